@@ -1,0 +1,338 @@
+"""Pins the CPU oracle before anything is compared against it.
+
+Sources of truth, strongest first: vectors the reference's own tests hold (IQ1_M), vectors written by
+the reference's numpy decoders (tests/golden/make_reference_fixtures.py), the reference's compiled
+C++ CPU kernels (oracle/_ref), torch's E4M3 cast, and hand-built blocks whose values follow from the
+format definition with one field live at a time.
+"""
+import hashlib
+import json
+import re
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import gguf_oracle as O
+from oracle import ref_ext
+
+REFERENCE = Path("/root/reference")
+
+
+def _load(golden_dir, name):
+    raw = json.loads((golden_dir / name).read_text())
+    blocks = np.frombuffer(bytes.fromhex(raw["blocks_u8"]), dtype=np.uint8)
+    values = np.frombuffer(bytes.fromhex(raw["values_f32"]), dtype="<f4")
+    return raw, blocks, values
+
+
+def test_iq1m_matches_reference_held_vector(golden_dir):
+    raw, blocks, values = _load(golden_dir, "iq1m_oracle.json")
+    blocks = blocks.reshape(raw["n_blocks"], raw["block_bytes"])
+    got = O.dequant_iq1_m(blocks)
+    np.testing.assert_array_equal(got, values.reshape(raw["n_blocks"], 256))
+
+
+@pytest.mark.parametrize("type_name", ["q8_0", "q4_k", "q5_k", "iq2_xxs"])
+def test_decoders_match_reference_decoder_vectors(golden_dir, type_name):
+    raw, blocks, values = _load(golden_dir, f"{type_name}_reference_decode.json")
+    blocks = blocks.reshape(raw["rows"], raw["blocks_per_row"], raw["block_bytes"])
+    got = O.dequant_rows(blocks, type_name)
+    want = values.reshape(raw["rows"], -1)
+    np.testing.assert_array_equal(got, want)
+
+
+def test_codebooks_match_reference_digests(golden_dir):
+    dig = json.loads((golden_dir / "codebook_digests.json").read_text())
+    signed = np.ascontiguousarray(O.iq2xxs_signed_grid())
+    iq1 = np.ascontiguousarray(O.iq1_grid_i8())
+    assert list(signed.shape) == dig["iq2xxs_signed_grid"]["shape"] and signed.dtype == np.int8
+    assert hashlib.sha256(signed.tobytes()).hexdigest() == dig["iq2xxs_signed_grid"]["sha256"]
+    assert list(iq1.shape) == dig["iq1_grid_i8"]["shape"] and iq1.dtype == np.int8
+    assert hashlib.sha256(iq1.tobytes()).hexdigest() == dig["iq1_grid_i8"]["sha256"]
+    assert set(np.unique(iq1).tolist()) == {-1, 0, 1}
+
+
+@pytest.mark.skipif(not REFERENCE.exists(), reason="reference checkout not mounted")
+def test_codebooks_match_ggml_header_text():
+    hdr = (REFERENCE / "src/csrc/llama_mmq/ggml-common.h").read_text()
+
+    def table(name, n):
+        m = re.search(r"GGML_TABLE_BEGIN\([^,]+,\s*%s,\s*%s\)(.*?)GGML_TABLE_END\(\)" % (name, n), hdr, flags=re.S)
+        return m.group(1)
+
+    g2 = np.asarray([int(v, 16) for v in re.findall(r"0x[0-9a-fA-F]+", table("iq2xxs_grid", 256))], dtype="<u8")
+    np.testing.assert_array_equal(g2.view(np.uint8).reshape(256, 8), O.iq2xxs_grid_u8())
+    g1 = np.asarray([int(v, 16) for v in re.findall(r"0x[0-9a-fA-F]+", table("iq1s_grid", "NGRID_IQ1S"))], dtype="<u8")
+    np.testing.assert_array_equal(g1.view(np.int8).reshape(2048, 8), O.iq1_grid_i8())
+    ks = np.asarray([int(v) for v in re.findall(r"\d+", table("ksigns_iq2xs", 128))], dtype=np.uint8)
+    np.testing.assert_array_equal(ks, O.ksigns_u8())
+
+
+@pytest.mark.skipif(not ref_ext.available(), reason="oracle/_ref not built")
+@pytest.mark.parametrize("type_name", ["iq2_xxs", "q2_k"])
+def test_decoders_match_compiled_reference_kernels_on_unit_vectors(type_name):
+    """dot(e_i, row) of the reference's C++ block dot returns weight i with no rounding beyond the
+    decoder's own, so unit vectors read the reference's dequantized row back bit for bit."""
+    rng = np.random.default_rng(7)
+    bb = O.BLOCK_BYTES[type_name]
+    blocks = rng.integers(0, 256, size=(5, 2, bb), dtype=np.uint8)
+    fields = [0] if type_name == "iq2_xxs" else [80, 82]
+    for off in fields:
+        vals = rng.uniform(0.002, 0.05, size=(5, 2)) * rng.choice([-1.0, 1.0], size=(5, 2))
+        blocks[..., off:off + 2] = vals.astype("<f2").view(np.uint8).reshape(5, 2, 2)
+    eye = np.eye(512, dtype=np.float32)
+    got = ref_ext.quantized_matmul(eye, blocks, O.TYPE_IDS[type_name], O.iq2xxs_signed_grid())   # [512, 5]
+    want = O.dequant_rows(blocks, type_name)
+    np.testing.assert_array_equal(got.T, want)
+
+
+@pytest.mark.skipif(not ref_ext.available(), reason="oracle/_ref not built")
+def test_moe_oracle_matches_compiled_reference_expert_forward():
+    rng = np.random.default_rng(11)
+    d, inter, t = 512, 256, 3
+    w1 = rng.integers(0, 256, size=(inter, d // 256, 66), dtype=np.uint8)
+    w3 = rng.integers(0, 256, size=(inter, d // 256, 66), dtype=np.uint8)
+    w2 = rng.integers(0, 256, size=(d, inter // 256, 84), dtype=np.uint8)
+    for w in (w1, w3):
+        w[..., 0:2] = rng.uniform(0.01, 0.04, size=w.shape[:2]).astype("<f2").view(np.uint8).reshape(w.shape[:2] + (2,))
+    for off in (80, 82):
+        w2[..., off:off + 2] = rng.uniform(0.01, 0.04, size=w2.shape[:2]).astype("<f2").view(np.uint8).reshape(w2.shape[:2] + (2,))
+    x = rng.standard_normal((t, d)).astype(np.float32)
+    rw = rng.uniform(0.1, 1.0, size=t).astype(np.float32)
+    for limit in (0.0, 0.75):
+        ref = ref_ext.expert_forward(x, rw, w1, w3, w2, 0, 0, 1, limit, O.iq2xxs_signed_grid())
+        got = O.moe_forward(x, np.arange(t), rw, np.zeros(t, dtype=np.int64),
+                            w1[None], w3[None], w2[None], "iq2_xxs", "iq2_xxs", "q2_k", limit)
+        assert O.rel_l2(ref, got) < 2e-6, limit
+
+
+# ---------------------------------------------------------------------------------------------
+# hand-built blocks: one live field at a time
+# ---------------------------------------------------------------------------------------------
+
+def _f16b(v):
+    return np.frombuffer(np.float16(v).tobytes(), dtype=np.uint8)
+
+
+def test_q8_0_closed_form():
+    b = np.zeros((1, 34), dtype=np.uint8)
+    b[0, 0:2] = _f16b(0.5)
+    b[0, 2:34] = np.arange(-16, 16, dtype=np.int8).view(np.uint8)
+    np.testing.assert_array_equal(O.dequant_q8_0(b)[0], 0.5 * np.arange(-16, 16, dtype=np.float32))
+
+
+def _k4_fields(sc, mn):
+    """Pack eight 6-bit scales and mins by the format definition, written index by index."""
+    s = [0] * 12
+    for j in range(8):
+        if j < 4:
+            s[j] |= sc[j]
+            s[j + 4] |= mn[j]
+        else:
+            s[j + 4] |= (sc[j] & 15) | ((mn[j] & 15) << 4)
+            s[j - 4] |= (sc[j] >> 4) << 6
+            s[j] |= (mn[j] >> 4) << 6
+    return np.asarray(s, dtype=np.uint8)
+
+
+@pytest.mark.parametrize("live", range(8))
+def test_q4_k_one_live_group(live):
+    """d = 1, dmin = 0, scale 1 in exactly one group: weights are the raw nibbles of that group."""
+    sc = [0] * 8
+    sc[live] = 1
+    b = np.zeros((1, 144), dtype=np.uint8)
+    b[0, 0:2] = _f16b(1.0)
+    b[0, 4:16] = _k4_fields(sc, [0] * 8)
+    rng = np.random.default_rng(live)
+    qs = rng.integers(0, 256, size=128, dtype=np.uint8)
+    b[0, 16:144] = qs
+    w = O.dequant_q4_k(b)[0]
+    pair, half = divmod(live, 2)
+    nib = (qs[32 * pair:32 * pair + 32] >> (4 * half)) & 15
+    want = np.zeros(256, dtype=np.float32)
+    want[32 * live:32 * live + 32] = nib
+    np.testing.assert_array_equal(w, want)
+
+
+@pytest.mark.parametrize("live", range(8))
+def test_q4_k_min_only(live):
+    """d = 0, dmin = 1: weights are minus the 6-bit min of their group, exercising both index branches."""
+    mn = [0] * 8
+    mn[live] = 37 + live          # > 15 so the high bits are exercised
+    b = np.zeros((1, 144), dtype=np.uint8)
+    b[0, 2:4] = _f16b(1.0)
+    b[0, 4:16] = _k4_fields([0] * 8, mn)
+    want = np.zeros(256, dtype=np.float32)
+    want[32 * live:32 * live + 32] = -(37 + live)
+    np.testing.assert_array_equal(O.dequant_q4_k(b)[0], want)
+    b5 = np.zeros((1, 176), dtype=np.uint8)
+    b5[0, 2:4] = _f16b(1.0)
+    b5[0, 4:16] = _k4_fields([0] * 8, mn)
+    np.testing.assert_array_equal(O.dequant_q5_k(b5)[0], want)
+
+
+@pytest.mark.parametrize("live", range(8))
+def test_q5_k_high_bit_plane(live):
+    """All nibbles zero, one qh bit plane set: exactly one group reads 16 * scale."""
+    sc = [3] * 8
+    b = np.zeros((1, 176), dtype=np.uint8)
+    b[0, 0:2] = _f16b(0.25)
+    b[0, 4:16] = _k4_fields(sc, [0] * 8)
+    b[0, 16:48] = 1 << live
+    want = np.zeros(256, dtype=np.float32)
+    want[32 * live:32 * live + 32] = 0.25 * 3 * 16
+    np.testing.assert_array_equal(O.dequant_q5_k(b)[0], want)
+
+
+def test_q2_k_closed_form_group_layout():
+    rng = np.random.default_rng(3)
+    b = np.zeros((1, 84), dtype=np.uint8)
+    scales = rng.integers(0, 256, size=16, dtype=np.uint8)
+    qs = rng.integers(0, 256, size=64, dtype=np.uint8)
+    b[0, 0:16] = scales
+    b[0, 16:80] = qs
+    b[0, 80:82] = _f16b(0.5)
+    b[0, 82:84] = _f16b(0.25)
+    w = O.dequant_q2_k(b)[0]
+    # ggml's dequantize_row_q2_K order: two halves of 128; inside a half four shifts, each shift
+    # yields two 16-weight groups (bytes 0..15 then 16..31 of the half).
+    want = np.empty(256, dtype=np.float32)
+    y = 0
+    is_ = 0
+    for half in range(2):
+        q = qs[32 * half:32 * half + 32]
+        for shift in (0, 2, 4, 6):
+            for part in range(2):
+                sc = scales[is_]
+                is_ += 1
+                for l in range(16):
+                    want[y] = np.float32(0.5 * (sc & 15) * ((q[16 * part + l] >> shift) & 3)) - np.float32(0.25 * (sc >> 4))
+                    y += 1
+    np.testing.assert_array_equal(w, want)
+
+
+def test_iq2_xxs_single_entry_signs_and_scale():
+    b = np.zeros((1, 66), dtype=np.uint8)
+    b[0, 0:2] = _f16b(2.0)
+    # sub-block 5: grid ids 7, 0, 0, 0; sign index of part 0 = 0b0000011 (odd parity -> bit 7 set); ls nibble 9
+    aux = (0b0000011) | (9 << 28)
+    b[0, 2 + 8 * 5:2 + 8 * 5 + 4] = [7, 0, 0, 0]
+    b[0, 2 + 8 * 5 + 4:2 + 8 * 5 + 8] = np.frombuffer(np.uint32(aux).tobytes(), dtype=np.uint8)
+    w = O.dequant_iq2_xxs(b)[0]
+    g = O.iq2xxs_grid_u8()[7].astype(np.float32)
+    sign = np.array([-1, -1, 1, 1, 1, 1, 1, 1], dtype=np.float32)   # bits 0, 1 set; popcount 2 -> parity 0
+    np.testing.assert_array_equal(w[160:168], 0.125 * 2.0 * 19 * g * sign)
+    # parity case: sign index 0b0000001 has odd popcount, so element 7 flips too
+    aux = (0b0000001) | (9 << 28)
+    b[0, 2 + 8 * 5 + 4:2 + 8 * 5 + 8] = np.frombuffer(np.uint32(aux).tobytes(), dtype=np.uint8)
+    w = O.dequant_iq2_xxs(b)[0]
+    sign = np.array([-1, 1, 1, 1, 1, 1, 1, -1], dtype=np.float32)
+    np.testing.assert_array_equal(w[160:168], 0.125 * 2.0 * 19 * g * sign)
+
+
+def test_fp8_decode_matches_torch_cast_on_all_codes():
+    codes = np.arange(256, dtype=np.uint8)
+    want = torch.from_numpy(codes.copy()).view(torch.float8_e4m3fn).to(torch.float32).numpy()
+    got = O.fp8_e4m3_decode(codes)
+    finite = np.isfinite(want)
+    assert (~finite).sum() == 2 and np.isnan(got[~finite]).all()
+    np.testing.assert_array_equal(got[finite], want[finite])
+
+
+def test_fp8_encode_rne_matches_torch_cast():
+    rng = np.random.default_rng(5)
+    x = np.concatenate([rng.standard_normal(20000).astype(np.float32) * 100,
+                        rng.standard_normal(20000).astype(np.float32) * 0.01,
+                        O.fp8_e4m3_decode(np.arange(127, dtype=np.uint8)),          # exact values
+                        np.array([448.0, -448.0, 0.0, 17.0, 18.0, 19.0, 21.0], dtype=np.float32)])
+    x = np.clip(x, -448, 448)
+    want = torch.from_numpy(x).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    got = O.fp8_e4m3_encode_rne(x)
+    # +0 / -0 codes may differ in sign bit for exact zeros only
+    nz = x != 0
+    np.testing.assert_array_equal(got[nz], want[nz])
+
+
+def test_fp8_block_scale_indexing_on_unaligned_shape():
+    rng = np.random.default_rng(9)
+    n, k = 130, 300
+    codes = rng.integers(0, 127, size=(n, k), dtype=np.uint8)
+    scale = rng.uniform(0.5, 2.0, size=(2, 3)).astype(np.float32)
+    w = O.dequant_fp8_block(codes, scale)
+    for r, c in [(0, 0), (127, 127), (128, 0), (129, 128), (5, 299), (129, 256)]:
+        assert w[r, c] == O.fp8_e4m3_decode(codes[r:r + 1, c:c + 1])[0, 0] * scale[r // 128, c // 128]
+
+
+@pytest.mark.parametrize("group", [16, 32])
+def test_q8_1_quantizer_invariants(group):
+    rng = np.random.default_rng(2)
+    x = rng.standard_normal((4, 256)).astype(np.float32)
+    x[1, 32:64] = 0.0
+    q, s = O.q8_1_quantize(x, group)
+    assert q.dtype == np.int8 and np.abs(q.astype(np.int32)).max() <= 127
+    rec = q.reshape(4, -1, group).astype(np.float32) * s[..., None]
+    assert (np.abs(rec - x.reshape(4, -1, group)) <= s[..., None] * 0.5000001).all()
+    amax_idx = np.abs(x.reshape(4, -1, group)).argmax(axis=-1)
+    top = np.take_along_axis(np.abs(q.reshape(4, -1, group).astype(np.int32)), amax_idx[..., None], axis=-1)[..., 0]
+    zero = (np.abs(x.reshape(4, -1, group)).max(axis=-1) == 0)
+    assert (top[~zero] == 127).all() and (q.reshape(4, -1, group)[zero] == 0).all()
+    assert (s[zero] == np.float32(1e-8)).all()
+
+
+def test_fp8_act_quant_matches_torch_recipe():
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal((3, 256)).astype(np.float32)
+    x[2, :128] = 0
+    codes, s = O.fp8_act_quant(x)
+    xt = torch.from_numpy(x)
+    st = xt.abs().view(3, 2, 128).amax(dim=-1).clamp_min(1e-4) / 448.0
+    qt = torch.clamp(xt / st.repeat_interleave(128, dim=-1), -448.0, 448.0).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    np.testing.assert_array_equal(s, st.numpy())
+    nz = x != 0
+    np.testing.assert_array_equal(codes[nz], qt[nz])
+
+
+def test_swiglu_route_closed_form():
+    g = np.array([[0.0, 2.0, -1.0, 10.0]], dtype=np.float32)
+    u = np.array([[3.0, -5.0, 0.5, 9.0]], dtype=np.float32)
+    w = np.array([0.5], dtype=np.float32)
+    h = O.swiglu_route(g, u, w, 0.0)[0]
+    silu = lambda v: v / (1 + np.exp(-v))
+    np.testing.assert_allclose(h, [0.0, silu(2.0) * -5.0 * 0.5, silu(-1.0) * 0.5 * 0.5, silu(10.0) * 9 * 0.5], rtol=1e-12)
+    h = O.swiglu_route(g, u, w, 4.0)[0]
+    np.testing.assert_allclose(h, [0.0, silu(2.0) * -4.0 * 0.5, silu(-1.0) * 0.5 * 0.5, silu(4.0) * 4 * 0.5], rtol=1e-12)
+
+
+def test_group_routes_invariants():
+    rng = np.random.default_rng(8)
+    t, k, e = 17, 4, 12
+    idx = np.stack([rng.choice(e + 6, size=k, replace=False) for _ in range(t)]).astype(np.int64)
+    w = rng.uniform(size=(t, k)).astype(np.float32)
+    start, n_local = 3, e
+    local_ids, toks, rw, seg = O.group_routes(idx, w, start, n_local)
+    assert seg[0] == 0 and (np.diff(seg) >= 0).all() and seg[-1] == len(toks) == len(rw)
+    for le in range(n_local):
+        got = sorted(zip(toks[seg[le]:seg[le + 1]].tolist(), rw[seg[le]:seg[le + 1]].tolist()))
+        want = sorted((tt, float(w[tt, kk])) for tt in range(t) for kk in range(k) if idx[tt, kk] - start == le)
+        assert got == want
+    assert local_ids.tolist() == [le for le in range(n_local) if seg[le + 1] > seg[le]]
+
+
+def test_kquant_int8_semantics_close_to_float_semantics():
+    """The int8-activation statement must agree with the float statement up to activation rounding
+    (a dropped min term or a swapped scale shows up as an O(1) difference)."""
+    from pocketllm_amd import block_codec as C
+    rng = np.random.default_rng(12)
+    w = (rng.standard_normal((24, 512)) * 0.02).astype(np.float32)
+    x = rng.standard_normal((5, 512)).astype(np.float32)
+    for name, enc in (("q4_k", C.quantize_q4_k), ("q5_k", C.quantize_q5_k)):
+        blocks = enc(w)
+        yf = O.matmul_f(x, O.dequant_rows(blocks, name))
+        yq = O.kquant_gemm_q(x, blocks, name)
+        assert O.rel_l2(yq, yf) < 1.5e-2, name
+        # exact agreement when the activations are already on the int8 lattice
+        xq, xs = O.q8_1_quantize(x)
+        xl = (xq.reshape(5, -1, 32).astype(np.float32) * xs[..., None]).reshape(5, 512)
+        assert O.rel_l2(O.kquant_gemm_q(xl, blocks, name), O.matmul_f(xl, O.dequant_rows(blocks, name))) < 1e-6, name
