@@ -1,0 +1,48 @@
+"""ctypes binding of libpllm_hip.so (the C ABI declared in include/pllm_hip.h)."""
+from __future__ import annotations
+
+import ctypes
+from pathlib import Path
+
+LIB_PATH = Path(__file__).resolve().parent / "libpllm_hip.so"
+
+PLLM_OK = 0
+DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
+
+_c_void_p = ctypes.c_void_p
+_i64 = ctypes.c_int64
+_int = ctypes.c_int
+
+# name -> (restype, argtypes); must list every symbol include/pllm_hip.h declares
+SIGNATURES = {
+    "pllm_status_string": (ctypes.c_char_p, [_int]),
+    "pllm_abi_version": (_int, []),
+    "pllm_gguf_block_bytes": (_int, [_int]),
+    "pllm_q8_0_gemm": (_int, [_c_void_p, _int, _c_void_p, _c_void_p, _int, _i64, _i64, _i64, _i64, _c_void_p]),
+    "pllm_gguf_quant_gemm": (_int, [_c_void_p, _int, _c_void_p, _int, _c_void_p, _int, _i64, _i64, _i64, _i64, _c_void_p]),
+}
+
+_LIB = None
+
+
+def load_library():
+    """Returns the loaded library, or None when libpllm_hip.so has not been built."""
+    global _LIB
+    if _LIB is not None:
+        return _LIB
+    if not LIB_PATH.exists():
+        return None
+    lib = ctypes.CDLL(str(LIB_PATH))
+    for name, (restype, argtypes) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = restype
+        fn.argtypes = argtypes
+    _LIB = lib
+    return lib
+
+
+def check(status: int, what: str) -> None:
+    if status != PLLM_OK:
+        lib = load_library()
+        msg = lib.pllm_status_string(status).decode() if lib is not None else str(status)
+        raise RuntimeError(f"{what}: {msg} (status {status})")

@@ -1,0 +1,140 @@
+// Device-side helpers shared by the raw-block kernels (gfx950, wave64).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/pllm_hip.h"
+
+namespace pllm {
+
+// ---- scalar conversions -------------------------------------------------------------------
+struct bf16_t { uint16_t bits; };
+struct f16_t { _Float16 v; };
+
+__device__ __forceinline__ float to_float(float v) { return v; }
+__device__ __forceinline__ float to_float(bf16_t v) { return __uint_as_float(static_cast<uint32_t>(v.bits) << 16); }
+__device__ __forceinline__ float to_float(f16_t v) { return static_cast<float>(v.v); }
+
+__device__ __forceinline__ float f16_bits_to_float(uint32_t bits) {
+    union { uint16_t u; _Float16 h; } c;
+    c.u = static_cast<uint16_t>(bits);
+    return static_cast<float>(c.h);
+}
+
+template <typename T> __device__ __forceinline__ T from_float(float v);
+template <> __device__ __forceinline__ float from_float<float>(float v) { return v; }
+template <> __device__ __forceinline__ f16_t from_float<f16_t>(float v) { f16_t r; r.v = static_cast<_Float16>(v); return r; }
+template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float v) {
+    // round to nearest even; NaN stays NaN
+    uint32_t u = __float_as_uint(v);
+    bf16_t r;
+    if ((u & 0x7fffffffu) > 0x7f800000u) { r.bits = static_cast<uint16_t>((u >> 16) | 0x40u); return r; }
+    u += 0x7fffu + ((u >> 16) & 1u);
+    r.bits = static_cast<uint16_t>(u >> 16);
+    return r;
+}
+
+// ---- integer dot and cross-lane ------------------------------------------------------------
+__device__ __forceinline__ int dot4(uint32_t a, uint32_t b, int c) {
+    return __builtin_amdgcn_sdot4(static_cast<int>(a), static_cast<int>(b), c, false);
+}
+
+// Sum over aligned groups of WIDTH lanes (WIDTH a power of two <= 64); every lane gets the total.
+template <int WIDTH>
+__device__ __forceinline__ float group_sum(float v) {
+#pragma unroll
+    for (int off = 1; off < WIDTH; off <<= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+template <int WIDTH>
+__device__ __forceinline__ float group_max(float v) {
+#pragma unroll
+    for (int off = 1; off < WIDTH; off <<= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+// ---- activation staging --------------------------------------------------------------------
+// Activations are split per 32 elements into two int8 terms,
+//     x[i] ~= xs[g] * (hi[i] + lo[i] / 254),   xs[g] = amax_g / 127,
+// so that integer dot products against the weight codes carry ~15 bits of each activation, enough
+// to stay far below 1e-3 relative error against float activations.  sum16[] holds the exact float
+// sum of every 16 activations for the "minus dmin * m" terms of the K-quants.
+constexpr float kLoInv = 1.0f / 254.0f;
+
+struct StagedX {
+    int8_t* hi;      // [kpad]
+    int8_t* lo;      // [kpad]
+    float* xs;       // [kpad / 32]
+    float* sum16;    // [kpad / 16]
+};
+
+__host__ __device__ inline size_t staged_x_bytes(int kpad) {
+    return static_cast<size_t>(kpad) * 2 + static_cast<size_t>(kpad / 32) * 4 + static_cast<size_t>(kpad / 16) * 4;
+}
+
+__device__ __forceinline__ StagedX carve_staged_x(unsigned char* smem, int kpad) {
+    StagedX s;
+    s.hi = reinterpret_cast<int8_t*>(smem);
+    s.lo = s.hi + kpad;
+    s.xs = reinterpret_cast<float*>(s.lo + kpad);
+    s.sum16 = s.xs + kpad / 32;
+    return s;
+}
+
+// Quantize four activations of one lane; the eight lanes of an aligned group share a 32-block.
+__device__ __forceinline__ void quantize4(const float v[4], uint32_t& hi, uint32_t& lo, float& scale) {
+    float am = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
+    am = group_max<8>(am);
+    const float inv = am > 0.0f ? 127.0f / am : 0.0f;
+    scale = am * (1.0f / 127.0f);
+    hi = 0; lo = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        float q = fminf(fmaxf(rintf(v[i] * inv), -127.0f), 127.0f);
+        float r = v[i] - q * scale;
+        float l = fminf(fmaxf(rintf(r * inv * 254.0f), -127.0f), 127.0f);
+        hi |= (static_cast<uint32_t>(static_cast<int>(q)) & 0xffu) << (8 * i);
+        lo |= (static_cast<uint32_t>(static_cast<int>(l)) & 0xffu) << (8 * i);
+    }
+}
+
+// All threads of the workgroup call this; k <= kpad, kpad a multiple of 256.  Caller synchronizes.
+template <typename XT>
+__device__ __forceinline__ void stage_activations(const XT* __restrict__ x, int k, int kpad, const StagedX& s) {
+    for (int e0 = threadIdx.x * 4; e0 < kpad; e0 += blockDim.x * 4) {
+        float v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = (e0 + i < k) ? to_float(x[e0 + i]) : 0.0f;
+        uint32_t hi, lo;
+        float scale;
+        quantize4(v, hi, lo, scale);
+        *reinterpret_cast<uint32_t*>(s.hi + e0) = hi;
+        *reinterpret_cast<uint32_t*>(s.lo + e0) = lo;
+        float sum = group_sum<4>((v[0] + v[1]) + (v[2] + v[3]));
+        if ((threadIdx.x & 3) == 0) s.sum16[e0 >> 4] = sum;
+        if ((threadIdx.x & 7) == 0) s.xs[e0 >> 5] = scale;
+    }
+}
+
+// Runtime-dtype front ends (the dtype is uniform, so the switch costs one scalar branch).
+__device__ __forceinline__ void stage_activations_any(const void* x, int x_dtype, size_t offset, int k, int kpad,
+                                                      const StagedX& s) {
+    if (x_dtype == PLLM_BF16) stage_activations(static_cast<const bf16_t*>(x) + offset, k, kpad, s);
+    else if (x_dtype == PLLM_F16) stage_activations(static_cast<const f16_t*>(x) + offset, k, kpad, s);
+    else stage_activations(static_cast<const float*>(x) + offset, k, kpad, s);
+}
+
+__device__ __forceinline__ float load_any(const void* x, int x_dtype, size_t i) {
+    if (x_dtype == PLLM_BF16) return to_float(static_cast<const bf16_t*>(x)[i]);
+    if (x_dtype == PLLM_F16) return to_float(static_cast<const f16_t*>(x)[i]);
+    return static_cast<const float*>(x)[i];
+}
+
+__device__ __forceinline__ void store_any(void* y, int y_dtype, size_t i, float v) {
+    if (y_dtype == PLLM_BF16) static_cast<bf16_t*>(y)[i] = from_float<bf16_t>(v);
+    else if (y_dtype == PLLM_F16) static_cast<f16_t*>(y)[i] = from_float<f16_t>(v);
+    else static_cast<float*>(y)[i] = v;
+}
+
+}  // namespace pllm

@@ -1,0 +1,148 @@
+"""GPU parity of the dense decode matvec operators against the float-activation oracle.
+
+Gate: rel-L2 <= 1e-3 on the float32 outputs (the bar the hot path is held to); the kernels carry the
+activations as two int8 terms, so the measured distance is around 1e-5.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import gguf_oracle as O
+from pocketllm_amd import block_codec as C
+from pocketllm_amd.cuda_loader import load_cuda_kernel
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-3
+ENCODERS = {"q4_k": C.quantize_q4_k, "q5_k": C.quantize_q5_k, "q2_k": C.quantize_q2_k}
+
+
+@pytest.fixture(scope="module")
+def mod():
+    m = load_cuda_kernel()
+    assert m is not None, "libpllm_hip.so missing: build it before running GPU tests"
+    assert torch.cuda.is_available()
+    return m
+
+
+def _weights(rng, n, k):
+    return (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
+
+
+def _run_dense(mod, type_name, blocks, x_np, x_dtype, k):
+    dev = torch.device("cuda:0")
+    x = torch.from_numpy(x_np).to(dev).to(x_dtype).contiguous()
+    b = torch.from_numpy(blocks).to(dev)
+    grid = torch.empty(0, dtype=torch.int8, device=dev)
+    y = mod.gguf_quant_gemm_forward(x, b, k, O.TYPE_IDS[type_name], grid, out_dtype=torch.float32)
+    torch.cuda.synchronize()
+    return x.float().cpu().numpy(), y.cpu().numpy()
+
+
+@pytest.mark.parametrize("type_name", ["q4_k", "q5_k", "q2_k"])
+@pytest.mark.parametrize("n,k,rows", [(64, 256, 1), (37, 768, 1), (100, 5120, 1), (16, 2048, 3), (9, 17408, 1), (33, 1000, 2)])
+def test_kquant_matvec_matches_oracle(mod, type_name, n, k, rows):
+    rng = np.random.default_rng(1000 + n + k)
+    blocks = ENCODERS[type_name](_weights(rng, n, k))
+    x_np = rng.standard_normal((rows, k)).astype(np.float32)
+    for dt in (torch.bfloat16, torch.float32, torch.float16):
+        print(f"case {type_name} n={n} k={k} rows={rows} {dt}", flush=True)
+        x_used, y = _run_dense(mod, type_name, blocks, x_np, dt, k)
+        want = O.matmul_f(x_used, O.dequant_rows(blocks, type_name, k))
+        err = O.rel_l2(y, want)
+        assert err <= TOL, (type_name, n, k, rows, dt, err)
+        assert err < 2e-4
+
+
+@pytest.mark.parametrize("type_name", ["q4_k", "q5_k", "q2_k"])
+def test_kquant_matvec_random_bytes(mod, type_name):
+    """Uniformly random block bytes reach every scale/min/high-bit code, not only what the encoder emits."""
+    rng = np.random.default_rng(77)
+    n, bpr = 48, 5
+    bb = O.BLOCK_BYTES[type_name]
+    blocks = rng.integers(0, 256, size=(n, bpr, bb), dtype=np.uint8)
+    for off in ([0, 2] if type_name != "q2_k" else [80, 82]):
+        vals = rng.uniform(0.001, 0.05, size=(n, bpr)) * rng.choice([-1.0, 1.0], size=(n, bpr))
+        blocks[..., off:off + 2] = vals.astype("<f2").view(np.uint8).reshape(n, bpr, 2)
+    x_np = rng.standard_normal((1, bpr * 256)).astype(np.float32)
+    x_used, y = _run_dense(mod, type_name, blocks, x_np, torch.float32, bpr * 256)
+    want = O.matmul_f(x_used, O.dequant_rows(blocks, type_name))
+    assert O.rel_l2(y, want) <= 2e-4
+
+
+@pytest.mark.parametrize("type_name,n,k", [("q4_k", 5120, 5120), ("q5_k", 5120, 5120), ("q4_k", 17408, 5120), ("q5_k", 17408, 5120)])
+def test_kquant_matvec_baseline_shapes(mod, type_name, n, k):
+    rng = np.random.default_rng(1002)
+    blocks = ENCODERS[type_name](_weights(rng, n, k))
+    x_np = rng.standard_normal((1, k)).astype(np.float32)
+    print(f"case {type_name} n={n} k={k}", flush=True)
+    x_used, y = _run_dense(mod, type_name, blocks, x_np, torch.bfloat16, k)
+    want = O.matmul_f(x_used, O.dequant_rows(blocks, type_name, k))
+    assert O.rel_l2(y, want) <= 2e-4
+
+
+def test_reference_output_dtype_is_bf16(mod):
+    rng = np.random.default_rng(5)
+    blocks = torch.from_numpy(C.quantize_q4_k(_weights(rng, 32, 512))).cuda()
+    x = torch.randn(2, 3, 512, device="cuda", dtype=torch.float16)
+    y = mod.gguf_quant_gemm_forward(x, blocks, 512, 3, torch.empty(0, dtype=torch.int8, device="cuda"))
+    assert y.dtype == torch.bfloat16 and tuple(y.shape) == (2, 3, 32)
+    y32 = mod.gguf_quant_gemm_prefill_forward(x, blocks, 512, 3, torch.empty(0, dtype=torch.int8, device="cuda"), out_dtype=torch.float32)
+    assert torch.equal(y32.to(torch.bfloat16), y)
+
+
+# ---------------------------------------------------------------------------------------------
+# Q8_0
+# ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("n,k,rows", [(96, 64, 2), (8, 256, 1), (130, 4096, 1), (4096, 4096, 1), (24, 1024, 3), (10, 200, 1), (5, 11008, 1)])
+def test_q8_0_matvec_matches_oracle(mod, n, k, rows):
+    rng = np.random.default_rng(1001 + n)
+    blocks = C.pack_q8_0(_weights(rng, n, k))
+    x_np = rng.standard_normal((rows, k)).astype(np.float32)
+    dev = torch.device("cuda:0")
+    b = torch.from_numpy(blocks).to(dev)
+    for dt in (torch.float32, torch.bfloat16):
+        print(f"case q8_0 n={n} k={k} rows={rows} {dt}", flush=True)
+        x = torch.from_numpy(x_np).to(dev).to(dt)
+        y = mod.q8_0_gemm_forward(x, b, k, out_dtype=torch.float32)
+        torch.cuda.synchronize()
+        want = O.matmul_f(x.float().cpu().numpy(), O.dequant_rows(blocks, "q8_0", k))
+        err = O.rel_l2(y.cpu().numpy(), want)
+        assert err <= 2e-4, (n, k, rows, dt, err)
+
+
+def test_q8_0_random_bytes_and_offset_base(mod):
+    rng = np.random.default_rng(3)
+    n, bpr = 40, 16
+    blocks = rng.integers(0, 256, size=(n + 1, bpr, 34), dtype=np.uint8)
+    vals = rng.uniform(0.001, 0.05, size=(n + 1, bpr)) * rng.choice([-1.0, 1.0], size=(n + 1, bpr))
+    blocks[..., 0:2] = vals.astype("<f2").view(np.uint8).reshape(n + 1, bpr, 2)
+    x_np = rng.standard_normal((1, bpr * 32)).astype(np.float32)
+    dev = torch.device("cuda:0")
+    full = torch.from_numpy(blocks).to(dev)
+    x = torch.from_numpy(x_np).to(dev)
+    for view, ref in ((full[:n], blocks[:n]), (full[1:], blocks[1:])):   # second view starts 544 B into the allocation
+        y = mod.q8_0_gemm_forward(x, view, bpr * 32, out_dtype=torch.float32)
+        torch.cuda.synchronize()
+        want = O.matmul_f(x_np, O.dequant_rows(ref, "q8_0"))
+        assert O.rel_l2(y.cpu().numpy(), want) <= 2e-4
+
+
+def test_argument_errors_match_reference_messages(mod):
+    dev = torch.device("cuda:0")
+    x = torch.randn(1, 512, device=dev)
+    blocks = torch.zeros(8, 2, 144, dtype=torch.uint8, device=dev)
+    grid = torch.empty(0, dtype=torch.int8, device=dev)
+    with pytest.raises(RuntimeError, match="inner dimension mismatch"):
+        mod.gguf_quant_gemm_forward(x, blocks, 256, 3, grid)
+    with pytest.raises(RuntimeError, match="unexpected GGUF block size for type_id"):
+        mod.gguf_quant_gemm_forward(x, blocks, 512, 4, grid)
+    with pytest.raises(RuntimeError, match="unsupported GGUF quant type_id"):
+        mod.gguf_quant_gemm_forward(x, blocks, 512, 11, grid)
+    with pytest.raises(RuntimeError, match="blocks do not cover row_elems"):
+        mod.gguf_quant_gemm_forward(torch.randn(1, 1024, device=dev), blocks, 1024, 3, grid)
+    with pytest.raises(RuntimeError, match="x must be float16, bfloat16, or float32"):
+        mod.gguf_quant_gemm_forward(x.double(), blocks, 512, 3, grid)
+    with pytest.raises(RuntimeError, match="q8_0 block size must be 34 bytes"):
+        mod.q8_0_gemm_forward(x, blocks, 512)
