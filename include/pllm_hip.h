@@ -56,11 +56,17 @@ int pllm_gguf_block_bytes(int type_id);
  *   blocks  [n, blocks_per_row, 34] uint8, blocks_per_row * 32 >= k (the tail is treated as zero
  *           activations)
  *   y       [rows, n]  y_dtype
+ *   workspace  device scratch of at least pllm_q8_0_gemm_workspace_bytes(...) bytes, 256-byte
+ *           aligned, private to this call until its kernels have run (it receives the
+ *           pre-quantized activations); the reference allocates its temporaries through torch in
+ *           the same place (src/csrc/cuda_kernel_impl.cu:9172-9175)
  * Replaces q8_0_gemm_forward (src/csrc/cuda_kernel.cpp:524-543, launcher
  * src/csrc/cuda_kernel_impl.cu:8472-8500, kernel 8345-8385).
  */
 int pllm_q8_0_gemm(const void* x, int x_dtype, const uint8_t* blocks, void* y, int y_dtype,
-                   int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row, void* stream);
+                   int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row,
+                   void* workspace, size_t workspace_bytes, void* stream);
+size_t pllm_q8_0_gemm_workspace_bytes(int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row);
 
 /*
  * Same contraction for 256-weight super-block types (type_id above).
@@ -72,7 +78,17 @@ int pllm_q8_0_gemm(const void* x, int x_dtype, const uint8_t* blocks, void* y, i
  * gguf_q2k_gemm_dp4a_forward (cuda_kernel.cpp:545-564).
  */
 int pllm_gguf_quant_gemm(const void* x, int x_dtype, const uint8_t* blocks, int type_id, void* y, int y_dtype,
-                         int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row, void* stream);
+                         int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row,
+                         void* workspace, size_t workspace_bytes, void* stream);
+size_t pllm_gguf_quant_gemm_workspace_bytes(int type_id, int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row);
+
+/*
+ * Measurement aids with no counterpart in the reference: a streaming copy and a streaming read of
+ * nbytes (a multiple of 16) with `blocks` workgroups of 256 threads.  They calibrate HBM byte
+ * counters against a transfer of known size.  sink: 4 writable bytes.
+ */
+int pllm_diag_stream_copy(const void* src, void* dst, size_t nbytes, int blocks, void* stream);
+int pllm_diag_stream_read(const void* src, void* sink, size_t nbytes, int blocks, void* stream);
 
 #ifdef __cplusplus
 }

@@ -12,14 +12,19 @@ DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
 _c_void_p = ctypes.c_void_p
 _i64 = ctypes.c_int64
 _int = ctypes.c_int
+_size_t = ctypes.c_size_t
 
 # name -> (restype, argtypes); must list every symbol include/pllm_hip.h declares
 SIGNATURES = {
     "pllm_status_string": (ctypes.c_char_p, [_int]),
     "pllm_abi_version": (_int, []),
     "pllm_gguf_block_bytes": (_int, [_int]),
-    "pllm_q8_0_gemm": (_int, [_c_void_p, _int, _c_void_p, _c_void_p, _int, _i64, _i64, _i64, _i64, _c_void_p]),
-    "pllm_gguf_quant_gemm": (_int, [_c_void_p, _int, _c_void_p, _int, _c_void_p, _int, _i64, _i64, _i64, _i64, _c_void_p]),
+    "pllm_q8_0_gemm": (_int, [_c_void_p, _int, _c_void_p, _c_void_p, _int, _i64, _i64, _i64, _i64, _c_void_p, _size_t, _c_void_p]),
+    "pllm_q8_0_gemm_workspace_bytes": (_size_t, [_i64, _i64, _i64, _i64]),
+    "pllm_gguf_quant_gemm": (_int, [_c_void_p, _int, _c_void_p, _int, _c_void_p, _int, _i64, _i64, _i64, _i64, _c_void_p, _size_t, _c_void_p]),
+    "pllm_gguf_quant_gemm_workspace_bytes": (_size_t, [_int, _i64, _i64, _i64, _i64]),
+    "pllm_diag_stream_copy": (_int, [_c_void_p, _c_void_p, _size_t, _int, _c_void_p]),
+    "pllm_diag_stream_read": (_int, [_c_void_p, _c_void_p, _size_t, _int, _c_void_p]),
 }
 
 _LIB = None

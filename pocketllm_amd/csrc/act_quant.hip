@@ -1,0 +1,101 @@
+// Activation pre-quantization: float / fp16 / bf16 rows -> int8 "images" the matvec kernels copy
+// into LDS (layouts in pllm_device.h and matvec_q8_0.hip).  One thread quantizes four values; the
+// eight threads of an aligned group share a 32-value block (amax by cross-lane max).
+#include "pllm_device.h"
+#include "pllm_internal.h"
+
+namespace pllm {
+namespace {
+
+constexpr int kThreads = 256;
+
+__global__ __launch_bounds__(kThreads) void act_image_256_kernel(
+    const void* __restrict__ x, int x_dtype, unsigned char* __restrict__ image, int k, int kpad, size_t image_stride) {
+    const int e0 = (blockIdx.x * kThreads + threadIdx.x) * 4;
+    if (e0 >= kpad) return;                                   // kpad is a multiple of 256: whole groups leave together
+    const size_t xoff = static_cast<size_t>(blockIdx.y) * k;
+    unsigned char* base = image + static_cast<size_t>(blockIdx.y) * image_stride;
+    int8_t* hi = reinterpret_cast<int8_t*>(base);
+    int8_t* lo = hi + kpad;
+    float2* gs = reinterpret_cast<float2*>(lo + kpad);
+    float* sum16 = reinterpret_cast<float*>(gs + kpad / 32);
+    float v[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = (e0 + i < k) ? load_any(x, x_dtype, xoff + e0 + i) : 0.0f;
+    uint32_t qh, ql;
+    float scale;
+    quantize4(v, qh, ql, scale);
+    *reinterpret_cast<uint32_t*>(hi + e0) = qh;
+    *reinterpret_cast<uint32_t*>(lo + e0) = ql;
+    const float sum = group_sum<4>((v[0] + v[1]) + (v[2] + v[3]));
+    const float sum32 = sum + __shfl_xor(sum, 4, 64);
+    if ((threadIdx.x & 3) == 0) sum16[e0 >> 4] = sum;
+    if ((threadIdx.x & 7) == 0) gs[e0 >> 5] = make_float2(scale * kLoInv, sum32);
+}
+
+// Q8_0 pair image: per pair of 32-value blocks 80 bytes that mirror the weight stream,
+//   [0,0, q0..q31, 0,0, q32..q63, 12 x 0],  then after all pairs: float xs[2 * pairs].
+__global__ __launch_bounds__(kThreads) void act_image_q8pair_kernel(
+    const void* __restrict__ x, int x_dtype, unsigned char* __restrict__ image, int k, int pairs, size_t image_stride) {
+    const int e0 = (blockIdx.x * kThreads + threadIdx.x) * 4;
+    if (e0 >= pairs * 64) return;
+    const size_t xoff = static_cast<size_t>(blockIdx.y) * k;
+    unsigned char* base = image + static_cast<size_t>(blockIdx.y) * image_stride;
+    unsigned char* hi = base;
+    unsigned char* lo = base + static_cast<size_t>(pairs) * 80;
+    float* xs = reinterpret_cast<float*>(lo + static_cast<size_t>(pairs) * 80);
+    float v[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = (e0 + i < k) ? load_any(x, x_dtype, xoff + e0 + i) : 0.0f;
+    uint32_t qh, ql;
+    float scale;
+    quantize4(v, qh, ql, scale);
+    const int b = e0 >> 5;
+    const int j = (e0 & 31) >> 2;
+    const int off = (b >> 1) * 80 + ((b & 1) ? 36 : 2) + 4 * j;   // 2-byte aligned
+    *reinterpret_cast<uint16_t*>(hi + off) = static_cast<uint16_t>(qh);
+    *reinterpret_cast<uint16_t*>(hi + off + 2) = static_cast<uint16_t>(qh >> 16);
+    *reinterpret_cast<uint16_t*>(lo + off) = static_cast<uint16_t>(ql);
+    *reinterpret_cast<uint16_t*>(lo + off + 2) = static_cast<uint16_t>(ql >> 16);
+    if (j == 0) {
+        const int p0 = (b >> 1) * 80;
+        if (b & 1) {
+            *reinterpret_cast<uint16_t*>(hi + p0 + 34) = 0;
+            *reinterpret_cast<uint16_t*>(lo + p0 + 34) = 0;
+#pragma unroll
+            for (int z = 68; z < 80; z += 4) {
+                *reinterpret_cast<uint32_t*>(hi + p0 + z) = 0;
+                *reinterpret_cast<uint32_t*>(lo + p0 + z) = 0;
+            }
+        } else {
+            *reinterpret_cast<uint16_t*>(hi + p0) = 0;
+            *reinterpret_cast<uint16_t*>(lo + p0) = 0;
+        }
+        xs[b] = scale;
+    }
+}
+
+}  // namespace
+
+size_t act_image_256_bytes(int bpr) { return (staged_x_bytes(bpr * 256) + 255) & ~static_cast<size_t>(255); }
+
+int act_image_256(const void* x, int x_dtype, int rows, int k, int bpr, void* image, hipStream_t stream) {
+    const int kpad = bpr * 256;
+    dim3 grid((kpad / 4 + kThreads - 1) / kThreads, rows);
+    hipLaunchKernelGGL(act_image_256_kernel, grid, dim3(kThreads), 0, stream, x, x_dtype,
+                       static_cast<unsigned char*>(image), k, kpad, act_image_256_bytes(bpr));
+    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+}
+
+size_t act_image_q8pair_bytes(int pairs) {
+    return (static_cast<size_t>(pairs) * 160 + static_cast<size_t>(pairs) * 8 + 255) & ~static_cast<size_t>(255);
+}
+
+int act_image_q8pair(const void* x, int x_dtype, int rows, int k, int pairs, void* image, hipStream_t stream) {
+    dim3 grid((pairs * 16 + kThreads - 1) / kThreads, rows);
+    hipLaunchKernelGGL(act_image_q8pair_kernel, grid, dim3(kThreads), 0, stream, x, x_dtype,
+                       static_cast<unsigned char*>(image), k, pairs, act_image_q8pair_bytes(pairs));
+    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+}
+
+}  // namespace pllm

@@ -35,17 +35,26 @@ int pllm_gguf_block_bytes(int type_id) {
 }
 
 int pllm_q8_0_gemm(const void* x, int x_dtype, const uint8_t* blocks, void* y, int y_dtype,
-                   int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row, void* stream) {
+                   int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row,
+                   void* workspace, size_t workspace_bytes, void* stream) {
     if (!x || !blocks || !y || !dtype_ok(x_dtype) || !dtype_ok(y_dtype)) return PLLM_ERR_INVALID_ARGUMENT;
     if (!fits_int(rows) || !fits_int(k) || !fits_int(n) || !fits_int(blocks_per_row)) return PLLM_ERR_INVALID_ARGUMENT;
     if (blocks_per_row * 32 < k) return PLLM_ERR_INVALID_ARGUMENT;
     if (rows > 65535) return PLLM_ERR_UNSUPPORTED;
     return pllm::q8_0_matvec(x, x_dtype, blocks, y, y_dtype, static_cast<int>(rows), static_cast<int>(k),
-                             static_cast<int>(n), static_cast<int>(blocks_per_row), static_cast<hipStream_t>(stream));
+                             static_cast<int>(n), static_cast<int>(blocks_per_row), workspace, workspace_bytes,
+                             static_cast<hipStream_t>(stream));
+}
+
+size_t pllm_q8_0_gemm_workspace_bytes(int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row) {
+    (void)k; (void)n;
+    if (!fits_int(rows) || !fits_int(blocks_per_row)) return 0;
+    return pllm::q8_0_matvec_workspace_bytes(static_cast<int>(rows), static_cast<int>(blocks_per_row));
 }
 
 int pllm_gguf_quant_gemm(const void* x, int x_dtype, const uint8_t* blocks, int type_id, void* y, int y_dtype,
-                         int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row, void* stream) {
+                         int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row,
+                         void* workspace, size_t workspace_bytes, void* stream) {
     if (!x || !blocks || !y || !dtype_ok(x_dtype) || !dtype_ok(y_dtype)) return PLLM_ERR_INVALID_ARGUMENT;
     if (!fits_int(rows) || !fits_int(k) || !fits_int(n) || !fits_int(blocks_per_row)) return PLLM_ERR_INVALID_ARGUMENT;
     if (blocks_per_row * 256 < k) return PLLM_ERR_INVALID_ARGUMENT;
@@ -57,10 +66,16 @@ int pllm_gguf_quant_gemm(const void* x, int x_dtype, const uint8_t* blocks, int 
         case PLLM_TYPE_Q5_K:
         case PLLM_TYPE_Q2_K:
             return pllm::kquant_matvec(x, x_dtype, blocks, type_id, y, y_dtype, static_cast<int>(rows), static_cast<int>(k),
-                                       static_cast<int>(n), static_cast<int>(blocks_per_row), s);
+                                       static_cast<int>(n), static_cast<int>(blocks_per_row), workspace, workspace_bytes, s);
         default:
             return PLLM_ERR_UNSUPPORTED;
     }
+}
+
+size_t pllm_gguf_quant_gemm_workspace_bytes(int type_id, int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row) {
+    (void)k; (void)n;
+    if (!fits_int(rows) || !fits_int(blocks_per_row) || pllm_gguf_block_bytes(type_id) == 0) return 0;
+    return pllm::kquant_matvec_workspace_bytes(static_cast<int>(rows), static_cast<int>(blocks_per_row));
 }
 
 }  // extern "C"

@@ -1,109 +1,186 @@
 // Decode matvec over raw Q4_K / Q5_K / Q2_K super-blocks (bandwidth-bound, wave64).
 //
-// Work split: a "team" of LPB adjacent lanes owns one 256-weight super-block at a time, every lane
-// loading 16 bytes of quants with one global_load_dwordx4 plus the block header shared by the team.
-// TPR teams stride over the super-blocks of one output row; a 256-thread workgroup therefore covers
-// (256 / LPB) / TPR rows.  All weight loads of a pass are issued before the workgroup quantizes the
-// activation row into LDS (two int8 terms per value), so the quantization hides under the HBM
-// latency.  Dots are v_dot4_i32_i8; scales and mins are unpacked in registers; the per-row sum is a
-// cross-lane reduction over the LPB * TPR lanes that share the row.
+// A wave owns 16 consecutive output rows and walks their super-blocks; the W waves of a workgroup
+// split a row's super-blocks between them (wave w takes blocks w, w + W, ...) and meet in a small
+// LDS reduction.  All weight loads of a pass are issued first; while they are in flight the
+// workgroup copies the pre-quantized activation image (two int8 terms per value, written once per
+// call by act_quant.hip) from L2 into LDS.
+//
+// Q4_K / Q5_K: the integer dots run on the matrix cores.  For one super-block index the wave forms
+//     C[m][n] = sum_k A[m][k] * B[k][n],     v_mfma_i32_16x16x64_i8, four of them per block,
+// with B = the 4/5-bit codes of the 16 rows (n = row, straight from the 16-byte global loads after
+// a nibble split) and A = the activation codes spread over 16 rows m = 2 * group + term, row m
+// holding the codes of 32-weight group `group` (term 0 = high int8 term, 1 = low term) and zeros
+// elsewhere.  One accumulator tile then holds, for every row, the eight per-group integer dots of
+// both terms; the lane that holds C[4s .. 4s+3][n] owns groups 2s and 2s+1 of row n and applies
+// their 6-bit scales and mins in float.  Which k sits where inside an MFMA is irrelevant as long
+// as A and B agree, and both are built per (lane / 16, byte) from the same positions.
+//
+// Q2_K keeps v_dot4_i32_i8 dots: four lanes share a block, 16 such teams (rows) per wave all on the
+// same block index, so that LDS reads of activations are broadcasts.
 #include "pllm_device.h"
+#include "pllm_internal.h"
 
 namespace pllm {
 namespace {
 
-constexpr int kThreads = 256;
+constexpr int kRowsPerWg = 16;
+constexpr int kMaxWaves = 8;
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ v4i as_v4i(const uint4& u) {
+    v4i r;
+    r.x = static_cast<int>(u.x); r.y = static_cast<int>(u.y); r.z = static_cast<int>(u.z); r.w = static_cast<int>(u.w);
+    return r;
+}
+
+// Eight 6-bit scales / mins of a K-quant header as bytes: lo word = entries 0..3, hi word = 4..7.
+struct K4Scales { uint32_t sc_lo, sc_hi, mn_lo, mn_hi; };
+__device__ __forceinline__ K4Scales k4_unpack(const uint4& hdr) {
+    const uint32_t u0 = hdr.y, u1 = hdr.z, u2 = hdr.w;
+    K4Scales r;
+    r.sc_lo = u0 & 0x3f3f3f3fu;
+    r.mn_lo = u1 & 0x3f3f3f3fu;
+    r.sc_hi = (u2 & 0x0f0f0f0fu) | (((u0 >> 6) & 0x03030303u) << 4);
+    r.mn_hi = ((u2 >> 4) & 0x0f0f0f0fu) | (((u1 >> 6) & 0x03030303u) << 4);
+    return r;
+}
+
+__device__ __forceinline__ uint4 nib_lo(const uint4& q) {
+    return make_uint4(q.x & 0x0f0f0f0fu, q.y & 0x0f0f0f0fu, q.z & 0x0f0f0f0fu, q.w & 0x0f0f0f0fu);
+}
+__device__ __forceinline__ uint4 nib_hi(const uint4& q) {
+    return make_uint4((q.x >> 4) & 0x0f0f0f0fu, (q.y >> 4) & 0x0f0f0f0fu, (q.z >> 4) & 0x0f0f0f0fu, (q.w >> 4) & 0x0f0f0f0fu);
+}
+__device__ __forceinline__ uint4 fifth_bit(const uint4& w, const uint4& qh, int bit) {
+    return make_uint4(w.x | (((qh.x >> bit) & 0x01010101u) << 4), w.y | (((qh.y >> bit) & 0x01010101u) << 4),
+                      w.z | (((qh.z >> bit) & 0x01010101u) << 4), w.w | (((qh.w >> bit) & 0x01010101u) << 4));
+}
 
 // ------------------------------------------------------------------------------------------------
-// Q4_K: 144 B = d(2) dmin(2) scales(12) qs(128).  8 lanes per block; lane j holds qs[16j, 16j+16):
-// low nibbles are weights 64p + 16h + i of group 2p, high nibbles the same offsets of group 2p+1
-// (p = j >> 1, h = j & 1).
+// Q4_K: 144 B = d(2) dmin(2) scales(12) qs(128).  Lane (n, ks) holds qs[16 ks, +16) and
+// qs[64 + 16 ks, +16).  With p = ks >> 1, h = ks & 1 the first chunk carries weights 16h + (0..15)
+// of group 2p in its low nibbles and of group 2p+1 in its high nibbles; the second chunk is the
+// same for groups 2p+4 and 2p+5.
+// Q5_K: 176 B = d dmin scales(12) qh(32) qs(128); same plus qh[16h, +16): bit g of qh byte 16h + t
+// is the fifth bit of weight 16h + t of group g.
 // ------------------------------------------------------------------------------------------------
 struct Q4K {
-    static constexpr int kLanesPerBlock = 8;
     static constexpr int kBlockBytes = 144;
-    struct Regs { uint4 hdr; uint4 qs; };
-    static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, int j) {
+    struct Regs { uint4 hdr; uint4 qa; uint4 qb; };
+    static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, int ks) {
         r.hdr = *reinterpret_cast<const uint4*>(blk);
-        r.qs = *reinterpret_cast<const uint4*>(blk + 16 + 16 * j);
+        r.qa = *reinterpret_cast<const uint4*>(blk + 16 + 16 * ks);
+        r.qb = *reinterpret_cast<const uint4*>(blk + 80 + 16 * ks);
     }
-    static __device__ __forceinline__ void zero(Regs& r) { r.hdr = make_uint4(0, 0, 0, 0); r.qs = r.hdr; }
+    // B operands of the four MFMAs of a block: groups 2p, 2p+1, 2p+4, 2p+5
+    static __device__ __forceinline__ void codes(const Regs& r, int, uint4 b[4]) {
+        b[0] = nib_lo(r.qa); b[1] = nib_hi(r.qa); b[2] = nib_lo(r.qb); b[3] = nib_hi(r.qb);
+    }
 };
 
-// Q5_K: 176 B = d dmin scales(12) qh(32) qs(128).  Same lane map as Q4_K plus qh[16h, 16h+16):
-// bit 2p of qh byte i is the fifth bit of the low-nibble weight, bit 2p+1 that of the high nibble.
 struct Q5K {
-    static constexpr int kLanesPerBlock = 8;
     static constexpr int kBlockBytes = 176;
-    struct Regs { uint4 hdr; uint4 qh; uint4 qs; };
-    static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, int j) {
+    struct Regs { uint4 hdr; uint4 qh; uint4 qa; uint4 qb; };
+    static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, int ks) {
         r.hdr = *reinterpret_cast<const uint4*>(blk);
-        r.qh = *reinterpret_cast<const uint4*>(blk + 16 + 16 * (j & 1));
-        r.qs = *reinterpret_cast<const uint4*>(blk + 48 + 16 * j);
+        r.qh = *reinterpret_cast<const uint4*>(blk + 16 + 16 * (ks & 1));
+        r.qa = *reinterpret_cast<const uint4*>(blk + 48 + 16 * ks);
+        r.qb = *reinterpret_cast<const uint4*>(blk + 112 + 16 * ks);
     }
-    static __device__ __forceinline__ void zero(Regs& r) { r.hdr = make_uint4(0, 0, 0, 0); r.qh = r.hdr; r.qs = r.hdr; }
+    static __device__ __forceinline__ void codes(const Regs& r, int ks, uint4 b[4]) {
+        const int g = 2 * (ks >> 1);
+        b[0] = fifth_bit(nib_lo(r.qa), r.qh, g);
+        b[1] = fifth_bit(nib_hi(r.qa), r.qh, g + 1);
+        b[2] = fifth_bit(nib_lo(r.qb), r.qh, g + 4);
+        b[3] = fifth_bit(nib_hi(r.qb), r.qh, g + 5);
+    }
 };
 
-// Eight 6-bit scales and mins of a K-quant header -> scale/min of groups 2p and 2p+1 as floats.
-__device__ __forceinline__ void k4_scales(const uint4& hdr, int p, float& sc0, float& sc1, float& m0, float& m1) {
-    const uint32_t u0 = hdr.y, u1 = hdr.z, u2 = hdr.w;
-    const uint32_t sc_lo = u0 & 0x3f3f3f3fu;
-    const uint32_t mn_lo = u1 & 0x3f3f3f3fu;
-    const uint32_t sc_hi = (u2 & 0x0f0f0f0fu) | (((u0 >> 6) & 0x03030303u) << 4);
-    const uint32_t mn_hi = ((u2 >> 4) & 0x0f0f0f0fu) | (((u1 >> 6) & 0x03030303u) << 4);
-    const uint32_t scw = (p < 2 ? sc_lo : sc_hi) >> ((p & 1) * 16);
-    const uint32_t mnw = (p < 2 ? mn_lo : mn_hi) >> ((p & 1) * 16);
-    sc0 = static_cast<float>(scw & 0xffu);
-    sc1 = static_cast<float>((scw >> 8) & 0xffu);
-    m0 = static_cast<float>(mnw & 0xffu);
-    m1 = static_cast<float>((mnw >> 8) & 0xffu);
-}
+template <typename FMT, int ITERS>
+__global__ __launch_bounds__(64 * kMaxWaves) void k45_mfma_matvec_kernel(
+    const unsigned char* __restrict__ image, size_t image_stride, const uint8_t* __restrict__ w,
+    void* __restrict__ y, int y_dtype, int n, int bpr) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int kpad = bpr * 256;
+    const int image_bytes = static_cast<int>(staged_x_bytes(kpad));
+    const StagedX sx = carve_staged_x(smem, kpad);
+    const int zero_off = image_bytes;                                        // 16 zero bytes
+    float* partial = reinterpret_cast<float*>(smem + image_bytes + 16);     // [waves][16]
 
-__device__ __forceinline__ float k45_finish(const uint4& hdr, int p, int h, int blk, const StagedX& sx,
-                                            const uint4& w0, const uint4& w1) {
-    const int base = blk * 256 + 64 * p + 16 * h;
-    const uint4 a0h = *reinterpret_cast<const uint4*>(sx.hi + base);
-    const uint4 a1h = *reinterpret_cast<const uint4*>(sx.hi + base + 32);
-    const uint4 a0l = *reinterpret_cast<const uint4*>(sx.lo + base);
-    const uint4 a1l = *reinterpret_cast<const uint4*>(sx.lo + base + 32);
-    int s0h = dot4(w0.x, a0h.x, 0); s0h = dot4(w0.y, a0h.y, s0h); s0h = dot4(w0.z, a0h.z, s0h); s0h = dot4(w0.w, a0h.w, s0h);
-    int s0l = dot4(w0.x, a0l.x, 0); s0l = dot4(w0.y, a0l.y, s0l); s0l = dot4(w0.z, a0l.z, s0l); s0l = dot4(w0.w, a0l.w, s0l);
-    int s1h = dot4(w1.x, a1h.x, 0); s1h = dot4(w1.y, a1h.y, s1h); s1h = dot4(w1.z, a1h.z, s1h); s1h = dot4(w1.w, a1h.w, s1h);
-    int s1l = dot4(w1.x, a1l.x, 0); s1l = dot4(w1.y, a1l.y, s1l); s1l = dot4(w1.z, a1l.z, s1l); s1l = dot4(w1.w, a1l.w, s1l);
-    float sc0, sc1, m0, m1;
-    k4_scales(hdr, p, sc0, sc1, m0, m1);
-    const float d = f16_bits_to_float(hdr.x & 0xffffu);
-    const float dmin = f16_bits_to_float(hdr.x >> 16);
-    const float xs0 = sx.xs[blk * 8 + 2 * p];
-    const float xs1 = sx.xs[blk * 8 + 2 * p + 1];
-    const float t0 = sx.sum16[blk * 16 + 4 * p + h];
-    const float t1 = sx.sum16[blk * 16 + 4 * p + 2 + h];
-    const float v0 = static_cast<float>(s0h) + static_cast<float>(s0l) * kLoInv;
-    const float v1 = static_cast<float>(s1h) + static_cast<float>(s1l) * kLoInv;
-    return d * (sc0 * xs0 * v0 + sc1 * xs1 * v1) - dmin * (m0 * t0 + m1 * t1);
-}
+    const int tid = threadIdx.x;
+    const int waves = blockDim.x >> 6;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    const int col = lane & 15;        // B/C column = output row within the tile; also A's row index m
+    const int ks = lane >> 4;         // k slice of A and B, row quad of C
+    const int row = blockIdx.x * kRowsPerWg + col;
+    const uint8_t* wrow = w + static_cast<size_t>(row < n ? row : 0) * bpr * FMT::kBlockBytes;
 
-__device__ __forceinline__ float lane_dot(const Q4K::Regs& r, int j, int blk, const StagedX& sx) {
-    const uint4 q = r.qs;
-    const uint4 w0 = make_uint4(q.x & 0x0f0f0f0fu, q.y & 0x0f0f0f0fu, q.z & 0x0f0f0f0fu, q.w & 0x0f0f0f0fu);
-    const uint4 w1 = make_uint4((q.x >> 4) & 0x0f0f0f0fu, (q.y >> 4) & 0x0f0f0f0fu, (q.z >> 4) & 0x0f0f0f0fu, (q.w >> 4) & 0x0f0f0f0fu);
-    return k45_finish(r.hdr, j >> 1, j & 1, blk, sx, w0, w1);
-}
+    // A side: this lane supplies row m = col = 2 * group + term of MFMA t, slice ks; it is non-zero
+    // only when MFMA t's slice ks belongs to `group`: G(t, ks) = 4 * (t >> 1) + 2 * (ks >> 1) + (t & 1)
+    int a_off[4], a_step[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        const int g = 4 * (t >> 1) + 2 * (ks >> 1) + (t & 1);
+        const bool active = (col >> 1) == g;
+        a_off[t] = active ? ((col & 1) ? kpad : 0) + 32 * g + 16 * (ks & 1) : zero_off;
+        a_step[t] = active ? 256 : 0;
+    }
 
-__device__ __forceinline__ float lane_dot(const Q5K::Regs& r, int j, int blk, const StagedX& sx) {
-    const int p = j >> 1;
-    const uint4 q = r.qs;
-    const uint4 b = r.qh;
-    const int s0 = 2 * p, s1 = 2 * p + 1;
-    const uint4 w0 = make_uint4((q.x & 0x0f0f0f0fu) | (((b.x >> s0) & 0x01010101u) << 4),
-                                (q.y & 0x0f0f0f0fu) | (((b.y >> s0) & 0x01010101u) << 4),
-                                (q.z & 0x0f0f0f0fu) | (((b.z >> s0) & 0x01010101u) << 4),
-                                (q.w & 0x0f0f0f0fu) | (((b.w >> s0) & 0x01010101u) << 4));
-    const uint4 w1 = make_uint4(((q.x >> 4) & 0x0f0f0f0fu) | (((b.x >> s1) & 0x01010101u) << 4),
-                                ((q.y >> 4) & 0x0f0f0f0fu) | (((b.y >> s1) & 0x01010101u) << 4),
-                                ((q.z >> 4) & 0x0f0f0f0fu) | (((b.z >> s1) & 0x01010101u) << 4),
-                                ((q.w >> 4) & 0x0f0f0f0fu) | (((b.w >> s1) & 0x01010101u) << 4));
-    return k45_finish(r.hdr, p, j & 1, blk, sx, w0, w1);
+    float acc = 0.0f;
+    bool staged = false;
+    for (int b0 = wave; b0 < bpr || !staged; b0 += waves * ITERS) {
+        typename FMT::Regs regs[ITERS];
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+            const int b = min(b0 + it * waves, bpr - 1);                    // clamped: always a valid address
+            FMT::load(regs[it], wrow + static_cast<size_t>(b) * FMT::kBlockBytes, ks);
+        }
+        if (!staged) {                       // first trip of every thread of the workgroup
+            copy_to_lds(smem, image + static_cast<size_t>(blockIdx.y) * image_stride, image_bytes);
+            if (tid < 4) reinterpret_cast<uint32_t*>(smem + zero_off)[tid] = 0;
+            __syncthreads();
+            staged = true;
+        }
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+            const int b = b0 + it * waves;
+            if (b < bpr) {                                                   // wave-uniform
+                uint4 bw[4];
+                FMT::codes(regs[it], ks, bw);
+                v4i c = {0, 0, 0, 0};
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const uint4 a = *reinterpret_cast<const uint4*>(smem + a_off[t] + b * a_step[t]);
+                    c = __builtin_amdgcn_mfma_i32_16x16x64_i8(as_v4i(a), as_v4i(bw[t]), c, 0, 0, 0);
+                }
+                // c = {group 2ks: hi, lo; group 2ks+1: hi, lo} for output row `col`
+                const float v0 = static_cast<float>(__mul24(c.x, 254) + c.y);
+                const float v1 = static_cast<float>(__mul24(c.z, 254) + c.w);
+                const float4 g2 = *reinterpret_cast<const float4*>(sx.gs + b * 8 + 2 * ks);   // {xs0, sum0, xs1, sum1}
+                const K4Scales sc = k4_unpack(regs[it].hdr);
+                const uint32_t scw = ((ks & 2) ? sc.sc_hi : sc.sc_lo) >> (16 * (ks & 1));
+                const uint32_t mnw = ((ks & 2) ? sc.mn_hi : sc.mn_lo) >> (16 * (ks & 1));
+                const float pos = static_cast<float>(scw & 0xffu) * g2.x * v0 + static_cast<float>((scw >> 8) & 0xffu) * g2.z * v1;
+                const float neg = static_cast<float>(mnw & 0xffu) * g2.y + static_cast<float>((mnw >> 8) & 0xffu) * g2.w;
+                const float d = f16_bits_to_float(regs[it].hdr.x & 0xffffu);
+                const float dmin = f16_bits_to_float(regs[it].hdr.x >> 16);
+                acc += d * pos - dmin * neg;
+            }
+        }
+    }
+    acc += __shfl_xor(acc, 16, 64);
+    acc += __shfl_xor(acc, 32, 64);
+    if (ks == 0) partial[wave * kRowsPerWg + col] = acc;
+    __syncthreads();
+    if (tid < kRowsPerWg) {
+        float total = 0.0f;
+        for (int v = 0; v < waves; ++v) total += partial[v * kRowsPerWg + tid];
+        const int out_row = blockIdx.x * kRowsPerWg + tid;
+        if (out_row < n) store_any(y, y_dtype, static_cast<size_t>(blockIdx.y) * n + out_row, total);
+    }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -111,7 +188,6 @@ __device__ __forceinline__ float lane_dot(const Q5K::Regs& r, int j, int blk, co
 // shift 2s of those bytes is group g = 8 * (j >> 1) + 2s + (j & 1), 16 weights each.
 // ------------------------------------------------------------------------------------------------
 struct Q2K {
-    static constexpr int kLanesPerBlock = 4;
     static constexpr int kBlockBytes = 84;
     struct Regs { uint4 sc; uint4 qs; uint32_t dd; };
     static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, int j) {
@@ -122,10 +198,9 @@ struct Q2K {
         r.qs = make_uint4(q[0], q[1], q[2], q[3]);
         r.dd = p[20];
     }
-    static __device__ __forceinline__ void zero(Regs& r) { r.sc = make_uint4(0, 0, 0, 0); r.qs = r.sc; r.dd = 0; }
 };
 
-__device__ __forceinline__ float lane_dot(const Q2K::Regs& r, int j, int blk, const StagedX& sx) {
+__device__ __forceinline__ float q2k_lane_dot(const Q2K::Regs& r, int j, int blk, const StagedX& sx) {
     const int half = j >> 1, odd = j & 1;
     const float d = f16_bits_to_float(r.dd & 0xffffu);
     const float dmin = f16_bits_to_float(r.dd >> 16);
@@ -147,110 +222,130 @@ __device__ __forceinline__ float lane_dot(const Q2K::Regs& r, int j, int blk, co
         const uint32_t w3 = (r.qs.w >> (2 * s)) & 0x03030303u;
         int sh = dot4(w0, ah.x, 0); sh = dot4(w1, ah.y, sh); sh = dot4(w2, ah.z, sh); sh = dot4(w3, ah.w, sh);
         int sl = dot4(w0, al.x, 0); sl = dot4(w1, al.y, sl); sl = dot4(w2, al.z, sl); sl = dot4(w3, al.w, sl);
-        const float xs = sx.xs[blk * 8 + (g >> 1)];
-        pos += static_cast<float>(sb & 15u) * xs * (static_cast<float>(sh) + static_cast<float>(sl) * kLoInv);
+        const float xs = sx.gs[blk * 8 + (g >> 1)].x;
+        pos += static_cast<float>(sb & 15u) * xs * static_cast<float>(__mul24(sh, 254) + sl);
         neg += static_cast<float>(sb >> 4) * sx.sum16[blk * 16 + g];
     }
     return d * pos - dmin * neg;
 }
 
-// ------------------------------------------------------------------------------------------------
-template <typename FMT, int ITERS>
-__global__ __launch_bounds__(kThreads) void kquant_matvec_kernel(
-    const void* __restrict__ x, int x_dtype, const uint8_t* __restrict__ w, void* __restrict__ y, int y_dtype,
-    int k, int n, int bpr, int tpr_log2) {
+template <int ITERS>
+__global__ __launch_bounds__(64 * kMaxWaves) void q2k_matvec_kernel(
+    const unsigned char* __restrict__ image, size_t image_stride, const uint8_t* __restrict__ w,
+    void* __restrict__ y, int y_dtype, int n, int bpr) {
     extern __shared__ __align__(16) unsigned char smem[];
-    constexpr int LPB = FMT::kLanesPerBlock;
     const int kpad = bpr * 256;
+    const int image_bytes = static_cast<int>(staged_x_bytes(kpad));
     const StagedX sx = carve_staged_x(smem, kpad);
+    float* partial = reinterpret_cast<float*>(smem + image_bytes + 16);
 
     const int tid = threadIdx.x;
-    const int j = tid % LPB;
-    const int team = tid / LPB;
-    const int tpr = 1 << tpr_log2;
-    const int rows_per_wg = (kThreads / LPB) >> tpr_log2;
-    const int row = blockIdx.x * rows_per_wg + (team >> tpr_log2);
-    const int slice = team & (tpr - 1);
-    const bool row_ok = row < n;
-    const uint8_t* wrow = w + static_cast<size_t>(row_ok ? row : 0) * bpr * FMT::kBlockBytes;
-    const size_t xoff = static_cast<size_t>(blockIdx.y) * k;
+    const int waves = blockDim.x >> 6;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    const int j = lane & 3;
+    const int team = lane >> 2;
+    const int row = blockIdx.x * kRowsPerWg + team;
+    const uint8_t* wrow = w + static_cast<size_t>(row < n ? row : 0) * bpr * Q2K::kBlockBytes;
 
     float acc = 0.0f;
     bool staged = false;
-    for (int b0 = slice; b0 < bpr || !staged; b0 += tpr * ITERS) {
-        typename FMT::Regs regs[ITERS];
+    for (int b0 = wave; b0 < bpr || !staged; b0 += waves * ITERS) {
+        Q2K::Regs regs[ITERS];
 #pragma unroll
         for (int it = 0; it < ITERS; ++it) {
-            const int b = b0 + it * tpr;
-            if (row_ok && b < bpr) FMT::load(regs[it], wrow + static_cast<size_t>(b) * FMT::kBlockBytes, j);
-            else FMT::zero(regs[it]);
+            const int b = min(b0 + it * waves, bpr - 1);
+            Q2K::load(regs[it], wrow + static_cast<size_t>(b) * Q2K::kBlockBytes, j);
         }
-        if (!staged) {                       // uniform across the workgroup: first trip of every thread
-            stage_activations_any(x, x_dtype, xoff, k, kpad, sx);
+        if (!staged) {
+            copy_to_lds(smem, image + static_cast<size_t>(blockIdx.y) * image_stride, image_bytes);
             __syncthreads();
             staged = true;
         }
 #pragma unroll
         for (int it = 0; it < ITERS; ++it) {
-            const int b = b0 + it * tpr;
-            if (row_ok && b < bpr) acc += lane_dot(regs[it], j, b, sx);
+            const int b = b0 + it * waves;
+            if (b < bpr) acc += q2k_lane_dot(regs[it], j, b, sx);           // wave-uniform guard
         }
     }
-    // lanes sharing the row are LPB * tpr consecutive lanes
-    const int width = LPB << tpr_log2;
-    for (int off = 1; off < width; off <<= 1) acc += __shfl_xor(acc, off, 64);
-    if (row_ok && (tid & (width - 1)) == 0) store_any(y, y_dtype, static_cast<size_t>(blockIdx.y) * n + row, acc);
+    acc += __shfl_xor(acc, 1, 64);
+    acc += __shfl_xor(acc, 2, 64);
+    if (j == 0) partial[wave * kRowsPerWg + team] = acc;
+    __syncthreads();
+    if (tid < kRowsPerWg) {
+        float total = 0.0f;
+        for (int v = 0; v < waves; ++v) total += partial[v * kRowsPerWg + tid];
+        const int out_row = blockIdx.x * kRowsPerWg + tid;
+        if (out_row < n) store_any(y, y_dtype, static_cast<size_t>(blockIdx.y) * n + out_row, total);
+    }
 }
 
-template <typename FMT, int ITERS>
-int launch_one(const void* x, int x_dtype, const uint8_t* w, void* y, int y_dtype, int rows, int k, int n, int bpr,
-               int tpr_log2, hipStream_t stream) {
-    const int rows_per_wg = (kThreads / FMT::kLanesPerBlock) >> tpr_log2;
-    const size_t smem = staged_x_bytes(bpr * 256);
-    auto kern = kquant_matvec_kernel<FMT, ITERS>;
+// ------------------------------------------------------------------------------------------------
+template <typename KERN>
+int launch_kernel(KERN kern, const unsigned char* image, size_t image_stride, const uint8_t* w, void* y, int y_dtype,
+                  int rows, int n, int bpr, int waves, hipStream_t stream) {
+    const size_t smem = staged_x_bytes(bpr * 256) + 16 + static_cast<size_t>(waves) * kRowsPerWg * sizeof(float);
     if (smem > 64 * 1024) {
         if (smem > 160 * 1024) return PLLM_ERR_UNSUPPORTED;
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                 static_cast<int>(smem)) != hipSuccess)
             return PLLM_ERR_UNSUPPORTED;
     }
-    dim3 grid((n + rows_per_wg - 1) / rows_per_wg, rows);
-    hipLaunchKernelGGL(kern, grid, dim3(kThreads), smem, stream, x, x_dtype, w, y, y_dtype, k, n, bpr, tpr_log2);
+    dim3 grid((n + kRowsPerWg - 1) / kRowsPerWg, rows);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * waves), smem, stream, image, image_stride, w, y, y_dtype, n, bpr);
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 
-template <typename FMT>
-int launch_fmt(const void* x, int x_dtype, const uint8_t* w, void* y, int y_dtype, int rows, int k, int n, int bpr,
-               hipStream_t stream) {
-    // teams per row: enough that a row's blocks are spread over lanes, few enough that every team
-    // still has several blocks in flight
-    int tpr_log2 = 0;
-    while (tpr_log2 < 3 && (bpr >> (tpr_log2 + 1)) >= 3) ++tpr_log2;
-    const int tpr = 1 << tpr_log2;
-    const int niter = (bpr + tpr - 1) / tpr;
+// waves per workgroup and blocks in flight per wave for a row of bpr super-blocks
+void split_blocks(int bpr, int& waves, int& iters) {
+    waves = 1;
+    while (waves < kMaxWaves && bpr / (waves * 2) >= 3) waves *= 2;
+    const int niter = (bpr + waves - 1) / waves;
     const int passes = (niter + 7) / 8;
-    const int iters = (niter + passes - 1) / passes;
-#define PLLM_CASE(I) return launch_one<FMT, I>(x, x_dtype, w, y, y_dtype, rows, k, n, bpr, tpr_log2, stream)
+    iters = (niter + passes - 1) / passes;
+    if (iters == 7) iters = 8;
+}
+
+template <typename FMT>
+int launch_k45(const unsigned char* image, size_t image_stride, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr,
+               hipStream_t stream) {
+    int waves, iters;
+    split_blocks(bpr, waves, iters);
+#define PLLM_CASE(I) case I: return launch_kernel(k45_mfma_matvec_kernel<FMT, I>, image, image_stride, w, y, y_dtype, rows, n, bpr, waves, stream)
     switch (iters) {
-        case 1: PLLM_CASE(1);
-        case 2: PLLM_CASE(2);
-        case 3: PLLM_CASE(3);
-        case 4: PLLM_CASE(4);
-        case 5: PLLM_CASE(5);
-        case 6: PLLM_CASE(6);
-        default: PLLM_CASE(8);
+        PLLM_CASE(1); PLLM_CASE(2); PLLM_CASE(3); PLLM_CASE(4); PLLM_CASE(5); PLLM_CASE(6);
+        default: return launch_kernel(k45_mfma_matvec_kernel<FMT, 8>, image, image_stride, w, y, y_dtype, rows, n, bpr, waves, stream);
+    }
+#undef PLLM_CASE
+}
+
+int launch_q2k(const unsigned char* image, size_t image_stride, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr,
+               hipStream_t stream) {
+    int waves, iters;
+    split_blocks(bpr, waves, iters);
+#define PLLM_CASE(I) case I: return launch_kernel(q2k_matvec_kernel<I>, image, image_stride, w, y, y_dtype, rows, n, bpr, waves, stream)
+    switch (iters) {
+        PLLM_CASE(1); PLLM_CASE(2); PLLM_CASE(3); PLLM_CASE(4); PLLM_CASE(5); PLLM_CASE(6);
+        default: return launch_kernel(q2k_matvec_kernel<8>, image, image_stride, w, y, y_dtype, rows, n, bpr, waves, stream);
     }
 #undef PLLM_CASE
 }
 
 }  // namespace
 
+size_t kquant_matvec_workspace_bytes(int rows, int bpr) { return act_image_256_bytes(bpr) * static_cast<size_t>(rows); }
+
 int kquant_matvec(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y, int y_dtype,
-                  int rows, int k, int n, int bpr, hipStream_t stream) {
+                  int rows, int k, int n, int bpr, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+    if (!workspace || workspace_bytes < kquant_matvec_workspace_bytes(rows, bpr)) return PLLM_ERR_WORKSPACE;
+    const int st = act_image_256(x, x_dtype, rows, k, bpr, workspace, stream);
+    if (st != PLLM_OK) return st;
+    const unsigned char* image = static_cast<const unsigned char*>(workspace);
+    const size_t stride = act_image_256_bytes(bpr);
     switch (type_id) {
-        case PLLM_TYPE_Q4_K: return launch_fmt<Q4K>(x, x_dtype, w, y, y_dtype, rows, k, n, bpr, stream);
-        case PLLM_TYPE_Q5_K: return launch_fmt<Q5K>(x, x_dtype, w, y, y_dtype, rows, k, n, bpr, stream);
-        case PLLM_TYPE_Q2_K: return launch_fmt<Q2K>(x, x_dtype, w, y, y_dtype, rows, k, n, bpr, stream);
+        case PLLM_TYPE_Q4_K: return launch_k45<Q4K>(image, stride, w, y, y_dtype, rows, n, bpr, stream);
+        case PLLM_TYPE_Q5_K: return launch_k45<Q5K>(image, stride, w, y, y_dtype, rows, n, bpr, stream);
+        case PLLM_TYPE_Q2_K: return launch_q2k(image, stride, w, y, y_dtype, rows, n, bpr, stream);
         default: return PLLM_ERR_UNSUPPORTED;
     }
 }

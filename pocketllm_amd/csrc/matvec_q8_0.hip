@@ -1,16 +1,18 @@
 // Decode matvec over raw Q8_0 blocks (34 B = fp16 scale + 32 int8), bandwidth-bound, wave64.
 //
-// 34-byte blocks are only 2-byte aligned, so lanes do not own blocks.  Instead a wave reads a row as
-// an aligned byte stream, lane l taking 16 bytes at offset 16 * (c0 + l) with one
-// global_load_dwordx4.  The activations are laid out in LDS as an IMAGE OF THE SAME STREAM: for
-// every block two zero bytes where the weight stream has its scale, then the 32 int8 activation
-// codes.  A dword of weights and the dword of the image at the same offset then line up byte for
-// byte, and v_dot4_i32_i8 of the two is a partial dot that belongs to exactly one block (the scale
-// bytes meet zeros).  The stream repeats every 17 dwords (two blocks): dwords 0..8 of a pair belong
-// to the even block, 9..16 to the odd one, so four consecutive dwords touch at most two blocks.
-// The fp16 scale of a lane's first block sits at most two lanes back and comes over with one
-// ds_bpermute; only the first two lanes of a pass fetch theirs from memory.
+// 34-byte blocks are only 2-byte aligned, but a PAIR of blocks is 68 bytes = 17 dwords and 4-byte
+// aligned whenever the row holds an even number of blocks.  A lane owns one pair at a time and pulls
+// it in with four 16-byte loads and one 4-byte load (dword alignment is all global_load_dwordx4
+// needs); neighbouring lanes sit 68 bytes apart, so a wave's five loads together sweep one
+// contiguous span of the row and every fetched cache line is used in full.  The activations sit in
+// LDS as an IMAGE OF THE SAME STREAM: per pair two zero bytes where the weight stream has a scale,
+// 32 int8 codes, two zeros, 32 codes (padded to 80 bytes so that ds_read_b128 stays aligned).  A
+// dword of weights and the image dword at the same offset line up byte for byte, v_dot4_i32_i8 of
+// the two is a partial dot of exactly one block (the scale bytes meet zeros): dwords 0..8 belong to
+// the even block, 9..16 to the odd one.  TL lanes share a row; their partial sums meet in a
+// cross-lane reduction.
 #include "pllm_device.h"
+#include "pllm_internal.h"
 
 namespace pllm {
 namespace {
@@ -18,144 +20,93 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / 64;
 
-struct Q8Image {
-    int8_t* hi;   // [bpr * 34]
-    int8_t* lo;   // [bpr * 34]
-    float* xs;    // [bpr]
-};
+struct PairRegs { uint4 a, b, c, d; uint32_t e; };
 
-__device__ __forceinline__ void stage_q8_image(const void* x, int x_dtype, size_t xoff, int k, int bpr, const Q8Image& im) {
-    const int kpad = bpr * 32;
-    for (int e0 = threadIdx.x * 4; e0 < kpad; e0 += kThreads * 4) {
-        float v[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) v[i] = (e0 + i < k) ? load_any(x, x_dtype, xoff + e0 + i) : 0.0f;
-        uint32_t hi, lo;
-        float scale;
-        quantize4(v, hi, lo, scale);
-        const int b = e0 >> 5;
-        const int j = (e0 & 31) >> 2;
-        const int off = 34 * b + 2 + 4 * j;                       // 2-byte aligned
-        *reinterpret_cast<uint16_t*>(im.hi + off) = static_cast<uint16_t>(hi);
-        *reinterpret_cast<uint16_t*>(im.hi + off + 2) = static_cast<uint16_t>(hi >> 16);
-        *reinterpret_cast<uint16_t*>(im.lo + off) = static_cast<uint16_t>(lo);
-        *reinterpret_cast<uint16_t*>(im.lo + off + 2) = static_cast<uint16_t>(lo >> 16);
-        if (j == 0) {
-            *reinterpret_cast<uint16_t*>(im.hi + 34 * b) = 0;
-            *reinterpret_cast<uint16_t*>(im.lo + 34 * b) = 0;
-            im.xs[b] = scale;
-        }
-    }
+__device__ __forceinline__ void load_pair(PairRegs& r, const uint8_t* p) {
+    const uint32_t* q = reinterpret_cast<const uint32_t*>(p);
+    r.a = make_uint4(q[0], q[1], q[2], q[3]);
+    r.b = make_uint4(q[4], q[5], q[6], q[7]);
+    r.c = make_uint4(q[8], q[9], q[10], q[11]);
+    r.d = make_uint4(q[12], q[13], q[14], q[15]);
+    r.e = q[16];
 }
 
-// Contribution of one 16-byte chunk (index c in the row stream) held in w.
-__device__ __forceinline__ float chunk_dot(const uint4& w, int c, int lane, uint32_t head_scale_bits, int bpr, const Q8Image& im) {
-    const int g0 = 4 * c;
-    const int pair = g0 / 17;
-    const int t0 = g0 - 17 * pair;
-    const int block_a = 2 * pair + (t0 >= 9 ? 1 : 0);
-    const int k_a = min(4, (t0 < 9 ? 9 : 17) - t0);           // dwords of this chunk inside block A
-
-    // the scale this lane carries, if any: low half of the dword at t == 0, high half of t == 8
-    const bool in_hi = (t0 >= 5 && t0 <= 8);
-    const int sel = (t0 == 0) ? 0 : (in_hi ? 8 - t0 : 17 - t0);
-    const uint32_t wsel = sel == 0 ? w.x : sel == 1 ? w.y : sel == 2 ? w.z : w.w;
-    const uint32_t own_bits = in_hi ? (wsel >> 16) : (wsel & 0xffffu);
-
-    // scale of block A: own (t0 == 0) or one/two lanes back
-    const int back = (t0 < 9) ? t0 : t0 - 8;                  // dwords back to the scale, 0..8
-    const int dlanes = (back + 3) >> 2;
-    const int src = lane - dlanes;
-    const uint32_t got = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute((src & 63) << 2, static_cast<int>(own_bits)));
-    const uint32_t a_bits = (t0 == 0) ? own_bits : (src >= 0 ? got : head_scale_bits);
-
-    const uint4 ah = *reinterpret_cast<const uint4*>(im.hi + 16 * c);
-    const uint4 al = *reinterpret_cast<const uint4*>(im.lo + 16 * c);
-    const int h0 = dot4(w.x, ah.x, 0), h1 = dot4(w.y, ah.y, 0), h2 = dot4(w.z, ah.z, 0), h3 = dot4(w.w, ah.w, 0);
-    const int l0 = dot4(w.x, al.x, 0), l1 = dot4(w.y, al.y, 0), l2 = dot4(w.z, al.z, 0), l3 = dot4(w.w, al.w, 0);
-    const int ha = h0 + (k_a > 1 ? h1 : 0) + (k_a > 2 ? h2 : 0) + (k_a > 3 ? h3 : 0);
-    const int la = l0 + (k_a > 1 ? l1 : 0) + (k_a > 2 ? l2 : 0) + (k_a > 3 ? l3 : 0);
-    const int hb = (h0 + h1 + h2 + h3) - ha;
-    const int lb = (l0 + l1 + l2 + l3) - la;
-
-    const float xs_a = im.xs[block_a];
-    float out = f16_bits_to_float(a_bits) * xs_a * (static_cast<float>(ha) + static_cast<float>(la) * kLoInv);
-    if (k_a < 4) {
-        const float xs_b = im.xs[min(block_a + 1, bpr - 1)];
-        out += f16_bits_to_float(own_bits) * xs_b * (static_cast<float>(hb) + static_cast<float>(lb) * kLoInv);
-    }
-    return out;
+__device__ __forceinline__ void zero_pair(PairRegs& r) {
+    r.a = make_uint4(0, 0, 0, 0); r.b = r.a; r.c = r.a; r.d = r.a; r.e = 0;
 }
 
-template <int ITERS, int RW>
-__global__ __launch_bounds__(kThreads) void q8_0_stream_kernel(
-    const void* __restrict__ x, int x_dtype, const uint8_t* __restrict__ w, void* __restrict__ y, int y_dtype,
-    int k, int n, int bpr) {
+// image: int8 [pairs][80] (hi) | int8 [pairs][80] (lo) | float xs[2 * pairs]
+__device__ __forceinline__ float pair_dot(const PairRegs& r, int pair, const unsigned char* img_hi, const unsigned char* img_lo,
+                                          const float* xs) {
+    const uint4* ih = reinterpret_cast<const uint4*>(img_hi + pair * 80);
+    const uint4* il = reinterpret_cast<const uint4*>(img_lo + pair * 80);
+    const uint4 h0 = ih[0], h1 = ih[1], h2 = ih[2], h3 = ih[3], h4 = ih[4];
+    const uint4 l0 = il[0], l1 = il[1], l2 = il[2], l3 = il[3], l4 = il[4];
+    // even block: dwords 0..8
+    int ah = dot4(r.a.x, h0.x, 0); ah = dot4(r.a.y, h0.y, ah); ah = dot4(r.a.z, h0.z, ah); ah = dot4(r.a.w, h0.w, ah);
+    ah = dot4(r.b.x, h1.x, ah); ah = dot4(r.b.y, h1.y, ah); ah = dot4(r.b.z, h1.z, ah); ah = dot4(r.b.w, h1.w, ah);
+    ah = dot4(r.c.x, h2.x, ah);
+    int al = dot4(r.a.x, l0.x, 0); al = dot4(r.a.y, l0.y, al); al = dot4(r.a.z, l0.z, al); al = dot4(r.a.w, l0.w, al);
+    al = dot4(r.b.x, l1.x, al); al = dot4(r.b.y, l1.y, al); al = dot4(r.b.z, l1.z, al); al = dot4(r.b.w, l1.w, al);
+    al = dot4(r.c.x, l2.x, al);
+    // odd block: dwords 9..16
+    int bh = dot4(r.c.y, h2.y, 0); bh = dot4(r.c.z, h2.z, bh); bh = dot4(r.c.w, h2.w, bh);
+    bh = dot4(r.d.x, h3.x, bh); bh = dot4(r.d.y, h3.y, bh); bh = dot4(r.d.z, h3.z, bh); bh = dot4(r.d.w, h3.w, bh);
+    bh = dot4(r.e, h4.x, bh);
+    int bl = dot4(r.c.y, l2.y, 0); bl = dot4(r.c.z, l2.z, bl); bl = dot4(r.c.w, l2.w, bl);
+    bl = dot4(r.d.x, l3.x, bl); bl = dot4(r.d.y, l3.y, bl); bl = dot4(r.d.z, l3.z, bl); bl = dot4(r.d.w, l3.w, bl);
+    bl = dot4(r.e, l4.x, bl);
+    const float da = f16_bits_to_float(r.a.x & 0xffffu);
+    const float db = f16_bits_to_float(r.c.x >> 16);
+    const float2 s = *reinterpret_cast<const float2*>(xs + 2 * pair);
+    return da * s.x * (static_cast<float>(ah) + static_cast<float>(al) * kLoInv) +
+           db * s.y * (static_cast<float>(bh) + static_cast<float>(bl) * kLoInv);
+}
+
+// TL = 1 << tl_log2 lanes share a row (4..64); a wave covers 64 / TL rows per pass.
+template <int ITERS>
+__global__ __launch_bounds__(kThreads) void q8_0_pair_kernel(
+    const unsigned char* __restrict__ image, size_t image_stride, const uint8_t* __restrict__ w,
+    void* __restrict__ y, int y_dtype, int n, int pairs, int tl_log2) {
     extern __shared__ __align__(16) unsigned char smem[];
-    const int row_bytes = bpr * 34;                               // multiple of 272
-    Q8Image im;
-    im.hi = reinterpret_cast<int8_t*>(smem);
-    im.lo = im.hi + row_bytes;
-    im.xs = reinterpret_cast<float*>(im.lo + row_bytes);
-    const int chunks = row_bytes >> 4;
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int row0 = (blockIdx.x * kWaves + wave) * RW;
-    const size_t xoff = static_cast<size_t>(blockIdx.y) * k;
+    const unsigned char* img_hi = smem;
+    const unsigned char* img_lo = smem + static_cast<size_t>(pairs) * 80;
+    const float* xs = reinterpret_cast<const float*>(smem + static_cast<size_t>(pairs) * 160);
+    const int tl = 1 << tl_log2;
+    const int tid = threadIdx.x;
+    const int rows_per_wg = kThreads >> tl_log2;
+    const int row = blockIdx.x * rows_per_wg + (tid >> tl_log2);
+    const int slot = tid & (tl - 1);
+    const bool row_ok = row < n;
+    const uint8_t* wrow = w + static_cast<size_t>(row_ok ? row : 0) * pairs * 68;
 
-    float acc[RW];
-#pragma unroll
-    for (int r = 0; r < RW; ++r) acc[r] = 0.0f;
-
+    float acc = 0.0f;
     bool staged = false;
-    for (int c0 = 0; c0 < chunks; c0 += 64 * ITERS) {
-        uint4 regs[RW][ITERS];
-        uint32_t head[RW][ITERS];
+    for (int p0 = slot; p0 < pairs || !staged; p0 += tl * ITERS) {
+        PairRegs regs[ITERS];
 #pragma unroll
-        for (int r = 0; r < RW; ++r) {
-            const int row = row0 + r;
-            const uint8_t* wrow = w + static_cast<size_t>(row < n ? row : 0) * row_bytes;
-#pragma unroll
-            for (int it = 0; it < ITERS; ++it) {
-                const int c = c0 + it * 64 + lane;
-                const int cc = c < chunks ? c : 0;
-                regs[r][it] = *reinterpret_cast<const uint4*>(wrow + 16 * cc);
-                head[r][it] = 0;
-                if (lane < 2) {
-                    const int g0 = 4 * cc;
-                    const int pair = g0 / 17;
-                    const int t0 = g0 - 17 * pair;
-                    const int block_a = 2 * pair + (t0 >= 9 ? 1 : 0);
-                    head[r][it] = *reinterpret_cast<const uint16_t*>(wrow + 34 * block_a);
-                }
-            }
+        for (int it = 0; it < ITERS; ++it) {
+            const int p = p0 + it * tl;
+            if (row_ok && p < pairs) load_pair(regs[it], wrow + static_cast<size_t>(p) * 68);
+            else zero_pair(regs[it]);
         }
         if (!staged) {
-            stage_q8_image(x, x_dtype, xoff, k, bpr, im);
+            copy_to_lds(smem, image + static_cast<size_t>(blockIdx.y) * image_stride, (pairs * 168 + 15) & ~15);
             __syncthreads();
             staged = true;
         }
 #pragma unroll
-        for (int r = 0; r < RW; ++r) {
-#pragma unroll
-            for (int it = 0; it < ITERS; ++it) {
-                const int c = c0 + it * 64 + lane;
-                const bool ok = c < chunks;
-                const float v = chunk_dot(regs[r][it], ok ? c : 0, lane, head[r][it], bpr, im);
-                acc[r] += ok ? v : 0.0f;
-            }
+        for (int it = 0; it < ITERS; ++it) {
+            const int p = p0 + it * tl;
+            if (row_ok && p < pairs) acc += pair_dot(regs[it], p, img_hi, img_lo, xs);
         }
     }
-#pragma unroll
-    for (int r = 0; r < RW; ++r) {
-        const float total = group_sum<64>(acc[r]);
-        const int row = row0 + r;
-        if (lane == 0 && row < n) store_any(y, y_dtype, static_cast<size_t>(blockIdx.y) * n + row, total);
-    }
+    for (int off = 1; off < tl; off <<= 1) acc += __shfl_xor(acc, off, 64);
+    if (row_ok && slot == 0) store_any(y, y_dtype, static_cast<size_t>(blockIdx.y) * n + row, acc);
 }
 
-// Any shape, any alignment: one wave per output row, one lane per block, byte loads.  Used when the
-// rows are not 16-byte aligned streams (blocks_per_row not a multiple of 8, or an offset base).
+// Any shape, any alignment: one wave per output row, one lane per block, byte loads.  Used when a
+// row holds an odd number of blocks or the base pointer is not dword aligned.
 __global__ __launch_bounds__(kThreads) void q8_0_generic_kernel(
     const void* __restrict__ x, int x_dtype, const uint8_t* __restrict__ w, void* __restrict__ y, int y_dtype,
     int k, int n, int bpr) {
@@ -180,56 +131,60 @@ __global__ __launch_bounds__(kThreads) void q8_0_generic_kernel(
     if (lane == 0 && row < n) store_any(y, y_dtype, static_cast<size_t>(blockIdx.y) * n + row, acc);
 }
 
-template <int ITERS, int RW>
-int launch_stream(const void* x, int x_dtype, const uint8_t* w, void* y, int y_dtype, int rows, int k, int n, int bpr,
-                  hipStream_t stream) {
-    const size_t smem = static_cast<size_t>(bpr) * 34 * 2 + static_cast<size_t>(bpr) * 4;
-    auto kern = q8_0_stream_kernel<ITERS, RW>;
+template <int ITERS>
+int launch_pair(const unsigned char* image, size_t image_stride, const uint8_t* w, void* y, int y_dtype, int rows, int n,
+                int pairs, int tl_log2, hipStream_t stream) {
+    const size_t smem = (static_cast<size_t>(pairs) * 168 + 15) & ~static_cast<size_t>(15);
+    auto kern = q8_0_pair_kernel<ITERS>;
     if (smem > 64 * 1024) {
         if (smem > 160 * 1024) return PLLM_ERR_UNSUPPORTED;
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                 static_cast<int>(smem)) != hipSuccess)
             return PLLM_ERR_UNSUPPORTED;
     }
-    const int rows_per_wg = kWaves * RW;
+    const int rows_per_wg = kThreads >> tl_log2;
     dim3 grid((n + rows_per_wg - 1) / rows_per_wg, rows);
-    hipLaunchKernelGGL(kern, grid, dim3(kThreads), smem, stream, x, x_dtype, w, y, y_dtype, k, n, bpr);
+    hipLaunchKernelGGL(kern, grid, dim3(kThreads), smem, stream, image, image_stride, w, y, y_dtype, n, pairs, tl_log2);
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 
-template <int RW>
-int launch_stream_rw(const void* x, int x_dtype, const uint8_t* w, void* y, int y_dtype, int rows, int k, int n, int bpr,
-                     hipStream_t stream) {
-    const int chunks = bpr * 34 / 16;
-    const int niter = (chunks + 63) / 64;
-    const int passes = (niter + 7) / 8;
+}  // namespace
+
+size_t q8_0_matvec_workspace_bytes(int rows, int bpr) {
+    return (bpr % 2 == 0) ? act_image_q8pair_bytes(bpr / 2) * static_cast<size_t>(rows) : 0;
+}
+
+int q8_0_matvec(const void* x, int x_dtype, const uint8_t* w, void* y, int y_dtype,
+                int rows, int k, int n, int bpr, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+    const bool pair_ok = (bpr % 2 == 0) && ((reinterpret_cast<uintptr_t>(w) & 3u) == 0);
+    if (!pair_ok) {
+        dim3 grid((n + kWaves - 1) / kWaves, rows);
+        hipLaunchKernelGGL(q8_0_generic_kernel, grid, dim3(kThreads), 0, stream, x, x_dtype, w, y, y_dtype, k, n, bpr);
+        return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+    }
+    if (!workspace || workspace_bytes < q8_0_matvec_workspace_bytes(rows, bpr)) return PLLM_ERR_WORKSPACE;
+    const int pairs = bpr / 2;
+    const int st = act_image_q8pair(x, x_dtype, rows, k, pairs, workspace, stream);
+    if (st != PLLM_OK) return st;
+    // lanes per row: leave every lane about four pairs
+    int tl_log2 = 2;
+    while (tl_log2 < 6 && (pairs >> (tl_log2 + 1)) >= 4) ++tl_log2;
+    const int tl = 1 << tl_log2;
+    const int niter = (pairs + tl - 1) / tl;
+    const int passes = (niter + 5) / 6;
     const int iters = (niter + passes - 1) / passes;
-#define PLLM_CASE(I) return launch_stream<I, RW>(x, x_dtype, w, y, y_dtype, rows, k, n, bpr, stream)
+    const unsigned char* image = static_cast<const unsigned char*>(workspace);
+    const size_t stride = act_image_q8pair_bytes(pairs);
+#define PLLM_CASE(I) return launch_pair<I>(image, stride, w, y, y_dtype, rows, n, pairs, tl_log2, stream)
     switch (iters) {
         case 1: PLLM_CASE(1);
         case 2: PLLM_CASE(2);
         case 3: PLLM_CASE(3);
         case 4: PLLM_CASE(4);
         case 5: PLLM_CASE(5);
-        case 6: PLLM_CASE(6);
-        default: PLLM_CASE(8);
+        default: PLLM_CASE(6);
     }
 #undef PLLM_CASE
-}
-
-}  // namespace
-
-int q8_0_matvec(const void* x, int x_dtype, const uint8_t* w, void* y, int y_dtype,
-                int rows, int k, int n, int bpr, hipStream_t stream) {
-    const bool stream_ok = (bpr % 8 == 0) && ((reinterpret_cast<uintptr_t>(w) & 15u) == 0);
-    if (!stream_ok) {
-        dim3 grid((n + kWaves - 1) / kWaves, rows);
-        hipLaunchKernelGGL(q8_0_generic_kernel, grid, dim3(kThreads), 0, stream, x, x_dtype, w, y, y_dtype, k, n, bpr);
-        return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
-    }
-    if (n >= 16384) return launch_stream_rw<4>(x, x_dtype, w, y, y_dtype, rows, k, n, bpr, stream);
-    if (n >= 2048) return launch_stream_rw<2>(x, x_dtype, w, y, y_dtype, rows, k, n, bpr, stream);
-    return launch_stream_rw<1>(x, x_dtype, w, y, y_dtype, rows, k, n, bpr, stream);
 }
 
 }  // namespace pllm

@@ -54,31 +54,37 @@ __device__ __forceinline__ float group_max(float v) {
     return v;
 }
 
-// ---- activation staging --------------------------------------------------------------------
-// Activations are split per 32 elements into two int8 terms,
+// ---- activation images ----------------------------------------------------------------------
+// Activations reach the matvec kernels pre-quantized, as an "image" a tiny kernel writes once per
+// call and every workgroup copies into LDS.  Per 32 values two int8 terms are kept,
 //     x[i] ~= xs[g] * (hi[i] + lo[i] / 254),   xs[g] = amax_g / 127,
 // so that integer dot products against the weight codes carry ~15 bits of each activation, enough
 // to stay far below 1e-3 relative error against float activations.  sum16[] holds the exact float
 // sum of every 16 activations for the "minus dmin * m" terms of the K-quants.
+//
+// Layout of one row's image for 256-weight super-block types (kpad = blocks_per_row * 256):
+//     int8 hi[kpad] | int8 lo[kpad] | float2 gs[kpad / 32] | float sum16[kpad / 16]
+// with gs[g] = { xs[g] / 254, exact float sum of the 32 activations of group g }, so that
+// xs * (hi + lo / 254) dotted with integer codes is gs.x * (254 * dot_hi + dot_lo).
 constexpr float kLoInv = 1.0f / 254.0f;
 
 struct StagedX {
-    int8_t* hi;      // [kpad]
-    int8_t* lo;      // [kpad]
-    float* xs;       // [kpad / 32]
-    float* sum16;    // [kpad / 16]
+    const int8_t* hi;
+    const int8_t* lo;
+    const float2* gs;
+    const float* sum16;
 };
 
 __host__ __device__ inline size_t staged_x_bytes(int kpad) {
-    return static_cast<size_t>(kpad) * 2 + static_cast<size_t>(kpad / 32) * 4 + static_cast<size_t>(kpad / 16) * 4;
+    return static_cast<size_t>(kpad) * 2 + static_cast<size_t>(kpad / 32) * 8 + static_cast<size_t>(kpad / 16) * 4;
 }
 
-__device__ __forceinline__ StagedX carve_staged_x(unsigned char* smem, int kpad) {
+__device__ __forceinline__ StagedX carve_staged_x(const unsigned char* base, int kpad) {
     StagedX s;
-    s.hi = reinterpret_cast<int8_t*>(smem);
+    s.hi = reinterpret_cast<const int8_t*>(base);
     s.lo = s.hi + kpad;
-    s.xs = reinterpret_cast<float*>(s.lo + kpad);
-    s.sum16 = s.xs + kpad / 32;
+    s.gs = reinterpret_cast<const float2*>(s.lo + kpad);
+    s.sum16 = reinterpret_cast<const float*>(s.gs + kpad / 32);
     return s;
 }
 
@@ -99,32 +105,14 @@ __device__ __forceinline__ void quantize4(const float v[4], uint32_t& hi, uint32
     }
 }
 
-// All threads of the workgroup call this; k <= kpad, kpad a multiple of 256.  Caller synchronizes.
-template <typename XT>
-__device__ __forceinline__ void stage_activations(const XT* __restrict__ x, int k, int kpad, const StagedX& s) {
-    for (int e0 = threadIdx.x * 4; e0 < kpad; e0 += blockDim.x * 4) {
-        float v[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) v[i] = (e0 + i < k) ? to_float(x[e0 + i]) : 0.0f;
-        uint32_t hi, lo;
-        float scale;
-        quantize4(v, hi, lo, scale);
-        *reinterpret_cast<uint32_t*>(s.hi + e0) = hi;
-        *reinterpret_cast<uint32_t*>(s.lo + e0) = lo;
-        float sum = group_sum<4>((v[0] + v[1]) + (v[2] + v[3]));
-        if ((threadIdx.x & 3) == 0) s.sum16[e0 >> 4] = sum;
-        if ((threadIdx.x & 7) == 0) s.xs[e0 >> 5] = scale;
-    }
+// Workgroup-wide copy of nbytes (a multiple of 16, both pointers 16-byte aligned) into LDS.
+__device__ __forceinline__ void copy_to_lds(unsigned char* dst, const unsigned char* __restrict__ src, int nbytes) {
+    const uint4* s = reinterpret_cast<const uint4*>(src);
+    uint4* d = reinterpret_cast<uint4*>(dst);
+    for (int i = threadIdx.x; i < (nbytes >> 4); i += blockDim.x) d[i] = s[i];
 }
 
 // Runtime-dtype front ends (the dtype is uniform, so the switch costs one scalar branch).
-__device__ __forceinline__ void stage_activations_any(const void* x, int x_dtype, size_t offset, int k, int kpad,
-                                                      const StagedX& s) {
-    if (x_dtype == PLLM_BF16) stage_activations(static_cast<const bf16_t*>(x) + offset, k, kpad, s);
-    else if (x_dtype == PLLM_F16) stage_activations(static_cast<const f16_t*>(x) + offset, k, kpad, s);
-    else stage_activations(static_cast<const float*>(x) + offset, k, kpad, s);
-}
-
 __device__ __forceinline__ float load_any(const void* x, int x_dtype, size_t i) {
     if (x_dtype == PLLM_BF16) return to_float(static_cast<const bf16_t*>(x)[i]);
     if (x_dtype == PLLM_F16) return to_float(static_cast<const f16_t*>(x)[i]);

@@ -2,16 +2,25 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <stddef.h>
 #include <stdint.h>
 
 #include "../../include/pllm_hip.h"
 
 namespace pllm {
 
-int q8_0_matvec(const void* x, int x_dtype, const uint8_t* w, void* y, int y_dtype,
-                int rows, int k, int n, int bpr, hipStream_t stream);
+// activation images (act_quant.hip); *_bytes is the per-row stride, a multiple of 256
+size_t act_image_256_bytes(int bpr);
+int act_image_256(const void* x, int x_dtype, int rows, int k, int bpr, void* image, hipStream_t stream);
+size_t act_image_q8pair_bytes(int pairs);
+int act_image_q8pair(const void* x, int x_dtype, int rows, int k, int pairs, void* image, hipStream_t stream);
 
+size_t q8_0_matvec_workspace_bytes(int rows, int bpr);
+int q8_0_matvec(const void* x, int x_dtype, const uint8_t* w, void* y, int y_dtype,
+                int rows, int k, int n, int bpr, void* workspace, size_t workspace_bytes, hipStream_t stream);
+
+size_t kquant_matvec_workspace_bytes(int rows, int bpr);
 int kquant_matvec(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y, int y_dtype,
-                  int rows, int k, int n, int bpr, hipStream_t stream);
+                  int rows, int k, int n, int bpr, void* workspace, size_t workspace_bytes, hipStream_t stream);
 
 }  // namespace pllm

@@ -30,6 +30,12 @@ def _lib():
     return lib
 
 
+def _workspace(nbytes: int, device: torch.device) -> torch.Tensor:
+    # scratch for the pre-quantized activations: a fresh tensor from torch's caching allocator, so
+    # stream ordering and lifetime follow torch's rules exactly as the reference's temporaries do
+    return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)
+
+
 def _stream(device: torch.device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
 
@@ -77,9 +83,12 @@ def q8_0_gemm_forward(x: torch.Tensor, blocks: torch.Tensor, row_elems: int, *, 
     y = torch.empty(*x.shape[:-1], n, dtype=out_dtype, device=x.device)
     if rows == 0 or n == 0:
         return y
+    lib = _lib()
     with torch.cuda.device(x.device):
-        st = _lib().pllm_q8_0_gemm(x.data_ptr(), _DTYPE_CODE[x.dtype], blocks.data_ptr(), y.data_ptr(), _DTYPE_CODE[out_dtype],
-                                   rows, row_elems, n, blocks.size(1), _stream(x.device))
+        ws_bytes = lib.pllm_q8_0_gemm_workspace_bytes(rows, row_elems, n, blocks.size(1))
+        ws = _workspace(ws_bytes, x.device)
+        st = lib.pllm_q8_0_gemm(x.data_ptr(), _DTYPE_CODE[x.dtype], blocks.data_ptr(), y.data_ptr(), _DTYPE_CODE[out_dtype],
+                                rows, row_elems, n, blocks.size(1), ws.data_ptr(), ws_bytes, _stream(x.device))
     _ffi.check(st, "q8_0_gemm_forward")
     return y
 
@@ -108,9 +117,13 @@ def _dense_gemm(name, x, blocks, row_elems, type_id, signed_grid, out_dtype):
     y = torch.empty(*x.shape[:-1], n, dtype=out_dtype, device=x.device)
     if rows == 0 or n == 0:
         return y
+    lib = _lib()
     with torch.cuda.device(x.device):
-        st = _lib().pllm_gguf_quant_gemm(x.data_ptr(), _DTYPE_CODE[x.dtype], blocks.data_ptr(), type_id, y.data_ptr(),
-                                         _DTYPE_CODE[out_dtype], rows, row_elems, n, blocks.size(1), _stream(x.device))
+        ws_bytes = lib.pllm_gguf_quant_gemm_workspace_bytes(type_id, rows, row_elems, n, blocks.size(1))
+        ws = _workspace(ws_bytes, x.device)
+        st = lib.pllm_gguf_quant_gemm(x.data_ptr(), _DTYPE_CODE[x.dtype], blocks.data_ptr(), type_id, y.data_ptr(),
+                                      _DTYPE_CODE[out_dtype], rows, row_elems, n, blocks.size(1), ws.data_ptr(), ws_bytes,
+                                      _stream(x.device))
     _ffi.check(st, name)
     return y
 
