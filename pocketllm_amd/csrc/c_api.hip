@@ -62,9 +62,13 @@ int pllm_gguf_quant_gemm(const void* x, int x_dtype, const uint8_t* blocks, int 
     if (rows > 65535) return PLLM_ERR_UNSUPPORTED;
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (type_id) {
+        case PLLM_TYPE_Q2_K:
+        case PLLM_TYPE_IQ2_XXS:
+        case PLLM_TYPE_IQ1_M:
+            return pllm::dot4_matvec(x, x_dtype, blocks, type_id, y, y_dtype, static_cast<int>(rows), static_cast<int>(k),
+                                     static_cast<int>(n), static_cast<int>(blocks_per_row), workspace, workspace_bytes, s);
         case PLLM_TYPE_Q4_K:
         case PLLM_TYPE_Q5_K:
-        case PLLM_TYPE_Q2_K:
             return pllm::kquant_matvec(x, x_dtype, blocks, type_id, y, y_dtype, static_cast<int>(rows), static_cast<int>(k),
                                        static_cast<int>(n), static_cast<int>(blocks_per_row), workspace, workspace_bytes, s);
         default:

@@ -1,0 +1,121 @@
+// Decode matvec over raw Q2_K / IQ2_XXS / IQ1_M super-blocks with v_dot4_i32_i8 (wave64).
+//
+// Four adjacent lanes share one super-block (block_dot4.h says which 64 weights each owns); the 16
+// such teams of a wave work on 16 consecutive output rows and on the same super-block index, so LDS
+// reads of activations are broadcasts.  The W waves of a workgroup split a row's super-blocks
+// between them (wave w takes blocks w, w + W, ...) and meet in a small LDS reduction.  All weight
+// loads of a pass are issued first; while they are in flight the workgroup fills LDS with the
+// pre-quantized activation image and the format's codebooks.
+#include "block_dot4.h"
+#include "pllm_internal.h"
+
+namespace pllm {
+namespace {
+
+constexpr int kRowsPerWg = 16;
+constexpr int kMaxWaves = 8;
+
+template <typename FMT, int ITERS>
+__global__ __launch_bounds__(64 * kMaxWaves) void dot4_matvec_kernel(
+    const unsigned char* __restrict__ image, size_t image_stride, const uint8_t* __restrict__ w,
+    void* __restrict__ y, int y_dtype, int n, int bpr) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int kpad = bpr * 256;
+    const int image_bytes = static_cast<int>(staged_x_bytes(kpad));
+    const StagedX sx = carve_staged_x(smem, kpad);
+    unsigned char* tables = smem + image_bytes;
+    float* partial = reinterpret_cast<float*>(tables + FMT::kTableBytes);        // [waves][16]
+
+    const int tid = threadIdx.x;
+    const int waves = blockDim.x >> 6;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    const int j = lane & 3;
+    const int team = lane >> 2;
+    const int row = blockIdx.x * kRowsPerWg + team;
+    const uint8_t* wrow = w + static_cast<size_t>(row < n ? row : 0) * bpr * FMT::kBlockBytes;
+
+    float acc = 0.0f;
+    bool staged = false;
+    for (int b0 = wave; b0 < bpr || !staged; b0 += waves * ITERS) {
+        typename FMT::Regs regs[ITERS];
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+            const int b = min(b0 + it * waves, bpr - 1);                        // clamped: always a valid address
+            FMT::load(regs[it], wrow + static_cast<size_t>(b) * FMT::kBlockBytes, j);
+        }
+        if (!staged) {                       // first trip of every thread of the workgroup
+            copy_to_lds(smem, image + static_cast<size_t>(blockIdx.y) * image_stride, image_bytes);
+            FMT::stage_tables(tables);
+            __syncthreads();
+            staged = true;
+        }
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+            const int b = b0 + it * waves;
+            if (b < bpr) acc += FMT::lane_dot(regs[it], j, b, sx, tables);      // wave-uniform guard
+        }
+    }
+    acc += __shfl_xor(acc, 1, 64);
+    acc += __shfl_xor(acc, 2, 64);
+    if (j == 0) partial[wave * kRowsPerWg + team] = acc;
+    __syncthreads();
+    if (tid < kRowsPerWg) {
+        float total = 0.0f;
+        for (int v = 0; v < waves; ++v) total += partial[v * kRowsPerWg + tid];
+        const int out_row = blockIdx.x * kRowsPerWg + tid;
+        if (out_row < n) store_any(y, y_dtype, static_cast<size_t>(blockIdx.y) * n + out_row, total);
+    }
+}
+
+template <typename FMT, int ITERS>
+int launch_one(const unsigned char* image, size_t image_stride, const uint8_t* w, void* y, int y_dtype,
+               int rows, int n, int bpr, int waves, hipStream_t stream) {
+    const size_t smem = staged_x_bytes(bpr * 256) + FMT::kTableBytes + static_cast<size_t>(waves) * kRowsPerWg * sizeof(float);
+    auto kern = dot4_matvec_kernel<FMT, ITERS>;
+    if (smem > 64 * 1024) {
+        if (smem > 160 * 1024) return PLLM_ERR_UNSUPPORTED;
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                static_cast<int>(smem)) != hipSuccess)
+            return PLLM_ERR_UNSUPPORTED;
+    }
+    dim3 grid((n + kRowsPerWg - 1) / kRowsPerWg, rows);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * waves), smem, stream, image, image_stride, w, y, y_dtype, n, bpr);
+    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+}
+
+template <typename FMT>
+int launch_fmt(const unsigned char* image, size_t image_stride, const uint8_t* w, void* y, int y_dtype,
+               int rows, int n, int bpr, hipStream_t stream) {
+    // waves per workgroup: split a row's blocks so that every wave keeps a handful in flight
+    int waves = 1;
+    while (waves < kMaxWaves && bpr / (waves * 2) >= 3) waves *= 2;
+    const int niter = (bpr + waves - 1) / waves;
+    const int passes = (niter + 5) / 6;
+    const int iters = (niter + passes - 1) / passes;
+#define PLLM_CASE(I) case I: return launch_one<FMT, I>(image, image_stride, w, y, y_dtype, rows, n, bpr, waves, stream)
+    switch (iters) {
+        PLLM_CASE(1); PLLM_CASE(2); PLLM_CASE(3); PLLM_CASE(4); PLLM_CASE(5);
+        default: return launch_one<FMT, 6>(image, image_stride, w, y, y_dtype, rows, n, bpr, waves, stream);
+    }
+#undef PLLM_CASE
+}
+
+}  // namespace
+
+int dot4_matvec(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y, int y_dtype,
+                int rows, int k, int n, int bpr, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+    if (!workspace || workspace_bytes < kquant_matvec_workspace_bytes(rows, bpr)) return PLLM_ERR_WORKSPACE;
+    const int st = act_image_256(x, x_dtype, rows, k, bpr, workspace, stream);
+    if (st != PLLM_OK) return st;
+    const unsigned char* image = static_cast<const unsigned char*>(workspace);
+    const size_t stride = act_image_256_bytes(bpr);
+    switch (type_id) {
+        case PLLM_TYPE_Q2_K: return launch_fmt<Q2K>(image, stride, w, y, y_dtype, rows, n, bpr, stream);
+        case PLLM_TYPE_IQ2_XXS: return launch_fmt<IQ2XXS>(image, stride, w, y, y_dtype, rows, n, bpr, stream);
+        case PLLM_TYPE_IQ1_M: return launch_fmt<IQ1M>(image, stride, w, y, y_dtype, rows, n, bpr, stream);
+        default: return PLLM_ERR_UNSUPPORTED;
+    }
+}
+
+}  // namespace pllm

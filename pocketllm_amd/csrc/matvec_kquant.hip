@@ -1,4 +1,4 @@
-// Decode matvec over raw Q4_K / Q5_K / Q2_K super-blocks (bandwidth-bound, wave64).
+// Decode matvec over raw Q4_K / Q5_K super-blocks (bandwidth-bound, wave64).
 //
 // A wave owns 16 consecutive output rows and walks their super-blocks; the W waves of a workgroup
 // split a row's super-blocks between them (wave w takes blocks w, w + W, ...) and meet in a small
@@ -6,7 +6,7 @@
 // workgroup copies the pre-quantized activation image (two int8 terms per value, written once per
 // call by act_quant.hip) from L2 into LDS.
 //
-// Q4_K / Q5_K: the integer dots run on the matrix cores.  For one super-block index the wave forms
+// The integer dots run on the matrix cores.  For one super-block index the wave forms
 //     C[m][n] = sum_k A[m][k] * B[k][n],     v_mfma_i32_16x16x64_i8, four of them per block,
 // with B = the 4/5-bit codes of the 16 rows (n = row, straight from the 16-byte global loads after
 // a nibble split) and A = the activation codes spread over 16 rows m = 2 * group + term, row m
@@ -15,9 +15,6 @@
 // both terms; the lane that holds C[4s .. 4s+3][n] owns groups 2s and 2s+1 of row n and applies
 // their 6-bit scales and mins in float.  Which k sits where inside an MFMA is irrelevant as long
 // as A and B agree, and both are built per (lane / 16, byte) from the same positions.
-//
-// Q2_K keeps v_dot4_i32_i8 dots: four lanes share a block, 16 such teams (rows) per wave all on the
-// same block index, so that LDS reads of activations are broadcasts.
 #include "pllm_device.h"
 #include "pllm_internal.h"
 
@@ -184,103 +181,6 @@ __global__ __launch_bounds__(64 * kMaxWaves) void k45_mfma_matvec_kernel(
 }
 
 // ------------------------------------------------------------------------------------------------
-// Q2_K: 84 B = scales(16) qs(64) d(2) dmin(2).  4 lanes per block; lane j holds qs[16j, 16j+16):
-// shift 2s of those bytes is group g = 8 * (j >> 1) + 2s + (j & 1), 16 weights each.
-// ------------------------------------------------------------------------------------------------
-struct Q2K {
-    static constexpr int kBlockBytes = 84;
-    struct Regs { uint4 sc; uint4 qs; uint32_t dd; };
-    static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, int j) {
-        // blocks are only 4-byte aligned: the loads below are dword-aligned vector loads
-        const uint32_t* p = reinterpret_cast<const uint32_t*>(blk);
-        r.sc = make_uint4(p[0], p[1], p[2], p[3]);
-        const uint32_t* q = p + 4 + 4 * j;
-        r.qs = make_uint4(q[0], q[1], q[2], q[3]);
-        r.dd = p[20];
-    }
-};
-
-__device__ __forceinline__ float q2k_lane_dot(const Q2K::Regs& r, int j, int blk, const StagedX& sx) {
-    const int half = j >> 1, odd = j & 1;
-    const float d = f16_bits_to_float(r.dd & 0xffffu);
-    const float dmin = f16_bits_to_float(r.dd >> 16);
-    // scale bytes of groups 8*half + 2s + odd, s = 0..3, live in dwords 2*half and 2*half+1
-    const uint32_t slo = half ? r.sc.z : r.sc.x;
-    const uint32_t shi = half ? r.sc.w : r.sc.y;
-    float pos = 0.0f, neg = 0.0f;
-#pragma unroll
-    for (int s = 0; s < 4; ++s) {
-        const uint32_t word = s < 2 ? slo : shi;
-        const uint32_t sb = (word >> (16 * (s & 1) + 8 * odd)) & 0xffu;
-        const int g = 8 * half + 2 * s + odd;
-        const int base = blk * 256 + 16 * g;
-        const uint4 ah = *reinterpret_cast<const uint4*>(sx.hi + base);
-        const uint4 al = *reinterpret_cast<const uint4*>(sx.lo + base);
-        const uint32_t w0 = (r.qs.x >> (2 * s)) & 0x03030303u;
-        const uint32_t w1 = (r.qs.y >> (2 * s)) & 0x03030303u;
-        const uint32_t w2 = (r.qs.z >> (2 * s)) & 0x03030303u;
-        const uint32_t w3 = (r.qs.w >> (2 * s)) & 0x03030303u;
-        int sh = dot4(w0, ah.x, 0); sh = dot4(w1, ah.y, sh); sh = dot4(w2, ah.z, sh); sh = dot4(w3, ah.w, sh);
-        int sl = dot4(w0, al.x, 0); sl = dot4(w1, al.y, sl); sl = dot4(w2, al.z, sl); sl = dot4(w3, al.w, sl);
-        const float xs = sx.gs[blk * 8 + (g >> 1)].x;
-        pos += static_cast<float>(sb & 15u) * xs * static_cast<float>(__mul24(sh, 254) + sl);
-        neg += static_cast<float>(sb >> 4) * sx.sum16[blk * 16 + g];
-    }
-    return d * pos - dmin * neg;
-}
-
-template <int ITERS>
-__global__ __launch_bounds__(64 * kMaxWaves) void q2k_matvec_kernel(
-    const unsigned char* __restrict__ image, size_t image_stride, const uint8_t* __restrict__ w,
-    void* __restrict__ y, int y_dtype, int n, int bpr) {
-    extern __shared__ __align__(16) unsigned char smem[];
-    const int kpad = bpr * 256;
-    const int image_bytes = static_cast<int>(staged_x_bytes(kpad));
-    const StagedX sx = carve_staged_x(smem, kpad);
-    float* partial = reinterpret_cast<float*>(smem + image_bytes + 16);
-
-    const int tid = threadIdx.x;
-    const int waves = blockDim.x >> 6;
-    const int wave = tid >> 6;
-    const int lane = tid & 63;
-    const int j = lane & 3;
-    const int team = lane >> 2;
-    const int row = blockIdx.x * kRowsPerWg + team;
-    const uint8_t* wrow = w + static_cast<size_t>(row < n ? row : 0) * bpr * Q2K::kBlockBytes;
-
-    float acc = 0.0f;
-    bool staged = false;
-    for (int b0 = wave; b0 < bpr || !staged; b0 += waves * ITERS) {
-        Q2K::Regs regs[ITERS];
-#pragma unroll
-        for (int it = 0; it < ITERS; ++it) {
-            const int b = min(b0 + it * waves, bpr - 1);
-            Q2K::load(regs[it], wrow + static_cast<size_t>(b) * Q2K::kBlockBytes, j);
-        }
-        if (!staged) {
-            copy_to_lds(smem, image + static_cast<size_t>(blockIdx.y) * image_stride, image_bytes);
-            __syncthreads();
-            staged = true;
-        }
-#pragma unroll
-        for (int it = 0; it < ITERS; ++it) {
-            const int b = b0 + it * waves;
-            if (b < bpr) acc += q2k_lane_dot(regs[it], j, b, sx);           // wave-uniform guard
-        }
-    }
-    acc += __shfl_xor(acc, 1, 64);
-    acc += __shfl_xor(acc, 2, 64);
-    if (j == 0) partial[wave * kRowsPerWg + team] = acc;
-    __syncthreads();
-    if (tid < kRowsPerWg) {
-        float total = 0.0f;
-        for (int v = 0; v < waves; ++v) total += partial[v * kRowsPerWg + tid];
-        const int out_row = blockIdx.x * kRowsPerWg + tid;
-        if (out_row < n) store_any(y, y_dtype, static_cast<size_t>(blockIdx.y) * n + out_row, total);
-    }
-}
-
-// ------------------------------------------------------------------------------------------------
 template <typename KERN>
 int launch_kernel(KERN kern, const unsigned char* image, size_t image_stride, const uint8_t* w, void* y, int y_dtype,
                   int rows, int n, int bpr, int waves, hipStream_t stream) {
@@ -319,18 +219,6 @@ int launch_k45(const unsigned char* image, size_t image_stride, const uint8_t* w
 #undef PLLM_CASE
 }
 
-int launch_q2k(const unsigned char* image, size_t image_stride, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr,
-               hipStream_t stream) {
-    int waves, iters;
-    split_blocks(bpr, waves, iters);
-#define PLLM_CASE(I) case I: return launch_kernel(q2k_matvec_kernel<I>, image, image_stride, w, y, y_dtype, rows, n, bpr, waves, stream)
-    switch (iters) {
-        PLLM_CASE(1); PLLM_CASE(2); PLLM_CASE(3); PLLM_CASE(4); PLLM_CASE(5); PLLM_CASE(6);
-        default: return launch_kernel(q2k_matvec_kernel<8>, image, image_stride, w, y, y_dtype, rows, n, bpr, waves, stream);
-    }
-#undef PLLM_CASE
-}
-
 }  // namespace
 
 size_t kquant_matvec_workspace_bytes(int rows, int bpr) { return act_image_256_bytes(bpr) * static_cast<size_t>(rows); }
@@ -345,7 +233,6 @@ int kquant_matvec(const void* x, int x_dtype, const uint8_t* w, int type_id, voi
     switch (type_id) {
         case PLLM_TYPE_Q4_K: return launch_k45<Q4K>(image, stride, w, y, y_dtype, rows, n, bpr, stream);
         case PLLM_TYPE_Q5_K: return launch_k45<Q5K>(image, stride, w, y, y_dtype, rows, n, bpr, stream);
-        case PLLM_TYPE_Q2_K: return launch_q2k(image, stride, w, y, y_dtype, rows, n, bpr, stream);
         default: return PLLM_ERR_UNSUPPORTED;
     }
 }

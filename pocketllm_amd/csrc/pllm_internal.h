@@ -23,4 +23,8 @@ size_t kquant_matvec_workspace_bytes(int rows, int bpr);
 int kquant_matvec(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y, int y_dtype,
                   int rows, int k, int n, int bpr, void* workspace, size_t workspace_bytes, hipStream_t stream);
 
+// Q2_K / IQ2_XXS / IQ1_M (matvec_dot4.hip); same workspace as kquant_matvec
+int dot4_matvec(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y, int y_dtype,
+                int rows, int k, int n, int bpr, void* workspace, size_t workspace_bytes, hipStream_t stream);
+
 }  // namespace pllm

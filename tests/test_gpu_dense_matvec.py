@@ -146,3 +146,60 @@ def test_argument_errors_match_reference_messages(mod):
         mod.gguf_quant_gemm_forward(x.double(), blocks, 512, 3, grid)
     with pytest.raises(RuntimeError, match="q8_0 block size must be 34 bytes"):
         mod.q8_0_gemm_forward(x, blocks, 512)
+
+
+# ---------------------------------------------------------------------------------------------
+# codebook types: IQ2_XXS and IQ1_M (random valid blocks, as the reference's own tests build them)
+# ---------------------------------------------------------------------------------------------
+
+def _grid_for(type_name, dev):
+    from pocketllm_amd import codebooks
+    if type_name == "iq2_xxs":
+        return codebooks.get_iq2xxs_signed_grid_tensor().to(dev)
+    return codebooks.get_iq1_grid_tensor().to(dev)
+
+
+@pytest.mark.parametrize("type_name", ["iq2_xxs", "iq1_m"])
+@pytest.mark.parametrize("n,k,rows", [(16, 256, 1), (50, 768, 1), (1536, 3072, 1), (3072, 1536, 1), (40, 2048, 3), (7, 5120, 1), (21, 1000, 2)])
+def test_iq_matvec_matches_oracle(mod, type_name, n, k, rows):
+    rng = np.random.default_rng(500 + n + k)
+    gen = C.random_iq2_xxs if type_name == "iq2_xxs" else C.random_iq1_m
+    blocks = gen(rng, n, (k + 255) // 256)
+    x_np = rng.standard_normal((rows, k)).astype(np.float32)
+    dev = torch.device("cuda:0")
+    grid = _grid_for(type_name, dev)
+    b = torch.from_numpy(blocks).to(dev)
+    for dt in (torch.bfloat16, torch.float32):
+        print(f"case {type_name} n={n} k={k} rows={rows} {dt}", flush=True)
+        x = torch.from_numpy(x_np).to(dev).to(dt)
+        y = mod.gguf_quant_gemm_forward(x, b, k, O.TYPE_IDS[type_name], grid, out_dtype=torch.float32)
+        torch.cuda.synchronize()
+        want = O.matmul_f(x.float().cpu().numpy(), O.dequant_rows(blocks, type_name, k))
+        err = O.rel_l2(y.cpu().numpy(), want)
+        assert err <= 2e-4, (type_name, n, k, rows, dt, err)
+
+
+def test_iq_fully_random_bytes(mod):
+    """Every byte random (all scale codes, all sign patterns, both deltas); only the fp16 scale is kept finite."""
+    rng = np.random.default_rng(91)
+    dev = torch.device("cuda:0")
+    for type_name, bb in (("iq2_xxs", 66), ("iq1_m", 56)):
+        n, bpr = 64, 6
+        gen = C.random_iq2_xxs if type_name == "iq2_xxs" else C.random_iq1_m
+        blocks = gen(rng, n, bpr, d_range=(0.001, 0.08))
+        x_np = rng.standard_normal((1, bpr * 256)).astype(np.float32)
+        y = mod.gguf_quant_gemm_forward(torch.from_numpy(x_np).to(dev), torch.from_numpy(blocks).to(dev), bpr * 256,
+                                        O.TYPE_IDS[type_name], _grid_for(type_name, dev), out_dtype=torch.float32)
+        torch.cuda.synchronize()
+        want = O.matmul_f(x_np, O.dequant_rows(blocks, type_name))
+        assert O.rel_l2(y.cpu().numpy(), want) <= 2e-4, type_name
+
+
+def test_codebook_grid_argument_is_validated(mod):
+    dev = torch.device("cuda:0")
+    x = torch.randn(1, 256, device=dev)
+    blocks = torch.zeros(4, 1, 66, dtype=torch.uint8, device=dev)
+    with pytest.raises(RuntimeError, match="256\\*128\\*8 entries for iq2_xxs"):
+        mod.gguf_quant_gemm_forward(x, blocks, 256, 0, torch.empty(0, dtype=torch.int8, device=dev))
+    with pytest.raises(RuntimeError, match="2048\\*8 entries for iq1_m"):
+        mod.gguf_quant_gemm_forward(x, torch.zeros(4, 1, 56, dtype=torch.uint8, device=dev), 256, 2, torch.empty(0, dtype=torch.int8, device=dev))
