@@ -40,7 +40,8 @@ enum {
     PLLM_TYPE_Q2_K = 1,    /* 84 B */
     PLLM_TYPE_IQ1_M = 2,   /* 56 B */
     PLLM_TYPE_Q4_K = 3,    /* 144 B */
-    PLLM_TYPE_Q5_K = 4     /* 176 B */
+    PLLM_TYPE_Q5_K = 4,    /* 176 B */
+    PLLM_TYPE_Q8_0 = 100   /* 34 B / 32 weights; the reference gives Q8_0 no id, this one is the library's own */
 };
 
 const char* pllm_status_string(int status);
@@ -81,6 +82,40 @@ int pllm_gguf_quant_gemm(const void* x, int x_dtype, const uint8_t* blocks, int 
                          int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row,
                          void* workspace, size_t workspace_bytes, void* stream);
 size_t pllm_gguf_quant_gemm_workspace_bytes(int type_id, int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row);
+
+/*
+ * Selected-row dequantization: out[i, :] = dequant(blocks[row_ids[i], :, :])[:k]  (row_ids == NULL
+ * selects rows 0 .. n_selected-1 in order).  type_id may also be PLLM_TYPE_Q8_0 (blocks_per_row then
+ * counts 32-weight blocks).  Results are bit-identical to the reference's numpy decoders.
+ *   row_ids int64 [n_selected] (ids outside [0, n_rows) produce zero rows), out [n_selected, k]
+ * Replaces gguf_quant_embedding_forward (src/csrc/cuda_kernel.cpp:669-687, kernel
+ * src/csrc/cuda_kernel_impl.cu:8387-8423, which serves q4_k/q5_k only) and stands in for the
+ * decoders of src/loader/gguf/tensor_reader.py:543-1009 and q8_0_weight_dequantize
+ * (src/kernels/ops.py:734-741).
+ */
+int pllm_gguf_dequantize_rows(const int64_t* row_ids, int64_t n_selected, const uint8_t* blocks, int type_id,
+                              int64_t n_rows, int64_t k, int64_t blocks_per_row, void* out, int out_dtype, void* stream);
+
+/*
+ * FP8 E4M3FN (OCP) weights with one float32 scale per 128 x 128 block.
+ *   weight [n, k] uint8 codes, scale [ceil(n/128), ceil(k/128)] float32
+ * pllm_fp8_block_dequantize: out[r, c] = f32(code[r, c]) * scale[r / 128, c / 128]
+ *   replaces _dequant_fp8_weight_torch (src/kernels/ops.py:144-147).
+ * pllm_fp8_block_gemm: y[t, r] = sum_c x[t, c] * out[r, c] without materialising `out`
+ *   replaces soft_fp8_blockfp8_gemm (src/kernels/ops.py:641-648, 910-954) on float activations.
+ */
+int pllm_fp8_block_dequantize(const uint8_t* weight, const float* scale, int64_t n, int64_t k, void* out, int out_dtype, void* stream);
+int pllm_fp8_block_gemm(const void* x, int x_dtype, const uint8_t* weight, const float* scale, void* y, int y_dtype,
+                        int64_t rows, int64_t k, int64_t n, void* stream);
+
+/*
+ * FP8 activation quantizer: per (row, 128 values) scale = max(amax, eps) / 448 (rounded up to a power
+ * of two when round_scale_pow2 != 0), code = E4M3FN round-to-nearest-even of clamp(x / scale, +-448).
+ *   x [rows, k] (k a multiple of 128) -> codes uint8 [rows, k], scales float32 [rows, k / 128]
+ * Replaces blockfp8_act_quant / act_quant (src/kernels/ops.py:501-516, 982-1001).
+ */
+int pllm_fp8_act_quant(const void* x, int x_dtype, int64_t rows, int64_t k, uint8_t* codes, float* scales,
+                       float eps, int round_scale_pow2, void* stream);
 
 /*
  * Measurement aids with no counterpart in the reference: a streaming copy and a streaming read of

@@ -8,6 +8,7 @@ LIB_PATH = Path(__file__).resolve().parent / "libpllm_hip.so"
 
 PLLM_OK = 0
 DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
+TYPE_Q8_0 = 100
 
 _c_void_p = ctypes.c_void_p
 _i64 = ctypes.c_int64
@@ -23,6 +24,10 @@ SIGNATURES = {
     "pllm_q8_0_gemm_workspace_bytes": (_size_t, [_i64, _i64, _i64, _i64]),
     "pllm_gguf_quant_gemm": (_int, [_c_void_p, _int, _c_void_p, _int, _c_void_p, _int, _i64, _i64, _i64, _i64, _c_void_p, _size_t, _c_void_p]),
     "pllm_gguf_quant_gemm_workspace_bytes": (_size_t, [_int, _i64, _i64, _i64, _i64]),
+    "pllm_gguf_dequantize_rows": (_int, [_c_void_p, _i64, _c_void_p, _int, _i64, _i64, _i64, _c_void_p, _int, _c_void_p]),
+    "pllm_fp8_block_dequantize": (_int, [_c_void_p, _c_void_p, _i64, _i64, _c_void_p, _int, _c_void_p]),
+    "pllm_fp8_block_gemm": (_int, [_c_void_p, _int, _c_void_p, _c_void_p, _c_void_p, _int, _i64, _i64, _i64, _c_void_p]),
+    "pllm_fp8_act_quant": (_int, [_c_void_p, _int, _i64, _i64, _c_void_p, _c_void_p, ctypes.c_float, _int, _c_void_p]),
     "pllm_diag_stream_copy": (_int, [_c_void_p, _c_void_p, _size_t, _int, _c_void_p]),
     "pllm_diag_stream_read": (_int, [_c_void_p, _c_void_p, _size_t, _int, _c_void_p]),
 }

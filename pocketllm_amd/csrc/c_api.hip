@@ -82,4 +82,13 @@ size_t pllm_gguf_quant_gemm_workspace_bytes(int type_id, int64_t rows, int64_t k
     return pllm::kquant_matvec_workspace_bytes(static_cast<int>(rows), static_cast<int>(blocks_per_row));
 }
 
+int pllm_fp8_block_gemm(const void* x, int x_dtype, const uint8_t* weight, const float* scale, void* y, int y_dtype,
+                        int64_t rows, int64_t k, int64_t n, void* stream) {
+    if (!x || !weight || !scale || !y || !dtype_ok(x_dtype) || !dtype_ok(y_dtype)) return PLLM_ERR_INVALID_ARGUMENT;
+    if (!fits_int(rows) || !fits_int(k) || !fits_int(n)) return PLLM_ERR_INVALID_ARGUMENT;
+    if (rows > 65535) return PLLM_ERR_UNSUPPORTED;
+    return pllm::fp8_matvec(x, x_dtype, weight, scale, y, y_dtype, static_cast<int>(rows), static_cast<int>(k),
+                            static_cast<int>(n), static_cast<hipStream_t>(stream));
+}
+
 }  // extern "C"

@@ -1,0 +1,152 @@
+// Block dequantization to float: selected rows of a raw-block matrix (the embedding operator) and
+// whole FP8 matrices.  One thread per weight, byte loads, the reference decoders' operand order.
+// Every product below is exact in float32, so only the K-quants' final subtraction rounds and the
+// results are bit-identical to the numpy decoders whatever the compiler contracts.
+#include "block_dot4.h"
+#include "pllm_internal.h"
+
+namespace pllm {
+namespace {
+
+__device__ __forceinline__ float f16_at(const uint8_t* p) {
+    return f16_bits_to_float(static_cast<uint32_t>(p[0]) | (static_cast<uint32_t>(p[1]) << 8));
+}
+
+__device__ __forceinline__ void scale_min_k4(const uint8_t* s, int j, int& sc, int& mn) {
+    if (j < 4) {
+        sc = s[j] & 63;
+        mn = s[j + 4] & 63;
+    } else {
+        sc = (s[j + 4] & 0x0f) | ((s[j - 4] >> 6) << 4);
+        mn = (s[j + 4] >> 4) | ((s[j] >> 6) << 4);
+    }
+}
+
+__device__ float dequant_q4_k(const uint8_t* b, int e) {
+    const int pair = e >> 6, in_pair = e & 63, hi = in_pair >> 5;
+    int sc, mn;
+    scale_min_k4(b + 4, 2 * pair + hi, sc, mn);
+    const int byte = b[16 + 32 * pair + (in_pair & 31)];
+    const int q = hi ? (byte >> 4) : (byte & 15);
+    return f16_at(b) * static_cast<float>(sc) * static_cast<float>(q) - f16_at(b + 2) * static_cast<float>(mn);
+}
+
+__device__ float dequant_q5_k(const uint8_t* b, int e) {
+    const int pair = e >> 6, in_pair = e & 63, hi = in_pair >> 5, pos = in_pair & 31;
+    int sc, mn;
+    scale_min_k4(b + 4, 2 * pair + hi, sc, mn);
+    const int byte = b[48 + 32 * pair + pos];
+    const int q = (hi ? (byte >> 4) : (byte & 15)) + (((b[16 + pos] >> (2 * pair + hi)) & 1) ? 16 : 0);
+    return f16_at(b) * static_cast<float>(sc) * static_cast<float>(q) - f16_at(b + 2) * static_cast<float>(mn);
+}
+
+__device__ float dequant_q2_k(const uint8_t* b, int e) {
+    const int group = e >> 4, half = group >> 3, gi = group & 7;
+    const int q = (b[16 + 32 * half + 16 * (gi & 1) + (e & 15)] >> (2 * (gi >> 1))) & 3;
+    const int s = b[group];
+    return f16_at(b + 80) * static_cast<float>(s & 15) * static_cast<float>(q) - f16_at(b + 82) * static_cast<float>(s >> 4);
+}
+
+__device__ float dequant_iq2_xxs(const uint8_t* b, int e) {
+    const int sub = e >> 5, part = (e >> 3) & 3, j = e & 7;
+    const uint8_t* c = b + 2 + 8 * sub;
+    const uint32_t aux = static_cast<uint32_t>(c[4]) | (static_cast<uint32_t>(c[5]) << 8) | (static_cast<uint32_t>(c[6]) << 16) |
+                         (static_cast<uint32_t>(c[7]) << 24);
+    const uint32_t sidx = (aux >> (7 * part)) & 127u;
+    const uint32_t sign8 = sidx | ((__popc(sidx) & 1u) << 7);
+    const float mag = static_cast<float>((PLLM_IQ2XXS_GRID[c[part]] >> (8 * j)) & 0xffull);
+    const float val = ((sign8 >> j) & 1u) ? -mag : mag;
+    return 0.125f * f16_at(b) * static_cast<float>(2 * (aux >> 28) + 1) * val;
+}
+
+__device__ float dequant_iq1_m(const uint8_t* b, int e) {
+    const int ent = e >> 3, t = e & 7, s = ent >> 1;
+    uint32_t sc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) sc[i] = static_cast<uint32_t>(b[48 + 2 * i]) | (static_cast<uint32_t>(b[49 + 2 * i]) << 8);
+    const uint32_t dbits = (sc[0] >> 12) | ((sc[1] >> 12) << 4) | ((sc[2] >> 12) << 8) | (sc[3] & 0xf000u);
+    const uint32_t ls = (sc[s >> 2] >> (3 * (s & 3))) & 7u;
+    const float dl = f16_bits_to_float(dbits) * static_cast<float>(2 * ls + 1);
+    const uint32_t h = (b[32 + (ent >> 1)] >> (4 * (ent & 1))) & 15u;
+    const uint32_t idx = b[ent] | ((h & 7u) << 8);
+    const float g = static_cast<float>(static_cast<int>((PLLM_IQ1_GRID_PACKED[idx] >> (2 * t)) & 3u) - 1);
+    return dl * (g + ((h & 8u) ? -0.125f : 0.125f));
+}
+
+// grid (selected rows, ceil(k / 256)), 256 threads
+__global__ __launch_bounds__(256) void dequant_rows_kernel(
+    const int64_t* __restrict__ row_ids, const uint8_t* __restrict__ blocks, int type_id, void* __restrict__ out, int out_dtype,
+    int k, int bpr, int block_bytes, int64_t n_rows) {
+    const int64_t row = row_ids ? row_ids[blockIdx.x] : static_cast<int64_t>(blockIdx.x);
+    const int e = threadIdx.x;
+    const int col = blockIdx.y * 256 + e;
+    if (col >= k) return;
+    float v = 0.0f;
+    if (row >= 0 && row < n_rows) {
+        if (type_id < 0) {                                                  // Q8_0: bpr counts 32-weight blocks
+            const uint8_t* b = blocks + (static_cast<size_t>(row) * bpr + (col >> 5)) * 34;
+            v = f16_at(b) * static_cast<float>(static_cast<int8_t>(b[2 + (col & 31)]));
+        } else {
+            const uint8_t* b = blocks + (static_cast<size_t>(row) * bpr + blockIdx.y) * block_bytes;
+            switch (type_id) {
+                case PLLM_TYPE_Q4_K: v = dequant_q4_k(b, e); break;
+                case PLLM_TYPE_Q5_K: v = dequant_q5_k(b, e); break;
+                case PLLM_TYPE_Q2_K: v = dequant_q2_k(b, e); break;
+                case PLLM_TYPE_IQ2_XXS: v = dequant_iq2_xxs(b, e); break;
+                default: v = dequant_iq1_m(b, e); break;
+            }
+        }
+    }
+    store_any(out, out_dtype, static_cast<size_t>(blockIdx.x) * k + col, v);
+}
+
+__device__ __forceinline__ float fp8_e4m3_to_float(uint32_t c) {
+    const uint32_t e = (c >> 3) & 15u, m = c & 7u;
+    float v;
+    if (e == 0) v = static_cast<float>(m) * 0.001953125f;                           // m / 8 * 2^-6
+    else if (e == 15 && m == 7) v = __uint_as_float(0x7fc00000u);
+    else v = __uint_as_float(((e + 120u) << 23) | (m << 20));                       // (1 + m / 8) * 2^(e - 7)
+    return (c & 0x80u) ? -v : v;
+}
+
+__global__ __launch_bounds__(256) void dequant_fp8_kernel(
+    const uint8_t* __restrict__ w, const float* __restrict__ scale, void* __restrict__ out, int out_dtype, int n, int k, int kb) {
+    const int col = blockIdx.y * 256 + threadIdx.x;
+    const int row = blockIdx.x;
+    if (col >= k) return;
+    const float v = fp8_e4m3_to_float(w[static_cast<size_t>(row) * k + col]) * scale[(row >> 7) * kb + (col >> 7)];
+    store_any(out, out_dtype, static_cast<size_t>(row) * k + col, v);
+}
+
+}  // namespace
+}  // namespace pllm
+
+extern "C" {
+
+int pllm_gguf_dequantize_rows(const int64_t* row_ids, int64_t n_selected, const uint8_t* blocks, int type_id,
+                              int64_t n_rows, int64_t k, int64_t blocks_per_row, void* out, int out_dtype, void* stream) {
+    if (!blocks || !out || n_selected < 0 || n_rows <= 0 || k <= 0 || blocks_per_row <= 0) return PLLM_ERR_INVALID_ARGUMENT;
+    if (out_dtype != PLLM_F32 && out_dtype != PLLM_F16 && out_dtype != PLLM_BF16) return PLLM_ERR_INVALID_ARGUMENT;
+    const bool q8 = type_id == PLLM_TYPE_Q8_0;
+    if (!q8 && pllm_gguf_block_bytes(type_id) == 0) return PLLM_ERR_UNSUPPORTED;
+    if (blocks_per_row * (q8 ? 32 : 256) < k) return PLLM_ERR_INVALID_ARGUMENT;
+    if (n_selected == 0) return PLLM_OK;
+    if (n_selected > 0x7fffffffLL || (k + 255) / 256 > 65535 || k > 0x7fffffffLL) return PLLM_ERR_UNSUPPORTED;
+    dim3 grid(static_cast<unsigned>(n_selected), static_cast<unsigned>((k + 255) / 256));
+    hipLaunchKernelGGL(pllm::dequant_rows_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream), row_ids, blocks,
+                       q8 ? -1 : type_id, out, out_dtype, static_cast<int>(k), static_cast<int>(blocks_per_row),
+                       q8 ? 34 : pllm_gguf_block_bytes(type_id), n_rows);
+    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+}
+
+int pllm_fp8_block_dequantize(const uint8_t* weight, const float* scale, int64_t n, int64_t k, void* out, int out_dtype, void* stream) {
+    if (!weight || !scale || !out || n <= 0 || k <= 0) return PLLM_ERR_INVALID_ARGUMENT;
+    if (out_dtype != PLLM_F32 && out_dtype != PLLM_F16 && out_dtype != PLLM_BF16) return PLLM_ERR_INVALID_ARGUMENT;
+    if (n > 0x7fffffffLL || (k + 255) / 256 > 65535) return PLLM_ERR_UNSUPPORTED;
+    dim3 grid(static_cast<unsigned>(n), static_cast<unsigned>((k + 255) / 256));
+    hipLaunchKernelGGL(pllm::dequant_fp8_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream), weight, scale, out,
+                       out_dtype, static_cast<int>(n), static_cast<int>(k), static_cast<int>((k + 127) / 128));
+    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+}
+
+}  // extern "C"

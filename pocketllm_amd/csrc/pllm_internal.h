@@ -27,4 +27,8 @@ int kquant_matvec(const void* x, int x_dtype, const uint8_t* w, int type_id, voi
 int dot4_matvec(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y, int y_dtype,
                 int rows, int k, int n, int bpr, void* workspace, size_t workspace_bytes, hipStream_t stream);
 
+// FP8 E4M3 weights [n, k] with float32 scales [ceil(n/128), ceil(k/128)] (matvec_fp8.hip)
+int fp8_matvec(const void* x, int x_dtype, const uint8_t* w, const float* scale, void* y, int y_dtype,
+               int rows, int k, int n, hipStream_t stream);
+
 }  // namespace pllm

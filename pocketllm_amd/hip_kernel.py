@@ -144,3 +144,108 @@ def gguf_q2k_gemm_dp4a_forward(x, blocks, row_elems, *, out_dtype: torch.dtype =
     _check(blocks.size(2) == 84, "q2_k block size must be 84 bytes")
     empty = torch.empty(0, dtype=torch.int8, device=x.device)
     return _dense_gemm("gguf_q2k_gemm_dp4a_forward", x, blocks, row_elems, 1, empty, out_dtype)
+
+
+def gguf_dequantize_rows(blocks: torch.Tensor, type_id: int, row_elems: int, row_ids: torch.Tensor | None = None, *,
+                         out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """Dequantize whole or selected rows of a raw-block matrix (type_id _ffi.TYPE_Q8_0 for Q8_0 blocks).
+
+    No direct counterpart in the reference extension: it is the device form of the numpy decoders of
+    src/loader/gguf/tensor_reader.py:543-1009, with bit-identical float32 results.
+    """
+    type_id, row_elems = int(type_id), int(row_elems)
+    q8 = type_id == _ffi.TYPE_Q8_0
+    if not q8:
+        _check_type(type_id)
+    _check(blocks.dim() == 3 and blocks.is_cuda and blocks.dtype == torch.uint8 and blocks.is_contiguous(),
+           "blocks must be a contiguous CUDA uint8 tensor [N, K_blocks, block_bytes]")
+    _check(blocks.size(2) == (34 if q8 else GGUF_BLOCK_BYTES[type_id]), "unexpected GGUF block size for type_id")
+    _check(row_elems > 0 and blocks.size(1) * (32 if q8 else 256) >= row_elems, "blocks do not cover row_elems")
+    if row_ids is not None:
+        _check(row_ids.is_cuda and row_ids.dtype == torch.int64 and row_ids.is_contiguous(), "row_ids must be contiguous CUDA int64")
+        lead, count = tuple(row_ids.shape), row_ids.numel()
+    else:
+        lead, count = (blocks.size(0),), blocks.size(0)
+    out = torch.empty(*lead, row_elems, dtype=out_dtype, device=blocks.device)
+    if count == 0:
+        return out
+    with torch.cuda.device(blocks.device):
+        st = _lib().pllm_gguf_dequantize_rows(None if row_ids is None else row_ids.data_ptr(), count, blocks.data_ptr(), type_id,
+                                              blocks.size(0), row_elems, blocks.size(1), out.data_ptr(), _DTYPE_CODE[out_dtype],
+                                              _stream(blocks.device))
+    _ffi.check(st, "gguf_dequantize_rows")
+    return out
+
+
+def gguf_quant_embedding_forward(token_ids, blocks, row_elems, type_id, signed_grid, *, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """src/csrc/cuda_kernel.cpp:669-687.  The reference serves q4_k/q5_k only; every implemented type works here."""
+    row_elems, type_id = int(row_elems), int(type_id)
+    _check(token_ids.dim() in (1, 2), "token_ids must have shape [T] or [B, S]")
+    _check(blocks.dim() == 3, "blocks must have shape [V, K_blocks, block_bytes]")
+    _check_type(type_id)
+    _check(row_elems > 0, "row_elems must be positive")
+    _check(blocks.size(1) * 256 >= row_elems, "blocks do not cover row_elems")
+    _check(blocks.size(2) == GGUF_BLOCK_BYTES[type_id], "unexpected GGUF block size for type_id")
+    _check(token_ids.is_cuda and blocks.is_cuda, "token_ids and blocks must be CUDA tensors")
+    _check(token_ids.is_contiguous() and blocks.is_contiguous(), "token_ids and blocks must be contiguous")
+    _check(token_ids.dtype == torch.int64, "token_ids must be int64")
+    _check(blocks.dtype == torch.uint8, "blocks has unexpected dtype")
+    _check_grid(signed_grid, type_id, "signed_grid")
+    return gguf_dequantize_rows(blocks, type_id, row_elems, token_ids, out_dtype=out_dtype)
+
+
+def fp8_block_dequantize(weight: torch.Tensor, scale: torch.Tensor, *, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """W[r, c] = f32(code) * scale[r // 128, c // 128]  (src/kernels/ops.py:144-147)."""
+    w8 = _fp8_bytes(weight)
+    n, k = w8.shape
+    _check(scale.is_cuda and scale.dtype == torch.float32 and scale.is_contiguous(), "scale must be a contiguous CUDA float32 tensor")
+    _check(tuple(scale.shape) == ((n + 127) // 128, (k + 127) // 128), "scale must have shape [ceil(N/128), ceil(K/128)]")
+    out = torch.empty(n, k, dtype=out_dtype, device=w8.device)
+    with torch.cuda.device(w8.device):
+        st = _lib().pllm_fp8_block_dequantize(w8.data_ptr(), scale.data_ptr(), n, k, out.data_ptr(), _DTYPE_CODE[out_dtype], _stream(w8.device))
+    _ffi.check(st, "fp8_block_dequantize")
+    return out
+
+
+def _fp8_bytes(weight: torch.Tensor) -> torch.Tensor:
+    _check(weight.dim() == 2 and weight.is_cuda and weight.is_contiguous(), "weight must be a contiguous CUDA tensor [N, K]")
+    if weight.dtype == torch.float8_e4m3fn:
+        return weight.view(torch.uint8)
+    _check(weight.dtype == torch.uint8, "weight must be float8_e4m3fn (or its uint8 bytes)")
+    return weight
+
+
+def fp8_block_gemm_forward(x: torch.Tensor, weight: torch.Tensor, scale: torch.Tensor, *, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """y = x @ (f32(weight) * block scales)^T from the FP8 bytes (src/kernels/ops.py:641-648)."""
+    w8 = _fp8_bytes(weight)
+    n, k = w8.shape
+    _check(x.is_cuda and x.is_contiguous() and x.size(-1) == k, "x must be a contiguous CUDA tensor [..., K]")
+    _check_x(x)
+    _check(scale.is_cuda and scale.dtype == torch.float32 and scale.is_contiguous(), "scale must be a contiguous CUDA float32 tensor")
+    _check(tuple(scale.shape) == ((n + 127) // 128, (k + 127) // 128), "scale must have shape [ceil(N/128), ceil(K/128)]")
+    rows = x.numel() // k
+    y = torch.empty(*x.shape[:-1], n, dtype=out_dtype, device=x.device)
+    if rows == 0:
+        return y
+    with torch.cuda.device(x.device):
+        st = _lib().pllm_fp8_block_gemm(x.data_ptr(), _DTYPE_CODE[x.dtype], w8.data_ptr(), scale.data_ptr(), y.data_ptr(),
+                                        _DTYPE_CODE[out_dtype], rows, k, n, _stream(x.device))
+    _ffi.check(st, "fp8_block_gemm_forward")
+    return y
+
+
+def fp8_act_quant_forward(x: torch.Tensor, eps: float = 1e-4, round_scale_pow2: bool = False):
+    """Per-(row, 128) FP8 activation quantizer (src/kernels/ops.py:501-516): returns (float8_e4m3fn codes, float32 scales)."""
+    _check(x.is_cuda and x.is_contiguous(), "x must be a contiguous CUDA tensor")
+    _check_x(x)
+    k = x.size(-1)
+    _check(k % 128 == 0, "last dimension must be a multiple of 128")
+    rows = x.numel() // k
+    codes = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    scales = torch.empty(*x.shape[:-1], k // 128, dtype=torch.float32, device=x.device)
+    if rows:
+        with torch.cuda.device(x.device):
+            st = _lib().pllm_fp8_act_quant(x.data_ptr(), _DTYPE_CODE[x.dtype], rows, k, codes.data_ptr(), scales.data_ptr(),
+                                           float(eps), int(bool(round_scale_pow2)), _stream(x.device))
+        _ffi.check(st, "fp8_act_quant_forward")
+    return codes.view(torch.float8_e4m3fn), scales
