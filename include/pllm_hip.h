@@ -84,6 +84,16 @@ int pllm_gguf_quant_gemm(const void* x, int x_dtype, const uint8_t* blocks, int 
 size_t pllm_gguf_quant_gemm_workspace_bytes(int type_id, int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row);
 
 /*
+ * Two weight matrices of the same [n, k] against one activation tensor (k/v projections): the
+ * activations are quantized once.  y [2, rows, n]; workspace as for pllm_gguf_quant_gemm.
+ * Replaces gguf_quant_gemm_pair_forward (src/csrc/cuda_kernel.cpp:615-666, launcher
+ * src/csrc/cuda_kernel_impl.cu:8598-8650).
+ */
+int pllm_gguf_quant_gemm_pair(const void* x, int x_dtype, const uint8_t* blocks0, int type_id0, const uint8_t* blocks1, int type_id1,
+                              void* y, int y_dtype, int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row,
+                              void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Selected-row dequantization: out[i, :] = dequant(blocks[row_ids[i], :, :])[:k]  (row_ids == NULL
  * selects rows 0 .. n_selected-1 in order).  type_id may also be PLLM_TYPE_Q8_0 (blocks_per_row then
  * counts 32-weight blocks).  Results are bit-identical to the reference's numpy decoders.
@@ -107,6 +117,40 @@ int pllm_gguf_dequantize_rows(const int64_t* row_ids, int64_t n_selected, const 
 int pllm_fp8_block_dequantize(const uint8_t* weight, const float* scale, int64_t n, int64_t k, void* out, int out_dtype, void* stream);
 int pllm_fp8_block_gemm(const void* x, int x_dtype, const uint8_t* weight, const float* scale, void* y, int y_dtype,
                         int64_t rows, int64_t k, int64_t n, void* stream);
+
+/*
+ * Fused routed-expert matmul over raw super-blocks (types Q2_K, IQ2_XXS, IQ1_M; gate/up share a type,
+ * the down projection may use another, so IQ2_XXS gate/up with IQ1_M down needs no special case):
+ *     y[t] = sum over routes r of token t:  W2_e ( silu(min(W1_e x_t, L)) * clamp(W3_e x_t, +-L) * w_r )
+ * with the clamp only when swiglu_limit L > 0.
+ *   x [tokens, dim]; w1, w3 [n_experts, inter, ceil(dim/256), bb]; w2 [n_experts, dim, ceil(inter/256), bb]
+ *   route_tokens  int64 [routes] token of each route (NULL when tokens == 1)
+ *   route_experts int64 [routes] expert of each route, or NULL with seg_starts int32 [n_experts + 1]
+ *                 giving expert e the routes [seg_starts[e], seg_starts[e+1])
+ *   route_weights float32 [routes];  y float32 [tokens, dim], fully overwritten
+ * Each token's routes are summed in ascending route order (deterministic).
+ * Replaces gguf_moe_prefill_grouped_forward, gguf_moe_single_token_iq2_q2k_forward and
+ * gguf_moe_single_token_iq1m_forward (src/csrc/cuda_kernel.cpp:689-865; launchers
+ * src/csrc/cuda_kernel_impl.cu:8688-9385).
+ */
+size_t pllm_gguf_moe_workspace_bytes(int64_t tokens, int64_t routes, int64_t dim, int64_t inter);
+int pllm_gguf_moe_forward(const void* x, int x_dtype, int64_t tokens, int64_t dim, int64_t inter,
+                          const int64_t* route_tokens, const int64_t* route_experts, const int32_t* seg_starts, int64_t n_experts,
+                          const float* route_weights, int64_t routes,
+                          const uint8_t* w1, const uint8_t* w3, int w13_type, const uint8_t* w2, int w2_type,
+                          float swiglu_limit, float* y, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Counting sort of the (token, k) routes of indices [tokens, topk] by local expert
+ * (local = expert - experts_start, kept when 0 <= local < n_local), stable in (token, k) order.
+ *   seg_starts int32 [n_local + 1]; route_tokens int64, route_weights float32, route_experts int32:
+ *   capacity tokens * topk each, the first seg_starts[n_local] entries are written.
+ * Replaces moe_group_routes (src/csrc/cuda_kernel.cpp:1228-1242, src/csrc/cuda_kernel_impl.cu:295-351,
+ * 4306-4377), whose order inside a segment depends on atomics.
+ */
+int pllm_moe_group_routes(const void* indices, int indices_are_i64, const float* weights, int64_t tokens, int64_t topk,
+                          int64_t experts_start, int64_t n_local, int32_t* seg_starts, int64_t* route_tokens, float* route_weights,
+                          int32_t* route_experts, void* stream);
 
 /*
  * FP8 activation quantizer: per (row, 128 values) scale = max(amax, eps) / 448 (rounded up to a power

@@ -52,6 +52,21 @@ size_t pllm_q8_0_gemm_workspace_bytes(int64_t rows, int64_t k, int64_t n, int64_
     return pllm::q8_0_matvec_workspace_bytes(static_cast<int>(rows), static_cast<int>(blocks_per_row));
 }
 
+static int superblock_matvec(const unsigned char* image, size_t stride, const uint8_t* blocks, int type_id, void* y, int y_dtype,
+                             int rows, int n, int bpr, hipStream_t s) {
+    switch (type_id) {
+        case PLLM_TYPE_Q2_K:
+        case PLLM_TYPE_IQ2_XXS:
+        case PLLM_TYPE_IQ1_M:
+            return pllm::dot4_matvec_from_image(image, stride, blocks, type_id, y, y_dtype, rows, n, bpr, s);
+        case PLLM_TYPE_Q4_K:
+        case PLLM_TYPE_Q5_K:
+            return pllm::kquant_matvec_from_image(image, stride, blocks, type_id, y, y_dtype, rows, n, bpr, s);
+        default:
+            return PLLM_ERR_UNSUPPORTED;
+    }
+}
+
 int pllm_gguf_quant_gemm(const void* x, int x_dtype, const uint8_t* blocks, int type_id, void* y, int y_dtype,
                          int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row,
                          void* workspace, size_t workspace_bytes, void* stream) {
@@ -60,26 +75,41 @@ int pllm_gguf_quant_gemm(const void* x, int x_dtype, const uint8_t* blocks, int 
     if (blocks_per_row * 256 < k) return PLLM_ERR_INVALID_ARGUMENT;
     if (pllm_gguf_block_bytes(type_id) == 0) return PLLM_ERR_UNSUPPORTED;
     if (rows > 65535) return PLLM_ERR_UNSUPPORTED;
+    if (!workspace || workspace_bytes < pllm_gguf_quant_gemm_workspace_bytes(type_id, rows, k, n, blocks_per_row)) return PLLM_ERR_WORKSPACE;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    switch (type_id) {
-        case PLLM_TYPE_Q2_K:
-        case PLLM_TYPE_IQ2_XXS:
-        case PLLM_TYPE_IQ1_M:
-            return pllm::dot4_matvec(x, x_dtype, blocks, type_id, y, y_dtype, static_cast<int>(rows), static_cast<int>(k),
-                                     static_cast<int>(n), static_cast<int>(blocks_per_row), workspace, workspace_bytes, s);
-        case PLLM_TYPE_Q4_K:
-        case PLLM_TYPE_Q5_K:
-            return pllm::kquant_matvec(x, x_dtype, blocks, type_id, y, y_dtype, static_cast<int>(rows), static_cast<int>(k),
-                                       static_cast<int>(n), static_cast<int>(blocks_per_row), workspace, workspace_bytes, s);
-        default:
-            return PLLM_ERR_UNSUPPORTED;
-    }
+    const int bpr = static_cast<int>(blocks_per_row);
+    const int st = pllm::act_image_256(x, x_dtype, static_cast<int>(rows), static_cast<int>(k), bpr, workspace, s);
+    if (st != PLLM_OK) return st;
+    return superblock_matvec(static_cast<const unsigned char*>(workspace), pllm::act_image_256_bytes(bpr), blocks, type_id, y, y_dtype,
+                             static_cast<int>(rows), static_cast<int>(n), bpr, s);
 }
 
 size_t pllm_gguf_quant_gemm_workspace_bytes(int type_id, int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row) {
     (void)k; (void)n;
     if (!fits_int(rows) || !fits_int(blocks_per_row) || pllm_gguf_block_bytes(type_id) == 0) return 0;
-    return pllm::kquant_matvec_workspace_bytes(static_cast<int>(rows), static_cast<int>(blocks_per_row));
+    return pllm::act_image_256_bytes(static_cast<int>(blocks_per_row)) * static_cast<size_t>(rows);
+}
+
+int pllm_gguf_quant_gemm_pair(const void* x, int x_dtype, const uint8_t* blocks0, int type_id0, const uint8_t* blocks1, int type_id1,
+                              void* y, int y_dtype, int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row,
+                              void* workspace, size_t workspace_bytes, void* stream) {
+    if (!x || !blocks0 || !blocks1 || !y || !dtype_ok(x_dtype) || !dtype_ok(y_dtype)) return PLLM_ERR_INVALID_ARGUMENT;
+    if (!fits_int(rows) || !fits_int(k) || !fits_int(n) || !fits_int(blocks_per_row)) return PLLM_ERR_INVALID_ARGUMENT;
+    if (blocks_per_row * 256 < k) return PLLM_ERR_INVALID_ARGUMENT;
+    if (pllm_gguf_block_bytes(type_id0) == 0 || pllm_gguf_block_bytes(type_id1) == 0) return PLLM_ERR_UNSUPPORTED;
+    if (rows > 65535) return PLLM_ERR_UNSUPPORTED;
+    if (!workspace || workspace_bytes < pllm_gguf_quant_gemm_workspace_bytes(type_id0, rows, k, n, blocks_per_row)) return PLLM_ERR_WORKSPACE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int bpr = static_cast<int>(blocks_per_row);
+    int st = pllm::act_image_256(x, x_dtype, static_cast<int>(rows), static_cast<int>(k), bpr, workspace, s);
+    if (st != PLLM_OK) return st;
+    const unsigned char* image = static_cast<const unsigned char*>(workspace);
+    const size_t stride = pllm::act_image_256_bytes(bpr);
+    const size_t esize = y_dtype == PLLM_F32 ? 4 : 2;
+    st = superblock_matvec(image, stride, blocks0, type_id0, y, y_dtype, static_cast<int>(rows), static_cast<int>(n), bpr, s);
+    if (st != PLLM_OK) return st;
+    return superblock_matvec(image, stride, blocks1, type_id1, static_cast<char*>(y) + static_cast<size_t>(rows) * n * esize, y_dtype,
+                             static_cast<int>(rows), static_cast<int>(n), bpr, s);
 }
 
 int pllm_fp8_block_gemm(const void* x, int x_dtype, const uint8_t* weight, const float* scale, void* y, int y_dtype,

@@ -18,12 +18,13 @@ constexpr int kMaxWaves = 8;
 template <typename FMT, int ITERS>
 __global__ __launch_bounds__(64 * kMaxWaves) void dot4_matvec_kernel(
     const unsigned char* __restrict__ image, size_t image_stride, const uint8_t* __restrict__ w,
-    void* __restrict__ y, int y_dtype, int n, int bpr) {
+    void* __restrict__ y, int y_dtype, int n, int bpr, const int32_t* __restrict__ y_expert, size_t expert_stride) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int kpad = bpr * 256;
     const int image_bytes = static_cast<int>(staged_x_bytes(kpad));
     const StagedX sx = carve_staged_x(smem, kpad);
     unsigned char* tables = smem + image_bytes;
+    if (y_expert) w += static_cast<size_t>(y_expert[blockIdx.y]) * expert_stride;   // routed: activation row r meets expert r's matrix
     float* partial = reinterpret_cast<float*>(tables + FMT::kTableBytes);        // [waves][16]
 
     const int tid = threadIdx.x;
@@ -70,7 +71,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void dot4_matvec_kernel(
 
 template <typename FMT, int ITERS>
 int launch_one(const unsigned char* image, size_t image_stride, const uint8_t* w, void* y, int y_dtype,
-               int rows, int n, int bpr, int waves, hipStream_t stream) {
+               int rows, int n, int bpr, int waves, const int32_t* y_expert, size_t expert_stride, hipStream_t stream) {
     const size_t smem = staged_x_bytes(bpr * 256) + FMT::kTableBytes + static_cast<size_t>(waves) * kRowsPerWg * sizeof(float);
     auto kern = dot4_matvec_kernel<FMT, ITERS>;
     if (smem > 64 * 1024) {
@@ -80,40 +81,40 @@ int launch_one(const unsigned char* image, size_t image_stride, const uint8_t* w
             return PLLM_ERR_UNSUPPORTED;
     }
     dim3 grid((n + kRowsPerWg - 1) / kRowsPerWg, rows);
-    hipLaunchKernelGGL(kern, grid, dim3(64 * waves), smem, stream, image, image_stride, w, y, y_dtype, n, bpr);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * waves), smem, stream, image, image_stride, w, y, y_dtype, n, bpr, y_expert, expert_stride);
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 
 template <typename FMT>
 int launch_fmt(const unsigned char* image, size_t image_stride, const uint8_t* w, void* y, int y_dtype,
-               int rows, int n, int bpr, hipStream_t stream) {
+               int rows, int n, int bpr, const int32_t* y_expert, size_t expert_stride, hipStream_t stream) {
     // waves per workgroup: split a row's blocks so that every wave keeps a handful in flight
     int waves = 1;
     while (waves < kMaxWaves && bpr / (waves * 2) >= 3) waves *= 2;
     const int niter = (bpr + waves - 1) / waves;
     const int passes = (niter + 5) / 6;
     const int iters = (niter + passes - 1) / passes;
-#define PLLM_CASE(I) case I: return launch_one<FMT, I>(image, image_stride, w, y, y_dtype, rows, n, bpr, waves, stream)
+#define PLLM_CASE(I) case I: return launch_one<FMT, I>(image, image_stride, w, y, y_dtype, rows, n, bpr, waves, y_expert, expert_stride, stream)
     switch (iters) {
         PLLM_CASE(1); PLLM_CASE(2); PLLM_CASE(3); PLLM_CASE(4); PLLM_CASE(5);
-        default: return launch_one<FMT, 6>(image, image_stride, w, y, y_dtype, rows, n, bpr, waves, stream);
+        default: return launch_one<FMT, 6>(image, image_stride, w, y, y_dtype, rows, n, bpr, waves, y_expert, expert_stride, stream);
     }
 #undef PLLM_CASE
 }
 
 }  // namespace
 
-int dot4_matvec(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y, int y_dtype,
-                int rows, int k, int n, int bpr, void* workspace, size_t workspace_bytes, hipStream_t stream) {
-    if (!workspace || workspace_bytes < kquant_matvec_workspace_bytes(rows, bpr)) return PLLM_ERR_WORKSPACE;
-    const int st = act_image_256(x, x_dtype, rows, k, bpr, workspace, stream);
-    if (st != PLLM_OK) return st;
-    const unsigned char* image = static_cast<const unsigned char*>(workspace);
-    const size_t stride = act_image_256_bytes(bpr);
+int dot4_matvec_from_image(const unsigned char* image, size_t stride, const uint8_t* w, int type_id, void* y, int y_dtype,
+                           int rows, int n, int bpr, hipStream_t stream) {
+    return dot4_routed_matvec_from_image(image, stride, w, type_id, y, y_dtype, rows, n, bpr, nullptr, 0, stream);
+}
+
+int dot4_routed_matvec_from_image(const unsigned char* image, size_t stride, const uint8_t* w, int type_id, void* y, int y_dtype,
+                                  int rows, int n, int bpr, const int32_t* y_expert, size_t expert_stride, hipStream_t stream) {
     switch (type_id) {
-        case PLLM_TYPE_Q2_K: return launch_fmt<Q2K>(image, stride, w, y, y_dtype, rows, n, bpr, stream);
-        case PLLM_TYPE_IQ2_XXS: return launch_fmt<IQ2XXS>(image, stride, w, y, y_dtype, rows, n, bpr, stream);
-        case PLLM_TYPE_IQ1_M: return launch_fmt<IQ1M>(image, stride, w, y, y_dtype, rows, n, bpr, stream);
+        case PLLM_TYPE_Q2_K: return launch_fmt<Q2K>(image, stride, w, y, y_dtype, rows, n, bpr, y_expert, expert_stride, stream);
+        case PLLM_TYPE_IQ2_XXS: return launch_fmt<IQ2XXS>(image, stride, w, y, y_dtype, rows, n, bpr, y_expert, expert_stride, stream);
+        case PLLM_TYPE_IQ1_M: return launch_fmt<IQ1M>(image, stride, w, y, y_dtype, rows, n, bpr, y_expert, expert_stride, stream);
         default: return PLLM_ERR_UNSUPPORTED;
     }
 }

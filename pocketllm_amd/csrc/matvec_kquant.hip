@@ -223,13 +223,8 @@ int launch_k45(const unsigned char* image, size_t image_stride, const uint8_t* w
 
 size_t kquant_matvec_workspace_bytes(int rows, int bpr) { return act_image_256_bytes(bpr) * static_cast<size_t>(rows); }
 
-int kquant_matvec(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y, int y_dtype,
-                  int rows, int k, int n, int bpr, void* workspace, size_t workspace_bytes, hipStream_t stream) {
-    if (!workspace || workspace_bytes < kquant_matvec_workspace_bytes(rows, bpr)) return PLLM_ERR_WORKSPACE;
-    const int st = act_image_256(x, x_dtype, rows, k, bpr, workspace, stream);
-    if (st != PLLM_OK) return st;
-    const unsigned char* image = static_cast<const unsigned char*>(workspace);
-    const size_t stride = act_image_256_bytes(bpr);
+int kquant_matvec_from_image(const unsigned char* image, size_t stride, const uint8_t* w, int type_id, void* y, int y_dtype,
+                             int rows, int n, int bpr, hipStream_t stream) {
     switch (type_id) {
         case PLLM_TYPE_Q4_K: return launch_k45<Q4K>(image, stride, w, y, y_dtype, rows, n, bpr, stream);
         case PLLM_TYPE_Q5_K: return launch_k45<Q5K>(image, stride, w, y, y_dtype, rows, n, bpr, stream);

@@ -1,0 +1,291 @@
+// Routed experts over raw GGUF super-blocks: route grouping and the fused expert matmul
+//     y[t] = sum over routes r of token t:  W2_e ( silu(W1_e x_t) * (W3_e x_t) * w_r ),   e = expert of r.
+//
+// Stages, all on one stream:
+//   1. act_image_256 quantizes every token's activations once (two int8 terms per value).
+//   2. moe_w13_kernel: one workgroup per (32 intermediate rows, route).  Waves 0/1 take the gate rows,
+//      waves 2/3 the up rows, v_dot4 block dots against the token's image in LDS.  The epilogue
+//      applies the clamp, SiLU and the route weight and QUANTIZES the 32 hidden values in place,
+//      writing the route's hidden activations straight into the image format the down projection
+//      reads: no float gate/up/hidden tensors are materialised.
+//   3. the routed matvec of matvec_dot4.hip computes W2_e h_r per route into a float32 [R, D] scratch.
+//   4. moe_reduce_kernel sums each token's routes in ascending route order: the result does not
+//      depend on scheduling (the reference accumulates with atomicAdd).
+#include "block_dot4.h"
+#include "pllm_internal.h"
+
+namespace pllm {
+namespace {
+
+constexpr int kW13Iters = 6;
+
+template <typename FMT>
+__global__ __launch_bounds__(256) void moe_w13_kernel(
+    const unsigned char* __restrict__ x_image, size_t x_image_stride, int bpr,
+    const int64_t* __restrict__ route_tokens, const int32_t* __restrict__ route_experts, const float* __restrict__ route_weights,
+    const uint8_t* __restrict__ w1, const uint8_t* __restrict__ w3, int inter, float limit,
+    unsigned char* __restrict__ h_image, size_t h_image_stride, int h_kpad) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int kpad = bpr * 256;
+    const int image_bytes = static_cast<int>(staged_x_bytes(kpad));
+    const StagedX sx = carve_staged_x(smem, kpad);
+    unsigned char* tables = smem + image_bytes;
+    float* exch = reinterpret_cast<float*>(tables + FMT::kTableBytes);           // [2][32]
+
+    const int route = blockIdx.y;
+    const int64_t token = route_tokens ? route_tokens[route] : 0;
+    const size_t expert_off = static_cast<size_t>(route_experts[route]) * inter * bpr * FMT::kBlockBytes;
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int j = lane & 3, team = lane >> 2;
+    const int mat = wave >> 1;
+    const int slot = 16 * (wave & 1) + team;                                     // 0..31 inside the tile
+    const int row = min(blockIdx.x * 32 + slot, inter - 1);
+    const uint8_t* wrow = (mat ? w3 : w1) + expert_off + static_cast<size_t>(row) * bpr * FMT::kBlockBytes;
+
+    float acc = 0.0f;
+    bool staged = false;
+    for (int b0 = 0; b0 < bpr; b0 += kW13Iters) {
+        typename FMT::Regs regs[kW13Iters];
+#pragma unroll
+        for (int it = 0; it < kW13Iters; ++it)
+            FMT::load(regs[it], wrow + static_cast<size_t>(min(b0 + it, bpr - 1)) * FMT::kBlockBytes, j);
+        if (!staged) {
+            copy_to_lds(smem, x_image + static_cast<size_t>(token) * x_image_stride, image_bytes);
+            FMT::stage_tables(tables);
+            __syncthreads();
+            staged = true;
+        }
+#pragma unroll
+        for (int it = 0; it < kW13Iters; ++it)
+            if (b0 + it < bpr) acc += FMT::lane_dot(regs[it], j, b0 + it, sx, tables);
+    }
+    acc += __shfl_xor(acc, 1, 64);
+    acc += __shfl_xor(acc, 2, 64);
+    if (j == 0) exch[mat * 32 + slot] = acc;
+    __syncthreads();
+    if (tid < 32) {
+        const int i = blockIdx.x * 32 + tid;
+        float g = exch[tid], u = exch[32 + tid];
+        if (limit > 0.0f) {
+            u = fminf(fmaxf(u, -limit), limit);
+            g = fminf(g, limit);
+        }
+        const float h = (i < inter) ? g / (1.0f + expf(-g)) * u * route_weights[route] : 0.0f;
+        // quantize the 32 hidden values of this tile (one activation group of the down projection)
+        float am = fabsf(h);
+#pragma unroll
+        for (int off = 1; off < 32; off <<= 1) am = fmaxf(am, __shfl_xor(am, off, 64));
+        const float inv = am > 0.0f ? 127.0f / am : 0.0f;
+        const float scale = am * (1.0f / 127.0f);
+        const float q = fminf(fmaxf(rintf(h * inv), -127.0f), 127.0f);
+        const float l = fminf(fmaxf(rintf((h - q * scale) * inv * 254.0f), -127.0f), 127.0f);
+        float s16 = h;
+#pragma unroll
+        for (int off = 1; off < 16; off <<= 1) s16 += __shfl_xor(s16, off, 64);
+        const float s32 = s16 + __shfl_xor(s16, 16, 64);
+        unsigned char* img = h_image + static_cast<size_t>(route) * h_image_stride;
+        if (i < h_kpad) {
+            reinterpret_cast<int8_t*>(img)[i] = static_cast<int8_t>(static_cast<int>(q));
+            reinterpret_cast<int8_t*>(img + h_kpad)[i] = static_cast<int8_t>(static_cast<int>(l));
+            float2* gs = reinterpret_cast<float2*>(img + 2 * static_cast<size_t>(h_kpad));
+            float* sum16 = reinterpret_cast<float*>(gs + h_kpad / 32);
+            if ((tid & 15) == 0) sum16[i >> 4] = s16;
+            if (tid == 0) gs[i >> 5] = make_float2(scale * kLoInv, s32);
+        }
+    }
+}
+
+// seg_starts [E + 1] -> route_experts [R]
+__global__ void expand_segments_kernel(const int32_t* __restrict__ seg, int32_t* __restrict__ route_experts, int n_experts) {
+    const int e = blockIdx.x;
+    if (e >= n_experts) return;
+    for (int r = seg[e] + threadIdx.x; r < seg[e + 1]; r += blockDim.x) route_experts[r] = e;
+}
+
+__global__ void zero_fill_kernel(float* __restrict__ p, size_t n) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0.0f;
+}
+
+__global__ void narrow_experts_kernel(const int64_t* __restrict__ src, int32_t* __restrict__ dst, int routes) {
+    const int r = blockIdx.x * blockDim.x + threadIdx.x;
+    if (r < routes) dst[r] = static_cast<int32_t>(src[r]);
+}
+
+// y[t, d] = sum_{r : route_tokens[r] == t} partial[r, d], ascending r.  grid (tokens, ceil(dim / 256))
+__global__ __launch_bounds__(256) void moe_reduce_kernel(const float* __restrict__ partial, const int64_t* __restrict__ route_tokens,
+                                                         float* __restrict__ y, int routes, int dim) {
+    const int t = blockIdx.x;
+    const int d = blockIdx.y * 256 + threadIdx.x;
+    float acc = 0.0f;
+    for (int r = 0; r < routes; ++r) {
+        const bool mine = route_tokens ? (route_tokens[r] == t) : true;         // uniform across the workgroup
+        if (mine && d < dim) acc += partial[static_cast<size_t>(r) * dim + d];
+    }
+    if (d < dim) y[static_cast<size_t>(t) * dim + d] = acc;
+}
+
+// ---- route grouping ---------------------------------------------------------------------------
+// counts per local expert and exclusive prefix; one workgroup
+__global__ __launch_bounds__(1024) void route_count_kernel(const void* __restrict__ indices, int idx_is_i64, int total, int start, int n_local,
+                                                           int32_t* __restrict__ seg_starts) {
+    extern __shared__ int32_t counts[];
+    for (int e = threadIdx.x; e <= n_local; e += blockDim.x) counts[e] = 0;
+    __syncthreads();
+    for (int i = threadIdx.x; i < total; i += blockDim.x) {
+        const int64_t ex = idx_is_i64 ? static_cast<const int64_t*>(indices)[i] : static_cast<const int32_t*>(indices)[i];
+        const int64_t local = ex - start;
+        if (local >= 0 && local < n_local) atomicAdd(&counts[local], 1);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int32_t run = 0;
+        for (int e = 0; e < n_local; ++e) {
+            const int32_t c = counts[e];
+            seg_starts[e] = run;
+            run += c;
+        }
+        seg_starts[n_local] = run;
+    }
+}
+
+// one wave per local expert: stable compaction of its (token, weight) pairs in (token, k) order
+__global__ __launch_bounds__(64) void route_fill_kernel(const void* __restrict__ indices, int idx_is_i64, const float* __restrict__ weights,
+                                                        int total, int topk, int start, const int32_t* __restrict__ seg_starts,
+                                                        int64_t* __restrict__ route_tokens, float* __restrict__ route_weights,
+                                                        int32_t* __restrict__ route_experts) {
+    const int e = blockIdx.x;
+    const int lane = threadIdx.x;
+    int out = seg_starts[e];
+    for (int base = 0; base < total; base += 64) {
+        const int i = base + lane;
+        bool hit = false;
+        if (i < total) {
+            const int64_t ex = idx_is_i64 ? static_cast<const int64_t*>(indices)[i] : static_cast<const int32_t*>(indices)[i];
+            hit = (ex - start) == e;
+        }
+        const unsigned long long mask = __ballot(hit);
+        if (hit) {
+            const int pos = out + __popcll(mask & ((1ull << lane) - 1ull));
+            route_tokens[pos] = i / topk;
+            route_weights[pos] = weights[i];
+            route_experts[pos] = e;
+        }
+        out += __popcll(mask);
+    }
+}
+
+template <typename FMT>
+int launch_w13(const unsigned char* x_image, size_t x_stride, int bpr, const int64_t* route_tokens, const int32_t* route_experts,
+               const float* route_weights, const uint8_t* w1, const uint8_t* w3, int inter, float limit, unsigned char* h_image,
+               size_t h_stride, int h_kpad, int routes, hipStream_t stream) {
+    const size_t smem = staged_x_bytes(bpr * 256) + FMT::kTableBytes + 64 * sizeof(float);
+    auto kern = moe_w13_kernel<FMT>;
+    if (smem > 64 * 1024) {
+        if (smem > 160 * 1024) return PLLM_ERR_UNSUPPORTED;
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                static_cast<int>(smem)) != hipSuccess)
+            return PLLM_ERR_UNSUPPORTED;
+    }
+    dim3 grid(h_kpad / 32, routes);
+    hipLaunchKernelGGL(kern, grid, dim3(256), smem, stream, x_image, x_stride, bpr, route_tokens, route_experts, route_weights, w1, w3,
+                       inter, limit, h_image, h_stride, h_kpad);
+    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+}
+
+bool dot4_type(int t) { return t == PLLM_TYPE_Q2_K || t == PLLM_TYPE_IQ2_XXS || t == PLLM_TYPE_IQ1_M; }
+
+size_t align256(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
+
+}  // namespace
+}  // namespace pllm
+
+extern "C" {
+
+size_t pllm_gguf_moe_workspace_bytes(int64_t tokens, int64_t routes, int64_t dim, int64_t inter) {
+    if (tokens <= 0 || routes < 0 || dim <= 0 || inter <= 0) return 0;
+    const int bpr_x = static_cast<int>((dim + 255) / 256), bpr_h = static_cast<int>((inter + 255) / 256);
+    return pllm::act_image_256_bytes(bpr_x) * static_cast<size_t>(tokens) + pllm::act_image_256_bytes(bpr_h) * static_cast<size_t>(routes) +
+           pllm::align256(static_cast<size_t>(routes) * dim * sizeof(float)) + pllm::align256(static_cast<size_t>(routes) * sizeof(int32_t)) + 256;
+}
+
+int pllm_gguf_moe_forward(const void* x, int x_dtype, int64_t tokens, int64_t dim, int64_t inter,
+                          const int64_t* route_tokens, const int64_t* route_experts, const int32_t* seg_starts, int64_t n_experts,
+                          const float* route_weights, int64_t routes,
+                          const uint8_t* w1, const uint8_t* w3, int w13_type, const uint8_t* w2, int w2_type,
+                          float swiglu_limit, float* y, void* workspace, size_t workspace_bytes, void* stream) {
+    using namespace pllm;
+    if (!x || !y || tokens <= 0 || dim <= 0 || inter <= 0 || routes < 0 || n_experts <= 0) return PLLM_ERR_INVALID_ARGUMENT;
+    if (x_dtype != PLLM_F32 && x_dtype != PLLM_F16 && x_dtype != PLLM_BF16) return PLLM_ERR_INVALID_ARGUMENT;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (routes == 0) {
+        const size_t count = static_cast<size_t>(tokens) * dim;                // a kernel, not a memset: callers may capture graphs
+        hipLaunchKernelGGL(zero_fill_kernel, dim3(static_cast<unsigned>((count + 255) / 256)), dim3(256), 0, s, y, count);
+        return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+    }
+    if (!w1 || !w3 || !w2 || !route_weights || (!route_experts && !seg_starts)) return PLLM_ERR_INVALID_ARGUMENT;
+    if (!dot4_type(w13_type) || !dot4_type(w2_type)) return PLLM_ERR_UNSUPPORTED;
+    if (tokens > 65535 || routes > 65535 || dim > (1 << 24) || inter > (1 << 24)) return PLLM_ERR_UNSUPPORTED;
+    if (tokens > 1 && !route_tokens) return PLLM_ERR_INVALID_ARGUMENT;
+    if (!workspace || workspace_bytes < pllm_gguf_moe_workspace_bytes(tokens, routes, dim, inter)) return PLLM_ERR_WORKSPACE;
+
+    const int bpr_x = static_cast<int>((dim + 255) / 256), bpr_h = static_cast<int>((inter + 255) / 256);
+    const size_t x_stride = act_image_256_bytes(bpr_x), h_stride = act_image_256_bytes(bpr_h);
+    unsigned char* ws = static_cast<unsigned char*>(workspace);
+    unsigned char* x_image = ws;
+    unsigned char* h_image = x_image + x_stride * tokens;
+    float* partial = reinterpret_cast<float*>(h_image + h_stride * routes);
+    int32_t* experts32 = reinterpret_cast<int32_t*>(reinterpret_cast<unsigned char*>(partial) + align256(static_cast<size_t>(routes) * dim * sizeof(float)));
+    const int R = static_cast<int>(routes);
+
+    if (route_experts) {
+        hipLaunchKernelGGL(narrow_experts_kernel, dim3((R + 255) / 256), dim3(256), 0, s, route_experts, experts32, R);
+    } else {
+        hipLaunchKernelGGL(expand_segments_kernel, dim3(static_cast<unsigned>(n_experts)), dim3(256), 0, s, seg_starts, experts32,
+                           static_cast<int>(n_experts));
+    }
+    if (hipGetLastError() != hipSuccess) return PLLM_ERR_LAUNCH;
+    int st = act_image_256(x, x_dtype, static_cast<int>(tokens), static_cast<int>(dim), bpr_x, x_image, s);
+    if (st != PLLM_OK) return st;
+
+    const int I = static_cast<int>(inter);
+    switch (w13_type) {
+        case PLLM_TYPE_IQ2_XXS:
+            st = launch_w13<IQ2XXS>(x_image, x_stride, bpr_x, route_tokens, experts32, route_weights, w1, w3, I, swiglu_limit, h_image, h_stride, bpr_h * 256, R, s);
+            break;
+        case PLLM_TYPE_IQ1_M:
+            st = launch_w13<IQ1M>(x_image, x_stride, bpr_x, route_tokens, experts32, route_weights, w1, w3, I, swiglu_limit, h_image, h_stride, bpr_h * 256, R, s);
+            break;
+        default:
+            st = launch_w13<Q2K>(x_image, x_stride, bpr_x, route_tokens, experts32, route_weights, w1, w3, I, swiglu_limit, h_image, h_stride, bpr_h * 256, R, s);
+            break;
+    }
+    if (st != PLLM_OK) return st;
+
+    const size_t w2_expert_stride = static_cast<size_t>(dim) * bpr_h * pllm_gguf_block_bytes(w2_type);
+    st = dot4_routed_matvec_from_image(h_image, h_stride, w2, w2_type, partial, PLLM_F32, R, static_cast<int>(dim), bpr_h, experts32,
+                                       w2_expert_stride, s);
+    if (st != PLLM_OK) return st;
+    dim3 rgrid(static_cast<unsigned>(tokens), static_cast<unsigned>((dim + 255) / 256));
+    hipLaunchKernelGGL(moe_reduce_kernel, rgrid, dim3(256), 0, s, partial, tokens > 1 ? route_tokens : nullptr, y, R, static_cast<int>(dim));
+    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+}
+
+int pllm_moe_group_routes(const void* indices, int indices_are_i64, const float* weights, int64_t tokens, int64_t topk,
+                          int64_t experts_start, int64_t n_local, int32_t* seg_starts, int64_t* route_tokens, float* route_weights,
+                          int32_t* route_experts, void* stream) {
+    using namespace pllm;
+    if (!indices || !weights || !seg_starts || !route_tokens || !route_weights || !route_experts) return PLLM_ERR_INVALID_ARGUMENT;
+    if (tokens <= 0 || topk <= 0 || n_local <= 0) return PLLM_ERR_INVALID_ARGUMENT;
+    if (tokens * topk > 0x7fffffffLL || n_local > 8192) return PLLM_ERR_UNSUPPORTED;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int total = static_cast<int>(tokens * topk);
+    hipLaunchKernelGGL(route_count_kernel, dim3(1), dim3(1024), (n_local + 1) * sizeof(int32_t), s, indices, indices_are_i64, total,
+                       static_cast<int>(experts_start), static_cast<int>(n_local), seg_starts);
+    hipLaunchKernelGGL(route_fill_kernel, dim3(static_cast<unsigned>(n_local)), dim3(64), 0, s, indices, indices_are_i64, weights, total,
+                       static_cast<int>(topk), static_cast<int>(experts_start), seg_starts, route_tokens, route_weights, route_experts);
+    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+}
+
+}  // extern "C"

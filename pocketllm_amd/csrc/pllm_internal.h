@@ -19,13 +19,16 @@ size_t q8_0_matvec_workspace_bytes(int rows, int bpr);
 int q8_0_matvec(const void* x, int x_dtype, const uint8_t* w, void* y, int y_dtype,
                 int rows, int k, int n, int bpr, void* workspace, size_t workspace_bytes, hipStream_t stream);
 
-size_t kquant_matvec_workspace_bytes(int rows, int bpr);
-int kquant_matvec(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y, int y_dtype,
-                  int rows, int k, int n, int bpr, void* workspace, size_t workspace_bytes, hipStream_t stream);
+// 256-weight super-block types: one activation image (act_image_256) serves any number of matvecs.
+// Q4_K / Q5_K run in matvec_kquant.hip, Q2_K / IQ2_XXS / IQ1_M in matvec_dot4.hip.
+int kquant_matvec_from_image(const unsigned char* image, size_t stride, const uint8_t* w, int type_id, void* y, int y_dtype,
+                             int rows, int n, int bpr, hipStream_t stream);
+int dot4_matvec_from_image(const unsigned char* image, size_t stride, const uint8_t* w, int type_id, void* y, int y_dtype,
+                           int rows, int n, int bpr, hipStream_t stream);
 
-// Q2_K / IQ2_XXS / IQ1_M (matvec_dot4.hip); same workspace as kquant_matvec
-int dot4_matvec(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y, int y_dtype,
-                int rows, int k, int n, int bpr, void* workspace, size_t workspace_bytes, hipStream_t stream);
+// routed form: activation row r (image r, output row r) meets the matrix at w + y_expert[r] * expert_stride
+int dot4_routed_matvec_from_image(const unsigned char* image, size_t stride, const uint8_t* w, int type_id, void* y, int y_dtype,
+                                  int rows, int n, int bpr, const int32_t* y_expert, size_t expert_stride, hipStream_t stream);
 
 // FP8 E4M3 weights [n, k] with float32 scales [ceil(n/128), ceil(k/128)] (matvec_fp8.hip)
 int fp8_matvec(const void* x, int x_dtype, const uint8_t* w, const float* scale, void* y, int y_dtype,

@@ -249,3 +249,247 @@ def fp8_act_quant_forward(x: torch.Tensor, eps: float = 1e-4, round_scale_pow2: 
                                            float(eps), int(bool(round_scale_pow2)), _stream(x.device))
         _ffi.check(st, "fp8_act_quant_forward")
     return codes.view(torch.float8_e4m3fn), scales
+
+
+def gguf_quant_gemm_pair_forward(x, blocks0, row_elems0, type_id0, blocks1, row_elems1, type_id1, signed_grid, *,
+                                 out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """src/csrc/cuda_kernel.cpp:615-666: returns the stack [2, ..., N]."""
+    row_elems0, row_elems1, type_id0, type_id1 = int(row_elems0), int(row_elems1), int(type_id0), int(type_id1)
+    _check(x.dim() in (2, 3), "x must have shape [M, K] or [B, S, K]")
+    _check(blocks0.dim() == 3 and blocks1.dim() == 3, "blocks must have shape [N, K_blocks, block_bytes]")
+    _check_type(type_id0, "type_id0")
+    _check_type(type_id1, "type_id1")
+    uses_iq2 = type_id0 == 0 or type_id1 == 0
+    uses_iq1 = type_id0 == 2 or type_id1 == 2
+    _check(not (uses_iq2 and uses_iq1), "paired GEMM cannot mix iq2_xxs and iq1_m because they require different grids")
+    _check(row_elems0 > 0 and row_elems1 > 0, "row_elems must be positive")
+    _check(row_elems0 == row_elems1, "paired GGUF GEMM requires matching input dimensions")
+    _check(x.size(-1) == row_elems0, "inner dimension mismatch")
+    _check(blocks0.size(0) == blocks1.size(0), "paired blocks must have same output rows")
+    _check(blocks0.size(1) * 256 >= row_elems0 and blocks1.size(1) * 256 >= row_elems1, "blocks do not cover row_elems")
+    _check(blocks0.size(2) == GGUF_BLOCK_BYTES[type_id0], "unexpected blocks0 GGUF block size")
+    _check(blocks1.size(2) == GGUF_BLOCK_BYTES[type_id1], "unexpected blocks1 GGUF block size")
+    _check(x.is_cuda and blocks0.is_cuda and blocks1.is_cuda, "x and blocks must be CUDA tensors")
+    _check(x.is_contiguous() and blocks0.is_contiguous() and blocks1.is_contiguous(), "x and blocks must be contiguous")
+    _check(blocks0.dtype == torch.uint8, "blocks0 has unexpected dtype")
+    _check(blocks1.dtype == torch.uint8, "blocks1 has unexpected dtype")
+    _check_x(x)
+    _check(blocks0.size(1) == blocks1.size(1), "paired blocks must have the same number of blocks per row")
+    if uses_iq2:
+        _check_grid(signed_grid, 0, "signed_grid")
+    elif uses_iq1:
+        _check_grid(signed_grid, 2, "signed_grid")
+    rows = x.numel() // row_elems0
+    n = blocks0.size(0)
+    y = torch.empty(2, *x.shape[:-1], n, dtype=out_dtype, device=x.device)
+    if rows == 0 or n == 0:
+        return y
+    lib = _lib()
+    with torch.cuda.device(x.device):
+        ws_bytes = lib.pllm_gguf_quant_gemm_workspace_bytes(type_id0, rows, row_elems0, n, blocks0.size(1))
+        ws = _workspace(ws_bytes, x.device)
+        st = lib.pllm_gguf_quant_gemm_pair(x.data_ptr(), _DTYPE_CODE[x.dtype], blocks0.data_ptr(), type_id0, blocks1.data_ptr(), type_id1,
+                                           y.data_ptr(), _DTYPE_CODE[out_dtype], rows, row_elems0, n, blocks0.size(1),
+                                           ws.data_ptr(), ws_bytes, _stream(x.device))
+    _ffi.check(st, "gguf_quant_gemm_pair_forward")
+    return y
+
+
+# ---- routed experts --------------------------------------------------------------------------------
+
+_MOE_TYPES = (0, 1, 2)   # iq2_xxs, q2_k, iq1_m: the types the fused expert kernels read
+
+
+def _grids_ok(grid, type_ids, name: str) -> None:
+    """The reference takes ONE grid tensor and refuses to mix iq2_xxs with iq1_m
+    (src/csrc/cuda_kernel.cpp:717-722).  Passing a tuple/list of grids lifts that limit: one entry
+    per codebook type in use, checked like the reference checks its single grid."""
+    need = sorted({t for t in type_ids if t in (0, 2)})
+    if isinstance(grid, (tuple, list)):
+        _check(len(grid) >= len(need), f"{name}: one grid per codebook type in use is required")
+        for g, t in zip(grid, need):
+            _check_grid(g, t, name)
+        return
+    _check(len(need) <= 1, "grouped GGUF kernel cannot mix iq2_xxs and iq1_m because they require different grids")
+    if need:
+        _check_grid(grid, need[0], name)
+
+
+def _moe_call(name, x, tokens, route_tokens, route_experts, seg_starts, route_weights, w1, w3, w2, w13_type, w2_type, swiglu_limit):
+    dim, inter, n_experts, routes = x.size(-1), w1.size(1), w1.size(0), route_weights.numel()
+    y = torch.empty(tokens, dim, dtype=torch.float32, device=x.device)
+    lib = _lib()
+    with torch.cuda.device(x.device):
+        ws_bytes = lib.pllm_gguf_moe_workspace_bytes(tokens, routes, dim, inter)
+        ws = _workspace(ws_bytes, x.device)
+        st = lib.pllm_gguf_moe_forward(
+            x.data_ptr(), _DTYPE_CODE[x.dtype], tokens, dim, inter,
+            None if route_tokens is None else route_tokens.data_ptr(),
+            None if route_experts is None else route_experts.data_ptr(),
+            None if seg_starts is None else seg_starts.data_ptr(), n_experts,
+            route_weights.data_ptr(), routes, w1.data_ptr(), w3.data_ptr(), w13_type, w2.data_ptr(), w2_type,
+            float(swiglu_limit), y.data_ptr(), ws.data_ptr(), ws_bytes, _stream(x.device))
+    _ffi.check(st, name)
+    return y
+
+
+def gguf_moe_prefill_grouped_forward(x, route_tokens, route_weights_sorted, seg_starts, w1_blocks, w3_blocks, w2_blocks,
+                                     w1_row_elems, w1_type_id, w3_row_elems, w3_type_id, w2_row_elems, w2_type_id,
+                                     signed_grid, swiglu_limit) -> torch.Tensor:
+    """src/csrc/cuda_kernel.cpp:689-767: float32 [T, D]."""
+    w1_type_id, w3_type_id, w2_type_id = int(w1_type_id), int(w3_type_id), int(w2_type_id)
+    _check(x.dim() == 2, "x must have shape [T, D]")
+    _check(route_tokens.dim() == 1, "route_tokens must have shape [R]")
+    _check(route_weights_sorted.dim() == 1, "route_weights_sorted must have shape [R]")
+    _check(seg_starts.dim() == 1, "seg_starts must have shape [E + 1]")
+    _check(w1_blocks.dim() == 4 and w3_blocks.dim() == 4 and w2_blocks.dim() == 4, "GGUF blocks must have shape [E, N, K_blocks, block_bytes]")
+    _check(route_tokens.size(0) == route_weights_sorted.size(0), "route count mismatch")
+    _check(seg_starts.size(0) == w1_blocks.size(0) + 1, "seg_starts/expert count mismatch")
+    _check(w1_blocks.size(0) == w3_blocks.size(0) == w2_blocks.size(0), "expert count mismatch")
+    _check(w1_blocks.size(2) * 256 >= w1_row_elems and w3_blocks.size(2) * 256 >= w3_row_elems and w2_blocks.size(2) * 256 >= w2_row_elems,
+           "blocks do not cover row_elems")
+    for t, nm in ((w1_type_id, "w1"), (w3_type_id, "w3"), (w2_type_id, "w2")):
+        _check(t in GGUF_BLOCK_BYTES, f"unsupported {nm} GGUF type: {t}")
+        _check(t in _MOE_TYPES, f"{nm} GGUF type {t} has no fused expert kernel in this build")
+    _grids_ok(signed_grid, (w1_type_id, w3_type_id, w2_type_id), "signed_grid")
+    _check(w1_type_id == w3_type_id, "w1 and w3 must share a GGUF type in this build")
+    _check(w1_blocks.size(3) == GGUF_BLOCK_BYTES[w1_type_id], "unexpected w1 GGUF block size")
+    _check(w3_blocks.size(3) == GGUF_BLOCK_BYTES[w3_type_id], "unexpected w3 GGUF block size")
+    _check(w2_blocks.size(3) == GGUF_BLOCK_BYTES[w2_type_id], "unexpected w2 GGUF block size")
+    _check(w1_row_elems == x.size(1) and w3_row_elems == x.size(1), "w1/w3 input dimension mismatch")
+    _check(w2_row_elems == w1_blocks.size(1) and w1_blocks.size(1) == w3_blocks.size(1), "w2 input dimension mismatch")
+    _check(w2_blocks.size(1) == x.size(1), "w2 output dimension mismatch")
+    _check(x.is_cuda and route_tokens.is_cuda and route_weights_sorted.is_cuda and seg_starts.is_cuda, "route tensors must be CUDA tensors")
+    _check(w1_blocks.is_cuda and w3_blocks.is_cuda and w2_blocks.is_cuda, "GGUF blocks must be CUDA tensors")
+    _check(x.is_contiguous() and route_tokens.is_contiguous() and route_weights_sorted.is_contiguous() and seg_starts.is_contiguous(),
+           "route tensors must be contiguous")
+    _check(w1_blocks.is_contiguous() and w3_blocks.is_contiguous() and w2_blocks.is_contiguous(), "GGUF blocks must be contiguous")
+    _check_x(x)
+    _check(route_tokens.dtype == torch.int64, "route_tokens must be int64")
+    _check(route_weights_sorted.dtype == torch.float32, "route_weights_sorted must be float32")
+    _check(seg_starts.dtype in (torch.int32, torch.int64), "seg_starts must be int32 or int64")
+    for b, nm in ((w1_blocks, "w1_blocks"), (w3_blocks, "w3_blocks"), (w2_blocks, "w2_blocks")):
+        _check(b.dtype == torch.uint8, f"{nm} has unexpected dtype")
+    seg32 = seg_starts if seg_starts.dtype == torch.int32 else seg_starts.to(torch.int32)
+    return _moe_call("gguf_moe_prefill_grouped_forward", x, x.size(0), route_tokens, None, seg32, route_weights_sorted,
+                     w1_blocks, w3_blocks, w2_blocks, w1_type_id, w2_type_id, swiglu_limit)
+
+
+def _single_token_checks(x, route_slots, route_weights, w1, w3, w2):
+    _check(x.dim() == 2 and x.size(0) == 1, "x must have shape [1, D]")
+    _check(route_slots.dim() == 1, "route_slots must have shape [K]")
+    _check(route_weights.dim() == 1, "route_weights must have shape [K]")
+    _check(route_slots.size(0) == route_weights.size(0), "route_slots/route_weights length mismatch")
+    _check(w1.dim() == 4 and w3.dim() == 4 and w2.dim() == 4, "GGUF blocks must have shape [E, N, K_blocks, block_bytes]")
+    _check(w1.size(0) == w3.size(0) == w2.size(0), "expert count mismatch")
+    _check(w1.size(1) == w3.size(1), "w1/w3 inter_dim mismatch")
+    _check(w1.size(2) == w3.size(2), "w1/w3 block count mismatch")
+    _check(w1.size(2) * 256 >= x.size(1), "w1/w3 blocks do not cover x dim")
+    _check(w2.size(1) == x.size(1), "w2 output dimension mismatch")
+    _check(w2.size(2) * 256 >= w1.size(1), "w2 blocks do not cover inter dim")
+    _check(x.is_cuda and route_slots.is_cuda and route_weights.is_cuda, "x/route tensors must be CUDA tensors")
+    _check(w1.is_cuda and w3.is_cuda and w2.is_cuda, "GGUF blocks must be CUDA tensors")
+    _check(x.is_contiguous() and route_slots.is_contiguous() and route_weights.is_contiguous(), "x/route tensors must be contiguous")
+    _check(w1.is_contiguous() and w3.is_contiguous() and w2.is_contiguous(), "GGUF blocks must be contiguous")
+    _check_x(x)
+    _check(route_slots.dtype == torch.int64, "route_slots must be int64")
+    _check(route_weights.dtype == torch.float32, "route_weights must be float32")
+    for b, nm in ((w1, "w1_blocks"), (w3, "w3_blocks"), (w2, "w2_blocks")):
+        _check(b.dtype == torch.uint8, f"{nm} has unexpected dtype")
+
+
+_TYPE_OF_BLOCK_BYTES = {66: 0, 84: 1, 56: 2}
+
+
+def gguf_moe_single_token_forward(x, route_slots, route_weights, w1_blocks, w3_blocks, w2_blocks, swiglu_limit) -> torch.Tensor:
+    """Single-token routed experts for any mix of IQ2_XXS / Q2_K / IQ1_M matrices (types read off the
+    block sizes): the case the reference cannot express because its operators take one grid tensor."""
+    _single_token_checks(x, route_slots, route_weights, w1_blocks, w3_blocks, w2_blocks)
+    _check(w1_blocks.size(3) == w3_blocks.size(3) and w1_blocks.size(3) in _TYPE_OF_BLOCK_BYTES, "w1/w3 must be IQ2_XXS, Q2_K or IQ1_M blocks")
+    _check(w2_blocks.size(3) in _TYPE_OF_BLOCK_BYTES, "w2 must be IQ2_XXS, Q2_K or IQ1_M blocks")
+    return _moe_call("gguf_moe_single_token_forward", x, 1, None, route_slots, None, route_weights, w1_blocks, w3_blocks, w2_blocks,
+                     _TYPE_OF_BLOCK_BYTES[w1_blocks.size(3)], _TYPE_OF_BLOCK_BYTES[w2_blocks.size(3)], swiglu_limit)
+
+
+def gguf_moe_single_token_iq2_q2k_forward(x, route_slots, route_weights, w1_blocks, w3_blocks, w2_blocks, signed_grid, swiglu_limit) -> torch.Tensor:
+    """src/csrc/cuda_kernel.cpp:769-818: float32 [1, D]."""
+    _single_token_checks(x, route_slots, route_weights, w1_blocks, w3_blocks, w2_blocks)
+    _check(w1_blocks.size(3) == 66 and w3_blocks.size(3) == 66, "w1/w3 must be IQ2_XXS blocks")
+    _check(w2_blocks.size(3) in (66, 84), "w2 must be IQ2_XXS or Q2_K blocks")
+    _check(signed_grid.is_cuda, "signed_grid must be CUDA for IQ2_XXS")
+    _check(signed_grid.is_contiguous(), "signed_grid must be contiguous")
+    _check(signed_grid.dtype == torch.int8, "signed_grid has unexpected dtype")
+    _check(signed_grid.numel() == 256 * 128 * 8, "signed_grid must contain 256*128*8 entries")
+    return _moe_call("gguf_moe_single_token_iq2_q2k_forward", x, 1, None, route_slots, None, route_weights, w1_blocks, w3_blocks, w2_blocks,
+                     0, _TYPE_OF_BLOCK_BYTES[w2_blocks.size(3)], swiglu_limit)
+
+
+def gguf_moe_single_token_iq1m_forward(x, route_slots, route_weights, w1_blocks, w3_blocks, w2_blocks, iq1_grid, swiglu_limit) -> torch.Tensor:
+    """src/csrc/cuda_kernel.cpp:820-865: float32 [1, D]."""
+    _single_token_checks(x, route_slots, route_weights, w1_blocks, w3_blocks, w2_blocks)
+    _check(w1_blocks.size(3) == 56 and w3_blocks.size(3) == 56 and w2_blocks.size(3) == 56, "w1/w3/w2 must be IQ1_M blocks")
+    _check_grid(iq1_grid, 2, "iq1_grid")
+    return _moe_call("gguf_moe_single_token_iq1m_forward", x, 1, None, route_slots, None, route_weights, w1_blocks, w3_blocks, w2_blocks,
+                     2, 2, swiglu_limit)
+
+
+def moe_group_routes(indices, weights, experts_start_idx, n_local_experts):
+    """src/csrc/cuda_kernel.cpp:1228-1242: [local_ids int64, route_tokens int64 [R], route_weights float32 [R], seg_starts int32 [E+1]].
+    Like the reference it reads the route count back to size the outputs (one host sync)."""
+    _check(indices.dim() == 2, "indices must have shape [T, K]")
+    _check(weights.dim() == 2, "weights must have shape [T, K]")
+    _check(indices.shape == weights.shape, "indices/weights shape mismatch")
+    _check(indices.is_cuda and weights.is_cuda, "indices and weights must be CUDA tensors")
+    _check(indices.is_contiguous() and weights.is_contiguous(), "indices and weights must be contiguous")
+    _check(weights.dtype == torch.float32, "weights must be float32")
+    _check(indices.dtype in (torch.int64, torch.int32), "indices must be int64 or int32")
+    n_local = int(n_local_experts)
+    _check(n_local > 0, "n_local_experts must be positive")
+    t, k = indices.shape
+    dev = indices.device
+    seg = torch.empty(n_local + 1, dtype=torch.int32, device=dev)
+    cap = max(t * k, 1)
+    toks = torch.empty(cap, dtype=torch.int64, device=dev)
+    wts = torch.empty(cap, dtype=torch.float32, device=dev)
+    exps = torch.empty(cap, dtype=torch.int32, device=dev)
+    if t * k:
+        with torch.cuda.device(dev):
+            st = _lib().pllm_moe_group_routes(indices.data_ptr(), int(indices.dtype == torch.int64), weights.data_ptr(), t, k,
+                                              int(experts_start_idx), n_local, seg.data_ptr(), toks.data_ptr(), wts.data_ptr(),
+                                              exps.data_ptr(), _stream(dev))
+        _ffi.check(st, "moe_group_routes")
+    else:
+        seg.zero_()
+    routes = int(seg[-1].item())
+    local_ids = (seg[1:] > seg[:-1]).nonzero().flatten().to(torch.long)
+    return [local_ids, toks[:routes], wts[:routes], seg]
+
+
+def gguf_single_token_route_slots(indices, weights, experts_start_idx, n_local_experts):
+    """Host-side compaction of one token's routes (src/csrc/cuda_kernel.cpp:1244-1327):
+    [local_ids (CPU int64), route_tokens, route_weights, route_slots, compact_starts (int32)]."""
+    _check(indices.dim() == 2 and indices.size(0) == 1, "indices must have shape [1, K]")
+    _check(weights.dim() == 2 and weights.size(0) == 1, "weights must have shape [1, K]")
+    _check(indices.size(1) == weights.size(1), "indices/weights shape mismatch")
+    _check(indices.is_cuda and weights.is_cuda, "indices and weights must be CUDA tensors")
+    _check(indices.is_contiguous() and weights.is_contiguous(), "indices and weights must be contiguous")
+    _check(weights.dtype == torch.float32, "weights must be float32")
+    _check(indices.dtype in (torch.int64, torch.int32), "indices must be int64 or int32")
+    _check(int(n_local_experts) > 0, "n_local_experts must be positive")
+    by_local: dict[int, list[int]] = {}
+    for pos, ex in enumerate(indices.view(-1).tolist()):
+        local = int(ex) - int(experts_start_idx)
+        if 0 <= local < int(n_local_experts):
+            by_local.setdefault(local, []).append(pos)
+    local_ids, slots, positions, starts = [], [], [], [0]
+    for slot, local in enumerate(sorted(by_local)):
+        local_ids.append(local)
+        for pos in by_local[local]:
+            slots.append(slot)
+            positions.append(pos)
+        starts.append(len(slots))
+    dev = indices.device
+    route_positions = torch.tensor(positions, dtype=torch.int64, device=dev)
+    return [torch.tensor(local_ids, dtype=torch.int64), torch.zeros(len(slots), dtype=torch.int64, device=dev),
+            weights.view(-1).index_select(0, route_positions), torch.tensor(slots, dtype=torch.int64, device=dev),
+            torch.tensor(starts, dtype=torch.int32, device=dev)]

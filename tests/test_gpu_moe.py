@@ -1,0 +1,187 @@
+"""GPU parity of the routed-expert operators, route grouping and the paired projection."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import gguf_oracle as O
+from pocketllm_amd import block_codec as C, codebooks
+from pocketllm_amd.cuda_loader import load_cuda_kernel
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+TOL = 1e-3
+GEN = {"iq2_xxs": C.random_iq2_xxs, "iq1_m": C.random_iq1_m}
+
+
+@pytest.fixture(scope="module")
+def mod():
+    m = load_cuda_kernel()
+    assert m is not None and torch.cuda.is_available()
+    return m
+
+
+def _expert_blocks(rng, type_name, e, n, k):
+    if type_name == "q2_k":
+        w = (rng.standard_normal((e * n, k)) * 0.05).astype(np.float32)
+        return C.quantize_q2_k(w).reshape(e, n, k // 256, 84)
+    # scales sized so that the hidden activations stay O(1)
+    return GEN[type_name](rng, e, n, (k + 255) // 256, d_range=(0.002, 0.006))
+
+
+def _route(rng, t, e, topk):
+    logits = rng.standard_normal((t, e)).astype(np.float32)
+    p = np.exp(logits - logits.max(axis=1, keepdims=True))
+    p /= p.sum(axis=1, keepdims=True)
+    idx = np.argsort(-p, axis=1)[:, :topk].astype(np.int64)
+    w = np.take_along_axis(p, idx, axis=1)
+    return idx, (w / w.sum(axis=1, keepdims=True)).astype(np.float32)
+
+
+@pytest.mark.parametrize("t13,t2", [("iq2_xxs", "iq1_m"), ("iq2_xxs", "iq2_xxs"), ("iq2_xxs", "q2_k"), ("iq1_m", "iq1_m")])
+@pytest.mark.parametrize("limit", [0.0, 0.6])
+def test_single_token_experts(mod, t13, t2, limit):
+    rng = np.random.default_rng(100 + len(t13) + len(t2))
+    e, d, inter, topk = 8, 512, 768, 4
+    w1 = _expert_blocks(rng, t13, e, inter, d)
+    w3 = _expert_blocks(rng, t13, e, inter, d)
+    w2 = _expert_blocks(rng, t2, e, d, inter)
+    idx, wts = _route(rng, 1, e, topk)
+    x = torch.from_numpy(rng.standard_normal((1, d)).astype(np.float32)).to(DEV).to(torch.bfloat16)
+    slots = torch.from_numpy(idx[0]).to(DEV)
+    rw = torch.from_numpy(wts[0]).to(DEV)
+    dw1, dw3, dw2 = (torch.from_numpy(a).to(DEV) for a in (w1, w3, w2))
+    print(f"case single {t13}/{t2} limit={limit}", flush=True)
+    y = mod.gguf_moe_single_token_forward(x, slots, rw, dw1, dw3, dw2, limit)
+    torch.cuda.synchronize()
+    want = O.moe_forward(x.float().cpu().numpy(), np.zeros(topk, dtype=np.int64), wts[0], idx[0], w1, w3, w2, t13, t13, t2, limit)
+    assert y.dtype == torch.float32 and tuple(y.shape) == (1, d)
+    assert O.rel_l2(y.cpu().numpy(), want) <= TOL
+    # the reference-named operators where they apply
+    if t13 == "iq2_xxs" and t2 in ("iq2_xxs", "q2_k"):
+        grid = codebooks.get_iq2xxs_signed_grid_tensor().to(DEV)
+        y2 = mod.gguf_moe_single_token_iq2_q2k_forward(x, slots, rw, dw1, dw3, dw2, grid, limit)
+        assert torch.equal(y2, y)
+    if t13 == "iq1_m" and t2 == "iq1_m":
+        y2 = mod.gguf_moe_single_token_iq1m_forward(x, slots, rw, dw1, dw3, dw2, codebooks.get_iq1_grid_tensor().to(DEV), limit)
+        assert torch.equal(y2, y)
+
+
+@pytest.mark.parametrize("t13,t2", [("iq2_xxs", "iq1_m"), ("iq2_xxs", "q2_k")])
+def test_grouped_experts_and_route_grouping(mod, t13, t2):
+    rng = np.random.default_rng(7)
+    e, d, inter, topk, t = 12, 512, 512, 3, 9
+    w1 = _expert_blocks(rng, t13, e, inter, d)
+    w3 = _expert_blocks(rng, t13, e, inter, d)
+    w2 = _expert_blocks(rng, t2, e, d, inter)
+    idx, wts = _route(rng, t, e + 4, topk)                 # experts 0..15, local window 2..13
+    start = 2
+    x = torch.from_numpy(rng.standard_normal((t, d)).astype(np.float32)).to(DEV).to(torch.bfloat16)
+    local_ids, toks, rws, seg = mod.moe_group_routes(torch.from_numpy(idx).to(DEV), torch.from_numpy(wts).to(DEV), start, e)
+    o_ids, o_toks, o_rws, o_seg = O.group_routes(idx, wts, start, e)
+    assert local_ids.cpu().tolist() == o_ids.tolist()
+    np.testing.assert_array_equal(seg.cpu().numpy(), o_seg)
+    np.testing.assert_array_equal(toks.cpu().numpy(), o_toks)          # stable order: same as the oracle's
+    np.testing.assert_array_equal(rws.cpu().numpy(), o_rws)
+    # int32 indices give the same grouping
+    _, toks32, _, seg32 = mod.moe_group_routes(torch.from_numpy(idx.astype(np.int32)).to(DEV), torch.from_numpy(wts).to(DEV), start, e)
+    assert torch.equal(toks32, toks) and torch.equal(seg32, seg)
+
+    grids = (codebooks.get_iq2xxs_signed_grid_tensor().to(DEV), codebooks.get_iq1_grid_tensor().to(DEV))
+    dw1, dw3, dw2 = (torch.from_numpy(a).to(DEV) for a in (w1, w3, w2))
+    tid = O.TYPE_IDS
+    y = mod.gguf_moe_prefill_grouped_forward(x, toks, rws, seg, dw1, dw3, dw2, d, tid[t13], d, tid[t13], inter, tid[t2], grids, 0.0)
+    torch.cuda.synchronize()
+    route_experts = np.repeat(np.arange(e), np.diff(o_seg))
+    want = O.moe_forward(x.float().cpu().numpy(), o_toks, o_rws, route_experts, w1, w3, w2, t13, t13, t2, 0.0)
+    assert O.rel_l2(y.cpu().numpy(), want) <= TOL
+    # run-to-run bitwise determinism (the reference's atomics cannot promise this)
+    y2 = mod.gguf_moe_prefill_grouped_forward(x, toks, rws, seg.to(torch.int64), dw1, dw3, dw2, d, tid[t13], d, tid[t13], inter, tid[t2], grids, 0.0)
+    assert torch.equal(y, y2)
+    if t2 == "iq1_m":
+        with pytest.raises(RuntimeError, match="cannot mix iq2_xxs and iq1_m"):
+            mod.gguf_moe_prefill_grouped_forward(x, toks, rws, seg, dw1, dw3, dw2, d, 0, d, 0, inter, 2, grids[0], 0.0)
+
+
+def test_no_routes_gives_zeros(mod):
+    e, d, inter = 2, 256, 256
+    z = torch.zeros(e, inter, 1, 66, dtype=torch.uint8, device=DEV)
+    z2 = torch.zeros(e, d, 1, 66, dtype=torch.uint8, device=DEV)
+    x = torch.randn(3, d, device=DEV)
+    y = mod.gguf_moe_prefill_grouped_forward(x, torch.empty(0, dtype=torch.int64, device=DEV), torch.empty(0, device=DEV),
+                                             torch.zeros(e + 1, dtype=torch.int32, device=DEV), z, z, z2, d, 0, d, 0, inter, 0,
+                                             codebooks.get_iq2xxs_signed_grid_tensor().to(DEV), 0.0)
+    assert tuple(y.shape) == (3, d) and float(y.abs().max()) == 0.0
+
+
+def test_baseline_config_single_token_shapes(mod):
+    """BASELINE config 5 at T = 1 with 16 of the 256 experts materialised (routing only touches 8)."""
+    rng = np.random.default_rng(1005)
+    e, d, inter, topk = 16, 3072, 1536, 8
+    w1 = _expert_blocks(rng, "iq2_xxs", e, inter, d)
+    w3 = _expert_blocks(rng, "iq2_xxs", e, inter, d)
+    w2 = _expert_blocks(rng, "iq1_m", e, d, inter)
+    idx, wts = _route(rng, 1, e, topk)
+    x = torch.from_numpy(rng.standard_normal((1, d)).astype(np.float32)).to(DEV).to(torch.bfloat16)
+    y = mod.gguf_moe_single_token_forward(x, torch.from_numpy(idx[0]).to(DEV), torch.from_numpy(wts[0]).to(DEV),
+                                          *(torch.from_numpy(a).to(DEV) for a in (w1, w3, w2)), 0.0)
+    torch.cuda.synchronize()
+    want = O.moe_forward(x.float().cpu().numpy(), np.zeros(topk, dtype=np.int64), wts[0], idx[0], w1, w3, w2, "iq2_xxs", "iq2_xxs", "iq1_m", 0.0)
+    assert O.rel_l2(y.cpu().numpy(), want) <= TOL
+
+
+def test_route_slots_host_compaction(mod):
+    idx = torch.tensor([[9, 3, 12, 4, 3]], device=DEV)
+    w = torch.tensor([[0.1, 0.2, 0.3, 0.25, 0.15]], device=DEV)
+    local_ids, toks, rw, slots, starts = mod.gguf_single_token_route_slots(idx, w, 3, 8)     # local window 3..10
+    assert local_ids.tolist() == [0, 1, 6] and not local_ids.is_cuda
+    assert slots.cpu().tolist() == [0, 0, 1, 2] and starts.cpu().tolist() == [0, 2, 3, 4]
+    assert toks.cpu().tolist() == [0, 0, 0, 0]
+    np.testing.assert_allclose(rw.cpu().numpy(), [0.2, 0.15, 0.25, 0.1])
+
+
+def test_paired_projection(mod):
+    rng = np.random.default_rng(21)
+    n, k = 48, 1024
+    wa = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
+    wb = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
+    x = torch.randn(1, 3, k, device=DEV, dtype=torch.bfloat16)
+    grid = torch.empty(0, dtype=torch.int8, device=DEV)
+    for tid, enc in ((3, C.quantize_q4_k), (4, C.quantize_q5_k)):
+        ba, bb = torch.from_numpy(enc(wa)).to(DEV), torch.from_numpy(enc(wb)).to(DEV)
+        y = mod.gguf_quant_gemm_pair_forward(x, ba, k, tid, bb, k, tid, grid)
+        assert y.dtype == torch.bfloat16 and tuple(y.shape) == (2, 1, 3, n)
+        # pair == the two separate calls, bit for bit (the reference's own test: tests/test_gguf_quantized_ops_cuda.py:83-92)
+        assert torch.equal(y[0], mod.gguf_quant_gemm_prefill_forward(x, ba, k, tid, grid))
+        assert torch.equal(y[1], mod.gguf_quant_gemm_prefill_forward(x, bb, k, tid, grid))
+    with pytest.raises(RuntimeError, match="paired blocks must have same output rows"):
+        mod.gguf_quant_gemm_pair_forward(x, ba, k, 4, bb[:8], k, 4, grid)
+
+
+def test_linear_modules(mod):
+    from pocketllm_amd.quantized_ops import Q8_0GGUFLinear, QuantizedGGUFEmbedding, QuantizedGGUFLinear
+    from pocketllm_amd.quantized_tensor import QuantizedGGUFTensor
+    rng = np.random.default_rng(2)
+    w = (rng.standard_normal((64, 512)) * 0.02).astype(np.float32)
+    blocks = C.quantize_q5_k(w)
+    t = QuantizedGGUFTensor.from_blocks(torch.from_numpy(blocks).to(DEV), "q5_k", 512, source_name="proj")
+    lin = QuantizedGGUFLinear(t)
+    assert (lin.in_dim, lin.out_dim, lin.row_start) == (512, 64, 0)
+    ref = O.dequant_rows(blocks, "q5_k")
+    for shape in ((1, 512), (5, 512), (2, 3, 512)):
+        x = torch.randn(*shape, device=DEV, dtype=torch.float16)
+        y = lin(x)
+        assert y.dtype == torch.float16 and tuple(y.shape) == shape[:-1] + (64,)
+        want = O.matmul_f(x.float().cpu().numpy().reshape(-1, 512), ref).reshape(shape[:-1] + (64,))
+        assert np.abs(y.float().cpu().numpy() - want).max() < 2e-2       # the reference's bound for this wrapper
+    with pytest.raises(ValueError, match="expected input dim 512"):
+        lin(torch.randn(1, 256, device=DEV))
+    y0, y1 = QuantizedGGUFLinear.pair(lin, lin, torch.randn(1, 512, device=DEV, dtype=torch.float16))
+    assert torch.equal(y0, y1)
+    emb = QuantizedGGUFEmbedding(t)
+    assert emb.dim == 512 and tuple(emb(torch.tensor([1, 2, 3], device=DEV, dtype=torch.int32)).shape) == (3, 512)
+    q8 = Q8_0GGUFLinear(torch.from_numpy(C.pack_q8_0(w)).to(DEV), 512, source_name="q8")
+    x = torch.randn(2, 512, device=DEV, dtype=torch.float16)
+    want = O.matmul_f(x.float().cpu().numpy(), O.dequant_rows(C.pack_q8_0(w), "q8_0"))
+    assert np.abs(q8(x).float().cpu().numpy() - want).max() < 2e-2
+    with pytest.raises(ValueError, match="q8_0 blocks must be"):
+        Q8_0GGUFLinear(torch.zeros(4, 2, 33, dtype=torch.uint8, device=DEV), 64)
