@@ -1,15 +1,21 @@
 #!/usr/bin/env python3
 """Benchmark of the raw-block quantized matmul path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--eager] [--no-extra] [--no-cpu-baseline]
 
 A step is one pass of the decode matvec over the Q4_K / Q5_K weights of the Qwen3-27B-like shapes
 (N x K = 5120 x 5120 and 17408 x 5120, one bf16 activation row): four operator calls, each on the
-next copy in a ring of weight copies larger than the 256 MB last-level cache, so the bytes come from
-HBM.  Inputs are synthetic (seeded N(0, 0.02) weights quantized by this package's encoders, N(0, 1)
-activations) and resident in HBM before the timed region.  The one JSON line printed at the end
-carries whole-step throughput (weight bytes / time), the roofline figures of the dominant kernel
-measured with HIP events on the launch stream, and the CPU dequantize-then-matmul baseline.
+next copy in a ring of weight copies that together exceed the 256 MB last-level cache several
+times, so the bytes come from HBM.  Inputs are synthetic (seeded N(0, 0.02) weights quantized by
+this package's encoders, N(0, 1) activations) and resident in HBM before the timed region.  Steps
+are replayed from one HIP graph that holds a step for every ring slot, so that the Python wrapper is
+not what is timed; --eager times the plain operator calls instead.  --pmc-pass runs only a few
+launches of the dominant kernel and of a plain copy of the same size: the short program the
+rocprofv3 counter passes under profiles/ are taken from.
+
+The one JSON line printed at the end carries whole-step throughput (weight bytes / time), the
+roofline figures of the dominant kernel measured with HIP events on the launch stream, the CPU
+dequantize-then-matmul baseline, and a table of the other formats of the path (`cases`).
 """
 from __future__ import annotations
 
@@ -23,7 +29,7 @@ import numpy as np
 import torch
 
 HBM_PEAK_GBS = 8000.0
-RING_BYTES = 640 << 20
+RING = 12                     # weight copies per case
 
 CASES = [  # (type name, type id, N, K)
     ("q4_k", 3, 5120, 5120),
@@ -33,34 +39,65 @@ CASES = [  # (type name, type id, N, K)
 ]
 DOMINANT = 3   # index into CASES: the launch the roofline object describes
 
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by
+# what the same counters read for a plain copy of known size (profiles/q5k_matvec_17408x5120_counters.md)
+TRAFFIC_FILE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "traffic.json")
+
 
 def _encoders():
     from pocketllm_amd import block_codec as C
-    return {"q4_k": C.quantize_q4_k, "q5_k": C.quantize_q5_k}
+    return {"q4_k": C.quantize_q4_k, "q5_k": C.quantize_q5_k, "q2_k": C.quantize_q2_k}
 
 
-def build_case(name, n, k, seed, device):
-    rng = np.random.default_rng(seed)
-    w = (rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02))
-    blocks = _encoders()[name](w)
+def ring_of(blocks: np.ndarray, device, copies: int = RING):
     first = torch.from_numpy(blocks).to(device)
-    copies = max(2, -(-RING_BYTES // first.numel()))
-    ring = [first] + [first.clone() for _ in range(copies - 1)]
-    return blocks, ring
+    return [first] + [first.clone() for _ in range(copies - 1)]
 
 
-def event_time_us(fn, ring, iters, warm):
+def event_time_us(fn, slots, iters, warm=5):
+    """Average duration of fn(slot) over `iters` back-to-back calls, HIP events on the current stream."""
     for i in range(warm):
-        fn(ring[i % len(ring)])
+        fn(i % slots)
     torch.cuda.synchronize()
     e0 = torch.cuda.Event(enable_timing=True)
     e1 = torch.cuda.Event(enable_timing=True)
     e0.record()
     for i in range(iters):
-        fn(ring[i % len(ring)])
+        fn(i % slots)
     e1.record()
     torch.cuda.synchronize()
     return e0.elapsed_time(e1) * 1e3 / iters
+
+
+def capture(fn, slots):
+    """One HIP graph holding fn(0) .. fn(slots - 1); returns (replay, True), or (None, False) if capture fails."""
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for s in range(slots):
+                fn(s)                                   # warm allocator and kernels on a side stream first
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for s in range(slots):
+                fn(s)
+        torch.cuda.synchronize()
+        return g.replay, True
+    except Exception as exc:                             # pragma: no cover - depends on the runtime
+        print(f"bench.py: graph capture failed ({exc!r}); timing eager calls", file=sys.stderr)
+        torch.cuda.synchronize()
+        return None, False
+
+
+def time_calls_us(fn, slots, iters, eager=False):
+    """Average duration of one fn(slot) call: a graph of `slots` calls replayed, or eager calls."""
+    replay, graphed = (None, False) if eager else capture(fn, slots)
+    if graphed:
+        reps = max(1, iters // slots)
+        return event_time_us(lambda _s: replay(), 1, reps, warm=2) / slots, True
+    return event_time_us(fn, slots, iters), False
 
 
 def cpu_baseline(blocks: np.ndarray, type_name: str, k: int, x: np.ndarray, budget_s: float = 15.0):
@@ -75,29 +112,115 @@ def cpu_baseline(blocks: np.ndarray, type_name: str, k: int, x: np.ndarray, budg
         t0 = time.perf_counter()
         w = O.dequant_rows(blocks, type_name, k)
         t1 = time.perf_counter()
-        y = torch.nn.functional.linear(xt, torch.from_numpy(w))
+        torch.nn.functional.linear(xt, torch.from_numpy(w))
         t2 = time.perf_counter()
         times.append((t2 - t0, t1 - t0, t2 - t1))
     times = times[1:] if len(times) > 1 else times          # first call warms the page cache
     total = float(np.median([t[0] for t in times]))
     return {
-        "value": blocks.size / total / 1e9,
+        "value": round(blocks.size / total / 1e9, 4),
         "unit": "GB/s",
         "cores": int(torch.get_num_threads()),
         "kind": "port",
         "sample": (f"{type_name} {blocks.shape[0]}x{k} matvec, numpy block decode ({np.median([t[1] for t in times]) * 1e3:.0f} ms, "
                    f"one thread) + torch F.linear fp32 ({np.median([t[2] for t in times]) * 1e3:.1f} ms, {torch.get_num_threads()} threads), "
                    f"median of {len(times)} calls"),
-        "ms_per_call": total * 1e3,
-    }, y.numpy()
+        "ms_per_call": round(total * 1e3, 3),
+    }
+
+
+def extra_cases(mod, dev, iters):
+    """Other formats of the path, one line each (event-timed eager launches are launch-bound for the
+    small ones, so these replay graphs as well)."""
+    from pocketllm_amd import block_codec as C, codebooks
+    rng = np.random.default_rng(3003)
+    out = []
+    empty = torch.empty(0, dtype=torch.int8, device=dev)
+
+    def run(label, nbytes, fn, slots, extra=None):
+        us, graphed = time_calls_us(fn, slots, iters)
+        rec = {"case": label, "weight_bytes": int(nbytes), "us_per_call": round(us, 3), "gbs": round(nbytes / us / 1e3, 1),
+               "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4), "graph": graphed}
+        if extra:
+            rec.update(extra)
+        out.append(rec)
+
+    # Q8_0, BASELINE config 1 and the large shape
+    for n, k in ((4096, 4096), (17408, 5120)):
+        blocks = C.pack_q8_0((rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02)))
+        ring = ring_of(blocks, dev, max(2, min(RING, (1 << 30) // blocks.size)))
+        x = torch.randn(1, k, device=dev)
+        run(f"q8_0 matvec {n}x{k} T=1", blocks.size, lambda s, ring=ring, x=x, k=k: mod.q8_0_gemm_forward(x, ring[s], k), len(ring))
+        del ring
+    # Q2_K at the large shape
+    blocks = C.quantize_q2_k((rng.standard_normal((17408, 5120), dtype=np.float32) * np.float32(0.02)))
+    ring = ring_of(blocks, dev)
+    x = torch.randn(1, 5120, device=dev, dtype=torch.bfloat16)
+    run("q2_k matvec 17408x5120 T=1", blocks.size, lambda s, ring=ring, x=x: mod.gguf_quant_gemm_forward(x, ring[s], 5120, 1, empty), len(ring))
+    del ring
+    # FP8 E4M3 + 128x128 scales, BASELINE config 4 at T=1
+    codes, scale = C.quantize_fp8_block((rng.standard_normal((17408, 5120), dtype=np.float32) * np.float32(0.02)))
+    ring = ring_of(codes, dev, 8)
+    sc = torch.from_numpy(scale).to(dev)
+    run("fp8_e4m3 matvec 17408x5120 T=1", codes.size + scale.size * 4,
+        lambda s, ring=ring, x=x, sc=sc: mod.fp8_block_gemm_forward(x, ring[s], sc), len(ring))
+    del ring
+    # IQ2_XXS / IQ1_M dense matvec at the expert shapes stacked 64 experts high
+    for name, tid, n, k, gen, grid in (("iq2_xxs", 0, 64 * 1536, 3072, C.random_iq2_xxs, codebooks.get_iq2xxs_signed_grid_tensor().to(dev)),
+                                       ("iq1_m", 2, 64 * 3072, 1536, C.random_iq1_m, codebooks.get_iq1_grid_tensor().to(dev))):
+        blocks = gen(rng, n, k // 256)
+        ring = ring_of(blocks, dev)
+        xx = torch.randn(1, k, device=dev, dtype=torch.bfloat16)
+        run(f"{name} matvec {n}x{k} T=1", blocks.size,
+            lambda s, ring=ring, xx=xx, k=k, tid=tid, grid=grid: mod.gguf_quant_gemm_forward(xx, ring[s], k, tid, grid), len(ring))
+        del ring
+    # fused routed experts, BASELINE config 5 at T=1: 256 experts, top-8
+    e, d, inter = 256, 3072, 1536
+    w1 = torch.from_numpy(C.random_iq2_xxs(rng, e, inter, d // 256, d_range=(0.002, 0.006))).to(dev)
+    w3 = torch.from_numpy(C.random_iq2_xxs(rng, e, inter, d // 256, d_range=(0.002, 0.006))).to(dev)
+    w2 = torch.from_numpy(C.random_iq1_m(rng, e, d, inter // 256, d_range=(0.002, 0.006))).to(dev)
+    logits = torch.from_numpy(rng.standard_normal((RING, e)).astype(np.float32))
+    probs = torch.softmax(logits, dim=-1)
+    topw, topi = probs.topk(8, dim=-1)
+    topw = (topw / topw.sum(dim=-1, keepdim=True)).to(dev)
+    topi = topi.to(dev)
+    xm = torch.randn(1, d, device=dev, dtype=torch.bfloat16)
+    per_call = 8 * (2 * inter * (d // 256) * 66 + d * (inter // 256) * 56)
+    run("fused experts iq2_xxs gate/up + iq1_m down, 256 experts top-8, T=1", per_call,
+        lambda s: mod.gguf_moe_single_token_forward(xm, topi[s], topw[s], w1, w3, w2, 0.0), RING,
+        {"note": "each slot routes to a different random top-8 of the 256 resident experts (887 MB)"})
+    return out
+
+
+def pmc_pass(mod, dev) -> None:
+    from pocketllm_amd import _ffi
+    name, tid, n, k = CASES[DOMINANT]
+    rng = np.random.default_rng(1002 + DOMINANT)
+    blocks = _encoders()[name]((rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02)))
+    ring = ring_of(blocks, dev, 6)
+    x = torch.randn(1, k, device=dev, dtype=torch.bfloat16)
+    grid = torch.empty(0, dtype=torch.int8, device=dev)
+    nbytes = blocks.size & ~15
+    dst = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    lib = _ffi.load_library()
+    stream = torch.cuda.current_stream().cuda_stream
+    for i in range(6):
+        mod.gguf_quant_gemm_forward(x, ring[i], k, tid, grid)
+    for i in range(6):
+        lib.pllm_diag_stream_copy(ring[i].data_ptr(), dst.data_ptr(), nbytes, 2048, stream)
+    torch.cuda.synchronize()
+    print(json.dumps({"pmc_pass": f"{name} matvec {n}x{k}", "weight_bytes": int(blocks.size), "copy_bytes": int(nbytes)}))
 
 
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=240)
+    ap.add_argument("--warmup", type=int, default=24)
+    ap.add_argument("--eager", action="store_true", help="time plain operator calls instead of graph replays")
+    ap.add_argument("--no-extra", action="store_true", help="skip the table of other formats")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--pmc-pass", action="store_true", help="short run for rocprofv3 --pmc: dominant kernel + a copy of the same size")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU (no sharding, no collectives); run with --gpus 1")
@@ -112,45 +235,74 @@ def main() -> None:
 
     dev = torch.device("cuda:0")
     grid = torch.empty(0, dtype=torch.int8, device=dev)
+    if args.pmc_pass:
+        pmc_pass(mod, dev)
+        return
     x_np = np.random.default_rng(2002).standard_normal((1, 5120), dtype=np.float32)
     x = torch.from_numpy(x_np).to(dev).to(torch.bfloat16)
 
     rings, host_blocks, fns = [], [], []
     for idx, (name, tid, n, k) in enumerate(CASES):
-        blocks, ring = build_case(name, n, k, 1002 + idx, dev)
+        rng = np.random.default_rng(1002 + idx)
+        blocks = _encoders()[name]((rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02)))
         host_blocks.append(blocks)
-        rings.append(ring)
-        fns.append(lambda b, tid=tid, k=k: mod.gguf_quant_gemm_forward(x, b, k, tid, grid))
+        rings.append(ring_of(blocks, dev))
+        fns.append(lambda s, ring=rings[-1], tid=tid, k=k: mod.gguf_quant_gemm_forward(x, ring[s], k, tid, grid))
     step_bytes = sum(b.size for b in host_blocks)
 
-    def step(i):
-        for ring, fn in zip(rings, fns):
-            fn(ring[i % len(ring)])
+    def step_eager(s):
+        for fn in fns:
+            fn(s)
 
-    for i in range(args.warmup):
-        step(i)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        step(args.warmup + i)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+    replay, graphed = (None, False) if args.eager else capture(step_eager, RING)
+    if graphed:
+        # one replay = RING steps (every ring slot once); steps and warmup are rounded up to whole replays
+        args.warmup = -(-args.warmup // RING) * RING
+        args.steps = max(RING, -(-args.steps // RING) * RING)
+        for _ in range(args.warmup // RING):
+            replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps // RING):
+            replay()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+    else:
+        for i in range(args.warmup):
+            step_eager(i % RING)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            step_eager((args.warmup + i) % RING)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
     ms_per_step = elapsed * 1e3 / args.steps
     value = step_bytes / (elapsed / args.steps) / 1e9
 
     # per-case launch durations with HIP events on the launch stream (torch's current stream)
     cases = []
-    for (name, tid, n, k), ring, fn, blocks in zip(CASES, rings, fns, host_blocks):
-        us = event_time_us(fn, ring, max(50, args.steps), 10)
-        hot = event_time_us(fn, ring[:1], max(50, args.steps), 10)
-        cases.append({"type": name, "n": n, "k": k, "t": 1, "weight_bytes": int(blocks.size), "us_per_call": round(us, 3),
+    iters = max(60, args.steps)
+    for (name, tid, n, k), fn, blocks in zip(CASES, fns, host_blocks):
+        us, g = time_calls_us(fn, RING, iters, eager=args.eager)
+        hot, _ = time_calls_us(lambda _s, fn=fn: fn(0), RING, iters, eager=args.eager)
+        cases.append({"case": f"{name} matvec {n}x{k} T=1", "weight_bytes": int(blocks.size), "us_per_call": round(us, 3),
                       "gbs": round(blocks.size / us / 1e3, 1), "frac_hbm_peak": round(blocks.size / us / 1e3 / HBM_PEAK_GBS, 4),
-                      "us_per_call_cache_hot": round(hot, 3)})
+                      "us_per_call_cache_hot": round(hot, 3), "graph": g})
     dom = cases[DOMINANT]
-    roofline = {"bound": "hbm", "achieved": dom["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(dom["gbs"] / HBM_PEAK_GBS, 4), "traffic": None,
-                "kernel": f"{dom['type']} matvec {dom['n']}x{dom['k']}", "bytes_per_launch": dom["weight_bytes"],
-                "us_per_launch": dom["us_per_call"]}
+    # the dominant kernel alone (activations quantized beforehand), for the roofline object
+    d_name, d_tid, d_n, d_k = CASES[DOMINANT]
+    image = mod.quantize_activations(x, d_k // 256)
+    kernel_us, _ = time_calls_us(lambda s: mod.gguf_quant_gemm_prequantized(image, rings[DOMINANT][s], d_tid), RING, iters, eager=args.eager)
+    kernel_gbs = host_blocks[DOMINANT].size / kernel_us / 1e3
+    traffic = None
+    if os.path.exists(TRAFFIC_FILE):
+        with open(TRAFFIC_FILE) as f:
+            traffic = json.load(f).get("q5_k matvec 17408x5120 T=1")
+    roofline = {"bound": "hbm", "achieved": round(kernel_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(kernel_gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
+                "kernel": "k45_mfma_matvec_kernel<Q5K, 5> (q5_k matvec 17408x5120, activations pre-quantized)",
+                "bytes_per_launch": dom["weight_bytes"], "us_per_launch": round(kernel_us, 3),
+                "us_per_operator_call": dom["us_per_call"]}
 
     # parity of what was just timed, against the float-activation oracle (small case only: seconds)
     from oracle import gguf_oracle as O
@@ -158,9 +310,11 @@ def main() -> None:
     want = O.matmul_f(x.float().cpu().numpy(), O.dequant_rows(host_blocks[0], "q4_k", 5120))
     parity = O.rel_l2(y_gpu, want)
 
-    cpu = None
-    if not args.no_cpu_baseline:
-        cpu, _ = cpu_baseline(host_blocks[0], "q4_k", 5120, x.float().cpu().numpy())
+    cpu = None if args.no_cpu_baseline else cpu_baseline(host_blocks[0], "q4_k", 5120, x.float().cpu().numpy())
+    del rings
+    torch.cuda.empty_cache()
+    if not args.no_extra:
+        cases += extra_cases(mod, dev, iters)
 
     out = {
         "metric": "decode matvec effective HBM GB/s (% of peak) + prefill TFLOPS, per quant type",
@@ -173,11 +327,11 @@ def main() -> None:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "int8 dot, f32 accumulate",
+        "dtype": "int8 dot (two int8 activation terms), f32 accumulate",
         "data": "synthetic (seeded N(0,0.02) weights quantized to Q4_K/Q5_K blocks, N(0,1) bf16 activations)",
-        "config": {"workload": "Q4_K + Q5_K decode matvec, N x K = 5120x5120 and 17408x5120, T=1, weights rotated through a "
-                               f"{RING_BYTES >> 20} MiB ring per case",
-                   "bytes_per_step": int(step_bytes), "calls_per_step": len(CASES)},
+        "config": {"workload": "Q4_K + Q5_K decode matvec, N x K = 5120x5120 and 17408x5120, T=1, weights rotated through a ring of "
+                               f"{RING} copies per case ({RING * step_bytes >> 20} MiB in all)",
+                   "bytes_per_step": int(step_bytes), "calls_per_step": len(CASES), "hip_graph_replay": graphed},
         "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "roofline": roofline,
         "cpu_baseline": cpu,

@@ -84,6 +84,18 @@ int pllm_gguf_quant_gemm(const void* x, int x_dtype, const uint8_t* blocks, int 
 size_t pllm_gguf_quant_gemm_workspace_bytes(int type_id, int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row);
 
 /*
+ * The two halves of pllm_gguf_quant_gemm, for callers that feed one activation tensor to several
+ * matrices (q/k/v, gate/up): quantize once into `image` (pllm_gguf_quant_gemm_workspace_bytes bytes,
+ * 256-byte aligned), then run any number of matmuls against it.  They have no counterpart in the
+ * reference, whose kernels re-read float activations; the reference's q8_1 activation quantizers
+ * (src/csrc/cuda_kernel_impl.cu:7090-7117) are the closest relative of the first.
+ */
+int pllm_quantize_activations(const void* x, int x_dtype, int64_t rows, int64_t k, int64_t blocks_per_row,
+                              void* image, size_t image_bytes, void* stream);
+int pllm_gguf_quant_gemm_prequantized(const void* image, const uint8_t* blocks, int type_id, void* y, int y_dtype,
+                                      int64_t rows, int64_t n, int64_t blocks_per_row, void* stream);
+
+/*
  * Two weight matrices of the same [n, k] against one activation tensor (k/v projections): the
  * activations are quantized once.  y [2, rows, n]; workspace as for pllm_gguf_quant_gemm.
  * Replaces gguf_quant_gemm_pair_forward (src/csrc/cuda_kernel.cpp:615-666, launcher

@@ -90,6 +90,26 @@ size_t pllm_gguf_quant_gemm_workspace_bytes(int type_id, int64_t rows, int64_t k
     return pllm::act_image_256_bytes(static_cast<int>(blocks_per_row)) * static_cast<size_t>(rows);
 }
 
+int pllm_quantize_activations(const void* x, int x_dtype, int64_t rows, int64_t k, int64_t blocks_per_row,
+                              void* image, size_t image_bytes, void* stream) {
+    if (!x || !image || !dtype_ok(x_dtype) || !fits_int(rows) || !fits_int(k) || !fits_int(blocks_per_row)) return PLLM_ERR_INVALID_ARGUMENT;
+    if (blocks_per_row * 256 < k) return PLLM_ERR_INVALID_ARGUMENT;
+    if (rows > 65535) return PLLM_ERR_UNSUPPORTED;
+    if (image_bytes < pllm_gguf_quant_gemm_workspace_bytes(PLLM_TYPE_Q4_K, rows, k, 0, blocks_per_row)) return PLLM_ERR_WORKSPACE;
+    return pllm::act_image_256(x, x_dtype, static_cast<int>(rows), static_cast<int>(k), static_cast<int>(blocks_per_row), image,
+                               static_cast<hipStream_t>(stream));
+}
+
+int pllm_gguf_quant_gemm_prequantized(const void* image, const uint8_t* blocks, int type_id, void* y, int y_dtype,
+                                      int64_t rows, int64_t n, int64_t blocks_per_row, void* stream) {
+    if (!image || !blocks || !y || !dtype_ok(y_dtype) || !fits_int(rows) || !fits_int(n) || !fits_int(blocks_per_row)) return PLLM_ERR_INVALID_ARGUMENT;
+    if (pllm_gguf_block_bytes(type_id) == 0) return PLLM_ERR_UNSUPPORTED;
+    if (rows > 65535) return PLLM_ERR_UNSUPPORTED;
+    const int bpr = static_cast<int>(blocks_per_row);
+    return superblock_matvec(static_cast<const unsigned char*>(image), pllm::act_image_256_bytes(bpr), blocks, type_id, y, y_dtype,
+                             static_cast<int>(rows), static_cast<int>(n), bpr, static_cast<hipStream_t>(stream));
+}
+
 int pllm_gguf_quant_gemm_pair(const void* x, int x_dtype, const uint8_t* blocks0, int type_id0, const uint8_t* blocks1, int type_id1,
                               void* y, int y_dtype, int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row,
                               void* workspace, size_t workspace_bytes, void* stream) {

@@ -493,3 +493,39 @@ def gguf_single_token_route_slots(indices, weights, experts_start_idx, n_local_e
     return [torch.tensor(local_ids, dtype=torch.int64), torch.zeros(len(slots), dtype=torch.int64, device=dev),
             weights.view(-1).index_select(0, route_positions), torch.tensor(slots, dtype=torch.int64, device=dev),
             torch.tensor(starts, dtype=torch.int32, device=dev)]
+
+
+def quantize_activations(x: torch.Tensor, blocks_per_row: int) -> torch.Tensor:
+    """Pre-quantize activations [..., K] for the super-block matmuls: returns the opaque uint8 image
+    (one row per activation row) that gguf_quant_gemm_prequantized reads."""
+    _check(x.is_cuda and x.is_contiguous(), "x must be a contiguous CUDA tensor")
+    _check_x(x)
+    k, bpr = x.size(-1), int(blocks_per_row)
+    _check(bpr * 256 >= k, "blocks do not cover row_elems")
+    rows = x.numel() // k
+    lib = _lib()
+    nbytes = lib.pllm_gguf_quant_gemm_workspace_bytes(3, rows, k, 0, bpr)
+    image = torch.empty(rows, nbytes // max(rows, 1), dtype=torch.uint8, device=x.device)
+    with torch.cuda.device(x.device):
+        st = lib.pllm_quantize_activations(x.data_ptr(), _DTYPE_CODE[x.dtype], rows, k, bpr, image.data_ptr(), nbytes, _stream(x.device))
+    _ffi.check(st, "quantize_activations")
+    return image
+
+
+def gguf_quant_gemm_prequantized(image: torch.Tensor, blocks: torch.Tensor, type_id: int, *, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """y [rows, N] from an activation image and raw super-blocks [N, K_blocks, block_bytes]."""
+    type_id = int(type_id)
+    _check_type(type_id)
+    _check(image.is_cuda and image.dtype == torch.uint8 and image.dim() == 2 and image.is_contiguous(), "image must come from quantize_activations")
+    _check(blocks.dim() == 3 and blocks.is_cuda and blocks.dtype == torch.uint8 and blocks.is_contiguous(),
+           "blocks must be a contiguous CUDA uint8 tensor [N, K_blocks, block_bytes]")
+    _check(blocks.size(2) == GGUF_BLOCK_BYTES[type_id], "unexpected GGUF block size for type_id")
+    lib = _lib()
+    rows, n = image.size(0), blocks.size(0)
+    _check(image.size(1) * rows == lib.pllm_gguf_quant_gemm_workspace_bytes(type_id, rows, 0, 0, blocks.size(1)), "image does not match blocks_per_row")
+    y = torch.empty(rows, n, dtype=out_dtype, device=image.device)
+    with torch.cuda.device(image.device):
+        st = lib.pllm_gguf_quant_gemm_prequantized(image.data_ptr(), blocks.data_ptr(), type_id, y.data_ptr(), _DTYPE_CODE[out_dtype],
+                                                   rows, n, blocks.size(1), _stream(image.device))
+    _ffi.check(st, "gguf_quant_gemm_prequantized")
+    return y
