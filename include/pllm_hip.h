@@ -85,11 +85,12 @@ size_t pllm_gguf_quant_gemm_workspace_bytes(int type_id, int64_t rows, int64_t k
 
 /*
  * The two halves of pllm_gguf_quant_gemm, for callers that feed one activation tensor to several
- * matrices (q/k/v, gate/up): quantize once into `image` (pllm_gguf_quant_gemm_workspace_bytes bytes,
- * 256-byte aligned), then run any number of matmuls against it.  They have no counterpart in the
+ * matrices (q/k/v, gate/up): quantize once into `image` (pllm_activation_image_bytes bytes, 256-byte
+ * aligned), then run any number of matmuls against it (the decode kernels, whatever the row count).  They have no counterpart in the
  * reference, whose kernels re-read float activations; the reference's q8_1 activation quantizers
  * (src/csrc/cuda_kernel_impl.cu:7090-7117) are the closest relative of the first.
  */
+size_t pllm_activation_image_bytes(int64_t rows, int64_t blocks_per_row);
 int pllm_quantize_activations(const void* x, int x_dtype, int64_t rows, int64_t k, int64_t blocks_per_row,
                               void* image, size_t image_bytes, void* stream);
 int pllm_gguf_quant_gemm_prequantized(const void* image, const uint8_t* blocks, int type_id, void* y, int y_dtype,

@@ -6,6 +6,9 @@ namespace {
 bool dtype_ok(int d) { return d == PLLM_F32 || d == PLLM_F16 || d == PLLM_BF16; }
 bool fits_int(int64_t v) { return v > 0 && v <= 0x7fffffffLL; }
 
+// from this many activation rows on, the tile GEMM replaces one matvec per row
+constexpr int64_t kGemmMinRows = 16;
+
 }  // namespace
 
 extern "C" {
@@ -78,6 +81,9 @@ int pllm_gguf_quant_gemm(const void* x, int x_dtype, const uint8_t* blocks, int 
     if (!workspace || workspace_bytes < pllm_gguf_quant_gemm_workspace_bytes(type_id, rows, k, n, blocks_per_row)) return PLLM_ERR_WORKSPACE;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int bpr = static_cast<int>(blocks_per_row);
+    if (rows >= kGemmMinRows && pllm::gemm_f16_supports(type_id))
+        return pllm::gemm_f16(x, x_dtype, blocks, type_id, y, y_dtype, static_cast<int>(rows), static_cast<int>(k), static_cast<int>(n), bpr,
+                              workspace, workspace_bytes, s);
     const int st = pllm::act_image_256(x, x_dtype, static_cast<int>(rows), static_cast<int>(k), bpr, workspace, s);
     if (st != PLLM_OK) return st;
     return superblock_matvec(static_cast<const unsigned char*>(workspace), pllm::act_image_256_bytes(bpr), blocks, type_id, y, y_dtype,
@@ -87,6 +93,13 @@ int pllm_gguf_quant_gemm(const void* x, int x_dtype, const uint8_t* blocks, int 
 size_t pllm_gguf_quant_gemm_workspace_bytes(int type_id, int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row) {
     (void)k; (void)n;
     if (!fits_int(rows) || !fits_int(blocks_per_row) || pllm_gguf_block_bytes(type_id) == 0) return 0;
+    if (rows >= kGemmMinRows && pllm::gemm_f16_supports(type_id))
+        return pllm::gemm_f16_workspace_bytes(static_cast<int>(rows), static_cast<int>(blocks_per_row));
+    return pllm::act_image_256_bytes(static_cast<int>(blocks_per_row)) * static_cast<size_t>(rows);
+}
+
+size_t pllm_activation_image_bytes(int64_t rows, int64_t blocks_per_row) {
+    if (!fits_int(rows) || !fits_int(blocks_per_row)) return 0;
     return pllm::act_image_256_bytes(static_cast<int>(blocks_per_row)) * static_cast<size_t>(rows);
 }
 
@@ -95,7 +108,7 @@ int pllm_quantize_activations(const void* x, int x_dtype, int64_t rows, int64_t 
     if (!x || !image || !dtype_ok(x_dtype) || !fits_int(rows) || !fits_int(k) || !fits_int(blocks_per_row)) return PLLM_ERR_INVALID_ARGUMENT;
     if (blocks_per_row * 256 < k) return PLLM_ERR_INVALID_ARGUMENT;
     if (rows > 65535) return PLLM_ERR_UNSUPPORTED;
-    if (image_bytes < pllm_gguf_quant_gemm_workspace_bytes(PLLM_TYPE_Q4_K, rows, k, 0, blocks_per_row)) return PLLM_ERR_WORKSPACE;
+    if (image_bytes < pllm_activation_image_bytes(rows, blocks_per_row)) return PLLM_ERR_WORKSPACE;
     return pllm::act_image_256(x, x_dtype, static_cast<int>(rows), static_cast<int>(k), static_cast<int>(blocks_per_row), image,
                                static_cast<hipStream_t>(stream));
 }
@@ -118,7 +131,7 @@ int pllm_gguf_quant_gemm_pair(const void* x, int x_dtype, const uint8_t* blocks0
     if (blocks_per_row * 256 < k) return PLLM_ERR_INVALID_ARGUMENT;
     if (pllm_gguf_block_bytes(type_id0) == 0 || pllm_gguf_block_bytes(type_id1) == 0) return PLLM_ERR_UNSUPPORTED;
     if (rows > 65535) return PLLM_ERR_UNSUPPORTED;
-    if (!workspace || workspace_bytes < pllm_gguf_quant_gemm_workspace_bytes(type_id0, rows, k, n, blocks_per_row)) return PLLM_ERR_WORKSPACE;
+    if (!workspace || workspace_bytes < pllm_activation_image_bytes(rows, blocks_per_row)) return PLLM_ERR_WORKSPACE;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int bpr = static_cast<int>(blocks_per_row);
     int st = pllm::act_image_256(x, x_dtype, static_cast<int>(rows), static_cast<int>(k), bpr, workspace, s);

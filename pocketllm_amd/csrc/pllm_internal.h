@@ -30,6 +30,12 @@ int dot4_matvec_from_image(const unsigned char* image, size_t stride, const uint
 int dot4_routed_matvec_from_image(const unsigned char* image, size_t stride, const uint8_t* w, int type_id, void* y, int y_dtype,
                                   int rows, int n, int bpr, const int32_t* y_expert, size_t expert_stride, hipStream_t stream);
 
+// prefill tile GEMM on f16 MFMA with decoded tiles (gemm_f16.hip)
+bool gemm_f16_supports(int type_id);
+size_t gemm_f16_workspace_bytes(int rows, int bpr);
+int gemm_f16(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y, int y_dtype,
+             int rows, int k, int n, int bpr, void* workspace, size_t workspace_bytes, hipStream_t stream);
+
 // FP8 E4M3 weights [n, k] with float32 scales [ceil(n/128), ceil(k/128)] (matvec_fp8.hip)
 int fp8_matvec(const void* x, int x_dtype, const uint8_t* w, const float* scale, void* y, int y_dtype,
                int rows, int k, int n, hipStream_t stream);

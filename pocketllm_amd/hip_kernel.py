@@ -286,7 +286,7 @@ def gguf_quant_gemm_pair_forward(x, blocks0, row_elems0, type_id0, blocks1, row_
         return y
     lib = _lib()
     with torch.cuda.device(x.device):
-        ws_bytes = lib.pllm_gguf_quant_gemm_workspace_bytes(type_id0, rows, row_elems0, n, blocks0.size(1))
+        ws_bytes = lib.pllm_activation_image_bytes(rows, blocks0.size(1))
         ws = _workspace(ws_bytes, x.device)
         st = lib.pllm_gguf_quant_gemm_pair(x.data_ptr(), _DTYPE_CODE[x.dtype], blocks0.data_ptr(), type_id0, blocks1.data_ptr(), type_id1,
                                            y.data_ptr(), _DTYPE_CODE[out_dtype], rows, row_elems0, n, blocks0.size(1),
@@ -504,7 +504,7 @@ def quantize_activations(x: torch.Tensor, blocks_per_row: int) -> torch.Tensor:
     _check(bpr * 256 >= k, "blocks do not cover row_elems")
     rows = x.numel() // k
     lib = _lib()
-    nbytes = lib.pllm_gguf_quant_gemm_workspace_bytes(3, rows, k, 0, bpr)
+    nbytes = lib.pllm_activation_image_bytes(rows, bpr)
     image = torch.empty(rows, nbytes // max(rows, 1), dtype=torch.uint8, device=x.device)
     with torch.cuda.device(x.device):
         st = lib.pllm_quantize_activations(x.data_ptr(), _DTYPE_CODE[x.dtype], rows, k, bpr, image.data_ptr(), nbytes, _stream(x.device))
@@ -522,7 +522,7 @@ def gguf_quant_gemm_prequantized(image: torch.Tensor, blocks: torch.Tensor, type
     _check(blocks.size(2) == GGUF_BLOCK_BYTES[type_id], "unexpected GGUF block size for type_id")
     lib = _lib()
     rows, n = image.size(0), blocks.size(0)
-    _check(image.size(1) * rows == lib.pllm_gguf_quant_gemm_workspace_bytes(type_id, rows, 0, 0, blocks.size(1)), "image does not match blocks_per_row")
+    _check(image.size(1) * rows == lib.pllm_activation_image_bytes(rows, blocks.size(1)), "image does not match blocks_per_row")
     y = torch.empty(rows, n, dtype=out_dtype, device=image.device)
     with torch.cuda.device(image.device):
         st = lib.pllm_gguf_quant_gemm_prequantized(image.data_ptr(), blocks.data_ptr(), type_id, y.data_ptr(), _DTYPE_CODE[out_dtype],

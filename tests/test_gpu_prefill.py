@@ -1,0 +1,73 @@
+"""GPU parity of the prefill matmul (tile GEMM on f16 MFMA with decoded tiles) against the float oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import gguf_oracle as O
+from pocketllm_amd import block_codec as C
+from pocketllm_amd.cuda_loader import load_cuda_kernel
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+ENC = {"q4_k": C.quantize_q4_k, "q5_k": C.quantize_q5_k}
+
+
+@pytest.fixture(scope="module")
+def mod():
+    m = load_cuda_kernel()
+    assert m is not None and torch.cuda.is_available()
+    return m
+
+
+@pytest.mark.parametrize("type_name", ["q4_k", "q5_k"])
+@pytest.mark.parametrize("t,n,k", [(16, 128, 256), (64, 300, 768), (130, 129, 1000), (512, 256, 5120), (257, 64, 2048)])
+def test_prefill_matches_float_oracle(mod, type_name, t, n, k):
+    rng = np.random.default_rng(t + n + k)
+    blocks = ENC[type_name]((rng.standard_normal((n, k)) * 0.02).astype(np.float32))
+    x_np = rng.standard_normal((t, k)).astype(np.float32)
+    x_np[3] *= 1e4                      # a token row with huge activations and one with tiny ones: the per-row power-of-two scaling must absorb both
+    x_np[5] *= 1e-6
+    ref_w = O.dequant_rows(blocks, type_name, k)
+    grid = torch.empty(0, dtype=torch.int8, device=DEV)
+    for dt, tol in ((torch.bfloat16, 4e-4), (torch.float32, 6e-4), (torch.float16, 4e-4)):
+        x = torch.from_numpy(x_np).to(DEV).to(dt)
+        if dt == torch.float16:
+            x = torch.from_numpy(np.clip(x_np, -6e4, 6e4)).to(DEV).to(dt)
+        print(f"case prefill {type_name} t={t} n={n} k={k} {dt}", flush=True)
+        y = mod.gguf_quant_gemm_prefill_forward(x, torch.from_numpy(blocks).to(DEV), k, O.TYPE_IDS[type_name], grid, out_dtype=torch.float32)
+        torch.cuda.synchronize()
+        want = O.matmul_f(x.float().cpu().numpy(), ref_w)
+        got = y.cpu().numpy()
+        assert O.rel_l2(got, want) <= 1e-3
+        # row by row as well: a scaling bug in one token must not hide in the total
+        row_err = np.sqrt(((got - want) ** 2).sum(axis=1) / np.maximum((want ** 2).sum(axis=1), 1e-300))
+        assert row_err.max() <= tol, (dt, row_err.argmax(), row_err.max())
+
+
+def test_prefill_3d_input_and_bf16_output(mod):
+    rng = np.random.default_rng(0)
+    blocks = torch.from_numpy(C.quantize_q4_k((rng.standard_normal((192, 512)) * 0.02).astype(np.float32))).to(DEV)
+    x = torch.randn(4, 8, 512, device=DEV, dtype=torch.bfloat16)
+    grid = torch.empty(0, dtype=torch.int8, device=DEV)
+    y = mod.gguf_quant_gemm_prefill_forward(x, blocks, 512, 3, grid)
+    assert y.dtype == torch.bfloat16 and tuple(y.shape) == (4, 8, 192)
+    y32 = mod.gguf_quant_gemm_prefill_forward(x, blocks, 512, 3, grid, out_dtype=torch.float32)
+    assert torch.equal(y32.to(torch.bfloat16), y)
+    # the tile GEMM and the decode kernels state the same operator
+    yd = torch.cat([mod.gguf_quant_gemm_forward(x.view(32, 512)[i:i + 1], blocks, 512, 3, grid, out_dtype=torch.float32) for i in range(32)])
+    assert O.rel_l2(y32.view(32, 192).cpu().numpy(), yd.cpu().numpy()) < 5e-4
+
+
+@pytest.mark.parametrize("type_name,n", [("q4_k", 5120), ("q5_k", 17408)])
+def test_prefill_baseline_shape_sampled(mod, type_name, n):
+    """BASELINE config 3 shape at T = 512; the oracle checks 64 sampled output columns (seconds on the host)."""
+    rng = np.random.default_rng(1003)
+    k, t = 5120, 512
+    blocks = ENC[type_name]((rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02)))
+    x = torch.from_numpy(rng.standard_normal((t, k)).astype(np.float32)).to(DEV).to(torch.bfloat16)
+    y = mod.gguf_quant_gemm_prefill_forward(x, torch.from_numpy(blocks).to(DEV), k, O.TYPE_IDS[type_name],
+                                            torch.empty(0, dtype=torch.int8, device=DEV), out_dtype=torch.float32)
+    torch.cuda.synchronize()
+    cols = rng.choice(n, size=64, replace=False)
+    want = O.matmul_f(x.float().cpu().numpy(), O.dequant_rows(blocks[cols], type_name, k))
+    assert O.rel_l2(y.cpu().numpy()[:, cols], want) <= 4e-4
