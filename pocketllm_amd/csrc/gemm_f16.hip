@@ -73,6 +73,18 @@ __device__ __forceinline__ K4Pair k4_pair(const uint4& hdr, int p) {
     return r;
 }
 
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+struct Half32 { half4 lo[4], hi[4]; };            // lo = weights [16 h, +16), hi = weights [32 + 16 h, +16) of the chunk
+
+__device__ __forceinline__ half4 affine4(uint32_t b0, uint32_t b1, uint32_t b2, uint32_t b3, float scale, float minus) {
+    half4 r;
+    r.x = static_cast<_Float16>(scale * static_cast<float>(b0) - minus);
+    r.y = static_cast<_Float16>(scale * static_cast<float>(b1) - minus);
+    r.z = static_cast<_Float16>(scale * static_cast<float>(b2) - minus);
+    r.w = static_cast<_Float16>(scale * static_cast<float>(b3) - minus);
+    return r;
+}
+
 struct GQ4K {
     static constexpr int kBlockBytes = 144;
     struct Regs { uint4 hdr; uint4 qs; };
@@ -80,15 +92,16 @@ struct GQ4K {
         r.hdr = *reinterpret_cast<const uint4*>(blk);
         r.qs = *reinterpret_cast<const uint4*>(blk + 16 + 32 * p + 16 * h);
     }
-    static __device__ __forceinline__ void decode(const Regs& r, int p, int, float lo[16], float hi[16]) {
+    static __device__ __forceinline__ void word(uint32_t q, const K4Pair& s, half4& lo, half4& hi) {
+        lo = affine4(q & 15u, (q >> 8) & 15u, (q >> 16) & 15u, (q >> 24) & 15u, s.d_sc0, s.dm0);
+        hi = affine4((q >> 4) & 15u, (q >> 12) & 15u, (q >> 20) & 15u, q >> 28, s.d_sc1, s.dm1);
+    }
+    static __device__ __forceinline__ void decode(const Regs& r, int p, Half32& o) {
         const K4Pair s = k4_pair(r.hdr, p);
-        const uint32_t q[4] = {r.qs.x, r.qs.y, r.qs.z, r.qs.w};
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const uint32_t b = (q[i >> 2] >> (8 * (i & 3))) & 0xffu;
-            lo[i] = s.d_sc0 * static_cast<float>(b & 15u) - s.dm0;
-            hi[i] = s.d_sc1 * static_cast<float>(b >> 4) - s.dm1;
-        }
+        word(r.qs.x, s, o.lo[0], o.hi[0]);
+        word(r.qs.y, s, o.lo[1], o.hi[1]);
+        word(r.qs.z, s, o.lo[2], o.hi[2]);
+        word(r.qs.w, s, o.lo[3], o.hi[3]);
     }
 };
 
@@ -100,27 +113,23 @@ struct GQ5K {
         r.qh = *reinterpret_cast<const uint4*>(blk + 16 + 16 * h);
         r.qs = *reinterpret_cast<const uint4*>(blk + 48 + 32 * p + 16 * h);
     }
-    static __device__ __forceinline__ void decode(const Regs& r, int p, int, float lo[16], float hi[16]) {
+    // g = the high-bit bytes shifted so that bit 0 of every byte belongs to the low nibble's weight
+    // and bit 1 to the high nibble's weight
+    static __device__ __forceinline__ void word(uint32_t q, uint32_t g, const K4Pair& s, half4& lo, half4& hi) {
+        const uint32_t l = (q & 0x0f0f0f0fu) | ((g & 0x01010101u) << 4);
+        const uint32_t u = ((q >> 4) & 0x0f0f0f0fu) | ((g & 0x02020202u) << 3);
+        lo = affine4(l & 31u, (l >> 8) & 31u, (l >> 16) & 31u, l >> 24, s.d_sc0, s.dm0);
+        hi = affine4(u & 31u, (u >> 8) & 31u, (u >> 16) & 31u, u >> 24, s.d_sc1, s.dm1);
+    }
+    static __device__ __forceinline__ void decode(const Regs& r, int p, Half32& o) {
         const K4Pair s = k4_pair(r.hdr, p);
-        const uint32_t q[4] = {r.qs.x, r.qs.y, r.qs.z, r.qs.w};
-        const uint32_t g[4] = {r.qh.x, r.qh.y, r.qh.z, r.qh.w};
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const uint32_t b = (q[i >> 2] >> (8 * (i & 3))) & 0xffu;
-            const uint32_t hb = (g[i >> 2] >> (8 * (i & 3))) & 0xffu;
-            lo[i] = s.d_sc0 * static_cast<float>((b & 15u) + (((hb >> (2 * p)) & 1u) << 4)) - s.dm0;
-            hi[i] = s.d_sc1 * static_cast<float>((b >> 4) + (((hb >> (2 * p + 1)) & 1u) << 4)) - s.dm1;
-        }
+        const int sft = 2 * p;
+        word(r.qs.x, r.qh.x >> sft, s, o.lo[0], o.hi[0]);
+        word(r.qs.y, r.qh.y >> sft, s, o.lo[1], o.hi[1]);
+        word(r.qs.z, r.qh.z >> sft, s, o.lo[2], o.hi[2]);
+        word(r.qs.w, r.qh.w >> sft, s, o.lo[3], o.hi[3]);
     }
 };
-
-__device__ __forceinline__ void store16(_Float16* dst, const float v[16]) {
-    half8 a, b;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) { a[i] = static_cast<_Float16>(v[i]); b[i] = static_cast<_Float16>(v[8 + i]); }
-    *reinterpret_cast<half8*>(dst) = a;
-    *reinterpret_cast<half8*>(dst + 8) = b;
-}
 
 template <typename FMT>
 __global__ __launch_bounds__(256) void gemm_f16_kernel(
@@ -150,29 +159,27 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    typename FMT::Regs wreg;
-    uint4 xreg[4];
-    auto fetch = [&](int c) {
-        FMT::load(wreg, wrow + static_cast<size_t>(c >> 2) * FMT::kBlockBytes, c & 3, sh);
+    // two register sets: while chunk c is multiplied, chunk c+1 is decoded into the other LDS buffer
+    // from one set and chunk c+2 is already being fetched into the other
+    typename FMT::Regs wreg0, wreg1;
+    // (the activation registers are separate variables on purpose: grouped in an aggregate the four
+    // copies fuse into one block copy that the compiler then keeps in scratch memory)
+    uint4 xa0, xb0, xc0, xd0, xa1, xb1, xc1, xd1;
+    auto fetch = [&](int c, typename FMT::Regs& wr, uint4& xa, uint4& xb, uint4& xc, uint4& xd) {
+        FMT::load(wr, wrow + static_cast<size_t>(c >> 2) * FMT::kBlockBytes, c & 3, sh);
         const uint4* xp = reinterpret_cast<const uint4*>(xrow + static_cast<size_t>(c) * kBK);
-        xreg[0] = xp[0]; xreg[1] = xp[1]; xreg[2] = xp[2]; xreg[3] = xp[3];
+        xa = xp[0]; xb = xp[1]; xc = xp[2]; xd = xp[3];
     };
-    auto stage = [&](int c, int buf) {
-        float lo[16], hi[16];
-        FMT::decode(wreg, c & 3, sh, lo, hi);
-        _Float16* wdst = ws_buf + buf * kTileHalves + srow * kLds;
-        store16(wdst + 16 * sh, lo);
-        store16(wdst + 32 + 16 * sh, hi);
+    auto stage = [&](int c, const typename FMT::Regs& wr, const uint4& xa, const uint4& xb, const uint4& xc, const uint4& xd, int buf) {
+        Half32 d;
+        FMT::decode(wr, c & 3, d);
+        half4* wlo = reinterpret_cast<half4*>(ws_buf + buf * kTileHalves + srow * kLds + 16 * sh);
+        wlo[0] = d.lo[0]; wlo[1] = d.lo[1]; wlo[2] = d.lo[2]; wlo[3] = d.lo[3];
+        wlo[8] = d.hi[0]; wlo[9] = d.hi[1]; wlo[10] = d.hi[2]; wlo[11] = d.hi[3];
         uint4* xdst = reinterpret_cast<uint4*>(xs_buf + buf * kTileHalves + srow * kLds + 32 * sh);
-        xdst[0] = xreg[0]; xdst[1] = xreg[1]; xdst[2] = xreg[2]; xdst[3] = xreg[3];
+        xdst[0] = xa; xdst[1] = xb; xdst[2] = xc; xdst[3] = xd;
     };
-
-    fetch(0);
-    stage(0, 0);
-    __syncthreads();
-    for (int c = 0; c < chunks; ++c) {
-        const int buf = c & 1;
-        if (c + 1 < chunks) fetch(c + 1);
+    auto multiply = [&](int buf) {
         const _Float16* xt = xs_buf + buf * kTileHalves + (wm * 64 + (lane & 31)) * kLds + 8 * (lane >> 5);
         const _Float16* wt = ws_buf + buf * kTileHalves + (wn * 64 + (lane & 31)) * kLds + 8 * (lane >> 5);
 #pragma unroll
@@ -186,7 +193,21 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(
             acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, b0, acc[1][0], 0, 0, 0);
             acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, b1, acc[1][1], 0, 0, 0);
         }
-        if (c + 1 < chunks) stage(c + 1, buf ^ 1);
+    };
+
+    // chunks is a multiple of 4, so the loop below runs in pairs with compile-time set/buffer indices
+    fetch(0, wreg0, xa0, xb0, xc0, xd0);
+    fetch(1, wreg1, xa1, xb1, xc1, xd1);
+    stage(0, wreg0, xa0, xb0, xc0, xd0, 0);
+    __syncthreads();
+    for (int c = 0; c < chunks; c += 2) {
+        if (c + 2 < chunks) fetch(c + 2, wreg0, xa0, xb0, xc0, xd0);
+        multiply(0);
+        stage(c + 1, wreg1, xa1, xb1, xc1, xd1, 1);
+        __syncthreads();
+        if (c + 3 < chunks) fetch(c + 3, wreg1, xa1, xb1, xc1, xd1);
+        multiply(1);
+        if (c + 2 < chunks) stage(c + 2, wreg0, xa0, xb0, xc0, xd0, 0);
         __syncthreads();
     }
 
