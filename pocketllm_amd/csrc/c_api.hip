@@ -91,10 +91,10 @@ int pllm_gguf_quant_gemm(const void* x, int x_dtype, const uint8_t* blocks, int 
 }
 
 size_t pllm_gguf_quant_gemm_workspace_bytes(int type_id, int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row) {
-    (void)k; (void)n;
-    if (!fits_int(rows) || !fits_int(blocks_per_row) || pllm_gguf_block_bytes(type_id) == 0) return 0;
+    (void)k;
+    if (!fits_int(rows) || !fits_int(n) || !fits_int(blocks_per_row) || pllm_gguf_block_bytes(type_id) == 0) return 0;
     if (rows >= kGemmMinRows && pllm::gemm_f16_supports(type_id))
-        return pllm::gemm_f16_workspace_bytes(static_cast<int>(rows), static_cast<int>(blocks_per_row));
+        return pllm::gemm_f16_workspace_bytes(static_cast<int>(rows), static_cast<int>(n), static_cast<int>(blocks_per_row));
     return pllm::act_image_256_bytes(static_cast<int>(blocks_per_row)) * static_cast<size_t>(rows);
 }
 

@@ -1,13 +1,18 @@
 // Prefill matmul y[T, N] = x[T, K] . dequant(W)[N, K]^T over raw super-blocks, on f16 MFMA.
 //
-// A workgroup owns a 128 (tokens) x 128 (weight rows) output tile and walks K in chunks of 64
-// weights (one quarter of a super-block).  Per chunk every thread pulls 16 bytes of codes plus the
-// block header straight from the raw tensor, decodes 32 weights in float32 exactly as the block
-// decoders do, rounds them once to fp16 and stores them in LDS; the activations arrive as fp16
-// (a pre-pass scales every token row by a power of two so that its largest value sits just below
-// 2^14, which keeps bf16 inputs exact and cannot overflow).  The four waves then run
-// v_mfma_f32_32x32x16_f16 on 64 x 64 sub-tiles with float32 accumulators.  LDS is double buffered:
-// the loads and the decode of chunk c+1 overlap the MFMAs of chunk c.
+// A workgroup owns a BM (tokens, 64 / 128 / 256) x 128 (weight rows) output tile and walks K in
+// chunks of 32 weights (one sub-block).  Per pair of chunks every thread pulls 16 bytes of codes plus
+// the block header straight from the raw tensor; per chunk it decodes 16 weights in float32 exactly
+// as the block decoders do, rounds them once to fp16 and stores them in LDS.  The activations arrive
+// as fp16 (a pre-pass scales every token row by a power of two so that its largest value sits just
+// below 2^14, which keeps bf16 inputs exact and cannot overflow).  The four waves (2 x 2) then run
+// v_mfma_f32_32x32x16_f16 on (BM/2) x 64 sub-tiles with float32 accumulators: with BM = 256 a wave
+// feeds eight MFMAs from six 16-byte LDS reads.  LDS is double buffered: the loads and the decode of
+// chunk c+1 overlap the MFMAs of chunk c, with one barrier per chunk.
+//
+// Small token counts leave too few tiles for 256 compute units, so K can be cut in slices
+// (blockIdx.z): every slice writes float32 partial tiles and a second kernel adds them in slice
+// order, which keeps the result independent of scheduling.
 //
 // Why fp16 tiles and not int8 MFMA here: with int8 activations every 32-wide group needs a float
 // fix-up per output (two scales that change along K), which costs more vector instructions than
@@ -20,11 +25,11 @@ namespace pllm {
 namespace {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr int kBM = 128, kBN = 128, kBK = 64;
-constexpr int kLds = kBK + 8;                       // halves per LDS row: 144 bytes, conflict-free for 16-byte reads
-constexpr int kTileHalves = 128 * kLds;
+constexpr int kBN = 128, kBK = 32;
+constexpr int kLds = kBK + 8;                       // halves per LDS row: 80 bytes, conflict-free for 16-byte reads
 
 // ---- activation pre-pass --------------------------------------------------------------------------
 // xh[t, 0..kp) = fp16(x[t, :] * 2^-e_t) (zero beyond k), scale[t] = 2^e_t, amax_t * 2^-e_t in [2^13, 2^14)
@@ -50,11 +55,10 @@ __global__ __launch_bounds__(256) void act_f16_kernel(const void* __restrict__ x
     if (threadIdx.x == 0) scale[blockIdx.x] = ldexpf(1.0f, e);
 }
 
-// ---- per-format decode of one 64-weight chunk ----------------------------------------------------
-// Thread (row, h) of the staging step decodes weights [64 c + 16 h, +16) and [64 c + 32 + 16 h, +16)
-// of its row (c = chunk index along K) into lo[16] and hi[16].
-struct K4Pair { float d_sc0, d_sc1, dm0, dm1; };
-__device__ __forceinline__ K4Pair k4_pair(const uint4& hdr, int p) {
+// ---- per-format decode of one 32-weight chunk -----------------------------------------------------
+// Staging thread (row, h) decodes weights [32 j + 16 h, +16) of its row for sub-block j = 2 p + e.
+struct K4Scale { float d_sc, dm; };
+__device__ __forceinline__ K4Scale k4_scale(const uint4& hdr, int p, int e) {
     const uint32_t u0 = hdr.y, u1 = hdr.z, u2 = hdr.w;
     uint32_t scw, mnw;
     if (p < 2) {
@@ -65,25 +69,23 @@ __device__ __forceinline__ K4Pair k4_pair(const uint4& hdr, int p) {
         mnw = (((u2 >> 4) & 0x0f0f0f0fu) | (((u1 >> 6) & 0x03030303u) << 4)) >> (16 * (p - 2));
     }
     const float d = f16_bits_to_float(hdr.x & 0xffffu), dmin = f16_bits_to_float(hdr.x >> 16);
-    K4Pair r;
-    r.d_sc0 = d * static_cast<float>(scw & 0xffu);
-    r.d_sc1 = d * static_cast<float>((scw >> 8) & 0xffu);
-    r.dm0 = dmin * static_cast<float>(mnw & 0xffu);
-    r.dm1 = dmin * static_cast<float>((mnw >> 8) & 0xffu);
+    K4Scale r;
+    r.d_sc = d * static_cast<float>((scw >> (8 * e)) & 0xffu);
+    r.dm = dmin * static_cast<float>((mnw >> (8 * e)) & 0xffu);
     return r;
 }
 
-typedef _Float16 half4 __attribute__((ext_vector_type(4)));
-struct Half32 { half4 lo[4], hi[4]; };            // lo = weights [16 h, +16), hi = weights [32 + 16 h, +16) of the chunk
-
-__device__ __forceinline__ half4 affine4(uint32_t b0, uint32_t b1, uint32_t b2, uint32_t b3, float scale, float minus) {
+// four byte-sized codes of one word -> fp16(scale * code - minus)
+__device__ __forceinline__ half4 affine4(uint32_t codes, float scale, float minus) {
     half4 r;
-    r.x = static_cast<_Float16>(scale * static_cast<float>(b0) - minus);
-    r.y = static_cast<_Float16>(scale * static_cast<float>(b1) - minus);
-    r.z = static_cast<_Float16>(scale * static_cast<float>(b2) - minus);
-    r.w = static_cast<_Float16>(scale * static_cast<float>(b3) - minus);
+    r.x = static_cast<_Float16>(scale * static_cast<float>(codes & 0xffu) - minus);
+    r.y = static_cast<_Float16>(scale * static_cast<float>((codes >> 8) & 0xffu) - minus);
+    r.z = static_cast<_Float16>(scale * static_cast<float>((codes >> 16) & 0xffu) - minus);
+    r.w = static_cast<_Float16>(scale * static_cast<float>(codes >> 24) - minus);
     return r;
 }
+
+struct Half16 { half4 a, b, c, d; };
 
 struct GQ4K {
     static constexpr int kBlockBytes = 144;
@@ -92,16 +94,13 @@ struct GQ4K {
         r.hdr = *reinterpret_cast<const uint4*>(blk);
         r.qs = *reinterpret_cast<const uint4*>(blk + 16 + 32 * p + 16 * h);
     }
-    static __device__ __forceinline__ void word(uint32_t q, const K4Pair& s, half4& lo, half4& hi) {
-        lo = affine4(q & 15u, (q >> 8) & 15u, (q >> 16) & 15u, (q >> 24) & 15u, s.d_sc0, s.dm0);
-        hi = affine4((q >> 4) & 15u, (q >> 12) & 15u, (q >> 20) & 15u, q >> 28, s.d_sc1, s.dm1);
-    }
-    static __device__ __forceinline__ void decode(const Regs& r, int p, Half32& o) {
-        const K4Pair s = k4_pair(r.hdr, p);
-        word(r.qs.x, s, o.lo[0], o.hi[0]);
-        word(r.qs.y, s, o.lo[1], o.hi[1]);
-        word(r.qs.z, s, o.lo[2], o.hi[2]);
-        word(r.qs.w, s, o.lo[3], o.hi[3]);
+    static __device__ __forceinline__ void decode(const Regs& r, int p, int e, Half16& o) {
+        const K4Scale s = k4_scale(r.hdr, p, e);
+        const int sft = 4 * e;
+        o.a = affine4((r.qs.x >> sft) & 0x0f0f0f0fu, s.d_sc, s.dm);
+        o.b = affine4((r.qs.y >> sft) & 0x0f0f0f0fu, s.d_sc, s.dm);
+        o.c = affine4((r.qs.z >> sft) & 0x0f0f0f0fu, s.d_sc, s.dm);
+        o.d = affine4((r.qs.w >> sft) & 0x0f0f0f0fu, s.d_sc, s.dm);
     }
 };
 
@@ -113,127 +112,186 @@ struct GQ5K {
         r.qh = *reinterpret_cast<const uint4*>(blk + 16 + 16 * h);
         r.qs = *reinterpret_cast<const uint4*>(blk + 48 + 32 * p + 16 * h);
     }
-    // g = the high-bit bytes shifted so that bit 0 of every byte belongs to the low nibble's weight
-    // and bit 1 to the high nibble's weight
-    static __device__ __forceinline__ void word(uint32_t q, uint32_t g, const K4Pair& s, half4& lo, half4& hi) {
-        const uint32_t l = (q & 0x0f0f0f0fu) | ((g & 0x01010101u) << 4);
-        const uint32_t u = ((q >> 4) & 0x0f0f0f0fu) | ((g & 0x02020202u) << 3);
-        lo = affine4(l & 31u, (l >> 8) & 31u, (l >> 16) & 31u, l >> 24, s.d_sc0, s.dm0);
-        hi = affine4(u & 31u, (u >> 8) & 31u, (u >> 16) & 31u, u >> 24, s.d_sc1, s.dm1);
+    static __device__ __forceinline__ uint32_t codes(uint32_t q, uint32_t g, int sft, int bit) {
+        return ((q >> sft) & 0x0f0f0f0fu) | (((g >> bit) & 0x01010101u) << 4);
     }
-    static __device__ __forceinline__ void decode(const Regs& r, int p, Half32& o) {
-        const K4Pair s = k4_pair(r.hdr, p);
-        const int sft = 2 * p;
-        word(r.qs.x, r.qh.x >> sft, s, o.lo[0], o.hi[0]);
-        word(r.qs.y, r.qh.y >> sft, s, o.lo[1], o.hi[1]);
-        word(r.qs.z, r.qh.z >> sft, s, o.lo[2], o.hi[2]);
-        word(r.qs.w, r.qh.w >> sft, s, o.lo[3], o.hi[3]);
+    static __device__ __forceinline__ void decode(const Regs& r, int p, int e, Half16& o) {
+        const K4Scale s = k4_scale(r.hdr, p, e);
+        const int sft = 4 * e, bit = 2 * p + e;
+        o.a = affine4(codes(r.qs.x, r.qh.x, sft, bit), s.d_sc, s.dm);
+        o.b = affine4(codes(r.qs.y, r.qh.y, sft, bit), s.d_sc, s.dm);
+        o.c = affine4(codes(r.qs.z, r.qh.z, sft, bit), s.d_sc, s.dm);
+        o.d = affine4(codes(r.qs.w, r.qh.w, sft, bit), s.d_sc, s.dm);
     }
 };
 
-template <typename FMT>
-__global__ __launch_bounds__(256) void gemm_f16_kernel(
+// MI = 32-row MFMA tiles per wave along the tokens; the workgroup tile is (64 MI) x 128.
+// partial == nullptr: the tile's result is scaled and stored into y; otherwise slice blockIdx.z
+// stores raw float32 sums into partial[slice, t, n].
+template <typename FMT, int MI>
+__global__ __launch_bounds__(256, 2) void gemm_f16_kernel(
     const _Float16* __restrict__ xh, const float* __restrict__ xscale, const uint8_t* __restrict__ w,
-    void* __restrict__ y, int y_dtype, int t_rows, int n, int bpr) {
+    void* __restrict__ y, int y_dtype, float* __restrict__ partial, int t_rows, int n, int bpr) {
+    constexpr int kBM = 64 * MI;
+    constexpr int kXTile = kBM * kLds, kWTile = kBN * kLds;
     extern __shared__ __align__(16) unsigned char smem[];
-    _Float16* xs_buf = reinterpret_cast<_Float16*>(smem);                 // [2][128][kLds]
-    _Float16* ws_buf = xs_buf + 2 * kTileHalves;                          // [2][128][kLds]
+    _Float16* xs_buf = reinterpret_cast<_Float16*>(smem);                 // [2][kBM][kLds]
+    _Float16* ws_buf = xs_buf + 2 * kXTile;                               // [2][kBN][kLds]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;                              // 2 x 2 waves, 64 x 64 each
+    const int wm = wave >> 1, wn = wave & 1;                              // 2 x 2 waves, (32 MI) x 64 each
     const int n0 = blockIdx.x * kBN, t0 = blockIdx.y * kBM;
     const int kp = bpr * 256;
-    const int chunks = bpr * 4;
+    const int slices = gridDim.z, slice = blockIdx.z;
+    const int c0 = 8 * static_cast<int>(static_cast<long long>(slice) * bpr / slices);
+    const int c1 = 8 * static_cast<int>(static_cast<long long>(slice + 1) * bpr / slices);
 
-    // staging roles: thread (row, h)
+    // staging roles: weights thread (row, h); activations MI pieces of 16 bytes: piece i of a
+    // thread covers row tid / 4 + 64 i, halves [8 (tid % 4), +8) of the chunk
     const int srow = tid >> 1, sh = tid & 1;
     const uint8_t* wrow = w + static_cast<size_t>(min(n0 + srow, n - 1)) * bpr * FMT::kBlockBytes;
-    const _Float16* xrow = xh + static_cast<size_t>(min(t0 + srow, t_rows - 1)) * kp + 32 * sh;
+    // (named variables, not arrays: indexed through the lambdas below, arrays end up in scratch memory)
+    auto xaddr = [&](int i) { return xh + static_cast<size_t>(min(t0 + (tid >> 2) + 64 * i, t_rows - 1)) * kp + 8 * (tid & 3); };
+    const _Float16* const xsrc0 = xaddr(0);
+    const _Float16* const xsrc1 = xaddr(MI > 1 ? 1 : 0);
+    const _Float16* const xsrc2 = xaddr(MI > 2 ? 2 : 0);
+    const _Float16* const xsrc3 = xaddr(MI > 2 ? 3 : 0);
 
-    floatx16 acc[2][2];
+    floatx16 acc[MI][2];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    // two register sets: while chunk c is multiplied, chunk c+1 is decoded into the other LDS buffer
-    // from one set and chunk c+2 is already being fetched into the other
-    typename FMT::Regs wreg0, wreg1;
-    // (the activation registers are separate variables on purpose: grouped in an aggregate the four
-    // copies fuse into one block copy that the compiler then keeps in scratch memory)
-    uint4 xa0, xb0, xc0, xd0, xa1, xb1, xc1, xd1;
-    auto fetch = [&](int c, typename FMT::Regs& wr, uint4& xa, uint4& xb, uint4& xc, uint4& xd) {
-        FMT::load(wr, wrow + static_cast<size_t>(c >> 2) * FMT::kBlockBytes, c & 3, sh);
-        const uint4* xp = reinterpret_cast<const uint4*>(xrow + static_cast<size_t>(c) * kBK);
-        xa = xp[0]; xb = xp[1]; xc = xp[2]; xd = xp[3];
+    typename FMT::Regs wreg;
+    uint4 xreg0, xreg1, xreg2, xreg3;
+    auto fetch = [&](int c) {
+        if ((c & 1) == 0) FMT::load(wreg, wrow + static_cast<size_t>(c >> 3) * FMT::kBlockBytes, (c >> 1) & 3, sh);
+        const size_t off = static_cast<size_t>(c) * kBK;
+        xreg0 = *reinterpret_cast<const uint4*>(xsrc0 + off);
+        if constexpr (MI > 1) xreg1 = *reinterpret_cast<const uint4*>(xsrc1 + off);
+        if constexpr (MI > 2) {
+            xreg2 = *reinterpret_cast<const uint4*>(xsrc2 + off);
+            xreg3 = *reinterpret_cast<const uint4*>(xsrc3 + off);
+        }
     };
-    auto stage = [&](int c, const typename FMT::Regs& wr, const uint4& xa, const uint4& xb, const uint4& xc, const uint4& xd, int buf) {
-        Half32 d;
-        FMT::decode(wr, c & 3, d);
-        half4* wlo = reinterpret_cast<half4*>(ws_buf + buf * kTileHalves + srow * kLds + 16 * sh);
-        wlo[0] = d.lo[0]; wlo[1] = d.lo[1]; wlo[2] = d.lo[2]; wlo[3] = d.lo[3];
-        wlo[8] = d.hi[0]; wlo[9] = d.hi[1]; wlo[10] = d.hi[2]; wlo[11] = d.hi[3];
-        uint4* xdst = reinterpret_cast<uint4*>(xs_buf + buf * kTileHalves + srow * kLds + 32 * sh);
-        xdst[0] = xa; xdst[1] = xb; xdst[2] = xc; xdst[3] = xd;
+    auto stage = [&](int c, int e, int buf) {
+        Half16 d;
+        FMT::decode(wreg, (c >> 1) & 3, e, d);
+        half4* wdst = reinterpret_cast<half4*>(ws_buf + buf * kWTile + srow * kLds + 16 * sh);
+        wdst[0] = d.a; wdst[1] = d.b; wdst[2] = d.c; wdst[3] = d.d;
+        uint4* xdst = reinterpret_cast<uint4*>(xs_buf + buf * kXTile + (tid >> 2) * kLds + 8 * (tid & 3));
+        constexpr int kStep = 64 * kLds * 2 / 16;          // 64 rows further, in 16-byte units
+        xdst[0] = xreg0;
+        if constexpr (MI > 1) xdst[kStep] = xreg1;
+        if constexpr (MI > 2) {
+            xdst[2 * kStep] = xreg2;
+            xdst[3 * kStep] = xreg3;
+        }
     };
     auto multiply = [&](int buf) {
-        const _Float16* xt = xs_buf + buf * kTileHalves + (wm * 64 + (lane & 31)) * kLds + 8 * (lane >> 5);
-        const _Float16* wt = ws_buf + buf * kTileHalves + (wn * 64 + (lane & 31)) * kLds + 8 * (lane >> 5);
+        const _Float16* xt = xs_buf + buf * kXTile + (wm * 32 * MI + (lane & 31)) * kLds + 8 * (lane >> 5);
+        const _Float16* wt = ws_buf + buf * kWTile + (wn * 64 + (lane & 31)) * kLds + 8 * (lane >> 5);
 #pragma unroll
         for (int ks = 0; ks < kBK / 16; ++ks) {
-            const half8 a0 = *reinterpret_cast<const half8*>(xt + 16 * ks);
-            const half8 a1 = *reinterpret_cast<const half8*>(xt + 32 * kLds + 16 * ks);
             const half8 b0 = *reinterpret_cast<const half8*>(wt + 16 * ks);
             const half8 b1 = *reinterpret_cast<const half8*>(wt + 32 * kLds + 16 * ks);
-            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0, b0, acc[0][0], 0, 0, 0);
-            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0, b1, acc[0][1], 0, 0, 0);
-            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, b0, acc[1][0], 0, 0, 0);
-            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, b1, acc[1][1], 0, 0, 0);
+#pragma unroll
+            for (int mi = 0; mi < MI; ++mi) {
+                const half8 a = *reinterpret_cast<const half8*>(xt + mi * 32 * kLds + 16 * ks);
+                acc[mi][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b0, acc[mi][0], 0, 0, 0);
+                acc[mi][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b1, acc[mi][1], 0, 0, 0);
+            }
         }
     };
 
-    // chunks is a multiple of 4, so the loop below runs in pairs with compile-time set/buffer indices
-    fetch(0, wreg0, xa0, xb0, xc0, xd0);
-    fetch(1, wreg1, xa1, xb1, xc1, xd1);
-    stage(0, wreg0, xa0, xb0, xc0, xd0, 0);
+    // c0 and c1 are multiples of 8, so chunks go in pairs: even chunks take the low nibbles of the
+    // codes fetched with them, odd chunks the high nibbles of the same registers
+    fetch(c0);
+    stage(c0, 0, 0);
     __syncthreads();
-    for (int c = 0; c < chunks; c += 2) {
-        if (c + 2 < chunks) fetch(c + 2, wreg0, xa0, xb0, xc0, xd0);
+    for (int c = c0; c < c1; c += 2) {
+        fetch(c + 1);
         multiply(0);
-        stage(c + 1, wreg1, xa1, xb1, xc1, xd1, 1);
+        stage(c + 1, 1, 1);
         __syncthreads();
-        if (c + 3 < chunks) fetch(c + 3, wreg1, xa1, xb1, xc1, xd1);
+        if (c + 2 < c1) fetch(c + 2);
         multiply(1);
-        if (c + 2 < chunks) stage(c + 2, wreg0, xa0, xb0, xc0, xd0, 0);
+        if (c + 2 < c1) stage(c + 2, 0, 0);
         __syncthreads();
     }
 
     // D[m][n]: lane holds column n = lane % 32 and rows 8 * (v / 4) + 4 * (lane / 32) + v % 4
 #pragma unroll
-    for (int mi = 0; mi < 2; ++mi)
+    for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
         for (int ni = 0; ni < 2; ++ni) {
             const int col = n0 + wn * 64 + ni * 32 + (lane & 31);
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const int row = t0 + wm * 64 + mi * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-                if (row < t_rows && col < n) store_any(y, y_dtype, static_cast<size_t>(row) * n + col, acc[mi][ni][v] * xscale[row]);
+                const int row = t0 + wm * 32 * MI + mi * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                if (row < t_rows && col < n) {
+                    if (partial) partial[(static_cast<size_t>(slice) * t_rows + row) * n + col] = acc[mi][ni][v];
+                    else store_any(y, y_dtype, static_cast<size_t>(row) * n + col, acc[mi][ni][v] * xscale[row]);
+                }
             }
         }
 }
 
-template <typename FMT>
-int launch_gemm(const _Float16* xh, const float* xscale, const uint8_t* w, void* y, int y_dtype, int t_rows, int n, int bpr, hipStream_t stream) {
-    const size_t smem = static_cast<size_t>(4) * kTileHalves * sizeof(_Float16);          // 73 728 bytes
-    auto kern = gemm_f16_kernel<FMT>;
+// y[t, n] = xscale[t] * sum over slices (in slice order) of partial[s, t, n]
+__global__ __launch_bounds__(256) void gemm_reduce_kernel(const float* __restrict__ partial, const float* __restrict__ xscale,
+                                                          void* __restrict__ y, int y_dtype, int t_rows, int n, int slices) {
+    const size_t total = static_cast<size_t>(t_rows) * n;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < total; i += static_cast<size_t>(gridDim.x) * 256) {
+        float s = 0.0f;
+        for (int k = 0; k < slices; ++k) s += partial[static_cast<size_t>(k) * total + i];
+        store_any(y, y_dtype, i, s * xscale[i / n]);
+    }
+}
+
+struct GemmPlan { int mi; int slices; };
+
+// Tile height by token count; K slices until the grid has about two workgroups per compute unit.
+GemmPlan plan_gemm(int t_rows, int n, int bpr) {
+    GemmPlan p;
+    p.mi = t_rows <= 64 ? 1 : (t_rows <= 1024 ? 2 : 4);
+    const long long tiles = static_cast<long long>((t_rows + 64 * p.mi - 1) / (64 * p.mi)) * ((n + kBN - 1) / kBN);
+    int s = 1;
+    while (s < 8 && s * 2 <= bpr && tiles * s < 448) s *= 2;
+    p.slices = s;
+    return p;
+}
+
+template <typename FMT, int MI>
+int launch_gemm(const _Float16* xh, const float* xscale, const uint8_t* w, void* y, int y_dtype, float* partial,
+                int t_rows, int n, int bpr, int slices, hipStream_t stream) {
+    const size_t smem = static_cast<size_t>(2) * (64 * MI + kBN) * kLds * sizeof(_Float16);
+    auto kern = gemm_f16_kernel<FMT, MI>;
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem)) != hipSuccess)
         return PLLM_ERR_UNSUPPORTED;
-    dim3 grid((n + kBN - 1) / kBN, (t_rows + kBM - 1) / kBM);
-    hipLaunchKernelGGL(kern, grid, dim3(256), smem, stream, xh, xscale, w, y, y_dtype, t_rows, n, bpr);
-    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+    dim3 grid((n + kBN - 1) / kBN, (t_rows + 64 * MI - 1) / (64 * MI), slices);
+    hipLaunchKernelGGL(kern, grid, dim3(256), smem, stream, xh, xscale, w, y, y_dtype, slices > 1 ? partial : nullptr, t_rows, n, bpr);
+    if (hipGetLastError() != hipSuccess) return PLLM_ERR_LAUNCH;
+    if (slices > 1) {
+        const size_t total = static_cast<size_t>(t_rows) * n;
+        const int blocks = static_cast<int>(std::min<size_t>((total + 255) / 256, 4096));
+        hipLaunchKernelGGL(gemm_reduce_kernel, dim3(blocks), dim3(256), 0, stream, partial, xscale, y, y_dtype, t_rows, n, slices);
+        if (hipGetLastError() != hipSuccess) return PLLM_ERR_LAUNCH;
+    }
+    return PLLM_OK;
+}
+
+template <typename FMT>
+int launch_gemm_mi(int mi, const _Float16* xh, const float* xscale, const uint8_t* w, void* y, int y_dtype, float* partial,
+                   int t_rows, int n, int bpr, int slices, hipStream_t stream) {
+    switch (mi) {
+        case 1: return launch_gemm<FMT, 1>(xh, xscale, w, y, y_dtype, partial, t_rows, n, bpr, slices, stream);
+        case 2: return launch_gemm<FMT, 2>(xh, xscale, w, y, y_dtype, partial, t_rows, n, bpr, slices, stream);
+        default: return launch_gemm<FMT, 4>(xh, xscale, w, y, y_dtype, partial, t_rows, n, bpr, slices, stream);
+    }
 }
 
 size_t align256(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
@@ -242,20 +300,27 @@ size_t align256(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
 
 bool gemm_f16_supports(int type_id) { return type_id == PLLM_TYPE_Q4_K || type_id == PLLM_TYPE_Q5_K; }
 
-size_t gemm_f16_workspace_bytes(int rows, int bpr) {
-    return align256(static_cast<size_t>(rows) * bpr * 256 * sizeof(_Float16)) + align256(static_cast<size_t>(rows) * sizeof(float));
+size_t gemm_f16_workspace_bytes(int rows, int n, int bpr) {
+    const GemmPlan p = plan_gemm(rows, n, bpr);
+    const size_t part = p.slices > 1 ? align256(static_cast<size_t>(p.slices) * rows * n * sizeof(float)) : 0;
+    return align256(static_cast<size_t>(rows) * bpr * 256 * sizeof(_Float16)) + align256(static_cast<size_t>(rows) * sizeof(float)) + part;
 }
 
 int gemm_f16(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y, int y_dtype,
              int rows, int k, int n, int bpr, void* workspace, size_t workspace_bytes, hipStream_t stream) {
-    if (!workspace || workspace_bytes < gemm_f16_workspace_bytes(rows, bpr)) return PLLM_ERR_WORKSPACE;
-    _Float16* xh = static_cast<_Float16*>(workspace);
-    float* xscale = reinterpret_cast<float*>(static_cast<unsigned char*>(workspace) + align256(static_cast<size_t>(rows) * bpr * 256 * sizeof(_Float16)));
+    if (!workspace || workspace_bytes < gemm_f16_workspace_bytes(rows, n, bpr)) return PLLM_ERR_WORKSPACE;
+    const GemmPlan p = plan_gemm(rows, n, bpr);
+    unsigned char* base = static_cast<unsigned char*>(workspace);
+    _Float16* xh = reinterpret_cast<_Float16*>(base);
+    base += align256(static_cast<size_t>(rows) * bpr * 256 * sizeof(_Float16));
+    float* xscale = reinterpret_cast<float*>(base);
+    base += align256(static_cast<size_t>(rows) * sizeof(float));
+    float* partial = reinterpret_cast<float*>(base);
     hipLaunchKernelGGL(act_f16_kernel, dim3(rows), dim3(256), 0, stream, x, x_dtype, xh, xscale, k, bpr * 256);
     if (hipGetLastError() != hipSuccess) return PLLM_ERR_LAUNCH;
     switch (type_id) {
-        case PLLM_TYPE_Q4_K: return launch_gemm<GQ4K>(xh, xscale, w, y, y_dtype, rows, n, bpr, stream);
-        case PLLM_TYPE_Q5_K: return launch_gemm<GQ5K>(xh, xscale, w, y, y_dtype, rows, n, bpr, stream);
+        case PLLM_TYPE_Q4_K: return launch_gemm_mi<GQ4K>(p.mi, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, p.slices, stream);
+        case PLLM_TYPE_Q5_K: return launch_gemm_mi<GQ5K>(p.mi, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, p.slices, stream);
         default: return PLLM_ERR_UNSUPPORTED;
     }
 }

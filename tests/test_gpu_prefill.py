@@ -20,7 +20,7 @@ def mod():
 
 
 @pytest.mark.parametrize("type_name", ["q4_k", "q5_k"])
-@pytest.mark.parametrize("t,n,k", [(16, 128, 256), (64, 300, 768), (130, 129, 1000), (512, 256, 5120), (257, 64, 2048)])
+@pytest.mark.parametrize("t,n,k", [(16, 128, 256), (64, 300, 768), (130, 129, 1000), (512, 256, 5120), (257, 64, 2048), (1100, 200, 512)])
 def test_prefill_matches_float_oracle(mod, type_name, t, n, k):
     rng = np.random.default_rng(t + n + k)
     blocks = ENC[type_name]((rng.standard_normal((n, k)) * 0.02).astype(np.float32))
