@@ -1,14 +1,16 @@
 // Prefill matmul y[T, N] = x[T, K] . dequant(W)[N, K]^T over raw super-blocks, on f16 MFMA.
 //
-// A workgroup owns a BM (tokens, 64 / 128 / 256) x 128 (weight rows) output tile and walks K in
-// chunks of 32 weights (one sub-block).  Per pair of chunks every thread pulls 16 bytes of codes plus
-// the block header straight from the raw tensor; per chunk it decodes 16 weights in float32 exactly
-// as the block decoders do, rounds them once to fp16 and stores them in LDS.  The activations arrive
-// as fp16 (a pre-pass scales every token row by a power of two so that its largest value sits just
-// below 2^14, which keeps bf16 inputs exact and cannot overflow).  The four waves (2 x 2) then run
-// v_mfma_f32_32x32x16_f16 on (BM/2) x 64 sub-tiles with float32 accumulators: with BM = 256 a wave
-// feeds eight MFMAs from six 16-byte LDS reads.  LDS is double buffered: the loads and the decode of
-// chunk c+1 overlap the MFMAs of chunk c, with one barrier per chunk.
+// A workgroup of eight waves owns a BM (tokens, 64 / 128 / 256) x 256 (weight rows) output tile and
+// walks K in chunks of 32 weights (one sub-block).  Per pair of chunks every thread pulls 16 bytes of
+// codes plus the block header straight from the raw tensor and its share of the activations; per
+// chunk it decodes 16 weights in float32 exactly as the block decoders do, rounds them once to fp16
+// and stores them in LDS.  The activations arrive as fp16 (a pre-pass scales every token row by a
+// power of two so that its largest value sits just below 2^14, which keeps bf16 inputs exact and
+// cannot overflow).  The waves (2 x 4) run v_mfma_f32_32x32x16_f16 on (BM/2) x 64 sub-tiles with
+// float32 accumulators: with BM = 256 a wave feeds eight MFMAs from six 16-byte LDS reads.  LDS is
+// double buffered and the raw registers come in two sets, so the loads of the chunk pair after next
+// and the decode of chunk c+1 overlap the MFMAs of chunk c, with one barrier per chunk; inside a
+// step the decode instructions are woven between the MFMAs so that both units stay busy.
 //
 // Small token counts leave too few tiles for 256 compute units, so K can be cut in slices
 // (blockIdx.z): every slice writes float32 partial tiles and a second kernel adds them in slice
@@ -28,7 +30,7 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr int kBN = 128, kBK = 32;
+constexpr int kBN = 256, kBK = 32, kThreads = 512;
 constexpr int kLds = kBK + 8;                       // halves per LDS row: 80 bytes, conflict-free for 16-byte reads
 
 // ---- activation pre-pass --------------------------------------------------------------------------
@@ -125,11 +127,11 @@ struct GQ5K {
     }
 };
 
-// MI = 32-row MFMA tiles per wave along the tokens; the workgroup tile is (64 MI) x 128.
+// MI = 32-row MFMA tiles per wave along the tokens; the workgroup tile is (64 MI) x 256.
 // partial == nullptr: the tile's result is scaled and stored into y; otherwise slice blockIdx.z
 // stores raw float32 sums into partial[slice, t, n].
 template <typename FMT, int MI>
-__global__ __launch_bounds__(256, 2) void gemm_f16_kernel(
+__global__ __launch_bounds__(kThreads) void gemm_f16_kernel(
     const _Float16* __restrict__ xh, const float* __restrict__ xscale, const uint8_t* __restrict__ w,
     void* __restrict__ y, int y_dtype, float* __restrict__ partial, int t_rows, int n, int bpr) {
     constexpr int kBM = 64 * MI;
@@ -140,23 +142,27 @@ __global__ __launch_bounds__(256, 2) void gemm_f16_kernel(
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;                              // 2 x 2 waves, (32 MI) x 64 each
+    const int wm = wave >> 2, wn = wave & 3;                              // 2 x 4 waves, (32 MI) x 64 each
     const int n0 = blockIdx.x * kBN, t0 = blockIdx.y * kBM;
     const int kp = bpr * 256;
     const int slices = gridDim.z, slice = blockIdx.z;
-    const int c0 = 8 * static_cast<int>(static_cast<long long>(slice) * bpr / slices);
-    const int c1 = 8 * static_cast<int>(static_cast<long long>(slice + 1) * bpr / slices);
+    const int b0 = static_cast<int>(static_cast<long long>(slice) * bpr / slices);
+    const int b1 = static_cast<int>(static_cast<long long>(slice + 1) * bpr / slices);
 
-    // staging roles: weights thread (row, h); activations MI pieces of 16 bytes: piece i of a
-    // thread covers row tid / 4 + 64 i, halves [8 (tid % 4), +8) of the chunk
+    // staging roles.  Weights: thread (row, h) owns 16 of the 32 weights of its row in every chunk.
+    // Activations: per chunk the tile has 4 pieces of 16 bytes per row; a thread moves piece
+    // tid % 4 of rows tid / 4 and tid / 4 + 128 (MI = 4), of row tid / 4 (MI = 2), and the first
+    // four waves of row tid / 4 (MI = 1).  Both chunks of a pair are fetched together, so the two
+    // halves of every 128-byte line are requested back to back.
+    // (named variables, not arrays: indexed through the lambdas below, arrays end up in scratch memory)
     const int srow = tid >> 1, sh = tid & 1;
     const uint8_t* wrow = w + static_cast<size_t>(min(n0 + srow, n - 1)) * bpr * FMT::kBlockBytes;
-    // (named variables, not arrays: indexed through the lambdas below, arrays end up in scratch memory)
-    auto xaddr = [&](int i) { return xh + static_cast<size_t>(min(t0 + (tid >> 2) + 64 * i, t_rows - 1)) * kp + 8 * (tid & 3); };
+    constexpr int kXRows = MI == 4 ? 2 : 1;                 // pieces per thread and chunk
+    const bool xmover = MI > 1 || tid < 256;
+    auto xaddr = [&](int i) { return xh + static_cast<size_t>(min(t0 + (tid >> 2) + 128 * i, t_rows - 1)) * kp + 8 * (tid & 3); };
     const _Float16* const xsrc0 = xaddr(0);
-    const _Float16* const xsrc1 = xaddr(MI > 1 ? 1 : 0);
-    const _Float16* const xsrc2 = xaddr(MI > 2 ? 2 : 0);
-    const _Float16* const xsrc3 = xaddr(MI > 2 ? 3 : 0);
+    const _Float16* const xsrc1 = xaddr(kXRows > 1 ? 1 : 0);
+    const int xdst_off = (tid >> 2) * kLds + 8 * (tid & 3);
 
     floatx16 acc[MI][2];
 #pragma unroll
@@ -166,30 +172,30 @@ __global__ __launch_bounds__(256, 2) void gemm_f16_kernel(
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    typename FMT::Regs wreg;
-    uint4 xreg0, xreg1, xreg2, xreg3;
-    auto fetch = [&](int c) {
-        if ((c & 1) == 0) FMT::load(wreg, wrow + static_cast<size_t>(c >> 3) * FMT::kBlockBytes, (c >> 1) & 3, sh);
-        const size_t off = static_cast<size_t>(c) * kBK;
-        xreg0 = *reinterpret_cast<const uint4*>(xsrc0 + off);
-        if constexpr (MI > 1) xreg1 = *reinterpret_cast<const uint4*>(xsrc1 + off);
-        if constexpr (MI > 2) {
-            xreg2 = *reinterpret_cast<const uint4*>(xsrc2 + off);
-            xreg3 = *reinterpret_cast<const uint4*>(xsrc3 + off);
+    typename FMT::Regs wset0, wset1;
+    uint4 xa0, xa1, xa2, xa3, xb0, xb1, xb2, xb3;            // [chunk of the pair][row piece] per set
+    // (blk, p) = super-block along K and chunk pair (64 weights) inside it
+    auto fetch = [&](int blk, int p, typename FMT::Regs& wr, uint4& x00, uint4& x01, uint4& x10, uint4& x11) {
+        FMT::load(wr, wrow + static_cast<size_t>(blk) * FMT::kBlockBytes, p, sh);
+        const size_t off = static_cast<size_t>(blk) * 256 + 64 * p;
+        if (xmover) {
+            x00 = *reinterpret_cast<const uint4*>(xsrc0 + off);
+            x10 = *reinterpret_cast<const uint4*>(xsrc0 + off + 32);
+            if constexpr (kXRows > 1) {
+                x01 = *reinterpret_cast<const uint4*>(xsrc1 + off);
+                x11 = *reinterpret_cast<const uint4*>(xsrc1 + off + 32);
+            }
         }
     };
-    auto stage = [&](int c, int e, int buf) {
+    auto stage = [&](int p, int e, int buf, const typename FMT::Regs& wr, const uint4& x0, const uint4& x1) {
         Half16 d;
-        FMT::decode(wreg, (c >> 1) & 3, e, d);
+        FMT::decode(wr, p, e, d);
         half4* wdst = reinterpret_cast<half4*>(ws_buf + buf * kWTile + srow * kLds + 16 * sh);
         wdst[0] = d.a; wdst[1] = d.b; wdst[2] = d.c; wdst[3] = d.d;
-        uint4* xdst = reinterpret_cast<uint4*>(xs_buf + buf * kXTile + (tid >> 2) * kLds + 8 * (tid & 3));
-        constexpr int kStep = 64 * kLds * 2 / 16;          // 64 rows further, in 16-byte units
-        xdst[0] = xreg0;
-        if constexpr (MI > 1) xdst[kStep] = xreg1;
-        if constexpr (MI > 2) {
-            xdst[2 * kStep] = xreg2;
-            xdst[3 * kStep] = xreg3;
+        if (xmover) {
+            uint4* xdst = reinterpret_cast<uint4*>(xs_buf + buf * kXTile + xdst_off);
+            xdst[0] = x0;
+            if constexpr (kXRows > 1) xdst[128 * kLds * 2 / 16] = x1;
         }
     };
     auto multiply = [&](int buf) {
@@ -207,20 +213,48 @@ __global__ __launch_bounds__(256, 2) void gemm_f16_kernel(
             }
         }
     };
+    // Asks the scheduler to weave one step's decode (vector ALU) and LDS reads between its MFMAs:
+    // a wave that issues its MFMAs in one run and decodes afterwards leaves each unit idle in turn.
+    auto weave = [&]() {
+        constexpr int kMfma = 4 * MI, kValuPer = 112 / kMfma, kReads = 2 * (2 + MI);
+        __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);                 // b0, b1, a0 of the first k-step
+#pragma unroll
+        for (int i = 0; i < kMfma; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);             // one MFMA
+            if (i < kReads - 3) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read ahead
+            __builtin_amdgcn_sched_group_barrier(0x002, kValuPer, 0);      // a slice of the decode
+        }
+    };
 
-    // c0 and c1 are multiples of 8, so chunks go in pairs: even chunks take the low nibbles of the
-    // codes fetched with them, odd chunks the high nibbles of the same registers
-    fetch(c0);
-    stage(c0, 0, 0);
+    // One turn of the loop is one super-block: eight chunks = four pairs, pairs 0 and 2 through
+    // register set a, pairs 1 and 3 through set b, so that the pair index is a compile-time constant
+    // in every step.  Even chunks use the low nibbles of their pair's codes, odd chunks the high ones.
+    // Past the end the loop re-fetches and re-stages the last block instead of branching: nobody reads it.
+    fetch(b0, 0, wset0, xa0, xa1, xa2, xa3);
+    fetch(b0, 1, wset1, xb0, xb1, xb2, xb3);
+    stage(0, 0, 0, wset0, xa0, xa1);
     __syncthreads();
-    for (int c = c0; c < c1; c += 2) {
-        fetch(c + 1);
-        multiply(0);
-        stage(c + 1, 1, 1);
+    for (int blk = b0; blk < b1; ++blk) {
+        const int nxt = min(blk + 1, b1 - 1);
+        multiply(0); stage(0, 1, 1, wset0, xa2, xa3); weave();
         __syncthreads();
-        if (c + 2 < c1) fetch(c + 2);
-        multiply(1);
-        if (c + 2 < c1) stage(c + 2, 0, 0);
+        fetch(blk, 2, wset0, xa0, xa1, xa2, xa3);
+        multiply(1); stage(1, 0, 0, wset1, xb0, xb1); weave();
+        __syncthreads();
+        multiply(0); stage(1, 1, 1, wset1, xb2, xb3); weave();
+        __syncthreads();
+        fetch(blk, 3, wset1, xb0, xb1, xb2, xb3);
+        multiply(1); stage(2, 0, 0, wset0, xa0, xa1); weave();
+        __syncthreads();
+        multiply(0); stage(2, 1, 1, wset0, xa2, xa3); weave();
+        __syncthreads();
+        fetch(nxt, 0, wset0, xa0, xa1, xa2, xa3);
+        multiply(1); stage(3, 0, 0, wset1, xb0, xb1); weave();
+        __syncthreads();
+        multiply(0); stage(3, 1, 1, wset1, xb2, xb3); weave();
+        __syncthreads();
+        fetch(nxt, 1, wset1, xb0, xb1, xb2, xb3);
+        multiply(1); stage(0, 0, 0, wset0, xa0, xa1); weave();
         __syncthreads();
     }
 
@@ -254,13 +288,13 @@ __global__ __launch_bounds__(256) void gemm_reduce_kernel(const float* __restric
 
 struct GemmPlan { int mi; int slices; };
 
-// Tile height by token count; K slices until the grid has about two workgroups per compute unit.
+// Tile height by token count; K slices until the grid has about one workgroup per compute unit.
 GemmPlan plan_gemm(int t_rows, int n, int bpr) {
     GemmPlan p;
-    p.mi = t_rows <= 64 ? 1 : (t_rows <= 1024 ? 2 : 4);
+    p.mi = t_rows <= 64 ? 1 : (t_rows <= 128 ? 2 : 4);
     const long long tiles = static_cast<long long>((t_rows + 64 * p.mi - 1) / (64 * p.mi)) * ((n + kBN - 1) / kBN);
     int s = 1;
-    while (s < 8 && s * 2 <= bpr && tiles * s < 448) s *= 2;
+    while (s < 16 && s * 2 <= bpr && tiles * s < 224) s *= 2;
     p.slices = s;
     return p;
 }
@@ -273,7 +307,7 @@ int launch_gemm(const _Float16* xh, const float* xscale, const uint8_t* w, void*
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem)) != hipSuccess)
         return PLLM_ERR_UNSUPPORTED;
     dim3 grid((n + kBN - 1) / kBN, (t_rows + 64 * MI - 1) / (64 * MI), slices);
-    hipLaunchKernelGGL(kern, grid, dim3(256), smem, stream, xh, xscale, w, y, y_dtype, slices > 1 ? partial : nullptr, t_rows, n, bpr);
+    hipLaunchKernelGGL(kern, grid, dim3(kThreads), smem, stream, xh, xscale, w, y, y_dtype, slices > 1 ? partial : nullptr, t_rows, n, bpr);
     if (hipGetLastError() != hipSuccess) return PLLM_ERR_LAUNCH;
     if (slices > 1) {
         const size_t total = static_cast<size_t>(t_rows) * n;
