@@ -12,9 +12,11 @@
 // and the decode of chunk c+1 overlap the MFMAs of chunk c, with one barrier per chunk; inside a
 // step the decode instructions are woven between the MFMAs so that both units stay busy.
 //
-// Small token counts leave too few tiles for 256 compute units, so K can be cut in slices
-// (blockIdx.z): every slice writes float32 partial tiles and a second kernel adds them in slice
-// order, which keeps the result independent of scheduling.
+// The grid is one-dimensional.  Tiles that fill whole rounds of the machine (one workgroup per
+// compute unit) run over all of K and store their result directly; the tiles left over, which
+// would occupy a fraction of the machine for a full round, are cut along K in slices: every slice
+// writes a float32 partial tile and a second kernel adds them in slice order, which keeps the
+// result independent of scheduling.  Small token counts consist of left-over tiles only.
 //
 // Why fp16 tiles and not int8 MFMA here: with int8 activations every 32-wide group needs a float
 // fix-up per output (two scales that change along K), which costs more vector instructions than
@@ -55,6 +57,56 @@ __global__ __launch_bounds__(256) void act_f16_kernel(const void* __restrict__ x
     for (int i = threadIdx.x; i < kp; i += 256)
         out[i] = static_cast<_Float16>(i < k ? load_any(x, x_dtype, xoff + i) * down : 0.0f);
     if (threadIdx.x == 0) scale[blockIdx.x] = ldexpf(1.0f, e);
+}
+
+// The same for rows of at most 8192 values with 16-bit inputs (the usual case): one wave per row
+// keeps the row in registers between the maximum and the conversion, so x is read once.
+// bits(v) = the value as float32: bf16 is the high half of a float32, fp16 converts in hardware.
+template <bool BF16>
+__global__ __launch_bounds__(256) void act_f16_rows_kernel(const uint16_t* __restrict__ x, _Float16* __restrict__ xh,
+                                                           float* __restrict__ scale, int rows, int k, int kp) {
+    const int lane = threadIdx.x & 63, row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const uint16_t* src = x + static_cast<size_t>(row) * k;
+    constexpr int kMaxPieces = 16;                 // 16 pieces x 64 lanes x 8 values
+    uint4 piece[kMaxPieces];
+    float am = 0.0f;
+    auto value = [](uint32_t word, int hi) -> float {
+        const uint32_t h = hi ? (word >> 16) : (word & 0xffffu);
+        if (BF16) return __uint_as_float(h << 16);
+        return f16_bits_to_float(h);
+    };
+#pragma unroll
+    for (int i = 0; i < kMaxPieces; ++i) {
+        const int e0 = (i * 64 + lane) * 8;
+        piece[i] = make_uint4(0, 0, 0, 0);
+        if (e0 < k) piece[i] = *reinterpret_cast<const uint4*>(src + e0);          // k is a multiple of 8 here
+        const uint32_t wds[4] = {piece[i].x, piece[i].y, piece[i].z, piece[i].w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) am = fmaxf(am, fmaxf(fabsf(value(wds[j], 0)), fabsf(value(wds[j], 1))));
+    }
+    am = group_max<64>(am);
+    int e = 0;
+    if (am > 0.0f && am < __uint_as_float(0x7f800000u)) {
+        (void)frexpf(am, &e);
+        e -= 14;
+    }
+    const float down = ldexpf(1.0f, -e);
+    _Float16* out = xh + static_cast<size_t>(row) * kp;
+#pragma unroll
+    for (int i = 0; i < kMaxPieces; ++i) {
+        const int e0 = (i * 64 + lane) * 8;
+        if (e0 >= kp) continue;
+        const uint32_t wds[4] = {piece[i].x, piece[i].y, piece[i].z, piece[i].w};
+        half8 o;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            o[2 * j] = static_cast<_Float16>(value(wds[j], 0) * down);
+            o[2 * j + 1] = static_cast<_Float16>(value(wds[j], 1) * down);
+        }
+        *reinterpret_cast<half8*>(out + e0) = o;
+    }
+    if (lane == 0) scale[row] = ldexpf(1.0f, e);
 }
 
 // ---- per-format decode of one 32-weight chunk -----------------------------------------------------
@@ -128,12 +180,14 @@ struct GQ5K {
 };
 
 // MI = 32-row MFMA tiles per wave along the tokens; the workgroup tile is (64 MI) x 256.
-// partial == nullptr: the tile's result is scaled and stored into y; otherwise slice blockIdx.z
-// stores raw float32 sums into partial[slice, t, n].
+// Workgroups [0, full_tiles) take whole tiles and store scaled results into y; workgroup
+// full_tiles + r takes slice r % slices of tile full_tiles + r / slices and stores raw float32 sums
+// into partial[r][kBM][kBN].  Tiles are numbered along N first.
 template <typename FMT, int MI>
 __global__ __launch_bounds__(kThreads) void gemm_f16_kernel(
     const _Float16* __restrict__ xh, const float* __restrict__ xscale, const uint8_t* __restrict__ w,
-    void* __restrict__ y, int y_dtype, float* __restrict__ partial, int t_rows, int n, int bpr) {
+    void* __restrict__ y, int y_dtype, float* __restrict__ partial, int t_rows, int n, int bpr,
+    int tiles_n, int full_tiles, int slices) {
     constexpr int kBM = 64 * MI;
     constexpr int kXTile = kBM * kLds, kWTile = kBN * kLds;
     extern __shared__ __align__(16) unsigned char smem[];
@@ -143,11 +197,15 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_kernel(
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 2, wn = wave & 3;                              // 2 x 4 waves, (32 MI) x 64 each
-    const int n0 = blockIdx.x * kBN, t0 = blockIdx.y * kBM;
+    const int wg = blockIdx.x;
+    const bool whole = wg < full_tiles;
+    const int rest = wg - full_tiles;
+    const int tile = whole ? wg : full_tiles + rest / slices;
+    const int slice = whole ? 0 : rest % slices, nsl = whole ? 1 : slices;
+    const int n0 = (tile % tiles_n) * kBN, t0 = (tile / tiles_n) * kBM;
     const int kp = bpr * 256;
-    const int slices = gridDim.z, slice = blockIdx.z;
-    const int b0 = static_cast<int>(static_cast<long long>(slice) * bpr / slices);
-    const int b1 = static_cast<int>(static_cast<long long>(slice + 1) * bpr / slices);
+    const int b0 = static_cast<int>(static_cast<long long>(slice) * bpr / nsl);
+    const int b1 = static_cast<int>(static_cast<long long>(slice + 1) * bpr / nsl);
 
     // staging roles.  Weights: thread (row, h) owns 16 of the 32 weights of its row in every chunk.
     // Activations: per chunk the tile has 4 pieces of 16 bytes per row; a thread moves piece
@@ -263,68 +321,108 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_kernel(
     for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
         for (int ni = 0; ni < 2; ++ni) {
-            const int col = n0 + wn * 64 + ni * 32 + (lane & 31);
+            const int lcol = wn * 64 + ni * 32 + (lane & 31), col = n0 + lcol;
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const int row = t0 + wm * 32 * MI + mi * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-                if (row < t_rows && col < n) {
-                    if (partial) partial[(static_cast<size_t>(slice) * t_rows + row) * n + col] = acc[mi][ni][v];
-                    else store_any(y, y_dtype, static_cast<size_t>(row) * n + col, acc[mi][ni][v] * xscale[row]);
-                }
+                const int lrow = wm * 32 * MI + mi * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3), row = t0 + lrow;
+                if (!whole) partial[(static_cast<size_t>(rest) * kBM + lrow) * kBN + lcol] = acc[mi][ni][v];
+                else if (row < t_rows && col < n) store_any(y, y_dtype, static_cast<size_t>(row) * n + col, acc[mi][ni][v] * xscale[row]);
             }
         }
 }
 
-// y[t, n] = xscale[t] * sum over slices (in slice order) of partial[s, t, n]
+// Split tile number blockIdx.y (tile full_tiles + blockIdx.y of the grid above), 1024 of its
+// elements per workgroup: y[t, n] = xscale[t] * sum over its slices, in slice order, of their
+// partial tiles.
 __global__ __launch_bounds__(256) void gemm_reduce_kernel(const float* __restrict__ partial, const float* __restrict__ xscale,
-                                                          void* __restrict__ y, int y_dtype, int t_rows, int n, int slices) {
-    const size_t total = static_cast<size_t>(t_rows) * n;
-    for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < total; i += static_cast<size_t>(gridDim.x) * 256) {
-        float s = 0.0f;
-        for (int k = 0; k < slices; ++k) s += partial[static_cast<size_t>(k) * total + i];
-        store_any(y, y_dtype, i, s * xscale[i / n]);
+                                                          void* __restrict__ y, int y_dtype, int t_rows, int n,
+                                                          int bm, int tiles_n, int full_tiles, int slices) {
+    const int tile = full_tiles + blockIdx.y;
+    const int n0 = (tile % tiles_n) * kBN, t0 = (tile / tiles_n) * bm;
+    const size_t tile_elems = static_cast<size_t>(bm) * kBN;
+    const int i = (blockIdx.x * 256 + threadIdx.x) * 4;
+    const int row = t0 + i / kBN, col = n0 + i % kBN;
+    if (row >= t_rows || col >= n) return;
+    const float* src = partial + static_cast<size_t>(blockIdx.y) * slices * tile_elems + i;
+    float4 s = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    for (int k = 0; k < slices; ++k) {
+        const float4 v = *reinterpret_cast<const float4*>(src + k * tile_elems);
+        s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
     }
+    const float sc = xscale[row];
+    const size_t o = static_cast<size_t>(row) * n + col;
+    store_any(y, y_dtype, o, s.x * sc);
+    if (col + 1 < n) store_any(y, y_dtype, o + 1, s.y * sc);
+    if (col + 2 < n) store_any(y, y_dtype, o + 2, s.z * sc);
+    if (col + 3 < n) store_any(y, y_dtype, o + 3, s.w * sc);
 }
 
-struct GemmPlan { int mi; int slices; };
+struct GemmPlan { int mi; int tiles_n; int tiles; int full_tiles; int slices; };
 
-// Tile height by token count; K slices until the grid has about one workgroup per compute unit.
+int compute_units() {
+    static int cus = 0;                      // one device kind per process: the count is read once
+    if (cus == 0) {
+        int dev = 0, v = 0;
+        if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) cus = v;
+        else cus = 256;
+    }
+    return cus;
+}
+
+// Tile height by token count.  The tiles beyond the last whole round of the machine are cut in the
+// number of K slices that minimises rounds per slice plus the cost of moving the partial tiles.
 GemmPlan plan_gemm(int t_rows, int n, int bpr) {
     GemmPlan p;
     p.mi = t_rows <= 64 ? 1 : (t_rows <= 128 ? 2 : 4);
-    const long long tiles = static_cast<long long>((t_rows + 64 * p.mi - 1) / (64 * p.mi)) * ((n + kBN - 1) / kBN);
-    int s = 1;
-    while (s < 16 && s * 2 <= bpr && tiles * s < 224) s *= 2;
-    p.slices = s;
+    const int bm = 64 * p.mi, cus = compute_units();
+    p.tiles_n = (n + kBN - 1) / kBN;
+    p.tiles = ((t_rows + bm - 1) / bm) * p.tiles_n;
+    p.full_tiles = (p.tiles / cus) * cus;
+    const int rem = p.tiles - p.full_tiles;
+    p.slices = 1;
+    if (rem > 0) {
+        // time of one unsplit tile in microseconds (about 1.1 per 32-weight step) against the
+        // write-plus-read of rem * s partial tiles at about 5 TB/s
+        const double tile_us = 8.8 * bpr;
+        double best = 1e30;
+        for (int s = 1; s <= 16 && s <= bpr; ++s) {
+            const double rounds = static_cast<double>((static_cast<long long>(rem) * s + cus - 1) / cus) / s;
+            const double move_us = s > 1 ? 2.0 * rem * s * bm * kBN * 4.0 / 5.0e6 : 0.0;
+            const double cost = rounds * tile_us + move_us;
+            if (cost < best - 1e-9) { best = cost; p.slices = s; }
+        }
+    }
     return p;
 }
 
 template <typename FMT, int MI>
-int launch_gemm(const _Float16* xh, const float* xscale, const uint8_t* w, void* y, int y_dtype, float* partial,
-                int t_rows, int n, int bpr, int slices, hipStream_t stream) {
+int launch_gemm(const GemmPlan& p, const _Float16* xh, const float* xscale, const uint8_t* w, void* y, int y_dtype, float* partial,
+                int t_rows, int n, int bpr, hipStream_t stream) {
     const size_t smem = static_cast<size_t>(2) * (64 * MI + kBN) * kLds * sizeof(_Float16);
     auto kern = gemm_f16_kernel<FMT, MI>;
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem)) != hipSuccess)
         return PLLM_ERR_UNSUPPORTED;
-    dim3 grid((n + kBN - 1) / kBN, (t_rows + 64 * MI - 1) / (64 * MI), slices);
-    hipLaunchKernelGGL(kern, grid, dim3(kThreads), smem, stream, xh, xscale, w, y, y_dtype, slices > 1 ? partial : nullptr, t_rows, n, bpr);
+    const int rem = p.tiles - p.full_tiles;
+    const int full = p.slices > 1 ? p.full_tiles : p.tiles;             // unsplit left-over tiles are whole tiles too
+    const int grid = full + (p.slices > 1 ? rem * p.slices : 0);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), smem, stream, xh, xscale, w, y, y_dtype, partial, t_rows, n, bpr,
+                       p.tiles_n, full, p.slices);
     if (hipGetLastError() != hipSuccess) return PLLM_ERR_LAUNCH;
-    if (slices > 1) {
-        const size_t total = static_cast<size_t>(t_rows) * n;
-        const int blocks = static_cast<int>(std::min<size_t>((total + 255) / 256, 4096));
-        hipLaunchKernelGGL(gemm_reduce_kernel, dim3(blocks), dim3(256), 0, stream, partial, xscale, y, y_dtype, t_rows, n, slices);
+    if (p.slices > 1) {
+        hipLaunchKernelGGL(gemm_reduce_kernel, dim3(64 * MI * kBN / 1024, rem), dim3(256), 0, stream, partial, xscale, y, y_dtype, t_rows, n,
+                           64 * MI, p.tiles_n, full, p.slices);
         if (hipGetLastError() != hipSuccess) return PLLM_ERR_LAUNCH;
     }
     return PLLM_OK;
 }
 
 template <typename FMT>
-int launch_gemm_mi(int mi, const _Float16* xh, const float* xscale, const uint8_t* w, void* y, int y_dtype, float* partial,
-                   int t_rows, int n, int bpr, int slices, hipStream_t stream) {
-    switch (mi) {
-        case 1: return launch_gemm<FMT, 1>(xh, xscale, w, y, y_dtype, partial, t_rows, n, bpr, slices, stream);
-        case 2: return launch_gemm<FMT, 2>(xh, xscale, w, y, y_dtype, partial, t_rows, n, bpr, slices, stream);
-        default: return launch_gemm<FMT, 4>(xh, xscale, w, y, y_dtype, partial, t_rows, n, bpr, slices, stream);
+int launch_gemm_mi(const GemmPlan& p, const _Float16* xh, const float* xscale, const uint8_t* w, void* y, int y_dtype, float* partial,
+                   int t_rows, int n, int bpr, hipStream_t stream) {
+    switch (p.mi) {
+        case 1: return launch_gemm<FMT, 1>(p, xh, xscale, w, y, y_dtype, partial, t_rows, n, bpr, stream);
+        case 2: return launch_gemm<FMT, 2>(p, xh, xscale, w, y, y_dtype, partial, t_rows, n, bpr, stream);
+        default: return launch_gemm<FMT, 4>(p, xh, xscale, w, y, y_dtype, partial, t_rows, n, bpr, stream);
     }
 }
 
@@ -336,7 +434,7 @@ bool gemm_f16_supports(int type_id) { return type_id == PLLM_TYPE_Q4_K || type_i
 
 size_t gemm_f16_workspace_bytes(int rows, int n, int bpr) {
     const GemmPlan p = plan_gemm(rows, n, bpr);
-    const size_t part = p.slices > 1 ? align256(static_cast<size_t>(p.slices) * rows * n * sizeof(float)) : 0;
+    const size_t part = p.slices > 1 ? align256(static_cast<size_t>(p.tiles - p.full_tiles) * p.slices * 64 * p.mi * kBN * sizeof(float)) : 0;
     return align256(static_cast<size_t>(rows) * bpr * 256 * sizeof(_Float16)) + align256(static_cast<size_t>(rows) * sizeof(float)) + part;
 }
 
@@ -350,11 +448,18 @@ int gemm_f16(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y,
     float* xscale = reinterpret_cast<float*>(base);
     base += align256(static_cast<size_t>(rows) * sizeof(float));
     float* partial = reinterpret_cast<float*>(base);
-    hipLaunchKernelGGL(act_f16_kernel, dim3(rows), dim3(256), 0, stream, x, x_dtype, xh, xscale, k, bpr * 256);
+    const bool narrow = (x_dtype == PLLM_BF16 || x_dtype == PLLM_F16) && k % 8 == 0 && bpr * 256 <= 8192 &&
+                        reinterpret_cast<uintptr_t>(x) % 16 == 0;
+    if (narrow && x_dtype == PLLM_BF16)
+        hipLaunchKernelGGL(act_f16_rows_kernel<true>, dim3((rows + 3) / 4), dim3(256), 0, stream, static_cast<const uint16_t*>(x), xh, xscale, rows, k, bpr * 256);
+    else if (narrow)
+        hipLaunchKernelGGL(act_f16_rows_kernel<false>, dim3((rows + 3) / 4), dim3(256), 0, stream, static_cast<const uint16_t*>(x), xh, xscale, rows, k, bpr * 256);
+    else
+        hipLaunchKernelGGL(act_f16_kernel, dim3(rows), dim3(256), 0, stream, x, x_dtype, xh, xscale, k, bpr * 256);
     if (hipGetLastError() != hipSuccess) return PLLM_ERR_LAUNCH;
     switch (type_id) {
-        case PLLM_TYPE_Q4_K: return launch_gemm_mi<GQ4K>(p.mi, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, p.slices, stream);
-        case PLLM_TYPE_Q5_K: return launch_gemm_mi<GQ5K>(p.mi, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, p.slices, stream);
+        case PLLM_TYPE_Q4_K: return launch_gemm_mi<GQ4K>(p, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, stream);
+        case PLLM_TYPE_Q5_K: return launch_gemm_mi<GQ5K>(p, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, stream);
         default: return PLLM_ERR_UNSUPPORTED;
     }
 }
