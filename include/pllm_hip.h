@@ -126,10 +126,14 @@ int pllm_gguf_dequantize_rows(const int64_t* row_ids, int64_t n_selected, const 
  *   replaces _dequant_fp8_weight_torch (src/kernels/ops.py:144-147).
  * pllm_fp8_block_gemm: y[t, r] = sum_c x[t, c] * out[r, c] without materialising `out`
  *   replaces soft_fp8_blockfp8_gemm (src/kernels/ops.py:641-648, 910-954) on float activations.
+ *   Few rows take the bandwidth-bound matvec; 16 rows or more with k a multiple of 256 take the
+ *   MFMA tile kernel, which needs `workspace` (pllm_fp8_block_gemm_workspace_bytes bytes, 256-byte
+ *   aligned, private to the call until its kernels have run; the query returns 0 when none is needed).
  */
 int pllm_fp8_block_dequantize(const uint8_t* weight, const float* scale, int64_t n, int64_t k, void* out, int out_dtype, void* stream);
 int pllm_fp8_block_gemm(const void* x, int x_dtype, const uint8_t* weight, const float* scale, void* y, int y_dtype,
-                        int64_t rows, int64_t k, int64_t n, void* stream);
+                        int64_t rows, int64_t k, int64_t n, void* workspace, size_t workspace_bytes, void* stream);
+size_t pllm_fp8_block_gemm_workspace_bytes(int64_t rows, int64_t k, int64_t n);
 
 /*
  * Fused routed-expert matmul over raw super-blocks (types Q2_K, IQ2_XXS, IQ1_M; gate/up share a type,

@@ -145,10 +145,21 @@ int pllm_gguf_quant_gemm_pair(const void* x, int x_dtype, const uint8_t* blocks0
                              static_cast<int>(rows), static_cast<int>(n), bpr, s);
 }
 
+// the tile GEMM serves many rows of 256-aligned k; everything else takes the matvec (no workspace)
+static bool fp8_uses_gemm(int64_t rows, int64_t k) { return rows >= kGemmMinRows && k % 256 == 0; }
+
+size_t pllm_fp8_block_gemm_workspace_bytes(int64_t rows, int64_t k, int64_t n) {
+    if (!fits_int(rows) || !fits_int(k) || !fits_int(n) || !fp8_uses_gemm(rows, k)) return 0;
+    return pllm::gemm_f16_workspace_bytes(static_cast<int>(rows), static_cast<int>(n), static_cast<int>(k / 256));
+}
+
 int pllm_fp8_block_gemm(const void* x, int x_dtype, const uint8_t* weight, const float* scale, void* y, int y_dtype,
-                        int64_t rows, int64_t k, int64_t n, void* stream) {
+                        int64_t rows, int64_t k, int64_t n, void* workspace, size_t workspace_bytes, void* stream) {
     if (!x || !weight || !scale || !y || !dtype_ok(x_dtype) || !dtype_ok(y_dtype)) return PLLM_ERR_INVALID_ARGUMENT;
     if (!fits_int(rows) || !fits_int(k) || !fits_int(n)) return PLLM_ERR_INVALID_ARGUMENT;
+    if (fp8_uses_gemm(rows, k))
+        return pllm::gemm_f16_fp8(x, x_dtype, weight, scale, y, y_dtype, static_cast<int>(rows), static_cast<int>(k), static_cast<int>(n),
+                                  workspace, workspace_bytes, static_cast<hipStream_t>(stream));
     if (rows > 65535) return PLLM_ERR_UNSUPPORTED;
     return pllm::fp8_matvec(x, x_dtype, weight, scale, y, y_dtype, static_cast<int>(rows), static_cast<int>(k),
                             static_cast<int>(n), static_cast<hipStream_t>(stream));

@@ -144,7 +144,7 @@ struct Half16 { half4 a, b, c, d; };
 struct GQ4K {
     static constexpr int kBlockBytes = 144;
     struct Regs { uint4 hdr; uint4 qs; };
-    static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, int p, int h) {
+    static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, const float*, int, int p, int h) {
         r.hdr = *reinterpret_cast<const uint4*>(blk);
         r.qs = *reinterpret_cast<const uint4*>(blk + 16 + 32 * p + 16 * h);
     }
@@ -161,7 +161,7 @@ struct GQ4K {
 struct GQ5K {
     static constexpr int kBlockBytes = 176;
     struct Regs { uint4 hdr; uint4 qh; uint4 qs; };
-    static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, int p, int h) {
+    static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, const float*, int, int p, int h) {
         r.hdr = *reinterpret_cast<const uint4*>(blk);
         r.qh = *reinterpret_cast<const uint4*>(blk + 16 + 16 * h);
         r.qs = *reinterpret_cast<const uint4*>(blk + 48 + 32 * p + 16 * h);
@@ -179,6 +179,32 @@ struct GQ5K {
     }
 };
 
+// FP8 E4M3 (OCP) codes, one byte per weight, rows of k bytes with k a multiple of 256 here; a
+// "block" is 256 consecutive codes of a row and carries no header.  The float32 scale of the
+// 128 x 128 block is folded into the fp16 weight: fp16(f32(code) * scale).
+struct GFP8 {
+    static constexpr int kBlockBytes = 256;
+    struct Regs { uint4 q0, q1; float scale; };
+    static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, const float* srow, int b, int p, int h) {
+        r.q0 = *reinterpret_cast<const uint4*>(blk + 64 * p + 16 * h);
+        r.q1 = *reinterpret_cast<const uint4*>(blk + 64 * p + 32 + 16 * h);
+        r.scale = srow[2 * b + (p >> 1)];
+    }
+    static __device__ __forceinline__ half4 word(uint32_t q, float sc) {
+        typedef float v2f __attribute__((ext_vector_type(2)));
+        const v2f lo = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(q), false);
+        const v2f hi = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(q), true);
+        half4 o;
+        o.x = static_cast<_Float16>(lo.x * sc); o.y = static_cast<_Float16>(lo.y * sc);
+        o.z = static_cast<_Float16>(hi.x * sc); o.w = static_cast<_Float16>(hi.y * sc);
+        return o;
+    }
+    static __device__ __forceinline__ void decode(const Regs& r, int, int e, Half16& o) {
+        const uint4 q = e ? r.q1 : r.q0;
+        o.a = word(q.x, r.scale); o.b = word(q.y, r.scale); o.c = word(q.z, r.scale); o.d = word(q.w, r.scale);
+    }
+};
+
 // MI = 32-row MFMA tiles per wave along the tokens; the workgroup tile is (64 MI) x 256.
 // Workgroups [0, full_tiles) take whole tiles and store scaled results into y; workgroup
 // full_tiles + r takes slice r % slices of tile full_tiles + r / slices and stores raw float32 sums
@@ -187,7 +213,7 @@ template <typename FMT, int MI>
 __global__ __launch_bounds__(kThreads) void gemm_f16_kernel(
     const _Float16* __restrict__ xh, const float* __restrict__ xscale, const uint8_t* __restrict__ w,
     void* __restrict__ y, int y_dtype, float* __restrict__ partial, int t_rows, int n, int bpr,
-    int tiles_n, int full_tiles, int slices) {
+    int tiles_n, int full_tiles, int slices, const float* __restrict__ wscale, int scale_kb) {
     constexpr int kBM = 64 * MI;
     constexpr int kXTile = kBM * kLds, kWTile = kBN * kLds;
     extern __shared__ __align__(16) unsigned char smem[];
@@ -215,6 +241,7 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_kernel(
     // (named variables, not arrays: indexed through the lambdas below, arrays end up in scratch memory)
     const int srow = tid >> 1, sh = tid & 1;
     const uint8_t* wrow = w + static_cast<size_t>(min(n0 + srow, n - 1)) * bpr * FMT::kBlockBytes;
+    const float* srow_scale = wscale + static_cast<size_t>(min(n0 + srow, n - 1) >> 7) * scale_kb;      // FP8 only
     constexpr int kXRows = MI == 4 ? 2 : 1;                 // pieces per thread and chunk
     const bool xmover = MI > 1 || tid < 256;
     auto xaddr = [&](int i) { return xh + static_cast<size_t>(min(t0 + (tid >> 2) + 128 * i, t_rows - 1)) * kp + 8 * (tid & 3); };
@@ -230,11 +257,11 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_kernel(
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    typename FMT::Regs wset0, wset1;
+    typename FMT::Regs wset0 = {}, wset1 = {};
     uint4 xa0, xa1, xa2, xa3, xb0, xb1, xb2, xb3;            // [chunk of the pair][row piece] per set
     // (blk, p) = super-block along K and chunk pair (64 weights) inside it
     auto fetch = [&](int blk, int p, typename FMT::Regs& wr, uint4& x00, uint4& x01, uint4& x10, uint4& x11) {
-        FMT::load(wr, wrow + static_cast<size_t>(blk) * FMT::kBlockBytes, p, sh);
+        FMT::load(wr, wrow + static_cast<size_t>(blk) * FMT::kBlockBytes, srow_scale, blk, p, sh);
         const size_t off = static_cast<size_t>(blk) * 256 + 64 * p;
         if (xmover) {
             x00 = *reinterpret_cast<const uint4*>(xsrc0 + off);
@@ -397,7 +424,7 @@ GemmPlan plan_gemm(int t_rows, int n, int bpr) {
 
 template <typename FMT, int MI>
 int launch_gemm(const GemmPlan& p, const _Float16* xh, const float* xscale, const uint8_t* w, void* y, int y_dtype, float* partial,
-                int t_rows, int n, int bpr, hipStream_t stream) {
+                int t_rows, int n, int bpr, const float* wscale, int scale_kb, hipStream_t stream) {
     const size_t smem = static_cast<size_t>(2) * (64 * MI + kBN) * kLds * sizeof(_Float16);
     auto kern = gemm_f16_kernel<FMT, MI>;
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem)) != hipSuccess)
@@ -406,7 +433,7 @@ int launch_gemm(const GemmPlan& p, const _Float16* xh, const float* xscale, cons
     const int full = p.slices > 1 ? p.full_tiles : p.tiles;             // unsplit left-over tiles are whole tiles too
     const int grid = full + (p.slices > 1 ? rem * p.slices : 0);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), smem, stream, xh, xscale, w, y, y_dtype, partial, t_rows, n, bpr,
-                       p.tiles_n, full, p.slices);
+                       p.tiles_n, full, p.slices, wscale, scale_kb);
     if (hipGetLastError() != hipSuccess) return PLLM_ERR_LAUNCH;
     if (p.slices > 1) {
         hipLaunchKernelGGL(gemm_reduce_kernel, dim3(64 * MI * kBN / 1024, rem), dim3(256), 0, stream, partial, xscale, y, y_dtype, t_rows, n,
@@ -418,11 +445,11 @@ int launch_gemm(const GemmPlan& p, const _Float16* xh, const float* xscale, cons
 
 template <typename FMT>
 int launch_gemm_mi(const GemmPlan& p, const _Float16* xh, const float* xscale, const uint8_t* w, void* y, int y_dtype, float* partial,
-                   int t_rows, int n, int bpr, hipStream_t stream) {
+                   int t_rows, int n, int bpr, const float* wscale, int scale_kb, hipStream_t stream) {
     switch (p.mi) {
-        case 1: return launch_gemm<FMT, 1>(p, xh, xscale, w, y, y_dtype, partial, t_rows, n, bpr, stream);
-        case 2: return launch_gemm<FMT, 2>(p, xh, xscale, w, y, y_dtype, partial, t_rows, n, bpr, stream);
-        default: return launch_gemm<FMT, 4>(p, xh, xscale, w, y, y_dtype, partial, t_rows, n, bpr, stream);
+        case 1: return launch_gemm<FMT, 1>(p, xh, xscale, w, y, y_dtype, partial, t_rows, n, bpr, wscale, scale_kb, stream);
+        case 2: return launch_gemm<FMT, 2>(p, xh, xscale, w, y, y_dtype, partial, t_rows, n, bpr, wscale, scale_kb, stream);
+        default: return launch_gemm<FMT, 4>(p, xh, xscale, w, y, y_dtype, partial, t_rows, n, bpr, wscale, scale_kb, stream);
     }
 }
 
@@ -438,16 +465,15 @@ size_t gemm_f16_workspace_bytes(int rows, int n, int bpr) {
     return align256(static_cast<size_t>(rows) * bpr * 256 * sizeof(_Float16)) + align256(static_cast<size_t>(rows) * sizeof(float)) + part;
 }
 
-int gemm_f16(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y, int y_dtype,
-             int rows, int k, int n, int bpr, void* workspace, size_t workspace_bytes, hipStream_t stream) {
-    if (!workspace || workspace_bytes < gemm_f16_workspace_bytes(rows, n, bpr)) return PLLM_ERR_WORKSPACE;
-    const GemmPlan p = plan_gemm(rows, n, bpr);
+namespace {
+// activations -> fp16 rows + per-row scales at the head of the workspace; returns the partial-tile area
+float* stage_activations(const void* x, int x_dtype, int rows, int k, int bpr, void* workspace, const _Float16*& xh_out, const float*& xscale_out,
+                         hipStream_t stream) {
     unsigned char* base = static_cast<unsigned char*>(workspace);
     _Float16* xh = reinterpret_cast<_Float16*>(base);
     base += align256(static_cast<size_t>(rows) * bpr * 256 * sizeof(_Float16));
     float* xscale = reinterpret_cast<float*>(base);
     base += align256(static_cast<size_t>(rows) * sizeof(float));
-    float* partial = reinterpret_cast<float*>(base);
     const bool narrow = (x_dtype == PLLM_BF16 || x_dtype == PLLM_F16) && k % 8 == 0 && bpr * 256 <= 8192 &&
                         reinterpret_cast<uintptr_t>(x) % 16 == 0;
     if (narrow && x_dtype == PLLM_BF16)
@@ -456,12 +482,39 @@ int gemm_f16(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y,
         hipLaunchKernelGGL(act_f16_rows_kernel<false>, dim3((rows + 3) / 4), dim3(256), 0, stream, static_cast<const uint16_t*>(x), xh, xscale, rows, k, bpr * 256);
     else
         hipLaunchKernelGGL(act_f16_kernel, dim3(rows), dim3(256), 0, stream, x, x_dtype, xh, xscale, k, bpr * 256);
+    xh_out = xh;
+    xscale_out = xscale;
+    return reinterpret_cast<float*>(base);
+}
+}  // namespace
+
+int gemm_f16(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y, int y_dtype,
+             int rows, int k, int n, int bpr, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+    if (!workspace || workspace_bytes < gemm_f16_workspace_bytes(rows, n, bpr)) return PLLM_ERR_WORKSPACE;
+    const GemmPlan p = plan_gemm(rows, n, bpr);
+    const _Float16* xh;
+    const float* xscale;
+    float* partial = stage_activations(x, x_dtype, rows, k, bpr, workspace, xh, xscale, stream);
     if (hipGetLastError() != hipSuccess) return PLLM_ERR_LAUNCH;
     switch (type_id) {
-        case PLLM_TYPE_Q4_K: return launch_gemm_mi<GQ4K>(p, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, stream);
-        case PLLM_TYPE_Q5_K: return launch_gemm_mi<GQ5K>(p, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, stream);
+        case PLLM_TYPE_Q4_K: return launch_gemm_mi<GQ4K>(p, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, nullptr, 0, stream);
+        case PLLM_TYPE_Q5_K: return launch_gemm_mi<GQ5K>(p, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, nullptr, 0, stream);
         default: return PLLM_ERR_UNSUPPORTED;
     }
+}
+
+// FP8 weights [n, k] (k a multiple of 256), scales [ceil(n/128), k/128]
+int gemm_f16_fp8(const void* x, int x_dtype, const uint8_t* w, const float* wscale, void* y, int y_dtype,
+                 int rows, int k, int n, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+    if (k % 256 != 0) return PLLM_ERR_UNSUPPORTED;
+    const int bpr = k / 256;
+    if (!workspace || workspace_bytes < gemm_f16_workspace_bytes(rows, n, bpr)) return PLLM_ERR_WORKSPACE;
+    const GemmPlan p = plan_gemm(rows, n, bpr);
+    const _Float16* xh;
+    const float* xscale;
+    float* partial = stage_activations(x, x_dtype, rows, k, bpr, workspace, xh, xscale, stream);
+    if (hipGetLastError() != hipSuccess) return PLLM_ERR_LAUNCH;
+    return launch_gemm_mi<GFP8>(p, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, wscale, k / 128, stream);
 }
 
 }  // namespace pllm

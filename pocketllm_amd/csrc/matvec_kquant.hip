@@ -50,9 +50,12 @@ __device__ __forceinline__ uint4 nib_lo(const uint4& q) {
 __device__ __forceinline__ uint4 nib_hi(const uint4& q) {
     return make_uint4((q.x >> 4) & 0x0f0f0f0fu, (q.y >> 4) & 0x0f0f0f0fu, (q.z >> 4) & 0x0f0f0f0fu, (q.w >> 4) & 0x0f0f0f0fu);
 }
+// bit `bit` of every byte of qh moves to bit 4 of the same byte by one rotation (a rotation only
+// wraps bits that the mask drops) and is merged into the nibble codes
 __device__ __forceinline__ uint4 fifth_bit(const uint4& w, const uint4& qh, int bit) {
-    return make_uint4(w.x | (((qh.x >> bit) & 0x01010101u) << 4), w.y | (((qh.y >> bit) & 0x01010101u) << 4),
-                      w.z | (((qh.z >> bit) & 0x01010101u) << 4), w.w | (((qh.w >> bit) & 0x01010101u) << 4));
+    const uint32_t r = static_cast<uint32_t>(bit + 28) & 31u;
+    return make_uint4(w.x | (__builtin_amdgcn_alignbit(qh.x, qh.x, r) & 0x10101010u), w.y | (__builtin_amdgcn_alignbit(qh.y, qh.y, r) & 0x10101010u),
+                      w.z | (__builtin_amdgcn_alignbit(qh.z, qh.z, r) & 0x10101010u), w.w | (__builtin_amdgcn_alignbit(qh.w, qh.w, r) & 0x10101010u));
 }
 
 // ------------------------------------------------------------------------------------------------

@@ -33,6 +33,8 @@ int dot4_routed_matvec_from_image(const unsigned char* image, size_t stride, con
 // prefill tile GEMM on f16 MFMA with decoded tiles (gemm_f16.hip)
 bool gemm_f16_supports(int type_id);
 size_t gemm_f16_workspace_bytes(int rows, int n, int bpr);
+int gemm_f16_fp8(const void* x, int x_dtype, const uint8_t* w, const float* wscale, void* y, int y_dtype,
+                 int rows, int k, int n, void* workspace, size_t workspace_bytes, hipStream_t stream);
 int gemm_f16(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y, int y_dtype,
              int rows, int k, int n, int bpr, void* workspace, size_t workspace_bytes, hipStream_t stream);
 

@@ -228,8 +228,11 @@ def fp8_block_gemm_forward(x: torch.Tensor, weight: torch.Tensor, scale: torch.T
     if rows == 0:
         return y
     with torch.cuda.device(x.device):
+        ws_bytes = _lib().pllm_fp8_block_gemm_workspace_bytes(rows, k, n)
+        ws = _workspace(ws_bytes, x.device) if ws_bytes else None
         st = _lib().pllm_fp8_block_gemm(x.data_ptr(), _DTYPE_CODE[x.dtype], w8.data_ptr(), scale.data_ptr(), y.data_ptr(),
-                                        _DTYPE_CODE[out_dtype], rows, k, n, _stream(x.device))
+                                        _DTYPE_CODE[out_dtype], rows, k, n, ws.data_ptr() if ws is not None else None, ws_bytes,
+                                        _stream(x.device))
     _ffi.check(st, "fp8_block_gemm_forward")
     return y
 

@@ -71,3 +71,40 @@ def test_prefill_baseline_shape_sampled(mod, type_name, n):
     cols = rng.choice(n, size=64, replace=False)
     want = O.matmul_f(x.float().cpu().numpy(), O.dequant_rows(blocks[cols], type_name, k))
     assert O.rel_l2(y.cpu().numpy()[:, cols], want) <= 4e-4
+
+
+# ---- FP8 E4M3 block-scaled weights through the same tile kernel ---------------------------------------
+
+@pytest.mark.parametrize("t,n,k", [(16, 128, 256), (64, 300, 768), (130, 129, 1024), (257, 520, 2048)])
+def test_fp8_prefill_matches_float_oracle(mod, t, n, k):
+    rng = np.random.default_rng(t * 7 + n + k)
+    codes = rng.integers(0, 256, size=(n, k), dtype=np.uint8)
+    codes[(codes & 0x7f) == 0x7f] = 0x3c                       # no NaN codes
+    scale = rng.uniform(0.001, 0.01, size=((n + 127) // 128, k // 128)).astype(np.float32)
+    x_np = rng.standard_normal((t, k)).astype(np.float32)
+    x_np[1] *= 300.0
+    for dt in (torch.bfloat16, torch.float32):
+        print(f"case fp8 prefill t={t} n={n} k={k} {dt}", flush=True)
+        x = torch.from_numpy(x_np).to(DEV).to(dt)
+        y = mod.fp8_block_gemm_forward(x, torch.from_numpy(codes).to(DEV), torch.from_numpy(scale).to(DEV))
+        torch.cuda.synchronize()
+        want = O.matmul_f(x.float().cpu().numpy(), O.dequant_fp8_block(codes, scale))
+        # rows compared one by one: the huge row must not hide errors in the others
+        got = y.cpu().numpy()
+        for r in (0, 1, t - 1):
+            assert O.rel_l2(got[r], want[r]) <= 1e-3, (t, n, k, dt, r)
+        assert O.rel_l2(got, want) <= 1e-3
+
+
+def test_fp8_prefill_baseline_shape_sampled(mod):
+    """BASELINE config 4 at T = 512 (N = 17408, K = 5120, weights N(0, 0.02) with blockmax/448 scales); 64 sampled columns."""
+    rng = np.random.default_rng(1004)
+    n, k, t = 17408, 5120, 512
+    codes, scale = C.quantize_fp8_block(rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02))
+    x = torch.from_numpy(rng.standard_normal((t, k)).astype(np.float32)).to(DEV).to(torch.bfloat16)
+    y = mod.fp8_block_gemm_forward(x, torch.from_numpy(codes).to(DEV), torch.from_numpy(scale).to(DEV))
+    torch.cuda.synchronize()
+    cols = rng.choice(n, size=64, replace=False)
+    w = O.dequant_fp8_block(codes, scale)[cols]
+    want = O.matmul_f(x.float().cpu().numpy(), w)
+    assert O.rel_l2(y.cpu().numpy()[:, cols], want) <= 1e-3
