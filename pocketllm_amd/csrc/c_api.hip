@@ -11,6 +11,18 @@ constexpr int64_t kGemmMinRows = 16;
 
 }  // namespace
 
+namespace pllm {
+int compute_units() {
+    static int cus = 0;                      // one device kind per process: the count is read once
+    if (cus == 0) {
+        int dev = 0, v = 0;
+        if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) cus = v;
+        else cus = 256;
+    }
+    return cus;
+}
+}  // namespace pllm
+
 extern "C" {
 
 const char* pllm_status_string(int status) {

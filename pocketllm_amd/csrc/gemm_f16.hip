@@ -386,16 +386,6 @@ __global__ __launch_bounds__(256) void gemm_reduce_kernel(const float* __restric
 
 struct GemmPlan { int mi; int tiles_n; int tiles; int full_tiles; int slices; };
 
-int compute_units() {
-    static int cus = 0;                      // one device kind per process: the count is read once
-    if (cus == 0) {
-        int dev = 0, v = 0;
-        if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) cus = v;
-        else cus = 256;
-    }
-    return cus;
-}
-
 // Tile height by token count.  The tiles beyond the last whole round of the machine are cut in the
 // number of K slices that minimises rounds per slice plus the cost of moving the partial tiles.
 GemmPlan plan_gemm(int t_rows, int n, int bpr) {

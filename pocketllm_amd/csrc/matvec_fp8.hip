@@ -8,6 +8,7 @@
 // applied once per chunk.  Row sums are 64-lane reductions.
 #include "pllm_device.h"
 #include "pllm_internal.h"
+#include <algorithm>
 
 namespace pllm {
 namespace {
@@ -91,6 +92,76 @@ __global__ __launch_bounds__(kThreads) void fp8_stream_matvec_kernel(
     }
 }
 
+// The same, persistent: the grid is sized to be resident at once, a workgroup stages the activation
+// row once and then walks groups of 8 weight rows (two per wave), always holding the loads of its
+// next group in a second register set while it multiplies the current one.  Rows of at most
+// 64 * 16 * ITERS bytes.
+template <int ITERS>
+__device__ __forceinline__ void fp8_fetch_group(uint4 (&r)[kRowsPerWave][ITERS], const uint8_t* __restrict__ w, int row0, int n, int k, int chunks, int lane) {
+#pragma unroll
+    for (int q = 0; q < kRowsPerWave; ++q) {
+        const uint8_t* wrow = w + static_cast<size_t>(min(row0 + q, n - 1)) * k;
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) r[q][it] = *reinterpret_cast<const uint4*>(wrow + 16 * min(it * 64 + lane, chunks - 1));
+    }
+}
+
+template <int ITERS>
+__device__ __forceinline__ void fp8_finish_group(const uint4 (&r)[kRowsPerWave][ITERS], const float* xs, const float* __restrict__ scale,
+                                                 void* __restrict__ y, int y_dtype, size_t yoff, int row0, int n, int kb, int chunks, int lane) {
+    float acc[kRowsPerWave];
+#pragma unroll
+    for (int q = 0; q < kRowsPerWave; ++q) acc[q] = 0.0f;
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int c = it * 64 + lane;
+        const bool ok = c < chunks;
+        const int cc = ok ? c : 0;
+#pragma unroll
+        for (int q = 0; q < kRowsPerWave; ++q) {
+            const float d = chunk_dot(r[q][it], xs + 16 * cc);
+            const float sc = scale[(min(row0 + q, n - 1) >> 7) * kb + (cc >> 3)];
+            acc[q] += ok ? d * sc : 0.0f;
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < kRowsPerWave; ++q) {
+        const float total = group_sum<64>(acc[q]);
+        if (lane == 0 && row0 + q < n) store_any(y, y_dtype, yoff + row0 + q, total);
+    }
+}
+
+template <int ITERS>
+__global__ __launch_bounds__(kThreads) void fp8_persistent_matvec_kernel(
+    const void* __restrict__ x, int x_dtype, const uint8_t* __restrict__ w, const float* __restrict__ scale,
+    void* __restrict__ y, int y_dtype, int k, int n, int kb, int groups) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    float* xs = reinterpret_cast<float*>(smem);
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int chunks = k >> 4;
+    const size_t xoff = static_cast<size_t>(blockIdx.y) * k;
+    const size_t yoff = static_cast<size_t>(blockIdx.y) * n;
+    const int rows_per_group = kWaves * kRowsPerWave, wave_row = wave * kRowsPerWave;
+
+    uint4 a[kRowsPerWave][ITERS], b[kRowsPerWave][ITERS];
+    int g = blockIdx.x;
+    const int step = gridDim.x;
+    fp8_fetch_group<ITERS>(a, w, g * rows_per_group + wave_row, n, k, chunks, lane);
+    for (int i = tid; i < k; i += kThreads) xs[i] = load_any(x, x_dtype, xoff + i);
+    __syncthreads();
+    while (g < groups) {
+        if (g + step < groups) fp8_fetch_group<ITERS>(b, w, (g + step) * rows_per_group + wave_row, n, k, chunks, lane);
+        fp8_finish_group<ITERS>(a, xs, scale, y, y_dtype, yoff, g * rows_per_group + wave_row, n, kb, chunks, lane);
+        g += step;
+        if (g >= groups) break;
+        if (g + step < groups) fp8_fetch_group<ITERS>(a, w, (g + step) * rows_per_group + wave_row, n, k, chunks, lane);
+        fp8_finish_group<ITERS>(b, xs, scale, y, y_dtype, yoff, g * rows_per_group + wave_row, n, kb, chunks, lane);
+        g += step;
+    }
+}
+
 __device__ __forceinline__ float fp8_to_float_sw(uint32_t c) {
     const uint32_t e = (c >> 3) & 15u, m = c & 7u;
     float v;
@@ -145,6 +216,18 @@ int fp8_matvec(const void* x, int x_dtype, const uint8_t* w, const float* scale,
         return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
     }
     const int niter = ((k >> 4) + 63) / 64;
+    if (niter <= 6) {
+        const int groups = (n + kWaves * kRowsPerWave - 1) / (kWaves * kRowsPerWave);
+        const int grid_x = std::min(groups, 2 * compute_units());   // two resident workgroups per compute unit (register-bound), groups dealt round-robin
+        const size_t smem = static_cast<size_t>(k) * sizeof(float);
+#define PLLM_PCASE(I) case I: hipLaunchKernelGGL(fp8_persistent_matvec_kernel<I>, dim3(grid_x, rows), dim3(kThreads), smem, stream, x, x_dtype, w, scale, y, y_dtype, k, n, (k + 127) / 128, groups); break
+        switch (niter) {
+            PLLM_PCASE(1); PLLM_PCASE(2); PLLM_PCASE(3); PLLM_PCASE(4); PLLM_PCASE(5);
+            default: hipLaunchKernelGGL(fp8_persistent_matvec_kernel<6>, dim3(grid_x, rows), dim3(kThreads), smem, stream, x, x_dtype, w, scale, y, y_dtype, k, n, (k + 127) / 128, groups); break;
+        }
+#undef PLLM_PCASE
+        return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+    }
     const int passes = (niter + 5) / 6;
     const int iters = (niter + passes - 1) / passes;
 #define PLLM_CASE(I) case I: return launch_stream<I>(x, x_dtype, w, scale, y, y_dtype, rows, k, n, stream)

@@ -30,6 +30,9 @@ int dot4_matvec_from_image(const unsigned char* image, size_t stride, const uint
 int dot4_routed_matvec_from_image(const unsigned char* image, size_t stride, const uint8_t* w, int type_id, void* y, int y_dtype,
                                   int rows, int n, int bpr, const int32_t* y_expert, size_t expert_stride, hipStream_t stream);
 
+// compute units of the current device (read once per process; 256 when no device answers)
+int compute_units();
+
 // prefill tile GEMM on f16 MFMA with decoded tiles (gemm_f16.hip)
 bool gemm_f16_supports(int type_id);
 size_t gemm_f16_workspace_bytes(int rows, int n, int bpr);
