@@ -189,6 +189,58 @@ def extra_cases(mod, dev, iters):
     run("fused experts iq2_xxs gate/up + iq1_m down, 256 experts top-8, T=1", per_call,
         lambda s: mod.gguf_moe_single_token_forward(xm, topi[s], topw[s], w1, w3, w2, 0.0), RING,
         {"note": "each slot routes to a different random top-8 of the 256 resident experts (887 MB)"})
+    # the same experts at T=256 (BASELINE config 5): 2048 routes grouped by expert
+    t = 256
+    logits = torch.from_numpy(rng.standard_normal((t, e)).astype(np.float32))
+    tw, ti = torch.softmax(logits, dim=-1).topk(8, dim=-1)
+    tw = (tw / tw.sum(dim=-1, keepdim=True)).to(dev)
+    _, toks, rws, seg = mod.moe_group_routes(ti.to(dev), tw, 0, e)
+    xt = torch.randn(t, d, device=dev, dtype=torch.bfloat16)
+    grids = (codebooks.get_iq2xxs_signed_grid_tensor().to(dev), codebooks.get_iq1_grid_tensor().to(dev))
+    touched = int((seg[1:] > seg[:-1]).sum().item())
+    flops = 2.0 * t * 8 * 3 * inter * d
+    us, graphed = time_calls_us(lambda s: mod.gguf_moe_prefill_grouped_forward(xt, toks, rws, seg, w1, w3, w2, d, 0, d, 0, inter, 2, grids, 0.0),
+                                4, max(8, iters // 8))
+    nbytes = touched * (2 * inter * (d // 256) * 66 + d * (inter // 256) * 56)
+    out.append({"case": "fused experts iq2_xxs gate/up + iq1_m down, 256 experts top-8, T=256", "weight_bytes": nbytes,
+                "us_per_call": round(us, 3), "gbs": round(nbytes / us / 1e3, 1), "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                "tflops": round(flops / us / 1e6, 2), "graph": graphed, "note": f"{touched} of 256 experts touched by the 2048 routes"})
+    del w1, w3, w2
+    return out + prefill_cases(mod, dev, iters)
+
+
+F16_MFMA_PEAK_TFLOPS = 2500.0
+
+
+def prefill_cases(mod, dev, iters):
+    """BASELINE configs 3 and 4 at T > 1: the MFMA tile kernel, TFLOPS = 2 T K N / t against the dense fp16 peak
+    (the tiles are decoded to fp16, see the kernel's header for why)."""
+    from pocketllm_amd import block_codec as C
+    rng = np.random.default_rng(4004)
+    out = []
+    empty = torch.empty(0, dtype=torch.int8, device=dev)
+    k = 5120
+
+    def run(label, t, n, fn):
+        us, graphed = time_calls_us(fn, 4, max(8, iters // 8))
+        tf = 2.0 * t * k * n / us / 1e6
+        out.append({"case": label, "us_per_call": round(us, 3), "tflops": round(tf, 1), "frac_mfma_peak": round(tf / F16_MFMA_PEAK_TFLOPS, 4),
+                    "peak": "fp16 dense 2.5 PFLOP/s", "graph": graphed})
+
+    for name, tid, enc in (("q4_k", 3, C.quantize_q4_k), ("q5_k", 4, C.quantize_q5_k)):
+        for n in (5120, 17408):
+            blocks = torch.from_numpy(enc(rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02))).to(dev)
+            for t in (64, 512, 2048):
+                x = torch.randn(t, k, device=dev, dtype=torch.bfloat16)
+                run(f"{name} prefill {n}x{k} T={t}", t, n,
+                    lambda s, x=x, blocks=blocks, tid=tid: mod.gguf_quant_gemm_prefill_forward(x, blocks, k, tid, empty))
+            del blocks
+    n = 17408
+    codes, scale = C.quantize_fp8_block(rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02))
+    codes = torch.from_numpy(codes).to(dev)
+    scale = torch.from_numpy(scale).to(dev)
+    x = torch.randn(512, k, device=dev, dtype=torch.bfloat16)
+    run(f"fp8_e4m3 prefill {n}x{k} T=512", 512, n, lambda s: mod.fp8_block_gemm_forward(x, codes, scale))
     return out
 
 

@@ -19,6 +19,38 @@ namespace {
 
 constexpr int kW13Iters = 6;
 
+// Epilogue of one 32-row tile of one route, run by lanes 0..31 of a wave (lane = row inside the tile):
+// clamp, SiLU, route weight, then the 32 hidden values are quantized in place into the image format
+// the down projection reads (one activation group).
+__device__ __forceinline__ void store_hidden(float g, float u, float limit, float route_weight, int i, int inter,
+                                             unsigned char* img, int h_kpad, int lane) {
+    if (limit > 0.0f) {
+        u = fminf(fmaxf(u, -limit), limit);
+        g = fminf(g, limit);
+    }
+    const float h = (i < inter) ? g / (1.0f + expf(-g)) * u * route_weight : 0.0f;
+    float am = fabsf(h);
+#pragma unroll
+    for (int off = 1; off < 32; off <<= 1) am = fmaxf(am, __shfl_xor(am, off, 64));
+    const float inv = am > 0.0f ? 127.0f / am : 0.0f;
+    const float scale = am * (1.0f / 127.0f);
+    const float q = fminf(fmaxf(rintf(h * inv), -127.0f), 127.0f);
+    const float l = fminf(fmaxf(rintf((h - q * scale) * inv * 254.0f), -127.0f), 127.0f);
+    float s16 = h;
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) s16 += __shfl_xor(s16, off, 64);
+    const float s32 = s16 + __shfl_xor(s16, 16, 64);
+    if (i < h_kpad) {
+        reinterpret_cast<int8_t*>(img)[i] = static_cast<int8_t>(static_cast<int>(q));
+        reinterpret_cast<int8_t*>(img + h_kpad)[i] = static_cast<int8_t>(static_cast<int>(l));
+        float2* gs = reinterpret_cast<float2*>(img + 2 * static_cast<size_t>(h_kpad));
+        float* sum16 = reinterpret_cast<float*>(gs + h_kpad / 32);
+        if ((lane & 15) == 0) sum16[i >> 4] = s16;
+        if (lane == 0) gs[i >> 5] = make_float2(scale * kLoInv, s32);
+    }
+}
+
+
 template <typename FMT>
 __global__ __launch_bounds__(256) void moe_w13_kernel(
     const unsigned char* __restrict__ x_image, size_t x_image_stride, int bpr,
@@ -64,35 +96,121 @@ __global__ __launch_bounds__(256) void moe_w13_kernel(
     acc += __shfl_xor(acc, 2, 64);
     if (j == 0) exch[mat * 32 + slot] = acc;
     __syncthreads();
-    if (tid < 32) {
-        const int i = blockIdx.x * 32 + tid;
-        float g = exch[tid], u = exch[32 + tid];
-        if (limit > 0.0f) {
-            u = fminf(fmaxf(u, -limit), limit);
-            g = fminf(g, limit);
-        }
-        const float h = (i < inter) ? g / (1.0f + expf(-g)) * u * route_weights[route] : 0.0f;
-        // quantize the 32 hidden values of this tile (one activation group of the down projection)
-        float am = fabsf(h);
+    if (tid < 32) store_hidden(exch[tid], exch[32 + tid], limit, route_weights[route], blockIdx.x * 32 + tid, inter,
+                               h_image + static_cast<size_t>(route) * h_image_stride, h_kpad, tid);
+}
+
+// ---- grouped forms: one workgroup per (row tile, expert) -----------------------------------------
+// With many tokens an expert serves several routes.  The workgroup brings up to kRouteBatch of the
+// expert's activation images into LDS and walks its rows' super-blocks kW13Iters at a time: every
+// pass of weights in registers is multiplied with all routes of the batch, so the weights cross the
+// memory system once per batch (for the usual handful of routes per expert: once per expert)
+// instead of once per route.  Per-route sums collect in LDS between the passes.
+constexpr int kRouteBatch = 8;
+
+template <typename FMT>
+__global__ __launch_bounds__(256) void moe_w13_grouped_kernel(
+    const unsigned char* __restrict__ x_image, size_t x_image_stride, int bpr,
+    const int64_t* __restrict__ route_tokens, const int32_t* __restrict__ seg, const float* __restrict__ route_weights,
+    const uint8_t* __restrict__ w1, const uint8_t* __restrict__ w3, int inter, float limit,
+    unsigned char* __restrict__ h_image, size_t h_image_stride, int h_kpad) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int kpad = bpr * 256;
+    const int image_bytes = static_cast<int>(staged_x_bytes(kpad));
+    unsigned char* tables = smem + kRouteBatch * image_bytes;
+    float* exch = reinterpret_cast<float*>(tables + FMT::kTableBytes);           // [kRouteBatch][2][32]
+
+    const int expert = blockIdx.y;
+    const int r0 = seg[expert], r1 = seg[expert + 1];
+    if (r0 >= r1) return;
+    const size_t expert_off = static_cast<size_t>(expert) * inter * bpr * FMT::kBlockBytes;
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int j = lane & 3, team = lane >> 2;
+    const int mat = wave >> 1;
+    const int slot = 16 * (wave & 1) + team;
+    const int row = min(blockIdx.x * 32 + slot, inter - 1);
+    const uint8_t* wrow = (mat ? w3 : w1) + expert_off + static_cast<size_t>(row) * bpr * FMT::kBlockBytes;
+    FMT::stage_tables(tables);
+
+    for (int rc = r0; rc < r1; rc += kRouteBatch) {
+        const int nr = min(kRouteBatch, r1 - rc);
+        for (int q = 0; q < nr; ++q)
+            copy_to_lds(smem + q * image_bytes, x_image + static_cast<size_t>(route_tokens[rc + q]) * x_image_stride, image_bytes);
+        __syncthreads();
+        for (int b0 = 0; b0 < bpr; b0 += kW13Iters) {
+            typename FMT::Regs regs[kW13Iters];
 #pragma unroll
-        for (int off = 1; off < 32; off <<= 1) am = fmaxf(am, __shfl_xor(am, off, 64));
-        const float inv = am > 0.0f ? 127.0f / am : 0.0f;
-        const float scale = am * (1.0f / 127.0f);
-        const float q = fminf(fmaxf(rintf(h * inv), -127.0f), 127.0f);
-        const float l = fminf(fmaxf(rintf((h - q * scale) * inv * 254.0f), -127.0f), 127.0f);
-        float s16 = h;
+            for (int it = 0; it < kW13Iters; ++it)
+                FMT::load(regs[it], wrow + static_cast<size_t>(min(b0 + it, bpr - 1)) * FMT::kBlockBytes, j);
+            for (int q = 0; q < nr; ++q) {
+                const StagedX sx = carve_staged_x(smem + q * image_bytes, kpad);
+                float acc = 0.0f;
 #pragma unroll
-        for (int off = 1; off < 16; off <<= 1) s16 += __shfl_xor(s16, off, 64);
-        const float s32 = s16 + __shfl_xor(s16, 16, 64);
-        unsigned char* img = h_image + static_cast<size_t>(route) * h_image_stride;
-        if (i < h_kpad) {
-            reinterpret_cast<int8_t*>(img)[i] = static_cast<int8_t>(static_cast<int>(q));
-            reinterpret_cast<int8_t*>(img + h_kpad)[i] = static_cast<int8_t>(static_cast<int>(l));
-            float2* gs = reinterpret_cast<float2*>(img + 2 * static_cast<size_t>(h_kpad));
-            float* sum16 = reinterpret_cast<float*>(gs + h_kpad / 32);
-            if ((tid & 15) == 0) sum16[i >> 4] = s16;
-            if (tid == 0) gs[i >> 5] = make_float2(scale * kLoInv, s32);
+                for (int it = 0; it < kW13Iters; ++it)
+                    if (b0 + it < bpr) acc += FMT::lane_dot(regs[it], j, b0 + it, sx, tables);
+                acc += __shfl_xor(acc, 1, 64);
+                acc += __shfl_xor(acc, 2, 64);
+                if (j == 0) {                                                    // every (route, row) slot has one owner lane
+                    float* dst = exch + q * 64 + mat * 32 + slot;
+                    *dst = b0 == 0 ? acc : *dst + acc;
+                }
+            }
         }
+        __syncthreads();
+        for (int q = wave; q < nr; q += 4)
+            if (lane < 32)
+                store_hidden(exch[q * 64 + lane], exch[q * 64 + 32 + lane], limit, route_weights[rc + q], blockIdx.x * 32 + lane, inter,
+                             h_image + static_cast<size_t>(rc + q) * h_image_stride, h_kpad, lane);
+        __syncthreads();
+    }
+}
+
+// partial[r, :] = W2_e h_r for the routes r of expert e = blockIdx.y; 64 rows per workgroup, one wave = 16 rows x all blocks
+template <typename FMT>
+__global__ __launch_bounds__(256) void moe_w2_grouped_kernel(
+    const unsigned char* __restrict__ h_image, size_t h_image_stride, int bpr, const int32_t* __restrict__ seg,
+    const uint8_t* __restrict__ w2, size_t expert_stride, float* __restrict__ partial, int dim) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int kpad = bpr * 256;
+    const int image_bytes = static_cast<int>(staged_x_bytes(kpad));
+    unsigned char* tables = smem + kRouteBatch * image_bytes;
+
+    const int expert = blockIdx.y;
+    const int r0 = seg[expert], r1 = seg[expert + 1];
+    if (r0 >= r1) return;
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int j = lane & 3, team = lane >> 2;
+    const int row = blockIdx.x * 64 + wave * 16 + team;
+    const uint8_t* wrow = w2 + static_cast<size_t>(expert) * expert_stride + static_cast<size_t>(min(row, dim - 1)) * bpr * FMT::kBlockBytes;
+    FMT::stage_tables(tables);
+
+    for (int rc = r0; rc < r1; rc += kRouteBatch) {
+        const int nr = min(kRouteBatch, r1 - rc);
+        for (int q = 0; q < nr; ++q)
+            copy_to_lds(smem + q * image_bytes, h_image + static_cast<size_t>(rc + q) * h_image_stride, image_bytes);
+        __syncthreads();
+        for (int b0 = 0; b0 < bpr; b0 += kW13Iters) {
+            typename FMT::Regs regs[kW13Iters];
+#pragma unroll
+            for (int it = 0; it < kW13Iters; ++it)
+                FMT::load(regs[it], wrow + static_cast<size_t>(min(b0 + it, bpr - 1)) * FMT::kBlockBytes, j);
+            for (int q = 0; q < nr; ++q) {
+                const StagedX sx = carve_staged_x(smem + q * image_bytes, kpad);
+                float acc = 0.0f;
+#pragma unroll
+                for (int it = 0; it < kW13Iters; ++it)
+                    if (b0 + it < bpr) acc += FMT::lane_dot(regs[it], j, b0 + it, sx, tables);
+                acc += __shfl_xor(acc, 1, 64);
+                acc += __shfl_xor(acc, 2, 64);
+                if (j == 0 && row < dim) {                                       // one owner lane per output: plain read-modify-write
+                    float* dst = partial + static_cast<size_t>(rc + q) * dim + row;
+                    *dst = b0 == 0 ? acc : *dst + acc;
+                }
+            }
+        }
+        __syncthreads();
     }
 }
 
@@ -194,6 +312,34 @@ int launch_w13(const unsigned char* x_image, size_t x_stride, int bpr, const int
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 
+template <typename FMT>
+int launch_w13_grouped(const unsigned char* x_image, size_t x_stride, int bpr, const int64_t* route_tokens, const int32_t* seg,
+                       const float* route_weights, const uint8_t* w1, const uint8_t* w3, int inter, float limit, unsigned char* h_image,
+                       size_t h_stride, int h_kpad, int n_experts, hipStream_t stream) {
+    const size_t smem = kRouteBatch * staged_x_bytes(bpr * 256) + FMT::kTableBytes + kRouteBatch * 64 * sizeof(float);
+    auto kern = moe_w13_grouped_kernel<FMT>;
+    if (smem > 160 * 1024) return PLLM_ERR_UNSUPPORTED;
+    if (smem > 64 * 1024 &&
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem)) != hipSuccess)
+        return PLLM_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(kern, dim3(h_kpad / 32, n_experts), dim3(256), smem, stream, x_image, x_stride, bpr, route_tokens, seg, route_weights,
+                       w1, w3, inter, limit, h_image, h_stride, h_kpad);
+    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+}
+
+template <typename FMT>
+int launch_w2_grouped(const unsigned char* h_image, size_t h_stride, int bpr, const int32_t* seg, const uint8_t* w2, size_t expert_stride,
+                      float* partial, int dim, int n_experts, hipStream_t stream) {
+    const size_t smem = kRouteBatch * staged_x_bytes(bpr * 256) + FMT::kTableBytes;
+    auto kern = moe_w2_grouped_kernel<FMT>;
+    if (smem > 160 * 1024) return PLLM_ERR_UNSUPPORTED;
+    if (smem > 64 * 1024 &&
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem)) != hipSuccess)
+        return PLLM_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(kern, dim3((dim + 63) / 64, n_experts), dim3(256), smem, stream, h_image, h_stride, bpr, seg, w2, expert_stride, partial, dim);
+    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+}
+
 bool dot4_type(int t) { return t == PLLM_TYPE_Q2_K || t == PLLM_TYPE_IQ2_XXS || t == PLLM_TYPE_IQ1_M; }
 
 size_t align256(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
@@ -250,6 +396,26 @@ int pllm_gguf_moe_forward(const void* x, int x_dtype, int64_t tokens, int64_t di
     if (st != PLLM_OK) return st;
 
     const int I = static_cast<int>(inter);
+    const bool grouped = seg_starts && tokens > 1;                 // several routes per expert: weights once per batch of routes
+    if (grouped) {
+        const int E = static_cast<int>(n_experts);
+        switch (w13_type) {
+            case PLLM_TYPE_IQ2_XXS: st = launch_w13_grouped<IQ2XXS>(x_image, x_stride, bpr_x, route_tokens, seg_starts, route_weights, w1, w3, I, swiglu_limit, h_image, h_stride, bpr_h * 256, E, s); break;
+            case PLLM_TYPE_IQ1_M: st = launch_w13_grouped<IQ1M>(x_image, x_stride, bpr_x, route_tokens, seg_starts, route_weights, w1, w3, I, swiglu_limit, h_image, h_stride, bpr_h * 256, E, s); break;
+            default: st = launch_w13_grouped<Q2K>(x_image, x_stride, bpr_x, route_tokens, seg_starts, route_weights, w1, w3, I, swiglu_limit, h_image, h_stride, bpr_h * 256, E, s); break;
+        }
+        if (st != PLLM_OK) return st;
+        const size_t stride2 = static_cast<size_t>(dim) * bpr_h * pllm_gguf_block_bytes(w2_type);
+        switch (w2_type) {
+            case PLLM_TYPE_IQ2_XXS: st = launch_w2_grouped<IQ2XXS>(h_image, h_stride, bpr_h, seg_starts, w2, stride2, partial, static_cast<int>(dim), E, s); break;
+            case PLLM_TYPE_IQ1_M: st = launch_w2_grouped<IQ1M>(h_image, h_stride, bpr_h, seg_starts, w2, stride2, partial, static_cast<int>(dim), E, s); break;
+            default: st = launch_w2_grouped<Q2K>(h_image, h_stride, bpr_h, seg_starts, w2, stride2, partial, static_cast<int>(dim), E, s); break;
+        }
+        if (st != PLLM_OK) return st;
+        dim3 rg(static_cast<unsigned>(tokens), static_cast<unsigned>((dim + 255) / 256));
+        hipLaunchKernelGGL(moe_reduce_kernel, rg, dim3(256), 0, s, partial, route_tokens, y, R, static_cast<int>(dim));
+        return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+    }
     switch (w13_type) {
         case PLLM_TYPE_IQ2_XXS:
             st = launch_w13<IQ2XXS>(x_image, x_stride, bpr_x, route_tokens, experts32, route_weights, w1, w3, I, swiglu_limit, h_image, h_stride, bpr_h * 256, R, s);
