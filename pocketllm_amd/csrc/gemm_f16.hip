@@ -38,9 +38,9 @@ constexpr int kLds = kBK + 8;                       // halves per LDS row: 80 by
 // ---- activation pre-pass --------------------------------------------------------------------------
 // xh[t, 0..kp) = fp16(x[t, :] * 2^-e_t) (zero beyond k), scale[t] = 2^e_t, amax_t * 2^-e_t in [2^13, 2^14)
 __global__ __launch_bounds__(256) void act_f16_kernel(const void* __restrict__ x, int x_dtype, _Float16* __restrict__ xh,
-                                                      float* __restrict__ scale, int k, int kp) {
+                                                      float* __restrict__ scale, int k, int kp, const int64_t* __restrict__ row_map) {
     __shared__ float red[4];
-    const size_t xoff = static_cast<size_t>(blockIdx.x) * k;
+    const size_t xoff = static_cast<size_t>(row_map ? row_map[blockIdx.x] : blockIdx.x) * k;      // row_map gathers source rows
     float am = 0.0f;
     for (int i = threadIdx.x; i < k; i += 256) am = fmaxf(am, fabsf(load_any(x, x_dtype, xoff + i)));
     am = group_max<64>(am);
@@ -64,10 +64,10 @@ __global__ __launch_bounds__(256) void act_f16_kernel(const void* __restrict__ x
 // bits(v) = the value as float32: bf16 is the high half of a float32, fp16 converts in hardware.
 template <bool BF16>
 __global__ __launch_bounds__(256) void act_f16_rows_kernel(const uint16_t* __restrict__ x, _Float16* __restrict__ xh,
-                                                           float* __restrict__ scale, int rows, int k, int kp) {
+                                                           float* __restrict__ scale, int rows, int k, int kp, const int64_t* __restrict__ row_map) {
     const int lane = threadIdx.x & 63, row = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= rows) return;
-    const uint16_t* src = x + static_cast<size_t>(row) * k;
+    const uint16_t* src = x + static_cast<size_t>(row_map ? row_map[row] : row) * k;
     constexpr int kMaxPieces = 16;                 // 16 pieces x 64 lanes x 8 values
     uint4 piece[kMaxPieces];
     float am = 0.0f;
@@ -109,6 +109,38 @@ __global__ __launch_bounds__(256) void act_f16_rows_kernel(const uint16_t* __res
     if (lane == 0) scale[row] = ldexpf(1.0f, e);
 }
 
+// Hidden activations of the routed experts, one wave per route: h = silu(min(g, L)) * clamp(u, +-L) * w_r
+// (L <= 0: no clamp) from the float32 gate / up products, written as fp16 rows scaled like the ones above.
+__global__ __launch_bounds__(256) void swiglu_f16_rows_kernel(const float* __restrict__ g, const float* __restrict__ u,
+                                                              const float* __restrict__ route_weights, float limit, _Float16* __restrict__ hh,
+                                                              float* __restrict__ scale, int rows, int inter, int kp) {
+    const int lane = threadIdx.x & 63, row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const float* gr = g + static_cast<size_t>(row) * inter;
+    const float* ur = u + static_cast<size_t>(row) * inter;
+    const float rw = route_weights[row];
+    auto hidden = [&](int i) {
+        float gv = gr[i], uv = ur[i];
+        if (limit > 0.0f) {
+            uv = fminf(fmaxf(uv, -limit), limit);
+            gv = fminf(gv, limit);
+        }
+        return gv / (1.0f + expf(-gv)) * uv * rw;
+    };
+    float am = 0.0f;
+    for (int i = lane; i < inter; i += 64) am = fmaxf(am, fabsf(hidden(i)));
+    am = group_max<64>(am);
+    int e = 0;
+    if (am > 0.0f && am < __uint_as_float(0x7f800000u)) {
+        (void)frexpf(am, &e);
+        e -= 14;
+    }
+    const float down = ldexpf(1.0f, -e);
+    _Float16* out = hh + static_cast<size_t>(row) * kp;
+    for (int i = lane; i < kp; i += 64) out[i] = static_cast<_Float16>(i < inter ? hidden(i) * down : 0.0f);
+    if (lane == 0) scale[row] = ldexpf(1.0f, e);
+}
+
 // ---- per-format decode of one 32-weight chunk -----------------------------------------------------
 // Staging thread (row, h) decodes weights [32 j + 16 h, +16) of its row for sub-block j = 2 p + e.
 struct K4Scale { float d_sc, dm; };
@@ -142,13 +174,15 @@ __device__ __forceinline__ half4 affine4(uint32_t codes, float scale, float minu
 struct Half16 { half4 a, b, c, d; };
 
 struct GQ4K {
+    static constexpr int kTableBytes = 0;
+    static __device__ __forceinline__ void stage_table(unsigned char*) {}
     static constexpr int kBlockBytes = 144;
     struct Regs { uint4 hdr; uint4 qs; };
     static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, const float*, int, int p, int h) {
         r.hdr = *reinterpret_cast<const uint4*>(blk);
         r.qs = *reinterpret_cast<const uint4*>(blk + 16 + 32 * p + 16 * h);
     }
-    static __device__ __forceinline__ void decode(const Regs& r, int p, int e, Half16& o) {
+    static __device__ __forceinline__ void decode(const Regs& r, int p, int e, int, const unsigned char*, Half16& o) {
         const K4Scale s = k4_scale(r.hdr, p, e);
         const int sft = 4 * e;
         o.a = affine4((r.qs.x >> sft) & 0x0f0f0f0fu, s.d_sc, s.dm);
@@ -159,6 +193,8 @@ struct GQ4K {
 };
 
 struct GQ5K {
+    static constexpr int kTableBytes = 0;
+    static __device__ __forceinline__ void stage_table(unsigned char*) {}
     static constexpr int kBlockBytes = 176;
     struct Regs { uint4 hdr; uint4 qh; uint4 qs; };
     static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, const float*, int, int p, int h) {
@@ -169,7 +205,7 @@ struct GQ5K {
     static __device__ __forceinline__ uint32_t codes(uint32_t q, uint32_t g, int sft, int bit) {
         return ((q >> sft) & 0x0f0f0f0fu) | (((g >> bit) & 0x01010101u) << 4);
     }
-    static __device__ __forceinline__ void decode(const Regs& r, int p, int e, Half16& o) {
+    static __device__ __forceinline__ void decode(const Regs& r, int p, int e, int, const unsigned char*, Half16& o) {
         const K4Scale s = k4_scale(r.hdr, p, e);
         const int sft = 4 * e, bit = 2 * p + e;
         o.a = affine4(codes(r.qs.x, r.qh.x, sft, bit), s.d_sc, s.dm);
@@ -179,10 +215,141 @@ struct GQ5K {
     }
 };
 
+// Q2_K: 84 B = scales(16) qs(64) d(2) dmin(2).  Chunk c = 2 p + e holds weights [32 c, +32): byte
+// qs[32 (c / 4) + l] >> 2 (c % 4), l = 0..31, so both chunks of a pair read the same 16 bytes per
+// thread at two shifts; the thread's 16 weights are group 2 c + h with scale byte scales[2 c + h]
+// (low nibble scale, high nibble min).
+struct GQ2K {
+    static constexpr int kTableBytes = 0;
+    static __device__ __forceinline__ void stage_table(unsigned char*) {}
+    static constexpr int kBlockBytes = 84;
+    struct Regs { uint4 sc; uint4 qs; uint32_t dd; };
+    static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, const float*, int, int p, int h) {
+        const uint32_t* w = reinterpret_cast<const uint32_t*>(blk);           // blocks are 4-byte aligned
+        r.sc = make_uint4(w[0], w[1], w[2], w[3]);
+        const uint32_t* q = w + 4 + 8 * (p >> 1) + 4 * h;
+        r.qs = make_uint4(q[0], q[1], q[2], q[3]);
+        r.dd = w[20];
+    }
+    static __device__ __forceinline__ void decode(const Regs& r, int p, int e, int h, const unsigned char*, Half16& o) {
+        const int c = 2 * p + e, sft = 2 * (c & 3), g = 2 * c + h;
+        const uint32_t word = (g < 4) ? r.sc.x : (g < 8) ? r.sc.y : (g < 12) ? r.sc.z : r.sc.w;
+        const uint32_t sb = (word >> (8 * (g & 3))) & 0xffu;
+        const float scale = f16_bits_to_float(r.dd & 0xffffu) * static_cast<float>(sb & 15u);
+        const float minus = f16_bits_to_float(r.dd >> 16) * static_cast<float>(sb >> 4);
+        o.a = affine4((r.qs.x >> sft) & 0x03030303u, scale, minus);
+        o.b = affine4((r.qs.y >> sft) & 0x03030303u, scale, minus);
+        o.c = affine4((r.qs.z >> sft) & 0x03030303u, scale, minus);
+        o.d = affine4((r.qs.w >> sft) & 0x03030303u, scale, minus);
+    }
+};
+
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+
+// two fp16 values in a dword, sign bits flipped by `flip`, times a float32 scale, rounded once to fp16
+// (mixed-precision multiplies: the scale keeps its float32 bits)
+__device__ __forceinline__ uint32_t scaled_pair(uint32_t bits, uint32_t flip, float scale) {
+    const half2v v = __builtin_bit_cast(half2v, bits ^ flip);
+    const half2v r = {static_cast<_Float16>(static_cast<float>(v.x) * scale), static_cast<_Float16>(static_cast<float>(v.y) * scale)};
+    return __builtin_bit_cast(uint32_t, r);
+}
+__device__ __forceinline__ half4 half4_of(uint32_t lo, uint32_t hi) {
+    return __builtin_bit_cast(half4, make_uint2(lo, hi));
+}
+
+// IQ2_XXS: 66 B = d(2) + 8 sub-blocks of 8 B (four grid ids, then a u32: four 7-bit sign indices and a
+// 4-bit scale).  A pair is sub-blocks 2 p and 2 p + 1; the thread takes grid entries 2 h and 2 h + 1 of
+// its sub-block.  w = d (2 s + 1) / 8 * magnitude, negated where the sign pattern (seven bits plus
+// their parity) says so.  The workgroup keeps two LDS tables in fp16: the 256 x 8 magnitudes (8, 25
+// and 43 are exact) and the 128 x 8 sign-bit masks, so eight weights cost two 16-byte LDS reads, four
+// XORs and eight mixed-precision multiplies by the float32 scale.
+struct GIQ2XXS {
+    static constexpr int kBlockBytes = 66;
+    struct Regs { uint4 q; uint32_t d; };
+    static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, const float*, int, int p, int) {
+        r.q = load16_a2(blk + 2 + 16 * p);
+        r.d = *reinterpret_cast<const uint16_t*>(blk);
+    }
+    static constexpr int kTableBytes = 4096 + 2048;
+    static __device__ __forceinline__ void stage_table(unsigned char* lds) {
+        _Float16* mag = reinterpret_cast<_Float16*>(lds);
+        uint16_t* sgn = reinterpret_cast<uint16_t*>(lds + 4096);
+        for (int i = threadIdx.x; i < 256 * 8; i += kThreads)
+            mag[i] = static_cast<_Float16>(static_cast<float>((PLLM_IQ2XXS_GRID[i >> 3] >> (8 * (i & 7))) & 0xffull));
+        for (int i = threadIdx.x; i < 128 * 8; i += kThreads) {
+            const uint32_t s7 = static_cast<uint32_t>(i >> 3);
+            const uint32_t s8 = s7 | ((__popc(s7) & 1u) << 7);
+            sgn[i] = ((s8 >> (i & 7)) & 1u) ? 0x8000u : 0u;
+        }
+    }
+    static __device__ __forceinline__ void entry(const unsigned char* table, uint32_t id, uint32_t s7, float scale, half4& lo, half4& hi) {
+        const uint4 m = *reinterpret_cast<const uint4*>(table + 16 * id);
+        const uint4 f = *reinterpret_cast<const uint4*>(table + 4096 + 16 * s7);
+        lo = half4_of(scaled_pair(m.x, f.x, scale), scaled_pair(m.y, f.y, scale));
+        hi = half4_of(scaled_pair(m.z, f.z, scale), scaled_pair(m.w, f.w, scale));
+    }
+    static __device__ __forceinline__ void decode(const Regs& r, int, int e, int h, const unsigned char* table, Half16& o) {
+        const uint32_t ids = e ? r.q.z : r.q.x, aux = e ? r.q.w : r.q.y;
+        const float scale = 0.125f * f16_bits_to_float(r.d) * static_cast<float>(2 * (aux >> 28) + 1);
+        entry(table, (ids >> (16 * h)) & 0xffu, (aux >> (14 * h)) & 127u, scale, o.a, o.b);
+        entry(table, (ids >> (16 * h + 8)) & 0xffu, (aux >> (14 * h + 7)) & 127u, scale, o.c, o.d);
+    }
+};
+
+// IQ1_M: 56 B = qs(32) qh(16) scales(8).  One codebook index per 8 weights (qs byte plus the low three
+// bits of its qh nibble; bit 3 of the nibble picks delta = -+0.125); sixteen 3-bit scales, one per 16
+// weights, in the low 12 bits of four u16 words whose top nibbles spell the fp16 block scale.
+// The thread's 16 weights are entries 8 p + 4 e + 2 h and the next one, scale group 4 p + 2 e + h.
+// LDS holds the 2048 x 16-bit codebook (two bits per element, value + 1) and a 2 x 16 table of fp16
+// pairs: for a delta and the four bits of two neighbouring elements, the pair (c0 - 1 + delta,
+// c1 - 1 + delta), all of them exact in fp16; mixed-precision multiplies by the float32 scale finish them.
+struct GIQ1M {
+    static constexpr int kBlockBytes = 56;
+    struct Regs { uint2 qs; uint32_t qh; uint2 sc; };
+    static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, const float*, int, int p, int) {
+        r.qs = *reinterpret_cast<const uint2*>(blk + 8 * p);                  // blocks are 8-byte aligned
+        r.qh = *reinterpret_cast<const uint32_t*>(blk + 32 + 4 * p);
+        r.sc = *reinterpret_cast<const uint2*>(blk + 48);
+    }
+    static constexpr int kTableBytes = 4096 + 128;
+    static __device__ __forceinline__ void stage_table(unsigned char* lds) {
+        uint16_t* t = reinterpret_cast<uint16_t*>(lds);
+        for (int i = threadIdx.x; i < 2048; i += kThreads) t[i] = PLLM_IQ1_GRID_PACKED[i];
+        half2v* pairs = reinterpret_cast<half2v*>(lds + 4096);
+        for (int i = threadIdx.x; i < 32; i += kThreads) {
+            const float delta = (i & 16) ? -0.125f : 0.125f;
+            pairs[i] = half2v{static_cast<_Float16>(static_cast<float>(i & 3) - 1.0f + delta),
+                              static_cast<_Float16>(static_cast<float>((i >> 2) & 3) - 1.0f + delta)};
+        }
+    }
+    static __device__ __forceinline__ void entry(const unsigned char* table, uint32_t qb, uint32_t nib, float scale, half4& lo, half4& hi) {
+        const uint32_t packed = reinterpret_cast<const uint16_t*>(table)[qb | ((nib & 7u) << 8)];      // element k in bits [2k, 2k+1], value + 1
+        const uint32_t* pairs = reinterpret_cast<const uint32_t*>(table + 4096) + ((nib & 8u) << 1);  // the delta's half of the pair table
+        const uint32_t w0 = scaled_pair(pairs[packed & 15u], 0u, scale), w1 = scaled_pair(pairs[(packed >> 4) & 15u], 0u, scale);
+        const uint32_t w2 = scaled_pair(pairs[(packed >> 8) & 15u], 0u, scale), w3 = scaled_pair(pairs[(packed >> 12) & 15u], 0u, scale);
+        lo = half4_of(w0, w1);
+        hi = half4_of(w2, w3);
+    }
+    static __device__ __forceinline__ void decode(const Regs& r, int p, int e, int h, const unsigned char* table, Half16& o) {
+        const uint32_t s01 = r.sc.x, s23 = r.sc.y;
+        const uint32_t dbits = ((s01 >> 12) & 0xfu) | ((s01 >> 24) & 0xf0u) | ((s23 >> 4) & 0xf00u) | ((s23 >> 16) & 0xf000u);
+        const int grp = 4 * p + 2 * e + h;                                     // 16-weight scale group of the block
+        const uint32_t word = ((grp & 8) ? s23 : s01) >> (16 * ((grp >> 2) & 1));
+        const float scale = f16_bits_to_float(dbits) * static_cast<float>(2 * ((word >> (3 * (grp & 3))) & 7u) + 1);
+        const int en = 4 * e + 2 * h;                                          // entry inside the pair, 0..7
+        const uint32_t qw = (en < 4) ? r.qs.x : r.qs.y;
+        const uint32_t q0 = (qw >> (8 * (en & 3))) & 0xffu, q1 = (qw >> (8 * (en & 3) + 8)) & 0xffu;
+        entry(table, q0, (r.qh >> (4 * en)) & 15u, scale, o.a, o.b);
+        entry(table, q1, (r.qh >> (4 * en + 4)) & 15u, scale, o.c, o.d);
+    }
+};
+
 // FP8 E4M3 (OCP) codes, one byte per weight, rows of k bytes with k a multiple of 256 here; a
 // "block" is 256 consecutive codes of a row and carries no header.  The float32 scale of the
 // 128 x 128 block is folded into the fp16 weight: fp16(f32(code) * scale).
 struct GFP8 {
+    static constexpr int kTableBytes = 0;
+    static __device__ __forceinline__ void stage_table(unsigned char*) {}
     static constexpr int kBlockBytes = 256;
     struct Regs { uint4 q0, q1; float scale; };
     static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, const float* srow, int b, int p, int h) {
@@ -199,7 +366,7 @@ struct GFP8 {
         o.z = static_cast<_Float16>(hi.x * sc); o.w = static_cast<_Float16>(hi.y * sc);
         return o;
     }
-    static __device__ __forceinline__ void decode(const Regs& r, int, int e, Half16& o) {
+    static __device__ __forceinline__ void decode(const Regs& r, int, int e, int, const unsigned char*, Half16& o) {
         const uint4 q = e ? r.q1 : r.q0;
         o.a = word(q.x, r.scale); o.b = word(q.y, r.scale); o.c = word(q.z, r.scale); o.d = word(q.w, r.scale);
     }
@@ -209,16 +376,21 @@ struct GFP8 {
 // Workgroups [0, full_tiles) take whole tiles and store scaled results into y; workgroup
 // full_tiles + r takes slice r % slices of tile full_tiles + r / slices and stores raw float32 sums
 // into partial[r][kBM][kBN].  Tiles are numbered along N first.
+// With `seg` the launch is a batch of matmuls (routed experts): grid.y counts the groups, every group
+// has its own weight matrix and a run of activation / output rows, and its tiles along the tokens are
+// counted from the start of that run (workgroups past the end of a short run leave at once).
 template <typename FMT, int MI>
 __global__ __launch_bounds__(kThreads) void gemm_f16_kernel(
     const _Float16* __restrict__ xh, const float* __restrict__ xscale, const uint8_t* __restrict__ w,
     void* __restrict__ y, int y_dtype, float* __restrict__ partial, int t_rows, int n, int bpr,
-    int tiles_n, int full_tiles, int slices, const float* __restrict__ wscale, int scale_kb) {
+    int tiles_n, int full_tiles, int slices, const float* __restrict__ wscale, int scale_kb,
+    const int32_t* __restrict__ seg, size_t group_stride) {
     constexpr int kBM = 64 * MI;
     constexpr int kXTile = kBM * kLds, kWTile = kBN * kLds;
     extern __shared__ __align__(16) unsigned char smem[];
     _Float16* xs_buf = reinterpret_cast<_Float16*>(smem);                 // [2][kBM][kLds]
     _Float16* ws_buf = xs_buf + 2 * kXTile;                               // [2][kBN][kLds]
+    unsigned char* table = reinterpret_cast<unsigned char*>(ws_buf + 2 * kWTile);   // the format's codebook, if any
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -228,7 +400,16 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_kernel(
     const int rest = wg - full_tiles;
     const int tile = whole ? wg : full_tiles + rest / slices;
     const int slice = whole ? 0 : rest % slices, nsl = whole ? 1 : slices;
-    const int n0 = (tile % tiles_n) * kBN, t0 = (tile / tiles_n) * kBM;
+    const int n0 = (tile % tiles_n) * kBN;
+    int t0 = (tile / tiles_n) * kBM;
+    if (seg) {
+        // grouped: group blockIdx.y owns activation rows [seg[g], seg[g + 1]) and the matrix at w + g * group_stride
+        const int g = blockIdx.y;
+        t0 += seg[g];
+        t_rows = seg[g + 1];
+        if (t0 >= t_rows) return;
+        w += static_cast<size_t>(g) * group_stride;
+    }
     const int kp = bpr * 256;
     const int b0 = static_cast<int>(static_cast<long long>(slice) * bpr / nsl);
     const int b1 = static_cast<int>(static_cast<long long>(slice + 1) * bpr / nsl);
@@ -274,7 +455,7 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_kernel(
     };
     auto stage = [&](int p, int e, int buf, const typename FMT::Regs& wr, const uint4& x0, const uint4& x1) {
         Half16 d;
-        FMT::decode(wr, p, e, d);
+        FMT::decode(wr, p, e, sh, table, d);
         half4* wdst = reinterpret_cast<half4*>(ws_buf + buf * kWTile + srow * kLds + 16 * sh);
         wdst[0] = d.a; wdst[1] = d.b; wdst[2] = d.c; wdst[3] = d.d;
         if (xmover) {
@@ -317,6 +498,10 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_kernel(
     // Past the end the loop re-fetches and re-stages the last block instead of branching: nobody reads it.
     fetch(b0, 0, wset0, xa0, xa1, xa2, xa3);
     fetch(b0, 1, wset1, xb0, xb1, xb2, xb3);
+    if constexpr (FMT::kTableBytes > 0) {
+        FMT::stage_table(table);
+        __syncthreads();
+    }
     stage(0, 0, 0, wset0, xa0, xa1);
     __syncthreads();
     for (int blk = b0; blk < b1; ++blk) {
@@ -414,16 +599,17 @@ GemmPlan plan_gemm(int t_rows, int n, int bpr) {
 
 template <typename FMT, int MI>
 int launch_gemm(const GemmPlan& p, const _Float16* xh, const float* xscale, const uint8_t* w, void* y, int y_dtype, float* partial,
-                int t_rows, int n, int bpr, const float* wscale, int scale_kb, hipStream_t stream) {
-    const size_t smem = static_cast<size_t>(2) * (64 * MI + kBN) * kLds * sizeof(_Float16);
+                int t_rows, int n, int bpr, const float* wscale, int scale_kb, const int32_t* seg, size_t group_stride, int groups,
+                hipStream_t stream) {
+    const size_t smem = static_cast<size_t>(2) * (64 * MI + kBN) * kLds * sizeof(_Float16) + FMT::kTableBytes;
     auto kern = gemm_f16_kernel<FMT, MI>;
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem)) != hipSuccess)
         return PLLM_ERR_UNSUPPORTED;
     const int rem = p.tiles - p.full_tiles;
     const int full = p.slices > 1 ? p.full_tiles : p.tiles;             // unsplit left-over tiles are whole tiles too
     const int grid = full + (p.slices > 1 ? rem * p.slices : 0);
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), smem, stream, xh, xscale, w, y, y_dtype, partial, t_rows, n, bpr,
-                       p.tiles_n, full, p.slices, wscale, scale_kb);
+    hipLaunchKernelGGL(kern, dim3(grid, seg ? groups : 1), dim3(kThreads), smem, stream, xh, xscale, w, y, y_dtype, partial, t_rows, n, bpr,
+                       p.tiles_n, full, p.slices, wscale, scale_kb, seg, group_stride);
     if (hipGetLastError() != hipSuccess) return PLLM_ERR_LAUNCH;
     if (p.slices > 1) {
         hipLaunchKernelGGL(gemm_reduce_kernel, dim3(64 * MI * kBN / 1024, rem), dim3(256), 0, stream, partial, xscale, y, y_dtype, t_rows, n,
@@ -435,11 +621,12 @@ int launch_gemm(const GemmPlan& p, const _Float16* xh, const float* xscale, cons
 
 template <typename FMT>
 int launch_gemm_mi(const GemmPlan& p, const _Float16* xh, const float* xscale, const uint8_t* w, void* y, int y_dtype, float* partial,
-                   int t_rows, int n, int bpr, const float* wscale, int scale_kb, hipStream_t stream) {
+                   int t_rows, int n, int bpr, const float* wscale, int scale_kb, const int32_t* seg, size_t group_stride, int groups,
+                   hipStream_t stream) {
     switch (p.mi) {
-        case 1: return launch_gemm<FMT, 1>(p, xh, xscale, w, y, y_dtype, partial, t_rows, n, bpr, wscale, scale_kb, stream);
-        case 2: return launch_gemm<FMT, 2>(p, xh, xscale, w, y, y_dtype, partial, t_rows, n, bpr, wscale, scale_kb, stream);
-        default: return launch_gemm<FMT, 4>(p, xh, xscale, w, y, y_dtype, partial, t_rows, n, bpr, wscale, scale_kb, stream);
+        case 1: return launch_gemm<FMT, 1>(p, xh, xscale, w, y, y_dtype, partial, t_rows, n, bpr, wscale, scale_kb, seg, group_stride, groups, stream);
+        case 2: return launch_gemm<FMT, 2>(p, xh, xscale, w, y, y_dtype, partial, t_rows, n, bpr, wscale, scale_kb, seg, group_stride, groups, stream);
+        default: return launch_gemm<FMT, 4>(p, xh, xscale, w, y, y_dtype, partial, t_rows, n, bpr, wscale, scale_kb, seg, group_stride, groups, stream);
     }
 }
 
@@ -447,7 +634,10 @@ size_t align256(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
 
 }  // namespace
 
-bool gemm_f16_supports(int type_id) { return type_id == PLLM_TYPE_Q4_K || type_id == PLLM_TYPE_Q5_K; }
+bool gemm_f16_supports(int type_id) {
+    return type_id == PLLM_TYPE_Q4_K || type_id == PLLM_TYPE_Q5_K || type_id == PLLM_TYPE_Q2_K || type_id == PLLM_TYPE_IQ2_XXS ||
+           type_id == PLLM_TYPE_IQ1_M;
+}
 
 size_t gemm_f16_workspace_bytes(int rows, int n, int bpr) {
     const GemmPlan p = plan_gemm(rows, n, bpr);
@@ -458,7 +648,7 @@ size_t gemm_f16_workspace_bytes(int rows, int n, int bpr) {
 namespace {
 // activations -> fp16 rows + per-row scales at the head of the workspace; returns the partial-tile area
 float* stage_activations(const void* x, int x_dtype, int rows, int k, int bpr, void* workspace, const _Float16*& xh_out, const float*& xscale_out,
-                         hipStream_t stream) {
+                         hipStream_t stream, const int64_t* row_map = nullptr) {
     unsigned char* base = static_cast<unsigned char*>(workspace);
     _Float16* xh = reinterpret_cast<_Float16*>(base);
     base += align256(static_cast<size_t>(rows) * bpr * 256 * sizeof(_Float16));
@@ -467,11 +657,11 @@ float* stage_activations(const void* x, int x_dtype, int rows, int k, int bpr, v
     const bool narrow = (x_dtype == PLLM_BF16 || x_dtype == PLLM_F16) && k % 8 == 0 && bpr * 256 <= 8192 &&
                         reinterpret_cast<uintptr_t>(x) % 16 == 0;
     if (narrow && x_dtype == PLLM_BF16)
-        hipLaunchKernelGGL(act_f16_rows_kernel<true>, dim3((rows + 3) / 4), dim3(256), 0, stream, static_cast<const uint16_t*>(x), xh, xscale, rows, k, bpr * 256);
+        hipLaunchKernelGGL(act_f16_rows_kernel<true>, dim3((rows + 3) / 4), dim3(256), 0, stream, static_cast<const uint16_t*>(x), xh, xscale, rows, k, bpr * 256, row_map);
     else if (narrow)
-        hipLaunchKernelGGL(act_f16_rows_kernel<false>, dim3((rows + 3) / 4), dim3(256), 0, stream, static_cast<const uint16_t*>(x), xh, xscale, rows, k, bpr * 256);
+        hipLaunchKernelGGL(act_f16_rows_kernel<false>, dim3((rows + 3) / 4), dim3(256), 0, stream, static_cast<const uint16_t*>(x), xh, xscale, rows, k, bpr * 256, row_map);
     else
-        hipLaunchKernelGGL(act_f16_kernel, dim3(rows), dim3(256), 0, stream, x, x_dtype, xh, xscale, k, bpr * 256);
+        hipLaunchKernelGGL(act_f16_kernel, dim3(rows), dim3(256), 0, stream, x, x_dtype, xh, xscale, k, bpr * 256, row_map);
     xh_out = xh;
     xscale_out = xscale;
     return reinterpret_cast<float*>(base);
@@ -487,8 +677,11 @@ int gemm_f16(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y,
     float* partial = stage_activations(x, x_dtype, rows, k, bpr, workspace, xh, xscale, stream);
     if (hipGetLastError() != hipSuccess) return PLLM_ERR_LAUNCH;
     switch (type_id) {
-        case PLLM_TYPE_Q4_K: return launch_gemm_mi<GQ4K>(p, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, nullptr, 0, stream);
-        case PLLM_TYPE_Q5_K: return launch_gemm_mi<GQ5K>(p, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, nullptr, 0, stream);
+        case PLLM_TYPE_Q4_K: return launch_gemm_mi<GQ4K>(p, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, nullptr, 0, nullptr, 0, 1, stream);
+        case PLLM_TYPE_Q5_K: return launch_gemm_mi<GQ5K>(p, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, nullptr, 0, nullptr, 0, 1, stream);
+        case PLLM_TYPE_Q2_K: return launch_gemm_mi<GQ2K>(p, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, nullptr, 0, nullptr, 0, 1, stream);
+        case PLLM_TYPE_IQ2_XXS: return launch_gemm_mi<GIQ2XXS>(p, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, nullptr, 0, nullptr, 0, 1, stream);
+        case PLLM_TYPE_IQ1_M: return launch_gemm_mi<GIQ1M>(p, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, nullptr, 0, nullptr, 0, 1, stream);
         default: return PLLM_ERR_UNSUPPORTED;
     }
 }
@@ -504,7 +697,50 @@ int gemm_f16_fp8(const void* x, int x_dtype, const uint8_t* w, const float* wsca
     const float* xscale;
     float* partial = stage_activations(x, x_dtype, rows, k, bpr, workspace, xh, xscale, stream);
     if (hipGetLastError() != hipSuccess) return PLLM_ERR_LAUNCH;
-    return launch_gemm_mi<GFP8>(p, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, wscale, k / 128, stream);
+    return launch_gemm_mi<GFP8>(p, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, wscale, k / 128, nullptr, 0, 1, stream);
+}
+
+// ---- routed experts as a batch of tile matmuls ---------------------------------------------------------
+size_t gemm_f16_staged_bytes(int rows, int bpr) {
+    return align256(static_cast<size_t>(rows) * bpr * 256 * sizeof(_Float16)) + align256(static_cast<size_t>(rows) * sizeof(float));
+}
+
+// x rows gathered through row_map (route -> token) into fp16 rows + scales at `staged` (gemm_f16_staged_bytes bytes)
+int gemm_f16_stage_rows(const void* x, int x_dtype, const int64_t* row_map, int rows, int k, int bpr, void* staged, hipStream_t stream) {
+    const _Float16* xh;
+    const float* xscale;
+    (void)stage_activations(x, x_dtype, rows, k, bpr, staged, xh, xscale, stream, row_map);
+    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+}
+
+int gemm_f16_stage_swiglu(const float* g, const float* u, const float* route_weights, float limit, int rows, int inter, int bpr, void* staged,
+                          hipStream_t stream) {
+    _Float16* hh = static_cast<_Float16*>(staged);
+    float* hscale = reinterpret_cast<float*>(static_cast<unsigned char*>(staged) + align256(static_cast<size_t>(rows) * bpr * 256 * sizeof(_Float16)));
+    hipLaunchKernelGGL(swiglu_f16_rows_kernel, dim3((rows + 3) / 4), dim3(256), 0, stream, g, u, route_weights, limit, hh, hscale, rows, inter, bpr * 256);
+    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+}
+
+// y[r, :] (float32 [rows, n]) = staged row r . dequant(W_g)^T for r in [seg[g], seg[g + 1]); no group has more than max_group_rows rows
+int gemm_f16_grouped(const void* staged, const uint8_t* w, int type_id, size_t group_stride, const int32_t* seg, int groups,
+                     float* y, int rows, int max_group_rows, int n, int bpr, hipStream_t stream) {
+    const _Float16* xh = static_cast<const _Float16*>(staged);
+    const float* xscale = reinterpret_cast<const float*>(static_cast<const unsigned char*>(staged) + align256(static_cast<size_t>(rows) * bpr * 256 * sizeof(_Float16)));
+    const int avg = (rows + groups - 1) / groups;
+    GemmPlan p;
+    p.mi = avg <= 48 ? 1 : (avg <= 128 ? 2 : 4);
+    p.tiles_n = (n + kBN - 1) / kBN;
+    p.tiles = p.tiles_n * ((max_group_rows + 64 * p.mi - 1) / (64 * p.mi));
+    p.full_tiles = p.tiles;
+    p.slices = 1;
+    switch (type_id) {
+        case PLLM_TYPE_Q4_K: return launch_gemm_mi<GQ4K>(p, xh, xscale, w, y, PLLM_F32, nullptr, rows, n, bpr, nullptr, 0, seg, group_stride, groups, stream);
+        case PLLM_TYPE_Q5_K: return launch_gemm_mi<GQ5K>(p, xh, xscale, w, y, PLLM_F32, nullptr, rows, n, bpr, nullptr, 0, seg, group_stride, groups, stream);
+        case PLLM_TYPE_Q2_K: return launch_gemm_mi<GQ2K>(p, xh, xscale, w, y, PLLM_F32, nullptr, rows, n, bpr, nullptr, 0, seg, group_stride, groups, stream);
+        case PLLM_TYPE_IQ2_XXS: return launch_gemm_mi<GIQ2XXS>(p, xh, xscale, w, y, PLLM_F32, nullptr, rows, n, bpr, nullptr, 0, seg, group_stride, groups, stream);
+        case PLLM_TYPE_IQ1_M: return launch_gemm_mi<GIQ1M>(p, xh, xscale, w, y, PLLM_F32, nullptr, rows, n, bpr, nullptr, 0, seg, group_stride, groups, stream);
+        default: return PLLM_ERR_UNSUPPORTED;
+    }
 }
 
 }  // namespace pllm

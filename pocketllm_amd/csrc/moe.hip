@@ -15,6 +15,9 @@
 #include "pllm_internal.h"
 
 namespace pllm {
+// from this many tokens on, an expert's routes are multiplied as one tile matmul on the matrix cores
+constexpr int kMoeGemmMinTokens = 16;
+
 namespace {
 
 constexpr int kW13Iters = 6;
@@ -231,15 +234,42 @@ __global__ void narrow_experts_kernel(const int64_t* __restrict__ src, int32_t* 
     if (r < routes) dst[r] = static_cast<int32_t>(src[r]);
 }
 
-// y[t, d] = sum_{r : route_tokens[r] == t} partial[r, d], ascending r.  grid (tokens, ceil(dim / 256))
+// y[t, d] = sum_{r : route_tokens[r] == t} partial[r, d], ascending r.  grid (tokens, ceil(dim / 256)).
+// The workgroup first lists the routes of its token in LDS (every thread scans a contiguous run of
+// the route table, an exclusive scan of the per-thread counts keeps the list in route order), then
+// adds them.  route_tokens == nullptr: a single token owns every route.
+constexpr int kReduceList = 2048;
 __global__ __launch_bounds__(256) void moe_reduce_kernel(const float* __restrict__ partial, const int64_t* __restrict__ route_tokens,
                                                          float* __restrict__ y, int routes, int dim) {
-    const int t = blockIdx.x;
-    const int d = blockIdx.y * 256 + threadIdx.x;
+    __shared__ int list[kReduceList];
+    __shared__ int offs[257];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const int d = blockIdx.y * 256 + tid;
     float acc = 0.0f;
-    for (int r = 0; r < routes; ++r) {
-        const bool mine = route_tokens ? (route_tokens[r] == t) : true;         // uniform across the workgroup
-        if (mine && d < dim) acc += partial[static_cast<size_t>(r) * dim + d];
+    if (!route_tokens) {
+        if (d < dim)
+            for (int r = 0; r < routes; ++r) acc += partial[static_cast<size_t>(r) * dim + d];
+    } else if (routes <= kReduceList) {
+        const int per = (routes + 255) / 256;
+        const int r0 = min(tid * per, routes), r1 = min(r0 + per, routes);
+        int cnt = 0;
+        for (int r = r0; r < r1; ++r) cnt += route_tokens[r] == t;
+        offs[tid + 1] = cnt;
+        if (tid == 0) offs[0] = 0;
+        __syncthreads();
+        if (tid == 0)
+            for (int i = 1; i <= 256; ++i) offs[i] += offs[i - 1];
+        __syncthreads();
+        int pos = offs[tid];
+        for (int r = r0; r < r1; ++r)
+            if (route_tokens[r] == t) list[pos++] = r;
+        __syncthreads();
+        const int total = offs[256];
+        if (d < dim)
+            for (int i = 0; i < total; ++i) acc += partial[static_cast<size_t>(list[i]) * dim + d];
+    } else if (d < dim) {
+        for (int r = 0; r < routes; ++r)
+            if (route_tokens[r] == t) acc += partial[static_cast<size_t>(r) * dim + d];
     }
     if (d < dim) y[static_cast<size_t>(t) * dim + d] = acc;
 }
@@ -352,8 +382,14 @@ extern "C" {
 size_t pllm_gguf_moe_workspace_bytes(int64_t tokens, int64_t routes, int64_t dim, int64_t inter) {
     if (tokens <= 0 || routes < 0 || dim <= 0 || inter <= 0) return 0;
     const int bpr_x = static_cast<int>((dim + 255) / 256), bpr_h = static_cast<int>((inter + 255) / 256);
-    return pllm::act_image_256_bytes(bpr_x) * static_cast<size_t>(tokens) + pllm::act_image_256_bytes(bpr_h) * static_cast<size_t>(routes) +
-           pllm::align256(static_cast<size_t>(routes) * dim * sizeof(float)) + pllm::align256(static_cast<size_t>(routes) * sizeof(int32_t)) + 256;
+    const size_t dot_path = pllm::act_image_256_bytes(bpr_x) * static_cast<size_t>(tokens) + pllm::act_image_256_bytes(bpr_h) * static_cast<size_t>(routes) +
+                            pllm::align256(static_cast<size_t>(routes) * dim * sizeof(float)) + pllm::align256(static_cast<size_t>(routes) * sizeof(int32_t)) + 256;
+    if (tokens < pllm::kMoeGemmMinTokens || routes > INT32_MAX) return dot_path;
+    const int R = static_cast<int>(routes);
+    const size_t tile_path = pllm::gemm_f16_staged_bytes(R, bpr_x) + pllm::gemm_f16_staged_bytes(R, bpr_h) +
+                             2 * pllm::align256(static_cast<size_t>(routes) * inter * sizeof(float)) +
+                             pllm::align256(static_cast<size_t>(routes) * dim * sizeof(float)) + 256;
+    return dot_path > tile_path ? dot_path : tile_path;
 }
 
 int pllm_gguf_moe_forward(const void* x, int x_dtype, int64_t tokens, int64_t dim, int64_t inter,
@@ -377,6 +413,34 @@ int pllm_gguf_moe_forward(const void* x, int x_dtype, int64_t tokens, int64_t di
     if (!workspace || workspace_bytes < pllm_gguf_moe_workspace_bytes(tokens, routes, dim, inter)) return PLLM_ERR_WORKSPACE;
 
     const int bpr_x = static_cast<int>((dim + 255) / 256), bpr_h = static_cast<int>((inter + 255) / 256);
+    if (seg_starts && tokens >= kMoeGemmMinTokens) {
+        // tile path: gather the routes' activation rows as fp16, gate and up as two batches of tile
+        // matmuls (one group per expert), SwiGLU into fp16 hidden rows, down as a third batch, then
+        // the ordered sum of every token's routes
+        const int R = static_cast<int>(routes), E = static_cast<int>(n_experts), I = static_cast<int>(inter), D = static_cast<int>(dim);
+        unsigned char* p = static_cast<unsigned char*>(workspace);
+        void* x_staged = p;  p += gemm_f16_staged_bytes(R, bpr_x);
+        void* h_staged = p;  p += gemm_f16_staged_bytes(R, bpr_h);
+        float* gate = reinterpret_cast<float*>(p);  p += align256(static_cast<size_t>(R) * I * sizeof(float));
+        float* up = reinterpret_cast<float*>(p);    p += align256(static_cast<size_t>(R) * I * sizeof(float));
+        float* part = reinterpret_cast<float*>(p);
+        const int max_group = static_cast<int>(tokens < routes ? tokens : routes);       // an expert sees a token at most once
+        const size_t stride13 = static_cast<size_t>(inter) * bpr_x * pllm_gguf_block_bytes(w13_type);
+        const size_t stride2 = static_cast<size_t>(dim) * bpr_h * pllm_gguf_block_bytes(w2_type);
+        int st = gemm_f16_stage_rows(x, x_dtype, route_tokens, R, D, bpr_x, x_staged, s);
+        if (st != PLLM_OK) return st;
+        st = gemm_f16_grouped(x_staged, w1, w13_type, stride13, seg_starts, E, gate, R, max_group, I, bpr_x, s);
+        if (st != PLLM_OK) return st;
+        st = gemm_f16_grouped(x_staged, w3, w13_type, stride13, seg_starts, E, up, R, max_group, I, bpr_x, s);
+        if (st != PLLM_OK) return st;
+        st = gemm_f16_stage_swiglu(gate, up, route_weights, swiglu_limit, R, I, bpr_h, h_staged, s);
+        if (st != PLLM_OK) return st;
+        st = gemm_f16_grouped(h_staged, w2, w2_type, stride2, seg_starts, E, part, R, max_group, D, bpr_h, s);
+        if (st != PLLM_OK) return st;
+        dim3 rg(static_cast<unsigned>(tokens), static_cast<unsigned>((dim + 255) / 256));
+        hipLaunchKernelGGL(moe_reduce_kernel, rg, dim3(256), 0, s, part, route_tokens, y, R, D);
+        return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+    }
     const size_t x_stride = act_image_256_bytes(bpr_x), h_stride = act_image_256_bytes(bpr_h);
     unsigned char* ws = static_cast<unsigned char*>(workspace);
     unsigned char* x_image = ws;

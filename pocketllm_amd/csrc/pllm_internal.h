@@ -36,6 +36,14 @@ int compute_units();
 // prefill tile GEMM on f16 MFMA with decoded tiles (gemm_f16.hip)
 bool gemm_f16_supports(int type_id);
 size_t gemm_f16_workspace_bytes(int rows, int n, int bpr);
+// routed experts as a batch of tile matmuls: activation rows staged once (fp16 rows + per-row scales),
+// then one launch per projection over all experts
+size_t gemm_f16_staged_bytes(int rows, int bpr);
+int gemm_f16_stage_rows(const void* x, int x_dtype, const int64_t* row_map, int rows, int k, int bpr, void* staged, hipStream_t stream);
+int gemm_f16_stage_swiglu(const float* g, const float* u, const float* route_weights, float limit, int rows, int inter, int bpr, void* staged,
+                          hipStream_t stream);
+int gemm_f16_grouped(const void* staged, const uint8_t* w, int type_id, size_t group_stride, const int32_t* seg, int groups,
+                     float* y, int rows, int max_group_rows, int n, int bpr, hipStream_t stream);
 int gemm_f16_fp8(const void* x, int x_dtype, const uint8_t* w, const float* wscale, void* y, int y_dtype,
                  int rows, int k, int n, void* workspace, size_t workspace_bytes, hipStream_t stream);
 int gemm_f16(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y, int y_dtype,

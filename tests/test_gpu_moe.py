@@ -185,3 +185,32 @@ def test_linear_modules(mod):
     assert np.abs(q8(x).float().cpu().numpy() - want).max() < 2e-2
     with pytest.raises(ValueError, match="q8_0 blocks must be"):
         Q8_0GGUFLinear(torch.zeros(4, 2, 33, dtype=torch.uint8, device=DEV), 64)
+
+
+@pytest.mark.parametrize("t13,t2,limit", [("iq2_xxs", "iq1_m", 0.0), ("iq2_xxs", "q2_k", 0.7), ("iq1_m", "iq1_m", 0.0)])
+def test_grouped_experts_tile_path(mod, t13, t2, limit):
+    """Sixteen tokens or more: the routes of every expert go through the MFMA tile kernel as one batch of matmuls
+    (some experts idle, one token count that is not a multiple of the tile)."""
+    rng = np.random.default_rng(11)
+    e, d, inter, topk, t = 10, 768, 512, 3, 77
+    w1 = _expert_blocks(rng, t13, e, inter, d)
+    w3 = _expert_blocks(rng, t13, e, inter, d)
+    w2 = _expert_blocks(rng, t2, e, d, inter)
+    idx, wts = _route(rng, t, e + 6, topk)                 # experts 0..15, local window 3..12
+    start = 3
+    x = torch.from_numpy(rng.standard_normal((t, d)).astype(np.float32)).to(DEV).to(torch.bfloat16)
+    _, toks, rws, seg = mod.moe_group_routes(torch.from_numpy(idx).to(DEV), torch.from_numpy(wts).to(DEV), start, e)
+    _, o_toks, o_rws, o_seg = O.group_routes(idx, wts, start, e)
+    grids = (codebooks.get_iq2xxs_signed_grid_tensor().to(DEV), codebooks.get_iq1_grid_tensor().to(DEV))
+    dw1, dw3, dw2 = (torch.from_numpy(a).to(DEV) for a in (w1, w3, w2))
+    tid = O.TYPE_IDS
+    if t13 == t2:                                          # one codebook in use: one grid, as the reference takes it
+        grids = grids[0] if t13 == "iq2_xxs" else grids[1]
+    print(f"case tile path {t13}/{t2} limit={limit}", flush=True)
+    y = mod.gguf_moe_prefill_grouped_forward(x, toks, rws, seg, dw1, dw3, dw2, d, tid[t13], d, tid[t13], inter, tid[t2], grids, limit)
+    torch.cuda.synchronize()
+    route_experts = np.repeat(np.arange(e), np.diff(o_seg))
+    want = O.moe_forward(x.float().cpu().numpy(), o_toks, o_rws, route_experts, w1, w3, w2, t13, t13, t2, limit)
+    assert O.rel_l2(y.cpu().numpy(), want) <= TOL
+    y2 = mod.gguf_moe_prefill_grouped_forward(x, toks, rws, seg, dw1, dw3, dw2, d, tid[t13], d, tid[t13], inter, tid[t2], grids, limit)
+    assert torch.equal(y, y2)

@@ -108,3 +108,27 @@ def test_fp8_prefill_baseline_shape_sampled(mod):
     w = O.dequant_fp8_block(codes, scale)[cols]
     want = O.matmul_f(x.float().cpu().numpy(), w)
     assert O.rel_l2(y.cpu().numpy()[:, cols], want) <= 1e-3
+
+
+# ---- the other super-block formats through the same tile kernel --------------------------------------
+
+@pytest.mark.parametrize("type_name", ["q2_k", "iq2_xxs", "iq1_m"])
+@pytest.mark.parametrize("t,n,k", [(16, 128, 256), (64, 300, 768), (130, 129, 1024), (300, 520, 3072)])
+def test_prefill_other_formats_match_float_oracle(mod, type_name, t, n, k):
+    from pocketllm_amd import codebooks
+    rng = np.random.default_rng(t + 3 * n + k)
+    if type_name == "q2_k":
+        blocks = C.quantize_q2_k((rng.standard_normal((n, k)) * 0.02).astype(np.float32))
+        grid = torch.empty(0, dtype=torch.int8, device=DEV)
+    elif type_name == "iq2_xxs":
+        blocks = C.random_iq2_xxs(rng, n, k // 256)
+        grid = codebooks.get_iq2xxs_signed_grid_tensor().to(DEV)
+    else:
+        blocks = C.random_iq1_m(rng, n, k // 256)
+        grid = codebooks.get_iq1_grid_tensor().to(DEV)
+    x = torch.from_numpy(rng.standard_normal((t, k)).astype(np.float32)).to(DEV).to(torch.bfloat16)
+    print(f"case {type_name} prefill t={t} n={n} k={k}", flush=True)
+    y = mod.gguf_quant_gemm_prefill_forward(x, torch.from_numpy(blocks).to(DEV), k, O.TYPE_IDS[type_name], grid, out_dtype=torch.float32)
+    torch.cuda.synchronize()
+    want = O.matmul_f(x.float().cpu().numpy(), O.dequant_rows(blocks, type_name, k))
+    assert O.rel_l2(y.cpu().numpy(), want) <= 1e-3, (type_name, t, n, k)
