@@ -264,6 +264,25 @@ def pmc_pass(mod, dev) -> None:
     print(json.dumps({"pmc_pass": f"{name} matvec {n}x{k}", "weight_bytes": int(blocks.size), "copy_bytes": int(nbytes)}))
 
 
+def prefill_pass(mod, dev) -> None:
+    """A few launches of the MFMA tile kernel for the profiler: Q4_K 17408x5120 at T=2048 and FP8 at T=512."""
+    from pocketllm_amd import block_codec as C
+    rng = np.random.default_rng(4004)
+    k, n = 5120, 17408
+    empty = torch.empty(0, dtype=torch.int8, device=dev)
+    blocks = torch.from_numpy(C.quantize_q4_k(rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02))).to(dev)
+    x = torch.randn(2048, k, device=dev, dtype=torch.bfloat16)
+    for _ in range(6):
+        mod.gguf_quant_gemm_prefill_forward(x, blocks, k, 3, empty)
+    codes, scale = C.quantize_fp8_block(rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02))
+    codes, scale = torch.from_numpy(codes).to(dev), torch.from_numpy(scale).to(dev)
+    x512 = x[:512].contiguous()
+    for _ in range(6):
+        mod.fp8_block_gemm_forward(x512, codes, scale)
+    torch.cuda.synchronize()
+    print(json.dumps({"prefill_pass": "q4_k 17408x5120 T=2048 x6, fp8 17408x5120 T=512 x6", "flops_q4k": 2.0 * 2048 * k * n, "flops_fp8": 2.0 * 512 * k * n}))
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -273,6 +292,7 @@ def main() -> None:
     ap.add_argument("--no-extra", action="store_true", help="skip the table of other formats")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--pmc-pass", action="store_true", help="short run for rocprofv3 --pmc: dominant kernel + a copy of the same size")
+    ap.add_argument("--prefill-pass", action="store_true", help="short run for rocprofv3: a few launches of the MFMA tile kernel")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU (no sharding, no collectives); run with --gpus 1")
@@ -289,6 +309,9 @@ def main() -> None:
     grid = torch.empty(0, dtype=torch.int8, device=dev)
     if args.pmc_pass:
         pmc_pass(mod, dev)
+        return
+    if args.prefill_pass:
+        prefill_pass(mod, dev)
         return
     x_np = np.random.default_rng(2002).standard_normal((1, 5120), dtype=np.float32)
     x = torch.from_numpy(x_np).to(dev).to(torch.bfloat16)
