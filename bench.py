@@ -241,6 +241,13 @@ def prefill_cases(mod, dev, iters):
     scale = torch.from_numpy(scale).to(dev)
     x = torch.randn(512, k, device=dev, dtype=torch.bfloat16)
     run(f"fp8_e4m3 prefill {n}x{k} T=512", 512, n, lambda s: mod.fp8_block_gemm_forward(x, codes, scale))
+    # the reference's FP8 linear: act_quant (E4M3 activations, 128-wide scales) + fp8_gemm on the native FP8 matrix path
+    a, a_s = mod.fp8_act_quant_forward(x)
+    us, graphed = time_calls_us(lambda s: mod.fp8_gemm_forward(a, a_s, codes, scale), 4, max(8, iters // 8))
+    usq, _ = time_calls_us(lambda s: mod.fp8_act_quant_forward(x), 4, max(8, iters // 8))
+    tf = 2.0 * 512 * k * n / us / 1e6
+    out.append({"case": f"fp8_e4m3 x fp8_e4m3 native MFMA prefill {n}x{k} T=512", "us_per_call": round(us, 3), "tflops": round(tf, 1),
+                "frac_mfma_peak": round(tf / 5000.0, 4), "peak": "fp8 dense 5.0 PFLOP/s", "act_quant_us": round(usq, 3), "graph": graphed})
     return out
 
 

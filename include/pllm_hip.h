@@ -136,6 +136,19 @@ int pllm_fp8_block_gemm(const void* x, int x_dtype, const uint8_t* weight, const
 size_t pllm_fp8_block_gemm_workspace_bytes(int64_t rows, int64_t k, int64_t n);
 
 /*
+ * FP8 activations times FP8 weights, both block-scaled, on the matrix cores' native OCP-FP8 path:
+ *     y[t, r] = sum over 128-wide K blocks kb of a_scale[t, kb] * scale[r / 128, kb] * sum_{c in kb} f32(a[t, c]) * f32(weight[r, c])
+ *   a [rows, k] E4M3 codes, a_scale [rows, k / 128] float32: the outputs of pllm_fp8_act_quant (block 128)
+ *   weight [n, k] E4M3 codes, scale [ceil(n / 128), k / 128] float32; k a multiple of 128, bases 16-byte aligned
+ *   y [rows, n] y_dtype, float32 accumulation
+ * Replaces fp8_gemm (src/kernels/ops.py:1043-1051), which dequantizes both sides and multiplies in
+ * floating point; together with pllm_fp8_act_quant this is the reference's FP8 linear
+ * (act_quant + fp8_gemm, src/models/deepseek_v4/runtime.py:639-643).
+ */
+int pllm_fp8_gemm(const uint8_t* a, const float* a_scale, const uint8_t* weight, const float* scale, void* y, int y_dtype,
+                  int64_t rows, int64_t k, int64_t n, void* stream);
+
+/*
  * Fused routed-expert matmul over raw super-blocks (types Q2_K, IQ2_XXS, IQ1_M; gate/up share a type,
  * the down projection may use another, so IQ2_XXS gate/up with IQ1_M down needs no special case):
  *     y[t] = sum over routes r of token t:  W2_e ( silu(min(W1_e x_t, L)) * clamp(W3_e x_t, +-L) * w_r )

@@ -157,6 +157,14 @@ int pllm_gguf_quant_gemm_pair(const void* x, int x_dtype, const uint8_t* blocks0
                              static_cast<int>(rows), static_cast<int>(n), bpr, s);
 }
 
+int pllm_fp8_gemm(const uint8_t* a, const float* a_scale, const uint8_t* weight, const float* scale, void* y, int y_dtype,
+                  int64_t rows, int64_t k, int64_t n, void* stream) {
+    if (!a || !a_scale || !weight || !scale || !y || !dtype_ok(y_dtype)) return PLLM_ERR_INVALID_ARGUMENT;
+    if (!fits_int(rows) || !fits_int(k) || !fits_int(n) || rows <= 0 || n <= 0) return PLLM_ERR_INVALID_ARGUMENT;
+    return pllm::fp8_gemm_native(a, a_scale, weight, scale, y, y_dtype, static_cast<int>(rows), static_cast<int>(k), static_cast<int>(n),
+                                 static_cast<hipStream_t>(stream));
+}
+
 // the tile GEMM serves many rows of 256-aligned k; everything else takes the matvec (no workspace)
 static bool fp8_uses_gemm(int64_t rows, int64_t k) { return rows >= kGemmMinRows && k % 256 == 0; }
 

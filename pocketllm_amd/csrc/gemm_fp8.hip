@@ -1,0 +1,168 @@
+// FP8 x FP8 block-scaled matmul on the matrix cores' native OCP-FP8 path:
+//     y[t, r] = sum over 128-wide K blocks kb of  a_s[t, kb] * b_s[r / 128, kb] * sum_{c in kb} f32(a[t, c]) * f32(b[r, c])
+// with E4M3 codes on both sides (activations as written by the 128-wide activation quantizer, weights
+// with their 128 x 128 block scales) and float32 accumulation.
+//
+// A workgroup of four waves (2 x 2) owns a 128 x 128 output tile and walks K one scale block (128
+// codes) at a time.  Codes need no decoding: 16-byte global loads go to registers one step ahead and
+// from there into a double-buffered LDS tile (rows padded to 144 bytes: 16-byte reads of 32 rows at
+// the same offset never share a bank).  Every wave runs v_mfma_scale_f32_32x32x64_f8f6f4 (both operands
+// E4M3, unit block scales) on its 64 x 64 sub-tile: two K halves of 64 into a fresh accumulator, which is then scaled
+// into the running sums with the product of the row's activation scale and the block's weight
+// scale.  Which code of a 64-chunk sits in which byte of a lane's operand does not matter as long
+// as both operands agree: lanes 0..31 take bytes [0, 32) and lanes 32..63 bytes [32, 64) of the
+// chunk on both sides.
+#include "pllm_device.h"
+#include "pllm_internal.h"
+
+namespace pllm {
+namespace {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int kTile = 128;                // rows of both operands per workgroup tile
+constexpr int kStep = 128;                // codes along K per step = one scale block
+constexpr int kRow = kStep + 16;          // LDS row stride in bytes
+
+__device__ __forceinline__ v8i operand(const unsigned char* p) {
+    const uint4 lo = *reinterpret_cast<const uint4*>(p);
+    const uint4 hi = *reinterpret_cast<const uint4*>(p + 16);
+    v8i r;
+    r[0] = static_cast<int>(lo.x); r[1] = static_cast<int>(lo.y); r[2] = static_cast<int>(lo.z); r[3] = static_cast<int>(lo.w);
+    r[4] = static_cast<int>(hi.x); r[5] = static_cast<int>(hi.y); r[6] = static_cast<int>(hi.z); r[7] = static_cast<int>(hi.w);
+    return r;
+}
+
+// both operands E4M3 (format selectors 0), both block scales 2^0 (E8M0 code 127)
+__device__ __forceinline__ floatx16 mfma_e4m3(const v8i& a, const v8i& b, const floatx16& c) {
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 127, 0, 127);
+}
+
+__global__ __launch_bounds__(256) void fp8_gemm_kernel(
+    const uint8_t* __restrict__ a, const float* __restrict__ a_s, const uint8_t* __restrict__ b, const float* __restrict__ b_s,
+    void* __restrict__ y, int y_dtype, int rows, int n, int k) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    unsigned char* a_tile = smem;                                         // [2][kTile * kRow]
+    unsigned char* b_tile = smem + 2 * kTile * kRow;                      // [2][kTile * kRow]
+    float* a_scale = reinterpret_cast<float*>(smem + 4 * kTile * kRow);   // [2][kTile]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int n0 = blockIdx.x * kTile, t0 = blockIdx.y * kTile;
+    const int steps = k / kStep;
+
+    // staging: piece q = tid + 256 i is bytes [16 (q % 8), +16) of tile row q / 8
+    const int prow = tid >> 3, pcol = 16 * (tid & 7);
+    // (named variables, not arrays: indexed through the lambdas below, arrays end up in scratch memory)
+    auto arow = [&](int i) { return a + static_cast<size_t>(min(t0 + prow + 32 * i, rows - 1)) * k + pcol; };
+    auto brow = [&](int i) { return b + static_cast<size_t>(min(n0 + prow + 32 * i, n - 1)) * k + pcol; };
+    const uint8_t* const as0 = arow(0); const uint8_t* const as1 = arow(1); const uint8_t* const as2 = arow(2); const uint8_t* const as3 = arow(3);
+    const uint8_t* const bs0 = brow(0); const uint8_t* const bs1 = brow(1); const uint8_t* const bs2 = brow(2); const uint8_t* const bs3 = brow(3);
+    const float* as_src = a_s + static_cast<size_t>(min(t0 + (tid & 127), rows - 1)) * steps;
+    // the wave's 64 weight rows lie inside one 128-row scale block
+    const float* bs_src = b_s + static_cast<size_t>(min(n0 + wn * 64, n - 1) >> 7) * steps;
+
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    uint4 ra0, ra1, ra2, ra3, rb0, rb1, rb2, rb3;
+    float rs = 0.0f;
+    auto fetch = [&](int s) {
+        const size_t off = static_cast<size_t>(s) * kStep;
+        ra0 = *reinterpret_cast<const uint4*>(as0 + off); ra1 = *reinterpret_cast<const uint4*>(as1 + off);
+        ra2 = *reinterpret_cast<const uint4*>(as2 + off); ra3 = *reinterpret_cast<const uint4*>(as3 + off);
+        rb0 = *reinterpret_cast<const uint4*>(bs0 + off); rb1 = *reinterpret_cast<const uint4*>(bs1 + off);
+        rb2 = *reinterpret_cast<const uint4*>(bs2 + off); rb3 = *reinterpret_cast<const uint4*>(bs3 + off);
+        if (tid < kTile) rs = as_src[s];
+    };
+    auto stage = [&](int buf) {
+        unsigned char* ad = a_tile + buf * kTile * kRow + prow * kRow + pcol;
+        unsigned char* bd = b_tile + buf * kTile * kRow + prow * kRow + pcol;
+        *reinterpret_cast<uint4*>(ad) = ra0; *reinterpret_cast<uint4*>(ad + 32 * kRow) = ra1;
+        *reinterpret_cast<uint4*>(ad + 64 * kRow) = ra2; *reinterpret_cast<uint4*>(ad + 96 * kRow) = ra3;
+        *reinterpret_cast<uint4*>(bd) = rb0; *reinterpret_cast<uint4*>(bd + 32 * kRow) = rb1;
+        *reinterpret_cast<uint4*>(bd + 64 * kRow) = rb2; *reinterpret_cast<uint4*>(bd + 96 * kRow) = rb3;
+        if (tid < kTile) a_scale[buf * kTile + tid] = rs;
+    };
+
+    fetch(0);
+    stage(0);
+    __syncthreads();
+    for (int s = 0; s < steps; ++s) {
+        const int buf = s & 1;
+        if (s + 1 < steps) fetch(s + 1);
+        const float ws = bs_src[s];
+        const unsigned char* at = a_tile + buf * kTile * kRow + (wm * 64 + (lane & 31)) * kRow + 32 * (lane >> 5);
+        const unsigned char* bt = b_tile + buf * kTile * kRow + (wn * 64 + (lane & 31)) * kRow + 32 * (lane >> 5);
+        floatx16 c[2][2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const v8i a0 = operand(at + 64 * h), a1 = operand(at + 32 * kRow + 64 * h);
+            const v8i b0 = operand(bt + 64 * h), b1 = operand(bt + 32 * kRow + 64 * h);
+            if (h == 0) {
+                const floatx16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                c[0][0] = mfma_e4m3(a0, b0, zero);
+                c[0][1] = mfma_e4m3(a0, b1, zero);
+                c[1][0] = mfma_e4m3(a1, b0, zero);
+                c[1][1] = mfma_e4m3(a1, b1, zero);
+            } else {
+                c[0][0] = mfma_e4m3(a0, b0, c[0][0]);
+                c[0][1] = mfma_e4m3(a0, b1, c[0][1]);
+                c[1][0] = mfma_e4m3(a1, b0, c[1][0]);
+                c[1][1] = mfma_e4m3(a1, b1, c[1][1]);
+            }
+        }
+        // D[m][n]: lane holds column n = lane % 32 and rows 8 * (v / 4) + 4 * (lane / 32) + v % 4
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const float4 sa = *reinterpret_cast<const float4*>(a_scale + buf * kTile + wm * 64 + mi * 32 + 8 * q + 4 * (lane >> 5));
+                const float f0 = sa.x * ws, f1 = sa.y * ws, f2 = sa.z * ws, f3 = sa.w * ws;
+#pragma unroll
+                for (int ni = 0; ni < 2; ++ni) {
+                    acc[mi][ni][4 * q + 0] += c[mi][ni][4 * q + 0] * f0;
+                    acc[mi][ni][4 * q + 1] += c[mi][ni][4 * q + 1] * f1;
+                    acc[mi][ni][4 * q + 2] += c[mi][ni][4 * q + 2] * f2;
+                    acc[mi][ni][4 * q + 3] += c[mi][ni][4 * q + 3] * f3;
+                }
+            }
+        if (s + 1 < steps) stage(buf ^ 1);
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni) {
+            const int col = n0 + wn * 64 + ni * 32 + (lane & 31);
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int row = t0 + wm * 64 + mi * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                if (row < rows && col < n) store_any(y, y_dtype, static_cast<size_t>(row) * n + col, acc[mi][ni][v]);
+            }
+        }
+}
+
+}  // namespace
+
+int fp8_gemm_native(const uint8_t* a, const float* a_s, const uint8_t* b, const float* b_s, void* y, int y_dtype,
+                    int rows, int k, int n, hipStream_t stream) {
+    if (k % kStep != 0 || k <= 0) return PLLM_ERR_UNSUPPORTED;
+    if ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15u) return PLLM_ERR_UNSUPPORTED;
+    const size_t smem = static_cast<size_t>(4) * kTile * kRow + 2 * kTile * sizeof(float);
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(fp8_gemm_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem)) != hipSuccess)
+        return PLLM_ERR_UNSUPPORTED;
+    dim3 grid((n + kTile - 1) / kTile, (rows + kTile - 1) / kTile);
+    hipLaunchKernelGGL(fp8_gemm_kernel, grid, dim3(256), smem, stream, a, a_s, b, b_s, y, y_dtype, rows, n, k);
+    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+}
+
+}  // namespace pllm

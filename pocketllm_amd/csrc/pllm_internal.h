@@ -44,6 +44,9 @@ int gemm_f16_stage_swiglu(const float* g, const float* u, const float* route_wei
                           hipStream_t stream);
 int gemm_f16_grouped(const void* staged, const uint8_t* w, int type_id, size_t group_stride, const int32_t* seg, int groups,
                      float* y, int rows, int max_group_rows, int n, int bpr, hipStream_t stream);
+// FP8 x FP8 block-scaled matmul on the native FP8 matrix path (gemm_fp8.hip); k a multiple of 128
+int fp8_gemm_native(const uint8_t* a, const float* a_s, const uint8_t* b, const float* b_s, void* y, int y_dtype,
+                    int rows, int k, int n, hipStream_t stream);
 int gemm_f16_fp8(const void* x, int x_dtype, const uint8_t* w, const float* wscale, void* y, int y_dtype,
                  int rows, int k, int n, void* workspace, size_t workspace_bytes, hipStream_t stream);
 int gemm_f16(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y, int y_dtype,

@@ -237,6 +237,31 @@ def fp8_block_gemm_forward(x: torch.Tensor, weight: torch.Tensor, scale: torch.T
     return y
 
 
+def fp8_gemm_forward(a: torch.Tensor, a_scale: torch.Tensor, weight: torch.Tensor, scale: torch.Tensor, *,
+                     out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """fp8_gemm(a, a_s, b, b_s) of src/kernels/ops.py:1043-1051 on the native FP8 matrix path: `a` / `a_scale` are the
+    codes and 128-wide scales of fp8_act_quant_forward, `weight` / `scale` the block-scaled FP8 weight."""
+    _check(a.dtype in (torch.float8_e4m3fn, torch.uint8), "a must be float8_e4m3fn (or its uint8 bytes)")
+    a8 = a.view(torch.uint8) if a.dtype == torch.float8_e4m3fn else a
+    w8 = _fp8_bytes(weight)
+    n, k = w8.shape
+    _check(a8.is_cuda and a8.is_contiguous() and a8.dim() >= 1 and a8.size(-1) == k, "a must be a contiguous CUDA FP8 tensor [..., K]")
+    _check(k % 128 == 0, "fp8_gemm needs K to be a multiple of 128")
+    rows = a8.numel() // k
+    _check(a_scale.is_cuda and a_scale.dtype == torch.float32 and a_scale.is_contiguous() and a_scale.numel() == rows * (k // 128),
+           "a_scale must be a contiguous CUDA float32 tensor [..., K/128]")
+    _check(scale.is_cuda and scale.dtype == torch.float32 and scale.is_contiguous(), "scale must be a contiguous CUDA float32 tensor")
+    _check(tuple(scale.shape) == ((n + 127) // 128, k // 128), "scale must have shape [ceil(N/128), K/128]")
+    y = torch.empty(*a8.shape[:-1], n, dtype=out_dtype, device=a8.device)
+    if rows == 0:
+        return y
+    with torch.cuda.device(a8.device):
+        st = _lib().pllm_fp8_gemm(a8.data_ptr(), a_scale.data_ptr(), w8.data_ptr(), scale.data_ptr(), y.data_ptr(), _DTYPE_CODE[out_dtype],
+                                  rows, k, n, _stream(a8.device))
+    _ffi.check(st, "fp8_gemm_forward")
+    return y
+
+
 def fp8_act_quant_forward(x: torch.Tensor, eps: float = 1e-4, round_scale_pow2: bool = False):
     """Per-(row, 128) FP8 activation quantizer (src/kernels/ops.py:501-516): returns (float8_e4m3fn codes, float32 scales)."""
     _check(x.is_cuda and x.is_contiguous(), "x must be a contiguous CUDA tensor")

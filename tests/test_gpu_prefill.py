@@ -132,3 +132,45 @@ def test_prefill_other_formats_match_float_oracle(mod, type_name, t, n, k):
     torch.cuda.synchronize()
     want = O.matmul_f(x.float().cpu().numpy(), O.dequant_rows(blocks, type_name, k))
     assert O.rel_l2(y.cpu().numpy(), want) <= 1e-3, (type_name, t, n, k)
+
+
+# ---- FP8 activations x FP8 weights on the native FP8 matrix path -----------------------------------
+
+@pytest.mark.parametrize("t,n,k", [(1, 128, 128), (16, 130, 256), (77, 300, 1024), (200, 512, 5120)])
+def test_fp8_gemm_native_matches_act_quant_semantics(mod, t, n, k):
+    """act_quant + fp8_gemm (ops.py:982-1051) against the oracle, which dequantizes both sides and multiplies in
+    float64.  The only differences are the matrix core's own summation of 64 products per instruction (full-range
+    random codes make that visible at a few 1e-5) and float32 accumulation across the K blocks."""
+    rng = np.random.default_rng(5 * t + n + k)
+    codes = rng.integers(0, 256, size=(n, k), dtype=np.uint8)
+    codes[(codes & 0x7f) == 0x7f] = 0x3c
+    scale = rng.uniform(0.001, 0.01, size=((n + 127) // 128, k // 128)).astype(np.float32)
+    x_np = rng.standard_normal((t, k)).astype(np.float32)
+    x_np[0] *= 50.0
+    x = torch.from_numpy(x_np).to(DEV)
+    a, a_s = mod.fp8_act_quant_forward(x)
+    print(f"case fp8 native t={t} n={n} k={k}", flush=True)
+    y = mod.fp8_gemm_forward(a, a_s, torch.from_numpy(codes).to(DEV), torch.from_numpy(scale).to(DEV))
+    torch.cuda.synchronize()
+    want = O.fp8_gemm_q(x_np, codes, scale)
+    assert O.rel_l2(y.cpu().numpy(), want) <= 2e-4
+    # the ops-layer name takes the same route
+    from pocketllm_amd import ops
+    y2 = ops.fp8_gemm(a, a_s, torch.from_numpy(codes).to(DEV).view(torch.float8_e4m3fn), torch.from_numpy(scale).to(DEV))
+    assert O.rel_l2(y2.float().cpu().numpy(), want) <= 1e-2       # default dtype may be 16-bit
+
+
+def test_fp8_gemm_native_baseline_shape_sampled(mod):
+    """BASELINE config 4 at T = 512 with the reference's FP8-activation semantics; 64 sampled columns."""
+    rng = np.random.default_rng(1005)
+    n, k, t = 17408, 5120, 512
+    codes, scale = C.quantize_fp8_block(rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02))
+    x_np = rng.standard_normal((t, k)).astype(np.float32)
+    a, a_s = mod.fp8_act_quant_forward(torch.from_numpy(x_np).to(DEV))
+    y = mod.fp8_gemm_forward(a, a_s, torch.from_numpy(codes).to(DEV), torch.from_numpy(scale).to(DEV))
+    torch.cuda.synchronize()
+    cols = np.sort(rng.choice(n, size=64, replace=False))
+    xa_codes, xs = O.fp8_act_quant(x_np)
+    xa = O.fp8_e4m3_decode(xa_codes).reshape(t, k // 128, 128) * xs[..., None]
+    want = O.matmul_f(xa.reshape(t, k), O.dequant_fp8_block(codes, scale)[cols])
+    assert O.rel_l2(y.cpu().numpy()[:, cols], want) <= 2e-4
