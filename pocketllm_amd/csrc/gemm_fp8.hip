@@ -39,7 +39,7 @@ __device__ __forceinline__ floatx16 mfma_e4m3(const v8i& a, const v8i& b, const 
     return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 127, 0, 127);
 }
 
-__global__ __launch_bounds__(256) void fp8_gemm_kernel(
+__global__ __launch_bounds__(256, 2) void fp8_gemm_kernel(
     const uint8_t* __restrict__ a, const float* __restrict__ a_s, const uint8_t* __restrict__ b, const float* __restrict__ b_s,
     void* __restrict__ y, int y_dtype, int rows, int n, int k) {
     extern __shared__ __align__(16) unsigned char smem[];
