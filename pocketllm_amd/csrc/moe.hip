@@ -21,6 +21,7 @@ constexpr int kMoeGemmMinTokens = 16;
 namespace {
 
 constexpr int kW13Iters = 6;
+constexpr int kW13Split = 2;               // waves that share one row's super-blocks in the per-route gate/up kernel
 
 // Epilogue of one 32-row tile of one route, run by lanes 0..31 of a wave (lane = row inside the tile):
 // clamp, SiLU, route weight, then the 32 hidden values are quantized in place into the image format
@@ -55,52 +56,120 @@ __device__ __forceinline__ void store_hidden(float g, float u, float limit, floa
 
 
 template <typename FMT>
-__global__ __launch_bounds__(256) void moe_w13_kernel(
+__global__ __launch_bounds__(256 * kW13Split) void moe_w13_kernel(
     const unsigned char* __restrict__ x_image, size_t x_image_stride, int bpr,
     const int64_t* __restrict__ route_tokens, const int32_t* __restrict__ route_experts, const float* __restrict__ route_weights,
     const uint8_t* __restrict__ w1, const uint8_t* __restrict__ w3, int inter, float limit,
-    unsigned char* __restrict__ h_image, size_t h_image_stride, int h_kpad) {
+    unsigned char* __restrict__ h_image, size_t h_image_stride, int h_kpad,
+    const void* __restrict__ x_raw, int x_dtype, int dim, const int64_t* __restrict__ route_experts64) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int kpad = bpr * 256;
     const int image_bytes = static_cast<int>(staged_x_bytes(kpad));
     const StagedX sx = carve_staged_x(smem, kpad);
     unsigned char* tables = smem + image_bytes;
-    float* exch = reinterpret_cast<float*>(tables + FMT::kTableBytes);           // [2][32]
+    float* exch = reinterpret_cast<float*>(tables + FMT::kTableBytes);           // [kW13Split][2 matrices][32]
 
     const int route = blockIdx.y;
     const int64_t token = route_tokens ? route_tokens[route] : 0;
-    const size_t expert_off = static_cast<size_t>(route_experts[route]) * inter * bpr * FMT::kBlockBytes;
+    // single-token calls skip the two helper launches: the expert ids are read as they come (int64)
+    // and the workgroup quantizes the activation row into LDS itself (x_raw)
+    const int expert = route_experts64 ? static_cast<int>(route_experts64[route]) : route_experts[route];
+    const size_t expert_off = static_cast<size_t>(expert) * inter * bpr * FMT::kBlockBytes;
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
     const int j = lane & 3, team = lane >> 2;
-    const int mat = wave >> 1;
+    // 4 kW13Split waves: (matrix, half of the 32 rows, share of the super-blocks); more waves in
+    // flight per row tile hide the latency of the codebook lookups
+    const int mat = (wave >> 1) & 1;
+    const int bhalf = wave >> 2;
     const int slot = 16 * (wave & 1) + team;                                     // 0..31 inside the tile
     const int row = min(blockIdx.x * 32 + slot, inter - 1);
     const uint8_t* wrow = (mat ? w3 : w1) + expert_off + static_cast<size_t>(row) * bpr * FMT::kBlockBytes;
 
     float acc = 0.0f;
     bool staged = false;
-    for (int b0 = 0; b0 < bpr; b0 += kW13Iters) {
-        typename FMT::Regs regs[kW13Iters];
+    for (int b0 = bhalf; b0 < bpr || !staged; b0 += kW13Split * kW13Iters) {
+        typename FMT::Regs regs[kW13Iters] = {};
 #pragma unroll
         for (int it = 0; it < kW13Iters; ++it)
-            FMT::load(regs[it], wrow + static_cast<size_t>(min(b0 + it, bpr - 1)) * FMT::kBlockBytes, j);
+            if (b0 + kW13Split * it < bpr) FMT::load(regs[it], wrow + static_cast<size_t>(b0 + kW13Split * it) * FMT::kBlockBytes, j);
         if (!staged) {
-            copy_to_lds(smem, x_image + static_cast<size_t>(token) * x_image_stride, image_bytes);
+            if (x_raw) quantize_row_to_lds(smem, x_raw, x_dtype, static_cast<size_t>(token) * dim, dim, kpad);
+            else copy_to_lds(smem, x_image + static_cast<size_t>(token) * x_image_stride, image_bytes);
             FMT::stage_tables(tables);
             __syncthreads();
             staged = true;
         }
 #pragma unroll
         for (int it = 0; it < kW13Iters; ++it)
-            if (b0 + it < bpr) acc += FMT::lane_dot(regs[it], j, b0 + it, sx, tables);
+            if (b0 + kW13Split * it < bpr) acc += FMT::lane_dot(regs[it], j, b0 + kW13Split * it, sx, tables);
     }
     acc += __shfl_xor(acc, 1, 64);
     acc += __shfl_xor(acc, 2, 64);
-    if (j == 0) exch[mat * 32 + slot] = acc;
+    if (j == 0) exch[bhalf * 64 + mat * 32 + slot] = acc;
     __syncthreads();
-    if (tid < 32) store_hidden(exch[tid], exch[32 + tid], limit, route_weights[route], blockIdx.x * 32 + tid, inter,
+    float gsum = 0.0f, usum = 0.0f;
+    if (tid < 32) {
+#pragma unroll
+        for (int v = 0; v < kW13Split; ++v) { gsum += exch[v * 64 + tid]; usum += exch[v * 64 + 32 + tid]; }
+    }
+    if (tid < 32) store_hidden(gsum, usum, limit, route_weights[route], blockIdx.x * 32 + tid, inter,
                                h_image + static_cast<size_t>(route) * h_image_stride, h_kpad, tid);
+}
+
+// Down projection of a single token with the sum over its routes inside the kernel:
+//     y[row] = sum over routes r, in route order, of W2_{e_r}[row, :] . h_r
+// One workgroup per 16 output rows; its waves split the routes and every expert row's super-blocks between them as
+// in the dense matvec, the hidden images of all routes sit in LDS.  No partial buffer, no second launch.
+// The sixteen waves' sums are added in wave order, so the result does not depend on scheduling.
+constexpr int kSumWaves = 16;             // wave = (route mod 8, super-block parity)
+constexpr int kSumIters = 4;
+
+template <typename FMT>
+__global__ __launch_bounds__(64 * kSumWaves) void moe_w2_sum_kernel(
+    const unsigned char* __restrict__ h_image, size_t h_image_stride, int bpr, const int64_t* __restrict__ route_experts, int routes,
+    const uint8_t* __restrict__ w2, size_t expert_stride, float* __restrict__ y, int dim) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int kpad = bpr * 256;
+    const int image_bytes = static_cast<int>(staged_x_bytes(kpad));
+    unsigned char* tables = smem + routes * image_bytes;
+    float* partial = reinterpret_cast<float*>(tables + FMT::kTableBytes);        // [waves][16]
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int j = lane & 3, team = lane >> 2;
+    const int row = blockIdx.x * 16 + team;
+    const size_t row_off = static_cast<size_t>(row < dim ? row : 0) * bpr * FMT::kBlockBytes;
+
+    for (int r = 0; r < routes; ++r) copy_to_lds(smem + r * image_bytes, h_image + static_cast<size_t>(r) * h_image_stride, image_bytes);
+    FMT::stage_tables(tables);
+    __syncthreads();
+
+    float acc = 0.0f;
+    for (int r = wave >> 1; r < routes; r += kSumWaves / 2) {
+        const uint8_t* wrow = w2 + static_cast<size_t>(route_experts[r]) * expert_stride + row_off;
+        const StagedX sx = carve_staged_x(smem + r * image_bytes, kpad);
+        for (int b0 = wave & 1; b0 < bpr; b0 += 2 * kSumIters) {
+            typename FMT::Regs regs[kSumIters];
+#pragma unroll
+            for (int it = 0; it < kSumIters; ++it)
+                FMT::load(regs[it], wrow + static_cast<size_t>(min(b0 + 2 * it, bpr - 1)) * FMT::kBlockBytes, j);
+#pragma unroll
+            for (int it = 0; it < kSumIters; ++it)
+                if (b0 + 2 * it < bpr) acc += FMT::lane_dot(regs[it], j, b0 + 2 * it, sx, tables);
+        }
+    }
+    acc += __shfl_xor(acc, 1, 64);
+    acc += __shfl_xor(acc, 2, 64);
+    if (j == 0) partial[wave * 16 + team] = acc;
+    __syncthreads();
+    if (tid < 16) {
+        float total = 0.0f;
+#pragma unroll
+        for (int v = 0; v < kSumWaves; ++v) total += partial[v * 16 + tid];
+        const int out_row = blockIdx.x * 16 + tid;
+        if (out_row < dim) y[out_row] = total;
+    }
 }
 
 // ---- grouped forms: one workgroup per (row tile, expert) -----------------------------------------
@@ -327,8 +396,9 @@ __global__ __launch_bounds__(64) void route_fill_kernel(const void* __restrict__
 template <typename FMT>
 int launch_w13(const unsigned char* x_image, size_t x_stride, int bpr, const int64_t* route_tokens, const int32_t* route_experts,
                const float* route_weights, const uint8_t* w1, const uint8_t* w3, int inter, float limit, unsigned char* h_image,
-               size_t h_stride, int h_kpad, int routes, hipStream_t stream) {
-    const size_t smem = staged_x_bytes(bpr * 256) + FMT::kTableBytes + 64 * sizeof(float);
+               size_t h_stride, int h_kpad, int routes, hipStream_t stream,
+               const void* x_raw = nullptr, int x_dtype = 0, int dim = 0, const int64_t* route_experts64 = nullptr) {
+    const size_t smem = staged_x_bytes(bpr * 256) + FMT::kTableBytes + kW13Split * 64 * sizeof(float);
     auto kern = moe_w13_kernel<FMT>;
     if (smem > 64 * 1024) {
         if (smem > 160 * 1024) return PLLM_ERR_UNSUPPORTED;
@@ -337,8 +407,21 @@ int launch_w13(const unsigned char* x_image, size_t x_stride, int bpr, const int
             return PLLM_ERR_UNSUPPORTED;
     }
     dim3 grid(h_kpad / 32, routes);
-    hipLaunchKernelGGL(kern, grid, dim3(256), smem, stream, x_image, x_stride, bpr, route_tokens, route_experts, route_weights, w1, w3,
-                       inter, limit, h_image, h_stride, h_kpad);
+    hipLaunchKernelGGL(kern, grid, dim3(256 * kW13Split), smem, stream, x_image, x_stride, bpr, route_tokens, route_experts, route_weights, w1, w3,
+                       inter, limit, h_image, h_stride, h_kpad, x_raw, x_dtype, dim, route_experts64);
+    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+}
+
+template <typename FMT>
+int launch_w2_sum(const unsigned char* h_image, size_t h_stride, int bpr, const int64_t* route_experts64, int routes, const uint8_t* w2,
+                  size_t expert_stride, float* y, int dim, hipStream_t stream) {
+    const size_t smem = static_cast<size_t>(routes) * staged_x_bytes(bpr * 256) + FMT::kTableBytes + kSumWaves * 16 * sizeof(float);
+    auto kern = moe_w2_sum_kernel<FMT>;
+    if (smem > 64 * 1024 &&
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem)) != hipSuccess)
+        return PLLM_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(kern, dim3((dim + 15) / 16), dim3(64 * kSumWaves), smem, stream, h_image, h_stride, bpr, route_experts64, routes, w2,
+                       expert_stride, y, dim);
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 
@@ -442,6 +525,25 @@ int pllm_gguf_moe_forward(const void* x, int x_dtype, int64_t tokens, int64_t di
         return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
     }
     const size_t x_stride = act_image_256_bytes(bpr_x), h_stride = act_image_256_bytes(bpr_h);
+    if (tokens == 1 && route_experts && routes * staged_x_bytes(bpr_h * 256) <= 96 * 1024) {
+        // single token: two launches.  Gate/up read the raw activation row and the int64 expert ids
+        // themselves; the down projection sums the routes in order inside the kernel.
+        unsigned char* himg = static_cast<unsigned char*>(workspace);
+        const int R1 = static_cast<int>(routes), I1 = static_cast<int>(inter), D1 = static_cast<int>(dim);
+        int st1;
+        switch (w13_type) {
+            case PLLM_TYPE_IQ2_XXS: st1 = launch_w13<IQ2XXS>(nullptr, 0, bpr_x, nullptr, nullptr, route_weights, w1, w3, I1, swiglu_limit, himg, h_stride, bpr_h * 256, R1, s, x, x_dtype, D1, route_experts); break;
+            case PLLM_TYPE_IQ1_M: st1 = launch_w13<IQ1M>(nullptr, 0, bpr_x, nullptr, nullptr, route_weights, w1, w3, I1, swiglu_limit, himg, h_stride, bpr_h * 256, R1, s, x, x_dtype, D1, route_experts); break;
+            default: st1 = launch_w13<Q2K>(nullptr, 0, bpr_x, nullptr, nullptr, route_weights, w1, w3, I1, swiglu_limit, himg, h_stride, bpr_h * 256, R1, s, x, x_dtype, D1, route_experts); break;
+        }
+        if (st1 != PLLM_OK) return st1;
+        const size_t stride2 = static_cast<size_t>(dim) * bpr_h * pllm_gguf_block_bytes(w2_type);
+        switch (w2_type) {
+            case PLLM_TYPE_IQ2_XXS: return launch_w2_sum<IQ2XXS>(himg, h_stride, bpr_h, route_experts, R1, w2, stride2, y, D1, s);
+            case PLLM_TYPE_IQ1_M: return launch_w2_sum<IQ1M>(himg, h_stride, bpr_h, route_experts, R1, w2, stride2, y, D1, s);
+            default: return launch_w2_sum<Q2K>(himg, h_stride, bpr_h, route_experts, R1, w2, stride2, y, D1, s);
+        }
+    }
     unsigned char* ws = static_cast<unsigned char*>(workspace);
     unsigned char* x_image = ws;
     unsigned char* h_image = x_image + x_stride * tokens;

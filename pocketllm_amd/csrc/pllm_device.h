@@ -105,13 +105,6 @@ __device__ __forceinline__ void quantize4(const float v[4], uint32_t& hi, uint32
     }
 }
 
-// Workgroup-wide copy of nbytes (a multiple of 16, both pointers 16-byte aligned) into LDS.
-__device__ __forceinline__ void copy_to_lds(unsigned char* dst, const unsigned char* __restrict__ src, int nbytes) {
-    const uint4* s = reinterpret_cast<const uint4*>(src);
-    uint4* d = reinterpret_cast<uint4*>(dst);
-    for (int i = threadIdx.x; i < (nbytes >> 4); i += blockDim.x) d[i] = s[i];
-}
-
 // Runtime-dtype front ends (the dtype is uniform, so the switch costs one scalar branch).
 __device__ __forceinline__ float load_any(const void* x, int x_dtype, size_t i) {
     if (x_dtype == PLLM_BF16) return to_float(static_cast<const bf16_t*>(x)[i]);
@@ -123,6 +116,49 @@ __device__ __forceinline__ void store_any(void* y, int y_dtype, size_t i, float 
     if (y_dtype == PLLM_BF16) static_cast<bf16_t*>(y)[i] = from_float<bf16_t>(v);
     else if (y_dtype == PLLM_F16) static_cast<f16_t*>(y)[i] = from_float<f16_t>(v);
     else static_cast<float*>(y)[i] = v;
+}
+
+// Workgroup-wide quantization of one activation row straight into LDS, the same image the
+// pre-pass kernel writes to memory (blockDim.x a multiple of 8, kpad a multiple of 256).  Four
+// consecutive values per lane: one 8-byte load for 16-bit inputs when the row allows it.
+__device__ __forceinline__ void quantize_row_to_lds(unsigned char* lds, const void* __restrict__ x, int x_dtype, size_t xoff, int k, int kpad) {
+    int8_t* hi = reinterpret_cast<int8_t*>(lds);
+    int8_t* lo = hi + kpad;
+    float2* gs = reinterpret_cast<float2*>(lo + kpad);
+    float* sum16 = reinterpret_cast<float*>(gs + kpad / 32);
+    const bool narrow = x_dtype != PLLM_F32 && ((reinterpret_cast<uintptr_t>(x) + 2 * xoff) & 7u) == 0;
+    for (int e0 = static_cast<int>(threadIdx.x) * 4; e0 < kpad; e0 += static_cast<int>(blockDim.x) * 4) {
+        float v[4];
+        if (narrow && e0 + 3 < k) {
+            const uint2 w = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(x) + xoff + e0);
+            if (x_dtype == PLLM_BF16) {
+                v[0] = __uint_as_float(w.x << 16); v[1] = __uint_as_float(w.x & 0xffff0000u);
+                v[2] = __uint_as_float(w.y << 16); v[3] = __uint_as_float(w.y & 0xffff0000u);
+            } else {
+                v[0] = f16_bits_to_float(w.x & 0xffffu); v[1] = f16_bits_to_float(w.x >> 16);
+                v[2] = f16_bits_to_float(w.y & 0xffffu); v[3] = f16_bits_to_float(w.y >> 16);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) v[i] = (e0 + i < k) ? load_any(x, x_dtype, xoff + e0 + i) : 0.0f;
+        }
+        uint32_t qh, ql;
+        float scale;
+        quantize4(v, qh, ql, scale);
+        *reinterpret_cast<uint32_t*>(hi + e0) = qh;
+        *reinterpret_cast<uint32_t*>(lo + e0) = ql;
+        const float sum = group_sum<4>((v[0] + v[1]) + (v[2] + v[3]));
+        const float sum32 = sum + __shfl_xor(sum, 4, 64);
+        if ((threadIdx.x & 3) == 0) sum16[e0 >> 4] = sum;
+        if ((threadIdx.x & 7) == 0) gs[e0 >> 5] = make_float2(scale * kLoInv, sum32);
+    }
+}
+
+// Workgroup-wide copy of nbytes (a multiple of 16, both pointers 16-byte aligned) into LDS.
+__device__ __forceinline__ void copy_to_lds(unsigned char* dst, const unsigned char* __restrict__ src, int nbytes) {
+    const uint4* s = reinterpret_cast<const uint4*>(src);
+    uint4* d = reinterpret_cast<uint4*>(dst);
+    for (int i = threadIdx.x; i < (nbytes >> 4); i += blockDim.x) d[i] = s[i];
 }
 
 }  // namespace pllm
