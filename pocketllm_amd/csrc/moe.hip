@@ -89,10 +89,10 @@ __global__ __launch_bounds__(256 * kW13Split) void moe_w13_kernel(
     float acc = 0.0f;
     bool staged = false;
     for (int b0 = bhalf; b0 < bpr || !staged; b0 += kW13Split * kW13Iters) {
-        typename FMT::Regs regs[kW13Iters] = {};
+        typename FMT::Regs regs[kW13Iters];
 #pragma unroll
         for (int it = 0; it < kW13Iters; ++it)
-            if (b0 + kW13Split * it < bpr) FMT::load(regs[it], wrow + static_cast<size_t>(b0 + kW13Split * it) * FMT::kBlockBytes, j);
+            FMT::load(regs[it], wrow + static_cast<size_t>(min(b0 + kW13Split * it, bpr - 1)) * FMT::kBlockBytes, j);
         if (!staged) {
             if (x_raw) quantize_row_to_lds(smem, x_raw, x_dtype, static_cast<size_t>(token) * dim, dim, kpad);
             else copy_to_lds(smem, x_image + static_cast<size_t>(token) * x_image_stride, image_bytes);
