@@ -12,13 +12,50 @@
 
 namespace pllm {
 
-#define PLLM_TABLE_U64(name, n) static __device__ const uint64_t name[n] = {
-#define PLLM_TABLE_U16(name, n) static __device__ const uint16_t name[n] = {
+#define PLLM_TABLE_U64(name, n) alignas(16) static __device__ constexpr uint64_t name[n] = {
+#define PLLM_TABLE_U16(name, n) alignas(16) static __device__ constexpr uint16_t name[n] = {
 #define PLLM_TABLE_END };
 #include "ggml_codebooks.inc"
 #undef PLLM_TABLE_U64
 #undef PLLM_TABLE_U16
 #undef PLLM_TABLE_END
+
+// Derived tables in the form the kernels keep in LDS, built at compile time so that staging them is
+// a plain copy.
+//   PLLM_IQ2XXS_SIGN_MASKS[s7]: 0xff in byte b where bit b of the 8-bit sign pattern is set (bit 7
+//     of a pattern is the parity of the other seven).
+//   PLLM_IQ1_GRID_NIBBLES[i]: the eight codes c = grid value + 1 in {0, 1, 2} of codebook entry i,
+//     nibble 2b = element b and nibble 2b + 1 = element 4 + b, so that two masks give the two dwords
+//     of int8 codes.
+struct alignas(16) Iq2xxsSignMasks { uint64_t v[128]; };
+struct alignas(16) Iq1GridNibbles { uint32_t v[2048]; };
+constexpr Iq2xxsSignMasks make_iq2xxs_sign_masks() {
+    Iq2xxsSignMasks t{};
+    for (uint32_t i = 0; i < 128; ++i) {
+        uint32_t parity = 0;
+        for (int b = 0; b < 7; ++b) parity ^= (i >> b) & 1u;
+        const uint32_t s8 = i | (parity << 7);
+        uint64_t m = 0;
+        for (int b = 0; b < 8; ++b) m |= ((s8 >> b) & 1u) ? (0xffull << (8 * b)) : 0ull;
+        t.v[i] = m;
+    }
+    return t;
+}
+constexpr Iq1GridNibbles make_iq1_grid_nibbles() {
+    Iq1GridNibbles t{};
+    for (int i = 0; i < 2048; ++i) {
+        const uint32_t p = PLLM_IQ1_GRID_PACKED[i];          // element e in bits [2e, 2e+1]
+        uint32_t v = 0;
+        for (int b = 0; b < 4; ++b) {
+            v |= ((p >> (2 * b)) & 3u) << (8 * b);
+            v |= ((p >> (2 * (4 + b))) & 3u) << (8 * b + 4);
+        }
+        t.v[i] = v;
+    }
+    return t;
+}
+static __device__ const Iq2xxsSignMasks PLLM_IQ2XXS_SIGN_MASKS = make_iq2xxs_sign_masks();
+static __device__ const Iq1GridNibbles PLLM_IQ1_GRID_NIBBLES = make_iq1_grid_nibbles();
 
 // 16 bytes from an address that is only 2-byte aligned
 struct __attribute__((packed, aligned(2))) Unaligned16 { uint32_t x, y, z, w; };
@@ -88,16 +125,8 @@ struct IQ2XXS {
         r.d = *reinterpret_cast<const uint16_t*>(blk);
     }
     static __device__ __forceinline__ void stage_tables(unsigned char* lds) {
-        uint64_t* grid = reinterpret_cast<uint64_t*>(lds);
-        uint64_t* sign = grid + 256;
-        for (int i = threadIdx.x; i < 256; i += blockDim.x) grid[i] = PLLM_IQ2XXS_GRID[i];
-        for (int i = threadIdx.x; i < 128; i += blockDim.x) {
-            const uint32_t s8 = static_cast<uint32_t>(i) | ((__popc(i) & 1u) << 7);
-            uint64_t m = 0;
-#pragma unroll
-            for (int b = 0; b < 8; ++b) m |= ((s8 >> b) & 1u) ? (0xffull << (8 * b)) : 0ull;
-            sign[i] = m;
-        }
+        copy_to_lds(lds, reinterpret_cast<const unsigned char*>(PLLM_IQ2XXS_GRID), 2048);
+        copy_to_lds(lds + 2048, reinterpret_cast<const unsigned char*>(PLLM_IQ2XXS_SIGN_MASKS.v), 1024);
     }
     static __device__ __forceinline__ float sub_block(uint32_t ids, uint32_t aux, int base, const StagedX& sx, const uint2* grid,
                                                        const uint2* sign) {
@@ -145,17 +174,7 @@ struct IQ1M {
         r.sc = *reinterpret_cast<const uint2*>(blk + 48);
     }
     static __device__ __forceinline__ void stage_tables(unsigned char* lds) {
-        uint32_t* t = reinterpret_cast<uint32_t*>(lds);
-        for (int i = threadIdx.x; i < 2048; i += blockDim.x) {
-            const uint32_t p = PLLM_IQ1_GRID_PACKED[i];          // element e in bits [2e, 2e+1]
-            uint32_t v = 0;
-#pragma unroll
-            for (int b = 0; b < 4; ++b) {
-                v |= ((p >> (2 * b)) & 3u) << (8 * b);
-                v |= ((p >> (2 * (4 + b))) & 3u) << (8 * b + 4);
-            }
-            t[i] = v;
-        }
+        copy_to_lds(lds, reinterpret_cast<const unsigned char*>(PLLM_IQ1_GRID_NIBBLES.v), 8192);
     }
     static __device__ __forceinline__ float lane_dot(const Regs& r, int j, int blk, const StagedX& sx, const unsigned char* lds) {
         const uint32_t* table = reinterpret_cast<const uint32_t*>(lds);

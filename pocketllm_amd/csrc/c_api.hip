@@ -71,9 +71,10 @@ static int superblock_matvec(const unsigned char* image, size_t stride, const ui
                              int rows, int n, int bpr, hipStream_t s) {
     switch (type_id) {
         case PLLM_TYPE_Q2_K:
+            return pllm::dot4_matvec_from_image(image, stride, blocks, type_id, y, y_dtype, rows, n, bpr, s);
         case PLLM_TYPE_IQ2_XXS:
         case PLLM_TYPE_IQ1_M:
-            return pllm::dot4_matvec_from_image(image, stride, blocks, type_id, y, y_dtype, rows, n, bpr, s);
+            return pllm::iq_mfma_matvec_from_image(image, stride, blocks, type_id, y, y_dtype, rows, n, bpr, s);
         case PLLM_TYPE_Q4_K:
         case PLLM_TYPE_Q5_K:
             return pllm::kquant_matvec_from_image(image, stride, blocks, type_id, y, y_dtype, rows, n, bpr, s);

@@ -20,11 +20,14 @@ int q8_0_matvec(const void* x, int x_dtype, const uint8_t* w, void* y, int y_dty
                 int rows, int k, int n, int bpr, void* workspace, size_t workspace_bytes, hipStream_t stream);
 
 // 256-weight super-block types: one activation image (act_image_256) serves any number of matvecs.
-// Q4_K / Q5_K run in matvec_kquant.hip, Q2_K / IQ2_XXS / IQ1_M in matvec_dot4.hip.
+// Q4_K / Q5_K run in matvec_kquant.hip, IQ2_XXS / IQ1_M in matvec_iq_mfma.hip (matrix cores),
+// Q2_K and the routed forms in matvec_dot4.hip (v_dot4).
 int kquant_matvec_from_image(const unsigned char* image, size_t stride, const uint8_t* w, int type_id, void* y, int y_dtype,
                              int rows, int n, int bpr, hipStream_t stream);
 int dot4_matvec_from_image(const unsigned char* image, size_t stride, const uint8_t* w, int type_id, void* y, int y_dtype,
                            int rows, int n, int bpr, hipStream_t stream);
+int iq_mfma_matvec_from_image(const unsigned char* image, size_t stride, const uint8_t* w, int type_id, void* y, int y_dtype,
+                              int rows, int n, int bpr, hipStream_t stream);
 
 // routed form: activation row r (image r, output row r) meets the matrix at w + y_expert[r] * expert_stride
 int dot4_routed_matvec_from_image(const unsigned char* image, size_t stride, const uint8_t* w, int type_id, void* y, int y_dtype,
