@@ -160,7 +160,8 @@ def _grid_for(type_name, dev):
 
 
 @pytest.mark.parametrize("type_name", ["iq2_xxs", "iq1_m"])
-@pytest.mark.parametrize("n,k,rows", [(16, 256, 1), (50, 768, 1), (1536, 3072, 1), (3072, 1536, 1), (40, 2048, 3), (7, 5120, 1), (21, 1000, 2)])
+@pytest.mark.parametrize("n,k,rows", [(16, 256, 1), (50, 768, 1), (1536, 3072, 1), (3072, 1536, 1), (40, 2048, 3), (7, 5120, 1), (21, 1000, 2),
+                                      (176, 768, 2), (208, 5120, 1), (64, 14336, 1)])
 def test_iq_matvec_matches_oracle(mod, type_name, n, k, rows):
     rng = np.random.default_rng(500 + n + k)
     gen = C.random_iq2_xxs if type_name == "iq2_xxs" else C.random_iq1_m
@@ -177,6 +178,25 @@ def test_iq_matvec_matches_oracle(mod, type_name, n, k, rows):
         want = O.matmul_f(x.float().cpu().numpy(), O.dequant_rows(blocks, type_name, k))
         err = O.rel_l2(y.cpu().numpy(), want)
         assert err <= 2e-4, (type_name, n, k, rows, dt, err)
+
+
+@pytest.mark.parametrize("type_name,n,k", [("iq2_xxs", 35200, 3072), ("iq1_m", 70400, 1536)])
+def test_iq_matvec_many_rows(mod, type_name, n, k):
+    """More row tiles than workgroups in flight: every workgroup walks several chunks of rows, the last ones
+    unevenly.  Checked on the first and last rows and a random sample in between."""
+    rng = np.random.default_rng(77)
+    gen = C.random_iq2_xxs if type_name == "iq2_xxs" else C.random_iq1_m
+    blocks = gen(rng, n, k // 256)
+    x_np = rng.standard_normal((1, k)).astype(np.float32)
+    dev = torch.device("cuda:0")
+    print(f"case {type_name} n={n} k={k}", flush=True)
+    y = mod.gguf_quant_gemm_forward(torch.from_numpy(x_np).to(dev), torch.from_numpy(blocks).to(dev), k, O.TYPE_IDS[type_name],
+                                    _grid_for(type_name, dev), out_dtype=torch.float32)
+    torch.cuda.synchronize()
+    pick = np.unique(np.concatenate([np.arange(256), np.arange(n - 256, n), rng.integers(0, n, size=4096)]))
+    want = O.matmul_f(x_np, O.dequant_rows(blocks[pick], type_name, k))
+    assert O.rel_l2(y.cpu().numpy()[:, pick], want) <= 2e-4
+    assert torch.isfinite(y).all()
 
 
 def test_iq_fully_random_bytes(mod):
