@@ -5,14 +5,14 @@
 // value) sits in LDS.  For one super-block index the wave forms
 //     C[m][n] = sum_k A[m][k] * B[k][n],     v_mfma_i32_16x16x64_i8,
 // with n = output row, B = the weights' integer codes and A = activation bytes arranged so that row
-// m collects one scale group of the block (the format structs below say which).  Lane (n, s)
+// m collects one scale group of the block (the format structs of block_mfma.h say which).  Lane (n, s)
 // supplies B for the 16-weight slice s of each MFMA from its own 64 weights of the block, and the
 // slices are assigned to A rows such that the lane finds the results for exactly those 64 weights
 // in its own C registers: C[4 s .. 4 s + 3][n].
 //
 // The codebook lookups happen once per weight and feed 16 rows of dots each, where the v_dot4 form
 // repeats the activation reads and the dots per lane.
-#include "block_dot4.h"
+#include "block_mfma.h"
 #include "pllm_internal.h"
 
 namespace pllm {
@@ -21,190 +21,6 @@ namespace {
 constexpr int kRowsPerTile = 16;
 constexpr int kWaves = 8;
 constexpr int kMaxRounds = 16;           // row-tile groups one workgroup works through at most
-
-typedef int v4i __attribute__((ext_vector_type(4)));
-
-__device__ __forceinline__ v4i as_v4i(uint32_t x, uint32_t y, uint32_t z, uint32_t w) {
-    v4i r;
-    r.x = static_cast<int>(x); r.y = static_cast<int>(y); r.z = static_cast<int>(z); r.w = static_cast<int>(w);
-    return r;
-}
-
-// LDS offsets of a lane's A operands: slot i of block b is read at off[i] + b * step[i]; slots whose
-// A row is not the lane's point at 16 zero bytes with step 0.
-template <int SLOTS>
-struct AMap { int off[SLOTS]; int step[SLOTS]; };
-
-// ------------------------------------------------------------------------------------------------
-// IQ2_XXS: 66 B = d(2) + 8 sub-blocks of 8 B (four grid ids, then a u32: four 7-bit sign indices and
-// a 4-bit scale).  Lane (n, s) holds sub-blocks 2 s and 2 s + 1 (two 32-weight groups).
-// A rows: m = 2 * group + term; MFMA t, slice s carries half t % 2 of group 2 s + t / 2, so
-// C[4 s .. 4 s + 3][n] = groups 2 s and 2 s + 1, both terms, in the lane's own registers.
-// LDS tables: 256 x 8 magnitude bytes g, 128 x 8 sign masks m (0xff where the weight is negative).
-// The signed code is (g ^ m) - m bytewise; instead of finishing that per byte, the wave runs two
-// MFMAs per slice, with B = g ^ m and with B = m, and subtracts the accumulators.
-// ------------------------------------------------------------------------------------------------
-struct IQ2XXSm {
-    static constexpr int kBlockBytes = 66;
-    static constexpr int kTableBytes = IQ2XXS::kTableBytes;
-    static constexpr int kSlots = 4;
-    static constexpr int kHoldBlocks = 3;                      // block indices whose activation side a wave may keep in registers
-    struct Regs { uint4 q; uint32_t d; };
-    static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, int s) {
-        r.q = load16_a2(blk + 2 + 16 * s);
-        r.d = *reinterpret_cast<const uint16_t*>(blk);
-    }
-    // the same share from a copy of the block in LDS (2-byte aligned there as in memory): five
-    // aligned dwords, shifted down by 16 bits where the share starts in the middle of a dword
-    static __device__ __forceinline__ void load_lds(Regs& r, const unsigned char* base, int off, int s) {   // base 4-byte aligned
-        const int a = off + 2 + 16 * s;
-        const uint32_t* p = reinterpret_cast<const uint32_t*>(base + (a & ~3));
-        const uint32_t sh = (static_cast<uint32_t>(a) & 2u) << 3;
-        const uint32_t d0 = p[0], d1 = p[1], d2 = p[2], d3 = p[3], d4 = p[4];
-        r.q = make_uint4(__builtin_amdgcn_alignbit(d1, d0, sh), __builtin_amdgcn_alignbit(d2, d1, sh),
-                         __builtin_amdgcn_alignbit(d3, d2, sh), __builtin_amdgcn_alignbit(d4, d3, sh));
-        r.d = *reinterpret_cast<const uint16_t*>(base + off);
-    }
-    static __device__ __forceinline__ void stage_tables(unsigned char* lds) { IQ2XXS::stage_tables(lds); }
-    static __device__ __forceinline__ void dma_tables(uint32_t lds_base, int wave, int lane);
-    static __device__ __forceinline__ void a_map(AMap<kSlots>& am, int col, int ks, int kpad, int zero_off) {
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            const int g = 2 * ks + (t >> 1);
-            const bool active = (col >> 1) == g;
-            am.off[t] = active ? ((col & 1) ? kpad : 0) + 32 * g + 16 * (t & 1) : zero_off;
-            am.step[t] = active ? 256 : 0;
-        }
-    }
-    // what a block index contributes from the activation side: the lane's A operands and its two
-    // groups' scales; a wave that meets the same block index in tile after tile keeps them in registers
-    struct Held { uint4 a[4]; float xs0, xs1; };
-    static __device__ __forceinline__ void hold(Held& h, int s, int b, const unsigned char* smem, const AMap<kSlots>& am, const StagedX& sx) {
-#pragma unroll
-        for (int t = 0; t < 4; ++t) h.a[t] = *reinterpret_cast<const uint4*>(smem + am.off[t] + b * am.step[t]);
-        const float4 g2 = *reinterpret_cast<const float4*>(sx.gs + b * 8 + 2 * s);   // {xs0 / 254, sum0, xs1 / 254, sum1}
-        h.xs0 = g2.x; h.xs1 = g2.z;
-    }
-    static __device__ __forceinline__ float block_held(const Regs& r, int, int, const Held& h, const unsigned char*, const AMap<kSlots>&,
-                                                       const unsigned char* tables) {
-        const uint2* grid = reinterpret_cast<const uint2*>(tables);
-        const uint2* sign = grid + 256;
-        v4i c = {0, 0, 0, 0}, cm = {0, 0, 0, 0};
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            const uint32_t ids = (t < 2) ? r.q.x : r.q.z, aux = (t < 2) ? r.q.y : r.q.w;
-            const int e = 2 * (t & 1);                                         // grid entries e and e + 1 of the sub-block
-            const uint2 g0 = grid[(ids >> (8 * e)) & 0xffu], m0 = sign[(aux >> (7 * e)) & 127u];
-            const uint2 g1 = grid[(ids >> (8 * e + 8)) & 0xffu], m1 = sign[(aux >> (7 * e + 7)) & 127u];
-            const v4i av = as_v4i(h.a[t].x, h.a[t].y, h.a[t].z, h.a[t].w);
-            c = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, as_v4i(g0.x ^ m0.x, g0.y ^ m0.y, g1.x ^ m1.x, g1.y ^ m1.y), c, 0, 0, 0);
-            cm = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, as_v4i(m0.x, m0.y, m1.x, m1.y), cm, 0, 0, 0);
-        }
-        const float v0 = static_cast<float>(__mul24(c.x - cm.x, 254) + (c.y - cm.y));   // group 2 s: 254 * high term + low term
-        const float v1 = static_cast<float>(__mul24(c.z - cm.z, 254) + (c.w - cm.w));   // group 2 s + 1
-        const float ls0 = static_cast<float>(2 * (r.q.y >> 28) + 1), ls1 = static_cast<float>(2 * (r.q.w >> 28) + 1);
-        return 0.125f * f16_bits_to_float(r.d) * (ls0 * h.xs0 * v0 + ls1 * h.xs1 * v1);
-    }
-    static __device__ __forceinline__ float block(const Regs& r, int s, int b, const unsigned char* smem, const AMap<kSlots>& am,
-                                                  const StagedX& sx, const unsigned char* tables) {
-        Held h;
-        hold(h, s, b, smem, am, sx);
-        return block_held(r, s, b, h, smem, am, tables);
-    }
-};
-
-// ------------------------------------------------------------------------------------------------
-// IQ1_M: 56 B = qs(32) qh(16) scales(8); w = dl (c - 1 + delta) with c in {0, 1, 2} from the
-// codebook (index: qs byte plus the low three bits of its qh nibble), dl = d (2 s3 + 1) per 16
-// weights, delta = -+1/8 per 8 weights (bit 3 of the nibble).  Lane (n, s) holds entries 8 s .. 8 s + 7
-// = four 16-weight groups.  With integer codes 8 c +- 1 = 8 (c + delta),
-//     sum w x = d sum over 16-groups j of (2 s3_j + 1) [ dot(8 c +- 1, x)_j / 8 - sum16(x)_j ].
-// A rows: m = 16-group of the block, one MFMA set per activation term; MFMA t, slice s carries group
-// 4 s + t, so C[4 s .. 4 s + 3][n] = the lane's own four groups.  sum16 comes from the image.
-// LDS table: 4096 x 8 code bytes, index = qs byte | nibble << 8 (the delta bit selects the half).
-// ------------------------------------------------------------------------------------------------
-struct alignas(16) Iq1DeltaCodes { uint64_t v[4096]; };
-constexpr Iq1DeltaCodes make_iq1_delta_codes() {
-    Iq1DeltaCodes t{};
-    for (int i = 0; i < 4096; ++i) {
-        const uint32_t p = PLLM_IQ1_GRID_PACKED[i & 2047];      // element e in bits [2e, 2e+1], value + 1
-        uint64_t v = 0;
-        for (int e = 0; e < 8; ++e) {
-            const int code = 8 * static_cast<int>((p >> (2 * e)) & 3u) + ((i & 2048) ? -1 : 1);
-            v |= static_cast<uint64_t>(static_cast<uint8_t>(code)) << (8 * e);
-        }
-        t.v[i] = v;
-    }
-    return t;
-}
-static __device__ const Iq1DeltaCodes PLLM_IQ1_DELTA_CODES = make_iq1_delta_codes();
-
-struct IQ1Mm {
-    static constexpr int kBlockBytes = 56;
-    static constexpr int kTableBytes = 32768;
-    static constexpr int kSlots = 8;                           // [term][t]
-    static constexpr int kHoldBlocks = 0;                      // (its held operands would cost a workgroup per compute unit)
-    struct Regs { uint2 qs; uint32_t qh; uint2 sc; };
-    static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, int s) {
-        r.qs = *reinterpret_cast<const uint2*>(blk + 8 * s);                   // blocks are 8-byte aligned
-        r.qh = *reinterpret_cast<const uint32_t*>(blk + 32 + 4 * s);
-        r.sc = *reinterpret_cast<const uint2*>(blk + 48);
-    }
-    static __device__ __forceinline__ void load_lds(Regs& r, const unsigned char* base, int off, int s) { load(r, base + off, s); }
-    static __device__ __forceinline__ void stage_tables(unsigned char* lds) {
-        copy_to_lds(lds, reinterpret_cast<const unsigned char*>(PLLM_IQ1_DELTA_CODES.v), kTableBytes);
-    }
-    static __device__ __forceinline__ void dma_tables(uint32_t lds_base, int wave, int lane);
-    static __device__ __forceinline__ void a_map(AMap<kSlots>& am, int col, int ks, int kpad, int zero_off) {
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            const bool active = col == 4 * ks + t;
-            am.off[t] = active ? 16 * col : zero_off;
-            am.off[4 + t] = active ? kpad + 16 * col : zero_off;
-            am.step[t] = am.step[4 + t] = active ? 256 : 0;
-        }
-    }
-    // activation side of a block index (see IQ2XXSm::Held): the high-term A operands, the groups'
-    // scales (already over 8) and the 16-value sums; the low-term operands are read when needed
-    struct Held { uint4 a[4]; float x0, x1; float4 s16; };
-    static __device__ __forceinline__ void hold(Held& h, int s, int b, const unsigned char* smem, const AMap<kSlots>& am, const StagedX& sx) {
-#pragma unroll
-        for (int t = 0; t < 4; ++t) h.a[t] = *reinterpret_cast<const uint4*>(smem + am.off[t] + b * am.step[t]);
-        const float4 g2 = *reinterpret_cast<const float4*>(sx.gs + b * 8 + 2 * s);   // {xs0 / 254, sum0, xs1 / 254, sum1}
-        h.x0 = 0.125f * g2.x; h.x1 = 0.125f * g2.z;
-        h.s16 = *reinterpret_cast<const float4*>(sx.sum16 + b * 16 + 4 * s);
-    }
-    static __device__ __forceinline__ float block_held(const Regs& r, int s, int b, const Held& h, const unsigned char* smem,
-                                                       const AMap<kSlots>& am, const unsigned char* tables) {
-        const uint2* table = reinterpret_cast<const uint2*>(tables);
-        const uint32_t s01 = r.sc.x, s23 = r.sc.y;
-        const uint32_t dbits = ((s01 >> 12) & 0xfu) | ((s01 >> 24) & 0xf0u) | ((s23 >> 4) & 0xf00u) | ((s23 >> 16) & 0xf000u);
-        // the lane's four 16-weight scales are the low 12 bits of scale word s
-        const uint32_t word = ((s & 2) ? s23 : s01) >> (16 * (s & 1));
-        v4i ch = {0, 0, 0, 0}, cl = {0, 0, 0, 0};
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {                                          // 16-weight group t of the lane = entries 2 t, 2 t + 1
-            const uint32_t qw = (t < 2) ? r.qs.x : r.qs.y;
-            const uint2 w0 = table[((qw >> (16 * (t & 1))) & 0xffu) | (((r.qh >> (8 * t)) & 15u) << 8)];
-            const uint2 w1 = table[((qw >> (16 * (t & 1) + 8)) & 0xffu) | (((r.qh >> (8 * t + 4)) & 15u) << 8)];
-            const v4i bw = as_v4i(w0.x, w0.y, w1.x, w1.y);
-            const uint4 al = *reinterpret_cast<const uint4*>(smem + am.off[4 + t] + b * am.step[4 + t]);
-            ch = __builtin_amdgcn_mfma_i32_16x16x64_i8(as_v4i(h.a[t].x, h.a[t].y, h.a[t].z, h.a[t].w), bw, ch, 0, 0, 0);
-            cl = __builtin_amdgcn_mfma_i32_16x16x64_i8(as_v4i(al.x, al.y, al.z, al.w), bw, cl, 0, 0, 0);
-        }
-        const float ls0 = static_cast<float>(2 * (word & 7u) + 1), ls1 = static_cast<float>(2 * ((word >> 3) & 7u) + 1);
-        const float ls2 = static_cast<float>(2 * ((word >> 6) & 7u) + 1), ls3 = static_cast<float>(2 * ((word >> 9) & 7u) + 1);
-        const float v = ls0 * (h.x0 * static_cast<float>(__mul24(ch.x, 254) + cl.x) - h.s16.x) + ls1 * (h.x0 * static_cast<float>(__mul24(ch.y, 254) + cl.y) - h.s16.y) +
-                        ls2 * (h.x1 * static_cast<float>(__mul24(ch.z, 254) + cl.z) - h.s16.z) + ls3 * (h.x1 * static_cast<float>(__mul24(ch.w, 254) + cl.w) - h.s16.w);
-        return f16_bits_to_float(dbits) * v;
-    }
-    static __device__ __forceinline__ float block(const Regs& r, int s, int b, const unsigned char* smem, const AMap<kSlots>& am,
-                                                  const StagedX& sx, const unsigned char* tables) {
-        Held h;
-        hold(h, s, b, smem, am, sx);
-        return block_held(r, s, b, h, smem, am, tables);
-    }
-};
 
 // The lane's share of ITERS super-blocks of one row tile: blocks part + (pass * ITERS + it) * split
 // (clamped: always a valid address)
@@ -342,44 +158,6 @@ int launch_one(const unsigned char* image, size_t image_stride, const uint8_t* w
 // Workgroups walk chunks blockIdx.x, blockIdx.x + gridDim.x, ...; several share a compute unit, so
 // some multiply while others wait for their chunk.  Needs n % 16 == 0 and a 16-byte aligned matrix.
 // ------------------------------------------------------------------------------------------------
-typedef __attribute__((address_space(3))) unsigned char* lds_byte_ptr;
-
-// 16 bytes per lane from memory to LDS[lds_base + 16 * lane] (lds_base wave-uniform), no registers in
-// between.  Issued through inline assembly so that the compiler does not put a wait for it in front
-// of every later LDS read: the kernel waits for its chunks itself (wait_vm).
-__device__ __forceinline__ void lds_dma16(const void* src, uint32_t lds_base) {
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(lds_base) : "memory", "m0");
-}
-template <int N> __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory"); }
-// until at most `newest` of this wave's memory operations are outstanding (they complete in order)
-__device__ __forceinline__ void wait_vm_all_but(int newest) {
-    switch (newest) {
-        case 1: wait_vm<1>(); break;
-        case 2: wait_vm<2>(); break;
-        case 3: wait_vm<3>(); break;
-        case 4: wait_vm<4>(); break;
-        default: wait_vm<0>(); break;
-    }
-}
-// the wave's share of a workgroup-wide copy of `bytes` (a multiple of 16) to LDS address lds_base:
-// 1 KB pieces wave, wave + 8, ...; returns the number of instructions issued
-__device__ __forceinline__ int dma_share(const unsigned char* src, uint32_t lds_base, int bytes, int wave, int lane) {
-    int issued = 0;
-    for (int o = wave * 1024; o < bytes; o += kWaves * 1024) {
-        if (o + lane * 16 < bytes) lds_dma16(src + o + lane * 16, lds_base + o);
-        ++issued;
-    }
-    return issued;
-}
-
-__device__ __forceinline__ void IQ2XXSm::dma_tables(uint32_t lds_base, int wave, int lane) {
-    dma_share(reinterpret_cast<const unsigned char*>(PLLM_IQ2XXS_GRID), lds_base, 2048, wave, lane);
-    dma_share(reinterpret_cast<const unsigned char*>(PLLM_IQ2XXS_SIGN_MASKS.v), lds_base + 2048, 1024, wave, lane);
-}
-__device__ __forceinline__ void IQ1Mm::dma_tables(uint32_t lds_base, int wave, int lane) {
-    dma_share(reinterpret_cast<const unsigned char*>(PLLM_IQ1_DELTA_CODES.v), lds_base, kTableBytes, wave, lane);
-}
-
 constexpr int kChunkBudget = 28 * 1024;
 
 // NB > 0: a wave meets at most NB block indices (part, part + split, ...) and keeps their activation
@@ -408,14 +186,14 @@ __global__ __launch_bounds__(64 * kWaves) void iq_stream_matvec_kernel(
     const int chunk_rows = tiles_per_chunk * kRowsPerTile;
 
     // activation image, codebooks and the first chunk: all in flight together
-    dma_share(image + static_cast<size_t>(blockIdx.y) * image_stride, lds0, image_bytes, wave, lane);
-    FMT::dma_tables(lds0 + table_off, wave, lane);
+    dma_share<kWaves>(image + static_cast<size_t>(blockIdx.y) * image_stride, lds0, image_bytes, wave, lane);
+    FMT::template dma_tables<kWaves>(lds0 + table_off, wave, lane);
     if (tid < 4) reinterpret_cast<uint32_t*>(smem + zero_off)[tid] = 0;
     AMap<FMT::kSlots> am;
     FMT::a_map(am, col, ks, kpad, zero_off);
 
     int c = blockIdx.x, buf = 0;
-    dma_share(w + static_cast<size_t>(c) * chunk_rows * row_bytes, lds0 + chunk_off, min(chunk_rows, n - c * chunk_rows) * row_bytes, wave, lane);
+    dma_share<kWaves>(w + static_cast<size_t>(c) * chunk_rows * row_bytes, lds0 + chunk_off, min(chunk_rows, n - c * chunk_rows) * row_bytes, wave, lane);
     typename FMT::Held held[NB > 0 ? NB : 1];
     bool holding = false;
     while (c < chunks) {
@@ -425,7 +203,7 @@ __global__ __launch_bounds__(64 * kWaves) void iq_stream_matvec_kernel(
         const int cn = c + gridDim.x;
         int newest = 0;
         if (cn < chunks)
-            newest = dma_share(w + static_cast<size_t>(cn) * chunk_rows * row_bytes, lds0 + chunk_off + (buf ^ 1) * chunk_stride,
+            newest = dma_share<kWaves>(w + static_cast<size_t>(cn) * chunk_rows * row_bytes, lds0 + chunk_off + (buf ^ 1) * chunk_stride,
                                min(chunk_rows, n - cn * chunk_rows) * row_bytes, wave, lane);
         wait_vm_all_but(newest);             // this wave's pieces of chunk c (and of the image and tables) have landed ...
         __syncthreads();                     // ... and everybody else's too

@@ -530,6 +530,11 @@ int pllm_gguf_moe_forward(const void* x, int x_dtype, int64_t tokens, int64_t di
         // themselves; the down projection sums the routes in order inside the kernel.
         unsigned char* himg = static_cast<unsigned char*>(workspace);
         const int R1 = static_cast<int>(routes), I1 = static_cast<int>(inter), D1 = static_cast<int>(dim);
+        if (moe_single_mfma_supports(w13_type, w2_type, D1, I1, R1, x, w1, w3, w2)) {
+            const int st = moe_single_w13_mfma(x, x_dtype, D1, route_experts, route_weights, R1, w1, w3, w13_type, I1, swiglu_limit, himg, h_stride, s);
+            if (st != PLLM_OK) return st;
+            return moe_single_w2_mfma(himg, h_stride, I1, route_experts, R1, w2, y, D1, s);
+        }
         int st1;
         switch (w13_type) {
             case PLLM_TYPE_IQ2_XXS: st1 = launch_w13<IQ2XXS>(nullptr, 0, bpr_x, nullptr, nullptr, route_weights, w1, w3, I1, swiglu_limit, himg, h_stride, bpr_h * 256, R1, s, x, x_dtype, D1, route_experts); break;

@@ -33,6 +33,18 @@ int iq_mfma_matvec_from_image(const unsigned char* image, size_t stride, const u
 int dot4_routed_matvec_from_image(const unsigned char* image, size_t stride, const uint8_t* w, int type_id, void* y, int y_dtype,
                                   int rows, int n, int bpr, const int32_t* y_expert, size_t expert_stride, hipStream_t stream);
 
+// Routed experts of a single token on the matrix cores (moe_single_mfma.hip): IQ2_XXS / IQ1_M gate and
+// up projections into per-route hidden images with one scale per 16 values, IQ1_M down projection
+// with the sum over the routes inside the kernel.  `supports` says whether types, shapes and
+// alignment fit; the hidden images need staged-image bytes per route (h_stride apart).
+bool moe_single_mfma_supports(int w13_type, int w2_type, int dim, int inter, int routes, const void* x, const uint8_t* w1,
+                              const uint8_t* w3, const uint8_t* w2);
+int moe_single_w13_mfma(const void* x, int x_dtype, int dim, const int64_t* route_experts, const float* route_weights, int routes,
+                        const uint8_t* w1, const uint8_t* w3, int w13_type, int inter, float limit, unsigned char* h_image, size_t h_stride,
+                        hipStream_t stream);
+int moe_single_w2_mfma(const unsigned char* h_image, size_t h_stride, int inter, const int64_t* route_experts, int routes, const uint8_t* w2,
+                       float* y, int dim, hipStream_t stream);
+
 // compute units of the current device (read once per process; 256 when no device answers)
 int compute_units();
 
