@@ -20,132 +20,100 @@ namespace {
 
 constexpr int kRowsPerTile = 16;
 constexpr int kWaves = 8;
-constexpr int kMaxRounds = 16;           // row-tile groups one workgroup works through at most
 
-// The lane's share of ITERS super-blocks of one row tile: blocks part + (pass * ITERS + it) * split
-// (clamped: always a valid address)
+// One workgroup per tile of 16 rows: its W waves split the row's super-blocks (wave w takes blocks w,
+// w + W, ...) and meet in a small LDS reduction.  All weight loads of a pass are issued first; while
+// they are in flight the workgroup fills LDS with the activation image and the format's codebooks.
 template <typename FMT, int ITERS>
-__device__ __forceinline__ void load_unit(typename FMT::Regs (&regs)[ITERS], const uint8_t* __restrict__ w, int n, int bpr,
-                                          int tile, int col, int ks, int part, int split, int pass) {
-    const int row = tile * kRowsPerTile + col;
-    const uint8_t* wrow = w + static_cast<size_t>(row < n ? row : 0) * bpr * FMT::kBlockBytes;
-#pragma unroll
-    for (int it = 0; it < ITERS; ++it) {
-        const int b = min(part + (pass * ITERS + it) * split, bpr - 1);
-        FMT::load(regs[it], wrow + static_cast<size_t>(b) * FMT::kBlockBytes, ks);
-    }
-}
-
-// A workgroup of 8 waves stages the activation image and the codebooks once and then works through
-// `rounds` groups of row tiles (group = blockIdx.x + round * gridDim.x, 8 / split tiles of 16 rows
-// each): `split` waves share a tile's super-blocks.  The blocks of the next unit of work are loaded
-// while the current one is computed.
-template <typename FMT, int ITERS>
-__global__ __launch_bounds__(64 * kWaves) void iq_mfma_matvec_kernel(
+__global__ __launch_bounds__(64 * kWaves) void mfma_tile_matvec_kernel(
     const unsigned char* __restrict__ image, size_t image_stride, const uint8_t* __restrict__ w,
-    void* __restrict__ y, int y_dtype, int n, int bpr, int split, int groups) {
+    void* __restrict__ y, int y_dtype, int n, int bpr) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int kpad = bpr * 256;
     const int image_bytes = static_cast<int>(staged_x_bytes(kpad));
     const StagedX sx = carve_staged_x(smem, kpad);
     const int zero_off = image_bytes;                                        // 16 zero bytes
     unsigned char* tables = smem + image_bytes + 16;
-    float* partial = reinterpret_cast<float*>(tables + FMT::kTableBytes);   // [rounds][waves][16]
+    float* partial = reinterpret_cast<float*>(tables + FMT::kTableBytes);   // [waves][16]
 
     const int tid = threadIdx.x;
+    const int waves = blockDim.x >> 6;
     const int wave = tid >> 6;
     const int lane = tid & 63;
     const int col = lane & 15;        // B/C column = output row within the tile; also A's row index m
     const int ks = lane >> 4;         // k slice of A and B, row quad of C
-    const int tiles_per_group = kWaves / split;
-    const int tile_in_group = wave / split, part = wave % split;
-    const int passes = (bpr + split * ITERS - 1) / (split * ITERS);
-    const int rounds = (groups - static_cast<int>(blockIdx.x) + static_cast<int>(gridDim.x) - 1) / static_cast<int>(gridDim.x);
-    const int units = rounds * passes;
-    const int tile0 = blockIdx.x * tiles_per_group + tile_in_group, tile_step = gridDim.x * tiles_per_group;
+    const int row = blockIdx.x * kRowsPerTile + col;
+    const uint8_t* wrow = w + static_cast<size_t>(row < n ? row : 0) * bpr * FMT::kBlockBytes;
 
     // A side: this lane supplies row m = col of every MFMA, slice ks; the format says which rows are its
     AMap<FMT::kSlots> am;
     FMT::a_map(am, col, ks, kpad, zero_off);
 
-    typename FMT::Regs cur[ITERS], nxt[ITERS];
-    load_unit<FMT, ITERS>(cur, w, n, bpr, tile0, col, ks, part, split, 0);
-    copy_to_lds(smem, image + static_cast<size_t>(blockIdx.y) * image_stride, image_bytes);
-    if (tid < 4) reinterpret_cast<uint32_t*>(smem + zero_off)[tid] = 0;
-    FMT::stage_tables(tables);
-    __syncthreads();
-
     float acc = 0.0f;
-    int round = 0, pass = 0;
-    for (int u = 0; u < units; ++u) {
-        int next_round = round, next_pass = pass + 1;
-        if (next_pass == passes) { next_pass = 0; ++next_round; }
-        if (u + 1 < units) load_unit<FMT, ITERS>(nxt, w, n, bpr, tile0 + next_round * tile_step, col, ks, part, split, next_pass);
+    bool staged = false;
+    for (int b0 = wave; b0 < bpr || !staged; b0 += waves * ITERS) {
+        typename FMT::Regs regs[ITERS];
 #pragma unroll
         for (int it = 0; it < ITERS; ++it) {
-            // no branch around a block past the row's end (its registers hold the clamped block's data):
-            // the blocks of a unit are then free to overlap; its result is dropped
-            const int b = part + (pass * ITERS + it) * split;
-            const float v = FMT::block(cur[it], ks, min(b, bpr - 1), smem, am, sx, tables);
-            acc += b < bpr ? v : 0.0f;
+            const int b = min(b0 + it * waves, bpr - 1);                    // clamped: always a valid address
+            FMT::load(regs[it], wrow + static_cast<size_t>(b) * FMT::kBlockBytes, ks);
         }
-        if (next_pass == 0) {                                                // the tile's last pass
-            acc += __shfl_xor(acc, 16, 64);
-            acc += __shfl_xor(acc, 32, 64);
-            if (split == 1) {
-                const int row = (tile0 + round * tile_step) * kRowsPerTile + col;
-                if (ks == 0 && row < n) store_any(y, y_dtype, static_cast<size_t>(blockIdx.y) * n + row, acc);
-            } else if (ks == 0) {
-                partial[(round * kWaves + wave) * kRowsPerTile + col] = acc;
-            }
-            acc = 0.0f;
+        if (!staged) {                       // first trip of every thread of the workgroup
+            copy_to_lds(smem, image + static_cast<size_t>(blockIdx.y) * image_stride, image_bytes);
+            if (tid < 4) reinterpret_cast<uint32_t*>(smem + zero_off)[tid] = 0;
+            FMT::stage_tables(tables);
+            __syncthreads();
+            staged = true;
         }
 #pragma unroll
-        for (int it = 0; it < ITERS; ++it) cur[it] = nxt[it];
-        round = next_round; pass = next_pass;
+        for (int it = 0; it < ITERS; ++it) {
+            const int b = b0 + it * waves;
+            if (b < bpr) acc += FMT::block(regs[it], ks, b, smem, am, sx, tables);   // wave-uniform guard
+        }
     }
-    if (split == 1) return;
+    acc += __shfl_xor(acc, 16, 64);
+    acc += __shfl_xor(acc, 32, 64);
+    if (ks == 0) partial[wave * kRowsPerTile + col] = acc;
     __syncthreads();
-    // thread i sums the `split` partials of (round, tile in group, row) = i
-    for (int i = tid; i < rounds * tiles_per_group * kRowsPerTile; i += blockDim.x) {
-        const int r = i / (tiles_per_group * kRowsPerTile), rest = i % (tiles_per_group * kRowsPerTile);
-        const int t = rest / kRowsPerTile, c = rest % kRowsPerTile;
+    if (tid < kRowsPerTile) {
         float total = 0.0f;
-        for (int v = 0; v < split; ++v) total += partial[(r * kWaves + t * split + v) * kRowsPerTile + c];
-        const int row = ((blockIdx.x + r * gridDim.x) * tiles_per_group + t) * kRowsPerTile + c;
-        if (row < n) store_any(y, y_dtype, static_cast<size_t>(blockIdx.y) * n + row, total);
+        for (int v = 0; v < waves; ++v) total += partial[v * kRowsPerTile + tid];
+        const int out_row = blockIdx.x * kRowsPerTile + tid;
+        if (out_row < n) store_any(y, y_dtype, static_cast<size_t>(blockIdx.y) * n + out_row, total);
     }
 }
 
 template <typename FMT, int ITERS>
-int launch_one(const unsigned char* image, size_t image_stride, const uint8_t* w, void* y, int y_dtype,
-               int rows, int n, int bpr, int split, hipStream_t stream) {
-    auto kern = iq_mfma_matvec_kernel<FMT, ITERS>;
-    const size_t fixed = staged_x_bytes(bpr * 256) + 16 + FMT::kTableBytes;
-    // workgroups that fit the device at once (per kernel, asked once)
-    static int resident = 0;
-    if (resident == 0) {
-        int per_cu = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, 64 * kWaves, fixed + 4096) != hipSuccess || per_cu < 1) per_cu = 2;
-        resident = per_cu * compute_units();
-    }
-    const int tiles = (n + kRowsPerTile - 1) / kRowsPerTile;
-    const int groups = (tiles * split + kWaves - 1) / kWaves;
-    int grid = groups;
-    if (groups > resident) {
-        const int rounds = min(kMaxRounds, (groups + resident - 1) / resident);
-        grid = (groups + rounds - 1) / rounds;
-    }
-    const int rounds = (groups + grid - 1) / grid;
-    const size_t smem = fixed + (split > 1 ? static_cast<size_t>(rounds) * kWaves * kRowsPerTile * sizeof(float) : 0);
+int launch_tile(const unsigned char* image, size_t image_stride, const uint8_t* w, void* y, int y_dtype,
+                int rows, int n, int bpr, int waves, hipStream_t stream) {
+    const size_t smem = staged_x_bytes(bpr * 256) + 16 + FMT::kTableBytes + static_cast<size_t>(waves) * kRowsPerTile * sizeof(float);
+    auto kern = mfma_tile_matvec_kernel<FMT, ITERS>;
     if (smem > 64 * 1024) {
         if (smem > 160 * 1024) return PLLM_ERR_UNSUPPORTED;
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                 static_cast<int>(smem)) != hipSuccess)
             return PLLM_ERR_UNSUPPORTED;
     }
-    hipLaunchKernelGGL(kern, dim3(grid, rows), dim3(64 * kWaves), smem, stream, image, image_stride, w, y, y_dtype, n, bpr, split, groups);
+    dim3 grid((n + kRowsPerTile - 1) / kRowsPerTile, rows);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * waves), smem, stream, image, image_stride, w, y, y_dtype, n, bpr);
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+}
+
+template <typename FMT>
+int launch_tiles(const unsigned char* image, size_t image_stride, const uint8_t* w, void* y, int y_dtype,
+                 int rows, int n, int bpr, hipStream_t stream) {
+    // waves per workgroup: split a row's blocks so that every wave keeps a handful in flight
+    int waves = 1;
+    while (waves < kWaves && bpr / (waves * 2) >= 3) waves *= 2;
+    const int niter = (bpr + waves - 1) / waves;
+    const int passes = (niter + 5) / 6;
+    const int iters = (niter + passes - 1) / passes;
+#define PLLM_CASE(I) case I: return launch_tile<FMT, I>(image, image_stride, w, y, y_dtype, rows, n, bpr, waves, stream)
+    switch (iters) {
+        PLLM_CASE(1); PLLM_CASE(2); PLLM_CASE(3); PLLM_CASE(4); PLLM_CASE(5);
+        default: return launch_tile<FMT, 6>(image, image_stride, w, y, y_dtype, rows, n, bpr, waves, stream);
+    }
+#undef PLLM_CASE
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -207,7 +175,7 @@ __global__ __launch_bounds__(64 * kWaves) void iq_stream_matvec_kernel(
                                min(chunk_rows, n - cn * chunk_rows) * row_bytes, wave, lane);
         wait_vm_all_but(newest);             // this wave's pieces of chunk c (and of the image and tables) have landed ...
         __syncthreads();                     // ... and everybody else's too
-        if (NB > 0 && !holding) {
+        if constexpr (NB > 0) if (!holding) {
 #pragma unroll
             for (int i = 0; i < NB; ++i) FMT::hold(held[i], ks, min(part + i * split, bpr - 1), smem, am, sx);
             holding = true;
@@ -217,7 +185,7 @@ __global__ __launch_bounds__(64 * kWaves) void iq_stream_matvec_kernel(
         float acc = 0.0f;
         if (tile_in_chunk * kRowsPerTile < valid_rows) {                     // wave-uniform
             const int row_off = (tile_in_chunk * kRowsPerTile + col) * row_bytes;
-            if (NB > 0) {
+            if constexpr (NB > 0) {
 #pragma unroll
                 for (int i = 0; i < NB; ++i) {
                     const int b = part + i * split;
@@ -259,9 +227,9 @@ template <typename FMT>
 int stream_split(const uint8_t* w, int n, int bpr) {
     if (n % kRowsPerTile != 0 || (reinterpret_cast<uintptr_t>(w) & 15u)) return 0;
     const int tile_bytes = kRowsPerTile * bpr * FMT::kBlockBytes;
-    // the most waves per tile first (smallest chunk) that leaves every wave at least three blocks
+    // the most waves per tile first (smallest chunk) that leaves every wave at least two blocks
     for (int split = kWaves; split >= 1; split /= 2)
-        if ((split == 1 || bpr >= 3 * split) && (kWaves / split) * tile_bytes <= kChunkBudget) return split;
+        if ((split == 1 || bpr >= 2 * split) && (kWaves / split) * tile_bytes <= kChunkBudget) return split;
     return 0;
 }
 
@@ -301,30 +269,18 @@ template <typename FMT>
 int launch_stream(const unsigned char* image, size_t image_stride, const uint8_t* w, void* y, int y_dtype,
                   int rows, int n, int bpr, int split, hipStream_t stream) {
     const int per_wave = (bpr + split - 1) / split;                          // block indices a wave meets
-    if (FMT::kHoldBlocks >= 2 && per_wave <= 2) return launch_stream_nb<FMT, 2>(image, image_stride, w, y, y_dtype, rows, n, bpr, split, stream);
-    if (FMT::kHoldBlocks >= 3 && per_wave == 3) return launch_stream_nb<FMT, 3>(image, image_stride, w, y, y_dtype, rows, n, bpr, split, stream);
+    if constexpr (FMT::kHoldBlocks >= 2) if (per_wave <= 2) return launch_stream_nb<FMT, 2>(image, image_stride, w, y, y_dtype, rows, n, bpr, split, stream);
+    if constexpr (FMT::kHoldBlocks >= 3) if (per_wave == 3) return launch_stream_nb<FMT, 3>(image, image_stride, w, y, y_dtype, rows, n, bpr, split, stream);
     return launch_stream_nb<FMT, 0>(image, image_stride, w, y, y_dtype, rows, n, bpr, split, stream);
 }
 
 template <typename FMT>
 int launch_fmt(const unsigned char* image, size_t image_stride, const uint8_t* w, void* y, int y_dtype,
                int rows, int n, int bpr, hipStream_t stream) {
+    // whole tiles streamed through long-lived workgroups (the codebooks are staged once per workgroup)
+    // where shape and alignment allow, else one short workgroup per tile
     if (const int split = stream_split<FMT>(w, n, bpr)) return launch_stream<FMT>(image, image_stride, w, y, y_dtype, rows, n, bpr, split, stream);
-    // waves per row tile: one when there are tiles enough to keep every wave of the device busy
-    // several times over, more (each with at least two super-blocks) for short matrices
-    const int tiles = (n + kRowsPerTile - 1) / kRowsPerTile;
-    const int want = 6 * compute_units();
-    int split = 1;
-    while (split < kWaves && split * 4 <= bpr && (tiles * split + kWaves - 1) / kWaves * rows < want) split *= 2;
-    const int niter = (bpr + split - 1) / split;
-    const int passes = (niter + 3) / 4;
-    const int iters = (niter + passes - 1) / passes;
-#define PLLM_CASE(I) case I: return launch_one<FMT, I>(image, image_stride, w, y, y_dtype, rows, n, bpr, split, stream)
-    switch (iters) {
-        PLLM_CASE(1); PLLM_CASE(2); PLLM_CASE(3);
-        default: return launch_one<FMT, 4>(image, image_stride, w, y, y_dtype, rows, n, bpr, split, stream);
-    }
-#undef PLLM_CASE
+    return launch_tiles<FMT>(image, image_stride, w, y, y_dtype, rows, n, bpr, stream);
 }
 
 }  // namespace
