@@ -271,6 +271,30 @@ def pmc_pass(mod, dev) -> None:
     print(json.dumps({"pmc_pass": f"{name} matvec {n}x{k}", "weight_bytes": int(blocks.size), "copy_bytes": int(nbytes)}))
 
 
+def iq_pass(mod, dev) -> None:
+    """A few launches of the codebook formats for the profiler: IQ2_XXS 98304x3072 and IQ1_M 196608x1536 matvec, then the
+    single-token routed experts of the 256-expert top-8 configuration."""
+    from pocketllm_amd import block_codec as C, codebooks
+    rng = np.random.default_rng(5005)
+    for tid, n, k, gen, grid in ((0, 64 * 1536, 3072, C.random_iq2_xxs, codebooks.get_iq2xxs_signed_grid_tensor()),
+                                 (2, 64 * 3072, 1536, C.random_iq1_m, codebooks.get_iq1_grid_tensor())):
+        ring = ring_of(gen(rng, n, k // 256), dev, 4)
+        x = torch.randn(1, k, device=dev, dtype=torch.bfloat16)
+        for i in range(8):
+            mod.gguf_quant_gemm_forward(x, ring[i % len(ring)], k, tid, grid.to(dev))
+        del ring
+    e, d, inter = 256, 3072, 1536
+    w1 = torch.from_numpy(C.random_iq2_xxs(rng, e, inter, d // 256, d_range=(0.002, 0.006))).to(dev)
+    w3 = torch.from_numpy(C.random_iq2_xxs(rng, e, inter, d // 256, d_range=(0.002, 0.006))).to(dev)
+    w2 = torch.from_numpy(C.random_iq1_m(rng, e, d, inter // 256, d_range=(0.002, 0.006))).to(dev)
+    x = torch.randn(1, d, device=dev, dtype=torch.bfloat16)
+    for _ in range(8):
+        topi = torch.from_numpy(rng.choice(e, size=8, replace=False).astype(np.int64)).to(dev)
+        mod.gguf_moe_single_token_forward(x, topi, torch.full((8,), 0.125, device=dev), w1, w3, w2, 0.0)
+    torch.cuda.synchronize()
+    print(json.dumps({"iq_pass": "iq2_xxs 98304x3072, iq1_m 196608x1536, single-token experts 256 x top-8"}))
+
+
 def prefill_pass(mod, dev) -> None:
     """A few launches of the MFMA tile kernel for the profiler: Q4_K 17408x5120 at T=2048 and FP8 at T=512."""
     from pocketllm_amd import block_codec as C
@@ -300,6 +324,7 @@ def main() -> None:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--pmc-pass", action="store_true", help="short run for rocprofv3 --pmc: dominant kernel + a copy of the same size")
     ap.add_argument("--prefill-pass", action="store_true", help="short run for rocprofv3: a few launches of the MFMA tile kernel")
+    ap.add_argument("--iq-pass", action="store_true", help="short run for rocprofv3: IQ2_XXS / IQ1_M matvec and the single-token experts")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU (no sharding, no collectives); run with --gpus 1")
@@ -319,6 +344,9 @@ def main() -> None:
         return
     if args.prefill_pass:
         prefill_pass(mod, dev)
+        return
+    if args.iq_pass:
+        iq_pass(mod, dev)
         return
     x_np = np.random.default_rng(2002).standard_normal((1, 5120), dtype=np.float32)
     x = torch.from_numpy(x_np).to(dev).to(torch.bfloat16)
