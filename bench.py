@@ -152,12 +152,14 @@ def extra_cases(mod, dev, iters):
         x = torch.randn(1, k, device=dev)
         run(f"q8_0 matvec {n}x{k} T=1", blocks.size, lambda s, ring=ring, x=x, k=k: mod.q8_0_gemm_forward(x, ring[s], k), len(ring))
         del ring
-    # Q2_K at the large shape
-    blocks = C.quantize_q2_k((rng.standard_normal((17408, 5120), dtype=np.float32) * np.float32(0.02)))
-    ring = ring_of(blocks, dev)
+    # Q2_K, Q6_K and IQ4_XS at the large shape (random valid blocks for the latter two: the kernels' work does not depend on the values)
     x = torch.randn(1, 5120, device=dev, dtype=torch.bfloat16)
-    run("q2_k matvec 17408x5120 T=1", blocks.size, lambda s, ring=ring, x=x: mod.gguf_quant_gemm_forward(x, ring[s], 5120, 1, empty), len(ring))
-    del ring
+    for name, tid, blocks in (("q2_k", 1, C.quantize_q2_k((rng.standard_normal((17408, 5120), dtype=np.float32) * np.float32(0.02)))),
+                              ("q6_k", 8, C.random_blocks(rng, "q6_k", 17408, 20)), ("iq4_xs", 7, C.random_blocks(rng, "iq4_xs", 17408, 20))):
+        ring = ring_of(blocks, dev, max(2, min(RING, (1 << 30) // blocks.size)))
+        run(f"{name} matvec 17408x5120 T=1", blocks.size,
+            lambda s, ring=ring, x=x, tid=tid: mod.gguf_quant_gemm_forward(x, ring[s], 5120, tid, empty), len(ring))
+        del ring
     # FP8 E4M3 + 128x128 scales, BASELINE config 4 at T=1
     codes, scale = C.quantize_fp8_block((rng.standard_normal((17408, 5120), dtype=np.float32) * np.float32(0.02)))
     ring = ring_of(codes, dev, 8)

@@ -16,6 +16,10 @@ How each function is pinned (what a wrong sign / index / transposed operand woul
   dequant_q4_k,
   dequant_q5_k       hand-built blocks that isolate every field (scale index j<4 / j>=4, nibble
                      halves, qh bit planes) plus fixtures written by the reference's numpy reader.
+  dequant_q6_k,
+  dequant_iq4_xs     fixtures written by the reference's numpy reader, hand-built blocks with one
+                     live field (every scale index, both nibble halves, every qh bit pair / high
+                     scale bit pair), and a per-weight scalar restatement of the ggml layout.
   fp8_e4m3_decode    torch's float8_e4m3fn cast over all 256 codes.
   q8_1_quantize,
   fp8_act_quant      invariants (|q*d - x| <= d/2, clamp range) and torch's e4m3 cast.
@@ -34,10 +38,10 @@ import numpy as np
 _CODEBOOK_FILE = Path(__file__).resolve().parents[1] / "pocketllm_amd" / "csrc" / "ggml_codebooks.inc"
 
 # type_id map of the reference: src/loader/gguf/quant_types.py:3-13, src/csrc/cuda_kernel.cpp:401-412
-TYPE_IDS = {"iq2_xxs": 0, "q2_k": 1, "iq1_m": 2, "q4_k": 3, "q5_k": 4}
+TYPE_IDS = {"iq2_xxs": 0, "q2_k": 1, "iq1_m": 2, "q4_k": 3, "q5_k": 4, "iq4_xs": 7, "q6_k": 8}
 TYPE_NAMES = {v: k for k, v in TYPE_IDS.items()}
-BLOCK_BYTES = {"q8_0": 34, "iq2_xxs": 66, "q2_k": 84, "iq1_m": 56, "q4_k": 144, "q5_k": 176}
-BLOCK_ELEMS = {"q8_0": 32, "iq2_xxs": 256, "q2_k": 256, "iq1_m": 256, "q4_k": 256, "q5_k": 256}
+BLOCK_BYTES = {"q8_0": 34, "iq2_xxs": 66, "q2_k": 84, "iq1_m": 56, "q4_k": 144, "q5_k": 176, "iq4_xs": 136, "q6_k": 210}
+BLOCK_ELEMS = {"q8_0": 32, "iq2_xxs": 256, "q2_k": 256, "iq1_m": 256, "q4_k": 256, "q5_k": 256, "iq4_xs": 256, "q6_k": 256}
 
 
 # --------------------------------------------------------------------------------------------
@@ -217,9 +221,60 @@ def dequant_iq1_m(blocks: np.ndarray) -> np.ndarray:
     return out.reshape(lead + (256,))
 
 
+def dequant_q6_k(blocks: np.ndarray) -> np.ndarray:
+    """Q6_K: ql(128) qh(64) scales int8(16) d(f16); w = d * scales[i // 16] * (q - 32), q = 4 low bits from ql and 2
+    high bits from qh.  Reference: tensor_reader.py:868-908."""
+    assert blocks.dtype == np.uint8 and blocks.shape[-1] == 210
+    ql = blocks[..., 0:128]
+    qh = blocks[..., 128:192]
+    scales = blocks[..., 192:208].view(np.int8).astype(np.float32)
+    d = _f16(blocks[..., 208:210])[..., None]
+    out = np.empty(blocks.shape[:-1] + (256,), dtype=np.float32)
+    for half in range(2):
+        ql_a = ql[..., 64 * half:64 * half + 32]
+        ql_b = ql[..., 64 * half + 32:64 * half + 64]
+        qh_h = qh[..., 32 * half:32 * half + 32]
+        sc = scales[..., 8 * half:8 * half + 8]
+        quads = (
+            (ql_a & 0x0F) | (((qh_h >> 0) & 3) << 4),
+            (ql_b & 0x0F) | (((qh_h >> 2) & 3) << 4),
+            (ql_a >> 4) | (((qh_h >> 4) & 3) << 4),
+            (ql_b >> 4) | (((qh_h >> 6) & 3) << 4),
+        )
+        for j, q in enumerate(quads):
+            # weights 128 half + 32 j + l, l < 32: scale index 2 j + l // 16 of the half
+            scale = np.repeat(sc[..., 2 * j:2 * j + 2], 16, axis=-1)
+            out[..., 128 * half + 32 * j:128 * half + 32 * j + 32] = d * scale * (q.astype(np.int16) - 32).astype(np.float32)
+    return out
+
+
+IQ4_KVALUES = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], dtype=np.float32)
+
+
+def dequant_iq4_xs(blocks: np.ndarray) -> np.ndarray:
+    """IQ4_XS: d(f16) scales_h(u16) scales_l(4) qs(128); per 32 weights a 6-bit scale (4 low bits from scales_l, 2 high
+    bits from scales_h) minus 32; 16 bytes per group, low nibbles = weights 0..15, high nibbles = weights 16..31, codes
+    through the 16-entry non-linear table.  Reference: tensor_reader.py:918-948."""
+    assert blocks.dtype == np.uint8 and blocks.shape[-1] == 136
+    d = _f16(blocks[..., 0:2])[..., None]
+    scales_h = (blocks[..., 2].astype(np.uint16) | (blocks[..., 3].astype(np.uint16) << 8))
+    scales_l = blocks[..., 4:8]
+    qs = blocks[..., 8:136]
+    out = np.empty(blocks.shape[:-1] + (256,), dtype=np.float32)
+    for g in range(8):
+        lo4 = (scales_l[..., g // 2] >> (4 if g & 1 else 0)) & 0x0F
+        hi2 = (scales_h >> (2 * g)) & 3
+        scale = ((lo4.astype(np.int16) | (hi2.astype(np.int16) << 4)) - 32).astype(np.float32)[..., None]
+        q = qs[..., 16 * g:16 * g + 16]
+        out[..., 32 * g:32 * g + 16] = d * scale * IQ4_KVALUES[q & 0x0F]
+        out[..., 32 * g + 16:32 * g + 32] = d * scale * IQ4_KVALUES[q >> 4]
+    return out
+
+
 _DECODERS = {
     "q8_0": dequant_q8_0, "q4_k": dequant_q4_k, "q5_k": dequant_q5_k,
     "q2_k": dequant_q2_k, "iq2_xxs": dequant_iq2_xxs, "iq1_m": dequant_iq1_m,
+    "q6_k": dequant_q6_k, "iq4_xs": dequant_iq4_xs,
 }
 
 

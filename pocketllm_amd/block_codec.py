@@ -6,7 +6,7 @@ activation quantizers.  Synthetic benchmarks and tests still need valid blocks, 
 simple encoders of this library's own.  Every correctness statement elsewhere is about
 blocks -> values, never about how good an encoder is.
 
-Layouts are the GGUF ones: Q8_0 34 B / 32 weights; Q2_K 84 B, Q4_K 144 B, Q5_K 176 B, IQ2_XXS 66 B,
+Layouts are the GGUF ones: Q8_0 34 B / 32 weights; Q2_K 84 B, Q4_K 144 B, Q5_K 176 B, Q6_K 210 B, IQ4_XS 136 B, IQ2_XXS 66 B,
 IQ1_M 56 B per 256 weights; FP8 is one OCP E4M3FN byte per weight plus a float32 scale per 128x128.
 """
 from __future__ import annotations
@@ -135,6 +135,66 @@ def quantize_q2_k(weight: np.ndarray) -> np.ndarray:
         blocks[..., start:start + 16] |= q[:, :, group] << shift
     blocks[..., 80:82] = _f16_bytes(d)
     blocks[..., 82:84] = _f16_bytes(dmin)
+    return blocks
+
+
+def quantize_q6_k(weight: np.ndarray) -> np.ndarray:
+    """float [N, K] -> uint8 [N, ceil(K/256), 210] (ql[128], qh[64], scales int8[16], d): w ~= d * scale[i // 16] * (q - 32)."""
+    w = _pad_rows(np.asarray(weight, dtype=np.float32), 256)
+    n = w.shape[0]
+    v = w.reshape(n, -1, 16, 16)
+    amax = np.abs(v).max(axis=-1)
+    gscale = amax / np.float32(31.0)                                         # per 16 weights
+    d = np.maximum(gscale.max(axis=-1), np.float32(1e-12)) / np.float32(127.0)
+    d = d.astype(np.float16).astype(np.float32)
+    sc = np.clip(np.rint(gscale / d[..., None]), 1, 127).astype(np.int8)
+    q = np.clip(np.rint(v / (d[..., None, None] * sc.astype(np.float32)[..., None])) + 32, 0, 63).astype(np.uint8)
+    q = q.reshape(n, -1, 2, 4, 32)                                           # [half][j][l]: weight 128 half + 32 j + l
+    blocks = np.zeros((n, v.shape[1], 210), dtype=np.uint8)
+    for half in range(2):
+        blocks[..., 64 * half:64 * half + 32] = (q[:, :, half, 0] & 15) | ((q[:, :, half, 2] & 15) << 4)
+        blocks[..., 64 * half + 32:64 * half + 64] = (q[:, :, half, 1] & 15) | ((q[:, :, half, 3] & 15) << 4)
+        blocks[..., 128 + 32 * half:160 + 32 * half] = ((q[:, :, half, 0] >> 4) | ((q[:, :, half, 1] >> 4) << 2) |
+                                                        ((q[:, :, half, 2] >> 4) << 4) | ((q[:, :, half, 3] >> 4) << 6))
+    blocks[..., 192:208] = sc.view(np.uint8)
+    blocks[..., 208:210] = _f16_bytes(d)
+    return blocks
+
+
+IQ4_KVALUES = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], dtype=np.float32)
+
+
+def quantize_iq4_xs(weight: np.ndarray) -> np.ndarray:
+    """float [N, K] -> uint8 [N, ceil(K/256), 136] (d, scales_h u16, scales_l[4], qs[128]): w ~= d * (ls - 32) * kvalues[code],
+    16 bytes per 32 weights with weights 0..15 in the low and 16..31 in the high nibbles."""
+    w = _pad_rows(np.asarray(weight, dtype=np.float32), 256)
+    n = w.shape[0]
+    v = w.reshape(n, -1, 8, 32)
+    gscale = np.abs(v).max(axis=-1) / np.float32(127.0)                      # per 32 weights
+    d = np.maximum(gscale.max(axis=-1), np.float32(1e-12)) / np.float32(31.0)
+    d = d.astype(np.float16).astype(np.float32)
+    ls = np.clip(np.rint(gscale / d[..., None]), 1, 31).astype(np.int16)      # scale - 32 in [1, 31]
+    target = v / (d[..., None, None] * ls.astype(np.float32)[..., None])
+    code = np.abs(target[..., None] - IQ4_KVALUES).argmin(axis=-1).astype(np.uint8)
+    blocks = np.zeros((n, v.shape[1], 136), dtype=np.uint8)
+    blocks[..., 0:2] = _f16_bytes(d)
+    stored = (ls + 32).astype(np.uint16)
+    sh = np.zeros(stored.shape[:-1], dtype=np.uint16)
+    for g in range(8):
+        sh |= ((stored[..., g] >> 4) & 3) << (2 * g)
+        blocks[..., 4 + g // 2] |= ((stored[..., g] & 15) << (4 if g & 1 else 0)).astype(np.uint8)
+        blocks[..., 8 + 16 * g:24 + 16 * g] = code[:, :, g, 0:16] | (code[:, :, g, 16:32] << 4)
+    blocks[..., 2] = (sh & 0xFF).astype(np.uint8)
+    blocks[..., 3] = (sh >> 8).astype(np.uint8)
+    return blocks
+
+
+def random_blocks(rng: np.random.Generator, type_name: str, *lead: int, d_range=(0.001, 0.02)) -> np.ndarray:
+    """Every byte random except the fp16 scale field (finite, drawn from d_range): q6_k or iq4_xs."""
+    nbytes, off = {"q6_k": (210, 208), "iq4_xs": (136, 0)}[type_name]
+    blocks = rng.integers(0, 256, size=tuple(lead) + (nbytes,), dtype=np.uint8)
+    d = rng.uniform(d_range[0], d_range[1], size=tuple(lead)).astype(np.float32)
+    blocks[..., off:off + 2] = _f16_bytes(d)
     return blocks
 
 

@@ -1,4 +1,4 @@
-// Per-format pieces of the matrix-core kernels over IQ2_XXS and IQ1_M super-blocks, and the
+// Per-format pieces of the matrix-core kernels over IQ2_XXS, IQ1_M, IQ4_XS and Q6_K super-blocks, and the
 // direct-to-LDS copy helpers they share.
 //
 // Lane map: lane (n, s) = (lane % 16, lane / 16) of a wave works on output row n of a 16-row tile and
@@ -76,6 +76,7 @@ struct IQ2XXSm {
     static constexpr int kBlockBytes = 66;
     static constexpr int kTableBytes = IQ2XXS::kTableBytes;
     static constexpr int kSlots = 4;
+    static constexpr bool kStreamed = true;                    // has LDS loaders and table copies for the streamed kernel
     static constexpr int kHoldBlocks = 3;                      // block indices whose activation side a wave may keep in registers
     struct Regs { uint4 q; uint32_t d; };
     static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, int s) {
@@ -171,6 +172,7 @@ struct IQ1Mm {
     static constexpr int kBlockBytes = 56;
     static constexpr int kTableBytes = 32768;
     static constexpr int kSlots = 8;                           // [term][t]
+    static constexpr bool kStreamed = true;
     static constexpr int kHoldBlocks = 0;                      // (its held operands would cost a workgroup per compute unit)
     struct Regs { uint2 qs; uint32_t qh; uint2 sc; };
     static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, int s) {
@@ -241,6 +243,129 @@ struct IQ1Mm {
         Held h;
         hold(h, s, b, smem, am, sx);
         return block_held(r, s, b, h, smem, am, tables);
+    }
+};
+
+// ------------------------------------------------------------------------------------------------
+// Q6_K: 210 B = ql(128) qh(64) scales int8(16) d(2); w = d * scale[i / 16] * (q - 32), q = a nibble of ql
+// plus two bits of qh.  Lane (n, s), half = s / 2, part = s % 2, holds ql[64 half + 16 part, +16),
+// ql[64 half + 32 + 16 part, +16) and qh[32 half + 16 part, +16): the 16-weight groups
+// 8 half + 2 t + part, t = 0..3 (low nibbles of the first piece, of the second, then their high
+// nibbles, with bit pair t of qh).  A rows: m = 16-group, one MFMA set per activation term; MFMA t,
+// slice s carries that group.  The codes stay unsigned (0..63): the "- 32" leaves through the
+// image's 16-value sums.  C[4 s .. 4 s + 3][n] are groups 4 s .. 4 s + 3, scale bytes = dword s of scales.
+// Blocks are only 2-byte aligned.
+// ------------------------------------------------------------------------------------------------
+struct __attribute__((packed, aligned(2))) Unaligned4 { uint32_t v; };
+
+struct Q6Km {
+    static constexpr int kBlockBytes = 210;
+    static constexpr int kTableBytes = 0;
+    static constexpr int kSlots = 8;                           // [term][t]
+    static constexpr bool kStreamed = false;
+    struct Regs { uint4 qa, qb, qh; uint32_t sc, d; };
+    static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, int s) {
+        const int half = s >> 1, part = s & 1;
+        r.qa = load16_a2(blk + 64 * half + 16 * part);
+        r.qb = load16_a2(blk + 64 * half + 32 + 16 * part);
+        r.qh = load16_a2(blk + 128 + 32 * half + 16 * part);
+        r.sc = reinterpret_cast<const Unaligned4*>(blk + 192 + 4 * s)->v;
+        r.d = *reinterpret_cast<const uint16_t*>(blk + 208);
+    }
+    static __device__ __forceinline__ void stage_tables(unsigned char*) {}
+    static __device__ __forceinline__ void a_map(AMap<kSlots>& am, int col, int ks, int kpad, int zero_off) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const bool active = col == 8 * (ks >> 1) + 2 * t + (ks & 1);
+            am.off[t] = active ? 16 * col : zero_off;
+            am.off[4 + t] = active ? kpad + 16 * col : zero_off;
+            am.step[t] = am.step[4 + t] = active ? 256 : 0;
+        }
+    }
+    static __device__ __forceinline__ uint32_t code4(uint32_t ql, uint32_t qh, int t) {
+        const uint32_t lo = (t < 2 ? ql : ql >> 4) & 0x0f0f0f0fu;
+        const uint32_t hi = (t == 0 ? qh << 4 : t == 1 ? qh << 2 : t == 2 ? qh : qh >> 2) & 0x30303030u;
+        return lo | hi;
+    }
+    static __device__ __forceinline__ float block(const Regs& r, int s, int b, const unsigned char* smem, const AMap<kSlots>& am,
+                                                  const StagedX& sx, const unsigned char*) {
+        v4i ch = {0, 0, 0, 0}, cl = {0, 0, 0, 0};
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const uint4 ql = (t & 1) ? r.qb : r.qa;
+            const v4i bw = as_v4i(code4(ql.x, r.qh.x, t), code4(ql.y, r.qh.y, t), code4(ql.z, r.qh.z, t), code4(ql.w, r.qh.w, t));
+            const uint4 ah = *reinterpret_cast<const uint4*>(smem + am.off[t] + b * am.step[t]);
+            const uint4 al = *reinterpret_cast<const uint4*>(smem + am.off[4 + t] + b * am.step[4 + t]);
+            ch = __builtin_amdgcn_mfma_i32_16x16x64_i8(as_v4i(ah.x, ah.y, ah.z, ah.w), bw, ch, 0, 0, 0);
+            cl = __builtin_amdgcn_mfma_i32_16x16x64_i8(as_v4i(al.x, al.y, al.z, al.w), bw, cl, 0, 0, 0);
+        }
+        const float4 g2 = *reinterpret_cast<const float4*>(sx.gs + b * 8 + 2 * s);   // {xs0 / 254, sum0, xs1 / 254, sum1}
+        const float4 s16 = *reinterpret_cast<const float4*>(sx.sum16 + b * 16 + 4 * s);
+        const int sc = static_cast<int>(r.sc);
+        const float v = static_cast<float>(static_cast<int8_t>(sc)) * (g2.x * static_cast<float>(__mul24(ch.x, 254) + cl.x) - 32.0f * s16.x) +
+                        static_cast<float>(static_cast<int8_t>(sc >> 8)) * (g2.x * static_cast<float>(__mul24(ch.y, 254) + cl.y) - 32.0f * s16.y) +
+                        static_cast<float>(static_cast<int8_t>(sc >> 16)) * (g2.z * static_cast<float>(__mul24(ch.z, 254) + cl.z) - 32.0f * s16.z) +
+                        static_cast<float>(sc >> 24) * (g2.z * static_cast<float>(__mul24(ch.w, 254) + cl.w) - 32.0f * s16.w);
+        return f16_bits_to_float(r.d) * v;
+    }
+};
+
+// ------------------------------------------------------------------------------------------------
+// IQ4_XS: 136 B = d(2) scales_h(2) scales_l(4) qs(128); w = d * (ls - 32) * kvalues[code], ls six bits per
+// 32 weights (low four in a nibble of scales_l, high two in scales_h), 16 bytes per group with
+// weights 0..15 in the low and 16..31 in the high nibbles.  Lane (n, s) holds qs[32 s, 32 s + 32) =
+// groups 2 s and 2 s + 1.  A rows as for IQ2_XXS: m = 2 * group + term; MFMA t, slice s carries half
+// t % 2 of group 2 s + t / 2.  The 16-entry code table sits in four registers; a byte permute picks
+// from its lower and upper half and a third one chooses between them by bit 3 of the code.
+// ------------------------------------------------------------------------------------------------
+struct IQ4XSm {
+    static constexpr int kBlockBytes = 136;
+    static constexpr int kTableBytes = 0;
+    static constexpr int kSlots = 4;
+    static constexpr bool kStreamed = false;
+    struct Regs { uint4 q0, q1; uint2 hdr; };
+    static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, int s) {
+        const uint2* p = reinterpret_cast<const uint2*>(blk);                  // blocks are 8-byte aligned
+        r.hdr = p[0];
+        r.q0 = make_uint4(p[1 + 4 * s].x, p[1 + 4 * s].y, p[2 + 4 * s].x, p[2 + 4 * s].y);
+        r.q1 = make_uint4(p[3 + 4 * s].x, p[3 + 4 * s].y, p[4 + 4 * s].x, p[4 + 4 * s].y);
+    }
+    static __device__ __forceinline__ void stage_tables(unsigned char*) {}
+    static __device__ __forceinline__ void a_map(AMap<kSlots>& am, int col, int ks, int kpad, int zero_off) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int g = 2 * ks + (t >> 1);
+            const bool active = (col >> 1) == g;
+            am.off[t] = active ? ((col & 1) ? kpad : 0) + 32 * g + 16 * (t & 1) : zero_off;
+            am.step[t] = active ? 256 : 0;
+        }
+    }
+    // four codes (one per byte, 0..15) -> four table values
+    static __device__ __forceinline__ uint32_t values4(uint32_t codes) {
+        const uint32_t low3 = codes & 0x07070707u;
+        const uint32_t lower = __builtin_amdgcn_perm(0xF6EADDCFu, 0xBFAD9881u, low3);   // -127 -104 -83 -65 | -49 -35 -22 -10
+        const uint32_t upper = __builtin_amdgcn_perm(0x71594535u, 0x26190D01u, low3);   // 1 13 25 38 | 53 69 89 113
+        return __builtin_amdgcn_perm(upper, lower, ((codes >> 1) & 0x04040404u) | 0x03020100u);
+    }
+    static __device__ __forceinline__ float block(const Regs& r, int s, int b, const unsigned char* smem, const AMap<kSlots>& am,
+                                                  const StagedX& sx, const unsigned char*) {
+        v4i c = {0, 0, 0, 0};
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const uint4 q = (t < 2) ? r.q0 : r.q1;
+            const int sh = 4 * (t & 1);
+            const v4i bw = as_v4i(values4((q.x >> sh) & 0x0f0f0f0fu), values4((q.y >> sh) & 0x0f0f0f0fu),
+                                  values4((q.z >> sh) & 0x0f0f0f0fu), values4((q.w >> sh) & 0x0f0f0f0fu));
+            const uint4 a = *reinterpret_cast<const uint4*>(smem + am.off[t] + b * am.step[t]);
+            c = __builtin_amdgcn_mfma_i32_16x16x64_i8(as_v4i(a.x, a.y, a.z, a.w), bw, c, 0, 0, 0);
+        }
+        const float v0 = static_cast<float>(__mul24(c.x, 254) + c.y);         // group 2 s: 254 * high term + low term
+        const float v1 = static_cast<float>(__mul24(c.z, 254) + c.w);         // group 2 s + 1
+        const float4 g2 = *reinterpret_cast<const float4*>(sx.gs + b * 8 + 2 * s);   // {xs0 / 254, sum0, xs1 / 254, sum1}
+        const uint32_t scales_h = r.hdr.x >> 16, sl = (r.hdr.y >> (8 * s)) & 0xffu;
+        const int ls0 = static_cast<int>((sl & 15u) | (((scales_h >> (4 * s)) & 3u) << 4)) - 32;
+        const int ls1 = static_cast<int>((sl >> 4) | (((scales_h >> (4 * s + 2)) & 3u) << 4)) - 32;
+        return f16_bits_to_float(r.hdr.x & 0xffffu) * (static_cast<float>(ls0) * g2.x * v0 + static_cast<float>(ls1) * g2.z * v1);
     }
 };
 

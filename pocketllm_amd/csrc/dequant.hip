@@ -73,6 +73,29 @@ __device__ float dequant_iq1_m(const uint8_t* b, int e) {
     return dl * (g + ((h & 8u) ? -0.125f : 0.125f));
 }
 
+// Q6_K: ql(128) qh(64) scales int8(16) d; weight e = 128 half + 32 j + l takes nibble j / 2 of ql[64 half + 32 (j % 2) + l],
+// bit pair j of qh[32 half + l] and scale e / 16
+__device__ float dequant_q6_k(const uint8_t* b, int e) {
+    const int half = e >> 7, j = (e >> 5) & 3, l = e & 31;
+    const uint32_t lo = (b[64 * half + 32 * (j & 1) + l] >> (4 * (j >> 1))) & 15u;
+    const uint32_t hi = (b[128 + 32 * half + l] >> (2 * j)) & 3u;
+    const int q = static_cast<int>(lo | (hi << 4)) - 32;
+    const float d = f16_at(b + 208);
+    return d * static_cast<float>(static_cast<int8_t>(b[192 + (e >> 4)])) * static_cast<float>(q);
+}
+
+__device__ const int8_t kIq4Values[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+
+// IQ4_XS: d, scales_h u16, scales_l(4), qs(128); group g = e / 32: 6-bit scale - 32, byte 16 g + e % 16, low nibble for the
+// first 16 weights of the group and high nibble for the others
+__device__ float dequant_iq4_xs(const uint8_t* b, int e) {
+    const int g = e >> 5, i = e & 31;
+    const uint32_t sh = static_cast<uint32_t>(b[2]) | (static_cast<uint32_t>(b[3]) << 8);
+    const int ls = static_cast<int>(((b[4 + (g >> 1)] >> (4 * (g & 1))) & 15u) | (((sh >> (2 * g)) & 3u) << 4)) - 32;
+    const uint32_t code = (b[8 + 16 * g + (i & 15)] >> (4 * (i >> 4))) & 15u;
+    return f16_at(b) * static_cast<float>(ls) * static_cast<float>(kIq4Values[code]);
+}
+
 // grid (selected rows, ceil(k / 256)), 256 threads
 __global__ __launch_bounds__(256) void dequant_rows_kernel(
     const int64_t* __restrict__ row_ids, const uint8_t* __restrict__ blocks, int type_id, void* __restrict__ out, int out_dtype,
@@ -93,6 +116,8 @@ __global__ __launch_bounds__(256) void dequant_rows_kernel(
                 case PLLM_TYPE_Q5_K: v = dequant_q5_k(b, e); break;
                 case PLLM_TYPE_Q2_K: v = dequant_q2_k(b, e); break;
                 case PLLM_TYPE_IQ2_XXS: v = dequant_iq2_xxs(b, e); break;
+                case PLLM_TYPE_Q6_K: v = dequant_q6_k(b, e); break;
+                case PLLM_TYPE_IQ4_XS: v = dequant_iq4_xs(b, e); break;
                 default: v = dequant_iq1_m(b, e); break;
             }
         }

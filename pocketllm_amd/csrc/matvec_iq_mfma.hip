@@ -1,4 +1,4 @@
-// Decode matvec over raw IQ2_XXS / IQ1_M super-blocks with the integer dots on the matrix cores.
+// Decode matvec over raw IQ2_XXS / IQ1_M / IQ4_XS / Q6_K super-blocks with the integer dots on the matrix cores.
 //
 // A wave owns a tile of 16 consecutive output rows (or, for short matrices, a share of the tile's
 // super-blocks; the shares meet in a small LDS reduction); the activation image (two int8 terms per
@@ -279,7 +279,8 @@ int launch_fmt(const unsigned char* image, size_t image_stride, const uint8_t* w
                int rows, int n, int bpr, hipStream_t stream) {
     // whole tiles streamed through long-lived workgroups (the codebooks are staged once per workgroup)
     // where shape and alignment allow, else one short workgroup per tile
-    if (const int split = stream_split<FMT>(w, n, bpr)) return launch_stream<FMT>(image, image_stride, w, y, y_dtype, rows, n, bpr, split, stream);
+    if constexpr (FMT::kStreamed)
+        if (const int split = stream_split<FMT>(w, n, bpr)) return launch_stream<FMT>(image, image_stride, w, y, y_dtype, rows, n, bpr, split, stream);
     return launch_tiles<FMT>(image, image_stride, w, y, y_dtype, rows, n, bpr, stream);
 }
 
@@ -290,6 +291,8 @@ int iq_mfma_matvec_from_image(const unsigned char* image, size_t stride, const u
     switch (type_id) {
         case PLLM_TYPE_IQ2_XXS: return launch_fmt<IQ2XXSm>(image, stride, w, y, y_dtype, rows, n, bpr, stream);
         case PLLM_TYPE_IQ1_M: return launch_fmt<IQ1Mm>(image, stride, w, y, y_dtype, rows, n, bpr, stream);
+        case PLLM_TYPE_IQ4_XS: return launch_fmt<IQ4XSm>(image, stride, w, y, y_dtype, rows, n, bpr, stream);
+        case PLLM_TYPE_Q6_K: return launch_fmt<Q6Km>(image, stride, w, y, y_dtype, rows, n, bpr, stream);
         default: return PLLM_ERR_UNSUPPORTED;
     }
 }

@@ -14,7 +14,7 @@ from pocketllm_amd.cuda_loader import load_cuda_kernel
 pytestmark = pytest.mark.gpu
 
 TOL = 1e-3
-ENCODERS = {"q4_k": C.quantize_q4_k, "q5_k": C.quantize_q5_k, "q2_k": C.quantize_q2_k}
+ENCODERS = {"q4_k": C.quantize_q4_k, "q5_k": C.quantize_q5_k, "q2_k": C.quantize_q2_k, "q6_k": C.quantize_q6_k, "iq4_xs": C.quantize_iq4_xs}
 
 
 @pytest.fixture(scope="module")
@@ -39,7 +39,7 @@ def _run_dense(mod, type_name, blocks, x_np, x_dtype, k):
     return x.float().cpu().numpy(), y.cpu().numpy()
 
 
-@pytest.mark.parametrize("type_name", ["q4_k", "q5_k", "q2_k"])
+@pytest.mark.parametrize("type_name", ["q4_k", "q5_k", "q2_k", "q6_k", "iq4_xs"])
 @pytest.mark.parametrize("n,k,rows", [(64, 256, 1), (37, 768, 1), (100, 5120, 1), (16, 2048, 3), (9, 17408, 1), (33, 1000, 2)])
 def test_kquant_matvec_matches_oracle(mod, type_name, n, k, rows):
     rng = np.random.default_rng(1000 + n + k)
@@ -54,14 +54,14 @@ def test_kquant_matvec_matches_oracle(mod, type_name, n, k, rows):
         assert err < 2e-4
 
 
-@pytest.mark.parametrize("type_name", ["q4_k", "q5_k", "q2_k"])
+@pytest.mark.parametrize("type_name", ["q4_k", "q5_k", "q2_k", "q6_k", "iq4_xs"])
 def test_kquant_matvec_random_bytes(mod, type_name):
     """Uniformly random block bytes reach every scale/min/high-bit code, not only what the encoder emits."""
     rng = np.random.default_rng(77)
     n, bpr = 48, 5
     bb = O.BLOCK_BYTES[type_name]
     blocks = rng.integers(0, 256, size=(n, bpr, bb), dtype=np.uint8)
-    for off in ([0, 2] if type_name != "q2_k" else [80, 82]):
+    for off in {"q2_k": [80, 82], "q6_k": [208], "iq4_xs": [0]}.get(type_name, [0, 2]):
         vals = rng.uniform(0.001, 0.05, size=(n, bpr)) * rng.choice([-1.0, 1.0], size=(n, bpr))
         blocks[..., off:off + 2] = vals.astype("<f2").view(np.uint8).reshape(n, bpr, 2)
     x_np = rng.standard_normal((1, bpr * 256)).astype(np.float32)
@@ -140,6 +140,8 @@ def test_argument_errors_match_reference_messages(mod):
         mod.gguf_quant_gemm_forward(x, blocks, 512, 4, grid)
     with pytest.raises(RuntimeError, match="unsupported GGUF quant type_id"):
         mod.gguf_quant_gemm_forward(x, blocks, 512, 11, grid)
+    with pytest.raises(RuntimeError, match="has no MI355X kernel"):
+        mod.gguf_quant_gemm_forward(x, torch.zeros(8, 2, 74, dtype=torch.uint8, device=dev), 512, 5, grid)
     with pytest.raises(RuntimeError, match="blocks do not cover row_elems"):
         mod.gguf_quant_gemm_forward(torch.randn(1, 1024, device=dev), blocks, 1024, 3, grid)
     with pytest.raises(RuntimeError, match="x must be float16, bfloat16, or float32"):

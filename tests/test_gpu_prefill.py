@@ -134,6 +134,22 @@ def test_prefill_other_formats_match_float_oracle(mod, type_name, t, n, k):
     assert O.rel_l2(y.cpu().numpy(), want) <= 1e-3, (type_name, t, n, k)
 
 
+@pytest.mark.parametrize("type_name", ["q6_k", "iq4_xs"])
+@pytest.mark.parametrize("t,n,k", [(16, 128, 256), (40, 96, 768), (130, 33, 1000)])
+def test_prefill_operator_serves_q6_k_and_iq4_xs(mod, type_name, t, n, k):
+    """No tile-kernel decoder for these two yet: the prefill operator runs the decode kernel once per activation row."""
+    rng = np.random.default_rng(t + n + k)
+    enc = C.quantize_q6_k if type_name == "q6_k" else C.quantize_iq4_xs
+    blocks = enc((rng.standard_normal((n, k)) * 0.02).astype(np.float32))
+    x = torch.from_numpy(rng.standard_normal((t, k)).astype(np.float32)).to(DEV).to(torch.bfloat16)
+    print(f"case {type_name} prefill t={t} n={n} k={k}", flush=True)
+    y = mod.gguf_quant_gemm_prefill_forward(x, torch.from_numpy(blocks).to(DEV), k, O.TYPE_IDS[type_name],
+                                            torch.empty(0, dtype=torch.int8, device=DEV), out_dtype=torch.float32)
+    torch.cuda.synchronize()
+    want = O.matmul_f(x.float().cpu().numpy(), O.dequant_rows(blocks, type_name, k))
+    assert O.rel_l2(y.cpu().numpy(), want) <= 2e-4, (type_name, t, n, k)
+
+
 # ---- FP8 activations x FP8 weights on the native FP8 matrix path -----------------------------------
 
 @pytest.mark.parametrize("t,n,k", [(1, 128, 128), (16, 130, 256), (77, 300, 1024), (200, 512, 5120)])

@@ -34,7 +34,7 @@ def test_iq1m_matches_reference_held_vector(golden_dir):
     np.testing.assert_array_equal(got, values.reshape(raw["n_blocks"], 256))
 
 
-@pytest.mark.parametrize("type_name", ["q8_0", "q4_k", "q5_k", "iq2_xxs"])
+@pytest.mark.parametrize("type_name", ["q8_0", "q4_k", "q5_k", "iq2_xxs", "q6_k", "iq4_xs"])
 def test_decoders_match_reference_decoder_vectors(golden_dir, type_name):
     raw, blocks, values = _load(golden_dir, f"{type_name}_reference_decode.json")
     blocks = blocks.reshape(raw["rows"], raw["blocks_per_row"], raw["block_bytes"])
@@ -211,6 +211,75 @@ def test_q2_k_closed_form_group_layout():
                     want[y] = np.float32(0.5 * (sc & 15) * ((q[16 * part + l] >> shift) & 3)) - np.float32(0.25 * (sc >> 4))
                     y += 1
     np.testing.assert_array_equal(w, want)
+
+
+def test_q6_k_scalar_restatement_of_the_ggml_layout():
+    """ggml's dequantize_row_q6_K, weight by weight: two halves of 128; for l < 32 the four weights l, l + 32, l + 64,
+    l + 96 of a half take the low / high nibbles of ql[l], ql[l + 32] and the four bit pairs of qh[l]; scale index
+    8 half + l // 16 + 2 j."""
+    rng = np.random.default_rng(11)
+    b = rng.integers(0, 256, size=(1, 210), dtype=np.uint8)
+    b[0, 208:210] = _f16b(-0.0625)
+    ql, qh, sc = b[0, 0:128], b[0, 128:192], b[0, 192:208].view(np.int8)
+    want = np.empty(256, dtype=np.float32)
+    for half in range(2):
+        for l in range(32):
+            h = int(qh[32 * half + l])
+            qs = (int(ql[64 * half + l]) & 15, int(ql[64 * half + 32 + l]) & 15, int(ql[64 * half + l]) >> 4, int(ql[64 * half + 32 + l]) >> 4)
+            for j in range(4):
+                q = (qs[j] | (((h >> (2 * j)) & 3) << 4)) - 32
+                want[128 * half + 32 * j + l] = np.float32(-0.0625) * np.float32(int(sc[8 * half + l // 16 + 2 * j])) * np.float32(q)
+    np.testing.assert_array_equal(O.dequant_q6_k(b)[0], want)
+
+
+@pytest.mark.parametrize("live", range(16))
+def test_q6_k_one_live_scale(live):
+    """All codes 33 (q - 32 = 1), one scale byte non-zero: exactly the 16 weights of that group read d * scale."""
+    b = np.zeros((1, 210), dtype=np.uint8)
+    b[0, 0:128] = 0x11                      # low four bits 1 everywhere
+    b[0, 128:192] = 0xAA                    # high two bits 2 everywhere: q = 33
+    b[0, 192 + live] = np.int8(-7).view(np.uint8)
+    b[0, 208:210] = _f16b(0.5)
+    want = np.zeros(256, dtype=np.float32)
+    want[16 * live:16 * live + 16] = 0.5 * -7 * 1
+    np.testing.assert_array_equal(O.dequant_q6_k(b)[0], want)
+
+
+@pytest.mark.parametrize("live", range(8))
+def test_iq4_xs_one_live_group(live):
+    """Stored scale 32 (zero after the offset) everywhere except one group with high bits 3 and low bits 5
+    (53 - 32 = 21); low nibbles 0 (-127), high nibbles 15 (113)."""
+    b = np.zeros((1, 136), dtype=np.uint8)
+    b[0, 0:2] = _f16b(0.125)
+    sh = 0
+    for g in range(8):
+        hi2 = 3 if g == live else 2         # stored 0b10_0000 = 32 elsewhere
+        sh |= hi2 << (2 * g)
+    b[0, 2] = sh & 0xFF
+    b[0, 3] = sh >> 8
+    b[0, 4 + live // 2] = 5 << (4 if live & 1 else 0)
+    b[0, 8:136] = 0xF0
+    want = np.zeros(256, dtype=np.float32)
+    want[32 * live:32 * live + 16] = 0.125 * 21 * -127
+    want[32 * live + 16:32 * live + 32] = 0.125 * 21 * 113
+    got = O.dequant_iq4_xs(b)[0]
+    np.testing.assert_array_equal(got, want)
+
+
+def test_iq4_xs_code_table_and_nibble_order():
+    """Group 0 with scale 33 - 32 = 1 and d = 1: byte i of the group holds code i in the low and 15 - i in the high nibble."""
+    b = np.zeros((1, 136), dtype=np.uint8)
+    b[0, 0:2] = _f16b(1.0)
+    b[0, 2] = 0b10                          # high bits of group 0 = 2 -> stored 32 + low
+    b[0, 4] = 1                             # low bits of group 0 = 1 -> stored 33
+    for g in range(1, 8):
+        b[0, 2 + (2 * g) // 8] |= 2 << ((2 * g) % 8)      # other groups: stored 32 -> scale 0
+    b[0, 8:24] = np.arange(16, dtype=np.uint8) | ((15 - np.arange(16, dtype=np.uint8)) << 4)
+    kv = [-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113]
+    got = O.dequant_iq4_xs(b)[0]
+    np.testing.assert_array_equal(got[0:16], np.asarray(kv, dtype=np.float32))
+    np.testing.assert_array_equal(got[16:32], np.asarray(kv[::-1], dtype=np.float32))
+    assert not got[32:].any()
 
 
 def test_iq2_xxs_single_entry_signs_and_scale():
