@@ -72,7 +72,7 @@ def test_dequant_matches_golden_vectors(mod, golden_dir, name):
 def test_embedding_operator(mod):
     rng = np.random.default_rng(8)
     w = (rng.standard_normal((50, 512)) * 0.02).astype(np.float32)
-    for type_name, enc in (("q4_k", C.quantize_q4_k), ("q5_k", C.quantize_q5_k)):
+    for type_name, enc in (("q4_k", C.quantize_q4_k), ("q5_k", C.quantize_q5_k), ("q6_k", C.quantize_q6_k), ("iq4_xs", C.quantize_iq4_xs)):
         blocks = enc(w)
         ids = torch.tensor([[3, 49, 0], [7, 7, 21]], device=DEV)
         grid = torch.empty(0, dtype=torch.int8, device=DEV)
@@ -81,7 +81,7 @@ def test_embedding_operator(mod):
         want = torch.from_numpy(O.dequant_rows(blocks, type_name)[ids.cpu().numpy()]).to(torch.bfloat16)
         assert torch.equal(y.cpu(), want)
     with pytest.raises(RuntimeError, match="token_ids must be int64"):
-        mod.gguf_quant_embedding_forward(ids.int(), torch.from_numpy(blocks).to(DEV), 512, 4, grid)
+        mod.gguf_quant_embedding_forward(ids.int(), torch.from_numpy(blocks).to(DEV), 512, O.TYPE_IDS[type_name], grid)
 
 
 def test_q8_0_ops_surface(mod):

@@ -179,6 +179,13 @@ def test_linear_modules(mod):
     assert torch.equal(y0, y1)
     emb = QuantizedGGUFEmbedding(t)
     assert emb.dim == 512 and tuple(emb(torch.tensor([1, 2, 3], device=DEV, dtype=torch.int32)).shape) == (3, 512)
+    # the two table-free types the reference's linear wrapper also serves (it passes an empty grid)
+    for name, enc in (("q6_k", C.quantize_q6_k), ("iq4_xs", C.quantize_iq4_xs)):
+        bl = enc(w)
+        lin2 = QuantizedGGUFLinear(QuantizedGGUFTensor.from_blocks(torch.from_numpy(bl).to(DEV), name, 512, source_name=name))
+        x = torch.randn(3, 512, device=DEV, dtype=torch.float16)
+        want = O.matmul_f(x.float().cpu().numpy(), O.dequant_rows(bl, name))
+        assert np.abs(lin2(x).float().cpu().numpy() - want).max() < 2e-2
     q8 = Q8_0GGUFLinear(torch.from_numpy(C.pack_q8_0(w)).to(DEV), 512, source_name="q8")
     x = torch.randn(2, 512, device=DEV, dtype=torch.float16)
     want = O.matmul_f(x.float().cpu().numpy(), O.dequant_rows(C.pack_q8_0(w), "q8_0"))
