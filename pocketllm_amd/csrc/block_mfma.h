@@ -146,10 +146,10 @@ struct IQ2XXSm {
 // IQ1_M: 56 B = qs(32) qh(16) scales(8); w = dl (c - 1 + delta) with c in {0, 1, 2} from the
 // codebook (index: qs byte plus the low three bits of its qh nibble), dl = d (2 s3 + 1) per 16
 // weights, delta = -+1/8 per 8 weights (bit 3 of the nibble).  Lane (n, s) holds entries 8 s .. 8 s + 7
-// = four 16-weight groups.  With integer codes 8 c +- 1 = 8 (c + delta),
-//     sum w x = d sum over 16-groups j of (2 s3_j + 1) [ dot(8 c +- 1, x)_j / 8 - sum16(x)_j ].
+// = four 16-weight groups.  With signed integer codes 8 (c - 1) +- 1 = 8 (c - 1 + delta) in {-9, -7, -1, 1, 7, 9},
+//     sum w x = d / 8 sum over 16-groups j of (2 s3_j + 1) dot(code, x)_j.
 // A rows: m = 16-group of the block, one MFMA set per activation term; MFMA t, slice s carries group
-// 4 s + t, so C[4 s .. 4 s + 3][n] = the lane's own four groups.  sum16 comes from the image.
+// 4 s + t, so C[4 s .. 4 s + 3][n] = the lane's own four groups.
 // LDS table: 4096 x 8 code bytes, index = qs byte | nibble << 8 (the delta bit selects the half).
 // ------------------------------------------------------------------------------------------------
 struct alignas(16) Iq1DeltaCodes { uint64_t v[4096]; };
@@ -159,7 +159,7 @@ constexpr Iq1DeltaCodes make_iq1_delta_codes() {
         const uint32_t p = PLLM_IQ1_GRID_PACKED[i & 2047];      // element e in bits [2e, 2e+1], value + 1
         uint64_t v = 0;
         for (int e = 0; e < 8; ++e) {
-            const int code = 8 * static_cast<int>((p >> (2 * e)) & 3u) + ((i & 2048) ? -1 : 1);
+            const int code = 8 * (static_cast<int>((p >> (2 * e)) & 3u) - 1) + ((i & 2048) ? -1 : 1);
             v |= static_cast<uint64_t>(static_cast<uint8_t>(code)) << (8 * e);
         }
         t.v[i] = v;
@@ -195,14 +195,13 @@ struct IQ1Mm {
         }
     }
     // activation side of a block index (see IQ2XXSm::Held): the high-term A operands, the groups'
-    // scales (already over 8) and the 16-value sums; the low-term operands are read when needed
-    struct Held { uint4 a[4]; float x0, x1; float4 s16; };
+    // scales (already over 8); the low-term operands are read when needed
+    struct Held { uint4 a[4]; float x0, x1; };
     static __device__ __forceinline__ void hold(Held& h, int s, int b, const unsigned char* smem, const AMap<kSlots>& am, const StagedX& sx) {
 #pragma unroll
         for (int t = 0; t < 4; ++t) h.a[t] = *reinterpret_cast<const uint4*>(smem + am.off[t] + b * am.step[t]);
         const float4 g2 = *reinterpret_cast<const float4*>(sx.gs + b * 8 + 2 * s);   // {xs0 / 254, sum0, xs1 / 254, sum1}
         h.x0 = 0.125f * g2.x; h.x1 = 0.125f * g2.z;
-        h.s16 = *reinterpret_cast<const float4*>(sx.sum16 + b * 16 + 4 * s);
     }
     // lookups and MFMAs of one block: ch / cl = the lane's four 16-weight groups against the high / low term
     static __device__ __forceinline__ void group_dots(const Regs& r, int b, const uint4 (&ah)[4], const unsigned char* smem, const AMap<kSlots>& am,
@@ -220,23 +219,23 @@ struct IQ1Mm {
             cl = __builtin_amdgcn_mfma_i32_16x16x64_i8(as_v4i(al.x, al.y, al.z, al.w), bw, cl, 0, 0, 0);
         }
     }
-    // scales and sums: x8 = the four groups' activation scales / (254 * 8), s16 = their exact activation sums
-    static __device__ __forceinline__ float finish(const Regs& r, int s, const v4i& ch, const v4i& cl, const float4& x8, const float4& s16) {
+    // scales: x8 = the four groups' activation scales / (254 * 8)
+    static __device__ __forceinline__ float finish(const Regs& r, int s, const v4i& ch, const v4i& cl, const float4& x8) {
         const uint32_t s01 = r.sc.x, s23 = r.sc.y;
         const uint32_t dbits = ((s01 >> 12) & 0xfu) | ((s01 >> 24) & 0xf0u) | ((s23 >> 4) & 0xf00u) | ((s23 >> 16) & 0xf000u);
         // the lane's four 16-weight scales are the low 12 bits of scale word s
         const uint32_t word = ((s & 2) ? s23 : s01) >> (16 * (s & 1));
         const float ls0 = static_cast<float>(2 * (word & 7u) + 1), ls1 = static_cast<float>(2 * ((word >> 3) & 7u) + 1);
         const float ls2 = static_cast<float>(2 * ((word >> 6) & 7u) + 1), ls3 = static_cast<float>(2 * ((word >> 9) & 7u) + 1);
-        const float v = ls0 * (x8.x * static_cast<float>(__mul24(ch.x, 254) + cl.x) - s16.x) + ls1 * (x8.y * static_cast<float>(__mul24(ch.y, 254) + cl.y) - s16.y) +
-                        ls2 * (x8.z * static_cast<float>(__mul24(ch.z, 254) + cl.z) - s16.z) + ls3 * (x8.w * static_cast<float>(__mul24(ch.w, 254) + cl.w) - s16.w);
+        const float v = ls0 * x8.x * static_cast<float>(__mul24(ch.x, 254) + cl.x) + ls1 * x8.y * static_cast<float>(__mul24(ch.y, 254) + cl.y) +
+                        ls2 * x8.z * static_cast<float>(__mul24(ch.z, 254) + cl.z) + ls3 * x8.w * static_cast<float>(__mul24(ch.w, 254) + cl.w);
         return f16_bits_to_float(dbits) * v;
     }
     static __device__ __forceinline__ float block_held(const Regs& r, int s, int b, const Held& h, const unsigned char* smem,
                                                        const AMap<kSlots>& am, const unsigned char* tables) {
         v4i ch, cl;
         group_dots(r, b, h.a, smem, am, tables, ch, cl);
-        return finish(r, s, ch, cl, make_float4(h.x0, h.x0, h.x1, h.x1), h.s16);
+        return finish(r, s, ch, cl, make_float4(h.x0, h.x0, h.x1, h.x1));
     }
     static __device__ __forceinline__ float block(const Regs& r, int s, int b, const unsigned char* smem, const AMap<kSlots>& am,
                                                   const StagedX& sx, const unsigned char* tables) {

@@ -157,7 +157,6 @@ __global__ __launch_bounds__(64 * kW2Waves) void moe_single_w2_kernel(
         AMap<FMT::kSlots> am;
         FMT::a_map(am, col, ks, kpad, zero_off - r * image_bytes);
         const float* xs16 = reinterpret_cast<const float*>(img + 2 * kpad);
-        const float* sum16 = xs16 + kpad / 16;
         const unsigned char* tile = smem + tile_off + r * tile_stride;
         for (int b = wave & 1; b < bpr; b += 2) {
             FMT::Regs regs;
@@ -168,8 +167,7 @@ __global__ __launch_bounds__(64 * kW2Waves) void moe_single_w2_kernel(
             v4i ch, cl;
             FMT::group_dots(regs, b, ah, img, am, tables, ch, cl);
             const float4 xs = *reinterpret_cast<const float4*>(xs16 + b * 16 + 4 * ks);
-            const float4 s16 = *reinterpret_cast<const float4*>(sum16 + b * 16 + 4 * ks);
-            acc += FMT::finish(regs, ks, ch, cl, make_float4(0.125f * xs.x, 0.125f * xs.y, 0.125f * xs.z, 0.125f * xs.w), s16);
+            acc += FMT::finish(regs, ks, ch, cl, make_float4(0.125f * xs.x, 0.125f * xs.y, 0.125f * xs.z, 0.125f * xs.w));
         }
     }
     acc += __shfl_xor(acc, 16, 64);
