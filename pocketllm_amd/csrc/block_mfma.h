@@ -59,9 +59,26 @@ __device__ __forceinline__ v4i as_v4i(uint32_t x, uint32_t y, uint32_t z, uint32
 }
 
 // LDS offsets of a lane's A operands: slot i of block b is read at off[i] + b * step[i]; slots whose
-// A row is not the lane's point at 16 zero bytes with step 0.
+// A row is not the lane's point at 16 zero bytes with step 0 (on[i] false).
 template <int SLOTS>
-struct AMap { int off[SLOTS]; int step[SLOTS]; };
+struct AMap { int off[SLOTS]; int step[SLOTS]; bool on[SLOTS]; };
+
+// A operands in registers.  Three quarters or more of a wave's lanes hold zero rows of A: cleared
+// once, they are never read again, and only the lanes a slot belongs to touch LDS (a 16-byte read of
+// every lane costs the LDS as much as a whole kilobyte of data, zeros included).
+template <int SLOTS>
+struct AOps { uint4 a[SLOTS]; };
+template <int SLOTS>
+__device__ __forceinline__ void clear_a(AOps<SLOTS>& ops) {
+#pragma unroll
+    for (int i = 0; i < SLOTS; ++i) ops.a[i] = make_uint4(0u, 0u, 0u, 0u);
+}
+template <int SLOTS>
+__device__ __forceinline__ void load_a(AOps<SLOTS>& ops, const AMap<SLOTS>& am, const unsigned char* base, int b) {
+#pragma unroll
+    for (int i = 0; i < SLOTS; ++i)
+        if (am.on[i]) ops.a[i] = *reinterpret_cast<const uint4*>(base + am.off[i] + b * 256);
+}
 
 // ------------------------------------------------------------------------------------------------
 // IQ2_XXS: 66 B = d(2) + 8 sub-blocks of 8 B (four grid ids, then a u32: four 7-bit sign indices and
@@ -103,6 +120,7 @@ struct IQ2XXSm {
             const bool active = (col >> 1) == g;
             am.off[t] = active ? ((col & 1) ? kpad : 0) + 32 * g + 16 * (t & 1) : zero_off;
             am.step[t] = active ? 256 : 0;
+            am.on[t] = active;
         }
     }
     // what a block index contributes from the activation side: the lane's A operands and its two
@@ -133,6 +151,37 @@ struct IQ2XXSm {
         const float v1 = static_cast<float>(__mul24(c.z - cm.z, 254) + (c.w - cm.w));   // group 2 s + 1
         const float ls0 = static_cast<float>(2 * (r.q.y >> 28) + 1), ls1 = static_cast<float>(2 * (r.q.w >> 28) + 1);
         return 0.125f * f16_bits_to_float(r.d) * (ls0 * h.xs0 * v0 + ls1 * h.xs1 * v1);
+    }
+    // A block decoded once for several activation vectors: finished signed codes (B operands of the
+    // four MFMAs) and the two groups' scales times d / 8.
+    struct Decoded { v4i b[4]; float ls0, ls1; };
+    static __device__ __forceinline__ void decode(const Regs& r, int, const unsigned char* tables, Decoded& o) {
+        const uint2* grid = reinterpret_cast<const uint2*>(tables);
+        const uint2* sign = grid + 256;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const uint32_t ids = (t < 2) ? r.q.x : r.q.z, aux = (t < 2) ? r.q.y : r.q.w;
+            const int e = 2 * (t & 1);
+            const uint2 g0 = grid[(ids >> (8 * e)) & 0xffu], m0 = sign[(aux >> (7 * e)) & 127u];
+            const uint2 g1 = grid[(ids >> (8 * e + 8)) & 0xffu], m1 = sign[(aux >> (7 * e + 7)) & 127u];
+            // negate the masked bytes: (g ^ 0xff) + 1 never carries out of a byte because g >= 8
+            o.b[t] = as_v4i((g0.x ^ m0.x) + (m0.x & 0x01010101u), (g0.y ^ m0.y) + (m0.y & 0x01010101u),
+                            (g1.x ^ m1.x) + (m1.x & 0x01010101u), (g1.y ^ m1.y) + (m1.y & 0x01010101u));
+        }
+        const float d8 = 0.125f * f16_bits_to_float(r.d);
+        o.ls0 = d8 * static_cast<float>(2 * (r.q.y >> 28) + 1);
+        o.ls1 = d8 * static_cast<float>(2 * (r.q.w >> 28) + 1);
+    }
+    // the decoded block against one activation image (img = its first byte in LDS, offsets of am relative to it)
+    static __device__ __forceinline__ float route_block(const Decoded& o, int s, int b, const unsigned char* img, const AMap<kSlots>& am, int kpad,
+                                                        AOps<kSlots>& ops) {
+        load_a(ops, am, img, b);
+        v4i c = {0, 0, 0, 0};
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            c = __builtin_amdgcn_mfma_i32_16x16x64_i8(as_v4i(ops.a[t].x, ops.a[t].y, ops.a[t].z, ops.a[t].w), o.b[t], c, 0, 0, 0);
+        const float4 g2 = *reinterpret_cast<const float4*>(img + 2 * kpad + (b * 8 + 2 * s) * 8);   // {xs0 / 254, sum0, xs1 / 254, sum1}
+        return o.ls0 * g2.x * static_cast<float>(__mul24(c.x, 254) + c.y) + o.ls1 * g2.z * static_cast<float>(__mul24(c.z, 254) + c.w);
     }
     static __device__ __forceinline__ float block(const Regs& r, int s, int b, const unsigned char* smem, const AMap<kSlots>& am,
                                                   const StagedX& sx, const unsigned char* tables) {
@@ -192,6 +241,7 @@ struct IQ1Mm {
             am.off[t] = active ? 16 * col : zero_off;
             am.off[4 + t] = active ? kpad + 16 * col : zero_off;
             am.step[t] = am.step[4 + t] = active ? 256 : 0;
+            am.on[t] = am.on[4 + t] = active;
         }
     }
     // activation side of a block index (see IQ2XXSm::Held): the high-term A operands, the groups'
@@ -237,6 +287,48 @@ struct IQ1Mm {
         group_dots(r, b, h.a, smem, am, tables, ch, cl);
         return finish(r, s, ch, cl, make_float4(h.x0, h.x0, h.x1, h.x1));
     }
+    // A block decoded once for several activation vectors: the codes of the lane's four 16-weight
+    // groups and their scales times d / 8.
+    struct Decoded { v4i b[4]; float l0, l1, l2, l3; };
+    static __device__ __forceinline__ void decode(const Regs& r, int s, const unsigned char* tables, Decoded& o) {
+        const uint2* table = reinterpret_cast<const uint2*>(tables);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const uint32_t qw = (t < 2) ? r.qs.x : r.qs.y;
+            const uint2 w0 = table[((qw >> (16 * (t & 1))) & 0xffu) | (((r.qh >> (8 * t)) & 15u) << 8)];
+            const uint2 w1 = table[((qw >> (16 * (t & 1) + 8)) & 0xffu) | (((r.qh >> (8 * t + 4)) & 15u) << 8)];
+            o.b[t] = as_v4i(w0.x, w0.y, w1.x, w1.y);
+        }
+        const uint32_t s01 = r.sc.x, s23 = r.sc.y;
+        const uint32_t dbits = ((s01 >> 12) & 0xfu) | ((s01 >> 24) & 0xf0u) | ((s23 >> 4) & 0xf00u) | ((s23 >> 16) & 0xf000u);
+        const uint32_t word = ((s & 2) ? s23 : s01) >> (16 * (s & 1));
+        const float d8 = 0.125f * f16_bits_to_float(dbits);
+        o.l0 = d8 * static_cast<float>(2 * (word & 7u) + 1); o.l1 = d8 * static_cast<float>(2 * ((word >> 3) & 7u) + 1);
+        o.l2 = d8 * static_cast<float>(2 * ((word >> 6) & 7u) + 1); o.l3 = d8 * static_cast<float>(2 * ((word >> 9) & 7u) + 1);
+    }
+    static __device__ __forceinline__ float route_dots(const Decoded& o, int b, const unsigned char* img, const AMap<kSlots>& am, const float4& xs,
+                                                       AOps<kSlots>& ops) {
+        load_a(ops, am, img, b);
+        v4i ch = {0, 0, 0, 0}, cl = {0, 0, 0, 0};
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            ch = __builtin_amdgcn_mfma_i32_16x16x64_i8(as_v4i(ops.a[t].x, ops.a[t].y, ops.a[t].z, ops.a[t].w), o.b[t], ch, 0, 0, 0);
+            cl = __builtin_amdgcn_mfma_i32_16x16x64_i8(as_v4i(ops.a[4 + t].x, ops.a[4 + t].y, ops.a[4 + t].z, ops.a[4 + t].w), o.b[t], cl, 0, 0, 0);
+        }
+        return o.l0 * xs.x * static_cast<float>(__mul24(ch.x, 254) + cl.x) + o.l1 * xs.y * static_cast<float>(__mul24(ch.y, 254) + cl.y) +
+               o.l2 * xs.z * static_cast<float>(__mul24(ch.z, 254) + cl.z) + o.l3 * xs.w * static_cast<float>(__mul24(ch.w, 254) + cl.w);
+    }
+    // against an activation image with one scale per 32 values (pllm_device.h) ...
+    static __device__ __forceinline__ float route_block(const Decoded& o, int s, int b, const unsigned char* img, const AMap<kSlots>& am, int kpad,
+                                                        AOps<kSlots>& ops) {
+        const float4 g2 = *reinterpret_cast<const float4*>(img + 2 * kpad + (b * 8 + 2 * s) * 8);   // {xs0 / 254, sum0, xs1 / 254, sum1}
+        return route_dots(o, b, img, am, make_float4(g2.x, g2.x, g2.z, g2.z), ops);
+    }
+    // ... and against one with a scale per 16 values (float xs16[kpad / 16] after the two int8 planes)
+    static __device__ __forceinline__ float route_block16(const Decoded& o, int s, int b, const unsigned char* img, const AMap<kSlots>& am, int kpad,
+                                                          AOps<kSlots>& ops) {
+        return route_dots(o, b, img, am, *reinterpret_cast<const float4*>(img + 2 * kpad + (b * 16 + 4 * s) * 4), ops);
+    }
     static __device__ __forceinline__ float block(const Regs& r, int s, int b, const unsigned char* smem, const AMap<kSlots>& am,
                                                   const StagedX& sx, const unsigned char* tables) {
         Held h;
@@ -279,6 +371,7 @@ struct Q6Km {
             am.off[t] = active ? 16 * col : zero_off;
             am.off[4 + t] = active ? kpad + 16 * col : zero_off;
             am.step[t] = am.step[4 + t] = active ? 256 : 0;
+            am.on[t] = am.on[4 + t] = active;
         }
     }
     static __device__ __forceinline__ uint32_t code4(uint32_t ql, uint32_t qh, int t) {
@@ -337,6 +430,7 @@ struct IQ4XSm {
             const bool active = (col >> 1) == g;
             am.off[t] = active ? ((col & 1) ? kpad : 0) + 32 * g + 16 * (t & 1) : zero_off;
             am.step[t] = active ? 256 : 0;
+            am.on[t] = active;
         }
     }
     // four codes (one per byte, 0..15) -> four table values

@@ -17,6 +17,10 @@
 namespace pllm {
 // from this many tokens on, an expert's routes are multiplied as one tile matmul on the matrix cores
 constexpr int kMoeGemmMinTokens = 16;
+// up to this many routes per expert on average the grouped matrix-core kernels (cost per route: MFMAs and a short
+// epilogue after one decode per expert; measured ~180 us + 0.5 us per route at 256 experts of 1536 x 3072) run ahead
+// of the tile matmuls (cost per expert: the fp16 decode of every weight, ~1450 us for the same experts)
+constexpr int kMoeGroupedMaxRoutesPerExpert = 8;
 
 namespace {
 
@@ -496,6 +500,25 @@ int pllm_gguf_moe_forward(const void* x, int x_dtype, int64_t tokens, int64_t di
     if (!workspace || workspace_bytes < pllm_gguf_moe_workspace_bytes(tokens, routes, dim, inter)) return PLLM_ERR_WORKSPACE;
 
     const int bpr_x = static_cast<int>((dim + 255) / 256), bpr_h = static_cast<int>((inter + 255) / 256);
+    if (seg_starts && tokens > 1 && routes <= kMoeGroupedMaxRoutesPerExpert * n_experts &&
+        moe_grouped_mfma_supports(w13_type, w2_type, static_cast<int>(dim), static_cast<int>(inter), w1, w3, w2)) {
+        // a few routes per expert: every expert's weights are decoded once on the matrix-core path and all its routes pass
+        // through; same workspace layout as the v_dot4 forms below
+        const size_t xs = act_image_256_bytes(bpr_x), hs = act_image_256_bytes(bpr_h);
+        unsigned char* x_img = static_cast<unsigned char*>(workspace);
+        unsigned char* h_img = x_img + xs * tokens;
+        float* part = reinterpret_cast<float*>(h_img + hs * routes);
+        const int R = static_cast<int>(routes), E = static_cast<int>(n_experts), I = static_cast<int>(inter), D = static_cast<int>(dim);
+        int st = act_image_256(x, x_dtype, static_cast<int>(tokens), D, bpr_x, x_img, s);
+        if (st != PLLM_OK) return st;
+        st = moe_grouped_w13_mfma(x_img, xs, D, route_tokens, seg_starts, route_weights, w1, w3, w13_type, I, swiglu_limit, h_img, hs, E, s);
+        if (st != PLLM_OK) return st;
+        st = moe_grouped_w2_mfma(h_img, hs, I, seg_starts, w2, part, D, E, s);
+        if (st != PLLM_OK) return st;
+        dim3 rg(static_cast<unsigned>(tokens), static_cast<unsigned>((dim + 255) / 256));
+        hipLaunchKernelGGL(moe_reduce_kernel, rg, dim3(256), 0, s, part, route_tokens, y, R, D);
+        return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+    }
     if (seg_starts && tokens >= kMoeGemmMinTokens) {
         // tile path: gather the routes' activation rows as fp16, gate and up as two batches of tile
         // matmuls (one group per expert), SwiGLU into fp16 hidden rows, down as a third batch, then

@@ -45,6 +45,15 @@ int moe_single_w13_mfma(const void* x, int x_dtype, int dim, const int64_t* rout
 int moe_single_w2_mfma(const unsigned char* h_image, size_t h_stride, int inter, const int64_t* route_experts, int routes, const uint8_t* w2,
                        float* y, int dim, hipStream_t stream);
 
+// Routed experts of several tokens on the matrix cores (same file): routes grouped by expert (seg), x images from
+// act_image_256, hidden images with one scale per 16 values, per-route outputs into partial [R, dim].
+bool moe_grouped_mfma_supports(int w13_type, int w2_type, int dim, int inter, const uint8_t* w1, const uint8_t* w3, const uint8_t* w2);
+int moe_grouped_w13_mfma(const unsigned char* x_image, size_t x_stride, int dim, const int64_t* route_tokens, const int32_t* seg,
+                         const float* route_weights, const uint8_t* w1, const uint8_t* w3, int w13_type, int inter, float limit,
+                         unsigned char* h_image, size_t h_stride, int n_experts, hipStream_t stream);
+int moe_grouped_w2_mfma(const unsigned char* h_image, size_t h_stride, int inter, const int32_t* seg, const uint8_t* w2, float* partial, int dim,
+                        int n_experts, hipStream_t stream);
+
 // compute units of the current device (read once per process; 256 when no device answers)
 int compute_units();
 

@@ -194,6 +194,36 @@ def test_linear_modules(mod):
         Q8_0GGUFLinear(torch.zeros(4, 2, 33, dtype=torch.uint8, device=DEV), 64)
 
 
+@pytest.mark.parametrize("t13,e,d,inter,topk,t,limit", [("iq2_xxs", 6, 3072, 1536, 2, 24, 0.0), ("iq2_xxs", 5, 768, 1072, 3, 14, 0.5),
+                                                        ("iq1_m", 7, 1024, 512, 2, 28, 0.0), ("iq2_xxs", 3, 256, 256, 3, 2, 0.0)])
+def test_grouped_experts_matrix_core_path(mod, t13, e, d, inter, topk, t, limit):
+    """Up to 8 routes per expert on average with an IQ1_M down projection: every expert's blocks are decoded once and its
+    routes pass through in batches (several batches for the busier experts, an intermediate size that is not a multiple of 256)."""
+    rng = np.random.default_rng(13 + t)
+    w1 = _expert_blocks(rng, t13, e, inter, d)
+    w3 = _expert_blocks(rng, t13, e, inter, d)
+    w2 = _expert_blocks(rng, "iq1_m", e, d, inter)
+    idx, wts = _route(rng, t, e + 2, topk)                 # local window 1..e
+    x = torch.from_numpy(rng.standard_normal((t, d)).astype(np.float32)).to(DEV).to(torch.bfloat16)
+    _, toks, rws, seg = mod.moe_group_routes(torch.from_numpy(idx).to(DEV), torch.from_numpy(wts).to(DEV), 1, e)
+    _, o_toks, o_rws, o_seg = O.group_routes(idx, wts, 1, e)
+    grids = (codebooks.get_iq2xxs_signed_grid_tensor().to(DEV), codebooks.get_iq1_grid_tensor().to(DEV))
+    if t13 == "iq1_m":
+        grids = grids[1]
+    dw1, dw3, dw2 = (torch.from_numpy(a).to(DEV) for a in (w1, w3, w2))
+    tid = O.TYPE_IDS
+    print(f"case matrix-core grouped {t13} e={e} d={d} inter={inter} t={t} routes={len(o_toks)}", flush=True)
+    assert 1 < t and len(o_toks) <= 8 * e, "shape no longer selects the grouped matrix-core kernels"
+    assert t == 2 or np.diff(o_seg).max() > 4, "no expert with more than one batch of routes"
+    y = mod.gguf_moe_prefill_grouped_forward(x, toks, rws, seg, dw1, dw3, dw2, d, tid[t13], d, tid[t13], inter, tid["iq1_m"], grids, limit)
+    torch.cuda.synchronize()
+    route_experts = np.repeat(np.arange(e), np.diff(o_seg))
+    want = O.moe_forward(x.float().cpu().numpy(), o_toks, o_rws, route_experts, w1, w3, w2, t13, t13, "iq1_m", limit)
+    assert O.rel_l2(y.cpu().numpy(), want) <= TOL
+    y2 = mod.gguf_moe_prefill_grouped_forward(x, toks, rws, seg, dw1, dw3, dw2, d, tid[t13], d, tid[t13], inter, tid["iq1_m"], grids, limit)
+    assert torch.equal(y, y2)
+
+
 @pytest.mark.parametrize("t13,t2,limit", [("iq2_xxs", "iq1_m", 0.0), ("iq2_xxs", "q2_k", 0.7), ("iq1_m", "iq1_m", 0.0)])
 def test_grouped_experts_tile_path(mod, t13, t2, limit):
     """Sixteen tokens or more: the routes of every expert go through the MFMA tile kernel as one batch of matmuls
