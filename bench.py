@@ -238,6 +238,12 @@ def prefill_cases(mod, dev, iters):
                     lambda s, x=x, blocks=blocks, tid=tid: mod.gguf_quant_gemm_prefill_forward(x, blocks, k, tid, empty))
             del blocks
     n = 17408
+    for name, tid in (("q6_k", 8), ("iq4_xs", 7)):             # random valid blocks: the work does not depend on the values
+        blocks = torch.from_numpy(C.random_blocks(rng, name, n, k // 256)).to(dev)
+        for t in (512, 2048):
+            x = torch.randn(t, k, device=dev, dtype=torch.bfloat16)
+            run(f"{name} prefill {n}x{k} T={t}", t, n, lambda s, x=x, blocks=blocks, tid=tid: mod.gguf_quant_gemm_prefill_forward(x, blocks, k, tid, empty))
+        del blocks
     codes, scale = C.quantize_fp8_block(rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02))
     codes = torch.from_numpy(codes).to(dev)
     scale = torch.from_numpy(scale).to(dev)

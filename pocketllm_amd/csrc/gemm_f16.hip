@@ -257,6 +257,72 @@ __device__ __forceinline__ half4 half4_of(uint32_t lo, uint32_t hi) {
     return __builtin_bit_cast(half4, make_uint2(lo, hi));
 }
 
+// Q6_K: 210 B = ql(128) qh(64) scales int8(16) d(2); weight 128 half + 32 j + l takes nibble j / 2 of ql[64 half + 32 (j % 2) + l], bit
+// pair j of qh[32 half + l] and scale 8 half + 2 j + l / 16; w = d * scale * (q - 32).  Here half = p / 2, j = 2 (p % 2) + e, l = 16 h + ...
+// Blocks are only 2-byte aligned.
+struct __attribute__((packed, aligned(2))) UnalignedWord { uint32_t v; };
+struct GQ6K {
+    static constexpr int kTableBytes = 0;
+    static __device__ __forceinline__ void stage_table(unsigned char*) {}
+    static constexpr int kBlockBytes = 210;
+    struct Regs { uint4 qa, qb, qh; uint32_t sc, d; };
+    static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, const float*, int, int p, int h) {
+        const int half = p >> 1;
+        r.qa = load16_a2(blk + 64 * half + 16 * h);
+        r.qb = load16_a2(blk + 64 * half + 32 + 16 * h);
+        r.qh = load16_a2(blk + 128 + 32 * half + 16 * h);
+        r.sc = reinterpret_cast<const UnalignedWord*>(blk + 192 + 8 * half + 4 * (p & 1))->v;   // scales 8 half + 4 (p % 2) + 0..3
+        r.d = *reinterpret_cast<const uint16_t*>(blk + 208);
+    }
+    static __device__ __forceinline__ uint32_t codes(uint32_t ql, uint32_t qh, int nib, int pair) {
+        return ((ql >> nib) & 0x0f0f0f0fu) | (((qh >> pair) & 0x03030303u) << 4);
+    }
+    static __device__ __forceinline__ void decode(const Regs& r, int p, int e, int h, const unsigned char*, Half16& o) {
+        const int nib = 4 * (p & 1), pair = 2 * (2 * (p & 1) + e);
+        const uint4 ql = e ? r.qb : r.qa;
+        const float scale = f16_bits_to_float(r.d) * static_cast<float>(static_cast<int8_t>(r.sc >> (8 * (2 * e + h))));
+        const float minus = 32.0f * scale;
+        o.a = affine4(codes(ql.x, r.qh.x, nib, pair), scale, minus);
+        o.b = affine4(codes(ql.y, r.qh.y, nib, pair), scale, minus);
+        o.c = affine4(codes(ql.z, r.qh.z, nib, pair), scale, minus);
+        o.d = affine4(codes(ql.w, r.qh.w, nib, pair), scale, minus);
+    }
+};
+
+// IQ4_XS: 136 B = d(2) scales_h(2) scales_l(4) qs(128); group g = 2 p + e of 32 weights: bytes qs[16 g, +16), low nibbles = its first
+// 16 weights (h = 0), high nibbles the others; w = d * (ls - 32) * kvalues[code].  The 16-entry table sits in four constants, biased
+// by 128 so that the codes stay unsigned bytes; three byte permutes pick four values.
+struct GIQ4XS {
+    static constexpr int kTableBytes = 0;
+    static __device__ __forceinline__ void stage_table(unsigned char*) {}
+    static constexpr int kBlockBytes = 136;
+    struct Regs { uint2 hdr; uint4 q0, q1; };
+    static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, const float*, int, int p, int) {
+        const uint2* w = reinterpret_cast<const uint2*>(blk);                 // blocks are 8-byte aligned
+        r.hdr = w[0];
+        r.q0 = make_uint4(w[1 + 4 * p].x, w[1 + 4 * p].y, w[2 + 4 * p].x, w[2 + 4 * p].y);
+        r.q1 = make_uint4(w[3 + 4 * p].x, w[3 + 4 * p].y, w[4 + 4 * p].x, w[4 + 4 * p].y);
+    }
+    static __device__ __forceinline__ uint32_t biased4(uint32_t codes) {     // kvalues[code] + 128, four at a time
+        const uint32_t low3 = codes & 0x07070707u;
+        const uint32_t lower = __builtin_amdgcn_perm(0x766A5D4Fu, 0x3F2D1801u, low3);   // 1 24 45 63 | 79 93 106 118
+        const uint32_t upper = __builtin_amdgcn_perm(0xF1D9C5B5u, 0xA6998D81u, low3);   // 129 141 153 166 | 181 197 217 241
+        return __builtin_amdgcn_perm(upper, lower, ((codes >> 1) & 0x04040404u) | 0x03020100u);
+    }
+    static __device__ __forceinline__ void decode(const Regs& r, int p, int e, int h, const unsigned char*, Half16& o) {
+        const uint4 q = e ? r.q1 : r.q0;
+        const int g = 2 * p + e, sft = 4 * h;
+        const uint32_t scales_h = r.hdr.x >> 16;
+        const int ls = static_cast<int>(((r.hdr.y >> (8 * p + 4 * e)) & 15u) | (((scales_h >> (2 * g)) & 3u) << 4)) - 32;
+        const float scale = f16_bits_to_float(r.hdr.x & 0xffffu) * static_cast<float>(ls);
+        const float minus = 128.0f * scale;
+        o.a = affine4(biased4((q.x >> sft) & 0x0f0f0f0fu), scale, minus);
+        o.b = affine4(biased4((q.y >> sft) & 0x0f0f0f0fu), scale, minus);
+        o.c = affine4(biased4((q.z >> sft) & 0x0f0f0f0fu), scale, minus);
+        o.d = affine4(biased4((q.w >> sft) & 0x0f0f0f0fu), scale, minus);
+    }
+};
+
 // IQ2_XXS: 66 B = d(2) + 8 sub-blocks of 8 B (four grid ids, then a u32: four 7-bit sign indices and a
 // 4-bit scale).  A pair is sub-blocks 2 p and 2 p + 1; the thread takes grid entries 2 h and 2 h + 1 of
 // its sub-block.  w = d (2 s + 1) / 8 * magnitude, negated where the sign pattern (seven bits plus
@@ -636,7 +702,7 @@ size_t align256(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
 
 bool gemm_f16_supports(int type_id) {
     return type_id == PLLM_TYPE_Q4_K || type_id == PLLM_TYPE_Q5_K || type_id == PLLM_TYPE_Q2_K || type_id == PLLM_TYPE_IQ2_XXS ||
-           type_id == PLLM_TYPE_IQ1_M;
+           type_id == PLLM_TYPE_IQ1_M || type_id == PLLM_TYPE_Q6_K || type_id == PLLM_TYPE_IQ4_XS;
 }
 
 size_t gemm_f16_workspace_bytes(int rows, int n, int bpr) {
@@ -682,6 +748,8 @@ int gemm_f16(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y,
         case PLLM_TYPE_Q2_K: return launch_gemm_mi<GQ2K>(p, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, nullptr, 0, nullptr, 0, 1, stream);
         case PLLM_TYPE_IQ2_XXS: return launch_gemm_mi<GIQ2XXS>(p, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, nullptr, 0, nullptr, 0, 1, stream);
         case PLLM_TYPE_IQ1_M: return launch_gemm_mi<GIQ1M>(p, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, nullptr, 0, nullptr, 0, 1, stream);
+        case PLLM_TYPE_Q6_K: return launch_gemm_mi<GQ6K>(p, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, nullptr, 0, nullptr, 0, 1, stream);
+        case PLLM_TYPE_IQ4_XS: return launch_gemm_mi<GIQ4XS>(p, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, nullptr, 0, nullptr, 0, 1, stream);
         default: return PLLM_ERR_UNSUPPORTED;
     }
 }

@@ -135,9 +135,9 @@ def test_prefill_other_formats_match_float_oracle(mod, type_name, t, n, k):
 
 
 @pytest.mark.parametrize("type_name", ["q6_k", "iq4_xs"])
-@pytest.mark.parametrize("t,n,k", [(16, 128, 256), (40, 96, 768), (130, 33, 1000)])
+@pytest.mark.parametrize("t,n,k", [(16, 128, 256), (40, 96, 768), (130, 33, 1000), (300, 520, 5120), (1100, 200, 512)])
 def test_prefill_operator_serves_q6_k_and_iq4_xs(mod, type_name, t, n, k):
-    """No tile-kernel decoder for these two yet: the prefill operator runs the decode kernel once per activation row."""
+    """Q6_K (2-byte aligned blocks, signed scales) and IQ4_XS (code table through byte permutes) in the tile kernel."""
     rng = np.random.default_rng(t + n + k)
     enc = C.quantize_q6_k if type_name == "q6_k" else C.quantize_iq4_xs
     blocks = enc((rng.standard_normal((n, k)) * 0.02).astype(np.float32))
@@ -147,7 +147,7 @@ def test_prefill_operator_serves_q6_k_and_iq4_xs(mod, type_name, t, n, k):
                                             torch.empty(0, dtype=torch.int8, device=DEV), out_dtype=torch.float32)
     torch.cuda.synchronize()
     want = O.matmul_f(x.float().cpu().numpy(), O.dequant_rows(blocks, type_name, k))
-    assert O.rel_l2(y.cpu().numpy(), want) <= 2e-4, (type_name, t, n, k)
+    assert O.rel_l2(y.cpu().numpy(), want) <= 1e-3, (type_name, t, n, k)
 
 
 # ---- FP8 activations x FP8 weights on the native FP8 matrix path -----------------------------------
