@@ -41,6 +41,8 @@ enum {
     PLLM_TYPE_IQ1_M = 2,   /* 56 B */
     PLLM_TYPE_Q4_K = 3,    /* 144 B */
     PLLM_TYPE_Q5_K = 4,    /* 176 B */
+    PLLM_TYPE_IQ2_XS = 5,  /* 74 B */
+    PLLM_TYPE_IQ3_XXS = 6, /* 98 B */
     PLLM_TYPE_IQ4_XS = 7,  /* 136 B */
     PLLM_TYPE_Q6_K = 8,    /* 210 B */
     PLLM_TYPE_Q8_0 = 100   /* 34 B / 32 weights; the reference gives Q8_0 no id, this one is the library's own */

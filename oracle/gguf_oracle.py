@@ -16,6 +16,9 @@ How each function is pinned (what a wrong sign / index / transposed operand woul
   dequant_q4_k,
   dequant_q5_k       hand-built blocks that isolate every field (scale index j<4 / j>=4, nibble
                      halves, qh bit planes) plus fixtures written by the reference's numpy reader.
+  dequant_iq2_xs,
+  dequant_iq3_xxs    fixtures written by the reference's numpy reader, hand-built blocks with one live
+                     entry (grid id, sign index and parity bit, both scale nibbles / the 4-bit scale).
   dequant_q6_k,
   dequant_iq4_xs     fixtures written by the reference's numpy reader, hand-built blocks with one
                      live field (every scale index, both nibble halves, every qh bit pair / high
@@ -38,10 +41,10 @@ import numpy as np
 _CODEBOOK_FILE = Path(__file__).resolve().parents[1] / "pocketllm_amd" / "csrc" / "ggml_codebooks.inc"
 
 # type_id map of the reference: src/loader/gguf/quant_types.py:3-13, src/csrc/cuda_kernel.cpp:401-412
-TYPE_IDS = {"iq2_xxs": 0, "q2_k": 1, "iq1_m": 2, "q4_k": 3, "q5_k": 4, "iq4_xs": 7, "q6_k": 8}
+TYPE_IDS = {"iq2_xxs": 0, "q2_k": 1, "iq1_m": 2, "q4_k": 3, "q5_k": 4, "iq2_xs": 5, "iq3_xxs": 6, "iq4_xs": 7, "q6_k": 8}
 TYPE_NAMES = {v: k for k, v in TYPE_IDS.items()}
-BLOCK_BYTES = {"q8_0": 34, "iq2_xxs": 66, "q2_k": 84, "iq1_m": 56, "q4_k": 144, "q5_k": 176, "iq4_xs": 136, "q6_k": 210}
-BLOCK_ELEMS = {"q8_0": 32, "iq2_xxs": 256, "q2_k": 256, "iq1_m": 256, "q4_k": 256, "q5_k": 256, "iq4_xs": 256, "q6_k": 256}
+BLOCK_BYTES = {"q8_0": 34, "iq2_xxs": 66, "q2_k": 84, "iq1_m": 56, "q4_k": 144, "q5_k": 176, "iq4_xs": 136, "q6_k": 210, "iq2_xs": 74, "iq3_xxs": 98}
+BLOCK_ELEMS = {"q8_0": 32, "iq2_xxs": 256, "q2_k": 256, "iq1_m": 256, "q4_k": 256, "q5_k": 256, "iq4_xs": 256, "q6_k": 256, "iq2_xs": 256, "iq3_xxs": 256}
 
 
 # --------------------------------------------------------------------------------------------
@@ -221,6 +224,74 @@ def dequant_iq1_m(blocks: np.ndarray) -> np.ndarray:
     return out.reshape(lead + (256,))
 
 
+@lru_cache(maxsize=1)
+def iq2xs_grid_u8() -> np.ndarray:
+    """(512, 8) uint8 magnitudes. Reference: tensor_reader.py:167-169 (parsed there from ggml-common.h)."""
+    return np.asarray(_parse_table("PLLM_IQ2XS_GRID"), dtype="<u8").view(np.uint8).reshape(512, 8).copy()
+
+
+@lru_cache(maxsize=1)
+def iq3xxs_grid_u8() -> np.ndarray:
+    """(256, 4) uint8 magnitudes. Reference: tensor_reader.py:172-174."""
+    return np.asarray(_parse_table("PLLM_IQ3XXS_GRID"), dtype="<u4").view(np.uint8).reshape(256, 4).copy()
+
+
+def _sign_table() -> np.ndarray:
+    """(128, 8) float32 of +-1: bit j of the 7-bit index, bit 7 = parity of the others (tensor_reader.py:183-187)."""
+    idx = np.arange(128)
+    parity = np.zeros(128, dtype=np.int64)
+    for b in range(7):
+        parity ^= (idx >> b) & 1
+    full = idx | (parity << 7)
+    return np.where((full[:, None] >> np.arange(8)) & 1, np.float32(-1.0), np.float32(1.0)).astype(np.float32)
+
+
+def dequant_iq2_xs(blocks: np.ndarray) -> np.ndarray:
+    """IQ2_XS: d(f16) qs u16[32] scales(8).  Entry e (8 weights): grid id = low 9 bits, sign index = high 7 bits of qs[e];
+    sub-block s = e // 4 (32 weights) has two 4-bit scales, the low nibble for its first 16 weights, the high nibble for the
+    others; w = 0.25 * d * (ls + 0.5) * grid * sign.  Reference: tensor_reader.py:663-690."""
+    assert blocks.dtype == np.uint8 and blocks.shape[-1] == 74
+    lead = blocks.shape[:-1]
+    b = blocks.reshape(-1, 74)
+    d = _f16(b[:, 0:2])
+    qs = b[:, 2:66].astype(np.uint16)
+    q = qs[:, 0::2] | (qs[:, 1::2] << 8)                                    # [n, 32]
+    scales = b[:, 66:74]
+    grid = iq2xs_grid_u8().astype(np.float32)
+    signs = _sign_table()
+    out = np.empty((b.shape[0], 256), dtype=np.float32)
+    for e in range(32):
+        sub, part = divmod(e, 4)
+        ls = ((scales[:, sub] & 0x0F) if part < 2 else (scales[:, sub] >> 4)).astype(np.float32)
+        values = grid[q[:, e] & 0x1FF] * signs[q[:, e] >> 9]
+        out[:, 8 * e:8 * e + 8] = np.float32(0.25) * d[:, None] * (ls + np.float32(0.5))[:, None] * values
+    return out.reshape(lead + (256,))
+
+
+def dequant_iq3_xxs(blocks: np.ndarray) -> np.ndarray:
+    """IQ3_XXS: d(f16) grid ids(64) aux u32[8].  Sub-block s (32 weights): ids qs[8 s + k] give four weights each from the
+    256-entry grid; aux_s holds four 7-bit sign indices (one per 8 weights) and a 4-bit scale; w = 0.5 * d * (ls + 0.5) * grid * sign.
+    Reference: tensor_reader.py:700-735."""
+    assert blocks.dtype == np.uint8 and blocks.shape[-1] == 98
+    lead = blocks.shape[:-1]
+    b = blocks.reshape(-1, 98)
+    d = _f16(b[:, 0:2])
+    ids = b[:, 2:66]
+    aux = b[:, 66:98].astype(np.uint32)
+    aux = aux[:, 0::4] | (aux[:, 1::4] << 8) | (aux[:, 2::4] << 16) | (aux[:, 3::4] << 24)      # [n, 8]
+    grid = iq3xxs_grid_u8().astype(np.float32)
+    signs = _sign_table()
+    out = np.empty((b.shape[0], 256), dtype=np.float32)
+    for sub in range(8):
+        ls = (aux[:, sub] >> 28).astype(np.float32)
+        for part in range(8):
+            sg = signs[(aux[:, sub] >> (7 * (part // 2))) & 127][:, 4 * (part % 2):4 * (part % 2) + 4]
+            values = grid[ids[:, 8 * sub + part]] * sg
+            start = 32 * sub + 4 * part
+            out[:, start:start + 4] = np.float32(0.5) * d[:, None] * (ls + np.float32(0.5))[:, None] * values
+    return out.reshape(lead + (256,))
+
+
 def dequant_q6_k(blocks: np.ndarray) -> np.ndarray:
     """Q6_K: ql(128) qh(64) scales int8(16) d(f16); w = d * scales[i // 16] * (q - 32), q = 4 low bits from ql and 2
     high bits from qh.  Reference: tensor_reader.py:868-908."""
@@ -274,7 +345,7 @@ def dequant_iq4_xs(blocks: np.ndarray) -> np.ndarray:
 _DECODERS = {
     "q8_0": dequant_q8_0, "q4_k": dequant_q4_k, "q5_k": dequant_q5_k,
     "q2_k": dequant_q2_k, "iq2_xxs": dequant_iq2_xxs, "iq1_m": dequant_iq1_m,
-    "q6_k": dequant_q6_k, "iq4_xs": dequant_iq4_xs,
+    "q6_k": dequant_q6_k, "iq4_xs": dequant_iq4_xs, "iq2_xs": dequant_iq2_xs, "iq3_xxs": dequant_iq3_xxs,
 }
 
 

@@ -190,8 +190,8 @@ def quantize_iq4_xs(weight: np.ndarray) -> np.ndarray:
 
 
 def random_blocks(rng: np.random.Generator, type_name: str, *lead: int, d_range=(0.001, 0.02)) -> np.ndarray:
-    """Every byte random except the fp16 scale field (finite, drawn from d_range): q6_k or iq4_xs."""
-    nbytes, off = {"q6_k": (210, 208), "iq4_xs": (136, 0)}[type_name]
+    """Every byte random except the fp16 scale field (finite, drawn from d_range): q6_k, iq4_xs, iq2_xs or iq3_xxs."""
+    nbytes, off = {"q6_k": (210, 208), "iq4_xs": (136, 0), "iq2_xs": (74, 0), "iq3_xxs": (98, 0)}[type_name]
     blocks = rng.integers(0, 256, size=tuple(lead) + (nbytes,), dtype=np.uint8)
     d = rng.uniform(d_range[0], d_range[1], size=tuple(lead)).astype(np.float32)
     blocks[..., off:off + 2] = _f16_bytes(d)

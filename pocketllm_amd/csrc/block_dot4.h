@@ -13,10 +13,12 @@
 namespace pllm {
 
 #define PLLM_TABLE_U64(name, n) alignas(16) static __device__ constexpr uint64_t name[n] = {
+#define PLLM_TABLE_U32(name, n) alignas(16) static __device__ constexpr uint32_t name[n] = {
 #define PLLM_TABLE_U16(name, n) alignas(16) static __device__ constexpr uint16_t name[n] = {
 #define PLLM_TABLE_END };
 #include "ggml_codebooks.inc"
 #undef PLLM_TABLE_U64
+#undef PLLM_TABLE_U32
 #undef PLLM_TABLE_U16
 #undef PLLM_TABLE_END
 

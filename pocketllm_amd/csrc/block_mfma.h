@@ -1,4 +1,4 @@
-// Per-format pieces of the matrix-core kernels over IQ2_XXS, IQ1_M, IQ4_XS and Q6_K super-blocks, and the
+// Per-format pieces of the matrix-core kernels over IQ2_XXS, IQ2_XS, IQ3_XXS, IQ1_M, IQ4_XS and Q6_K super-blocks, and the
 // direct-to-LDS copy helpers they share.
 //
 // Lane map: lane (n, s) = (lane % 16, lane / 16) of a wave works on output row n of a 16-row tile and
@@ -459,6 +459,124 @@ struct IQ4XSm {
         const int ls0 = static_cast<int>((sl & 15u) | (((scales_h >> (4 * s)) & 3u) << 4)) - 32;
         const int ls1 = static_cast<int>((sl >> 4) | (((scales_h >> (4 * s + 2)) & 3u) << 4)) - 32;
         return f16_bits_to_float(r.hdr.x & 0xffffu) * (static_cast<float>(ls0) * g2.x * v0 + static_cast<float>(ls1) * g2.z * v1);
+    }
+};
+
+// ------------------------------------------------------------------------------------------------
+// IQ2_XS: 74 B = d(2) qs u16[32] scales(8).  Entry e (8 weights): grid id = low 9 bits of qs[e], sign
+// index = high 7 bits; two 4-bit scales per 32 weights (low nibble: first 16); w = d (2 ls + 1) / 8 *
+// grid * sign.  Lane (n, s) holds qs[8 s, 8 s + 8) = four 16-weight groups and scale bytes 2 s, 2 s + 1.
+// A rows as for IQ1_M: m = 16-group, one MFMA set per activation term, MFMA t, slice s carries group
+// 4 s + t.  LDS tables: 512 x 8 magnitude bytes, then the 128 x 8 sign masks.  Blocks are 2-byte aligned.
+// ------------------------------------------------------------------------------------------------
+struct IQ2XSm {
+    static constexpr int kBlockBytes = 74;
+    static constexpr int kTableBytes = 4096 + 1024;
+    static constexpr int kSlots = 8;                           // [term][t]
+    static constexpr bool kStreamed = false;
+    struct Regs { uint4 q; uint32_t sc, d; };
+    static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, int s) {
+        r.q = load16_a2(blk + 2 + 16 * s);
+        r.sc = *reinterpret_cast<const uint16_t*>(blk + 66 + 2 * s);
+        r.d = *reinterpret_cast<const uint16_t*>(blk);
+    }
+    static __device__ __forceinline__ void stage_tables(unsigned char* lds) {
+        copy_to_lds(lds, reinterpret_cast<const unsigned char*>(PLLM_IQ2XS_GRID), 4096);
+        copy_to_lds(lds + 4096, reinterpret_cast<const unsigned char*>(PLLM_IQ2XXS_SIGN_MASKS.v), 1024);
+    }
+    static __device__ __forceinline__ void a_map(AMap<kSlots>& am, int col, int ks, int kpad, int zero_off) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const bool active = col == 4 * ks + t;
+            am.off[t] = active ? 16 * col : zero_off;
+            am.off[4 + t] = active ? kpad + 16 * col : zero_off;
+            am.step[t] = am.step[4 + t] = active ? 256 : 0;
+            am.on[t] = am.on[4 + t] = active;
+        }
+    }
+    static __device__ __forceinline__ uint2 signed8(const uint2* grid, const uint2* sign, uint32_t q16) {
+        const uint2 g = grid[q16 & 511u], m = sign[q16 >> 9];
+        // negate the masked bytes: (g ^ 0xff) + 1 never carries out of a byte because g >= 8
+        return make_uint2((g.x ^ m.x) + (m.x & 0x01010101u), (g.y ^ m.y) + (m.y & 0x01010101u));
+    }
+    static __device__ __forceinline__ float block(const Regs& r, int s, int b, const unsigned char* smem, const AMap<kSlots>& am,
+                                                  const StagedX& sx, const unsigned char* tables) {
+        const uint2* grid = reinterpret_cast<const uint2*>(tables);
+        const uint2* sign = grid + 512;
+        v4i ch = {0, 0, 0, 0}, cl = {0, 0, 0, 0};
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {                                          // 16-weight group t of the lane = entries 2 t, 2 t + 1
+            const uint32_t pair = t == 0 ? r.q.x : t == 1 ? r.q.y : t == 2 ? r.q.z : r.q.w;
+            const uint2 w0 = signed8(grid, sign, pair & 0xffffu), w1 = signed8(grid, sign, pair >> 16);
+            const v4i bw = as_v4i(w0.x, w0.y, w1.x, w1.y);
+            const uint4 ah = *reinterpret_cast<const uint4*>(smem + am.off[t] + b * am.step[t]);
+            const uint4 al = *reinterpret_cast<const uint4*>(smem + am.off[4 + t] + b * am.step[4 + t]);
+            ch = __builtin_amdgcn_mfma_i32_16x16x64_i8(as_v4i(ah.x, ah.y, ah.z, ah.w), bw, ch, 0, 0, 0);
+            cl = __builtin_amdgcn_mfma_i32_16x16x64_i8(as_v4i(al.x, al.y, al.z, al.w), bw, cl, 0, 0, 0);
+        }
+        const float4 g2 = *reinterpret_cast<const float4*>(sx.gs + b * 8 + 2 * s);   // {xs0 / 254, sum0, xs1 / 254, sum1}
+        const float l0 = static_cast<float>(2 * (r.sc & 15u) + 1), l1 = static_cast<float>(2 * ((r.sc >> 4) & 15u) + 1);
+        const float l2 = static_cast<float>(2 * ((r.sc >> 8) & 15u) + 1), l3 = static_cast<float>(2 * (r.sc >> 12) + 1);
+        const float v = l0 * g2.x * static_cast<float>(__mul24(ch.x, 254) + cl.x) + l1 * g2.x * static_cast<float>(__mul24(ch.y, 254) + cl.y) +
+                        l2 * g2.z * static_cast<float>(__mul24(ch.z, 254) + cl.z) + l3 * g2.z * static_cast<float>(__mul24(ch.w, 254) + cl.w);
+        return 0.125f * f16_bits_to_float(r.d) * v;
+    }
+};
+
+// ------------------------------------------------------------------------------------------------
+// IQ3_XXS: 98 B = d(2) grid ids(64) aux u32[8].  An id gives four weights from a 256-entry grid; aux of a
+// sub-block (32 weights) holds four 7-bit sign indices (one per 8 weights) and a 4-bit scale;
+// w = d (2 ls + 1) / 4 * grid * sign.  Lane (n, s) holds ids [16 s, 16 s + 16) = groups 2 s, 2 s + 1 and their
+// two aux words.  A rows as for IQ2_XXS.  LDS tables: 256 x 4 magnitude bytes, then the 128 x 8 sign
+// masks.  Blocks are 2-byte aligned.
+// ------------------------------------------------------------------------------------------------
+struct IQ3XXSm {
+    static constexpr int kBlockBytes = 98;
+    static constexpr int kTableBytes = 1024 + 1024;
+    static constexpr int kSlots = 4;
+    static constexpr bool kStreamed = false;
+    struct Regs { uint4 ids; uint32_t aux0, aux1, d; };
+    static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, int s) {
+        r.ids = load16_a2(blk + 2 + 16 * s);
+        r.aux0 = reinterpret_cast<const Unaligned4*>(blk + 66 + 8 * s)->v;
+        r.aux1 = reinterpret_cast<const Unaligned4*>(blk + 70 + 8 * s)->v;
+        r.d = *reinterpret_cast<const uint16_t*>(blk);
+    }
+    static __device__ __forceinline__ void stage_tables(unsigned char* lds) {
+        copy_to_lds(lds, reinterpret_cast<const unsigned char*>(PLLM_IQ3XXS_GRID), 1024);
+        copy_to_lds(lds + 1024, reinterpret_cast<const unsigned char*>(PLLM_IQ2XXS_SIGN_MASKS.v), 1024);
+    }
+    static __device__ __forceinline__ void a_map(AMap<kSlots>& am, int col, int ks, int kpad, int zero_off) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int g = 2 * ks + (t >> 1);
+            const bool active = (col >> 1) == g;
+            am.off[t] = active ? ((col & 1) ? kpad : 0) + 32 * g + 16 * (t & 1) : zero_off;
+            am.step[t] = active ? 256 : 0;
+            am.on[t] = active;
+        }
+    }
+    static __device__ __forceinline__ uint32_t signed4(uint32_t g, uint32_t m) { return (g ^ m) + (m & 0x01010101u); }   // g >= 4: no carry
+    static __device__ __forceinline__ float block(const Regs& r, int s, int b, const unsigned char* smem, const AMap<kSlots>& am,
+                                                  const StagedX& sx, const unsigned char* tables) {
+        const uint32_t* grid = reinterpret_cast<const uint32_t*>(tables);
+        const uint2* sign = reinterpret_cast<const uint2*>(tables + 1024);
+        v4i c = {0, 0, 0, 0};
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {                                          // half t % 2 of group 2 s + t / 2: four ids, two sign indices
+            const uint32_t ids = t == 0 ? r.ids.x : t == 1 ? r.ids.y : t == 2 ? r.ids.z : r.ids.w;
+            const uint32_t aux = (t < 2) ? r.aux0 : r.aux1;
+            const uint2 m0 = sign[(aux >> (14 * (t & 1))) & 127u], m1 = sign[(aux >> (14 * (t & 1) + 7)) & 127u];
+            const v4i bw = as_v4i(signed4(grid[ids & 0xffu], m0.x), signed4(grid[(ids >> 8) & 0xffu], m0.y),
+                                  signed4(grid[(ids >> 16) & 0xffu], m1.x), signed4(grid[ids >> 24], m1.y));
+            const uint4 a = *reinterpret_cast<const uint4*>(smem + am.off[t] + b * am.step[t]);
+            c = __builtin_amdgcn_mfma_i32_16x16x64_i8(as_v4i(a.x, a.y, a.z, a.w), bw, c, 0, 0, 0);
+        }
+        const float v0 = static_cast<float>(__mul24(c.x, 254) + c.y);         // group 2 s: 254 * high term + low term
+        const float v1 = static_cast<float>(__mul24(c.z, 254) + c.w);         // group 2 s + 1
+        const float4 g2 = *reinterpret_cast<const float4*>(sx.gs + b * 8 + 2 * s);   // {xs0 / 254, sum0, xs1 / 254, sum1}
+        const float ls0 = static_cast<float>(2 * (r.aux0 >> 28) + 1), ls1 = static_cast<float>(2 * (r.aux1 >> 28) + 1);
+        return 0.25f * f16_bits_to_float(r.d) * (ls0 * g2.x * v0 + ls1 * g2.z * v1);
     }
 };
 

@@ -45,6 +45,8 @@ int pllm_gguf_block_bytes(int type_id) {
         case PLLM_TYPE_IQ1_M: return 56;
         case PLLM_TYPE_Q4_K: return 144;
         case PLLM_TYPE_Q5_K: return 176;
+        case PLLM_TYPE_IQ2_XS: return 74;
+        case PLLM_TYPE_IQ3_XXS: return 98;
         case PLLM_TYPE_IQ4_XS: return 136;
         case PLLM_TYPE_Q6_K: return 210;
         default: return 0;
@@ -76,6 +78,8 @@ static int superblock_matvec(const unsigned char* image, size_t stride, const ui
             return pllm::dot4_matvec_from_image(image, stride, blocks, type_id, y, y_dtype, rows, n, bpr, s);
         case PLLM_TYPE_IQ2_XXS:
         case PLLM_TYPE_IQ1_M:
+        case PLLM_TYPE_IQ2_XS:
+        case PLLM_TYPE_IQ3_XXS:
         case PLLM_TYPE_IQ4_XS:
         case PLLM_TYPE_Q6_K:
             return pllm::iq_mfma_matvec_from_image(image, stride, blocks, type_id, y, y_dtype, rows, n, bpr, s);

@@ -73,6 +73,31 @@ __device__ float dequant_iq1_m(const uint8_t* b, int e) {
     return dl * (g + ((h & 8u) ? -0.125f : 0.125f));
 }
 
+// sign of weight j under a 7-bit sign index (bit 7 = parity of the other seven)
+__device__ __forceinline__ float sign_of(uint32_t s7, int j) {
+    const uint32_t s8 = s7 | ((__popc(s7) & 1u) << 7);
+    return ((s8 >> j) & 1u) ? -1.0f : 1.0f;
+}
+
+// IQ2_XS: d, qs u16[32] (9-bit grid id, 7-bit sign index per 8 weights), scales(8): two 4-bit scales per 32 weights
+__device__ float dequant_iq2_xs(const uint8_t* b, int e) {
+    const int ent = e >> 3, j = e & 7;
+    const uint32_t q = static_cast<uint32_t>(b[2 + 2 * ent]) | (static_cast<uint32_t>(b[3 + 2 * ent]) << 8);
+    const uint32_t ls = (b[66 + (ent >> 2)] >> (4 * ((ent >> 1) & 1))) & 15u;
+    const float mag = static_cast<float>((PLLM_IQ2XS_GRID[q & 511u] >> (8 * j)) & 0xffull);
+    return 0.25f * f16_at(b) * (static_cast<float>(ls) + 0.5f) * (mag * sign_of(q >> 9, j));
+}
+
+// IQ3_XXS: d, grid ids(64: four weights each), aux u32[8] (four 7-bit sign indices per 32 weights, 4-bit scale)
+__device__ float dequant_iq3_xxs(const uint8_t* b, int e) {
+    const int sub = e >> 5, part = (e >> 2) & 7, j = e & 3;
+    const uint8_t* a = b + 66 + 4 * sub;
+    const uint32_t aux = static_cast<uint32_t>(a[0]) | (static_cast<uint32_t>(a[1]) << 8) | (static_cast<uint32_t>(a[2]) << 16) | (static_cast<uint32_t>(a[3]) << 24);
+    const float mag = static_cast<float>((PLLM_IQ3XXS_GRID[b[2 + 8 * sub + part]] >> (8 * j)) & 0xffu);
+    const float sgn = sign_of((aux >> (7 * (part >> 1))) & 127u, 4 * (part & 1) + j);
+    return 0.5f * f16_at(b) * (static_cast<float>(aux >> 28) + 0.5f) * (mag * sgn);
+}
+
 // Q6_K: ql(128) qh(64) scales int8(16) d; weight e = 128 half + 32 j + l takes nibble j / 2 of ql[64 half + 32 (j % 2) + l],
 // bit pair j of qh[32 half + l] and scale e / 16
 __device__ float dequant_q6_k(const uint8_t* b, int e) {
@@ -117,6 +142,8 @@ __global__ __launch_bounds__(256) void dequant_rows_kernel(
                 case PLLM_TYPE_Q2_K: v = dequant_q2_k(b, e); break;
                 case PLLM_TYPE_IQ2_XXS: v = dequant_iq2_xxs(b, e); break;
                 case PLLM_TYPE_Q6_K: v = dequant_q6_k(b, e); break;
+                case PLLM_TYPE_IQ2_XS: v = dequant_iq2_xs(b, e); break;
+                case PLLM_TYPE_IQ3_XXS: v = dequant_iq3_xxs(b, e); break;
                 case PLLM_TYPE_IQ4_XS: v = dequant_iq4_xs(b, e); break;
                 default: v = dequant_iq1_m(b, e); break;
             }

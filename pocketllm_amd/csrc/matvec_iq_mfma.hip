@@ -1,4 +1,4 @@
-// Decode matvec over raw IQ2_XXS / IQ1_M / IQ4_XS / Q6_K super-blocks with the integer dots on the matrix cores.
+// Decode matvec over raw IQ2_XXS / IQ2_XS / IQ3_XXS / IQ1_M / IQ4_XS / Q6_K super-blocks with the integer dots on the matrix cores.
 //
 // A wave owns a tile of 16 consecutive output rows (or, for short matrices, a share of the tile's
 // super-blocks; the shares meet in a small LDS reduction); the activation image (two int8 terms per
@@ -291,6 +291,8 @@ int iq_mfma_matvec_from_image(const unsigned char* image, size_t stride, const u
     switch (type_id) {
         case PLLM_TYPE_IQ2_XXS: return launch_fmt<IQ2XXSm>(image, stride, w, y, y_dtype, rows, n, bpr, stream);
         case PLLM_TYPE_IQ1_M: return launch_fmt<IQ1Mm>(image, stride, w, y, y_dtype, rows, n, bpr, stream);
+        case PLLM_TYPE_IQ2_XS: return launch_fmt<IQ2XSm>(image, stride, w, y, y_dtype, rows, n, bpr, stream);
+        case PLLM_TYPE_IQ3_XXS: return launch_fmt<IQ3XXSm>(image, stride, w, y, y_dtype, rows, n, bpr, stream);
         case PLLM_TYPE_IQ4_XS: return launch_fmt<IQ4XSm>(image, stride, w, y, y_dtype, rows, n, bpr, stream);
         case PLLM_TYPE_Q6_K: return launch_fmt<Q6Km>(image, stride, w, y, y_dtype, rows, n, bpr, stream);
         default: return PLLM_ERR_UNSUPPORTED;

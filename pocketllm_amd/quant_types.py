@@ -22,7 +22,7 @@ GGUF_DENSE_TYPE_NAMES = {v: k for k, v in GGUF_DENSE_TYPE_IDS.items()}
 GGUF_BLOCK_BYTES = {0: 66, 1: 84, 2: 56, 3: 144, 4: 176, 5: 74, 6: 98, 7: 136, 8: 210}
 
 # type ids this library has kernels for; the others are known to the id map but raise
-IMPLEMENTED_TYPE_IDS = (0, 1, 2, 3, 4, 7, 8)
+IMPLEMENTED_TYPE_IDS = (0, 1, 2, 3, 4, 5, 6, 7, 8)
 
 Q8_0_BLOCK_BYTES = 34
 Q8_0_BLOCK_ELEMS = 32

@@ -54,14 +54,14 @@ def test_kquant_matvec_matches_oracle(mod, type_name, n, k, rows):
         assert err < 2e-4
 
 
-@pytest.mark.parametrize("type_name", ["q4_k", "q5_k", "q2_k", "q6_k", "iq4_xs"])
+@pytest.mark.parametrize("type_name", ["q4_k", "q5_k", "q2_k", "q6_k", "iq4_xs", "iq2_xs", "iq3_xxs"])
 def test_kquant_matvec_random_bytes(mod, type_name):
     """Uniformly random block bytes reach every scale/min/high-bit code, not only what the encoder emits."""
     rng = np.random.default_rng(77)
     n, bpr = 48, 5
     bb = O.BLOCK_BYTES[type_name]
     blocks = rng.integers(0, 256, size=(n, bpr, bb), dtype=np.uint8)
-    for off in {"q2_k": [80, 82], "q6_k": [208], "iq4_xs": [0]}.get(type_name, [0, 2]):
+    for off in {"q2_k": [80, 82], "q6_k": [208], "iq4_xs": [0], "iq2_xs": [0], "iq3_xxs": [0]}.get(type_name, [0, 2]):
         vals = rng.uniform(0.001, 0.05, size=(n, bpr)) * rng.choice([-1.0, 1.0], size=(n, bpr))
         blocks[..., off:off + 2] = vals.astype("<f2").view(np.uint8).reshape(n, bpr, 2)
     x_np = rng.standard_normal((1, bpr * 256)).astype(np.float32)
@@ -140,8 +140,6 @@ def test_argument_errors_match_reference_messages(mod):
         mod.gguf_quant_gemm_forward(x, blocks, 512, 4, grid)
     with pytest.raises(RuntimeError, match="unsupported GGUF quant type_id"):
         mod.gguf_quant_gemm_forward(x, blocks, 512, 11, grid)
-    with pytest.raises(RuntimeError, match="has no MI355X kernel"):
-        mod.gguf_quant_gemm_forward(x, torch.zeros(8, 2, 74, dtype=torch.uint8, device=dev), 512, 5, grid)
     with pytest.raises(RuntimeError, match="blocks do not cover row_elems"):
         mod.gguf_quant_gemm_forward(torch.randn(1, 1024, device=dev), blocks, 1024, 3, grid)
     with pytest.raises(RuntimeError, match="x must be float16, bfloat16, or float32"):
@@ -199,6 +197,22 @@ def test_iq_matvec_many_rows(mod, type_name, n, k):
     want = O.matmul_f(x_np, O.dequant_rows(blocks[pick], type_name, k))
     assert O.rel_l2(y.cpu().numpy()[:, pick], want) <= 2e-4
     assert torch.isfinite(y).all()
+
+
+@pytest.mark.parametrize("type_name", ["iq2_xs", "iq3_xxs"])
+@pytest.mark.parametrize("n,k,rows", [(16, 256, 1), (50, 768, 2), (1536, 3072, 1), (7, 5120, 1), (64, 14336, 1)])
+def test_iq2xs_iq3xxs_matvec_matches_oracle(mod, type_name, n, k, rows):
+    rng = np.random.default_rng(900 + n + k)
+    blocks = C.random_blocks(rng, type_name, n, (k + 255) // 256)
+    x_np = rng.standard_normal((rows, k)).astype(np.float32)
+    dev = torch.device("cuda:0")
+    print(f"case {type_name} n={n} k={k} rows={rows}", flush=True)
+    y = mod.gguf_quant_gemm_forward(torch.from_numpy(x_np).to(dev).to(torch.bfloat16), torch.from_numpy(blocks).to(dev), k, O.TYPE_IDS[type_name],
+                                    torch.empty(0, dtype=torch.int8, device=dev), out_dtype=torch.float32)
+    torch.cuda.synchronize()
+    x_used = torch.from_numpy(x_np).to(torch.bfloat16).float().numpy()
+    want = O.matmul_f(x_used, O.dequant_rows(blocks, type_name, k))
+    assert O.rel_l2(y.cpu().numpy(), want) <= 2e-4, (type_name, n, k, rows)
 
 
 def test_iq_fully_random_bytes(mod):

@@ -34,7 +34,7 @@ def test_iq1m_matches_reference_held_vector(golden_dir):
     np.testing.assert_array_equal(got, values.reshape(raw["n_blocks"], 256))
 
 
-@pytest.mark.parametrize("type_name", ["q8_0", "q4_k", "q5_k", "iq2_xxs", "q6_k", "iq4_xs"])
+@pytest.mark.parametrize("type_name", ["q8_0", "q4_k", "q5_k", "iq2_xxs", "q6_k", "iq4_xs", "iq2_xs", "iq3_xxs"])
 def test_decoders_match_reference_decoder_vectors(golden_dir, type_name):
     raw, blocks, values = _load(golden_dir, f"{type_name}_reference_decode.json")
     blocks = blocks.reshape(raw["rows"], raw["blocks_per_row"], raw["block_bytes"])
@@ -280,6 +280,79 @@ def test_iq4_xs_code_table_and_nibble_order():
     np.testing.assert_array_equal(got[0:16], np.asarray(kv, dtype=np.float32))
     np.testing.assert_array_equal(got[16:32], np.asarray(kv[::-1], dtype=np.float32))
     assert not got[32:].any()
+
+
+def _ggml_grid(name, count):
+    """The named table of ggml-common.h, read as text from the mounted checkout (skipped where it is absent)."""
+    header = REFERENCE / "src" / "csrc" / "llama_mmq" / "ggml-common.h"
+    if not header.exists():
+        pytest.skip("reference checkout not mounted")
+    m = re.search(r"GGML_TABLE_BEGIN\([^,]+,\s*%s,\s*%d\)(.*?)GGML_TABLE_END\(\)" % (name, count), header.read_text(), flags=re.S)
+    return [int(v, 16) for v in re.findall(r"0x[0-9a-fA-F]+", m.group(1))]
+
+
+def test_iq2xs_and_iq3xxs_grids_match_ggml_header_text():
+    g2 = np.asarray(_ggml_grid("iq2xs_grid", 512), dtype="<u8").view(np.uint8).reshape(512, 8)
+    np.testing.assert_array_equal(O.iq2xs_grid_u8(), g2)
+    g3 = np.asarray(_ggml_grid("iq3xxs_grid", 256), dtype="<u4").view(np.uint8).reshape(256, 4)
+    np.testing.assert_array_equal(O.iq3xxs_grid_u8(), g3)
+
+
+@pytest.mark.parametrize("entry", [0, 5, 13, 31])
+def test_iq2_xs_single_entry(entry):
+    """One entry live: grid id 300 with sign index 0b0000101 (bits 0 and 2 set, parity even -> weight 7 positive), scale nibble 9
+    in the half of the scale byte that covers this entry, every other scale nibble 0 (which still means ls + 0.5 = 0.5)."""
+    b = np.zeros((1, 74), dtype=np.uint8)
+    b[0, 0:2] = _f16b(2.0)
+    q = 300 | (0b0000101 << 9)
+    b[0, 2 + 2 * entry] = q & 0xFF
+    b[0, 3 + 2 * entry] = q >> 8
+    sub, part = divmod(entry, 4)
+    b[0, 66 + sub] = 9 << (4 if part >= 2 else 0)
+    got = O.dequant_iq2_xs(b)[0]
+    g = O.iq2xs_grid_u8()
+    sign = np.array([-1, 1, -1, 1, 1, 1, 1, 1], dtype=np.float32)
+    np.testing.assert_array_equal(got[8 * entry:8 * entry + 8], 0.25 * 2.0 * 9.5 * g[300].astype(np.float32) * sign)
+    other = np.delete(np.arange(32), entry)
+    # all other entries: grid id 0, no signs, scale 0.5 (their nibble is 0) unless they share the live nibble
+    for e in other[:6]:
+        shared = (e // 4 == sub) and ((e % 4 >= 2) == (part >= 2))
+        np.testing.assert_array_equal(got[8 * e:8 * e + 8], 0.25 * 2.0 * (9.5 if shared else 0.5) * g[0].astype(np.float32))
+
+
+def test_iq2_xs_parity_bit():
+    """Sign index with an odd number of bits set flips weight 7 as well."""
+    b = np.zeros((1, 74), dtype=np.uint8)
+    b[0, 0:2] = _f16b(1.0)
+    q = 17 | (0b0000111 << 9)
+    b[0, 2], b[0, 3] = q & 0xFF, q >> 8
+    got = O.dequant_iq2_xs(b)[0, :8]
+    g = O.iq2xs_grid_u8()[17].astype(np.float32)
+    np.testing.assert_array_equal(got, 0.25 * 0.5 * g * np.array([-1, -1, -1, 1, 1, 1, 1, -1], dtype=np.float32))
+
+
+@pytest.mark.parametrize("sub", [0, 3, 7])
+def test_iq3_xxs_single_sub_block(sub):
+    """One sub-block live: ids 8 s .. 8 s + 7 = 10, 20, ..., 80; sign index of pair k = 1 << k (one weight negative, parity odd ->
+    weight 7 of the pair negative too); scale 6."""
+    b = np.zeros((1, 98), dtype=np.uint8)
+    b[0, 0:2] = _f16b(0.5)
+    ids = np.arange(1, 9, dtype=np.uint8) * 10
+    b[0, 2 + 8 * sub:10 + 8 * sub] = ids
+    aux = (6 << 28) | sum((1 << k) << (7 * k) for k in range(4))
+    b[0, 66 + 4 * sub:70 + 4 * sub] = np.frombuffer(np.uint32(aux).tobytes(), dtype=np.uint8)
+    got = O.dequant_iq3_xxs(b)[0]
+    g = O.iq3xxs_grid_u8().astype(np.float32)
+    want = np.zeros(32, dtype=np.float32)
+    for part in range(8):
+        k = part // 2
+        sign8 = np.ones(8, dtype=np.float32)
+        sign8[k] = -1
+        sign8[7] = -1
+        want[4 * part:4 * part + 4] = 0.5 * 0.5 * 6.5 * g[ids[part]] * sign8[4 * (part % 2):4 * (part % 2) + 4]
+    np.testing.assert_array_equal(got[32 * sub:32 * sub + 32], want)
+    rest = np.delete(got.reshape(8, 32), sub, axis=0)
+    np.testing.assert_array_equal(rest, np.tile(0.5 * 0.5 * 0.5 * np.tile(g[0], 8), (7, 1)))
 
 
 def test_iq2_xxs_single_entry_signs_and_scale():
