@@ -362,6 +362,86 @@ struct GIQ2XXS {
     }
 };
 
+// IQ2_XS: 74 B = d(2) qs u16[32] scales(8).  Entry (8 weights) = 9-bit grid id + 7-bit sign index; two 4-bit scales per 32
+// weights (low nibble: first 16).  The thread's 16 weights are entries 8 p + 4 e + 2 h and the next one.  LDS tables as for
+// IQ2_XXS with 512 grid entries.
+struct GIQ2XS {
+    static constexpr int kBlockBytes = 74;
+    struct Regs { uint32_t q0, q1, sc, d; };
+    static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, const float*, int, int p, int h) {
+        r.q0 = reinterpret_cast<const UnalignedWord*>(blk + 2 + 16 * p + 4 * h)->v;
+        r.q1 = reinterpret_cast<const UnalignedWord*>(blk + 10 + 16 * p + 4 * h)->v;
+        r.sc = *reinterpret_cast<const uint16_t*>(blk + 66 + 2 * p);
+        r.d = *reinterpret_cast<const uint16_t*>(blk);
+    }
+    static constexpr int kTableBytes = 8192 + 2048;
+    static __device__ __forceinline__ void stage_table(unsigned char* lds) {
+        _Float16* mag = reinterpret_cast<_Float16*>(lds);
+        uint16_t* sgn = reinterpret_cast<uint16_t*>(lds + 8192);
+        for (int i = threadIdx.x; i < 512 * 8; i += kThreads)
+            mag[i] = static_cast<_Float16>(static_cast<float>((PLLM_IQ2XS_GRID[i >> 3] >> (8 * (i & 7))) & 0xffull));
+        for (int i = threadIdx.x; i < 128 * 8; i += kThreads) {
+            const uint32_t s7 = static_cast<uint32_t>(i >> 3);
+            const uint32_t s8 = s7 | ((__popc(s7) & 1u) << 7);
+            sgn[i] = ((s8 >> (i & 7)) & 1u) ? 0x8000u : 0u;
+        }
+    }
+    static __device__ __forceinline__ void entry(const unsigned char* table, uint32_t q16, float scale, half4& lo, half4& hi) {
+        const uint4 m = *reinterpret_cast<const uint4*>(table + 16 * (q16 & 511u));
+        const uint4 f = *reinterpret_cast<const uint4*>(table + 8192 + 16 * (q16 >> 9));
+        lo = half4_of(scaled_pair(m.x, f.x, scale), scaled_pair(m.y, f.y, scale));
+        hi = half4_of(scaled_pair(m.z, f.z, scale), scaled_pair(m.w, f.w, scale));
+    }
+    static __device__ __forceinline__ void decode(const Regs& r, int, int e, int h, const unsigned char* table, Half16& o) {
+        const uint32_t pair = e ? r.q1 : r.q0;
+        const uint32_t ls = (r.sc >> (8 * e + 4 * h)) & 15u;
+        const float scale = 0.125f * f16_bits_to_float(r.d) * static_cast<float>(2 * ls + 1);
+        entry(table, pair & 0xffffu, scale, o.a, o.b);
+        entry(table, pair >> 16, scale, o.c, o.d);
+    }
+};
+
+// IQ3_XXS: 98 B = d(2) grid ids(64) aux u32[8].  An id gives four weights; aux of a 32-weight sub-block = four 7-bit sign indices
+// (one per 8 weights) and a 4-bit scale.  The thread's 16 weights are ids 8 (2 p + e) + 4 h .. + 3 with sign indices 2 h, 2 h + 1.
+// LDS tables: 256 x 4 magnitudes as fp16, then the 128 x 8 sign bits.
+struct GIQ3XXS {
+    static constexpr int kBlockBytes = 98;
+    struct Regs { uint32_t i0, i1, a0, a1, d; };
+    static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, const float*, int, int p, int h) {
+        r.i0 = reinterpret_cast<const UnalignedWord*>(blk + 2 + 16 * p + 4 * h)->v;
+        r.i1 = reinterpret_cast<const UnalignedWord*>(blk + 10 + 16 * p + 4 * h)->v;
+        r.a0 = reinterpret_cast<const UnalignedWord*>(blk + 66 + 8 * p)->v;
+        r.a1 = reinterpret_cast<const UnalignedWord*>(blk + 70 + 8 * p)->v;
+        r.d = *reinterpret_cast<const uint16_t*>(blk);
+    }
+    static constexpr int kTableBytes = 2048 + 2048;
+    static __device__ __forceinline__ void stage_table(unsigned char* lds) {
+        _Float16* mag = reinterpret_cast<_Float16*>(lds);
+        uint16_t* sgn = reinterpret_cast<uint16_t*>(lds + 2048);
+        for (int i = threadIdx.x; i < 256 * 4; i += kThreads)
+            mag[i] = static_cast<_Float16>(static_cast<float>((PLLM_IQ3XXS_GRID[i >> 2] >> (8 * (i & 3))) & 0xffu));
+        for (int i = threadIdx.x; i < 128 * 8; i += kThreads) {
+            const uint32_t s7 = static_cast<uint32_t>(i >> 3);
+            const uint32_t s8 = s7 | ((__popc(s7) & 1u) << 7);
+            sgn[i] = ((s8 >> (i & 7)) & 1u) ? 0x8000u : 0u;
+        }
+    }
+    static __device__ __forceinline__ half4 four(const unsigned char* table, uint32_t id, uint32_t flip_lo, uint32_t flip_hi, float scale) {
+        const uint2 m = *reinterpret_cast<const uint2*>(table + 8 * id);
+        return half4_of(scaled_pair(m.x, flip_lo, scale), scaled_pair(m.y, flip_hi, scale));
+    }
+    static __device__ __forceinline__ void decode(const Regs& r, int, int e, int h, const unsigned char* table, Half16& o) {
+        const uint32_t ids = e ? r.i1 : r.i0, aux = e ? r.a1 : r.a0;
+        const float scale = 0.25f * f16_bits_to_float(r.d) * static_cast<float>(2 * (aux >> 28) + 1);
+        const uint4 f0 = *reinterpret_cast<const uint4*>(table + 2048 + 16 * ((aux >> (14 * h)) & 127u));
+        const uint4 f1 = *reinterpret_cast<const uint4*>(table + 2048 + 16 * ((aux >> (14 * h + 7)) & 127u));
+        o.a = four(table, ids & 0xffu, f0.x, f0.y, scale);
+        o.b = four(table, (ids >> 8) & 0xffu, f0.z, f0.w, scale);
+        o.c = four(table, (ids >> 16) & 0xffu, f1.x, f1.y, scale);
+        o.d = four(table, ids >> 24, f1.z, f1.w, scale);
+    }
+};
+
 // IQ1_M: 56 B = qs(32) qh(16) scales(8).  One codebook index per 8 weights (qs byte plus the low three
 // bits of its qh nibble; bit 3 of the nibble picks delta = -+0.125); sixteen 3-bit scales, one per 16
 // weights, in the low 12 bits of four u16 words whose top nibbles spell the fp16 block scale.
@@ -702,7 +782,8 @@ size_t align256(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
 
 bool gemm_f16_supports(int type_id) {
     return type_id == PLLM_TYPE_Q4_K || type_id == PLLM_TYPE_Q5_K || type_id == PLLM_TYPE_Q2_K || type_id == PLLM_TYPE_IQ2_XXS ||
-           type_id == PLLM_TYPE_IQ1_M || type_id == PLLM_TYPE_Q6_K || type_id == PLLM_TYPE_IQ4_XS;
+           type_id == PLLM_TYPE_IQ1_M || type_id == PLLM_TYPE_Q6_K || type_id == PLLM_TYPE_IQ4_XS || type_id == PLLM_TYPE_IQ2_XS ||
+           type_id == PLLM_TYPE_IQ3_XXS;
 }
 
 size_t gemm_f16_workspace_bytes(int rows, int n, int bpr) {
@@ -750,6 +831,8 @@ int gemm_f16(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y,
         case PLLM_TYPE_IQ1_M: return launch_gemm_mi<GIQ1M>(p, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, nullptr, 0, nullptr, 0, 1, stream);
         case PLLM_TYPE_Q6_K: return launch_gemm_mi<GQ6K>(p, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, nullptr, 0, nullptr, 0, 1, stream);
         case PLLM_TYPE_IQ4_XS: return launch_gemm_mi<GIQ4XS>(p, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, nullptr, 0, nullptr, 0, 1, stream);
+        case PLLM_TYPE_IQ2_XS: return launch_gemm_mi<GIQ2XS>(p, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, nullptr, 0, nullptr, 0, 1, stream);
+        case PLLM_TYPE_IQ3_XXS: return launch_gemm_mi<GIQ3XXS>(p, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, nullptr, 0, nullptr, 0, 1, stream);
         default: return PLLM_ERR_UNSUPPORTED;
     }
 }

@@ -134,13 +134,17 @@ def test_prefill_other_formats_match_float_oracle(mod, type_name, t, n, k):
     assert O.rel_l2(y.cpu().numpy(), want) <= 1e-3, (type_name, t, n, k)
 
 
-@pytest.mark.parametrize("type_name", ["q6_k", "iq4_xs"])
+@pytest.mark.parametrize("type_name", ["q6_k", "iq4_xs", "iq2_xs", "iq3_xxs"])
 @pytest.mark.parametrize("t,n,k", [(16, 128, 256), (40, 96, 768), (130, 33, 1000), (300, 520, 5120), (1100, 200, 512)])
 def test_prefill_operator_serves_q6_k_and_iq4_xs(mod, type_name, t, n, k):
-    """Q6_K (2-byte aligned blocks, signed scales) and IQ4_XS (code table through byte permutes) in the tile kernel."""
+    """Q6_K (2-byte aligned blocks, signed scales), IQ4_XS (code table through byte permutes), IQ2_XS and IQ3_XXS (grid and sign
+    tables in LDS) in the tile kernel."""
     rng = np.random.default_rng(t + n + k)
-    enc = C.quantize_q6_k if type_name == "q6_k" else C.quantize_iq4_xs
-    blocks = enc((rng.standard_normal((n, k)) * 0.02).astype(np.float32))
+    if type_name in ("q6_k", "iq4_xs"):
+        enc = C.quantize_q6_k if type_name == "q6_k" else C.quantize_iq4_xs
+        blocks = enc((rng.standard_normal((n, k)) * 0.02).astype(np.float32))
+    else:
+        blocks = C.random_blocks(rng, type_name, n, (k + 255) // 256)
     x = torch.from_numpy(rng.standard_normal((t, k)).astype(np.float32)).to(DEV).to(torch.bfloat16)
     print(f"case {type_name} prefill t={t} n={n} k={k}", flush=True)
     y = mod.gguf_quant_gemm_prefill_forward(x, torch.from_numpy(blocks).to(DEV), k, O.TYPE_IDS[type_name],
