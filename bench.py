@@ -152,13 +152,15 @@ def extra_cases(mod, dev, iters):
         x = torch.randn(1, k, device=dev)
         run(f"q8_0 matvec {n}x{k} T=1", blocks.size, lambda s, ring=ring, x=x, k=k: mod.q8_0_gemm_forward(x, ring[s], k), len(ring))
         del ring
-    # Q2_K, Q6_K and IQ4_XS at the large shape (random valid blocks for the latter two: the kernels' work does not depend on the values)
+    # Q2_K and the other five formats at the large shape (random valid blocks for those: the kernels' work does not depend on the values)
     x = torch.randn(1, 5120, device=dev, dtype=torch.bfloat16)
     for name, tid, blocks in (("q2_k", 1, C.quantize_q2_k((rng.standard_normal((17408, 5120), dtype=np.float32) * np.float32(0.02)))),
-                              ("q6_k", 8, C.random_blocks(rng, "q6_k", 17408, 20)), ("iq4_xs", 7, C.random_blocks(rng, "iq4_xs", 17408, 20))):
+                              ("q6_k", 8, C.random_blocks(rng, "q6_k", 17408, 20)), ("iq4_xs", 7, C.random_blocks(rng, "iq4_xs", 17408, 20)),
+                              ("iq3_xxs", 6, C.random_blocks(rng, "iq3_xxs", 17408, 20)), ("iq2_xs", 5, C.random_blocks(rng, "iq2_xs", 17408, 20))):
         ring = ring_of(blocks, dev, max(2, min(RING, (1 << 30) // blocks.size)))
+        grid = codebooks.grid_tensor_for_type(tid).to(dev)
         run(f"{name} matvec 17408x5120 T=1", blocks.size,
-            lambda s, ring=ring, x=x, tid=tid: mod.gguf_quant_gemm_forward(x, ring[s], 5120, tid, empty), len(ring))
+            lambda s, ring=ring, x=x, tid=tid, grid=grid: mod.gguf_quant_gemm_forward(x, ring[s], 5120, tid, grid), len(ring))
         del ring
     # FP8 E4M3 + 128x128 scales, BASELINE config 4 at T=1
     codes, scale = C.quantize_fp8_block((rng.standard_normal((17408, 5120), dtype=np.float32) * np.float32(0.02)))
@@ -217,7 +219,7 @@ F16_MFMA_PEAK_TFLOPS = 2500.0
 def prefill_cases(mod, dev, iters):
     """BASELINE configs 3 and 4 at T > 1: the MFMA tile kernel, TFLOPS = 2 T K N / t against the dense fp16 peak
     (the tiles are decoded to fp16, see the kernel's header for why)."""
-    from pocketllm_amd import block_codec as C
+    from pocketllm_amd import block_codec as C, codebooks
     rng = np.random.default_rng(4004)
     out = []
     empty = torch.empty(0, dtype=torch.int8, device=dev)
@@ -238,11 +240,13 @@ def prefill_cases(mod, dev, iters):
                     lambda s, x=x, blocks=blocks, tid=tid: mod.gguf_quant_gemm_prefill_forward(x, blocks, k, tid, empty))
             del blocks
     n = 17408
-    for name, tid in (("q6_k", 8), ("iq4_xs", 7)):             # random valid blocks: the work does not depend on the values
+    for name, tid in (("q6_k", 8), ("iq4_xs", 7), ("iq3_xxs", 6), ("iq2_xs", 5)):   # random valid blocks: the work does not depend on the values
         blocks = torch.from_numpy(C.random_blocks(rng, name, n, k // 256)).to(dev)
+        grid = codebooks.grid_tensor_for_type(tid).to(dev)
         for t in (512, 2048):
             x = torch.randn(t, k, device=dev, dtype=torch.bfloat16)
-            run(f"{name} prefill {n}x{k} T={t}", t, n, lambda s, x=x, blocks=blocks, tid=tid: mod.gguf_quant_gemm_prefill_forward(x, blocks, k, tid, empty))
+            run(f"{name} prefill {n}x{k} T={t}", t, n,
+                lambda s, x=x, blocks=blocks, tid=tid, grid=grid: mod.gguf_quant_gemm_prefill_forward(x, blocks, k, tid, grid))
         del blocks
     codes, scale = C.quantize_fp8_block(rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02))
     codes = torch.from_numpy(codes).to(dev)
@@ -305,7 +309,7 @@ def iq_pass(mod, dev) -> None:
 
 def prefill_pass(mod, dev) -> None:
     """A few launches of the MFMA tile kernel for the profiler: Q4_K 17408x5120 at T=2048 and FP8 at T=512."""
-    from pocketllm_amd import block_codec as C
+    from pocketllm_amd import block_codec as C, codebooks
     rng = np.random.default_rng(4004)
     k, n = 5120, 17408
     empty = torch.empty(0, dtype=torch.int8, device=dev)

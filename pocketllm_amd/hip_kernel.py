@@ -57,6 +57,12 @@ def _check_grid(grid: torch.Tensor, type_id: int, name: str) -> None:
         _check(grid.dtype == torch.int8, f"{name} must be int8")
         _check(grid.is_contiguous(), f"{name} must be contiguous")
         _check(grid.numel() == 2048 * 8, f"{name} must contain 2048*8 entries for iq1_m")
+    elif type_id in (5, 6):
+        _check(grid.is_cuda, f"{name} must be CUDA for iq2_xs/iq3_xxs")
+        _check(grid.dtype == torch.int8, f"{name} must be int8")
+        _check(grid.is_contiguous(), f"{name} must be contiguous")
+        _check(grid.numel() >= 512 * 128 * 8 + 256 * 128 * 8,
+               f"{name} must contain packed iq2_xs and iq3_xxs signed grids")
 
 
 def _check_type(type_id: int, what: str = "type_id") -> None:
@@ -289,7 +295,10 @@ def gguf_quant_gemm_pair_forward(x, blocks0, row_elems0, type_id0, blocks1, row_
     _check_type(type_id1, "type_id1")
     uses_iq2 = type_id0 == 0 or type_id1 == 0
     uses_iq1 = type_id0 == 2 or type_id1 == 2
+    uses_xs = type_id0 in (5, 6) or type_id1 in (5, 6)
     _check(not (uses_iq2 and uses_iq1), "paired GEMM cannot mix iq2_xxs and iq1_m because they require different grids")
+    _check(not (uses_iq2 and uses_xs), "paired GEMM cannot mix iq2_xxs with iq2_xs/iq3_xxs because they require different grids")
+    _check(not (uses_iq1 and uses_xs), "paired GEMM cannot mix iq1_m with iq2_xs/iq3_xxs because they require different grids")
     _check(row_elems0 > 0 and row_elems1 > 0, "row_elems must be positive")
     _check(row_elems0 == row_elems1, "paired GGUF GEMM requires matching input dimensions")
     _check(x.size(-1) == row_elems0, "inner dimension mismatch")
@@ -307,6 +316,8 @@ def gguf_quant_gemm_pair_forward(x, blocks0, row_elems0, type_id0, blocks1, row_
         _check_grid(signed_grid, 0, "signed_grid")
     elif uses_iq1:
         _check_grid(signed_grid, 2, "signed_grid")
+    elif uses_xs:
+        _check_grid(signed_grid, 5, "signed_grid")
     rows = x.numel() // row_elems0
     n = blocks0.size(0)
     y = torch.empty(2, *x.shape[:-1], n, dtype=out_dtype, device=x.device)

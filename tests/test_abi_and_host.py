@@ -95,6 +95,18 @@ def test_codebooks_agree_with_oracle_copy():
     np.testing.assert_array_equal(codebooks.iq1_grid(), O.iq1_grid_i8())
     assert tuple(codebooks.get_iq2xxs_signed_grid_tensor().shape) == (256, 128, 8)
     assert codebooks.get_iq1_grid_tensor().dtype == torch.int8
+    np.testing.assert_array_equal(codebooks.iq2xs_grid(), O.iq2xs_grid_u8())
+    np.testing.assert_array_equal(codebooks.iq3xxs_grid(), O.iq3xxs_grid_u8())
+    # the packed tensor for type ids 5 and 6: entry x sign pattern, IQ3_XXS entries doubled under the two sign halves
+    packed = codebooks.get_iq2xs_iq3xxs_signed_grid_tensor()
+    assert packed.dtype == torch.int8 and packed.numel() == 512 * 128 * 8 + 256 * 128 * 8
+    xs, xxs = codebooks.iq2xs_signed_grid(), codebooks.iq3xxs_signed_grid()
+    ks = codebooks.ksigns()
+    for g, s_ in ((0, 0), (511, 127), (300, 77)):
+        sign = np.where((ks[s_] >> np.arange(8)) & 1, -1, 1)
+        np.testing.assert_array_equal(xs[g, s_], O.iq2xs_grid_u8()[g].astype(np.int16) * sign)
+        np.testing.assert_array_equal(xxs[g % 256, s_], np.tile(O.iq3xxs_grid_u8()[g % 256].astype(np.int16), 2) * sign)
+    assert codebooks.grid_tensor_for_type(3).numel() == 0 and codebooks.grid_tensor_for_type(6).numel() == packed.numel()
 
 
 @pytest.mark.parametrize("name,enc,bits", [("q4_k", C.quantize_q4_k, 4), ("q5_k", C.quantize_q5_k, 5), ("q2_k", C.quantize_q2_k, 2)])

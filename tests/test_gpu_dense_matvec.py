@@ -8,7 +8,7 @@ import pytest
 import torch
 
 from oracle import gguf_oracle as O
-from pocketllm_amd import block_codec as C
+from pocketllm_amd import block_codec as C, codebooks
 from pocketllm_amd.cuda_loader import load_cuda_kernel
 
 pytestmark = pytest.mark.gpu
@@ -33,7 +33,7 @@ def _run_dense(mod, type_name, blocks, x_np, x_dtype, k):
     dev = torch.device("cuda:0")
     x = torch.from_numpy(x_np).to(dev).to(x_dtype).contiguous()
     b = torch.from_numpy(blocks).to(dev)
-    grid = torch.empty(0, dtype=torch.int8, device=dev)
+    grid = codebooks.grid_tensor_for_type(O.TYPE_IDS[type_name]).to(dev)
     y = mod.gguf_quant_gemm_forward(x, b, k, O.TYPE_IDS[type_name], grid, out_dtype=torch.float32)
     torch.cuda.synchronize()
     return x.float().cpu().numpy(), y.cpu().numpy()
@@ -208,7 +208,7 @@ def test_iq2xs_iq3xxs_matvec_matches_oracle(mod, type_name, n, k, rows):
     dev = torch.device("cuda:0")
     print(f"case {type_name} n={n} k={k} rows={rows}", flush=True)
     y = mod.gguf_quant_gemm_forward(torch.from_numpy(x_np).to(dev).to(torch.bfloat16), torch.from_numpy(blocks).to(dev), k, O.TYPE_IDS[type_name],
-                                    torch.empty(0, dtype=torch.int8, device=dev), out_dtype=torch.float32)
+                                    codebooks.grid_tensor_for_type(O.TYPE_IDS[type_name]).to(dev), out_dtype=torch.float32)
     torch.cuda.synchronize()
     x_used = torch.from_numpy(x_np).to(torch.bfloat16).float().numpy()
     want = O.matmul_f(x_used, O.dequant_rows(blocks, type_name, k))
@@ -239,3 +239,10 @@ def test_codebook_grid_argument_is_validated(mod):
         mod.gguf_quant_gemm_forward(x, blocks, 256, 0, torch.empty(0, dtype=torch.int8, device=dev))
     with pytest.raises(RuntimeError, match="2048\\*8 entries for iq1_m"):
         mod.gguf_quant_gemm_forward(x, torch.zeros(4, 1, 56, dtype=torch.uint8, device=dev), 256, 2, torch.empty(0, dtype=torch.int8, device=dev))
+    for tid, bb in ((5, 74), (6, 98)):
+        with pytest.raises(RuntimeError, match="packed iq2_xs and iq3_xxs signed grids"):
+            mod.gguf_quant_gemm_forward(x, torch.zeros(4, 1, bb, dtype=torch.uint8, device=dev), 256, tid,
+                                        codebooks.get_iq2xs_signed_grid_tensor().to(dev))
+    with pytest.raises(RuntimeError, match="cannot mix iq1_m with iq2_xs/iq3_xxs"):
+        mod.gguf_quant_gemm_pair_forward(x, torch.zeros(4, 1, 56, dtype=torch.uint8, device=dev), 256, 2,
+                                         torch.zeros(4, 1, 74, dtype=torch.uint8, device=dev), 256, 5, codebooks.get_iq1_grid_tensor().to(dev))

@@ -4,7 +4,7 @@ import pytest
 import torch
 
 from oracle import gguf_oracle as O
-from pocketllm_amd import block_codec as C
+from pocketllm_amd import block_codec as C, codebooks
 from pocketllm_amd.cuda_loader import load_cuda_kernel
 
 pytestmark = pytest.mark.gpu
@@ -66,7 +66,7 @@ def test_prefill_baseline_shape_sampled(mod, type_name, n):
     blocks = ENC[type_name]((rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02)))
     x = torch.from_numpy(rng.standard_normal((t, k)).astype(np.float32)).to(DEV).to(torch.bfloat16)
     y = mod.gguf_quant_gemm_prefill_forward(x, torch.from_numpy(blocks).to(DEV), k, O.TYPE_IDS[type_name],
-                                            torch.empty(0, dtype=torch.int8, device=DEV), out_dtype=torch.float32)
+                                            codebooks.grid_tensor_for_type(O.TYPE_IDS[type_name]).to(DEV), out_dtype=torch.float32)
     torch.cuda.synchronize()
     cols = rng.choice(n, size=64, replace=False)
     want = O.matmul_f(x.float().cpu().numpy(), O.dequant_rows(blocks[cols], type_name, k))
@@ -148,7 +148,7 @@ def test_prefill_operator_serves_q6_k_and_iq4_xs(mod, type_name, t, n, k):
     x = torch.from_numpy(rng.standard_normal((t, k)).astype(np.float32)).to(DEV).to(torch.bfloat16)
     print(f"case {type_name} prefill t={t} n={n} k={k}", flush=True)
     y = mod.gguf_quant_gemm_prefill_forward(x, torch.from_numpy(blocks).to(DEV), k, O.TYPE_IDS[type_name],
-                                            torch.empty(0, dtype=torch.int8, device=DEV), out_dtype=torch.float32)
+                                            codebooks.grid_tensor_for_type(O.TYPE_IDS[type_name]).to(DEV), out_dtype=torch.float32)
     torch.cuda.synchronize()
     want = O.matmul_f(x.float().cpu().numpy(), O.dequant_rows(blocks, type_name, k))
     assert O.rel_l2(y.cpu().numpy(), want) <= 1e-3, (type_name, t, n, k)
