@@ -22,15 +22,7 @@ __global__ __launch_bounds__(kThreads) void act_image_256_kernel(
     float v[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) v[i] = (e0 + i < k) ? load_any(x, x_dtype, xoff + e0 + i) : 0.0f;
-    uint32_t qh, ql;
-    float scale;
-    quantize4(v, qh, ql, scale);
-    *reinterpret_cast<uint32_t*>(hi + e0) = qh;
-    *reinterpret_cast<uint32_t*>(lo + e0) = ql;
-    const float sum = group_sum<4>((v[0] + v[1]) + (v[2] + v[3]));
-    const float sum32 = sum + __shfl_xor(sum, 4, 64);
-    if ((threadIdx.x & 3) == 0) sum16[e0 >> 4] = sum;
-    if ((threadIdx.x & 7) == 0) gs[e0 >> 5] = make_float2(scale * kLoInv, sum32);
+    quantize4_to_image(v, e0, hi, lo, gs, sum16);
 }
 
 // Q8_0 pair image: per pair of 32-value blocks 80 bytes that mirror the weight stream,
@@ -47,32 +39,7 @@ __global__ __launch_bounds__(kThreads) void act_image_q8pair_kernel(
     float v[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) v[i] = (e0 + i < k) ? load_any(x, x_dtype, xoff + e0 + i) : 0.0f;
-    uint32_t qh, ql;
-    float scale;
-    quantize4(v, qh, ql, scale);
-    const int b = e0 >> 5;
-    const int j = (e0 & 31) >> 2;
-    const int off = (b >> 1) * 80 + ((b & 1) ? 36 : 2) + 4 * j;   // 2-byte aligned
-    *reinterpret_cast<uint16_t*>(hi + off) = static_cast<uint16_t>(qh);
-    *reinterpret_cast<uint16_t*>(hi + off + 2) = static_cast<uint16_t>(qh >> 16);
-    *reinterpret_cast<uint16_t*>(lo + off) = static_cast<uint16_t>(ql);
-    *reinterpret_cast<uint16_t*>(lo + off + 2) = static_cast<uint16_t>(ql >> 16);
-    if (j == 0) {
-        const int p0 = (b >> 1) * 80;
-        if (b & 1) {
-            *reinterpret_cast<uint16_t*>(hi + p0 + 34) = 0;
-            *reinterpret_cast<uint16_t*>(lo + p0 + 34) = 0;
-#pragma unroll
-            for (int z = 68; z < 80; z += 4) {
-                *reinterpret_cast<uint32_t*>(hi + p0 + z) = 0;
-                *reinterpret_cast<uint32_t*>(lo + p0 + z) = 0;
-            }
-        } else {
-            *reinterpret_cast<uint16_t*>(hi + p0) = 0;
-            *reinterpret_cast<uint16_t*>(lo + p0) = 0;
-        }
-        xs[b] = scale;
-    }
+    quantize4_to_pair_image(v, e0, hi, lo, xs);
 }
 
 }  // namespace

@@ -71,21 +71,32 @@ size_t pllm_q8_0_gemm_workspace_bytes(int64_t rows, int64_t k, int64_t n, int64_
     return pllm::q8_0_matvec_workspace_bytes(static_cast<int>(rows), static_cast<int>(blocks_per_row));
 }
 
-static int superblock_matvec(const unsigned char* image, size_t stride, const uint8_t* blocks, int type_id, void* y, int y_dtype,
+// Calls of up to this many rows skip the activation pre-pass where the kernel can quantize its row itself.  The Q4_K / Q5_K
+// kernel runs one short workgroup per 16 rows and every one of them repeats the quantization: that beats the extra launch
+// (~3 us) up to about a thousand workgroups of a 5120-wide row; the other kernels are longer per workgroup or persistent.
+constexpr int64_t kInKernelQuantMaxRows = 4;
+constexpr int64_t kInKernelQuantMaxWeightsK45 = int64_t{64} << 20;
+
+static bool quantizes_in_kernel(int type_id, int64_t n, int64_t bpr) {
+    if (type_id == PLLM_TYPE_Q4_K || type_id == PLLM_TYPE_Q5_K) return n * bpr * 256 <= kInKernelQuantMaxWeightsK45;
+    return pllm_gguf_block_bytes(type_id) != 0;
+}
+
+static int superblock_matvec(const pllm::ActRows& act, const uint8_t* blocks, int type_id, void* y, int y_dtype,
                              int rows, int n, int bpr, hipStream_t s) {
     switch (type_id) {
         case PLLM_TYPE_Q2_K:
-            return pllm::dot4_matvec_from_image(image, stride, blocks, type_id, y, y_dtype, rows, n, bpr, s);
+            return pllm::dot4_matvec_from_image(act, blocks, type_id, y, y_dtype, rows, n, bpr, s);
         case PLLM_TYPE_IQ2_XXS:
         case PLLM_TYPE_IQ1_M:
         case PLLM_TYPE_IQ2_XS:
         case PLLM_TYPE_IQ3_XXS:
         case PLLM_TYPE_IQ4_XS:
         case PLLM_TYPE_Q6_K:
-            return pllm::iq_mfma_matvec_from_image(image, stride, blocks, type_id, y, y_dtype, rows, n, bpr, s);
+            return pllm::iq_mfma_matvec_from_image(act, blocks, type_id, y, y_dtype, rows, n, bpr, s);
         case PLLM_TYPE_Q4_K:
         case PLLM_TYPE_Q5_K:
-            return pllm::kquant_matvec_from_image(image, stride, blocks, type_id, y, y_dtype, rows, n, bpr, s);
+            return pllm::kquant_matvec_from_image(act, blocks, type_id, y, y_dtype, rows, n, bpr, s);
         default:
             return PLLM_ERR_UNSUPPORTED;
     }
@@ -105,10 +116,13 @@ int pllm_gguf_quant_gemm(const void* x, int x_dtype, const uint8_t* blocks, int 
     if (rows >= kGemmMinRows && pllm::gemm_f16_supports(type_id))
         return pllm::gemm_f16(x, x_dtype, blocks, type_id, y, y_dtype, static_cast<int>(rows), static_cast<int>(k), static_cast<int>(n), bpr,
                               workspace, workspace_bytes, s);
+    if (rows <= kInKernelQuantMaxRows && quantizes_in_kernel(type_id, n, blocks_per_row))
+        return superblock_matvec(pllm::act_rows_raw(x, x_dtype, static_cast<int>(k)), blocks, type_id, y, y_dtype,
+                                 static_cast<int>(rows), static_cast<int>(n), bpr, s);
     const int st = pllm::act_image_256(x, x_dtype, static_cast<int>(rows), static_cast<int>(k), bpr, workspace, s);
     if (st != PLLM_OK) return st;
-    return superblock_matvec(static_cast<const unsigned char*>(workspace), pllm::act_image_256_bytes(bpr), blocks, type_id, y, y_dtype,
-                             static_cast<int>(rows), static_cast<int>(n), bpr, s);
+    return superblock_matvec(pllm::act_rows_from_image(static_cast<const unsigned char*>(workspace), pllm::act_image_256_bytes(bpr)), blocks,
+                             type_id, y, y_dtype, static_cast<int>(rows), static_cast<int>(n), bpr, s);
 }
 
 size_t pllm_gguf_quant_gemm_workspace_bytes(int type_id, int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row) {
@@ -140,8 +154,8 @@ int pllm_gguf_quant_gemm_prequantized(const void* image, const uint8_t* blocks, 
     if (pllm_gguf_block_bytes(type_id) == 0) return PLLM_ERR_UNSUPPORTED;
     if (rows > 65535) return PLLM_ERR_UNSUPPORTED;
     const int bpr = static_cast<int>(blocks_per_row);
-    return superblock_matvec(static_cast<const unsigned char*>(image), pllm::act_image_256_bytes(bpr), blocks, type_id, y, y_dtype,
-                             static_cast<int>(rows), static_cast<int>(n), bpr, static_cast<hipStream_t>(stream));
+    return superblock_matvec(pllm::act_rows_from_image(static_cast<const unsigned char*>(image), pllm::act_image_256_bytes(bpr)), blocks,
+                             type_id, y, y_dtype, static_cast<int>(rows), static_cast<int>(n), bpr, static_cast<hipStream_t>(stream));
 }
 
 int pllm_gguf_quant_gemm_pair(const void* x, int x_dtype, const uint8_t* blocks0, int type_id0, const uint8_t* blocks1, int type_id1,
@@ -155,14 +169,17 @@ int pllm_gguf_quant_gemm_pair(const void* x, int x_dtype, const uint8_t* blocks0
     if (!workspace || workspace_bytes < pllm_activation_image_bytes(rows, blocks_per_row)) return PLLM_ERR_WORKSPACE;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int bpr = static_cast<int>(blocks_per_row);
-    int st = pllm::act_image_256(x, x_dtype, static_cast<int>(rows), static_cast<int>(k), bpr, workspace, s);
-    if (st != PLLM_OK) return st;
-    const unsigned char* image = static_cast<const unsigned char*>(workspace);
-    const size_t stride = pllm::act_image_256_bytes(bpr);
+    pllm::ActRows act = pllm::act_rows_raw(x, x_dtype, static_cast<int>(k));
+    int st = PLLM_OK;
+    if (rows > kInKernelQuantMaxRows || !quantizes_in_kernel(type_id0, n, blocks_per_row) || !quantizes_in_kernel(type_id1, n, blocks_per_row)) {
+        st = pllm::act_image_256(x, x_dtype, static_cast<int>(rows), static_cast<int>(k), bpr, workspace, s);
+        if (st != PLLM_OK) return st;
+        act = pllm::act_rows_from_image(static_cast<const unsigned char*>(workspace), pllm::act_image_256_bytes(bpr));
+    }
     const size_t esize = y_dtype == PLLM_F32 ? 4 : 2;
-    st = superblock_matvec(image, stride, blocks0, type_id0, y, y_dtype, static_cast<int>(rows), static_cast<int>(n), bpr, s);
+    st = superblock_matvec(act, blocks0, type_id0, y, y_dtype, static_cast<int>(rows), static_cast<int>(n), bpr, s);
     if (st != PLLM_OK) return st;
-    return superblock_matvec(image, stride, blocks1, type_id1, static_cast<char*>(y) + static_cast<size_t>(rows) * n * esize, y_dtype,
+    return superblock_matvec(act, blocks1, type_id1, static_cast<char*>(y) + static_cast<size_t>(rows) * n * esize, y_dtype,
                              static_cast<int>(rows), static_cast<int>(n), bpr, s);
 }
 

@@ -15,9 +15,9 @@ namespace {
 constexpr int kRowsPerWg = 16;
 constexpr int kMaxWaves = 8;
 
-template <typename FMT, int ITERS>
+template <typename FMT, int ITERS, bool RAW>
 __global__ __launch_bounds__(64 * kMaxWaves) void dot4_matvec_kernel(
-    const unsigned char* __restrict__ image, size_t image_stride, const uint8_t* __restrict__ w,
+    const ActRows act, const uint8_t* __restrict__ w,
     void* __restrict__ y, int y_dtype, int n, int bpr, const int32_t* __restrict__ y_expert, size_t expert_stride) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int kpad = bpr * 256;
@@ -38,6 +38,8 @@ __global__ __launch_bounds__(64 * kMaxWaves) void dot4_matvec_kernel(
 
     float acc = 0.0f;
     bool staged = false;
+    if constexpr (RAW)                       // raw activation row: quantized here, before the loads take their registers
+        quantize_row_to_lds(smem, act.x, act.x_dtype, static_cast<size_t>(blockIdx.y) * act.k, act.k, kpad);
     for (int b0 = wave; b0 < bpr || !staged; b0 += waves * ITERS) {
         typename FMT::Regs regs[ITERS];
 #pragma unroll
@@ -46,7 +48,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void dot4_matvec_kernel(
             FMT::load(regs[it], wrow + static_cast<size_t>(b) * FMT::kBlockBytes, j);
         }
         if (!staged) {                       // first trip of every thread of the workgroup
-            copy_to_lds(smem, image + static_cast<size_t>(blockIdx.y) * image_stride, image_bytes);
+            if constexpr (!RAW) copy_to_lds(smem, act.image + static_cast<size_t>(blockIdx.y) * act.stride, image_bytes);
             FMT::stage_tables(tables);
             __syncthreads();
             staged = true;
@@ -69,11 +71,11 @@ __global__ __launch_bounds__(64 * kMaxWaves) void dot4_matvec_kernel(
     }
 }
 
-template <typename FMT, int ITERS>
-int launch_one(const unsigned char* image, size_t image_stride, const uint8_t* w, void* y, int y_dtype,
+template <typename FMT, int ITERS, bool RAW>
+int launch_one(const ActRows& act, const uint8_t* w, void* y, int y_dtype,
                int rows, int n, int bpr, int waves, const int32_t* y_expert, size_t expert_stride, hipStream_t stream) {
     const size_t smem = staged_x_bytes(bpr * 256) + FMT::kTableBytes + static_cast<size_t>(waves) * kRowsPerWg * sizeof(float);
-    auto kern = dot4_matvec_kernel<FMT, ITERS>;
+    auto kern = dot4_matvec_kernel<FMT, ITERS, RAW>;
     if (smem > 64 * 1024) {
         if (smem > 160 * 1024) return PLLM_ERR_UNSUPPORTED;
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -81,12 +83,12 @@ int launch_one(const unsigned char* image, size_t image_stride, const uint8_t* w
             return PLLM_ERR_UNSUPPORTED;
     }
     dim3 grid((n + kRowsPerWg - 1) / kRowsPerWg, rows);
-    hipLaunchKernelGGL(kern, grid, dim3(64 * waves), smem, stream, image, image_stride, w, y, y_dtype, n, bpr, y_expert, expert_stride);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * waves), smem, stream, act, w, y, y_dtype, n, bpr, y_expert, expert_stride);
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 
 template <typename FMT>
-int launch_fmt(const unsigned char* image, size_t image_stride, const uint8_t* w, void* y, int y_dtype,
+int launch_fmt(const ActRows& act, const uint8_t* w, void* y, int y_dtype,
                int rows, int n, int bpr, const int32_t* y_expert, size_t expert_stride, hipStream_t stream) {
     // waves per workgroup: split a row's blocks so that every wave keeps a handful in flight
     int waves = 1;
@@ -94,29 +96,35 @@ int launch_fmt(const unsigned char* image, size_t image_stride, const uint8_t* w
     const int niter = (bpr + waves - 1) / waves;
     const int passes = (niter + 5) / 6;
     const int iters = (niter + passes - 1) / passes;
-#define PLLM_CASE(I) case I: return launch_one<FMT, I>(image, image_stride, w, y, y_dtype, rows, n, bpr, waves, y_expert, expert_stride, stream)
+#define PLLM_CASE(I) case I: return act.x ? launch_one<FMT, I, true>(act, w, y, y_dtype, rows, n, bpr, waves, y_expert, expert_stride, stream) \
+                                          : launch_one<FMT, I, false>(act, w, y, y_dtype, rows, n, bpr, waves, y_expert, expert_stride, stream)
     switch (iters) {
         PLLM_CASE(1); PLLM_CASE(2); PLLM_CASE(3); PLLM_CASE(4); PLLM_CASE(5);
-        default: return launch_one<FMT, 6>(image, image_stride, w, y, y_dtype, rows, n, bpr, waves, y_expert, expert_stride, stream);
+        default: PLLM_CASE(6);
     }
 #undef PLLM_CASE
 }
 
 }  // namespace
 
-int dot4_matvec_from_image(const unsigned char* image, size_t stride, const uint8_t* w, int type_id, void* y, int y_dtype,
+static int dot4_dispatch(const ActRows& act, const uint8_t* w, int type_id, void* y, int y_dtype,
+                         int rows, int n, int bpr, const int32_t* y_expert, size_t expert_stride, hipStream_t stream) {
+    switch (type_id) {
+        case PLLM_TYPE_Q2_K: return launch_fmt<Q2K>(act, w, y, y_dtype, rows, n, bpr, y_expert, expert_stride, stream);
+        case PLLM_TYPE_IQ2_XXS: return launch_fmt<IQ2XXS>(act, w, y, y_dtype, rows, n, bpr, y_expert, expert_stride, stream);
+        case PLLM_TYPE_IQ1_M: return launch_fmt<IQ1M>(act, w, y, y_dtype, rows, n, bpr, y_expert, expert_stride, stream);
+        default: return PLLM_ERR_UNSUPPORTED;
+    }
+}
+
+int dot4_matvec_from_image(const ActRows& act, const uint8_t* w, int type_id, void* y, int y_dtype,
                            int rows, int n, int bpr, hipStream_t stream) {
-    return dot4_routed_matvec_from_image(image, stride, w, type_id, y, y_dtype, rows, n, bpr, nullptr, 0, stream);
+    return dot4_dispatch(act, w, type_id, y, y_dtype, rows, n, bpr, nullptr, 0, stream);
 }
 
 int dot4_routed_matvec_from_image(const unsigned char* image, size_t stride, const uint8_t* w, int type_id, void* y, int y_dtype,
                                   int rows, int n, int bpr, const int32_t* y_expert, size_t expert_stride, hipStream_t stream) {
-    switch (type_id) {
-        case PLLM_TYPE_Q2_K: return launch_fmt<Q2K>(image, stride, w, y, y_dtype, rows, n, bpr, y_expert, expert_stride, stream);
-        case PLLM_TYPE_IQ2_XXS: return launch_fmt<IQ2XXS>(image, stride, w, y, y_dtype, rows, n, bpr, y_expert, expert_stride, stream);
-        case PLLM_TYPE_IQ1_M: return launch_fmt<IQ1M>(image, stride, w, y, y_dtype, rows, n, bpr, y_expert, expert_stride, stream);
-        default: return PLLM_ERR_UNSUPPORTED;
-    }
+    return dot4_dispatch(act_rows_from_image(image, stride), w, type_id, y, y_dtype, rows, n, bpr, y_expert, expert_stride, stream);
 }
 
 }  // namespace pllm

@@ -24,10 +24,9 @@ constexpr int kWaves = 8;
 // One workgroup per tile of 16 rows: its W waves split the row's super-blocks (wave w takes blocks w,
 // w + W, ...) and meet in a small LDS reduction.  All weight loads of a pass are issued first; while
 // they are in flight the workgroup fills LDS with the activation image and the format's codebooks.
-template <typename FMT, int ITERS>
+template <typename FMT, int ITERS, bool RAW>
 __global__ __launch_bounds__(64 * kWaves) void mfma_tile_matvec_kernel(
-    const unsigned char* __restrict__ image, size_t image_stride, const uint8_t* __restrict__ w,
-    void* __restrict__ y, int y_dtype, int n, int bpr) {
+    const ActRows act, const uint8_t* __restrict__ w, void* __restrict__ y, int y_dtype, int n, int bpr) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int kpad = bpr * 256;
     const int image_bytes = static_cast<int>(staged_x_bytes(kpad));
@@ -51,6 +50,8 @@ __global__ __launch_bounds__(64 * kWaves) void mfma_tile_matvec_kernel(
 
     float acc = 0.0f;
     bool staged = false;
+    if constexpr (RAW)                       // raw activation row: quantized here, before the loads take their registers
+        quantize_row_to_lds(smem, act.x, act.x_dtype, static_cast<size_t>(blockIdx.y) * act.k, act.k, kpad);
     for (int b0 = wave; b0 < bpr || !staged; b0 += waves * ITERS) {
         typename FMT::Regs regs[ITERS];
 #pragma unroll
@@ -59,7 +60,7 @@ __global__ __launch_bounds__(64 * kWaves) void mfma_tile_matvec_kernel(
             FMT::load(regs[it], wrow + static_cast<size_t>(b) * FMT::kBlockBytes, ks);
         }
         if (!staged) {                       // first trip of every thread of the workgroup
-            copy_to_lds(smem, image + static_cast<size_t>(blockIdx.y) * image_stride, image_bytes);
+            if constexpr (!RAW) copy_to_lds(smem, act.image + static_cast<size_t>(blockIdx.y) * act.stride, image_bytes);
             if (tid < 4) reinterpret_cast<uint32_t*>(smem + zero_off)[tid] = 0;
             FMT::stage_tables(tables);
             __syncthreads();
@@ -83,11 +84,11 @@ __global__ __launch_bounds__(64 * kWaves) void mfma_tile_matvec_kernel(
     }
 }
 
-template <typename FMT, int ITERS>
-int launch_tile(const unsigned char* image, size_t image_stride, const uint8_t* w, void* y, int y_dtype,
+template <typename FMT, int ITERS, bool RAW>
+int launch_tile(const ActRows& act, const uint8_t* w, void* y, int y_dtype,
                 int rows, int n, int bpr, int waves, hipStream_t stream) {
     const size_t smem = staged_x_bytes(bpr * 256) + 16 + FMT::kTableBytes + static_cast<size_t>(waves) * kRowsPerTile * sizeof(float);
-    auto kern = mfma_tile_matvec_kernel<FMT, ITERS>;
+    auto kern = mfma_tile_matvec_kernel<FMT, ITERS, RAW>;
     if (smem > 64 * 1024) {
         if (smem > 160 * 1024) return PLLM_ERR_UNSUPPORTED;
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -95,12 +96,12 @@ int launch_tile(const unsigned char* image, size_t image_stride, const uint8_t* 
             return PLLM_ERR_UNSUPPORTED;
     }
     dim3 grid((n + kRowsPerTile - 1) / kRowsPerTile, rows);
-    hipLaunchKernelGGL(kern, grid, dim3(64 * waves), smem, stream, image, image_stride, w, y, y_dtype, n, bpr);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * waves), smem, stream, act, w, y, y_dtype, n, bpr);
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 
 template <typename FMT>
-int launch_tiles(const unsigned char* image, size_t image_stride, const uint8_t* w, void* y, int y_dtype,
+int launch_tiles(const ActRows& act, const uint8_t* w, void* y, int y_dtype,
                  int rows, int n, int bpr, hipStream_t stream) {
     // waves per workgroup: split a row's blocks so that every wave keeps a handful in flight
     int waves = 1;
@@ -108,10 +109,11 @@ int launch_tiles(const unsigned char* image, size_t image_stride, const uint8_t*
     const int niter = (bpr + waves - 1) / waves;
     const int passes = (niter + 5) / 6;
     const int iters = (niter + passes - 1) / passes;
-#define PLLM_CASE(I) case I: return launch_tile<FMT, I>(image, image_stride, w, y, y_dtype, rows, n, bpr, waves, stream)
+#define PLLM_CASE(I) case I: return act.x ? launch_tile<FMT, I, true>(act, w, y, y_dtype, rows, n, bpr, waves, stream) \
+                                          : launch_tile<FMT, I, false>(act, w, y, y_dtype, rows, n, bpr, waves, stream)
     switch (iters) {
         PLLM_CASE(1); PLLM_CASE(2); PLLM_CASE(3); PLLM_CASE(4); PLLM_CASE(5);
-        default: return launch_tile<FMT, 6>(image, image_stride, w, y, y_dtype, rows, n, bpr, waves, stream);
+        default: PLLM_CASE(6);
     }
 #undef PLLM_CASE
 }
@@ -130,9 +132,9 @@ constexpr int kChunkBudget = 28 * 1024;
 
 // NB > 0: a wave meets at most NB block indices (part, part + split, ...) and keeps their activation
 // side in registers across all its chunks; NB == 0: any number, read from LDS every time.
-template <typename FMT, int NB>
+template <typename FMT, int NB, bool RAW>
 __global__ __launch_bounds__(64 * kWaves) void iq_stream_matvec_kernel(
-    const unsigned char* __restrict__ image, size_t image_stride, const uint8_t* __restrict__ w,
+    const ActRows act, const uint8_t* __restrict__ w,
     void* __restrict__ y, int y_dtype, int n, int bpr, int split, int chunks, int chunk_off, int chunk_stride) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int kpad = bpr * 256;
@@ -154,7 +156,7 @@ __global__ __launch_bounds__(64 * kWaves) void iq_stream_matvec_kernel(
     const int chunk_rows = tiles_per_chunk * kRowsPerTile;
 
     // activation image, codebooks and the first chunk: all in flight together
-    dma_share<kWaves>(image + static_cast<size_t>(blockIdx.y) * image_stride, lds0, image_bytes, wave, lane);
+    if constexpr (!RAW) dma_share<kWaves>(act.image + static_cast<size_t>(blockIdx.y) * act.stride, lds0, image_bytes, wave, lane);
     FMT::template dma_tables<kWaves>(lds0 + table_off, wave, lane);
     if (tid < 4) reinterpret_cast<uint32_t*>(smem + zero_off)[tid] = 0;
     AMap<FMT::kSlots> am;
@@ -162,6 +164,8 @@ __global__ __launch_bounds__(64 * kWaves) void iq_stream_matvec_kernel(
 
     int c = blockIdx.x, buf = 0;
     dma_share<kWaves>(w + static_cast<size_t>(c) * chunk_rows * row_bytes, lds0 + chunk_off, min(chunk_rows, n - c * chunk_rows) * row_bytes, wave, lane);
+    if constexpr (RAW)                       // raw activation row: quantized once per workgroup while the first chunk is on its way
+        quantize_row_to_lds(smem, act.x, act.x_dtype, static_cast<size_t>(blockIdx.y) * act.k, act.k, kpad);
     typename FMT::Held held[NB > 0 ? NB : 1];
     bool holding = false;
     while (c < chunks) {
@@ -233,10 +237,10 @@ int stream_split(const uint8_t* w, int n, int bpr) {
     return 0;
 }
 
-template <typename FMT, int NB>
-int launch_stream_nb(const unsigned char* image, size_t image_stride, const uint8_t* w, void* y, int y_dtype,
-                     int rows, int n, int bpr, int split, hipStream_t stream) {
-    auto kern = iq_stream_matvec_kernel<FMT, NB>;
+template <typename FMT, int NB, bool RAW>
+int launch_stream_raw(const ActRows& act, const uint8_t* w, void* y, int y_dtype,
+                      int rows, int n, int bpr, int split, hipStream_t stream) {
+    auto kern = iq_stream_matvec_kernel<FMT, NB, RAW>;
     const int tiles_per_chunk = kWaves / split;
     const int chunk_bytes = tiles_per_chunk * kRowsPerTile * bpr * FMT::kBlockBytes;
     const size_t head = staged_x_bytes(bpr * 256) + 16 + FMT::kTableBytes + kWaves * kRowsPerTile * sizeof(float);
@@ -260,41 +264,47 @@ int launch_stream_nb(const unsigned char* image, size_t image_stride, const uint
         const int rounds = (chunks + resident - 1) / resident;
         grid = (chunks + rounds - 1) / rounds;
     }
-    hipLaunchKernelGGL(kern, dim3(grid, rows), dim3(64 * kWaves), smem, stream, image, image_stride, w, y, y_dtype, n, bpr, split, chunks,
+    hipLaunchKernelGGL(kern, dim3(grid, rows), dim3(64 * kWaves), smem, stream, act, w, y, y_dtype, n, bpr, split, chunks,
                        chunk_off, chunk_stride);
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 
-template <typename FMT>
-int launch_stream(const unsigned char* image, size_t image_stride, const uint8_t* w, void* y, int y_dtype,
-                  int rows, int n, int bpr, int split, hipStream_t stream) {
-    const int per_wave = (bpr + split - 1) / split;                          // block indices a wave meets
-    if constexpr (FMT::kHoldBlocks >= 2) if (per_wave <= 2) return launch_stream_nb<FMT, 2>(image, image_stride, w, y, y_dtype, rows, n, bpr, split, stream);
-    if constexpr (FMT::kHoldBlocks >= 3) if (per_wave == 3) return launch_stream_nb<FMT, 3>(image, image_stride, w, y, y_dtype, rows, n, bpr, split, stream);
-    return launch_stream_nb<FMT, 0>(image, image_stride, w, y, y_dtype, rows, n, bpr, split, stream);
+template <typename FMT, int NB>
+int launch_stream_nb(const ActRows& act, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, int split, hipStream_t stream) {
+    return act.x ? launch_stream_raw<FMT, NB, true>(act, w, y, y_dtype, rows, n, bpr, split, stream)
+                 : launch_stream_raw<FMT, NB, false>(act, w, y, y_dtype, rows, n, bpr, split, stream);
 }
 
 template <typename FMT>
-int launch_fmt(const unsigned char* image, size_t image_stride, const uint8_t* w, void* y, int y_dtype,
+int launch_stream(const ActRows& act, const uint8_t* w, void* y, int y_dtype,
+                  int rows, int n, int bpr, int split, hipStream_t stream) {
+    const int per_wave = (bpr + split - 1) / split;                          // block indices a wave meets
+    if constexpr (FMT::kHoldBlocks >= 2) if (per_wave <= 2) return launch_stream_nb<FMT, 2>(act, w, y, y_dtype, rows, n, bpr, split, stream);
+    if constexpr (FMT::kHoldBlocks >= 3) if (per_wave == 3) return launch_stream_nb<FMT, 3>(act, w, y, y_dtype, rows, n, bpr, split, stream);
+    return launch_stream_nb<FMT, 0>(act, w, y, y_dtype, rows, n, bpr, split, stream);
+}
+
+template <typename FMT>
+int launch_fmt(const ActRows& act, const uint8_t* w, void* y, int y_dtype,
                int rows, int n, int bpr, hipStream_t stream) {
     // whole tiles streamed through long-lived workgroups (the codebooks are staged once per workgroup)
     // where shape and alignment allow, else one short workgroup per tile
     if constexpr (FMT::kStreamed)
-        if (const int split = stream_split<FMT>(w, n, bpr)) return launch_stream<FMT>(image, image_stride, w, y, y_dtype, rows, n, bpr, split, stream);
-    return launch_tiles<FMT>(image, image_stride, w, y, y_dtype, rows, n, bpr, stream);
+        if (const int split = stream_split<FMT>(w, n, bpr)) return launch_stream<FMT>(act, w, y, y_dtype, rows, n, bpr, split, stream);
+    return launch_tiles<FMT>(act, w, y, y_dtype, rows, n, bpr, stream);
 }
 
 }  // namespace
 
-int iq_mfma_matvec_from_image(const unsigned char* image, size_t stride, const uint8_t* w, int type_id, void* y, int y_dtype,
+int iq_mfma_matvec_from_image(const ActRows& act, const uint8_t* w, int type_id, void* y, int y_dtype,
                               int rows, int n, int bpr, hipStream_t stream) {
     switch (type_id) {
-        case PLLM_TYPE_IQ2_XXS: return launch_fmt<IQ2XXSm>(image, stride, w, y, y_dtype, rows, n, bpr, stream);
-        case PLLM_TYPE_IQ1_M: return launch_fmt<IQ1Mm>(image, stride, w, y, y_dtype, rows, n, bpr, stream);
-        case PLLM_TYPE_IQ2_XS: return launch_fmt<IQ2XSm>(image, stride, w, y, y_dtype, rows, n, bpr, stream);
-        case PLLM_TYPE_IQ3_XXS: return launch_fmt<IQ3XXSm>(image, stride, w, y, y_dtype, rows, n, bpr, stream);
-        case PLLM_TYPE_IQ4_XS: return launch_fmt<IQ4XSm>(image, stride, w, y, y_dtype, rows, n, bpr, stream);
-        case PLLM_TYPE_Q6_K: return launch_fmt<Q6Km>(image, stride, w, y, y_dtype, rows, n, bpr, stream);
+        case PLLM_TYPE_IQ2_XXS: return launch_fmt<IQ2XXSm>(act, w, y, y_dtype, rows, n, bpr, stream);
+        case PLLM_TYPE_IQ1_M: return launch_fmt<IQ1Mm>(act, w, y, y_dtype, rows, n, bpr, stream);
+        case PLLM_TYPE_IQ2_XS: return launch_fmt<IQ2XSm>(act, w, y, y_dtype, rows, n, bpr, stream);
+        case PLLM_TYPE_IQ3_XXS: return launch_fmt<IQ3XXSm>(act, w, y, y_dtype, rows, n, bpr, stream);
+        case PLLM_TYPE_IQ4_XS: return launch_fmt<IQ4XSm>(act, w, y, y_dtype, rows, n, bpr, stream);
+        case PLLM_TYPE_Q6_K: return launch_fmt<Q6Km>(act, w, y, y_dtype, rows, n, bpr, stream);
         default: return PLLM_ERR_UNSUPPORTED;
     }
 }

@@ -3,8 +3,8 @@
 // A wave owns 16 consecutive output rows and walks their super-blocks; the W waves of a workgroup
 // split a row's super-blocks between them (wave w takes blocks w, w + W, ...) and meet in a small
 // LDS reduction.  All weight loads of a pass are issued first; while they are in flight the
-// workgroup copies the pre-quantized activation image (two int8 terms per value, written once per
-// call by act_quant.hip) from L2 into LDS.
+// workgroup brings the activation image (two int8 terms per value) into LDS: copied from the image
+// act_quant.hip wrote, or, for calls of a few rows, quantized from the raw row on the spot.
 //
 // The integer dots run on the matrix cores.  For one super-block index the wave forms
 //     C[m][n] = sum_k A[m][k] * B[k][n],     v_mfma_i32_16x16x64_i8, four of them per block,
@@ -98,10 +98,9 @@ struct Q5K {
     }
 };
 
-template <typename FMT, int ITERS>
+template <typename FMT, int ITERS, bool RAW>
 __global__ __launch_bounds__(64 * kMaxWaves) void k45_mfma_matvec_kernel(
-    const unsigned char* __restrict__ image, size_t image_stride, const uint8_t* __restrict__ w,
-    void* __restrict__ y, int y_dtype, int n, int bpr) {
+    const ActRows act, const uint8_t* __restrict__ w, void* __restrict__ y, int y_dtype, int n, int bpr) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int kpad = bpr * 256;
     const int image_bytes = static_cast<int>(staged_x_bytes(kpad));
@@ -131,6 +130,12 @@ __global__ __launch_bounds__(64 * kMaxWaves) void k45_mfma_matvec_kernel(
 
     float acc = 0.0f;
     bool staged = false;
+    if constexpr (RAW) {                     // quantize before the loads take their registers
+        quantize_row_to_lds(smem, act.x, act.x_dtype, static_cast<size_t>(blockIdx.y) * act.k, act.k, kpad);
+        if (tid < 4) reinterpret_cast<uint32_t*>(smem + zero_off)[tid] = 0;
+        __syncthreads();
+        staged = true;
+    }
     for (int b0 = wave; b0 < bpr || !staged; b0 += waves * ITERS) {
         typename FMT::Regs regs[ITERS];
 #pragma unroll
@@ -139,7 +144,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void k45_mfma_matvec_kernel(
             FMT::load(regs[it], wrow + static_cast<size_t>(b) * FMT::kBlockBytes, ks);
         }
         if (!staged) {                       // first trip of every thread of the workgroup
-            copy_to_lds(smem, image + static_cast<size_t>(blockIdx.y) * image_stride, image_bytes);
+            copy_to_lds(smem, act.image + static_cast<size_t>(blockIdx.y) * act.stride, image_bytes);
             if (tid < 4) reinterpret_cast<uint32_t*>(smem + zero_off)[tid] = 0;
             __syncthreads();
             staged = true;
@@ -185,7 +190,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void k45_mfma_matvec_kernel(
 
 // ------------------------------------------------------------------------------------------------
 template <typename KERN>
-int launch_kernel(KERN kern, const unsigned char* image, size_t image_stride, const uint8_t* w, void* y, int y_dtype,
+int launch_kernel(KERN kern, const ActRows& act, const uint8_t* w, void* y, int y_dtype,
                   int rows, int n, int bpr, int waves, hipStream_t stream) {
     const size_t smem = staged_x_bytes(bpr * 256) + 16 + static_cast<size_t>(waves) * kRowsPerWg * sizeof(float);
     if (smem > 64 * 1024) {
@@ -195,7 +200,7 @@ int launch_kernel(KERN kern, const unsigned char* image, size_t image_stride, co
             return PLLM_ERR_UNSUPPORTED;
     }
     dim3 grid((n + kRowsPerWg - 1) / kRowsPerWg, rows);
-    hipLaunchKernelGGL(kern, grid, dim3(64 * waves), smem, stream, image, image_stride, w, y, y_dtype, n, bpr);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * waves), smem, stream, act, w, y, y_dtype, n, bpr);
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 
@@ -210,14 +215,14 @@ void split_blocks(int bpr, int& waves, int& iters) {
 }
 
 template <typename FMT>
-int launch_k45(const unsigned char* image, size_t image_stride, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr,
-               hipStream_t stream) {
+int launch_k45(const ActRows& act, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream) {
     int waves, iters;
     split_blocks(bpr, waves, iters);
-#define PLLM_CASE(I) case I: return launch_kernel(k45_mfma_matvec_kernel<FMT, I>, image, image_stride, w, y, y_dtype, rows, n, bpr, waves, stream)
+#define PLLM_CASE(I) case I: return act.x ? launch_kernel(k45_mfma_matvec_kernel<FMT, I, true>, act, w, y, y_dtype, rows, n, bpr, waves, stream) \
+                                          : launch_kernel(k45_mfma_matvec_kernel<FMT, I, false>, act, w, y, y_dtype, rows, n, bpr, waves, stream)
     switch (iters) {
         PLLM_CASE(1); PLLM_CASE(2); PLLM_CASE(3); PLLM_CASE(4); PLLM_CASE(5); PLLM_CASE(6);
-        default: return launch_kernel(k45_mfma_matvec_kernel<FMT, 8>, image, image_stride, w, y, y_dtype, rows, n, bpr, waves, stream);
+        default: PLLM_CASE(8);
     }
 #undef PLLM_CASE
 }
@@ -226,11 +231,11 @@ int launch_k45(const unsigned char* image, size_t image_stride, const uint8_t* w
 
 size_t kquant_matvec_workspace_bytes(int rows, int bpr) { return act_image_256_bytes(bpr) * static_cast<size_t>(rows); }
 
-int kquant_matvec_from_image(const unsigned char* image, size_t stride, const uint8_t* w, int type_id, void* y, int y_dtype,
+int kquant_matvec_from_image(const ActRows& act, const uint8_t* w, int type_id, void* y, int y_dtype,
                              int rows, int n, int bpr, hipStream_t stream) {
     switch (type_id) {
-        case PLLM_TYPE_Q4_K: return launch_k45<Q4K>(image, stride, w, y, y_dtype, rows, n, bpr, stream);
-        case PLLM_TYPE_Q5_K: return launch_k45<Q5K>(image, stride, w, y, y_dtype, rows, n, bpr, stream);
+        case PLLM_TYPE_Q4_K: return launch_k45<Q4K>(act, w, y, y_dtype, rows, n, bpr, stream);
+        case PLLM_TYPE_Q5_K: return launch_k45<Q5K>(act, w, y, y_dtype, rows, n, bpr, stream);
         default: return PLLM_ERR_UNSUPPORTED;
     }
 }

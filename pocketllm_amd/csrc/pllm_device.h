@@ -40,17 +40,42 @@ __device__ __forceinline__ int dot4(uint32_t a, uint32_t b, int c) {
     return __builtin_amdgcn_sdot4(static_cast<int>(a), static_cast<int>(b), c, false);
 }
 
-// Sum over aligned groups of WIDTH lanes (WIDTH a power of two <= 64); every lane gets the total.
+// One step of a butterfly reduction without the LDS crossbar: the value lane (id ^ OFF) holds,
+// for a v that is already equal over aligned groups of OFF lanes (which is what step OFF of a
+// butterfly sees).  Steps 1 and 2 swap inside the quad, 4 and 8 mirror the half row / the row,
+// which pairs each group with its partner group; wider steps go through ds_bpermute.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+template <int OFF>
+__device__ __forceinline__ float butterfly_peer(float v) {
+    if constexpr (OFF == 1) return dpp_move<0xB1>(v);            // quad_perm:[1,0,3,2]
+    else if constexpr (OFF == 2) return dpp_move<0x4E>(v);       // quad_perm:[2,3,0,1]
+    else if constexpr (OFF == 4) return dpp_move<0x141>(v);      // row_half_mirror
+    else if constexpr (OFF == 8) return dpp_move<0x140>(v);      // row_mirror
+    else return __shfl_xor(v, OFF, 64);
+}
+
+// Sum / maximum over aligned groups of WIDTH lanes (WIDTH a power of two <= 64); every lane gets the result.
 template <int WIDTH>
 __device__ __forceinline__ float group_sum(float v) {
-#pragma unroll
-    for (int off = 1; off < WIDTH; off <<= 1) v += __shfl_xor(v, off, 64);
+    if constexpr (WIDTH > 1) v += butterfly_peer<1>(v);
+    if constexpr (WIDTH > 2) v += butterfly_peer<2>(v);
+    if constexpr (WIDTH > 4) v += butterfly_peer<4>(v);
+    if constexpr (WIDTH > 8) v += butterfly_peer<8>(v);
+    if constexpr (WIDTH > 16) v += butterfly_peer<16>(v);
+    if constexpr (WIDTH > 32) v += butterfly_peer<32>(v);
     return v;
 }
 template <int WIDTH>
 __device__ __forceinline__ float group_max(float v) {
-#pragma unroll
-    for (int off = 1; off < WIDTH; off <<= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    if constexpr (WIDTH > 1) v = fmaxf(v, butterfly_peer<1>(v));
+    if constexpr (WIDTH > 2) v = fmaxf(v, butterfly_peer<2>(v));
+    if constexpr (WIDTH > 4) v = fmaxf(v, butterfly_peer<4>(v));
+    if constexpr (WIDTH > 8) v = fmaxf(v, butterfly_peer<8>(v));
+    if constexpr (WIDTH > 16) v = fmaxf(v, butterfly_peer<16>(v));
+    if constexpr (WIDTH > 32) v = fmaxf(v, butterfly_peer<32>(v));
     return v;
 }
 
@@ -89,20 +114,33 @@ __device__ __forceinline__ StagedX carve_staged_x(const unsigned char* base, int
 }
 
 // Quantize four activations of one lane; the eight lanes of an aligned group share a 32-block.
+// Rounding and the int8 cast ride on one fused multiply-add each: for |t| < 2^22 the float
+// t + 1.5 * 2^23 has round-to-nearest-even(t) in its low mantissa bits, two's complement included, so
+// its low byte is the code and (sum - 1.5 * 2^23) the rounded value.  |v * inv| <= 127 and
+// |r * inv * 254| <= 127.01 by construction (inv and scale are reciprocal to 2^-22), so neither term
+// needs a clamp.  inv comes from v_rcp_f32: it only steers the rounding, the image carries `scale`.
+__device__ __forceinline__ uint32_t pack_low_bytes(uint32_t b0, uint32_t b1, uint32_t b2, uint32_t b3) {
+    const uint32_t lo = __builtin_amdgcn_perm(b1, b0, 0x0c0c0400u);
+    const uint32_t hi = __builtin_amdgcn_perm(b3, b2, 0x0c0c0400u);
+    return __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+}
 __device__ __forceinline__ void quantize4(const float v[4], uint32_t& hi, uint32_t& lo, float& scale) {
+    constexpr float kRound = 12582912.0f;                       // 1.5 * 2^23
     float am = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
     am = group_max<8>(am);
-    const float inv = am > 0.0f ? 127.0f / am : 0.0f;
+    const float inv = am > 0.0f ? 127.0f * __builtin_amdgcn_rcpf(am) : 0.0f;
+    const float inv_lo = inv * 254.0f;
     scale = am * (1.0f / 127.0f);
-    hi = 0; lo = 0;
+    uint32_t qb[4], lb[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        float q = fminf(fmaxf(rintf(v[i] * inv), -127.0f), 127.0f);
-        float r = v[i] - q * scale;
-        float l = fminf(fmaxf(rintf(r * inv * 254.0f), -127.0f), 127.0f);
-        hi |= (static_cast<uint32_t>(static_cast<int>(q)) & 0xffu) << (8 * i);
-        lo |= (static_cast<uint32_t>(static_cast<int>(l)) & 0xffu) << (8 * i);
+        const float qm = fmaf(v[i], inv, kRound);
+        const float r = fmaf(kRound - qm, scale, v[i]);         // v - q * scale
+        qb[i] = __float_as_uint(qm);
+        lb[i] = __float_as_uint(fmaf(r, inv_lo, kRound));
     }
+    hi = pack_low_bytes(qb[0], qb[1], qb[2], qb[3]);
+    lo = pack_low_bytes(lb[0], lb[1], lb[2], lb[3]);
 }
 
 // Runtime-dtype front ends (the dtype is uniform, so the switch costs one scalar branch).
@@ -120,37 +158,84 @@ __device__ __forceinline__ void store_any(void* y, int y_dtype, size_t i, float 
 
 // Workgroup-wide quantization of one activation row straight into LDS, the same image the
 // pre-pass kernel writes to memory (blockDim.x a multiple of 8, kpad a multiple of 256).  Four
-// consecutive values per lane: one 8-byte load for 16-bit inputs when the row allows it.
+// consecutive values per lane and trip: one 8-byte load for 16-bit inputs when the row allows it.
+// The loads of BATCH trips are issued together so that a row costs one or two memory round trips.
+__device__ __forceinline__ void load_row4(float v[4], const void* __restrict__ x, int x_dtype, size_t xoff, int e0, int k, bool narrow) {
+    if (narrow && e0 + 3 < k) {
+        const uint2 w = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(x) + xoff + e0);
+        if (x_dtype == PLLM_BF16) {
+            v[0] = __uint_as_float(w.x << 16); v[1] = __uint_as_float(w.x & 0xffff0000u);
+            v[2] = __uint_as_float(w.y << 16); v[3] = __uint_as_float(w.y & 0xffff0000u);
+        } else {
+            v[0] = f16_bits_to_float(w.x & 0xffffu); v[1] = f16_bits_to_float(w.x >> 16);
+            v[2] = f16_bits_to_float(w.y & 0xffffu); v[3] = f16_bits_to_float(w.y >> 16);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = (e0 + i < k) ? load_any(x, x_dtype, xoff + e0 + i) : 0.0f;
+    }
+}
+
+// One lane's four values into the image at e0 (hi, lo, and the group figures from the lanes that own them).
+__device__ __forceinline__ void quantize4_to_image(const float v[4], int e0, int8_t* hi, int8_t* lo, float2* gs, float* sum16) {
+    uint32_t qh, ql;
+    float scale;
+    quantize4(v, qh, ql, scale);
+    *reinterpret_cast<uint32_t*>(hi + e0) = qh;
+    *reinterpret_cast<uint32_t*>(lo + e0) = ql;
+    const float sum = group_sum<4>((v[0] + v[1]) + (v[2] + v[3]));
+    const float sum32 = sum + butterfly_peer<4>(sum);
+    if ((threadIdx.x & 3) == 0) sum16[e0 >> 4] = sum;
+    if ((threadIdx.x & 7) == 0) gs[e0 >> 5] = make_float2(scale * kLoInv, sum32);
+}
+
+template <int BATCH = 6>
 __device__ __forceinline__ void quantize_row_to_lds(unsigned char* lds, const void* __restrict__ x, int x_dtype, size_t xoff, int k, int kpad) {
     int8_t* hi = reinterpret_cast<int8_t*>(lds);
     int8_t* lo = hi + kpad;
     float2* gs = reinterpret_cast<float2*>(lo + kpad);
     float* sum16 = reinterpret_cast<float*>(gs + kpad / 32);
     const bool narrow = x_dtype != PLLM_F32 && ((reinterpret_cast<uintptr_t>(x) + 2 * xoff) & 7u) == 0;
-    for (int e0 = static_cast<int>(threadIdx.x) * 4; e0 < kpad; e0 += static_cast<int>(blockDim.x) * 4) {
-        float v[4];
-        if (narrow && e0 + 3 < k) {
-            const uint2 w = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(x) + xoff + e0);
-            if (x_dtype == PLLM_BF16) {
-                v[0] = __uint_as_float(w.x << 16); v[1] = __uint_as_float(w.x & 0xffff0000u);
-                v[2] = __uint_as_float(w.y << 16); v[3] = __uint_as_float(w.y & 0xffff0000u);
-            } else {
-                v[0] = f16_bits_to_float(w.x & 0xffffu); v[1] = f16_bits_to_float(w.x >> 16);
-                v[2] = f16_bits_to_float(w.y & 0xffffu); v[3] = f16_bits_to_float(w.y >> 16);
+    const int trip = static_cast<int>(blockDim.x) * 4;
+    for (int base = static_cast<int>(threadIdx.x) * 4; base < kpad; base += trip * BATCH) {
+        float v[BATCH][4];
+#pragma unroll
+        for (int j = 0; j < BATCH; ++j)
+            if (base + j * trip < kpad) load_row4(v[j], x, x_dtype, xoff, base + j * trip, k, narrow);
+#pragma unroll
+        for (int j = 0; j < BATCH; ++j)
+            if (base + j * trip < kpad) quantize4_to_image(v[j], base + j * trip, hi, lo, gs, sum16);
+    }
+}
+
+// The Q8_0 pair image (layout in matvec_q8_0.hip): per pair of 32-value blocks 80 bytes that mirror the
+// weight stream, [0,0, q0..q31, 0,0, q32..q63, 12 x 0], hi term then lo term, then float xs[2 * pairs].
+__device__ __forceinline__ void quantize4_to_pair_image(const float v[4], int e0, unsigned char* hi, unsigned char* lo, float* xs) {
+    uint32_t qh, ql;
+    float scale;
+    quantize4(v, qh, ql, scale);
+    const int b = e0 >> 5;
+    const int j = (e0 & 31) >> 2;
+    const int off = (b >> 1) * 80 + ((b & 1) ? 36 : 2) + 4 * j;   // 2-byte aligned
+    *reinterpret_cast<uint16_t*>(hi + off) = static_cast<uint16_t>(qh);
+    *reinterpret_cast<uint16_t*>(hi + off + 2) = static_cast<uint16_t>(qh >> 16);
+    *reinterpret_cast<uint16_t*>(lo + off) = static_cast<uint16_t>(ql);
+    *reinterpret_cast<uint16_t*>(lo + off + 2) = static_cast<uint16_t>(ql >> 16);
+    if (j == 0) {
+        const int p0 = (b >> 1) * 80;
+        if (b & 1) {
+            *reinterpret_cast<uint16_t*>(hi + p0 + 34) = 0;
+            *reinterpret_cast<uint16_t*>(lo + p0 + 34) = 0;
+#pragma unroll
+            for (int z = 68; z < 80; z += 4) {
+                *reinterpret_cast<uint32_t*>(hi + p0 + z) = 0;
+                *reinterpret_cast<uint32_t*>(lo + p0 + z) = 0;
             }
         } else {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) v[i] = (e0 + i < k) ? load_any(x, x_dtype, xoff + e0 + i) : 0.0f;
+            *reinterpret_cast<uint16_t*>(hi + p0) = 0;
+            *reinterpret_cast<uint16_t*>(lo + p0) = 0;
         }
-        uint32_t qh, ql;
-        float scale;
-        quantize4(v, qh, ql, scale);
-        *reinterpret_cast<uint32_t*>(hi + e0) = qh;
-        *reinterpret_cast<uint32_t*>(lo + e0) = ql;
-        const float sum = group_sum<4>((v[0] + v[1]) + (v[2] + v[3]));
-        const float sum32 = sum + __shfl_xor(sum, 4, 64);
-        if ((threadIdx.x & 3) == 0) sum16[e0 >> 4] = sum;
-        if ((threadIdx.x & 7) == 0) gs[e0 >> 5] = make_float2(scale * kLoInv, sum32);
+        xs[b] = scale;
     }
 }
 

@@ -19,14 +19,28 @@ size_t q8_0_matvec_workspace_bytes(int rows, int bpr);
 int q8_0_matvec(const void* x, int x_dtype, const uint8_t* w, void* y, int y_dtype,
                 int rows, int k, int n, int bpr, void* workspace, size_t workspace_bytes, hipStream_t stream);
 
+// Where a super-block matvec kernel finds its activation rows.  x == nullptr: images written by
+// act_image_256, `stride` bytes apart.  Otherwise the raw rows ([rows, k] of x_dtype): every
+// workgroup quantizes its row into LDS itself (the same image, bit for bit), which saves the
+// pre-pass launch when there are only a few rows.
+struct ActRows {
+    const unsigned char* image;
+    size_t stride;
+    const void* x;
+    int x_dtype;
+    int k;
+};
+inline ActRows act_rows_from_image(const unsigned char* image, size_t stride) { return ActRows{image, stride, nullptr, 0, 0}; }
+inline ActRows act_rows_raw(const void* x, int x_dtype, int k) { return ActRows{nullptr, 0, x, x_dtype, k}; }
+
 // 256-weight super-block types: one activation image (act_image_256) serves any number of matvecs.
 // Q4_K / Q5_K run in matvec_kquant.hip, IQ2_XXS / IQ1_M in matvec_iq_mfma.hip (matrix cores),
 // Q2_K and the routed forms in matvec_dot4.hip (v_dot4).
-int kquant_matvec_from_image(const unsigned char* image, size_t stride, const uint8_t* w, int type_id, void* y, int y_dtype,
+int kquant_matvec_from_image(const ActRows& act, const uint8_t* w, int type_id, void* y, int y_dtype,
                              int rows, int n, int bpr, hipStream_t stream);
-int dot4_matvec_from_image(const unsigned char* image, size_t stride, const uint8_t* w, int type_id, void* y, int y_dtype,
+int dot4_matvec_from_image(const ActRows& act, const uint8_t* w, int type_id, void* y, int y_dtype,
                            int rows, int n, int bpr, hipStream_t stream);
-int iq_mfma_matvec_from_image(const unsigned char* image, size_t stride, const uint8_t* w, int type_id, void* y, int y_dtype,
+int iq_mfma_matvec_from_image(const ActRows& act, const uint8_t* w, int type_id, void* y, int y_dtype,
                               int rows, int n, int bpr, hipStream_t stream);
 
 // routed form: activation row r (image r, output row r) meets the matrix at w + y_expert[r] * expert_stride

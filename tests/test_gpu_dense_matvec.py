@@ -246,3 +246,57 @@ def test_codebook_grid_argument_is_validated(mod):
     with pytest.raises(RuntimeError, match="cannot mix iq1_m with iq2_xs/iq3_xxs"):
         mod.gguf_quant_gemm_pair_forward(x, torch.zeros(4, 1, 56, dtype=torch.uint8, device=dev), 256, 2,
                                          torch.zeros(4, 1, 74, dtype=torch.uint8, device=dev), 256, 5, codebooks.get_iq1_grid_tensor().to(dev))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_activation_image_holds_two_int8_terms_per_value(mod, dtype):
+    """The image the matvec kernels read: per 32 values x ~= xs * (hi + lo / 254) with xs = amax / 127, plus exact-order float sums
+    of every 16 and 32 values.  Checked against the definition (not against another quantizer): reconstruction error below
+    amax / 127 / 254 * 0.51 per value, scale and sums as stated, padding zero."""
+    rng = np.random.default_rng(77)
+    dev = torch.device("cuda:0")
+    k, bpr = 1000, 4
+    x_np = rng.standard_normal((3, k)).astype(np.float32) * np.array([[1.0], [1e-3], [300.0]], dtype=np.float32)
+    x_np[0, 64:96] = 0.0                                       # an all-zero group
+    x = torch.from_numpy(x_np).to(dev).to(dtype)
+    xf = x.float().cpu().numpy()
+    image = mod.quantize_activations(x, bpr).cpu().numpy()
+    kpad = bpr * 256
+    xp = np.zeros((3, kpad), dtype=np.float32)
+    xp[:, :k] = xf
+    hi = image[:, :kpad].view(np.int8).astype(np.float32)
+    lo = image[:, kpad:2 * kpad].view(np.int8).astype(np.float32)
+    gs = image[:, 2 * kpad:2 * kpad + kpad // 32 * 8].copy().view(np.float32).reshape(3, kpad // 32, 2)
+    sum16 = image[:, 2 * kpad + kpad // 32 * 8:2 * kpad + kpad // 32 * 8 + kpad // 16 * 4].copy().view(np.float32)
+    amax = np.abs(xp).reshape(3, -1, 32).max(axis=2)
+    np.testing.assert_allclose(gs[..., 0] * 254.0, amax / 127.0, rtol=3e-7)
+    recon = (gs[..., 0:1] * (hi.reshape(3, -1, 32) * 254.0 + lo.reshape(3, -1, 32))).reshape(3, kpad)
+    assert np.all(np.abs(recon - xp) <= np.repeat(amax, 32, axis=1) / 127.0 / 254.0 * 0.51 + 1e-30)
+    assert np.all(np.abs(hi) <= 127) and np.all(np.abs(lo) <= 127)
+    np.testing.assert_allclose(sum16, xp.reshape(3, -1, 16).sum(axis=2), rtol=0, atol=np.abs(xp).max() * 4e-6)
+    np.testing.assert_allclose(gs[..., 1], xp.reshape(3, -1, 32).sum(axis=2), rtol=0, atol=np.abs(xp).max() * 8e-6)
+    assert not hi[:, k:].any() and not lo[:, k:].any()
+
+
+@pytest.mark.parametrize("type_name", ["q4_k", "q5_k", "q2_k", "q6_k", "iq4_xs", "iq2_xxs", "iq1_m", "iq2_xs", "iq3_xxs"])
+def test_few_row_calls_equal_the_prequantized_path(mod, type_name):
+    """Calls of a few rows may quantize the activations inside the matvec kernel; the result is the same bits as quantizing ahead."""
+    rng = np.random.default_rng(78)
+    dev = torch.device("cuda:0")
+    tid = O.TYPE_IDS[type_name]
+    for n, k, rows in ((48, 5120, 1), (130, 1002, 3), (16, 17408, 2), (20, 256, 4)):
+        bpr = (k + 255) // 256
+        if type_name in ("q4_k", "q5_k", "q2_k"):
+            enc = {"q4_k": C.quantize_q4_k, "q5_k": C.quantize_q5_k, "q2_k": C.quantize_q2_k}[type_name]
+            blocks = enc(np.pad(_weights(rng, n, k), ((0, 0), (0, bpr * 256 - k))))
+        elif type_name in ("iq2_xxs", "iq1_m"):
+            blocks = (C.random_iq2_xxs if type_name == "iq2_xxs" else C.random_iq1_m)(rng, n, bpr)
+        else:
+            blocks = C.random_blocks(rng, type_name, n, bpr)
+        blocks = torch.from_numpy(blocks).to(dev)
+        for dt in (torch.bfloat16, torch.float32, torch.float16):
+            x = torch.from_numpy(rng.standard_normal((rows, k)).astype(np.float32)).to(dev).to(dt)
+            print(f"case few-row {type_name} n={n} k={k} rows={rows} {dt}", flush=True)
+            y = mod.gguf_quant_gemm_forward(x, blocks, k, tid, codebooks.grid_tensor_for_type(tid).to(dev), out_dtype=torch.float32)
+            y_pre = mod.gguf_quant_gemm_prequantized(mod.quantize_activations(x, bpr), blocks, tid, out_dtype=torch.float32)
+            assert torch.equal(y, y_pre)
