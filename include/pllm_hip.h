@@ -153,6 +153,37 @@ int pllm_fp8_gemm(const uint8_t* a, const float* a_scale, const uint8_t* weight,
                   int64_t rows, int64_t k, int64_t n, void* stream);
 
 /*
+ * FP8 E4M3 weights with IEEE fp16 scale bits per 128 x 128 block and explicit pitches: the raw-pointer
+ * operators of the reference's C++ engine (cpp_engine/include/qwen_cuda_ops.hpp), which take device
+ * pointers, ints and an opaque stream and return false on bad arguments; these return a status.
+ * In the reference's naming `rows` counts OUTPUT rows (N) and `cols` is the inner dimension (K):
+ *   weight [rows, weight_stride >= cols] codes; scale_fp16 [ceil(rows / 128), scale_stride >= ceil(cols / 128)];
+ *   x [batch, x_stride >= cols], y [batch, y_stride >= rows]; float32 accumulation, any x / y dtype code.
+ * pllm_fp8_fp16scale_matvec: y[r] = sum_c x[c] * f32(code[r, c]) * f32(scale[r / 128, c / 128])
+ *   replaces qwen_fp8_e4m3_fp16scale_matvec_cuda and ..._matvec_f16_cuda (qwen_cuda_ops.hpp:59-69, 102-111;
+ *   cpp_engine/cuda/qwen_fp8_ops.cu:959-1007).
+ * pllm_fp8_fp16scale_swiglu_matvec: y[b, r] = silu(gate . x_b) * (up . x_b), neither projection written out
+ *   replaces ..._swiglu_matvec_cuda, ..._swiglu_matvec_f16_cuda (batch 1) and ..._swiglu_small_batch_f16_cuda
+ *   (qwen_cuda_ops.hpp:72-83, 113-140; qwen_fp8_ops.cu:1009-1033).
+ * pllm_fp8_fp16scale_matmul_rows: the matvec over `batch` activation rows
+ *   replaces ..._matmul_rows_cuda, ..._matmul_rows_f16_cuda and ..._matmul_simt_cuda (qwen_cuda_ops.hpp:85-97,
+ *   142-170; qwen_fp8_ops.cu:1035-1124).  16 rows or more of fp16 / bf16 activations with dense pitches and cols a
+ *   multiple of 256 run on the MFMA tile kernel (fp16 operands, float32 accumulation) when `workspace` holds pllm_fp8_fp16scale_matmul_rows_workspace_bytes bytes (256-byte
+ *   aligned, private to the call until its kernels have run); otherwise, or with a null workspace, every
+ *   activation row takes the matvec kernel.
+ */
+int pllm_fp8_fp16scale_matvec(const void* x, int x_dtype, const uint8_t* weight, const uint16_t* scale_fp16, void* y, int y_dtype,
+                              int64_t rows, int64_t cols, int64_t weight_stride, int64_t scale_stride, void* stream);
+int pllm_fp8_fp16scale_swiglu_matvec(const void* x, int x_dtype, const uint8_t* gate_weight, const uint16_t* gate_scale_fp16,
+                                     const uint8_t* up_weight, const uint16_t* up_scale_fp16, void* y, int y_dtype,
+                                     int64_t batch, int64_t rows, int64_t cols, int64_t x_stride, int64_t y_stride,
+                                     int64_t weight_stride, int64_t scale_stride, void* stream);
+int pllm_fp8_fp16scale_matmul_rows(const void* x, int x_dtype, const uint8_t* weight, const uint16_t* scale_fp16, void* y, int y_dtype,
+                                   int64_t batch, int64_t rows, int64_t cols, int64_t x_stride, int64_t y_stride,
+                                   int64_t weight_stride, int64_t scale_stride, void* workspace, size_t workspace_bytes, void* stream);
+size_t pllm_fp8_fp16scale_matmul_rows_workspace_bytes(int64_t batch, int64_t rows, int64_t cols);
+
+/*
  * Fused routed-expert matmul over raw super-blocks (types Q2_K, IQ2_XXS, IQ1_M; gate/up share a type,
  * the down projection may use another, so IQ2_XXS gate/up with IQ1_M down needs no special case):
  *     y[t] = sum over routes r of token t:  W2_e ( silu(min(W1_e x_t, L)) * clamp(W3_e x_t, +-L) * w_r )

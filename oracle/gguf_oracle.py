@@ -389,6 +389,27 @@ def dequant_fp8_block(weight: np.ndarray, scale: np.ndarray, block: int = 128) -
     return fp8_e4m3_decode(weight) * s
 
 
+def fp8_fp16scale_matmul(x: np.ndarray, weight: np.ndarray, scale_bits: np.ndarray, rows: int, cols: int,
+                          weight_stride: int, scale_stride: int) -> np.ndarray:
+    """y[b, r] = sum_c x[b, c] * f32(code[r, c]) * f32(f16 scale[r // 128, c // 128]) in float64: the expectation the
+    reference's own test builds for its C++ engine operators (cpp_engine/tests/test_qwen_fp8_online.cpp:159-171), with
+    their pitches: weight is a flat byte array read at r * weight_stride + c, scale_bits a flat uint16 array read at
+    (r // 128) * scale_stride + c // 128.  Pinned by: the decode (torch's cast, all codes), the fp16 bits (numpy's
+    float16 view), the indexing (brute-force loop on a small unaligned case in tests/test_oracle_pinning.py)."""
+    w = np.lib.stride_tricks.as_strided(weight, shape=(rows, cols), strides=(weight_stride, 1))
+    tr, tc = (rows + 127) // 128, (cols + 127) // 128
+    sc = np.lib.stride_tricks.as_strided(scale_bits, shape=(tr, tc), strides=(2 * scale_stride, 2)).view(np.float16).astype(np.float64)
+    wf = fp8_e4m3_decode(np.ascontiguousarray(w)).astype(np.float64) * np.repeat(np.repeat(sc, 128, axis=0)[:rows], 128, axis=1)[:, :cols]
+    return x.astype(np.float64) @ wf.T
+
+
+def silu_mul(gate: np.ndarray, up: np.ndarray) -> np.ndarray:
+    """silu(g) * u, the epilogue of the fused gate/up matvec (cpp_engine/cuda/qwen_fp8_ops.cu:41-43, 815-896)."""
+    g = gate.astype(np.float64)
+    with np.errstate(over="ignore"):                         # exp(-g) = inf for very negative g: silu -> -0, as in float arithmetic
+        return g / (1.0 + np.exp(-g)) * up.astype(np.float64)
+
+
 def fp8_e4m3_encode_rne(x: np.ndarray) -> np.ndarray:
     """float32 -> nearest E4M3FN code, ties to even, saturating at +-448 (test helper)."""
     table = fp8_e4m3_decode(np.arange(256, dtype=np.uint8))

@@ -211,4 +211,75 @@ int pllm_fp8_block_gemm(const void* x, int x_dtype, const uint8_t* weight, const
                             static_cast<int>(n), static_cast<hipStream_t>(stream));
 }
 
+// ---- FP8 with fp16 scales: the raw-pointer operators of the reference's C++ engine -----------------------------------
+
+static bool fp16scale_args_ok(const void* x, const void* w, const void* scale, const void* y, int64_t rows, int64_t cols,
+                              int64_t weight_stride, int64_t scale_stride) {
+    // cpp_engine/cuda/qwen_fp8_ops.cu:951-955 (valid_common) plus the pitch check every entry point adds
+    return x && w && scale && y && rows > 0 && cols > 0 && fits_int(rows) && fits_int(cols) && fits_int(scale_stride) &&
+           scale_stride >= (cols + 127) / 128 && weight_stride >= cols;
+}
+
+int pllm_fp8_fp16scale_matvec(const void* x, int x_dtype, const uint8_t* weight, const uint16_t* scale_fp16, void* y, int y_dtype,
+                              int64_t rows, int64_t cols, int64_t weight_stride, int64_t scale_stride, void* stream) {
+    if (!dtype_ok(x_dtype) || !dtype_ok(y_dtype) || !fp16scale_args_ok(x, weight, scale_fp16, y, rows, cols, weight_stride, scale_stride))
+        return PLLM_ERR_INVALID_ARGUMENT;
+    return pllm::fp8_f16scale_matvec(x, x_dtype, static_cast<size_t>(cols), weight, scale_fp16, static_cast<size_t>(weight_stride),
+                                     static_cast<int>(scale_stride), y, y_dtype, static_cast<size_t>(rows), 1, static_cast<int>(cols),
+                                     static_cast<int>(rows), static_cast<hipStream_t>(stream));
+}
+
+int pllm_fp8_fp16scale_swiglu_matvec(const void* x, int x_dtype, const uint8_t* gate_weight, const uint16_t* gate_scale_fp16,
+                                     const uint8_t* up_weight, const uint16_t* up_scale_fp16, void* y, int y_dtype,
+                                     int64_t batch, int64_t rows, int64_t cols, int64_t x_stride, int64_t y_stride,
+                                     int64_t weight_stride, int64_t scale_stride, void* stream) {
+    if (!dtype_ok(x_dtype) || !dtype_ok(y_dtype) || !up_weight || !up_scale_fp16 ||
+        !fp16scale_args_ok(x, gate_weight, gate_scale_fp16, y, rows, cols, weight_stride, scale_stride))
+        return PLLM_ERR_INVALID_ARGUMENT;
+    if (batch <= 0 || x_stride < cols || y_stride < rows) return PLLM_ERR_INVALID_ARGUMENT;
+    if (batch > 65535) return PLLM_ERR_UNSUPPORTED;
+    return pllm::fp8_f16scale_swiglu_matvec(x, x_dtype, static_cast<size_t>(x_stride), gate_weight, gate_scale_fp16, up_weight, up_scale_fp16,
+                                            static_cast<size_t>(weight_stride), static_cast<int>(scale_stride), y, y_dtype,
+                                            static_cast<size_t>(y_stride), static_cast<int>(batch), static_cast<int>(cols),
+                                            static_cast<int>(rows), static_cast<hipStream_t>(stream));
+}
+
+// Many rows of 16-bit activations with dense pitches and 256-aligned cols run on the tile kernel (float32 scale table in
+// the workspace).  float32 activations stay on the float32 matvec, row by row: the tile kernel rounds its operands to fp16,
+// which is inside the bound the reference sets for its fp16-storage variants (2e-2) but not the 2e-4 of its float32 ones.
+static bool fp16scale_uses_gemm(int x_dtype, int64_t batch, int64_t rows, int64_t cols, int64_t x_stride, int64_t y_stride, int64_t weight_stride) {
+    return x_dtype != PLLM_F32 && fp8_uses_gemm(batch, cols) && x_stride == cols && y_stride == rows && weight_stride == cols;
+}
+
+static size_t fp16scale_table_bytes(int64_t rows, int64_t cols) {
+    return (static_cast<size_t>((rows + 127) / 128) * static_cast<size_t>((cols + 127) / 128) * sizeof(float) + 255) & ~static_cast<size_t>(255);
+}
+
+size_t pllm_fp8_fp16scale_matmul_rows_workspace_bytes(int64_t batch, int64_t rows, int64_t cols) {
+    if (!fits_int(batch) || !fits_int(rows) || !fits_int(cols) || !fp8_uses_gemm(batch, cols)) return 0;
+    return fp16scale_table_bytes(rows, cols) + pllm::gemm_f16_workspace_bytes(static_cast<int>(batch), static_cast<int>(rows), static_cast<int>(cols / 256));
+}
+
+int pllm_fp8_fp16scale_matmul_rows(const void* x, int x_dtype, const uint8_t* weight, const uint16_t* scale_fp16, void* y, int y_dtype,
+                                   int64_t batch, int64_t rows, int64_t cols, int64_t x_stride, int64_t y_stride,
+                                   int64_t weight_stride, int64_t scale_stride, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!dtype_ok(x_dtype) || !dtype_ok(y_dtype) || !fp16scale_args_ok(x, weight, scale_fp16, y, rows, cols, weight_stride, scale_stride))
+        return PLLM_ERR_INVALID_ARGUMENT;
+    if (batch <= 0 || !fits_int(batch) || x_stride < cols || y_stride < rows) return PLLM_ERR_INVALID_ARGUMENT;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (fp16scale_uses_gemm(x_dtype, batch, rows, cols, x_stride, y_stride, weight_stride) && workspace &&
+        workspace_bytes >= pllm_fp8_fp16scale_matmul_rows_workspace_bytes(batch, rows, cols)) {
+        float* table = static_cast<float*>(workspace);
+        const size_t table_bytes = fp16scale_table_bytes(rows, cols);
+        const int st = pllm::fp8_f16scale_table_to_f32(scale_fp16, static_cast<int>(scale_stride), table, static_cast<int>(rows), static_cast<int>(cols), s);
+        if (st != PLLM_OK) return st;
+        return pllm::gemm_f16_fp8(x, x_dtype, weight, table, y, y_dtype, static_cast<int>(batch), static_cast<int>(cols), static_cast<int>(rows),
+                                  static_cast<char*>(workspace) + table_bytes, workspace_bytes - table_bytes, s);
+    }
+    if (batch > 65535) return PLLM_ERR_UNSUPPORTED;
+    return pllm::fp8_f16scale_matvec(x, x_dtype, static_cast<size_t>(x_stride), weight, scale_fp16, static_cast<size_t>(weight_stride),
+                                     static_cast<int>(scale_stride), y, y_dtype, static_cast<size_t>(y_stride), static_cast<int>(batch),
+                                     static_cast<int>(cols), static_cast<int>(rows), s);
+}
+
 }  // extern "C"

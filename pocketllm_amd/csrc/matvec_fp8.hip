@@ -1,4 +1,6 @@
-// Decode matvec over FP8 E4M3 (OCP) weights with float32 scales per 128 x 128 block.
+// Decode matvec over FP8 E4M3 (OCP) weights with one scale per 128 x 128 block (float32, or IEEE
+// fp16 bits with a row pitch for the scale table, the form the reference's C++ engine uploads), and
+// the fused gate/up form y = silu(G x) * (U x) of the same kernels.
 //
 // One byte per weight, rows contiguous: a wave reads a row as a stream, lane l taking 16 bytes at
 // offset 16 * (l + 64 * it) with one global_load_dwordx4, two rows in flight per wave.  The
@@ -19,6 +21,29 @@ constexpr int kRowsPerWave = 2;
 
 typedef float v2f __attribute__((ext_vector_type(2)));
 
+// One weight matrix as the kernels see it: codes with a row pitch, scale table with a row pitch.
+struct Fp8Mat {
+    const uint8_t* w;
+    const void* scale;      // float32 or fp16 bits, chosen by the kernels' F16S parameter
+    size_t wstride;         // bytes between rows of codes
+    int sstride;            // entries between rows of the scale table
+};
+
+template <bool F16S>
+__device__ __forceinline__ float scale_at(const void* __restrict__ scale, size_t i) {
+    if constexpr (F16S) return f16_bits_to_float(static_cast<const uint16_t*>(scale)[i]);
+    else return static_cast<const float*>(scale)[i];
+}
+
+__device__ __forceinline__ float silu(float v) { return v / (1.0f + __expf(-v)); }
+
+// Two register slots per wave: two consecutive rows of one matrix, or (SWIGLU) the same row of the
+// gate and of the up matrix.
+template <bool SWIGLU>
+__device__ __forceinline__ const Fp8Mat& slot_mat(const Fp8Mat& a, const Fp8Mat& b, int q) { return (SWIGLU && q == 1) ? b : a; }
+template <bool SWIGLU>
+__device__ __forceinline__ int slot_row(int row0, int q, int n) { return min(SWIGLU ? row0 : row0 + q, n - 1); }
+
 __device__ __forceinline__ float chunk_dot(const uint4& w, const float* xp) {
     const float4 x0 = *reinterpret_cast<const float4*>(xp);
     const float4 x1 = *reinterpret_cast<const float4*>(xp + 4);
@@ -37,19 +62,19 @@ __device__ __forceinline__ float chunk_dot(const uint4& w, const float* xp) {
     return s;
 }
 
-// k a multiple of 16, weight base 16-byte aligned
-template <int ITERS>
+// k a multiple of 16, weight base and row pitch 16-byte aligned
+template <int ITERS, bool F16S, bool SWIGLU>
 __global__ __launch_bounds__(kThreads) void fp8_stream_matvec_kernel(
-    const void* __restrict__ x, int x_dtype, const uint8_t* __restrict__ w, const float* __restrict__ scale,
-    void* __restrict__ y, int y_dtype, int k, int n, int kb) {
+    const void* __restrict__ x, int x_dtype, size_t x_stride, const Fp8Mat ma, const Fp8Mat mb,
+    void* __restrict__ y, int y_dtype, size_t y_stride, int k, int n) {
     extern __shared__ __align__(16) unsigned char smem[];
     float* xs = reinterpret_cast<float*>(smem);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int chunks = k >> 4;
-    const int row0 = (blockIdx.x * kWaves + wave) * kRowsPerWave;
-    const size_t xoff = static_cast<size_t>(blockIdx.y) * k;
+    const int row0 = (blockIdx.x * kWaves + wave) * (SWIGLU ? 1 : kRowsPerWave);
+    const size_t xoff = static_cast<size_t>(blockIdx.y) * x_stride;
 
     float acc[kRowsPerWave];
 #pragma unroll
@@ -60,7 +85,7 @@ __global__ __launch_bounds__(kThreads) void fp8_stream_matvec_kernel(
         uint4 regs[kRowsPerWave][ITERS];
 #pragma unroll
         for (int r = 0; r < kRowsPerWave; ++r) {
-            const uint8_t* wrow = w + static_cast<size_t>(min(row0 + r, n - 1)) * k;
+            const uint8_t* wrow = slot_mat<SWIGLU>(ma, mb, r).w + static_cast<size_t>(slot_row<SWIGLU>(row0, r, n)) * slot_mat<SWIGLU>(ma, mb, r).wstride;
 #pragma unroll
             for (int it = 0; it < ITERS; ++it) {
                 const int c = min(c0 + it * 64 + lane, chunks - 1);
@@ -80,15 +105,22 @@ __global__ __launch_bounds__(kThreads) void fp8_stream_matvec_kernel(
 #pragma unroll
             for (int r = 0; r < kRowsPerWave; ++r) {
                 const float s = chunk_dot(regs[r][it], xs + 16 * cc);
-                const float sc = scale[(min(row0 + r, n - 1) >> 7) * kb + (cc >> 3)];
+                const Fp8Mat& m = slot_mat<SWIGLU>(ma, mb, r);
+                const float sc = scale_at<F16S>(m.scale, static_cast<size_t>(slot_row<SWIGLU>(row0, r, n) >> 7) * m.sstride + (cc >> 3));
                 acc[r] += ok ? s * sc : 0.0f;
             }
         }
     }
+    float total[kRowsPerWave];
 #pragma unroll
-    for (int r = 0; r < kRowsPerWave; ++r) {
-        const float total = group_sum<64>(acc[r]);
-        if (lane == 0 && row0 + r < n) store_any(y, y_dtype, static_cast<size_t>(blockIdx.y) * n + row0 + r, total);
+    for (int r = 0; r < kRowsPerWave; ++r) total[r] = group_sum<64>(acc[r]);
+    const size_t yoff = static_cast<size_t>(blockIdx.y) * y_stride;
+    if constexpr (SWIGLU) {
+        if (lane == 0 && row0 < n) store_any(y, y_dtype, yoff + row0, silu(total[0]) * total[1]);
+    } else {
+#pragma unroll
+        for (int r = 0; r < kRowsPerWave; ++r)
+            if (lane == 0 && row0 + r < n) store_any(y, y_dtype, yoff + row0 + r, total[r]);
     }
 }
 
@@ -96,19 +128,19 @@ __global__ __launch_bounds__(kThreads) void fp8_stream_matvec_kernel(
 // row once and then walks groups of 8 weight rows (two per wave), always holding the loads of its
 // next group in a second register set while it multiplies the current one.  Rows of at most
 // 64 * 16 * ITERS bytes.
-template <int ITERS>
-__device__ __forceinline__ void fp8_fetch_group(uint4 (&r)[kRowsPerWave][ITERS], const uint8_t* __restrict__ w, int row0, int n, int k, int chunks, int lane) {
+template <int ITERS, bool SWIGLU>
+__device__ __forceinline__ void fp8_fetch_group(uint4 (&r)[kRowsPerWave][ITERS], const Fp8Mat& ma, const Fp8Mat& mb, int row0, int n, int chunks, int lane) {
 #pragma unroll
     for (int q = 0; q < kRowsPerWave; ++q) {
-        const uint8_t* wrow = w + static_cast<size_t>(min(row0 + q, n - 1)) * k;
+        const uint8_t* wrow = slot_mat<SWIGLU>(ma, mb, q).w + static_cast<size_t>(slot_row<SWIGLU>(row0, q, n)) * slot_mat<SWIGLU>(ma, mb, q).wstride;
 #pragma unroll
         for (int it = 0; it < ITERS; ++it) r[q][it] = *reinterpret_cast<const uint4*>(wrow + 16 * min(it * 64 + lane, chunks - 1));
     }
 }
 
-template <int ITERS>
-__device__ __forceinline__ void fp8_finish_group(const uint4 (&r)[kRowsPerWave][ITERS], const float* xs, const float* __restrict__ scale,
-                                                 void* __restrict__ y, int y_dtype, size_t yoff, int row0, int n, int kb, int chunks, int lane) {
+template <int ITERS, bool F16S, bool SWIGLU>
+__device__ __forceinline__ void fp8_finish_group(const uint4 (&r)[kRowsPerWave][ITERS], const float* xs, const Fp8Mat& ma, const Fp8Mat& mb,
+                                                 void* __restrict__ y, int y_dtype, size_t yoff, int row0, int n, int chunks, int lane) {
     float acc[kRowsPerWave];
 #pragma unroll
     for (int q = 0; q < kRowsPerWave; ++q) acc[q] = 0.0f;
@@ -120,44 +152,51 @@ __device__ __forceinline__ void fp8_finish_group(const uint4 (&r)[kRowsPerWave][
 #pragma unroll
         for (int q = 0; q < kRowsPerWave; ++q) {
             const float d = chunk_dot(r[q][it], xs + 16 * cc);
-            const float sc = scale[(min(row0 + q, n - 1) >> 7) * kb + (cc >> 3)];
+            const Fp8Mat& m = slot_mat<SWIGLU>(ma, mb, q);
+            const float sc = scale_at<F16S>(m.scale, static_cast<size_t>(slot_row<SWIGLU>(row0, q, n) >> 7) * m.sstride + (cc >> 3));
             acc[q] += ok ? d * sc : 0.0f;
         }
     }
+    float total[kRowsPerWave];
 #pragma unroll
-    for (int q = 0; q < kRowsPerWave; ++q) {
-        const float total = group_sum<64>(acc[q]);
-        if (lane == 0 && row0 + q < n) store_any(y, y_dtype, yoff + row0 + q, total);
+    for (int q = 0; q < kRowsPerWave; ++q) total[q] = group_sum<64>(acc[q]);
+    if constexpr (SWIGLU) {
+        if (lane == 0 && row0 < n) store_any(y, y_dtype, yoff + row0, silu(total[0]) * total[1]);
+    } else {
+#pragma unroll
+        for (int q = 0; q < kRowsPerWave; ++q)
+            if (lane == 0 && row0 + q < n) store_any(y, y_dtype, yoff + row0 + q, total[q]);
     }
 }
 
-template <int ITERS>
+template <int ITERS, bool F16S, bool SWIGLU>
 __global__ __launch_bounds__(kThreads) void fp8_persistent_matvec_kernel(
-    const void* __restrict__ x, int x_dtype, const uint8_t* __restrict__ w, const float* __restrict__ scale,
-    void* __restrict__ y, int y_dtype, int k, int n, int kb, int groups) {
+    const void* __restrict__ x, int x_dtype, size_t x_stride, const Fp8Mat ma, const Fp8Mat mb,
+    void* __restrict__ y, int y_dtype, size_t y_stride, int k, int n, int groups) {
     extern __shared__ __align__(16) unsigned char smem[];
     float* xs = reinterpret_cast<float*>(smem);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int chunks = k >> 4;
-    const size_t xoff = static_cast<size_t>(blockIdx.y) * k;
-    const size_t yoff = static_cast<size_t>(blockIdx.y) * n;
-    const int rows_per_group = kWaves * kRowsPerWave, wave_row = wave * kRowsPerWave;
+    const size_t xoff = static_cast<size_t>(blockIdx.y) * x_stride;
+    const size_t yoff = static_cast<size_t>(blockIdx.y) * y_stride;
+    constexpr int per_wave = SWIGLU ? 1 : kRowsPerWave;
+    const int rows_per_group = kWaves * per_wave, wave_row = wave * per_wave;
 
     uint4 a[kRowsPerWave][ITERS], b[kRowsPerWave][ITERS];
     int g = blockIdx.x;
     const int step = gridDim.x;
-    fp8_fetch_group<ITERS>(a, w, g * rows_per_group + wave_row, n, k, chunks, lane);
+    fp8_fetch_group<ITERS, SWIGLU>(a, ma, mb, g * rows_per_group + wave_row, n, chunks, lane);
     for (int i = tid; i < k; i += kThreads) xs[i] = load_any(x, x_dtype, xoff + i);
     __syncthreads();
     while (g < groups) {
-        if (g + step < groups) fp8_fetch_group<ITERS>(b, w, (g + step) * rows_per_group + wave_row, n, k, chunks, lane);
-        fp8_finish_group<ITERS>(a, xs, scale, y, y_dtype, yoff, g * rows_per_group + wave_row, n, kb, chunks, lane);
+        if (g + step < groups) fp8_fetch_group<ITERS, SWIGLU>(b, ma, mb, (g + step) * rows_per_group + wave_row, n, chunks, lane);
+        fp8_finish_group<ITERS, F16S, SWIGLU>(a, xs, ma, mb, y, y_dtype, yoff, g * rows_per_group + wave_row, n, chunks, lane);
         g += step;
         if (g >= groups) break;
-        if (g + step < groups) fp8_fetch_group<ITERS>(a, w, (g + step) * rows_per_group + wave_row, n, k, chunks, lane);
-        fp8_finish_group<ITERS>(b, xs, scale, y, y_dtype, yoff, g * rows_per_group + wave_row, n, kb, chunks, lane);
+        if (g + step < groups) fp8_fetch_group<ITERS, SWIGLU>(a, ma, mb, (g + step) * rows_per_group + wave_row, n, chunks, lane);
+        fp8_finish_group<ITERS, F16S, SWIGLU>(b, xs, ma, mb, y, y_dtype, yoff, g * rows_per_group + wave_row, n, chunks, lane);
         g += step;
     }
 }
@@ -172,35 +211,81 @@ __device__ __forceinline__ float fp8_to_float_sw(uint32_t c) {
 }
 
 // any k, any alignment: one wave per row, byte loads
+template <bool F16S, bool SWIGLU>
 __global__ __launch_bounds__(kThreads) void fp8_generic_matvec_kernel(
-    const void* __restrict__ x, int x_dtype, const uint8_t* __restrict__ w, const float* __restrict__ scale,
-    void* __restrict__ y, int y_dtype, int k, int n, int kb) {
+    const void* __restrict__ x, int x_dtype, size_t x_stride, const Fp8Mat ma, const Fp8Mat mb,
+    void* __restrict__ y, int y_dtype, size_t y_stride, int k, int n) {
     const int lane = threadIdx.x & 63;
     const int row = blockIdx.x * kWaves + (threadIdx.x >> 6);
-    const size_t xoff = static_cast<size_t>(blockIdx.y) * k;
-    float acc = 0.0f;
+    const size_t xoff = static_cast<size_t>(blockIdx.y) * x_stride;
+    float acc = 0.0f, acc_up = 0.0f;
     if (row < n) {
-        const uint8_t* wrow = w + static_cast<size_t>(row) * k;
-        for (int c = lane; c < k; c += 64)
-            acc += load_any(x, x_dtype, xoff + c) * (fp8_to_float_sw(wrow[c]) * scale[(row >> 7) * kb + (c >> 7)]);
+        const uint8_t* wrow = ma.w + static_cast<size_t>(row) * ma.wstride;
+        for (int c = lane; c < k; c += 64) {
+            const float xv = load_any(x, x_dtype, xoff + c);
+            acc += xv * (fp8_to_float_sw(wrow[c]) * scale_at<F16S>(ma.scale, static_cast<size_t>(row >> 7) * ma.sstride + (c >> 7)));
+            if constexpr (SWIGLU)
+                acc_up += xv * (fp8_to_float_sw(mb.w[static_cast<size_t>(row) * mb.wstride + c]) *
+                                scale_at<F16S>(mb.scale, static_cast<size_t>(row >> 7) * mb.sstride + (c >> 7)));
+        }
     }
     acc = group_sum<64>(acc);
-    if (lane == 0 && row < n) store_any(y, y_dtype, static_cast<size_t>(blockIdx.y) * n + row, acc);
+    if constexpr (SWIGLU) acc = silu(acc) * group_sum<64>(acc_up);
+    if (lane == 0 && row < n) store_any(y, y_dtype, static_cast<size_t>(blockIdx.y) * y_stride + row, acc);
 }
 
-template <int ITERS>
-int launch_stream(const void* x, int x_dtype, const uint8_t* w, const float* scale, void* y, int y_dtype,
-                  int rows, int k, int n, hipStream_t stream) {
-    const size_t smem = static_cast<size_t>(k) * sizeof(float);
-    auto kern = fp8_stream_matvec_kernel<ITERS>;
-    if (smem > 64 * 1024) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                static_cast<int>(smem)) != hipSuccess)
-            return PLLM_ERR_UNSUPPORTED;
+// fp16 scale table with a row pitch -> dense float32 table (what the tile kernel reads)
+__global__ __launch_bounds__(kThreads) void f16_scale_table_kernel(const uint16_t* __restrict__ src, int src_stride, float* __restrict__ dst,
+                                                                   int table_rows, int table_cols) {
+    const int i = blockIdx.x * kThreads + threadIdx.x;
+    if (i < table_rows * table_cols) dst[i] = f16_bits_to_float(src[static_cast<size_t>(i / table_cols) * src_stride + i % table_cols]);
+}
+
+template <bool F16S, bool SWIGLU>
+int launch_any(const void* x, int x_dtype, size_t x_stride, const Fp8Mat& ma, const Fp8Mat& mb, void* y, int y_dtype, size_t y_stride,
+               int rows, int k, int n, hipStream_t stream) {
+    const bool aligned = (k % 16 == 0) && (static_cast<size_t>(k) * 4 <= 160 * 1024) &&
+                         ((reinterpret_cast<uintptr_t>(ma.w) | ma.wstride) & 15u) == 0 &&
+                         (!SWIGLU || ((reinterpret_cast<uintptr_t>(mb.w) | mb.wstride) & 15u) == 0);
+    if (!aligned) {
+        dim3 grid((n + kWaves - 1) / kWaves, rows);
+        hipLaunchKernelGGL((fp8_generic_matvec_kernel<F16S, SWIGLU>), grid, dim3(kThreads), 0, stream, x, x_dtype, x_stride, ma, mb,
+                           y, y_dtype, y_stride, k, n);
+        return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
     }
-    const int rows_per_wg = kWaves * kRowsPerWave;
-    dim3 grid((n + rows_per_wg - 1) / rows_per_wg, rows);
-    hipLaunchKernelGGL(kern, grid, dim3(kThreads), smem, stream, x, x_dtype, w, scale, y, y_dtype, k, n, (k + 127) / 128);
+    const size_t smem = static_cast<size_t>(k) * sizeof(float);
+    const int rows_per_group = kWaves * (SWIGLU ? 1 : kRowsPerWave);
+    const int groups = (n + rows_per_group - 1) / rows_per_group;
+    const int niter = ((k >> 4) + 63) / 64;
+    if (niter <= 6) {
+        // persistent: two resident workgroups per compute unit (register-bound), groups dealt round-robin
+        const int grid_x = std::min(groups, 2 * compute_units());
+#define PLLM_PCASE(I) case I: { \
+            auto kern = fp8_persistent_matvec_kernel<I, F16S, SWIGLU>; \
+            if (smem > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                                        static_cast<int>(smem)) != hipSuccess) return PLLM_ERR_UNSUPPORTED; \
+            hipLaunchKernelGGL(kern, dim3(grid_x, rows), dim3(kThreads), smem, stream, x, x_dtype, x_stride, ma, mb, y, y_dtype, y_stride, k, n, groups); \
+            break; }
+        switch (niter) {
+            PLLM_PCASE(1) PLLM_PCASE(2) PLLM_PCASE(3) PLLM_PCASE(4) PLLM_PCASE(5)
+            default: PLLM_PCASE(6)
+        }
+#undef PLLM_PCASE
+        return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+    }
+    const int passes = (niter + 5) / 6;
+    const int iters = (niter + passes - 1) / passes;
+#define PLLM_CASE(I) case I: { \
+            auto kern = fp8_stream_matvec_kernel<I, F16S, SWIGLU>; \
+            if (smem > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                                        static_cast<int>(smem)) != hipSuccess) return PLLM_ERR_UNSUPPORTED; \
+            hipLaunchKernelGGL(kern, dim3(groups, rows), dim3(kThreads), smem, stream, x, x_dtype, x_stride, ma, mb, y, y_dtype, y_stride, k, n); \
+            break; }
+    switch (iters) {
+        PLLM_CASE(1) PLLM_CASE(2) PLLM_CASE(3) PLLM_CASE(4) PLLM_CASE(5)
+        default: PLLM_CASE(6)
+    }
+#undef PLLM_CASE
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 
@@ -208,34 +293,28 @@ int launch_stream(const void* x, int x_dtype, const uint8_t* w, const float* sca
 
 int fp8_matvec(const void* x, int x_dtype, const uint8_t* w, const float* scale, void* y, int y_dtype,
                int rows, int k, int n, hipStream_t stream) {
-    const bool stream_ok = (k % 16 == 0) && ((reinterpret_cast<uintptr_t>(w) & 15u) == 0) && (static_cast<size_t>(k) * 4 <= 160 * 1024);
-    if (!stream_ok) {
-        dim3 grid((n + kWaves - 1) / kWaves, rows);
-        hipLaunchKernelGGL(fp8_generic_matvec_kernel, grid, dim3(kThreads), 0, stream, x, x_dtype, w, scale, y, y_dtype, k, n,
-                           (k + 127) / 128);
-        return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
-    }
-    const int niter = ((k >> 4) + 63) / 64;
-    if (niter <= 6) {
-        const int groups = (n + kWaves * kRowsPerWave - 1) / (kWaves * kRowsPerWave);
-        const int grid_x = std::min(groups, 2 * compute_units());   // two resident workgroups per compute unit (register-bound), groups dealt round-robin
-        const size_t smem = static_cast<size_t>(k) * sizeof(float);
-#define PLLM_PCASE(I) case I: hipLaunchKernelGGL(fp8_persistent_matvec_kernel<I>, dim3(grid_x, rows), dim3(kThreads), smem, stream, x, x_dtype, w, scale, y, y_dtype, k, n, (k + 127) / 128, groups); break
-        switch (niter) {
-            PLLM_PCASE(1); PLLM_PCASE(2); PLLM_PCASE(3); PLLM_PCASE(4); PLLM_PCASE(5);
-            default: hipLaunchKernelGGL(fp8_persistent_matvec_kernel<6>, dim3(grid_x, rows), dim3(kThreads), smem, stream, x, x_dtype, w, scale, y, y_dtype, k, n, (k + 127) / 128, groups); break;
-        }
-#undef PLLM_PCASE
-        return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
-    }
-    const int passes = (niter + 5) / 6;
-    const int iters = (niter + passes - 1) / passes;
-#define PLLM_CASE(I) case I: return launch_stream<I>(x, x_dtype, w, scale, y, y_dtype, rows, k, n, stream)
-    switch (iters) {
-        PLLM_CASE(1); PLLM_CASE(2); PLLM_CASE(3); PLLM_CASE(4); PLLM_CASE(5);
-        default: return launch_stream<6>(x, x_dtype, w, scale, y, y_dtype, rows, k, n, stream);
-    }
-#undef PLLM_CASE
+    const Fp8Mat m{w, scale, static_cast<size_t>(k), (k + 127) / 128};
+    return launch_any<false, false>(x, x_dtype, static_cast<size_t>(k), m, m, y, y_dtype, static_cast<size_t>(n), rows, k, n, stream);
+}
+
+int fp8_f16scale_matvec(const void* x, int x_dtype, size_t x_stride, const uint8_t* w, const uint16_t* scale, size_t weight_stride,
+                        int scale_stride, void* y, int y_dtype, size_t y_stride, int rows, int k, int n, hipStream_t stream) {
+    const Fp8Mat m{w, scale, weight_stride, scale_stride};
+    return launch_any<true, false>(x, x_dtype, x_stride, m, m, y, y_dtype, y_stride, rows, k, n, stream);
+}
+
+int fp8_f16scale_table_to_f32(const uint16_t* scale, int scale_stride, float* out, int n, int k, hipStream_t stream) {
+    const int tr = (n + 127) / 128, tc = (k + 127) / 128;
+    hipLaunchKernelGGL(f16_scale_table_kernel, dim3((tr * tc + kThreads - 1) / kThreads), dim3(kThreads), 0, stream, scale, scale_stride, out, tr, tc);
+    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+}
+
+int fp8_f16scale_swiglu_matvec(const void* x, int x_dtype, size_t x_stride, const uint8_t* gate_w, const uint16_t* gate_scale,
+                               const uint8_t* up_w, const uint16_t* up_scale, size_t weight_stride, int scale_stride,
+                               void* y, int y_dtype, size_t y_stride, int rows, int k, int n, hipStream_t stream) {
+    const Fp8Mat g{gate_w, gate_scale, weight_stride, scale_stride};
+    const Fp8Mat u{up_w, up_scale, weight_stride, scale_stride};
+    return launch_any<true, true>(x, x_dtype, x_stride, g, u, y, y_dtype, y_stride, rows, k, n, stream);
 }
 
 }  // namespace pllm

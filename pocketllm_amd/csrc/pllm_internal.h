@@ -93,5 +93,13 @@ int gemm_f16(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y,
 // FP8 E4M3 weights [n, k] with float32 scales [ceil(n/128), ceil(k/128)] (matvec_fp8.hip)
 int fp8_matvec(const void* x, int x_dtype, const uint8_t* w, const float* scale, void* y, int y_dtype,
                int rows, int k, int n, hipStream_t stream);
+// the same with fp16 scale bits and explicit pitches (elements between activation / output rows, bytes between
+// weight rows, entries between scale-table rows), and the fused form y = silu(gate . x) * (up . x)
+int fp8_f16scale_matvec(const void* x, int x_dtype, size_t x_stride, const uint8_t* w, const uint16_t* scale, size_t weight_stride,
+                        int scale_stride, void* y, int y_dtype, size_t y_stride, int rows, int k, int n, hipStream_t stream);
+int fp8_f16scale_swiglu_matvec(const void* x, int x_dtype, size_t x_stride, const uint8_t* gate_w, const uint16_t* gate_scale,
+                               const uint8_t* up_w, const uint16_t* up_scale, size_t weight_stride, int scale_stride,
+                               void* y, int y_dtype, size_t y_stride, int rows, int k, int n, hipStream_t stream);
+int fp8_f16scale_table_to_f32(const uint16_t* scale, int scale_stride, float* out, int n, int k, hipStream_t stream);
 
 }  // namespace pllm

@@ -478,3 +478,31 @@ def test_kquant_int8_semantics_close_to_float_semantics():
         xq, xs = O.q8_1_quantize(x)
         xl = (xq.reshape(5, -1, 32).astype(np.float32) * xs[..., None]).reshape(5, 512)
         assert O.rel_l2(O.kquant_gemm_q(xl, blocks, name), O.matmul_f(xl, O.dequant_rows(blocks, name))) < 1e-6, name
+
+
+def test_fp8_fp16scale_expectation_indexing_and_reference_bit_decode():
+    """The C++ engine's FP8 statement: (a) its bit-trick decoder (cpp_engine/cuda/qwen_fp8_ops.cu:16-31), restated here from
+    its description (normal codes: exponent + 120, mantissa << 20; subnormals m * 2^-9), agrees with the oracle decode on all
+    254 non-NaN codes; (b) the pitched indexing of the expectation against a plain loop on an unaligned case."""
+    codes = np.array([c for c in range(256) if (c & 0x7F) != 0x7F], dtype=np.uint8)
+    e, m = (codes >> 3) & 15, codes & 7
+    bits = np.where(e != 0, ((e.astype(np.uint32) + 120) << 23) | (m.astype(np.uint32) << 20), 0).astype(np.uint32)
+    ref = np.where(e != 0, bits.view(np.float32), m.astype(np.float32) * np.float32(2.0 ** -9))
+    ref = np.where(codes & 0x80, -ref, ref).astype(np.float32)
+    np.testing.assert_array_equal(O.fp8_e4m3_decode(codes), ref)
+
+    rng = np.random.default_rng(5)
+    rows, cols, wstride, sstride = 130, 300, 304, 5
+    weight = rng.integers(0, 256, size=rows * wstride, dtype=np.uint8)
+    weight[(weight & 0x7F) == 0x7F] = 0x70
+    scale = rng.uniform(0.01, 0.4, size=2 * sstride).astype(np.float16)
+    x = rng.uniform(-1.5, 1.5, size=(2, cols)).astype(np.float32)
+    got = O.fp8_fp16scale_matmul(x, weight, scale.view(np.uint16), rows, cols, wstride, sstride)
+    dec = O.fp8_e4m3_decode(np.arange(256, dtype=np.uint8))
+    for b, r in ((0, 0), (1, 127), (0, 128), (1, 129)):
+        want = 0.0
+        for c in range(cols):
+            want += float(x[b, c]) * float(dec[weight[r * wstride + c]]) * float(scale[(r // 128) * sstride + c // 128])
+        assert abs(got[b, r] - want) <= 1e-9 * max(1.0, abs(want))
+    g, u = np.array([0.0, 1.0, -2.0]), np.array([3.0, 2.0, 1.0])
+    np.testing.assert_allclose(O.silu_mul(g, u), [0.0, 2.0 / (1.0 + np.exp(-1.0)), -2.0 / (1.0 + np.exp(2.0))], rtol=1e-15)
