@@ -184,6 +184,16 @@ int pllm_fp8_fp16scale_matmul_rows(const void* x, int x_dtype, const uint8_t* we
 size_t pllm_fp8_fp16scale_matmul_rows_workspace_bytes(int64_t batch, int64_t rows, int64_t cols);
 
 /*
+ * The same matvec over `batch` rows with the scale table kept as bf16 bits, the checkpoint's own storage:
+ * replaces qwen_fp8_e4m3_bf16_matvec_cuda (batch 1, x_stride = cols, y_stride = rows) and
+ * qwen_fp8_e4m3_bf16_matmul_rows_cuda (cpp_engine/include/qwen_cuda_ops.hpp:172-197), which the reference keeps
+ * as its compatibility path; every row takes the float32 matvec kernel.
+ */
+int pllm_fp8_bf16scale_matmul_rows(const void* x, int x_dtype, const uint8_t* weight, const uint16_t* scale_bf16, void* y, int y_dtype,
+                                   int64_t batch, int64_t rows, int64_t cols, int64_t x_stride, int64_t y_stride,
+                                   int64_t weight_stride, int64_t scale_stride, void* stream);
+
+/*
  * Fused routed-expert matmul over raw super-blocks (types Q2_K, IQ2_XXS, IQ1_M; gate/up share a type,
  * the down projection may use another, so IQ2_XXS gate/up with IQ1_M down needs no special case):
  *     y[t] = sum over routes r of token t:  W2_e ( silu(min(W1_e x_t, L)) * clamp(W3_e x_t, +-L) * w_r )

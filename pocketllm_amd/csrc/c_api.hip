@@ -244,6 +244,18 @@ int pllm_fp8_fp16scale_swiglu_matvec(const void* x, int x_dtype, const uint8_t* 
                                             static_cast<int>(rows), static_cast<hipStream_t>(stream));
 }
 
+int pllm_fp8_bf16scale_matmul_rows(const void* x, int x_dtype, const uint8_t* weight, const uint16_t* scale_bf16, void* y, int y_dtype,
+                                   int64_t batch, int64_t rows, int64_t cols, int64_t x_stride, int64_t y_stride,
+                                   int64_t weight_stride, int64_t scale_stride, void* stream) {
+    if (!dtype_ok(x_dtype) || !dtype_ok(y_dtype) || !fp16scale_args_ok(x, weight, scale_bf16, y, rows, cols, weight_stride, scale_stride))
+        return PLLM_ERR_INVALID_ARGUMENT;
+    if (batch <= 0 || x_stride < cols || y_stride < rows) return PLLM_ERR_INVALID_ARGUMENT;
+    if (batch > 65535) return PLLM_ERR_UNSUPPORTED;
+    return pllm::fp8_bf16scale_matvec(x, x_dtype, static_cast<size_t>(x_stride), weight, scale_bf16, static_cast<size_t>(weight_stride),
+                                      static_cast<int>(scale_stride), y, y_dtype, static_cast<size_t>(y_stride), static_cast<int>(batch),
+                                      static_cast<int>(cols), static_cast<int>(rows), static_cast<hipStream_t>(stream));
+}
+
 // Many rows of 16-bit activations with dense pitches and 256-aligned cols run on the tile kernel (float32 scale table in
 // the workspace).  float32 activations stay on the float32 matvec, row by row: the tile kernel rounds its operands to fp16,
 // which is inside the bound the reference sets for its fp16-storage variants (2e-2) but not the 2e-4 of its float32 ones.

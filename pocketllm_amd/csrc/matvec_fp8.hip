@@ -24,14 +24,16 @@ typedef float v2f __attribute__((ext_vector_type(2)));
 // One weight matrix as the kernels see it: codes with a row pitch, scale table with a row pitch.
 struct Fp8Mat {
     const uint8_t* w;
-    const void* scale;      // float32 or fp16 bits, chosen by the kernels' F16S parameter
+    const void* scale;      // float32, fp16 bits or bf16 bits, chosen by the kernels' F16S parameter
     size_t wstride;         // bytes between rows of codes
     int sstride;            // entries between rows of the scale table
 };
 
-template <bool F16S>
+// scale storage: 0 float32, 1 IEEE fp16 bits, 2 bf16 bits
+template <int F16S>
 __device__ __forceinline__ float scale_at(const void* __restrict__ scale, size_t i) {
-    if constexpr (F16S) return f16_bits_to_float(static_cast<const uint16_t*>(scale)[i]);
+    if constexpr (F16S == 1) return f16_bits_to_float(static_cast<const uint16_t*>(scale)[i]);
+    else if constexpr (F16S == 2) return __uint_as_float(static_cast<uint32_t>(static_cast<const uint16_t*>(scale)[i]) << 16);
     else return static_cast<const float*>(scale)[i];
 }
 
@@ -63,7 +65,7 @@ __device__ __forceinline__ float chunk_dot(const uint4& w, const float* xp) {
 }
 
 // k a multiple of 16, weight base and row pitch 16-byte aligned
-template <int ITERS, bool F16S, bool SWIGLU>
+template <int ITERS, int F16S, bool SWIGLU>
 __global__ __launch_bounds__(kThreads) void fp8_stream_matvec_kernel(
     const void* __restrict__ x, int x_dtype, size_t x_stride, const Fp8Mat ma, const Fp8Mat mb,
     void* __restrict__ y, int y_dtype, size_t y_stride, int k, int n) {
@@ -138,7 +140,7 @@ __device__ __forceinline__ void fp8_fetch_group(uint4 (&r)[kRowsPerWave][ITERS],
     }
 }
 
-template <int ITERS, bool F16S, bool SWIGLU>
+template <int ITERS, int F16S, bool SWIGLU>
 __device__ __forceinline__ void fp8_finish_group(const uint4 (&r)[kRowsPerWave][ITERS], const float* xs, const Fp8Mat& ma, const Fp8Mat& mb,
                                                  void* __restrict__ y, int y_dtype, size_t yoff, int row0, int n, int chunks, int lane) {
     float acc[kRowsPerWave];
@@ -169,7 +171,7 @@ __device__ __forceinline__ void fp8_finish_group(const uint4 (&r)[kRowsPerWave][
     }
 }
 
-template <int ITERS, bool F16S, bool SWIGLU>
+template <int ITERS, int F16S, bool SWIGLU>
 __global__ __launch_bounds__(kThreads) void fp8_persistent_matvec_kernel(
     const void* __restrict__ x, int x_dtype, size_t x_stride, const Fp8Mat ma, const Fp8Mat mb,
     void* __restrict__ y, int y_dtype, size_t y_stride, int k, int n, int groups) {
@@ -211,7 +213,7 @@ __device__ __forceinline__ float fp8_to_float_sw(uint32_t c) {
 }
 
 // any k, any alignment: one wave per row, byte loads
-template <bool F16S, bool SWIGLU>
+template <int F16S, bool SWIGLU>
 __global__ __launch_bounds__(kThreads) void fp8_generic_matvec_kernel(
     const void* __restrict__ x, int x_dtype, size_t x_stride, const Fp8Mat ma, const Fp8Mat mb,
     void* __restrict__ y, int y_dtype, size_t y_stride, int k, int n) {
@@ -241,7 +243,7 @@ __global__ __launch_bounds__(kThreads) void f16_scale_table_kernel(const uint16_
     if (i < table_rows * table_cols) dst[i] = f16_bits_to_float(src[static_cast<size_t>(i / table_cols) * src_stride + i % table_cols]);
 }
 
-template <bool F16S, bool SWIGLU>
+template <int F16S, bool SWIGLU>
 int launch_any(const void* x, int x_dtype, size_t x_stride, const Fp8Mat& ma, const Fp8Mat& mb, void* y, int y_dtype, size_t y_stride,
                int rows, int k, int n, hipStream_t stream) {
     const bool aligned = (k % 16 == 0) && (static_cast<size_t>(k) * 4 <= 160 * 1024) &&
@@ -294,13 +296,19 @@ int launch_any(const void* x, int x_dtype, size_t x_stride, const Fp8Mat& ma, co
 int fp8_matvec(const void* x, int x_dtype, const uint8_t* w, const float* scale, void* y, int y_dtype,
                int rows, int k, int n, hipStream_t stream) {
     const Fp8Mat m{w, scale, static_cast<size_t>(k), (k + 127) / 128};
-    return launch_any<false, false>(x, x_dtype, static_cast<size_t>(k), m, m, y, y_dtype, static_cast<size_t>(n), rows, k, n, stream);
+    return launch_any<0, false>(x, x_dtype, static_cast<size_t>(k), m, m, y, y_dtype, static_cast<size_t>(n), rows, k, n, stream);
 }
 
 int fp8_f16scale_matvec(const void* x, int x_dtype, size_t x_stride, const uint8_t* w, const uint16_t* scale, size_t weight_stride,
                         int scale_stride, void* y, int y_dtype, size_t y_stride, int rows, int k, int n, hipStream_t stream) {
     const Fp8Mat m{w, scale, weight_stride, scale_stride};
-    return launch_any<true, false>(x, x_dtype, x_stride, m, m, y, y_dtype, y_stride, rows, k, n, stream);
+    return launch_any<1, false>(x, x_dtype, x_stride, m, m, y, y_dtype, y_stride, rows, k, n, stream);
+}
+
+int fp8_bf16scale_matvec(const void* x, int x_dtype, size_t x_stride, const uint8_t* w, const uint16_t* scale, size_t weight_stride,
+                         int scale_stride, void* y, int y_dtype, size_t y_stride, int rows, int k, int n, hipStream_t stream) {
+    const Fp8Mat m{w, scale, weight_stride, scale_stride};
+    return launch_any<2, false>(x, x_dtype, x_stride, m, m, y, y_dtype, y_stride, rows, k, n, stream);
 }
 
 int fp8_f16scale_table_to_f32(const uint16_t* scale, int scale_stride, float* out, int n, int k, hipStream_t stream) {
@@ -314,7 +322,7 @@ int fp8_f16scale_swiglu_matvec(const void* x, int x_dtype, size_t x_stride, cons
                                void* y, int y_dtype, size_t y_stride, int rows, int k, int n, hipStream_t stream) {
     const Fp8Mat g{gate_w, gate_scale, weight_stride, scale_stride};
     const Fp8Mat u{up_w, up_scale, weight_stride, scale_stride};
-    return launch_any<true, true>(x, x_dtype, x_stride, g, u, y, y_dtype, y_stride, rows, k, n, stream);
+    return launch_any<1, true>(x, x_dtype, x_stride, g, u, y, y_dtype, y_stride, rows, k, n, stream);
 }
 
 }  // namespace pllm

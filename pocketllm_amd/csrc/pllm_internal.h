@@ -97,6 +97,8 @@ int fp8_matvec(const void* x, int x_dtype, const uint8_t* w, const float* scale,
 // weight rows, entries between scale-table rows), and the fused form y = silu(gate . x) * (up . x)
 int fp8_f16scale_matvec(const void* x, int x_dtype, size_t x_stride, const uint8_t* w, const uint16_t* scale, size_t weight_stride,
                         int scale_stride, void* y, int y_dtype, size_t y_stride, int rows, int k, int n, hipStream_t stream);
+int fp8_bf16scale_matvec(const void* x, int x_dtype, size_t x_stride, const uint8_t* w, const uint16_t* scale, size_t weight_stride,
+                         int scale_stride, void* y, int y_dtype, size_t y_stride, int rows, int k, int n, hipStream_t stream);
 int fp8_f16scale_swiglu_matvec(const void* x, int x_dtype, size_t x_stride, const uint8_t* gate_w, const uint16_t* gate_scale,
                                const uint8_t* up_w, const uint16_t* up_scale, size_t weight_stride, int scale_stride,
                                void* y, int y_dtype, size_t y_stride, int rows, int k, int n, hipStream_t stream);

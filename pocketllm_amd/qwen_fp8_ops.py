@@ -77,3 +77,19 @@ def qwen_fp8_e4m3_fp16scale_matmul_rows(x, weight, scale_fp16, y, batch: int, ro
                                                 int(batch), int(rows), int(cols), int(x_stride), int(y_stride), int(weight_stride),
                                                 int(scale_stride), _ptr(ws), ws_bytes, torch.cuda.current_stream(x.device).cuda_stream)
     return st == 0
+
+
+def qwen_fp8_e4m3_bf16_matmul_rows(x, weight, scale_bf16, y, batch: int, rows: int, cols: int, x_stride: int, y_stride: int,
+                                   weight_stride: int, scale_stride: int) -> bool:
+    """The compatibility forms with bf16 scale bits (qwen_cuda_ops.hpp:172-197); batch 1 is qwen_fp8_e4m3_bf16_matvec_cuda."""
+    if not _on_one_gpu(x, weight, scale_bf16, y) or not _codes_ok(x, y):
+        return False
+    with torch.cuda.device(x.device):
+        st = _lib().pllm_fp8_bf16scale_matmul_rows(_ptr(x), _DTYPE_CODE[x.dtype], _ptr(weight), _ptr(scale_bf16), _ptr(y), _DTYPE_CODE[y.dtype],
+                                                   int(batch), int(rows), int(cols), int(x_stride), int(y_stride), int(weight_stride),
+                                                   int(scale_stride), torch.cuda.current_stream(x.device).cuda_stream)
+    return st == 0
+
+
+def qwen_fp8_e4m3_bf16_matvec(x, weight, scale_bf16, y, rows: int, cols: int, weight_stride: int, scale_stride: int) -> bool:
+    return qwen_fp8_e4m3_bf16_matmul_rows(x, weight, scale_bf16, y, 1, rows, cols, cols, rows, weight_stride, scale_stride)

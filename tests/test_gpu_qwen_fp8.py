@@ -129,6 +129,25 @@ def test_fp16_storage_rows_take_the_tile_kernel(batch, rows, cols):
     assert O.rel_l2(y.float().cpu().numpy(), want) < 2.0e-3
 
 
+@pytest.mark.parametrize("batch,rows,cols", [(1, 384, 640), (1, 130, 300), (9, 128, 256)])
+def test_bf16_scale_compatibility_forms(batch, rows, cols):
+    """Scale table as bf16 bits (the checkpoint's storage, cpp_engine/tests/test_qwen_fp8_online.cpp:150-156): the expectation is the
+    fp16-scale statement evaluated on the same scale values, which are chosen exactly representable in both formats."""
+    rng = np.random.default_rng(rows + batch)
+    x, weight, _, wstride, sstride = _case(rng, batch, rows, cols)
+    sc = (rng.integers(3, 100, size=((rows + 127) // 128) * sstride).astype(np.float32) / np.float32(256.0))   # 7 significant bits
+    bf16_bits = (sc.view(np.uint32) >> 16).astype(np.uint16)
+    want = O.fp8_fp16scale_matmul(x, weight, sc.astype(np.float16).view(np.uint16), rows, cols, wstride, sstride)
+    y = torch.empty(batch, rows, device=DEV)
+    dev = lambda a: torch.from_numpy(a.view(np.int16) if a.dtype == np.uint16 else a).to(DEV)
+    if batch == 1:
+        assert Q.qwen_fp8_e4m3_bf16_matvec(dev(x), dev(weight), dev(bf16_bits), y, rows, cols, wstride, sstride)
+    else:
+        assert Q.qwen_fp8_e4m3_bf16_matmul_rows(dev(x), dev(weight), dev(bf16_bits), y, batch, rows, cols, cols, rows, wstride, sstride)
+    torch.cuda.synchronize()
+    assert _max_rel(y.cpu().numpy(), want) < 2.0e-4
+
+
 def test_bad_arguments_return_false_and_write_nothing():
     """cpp_engine/cuda/qwen_fp8_ops.cu:951-955, 969-970, 1087-1088: null pointers, non-positive sizes, pitches below the
     extent: false, no launch."""
