@@ -204,6 +204,14 @@ def extra_cases(mod, dev, iters):
     run("fused experts iq2_xxs gate/up + iq1_m down, 256 experts top-8, T=1", per_call,
         lambda s: mod.gguf_moe_single_token_forward(xm, topi[s], topw[s], w1, w3, w2, 0.0), RING,
         {"note": "each slot routes to a different random top-8 of the 256 resident experts (887 MB)"})
+    # routing ahead of the experts: gate logits + sigmoid + top-8 + renormalisation (256 experts x 3072, float32 gate)
+    gate = torch.randn(e, d, device=dev) * (d ** -0.5)
+    gbias = torch.zeros(e, device=dev)
+    for tt in (1, 256):
+        xr = torch.randn(tt, d, device=dev, dtype=torch.bfloat16)
+        us, graphed = time_calls_us(lambda s, xr=xr: mod.moe_route(xr, gate, gbias, 8), 4, max(8, iters // 4))
+        out.append({"case": f"expert routing (gate 256x3072 f32, sigmoid + bias, top-8) T={tt}", "us_per_call": round(us, 3), "graph": graphed,
+                    "weight_bytes": e * d * 4, "gbs": round(e * d * 4 / us / 1e3, 1)})
     # the same experts at T=256 (BASELINE config 5): 2048 routes grouped by expert
     t = 256
     logits = torch.from_numpy(rng.standard_normal((t, e)).astype(np.float32))

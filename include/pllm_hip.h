@@ -228,6 +228,21 @@ int pllm_moe_group_routes(const void* indices, int indices_are_i64, const float*
                           int32_t* route_experts, void* stream);
 
 /*
+ * Expert routing ahead of the fused expert matmul: gate logits, scores, top-k, renormalised route weights.
+ *   logits[t, e] = x[t, :] . gate_weight[e, :]   (gate_weight float32 [n_experts, dim], float32 accumulation)
+ *   softmax_mode == 0: p = sigmoid(logits); the top_k of p + gate_bias (gate_bias float32 [n_experts] or null) are picked;
+ *                      weights = p[picked] / max(sum of p[picked], 1e-20)
+ *   softmax_mode != 0: the top_k logits are picked; weights = softmax over the picked logits
+ *   indices int64 [tokens, top_k] in descending score order (lower expert id first on equal scores), weights float32 [tokens, top_k];
+ *   logits float32 [tokens, n_experts] is caller-provided scratch that holds the logits afterwards.
+ * Replaces MiniMaxMoE.route (src/models/minimax_m2/architecture.py:291-298), a chain of six framework ops on the caller's side
+ * of the expert operators; the softmax form is the routing of the grouped-expert benchmark (tests/bench_gguf_fused_expert.py).
+ * n_experts <= 1024, top_k <= 64.
+ */
+int pllm_moe_route(const void* x, int x_dtype, int64_t tokens, int64_t dim, const float* gate_weight, const float* gate_bias,
+                   int64_t n_experts, int64_t top_k, int softmax_mode, float* logits, int64_t* indices, float* weights, void* stream);
+
+/*
  * FP8 activation quantizer: per (row, 128 values) scale = max(amax, eps) / 448 (rounded up to a power
  * of two when round_scale_pow2 != 0), code = E4M3FN round-to-nearest-even of clamp(x / scale, +-448).
  *   x [rows, k] (k a multiple of 128) -> codes uint8 [rows, k], scales float32 [rows, k / 128]

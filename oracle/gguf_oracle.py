@@ -544,6 +544,30 @@ def swiglu_route(gate: np.ndarray, up: np.ndarray, route_w: np.ndarray, limit: f
     return g / (1.0 + np.exp(-g)) * u * route_w.astype(np.float64)[:, None]
 
 
+def route_topk(logits: np.ndarray, bias, top_k: int, softmax: bool = False):
+    """Scores, top-k and renormalised weights from gate logits [T, E] (float64 arithmetic on the given logits).
+
+    Reference: MiniMaxMoE.route, src/models/minimax_m2/architecture.py:291-298 (sigmoid, optional bias added for the
+    selection only, weights = picked probabilities / max(their sum, 1e-20)); softmax=True is softmax -> top-k ->
+    renormalise, which equals the softmax over the picked logits.  Picks come in descending score order, the lower expert id
+    first on equal scores (the reference's topk leaves ties unspecified).  Pinned by closed-form cases in
+    tests/test_oracle_pinning.py."""
+    l = logits.astype(np.float64)
+    if softmax:
+        score, prob = l, l
+    else:
+        prob = 1.0 / (1.0 + np.exp(-l))
+        score = prob if bias is None else prob + bias.astype(np.float64)[None, :]
+    order = np.argsort(-score, axis=1, kind="stable")[:, :top_k]
+    picked = np.take_along_axis(prob, order, axis=1)
+    if softmax:
+        ex = np.exp(picked - picked.max(axis=1, keepdims=True))
+        w = ex / ex.sum(axis=1, keepdims=True)
+    else:
+        w = picked / np.maximum(picked.sum(axis=1, keepdims=True), 1.0e-20)
+    return order.astype(np.int64), w
+
+
 def group_routes(indices: np.ndarray, weights: np.ndarray, experts_start: int, n_local: int):
     """Counting sort of (token, k) routes by local expert.
 

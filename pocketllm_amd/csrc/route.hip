@@ -1,0 +1,130 @@
+// Expert routing of the fused expert path's callers: gate logits, scores, top-k and renormalised
+// route weights in two launches instead of six framework ops.
+//
+//   logits[t, e] = x[t, :] . gate_weight[e, :]                (float32 accumulate)
+//   sigmoid mode: p = sigmoid(logits); pick the top_k of p + bias (bias optional); weight = p / max(sum of picked p, 1e-20)
+//   softmax mode: pick the top_k logits; weight = softmax over the picked logits (= softmax probabilities renormalised)
+//
+// Launch 1: one wave per (expert, token), 16-byte loads of the gate row, 64-lane sum.  Launch 2: one
+// wave per token, every lane keeps E / 64 candidates in registers, top_k rounds of a wave-wide
+// argmax (larger score first, lower expert id on equal scores), picked in descending order.
+#include "pllm_device.h"
+#include "pllm_internal.h"
+
+namespace pllm {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWavesPerWg = kThreads / 64;
+constexpr int kMaxPerLane = 16;          // experts per lane: up to 1024 experts
+
+__global__ __launch_bounds__(kThreads) void route_logits_kernel(
+    const void* __restrict__ x, int x_dtype, const float* __restrict__ gate, float* __restrict__ logits, int dim, int n_experts) {
+    const int lane = threadIdx.x & 63;
+    const int e = blockIdx.x * kWavesPerWg + (threadIdx.x >> 6);
+    if (e >= n_experts) return;                                             // whole waves leave together
+    const size_t xoff = static_cast<size_t>(blockIdx.y) * dim;
+    const float* grow = gate + static_cast<size_t>(e) * dim;
+    float acc = 0.0f;
+    const bool vec = (dim % 4 == 0) && ((reinterpret_cast<uintptr_t>(gate) & 15u) == 0);
+    if (vec) {
+        for (int c = lane * 4; c < dim; c += 256) {
+            const float4 g = *reinterpret_cast<const float4*>(grow + c);
+            acc += g.x * load_any(x, x_dtype, xoff + c) + g.y * load_any(x, x_dtype, xoff + c + 1) +
+                   g.z * load_any(x, x_dtype, xoff + c + 2) + g.w * load_any(x, x_dtype, xoff + c + 3);
+        }
+    } else {
+        for (int c = lane; c < dim; c += 64) acc += grow[c] * load_any(x, x_dtype, xoff + c);
+    }
+    acc = group_sum<64>(acc);
+    if (lane == 0) logits[static_cast<size_t>(blockIdx.y) * n_experts + e] = acc;
+}
+
+__device__ __forceinline__ float wave_max(float v) { return group_max<64>(v); }
+
+__global__ __launch_bounds__(64) void route_topk_kernel(
+    const float* __restrict__ logits, const float* __restrict__ bias, int n_experts, int top_k, int softmax_mode,
+    int64_t* __restrict__ indices, float* __restrict__ weights) {
+    const int lane = threadIdx.x;
+    const size_t t = blockIdx.x;
+    const float* row = logits + t * n_experts;
+    constexpr float kGone = -3.0e38f;
+    float score[kMaxPerLane], prob[kMaxPerLane];
+#pragma unroll
+    for (int i = 0; i < kMaxPerLane; ++i) {
+        const int e = lane + 64 * i;
+        score[i] = kGone;
+        prob[i] = 0.0f;
+        if (e < n_experts) {
+            const float l = row[e];
+            if (softmax_mode) {
+                score[i] = l;
+                prob[i] = l;
+            } else {
+                const float p = 1.0f / (1.0f + expf(-l));
+                prob[i] = p;
+                score[i] = bias ? p + bias[e] : p;
+            }
+        }
+    }
+    // top_k rounds; lane r keeps the r-th pick
+    int my_pick = -1;
+    float my_prob = 0.0f;
+    for (int r = 0; r < top_k; ++r) {
+        float best = kGone;
+        int best_e = 0x7fffffff;
+#pragma unroll
+        for (int i = 0; i < kMaxPerLane; ++i) {                             // ascending expert id inside the lane: strict > keeps the lowest
+            if (score[i] > best) { best = score[i]; best_e = lane + 64 * i; }
+        }
+        const float top = wave_max(best);
+        // the lowest expert id among the lanes that hold the maximum
+        int cand = (best == top) ? best_e : 0x7fffffff;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) cand = min(cand, __shfl_xor(cand, off, 64));
+        const int owner = cand & 63, slot = cand >> 6;
+        float p = 0.0f;
+#pragma unroll
+        for (int i = 0; i < kMaxPerLane; ++i) {
+            if (lane == owner && i == slot) { p = prob[i]; score[i] = kGone; }
+        }
+        p = __shfl(p, owner, 64);
+        if (lane == r) { my_pick = cand; my_prob = p; }
+    }
+    // renormalise over the picks (lanes 0 .. top_k - 1)
+    float w;
+    if (softmax_mode) {
+        const float m = wave_max(lane < top_k ? my_prob : kGone);
+        const float ex = lane < top_k ? expf(my_prob - m) : 0.0f;
+        w = ex / group_sum<64>(ex);
+    } else {
+        const float total = group_sum<64>(lane < top_k ? my_prob : 0.0f);
+        w = my_prob / fmaxf(total, 1.0e-20f);
+    }
+    if (lane < top_k) {
+        indices[t * top_k + lane] = my_pick;
+        weights[t * top_k + lane] = w;
+    }
+}
+
+}  // namespace
+}  // namespace pllm
+
+extern "C" {
+
+int pllm_moe_route(const void* x, int x_dtype, int64_t tokens, int64_t dim, const float* gate_weight, const float* gate_bias,
+                   int64_t n_experts, int64_t top_k, int softmax_mode, float* logits, int64_t* indices, float* weights, void* stream) {
+    using namespace pllm;
+    if (!x || !gate_weight || !logits || !indices || !weights) return PLLM_ERR_INVALID_ARGUMENT;
+    if (x_dtype != PLLM_F32 && x_dtype != PLLM_F16 && x_dtype != PLLM_BF16) return PLLM_ERR_INVALID_ARGUMENT;
+    if (tokens <= 0 || dim <= 0 || n_experts <= 0 || top_k <= 0 || top_k > n_experts) return PLLM_ERR_INVALID_ARGUMENT;
+    if (n_experts > 64 * kMaxPerLane || top_k > 64 || tokens > 65535 || dim > 0x7fffffffLL) return PLLM_ERR_UNSUPPORTED;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(route_logits_kernel, dim3(static_cast<unsigned>((n_experts + kWavesPerWg - 1) / kWavesPerWg), static_cast<unsigned>(tokens)),
+                       dim3(kThreads), 0, s, x, x_dtype, gate_weight, logits, static_cast<int>(dim), static_cast<int>(n_experts));
+    hipLaunchKernelGGL(route_topk_kernel, dim3(static_cast<unsigned>(tokens)), dim3(64), 0, s, logits, gate_bias, static_cast<int>(n_experts),
+                       static_cast<int>(top_k), softmax_mode, indices, weights);
+    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+}
+
+}  // extern "C"

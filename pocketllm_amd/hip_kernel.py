@@ -504,6 +504,33 @@ def moe_group_routes(indices, weights, experts_start_idx, n_local_experts):
     return [local_ids, toks[:routes], wts[:routes], seg]
 
 
+def moe_route(x_flat: torch.Tensor, gate_weight: torch.Tensor, gate_bias, top_k: int, *, softmax: bool = False):
+    """MiniMaxMoE.route (src/models/minimax_m2/architecture.py:291-298) in two launches: (indices int64 [T, top_k],
+    weights float32 [T, top_k]) from x_flat [T, dim], gate_weight float32 [E, dim] and an optional gate_bias [E].
+    softmax=True picks the top_k logits and returns their softmax instead (the renormalised softmax routing)."""
+    _check(x_flat.dim() == 2 and gate_weight.dim() == 2 and x_flat.size(1) == gate_weight.size(1), "x_flat [T, dim] and gate_weight [E, dim] must agree on dim")
+    _check(x_flat.is_cuda and gate_weight.is_cuda and x_flat.is_contiguous() and gate_weight.is_contiguous(), "x_flat and gate_weight must be contiguous CUDA tensors")
+    _check_x(x_flat)
+    _check(gate_weight.dtype == torch.float32, "gate_weight must be float32")
+    if gate_bias is not None:
+        _check(gate_bias.is_cuda and gate_bias.dtype == torch.float32 and gate_bias.is_contiguous() and gate_bias.numel() == gate_weight.size(0),
+               "gate_bias must be a contiguous CUDA float32 tensor [E]")
+    t, e, k = x_flat.size(0), gate_weight.size(0), int(top_k)
+    _check(0 < k <= e, "top_k must be in 1..E")
+    dev = x_flat.device
+    indices = torch.empty(t, k, dtype=torch.int64, device=dev)
+    weights = torch.empty(t, k, dtype=torch.float32, device=dev)
+    if t == 0:
+        return indices, weights
+    logits = torch.empty(t, e, dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        st = _lib().pllm_moe_route(x_flat.data_ptr(), _DTYPE_CODE[x_flat.dtype], t, x_flat.size(1), gate_weight.data_ptr(),
+                                   gate_bias.data_ptr() if gate_bias is not None else None, e, k, int(bool(softmax)),
+                                   logits.data_ptr(), indices.data_ptr(), weights.data_ptr(), _stream(dev))
+    _ffi.check(st, "moe_route")
+    return indices, weights
+
+
 def gguf_single_token_route_slots(indices, weights, experts_start_idx, n_local_experts):
     """Host-side compaction of one token's routes (src/csrc/cuda_kernel.cpp:1244-1327):
     [local_ids (CPU int64), route_tokens, route_weights, route_slots, compact_starts (int32)]."""

@@ -4,7 +4,7 @@ import pytest
 import torch
 
 from oracle import gguf_oracle as O
-from pocketllm_amd import block_codec as C, codebooks
+from pocketllm_amd import _ffi, block_codec as C, codebooks
 from pocketllm_amd.cuda_loader import load_cuda_kernel
 
 pytestmark = pytest.mark.gpu
@@ -251,3 +251,52 @@ def test_grouped_experts_tile_path(mod, t13, t2, limit):
     assert O.rel_l2(y.cpu().numpy(), want) <= TOL
     y2 = mod.gguf_moe_prefill_grouped_forward(x, toks, rws, seg, dw1, dw3, dw2, d, tid[t13], d, tid[t13], inter, tid[t2], grids, limit)
     assert torch.equal(y, y2)
+
+
+@pytest.mark.parametrize("tokens,dim,n_experts,top_k", [(1, 3072, 256, 8), (7, 3072, 256, 8), (3, 1000, 60, 6), (2, 257, 1024, 64), (5, 64, 8, 8)])
+def test_router_matches_the_reference_statement(mod, tokens, dim, n_experts, top_k):
+    """MiniMaxMoE.route on the device: logits against float64, then selection and weights against the oracle evaluated on the
+    device's own logits (a float dot in another order may legitimately swap two experts whose scores differ in the last bits,
+    so the integer part of the comparison starts from identical inputs), sigmoid with and without bias and the softmax form."""
+    rng = np.random.default_rng(tokens * 31 + n_experts)
+    x = torch.from_numpy(rng.standard_normal((tokens, dim)).astype(np.float32)).to(DEV)
+    gate = torch.from_numpy((rng.standard_normal((n_experts, dim)) / np.sqrt(dim)).astype(np.float32)).to(DEV)
+    bias = torch.from_numpy(rng.uniform(-0.3, 0.3, size=n_experts).astype(np.float32)).to(DEV)
+    lib = _ffi.load_library()
+    for xd in (x, x.to(torch.bfloat16)):
+        for b, softmax in ((None, False), (bias, False), (None, True)):
+            print(f"case route t={tokens} dim={dim} e={n_experts} k={top_k} {xd.dtype} bias={b is not None} softmax={softmax}", flush=True)
+            logits = torch.empty(tokens, n_experts, device=DEV)
+            idx = torch.empty(tokens, top_k, dtype=torch.int64, device=DEV)
+            w = torch.empty(tokens, top_k, device=DEV)
+            st = lib.pllm_moe_route(xd.data_ptr(), {torch.float32: _ffi.DTYPE_F32, torch.bfloat16: _ffi.DTYPE_BF16}[xd.dtype], tokens, dim,
+                                    gate.data_ptr(), b.data_ptr() if b is not None else None, n_experts, top_k, int(softmax),
+                                    logits.data_ptr(), idx.data_ptr(), w.data_ptr(), torch.cuda.current_stream().cuda_stream)
+            assert st == 0
+            torch.cuda.synchronize()
+            want_logits = xd.double().cpu().numpy() @ gate.double().cpu().numpy().T
+            assert O.rel_l2(logits.cpu().numpy(), want_logits) < 1e-6
+            want_idx, want_w = O.route_topk(logits.cpu().numpy(), None if b is None else b.cpu().numpy(), top_k, softmax)
+            # float32 sigmoid on the device against float64 in the oracle: equal picks unless two scores sit within 1e-6
+            got_idx = idx.cpu().numpy()
+            if not np.array_equal(got_idx, want_idx):
+                l64 = logits.double().cpu().numpy()
+                sc = l64 if softmax else 1.0 / (1.0 + np.exp(-l64)) + (0.0 if b is None else b.double().cpu().numpy()[None, :])
+                for t in range(tokens):
+                    assert sorted(got_idx[t].tolist()) == sorted(want_idx[t].tolist()) or \
+                        np.abs(np.sort(np.take(sc[t], got_idx[t])) - np.sort(np.take(sc[t], want_idx[t]))).max() < 1e-6
+                    assert np.all(np.diff(np.take(sc[t], got_idx[t])) <= 1e-6)      # descending
+            else:
+                np.testing.assert_allclose(w.cpu().numpy(), want_w, rtol=2e-6, atol=1e-8)
+            assert np.allclose(w.sum(dim=1).cpu().numpy(), 1.0, atol=1e-5)
+    # the operator form, and what the reference's own op chain gives
+    i2, w2 = mod.moe_route(x, gate, bias, top_k)
+    probs = torch.sigmoid(x @ gate.t())
+    _, ri = torch.topk(probs + bias, k=top_k, dim=-1)
+    rw = torch.gather(probs, -1, ri)
+    rw = rw / rw.sum(dim=-1, keepdim=True).clamp_min(1e-20)
+    same = (i2 == ri).all(dim=1)
+    assert same.float().mean() >= 0.5                      # rows without near-ties agree pick for pick
+    assert torch.allclose(w2[same], rw[same], rtol=1e-4, atol=1e-7)
+    with pytest.raises(RuntimeError, match="top_k must be in"):
+        mod.moe_route(x, gate, None, n_experts + 1)

@@ -506,3 +506,27 @@ def test_fp8_fp16scale_expectation_indexing_and_reference_bit_decode():
         assert abs(got[b, r] - want) <= 1e-9 * max(1.0, abs(want))
     g, u = np.array([0.0, 1.0, -2.0]), np.array([3.0, 2.0, 1.0])
     np.testing.assert_allclose(O.silu_mul(g, u), [0.0, 2.0 / (1.0 + np.exp(-1.0)), -2.0 / (1.0 + np.exp(2.0))], rtol=1e-15)
+
+
+def test_route_topk_closed_forms():
+    """Routing restatement against hand-computed cases: sigmoid scores with a bias that changes the selection but not the
+    weights; softmax routing equals softmax -> top-k -> renormalise."""
+    logits = np.array([[0.0, 2.0, -1.0, 1.0]])
+    idx, w = O.route_topk(logits, None, 2)
+    p = 1.0 / (1.0 + np.exp(-np.array([2.0, 1.0])))
+    assert idx.tolist() == [[1, 3]]
+    np.testing.assert_allclose(w[0], p / p.sum(), rtol=1e-15)
+    idx, w = O.route_topk(logits, np.array([0.0, -1.0, 0.9, 0.0]), 2)       # scores 0.5, -0.119, 1.169, 0.731: picks 2 then 3
+    p = 1.0 / (1.0 + np.exp(-np.array([-1.0, 1.0])))
+    assert idx.tolist() == [[2, 3]]
+    np.testing.assert_allclose(w[0], p / p.sum(), rtol=1e-15)                 # the bias never enters the weights
+    rng = np.random.default_rng(0)
+    lg = rng.standard_normal((5, 32))
+    idx, w = O.route_topk(lg, None, 4, softmax=True)
+    sm = np.exp(lg) / np.exp(lg).sum(axis=1, keepdims=True)
+    for t in range(5):
+        top = np.argsort(-sm[t])[:4]
+        assert idx[t].tolist() == top.tolist()
+        np.testing.assert_allclose(w[t], sm[t, top] / sm[t, top].sum(), rtol=1e-12)
+    idx, _ = O.route_topk(np.zeros((1, 6)), None, 3)
+    assert idx.tolist() == [[0, 1, 2]]                                        # equal scores: lower expert id first
