@@ -158,10 +158,13 @@ __device__ __forceinline__ void store_any(void* y, int y_dtype, size_t i, float 
 
 // Workgroup-wide quantization of one activation row straight into LDS, the same image the
 // pre-pass kernel writes to memory (blockDim.x a multiple of 8, kpad a multiple of 256).  Four
-// consecutive values per lane and trip: one 8-byte load for 16-bit inputs when the row allows it.
+// consecutive values per lane and trip, fetched by one vector load when the row's alignment allows it.
 // The loads of BATCH trips are issued together so that a row costs one or two memory round trips.
-__device__ __forceinline__ void load_row4(float v[4], const void* __restrict__ x, int x_dtype, size_t xoff, int e0, int k, bool narrow) {
-    if (narrow && e0 + 3 < k) {
+__device__ __forceinline__ void load_row4(float v[4], const void* __restrict__ x, int x_dtype, size_t xoff, int e0, int k, bool vec) {
+    if (vec && e0 + 3 < k && x_dtype == PLLM_F32) {
+        const float4 w = *reinterpret_cast<const float4*>(static_cast<const float*>(x) + xoff + e0);
+        v[0] = w.x; v[1] = w.y; v[2] = w.z; v[3] = w.w;
+    } else if (vec && e0 + 3 < k) {
         const uint2 w = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(x) + xoff + e0);
         if (x_dtype == PLLM_BF16) {
             v[0] = __uint_as_float(w.x << 16); v[1] = __uint_as_float(w.x & 0xffff0000u);
@@ -195,13 +198,15 @@ __device__ __forceinline__ void quantize_row_to_lds(unsigned char* lds, const vo
     int8_t* lo = hi + kpad;
     float2* gs = reinterpret_cast<float2*>(lo + kpad);
     float* sum16 = reinterpret_cast<float*>(gs + kpad / 32);
-    const bool narrow = x_dtype != PLLM_F32 && ((reinterpret_cast<uintptr_t>(x) + 2 * xoff) & 7u) == 0;
+    // one 8-byte (16-bit inputs) or 16-byte (float32) load per lane and trip when the row starts on that boundary
+    const bool vec = x_dtype == PLLM_F32 ? ((reinterpret_cast<uintptr_t>(x) + 4 * xoff) & 15u) == 0
+                                         : ((reinterpret_cast<uintptr_t>(x) + 2 * xoff) & 7u) == 0;
     const int trip = static_cast<int>(blockDim.x) * 4;
     for (int base = static_cast<int>(threadIdx.x) * 4; base < kpad; base += trip * BATCH) {
         float v[BATCH][4];
 #pragma unroll
         for (int j = 0; j < BATCH; ++j)
-            if (base + j * trip < kpad) load_row4(v[j], x, x_dtype, xoff, base + j * trip, k, narrow);
+            if (base + j * trip < kpad) load_row4(v[j], x, x_dtype, xoff, base + j * trip, k, vec);
 #pragma unroll
         for (int j = 0; j < BATCH; ++j)
             if (base + j * trip < kpad) quantize4_to_image(v[j], base + j * trip, hi, lo, gs, sum16);
