@@ -82,25 +82,32 @@ static bool quantizes_in_kernel(int type_id, int64_t n, int64_t bpr) {
     return pllm_gguf_block_bytes(type_id) != 0;
 }
 
-static int superblock_matvec(const pllm::ActRows& act, const uint8_t* blocks, int type_id, void* y, int y_dtype,
-                             int rows, int n, int bpr, hipStream_t s) {
+}  // extern "C"
+
+namespace pllm {
+int superblock_matvec(const ActRows& act, const uint8_t* blocks, int type_id, void* y, int y_dtype,
+                      int rows, int n, int bpr, hipStream_t s, WeightRoute route) {
     switch (type_id) {
         case PLLM_TYPE_Q2_K:
-            return pllm::dot4_matvec_from_image(act, blocks, type_id, y, y_dtype, rows, n, bpr, s);
+            return dot4_matvec_from_image(act, blocks, type_id, y, y_dtype, rows, n, bpr, s, route);
         case PLLM_TYPE_IQ2_XXS:
         case PLLM_TYPE_IQ1_M:
         case PLLM_TYPE_IQ2_XS:
         case PLLM_TYPE_IQ3_XXS:
         case PLLM_TYPE_IQ4_XS:
         case PLLM_TYPE_Q6_K:
-            return pllm::iq_mfma_matvec_from_image(act, blocks, type_id, y, y_dtype, rows, n, bpr, s);
+            return iq_mfma_matvec_from_image(act, blocks, type_id, y, y_dtype, rows, n, bpr, s, route);
         case PLLM_TYPE_Q4_K:
         case PLLM_TYPE_Q5_K:
-            return pllm::kquant_matvec_from_image(act, blocks, type_id, y, y_dtype, rows, n, bpr, s);
+            return kquant_matvec_from_image(act, blocks, type_id, y, y_dtype, rows, n, bpr, s, route);
         default:
             return PLLM_ERR_UNSUPPORTED;
     }
 }
+}  // namespace pllm
+using pllm::superblock_matvec;
+
+extern "C" {
 
 int pllm_gguf_quant_gemm(const void* x, int x_dtype, const uint8_t* blocks, int type_id, void* y, int y_dtype,
                          int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row,

@@ -890,6 +890,10 @@ int gemm_f16_grouped(const void* staged, const uint8_t* w, int type_id, size_t g
         case PLLM_TYPE_Q2_K: return launch_gemm_mi<GQ2K>(p, xh, xscale, w, y, PLLM_F32, nullptr, rows, n, bpr, nullptr, 0, seg, group_stride, groups, stream);
         case PLLM_TYPE_IQ2_XXS: return launch_gemm_mi<GIQ2XXS>(p, xh, xscale, w, y, PLLM_F32, nullptr, rows, n, bpr, nullptr, 0, seg, group_stride, groups, stream);
         case PLLM_TYPE_IQ1_M: return launch_gemm_mi<GIQ1M>(p, xh, xscale, w, y, PLLM_F32, nullptr, rows, n, bpr, nullptr, 0, seg, group_stride, groups, stream);
+        case PLLM_TYPE_Q6_K: return launch_gemm_mi<GQ6K>(p, xh, xscale, w, y, PLLM_F32, nullptr, rows, n, bpr, nullptr, 0, seg, group_stride, groups, stream);
+        case PLLM_TYPE_IQ4_XS: return launch_gemm_mi<GIQ4XS>(p, xh, xscale, w, y, PLLM_F32, nullptr, rows, n, bpr, nullptr, 0, seg, group_stride, groups, stream);
+        case PLLM_TYPE_IQ2_XS: return launch_gemm_mi<GIQ2XS>(p, xh, xscale, w, y, PLLM_F32, nullptr, rows, n, bpr, nullptr, 0, seg, group_stride, groups, stream);
+        case PLLM_TYPE_IQ3_XXS: return launch_gemm_mi<GIQ3XXS>(p, xh, xscale, w, y, PLLM_F32, nullptr, rows, n, bpr, nullptr, 0, seg, group_stride, groups, stream);
         default: return PLLM_ERR_UNSUPPORTED;
     }
 }

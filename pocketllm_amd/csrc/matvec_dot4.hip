@@ -48,7 +48,8 @@ __global__ __launch_bounds__(64 * kMaxWaves) void dot4_matvec_kernel(
             FMT::load(regs[it], wrow + static_cast<size_t>(b) * FMT::kBlockBytes, j);
         }
         if (!staged) {                       // first trip of every thread of the workgroup
-            if constexpr (!RAW) copy_to_lds(smem, act.image + static_cast<size_t>(blockIdx.y) * act.stride, image_bytes);
+            if constexpr (!RAW)
+                copy_to_lds(smem, act.image + (act.row_token ? static_cast<size_t>(act.row_token[blockIdx.y]) : blockIdx.y) * act.stride, image_bytes);
             FMT::stage_tables(tables);
             __syncthreads();
             staged = true;
@@ -118,8 +119,8 @@ static int dot4_dispatch(const ActRows& act, const uint8_t* w, int type_id, void
 }
 
 int dot4_matvec_from_image(const ActRows& act, const uint8_t* w, int type_id, void* y, int y_dtype,
-                           int rows, int n, int bpr, hipStream_t stream) {
-    return dot4_dispatch(act, w, type_id, y, y_dtype, rows, n, bpr, nullptr, 0, stream);
+                           int rows, int n, int bpr, hipStream_t stream, WeightRoute route) {
+    return dot4_dispatch(act, w, type_id, y, y_dtype, rows, n, bpr, route.expert, route.expert_stride, stream);
 }
 
 int dot4_routed_matvec_from_image(const unsigned char* image, size_t stride, const uint8_t* w, int type_id, void* y, int y_dtype,

@@ -26,13 +26,15 @@ constexpr int kWaves = 8;
 // they are in flight the workgroup fills LDS with the activation image and the format's codebooks.
 template <typename FMT, int ITERS, bool RAW>
 __global__ __launch_bounds__(64 * kWaves) void mfma_tile_matvec_kernel(
-    const ActRows act, const uint8_t* __restrict__ w, void* __restrict__ y, int y_dtype, int n, int bpr) {
+    const ActRows act, const WeightRoute route, const uint8_t* __restrict__ w, void* __restrict__ y, int y_dtype, int n, int bpr) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int kpad = bpr * 256;
     const int image_bytes = static_cast<int>(staged_x_bytes(kpad));
     const StagedX sx = carve_staged_x(smem, kpad);
     const int zero_off = image_bytes;                                        // 16 zero bytes
     unsigned char* tables = smem + image_bytes + 16;
+    if (route.expert) w += static_cast<size_t>(route.expert[blockIdx.y]) * route.expert_stride;
+    const size_t image_row = act.row_token ? static_cast<size_t>(act.row_token[blockIdx.y]) : blockIdx.y;
     float* partial = reinterpret_cast<float*>(tables + FMT::kTableBytes);   // [waves][16]
 
     const int tid = threadIdx.x;
@@ -60,7 +62,7 @@ __global__ __launch_bounds__(64 * kWaves) void mfma_tile_matvec_kernel(
             FMT::load(regs[it], wrow + static_cast<size_t>(b) * FMT::kBlockBytes, ks);
         }
         if (!staged) {                       // first trip of every thread of the workgroup
-            if constexpr (!RAW) copy_to_lds(smem, act.image + static_cast<size_t>(blockIdx.y) * act.stride, image_bytes);
+            if constexpr (!RAW) copy_to_lds(smem, act.image + image_row * act.stride, image_bytes);
             if (tid < 4) reinterpret_cast<uint32_t*>(smem + zero_off)[tid] = 0;
             FMT::stage_tables(tables);
             __syncthreads();
@@ -85,7 +87,7 @@ __global__ __launch_bounds__(64 * kWaves) void mfma_tile_matvec_kernel(
 }
 
 template <typename FMT, int ITERS, bool RAW>
-int launch_tile(const ActRows& act, const uint8_t* w, void* y, int y_dtype,
+int launch_tile(const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype,
                 int rows, int n, int bpr, int waves, hipStream_t stream) {
     const size_t smem = staged_x_bytes(bpr * 256) + 16 + FMT::kTableBytes + static_cast<size_t>(waves) * kRowsPerTile * sizeof(float);
     auto kern = mfma_tile_matvec_kernel<FMT, ITERS, RAW>;
@@ -96,12 +98,12 @@ int launch_tile(const ActRows& act, const uint8_t* w, void* y, int y_dtype,
             return PLLM_ERR_UNSUPPORTED;
     }
     dim3 grid((n + kRowsPerTile - 1) / kRowsPerTile, rows);
-    hipLaunchKernelGGL(kern, grid, dim3(64 * waves), smem, stream, act, w, y, y_dtype, n, bpr);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * waves), smem, stream, act, route, w, y, y_dtype, n, bpr);
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 
 template <typename FMT>
-int launch_tiles(const ActRows& act, const uint8_t* w, void* y, int y_dtype,
+int launch_tiles(const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype,
                  int rows, int n, int bpr, hipStream_t stream) {
     // waves per workgroup: split a row's blocks so that every wave keeps a handful in flight
     int waves = 1;
@@ -109,8 +111,8 @@ int launch_tiles(const ActRows& act, const uint8_t* w, void* y, int y_dtype,
     const int niter = (bpr + waves - 1) / waves;
     const int passes = (niter + 5) / 6;
     const int iters = (niter + passes - 1) / passes;
-#define PLLM_CASE(I) case I: return act.x ? launch_tile<FMT, I, true>(act, w, y, y_dtype, rows, n, bpr, waves, stream) \
-                                          : launch_tile<FMT, I, false>(act, w, y, y_dtype, rows, n, bpr, waves, stream)
+#define PLLM_CASE(I) case I: return act.x ? launch_tile<FMT, I, true>(act, route, w, y, y_dtype, rows, n, bpr, waves, stream) \
+                                          : launch_tile<FMT, I, false>(act, route, w, y, y_dtype, rows, n, bpr, waves, stream)
     switch (iters) {
         PLLM_CASE(1); PLLM_CASE(2); PLLM_CASE(3); PLLM_CASE(4); PLLM_CASE(5);
         default: PLLM_CASE(6);
@@ -285,26 +287,27 @@ int launch_stream(const ActRows& act, const uint8_t* w, void* y, int y_dtype,
 }
 
 template <typename FMT>
-int launch_fmt(const ActRows& act, const uint8_t* w, void* y, int y_dtype,
+int launch_fmt(const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype,
                int rows, int n, int bpr, hipStream_t stream) {
     // whole tiles streamed through long-lived workgroups (the codebooks are staged once per workgroup)
-    // where shape and alignment allow, else one short workgroup per tile
+    // where shape and alignment allow, else one short workgroup per tile; routed calls always take the latter
     if constexpr (FMT::kStreamed)
-        if (const int split = stream_split<FMT>(w, n, bpr)) return launch_stream<FMT>(act, w, y, y_dtype, rows, n, bpr, split, stream);
-    return launch_tiles<FMT>(act, w, y, y_dtype, rows, n, bpr, stream);
+        if (!route.expert && !act.row_token)
+            if (const int split = stream_split<FMT>(w, n, bpr)) return launch_stream<FMT>(act, w, y, y_dtype, rows, n, bpr, split, stream);
+    return launch_tiles<FMT>(act, route, w, y, y_dtype, rows, n, bpr, stream);
 }
 
 }  // namespace
 
 int iq_mfma_matvec_from_image(const ActRows& act, const uint8_t* w, int type_id, void* y, int y_dtype,
-                              int rows, int n, int bpr, hipStream_t stream) {
+                              int rows, int n, int bpr, hipStream_t stream, WeightRoute route) {
     switch (type_id) {
-        case PLLM_TYPE_IQ2_XXS: return launch_fmt<IQ2XXSm>(act, w, y, y_dtype, rows, n, bpr, stream);
-        case PLLM_TYPE_IQ1_M: return launch_fmt<IQ1Mm>(act, w, y, y_dtype, rows, n, bpr, stream);
-        case PLLM_TYPE_IQ2_XS: return launch_fmt<IQ2XSm>(act, w, y, y_dtype, rows, n, bpr, stream);
-        case PLLM_TYPE_IQ3_XXS: return launch_fmt<IQ3XXSm>(act, w, y, y_dtype, rows, n, bpr, stream);
-        case PLLM_TYPE_IQ4_XS: return launch_fmt<IQ4XSm>(act, w, y, y_dtype, rows, n, bpr, stream);
-        case PLLM_TYPE_Q6_K: return launch_fmt<Q6Km>(act, w, y, y_dtype, rows, n, bpr, stream);
+        case PLLM_TYPE_IQ2_XXS: return launch_fmt<IQ2XXSm>(act, route, w, y, y_dtype, rows, n, bpr, stream);
+        case PLLM_TYPE_IQ1_M: return launch_fmt<IQ1Mm>(act, route, w, y, y_dtype, rows, n, bpr, stream);
+        case PLLM_TYPE_IQ2_XS: return launch_fmt<IQ2XSm>(act, route, w, y, y_dtype, rows, n, bpr, stream);
+        case PLLM_TYPE_IQ3_XXS: return launch_fmt<IQ3XXSm>(act, route, w, y, y_dtype, rows, n, bpr, stream);
+        case PLLM_TYPE_IQ4_XS: return launch_fmt<IQ4XSm>(act, route, w, y, y_dtype, rows, n, bpr, stream);
+        case PLLM_TYPE_Q6_K: return launch_fmt<Q6Km>(act, route, w, y, y_dtype, rows, n, bpr, stream);
         default: return PLLM_ERR_UNSUPPORTED;
     }
 }

@@ -100,7 +100,7 @@ struct Q5K {
 
 template <typename FMT, int ITERS, bool RAW>
 __global__ __launch_bounds__(64 * kMaxWaves) void k45_mfma_matvec_kernel(
-    const ActRows act, const uint8_t* __restrict__ w, void* __restrict__ y, int y_dtype, int n, int bpr) {
+    const ActRows act, const WeightRoute route, const uint8_t* __restrict__ w, void* __restrict__ y, int y_dtype, int n, int bpr) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int kpad = bpr * 256;
     const int image_bytes = static_cast<int>(staged_x_bytes(kpad));
@@ -115,6 +115,8 @@ __global__ __launch_bounds__(64 * kMaxWaves) void k45_mfma_matvec_kernel(
     const int col = lane & 15;        // B/C column = output row within the tile; also A's row index m
     const int ks = lane >> 4;         // k slice of A and B, row quad of C
     const int row = blockIdx.x * kRowsPerWg + col;
+    if (route.expert) w += static_cast<size_t>(route.expert[blockIdx.y]) * route.expert_stride;
+    const size_t image_row = act.row_token ? static_cast<size_t>(act.row_token[blockIdx.y]) : blockIdx.y;
     const uint8_t* wrow = w + static_cast<size_t>(row < n ? row : 0) * bpr * FMT::kBlockBytes;
 
     // A side: this lane supplies row m = col = 2 * group + term of MFMA t, slice ks; it is non-zero
@@ -144,7 +146,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void k45_mfma_matvec_kernel(
             FMT::load(regs[it], wrow + static_cast<size_t>(b) * FMT::kBlockBytes, ks);
         }
         if (!staged) {                       // first trip of every thread of the workgroup
-            copy_to_lds(smem, act.image + static_cast<size_t>(blockIdx.y) * act.stride, image_bytes);
+            copy_to_lds(smem, act.image + image_row * act.stride, image_bytes);
             if (tid < 4) reinterpret_cast<uint32_t*>(smem + zero_off)[tid] = 0;
             __syncthreads();
             staged = true;
@@ -190,7 +192,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void k45_mfma_matvec_kernel(
 
 // ------------------------------------------------------------------------------------------------
 template <typename KERN>
-int launch_kernel(KERN kern, const ActRows& act, const uint8_t* w, void* y, int y_dtype,
+int launch_kernel(KERN kern, const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype,
                   int rows, int n, int bpr, int waves, hipStream_t stream) {
     const size_t smem = staged_x_bytes(bpr * 256) + 16 + static_cast<size_t>(waves) * kRowsPerWg * sizeof(float);
     if (smem > 64 * 1024) {
@@ -200,7 +202,7 @@ int launch_kernel(KERN kern, const ActRows& act, const uint8_t* w, void* y, int 
             return PLLM_ERR_UNSUPPORTED;
     }
     dim3 grid((n + kRowsPerWg - 1) / kRowsPerWg, rows);
-    hipLaunchKernelGGL(kern, grid, dim3(64 * waves), smem, stream, act, w, y, y_dtype, n, bpr);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * waves), smem, stream, act, route, w, y, y_dtype, n, bpr);
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 
@@ -215,11 +217,11 @@ void split_blocks(int bpr, int& waves, int& iters) {
 }
 
 template <typename FMT>
-int launch_k45(const ActRows& act, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream) {
+int launch_k45(const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream) {
     int waves, iters;
     split_blocks(bpr, waves, iters);
-#define PLLM_CASE(I) case I: return act.x ? launch_kernel(k45_mfma_matvec_kernel<FMT, I, true>, act, w, y, y_dtype, rows, n, bpr, waves, stream) \
-                                          : launch_kernel(k45_mfma_matvec_kernel<FMT, I, false>, act, w, y, y_dtype, rows, n, bpr, waves, stream)
+#define PLLM_CASE(I) case I: return act.x ? launch_kernel(k45_mfma_matvec_kernel<FMT, I, true>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream) \
+                                          : launch_kernel(k45_mfma_matvec_kernel<FMT, I, false>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream)
     switch (iters) {
         PLLM_CASE(1); PLLM_CASE(2); PLLM_CASE(3); PLLM_CASE(4); PLLM_CASE(5); PLLM_CASE(6);
         default: PLLM_CASE(8);
@@ -232,10 +234,10 @@ int launch_k45(const ActRows& act, const uint8_t* w, void* y, int y_dtype, int r
 size_t kquant_matvec_workspace_bytes(int rows, int bpr) { return act_image_256_bytes(bpr) * static_cast<size_t>(rows); }
 
 int kquant_matvec_from_image(const ActRows& act, const uint8_t* w, int type_id, void* y, int y_dtype,
-                             int rows, int n, int bpr, hipStream_t stream) {
+                             int rows, int n, int bpr, hipStream_t stream, WeightRoute route) {
     switch (type_id) {
-        case PLLM_TYPE_Q4_K: return launch_k45<Q4K>(act, w, y, y_dtype, rows, n, bpr, stream);
-        case PLLM_TYPE_Q5_K: return launch_k45<Q5K>(act, w, y, y_dtype, rows, n, bpr, stream);
+        case PLLM_TYPE_Q4_K: return launch_k45<Q4K>(act, route, w, y, y_dtype, rows, n, bpr, stream);
+        case PLLM_TYPE_Q5_K: return launch_k45<Q5K>(act, route, w, y, y_dtype, rows, n, bpr, stream);
         default: return PLLM_ERR_UNSUPPORTED;
     }
 }

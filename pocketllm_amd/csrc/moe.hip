@@ -59,6 +59,38 @@ __device__ __forceinline__ void store_hidden(float g, float u, float limit, floa
 }
 
 
+// Hidden images of the route-by-route path: h = SiLU(min(g, L)) * clamp(u, +-L) * route weight (the clamp only for L > 0)
+// from the float32 gate and up products [routes, inter], quantized into the image the down projection reads.
+__global__ __launch_bounds__(256) void swiglu_image_kernel(
+    const float* __restrict__ gate, const float* __restrict__ up, const float* __restrict__ route_weights, float limit, int inter, int h_kpad,
+    unsigned char* __restrict__ h_image, size_t h_stride) {
+    const int e0 = (blockIdx.x * 256 + threadIdx.x) * 4;
+    if (e0 >= h_kpad) return;                                   // h_kpad is a multiple of 256: whole groups leave together
+    const size_t r = blockIdx.y;
+    unsigned char* base = h_image + r * h_stride;
+    int8_t* hi = reinterpret_cast<int8_t*>(base);
+    int8_t* lo = hi + h_kpad;
+    float2* gs = reinterpret_cast<float2*>(lo + h_kpad);
+    float* sum16 = reinterpret_cast<float*>(gs + h_kpad / 32);
+    const float rw = route_weights[r];
+    float v[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        float h = 0.0f;
+        if (e0 + i < inter) {
+            float g = gate[r * inter + e0 + i], u = up[r * inter + e0 + i];
+            if (limit > 0.0f) {
+                u = fminf(fmaxf(u, -limit), limit);
+                g = fminf(g, limit);
+            }
+            h = g / (1.0f + expf(-g)) * u * rw;
+        }
+        v[i] = h;
+    }
+    quantize4_to_image(v, e0, hi, lo, gs, sum16);
+}
+
+
 template <typename FMT>
 __global__ __launch_bounds__(256 * kW13Split) void moe_w13_kernel(
     const unsigned char* __restrict__ x_image, size_t x_image_stride, int bpr,
@@ -469,8 +501,11 @@ extern "C" {
 size_t pllm_gguf_moe_workspace_bytes(int64_t tokens, int64_t routes, int64_t dim, int64_t inter) {
     if (tokens <= 0 || routes < 0 || dim <= 0 || inter <= 0) return 0;
     const int bpr_x = static_cast<int>((dim + 255) / 256), bpr_h = static_cast<int>((inter + 255) / 256);
+    // images of the tokens and of the routes' hidden rows, per-route outputs, narrow expert ids, and (route-by-route path of the
+    // types without fused expert kernels) the float32 gate and up products
     const size_t dot_path = pllm::act_image_256_bytes(bpr_x) * static_cast<size_t>(tokens) + pllm::act_image_256_bytes(bpr_h) * static_cast<size_t>(routes) +
-                            pllm::align256(static_cast<size_t>(routes) * dim * sizeof(float)) + pllm::align256(static_cast<size_t>(routes) * sizeof(int32_t)) + 256;
+                            pllm::align256(static_cast<size_t>(routes) * dim * sizeof(float)) + pllm::align256(static_cast<size_t>(routes) * sizeof(int32_t)) +
+                            2 * pllm::align256(static_cast<size_t>(routes) * inter * sizeof(float)) + 256;
     if (tokens < pllm::kMoeGemmMinTokens || routes > INT32_MAX) return dot_path;
     const int R = static_cast<int>(routes);
     const size_t tile_path = pllm::gemm_f16_staged_bytes(R, bpr_x) + pllm::gemm_f16_staged_bytes(R, bpr_h) +
@@ -494,7 +529,7 @@ int pllm_gguf_moe_forward(const void* x, int x_dtype, int64_t tokens, int64_t di
         return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
     }
     if (!w1 || !w3 || !w2 || !route_weights || (!route_experts && !seg_starts)) return PLLM_ERR_INVALID_ARGUMENT;
-    if (!dot4_type(w13_type) || !dot4_type(w2_type)) return PLLM_ERR_UNSUPPORTED;
+    if (pllm_gguf_block_bytes(w13_type) == 0 || pllm_gguf_block_bytes(w2_type) == 0) return PLLM_ERR_UNSUPPORTED;
     if (tokens > 65535 || routes > 65535 || dim > (1 << 24) || inter > (1 << 24)) return PLLM_ERR_UNSUPPORTED;
     if (tokens > 1 && !route_tokens) return PLLM_ERR_INVALID_ARGUMENT;
     if (!workspace || workspace_bytes < pllm_gguf_moe_workspace_bytes(tokens, routes, dim, inter)) return PLLM_ERR_WORKSPACE;
@@ -548,6 +583,41 @@ int pllm_gguf_moe_forward(const void* x, int x_dtype, int64_t tokens, int64_t di
         return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
     }
     const size_t x_stride = act_image_256_bytes(bpr_x), h_stride = act_image_256_bytes(bpr_h);
+    if (!dot4_type(w13_type) || !dot4_type(w2_type)) {
+        // Types without fused expert kernels (Q4_K, Q5_K, Q6_K, IQ4_XS, IQ2_XS, IQ3_XXS), below the tile path's token count: route
+        // by route through the dense decode kernels in their routed form (grid row = route, matrix = the route's expert, activation
+        // image = the route's token): gate, up, SwiGLU into hidden images, down, ordered sum per token.
+        unsigned char* p = static_cast<unsigned char*>(workspace);
+        unsigned char* x_image = p;  p += x_stride * tokens;
+        unsigned char* h_image = p;  p += h_stride * routes;
+        float* partial = reinterpret_cast<float*>(p);  p += align256(static_cast<size_t>(routes) * dim * sizeof(float));
+        int32_t* experts32 = reinterpret_cast<int32_t*>(p);  p += align256(static_cast<size_t>(routes) * sizeof(int32_t));
+        float* gate = reinterpret_cast<float*>(p);  p += align256(static_cast<size_t>(routes) * inter * sizeof(float));
+        float* up = reinterpret_cast<float*>(p);
+        const int R = static_cast<int>(routes), I = static_cast<int>(inter), D = static_cast<int>(dim);
+        if (route_experts) hipLaunchKernelGGL(narrow_experts_kernel, dim3((R + 255) / 256), dim3(256), 0, s, route_experts, experts32, R);
+        else hipLaunchKernelGGL(expand_segments_kernel, dim3(static_cast<unsigned>(n_experts)), dim3(256), 0, s, seg_starts, experts32, static_cast<int>(n_experts));
+        if (hipGetLastError() != hipSuccess) return PLLM_ERR_LAUNCH;
+        int st = act_image_256(x, x_dtype, static_cast<int>(tokens), D, bpr_x, x_image, s);
+        if (st != PLLM_OK) return st;
+        // one token: every route reads image 0 (stride 0); several: the route's token picks the image
+        const ActRows xa = act_rows_from_image(x_image, tokens > 1 ? x_stride : 0, tokens > 1 ? route_tokens : nullptr);
+        const WeightRoute r13{experts32, static_cast<size_t>(inter) * bpr_x * pllm_gguf_block_bytes(w13_type)};
+        const WeightRoute r2{experts32, static_cast<size_t>(dim) * bpr_h * pllm_gguf_block_bytes(w2_type)};
+        st = superblock_matvec(xa, w1, w13_type, gate, PLLM_F32, R, I, bpr_x, s, r13);
+        if (st != PLLM_OK) return st;
+        st = superblock_matvec(xa, w3, w13_type, up, PLLM_F32, R, I, bpr_x, s, r13);
+        if (st != PLLM_OK) return st;
+        const int h_kpad = bpr_h * 256;
+        hipLaunchKernelGGL(swiglu_image_kernel, dim3((h_kpad / 4 + 255) / 256, R), dim3(256), 0, s, gate, up, route_weights, swiglu_limit, I, h_kpad,
+                           h_image, h_stride);
+        if (hipGetLastError() != hipSuccess) return PLLM_ERR_LAUNCH;
+        st = superblock_matvec(act_rows_from_image(h_image, h_stride), w2, w2_type, partial, PLLM_F32, R, D, bpr_h, s, r2);
+        if (st != PLLM_OK) return st;
+        dim3 rg(static_cast<unsigned>(tokens), static_cast<unsigned>((dim + 255) / 256));
+        hipLaunchKernelGGL(moe_reduce_kernel, rg, dim3(256), 0, s, partial, tokens > 1 ? route_tokens : nullptr, y, R, D);
+        return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+    }
     if (tokens == 1 && route_experts && routes * staged_x_bytes(bpr_h * 256) <= 96 * 1024) {
         // single token: two launches.  Gate/up read the raw activation row and the int64 expert ids
         // themselves; the down projection sums the routes in order inside the kernel.

@@ -336,20 +336,27 @@ def gguf_quant_gemm_pair_forward(x, blocks0, row_elems0, type_id0, blocks1, row_
 
 # ---- routed experts --------------------------------------------------------------------------------
 
-_MOE_TYPES = (0, 1, 2)   # iq2_xxs, q2_k, iq1_m: the types the fused expert kernels read
+_MOE_TYPES = IMPLEMENTED_TYPE_IDS   # iq2_xxs, q2_k, iq1_m have fused expert kernels; the other six run route by route or as tile matmuls
+
+# codebook families: one grid tensor serves a family (src/csrc/cuda_kernel.cpp:717-722)
+_GRID_FAMILY = {0: 0, 2: 2, 5: 5, 6: 5}
+_FAMILY_NAME = {0: "iq2_xxs", 2: "iq1_m", 5: "iq2_xs/iq3_xxs"}
 
 
 def _grids_ok(grid, type_ids, name: str) -> None:
-    """The reference takes ONE grid tensor and refuses to mix iq2_xxs with iq1_m
-    (src/csrc/cuda_kernel.cpp:717-722).  Passing a tuple/list of grids lifts that limit: one entry
-    per codebook type in use, checked like the reference checks its single grid."""
-    need = sorted({t for t in type_ids if t in (0, 2)})
+    """The reference takes ONE grid tensor and refuses to mix codebook families (iq2_xxs, iq1_m, iq2_xs/iq3_xxs:
+    src/csrc/cuda_kernel.cpp:717-722).  Passing a tuple/list of grids lifts that limit: one entry per family in use,
+    in the order iq2_xxs, iq1_m, iq2_xs/iq3_xxs, each checked like the reference checks its single grid."""
+    need = sorted({_GRID_FAMILY[t] for t in type_ids if t in _GRID_FAMILY})
     if isinstance(grid, (tuple, list)):
         _check(len(grid) >= len(need), f"{name}: one grid per codebook type in use is required")
         for g, t in zip(grid, need):
             _check_grid(g, t, name)
         return
-    _check(len(need) <= 1, "grouped GGUF kernel cannot mix iq2_xxs and iq1_m because they require different grids")
+    if len(need) > 1:
+        a, b = _FAMILY_NAME[need[0]], _FAMILY_NAME[need[1]]
+        joiner = "and" if (need[0], need[1]) == (0, 2) else "with"
+        _check(False, f"grouped GGUF kernel cannot mix {a} {joiner} {b} because they require different grids")
     if need:
         _check_grid(grid, need[0], name)
 
@@ -437,15 +444,15 @@ def _single_token_checks(x, route_slots, route_weights, w1, w3, w2):
         _check(b.dtype == torch.uint8, f"{nm} has unexpected dtype")
 
 
-_TYPE_OF_BLOCK_BYTES = {66: 0, 84: 1, 56: 2}
+_TYPE_OF_BLOCK_BYTES = {GGUF_BLOCK_BYTES[t]: t for t in IMPLEMENTED_TYPE_IDS}   # the nine block sizes are distinct
 
 
 def gguf_moe_single_token_forward(x, route_slots, route_weights, w1_blocks, w3_blocks, w2_blocks, swiglu_limit) -> torch.Tensor:
     """Single-token routed experts for any mix of IQ2_XXS / Q2_K / IQ1_M matrices (types read off the
     block sizes): the case the reference cannot express because its operators take one grid tensor."""
     _single_token_checks(x, route_slots, route_weights, w1_blocks, w3_blocks, w2_blocks)
-    _check(w1_blocks.size(3) == w3_blocks.size(3) and w1_blocks.size(3) in _TYPE_OF_BLOCK_BYTES, "w1/w3 must be IQ2_XXS, Q2_K or IQ1_M blocks")
-    _check(w2_blocks.size(3) in _TYPE_OF_BLOCK_BYTES, "w2 must be IQ2_XXS, Q2_K or IQ1_M blocks")
+    _check(w1_blocks.size(3) == w3_blocks.size(3) and w1_blocks.size(3) in _TYPE_OF_BLOCK_BYTES, "w1/w3 must be blocks of one supported GGUF type")
+    _check(w2_blocks.size(3) in _TYPE_OF_BLOCK_BYTES, "w2 must be blocks of a supported GGUF type")
     return _moe_call("gguf_moe_single_token_forward", x, 1, None, route_slots, None, route_weights, w1_blocks, w3_blocks, w2_blocks,
                      _TYPE_OF_BLOCK_BYTES[w1_blocks.size(3)], _TYPE_OF_BLOCK_BYTES[w2_blocks.size(3)], swiglu_limit)
 

@@ -300,3 +300,62 @@ def test_router_matches_the_reference_statement(mod, tokens, dim, n_experts, top
     assert torch.allclose(w2[same], rw[same], rtol=1e-4, atol=1e-7)
     with pytest.raises(RuntimeError, match="top_k must be in"):
         mod.moe_route(x, gate, None, n_experts + 1)
+
+
+def _any_expert_blocks(rng, type_name, e, n, k):
+    if type_name in ("iq2_xxs", "iq1_m", "q2_k"):
+        return _expert_blocks(rng, type_name, e, n, k)
+    bpr = (k + 255) // 256
+    if type_name in ("iq2_xs", "iq3_xxs"):
+        return C.random_blocks(rng, type_name, e, n, bpr, d_range=(0.002, 0.006))
+    enc = {"q4_k": C.quantize_q4_k, "q5_k": C.quantize_q5_k, "q6_k": C.quantize_q6_k, "iq4_xs": C.quantize_iq4_xs}[type_name]
+    w = (rng.standard_normal((e * n, bpr * 256)) * 0.05).astype(np.float32)
+    w[:, k:] = 0.0
+    return enc(w).reshape(e, n, bpr, O.BLOCK_BYTES[type_name])
+
+
+@pytest.mark.parametrize("t13,t2", [("iq2_xs", "iq3_xxs"), ("q4_k", "q5_k"), ("q6_k", "iq4_xs"), ("iq2_xxs", "q4_k"), ("q5_k", "iq1_m")])
+@pytest.mark.parametrize("tokens", [1, 5, 40])
+def test_experts_in_every_block_type(mod, t13, t2, tokens):
+    """The routed operators accept all nine block types like the reference (src/csrc/cuda_kernel.cpp:714-725): types without a
+    fused expert kernel run route by route through the dense decode kernels below 16 tokens and as tile matmuls from 16 on."""
+    rng = np.random.default_rng(300 + tokens + len(t13) * 7 + len(t2))
+    e, d, inter, topk = 6, 512, 768, 3
+    w1 = _any_expert_blocks(rng, t13, e, inter, d)
+    w3 = _any_expert_blocks(rng, t13, e, inter, d)
+    w2 = _any_expert_blocks(rng, t2, e, d, inter)
+    idx, wts = _route(rng, tokens, e, topk)
+    x = torch.from_numpy(rng.standard_normal((tokens, d)).astype(np.float32)).to(DEV).to(torch.bfloat16)
+    dw1, dw3, dw2 = (torch.from_numpy(a).to(DEV) for a in (w1, w3, w2))
+    tid = O.TYPE_IDS
+    grids = tuple(codebooks.grid_tensor_for_type(t).to(DEV) for t in (0, 2, 5))
+    used = sorted({{0: 0, 2: 1, 5: 2, 6: 2}[tid[t]] for t in (t13, t2) if tid[t] in (0, 2, 5, 6)})
+    grid_arg = tuple(grids[i] for i in used) if used else torch.empty(0, dtype=torch.int8, device=DEV)
+    print(f"case experts {t13}/{t2} tokens={tokens}", flush=True)
+    for limit in (0.0, 0.5):
+        if tokens == 1:
+            y = mod.gguf_moe_single_token_forward(x, torch.from_numpy(idx[0]).to(DEV), torch.from_numpy(wts[0]).to(DEV), dw1, dw3, dw2, limit)
+            want = O.moe_forward(x.float().cpu().numpy(), np.zeros(topk, dtype=np.int64), wts[0], idx[0], w1, w3, w2, t13, t13, t2, limit)
+        else:
+            _, toks, rws, seg = mod.moe_group_routes(torch.from_numpy(idx).to(DEV), torch.from_numpy(wts).to(DEV), 0, e)
+            y = mod.gguf_moe_prefill_grouped_forward(x, toks, rws, seg, dw1, dw3, dw2, d, tid[t13], d, tid[t13], inter, tid[t2], grid_arg, limit)
+            _, o_toks, o_rws, o_seg = O.group_routes(idx, wts, 0, e)
+            want = O.moe_forward(x.float().cpu().numpy(), o_toks, o_rws, np.repeat(np.arange(e), np.diff(o_seg)), w1, w3, w2, t13, t13, t2, limit)
+        torch.cuda.synchronize()
+        assert tuple(y.shape) == (tokens, d) and y.dtype == torch.float32
+        assert O.rel_l2(y.cpu().numpy(), want) <= TOL, (t13, t2, tokens, limit)
+
+
+def test_expert_grid_families_are_checked(mod):
+    e, d, inter = 2, 256, 256
+    x = torch.randn(2, d, device=DEV)
+    toks = torch.zeros(1, dtype=torch.int64, device=DEV)
+    rws = torch.ones(1, device=DEV)
+    seg = torch.tensor([0, 1, 1], dtype=torch.int32, device=DEV)
+    w_xs = torch.zeros(e, inter, 1, 74, dtype=torch.uint8, device=DEV)
+    w_xxs = torch.zeros(e, d, 1, 66, dtype=torch.uint8, device=DEV)
+    with pytest.raises(RuntimeError, match="cannot mix iq2_xxs with iq2_xs/iq3_xxs"):
+        mod.gguf_moe_prefill_grouped_forward(x, toks, rws, seg, w_xs, w_xs, w_xxs, d, 5, d, 5, inter, 0, codebooks.grid_tensor_for_type(5).to(DEV), 0.0)
+    with pytest.raises(RuntimeError, match="packed iq2_xs and iq3_xxs signed grids"):
+        mod.gguf_moe_prefill_grouped_forward(x, toks, rws, seg, w_xs, w_xs, torch.zeros(e, d, 1, 98, dtype=torch.uint8, device=DEV), d, 5, d, 5, inter, 6,
+                                             codebooks.get_iq2xxs_signed_grid_tensor().to(DEV), 0.0)
