@@ -162,6 +162,15 @@ def extra_cases(mod, dev, iters):
         run(f"{name} matvec 17408x5120 T=1", blocks.size,
             lambda s, ring=ring, x=x, tid=tid, grid=grid: mod.gguf_quant_gemm_forward(x, ring[s], 5120, tid, grid), len(ring))
         del ring
+    # normalisation + projection as one decode operator against the two operators one after the other (Q4_K 5120x5120)
+    blocks = C.quantize_q4_k((rng.standard_normal((5120, 5120), dtype=np.float32) * np.float32(0.02)))
+    ring = ring_of(blocks, dev, max(2, min(RING, (1 << 30) // blocks.size)))
+    gamma = torch.ones(5120, device=dev)
+    run("rmsnorm + q4_k matvec 5120x5120 T=1, one operator", blocks.size,
+        lambda s, ring=ring: mod.gguf_quant_gemm_rmsnorm_forward(x, gamma, 1e-6, ring[s], 5120, 3, empty), len(ring))
+    run("rmsnorm + q4_k matvec 5120x5120 T=1, two operators", blocks.size,
+        lambda s, ring=ring: mod.gguf_quant_gemm_forward(mod.fused_rms_norm_forward(x, gamma, 1e-6), ring[s], 5120, 3, empty), len(ring))
+    del ring
     # FP8 E4M3 + 128x128 scales, BASELINE config 4 at T=1
     codes, scale = C.quantize_fp8_block((rng.standard_normal((17408, 5120), dtype=np.float32) * np.float32(0.02)))
     ring = ring_of(codes, dev, 8)

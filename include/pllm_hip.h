@@ -88,6 +88,26 @@ int pllm_gguf_quant_gemm(const void* x, int x_dtype, const uint8_t* blocks, int 
 size_t pllm_gguf_quant_gemm_workspace_bytes(int type_id, int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row);
 
 /*
+ * RMS normalisation of rows, y[r, :] = x[r, :] * rsqrt(mean(x[r, :]^2) + eps) * weight, float32 arithmetic and one rounding to
+ * y_dtype (the reference writes fp16).  Replaces fused_rms_norm_forward (src/csrc/cuda_kernel_impl.cu:9639-9730,
+ * src/csrc/cuda_kernel.cpp:2012), the normalisation the reference runs ahead of its quantized projections
+ * (src/models/minimax_m2/architecture.py:57-85).
+ *
+ * pllm_gguf_quant_gemm_rmsnorm: pllm_gguf_quant_gemm on the normalized rows without the round trip through memory,
+ *     y = W . (x * rsqrt(mean(x^2) + eps) * norm_weight).
+ * It has no counterpart in the reference (which runs the two operators one after the other) and is for decode callers: up to
+ * 4 rows are normalized and quantized inside the matvec kernel, one launch in all.  round_fp16 != 0 rounds the normalized values
+ * through fp16 first, which is what the reference's two-operator chain hands to its projection; 0 keeps float32.  More rows run
+ * the normalisation into the workspace (fp16 rows) and then the ordinary operator.
+ */
+int pllm_fused_rms_norm(const void* x, int x_dtype, const float* weight, void* y, int y_dtype, int64_t rows, int64_t dim, float eps, void* stream);
+int pllm_gguf_quant_gemm_rmsnorm(const void* x, int x_dtype, const float* norm_weight, float eps, int round_fp16,
+                                 const uint8_t* blocks, int type_id, void* y, int y_dtype,
+                                 int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row,
+                                 void* workspace, size_t workspace_bytes, void* stream);
+size_t pllm_gguf_quant_gemm_rmsnorm_workspace_bytes(int type_id, int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row);
+
+/*
  * The two halves of pllm_gguf_quant_gemm, for callers that feed one activation tensor to several
  * matrices (q/k/v, gate/up): quantize once into `image` (pllm_activation_image_bytes bytes, 256-byte
  * aligned), then run any number of matmuls against it (the decode kernels, whatever the row count).  They have no counterpart in the

@@ -544,6 +544,16 @@ def swiglu_route(gate: np.ndarray, up: np.ndarray, route_w: np.ndarray, limit: f
     return g / (1.0 + np.exp(-g)) * u * route_w.astype(np.float64)[:, None]
 
 
+def rms_norm(x: np.ndarray, weight: np.ndarray, eps: float) -> np.ndarray:
+    """x * rsqrt(mean(x^2) + eps) * weight per row, in float64 (no output rounding).
+
+    Reference: fused_rms_norm_kernel, src/csrc/cuda_kernel_impl.cu:9639-9697 (float32 there, output rounded to fp16), and the
+    framework fallback src/models/minimax_m2/architecture.py:77-85.  Pinned by closed forms in tests/test_oracle_pinning.py."""
+    xf = x.astype(np.float64)
+    inv = 1.0 / np.sqrt((xf * xf).mean(axis=-1, keepdims=True) + float(eps))
+    return xf * inv * weight.astype(np.float64)
+
+
 def route_topk(logits: np.ndarray, bias, top_k: int, softmax: bool = False):
     """Scores, top-k and renormalised weights from gate logits [T, E] (float64 arithmetic on the given logits).
 

@@ -42,7 +42,32 @@ __global__ __launch_bounds__(kThreads) void act_image_q8pair_kernel(
     quantize4_to_pair_image(v, e0, hi, lo, xs);
 }
 
+// RMS normalisation of rows: one workgroup per row, the row is read twice (sum of squares, then the scaled values).
+__global__ __launch_bounds__(kThreads) void rms_norm_rows_kernel(
+    const void* __restrict__ x, int x_dtype, const float* __restrict__ weight, void* __restrict__ y, int y_dtype, int dim, float eps) {
+    __shared__ float red[kThreads / 64];
+    const size_t off = static_cast<size_t>(blockIdx.x) * dim;
+    float ss = 0.0f;
+    for (int i = threadIdx.x; i < dim; i += kThreads) {
+        const float v = load_any(x, x_dtype, off + i);
+        ss += v * v;
+    }
+    ss = group_sum<64>(ss);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    float total = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kThreads / 64; ++w) total += red[w];
+    const float rstd = rsqrtf(total / static_cast<float>(dim) + eps);
+    for (int i = threadIdx.x; i < dim; i += kThreads) store_any(y, y_dtype, off + i, load_any(x, x_dtype, off + i) * rstd * weight[i]);
+}
+
 }  // namespace
+
+int rms_norm_rows(const void* x, int x_dtype, const float* weight, void* y, int y_dtype, int rows, int dim, float eps, hipStream_t stream) {
+    hipLaunchKernelGGL(rms_norm_rows_kernel, dim3(rows), dim3(kThreads), 0, stream, x, x_dtype, weight, y, y_dtype, dim, eps);
+    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+}
 
 size_t act_image_256_bytes(int bpr) { return (staged_x_bytes(bpr * 256) + 255) & ~static_cast<size_t>(255); }
 

@@ -140,6 +140,44 @@ size_t pllm_gguf_quant_gemm_workspace_bytes(int type_id, int64_t rows, int64_t k
     return pllm::act_image_256_bytes(static_cast<int>(blocks_per_row)) * static_cast<size_t>(rows);
 }
 
+int pllm_fused_rms_norm(const void* x, int x_dtype, const float* weight, void* y, int y_dtype, int64_t rows, int64_t dim, float eps, void* stream) {
+    if (!x || !weight || !y || !dtype_ok(x_dtype) || !dtype_ok(y_dtype) || rows <= 0 || dim <= 0 || !fits_int(rows) || !fits_int(dim))
+        return PLLM_ERR_INVALID_ARGUMENT;
+    return pllm::rms_norm_rows(x, x_dtype, weight, y, y_dtype, static_cast<int>(rows), static_cast<int>(dim), eps, static_cast<hipStream_t>(stream));
+}
+
+// normalized rows (fp16) ahead of the matmul's own workspace when the call has too many rows for the in-kernel form
+static size_t rmsnorm_rows_bytes(int64_t rows, int64_t k) {
+    return rows <= kInKernelQuantMaxRows ? 0 : (static_cast<size_t>(rows) * static_cast<size_t>(k) * 2 + 255) & ~static_cast<size_t>(255);
+}
+
+size_t pllm_gguf_quant_gemm_rmsnorm_workspace_bytes(int type_id, int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row) {
+    const size_t inner = pllm_gguf_quant_gemm_workspace_bytes(type_id, rows, k, n, blocks_per_row);
+    return inner == 0 ? 0 : inner + rmsnorm_rows_bytes(rows, k);
+}
+
+int pllm_gguf_quant_gemm_rmsnorm(const void* x, int x_dtype, const float* norm_weight, float eps, int round_fp16,
+                                 const uint8_t* blocks, int type_id, void* y, int y_dtype,
+                                 int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row,
+                                 void* workspace, size_t workspace_bytes, void* stream) {
+    if (!x || !norm_weight || !blocks || !y || !dtype_ok(x_dtype) || !dtype_ok(y_dtype)) return PLLM_ERR_INVALID_ARGUMENT;
+    if (!fits_int(rows) || !fits_int(k) || !fits_int(n) || !fits_int(blocks_per_row) || rows <= 0 || k <= 0) return PLLM_ERR_INVALID_ARGUMENT;
+    if (blocks_per_row * 256 < k) return PLLM_ERR_INVALID_ARGUMENT;
+    if (pllm_gguf_block_bytes(type_id) == 0) return PLLM_ERR_UNSUPPORTED;
+    if (rows > 65535) return PLLM_ERR_UNSUPPORTED;
+    if (!workspace || workspace_bytes < pllm_gguf_quant_gemm_rmsnorm_workspace_bytes(type_id, rows, k, n, blocks_per_row)) return PLLM_ERR_WORKSPACE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (rows <= kInKernelQuantMaxRows)       // every workgroup normalizes and quantizes its activation row itself: one launch
+        return superblock_matvec(pllm::act_rows_raw(x, x_dtype, static_cast<int>(k), norm_weight, eps, round_fp16), blocks, type_id, y, y_dtype,
+                                 static_cast<int>(rows), static_cast<int>(n), static_cast<int>(blocks_per_row), s);
+    // many rows: normalized fp16 rows into the head of the workspace, then the ordinary operator on them
+    const size_t head = rmsnorm_rows_bytes(rows, k);
+    const int st = pllm::rms_norm_rows(x, x_dtype, norm_weight, workspace, PLLM_F16, static_cast<int>(rows), static_cast<int>(k), eps, s);
+    if (st != PLLM_OK) return st;
+    return pllm_gguf_quant_gemm(workspace, PLLM_F16, blocks, type_id, y, y_dtype, rows, k, n, blocks_per_row,
+                                static_cast<char*>(workspace) + head, workspace_bytes - head, stream);
+}
+
 size_t pllm_activation_image_bytes(int64_t rows, int64_t blocks_per_row) {
     if (!fits_int(rows) || !fits_int(blocks_per_row)) return 0;
     return pllm::act_image_256_bytes(static_cast<int>(blocks_per_row)) * static_cast<size_t>(rows);

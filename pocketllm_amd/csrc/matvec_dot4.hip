@@ -39,7 +39,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void dot4_matvec_kernel(
     float acc = 0.0f;
     bool staged = false;
     if constexpr (RAW)                       // raw activation row: quantized here, before the loads take their registers
-        quantize_row_to_lds(smem, act.x, act.x_dtype, static_cast<size_t>(blockIdx.y) * act.k, act.k, kpad);
+        quantize_row_to_lds(smem, act.x, act.x_dtype, static_cast<size_t>(blockIdx.y) * act.k, act.k, kpad, RowNorm{act.gamma, act.eps, act.round_f16});
     for (int b0 = wave; b0 < bpr || !staged; b0 += waves * ITERS) {
         typename FMT::Regs regs[ITERS];
 #pragma unroll

@@ -53,7 +53,7 @@ __global__ __launch_bounds__(64 * kWaves) void mfma_tile_matvec_kernel(
     float acc = 0.0f;
     bool staged = false;
     if constexpr (RAW)                       // raw activation row: quantized here, before the loads take their registers
-        quantize_row_to_lds(smem, act.x, act.x_dtype, static_cast<size_t>(blockIdx.y) * act.k, act.k, kpad);
+        quantize_row_to_lds(smem, act.x, act.x_dtype, static_cast<size_t>(blockIdx.y) * act.k, act.k, kpad, RowNorm{act.gamma, act.eps, act.round_f16});
     for (int b0 = wave; b0 < bpr || !staged; b0 += waves * ITERS) {
         typename FMT::Regs regs[ITERS];
 #pragma unroll
@@ -167,7 +167,7 @@ __global__ __launch_bounds__(64 * kWaves) void iq_stream_matvec_kernel(
     int c = blockIdx.x, buf = 0;
     dma_share<kWaves>(w + static_cast<size_t>(c) * chunk_rows * row_bytes, lds0 + chunk_off, min(chunk_rows, n - c * chunk_rows) * row_bytes, wave, lane);
     if constexpr (RAW)                       // raw activation row: quantized once per workgroup while the first chunk is on its way
-        quantize_row_to_lds(smem, act.x, act.x_dtype, static_cast<size_t>(blockIdx.y) * act.k, act.k, kpad);
+        quantize_row_to_lds(smem, act.x, act.x_dtype, static_cast<size_t>(blockIdx.y) * act.k, act.k, kpad, RowNorm{act.gamma, act.eps, act.round_f16});
     typename FMT::Held held[NB > 0 ? NB : 1];
     bool holding = false;
     while (c < chunks) {

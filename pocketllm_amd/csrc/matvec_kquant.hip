@@ -133,7 +133,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void k45_mfma_matvec_kernel(
     float acc = 0.0f;
     bool staged = false;
     if constexpr (RAW) {                     // quantize before the loads take their registers
-        quantize_row_to_lds(smem, act.x, act.x_dtype, static_cast<size_t>(blockIdx.y) * act.k, act.k, kpad);
+        quantize_row_to_lds(smem, act.x, act.x_dtype, static_cast<size_t>(blockIdx.y) * act.k, act.k, kpad, RowNorm{act.gamma, act.eps, act.round_f16});
         if (tid < 4) reinterpret_cast<uint32_t*>(smem + zero_off)[tid] = 0;
         __syncthreads();
         staged = true;

@@ -192,8 +192,17 @@ __device__ __forceinline__ void quantize4_to_image(const float v[4], int e0, int
     if ((threadIdx.x & 7) == 0) gs[e0 >> 5] = make_float2(scale * kLoInv, sum32);
 }
 
+// Optional RMS normalisation ahead of the quantization: v = x * rsqrt(mean(x^2) + eps) * gamma, optionally rounded through fp16
+// (what a separate normalisation kernel with an fp16 output would hand over).  gamma == nullptr: none.
+struct RowNorm {
+    const float* gamma;
+    float eps;
+    int round_f16;
+};
+
 template <int BATCH = 6>
-__device__ __forceinline__ void quantize_row_to_lds(unsigned char* lds, const void* __restrict__ x, int x_dtype, size_t xoff, int k, int kpad) {
+__device__ __forceinline__ void quantize_row_to_lds(unsigned char* lds, const void* __restrict__ x, int x_dtype, size_t xoff, int k, int kpad,
+                                                    const RowNorm norm = RowNorm{nullptr, 0.0f, 0}) {
     int8_t* hi = reinterpret_cast<int8_t*>(lds);
     int8_t* lo = hi + kpad;
     float2* gs = reinterpret_cast<float2*>(lo + kpad);
@@ -202,11 +211,45 @@ __device__ __forceinline__ void quantize_row_to_lds(unsigned char* lds, const vo
     const bool vec = x_dtype == PLLM_F32 ? ((reinterpret_cast<uintptr_t>(x) + 4 * xoff) & 15u) == 0
                                          : ((reinterpret_cast<uintptr_t>(x) + 2 * xoff) & 7u) == 0;
     const int trip = static_cast<int>(blockDim.x) * 4;
+    float rstd = 1.0f;
+    if (norm.gamma) {
+        // sum of squares of the row: per-wave sums meet in the first floats of the image area, which nobody has written yet
+        float ss = 0.0f;
+        for (int e0 = static_cast<int>(threadIdx.x) * 4; e0 < k; e0 += trip) {
+            float v[4];
+            load_row4(v, x, x_dtype, xoff, e0, k, vec);
+            ss += (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
+        }
+        ss = group_sum<64>(ss);
+        float* red = reinterpret_cast<float*>(lds);
+        if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+        __syncthreads();
+        float total = 0.0f;
+        for (int w = 0; w < static_cast<int>(blockDim.x >> 6); ++w) total += red[w];
+        __syncthreads();                                                     // read by everybody before the image overwrites it
+        rstd = rsqrtf(total / static_cast<float>(k) + norm.eps);
+    }
     for (int base = static_cast<int>(threadIdx.x) * 4; base < kpad; base += trip * BATCH) {
         float v[BATCH][4];
 #pragma unroll
         for (int j = 0; j < BATCH; ++j)
             if (base + j * trip < kpad) load_row4(v[j], x, x_dtype, xoff, base + j * trip, k, vec);
+        if (norm.gamma) {
+#pragma unroll
+            for (int j = 0; j < BATCH; ++j) {
+                const int e0 = base + j * trip;
+                if (e0 < kpad) {
+                    float g[4];
+                    load_row4(g, norm.gamma, PLLM_F32, 0, e0, k, (reinterpret_cast<uintptr_t>(norm.gamma) & 15u) == 0);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        float t = v[j][i] * rstd * g[i];                     // values past k are zeros on both sides
+                        if (norm.round_f16) t = static_cast<float>(static_cast<_Float16>(t));
+                        v[j][i] = t;
+                    }
+                }
+            }
+        }
 #pragma unroll
         for (int j = 0; j < BATCH; ++j)
             if (base + j * trip < kpad) quantize4_to_image(v[j], base + j * trip, hi, lo, gs, sum16);

@@ -12,6 +12,8 @@ namespace pllm {
 // activation images (act_quant.hip); *_bytes is the per-row stride, a multiple of 256
 size_t act_image_256_bytes(int bpr);
 int act_image_256(const void* x, int x_dtype, int rows, int k, int bpr, void* image, hipStream_t stream);
+// y[r, :] = x[r, :] * rsqrt(mean(x[r, :]^2) + eps) * weight (float32 arithmetic, one rounding to y_dtype)
+int rms_norm_rows(const void* x, int x_dtype, const float* weight, void* y, int y_dtype, int rows, int dim, float eps, hipStream_t stream);
 size_t act_image_q8pair_bytes(int pairs);
 int act_image_q8pair(const void* x, int x_dtype, int rows, int k, int pairs, void* image, hipStream_t stream);
 
@@ -30,6 +32,9 @@ struct ActRows {
     int x_dtype;
     int k;
     const int64_t* row_token;     // routed calls: grid row r reads image row_token[r] (null: image r)
+    const float* gamma;           // raw rows only: RMS normalisation ahead of the quantization (null: none)
+    float eps;
+    int round_f16;
 };
 // Routed calls: grid row r multiplies with the matrix at w + expert[r] * expert_stride (null: one matrix for every row).
 struct WeightRoute {
@@ -37,9 +42,11 @@ struct WeightRoute {
     size_t expert_stride;
 };
 inline ActRows act_rows_from_image(const unsigned char* image, size_t stride, const int64_t* row_token = nullptr) {
-    return ActRows{image, stride, nullptr, 0, 0, row_token};
+    return ActRows{image, stride, nullptr, 0, 0, row_token, nullptr, 0.0f, 0};
 }
-inline ActRows act_rows_raw(const void* x, int x_dtype, int k) { return ActRows{nullptr, 0, x, x_dtype, k, nullptr}; }
+inline ActRows act_rows_raw(const void* x, int x_dtype, int k, const float* gamma = nullptr, float eps = 0.0f, int round_f16 = 0) {
+    return ActRows{nullptr, 0, x, x_dtype, k, nullptr, gamma, eps, round_f16};
+}
 
 // 256-weight super-block types: one activation image (act_image_256) serves any number of matvecs.
 // Q4_K / Q5_K run in matvec_kquant.hip, IQ2_XXS / IQ1_M in matvec_iq_mfma.hip (matrix cores),

@@ -144,6 +144,49 @@ def gguf_quant_gemm_prefill_forward(x, blocks, row_elems, type_id, signed_grid, 
     return _dense_gemm("gguf_quant_gemm_prefill_forward", x, blocks, row_elems, type_id, signed_grid, out_dtype)
 
 
+def fused_rms_norm_forward(x: torch.Tensor, weight: torch.Tensor, eps: float, *, out_dtype: torch.dtype = torch.float16) -> torch.Tensor:
+    """src/csrc/cuda_kernel_impl.cu:9699-9730: fp16 [batch, dim] = x * rsqrt(mean(x^2) + eps) * weight."""
+    _check(x.dim() == 2, "fused_rms_norm: x must be 2D [batch, dim]")
+    _check(weight.dim() == 1, "fused_rms_norm: weight must be 1D [dim]")
+    _check(weight.dtype == torch.float32, "fused_rms_norm: weight must be fp32")
+    _check(weight.size(0) == x.size(1), "fused_rms_norm: weight.size(0) must == dim")
+    _check(x.is_cuda and weight.is_cuda, "fused_rms_norm: tensors must be CUDA tensors")
+    _check_x(x)
+    x, weight = x.contiguous(), weight.contiguous()
+    y = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    if x.numel() == 0:
+        return y
+    with torch.cuda.device(x.device):
+        st = _lib().pllm_fused_rms_norm(x.data_ptr(), _DTYPE_CODE[x.dtype], weight.data_ptr(), y.data_ptr(), _DTYPE_CODE[out_dtype],
+                                        x.size(0), x.size(1), float(eps), _stream(x.device))
+    _ffi.check(st, "fused_rms_norm_forward")
+    return y
+
+
+def gguf_quant_gemm_rmsnorm_forward(x, norm_weight, eps, blocks, row_elems, type_id, signed_grid, *, round_fp16: bool = True,
+                                    out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """gguf_quant_gemm_forward(fused_rms_norm_forward(x, norm_weight, eps), ...) as one operator (decode: one launch).
+    round_fp16=True rounds the normalized activations through fp16 like the two-operator chain, False keeps them in float32."""
+    row_elems, type_id = int(row_elems), int(type_id)
+    _dense_checks(x, blocks, row_elems, type_id, signed_grid)
+    _check(norm_weight.dim() == 1 and norm_weight.size(0) == row_elems, "fused_rms_norm: weight.size(0) must == dim")
+    _check(norm_weight.is_cuda and norm_weight.dtype == torch.float32 and norm_weight.is_contiguous(), "fused_rms_norm: weight must be fp32")
+    rows = x.numel() // row_elems
+    n = blocks.size(0)
+    y = torch.empty(*x.shape[:-1], n, dtype=out_dtype, device=x.device)
+    if rows == 0 or n == 0:
+        return y
+    lib = _lib()
+    with torch.cuda.device(x.device):
+        ws_bytes = lib.pllm_gguf_quant_gemm_rmsnorm_workspace_bytes(type_id, rows, row_elems, n, blocks.size(1))
+        ws = _workspace(ws_bytes, x.device)
+        st = lib.pllm_gguf_quant_gemm_rmsnorm(x.data_ptr(), _DTYPE_CODE[x.dtype], norm_weight.data_ptr(), float(eps), int(bool(round_fp16)),
+                                              blocks.data_ptr(), type_id, y.data_ptr(), _DTYPE_CODE[out_dtype], rows, row_elems, n,
+                                              blocks.size(1), ws.data_ptr(), ws_bytes, _stream(x.device))
+    _ffi.check(st, "gguf_quant_gemm_rmsnorm_forward")
+    return y
+
+
 def gguf_q2k_gemm_dp4a_forward(x, blocks, row_elems, *, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
     """src/csrc/cuda_kernel.cpp:545-564."""
     _check(blocks.dim() == 3, "blocks must have shape [N, K_blocks, 84]")

@@ -530,3 +530,15 @@ def test_route_topk_closed_forms():
         np.testing.assert_allclose(w[t], sm[t, top] / sm[t, top].sum(), rtol=1e-12)
     idx, _ = O.route_topk(np.zeros((1, 6)), None, 3)
     assert idx.tolist() == [[0, 1, 2]]                                        # equal scores: lower expert id first
+
+
+def test_rms_norm_closed_forms():
+    w = np.array([1.0, 2.0, -1.0, 0.5])
+    np.testing.assert_allclose(O.rms_norm(np.array([[3.0, 3.0, 3.0, 3.0]]), w, 0.0), [w], rtol=1e-15)          # constant row: x / |x| * w
+    np.testing.assert_allclose(O.rms_norm(np.array([[-2.0, -2.0, -2.0, -2.0]]), w, 0.0), [-w], rtol=1e-15)
+    x = np.array([[1.0, -2.0, 3.0, 0.0], [0.0, 0.0, 4.0, 0.0]])
+    got = O.rms_norm(x, w, 1e-6)
+    np.testing.assert_allclose(got[0], x[0] / np.sqrt(14.0 / 4.0 + 1e-6) * w, rtol=1e-15)
+    np.testing.assert_allclose(got[1], x[1] / np.sqrt(4.0 + 1e-6) * w, rtol=1e-15)
+    np.testing.assert_allclose(O.rms_norm(7.0 * x, w, 0.0), O.rms_norm(x, w, 0.0), rtol=1e-14)                  # scale invariance at eps = 0
+    np.testing.assert_allclose(O.rms_norm(np.zeros((1, 4)), w, 1e-6), np.zeros((1, 4)))                          # eps keeps a zero row finite
