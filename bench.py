@@ -162,6 +162,12 @@ def extra_cases(mod, dev, iters):
         run(f"{name} matvec 17408x5120 T=1", blocks.size,
             lambda s, ring=ring, x=x, tid=tid, grid=grid: mod.gguf_quant_gemm_forward(x, ring[s], 5120, tid, grid), len(ring))
         del ring
+    # paired projection (gate and up of a dense MLP): two Q4_K matrices 17408x5120 against one activation row
+    blocks = C.quantize_q4_k((rng.standard_normal((17408, 5120), dtype=np.float32) * np.float32(0.02)))
+    ring = ring_of(blocks, dev, 12)
+    run("q4_k paired projection 2 x 17408x5120 T=1", 2 * blocks.size,
+        lambda s, ring=ring: mod.gguf_quant_gemm_pair_forward(x, ring[s], 5120, 3, ring[(s + 6) % 12], 5120, 3, empty), len(ring))
+    del ring
     # normalisation + projection as one decode operator against the two operators one after the other (Q4_K 5120x5120)
     blocks = C.quantize_q4_k((rng.standard_normal((5120, 5120), dtype=np.float32) * np.float32(0.02)))
     ring = ring_of(blocks, dev, max(2, min(RING, (1 << 30) // blocks.size)))

@@ -214,18 +214,24 @@ int pllm_gguf_quant_gemm_pair(const void* x, int x_dtype, const uint8_t* blocks0
     if (!workspace || workspace_bytes < pllm_activation_image_bytes(rows, blocks_per_row)) return PLLM_ERR_WORKSPACE;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int bpr = static_cast<int>(blocks_per_row);
+    const int R = static_cast<int>(rows), N = static_cast<int>(n);
+    const size_t esize = y_dtype == PLLM_F32 ? 4 : 2;
+    const bool k45 = type_id0 == type_id1 && (type_id0 == PLLM_TYPE_Q4_K || type_id0 == PLLM_TYPE_Q5_K);
+    const bool raw = rows <= kInKernelQuantMaxRows &&
+                     (k45 ? quantizes_in_kernel(type_id0, 2 * n, blocks_per_row)
+                          : quantizes_in_kernel(type_id0, n, blocks_per_row) && quantizes_in_kernel(type_id1, n, blocks_per_row));
     pllm::ActRows act = pllm::act_rows_raw(x, x_dtype, static_cast<int>(k));
-    int st = PLLM_OK;
-    if (rows > kInKernelQuantMaxRows || !quantizes_in_kernel(type_id0, n, blocks_per_row) || !quantizes_in_kernel(type_id1, n, blocks_per_row)) {
-        st = pllm::act_image_256(x, x_dtype, static_cast<int>(rows), static_cast<int>(k), bpr, workspace, s);
+    if (!raw) {
+        const int st = pllm::act_image_256(x, x_dtype, R, static_cast<int>(k), bpr, workspace, s);
         if (st != PLLM_OK) return st;
         act = pllm::act_rows_from_image(static_cast<const unsigned char*>(workspace), pllm::act_image_256_bytes(bpr));
     }
-    const size_t esize = y_dtype == PLLM_F32 ? 4 : 2;
-    st = superblock_matvec(act, blocks0, type_id0, y, y_dtype, static_cast<int>(rows), static_cast<int>(n), bpr, s);
+    if (k45)                                 // one launch over both matrices (grid.z)
+        return superblock_matvec(act, blocks0, type_id0, y, y_dtype, R, N, bpr, s,
+                                 pllm::WeightRoute{nullptr, 0, blocks1, static_cast<size_t>(rows) * static_cast<size_t>(n)});
+    const int st = superblock_matvec(act, blocks0, type_id0, y, y_dtype, R, N, bpr, s);
     if (st != PLLM_OK) return st;
-    return superblock_matvec(act, blocks1, type_id1, static_cast<char*>(y) + static_cast<size_t>(rows) * n * esize, y_dtype,
-                             static_cast<int>(rows), static_cast<int>(n), bpr, s);
+    return superblock_matvec(act, blocks1, type_id1, static_cast<char*>(y) + static_cast<size_t>(rows) * n * esize, y_dtype, R, N, bpr, s);
 }
 
 int pllm_fp8_gemm(const uint8_t* a, const float* a_scale, const uint8_t* weight, const float* scale, void* y, int y_dtype,

@@ -116,6 +116,8 @@ __global__ __launch_bounds__(64 * kMaxWaves) void k45_mfma_matvec_kernel(
     const int ks = lane >> 4;         // k slice of A and B, row quad of C
     const int row = blockIdx.x * kRowsPerWg + col;
     if (route.expert) w += static_cast<size_t>(route.expert[blockIdx.y]) * route.expert_stride;
+    const size_t y_base = blockIdx.z ? route.second_y_offset : 0;           // paired projections: the second matrix and its output
+    if (blockIdx.z) w = route.second;
     const size_t image_row = act.row_token ? static_cast<size_t>(act.row_token[blockIdx.y]) : blockIdx.y;
     const uint8_t* wrow = w + static_cast<size_t>(row < n ? row : 0) * bpr * FMT::kBlockBytes;
 
@@ -186,7 +188,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void k45_mfma_matvec_kernel(
         float total = 0.0f;
         for (int v = 0; v < waves; ++v) total += partial[v * kRowsPerWg + tid];
         const int out_row = blockIdx.x * kRowsPerWg + tid;
-        if (out_row < n) store_any(y, y_dtype, static_cast<size_t>(blockIdx.y) * n + out_row, total);
+        if (out_row < n) store_any(y, y_dtype, y_base + static_cast<size_t>(blockIdx.y) * n + out_row, total);
     }
 }
 
@@ -201,7 +203,7 @@ int launch_kernel(KERN kern, const ActRows& act, const WeightRoute& route, const
                                 static_cast<int>(smem)) != hipSuccess)
             return PLLM_ERR_UNSUPPORTED;
     }
-    dim3 grid((n + kRowsPerWg - 1) / kRowsPerWg, rows);
+    dim3 grid((n + kRowsPerWg - 1) / kRowsPerWg, rows, route.second ? 2 : 1);
     hipLaunchKernelGGL(kern, grid, dim3(64 * waves), smem, stream, act, route, w, y, y_dtype, n, bpr);
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }

@@ -153,6 +153,14 @@ def test_paired_projection(mod):
         # pair == the two separate calls, bit for bit (the reference's own test: tests/test_gguf_quantized_ops_cuda.py:83-92)
         assert torch.equal(y[0], mod.gguf_quant_gemm_prefill_forward(x, ba, k, tid, grid))
         assert torch.equal(y[1], mod.gguf_quant_gemm_prefill_forward(x, bb, k, tid, grid))
+    # one launch over both matrices: also with rows that take the activation pre-pass and with mixed types (two launches)
+    for rows, ta, tb in ((1, 4, 4), (6, 3, 3), (2, 3, 4)):
+        xr = torch.randn(rows, k, device=DEV, dtype=torch.bfloat16)
+        ea, eb = ({3: C.quantize_q4_k, 4: C.quantize_q5_k}[t] for t in (ta, tb))
+        ba, bb = torch.from_numpy(ea(wa)).to(DEV), torch.from_numpy(eb(wb)).to(DEV)
+        y = mod.gguf_quant_gemm_pair_forward(xr, ba, k, ta, bb, k, tb, grid, out_dtype=torch.float32)
+        assert torch.equal(y[0], mod.gguf_quant_gemm_forward(xr, ba, k, ta, grid, out_dtype=torch.float32))
+        assert torch.equal(y[1], mod.gguf_quant_gemm_forward(xr, bb, k, tb, grid, out_dtype=torch.float32))
     with pytest.raises(RuntimeError, match="paired blocks must have same output rows"):
         mod.gguf_quant_gemm_pair_forward(x, ba, k, 4, bb[:8], k, 4, grid)
 
