@@ -28,6 +28,13 @@ How each function is pinned (what a wrong sign / index / transposed operand woul
   fp8_act_quant      invariants (|q*d - x| <= d/2, clamp range) and torch's e4m3 cast.
   swiglu_route       closed form on hand values, both with and without the clamp.
   group_routes       invariants (monotone segment starts, multiset of routes preserved).
+  fp8_fp16scale_matmul  the decode against the C++ engine's bit-trick decoder restated from its description (all 254
+                     non-NaN codes), the pitched indexing against a plain loop on an unaligned case.
+  silu_mul, rms_norm closed forms on hand values (constant rows, scale invariance at eps = 0, zero row).
+  route_topk         hand-computed cases: a bias that changes the selection but not the weights, softmax routing
+                     against softmax -> top-k -> renormalise, equal scores in expert order.
+  matmul_f, moe_forward, fp8_gemm_q   float64 compositions of the pinned pieces above (no arithmetic of their own
+                     beyond a matrix product).
 """
 from __future__ import annotations
 
