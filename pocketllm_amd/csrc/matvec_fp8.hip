@@ -39,6 +39,23 @@ __device__ __forceinline__ float scale_at(const void* __restrict__ scale, size_t
 
 __device__ __forceinline__ float silu(float v) { return v / (1.0f + __expf(-v)); }
 
+// The activation row as float32 in LDS (k a multiple of 16 on the callers' path): four values per lane and trip, one vector
+// load each where the row's alignment allows, all trips of a pass issued together.
+__device__ __forceinline__ void stage_row_f32(float* xs, const void* __restrict__ x, int x_dtype, size_t xoff, int k) {
+    const bool vec = x_dtype == PLLM_F32 ? ((reinterpret_cast<uintptr_t>(x) + 4 * xoff) & 15u) == 0
+                                         : ((reinterpret_cast<uintptr_t>(x) + 2 * xoff) & 7u) == 0;
+    constexpr int kBatch = 6;
+    for (int base = static_cast<int>(threadIdx.x) * 4; base < k; base += kThreads * 4 * kBatch) {
+        float v[kBatch][4];
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j)
+            if (base + j * kThreads * 4 < k) load_row4(v[j], x, x_dtype, xoff, base + j * kThreads * 4, k, vec);
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j)
+            if (base + j * kThreads * 4 < k) *reinterpret_cast<float4*>(xs + base + j * kThreads * 4) = make_float4(v[j][0], v[j][1], v[j][2], v[j][3]);
+    }
+}
+
 // Two register slots per wave: two consecutive rows of one matrix, or (SWIGLU) the same row of the
 // gate and of the up matrix.
 template <bool SWIGLU>
@@ -95,7 +112,7 @@ __global__ __launch_bounds__(kThreads) void fp8_stream_matvec_kernel(
             }
         }
         if (!staged) {
-            for (int i = tid; i < k; i += kThreads) xs[i] = load_any(x, x_dtype, xoff + i);
+            stage_row_f32(xs, x, x_dtype, xoff, k);
             __syncthreads();
             staged = true;
         }
@@ -190,7 +207,7 @@ __global__ __launch_bounds__(kThreads) void fp8_persistent_matvec_kernel(
     int g = blockIdx.x;
     const int step = gridDim.x;
     fp8_fetch_group<ITERS, SWIGLU>(a, ma, mb, g * rows_per_group + wave_row, n, chunks, lane);
-    for (int i = tid; i < k; i += kThreads) xs[i] = load_any(x, x_dtype, xoff + i);
+    stage_row_f32(xs, x, x_dtype, xoff, k);
     __syncthreads();
     while (g < groups) {
         if (g + step < groups) fp8_fetch_group<ITERS, SWIGLU>(b, ma, mb, (g + step) * rows_per_group + wave_row, n, chunks, lane);
