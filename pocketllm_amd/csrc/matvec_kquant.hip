@@ -209,9 +209,11 @@ int launch_kernel(KERN kern, const ActRows& act, const WeightRoute& route, const
 }
 
 // waves per workgroup and blocks in flight per wave for a row of bpr super-blocks
-void split_blocks(int bpr, int& waves, int& iters) {
+void split_blocks(int bpr, int work_items, int& waves, int& iters) {
     waves = 1;
     while (waves < kMaxWaves && bpr / (waves * 2) >= 3) waves *= 2;
+    // few tiles (less than two workgroups per compute unit): twice the waves with half the blocks each keep more loads in flight
+    if (waves < kMaxWaves && bpr / (waves * 2) >= 2 && work_items < 2 * compute_units()) waves *= 2;
     const int niter = (bpr + waves - 1) / waves;
     const int passes = (niter + 7) / 8;
     iters = (niter + passes - 1) / passes;
@@ -221,7 +223,7 @@ void split_blocks(int bpr, int& waves, int& iters) {
 template <typename FMT>
 int launch_k45(const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream) {
     int waves, iters;
-    split_blocks(bpr, waves, iters);
+    split_blocks(bpr, ((n + kRowsPerWg - 1) / kRowsPerWg) * rows * (route.second ? 2 : 1), waves, iters);
 #define PLLM_CASE(I) case I: return act.x ? launch_kernel(k45_mfma_matvec_kernel<FMT, I, true>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream) \
                                           : launch_kernel(k45_mfma_matvec_kernel<FMT, I, false>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream)
     switch (iters) {
