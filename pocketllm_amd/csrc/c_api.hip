@@ -9,6 +9,16 @@ bool fits_int(int64_t v) { return v > 0 && v <= 0x7fffffffLL; }
 // from this many activation rows on, the tile GEMM replaces one matvec per row
 constexpr int64_t kGemmMinRows = 16;
 
+// From how many activation rows on the MFMA tile kernel serves a super-block matmul.  The decode kernels read the matrix once
+// per activation row (from cache after the first), the tile kernel decodes it once for up to 64 rows at a fixed cost: measured
+// crossovers for Q4_K are 5 rows at 17408x5120 (46.7 us against 44) and 12 rows at 5120x5120 (27.0 against 26.1).
+static bool gguf_uses_tile_gemm(int type_id, int64_t rows, int64_t n, int64_t blocks_per_row) {
+    if (!pllm::gemm_f16_supports(type_id)) return false;
+    const int64_t weights = n * blocks_per_row * 256;
+    const int64_t min_rows = weights >= (int64_t{64} << 20) ? 5 : (weights >= (int64_t{16} << 20) ? 12 : kGemmMinRows);
+    return rows >= min_rows;
+}
+
 }  // namespace
 
 namespace pllm {
@@ -120,7 +130,7 @@ int pllm_gguf_quant_gemm(const void* x, int x_dtype, const uint8_t* blocks, int 
     if (!workspace || workspace_bytes < pllm_gguf_quant_gemm_workspace_bytes(type_id, rows, k, n, blocks_per_row)) return PLLM_ERR_WORKSPACE;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int bpr = static_cast<int>(blocks_per_row);
-    if (rows >= kGemmMinRows && pllm::gemm_f16_supports(type_id))
+    if (gguf_uses_tile_gemm(type_id, rows, n, blocks_per_row))
         return pllm::gemm_f16(x, x_dtype, blocks, type_id, y, y_dtype, static_cast<int>(rows), static_cast<int>(k), static_cast<int>(n), bpr,
                               workspace, workspace_bytes, s);
     if (rows <= kInKernelQuantMaxRows && quantizes_in_kernel(type_id, n, blocks_per_row))
@@ -135,7 +145,7 @@ int pllm_gguf_quant_gemm(const void* x, int x_dtype, const uint8_t* blocks, int 
 size_t pllm_gguf_quant_gemm_workspace_bytes(int type_id, int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row) {
     (void)k;
     if (!fits_int(rows) || !fits_int(n) || !fits_int(blocks_per_row) || pllm_gguf_block_bytes(type_id) == 0) return 0;
-    if (rows >= kGemmMinRows && pllm::gemm_f16_supports(type_id))
+    if (gguf_uses_tile_gemm(type_id, rows, n, blocks_per_row))
         return pllm::gemm_f16_workspace_bytes(static_cast<int>(rows), static_cast<int>(n), static_cast<int>(blocks_per_row));
     return pllm::act_image_256_bytes(static_cast<int>(blocks_per_row)) * static_cast<size_t>(rows);
 }
