@@ -59,11 +59,13 @@ constexpr Iq1GridNibbles make_iq1_grid_nibbles() {
 static __device__ const Iq2xxsSignMasks PLLM_IQ2XXS_SIGN_MASKS = make_iq2xxs_sign_masks();
 static __device__ const Iq1GridNibbles PLLM_IQ1_GRID_NIBBLES = make_iq1_grid_nibbles();
 
-// 16 bytes from an address that is only 2-byte aligned
-struct __attribute__((packed, aligned(2))) Unaligned16 { uint32_t x, y, z, w; };
+// 16 bytes from an address that is only 2-byte aligned.  The vector member keeps it one 16-byte load instruction (global
+// memory takes any alignment); four separate words would become four loads.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+struct __attribute__((packed, aligned(2))) Unaligned16 { u32x4 v; };
 __device__ __forceinline__ uint4 load16_a2(const uint8_t* p) {
-    const Unaligned16 v = *reinterpret_cast<const Unaligned16*>(p);
-    return make_uint4(v.x, v.y, v.z, v.w);
+    const Unaligned16 u = *reinterpret_cast<const Unaligned16*>(p);
+    return make_uint4(u.v.x, u.v.y, u.v.z, u.v.w);
 }
 
 // ------------------------------------------------------------------------------------------------

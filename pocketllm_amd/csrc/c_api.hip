@@ -9,14 +9,31 @@ bool fits_int(int64_t v) { return v > 0 && v <= 0x7fffffffLL; }
 // from this many activation rows on, the tile GEMM replaces one matvec per row
 constexpr int64_t kGemmMinRows = 16;
 
-// From how many activation rows on the MFMA tile kernel serves a super-block matmul.  The decode kernels read the matrix once
-// per activation row (from cache after the first), the tile kernel decodes it once for up to 64 rows at a fixed cost: measured
-// crossovers for Q4_K are 5 rows at 17408x5120 (46.7 us against 44) and 12 rows at 5120x5120 (27.0 against 26.1).
+// From how many activation rows on the MFMA tile kernel serves a matmul.  The decode kernels read the matrix once per
+// activation row (from cache after the first), the tile kernel decodes it once for up to 64 rows at a fixed cost.  Measured
+// crossovers (us, decode kernel against tile kernel): at 17408x5120 Q4_K 5 rows (46.7 / 44), IQ1_M, IQ2_XS and IQ3_XXS 4 rows
+// (50 - 56 / 45), Q6_K 3 rows (88.6 at 4 rows / 56); at 5120x5120 Q4_K 12 rows (27.0 / 26.1), IQ1_M, IQ2_XS, IQ3_XXS 8 rows
+// (27 - 30 / 28.5), Q6_K 5 rows (34.0 / 30.6); FP8 (one matvec per row) 3 rows (34.4 at 2 rows / 42) and 5 rows (22.6 at 4 rows / 24.1).
+enum class RowClass { kKQuant, kCodebook, kQ6K, kFp8 };
+
+static int64_t tile_gemm_min_rows(RowClass cls, int64_t weights) {
+    const int size = weights >= (int64_t{64} << 20) ? 2 : (weights >= (int64_t{16} << 20) ? 1 : 0);
+    if (size == 0) return kGemmMinRows;
+    switch (cls) {
+        case RowClass::kKQuant: return size == 2 ? 5 : 12;
+        case RowClass::kCodebook: return size == 2 ? 4 : 8;
+        case RowClass::kQ6K: return size == 2 ? 3 : 5;
+        case RowClass::kFp8: return size == 2 ? 3 : 5;
+    }
+    return kGemmMinRows;
+}
+
 static bool gguf_uses_tile_gemm(int type_id, int64_t rows, int64_t n, int64_t blocks_per_row) {
     if (!pllm::gemm_f16_supports(type_id)) return false;
-    const int64_t weights = n * blocks_per_row * 256;
-    const int64_t min_rows = weights >= (int64_t{64} << 20) ? 5 : (weights >= (int64_t{16} << 20) ? 12 : kGemmMinRows);
-    return rows >= min_rows;
+    const RowClass cls = type_id == PLLM_TYPE_Q6_K ? RowClass::kQ6K
+                         : (type_id == PLLM_TYPE_IQ1_M || type_id == PLLM_TYPE_IQ2_XS || type_id == PLLM_TYPE_IQ3_XXS) ? RowClass::kCodebook
+                                                                                                                       : RowClass::kKQuant;
+    return rows >= tile_gemm_min_rows(cls, n * blocks_per_row * 256);
 }
 
 }  // namespace
@@ -253,10 +270,10 @@ int pllm_fp8_gemm(const uint8_t* a, const float* a_scale, const uint8_t* weight,
 }
 
 // the tile GEMM serves many rows of 256-aligned k; everything else takes the matvec (no workspace)
-static bool fp8_uses_gemm(int64_t rows, int64_t k) { return rows >= kGemmMinRows && k % 256 == 0; }
+static bool fp8_uses_gemm(int64_t rows, int64_t k, int64_t n) { return k % 256 == 0 && rows >= tile_gemm_min_rows(RowClass::kFp8, n * k); }
 
 size_t pllm_fp8_block_gemm_workspace_bytes(int64_t rows, int64_t k, int64_t n) {
-    if (!fits_int(rows) || !fits_int(k) || !fits_int(n) || !fp8_uses_gemm(rows, k)) return 0;
+    if (!fits_int(rows) || !fits_int(k) || !fits_int(n) || !fp8_uses_gemm(rows, k, n)) return 0;
     return pllm::gemm_f16_workspace_bytes(static_cast<int>(rows), static_cast<int>(n), static_cast<int>(k / 256));
 }
 
@@ -264,7 +281,7 @@ int pllm_fp8_block_gemm(const void* x, int x_dtype, const uint8_t* weight, const
                         int64_t rows, int64_t k, int64_t n, void* workspace, size_t workspace_bytes, void* stream) {
     if (!x || !weight || !scale || !y || !dtype_ok(x_dtype) || !dtype_ok(y_dtype)) return PLLM_ERR_INVALID_ARGUMENT;
     if (!fits_int(rows) || !fits_int(k) || !fits_int(n)) return PLLM_ERR_INVALID_ARGUMENT;
-    if (fp8_uses_gemm(rows, k))
+    if (fp8_uses_gemm(rows, k, n))
         return pllm::gemm_f16_fp8(x, x_dtype, weight, scale, y, y_dtype, static_cast<int>(rows), static_cast<int>(k), static_cast<int>(n),
                                   workspace, workspace_bytes, static_cast<hipStream_t>(stream));
     if (rows > 65535) return PLLM_ERR_UNSUPPORTED;
@@ -321,7 +338,7 @@ int pllm_fp8_bf16scale_matmul_rows(const void* x, int x_dtype, const uint8_t* we
 // the workspace).  float32 activations stay on the float32 matvec, row by row: the tile kernel rounds its operands to fp16,
 // which is inside the bound the reference sets for its fp16-storage variants (2e-2) but not the 2e-4 of its float32 ones.
 static bool fp16scale_uses_gemm(int x_dtype, int64_t batch, int64_t rows, int64_t cols, int64_t x_stride, int64_t y_stride, int64_t weight_stride) {
-    return x_dtype != PLLM_F32 && fp8_uses_gemm(batch, cols) && x_stride == cols && y_stride == rows && weight_stride == cols;
+    return x_dtype != PLLM_F32 && fp8_uses_gemm(batch, cols, rows) && x_stride == cols && y_stride == rows && weight_stride == cols;
 }
 
 static size_t fp16scale_table_bytes(int64_t rows, int64_t cols) {
@@ -329,7 +346,7 @@ static size_t fp16scale_table_bytes(int64_t rows, int64_t cols) {
 }
 
 size_t pllm_fp8_fp16scale_matmul_rows_workspace_bytes(int64_t batch, int64_t rows, int64_t cols) {
-    if (!fits_int(batch) || !fits_int(rows) || !fits_int(cols) || !fp8_uses_gemm(batch, cols)) return 0;
+    if (!fits_int(batch) || !fits_int(rows) || !fits_int(cols) || !fp8_uses_gemm(batch, cols, rows)) return 0;
     return fp16scale_table_bytes(rows, cols) + pllm::gemm_f16_workspace_bytes(static_cast<int>(batch), static_cast<int>(rows), static_cast<int>(cols / 256));
 }
 

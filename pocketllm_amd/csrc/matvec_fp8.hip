@@ -81,91 +81,26 @@ __device__ __forceinline__ float chunk_dot(const uint4& w, const float* xp) {
     return s;
 }
 
-// k a multiple of 16, weight base and row pitch 16-byte aligned
-template <int ITERS, int F16S, bool SWIGLU>
-__global__ __launch_bounds__(kThreads) void fp8_stream_matvec_kernel(
-    const void* __restrict__ x, int x_dtype, size_t x_stride, const Fp8Mat ma, const Fp8Mat mb,
-    void* __restrict__ y, int y_dtype, size_t y_stride, int k, int n) {
-    extern __shared__ __align__(16) unsigned char smem[];
-    float* xs = reinterpret_cast<float*>(smem);
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
-    const int chunks = k >> 4;
-    const int row0 = (blockIdx.x * kWaves + wave) * (SWIGLU ? 1 : kRowsPerWave);
-    const size_t xoff = static_cast<size_t>(blockIdx.y) * x_stride;
-
-    float acc[kRowsPerWave];
-#pragma unroll
-    for (int r = 0; r < kRowsPerWave; ++r) acc[r] = 0.0f;
-
-    bool staged = false;
-    for (int c0 = 0; c0 < chunks; c0 += 64 * ITERS) {
-        uint4 regs[kRowsPerWave][ITERS];
-#pragma unroll
-        for (int r = 0; r < kRowsPerWave; ++r) {
-            const uint8_t* wrow = slot_mat<SWIGLU>(ma, mb, r).w + static_cast<size_t>(slot_row<SWIGLU>(row0, r, n)) * slot_mat<SWIGLU>(ma, mb, r).wstride;
-#pragma unroll
-            for (int it = 0; it < ITERS; ++it) {
-                const int c = min(c0 + it * 64 + lane, chunks - 1);
-                regs[r][it] = *reinterpret_cast<const uint4*>(wrow + 16 * c);
-            }
-        }
-        if (!staged) {
-            stage_row_f32(xs, x, x_dtype, xoff, k);
-            __syncthreads();
-            staged = true;
-        }
-#pragma unroll
-        for (int it = 0; it < ITERS; ++it) {
-            const int c = c0 + it * 64 + lane;
-            const bool ok = c < chunks;
-            const int cc = ok ? c : 0;
-#pragma unroll
-            for (int r = 0; r < kRowsPerWave; ++r) {
-                const float s = chunk_dot(regs[r][it], xs + 16 * cc);
-                const Fp8Mat& m = slot_mat<SWIGLU>(ma, mb, r);
-                const float sc = scale_at<F16S>(m.scale, static_cast<size_t>(slot_row<SWIGLU>(row0, r, n) >> 7) * m.sstride + (cc >> 3));
-                acc[r] += ok ? s * sc : 0.0f;
-            }
-        }
-    }
-    float total[kRowsPerWave];
-#pragma unroll
-    for (int r = 0; r < kRowsPerWave; ++r) total[r] = group_sum<64>(acc[r]);
-    const size_t yoff = static_cast<size_t>(blockIdx.y) * y_stride;
-    if constexpr (SWIGLU) {
-        if (lane == 0 && row0 < n) store_any(y, y_dtype, yoff + row0, silu(total[0]) * total[1]);
-    } else {
-#pragma unroll
-        for (int r = 0; r < kRowsPerWave; ++r)
-            if (lane == 0 && row0 + r < n) store_any(y, y_dtype, yoff + row0 + r, total[r]);
-    }
-}
-
-// The same, persistent: the grid is sized to be resident at once, a workgroup stages the activation
-// row once and then walks groups of 8 weight rows (two per wave), always holding the loads of its
-// next group in a second register set while it multiplies the current one.  Rows of at most
-// 64 * 16 * ITERS bytes.
+// k a multiple of 16, weight base and row pitch 16-byte aligned.  Persistent: the grid is sized to be resident at once, a workgroup stages the activation
+// row once and then walks groups of 8 weight rows (two per wave) in passes of 64 * 16 * ITERS bytes
+// per row, always holding the loads of its next pass (of the same group or of its next group) in a
+// second register set while it multiplies the current one.
 template <int ITERS, bool SWIGLU>
-__device__ __forceinline__ void fp8_fetch_group(uint4 (&r)[kRowsPerWave][ITERS], const Fp8Mat& ma, const Fp8Mat& mb, int row0, int n, int chunks, int lane) {
+__device__ __forceinline__ void fp8_fetch_pass(uint4 (&r)[kRowsPerWave][ITERS], const Fp8Mat& ma, const Fp8Mat& mb, int row0, int n, int chunks, int c0, int lane) {
 #pragma unroll
     for (int q = 0; q < kRowsPerWave; ++q) {
         const uint8_t* wrow = slot_mat<SWIGLU>(ma, mb, q).w + static_cast<size_t>(slot_row<SWIGLU>(row0, q, n)) * slot_mat<SWIGLU>(ma, mb, q).wstride;
 #pragma unroll
-        for (int it = 0; it < ITERS; ++it) r[q][it] = *reinterpret_cast<const uint4*>(wrow + 16 * min(it * 64 + lane, chunks - 1));
+        for (int it = 0; it < ITERS; ++it) r[q][it] = *reinterpret_cast<const uint4*>(wrow + 16 * min(c0 + it * 64 + lane, chunks - 1));
     }
 }
 
 template <int ITERS, int F16S, bool SWIGLU>
-__device__ __forceinline__ void fp8_finish_group(const uint4 (&r)[kRowsPerWave][ITERS], const float* xs, const Fp8Mat& ma, const Fp8Mat& mb,
-                                                 void* __restrict__ y, int y_dtype, size_t yoff, int row0, int n, int chunks, int lane) {
-    float acc[kRowsPerWave];
-#pragma unroll
-    for (int q = 0; q < kRowsPerWave; ++q) acc[q] = 0.0f;
+__device__ __forceinline__ void fp8_multiply_pass(float (&acc)[kRowsPerWave], const uint4 (&r)[kRowsPerWave][ITERS], const float* xs, const Fp8Mat& ma,
+                                                  const Fp8Mat& mb, int row0, int n, int chunks, int c0, int lane) {
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
-        const int c = it * 64 + lane;
+        const int c = c0 + it * 64 + lane;
         const bool ok = c < chunks;
         const int cc = ok ? c : 0;
 #pragma unroll
@@ -176,9 +111,13 @@ __device__ __forceinline__ void fp8_finish_group(const uint4 (&r)[kRowsPerWave][
             acc[q] += ok ? d * sc : 0.0f;
         }
     }
+}
+
+template <bool SWIGLU>
+__device__ __forceinline__ void fp8_store_rows(float (&acc)[kRowsPerWave], void* __restrict__ y, int y_dtype, size_t yoff, int row0, int n, int lane) {
     float total[kRowsPerWave];
 #pragma unroll
-    for (int q = 0; q < kRowsPerWave; ++q) total[q] = group_sum<64>(acc[q]);
+    for (int q = 0; q < kRowsPerWave; ++q) { total[q] = group_sum<64>(acc[q]); acc[q] = 0.0f; }
     if constexpr (SWIGLU) {
         if (lane == 0 && row0 < n) store_any(y, y_dtype, yoff + row0, silu(total[0]) * total[1]);
     } else {
@@ -188,10 +127,11 @@ __device__ __forceinline__ void fp8_finish_group(const uint4 (&r)[kRowsPerWave][
     }
 }
 
-template <int ITERS, int F16S, bool SWIGLU>
+template <int ITERS, int F16S, bool SWIGLU, bool LONG_ROWS>
 __global__ __launch_bounds__(kThreads) void fp8_persistent_matvec_kernel(
     const void* __restrict__ x, int x_dtype, size_t x_stride, const Fp8Mat ma, const Fp8Mat mb,
-    void* __restrict__ y, int y_dtype, size_t y_stride, int k, int n, int groups) {
+    void* __restrict__ y, int y_dtype, size_t y_stride, int k, int n, int groups, int passes_of_long_rows) {
+    const int passes = LONG_ROWS ? passes_of_long_rows : 1;                  // a constant for rows that fit one pass
     extern __shared__ __align__(16) unsigned char smem[];
     float* xs = reinterpret_cast<float*>(smem);
     const int tid = threadIdx.x;
@@ -201,22 +141,31 @@ __global__ __launch_bounds__(kThreads) void fp8_persistent_matvec_kernel(
     const size_t xoff = static_cast<size_t>(blockIdx.y) * x_stride;
     const size_t yoff = static_cast<size_t>(blockIdx.y) * y_stride;
     constexpr int per_wave = SWIGLU ? 1 : kRowsPerWave;
+    constexpr int kPassChunks = 64 * ITERS;
     const int rows_per_group = kWaves * per_wave, wave_row = wave * per_wave;
+    const int step = gridDim.x;
 
     uint4 a[kRowsPerWave][ITERS], b[kRowsPerWave][ITERS];
-    int g = blockIdx.x;
-    const int step = gridDim.x;
-    fp8_fetch_group<ITERS, SWIGLU>(a, ma, mb, g * rows_per_group + wave_row, n, chunks, lane);
+    float acc[kRowsPerWave];
+#pragma unroll
+    for (int q = 0; q < kRowsPerWave; ++q) acc[q] = 0.0f;
+    int g = blockIdx.x, p = 0;               // the pass being multiplied
+    int gn = g, pn = 0;                      // the pass being fetched
+    fp8_fetch_pass<ITERS, SWIGLU>(a, ma, mb, g * rows_per_group + wave_row, n, chunks, 0, lane);
     stage_row_f32(xs, x, x_dtype, xoff, k);
     __syncthreads();
     while (g < groups) {
-        if (g + step < groups) fp8_fetch_group<ITERS, SWIGLU>(b, ma, mb, (g + step) * rows_per_group + wave_row, n, chunks, lane);
-        fp8_finish_group<ITERS, F16S, SWIGLU>(a, xs, ma, mb, y, y_dtype, yoff, g * rows_per_group + wave_row, n, chunks, lane);
-        g += step;
+        if (++pn == passes) { pn = 0; gn += step; }
+        if (gn < groups) fp8_fetch_pass<ITERS, SWIGLU>(b, ma, mb, gn * rows_per_group + wave_row, n, chunks, pn * kPassChunks, lane);
+        fp8_multiply_pass<ITERS, F16S, SWIGLU>(acc, a, xs, ma, mb, g * rows_per_group + wave_row, n, chunks, p * kPassChunks, lane);
+        if (p == passes - 1) fp8_store_rows<SWIGLU>(acc, y, y_dtype, yoff, g * rows_per_group + wave_row, n, lane);
+        g = gn; p = pn;
         if (g >= groups) break;
-        if (g + step < groups) fp8_fetch_group<ITERS, SWIGLU>(a, ma, mb, (g + step) * rows_per_group + wave_row, n, chunks, lane);
-        fp8_finish_group<ITERS, F16S, SWIGLU>(b, xs, ma, mb, y, y_dtype, yoff, g * rows_per_group + wave_row, n, chunks, lane);
-        g += step;
+        if (++pn == passes) { pn = 0; gn += step; }
+        if (gn < groups) fp8_fetch_pass<ITERS, SWIGLU>(a, ma, mb, gn * rows_per_group + wave_row, n, chunks, pn * kPassChunks, lane);
+        fp8_multiply_pass<ITERS, F16S, SWIGLU>(acc, b, xs, ma, mb, g * rows_per_group + wave_row, n, chunks, p * kPassChunks, lane);
+        if (p == passes - 1) fp8_store_rows<SWIGLU>(acc, y, y_dtype, yoff, g * rows_per_group + wave_row, n, lane);
+        g = gn; p = pn;
     }
 }
 
@@ -276,35 +225,23 @@ int launch_any(const void* x, int x_dtype, size_t x_stride, const Fp8Mat& ma, co
     const int rows_per_group = kWaves * (SWIGLU ? 1 : kRowsPerWave);
     const int groups = (n + rows_per_group - 1) / rows_per_group;
     const int niter = ((k >> 4) + 63) / 64;
-    if (niter <= 6) {
-        // persistent: two resident workgroups per compute unit (register-bound), groups dealt round-robin
-        const int grid_x = std::min(groups, 2 * compute_units());
-#define PLLM_PCASE(I) case I: { \
-            auto kern = fp8_persistent_matvec_kernel<I, F16S, SWIGLU>; \
-            if (smem > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, \
-                                                        static_cast<int>(smem)) != hipSuccess) return PLLM_ERR_UNSUPPORTED; \
-            hipLaunchKernelGGL(kern, dim3(grid_x, rows), dim3(kThreads), smem, stream, x, x_dtype, x_stride, ma, mb, y, y_dtype, y_stride, k, n, groups); \
-            break; }
-        switch (niter) {
-            PLLM_PCASE(1) PLLM_PCASE(2) PLLM_PCASE(3) PLLM_PCASE(4) PLLM_PCASE(5)
-            default: PLLM_PCASE(6)
-        }
-#undef PLLM_PCASE
-        return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
-    }
     const int passes = (niter + 5) / 6;
     const int iters = (niter + passes - 1) / passes;
-#define PLLM_CASE(I) case I: { \
-            auto kern = fp8_stream_matvec_kernel<I, F16S, SWIGLU>; \
-            if (smem > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, \
-                                                        static_cast<int>(smem)) != hipSuccess) return PLLM_ERR_UNSUPPORTED; \
-            hipLaunchKernelGGL(kern, dim3(groups, rows), dim3(kThreads), smem, stream, x, x_dtype, x_stride, ma, mb, y, y_dtype, y_stride, k, n); \
-            break; }
+    // persistent: the workgroups that fit a compute unit at once (two by registers, fewer when the activation row fills LDS),
+    // groups dealt round-robin
+    const int per_cu = std::max(1, std::min(2, static_cast<int>((160 * 1024) / std::max<size_t>(smem, 1))));
+    const int grid_x = std::min(groups, per_cu * compute_units());
+#define PLLM_PCASE(I) case I: { \
+        auto kern = passes > 1 ? fp8_persistent_matvec_kernel<I, F16S, SWIGLU, true> : fp8_persistent_matvec_kernel<I, F16S, SWIGLU, false>; \
+        if (smem > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                                    static_cast<int>(smem)) != hipSuccess) return PLLM_ERR_UNSUPPORTED; \
+        hipLaunchKernelGGL(kern, dim3(grid_x, rows), dim3(kThreads), smem, stream, x, x_dtype, x_stride, ma, mb, y, y_dtype, y_stride, k, n, groups, passes); \
+        break; }
     switch (iters) {
-        PLLM_CASE(1) PLLM_CASE(2) PLLM_CASE(3) PLLM_CASE(4) PLLM_CASE(5)
-        default: PLLM_CASE(6)
+        PLLM_PCASE(1) PLLM_PCASE(2) PLLM_PCASE(3) PLLM_PCASE(4) PLLM_PCASE(5)
+        default: PLLM_PCASE(6)
     }
-#undef PLLM_CASE
+#undef PLLM_PCASE
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 

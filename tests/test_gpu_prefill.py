@@ -73,6 +73,36 @@ def test_prefill_baseline_shape_sampled(mod, type_name, n):
     assert O.rel_l2(y.cpu().numpy()[:, cols], want) <= 4e-4
 
 
+@pytest.mark.parametrize("type_name,n,rows", [("q4_k", 17408, 5), ("q5_k", 17408, 7), ("q4_k", 5120, 11), ("q4_k", 5120, 12), ("q5_k", 5120, 15),
+                                              ("iq1_m", 17408, 3), ("iq1_m", 17408, 4), ("q6_k", 17408, 2), ("q6_k", 17408, 3),
+                                              ("iq3_xxs", 5120, 7), ("iq3_xxs", 5120, 8), ("q6_k", 5120, 5), ("iq2_xs", 5120, 9)])
+def test_operator_few_rows_on_large_matrices(mod, type_name, n, rows):
+    """Between 2 and 15 activation rows the operator chooses between the decode kernels and the tile
+    kernel by matrix size and format; either side of that choice states the same product (64 sampled columns)."""
+    rng = np.random.default_rng(n + rows)
+    k = 5120
+    if type_name in ENC:
+        blocks = ENC[type_name]((rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02)))
+    elif type_name == "iq1_m":
+        blocks = C.random_iq1_m(rng, n, k // 256)
+    else:
+        blocks = C.random_blocks(rng, type_name, n, k // 256)
+    x_np = rng.standard_normal((rows, k)).astype(np.float32)
+    x_np[1] *= 1e3
+    x_np[rows - 1] *= 1e-5
+    x = torch.from_numpy(x_np).to(DEV).to(torch.bfloat16)
+    grid = codebooks.grid_tensor_for_type(O.TYPE_IDS[type_name]).to(DEV)
+    print(f"case operator {type_name} n={n} rows={rows}", flush=True)
+    y = mod.gguf_quant_gemm_forward(x, torch.from_numpy(blocks).to(DEV), k, O.TYPE_IDS[type_name], grid, out_dtype=torch.float32)
+    torch.cuda.synchronize()
+    assert tuple(y.shape) == (rows, n)
+    cols = rng.choice(n, size=64, replace=False)
+    want = O.matmul_f(x.float().cpu().numpy(), O.dequant_rows(blocks[cols], type_name, k))
+    got = y.cpu().numpy()[:, cols]
+    row_err = np.sqrt(((got - want) ** 2).sum(axis=1) / np.maximum((want ** 2).sum(axis=1), 1e-300))
+    assert row_err.max() <= 6e-4, (row_err.argmax(), row_err.max())
+
+
 # ---- FP8 E4M3 block-scaled weights through the same tile kernel ---------------------------------------
 
 @pytest.mark.parametrize("t,n,k", [(16, 128, 256), (64, 300, 768), (130, 129, 1024), (257, 520, 2048)])
@@ -108,6 +138,28 @@ def test_fp8_prefill_baseline_shape_sampled(mod):
     w = O.dequant_fp8_block(codes, scale)[cols]
     want = O.matmul_f(x.float().cpu().numpy(), w)
     assert O.rel_l2(y.cpu().numpy()[:, cols], want) <= 1e-3
+
+
+@pytest.mark.parametrize("n,rows", [(17408, 2), (17408, 3), (5120, 4), (5120, 5)])
+def test_fp8_operator_few_rows_on_large_matrices(mod, n, rows):
+    """FP8 with a few activation rows: one matvec per row below the crossover, the tile kernel from it on."""
+    rng = np.random.default_rng(n + rows)
+    k = 5120
+    codes = rng.integers(0, 256, size=(n, k), dtype=np.uint8)
+    codes[(codes & 0x7f) == 0x7f] = 0x3c
+    scale = rng.uniform(0.001, 0.01, size=((n + 127) // 128, k // 128)).astype(np.float32)
+    x_np = rng.standard_normal((rows, k)).astype(np.float32)
+    x_np[1] *= 300.0
+    x = torch.from_numpy(x_np).to(DEV).to(torch.bfloat16)
+    print(f"case fp8 operator n={n} rows={rows}", flush=True)
+    y = mod.fp8_block_gemm_forward(x, torch.from_numpy(codes).to(DEV), torch.from_numpy(scale).to(DEV))
+    torch.cuda.synchronize()
+    cols = rng.choice(n, size=64, replace=False)
+    w = O.dequant_fp8_block(codes, scale)[cols]
+    want = O.matmul_f(x.float().cpu().numpy(), w)
+    got = y.cpu().numpy()[:, cols]
+    for r in range(rows):
+        assert O.rel_l2(got[r], want[r]) <= 1e-3, (n, rows, r)
 
 
 # ---- the other super-block formats through the same tile kernel --------------------------------------
