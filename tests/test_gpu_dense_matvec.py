@@ -40,7 +40,7 @@ def _run_dense(mod, type_name, blocks, x_np, x_dtype, k):
 
 
 @pytest.mark.parametrize("type_name", ["q4_k", "q5_k", "q2_k", "q6_k", "iq4_xs"])
-@pytest.mark.parametrize("n,k,rows", [(64, 256, 1), (37, 768, 1), (100, 5120, 1), (16, 2048, 3), (9, 17408, 1), (33, 1000, 2)])
+@pytest.mark.parametrize("n,k,rows", [(64, 256, 1), (37, 768, 1), (100, 5120, 1), (16, 2048, 3), (9, 17408, 1), (33, 1000, 2), (20, 33024, 2), (48, 20480, 1)])
 def test_kquant_matvec_matches_oracle(mod, type_name, n, k, rows):
     rng = np.random.default_rng(1000 + n + k)
     blocks = ENCODERS[type_name](_weights(rng, n, k))
