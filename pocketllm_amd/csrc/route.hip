@@ -5,7 +5,7 @@
 //   sigmoid mode: p = sigmoid(logits); pick the top_k of p + bias (bias optional); weight = p / max(sum of picked p, 1e-20)
 //   softmax mode: pick the top_k logits; weight = softmax over the picked logits (= softmax probabilities renormalised)
 //
-// Launch 1: one wave per (expert, group of 16 tokens), 16-byte loads, the gate row held in registers, 64-lane sums.  Launch 2: one
+// Launch 1: one wave per (expert, group of 4 tokens), 16-byte loads, the gate row held in registers, the tokens side by side, 64-lane sums.  Launch 2: one
 // wave per token, every lane keeps E / 64 candidates in registers, top_k rounds of a wave-wide
 // argmax (larger score first, lower expert id on equal scores), picked in descending order.
 #include "pllm_device.h"
@@ -20,16 +20,17 @@ constexpr int kMaxPerLane = 16;          // experts per lane: up to 1024 experts
 
 // One wave per (expert, group of kTokensPerWave tokens): the gate row is read once per group (its
 // first kHeld float4 pieces per lane stay in registers), the tokens' rows come from cache.
-constexpr int kTokensPerWave = 16;
+constexpr int kTokensPerWave = 4;        // their x loads are in flight together; a single token (decode) runs alone
 constexpr int kHeld = 12;                // 12 x 256 floats: gate rows up to 3072 wide are held whole
 
+template <int NT>
 __global__ __launch_bounds__(kThreads) void route_logits_kernel(
     const void* __restrict__ x, int x_dtype, const float* __restrict__ gate, float* __restrict__ logits, int dim, int n_experts, int tokens) {
     const int lane = threadIdx.x & 63;
     const int e = blockIdx.x * kWavesPerWg + (threadIdx.x >> 6);
     if (e >= n_experts) return;                                             // whole waves leave together
     const float* grow = gate + static_cast<size_t>(e) * dim;
-    const int t0 = blockIdx.y * kTokensPerWave, t1 = min(tokens, t0 + kTokensPerWave);
+    const int t0 = blockIdx.y * NT, t1 = min(tokens, t0 + NT);
     const bool vec = (dim % 4 == 0) && ((reinterpret_cast<uintptr_t>(gate) & 15u) == 0);
     if (!vec) {
         for (int t = t0; t < t1; ++t) {
@@ -46,25 +47,38 @@ __global__ __launch_bounds__(kThreads) void route_logits_kernel(
         const int c = lane * 4 + 256 * i;
         held[i] = c < dim ? *reinterpret_cast<const float4*>(grow + c) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     }
-    for (int t = t0; t < t1; ++t) {
-        const size_t xoff = static_cast<size_t>(t) * dim;
-        float acc = 0.0f;
+    // all tokens of the group side by side: their loads are independent and go out together
+    const bool xvec = ((reinterpret_cast<uintptr_t>(x) & 15u) == 0) && (x_dtype != PLLM_F32 ? dim % 4 == 0 : true);
+    float acc[NT];
+    size_t xoff[NT];
 #pragma unroll
-        for (int i = 0; i < kHeld; ++i) {
-            const int c = lane * 4 + 256 * i;
-            if (c < dim) {
+    for (int j = 0; j < NT; ++j) {
+        acc[j] = 0.0f;
+        xoff[j] = static_cast<size_t>(min(t0 + j, t1 - 1)) * dim;            // past the end: the last token again, result dropped
+    }
+#pragma unroll
+    for (int i = 0; i < kHeld; ++i) {
+        const int c = lane * 4 + 256 * i;
+        if (c < dim) {
+#pragma unroll
+            for (int j = 0; j < NT; ++j) {
                 float v[4];
-                load_row4(v, x, x_dtype, xoff, c, dim, ((reinterpret_cast<uintptr_t>(x) & 15u) == 0) && (x_dtype != PLLM_F32 ? dim % 4 == 0 : true));
-                acc += held[i].x * v[0] + held[i].y * v[1] + held[i].z * v[2] + held[i].w * v[3];
+                load_row4(v, x, x_dtype, xoff[j], c, dim, xvec);
+                acc[j] += held[i].x * v[0] + held[i].y * v[1] + held[i].z * v[2] + held[i].w * v[3];
             }
         }
-        for (int c = lane * 4 + 256 * kHeld; c < dim; c += 256) {           // rows wider than the held part
-            const float4 g = *reinterpret_cast<const float4*>(grow + c);
-            acc += g.x * load_any(x, x_dtype, xoff + c) + g.y * load_any(x, x_dtype, xoff + c + 1) +
-                   g.z * load_any(x, x_dtype, xoff + c + 2) + g.w * load_any(x, x_dtype, xoff + c + 3);
-        }
-        acc = group_sum<64>(acc);
-        if (lane == 0) logits[static_cast<size_t>(t) * n_experts + e] = acc;
+    }
+    for (int c = lane * 4 + 256 * kHeld; c < dim; c += 256) {               // rows wider than the held part
+        const float4 g = *reinterpret_cast<const float4*>(grow + c);
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+            acc[j] += g.x * load_any(x, x_dtype, xoff[j] + c) + g.y * load_any(x, x_dtype, xoff[j] + c + 1) +
+                      g.z * load_any(x, x_dtype, xoff[j] + c + 2) + g.w * load_any(x, x_dtype, xoff[j] + c + 3);
+    }
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+        const float total = group_sum<64>(acc[j]);
+        if (lane == 0 && t0 + j < t1) logits[static_cast<size_t>(t0 + j) * n_experts + e] = total;
     }
 }
 
@@ -148,9 +162,14 @@ int pllm_moe_route(const void* x, int x_dtype, int64_t tokens, int64_t dim, cons
     if (tokens <= 0 || dim <= 0 || n_experts <= 0 || top_k <= 0 || top_k > n_experts) return PLLM_ERR_INVALID_ARGUMENT;
     if (n_experts > 64 * kMaxPerLane || top_k > 64 || tokens > 65535 || dim > 0x7fffffffLL) return PLLM_ERR_UNSUPPORTED;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    hipLaunchKernelGGL(route_logits_kernel,
-                       dim3(static_cast<unsigned>((n_experts + kWavesPerWg - 1) / kWavesPerWg), static_cast<unsigned>((tokens + kTokensPerWave - 1) / kTokensPerWave)),
-                       dim3(kThreads), 0, s, x, x_dtype, gate_weight, logits, static_cast<int>(dim), static_cast<int>(n_experts), static_cast<int>(tokens));
+    const dim3 wgs(static_cast<unsigned>((n_experts + kWavesPerWg - 1) / kWavesPerWg),
+                   static_cast<unsigned>(tokens == 1 ? 1 : (tokens + kTokensPerWave - 1) / kTokensPerWave));
+    if (tokens == 1)
+        hipLaunchKernelGGL(route_logits_kernel<1>, wgs, dim3(kThreads), 0, s, x, x_dtype, gate_weight, logits, static_cast<int>(dim),
+                           static_cast<int>(n_experts), static_cast<int>(tokens));
+    else
+        hipLaunchKernelGGL(route_logits_kernel<kTokensPerWave>, wgs, dim3(kThreads), 0, s, x, x_dtype, gate_weight, logits, static_cast<int>(dim),
+                           static_cast<int>(n_experts), static_cast<int>(tokens));
     hipLaunchKernelGGL(route_topk_kernel, dim3(static_cast<unsigned>(tokens)), dim3(64), 0, s, logits, gate_bias, static_cast<int>(n_experts),
                        static_cast<int>(top_k), softmax_mode, indices, weights);
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
