@@ -150,8 +150,8 @@ int pllm_gguf_dequantize_rows(const int64_t* row_ids, int64_t n_selected, const 
  *   replaces _dequant_fp8_weight_torch (src/kernels/ops.py:144-147).
  * pllm_fp8_block_gemm: y[t, r] = sum_c x[t, c] * out[r, c] without materialising `out`
  *   replaces soft_fp8_blockfp8_gemm (src/kernels/ops.py:641-648, 910-954) on float activations.
- *   Few rows take the bandwidth-bound matvec; 16 rows or more with k a multiple of 256 take the
- *   MFMA tile kernel, which needs `workspace` (pllm_fp8_block_gemm_workspace_bytes bytes, 256-byte
+ *   Few rows take the bandwidth-bound matvec; 16 rows or more with k a multiple of 256 (5 or more when the matrix has
+ *   16M weights, 3 or more when it has 64M) take the MFMA tile kernel, which needs `workspace` (pllm_fp8_block_gemm_workspace_bytes bytes, 256-byte
  *   aligned, private to the call until its kernels have run; the query returns 0 when none is needed).
  */
 int pllm_fp8_block_dequantize(const uint8_t* weight, const float* scale, int64_t n, int64_t k, void* out, int out_dtype, void* stream);
@@ -187,7 +187,7 @@ int pllm_fp8_gemm(const uint8_t* a, const float* a_scale, const uint8_t* weight,
  *   (qwen_cuda_ops.hpp:72-83, 113-140; qwen_fp8_ops.cu:1009-1033).
  * pllm_fp8_fp16scale_matmul_rows: the matvec over `batch` activation rows
  *   replaces ..._matmul_rows_cuda, ..._matmul_rows_f16_cuda and ..._matmul_simt_cuda (qwen_cuda_ops.hpp:85-97,
- *   142-170; qwen_fp8_ops.cu:1035-1124).  16 rows or more of fp16 / bf16 activations with dense pitches and cols a
+ *   142-170; qwen_fp8_ops.cu:1035-1124).  16 rows or more (5 / 3 or more from 16M / 64M weights) of fp16 / bf16 activations with dense pitches and cols a
  *   multiple of 256 run on the MFMA tile kernel (fp16 operands, float32 accumulation) when `workspace` holds pllm_fp8_fp16scale_matmul_rows_workspace_bytes bytes (256-byte
  *   aligned, private to the call until its kernels have run); otherwise, or with a null workspace, every
  *   activation row takes the matvec kernel.
