@@ -118,7 +118,7 @@ def test_fp8_dequant_all_codes_and_block_scales(mod):
     np.testing.assert_array_equal(got2.cpu().numpy(), got)
 
 
-@pytest.mark.parametrize("n,k,rows", [(130, 304, 1), (256, 1024, 1), (17408, 5120, 1), (64, 5120, 3), (33, 300, 2), (16, 40960, 1)])
+@pytest.mark.parametrize("n,k,rows", [(130, 304, 1), (256, 1024, 1), (17408, 5120, 1), (64, 5120, 3), (33, 300, 2), (16, 40960, 1), (4500, 8192, 1)])
 def test_fp8_matvec_matches_oracle(mod, n, k, rows):
     rng = np.random.default_rng(40 + n)
     if n * k <= 4_000_000:

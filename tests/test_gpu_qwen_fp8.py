@@ -91,7 +91,7 @@ def test_fused_swiglu_matches_two_matvecs_and_the_float64_statement():
     assert O.rel_l2(fused.cpu().numpy(), want) < 1.0e-5       # outputs are products of two sums of ~1e3: judged on the whole vector
 
 
-@pytest.mark.parametrize("batch,rows,cols", [(1, 130, 300), (4, 100, 512), (3, 37, 17408)])
+@pytest.mark.parametrize("batch,rows,cols", [(1, 130, 300), (4, 100, 512), (3, 37, 17408), (1, 2100, 8192)])
 def test_fused_swiglu_small_batch_and_fp16_storage(batch, rows, cols):
     rng = np.random.default_rng(rows * 3 + cols)
     x, gate, gscale, wstride, sstride = _case(rng, batch, rows, cols)
