@@ -251,19 +251,20 @@ def extra_cases(mod, dev, iters):
     wq, wk, wv, wo = q5(6144, d), q5(1024, d), q5(1024, d), q5(d, 6144)
     g1, g2 = torch.ones(d, device=dev), torch.ones(d, device=dev)
     hx = torch.randn(1, d, device=dev, dtype=torch.bfloat16)
+    hres = torch.zeros(1, d, device=dev, dtype=torch.float32)
 
     def layer(_s):
         q = mod.gguf_quant_gemm_rmsnorm_forward(hx, g1, 1e-6, wq, d, 4, empty)
         mod.gguf_quant_gemm_rmsnorm_forward(hx, g1, 1e-6, wk, d, 4, empty)
         mod.gguf_quant_gemm_rmsnorm_forward(hx, g1, 1e-6, wv, d, 4, empty)
-        o = mod.gguf_quant_gemm_forward(q, wo, 6144, 4, empty)
+        o = mod.gguf_quant_gemm_accumulate_forward(q, wo, 6144, 4, empty, hres)     # residual connection folded into the projection
         h2 = mod.fused_rms_norm_forward(o, g2, 1e-6)
         ridx, rw = mod.moe_route(h2, gate, gbias, 8)
         return mod.gguf_moe_single_token_forward(h2, ridx[0], rw[0], w1, w3, w2, 0.0)
 
     layer_bytes = (wq.numel() + wk.numel() + wv.numel() + wo.numel()) + per_call + e * d * 4
     us, graphed = time_calls_us(layer, 4, max(8, iters // 4))
-    out.append({"case": "decoder layer matmul path, MiniMax-M2 shapes, T=1 (3 norm+projection, output projection, norm, routing, experts)",
+    out.append({"case": "decoder layer matmul path, MiniMax-M2 shapes, T=1 (3 norm+projection, output projection + residual, norm, routing, experts)",
                 "weight_bytes": int(layer_bytes), "us_per_call": round(us, 3), "gbs": round(layer_bytes / us / 1e3, 1),
                 "frac_hbm_peak": round(layer_bytes / us / 1e3 / HBM_PEAK_GBS, 4), "graph": graphed,
                 "note": "9 launches; the experts and the routing gate stay cache-resident between replays (same routes every replay)"})

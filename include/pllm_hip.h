@@ -88,6 +88,17 @@ int pllm_gguf_quant_gemm(const void* x, int x_dtype, const uint8_t* blocks, int 
 size_t pllm_gguf_quant_gemm_workspace_bytes(int type_id, int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row);
 
 /*
+ * The residual form of pllm_gguf_quant_gemm: y[t, r] += sum_c x[t, c] * W[r, c], the sum formed in float32 and rounded to y's
+ * type once.  Replaces the matmul followed by the separate addition of the transformer block's residual connection
+ * (src/models/minimax_m2/architecture.py:412-413, `x = x + ...` after the output and expert projections) for decode calls.
+ * Same arguments and workspace as pllm_gguf_quant_gemm; y is read and written.  Served by the decode kernels only: a row count
+ * that pllm_gguf_quant_gemm would hand to the tile kernel returns PLLM_ERR_UNSUPPORTED (the caller then adds separately).
+ */
+int pllm_gguf_quant_gemm_accumulate(const void* x, int x_dtype, const uint8_t* blocks, int type_id, void* y, int y_dtype,
+                                    int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row,
+                                    void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * RMS normalisation of rows, y[r, :] = x[r, :] * rsqrt(mean(x[r, :]^2) + eps) * weight, float32 arithmetic and one rounding to
  * y_dtype (the reference writes fp16).  Replaces fused_rms_norm_forward (src/csrc/cuda_kernel_impl.cu:9639-9730,
  * src/csrc/cuda_kernel.cpp:2012), the normalisation the reference runs ahead of its quantized projections

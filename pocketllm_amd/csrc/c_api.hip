@@ -159,6 +159,28 @@ int pllm_gguf_quant_gemm(const void* x, int x_dtype, const uint8_t* blocks, int 
                              type_id, y, y_dtype, static_cast<int>(rows), static_cast<int>(n), bpr, s);
 }
 
+int pllm_gguf_quant_gemm_accumulate(const void* x, int x_dtype, const uint8_t* blocks, int type_id, void* y, int y_dtype,
+                                    int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row,
+                                    void* workspace, size_t workspace_bytes, void* stream) {
+    if (!x || !blocks || !y || !dtype_ok(x_dtype) || !dtype_ok(y_dtype)) return PLLM_ERR_INVALID_ARGUMENT;
+    if (!fits_int(rows) || !fits_int(k) || !fits_int(n) || !fits_int(blocks_per_row)) return PLLM_ERR_INVALID_ARGUMENT;
+    if (blocks_per_row * 256 < k) return PLLM_ERR_INVALID_ARGUMENT;
+    if (pllm_gguf_block_bytes(type_id) == 0) return PLLM_ERR_UNSUPPORTED;
+    // the decode kernels only: the row counts the plain operator hands to the tile kernel are not served
+    if (rows > 65535 || gguf_uses_tile_gemm(type_id, rows, n, blocks_per_row)) return PLLM_ERR_UNSUPPORTED;
+    if (!workspace || workspace_bytes < pllm_gguf_quant_gemm_workspace_bytes(type_id, rows, k, n, blocks_per_row)) return PLLM_ERR_WORKSPACE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int bpr = static_cast<int>(blocks_per_row);
+    const int into = y_dtype | pllm::kAccumulateInto;
+    if (rows <= kInKernelQuantMaxRows && quantizes_in_kernel(type_id, n, blocks_per_row))
+        return superblock_matvec(pllm::act_rows_raw(x, x_dtype, static_cast<int>(k)), blocks, type_id, y, into,
+                                 static_cast<int>(rows), static_cast<int>(n), bpr, s);
+    const int st = pllm::act_image_256(x, x_dtype, static_cast<int>(rows), static_cast<int>(k), bpr, workspace, s);
+    if (st != PLLM_OK) return st;
+    return superblock_matvec(pllm::act_rows_from_image(static_cast<const unsigned char*>(workspace), pllm::act_image_256_bytes(bpr)), blocks,
+                             type_id, y, into, static_cast<int>(rows), static_cast<int>(n), bpr, s);
+}
+
 size_t pllm_gguf_quant_gemm_workspace_bytes(int type_id, int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row) {
     (void)k;
     if (!fits_int(rows) || !fits_int(n) || !fits_int(blocks_per_row) || pllm_gguf_block_bytes(type_id) == 0) return 0;

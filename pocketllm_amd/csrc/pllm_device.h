@@ -150,7 +150,13 @@ __device__ __forceinline__ float load_any(const void* x, int x_dtype, size_t i) 
     return static_cast<const float*>(x)[i];
 }
 
+// Output element i.  With bit 0x100 (kAccumulateInto of pllm_internal.h) set in y_dtype the value is added to what y holds
+// (in float32, rounded once): the residual connection y += W x of the operators that state it.
 __device__ __forceinline__ void store_any(void* y, int y_dtype, size_t i, float v) {
+    if (y_dtype & 0x100) {
+        y_dtype &= ~0x100;
+        v += load_any(y, y_dtype, i);
+    }
     if (y_dtype == PLLM_BF16) static_cast<bf16_t*>(y)[i] = from_float<bf16_t>(v);
     else if (y_dtype == PLLM_F16) static_cast<f16_t*>(y)[i] = from_float<f16_t>(v);
     else static_cast<float*>(y)[i] = v;

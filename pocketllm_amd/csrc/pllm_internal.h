@@ -9,6 +9,10 @@
 
 namespace pllm {
 
+// Set in the output dtype code a matvec launcher receives: the kernels add their result to what y holds (float32 sum,
+// rounded once) instead of overwriting it.
+constexpr int kAccumulateInto = 0x100;
+
 // activation images (act_quant.hip); *_bytes is the per-row stride, a multiple of 256
 size_t act_image_256_bytes(int bpr);
 int act_image_256(const void* x, int x_dtype, int rows, int k, int bpr, void* image, hipStream_t stream);

@@ -139,6 +139,33 @@ def gguf_quant_gemm_forward(x, blocks, row_elems, type_id, signed_grid, *, out_d
     return _dense_gemm("gguf_quant_gemm_forward", x, blocks, row_elems, type_id, signed_grid, out_dtype)
 
 
+def gguf_quant_gemm_accumulate_forward(x, blocks, row_elems, type_id, signed_grid, y: torch.Tensor) -> torch.Tensor:
+    """y += gguf_quant_gemm_forward(x, ...) in place, the residual connection of a transformer block
+    (src/models/minimax_m2/architecture.py:412-413) folded into the projection: one launch for decode calls, the sum formed in
+    float32 and rounded to y's type once.  Row counts that the plain operator hands to the tile kernel run it and add separately."""
+    row_elems, type_id = int(row_elems), int(type_id)
+    _dense_checks(x, blocks, row_elems, type_id, signed_grid)
+    rows = x.numel() // row_elems
+    n = blocks.size(0)
+    _check(y.is_cuda and y.device == x.device and y.is_contiguous() and y.dtype in _DTYPE_CODE, "y must be a contiguous CUDA tensor of float16, bfloat16 or float32")
+    _check(tuple(y.shape) == (*x.shape[:-1], n), "y must have x's leading shape and blocks.size(0) columns")
+    if rows == 0 or n == 0:
+        return y
+    lib = _lib()
+    with torch.cuda.device(x.device):
+        ws_bytes = lib.pllm_gguf_quant_gemm_workspace_bytes(type_id, rows, row_elems, n, blocks.size(1))
+        ws = _workspace(ws_bytes, x.device)
+        st = lib.pllm_gguf_quant_gemm_accumulate(x.data_ptr(), _DTYPE_CODE[x.dtype], blocks.data_ptr(), type_id, y.data_ptr(),
+                                                 _DTYPE_CODE[y.dtype], rows, row_elems, n, blocks.size(1), ws.data_ptr(), ws_bytes,
+                                                 _stream(x.device))
+    if st == -2:                             # PLLM_ERR_UNSUPPORTED: a row count of the tile kernel
+        prod = _dense_gemm("gguf_quant_gemm_accumulate_forward", x, blocks, row_elems, type_id, signed_grid, torch.float32)
+        y.copy_((y.float() + prod).to(y.dtype))
+        return y
+    _ffi.check(st, "gguf_quant_gemm_accumulate_forward")
+    return y
+
+
 def gguf_quant_gemm_prefill_forward(x, blocks, row_elems, type_id, signed_grid, *, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
     """Prefill-regime operator, src/csrc/cuda_kernel.cpp:591-614."""
     return _dense_gemm("gguf_quant_gemm_prefill_forward", x, blocks, row_elems, type_id, signed_grid, out_dtype)

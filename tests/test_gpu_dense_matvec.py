@@ -300,3 +300,37 @@ def test_few_row_calls_equal_the_prequantized_path(mod, type_name):
             y = mod.gguf_quant_gemm_forward(x, blocks, k, tid, codebooks.grid_tensor_for_type(tid).to(dev), out_dtype=torch.float32)
             y_pre = mod.gguf_quant_gemm_prequantized(mod.quantize_activations(x, bpr), blocks, tid, out_dtype=torch.float32)
             assert torch.equal(y, y_pre)
+
+
+@pytest.mark.parametrize("type_name", ["q4_k", "q5_k", "q2_k", "q6_k", "iq4_xs", "iq2_xxs", "iq1_m", "iq2_xs", "iq3_xxs"])
+def test_accumulate_adds_the_product_to_y(mod, type_name):
+    """The residual form y += W x: equal to the plain operator's float32 product plus the old y, rounded once to y's type,
+    for the in-kernel and the pre-pass activation paths, the streamed and the tile-frame kernels; rows of the tile kernel
+    take the composed path of the wrapper."""
+    rng = np.random.default_rng(91)
+    dev = torch.device("cuda:0")
+    tid = O.TYPE_IDS[type_name]
+    grid = codebooks.grid_tensor_for_type(tid).to(dev)
+    for n, k, rows in ((48, 5120, 1), (130, 1002, 3), (1536, 3072, 2), (64, 512, 7), (40, 768, 20)):
+        bpr = (k + 255) // 256
+        if type_name in ("q4_k", "q5_k", "q2_k"):
+            enc = {"q4_k": C.quantize_q4_k, "q5_k": C.quantize_q5_k, "q2_k": C.quantize_q2_k}[type_name]
+            blocks = enc(np.pad(_weights(rng, n, k), ((0, 0), (0, bpr * 256 - k))))
+        elif type_name in ("iq2_xxs", "iq1_m"):
+            blocks = (C.random_iq2_xxs if type_name == "iq2_xxs" else C.random_iq1_m)(rng, n, bpr)
+        else:
+            blocks = C.random_blocks(rng, type_name, n, bpr)
+        blocks = torch.from_numpy(blocks).to(dev)
+        x = torch.from_numpy(rng.standard_normal((rows, k)).astype(np.float32)).to(dev).to(torch.bfloat16)
+        prod = mod.gguf_quant_gemm_forward(x, blocks, k, tid, grid, out_dtype=torch.float32)
+        for ydt in (torch.float32, torch.bfloat16, torch.float16):
+            print(f"case accumulate {type_name} n={n} k={k} rows={rows} {ydt}", flush=True)
+            y0 = torch.from_numpy(rng.standard_normal((rows, n)).astype(np.float32)).to(dev).to(ydt)
+            y = y0.clone()
+            out = mod.gguf_quant_gemm_accumulate_forward(x, blocks, k, tid, grid, y)
+            torch.cuda.synchronize()
+            assert out is y
+            want = (y0.float() + prod).to(ydt)
+            assert torch.equal(y, want), (n, k, rows, ydt, (y.float() - want.float()).abs().max().item())
+    with pytest.raises(RuntimeError, match="leading shape"):
+        mod.gguf_quant_gemm_accumulate_forward(x, blocks, k, tid, grid, torch.zeros(rows, n + 1, device=dev))
