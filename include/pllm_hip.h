@@ -142,6 +142,20 @@ int pllm_gguf_quant_gemm_pair(const void* x, int x_dtype, const uint8_t* blocks0
                               void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * Up to four weight matrices of the same row length and format against one activation tensor, in one launch: the q / k / v
+ * (or gate / up) projections of a decode step.  y[m] [rows, n[m]] = x (optionally RMS-normalized first, as in
+ * pllm_gguf_quant_gemm_rmsnorm; norm_weight may be null) times blocks[m] [n[m], blocks_per_row, block bytes] transposed.
+ * `blocks`, `n` and `y` are host arrays of `count` entries.  Generalizes gguf_quant_gemm_pair_forward
+ * (src/csrc/cuda_kernel.cpp:615-666), which takes two matrices of equal height, to the unequal heights of q and k / v.
+ * One launch exists for Q4_K and Q5_K at decode row counts; other formats, row counts of the tile kernel, and a normalisation
+ * with more than four rows return PLLM_ERR_UNSUPPORTED (call pllm_gguf_quant_gemm[_rmsnorm] per matrix instead).
+ * workspace: pllm_activation_image_bytes(rows, blocks_per_row) bytes (unused when the kernel quantizes the rows itself).
+ */
+int pllm_gguf_quant_gemm_multi(const void* x, int x_dtype, const float* norm_weight, float eps, int round_fp16,
+                               int count, const uint8_t* const* blocks, const int64_t* n, int type_id, void* const* y, int y_dtype,
+                               int64_t rows, int64_t k, int64_t blocks_per_row, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Selected-row dequantization: out[i, :] = dequant(blocks[row_ids[i], :, :])[:k]  (row_ids == NULL
  * selects rows 0 .. n_selected-1 in order).  type_id may also be PLLM_TYPE_Q8_0 (blocks_per_row then
  * counts 32-weight blocks).  Results are bit-identical to the reference's numpy decoders.

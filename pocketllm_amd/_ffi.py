@@ -23,6 +23,8 @@ SIGNATURES = {
     "pllm_q8_0_gemm": (_int, [_c_void_p, _int, _c_void_p, _c_void_p, _int, _i64, _i64, _i64, _i64, _c_void_p, _size_t, _c_void_p]),
     "pllm_q8_0_gemm_workspace_bytes": (_size_t, [_i64, _i64, _i64, _i64]),
     "pllm_gguf_quant_gemm": (_int, [_c_void_p, _int, _c_void_p, _int, _c_void_p, _int, _i64, _i64, _i64, _i64, _c_void_p, _size_t, _c_void_p]),
+    "pllm_gguf_quant_gemm_multi": (_int, [_c_void_p, _int, _c_void_p, ctypes.c_float, _int, _int, _c_void_p, _c_void_p, _int, _c_void_p, _int,
+                                          _i64, _i64, _i64, _c_void_p, _size_t, _c_void_p]),
     "pllm_gguf_quant_gemm_accumulate": (_int, [_c_void_p, _int, _c_void_p, _int, _c_void_p, _int, _i64, _i64, _i64, _i64, _c_void_p, _size_t, _c_void_p]),
     "pllm_gguf_quant_gemm_workspace_bytes": (_size_t, [_int, _i64, _i64, _i64, _i64]),
     "pllm_activation_image_bytes": (_size_t, [_i64, _i64]),

@@ -227,6 +227,42 @@ int pllm_gguf_quant_gemm_rmsnorm(const void* x, int x_dtype, const float* norm_w
                                 static_cast<char*>(workspace) + head, workspace_bytes - head, stream);
 }
 
+int pllm_gguf_quant_gemm_multi(const void* x, int x_dtype, const float* norm_weight, float eps, int round_fp16,
+                               int count, const uint8_t* const* blocks, const int64_t* n, int type_id, void* const* y, int y_dtype,
+                               int64_t rows, int64_t k, int64_t blocks_per_row, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!x || !blocks || !n || !y || !dtype_ok(x_dtype) || !dtype_ok(y_dtype)) return PLLM_ERR_INVALID_ARGUMENT;
+    if (count < 1 || count > 4 || !fits_int(rows) || !fits_int(k) || !fits_int(blocks_per_row) || rows <= 0 || k <= 0) return PLLM_ERR_INVALID_ARGUMENT;
+    if (blocks_per_row * 256 < k) return PLLM_ERR_INVALID_ARGUMENT;
+    int64_t total_n = 0;
+    for (int m = 0; m < count; ++m) {
+        if (!blocks[m] || !y[m] || n[m] <= 0 || !fits_int(n[m])) return PLLM_ERR_INVALID_ARGUMENT;
+        total_n += n[m];
+    }
+    if (pllm_gguf_block_bytes(type_id) == 0) return PLLM_ERR_UNSUPPORTED;
+    // one launch exists for the Q4_K / Q5_K decode kernel; everything else is left to one call per matrix
+    if (type_id != PLLM_TYPE_Q4_K && type_id != PLLM_TYPE_Q5_K) return PLLM_ERR_UNSUPPORTED;
+    if (rows > 65535 || gguf_uses_tile_gemm(type_id, rows, total_n, blocks_per_row)) return PLLM_ERR_UNSUPPORTED;
+    const bool raw = rows <= kInKernelQuantMaxRows && (norm_weight || quantizes_in_kernel(type_id, total_n, blocks_per_row));
+    if (norm_weight && !raw) return PLLM_ERR_UNSUPPORTED;                    // the normalisation exists inside the kernel only
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int bpr = static_cast<int>(blocks_per_row);
+    pllm::ActRows act = pllm::act_rows_raw(x, x_dtype, static_cast<int>(k), norm_weight, eps, round_fp16);
+    if (!raw) {
+        if (!workspace || workspace_bytes < pllm_activation_image_bytes(rows, blocks_per_row)) return PLLM_ERR_WORKSPACE;
+        const int st = pllm::act_image_256(x, x_dtype, static_cast<int>(rows), static_cast<int>(k), bpr, workspace, s);
+        if (st != PLLM_OK) return st;
+        act = pllm::act_rows_from_image(static_cast<const unsigned char*>(workspace), pllm::act_image_256_bytes(bpr));
+    }
+    pllm::WeightRoute all{};
+    for (int m = 1; m < count; ++m) {
+        all.more_w[m - 1] = blocks[m];
+        all.more_y[m - 1] = y[m];
+        all.more_n[m - 1] = static_cast<int>(n[m]);
+    }
+    all.extra = count - 1;
+    return superblock_matvec(act, blocks[0], type_id, y[0], y_dtype, static_cast<int>(rows), static_cast<int>(n[0]), bpr, s, all);
+}
+
 size_t pllm_activation_image_bytes(int64_t rows, int64_t blocks_per_row) {
     if (!fits_int(rows) || !fits_int(blocks_per_row)) return 0;
     return pllm::act_image_256_bytes(static_cast<int>(blocks_per_row)) * static_cast<size_t>(rows);
@@ -275,9 +311,14 @@ int pllm_gguf_quant_gemm_pair(const void* x, int x_dtype, const uint8_t* blocks0
         if (st != PLLM_OK) return st;
         act = pllm::act_rows_from_image(static_cast<const unsigned char*>(workspace), pllm::act_image_256_bytes(bpr));
     }
-    if (k45)                                 // one launch over both matrices (grid.z)
-        return superblock_matvec(act, blocks0, type_id0, y, y_dtype, R, N, bpr, s,
-                                 pllm::WeightRoute{nullptr, 0, blocks1, static_cast<size_t>(rows) * static_cast<size_t>(n)});
+    if (k45) {                               // one launch over both matrices (grid.z)
+        pllm::WeightRoute both{};
+        both.more_w[0] = blocks1;
+        both.more_y[0] = static_cast<char*>(y) + static_cast<size_t>(rows) * n * esize;
+        both.more_n[0] = N;
+        both.extra = 1;
+        return superblock_matvec(act, blocks0, type_id0, y, y_dtype, R, N, bpr, s, both);
+    }
     const int st = superblock_matvec(act, blocks0, type_id0, y, y_dtype, R, N, bpr, s);
     if (st != PLLM_OK) return st;
     return superblock_matvec(act, blocks1, type_id1, static_cast<char*>(y) + static_cast<size_t>(rows) * n * esize, y_dtype, R, N, bpr, s);

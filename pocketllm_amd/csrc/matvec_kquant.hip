@@ -114,11 +114,16 @@ __global__ __launch_bounds__(64 * kMaxWaves) void k45_mfma_matvec_kernel(
     const int lane = tid & 63;
     const int col = lane & 15;        // B/C column = output row within the tile; also A's row index m
     const int ks = lane >> 4;         // k slice of A and B, row quad of C
-    const int row = blockIdx.x * kRowsPerWg + col;
     if (route.expert) w += static_cast<size_t>(route.expert[blockIdx.y]) * route.expert_stride;
-    const size_t y_base = blockIdx.z ? route.second_y_offset : 0;           // paired projections: the second matrix and its output
-    if (blockIdx.z) w = route.second;
+    if (blockIdx.z) {                        // several projections in one launch: this one's matrix, row count and output
+        const int m = blockIdx.z - 1;
+        w = route.more_w[m];
+        y = route.more_y[m];
+        n = route.more_n[m];
+    }
+    if (static_cast<int>(blockIdx.x) * kRowsPerWg >= n) return;             // the grid covers the tallest matrix
     const size_t image_row = act.row_token ? static_cast<size_t>(act.row_token[blockIdx.y]) : blockIdx.y;
+    const int row = blockIdx.x * kRowsPerWg + col;
     const uint8_t* wrow = w + static_cast<size_t>(row < n ? row : 0) * bpr * FMT::kBlockBytes;
 
     // A side: this lane supplies row m = col = 2 * group + term of MFMA t, slice ks; it is non-zero
@@ -188,7 +193,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void k45_mfma_matvec_kernel(
         float total = 0.0f;
         for (int v = 0; v < waves; ++v) total += partial[v * kRowsPerWg + tid];
         const int out_row = blockIdx.x * kRowsPerWg + tid;
-        if (out_row < n) store_any(y, y_dtype, y_base + static_cast<size_t>(blockIdx.y) * n + out_row, total);
+        if (out_row < n) store_any(y, y_dtype, static_cast<size_t>(blockIdx.y) * n + out_row, total);
     }
 }
 
@@ -203,7 +208,9 @@ int launch_kernel(KERN kern, const ActRows& act, const WeightRoute& route, const
                                 static_cast<int>(smem)) != hipSuccess)
             return PLLM_ERR_UNSUPPORTED;
     }
-    dim3 grid((n + kRowsPerWg - 1) / kRowsPerWg, rows, route.second ? 2 : 1);
+    int tallest = n;
+    for (int m = 0; m < route.extra; ++m) tallest = tallest > route.more_n[m] ? tallest : route.more_n[m];
+    dim3 grid((tallest + kRowsPerWg - 1) / kRowsPerWg, rows, 1 + route.extra);
     hipLaunchKernelGGL(kern, grid, dim3(64 * waves), smem, stream, act, route, w, y, y_dtype, n, bpr);
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
@@ -223,7 +230,9 @@ void split_blocks(int bpr, int work_items, int& waves, int& iters) {
 template <typename FMT>
 int launch_k45(const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream) {
     int waves, iters;
-    split_blocks(bpr, ((n + kRowsPerWg - 1) / kRowsPerWg) * rows * (route.second ? 2 : 1), waves, iters);
+    int tiles = (n + kRowsPerWg - 1) / kRowsPerWg;
+    for (int m = 0; m < route.extra; ++m) tiles += (route.more_n[m] + kRowsPerWg - 1) / kRowsPerWg;
+    split_blocks(bpr, tiles * rows, waves, iters);
 #define PLLM_CASE(I) case I: return act.x ? launch_kernel(k45_mfma_matvec_kernel<FMT, I, true>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream) \
                                           : launch_kernel(k45_mfma_matvec_kernel<FMT, I, false>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream)
     switch (iters) {

@@ -602,8 +602,12 @@ int pllm_gguf_moe_forward(const void* x, int x_dtype, int64_t tokens, int64_t di
         if (st != PLLM_OK) return st;
         // one token: every route reads image 0 (stride 0); several: the route's token picks the image
         const ActRows xa = act_rows_from_image(x_image, tokens > 1 ? x_stride : 0, tokens > 1 ? route_tokens : nullptr);
-        const WeightRoute r13{experts32, static_cast<size_t>(inter) * bpr_x * pllm_gguf_block_bytes(w13_type), nullptr, 0};
-        const WeightRoute r2{experts32, static_cast<size_t>(dim) * bpr_h * pllm_gguf_block_bytes(w2_type), nullptr, 0};
+        WeightRoute r13{};
+        r13.expert = experts32;
+        r13.expert_stride = static_cast<size_t>(inter) * bpr_x * pllm_gguf_block_bytes(w13_type);
+        WeightRoute r2{};
+        r2.expert = experts32;
+        r2.expert_stride = static_cast<size_t>(dim) * bpr_h * pllm_gguf_block_bytes(w2_type);
         st = superblock_matvec(xa, w1, w13_type, gate, PLLM_F32, R, I, bpr_x, s, r13);
         if (st != PLLM_OK) return st;
         st = superblock_matvec(xa, w3, w13_type, up, PLLM_F32, R, I, bpr_x, s, r13);

@@ -44,10 +44,12 @@ struct ActRows {
 struct WeightRoute {
     const int32_t* expert;
     size_t expert_stride;
-    // paired projections in one launch (kernels that support it): grid.z = 1 multiplies with `second` and writes its rows
-    // `second_y_offset` elements further into y
-    const uint8_t* second;
-    size_t second_y_offset;
+    // several projections of one activation tensor in one launch (kernels that support it): grid.z = 1 + m multiplies with
+    // more_w[m] (more_n[m] rows of the same length and format) and writes to more_y[m]; `extra` counts them
+    const uint8_t* more_w[3];
+    void* more_y[3];
+    int more_n[3];
+    int extra;
 };
 inline ActRows act_rows_from_image(const unsigned char* image, size_t stride, const int64_t* row_token = nullptr) {
     return ActRows{image, stride, nullptr, 0, 0, row_token, nullptr, 0.0f, 0};
@@ -60,14 +62,14 @@ inline ActRows act_rows_raw(const void* x, int x_dtype, int k, const float* gamm
 // Q4_K / Q5_K run in matvec_kquant.hip, IQ2_XXS / IQ1_M in matvec_iq_mfma.hip (matrix cores),
 // Q2_K and the routed forms in matvec_dot4.hip (v_dot4).
 int kquant_matvec_from_image(const ActRows& act, const uint8_t* w, int type_id, void* y, int y_dtype,
-                             int rows, int n, int bpr, hipStream_t stream, WeightRoute route = WeightRoute{nullptr, 0, nullptr, 0});
+                             int rows, int n, int bpr, hipStream_t stream, WeightRoute route = WeightRoute{});
 int dot4_matvec_from_image(const ActRows& act, const uint8_t* w, int type_id, void* y, int y_dtype,
-                           int rows, int n, int bpr, hipStream_t stream, WeightRoute route = WeightRoute{nullptr, 0, nullptr, 0});
+                           int rows, int n, int bpr, hipStream_t stream, WeightRoute route = WeightRoute{});
 int iq_mfma_matvec_from_image(const ActRows& act, const uint8_t* w, int type_id, void* y, int y_dtype,
-                              int rows, int n, int bpr, hipStream_t stream, WeightRoute route = WeightRoute{nullptr, 0, nullptr, 0});
+                              int rows, int n, int bpr, hipStream_t stream, WeightRoute route = WeightRoute{});
 // any of the nine super-block types, dense or routed (defined beside the C ABI)
 int superblock_matvec(const ActRows& act, const uint8_t* blocks, int type_id, void* y, int y_dtype,
-                      int rows, int n, int bpr, hipStream_t stream, WeightRoute route = WeightRoute{nullptr, 0, nullptr, 0});
+                      int rows, int n, int bpr, hipStream_t stream, WeightRoute route = WeightRoute{});
 
 // routed form: activation row r (image r, output row r) meets the matrix at w + y_expert[r] * expert_stride
 int dot4_routed_matvec_from_image(const unsigned char* image, size_t stride, const uint8_t* w, int type_id, void* y, int y_dtype,

@@ -139,6 +139,50 @@ def gguf_quant_gemm_forward(x, blocks, row_elems, type_id, signed_grid, *, out_d
     return _dense_gemm("gguf_quant_gemm_forward", x, blocks, row_elems, type_id, signed_grid, out_dtype)
 
 
+def gguf_quant_gemm_multi_forward(x, blocks_list, row_elems, type_id, signed_grid, *, norm_weight=None, eps: float = 1e-6,
+                                  round_fp16: bool = True, out_dtype: torch.dtype = torch.bfloat16):
+    """Several projections of one activation tensor, [gguf_quant_gemm_forward(x, b, ...) for b in blocks_list] (with norm_weight:
+    gguf_quant_gemm_rmsnorm_forward), as ONE launch where the library has one: up to four Q4_K or Q5_K matrices of any heights
+    at decode row counts.  The generalization of gguf_quant_gemm_pair_forward (src/csrc/cuda_kernel.cpp:615-666) to q / k / v.
+    Everything else runs one operator call per matrix.  Returns the list of outputs."""
+    import ctypes
+    row_elems, type_id = int(row_elems), int(type_id)
+    blocks_list = list(blocks_list)
+    _check(len(blocks_list) >= 1, "blocks_list must hold at least one matrix")
+    for b in blocks_list:
+        _dense_checks(x, b, row_elems, type_id, signed_grid)
+        _check(b.size(1) == blocks_list[0].size(1), "all matrices must have the same number of blocks per row")
+    if norm_weight is not None:
+        _check(norm_weight.dim() == 1 and norm_weight.size(0) == row_elems, "fused_rms_norm: weight.size(0) must == dim")
+        _check(norm_weight.is_cuda and norm_weight.dtype == torch.float32 and norm_weight.is_contiguous(), "fused_rms_norm: weight must be fp32")
+    rows = x.numel() // row_elems
+
+    def one_by_one():
+        if norm_weight is None:
+            return [_dense_gemm("gguf_quant_gemm_multi_forward", x, b, row_elems, type_id, signed_grid, out_dtype) for b in blocks_list]
+        return [gguf_quant_gemm_rmsnorm_forward(x, norm_weight, eps, b, row_elems, type_id, signed_grid, round_fp16=round_fp16, out_dtype=out_dtype)
+                for b in blocks_list]
+
+    count = len(blocks_list)
+    if rows == 0 or count > 4 or any(b.size(0) == 0 for b in blocks_list):
+        return one_by_one()
+    ys = [torch.empty(*x.shape[:-1], b.size(0), dtype=out_dtype, device=x.device) for b in blocks_list]
+    lib = _lib()
+    bpr = blocks_list[0].size(1)
+    with torch.cuda.device(x.device):
+        ws_bytes = lib.pllm_activation_image_bytes(rows, bpr)
+        ws = _workspace(ws_bytes, x.device)
+        st = lib.pllm_gguf_quant_gemm_multi(
+            x.data_ptr(), _DTYPE_CODE[x.dtype], norm_weight.data_ptr() if norm_weight is not None else None, float(eps), int(bool(round_fp16)),
+            count, (ctypes.c_void_p * count)(*[b.data_ptr() for b in blocks_list]), (ctypes.c_int64 * count)(*[b.size(0) for b in blocks_list]),
+            type_id, (ctypes.c_void_p * count)(*[t.data_ptr() for t in ys]), _DTYPE_CODE[out_dtype], rows, row_elems, bpr,
+            ws.data_ptr(), ws_bytes, _stream(x.device))
+    if st == -2:                             # PLLM_ERR_UNSUPPORTED: no single launch for this format or row count
+        return one_by_one()
+    _ffi.check(st, "gguf_quant_gemm_multi_forward")
+    return ys
+
+
 def gguf_quant_gemm_accumulate_forward(x, blocks, row_elems, type_id, signed_grid, y: torch.Tensor) -> torch.Tensor:
     """y += gguf_quant_gemm_forward(x, ...) in place, the residual connection of a transformer block
     (src/models/minimax_m2/architecture.py:412-413) folded into the projection: one launch for decode calls, the sum formed in

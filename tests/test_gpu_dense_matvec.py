@@ -334,3 +334,39 @@ def test_accumulate_adds_the_product_to_y(mod, type_name):
             assert torch.equal(y, want), (n, k, rows, ydt, (y.float() - want.float()).abs().max().item())
     with pytest.raises(RuntimeError, match="leading shape"):
         mod.gguf_quant_gemm_accumulate_forward(x, blocks, k, tid, grid, torch.zeros(rows, n + 1, device=dev))
+
+
+@pytest.mark.parametrize("type_name", ["q4_k", "q5_k", "q6_k"])
+def test_multi_projection_equals_separate_calls(mod, type_name):
+    """q / k / v style projections of one activation tensor in one launch (Q4_K, Q5_K) or one call each (other formats):
+    the same bits as the separate operators, with and without the fused RMS normalisation, heights in any order."""
+    rng = np.random.default_rng(93)
+    dev = torch.device("cuda:0")
+    tid = O.TYPE_IDS[type_name]
+    grid = codebooks.grid_tensor_for_type(tid).to(dev)
+    for k, heights, rows in ((3072, (6144, 1024, 1024), 1), (1002, (40, 130, 16, 7), 3), (512, (33,), 2), (768, (64, 200), 20)):
+        bpr = (k + 255) // 256
+        mats = []
+        for n in heights:
+            if type_name == "q6_k":
+                mats.append(torch.from_numpy(C.random_blocks(rng, type_name, n, bpr)).to(dev))
+            else:
+                enc = C.quantize_q4_k if type_name == "q4_k" else C.quantize_q5_k
+                mats.append(torch.from_numpy(enc(np.pad(_weights(rng, n, k), ((0, 0), (0, bpr * 256 - k))))).to(dev))
+        gamma = torch.from_numpy(rng.uniform(0.5, 1.5, size=k).astype(np.float32)).to(dev)
+        for dt in (torch.bfloat16, torch.float32):
+            x = torch.from_numpy(rng.standard_normal((rows, k)).astype(np.float32)).to(dev).to(dt)
+            print(f"case multi {type_name} k={k} heights={heights} rows={rows} {dt}", flush=True)
+            got = mod.gguf_quant_gemm_multi_forward(x, mats, k, tid, grid, out_dtype=torch.float32)
+            want = [mod.gguf_quant_gemm_forward(x, m, k, tid, grid, out_dtype=torch.float32) for m in mats]
+            assert len(got) == len(want)
+            for a, b in zip(got, want):
+                assert a.shape == b.shape and torch.equal(a, b)
+            got = mod.gguf_quant_gemm_multi_forward(x, mats, k, tid, grid, norm_weight=gamma, eps=1e-5, out_dtype=torch.float32)
+            want = [mod.gguf_quant_gemm_rmsnorm_forward(x, gamma, 1e-5, m, k, tid, grid, out_dtype=torch.float32) for m in mats]
+            for a, b in zip(got, want):
+                assert torch.equal(a, b)
+    bb = mats[0].size(2)
+    one, two = torch.zeros(8, 1, bb, dtype=torch.uint8, device=dev), torch.zeros(8, 2, bb, dtype=torch.uint8, device=dev)
+    with pytest.raises(RuntimeError, match="same number of blocks per row"):
+        mod.gguf_quant_gemm_multi_forward(torch.zeros(1, 256, device=dev), [one, two], 256, tid, grid)
