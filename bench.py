@@ -267,6 +267,39 @@ def extra_cases(mod, dev, iters):
                 "frac_hbm_peak": round(layer_bytes / us / 1e3 / HBM_PEAK_GBS, 4), "graph": graphed,
                 "note": "7 launches; the experts and the routing gate stay cache-resident between replays (same routes every replay)"})
     del w1, w3, w2, wq, wk, wv, wo
+    # one dense feed-forward block at T=1, hidden 5120, intermediate 17408, Q4_K: y += W_down (SiLU(W_gate n(x)) * W_up n(x)), as three
+    # launches (norm + gate/up in one, SiLU * up into the activation image, down projection with the residual in its store) and as the
+    # chain of separate operators a runtime would otherwise issue
+    dff, iff = 5120, 17408
+    def q4(n, k):
+        return torch.from_numpy(C.quantize_q4_k((rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02)))).to(dev)
+    base = (q4(iff, dff), q4(iff, dff), q4(dff, iff))
+    rings = [base] + [tuple(t.clone() for t in base) for _ in range(2)]        # 450 MB in rotation: the weights come from HBM
+    gff = torch.ones(dff, device=dev)
+    xff = torch.randn(1, dff, device=dev, dtype=torch.bfloat16)
+    yres = torch.zeros(1, dff, device=dev, dtype=torch.float32)
+
+    def ffn_fused(sl):
+        wg, wu, wd = rings[sl]
+        g, u = mod.gguf_quant_gemm_multi_forward(xff, (wg, wu), dff, 3, empty, norm_weight=gff, eps=1e-6, out_dtype=torch.float32)
+        image = mod.swiglu_quantize_activations(g, u, iff // 256, round_dtype=torch.bfloat16)
+        return mod.gguf_quant_gemm_prequantized(image, wd, 3, accumulate_into=yres)
+
+    def ffn_chain(sl):
+        wg, wu, wd = rings[sl]
+        hn = mod.fused_rms_norm_forward(xff, gff, 1e-6)
+        gu = mod.gguf_quant_gemm_pair_forward(hn, wg, dff, 3, wu, dff, 3, empty)
+        h = torch.nn.functional.silu(gu[0]) * gu[1]
+        yres.add_(mod.gguf_quant_gemm_forward(h, wd, iff, 3, empty, out_dtype=torch.float32))
+        return yres
+
+    ffn_bytes = sum(t.numel() for t in rings[0])
+    for label, fn in (("three launches (norm + gate/up, SiLU * up image, down + residual)", ffn_fused), ("separate operators", ffn_chain)):
+        us, graphed = time_calls_us(fn, 3, max(6, iters // 4))
+        out.append({"case": f"dense feed-forward block q4_k 5120 -> 17408 -> 5120, T=1, {label}", "weight_bytes": int(ffn_bytes),
+                    "us_per_call": round(us, 3), "gbs": round(ffn_bytes / us / 1e3, 1),
+                    "frac_hbm_peak": round(ffn_bytes / us / 1e3 / HBM_PEAK_GBS, 4), "graph": graphed})
+    del rings, base
     return out + prefill_cases(mod, dev, iters)
 
 

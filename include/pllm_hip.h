@@ -132,6 +132,21 @@ int pllm_gguf_quant_gemm_prequantized(const void* image, const uint8_t* blocks, 
                                       int64_t rows, int64_t n, int64_t blocks_per_row, void* stream);
 
 /*
+ * The feed-forward tail of a decode step in two launches: the image of h = SiLU(gate) * up straight from the gate and up
+ * projections [rows, k] (float16, bfloat16 or float32), then the down projection on that image with the residual added
+ * (y += W h).  swiglu_limit > 0 caps gate at the limit and clamps up to +-limit first (src/csrc/cuda_kernel_impl.cu:241-262);
+ * round_dtype PLLM_F16 / PLLM_BF16 rounds h through that type before quantizing, which is what the chain
+ * "F.silu(gate) * up in the model's dtype, then the down projection" feeds its matmul; PLLM_F32 keeps h in float32.
+ * They have no counterpart in the reference, whose dense feed-forward runs activation, multiplication, projection and residual
+ * addition as separate framework ops around gguf_quant_gemm_forward (src/components/gguf/quantized_ops.py:9-151).
+ * image: pllm_activation_image_bytes(rows, blocks_per_row) bytes, 256-byte aligned.
+ */
+int pllm_swiglu_quantize_activations(const void* gate, const void* up, int gu_dtype, int64_t rows, int64_t k, int64_t blocks_per_row,
+                                     float swiglu_limit, int round_dtype, void* image, size_t image_bytes, void* stream);
+int pllm_gguf_quant_gemm_prequantized_accumulate(const void* image, const uint8_t* blocks, int type_id, void* y, int y_dtype,
+                                                 int64_t rows, int64_t n, int64_t blocks_per_row, void* stream);
+
+/*
  * Two weight matrices of the same [n, k] against one activation tensor (k/v projections): the
  * activations are quantized once.  y [2, rows, n]; workspace as for pllm_gguf_quant_gemm.
  * Replaces gguf_quant_gemm_pair_forward (src/csrc/cuda_kernel.cpp:615-666, launcher

@@ -30,6 +30,8 @@ SIGNATURES = {
     "pllm_activation_image_bytes": (_size_t, [_i64, _i64]),
     "pllm_quantize_activations": (_int, [_c_void_p, _int, _i64, _i64, _i64, _c_void_p, _size_t, _c_void_p]),
     "pllm_gguf_quant_gemm_prequantized": (_int, [_c_void_p, _c_void_p, _int, _c_void_p, _int, _i64, _i64, _i64, _c_void_p]),
+    "pllm_gguf_quant_gemm_prequantized_accumulate": (_int, [_c_void_p, _c_void_p, _int, _c_void_p, _int, _i64, _i64, _i64, _c_void_p]),
+    "pllm_swiglu_quantize_activations": (_int, [_c_void_p, _c_void_p, _int, _i64, _i64, _i64, ctypes.c_float, _int, _c_void_p, _size_t, _c_void_p]),
     "pllm_gguf_quant_gemm_pair": (_int, [_c_void_p, _int, _c_void_p, _int, _c_void_p, _int, _c_void_p, _int, _i64, _i64, _i64, _i64, _c_void_p, _size_t, _c_void_p]),
     "pllm_gguf_moe_workspace_bytes": (_size_t, [_i64, _i64, _i64, _i64]),
     "pllm_gguf_moe_forward": (_int, [_c_void_p, _int, _i64, _i64, _i64, _c_void_p, _c_void_p, _c_void_p, _i64, _c_void_p, _i64,

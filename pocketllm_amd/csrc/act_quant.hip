@@ -25,6 +25,38 @@ __global__ __launch_bounds__(kThreads) void act_image_256_kernel(
     quantize4_to_image(v, e0, hi, lo, gs, sum16);
 }
 
+// The image of h = SiLU(g) * u (g capped at L from above and u clamped to +-L when L > 0), optionally rounded through a 16-bit
+// type first, as the two-operator chain "activation in the model's dtype, then the down projection" rounds it.
+__global__ __launch_bounds__(kThreads) void swiglu_image_256_kernel(
+    const void* __restrict__ gate, const void* __restrict__ up, int gu_dtype, float limit, int round_dtype,
+    unsigned char* __restrict__ image, int k, int kpad, size_t image_stride) {
+    const int e0 = (blockIdx.x * kThreads + threadIdx.x) * 4;
+    if (e0 >= kpad) return;
+    const size_t xoff = static_cast<size_t>(blockIdx.y) * k;
+    unsigned char* base = image + static_cast<size_t>(blockIdx.y) * image_stride;
+    int8_t* hi = reinterpret_cast<int8_t*>(base);
+    int8_t* lo = hi + kpad;
+    float2* gs = reinterpret_cast<float2*>(lo + kpad);
+    float* sum16 = reinterpret_cast<float*>(gs + kpad / 32);
+    float v[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        float h = 0.0f;
+        if (e0 + i < k) {
+            float g = load_any(gate, gu_dtype, xoff + e0 + i), u = load_any(up, gu_dtype, xoff + e0 + i);
+            if (limit > 0.0f) {
+                u = fminf(fmaxf(u, -limit), limit);
+                g = fminf(g, limit);
+            }
+            h = g / (1.0f + expf(-g)) * u;
+            if (round_dtype == PLLM_F16) h = to_float(from_float<f16_t>(h));
+            else if (round_dtype == PLLM_BF16) h = to_float(from_float<bf16_t>(h));
+        }
+        v[i] = h;
+    }
+    quantize4_to_image(v, e0, hi, lo, gs, sum16);
+}
+
 // Q8_0 pair image: per pair of 32-value blocks 80 bytes that mirror the weight stream,
 //   [0,0, q0..q31, 0,0, q32..q63, 12 x 0],  then after all pairs: float xs[2 * pairs].
 __global__ __launch_bounds__(kThreads) void act_image_q8pair_kernel(
@@ -75,6 +107,15 @@ int act_image_256(const void* x, int x_dtype, int rows, int k, int bpr, void* im
     const int kpad = bpr * 256;
     dim3 grid((kpad / 4 + kThreads - 1) / kThreads, rows);
     hipLaunchKernelGGL(act_image_256_kernel, grid, dim3(kThreads), 0, stream, x, x_dtype,
+                       static_cast<unsigned char*>(image), k, kpad, act_image_256_bytes(bpr));
+    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+}
+
+int swiglu_image_256(const void* gate, const void* up, int gu_dtype, float limit, int round_dtype, int rows, int k, int bpr, void* image,
+                     hipStream_t stream) {
+    const int kpad = bpr * 256;
+    dim3 grid((kpad / 4 + kThreads - 1) / kThreads, rows);
+    hipLaunchKernelGGL(swiglu_image_256_kernel, grid, dim3(kThreads), 0, stream, gate, up, gu_dtype, limit, round_dtype,
                        static_cast<unsigned char*>(image), k, kpad, act_image_256_bytes(bpr));
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }

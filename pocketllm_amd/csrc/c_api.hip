@@ -278,14 +278,35 @@ int pllm_quantize_activations(const void* x, int x_dtype, int64_t rows, int64_t 
                                static_cast<hipStream_t>(stream));
 }
 
-int pllm_gguf_quant_gemm_prequantized(const void* image, const uint8_t* blocks, int type_id, void* y, int y_dtype,
-                                      int64_t rows, int64_t n, int64_t blocks_per_row, void* stream) {
+static int prequantized_matvec(const void* image, const uint8_t* blocks, int type_id, void* y, int y_dtype, int into,
+                               int64_t rows, int64_t n, int64_t blocks_per_row, void* stream) {
     if (!image || !blocks || !y || !dtype_ok(y_dtype) || !fits_int(rows) || !fits_int(n) || !fits_int(blocks_per_row)) return PLLM_ERR_INVALID_ARGUMENT;
     if (pllm_gguf_block_bytes(type_id) == 0) return PLLM_ERR_UNSUPPORTED;
     if (rows > 65535) return PLLM_ERR_UNSUPPORTED;
     const int bpr = static_cast<int>(blocks_per_row);
     return superblock_matvec(pllm::act_rows_from_image(static_cast<const unsigned char*>(image), pllm::act_image_256_bytes(bpr)), blocks,
-                             type_id, y, y_dtype, static_cast<int>(rows), static_cast<int>(n), bpr, static_cast<hipStream_t>(stream));
+                             type_id, y, y_dtype | into, static_cast<int>(rows), static_cast<int>(n), bpr, static_cast<hipStream_t>(stream));
+}
+
+int pllm_gguf_quant_gemm_prequantized(const void* image, const uint8_t* blocks, int type_id, void* y, int y_dtype,
+                                      int64_t rows, int64_t n, int64_t blocks_per_row, void* stream) {
+    return prequantized_matvec(image, blocks, type_id, y, y_dtype, 0, rows, n, blocks_per_row, stream);
+}
+
+int pllm_gguf_quant_gemm_prequantized_accumulate(const void* image, const uint8_t* blocks, int type_id, void* y, int y_dtype,
+                                                 int64_t rows, int64_t n, int64_t blocks_per_row, void* stream) {
+    return prequantized_matvec(image, blocks, type_id, y, y_dtype, pllm::kAccumulateInto, rows, n, blocks_per_row, stream);
+}
+
+int pllm_swiglu_quantize_activations(const void* gate, const void* up, int gu_dtype, int64_t rows, int64_t k, int64_t blocks_per_row,
+                                     float swiglu_limit, int round_dtype, void* image, size_t image_bytes, void* stream) {
+    if (!gate || !up || !image || !dtype_ok(gu_dtype) || !dtype_ok(round_dtype)) return PLLM_ERR_INVALID_ARGUMENT;
+    if (!fits_int(rows) || !fits_int(k) || !fits_int(blocks_per_row) || rows <= 0 || k <= 0) return PLLM_ERR_INVALID_ARGUMENT;
+    if (blocks_per_row * 256 < k) return PLLM_ERR_INVALID_ARGUMENT;
+    if (rows > 65535) return PLLM_ERR_UNSUPPORTED;
+    if (image_bytes < pllm_activation_image_bytes(rows, blocks_per_row)) return PLLM_ERR_WORKSPACE;
+    return pllm::swiglu_image_256(gate, up, gu_dtype, swiglu_limit, round_dtype, static_cast<int>(rows), static_cast<int>(k),
+                                  static_cast<int>(blocks_per_row), image, static_cast<hipStream_t>(stream));
 }
 
 int pllm_gguf_quant_gemm_pair(const void* x, int x_dtype, const uint8_t* blocks0, int type_id0, const uint8_t* blocks1, int type_id1,

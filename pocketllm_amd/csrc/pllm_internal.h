@@ -16,6 +16,9 @@ constexpr int kAccumulateInto = 0x100;
 // activation images (act_quant.hip); *_bytes is the per-row stride, a multiple of 256
 size_t act_image_256_bytes(int bpr);
 int act_image_256(const void* x, int x_dtype, int rows, int k, int bpr, void* image, hipStream_t stream);
+// the image of SiLU(gate) * up (clamped by `limit` when positive, rounded through round_dtype when that is a 16-bit type)
+int swiglu_image_256(const void* gate, const void* up, int gu_dtype, float limit, int round_dtype, int rows, int k, int bpr, void* image,
+                     hipStream_t stream);
 // y[r, :] = x[r, :] * rsqrt(mean(x[r, :]^2) + eps) * weight (float32 arithmetic, one rounding to y_dtype)
 int rms_norm_rows(const void* x, int x_dtype, const float* weight, void* y, int y_dtype, int rows, int dim, float eps, hipStream_t stream);
 size_t act_image_q8pair_bytes(int pairs);

@@ -699,8 +699,34 @@ def quantize_activations(x: torch.Tensor, blocks_per_row: int) -> torch.Tensor:
     return image
 
 
-def gguf_quant_gemm_prequantized(image: torch.Tensor, blocks: torch.Tensor, type_id: int, *, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
-    """y [rows, N] from an activation image and raw super-blocks [N, K_blocks, block_bytes]."""
+def swiglu_quantize_activations(gate: torch.Tensor, up: torch.Tensor, blocks_per_row: int, *, swiglu_limit: float = 0.0,
+                                round_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """The activation image of SiLU(gate) * up for the down projection (gguf_quant_gemm_prequantized), one launch in place of the
+    activation, the multiplication and the quantization pre-pass.  swiglu_limit > 0 caps gate and clamps up as the fused expert
+    operators do (src/csrc/cuda_kernel_impl.cu:241-262); round_dtype float16 / bfloat16 rounds the product through that type
+    first, as a chain that forms it in the model's dtype does."""
+    _check(gate.is_cuda and up.is_cuda and gate.is_contiguous() and up.is_contiguous(), "gate and up must be contiguous CUDA tensors")
+    _check(gate.shape == up.shape and gate.dtype == up.dtype, "gate and up must agree in shape and dtype")
+    _check_x(gate)
+    _check(round_dtype in _DTYPE_CODE, "round_dtype must be float16, bfloat16, or float32")
+    k, bpr = gate.size(-1), int(blocks_per_row)
+    _check(bpr * 256 >= k, "blocks do not cover row_elems")
+    rows = gate.numel() // max(k, 1)
+    _check(rows > 0 and k > 0, "gate and up must not be empty")
+    lib = _lib()
+    nbytes = lib.pllm_activation_image_bytes(rows, bpr)
+    image = torch.empty(rows, nbytes // rows, dtype=torch.uint8, device=gate.device)
+    with torch.cuda.device(gate.device):
+        st = lib.pllm_swiglu_quantize_activations(gate.data_ptr(), up.data_ptr(), _DTYPE_CODE[gate.dtype], rows, k, bpr, float(swiglu_limit),
+                                                  _DTYPE_CODE[round_dtype], image.data_ptr(), nbytes, _stream(gate.device))
+    _ffi.check(st, "swiglu_quantize_activations")
+    return image
+
+
+def gguf_quant_gemm_prequantized(image: torch.Tensor, blocks: torch.Tensor, type_id: int, *, out_dtype: torch.dtype = torch.bfloat16,
+                                 accumulate_into: torch.Tensor = None) -> torch.Tensor:
+    """y [rows, N] from an activation image and raw super-blocks [N, K_blocks, block_bytes]; with accumulate_into the product is
+    added to that tensor in place (the residual connection) and it is returned."""
     type_id = int(type_id)
     _check_type(type_id)
     _check(image.is_cuda and image.dtype == torch.uint8 and image.dim() == 2 and image.is_contiguous(), "image must come from quantize_activations")
@@ -710,9 +736,15 @@ def gguf_quant_gemm_prequantized(image: torch.Tensor, blocks: torch.Tensor, type
     lib = _lib()
     rows, n = image.size(0), blocks.size(0)
     _check(image.size(1) * rows == lib.pllm_activation_image_bytes(rows, blocks.size(1)), "image does not match blocks_per_row")
-    y = torch.empty(rows, n, dtype=out_dtype, device=image.device)
+    if accumulate_into is not None:
+        y = accumulate_into
+        _check(y.is_cuda and y.device == image.device and y.is_contiguous() and y.dtype in _DTYPE_CODE and y.numel() == rows * n and y.size(-1) == n,
+               "accumulate_into must be a contiguous CUDA tensor [rows, N] of float16, bfloat16 or float32")
+        fn = lib.pllm_gguf_quant_gemm_prequantized_accumulate
+    else:
+        y = torch.empty(rows, n, dtype=out_dtype, device=image.device)
+        fn = lib.pllm_gguf_quant_gemm_prequantized
     with torch.cuda.device(image.device):
-        st = lib.pllm_gguf_quant_gemm_prequantized(image.data_ptr(), blocks.data_ptr(), type_id, y.data_ptr(), _DTYPE_CODE[out_dtype],
-                                                   rows, n, blocks.size(1), _stream(image.device))
+        st = fn(image.data_ptr(), blocks.data_ptr(), type_id, y.data_ptr(), _DTYPE_CODE[y.dtype], rows, n, blocks.size(1), _stream(image.device))
     _ffi.check(st, "gguf_quant_gemm_prequantized")
     return y

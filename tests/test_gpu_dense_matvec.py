@@ -370,3 +370,44 @@ def test_multi_projection_equals_separate_calls(mod, type_name):
     one, two = torch.zeros(8, 1, bb, dtype=torch.uint8, device=dev), torch.zeros(8, 2, bb, dtype=torch.uint8, device=dev)
     with pytest.raises(RuntimeError, match="same number of blocks per row"):
         mod.gguf_quant_gemm_multi_forward(torch.zeros(1, 256, device=dev), [one, two], 256, tid, grid)
+
+
+@pytest.mark.parametrize("type_name", ["q4_k", "q6_k", "iq2_xxs"])
+def test_swiglu_image_feeds_the_down_projection(mod, type_name):
+    """SiLU(gate) * up quantized in one launch, then the down projection on the image with the residual added: against the chain of
+    separate operators on the same float values (image bit-equal when the product is formed identically), and against the float oracle."""
+    rng = np.random.default_rng(95)
+    dev = torch.device("cuda:0")
+    tid = O.TYPE_IDS[type_name]
+    for inter, d, rows, limit in ((1536, 96, 1, 0.0), (1002, 40, 3, 0.0), (2048, 64, 2, 1.5)):
+        bpr = (inter + 255) // 256
+        if type_name == "q4_k":
+            wd = C.quantize_q4_k(np.pad(_weights(rng, d, inter), ((0, 0), (0, bpr * 256 - inter))))
+        elif type_name == "q6_k":
+            wd = C.random_blocks(rng, type_name, d, bpr)
+        else:
+            wd = C.random_iq2_xxs(rng, d, bpr)
+        wd_dev = torch.from_numpy(wd).to(dev)
+        g_np = rng.standard_normal((rows, inter)).astype(np.float32) * 2
+        u_np = rng.standard_normal((rows, inter)).astype(np.float32) * 2
+        for gu_dt, round_dt in ((torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16), (torch.float32, torch.float16)):
+            print(f"case swiglu image {type_name} inter={inter} d={d} rows={rows} limit={limit} {gu_dt} round {round_dt}", flush=True)
+            g, u = torch.from_numpy(g_np).to(dev).to(gu_dt), torch.from_numpy(u_np).to(dev).to(gu_dt)
+            image = mod.swiglu_quantize_activations(g, u, bpr, swiglu_limit=limit, round_dtype=round_dt)
+            gf, uf = g.float().cpu().numpy().astype(np.float64), u.float().cpu().numpy().astype(np.float64)
+            if limit > 0:
+                uf, gf = np.clip(uf, -limit, limit), np.minimum(gf, limit)
+            h64 = gf / (1.0 + np.exp(-gf)) * uf
+            h = torch.from_numpy(h64.astype(np.float32)).to(round_dt)              # the chain's activation tensor
+            y0 = torch.from_numpy(rng.standard_normal((rows, d)).astype(np.float32)).to(dev)
+            y = mod.gguf_quant_gemm_prequantized(image, wd_dev, tid, accumulate_into=y0.clone())
+            torch.cuda.synchronize()
+            want = y0.cpu().numpy() + O.matmul_f(h.float().numpy(), O.dequant_rows(wd, type_name, inter))
+            assert O.rel_l2(y.cpu().numpy(), want) <= 1e-3
+            # the same through the separate operators: identical up to the last-bit differences of the device's expf
+            chain = y0 + mod.gguf_quant_gemm_forward(h.to(dev), wd_dev, inter, tid, codebooks.grid_tensor_for_type(tid).to(dev), out_dtype=torch.float32)
+            assert O.rel_l2(y.cpu().numpy(), chain.cpu().numpy()) <= 2e-4
+            plain = mod.gguf_quant_gemm_prequantized(image, wd_dev, tid, out_dtype=torch.float32)
+            assert torch.equal((y0 + plain), y)
+    with pytest.raises(RuntimeError, match="agree in shape"):
+        mod.swiglu_quantize_activations(g, u[:, :-1].contiguous(), bpr)
