@@ -162,7 +162,7 @@ int pllm_gguf_quant_gemm_pair(const void* x, int x_dtype, const uint8_t* blocks0
  * pllm_gguf_quant_gemm_rmsnorm; norm_weight may be null) times blocks[m] [n[m], blocks_per_row, block bytes] transposed.
  * `blocks`, `n` and `y` are host arrays of `count` entries.  Generalizes gguf_quant_gemm_pair_forward
  * (src/csrc/cuda_kernel.cpp:615-666), which takes two matrices of equal height, to the unequal heights of q and k / v.
- * One launch exists for Q4_K and Q5_K at decode row counts; other formats, row counts of the tile kernel, and a normalisation
+ * One launch exists for every format but Q2_K at decode row counts; Q2_K, row counts of the tile kernel, and a normalisation
  * with more than four rows return PLLM_ERR_UNSUPPORTED (call pllm_gguf_quant_gemm[_rmsnorm] per matrix instead).
  * workspace: pllm_activation_image_bytes(rows, blocks_per_row) bytes (unused when the kernel quantizes the rows itself).
  */

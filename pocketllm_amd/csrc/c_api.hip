@@ -239,8 +239,8 @@ int pllm_gguf_quant_gemm_multi(const void* x, int x_dtype, const float* norm_wei
         total_n += n[m];
     }
     if (pllm_gguf_block_bytes(type_id) == 0) return PLLM_ERR_UNSUPPORTED;
-    // one launch exists for the Q4_K / Q5_K decode kernel; everything else is left to one call per matrix
-    if (type_id != PLLM_TYPE_Q4_K && type_id != PLLM_TYPE_Q5_K) return PLLM_ERR_UNSUPPORTED;
+    // one launch exists in the matrix-core decode kernels; Q2_K (and anything else) is left to one call per matrix
+    if (type_id == PLLM_TYPE_Q2_K) return PLLM_ERR_UNSUPPORTED;
     if (rows > 65535 || gguf_uses_tile_gemm(type_id, rows, total_n, blocks_per_row)) return PLLM_ERR_UNSUPPORTED;
     const bool raw = rows <= kInKernelQuantMaxRows && (norm_weight || quantizes_in_kernel(type_id, total_n, blocks_per_row));
     if (norm_weight && !raw) return PLLM_ERR_UNSUPPORTED;                    // the normalisation exists inside the kernel only

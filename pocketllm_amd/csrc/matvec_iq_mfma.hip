@@ -34,6 +34,13 @@ __global__ __launch_bounds__(64 * kWaves) void mfma_tile_matvec_kernel(
     const int zero_off = image_bytes;                                        // 16 zero bytes
     unsigned char* tables = smem + image_bytes + 16;
     if (route.expert) w += static_cast<size_t>(route.expert[blockIdx.y]) * route.expert_stride;
+    if (blockIdx.z) {                        // several projections in one launch: this one's matrix, row count and output
+        const int m = blockIdx.z - 1;
+        w = route.more_w[m];
+        y = route.more_y[m];
+        n = route.more_n[m];
+    }
+    if (static_cast<int>(blockIdx.x) * kRowsPerTile >= n) return;           // the grid covers the tallest matrix
     const size_t image_row = act.row_token ? static_cast<size_t>(act.row_token[blockIdx.y]) : blockIdx.y;
     float* partial = reinterpret_cast<float*>(tables + FMT::kTableBytes);   // [waves][16]
 
@@ -97,7 +104,9 @@ int launch_tile(const ActRows& act, const WeightRoute& route, const uint8_t* w, 
                                 static_cast<int>(smem)) != hipSuccess)
             return PLLM_ERR_UNSUPPORTED;
     }
-    dim3 grid((n + kRowsPerTile - 1) / kRowsPerTile, rows);
+    int tallest = n;
+    for (int m = 0; m < route.extra; ++m) tallest = tallest > route.more_n[m] ? tallest : route.more_n[m];
+    dim3 grid((tallest + kRowsPerTile - 1) / kRowsPerTile, rows, 1 + route.extra);
     hipLaunchKernelGGL(kern, grid, dim3(64 * waves), smem, stream, act, route, w, y, y_dtype, n, bpr);
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
@@ -290,9 +299,10 @@ template <typename FMT>
 int launch_fmt(const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype,
                int rows, int n, int bpr, hipStream_t stream) {
     // whole tiles streamed through long-lived workgroups (the codebooks are staged once per workgroup)
-    // where shape and alignment allow, else one short workgroup per tile; routed calls always take the latter
+    // where shape and alignment allow, else one short workgroup per tile; routed calls and several projections in one launch
+    // always take the latter
     if constexpr (FMT::kStreamed)
-        if (!route.expert && !act.row_token)
+        if (!route.expert && !act.row_token && route.extra == 0)
             if (const int split = stream_split<FMT>(w, n, bpr)) return launch_stream<FMT>(act, w, y, y_dtype, rows, n, bpr, split, stream);
     return launch_tiles<FMT>(act, route, w, y, y_dtype, rows, n, bpr, stream);
 }

@@ -142,8 +142,8 @@ def gguf_quant_gemm_forward(x, blocks, row_elems, type_id, signed_grid, *, out_d
 def gguf_quant_gemm_multi_forward(x, blocks_list, row_elems, type_id, signed_grid, *, norm_weight=None, eps: float = 1e-6,
                                   round_fp16: bool = True, out_dtype: torch.dtype = torch.bfloat16):
     """Several projections of one activation tensor, [gguf_quant_gemm_forward(x, b, ...) for b in blocks_list] (with norm_weight:
-    gguf_quant_gemm_rmsnorm_forward), as ONE launch where the library has one: up to four Q4_K or Q5_K matrices of any heights
-    at decode row counts.  The generalization of gguf_quant_gemm_pair_forward (src/csrc/cuda_kernel.cpp:615-666) to q / k / v.
+    gguf_quant_gemm_rmsnorm_forward), as ONE launch where the library has one: up to four matrices of any heights and one format
+    (any but Q2_K) at decode row counts.  The generalization of gguf_quant_gemm_pair_forward (src/csrc/cuda_kernel.cpp:615-666) to q / k / v.
     Everything else runs one operator call per matrix.  Returns the list of outputs."""
     import ctypes
     row_elems, type_id = int(row_elems), int(type_id)

@@ -336,10 +336,10 @@ def test_accumulate_adds_the_product_to_y(mod, type_name):
         mod.gguf_quant_gemm_accumulate_forward(x, blocks, k, tid, grid, torch.zeros(rows, n + 1, device=dev))
 
 
-@pytest.mark.parametrize("type_name", ["q4_k", "q5_k", "q6_k"])
+@pytest.mark.parametrize("type_name", ["q4_k", "q5_k", "q6_k", "iq4_xs", "iq2_xxs", "iq1_m", "iq3_xxs", "q2_k"])
 def test_multi_projection_equals_separate_calls(mod, type_name):
-    """q / k / v style projections of one activation tensor in one launch (Q4_K, Q5_K) or one call each (other formats):
-    the same bits as the separate operators, with and without the fused RMS normalisation, heights in any order."""
+    """q / k / v style projections of one activation tensor in one launch (one call each for Q2_K): the results of the separate
+    operators, with and without the fused RMS normalisation, heights in any order."""
     rng = np.random.default_rng(93)
     dev = torch.device("cuda:0")
     tid = O.TYPE_IDS[type_name]
@@ -348,11 +348,13 @@ def test_multi_projection_equals_separate_calls(mod, type_name):
         bpr = (k + 255) // 256
         mats = []
         for n in heights:
-            if type_name == "q6_k":
-                mats.append(torch.from_numpy(C.random_blocks(rng, type_name, n, bpr)).to(dev))
-            else:
-                enc = C.quantize_q4_k if type_name == "q4_k" else C.quantize_q5_k
+            if type_name in ("q4_k", "q5_k", "q2_k"):
+                enc = {"q4_k": C.quantize_q4_k, "q5_k": C.quantize_q5_k, "q2_k": C.quantize_q2_k}[type_name]
                 mats.append(torch.from_numpy(enc(np.pad(_weights(rng, n, k), ((0, 0), (0, bpr * 256 - k))))).to(dev))
+            elif type_name in ("iq2_xxs", "iq1_m"):
+                mats.append(torch.from_numpy((C.random_iq2_xxs if type_name == "iq2_xxs" else C.random_iq1_m)(rng, n, bpr)).to(dev))
+            else:
+                mats.append(torch.from_numpy(C.random_blocks(rng, type_name, n, bpr)).to(dev))
         gamma = torch.from_numpy(rng.uniform(0.5, 1.5, size=k).astype(np.float32)).to(dev)
         for dt in (torch.bfloat16, torch.float32):
             x = torch.from_numpy(rng.standard_normal((rows, k)).astype(np.float32)).to(dev).to(dt)
@@ -360,12 +362,16 @@ def test_multi_projection_equals_separate_calls(mod, type_name):
             got = mod.gguf_quant_gemm_multi_forward(x, mats, k, tid, grid, out_dtype=torch.float32)
             want = [mod.gguf_quant_gemm_forward(x, m, k, tid, grid, out_dtype=torch.float32) for m in mats]
             assert len(got) == len(want)
+            # The joint launch and the single calls may split a row's blocks over different numbers of waves (and IQ2_XXS / IQ1_M
+            # single calls may stream whole tiles), which sums in another order; with the normalisation the row's sum of squares
+            # is summed in another order too, which can move an activation code by one step.  A wrong matrix, height or output
+            # would be an error of order one.
             for a, b in zip(got, want):
-                assert a.shape == b.shape and torch.equal(a, b)
+                assert a.shape == b.shape and O.rel_l2(a.cpu().numpy(), b.cpu().numpy()) <= 2e-6
             got = mod.gguf_quant_gemm_multi_forward(x, mats, k, tid, grid, norm_weight=gamma, eps=1e-5, out_dtype=torch.float32)
             want = [mod.gguf_quant_gemm_rmsnorm_forward(x, gamma, 1e-5, m, k, tid, grid, out_dtype=torch.float32) for m in mats]
             for a, b in zip(got, want):
-                assert torch.equal(a, b)
+                assert a.shape == b.shape and O.rel_l2(a.cpu().numpy(), b.cpu().numpy()) <= 5e-5
     bb = mats[0].size(2)
     one, two = torch.zeros(8, 1, bb, dtype=torch.uint8, device=dev), torch.zeros(8, 2, bb, dtype=torch.uint8, device=dev)
     with pytest.raises(RuntimeError, match="same number of blocks per row"):
