@@ -5,7 +5,8 @@
 //   sigmoid mode: p = sigmoid(logits); pick the top_k of p + bias (bias optional); weight = p / max(sum of picked p, 1e-20)
 //   softmax mode: pick the top_k logits; weight = softmax over the picked logits (= softmax probabilities renormalised)
 //
-// Launch 1: one wave per (expert, group of 4 tokens), 16-byte loads, the gate row held in registers, the tokens side by side, 64-lane sums.  Launch 2: one
+// Launch 1: one wave per (expert, group of 4 tokens), 16-byte loads, the gate row held in registers, the tokens side by side, 64-lane sums;
+// from 80 tokens on 16 x 16 blocks of logits on the float32 matrix cores instead.  Launch 2: one
 // wave per token, every lane keeps E / 64 candidates in registers, top_k rounds of a wave-wide
 // argmax (larger score first, lower expert id on equal scores), picked in descending order.
 #include "pllm_device.h"
@@ -21,6 +22,7 @@ constexpr int kMaxPerLane = 16;          // experts per lane: up to 1024 experts
 // One wave per (expert, group of kTokensPerWave tokens): the gate row is read once per group (its
 // first kHeld float4 pieces per lane stay in registers), the tokens' rows come from cache.
 constexpr int kTokensPerWave = 4;        // their x loads are in flight together; a single token (decode) runs alone
+constexpr int kMfmaMinTokens = 80;       // from here on the logits are formed block by block on the matrix cores
 constexpr int kHeld = 12;                // 12 x 256 floats: gate rows up to 3072 wide are held whole
 
 template <int NT>
@@ -80,6 +82,56 @@ __global__ __launch_bounds__(kThreads) void route_logits_kernel(
         const float total = group_sum<64>(acc[j]);
         if (lane == 0 && t0 + j < t1) logits[static_cast<size_t>(t0 + j) * n_experts + e] = total;
     }
+}
+
+// Many tokens: a workgroup forms the 16 x 16 block logits[t0 .. t0 + 15, e0 .. e0 + 15] on the float32 matrix cores
+// (v_mfma_f32_16x16x4_f32, C[m][n] = sum_k A[m][k] B[k][n] with m = token, n = expert).  Lane (r, q) = (lane % 16, lane / 16)
+// loads four consecutive values of token row r and of gate row r at column k0 + 4 q; value i of both goes to MFMA i of the step,
+// where the lane's k index is q on either side.  The four waves split the row's columns and meet in LDS.  A block reads
+// 16 gate rows and 16 token rows once: an eighth of the cache traffic of the one-wave-per-expert form.  dim % 16 == 0.
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(kThreads) void route_logits_mfma_kernel(
+    const void* __restrict__ x, int x_dtype, const float* __restrict__ gate, float* __restrict__ logits, int dim, int n_experts, int tokens) {
+    __shared__ float partial[kWavesPerWg][16 * 16];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 15, q = lane >> 4;
+    const int e0 = blockIdx.x * 16, t0 = blockIdx.y * 16;
+    const float* grow = gate + static_cast<size_t>(min(e0 + r, n_experts - 1)) * dim;       // past the end: a valid row, result dropped
+    const size_t xoff = static_cast<size_t>(min(t0 + r, tokens - 1)) * dim;
+    const bool xvec = ((reinterpret_cast<uintptr_t>(x) & 15u) == 0);
+    const int per_wave = (dim / 16 + kWavesPerWg - 1) / kWavesPerWg * 16;                    // columns per wave, a multiple of 16
+    const int k_begin = wave * per_wave, k_end = min(dim, k_begin + per_wave);
+    v4f c = {0.0f, 0.0f, 0.0f, 0.0f};
+    constexpr int kUnroll = 4;
+    for (int k0 = k_begin; k0 < k_end; k0 += 16 * kUnroll) {
+        float4 g[kUnroll];
+        float xv[kUnroll][4];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const int col = min(k0 + 16 * u, k_end - 16) + 4 * q;                            // a step past the end repeats the last one ...
+            g[u] = *reinterpret_cast<const float4*>(grow + col);
+            load_row4(xv[u], x, x_dtype, xoff, col, dim, xvec);
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            if (k0 + 16 * u < k_end) {                                                       // ... and is not multiplied (wave-uniform)
+                c = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[u][0], g[u].x, c, 0, 0, 0);
+                c = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[u][1], g[u].y, c, 0, 0, 0);
+                c = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[u][2], g[u].z, c, 0, 0, 0);
+                c = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[u][3], g[u].w, c, 0, 0, 0);
+            }
+        }
+    }
+    // lane (n = r, quad q) holds C[4 q + i][n], i = 0..3: token t0 + 4 q + i, expert e0 + r
+#pragma unroll
+    for (int i = 0; i < 4; ++i) partial[wave][(4 * q + i) * 16 + r] = c[i];
+    __syncthreads();
+    const int m = threadIdx.x >> 4, n = threadIdx.x & 15;                                    // 256 threads, 256 outputs
+    float total = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kWavesPerWg; ++w) total += partial[w][m * 16 + n];
+    if (t0 + m < tokens && e0 + n < n_experts) logits[static_cast<size_t>(t0 + m) * n_experts + e0 + n] = total;
 }
 
 __device__ __forceinline__ float wave_max(float v) { return group_max<64>(v); }
@@ -164,7 +216,11 @@ int pllm_moe_route(const void* x, int x_dtype, int64_t tokens, int64_t dim, cons
     hipStream_t s = static_cast<hipStream_t>(stream);
     const dim3 wgs(static_cast<unsigned>((n_experts + kWavesPerWg - 1) / kWavesPerWg),
                    static_cast<unsigned>(tokens == 1 ? 1 : (tokens + kTokensPerWave - 1) / kTokensPerWave));
-    if (tokens == 1)
+    if (tokens >= kMfmaMinTokens && dim % 16 == 0 && dim >= 16 && ((reinterpret_cast<uintptr_t>(gate_weight) & 15u) == 0))
+        hipLaunchKernelGGL(route_logits_mfma_kernel, dim3(static_cast<unsigned>((n_experts + 15) / 16), static_cast<unsigned>((tokens + 15) / 16)),
+                           dim3(kThreads), 0, s, x, x_dtype, gate_weight, logits, static_cast<int>(dim), static_cast<int>(n_experts),
+                           static_cast<int>(tokens));
+    else if (tokens == 1)
         hipLaunchKernelGGL(route_logits_kernel<1>, wgs, dim3(kThreads), 0, s, x, x_dtype, gate_weight, logits, static_cast<int>(dim),
                            static_cast<int>(n_experts), static_cast<int>(tokens));
     else

@@ -261,7 +261,9 @@ def test_grouped_experts_tile_path(mod, t13, t2, limit):
     assert torch.equal(y, y2)
 
 
-@pytest.mark.parametrize("tokens,dim,n_experts,top_k", [(1, 3072, 256, 8), (7, 3072, 256, 8), (3, 1000, 60, 6), (2, 257, 1024, 64), (5, 64, 8, 8)])
+@pytest.mark.parametrize("tokens,dim,n_experts,top_k", [(1, 3072, 256, 8), (7, 3072, 256, 8), (3, 1000, 60, 6), (2, 257, 1024, 64), (5, 64, 8, 8),
+                                                        (16, 3072, 256, 8), (80, 1024, 60, 6), (256, 3072, 256, 8), (97, 48, 20, 4), (90, 1000, 60, 6),
+                                                        (81, 16, 5, 2)])
 def test_router_matches_the_reference_statement(mod, tokens, dim, n_experts, top_k):
     """MiniMaxMoE.route on the device: logits against float64, then selection and weights against the oracle evaluated on the
     device's own logits (a float dot in another order may legitimately swap two experts whose scores differ in the last bits,
