@@ -197,6 +197,15 @@ int pllm_gguf_dequantize_rows(const int64_t* row_ids, int64_t n_selected, const 
 int pllm_fp8_block_dequantize(const uint8_t* weight, const float* scale, int64_t n, int64_t k, void* out, int out_dtype, void* stream);
 int pllm_fp8_block_gemm(const void* x, int x_dtype, const uint8_t* weight, const float* scale, void* y, int y_dtype,
                         int64_t rows, int64_t k, int64_t n, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * The residual form of pllm_fp8_block_gemm for decode calls: y[t, r] += sum_c x[t, c] * out[r, c], the sum formed in float32 and
+ * rounded to y's type once (no workspace: the matvec kernel only; a row count of the tile kernel returns PLLM_ERR_UNSUPPORTED).
+ * Replaces soft_fp8_blockfp8_gemm (src/kernels/ops.py:641-648) followed by the separate addition of a transformer block's
+ * residual connection.
+ */
+int pllm_fp8_block_gemm_accumulate(const void* x, int x_dtype, const uint8_t* weight, const float* scale, void* y, int y_dtype,
+                                   int64_t rows, int64_t k, int64_t n, void* stream);
 size_t pllm_fp8_block_gemm_workspace_bytes(int64_t rows, int64_t k, int64_t n);
 
 /*

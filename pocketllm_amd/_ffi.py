@@ -40,6 +40,7 @@ SIGNATURES = {
     "pllm_gguf_dequantize_rows": (_int, [_c_void_p, _i64, _c_void_p, _int, _i64, _i64, _i64, _c_void_p, _int, _c_void_p]),
     "pllm_fp8_block_dequantize": (_int, [_c_void_p, _c_void_p, _i64, _i64, _c_void_p, _int, _c_void_p]),
     "pllm_fp8_block_gemm": (_int, [_c_void_p, _int, _c_void_p, _c_void_p, _c_void_p, _int, _i64, _i64, _i64, _c_void_p, _size_t, _c_void_p]),
+    "pllm_fp8_block_gemm_accumulate": (_int, [_c_void_p, _int, _c_void_p, _c_void_p, _c_void_p, _int, _i64, _i64, _i64, _c_void_p]),
     "pllm_fp8_block_gemm_workspace_bytes": (_size_t, [_i64, _i64, _i64]),
     "pllm_fp8_fp16scale_matvec": (_int, [_c_void_p, _int, _c_void_p, _c_void_p, _c_void_p, _int, _i64, _i64, _i64, _i64, _c_void_p]),
     "pllm_fp8_fp16scale_swiglu_matvec": (_int, [_c_void_p, _int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _int,

@@ -373,6 +373,16 @@ int pllm_fp8_block_gemm(const void* x, int x_dtype, const uint8_t* weight, const
                             static_cast<int>(n), static_cast<hipStream_t>(stream));
 }
 
+int pllm_fp8_block_gemm_accumulate(const void* x, int x_dtype, const uint8_t* weight, const float* scale, void* y, int y_dtype,
+                                   int64_t rows, int64_t k, int64_t n, void* stream) {
+    if (!x || !weight || !scale || !y || !dtype_ok(x_dtype) || !dtype_ok(y_dtype)) return PLLM_ERR_INVALID_ARGUMENT;
+    if (!fits_int(rows) || !fits_int(k) || !fits_int(n)) return PLLM_ERR_INVALID_ARGUMENT;
+    // the matvec only: the row counts pllm_fp8_block_gemm hands to the tile kernel are not served
+    if (rows > 65535 || fp8_uses_gemm(rows, k, n)) return PLLM_ERR_UNSUPPORTED;
+    return pllm::fp8_matvec(x, x_dtype, weight, scale, y, y_dtype | pllm::kAccumulateInto, static_cast<int>(rows), static_cast<int>(k),
+                            static_cast<int>(n), static_cast<hipStream_t>(stream));
+}
+
 // ---- FP8 with fp16 scales: the raw-pointer operators of the reference's C++ engine -----------------------------------
 
 static bool fp16scale_args_ok(const void* x, const void* w, const void* scale, const void* y, int64_t rows, int64_t cols,

@@ -357,6 +357,30 @@ def fp8_block_gemm_forward(x: torch.Tensor, weight: torch.Tensor, scale: torch.T
     return y
 
 
+def fp8_block_gemm_accumulate_forward(x: torch.Tensor, weight: torch.Tensor, scale: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
+    """y += fp8_block_gemm_forward(x, weight, scale) in place (a block's residual connection folded into the projection): one
+    launch for decode calls; row counts of the tile kernel run it and add separately."""
+    w8 = _fp8_bytes(weight)
+    n, k = w8.shape
+    _check(x.is_cuda and x.is_contiguous() and x.size(-1) == k, "x must be a contiguous CUDA tensor [..., K]")
+    _check_x(x)
+    _check(scale.is_cuda and scale.dtype == torch.float32 and scale.is_contiguous(), "scale must be a contiguous CUDA float32 tensor")
+    _check(tuple(scale.shape) == ((n + 127) // 128, (k + 127) // 128), "scale must have shape [ceil(N/128), ceil(K/128)]")
+    _check(y.is_cuda and y.device == x.device and y.is_contiguous() and y.dtype in _DTYPE_CODE, "y must be a contiguous CUDA tensor of float16, bfloat16 or float32")
+    _check(tuple(y.shape) == (*x.shape[:-1], n), "y must have x's leading shape and weight.size(0) columns")
+    rows = x.numel() // k
+    if rows == 0:
+        return y
+    with torch.cuda.device(x.device):
+        st = _lib().pllm_fp8_block_gemm_accumulate(x.data_ptr(), _DTYPE_CODE[x.dtype], w8.data_ptr(), scale.data_ptr(), y.data_ptr(),
+                                                   _DTYPE_CODE[y.dtype], rows, k, n, _stream(x.device))
+    if st == -2:                             # PLLM_ERR_UNSUPPORTED: a row count of the tile kernel
+        y.copy_((y.float() + fp8_block_gemm_forward(x, weight, scale, out_dtype=torch.float32)).to(y.dtype))
+        return y
+    _ffi.check(st, "fp8_block_gemm_accumulate_forward")
+    return y
+
+
 def fp8_gemm_forward(a: torch.Tensor, a_scale: torch.Tensor, weight: torch.Tensor, scale: torch.Tensor, *,
                      out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
     """fp8_gemm(a, a_s, b, b_s) of src/kernels/ops.py:1043-1051 on the native FP8 matrix path: `a` / `a_scale` are the

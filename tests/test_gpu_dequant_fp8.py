@@ -166,3 +166,22 @@ def test_fp8_act_quant_matches_reference_recipe(mod):
     want = O.fp8_gemm_q(xt.float().cpu().numpy(), w_codes, w_scale)
     # the native FP8 matrix-core path sums each 128-wide block in the hardware's own order and width
     assert O.rel_l2(y.cpu().numpy(), want) <= 2e-4
+
+
+@pytest.mark.parametrize("n,k,rows", [(130, 304, 1), (256, 1024, 3), (4500, 8192, 1), (64, 512, 20)])
+def test_fp8_accumulate_adds_the_product_to_y(mod, n, k, rows):
+    """y += W x for FP8 weights: the plain operator's float32 product plus the old y, rounded once to y's type."""
+    rng = np.random.default_rng(60 + n)
+    codes = rng.integers(0, 256, size=(n, k), dtype=np.uint8)
+    codes[(codes & 0x7f) == 0x7f] = 0x3c
+    scale = rng.uniform(0.001, 0.01, size=((n + 127) // 128, (k + 127) // 128)).astype(np.float32)
+    w, sc = torch.from_numpy(codes).to(DEV), torch.from_numpy(scale).to(DEV)
+    x = torch.from_numpy(rng.standard_normal((rows, k)).astype(np.float32)).to(DEV).to(torch.bfloat16)
+    prod = mod.fp8_block_gemm_forward(x, w, sc)
+    for ydt in (torch.float32, torch.bfloat16, torch.float16):
+        print(f"case fp8 accumulate n={n} k={k} rows={rows} {ydt}", flush=True)
+        y0 = torch.from_numpy(rng.standard_normal((rows, n)).astype(np.float32)).to(DEV).to(ydt)
+        y = y0.clone()
+        assert mod.fp8_block_gemm_accumulate_forward(x, w, sc, y) is y
+        torch.cuda.synchronize()
+        assert torch.equal(y, (y0.float() + prod).to(ydt))
