@@ -98,15 +98,17 @@ struct Q5K {
     }
 };
 
-template <typename FMT, int ITERS, bool RAW>
+// R activation rows per workgroup (1, 2 or 4): the weights of a super-block are loaded and split into codes once and multiplied
+// with the images of R rows, which sit side by side in LDS; grid row blockIdx.y serves activation rows R * blockIdx.y ...
+template <typename FMT, int ITERS, bool RAW, int R>
 __global__ __launch_bounds__(64 * kMaxWaves) void k45_mfma_matvec_kernel(
-    const ActRows act, const WeightRoute route, const uint8_t* __restrict__ w, void* __restrict__ y, int y_dtype, int n, int bpr) {
+    const ActRows act, const WeightRoute route, const uint8_t* __restrict__ w, void* __restrict__ y, int y_dtype, int n, int bpr, int total_rows) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int kpad = bpr * 256;
-    const int image_bytes = static_cast<int>(staged_x_bytes(kpad));
+    const int image_bytes = static_cast<int>(staged_x_bytes(kpad));          // a multiple of 16
     const StagedX sx = carve_staged_x(smem, kpad);
-    const int zero_off = image_bytes;                                        // 16 zero bytes
-    float* partial = reinterpret_cast<float*>(smem + image_bytes + 16);     // [waves][16]
+    const int zero_off = R * image_bytes;                                    // 16 zero bytes
+    float* partial = reinterpret_cast<float*>(smem + R * image_bytes + 16); // [R][waves][16]
 
     const int tid = threadIdx.x;
     const int waves = blockDim.x >> 6;
@@ -122,25 +124,31 @@ __global__ __launch_bounds__(64 * kMaxWaves) void k45_mfma_matvec_kernel(
         n = route.more_n[m];
     }
     if (static_cast<int>(blockIdx.x) * kRowsPerWg >= n) return;             // the grid covers the tallest matrix
-    const size_t image_row = act.row_token ? static_cast<size_t>(act.row_token[blockIdx.y]) : blockIdx.y;
+    const int row0 = blockIdx.y * R;                                         // first activation row of this workgroup
     const int row = blockIdx.x * kRowsPerWg + col;
     const uint8_t* wrow = w + static_cast<size_t>(row < n ? row : 0) * bpr * FMT::kBlockBytes;
 
     // A side: this lane supplies row m = col = 2 * group + term of MFMA t, slice ks; it is non-zero
     // only when MFMA t's slice ks belongs to `group`: G(t, ks) = 4 * (t >> 1) + 2 * (ks >> 1) + (t & 1)
-    int a_off[4], a_step[4];
+    int a_off[4], a_step[4], a_row[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
         const int g = 4 * (t >> 1) + 2 * (ks >> 1) + (t & 1);
         const bool active = (col >> 1) == g;
         a_off[t] = active ? ((col & 1) ? kpad : 0) + 32 * g + 16 * (ks & 1) : zero_off;
         a_step[t] = active ? 256 : 0;
+        a_row[t] = active ? image_bytes : 0;                                 // distance to the next activation row's image
     }
 
-    float acc = 0.0f;
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = 0.0f;
     bool staged = false;
     if constexpr (RAW) {                     // quantize before the loads take their registers
-        quantize_row_to_lds(smem, act.x, act.x_dtype, static_cast<size_t>(blockIdx.y) * act.k, act.k, kpad, RowNorm{act.gamma, act.eps, act.round_f16});
+#pragma unroll 1
+        for (int r = 0; r < R; ++r)          // rows past the end: the last row again, result dropped
+            quantize_row_to_lds(smem + r * image_bytes, act.x, act.x_dtype, static_cast<size_t>(min(row0 + r, total_rows - 1)) * act.k, act.k, kpad,
+                                RowNorm{act.gamma, act.eps, act.round_f16});
         if (tid < 4) reinterpret_cast<uint32_t*>(smem + zero_off)[tid] = 0;
         __syncthreads();
         staged = true;
@@ -153,7 +161,12 @@ __global__ __launch_bounds__(64 * kMaxWaves) void k45_mfma_matvec_kernel(
             FMT::load(regs[it], wrow + static_cast<size_t>(b) * FMT::kBlockBytes, ks);
         }
         if (!staged) {                       // first trip of every thread of the workgroup
-            copy_to_lds(smem, act.image + image_row * act.stride, image_bytes);
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const int arow = min(row0 + r, total_rows - 1);
+                const size_t image_row = act.row_token ? static_cast<size_t>(act.row_token[arow]) : static_cast<size_t>(arow);
+                copy_to_lds(smem + r * image_bytes, act.image + image_row * act.stride, image_bytes);
+            }
             if (tid < 4) reinterpret_cast<uint32_t*>(smem + zero_off)[tid] = 0;
             __syncthreads();
             staged = true;
@@ -164,44 +177,54 @@ __global__ __launch_bounds__(64 * kMaxWaves) void k45_mfma_matvec_kernel(
             if (b < bpr) {                                                   // wave-uniform
                 uint4 bw[4];
                 FMT::codes(regs[it], ks, bw);
-                v4i c = {0, 0, 0, 0};
-#pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    const uint4 a = *reinterpret_cast<const uint4*>(smem + a_off[t] + b * a_step[t]);
-                    c = __builtin_amdgcn_mfma_i32_16x16x64_i8(as_v4i(a), as_v4i(bw[t]), c, 0, 0, 0);
-                }
-                // c = {group 2ks: hi, lo; group 2ks+1: hi, lo} for output row `col`
-                const float v0 = static_cast<float>(__mul24(c.x, 254) + c.y);
-                const float v1 = static_cast<float>(__mul24(c.z, 254) + c.w);
-                const float4 g2 = *reinterpret_cast<const float4*>(sx.gs + b * 8 + 2 * ks);   // {xs0, sum0, xs1, sum1}
                 const K4Scales sc = k4_unpack(regs[it].hdr);
                 const uint32_t scw = ((ks & 2) ? sc.sc_hi : sc.sc_lo) >> (16 * (ks & 1));
                 const uint32_t mnw = ((ks & 2) ? sc.mn_hi : sc.mn_lo) >> (16 * (ks & 1));
-                const float pos = static_cast<float>(scw & 0xffu) * g2.x * v0 + static_cast<float>((scw >> 8) & 0xffu) * g2.z * v1;
-                const float neg = static_cast<float>(mnw & 0xffu) * g2.y + static_cast<float>((mnw >> 8) & 0xffu) * g2.w;
                 const float d = f16_bits_to_float(regs[it].hdr.x & 0xffffu);
                 const float dmin = f16_bits_to_float(regs[it].hdr.x >> 16);
-                acc += d * pos - dmin * neg;
+                const float s0 = static_cast<float>(scw & 0xffu), s1 = static_cast<float>((scw >> 8) & 0xffu);
+                const float m0 = static_cast<float>(mnw & 0xffu), m1 = static_cast<float>((mnw >> 8) & 0xffu);
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    v4i c = {0, 0, 0, 0};
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        const uint4 a = *reinterpret_cast<const uint4*>(smem + a_off[t] + b * a_step[t] + r * a_row[t]);
+                        c = __builtin_amdgcn_mfma_i32_16x16x64_i8(as_v4i(a), as_v4i(bw[t]), c, 0, 0, 0);
+                    }
+                    // c = {group 2ks: hi, lo; group 2ks+1: hi, lo} for output row `col`
+                    const float v0 = static_cast<float>(__mul24(c.x, 254) + c.y);
+                    const float v1 = static_cast<float>(__mul24(c.z, 254) + c.w);
+                    const float4 g2 = *reinterpret_cast<const float4*>(reinterpret_cast<const unsigned char*>(sx.gs + b * 8 + 2 * ks) + r * image_bytes);   // {xs0, sum0, xs1, sum1}
+                    const float pos = s0 * g2.x * v0 + s1 * g2.z * v1;
+                    const float neg = m0 * g2.y + m1 * g2.w;
+                    acc[r] += d * pos - dmin * neg;
+                }
             }
         }
     }
-    acc += __shfl_xor(acc, 16, 64);
-    acc += __shfl_xor(acc, 32, 64);
-    if (ks == 0) partial[wave * kRowsPerWg + col] = acc;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        float a = acc[r];
+        a += __shfl_xor(a, 16, 64);
+        a += __shfl_xor(a, 32, 64);
+        if (ks == 0) partial[(r * waves + wave) * kRowsPerWg + col] = a;
+    }
     __syncthreads();
-    if (tid < kRowsPerWg) {
+    if (tid < kRowsPerWg * R) {
+        const int r = tid / kRowsPerWg, c = tid % kRowsPerWg;
         float total = 0.0f;
-        for (int v = 0; v < waves; ++v) total += partial[v * kRowsPerWg + tid];
-        const int out_row = blockIdx.x * kRowsPerWg + tid;
-        if (out_row < n) store_any(y, y_dtype, static_cast<size_t>(blockIdx.y) * n + out_row, total);
+        for (int v = 0; v < waves; ++v) total += partial[(r * waves + v) * kRowsPerWg + c];
+        const int out_row = blockIdx.x * kRowsPerWg + c;
+        if (out_row < n && row0 + r < total_rows) store_any(y, y_dtype, static_cast<size_t>(row0 + r) * n + out_row, total);
     }
 }
 
 // ------------------------------------------------------------------------------------------------
 template <typename KERN>
 int launch_kernel(KERN kern, const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype,
-                  int rows, int n, int bpr, int waves, hipStream_t stream) {
-    const size_t smem = staged_x_bytes(bpr * 256) + 16 + static_cast<size_t>(waves) * kRowsPerWg * sizeof(float);
+                  int rows, int n, int bpr, int waves, int rows_per_wg, hipStream_t stream) {
+    const size_t smem = rows_per_wg * staged_x_bytes(bpr * 256) + 16 + static_cast<size_t>(rows_per_wg) * waves * kRowsPerWg * sizeof(float);
     if (smem > 64 * 1024) {
         if (smem > 160 * 1024) return PLLM_ERR_UNSUPPORTED;
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -210,8 +233,8 @@ int launch_kernel(KERN kern, const ActRows& act, const WeightRoute& route, const
     }
     int tallest = n;
     for (int m = 0; m < route.extra; ++m) tallest = tallest > route.more_n[m] ? tallest : route.more_n[m];
-    dim3 grid((tallest + kRowsPerWg - 1) / kRowsPerWg, rows, 1 + route.extra);
-    hipLaunchKernelGGL(kern, grid, dim3(64 * waves), smem, stream, act, route, w, y, y_dtype, n, bpr);
+    dim3 grid((tallest + kRowsPerWg - 1) / kRowsPerWg, (rows + rows_per_wg - 1) / rows_per_wg, 1 + route.extra);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * waves), smem, stream, act, route, w, y, y_dtype, n, bpr, rows);
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 
@@ -227,19 +250,34 @@ void split_blocks(int bpr, int work_items, int& waves, int& iters) {
     if (iters == 7) iters = 8;
 }
 
-template <typename FMT>
-int launch_k45(const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream) {
+template <typename FMT, int R>
+int launch_k45_rows(const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream) {
     int waves, iters;
     int tiles = (n + kRowsPerWg - 1) / kRowsPerWg;
     for (int m = 0; m < route.extra; ++m) tiles += (route.more_n[m] + kRowsPerWg - 1) / kRowsPerWg;
-    split_blocks(bpr, tiles * rows, waves, iters);
-#define PLLM_CASE(I) case I: return act.x ? launch_kernel(k45_mfma_matvec_kernel<FMT, I, true>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream) \
-                                          : launch_kernel(k45_mfma_matvec_kernel<FMT, I, false>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream)
+    split_blocks(bpr, tiles * ((rows + R - 1) / R), waves, iters);
+#define PLLM_CASE(I) case I: \
+        if constexpr (R == 1) if (act.x) return launch_kernel(k45_mfma_matvec_kernel<FMT, I, true, 1>, act, route, w, y, y_dtype, rows, n, bpr, waves, 1, stream); \
+        return launch_kernel(k45_mfma_matvec_kernel<FMT, I, false, R>, act, route, w, y, y_dtype, rows, n, bpr, waves, R, stream)
     switch (iters) {
         PLLM_CASE(1); PLLM_CASE(2); PLLM_CASE(3); PLLM_CASE(4); PLLM_CASE(5); PLLM_CASE(6);
         default: PLLM_CASE(8);
     }
 #undef PLLM_CASE
+}
+
+// Activation rows per workgroup: routed calls address experts and image rows per grid row and stay at one, and so do calls that
+// quantize their rows in the kernel (measured: four rows quantized one after the other cost more than the shared weight pass
+// saves, Q4_K 5120x5120 at 4 rows 16.9 us against 14.2); calls on pre-quantized images take pairs at two rows and fours
+// from three on (three rows as two pairs: 31.5 us against 28.4 as one four), as long as the images leave room in LDS for three workgroups per compute unit (Q4_K 17408x5120: 24.8 -> 21.9 us
+// at 2 rows, 39.5 -> 29.1 us at 4).
+template <typename FMT>
+int launch_k45(const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream) {
+    const size_t image = staged_x_bytes(bpr * 256);
+    const bool plain = !route.expert && !act.row_token && !act.x;
+    if (plain && rows >= 3 && 4 * image <= 52 * 1024) return launch_k45_rows<FMT, 4>(act, route, w, y, y_dtype, rows, n, bpr, stream);
+    if (plain && rows >= 2 && 2 * image <= 52 * 1024) return launch_k45_rows<FMT, 2>(act, route, w, y, y_dtype, rows, n, bpr, stream);
+    return launch_k45_rows<FMT, 1>(act, route, w, y, y_dtype, rows, n, bpr, stream);
 }
 
 }  // namespace
