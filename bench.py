@@ -513,7 +513,7 @@ def main() -> None:
             traffic = json.load(f).get("q5_k matvec 17408x5120 T=1")
     roofline = {"bound": "hbm", "achieved": round(kernel_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(kernel_gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
-                "kernel": "k45_mfma_matvec_kernel<Q5K, 5, false> (q5_k matvec 17408x5120, activation image prepared by act_image_256_kernel)",
+                "kernel": "k45_mfma_matvec_kernel<Q5K, 5, false, 1> (q5_k matvec 17408x5120, activation image prepared by act_image_256_kernel)",
                 "bytes_per_launch": dom["weight_bytes"], "us_per_launch": round(kernel_us, 3),
                 "us_per_operator_call": dom["us_per_call"]}
 
