@@ -95,9 +95,36 @@ __device__ __forceinline__ void fp8_fetch_pass(uint4 (&r)[kRowsPerWave][ITERS], 
     }
 }
 
-template <int ITERS, int F16S, bool SWIGLU>
-__device__ __forceinline__ void fp8_multiply_pass(float (&acc)[kRowsPerWave], const uint4 (&r)[kRowsPerWave][ITERS], const float* xs, const Fp8Mat& ma,
-                                                  const Fp8Mat& mb, int row0, int n, int chunks, int c0, int lane) {
+// 16 codes as floats, converted once for all activation rows
+__device__ __forceinline__ void chunk_floats(float (&f)[16], const uint4& w) {
+    v2f a;
+    a = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w.x), false); f[0] = a.x; f[1] = a.y;
+    a = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w.x), true);  f[2] = a.x; f[3] = a.y;
+    a = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w.y), false); f[4] = a.x; f[5] = a.y;
+    a = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w.y), true);  f[6] = a.x; f[7] = a.y;
+    a = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w.z), false); f[8] = a.x; f[9] = a.y;
+    a = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w.z), true);  f[10] = a.x; f[11] = a.y;
+    a = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w.w), false); f[12] = a.x; f[13] = a.y;
+    a = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w.w), true);  f[14] = a.x; f[15] = a.y;
+}
+
+// the same summation order as chunk_dot
+__device__ __forceinline__ float floats_dot(const float (&f)[16], const float* xp) {
+    const float4 x0 = *reinterpret_cast<const float4*>(xp);
+    const float4 x1 = *reinterpret_cast<const float4*>(xp + 4);
+    const float4 x2 = *reinterpret_cast<const float4*>(xp + 8);
+    const float4 x3 = *reinterpret_cast<const float4*>(xp + 12);
+    float s = f[0] * x0.x; s += f[1] * x0.y; s += f[2] * x0.z; s += f[3] * x0.w;
+    s += f[4] * x1.x; s += f[5] * x1.y; s += f[6] * x1.z; s += f[7] * x1.w;
+    s += f[8] * x2.x; s += f[9] * x2.y; s += f[10] * x2.z; s += f[11] * x2.w;
+    s += f[12] * x3.x; s += f[13] * x3.y; s += f[14] * x3.z; s += f[15] * x3.w;
+    return s;
+}
+
+// R activation rows (xs holds them k floats apart) against the pass's weights: the codes are converted once per chunk
+template <int ITERS, int F16S, bool SWIGLU, int R>
+__device__ __forceinline__ void fp8_multiply_pass(float (&acc)[kRowsPerWave][R], const uint4 (&r)[kRowsPerWave][ITERS], const float* xs, int k,
+                                                  const Fp8Mat& ma, const Fp8Mat& mb, int row0, int n, int chunks, int c0, int lane) {
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
         const int c = c0 + it * 64 + lane;
@@ -105,66 +132,86 @@ __device__ __forceinline__ void fp8_multiply_pass(float (&acc)[kRowsPerWave], co
         const int cc = ok ? c : 0;
 #pragma unroll
         for (int q = 0; q < kRowsPerWave; ++q) {
-            const float d = chunk_dot(r[q][it], xs + 16 * cc);
             const Fp8Mat& m = slot_mat<SWIGLU>(ma, mb, q);
             const float sc = scale_at<F16S>(m.scale, static_cast<size_t>(slot_row<SWIGLU>(row0, q, n) >> 7) * m.sstride + (cc >> 3));
-            acc[q] += ok ? d * sc : 0.0f;
+            if constexpr (R == 1) {
+                const float d = chunk_dot(r[q][it], xs + 16 * cc);
+                acc[q][0] += ok ? d * sc : 0.0f;
+            } else {
+                float f[16];
+                chunk_floats(f, r[q][it]);
+#pragma unroll
+                for (int a = 0; a < R; ++a) {
+                    const float d = floats_dot(f, xs + static_cast<size_t>(a) * k + 16 * cc);
+                    acc[q][a] += ok ? d * sc : 0.0f;
+                }
+            }
         }
     }
 }
 
-template <bool SWIGLU>
-__device__ __forceinline__ void fp8_store_rows(float (&acc)[kRowsPerWave], void* __restrict__ y, int y_dtype, size_t yoff, int row0, int n, int lane) {
-    float total[kRowsPerWave];
+// activation rows arow0 .. arow0 + R - 1 (those below total_rows) of output row(s) row0
+template <bool SWIGLU, int R>
+__device__ __forceinline__ void fp8_store_rows(float (&acc)[kRowsPerWave][R], void* __restrict__ y, int y_dtype, size_t y_stride, int arow0, int total_rows,
+                                               int row0, int n, int lane) {
 #pragma unroll
-    for (int q = 0; q < kRowsPerWave; ++q) { total[q] = group_sum<64>(acc[q]); acc[q] = 0.0f; }
-    if constexpr (SWIGLU) {
-        if (lane == 0 && row0 < n) store_any(y, y_dtype, yoff + row0, silu(total[0]) * total[1]);
-    } else {
+    for (int a = 0; a < R; ++a) {
+        float total[kRowsPerWave];
 #pragma unroll
-        for (int q = 0; q < kRowsPerWave; ++q)
-            if (lane == 0 && row0 + q < n) store_any(y, y_dtype, yoff + row0 + q, total[q]);
+        for (int q = 0; q < kRowsPerWave; ++q) { total[q] = group_sum<64>(acc[q][a]); acc[q][a] = 0.0f; }
+        if (arow0 + a >= total_rows) continue;
+        const size_t yoff = static_cast<size_t>(arow0 + a) * y_stride;
+        if constexpr (SWIGLU) {
+            if (lane == 0 && row0 < n) store_any(y, y_dtype, yoff + row0, silu(total[0]) * total[1]);
+        } else {
+#pragma unroll
+            for (int q = 0; q < kRowsPerWave; ++q)
+                if (lane == 0 && row0 + q < n) store_any(y, y_dtype, yoff + row0 + q, total[q]);
+        }
     }
 }
 
-template <int ITERS, int F16S, bool SWIGLU, bool LONG_ROWS>
+template <int ITERS, int F16S, bool SWIGLU, bool LONG_ROWS, int R>
 __global__ __launch_bounds__(kThreads) void fp8_persistent_matvec_kernel(
     const void* __restrict__ x, int x_dtype, size_t x_stride, const Fp8Mat ma, const Fp8Mat mb,
-    void* __restrict__ y, int y_dtype, size_t y_stride, int k, int n, int groups, int passes_of_long_rows) {
+    void* __restrict__ y, int y_dtype, size_t y_stride, int k, int n, int groups, int passes_of_long_rows, int total_rows) {
     const int passes = LONG_ROWS ? passes_of_long_rows : 1;                  // a constant for rows that fit one pass
     extern __shared__ __align__(16) unsigned char smem[];
-    float* xs = reinterpret_cast<float*>(smem);
+    float* xs = reinterpret_cast<float*>(smem);                              // R activation rows, k floats apart
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int chunks = k >> 4;
-    const size_t xoff = static_cast<size_t>(blockIdx.y) * x_stride;
-    const size_t yoff = static_cast<size_t>(blockIdx.y) * y_stride;
+    const int arow0 = blockIdx.y * R;                                        // this workgroup's first activation row
     constexpr int per_wave = SWIGLU ? 1 : kRowsPerWave;
     constexpr int kPassChunks = 64 * ITERS;
     const int rows_per_group = kWaves * per_wave, wave_row = wave * per_wave;
     const int step = gridDim.x;
 
     uint4 a[kRowsPerWave][ITERS], b[kRowsPerWave][ITERS];
-    float acc[kRowsPerWave];
+    float acc[kRowsPerWave][R];
 #pragma unroll
-    for (int q = 0; q < kRowsPerWave; ++q) acc[q] = 0.0f;
+    for (int q = 0; q < kRowsPerWave; ++q)
+#pragma unroll
+        for (int r = 0; r < R; ++r) acc[q][r] = 0.0f;
     int g = blockIdx.x, p = 0;               // the pass being multiplied
     int gn = g, pn = 0;                      // the pass being fetched
     fp8_fetch_pass<ITERS, SWIGLU>(a, ma, mb, g * rows_per_group + wave_row, n, chunks, 0, lane);
-    stage_row_f32(xs, x, x_dtype, xoff, k);
+#pragma unroll 1
+    for (int r = 0; r < R; ++r)              // rows past the end: the last row again, result dropped
+        stage_row_f32(xs + static_cast<size_t>(r) * k, x, x_dtype, static_cast<size_t>(min(arow0 + r, total_rows - 1)) * x_stride, k);
     __syncthreads();
     while (g < groups) {
         if (++pn == passes) { pn = 0; gn += step; }
         if (gn < groups) fp8_fetch_pass<ITERS, SWIGLU>(b, ma, mb, gn * rows_per_group + wave_row, n, chunks, pn * kPassChunks, lane);
-        fp8_multiply_pass<ITERS, F16S, SWIGLU>(acc, a, xs, ma, mb, g * rows_per_group + wave_row, n, chunks, p * kPassChunks, lane);
-        if (p == passes - 1) fp8_store_rows<SWIGLU>(acc, y, y_dtype, yoff, g * rows_per_group + wave_row, n, lane);
+        fp8_multiply_pass<ITERS, F16S, SWIGLU, R>(acc, a, xs, k, ma, mb, g * rows_per_group + wave_row, n, chunks, p * kPassChunks, lane);
+        if (p == passes - 1) fp8_store_rows<SWIGLU, R>(acc, y, y_dtype, y_stride, arow0, total_rows, g * rows_per_group + wave_row, n, lane);
         g = gn; p = pn;
         if (g >= groups) break;
         if (++pn == passes) { pn = 0; gn += step; }
         if (gn < groups) fp8_fetch_pass<ITERS, SWIGLU>(a, ma, mb, gn * rows_per_group + wave_row, n, chunks, pn * kPassChunks, lane);
-        fp8_multiply_pass<ITERS, F16S, SWIGLU>(acc, b, xs, ma, mb, g * rows_per_group + wave_row, n, chunks, p * kPassChunks, lane);
-        if (p == passes - 1) fp8_store_rows<SWIGLU>(acc, y, y_dtype, yoff, g * rows_per_group + wave_row, n, lane);
+        fp8_multiply_pass<ITERS, F16S, SWIGLU, R>(acc, b, xs, k, ma, mb, g * rows_per_group + wave_row, n, chunks, p * kPassChunks, lane);
+        if (p == passes - 1) fp8_store_rows<SWIGLU, R>(acc, y, y_dtype, y_stride, arow0, total_rows, g * rows_per_group + wave_row, n, lane);
         g = gn; p = pn;
     }
 }
@@ -221,27 +268,34 @@ int launch_any(const void* x, int x_dtype, size_t x_stride, const Fp8Mat& ma, co
                            y, y_dtype, y_stride, k, n);
         return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
     }
-    const size_t smem = static_cast<size_t>(k) * sizeof(float);
     const int rows_per_group = kWaves * (SWIGLU ? 1 : kRowsPerWave);
     const int groups = (n + rows_per_group - 1) / rows_per_group;
     const int niter = ((k >> 4) + 63) / 64;
     const int passes = (niter + 5) / 6;
     const int iters = (niter + passes - 1) / passes;
-    // persistent: the workgroups that fit a compute unit at once (two by registers, fewer when the activation row fills LDS),
+    // activation rows per workgroup: pairs from two rows on and fours from three on share one pass over the weights, as long as two
+    // workgroups' rows fit LDS
+    const int share = (rows >= 3 && static_cast<size_t>(k) * 4 * 4 <= 80 * 1024) ? 4 : (rows >= 2 && static_cast<size_t>(k) * 4 * 2 <= 80 * 1024) ? 2 : 1;
+    const size_t smem = static_cast<size_t>(share) * k * sizeof(float);
+    // persistent: the workgroups that fit a compute unit at once (two by registers, fewer when the activation rows fill LDS),
     // groups dealt round-robin
     const int per_cu = std::max(1, std::min(2, static_cast<int>((160 * 1024) / std::max<size_t>(smem, 1))));
     const int grid_x = std::min(groups, per_cu * compute_units());
-#define PLLM_PCASE(I) case I: { \
-        auto kern = passes > 1 ? fp8_persistent_matvec_kernel<I, F16S, SWIGLU, true> : fp8_persistent_matvec_kernel<I, F16S, SWIGLU, false>; \
+    const dim3 grid(grid_x, (rows + share - 1) / share);
+    // (the form with a compile-time pass count keeps both register sets and all accumulators of several rows live at once and spills;
+    // several activation rows always run the form with the pass count as a variable)
+#define PLLM_LAUNCH(I, RR) { \
+        auto kern = (passes > 1 || RR > 1) ? fp8_persistent_matvec_kernel<I, F16S, SWIGLU, true, RR> : fp8_persistent_matvec_kernel<I, F16S, SWIGLU, false, 1>; \
         if (smem > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, \
                                                     static_cast<int>(smem)) != hipSuccess) return PLLM_ERR_UNSUPPORTED; \
-        hipLaunchKernelGGL(kern, dim3(grid_x, rows), dim3(kThreads), smem, stream, x, x_dtype, x_stride, ma, mb, y, y_dtype, y_stride, k, n, groups, passes); \
-        break; }
+        hipLaunchKernelGGL(kern, grid, dim3(kThreads), smem, stream, x, x_dtype, x_stride, ma, mb, y, y_dtype, y_stride, k, n, groups, passes, rows); }
+#define PLLM_PCASE(I) case I: if (share == 4) PLLM_LAUNCH(I, 4) else if (share == 2) PLLM_LAUNCH(I, 2) else PLLM_LAUNCH(I, 1) break;
     switch (iters) {
         PLLM_PCASE(1) PLLM_PCASE(2) PLLM_PCASE(3) PLLM_PCASE(4) PLLM_PCASE(5)
         default: PLLM_PCASE(6)
     }
 #undef PLLM_PCASE
+#undef PLLM_LAUNCH
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 
