@@ -167,6 +167,10 @@ def extra_cases(mod, dev, iters):
     ring = ring_of(blocks, dev, 12)
     run("q4_k paired projection 2 x 17408x5120 T=1", 2 * blocks.size,
         lambda s, ring=ring: mod.gguf_quant_gemm_pair_forward(x, ring[s], 5120, 3, ring[(s + 6) % 12], 5120, 3, empty), len(ring))
+    # a few activation rows (speculative decoding, small batches): two or four rows share one pass over the weights
+    for t in (2, 4):
+        xt = torch.randn(t, 5120, device=dev, dtype=torch.bfloat16)
+        run(f"q4_k matvec 17408x5120 T={t}", blocks.size, lambda s, ring=ring, xt=xt: mod.gguf_quant_gemm_forward(xt, ring[s], 5120, 3, empty), len(ring))
     del ring
     # normalisation + projection as one decode operator against the two operators one after the other (Q4_K 5120x5120)
     blocks = C.quantize_q4_k((rng.standard_normal((5120, 5120), dtype=np.float32) * np.float32(0.02)))
@@ -183,6 +187,9 @@ def extra_cases(mod, dev, iters):
     sc = torch.from_numpy(scale).to(dev)
     run("fp8_e4m3 matvec 17408x5120 T=1", codes.size + scale.size * 4,
         lambda s, ring=ring, x=x, sc=sc: mod.fp8_block_gemm_forward(x, ring[s], sc), len(ring))
+    x2 = torch.randn(2, 5120, device=dev, dtype=torch.bfloat16)
+    run("fp8_e4m3 matvec 17408x5120 T=2", codes.size + scale.size * 4,
+        lambda s, ring=ring, x2=x2, sc=sc: mod.fp8_block_gemm_forward(x2, ring[s], sc), len(ring))
     del ring
     # the same weights with fp16 scales behind the C++ engine's operator forms: matvec and fused gate/up SwiGLU (float32 activations)
     from pocketllm_amd import qwen_fp8_ops as Q
