@@ -7,6 +7,7 @@ from pathlib import Path
 LIB_PATH = Path(__file__).resolve().parent / "libpllm_hip.so"
 
 PLLM_OK = 0
+PLLM_ERR_UNSUPPORTED = -2        # include/pllm_hip.h: type id or shape outside what the kernels implement
 DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
 TYPE_Q8_0 = 100
 

@@ -10,6 +10,8 @@ parity checks can read the float32 accumulators before the bf16 rounding.
 """
 from __future__ import annotations
 
+import ctypes
+
 import torch
 
 from pocketllm_amd import _ffi
@@ -145,7 +147,6 @@ def gguf_quant_gemm_multi_forward(x, blocks_list, row_elems, type_id, signed_gri
     gguf_quant_gemm_rmsnorm_forward), as ONE launch where the library has one: up to four matrices of any heights and one format
     (any but Q2_K) at decode row counts.  The generalization of gguf_quant_gemm_pair_forward (src/csrc/cuda_kernel.cpp:615-666) to q / k / v.
     Everything else runs one operator call per matrix.  Returns the list of outputs."""
-    import ctypes
     row_elems, type_id = int(row_elems), int(type_id)
     blocks_list = list(blocks_list)
     _check(len(blocks_list) >= 1, "blocks_list must hold at least one matrix")
@@ -177,7 +178,7 @@ def gguf_quant_gemm_multi_forward(x, blocks_list, row_elems, type_id, signed_gri
             count, (ctypes.c_void_p * count)(*[b.data_ptr() for b in blocks_list]), (ctypes.c_int64 * count)(*[b.size(0) for b in blocks_list]),
             type_id, (ctypes.c_void_p * count)(*[t.data_ptr() for t in ys]), _DTYPE_CODE[out_dtype], rows, row_elems, bpr,
             ws.data_ptr(), ws_bytes, _stream(x.device))
-    if st == -2:                             # PLLM_ERR_UNSUPPORTED: no single launch for this format or row count
+    if st == _ffi.PLLM_ERR_UNSUPPORTED:      # no single launch for this format or row count
         return one_by_one()
     _ffi.check(st, "gguf_quant_gemm_multi_forward")
     return ys
@@ -202,7 +203,7 @@ def gguf_quant_gemm_accumulate_forward(x, blocks, row_elems, type_id, signed_gri
         st = lib.pllm_gguf_quant_gemm_accumulate(x.data_ptr(), _DTYPE_CODE[x.dtype], blocks.data_ptr(), type_id, y.data_ptr(),
                                                  _DTYPE_CODE[y.dtype], rows, row_elems, n, blocks.size(1), ws.data_ptr(), ws_bytes,
                                                  _stream(x.device))
-    if st == -2:                             # PLLM_ERR_UNSUPPORTED: a row count of the tile kernel
+    if st == _ffi.PLLM_ERR_UNSUPPORTED:      # a row count of the tile kernel
         prod = _dense_gemm("gguf_quant_gemm_accumulate_forward", x, blocks, row_elems, type_id, signed_grid, torch.float32)
         y.copy_((y.float() + prod).to(y.dtype))
         return y
@@ -374,7 +375,7 @@ def fp8_block_gemm_accumulate_forward(x: torch.Tensor, weight: torch.Tensor, sca
     with torch.cuda.device(x.device):
         st = _lib().pllm_fp8_block_gemm_accumulate(x.data_ptr(), _DTYPE_CODE[x.dtype], w8.data_ptr(), scale.data_ptr(), y.data_ptr(),
                                                    _DTYPE_CODE[y.dtype], rows, k, n, _stream(x.device))
-    if st == -2:                             # PLLM_ERR_UNSUPPORTED: a row count of the tile kernel
+    if st == _ffi.PLLM_ERR_UNSUPPORTED:      # a row count of the tile kernel
         y.copy_((y.float() + fp8_block_gemm_forward(x, weight, scale, out_dtype=torch.float32)).to(y.dtype))
         return y
     _ffi.check(st, "fp8_block_gemm_accumulate_forward")
