@@ -266,8 +266,15 @@ int launch_stream_raw(const ActRows& act, const uint8_t* w, void* y, int y_dtype
             return PLLM_ERR_UNSUPPORTED;
         attr_smem = smem;
     }
-    int per_cu = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, 64 * kWaves, smem) != hipSuccess || per_cu < 1) per_cu = 1;
+    // resident workgroups per compute unit for this LDS size: asked once per size (the query costs microseconds of host time)
+    static size_t occ_smem = ~static_cast<size_t>(0);
+    static int occ_per_cu = 1;
+    if (smem != occ_smem) {
+        int q = 0;
+        occ_per_cu = (hipOccupancyMaxActiveBlocksPerMultiprocessor(&q, kern, 64 * kWaves, smem) == hipSuccess && q >= 1) ? q : 1;
+        occ_smem = smem;
+    }
+    const int per_cu = occ_per_cu;
     const int chunks = (n / kRowsPerTile + tiles_per_chunk - 1) / tiles_per_chunk;
     const int resident = per_cu * compute_units();
     int grid = chunks;

@@ -383,10 +383,19 @@ int launch_single_w13(const void* x, int x_dtype, int dim, int bpr, const int64_
 }
 
 // workgroups of a persistent kernel that fit the device at once
+// (asked again only when kernel, threads or LDS size change: the query costs microseconds of host time)
 template <typename KERN>
 int resident_workgroups(KERN kern, int threads, size_t smem) {
-    int per_cu = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, threads, smem) != hipSuccess || per_cu < 1) per_cu = 1;
+    static const void* asked_kern = nullptr;                 // kernels of one signature share this instantiation
+    static size_t asked_smem = ~static_cast<size_t>(0);
+    static int asked_threads = 0, per_cu = 1;
+    if (reinterpret_cast<const void*>(kern) != asked_kern || smem != asked_smem || threads != asked_threads) {
+        int q = 0;
+        per_cu = (hipOccupancyMaxActiveBlocksPerMultiprocessor(&q, kern, threads, smem) == hipSuccess && q >= 1) ? q : 1;
+        asked_kern = reinterpret_cast<const void*>(kern);
+        asked_smem = smem;
+        asked_threads = threads;
+    }
     return per_cu * compute_units();
 }
 
