@@ -10,6 +10,7 @@ parity checks can read the float32 accumulators before the bf16 rounding.
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes
 
 import torch
@@ -36,6 +37,14 @@ def _workspace(nbytes: int, device: torch.device) -> torch.Tensor:
     # scratch for the pre-quantized activations: a fresh tensor from torch's caching allocator, so
     # stream ordering and lifetime follow torch's rules exactly as the reference's temporaries do
     return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)
+
+
+def _on_device(device: torch.device):
+    """Device guard for the launch: torch's context manager only when the tensor's device is not the current one (entering
+    and leaving it costs a few microseconds of host time per call, which shows in eager decode loops)."""
+    if device.index is None or device.index == torch.cuda.current_device():
+        return contextlib.nullcontext()
+    return torch.cuda.device(device)
 
 
 def _stream(device: torch.device) -> int:
@@ -92,7 +101,7 @@ def q8_0_gemm_forward(x: torch.Tensor, blocks: torch.Tensor, row_elems: int, *, 
     if rows == 0 or n == 0:
         return y
     lib = _lib()
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         ws_bytes = lib.pllm_q8_0_gemm_workspace_bytes(rows, row_elems, n, blocks.size(1))
         ws = _workspace(ws_bytes, x.device)
         st = lib.pllm_q8_0_gemm(x.data_ptr(), _DTYPE_CODE[x.dtype], blocks.data_ptr(), y.data_ptr(), _DTYPE_CODE[out_dtype],
@@ -126,7 +135,7 @@ def _dense_gemm(name, x, blocks, row_elems, type_id, signed_grid, out_dtype):
     if rows == 0 or n == 0:
         return y
     lib = _lib()
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         ws_bytes = lib.pllm_gguf_quant_gemm_workspace_bytes(type_id, rows, row_elems, n, blocks.size(1))
         ws = _workspace(ws_bytes, x.device)
         st = lib.pllm_gguf_quant_gemm(x.data_ptr(), _DTYPE_CODE[x.dtype], blocks.data_ptr(), type_id, y.data_ptr(),
@@ -170,7 +179,7 @@ def gguf_quant_gemm_multi_forward(x, blocks_list, row_elems, type_id, signed_gri
     ys = [torch.empty(*x.shape[:-1], b.size(0), dtype=out_dtype, device=x.device) for b in blocks_list]
     lib = _lib()
     bpr = blocks_list[0].size(1)
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         ws_bytes = lib.pllm_activation_image_bytes(rows, bpr)
         ws = _workspace(ws_bytes, x.device)
         st = lib.pllm_gguf_quant_gemm_multi(
@@ -197,7 +206,7 @@ def gguf_quant_gemm_accumulate_forward(x, blocks, row_elems, type_id, signed_gri
     if rows == 0 or n == 0:
         return y
     lib = _lib()
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         ws_bytes = lib.pllm_gguf_quant_gemm_workspace_bytes(type_id, rows, row_elems, n, blocks.size(1))
         ws = _workspace(ws_bytes, x.device)
         st = lib.pllm_gguf_quant_gemm_accumulate(x.data_ptr(), _DTYPE_CODE[x.dtype], blocks.data_ptr(), type_id, y.data_ptr(),
@@ -228,7 +237,7 @@ def fused_rms_norm_forward(x: torch.Tensor, weight: torch.Tensor, eps: float, *,
     y = torch.empty(x.shape, dtype=out_dtype, device=x.device)
     if x.numel() == 0:
         return y
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         st = _lib().pllm_fused_rms_norm(x.data_ptr(), _DTYPE_CODE[x.dtype], weight.data_ptr(), y.data_ptr(), _DTYPE_CODE[out_dtype],
                                         x.size(0), x.size(1), float(eps), _stream(x.device))
     _ffi.check(st, "fused_rms_norm_forward")
@@ -249,7 +258,7 @@ def gguf_quant_gemm_rmsnorm_forward(x, norm_weight, eps, blocks, row_elems, type
     if rows == 0 or n == 0:
         return y
     lib = _lib()
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         ws_bytes = lib.pllm_gguf_quant_gemm_rmsnorm_workspace_bytes(type_id, rows, row_elems, n, blocks.size(1))
         ws = _workspace(ws_bytes, x.device)
         st = lib.pllm_gguf_quant_gemm_rmsnorm(x.data_ptr(), _DTYPE_CODE[x.dtype], norm_weight.data_ptr(), float(eps), int(bool(round_fp16)),
@@ -290,7 +299,7 @@ def gguf_dequantize_rows(blocks: torch.Tensor, type_id: int, row_elems: int, row
     out = torch.empty(*lead, row_elems, dtype=out_dtype, device=blocks.device)
     if count == 0:
         return out
-    with torch.cuda.device(blocks.device):
+    with _on_device(blocks.device):
         st = _lib().pllm_gguf_dequantize_rows(None if row_ids is None else row_ids.data_ptr(), count, blocks.data_ptr(), type_id,
                                               blocks.size(0), row_elems, blocks.size(1), out.data_ptr(), _DTYPE_CODE[out_dtype],
                                               _stream(blocks.device))
@@ -322,7 +331,7 @@ def fp8_block_dequantize(weight: torch.Tensor, scale: torch.Tensor, *, out_dtype
     _check(scale.is_cuda and scale.dtype == torch.float32 and scale.is_contiguous(), "scale must be a contiguous CUDA float32 tensor")
     _check(tuple(scale.shape) == ((n + 127) // 128, (k + 127) // 128), "scale must have shape [ceil(N/128), ceil(K/128)]")
     out = torch.empty(n, k, dtype=out_dtype, device=w8.device)
-    with torch.cuda.device(w8.device):
+    with _on_device(w8.device):
         st = _lib().pllm_fp8_block_dequantize(w8.data_ptr(), scale.data_ptr(), n, k, out.data_ptr(), _DTYPE_CODE[out_dtype], _stream(w8.device))
     _ffi.check(st, "fp8_block_dequantize")
     return out
@@ -348,7 +357,7 @@ def fp8_block_gemm_forward(x: torch.Tensor, weight: torch.Tensor, scale: torch.T
     y = torch.empty(*x.shape[:-1], n, dtype=out_dtype, device=x.device)
     if rows == 0:
         return y
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         ws_bytes = _lib().pllm_fp8_block_gemm_workspace_bytes(rows, k, n)
         ws = _workspace(ws_bytes, x.device) if ws_bytes else None
         st = _lib().pllm_fp8_block_gemm(x.data_ptr(), _DTYPE_CODE[x.dtype], w8.data_ptr(), scale.data_ptr(), y.data_ptr(),
@@ -372,7 +381,7 @@ def fp8_block_gemm_accumulate_forward(x: torch.Tensor, weight: torch.Tensor, sca
     rows = x.numel() // k
     if rows == 0:
         return y
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         st = _lib().pllm_fp8_block_gemm_accumulate(x.data_ptr(), _DTYPE_CODE[x.dtype], w8.data_ptr(), scale.data_ptr(), y.data_ptr(),
                                                    _DTYPE_CODE[y.dtype], rows, k, n, _stream(x.device))
     if st == _ffi.PLLM_ERR_UNSUPPORTED:      # a row count of the tile kernel
@@ -400,7 +409,7 @@ def fp8_gemm_forward(a: torch.Tensor, a_scale: torch.Tensor, weight: torch.Tenso
     y = torch.empty(*a8.shape[:-1], n, dtype=out_dtype, device=a8.device)
     if rows == 0:
         return y
-    with torch.cuda.device(a8.device):
+    with _on_device(a8.device):
         st = _lib().pllm_fp8_gemm(a8.data_ptr(), a_scale.data_ptr(), w8.data_ptr(), scale.data_ptr(), y.data_ptr(), _DTYPE_CODE[out_dtype],
                                   rows, k, n, _stream(a8.device))
     _ffi.check(st, "fp8_gemm_forward")
@@ -417,7 +426,7 @@ def fp8_act_quant_forward(x: torch.Tensor, eps: float = 1e-4, round_scale_pow2: 
     codes = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
     scales = torch.empty(*x.shape[:-1], k // 128, dtype=torch.float32, device=x.device)
     if rows:
-        with torch.cuda.device(x.device):
+        with _on_device(x.device):
             st = _lib().pllm_fp8_act_quant(x.data_ptr(), _DTYPE_CODE[x.dtype], rows, k, codes.data_ptr(), scales.data_ptr(),
                                            float(eps), int(bool(round_scale_pow2)), _stream(x.device))
         _ffi.check(st, "fp8_act_quant_forward")
@@ -463,7 +472,7 @@ def gguf_quant_gemm_pair_forward(x, blocks0, row_elems0, type_id0, blocks1, row_
     if rows == 0 or n == 0:
         return y
     lib = _lib()
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         ws_bytes = lib.pllm_activation_image_bytes(rows, blocks0.size(1))
         ws = _workspace(ws_bytes, x.device)
         st = lib.pllm_gguf_quant_gemm_pair(x.data_ptr(), _DTYPE_CODE[x.dtype], blocks0.data_ptr(), type_id0, blocks1.data_ptr(), type_id1,
@@ -504,7 +513,7 @@ def _moe_call(name, x, tokens, route_tokens, route_experts, seg_starts, route_we
     dim, inter, n_experts, routes = x.size(-1), w1.size(1), w1.size(0), route_weights.numel()
     y = torch.empty(tokens, dim, dtype=torch.float32, device=x.device)
     lib = _lib()
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         ws_bytes = lib.pllm_gguf_moe_workspace_bytes(tokens, routes, dim, inter)
         ws = _workspace(ws_bytes, x.device)
         st = lib.pllm_gguf_moe_forward(
@@ -638,7 +647,7 @@ def moe_group_routes(indices, weights, experts_start_idx, n_local_experts):
     wts = torch.empty(cap, dtype=torch.float32, device=dev)
     exps = torch.empty(cap, dtype=torch.int32, device=dev)
     if t * k:
-        with torch.cuda.device(dev):
+        with _on_device(dev):
             st = _lib().pllm_moe_group_routes(indices.data_ptr(), int(indices.dtype == torch.int64), weights.data_ptr(), t, k,
                                               int(experts_start_idx), n_local, seg.data_ptr(), toks.data_ptr(), wts.data_ptr(),
                                               exps.data_ptr(), _stream(dev))
@@ -669,7 +678,7 @@ def moe_route(x_flat: torch.Tensor, gate_weight: torch.Tensor, gate_bias, top_k:
     if t == 0:
         return indices, weights
     logits = torch.empty(t, e, dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         st = _lib().pllm_moe_route(x_flat.data_ptr(), _DTYPE_CODE[x_flat.dtype], t, x_flat.size(1), gate_weight.data_ptr(),
                                    gate_bias.data_ptr() if gate_bias is not None else None, e, k, int(bool(softmax)),
                                    logits.data_ptr(), indices.data_ptr(), weights.data_ptr(), _stream(dev))
@@ -718,7 +727,7 @@ def quantize_activations(x: torch.Tensor, blocks_per_row: int) -> torch.Tensor:
     lib = _lib()
     nbytes = lib.pllm_activation_image_bytes(rows, bpr)
     image = torch.empty(rows, nbytes // max(rows, 1), dtype=torch.uint8, device=x.device)
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         st = lib.pllm_quantize_activations(x.data_ptr(), _DTYPE_CODE[x.dtype], rows, k, bpr, image.data_ptr(), nbytes, _stream(x.device))
     _ffi.check(st, "quantize_activations")
     return image
@@ -741,7 +750,7 @@ def swiglu_quantize_activations(gate: torch.Tensor, up: torch.Tensor, blocks_per
     lib = _lib()
     nbytes = lib.pllm_activation_image_bytes(rows, bpr)
     image = torch.empty(rows, nbytes // rows, dtype=torch.uint8, device=gate.device)
-    with torch.cuda.device(gate.device):
+    with _on_device(gate.device):
         st = lib.pllm_swiglu_quantize_activations(gate.data_ptr(), up.data_ptr(), _DTYPE_CODE[gate.dtype], rows, k, bpr, float(swiglu_limit),
                                                   _DTYPE_CODE[round_dtype], image.data_ptr(), nbytes, _stream(gate.device))
     _ffi.check(st, "swiglu_quantize_activations")
@@ -769,7 +778,7 @@ def gguf_quant_gemm_prequantized(image: torch.Tensor, blocks: torch.Tensor, type
     else:
         y = torch.empty(rows, n, dtype=out_dtype, device=image.device)
         fn = lib.pllm_gguf_quant_gemm_prequantized
-    with torch.cuda.device(image.device):
+    with _on_device(image.device):
         st = fn(image.data_ptr(), blocks.data_ptr(), type_id, y.data_ptr(), _DTYPE_CODE[y.dtype], rows, n, blocks.size(1), _stream(image.device))
     _ffi.check(st, "gguf_quant_gemm_prequantized")
     return y
