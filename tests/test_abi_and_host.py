@@ -151,3 +151,12 @@ def test_random_iq_blocks_have_finite_scales():
         blocks = gen(rng, 3, 2)
         vals = O.dequant_rows(blocks, name)
         assert np.isfinite(vals).all() and vals.std() > 0
+
+
+def test_product_never_touches_the_oracle():
+    """The oracle is test infrastructure: nothing under the package imports, reads or links it."""
+    import pathlib
+    root = pathlib.Path(__file__).resolve().parents[1] / "pocketllm_amd"
+    for path in list(root.glob("*.py")) + list((root / "csrc").glob("*")):
+        if path.is_file() and path.suffix in (".py", ".hip", ".h", ".inc"):
+            assert "oracle" not in path.read_text(errors="replace"), path.name
