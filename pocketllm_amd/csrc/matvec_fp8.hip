@@ -56,6 +56,32 @@ __device__ __forceinline__ void stage_row_f32(float* xs, const void* __restrict_
     }
 }
 
+// The first batch of stage_row_f32 in two halves, so that the row's loads can be issued ahead of the weight loads (loads return
+// in order: a row requested after the weights would arrive after all of them) and stored once the weights are on their way.
+constexpr int kStageBatch = 6;
+__device__ __forceinline__ void stage_row_request(float (&v)[kStageBatch][4], const void* __restrict__ x, int x_dtype, size_t xoff, int k) {
+    const bool vec = x_dtype == PLLM_F32 ? ((reinterpret_cast<uintptr_t>(x) + 4 * xoff) & 15u) == 0
+                                         : ((reinterpret_cast<uintptr_t>(x) + 2 * xoff) & 7u) == 0;
+    const int base = static_cast<int>(threadIdx.x) * 4;
+#pragma unroll
+    for (int j = 0; j < kStageBatch; ++j)
+        if (base + j * kThreads * 4 < k) load_row4(v[j], x, x_dtype, xoff, base + j * kThreads * 4, k, vec);
+}
+__device__ __forceinline__ void stage_row_finish(float* xs, const float (&v)[kStageBatch][4], const void* __restrict__ x, int x_dtype, size_t xoff, int k) {
+    const int base = static_cast<int>(threadIdx.x) * 4;
+#pragma unroll
+    for (int j = 0; j < kStageBatch; ++j)
+        if (base + j * kThreads * 4 < k) *reinterpret_cast<float4*>(xs + base + j * kThreads * 4) = make_float4(v[j][0], v[j][1], v[j][2], v[j][3]);
+    // rows longer than one batch: the rest the ordinary way
+    const bool vec = x_dtype == PLLM_F32 ? ((reinterpret_cast<uintptr_t>(x) + 4 * xoff) & 15u) == 0
+                                         : ((reinterpret_cast<uintptr_t>(x) + 2 * xoff) & 7u) == 0;
+    for (int e0 = base + kStageBatch * kThreads * 4; e0 < k; e0 += kThreads * 4) {
+        float t[4];
+        load_row4(t, x, x_dtype, xoff, e0, k, vec);
+        *reinterpret_cast<float4*>(xs + e0) = make_float4(t[0], t[1], t[2], t[3]);
+    }
+}
+
 // Two register slots per wave: two consecutive rows of one matrix, or (SWIGLU) the same row of the
 // gate and of the up matrix.
 template <bool SWIGLU>
@@ -196,10 +222,18 @@ __global__ __launch_bounds__(kThreads) void fp8_persistent_matvec_kernel(
         for (int r = 0; r < R; ++r) acc[q][r] = 0.0f;
     int g = blockIdx.x, p = 0;               // the pass being multiplied
     int gn = g, pn = 0;                      // the pass being fetched
-    fp8_fetch_pass<ITERS, SWIGLU>(a, ma, mb, g * rows_per_group + wave_row, n, chunks, 0, lane);
+    if constexpr (R == 1) {                  // the activation row is requested first and stored once the weights are on their way
+        float head[kStageBatch][4];
+        const size_t xoff = static_cast<size_t>(arow0) * x_stride;
+        stage_row_request(head, x, x_dtype, xoff, k);
+        fp8_fetch_pass<ITERS, SWIGLU>(a, ma, mb, g * rows_per_group + wave_row, n, chunks, 0, lane);
+        stage_row_finish(xs, head, x, x_dtype, xoff, k);
+    } else {
+        fp8_fetch_pass<ITERS, SWIGLU>(a, ma, mb, g * rows_per_group + wave_row, n, chunks, 0, lane);
 #pragma unroll 1
-    for (int r = 0; r < R; ++r)              // rows past the end: the last row again, result dropped
-        stage_row_f32(xs + static_cast<size_t>(r) * k, x, x_dtype, static_cast<size_t>(min(arow0 + r, total_rows - 1)) * x_stride, k);
+        for (int r = 0; r < R; ++r)          // rows past the end: the last row again, result dropped
+            stage_row_f32(xs + static_cast<size_t>(r) * k, x, x_dtype, static_cast<size_t>(min(arow0 + r, total_rows - 1)) * x_stride, k);
+    }
     __syncthreads();
     while (g < groups) {
         if (++pn == passes) { pn = 0; gn += step; }
