@@ -54,19 +54,31 @@ def ring_of(blocks: np.ndarray, device, copies: int = RING):
     return [first] + [first.clone() for _ in range(copies - 1)]
 
 
+MIN_TIMED_LAUNCHES = 200      # per repeat
+REPEATS = 5                   # the median of this many repeats is reported
+RING_BYTES = 512 << 20        # a case's weight copies in rotation: twice the 256 MB last-level cache
+
+
+def ring_copies(nbytes: int, least: int = 2) -> int:
+    return max(least, -(-RING_BYTES // max(1, nbytes)))
+
+
 def event_time_us(fn, slots, iters, warm=5):
-    """Average duration of fn(slot) over `iters` back-to-back calls, HIP events on the current stream."""
+    """Median over REPEATS of the average duration of fn(slot) over `iters` back-to-back calls, HIP events on the current stream."""
     for i in range(warm):
         fn(i % slots)
     torch.cuda.synchronize()
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for i in range(iters):
-        fn(i % slots)
-    e1.record()
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) * 1e3 / iters
+    samples = []
+    for _ in range(REPEATS):
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(iters):
+            fn(i % slots)
+        e1.record()
+        torch.cuda.synchronize()
+        samples.append(e0.elapsed_time(e1) * 1e3 / iters)
+    return float(np.median(samples))
 
 
 def capture(fn, slots):
@@ -91,45 +103,103 @@ def capture(fn, slots):
         return None, False
 
 
-def time_calls_us(fn, slots, iters, eager=False):
-    """Average duration of one fn(slot) call: a graph of `slots` calls replayed, or eager calls."""
+def time_calls_us(fn, slots, iters=MIN_TIMED_LAUNCHES, eager=False):
+    """Duration of one fn(slot) call: a graph of `slots` calls replayed until at least `iters` calls have run, or eager calls;
+    the median of REPEATS such measurements."""
     replay, graphed = (None, False) if eager else capture(fn, slots)
     if graphed:
-        reps = max(1, iters // slots)
+        reps = max(1, -(-iters // slots))
         return event_time_us(lambda _s: replay(), 1, reps, warm=2) / slots, True
-    return event_time_us(fn, slots, iters), False
+    return event_time_us(fn, slots, max(iters, slots)), False
 
 
-def cpu_baseline(blocks: np.ndarray, type_name: str, k: int, x: np.ndarray, budget_s: float = 15.0):
+def _median_time(fn, budget_s: float, most: int = 10):
+    """Median wall time of fn() over up to `most` calls within the budget (at least two; the first call only warms up)."""
+    times = []
+    t_begin = time.perf_counter()
+    while len(times) < most + 1 and (time.perf_counter() - t_begin < budget_s or len(times) < 2):
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    times = times[1:]
+    return float(np.median(times)), len(times)
+
+
+def cpu_baseline(blocks: np.ndarray, type_name: str, k: int, x: np.ndarray, budget_s: float = 8.0):
     """The reference's CPU path restated: numpy block decode to float32, then torch matmul."""
     from oracle import gguf_oracle as O
     threads = os.cpu_count() or 1
     torch.set_num_threads(threads)
     xt = torch.from_numpy(x.astype(np.float32))
-    times = []
-    t_begin = time.perf_counter()
-    while len(times) < 5 and (time.perf_counter() - t_begin < budget_s or len(times) < 2):
+    parts = []
+
+    def call():
         t0 = time.perf_counter()
         w = O.dequant_rows(blocks, type_name, k)
         t1 = time.perf_counter()
         torch.nn.functional.linear(xt, torch.from_numpy(w))
-        t2 = time.perf_counter()
-        times.append((t2 - t0, t1 - t0, t2 - t1))
-    times = times[1:] if len(times) > 1 else times          # first call warms the page cache
-    total = float(np.median([t[0] for t in times]))
+        parts.append((t1 - t0, time.perf_counter() - t1))
+
+    total, calls = _median_time(call, budget_s, most=5)
+    parts = parts[1:]
     return {
         "value": round(blocks.size / total / 1e9, 4),
         "unit": "GB/s",
         "cores": int(torch.get_num_threads()),
         "kind": "port",
-        "sample": (f"{type_name} {blocks.shape[0]}x{k} matvec, numpy block decode ({np.median([t[1] for t in times]) * 1e3:.0f} ms, "
-                   f"one thread) + torch F.linear fp32 ({np.median([t[2] for t in times]) * 1e3:.1f} ms, {torch.get_num_threads()} threads), "
-                   f"median of {len(times)} calls"),
+        "sample": (f"{type_name} {blocks.shape[0]}x{k} matvec, numpy block decode ({np.median([t[0] for t in parts]) * 1e3:.0f} ms, "
+                   f"one thread) + torch F.linear fp32 ({np.median([t[1] for t in parts]) * 1e3:.1f} ms, {torch.get_num_threads()} threads), "
+                   f"median of {calls} calls"),
         "ms_per_call": round(total * 1e3, 3),
     }
 
 
-def extra_cases(mod, dev, iters):
+def cpu_baselines_more(q4k_blocks: np.ndarray, x5120: np.ndarray):
+    """Further CPU lines, each a few seconds of host work:
+      * BASELINE config 1 as the reference runs it on the CPU (src/kernels/ops.py:766-792): Q8_0 4096x4096 dequantized to a
+        float32 matrix, then F.linear, restated with the oracle's decoder;
+      * this repository's plain-C raw-block matvec (oracle/rawblock_cpu.c, OpenMP over rows, no float copy of the matrix) on
+        the same Q8_0 matrix and on Q4_K 5120x5120;
+      * the reference's own compiled CPU kernel gguf_quantized_matmul (src/csrc/deepseek_cpu_moe_ext.cpp:2759-2803, AVX2 +
+        OpenMP; it serves IQ2_XXS and Q2_K) where oracle/_ref holds it: Q2_K 5120x5120, kind "reference"."""
+    from oracle import gguf_oracle as O
+    from pocketllm_amd import block_codec as C
+    threads = os.cpu_count() or 1
+    torch.set_num_threads(threads)
+    rng = np.random.default_rng(1001)
+    out = []
+    w = rng.standard_normal((4096, 4096), dtype=np.float32) * np.float32(0.02)
+    q8 = C.pack_q8_0(w)
+    x1 = rng.standard_normal((1, 4096), dtype=np.float32)
+    xt = torch.from_numpy(x1)
+    total, calls = _median_time(lambda: torch.nn.functional.linear(xt, torch.from_numpy(O.dequant_rows(q8, "q8_0", 4096))), 4.0, most=8)
+    out.append({"case": "q8_0 4096x4096 T=1 (BASELINE config 1): dequantize to float32 + F.linear", "kind": "port", "cores": threads,
+                "ms_per_call": round(total * 1e3, 3), "value": round(q8.size / total / 1e9, 4), "unit": "GB/s", "calls": calls})
+    try:
+        from oracle import rawblock_cpu as R
+        if R.available():
+            for label, blocks, name, xx in (("q8_0 4096x4096 T=1", q8, "q8_0", x1), ("q4_k 5120x5120 T=1", q4k_blocks, "q4_k", x5120)):
+                total, calls = _median_time(lambda: R.matvec(blocks, name, xx), 2.0, most=20)
+                out.append({"case": f"{label}: raw-block matvec in plain C, OpenMP over rows (oracle/rawblock_cpu.c)", "kind": "port",
+                            "cores": threads, "ms_per_call": round(total * 1e3, 3), "value": round(blocks.size / total / 1e9, 4),
+                            "unit": "GB/s", "calls": calls})
+    except OSError as exc:                                # pragma: no cover - a library built for another host
+        print(f"bench.py: oracle/_build not usable here ({exc})", file=sys.stderr)
+    try:
+        from oracle import ref_ext
+        if ref_ext.available():
+            q2 = C.quantize_q2_k(rng.standard_normal((5120, 5120), dtype=np.float32) * np.float32(0.02))
+            grid = O.iq2xxs_signed_grid()
+            total, calls = _median_time(lambda: ref_ext.quantized_matmul(x5120, q2, 1, grid), 2.0, most=20)
+            out.append({"case": "q2_k 5120x5120 T=1: the reference's compiled CPU kernel gguf_quantized_matmul (oracle/_ref)", "kind": "reference",
+                        "cores": threads, "ms_per_call": round(total * 1e3, 3), "value": round(q2.size / total / 1e9, 4), "unit": "GB/s",
+                        "calls": calls})
+    except (OSError, ImportError) as exc:                 # pragma: no cover
+        print(f"bench.py: oracle/_ref not usable here ({exc})", file=sys.stderr)
+    return out
+
+
+def extra_cases(mod, dev):
     """Other formats of the path, one line each (event-timed eager launches are launch-bound for the
     small ones, so these replay graphs as well)."""
     from pocketllm_amd import block_codec as C, codebooks
@@ -138,7 +208,7 @@ def extra_cases(mod, dev, iters):
     empty = torch.empty(0, dtype=torch.int8, device=dev)
 
     def run(label, nbytes, fn, slots, extra=None):
-        us, graphed = time_calls_us(fn, slots, iters)
+        us, graphed = time_calls_us(fn, slots)
         rec = {"case": label, "weight_bytes": int(nbytes), "us_per_call": round(us, 3), "gbs": round(nbytes / us / 1e3, 1),
                "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4), "graph": graphed}
         if extra:
@@ -148,7 +218,7 @@ def extra_cases(mod, dev, iters):
     # Q8_0, BASELINE config 1 and the large shape
     for n, k in ((4096, 4096), (17408, 5120)):
         blocks = C.pack_q8_0((rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02)))
-        ring = ring_of(blocks, dev, max(2, min(RING, (1 << 30) // blocks.size)))
+        ring = ring_of(blocks, dev, ring_copies(blocks.size))
         x = torch.randn(1, k, device=dev)
         run(f"q8_0 matvec {n}x{k} T=1", blocks.size, lambda s, ring=ring, x=x, k=k: mod.q8_0_gemm_forward(x, ring[s], k), len(ring))
         del ring
@@ -157,7 +227,7 @@ def extra_cases(mod, dev, iters):
     for name, tid, blocks in (("q2_k", 1, C.quantize_q2_k((rng.standard_normal((17408, 5120), dtype=np.float32) * np.float32(0.02)))),
                               ("q6_k", 8, C.random_blocks(rng, "q6_k", 17408, 20)), ("iq4_xs", 7, C.random_blocks(rng, "iq4_xs", 17408, 20)),
                               ("iq3_xxs", 6, C.random_blocks(rng, "iq3_xxs", 17408, 20)), ("iq2_xs", 5, C.random_blocks(rng, "iq2_xs", 17408, 20))):
-        ring = ring_of(blocks, dev, max(2, min(RING, (1 << 30) // blocks.size)))
+        ring = ring_of(blocks, dev, ring_copies(blocks.size))
         grid = codebooks.grid_tensor_for_type(tid).to(dev)
         run(f"{name} matvec 17408x5120 T=1", blocks.size,
             lambda s, ring=ring, x=x, tid=tid, grid=grid: mod.gguf_quant_gemm_forward(x, ring[s], 5120, tid, grid), len(ring))
@@ -174,7 +244,7 @@ def extra_cases(mod, dev, iters):
     del ring
     # normalisation + projection as one decode operator against the two operators one after the other (Q4_K 5120x5120)
     blocks = C.quantize_q4_k((rng.standard_normal((5120, 5120), dtype=np.float32) * np.float32(0.02)))
-    ring = ring_of(blocks, dev, max(2, min(RING, (1 << 30) // blocks.size)))
+    ring = ring_of(blocks, dev, ring_copies(blocks.size))
     gamma = torch.ones(5120, device=dev)
     run("rmsnorm + q4_k matvec 5120x5120 T=1, one operator", blocks.size,
         lambda s, ring=ring: mod.gguf_quant_gemm_rmsnorm_forward(x, gamma, 1e-6, ring[s], 5120, 3, empty), len(ring))
@@ -206,7 +276,7 @@ def extra_cases(mod, dev, iters):
     for name, tid, n, k, gen, grid in (("iq2_xxs", 0, 64 * 1536, 3072, C.random_iq2_xxs, codebooks.get_iq2xxs_signed_grid_tensor().to(dev)),
                                        ("iq1_m", 2, 64 * 3072, 1536, C.random_iq1_m, codebooks.get_iq1_grid_tensor().to(dev))):
         blocks = gen(rng, n, k // 256)
-        ring = ring_of(blocks, dev)
+        ring = ring_of(blocks, dev, ring_copies(blocks.size))
         xx = torch.randn(1, k, device=dev, dtype=torch.bfloat16)
         run(f"{name} matvec {n}x{k} T=1", blocks.size,
             lambda s, ring=ring, xx=xx, k=k, tid=tid, grid=grid: mod.gguf_quant_gemm_forward(xx, ring[s], k, tid, grid), len(ring))
@@ -231,7 +301,7 @@ def extra_cases(mod, dev, iters):
     gbias = torch.zeros(e, device=dev)
     for tt in (1, 256):
         xr = torch.randn(tt, d, device=dev, dtype=torch.bfloat16)
-        us, graphed = time_calls_us(lambda s, xr=xr: mod.moe_route(xr, gate, gbias, 8), 4, max(8, iters // 4))
+        us, graphed = time_calls_us(lambda s, xr=xr: mod.moe_route(xr, gate, gbias, 8), 4)
         out.append({"case": f"expert routing (gate 256x3072 f32, sigmoid + bias, top-8) T={tt}", "us_per_call": round(us, 3), "graph": graphed,
                     "weight_bytes": e * d * 4, "gbs": round(e * d * 4 / us / 1e3, 1)})
     # the same experts at T=256 (BASELINE config 5): 2048 routes grouped by expert
@@ -245,7 +315,7 @@ def extra_cases(mod, dev, iters):
     touched = int((seg[1:] > seg[:-1]).sum().item())
     flops = 2.0 * t * 8 * 3 * inter * d
     us, graphed = time_calls_us(lambda s: mod.gguf_moe_prefill_grouped_forward(xt, toks, rws, seg, w1, w3, w2, d, 0, d, 0, inter, 2, grids, 0.0),
-                                4, max(8, iters // 8))
+                                4)
     nbytes = touched * (2 * inter * (d // 256) * 66 + d * (inter // 256) * 56)
     out.append({"case": "fused experts iq2_xxs gate/up + iq1_m down, 256 experts top-8, T=256", "weight_bytes": nbytes,
                 "us_per_call": round(us, 3), "gbs": round(nbytes / us / 1e3, 1), "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
@@ -268,7 +338,7 @@ def extra_cases(mod, dev, iters):
         return mod.gguf_moe_single_token_forward(h2, ridx[0], rw[0], w1, w3, w2, 0.0)
 
     layer_bytes = (wq.numel() + wk.numel() + wv.numel() + wo.numel()) + per_call + e * d * 4
-    us, graphed = time_calls_us(layer, 4, max(8, iters // 4))
+    us, graphed = time_calls_us(layer, 4)
     out.append({"case": "decoder layer matmul path, MiniMax-M2 shapes, T=1 (norm + q/k/v projections in one launch, output projection + residual, norm, routing, experts)",
                 "weight_bytes": int(layer_bytes), "us_per_call": round(us, 3), "gbs": round(layer_bytes / us / 1e3, 1),
                 "frac_hbm_peak": round(layer_bytes / us / 1e3 / HBM_PEAK_GBS, 4), "graph": graphed,
@@ -302,18 +372,18 @@ def extra_cases(mod, dev, iters):
 
     ffn_bytes = sum(t.numel() for t in rings[0])
     for label, fn in (("three launches (norm + gate/up, SiLU * up image, down + residual)", ffn_fused), ("separate operators", ffn_chain)):
-        us, graphed = time_calls_us(fn, 3, max(6, iters // 4))
+        us, graphed = time_calls_us(fn, 3)
         out.append({"case": f"dense feed-forward block q4_k 5120 -> 17408 -> 5120, T=1, {label}", "weight_bytes": int(ffn_bytes),
                     "us_per_call": round(us, 3), "gbs": round(ffn_bytes / us / 1e3, 1),
                     "frac_hbm_peak": round(ffn_bytes / us / 1e3 / HBM_PEAK_GBS, 4), "graph": graphed})
     del rings, base
-    return out + prefill_cases(mod, dev, iters)
+    return out + prefill_cases(mod, dev)
 
 
 F16_MFMA_PEAK_TFLOPS = 2500.0
 
 
-def prefill_cases(mod, dev, iters):
+def prefill_cases(mod, dev):
     """BASELINE configs 3 and 4 at T > 1: the MFMA tile kernel, TFLOPS = 2 T K N / t against the dense fp16 peak
     (the tiles are decoded to fp16, see the kernel's header for why)."""
     from pocketllm_amd import block_codec as C, codebooks
@@ -323,7 +393,7 @@ def prefill_cases(mod, dev, iters):
     k = 5120
 
     def run(label, t, n, fn):
-        us, graphed = time_calls_us(fn, 4, max(8, iters // 8))
+        us, graphed = time_calls_us(fn, 4)
         tf = 2.0 * t * k * n / us / 1e6
         out.append({"case": label, "us_per_call": round(us, 3), "tflops": round(tf, 1), "frac_mfma_peak": round(tf / F16_MFMA_PEAK_TFLOPS, 4),
                     "peak": "fp16 dense 2.5 PFLOP/s", "graph": graphed})
@@ -352,8 +422,8 @@ def prefill_cases(mod, dev, iters):
     run(f"fp8_e4m3 prefill {n}x{k} T=512", 512, n, lambda s: mod.fp8_block_gemm_forward(x, codes, scale))
     # the reference's FP8 linear: act_quant (E4M3 activations, 128-wide scales) + fp8_gemm on the native FP8 matrix path
     a, a_s = mod.fp8_act_quant_forward(x)
-    us, graphed = time_calls_us(lambda s: mod.fp8_gemm_forward(a, a_s, codes, scale), 4, max(8, iters // 8))
-    usq, _ = time_calls_us(lambda s: mod.fp8_act_quant_forward(x), 4, max(8, iters // 8))
+    us, graphed = time_calls_us(lambda s: mod.fp8_gemm_forward(a, a_s, codes, scale), 4)
+    usq, _ = time_calls_us(lambda s: mod.fp8_act_quant_forward(x), 4)
     tf = 2.0 * 512 * k * n / us / 1e6
     out.append({"case": f"fp8_e4m3 x fp8_e4m3 native MFMA prefill {n}x{k} T=512", "us_per_call": round(us, 3), "tflops": round(tf, 1),
                 "frac_mfma_peak": round(tf / 5000.0, 4), "peak": "fp8 dense 5.0 PFLOP/s", "act_quant_us": round(usq, 3), "graph": graphed})
@@ -361,7 +431,7 @@ def prefill_cases(mod, dev, iters):
 
 
 def pmc_pass(mod, dev) -> None:
-    from pocketllm_amd import _ffi
+    import ctypes
     name, tid, n, k = CASES[DOMINANT]
     rng = np.random.default_rng(1002 + DOMINANT)
     blocks = _encoders()[name]((rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02)))
@@ -370,12 +440,13 @@ def pmc_pass(mod, dev) -> None:
     grid = torch.empty(0, dtype=torch.int8, device=dev)
     nbytes = blocks.size & ~15
     dst = torch.empty(nbytes, dtype=torch.uint8, device=dev)
-    lib = _ffi.load_library()
+    probe = ctypes.CDLL(os.path.join(os.path.dirname(os.path.abspath(__file__)), "pocketllm_amd", "libpllm_probe.so"))
+    probe.pllm_probe_stream_copy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p]
     stream = torch.cuda.current_stream().cuda_stream
     for i in range(6):
         mod.gguf_quant_gemm_forward(x, ring[i], k, tid, grid)
     for i in range(6):
-        lib.pllm_diag_stream_copy(ring[i].data_ptr(), dst.data_ptr(), nbytes, 2048, stream)
+        probe.pllm_probe_stream_copy(ring[i].data_ptr(), dst.data_ptr(), nbytes, 2048, stream)
     torch.cuda.synchronize()
     print(json.dumps({"pmc_pass": f"{name} matvec {n}x{k}", "weight_bytes": int(blocks.size), "copy_bytes": int(nbytes)}))
 
@@ -426,7 +497,7 @@ def prefill_pass(mod, dev) -> None:
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=240)
+    ap.add_argument("--steps", type=int, default=240, help="timed steps (run exactly, five times over; the median is reported)")
     ap.add_argument("--warmup", type=int, default=24)
     ap.add_argument("--eager", action="store_true", help="time plain operator calls instead of graph replays")
     ap.add_argument("--no-extra", action="store_true", help="skip the table of other formats")
@@ -465,54 +536,61 @@ def main() -> None:
         rng = np.random.default_rng(1002 + idx)
         blocks = _encoders()[name]((rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02)))
         host_blocks.append(blocks)
-        rings.append(ring_of(blocks, dev))
-        fns.append(lambda s, ring=rings[-1], tid=tid, k=k: mod.gguf_quant_gemm_forward(x, ring[s], k, tid, grid))
+        rings.append(ring_of(blocks, dev, ring_copies(blocks.size, RING)))
+        fns.append(lambda s, ring=rings[-1], tid=tid, k=k: mod.gguf_quant_gemm_forward(x, ring[s % len(ring)], k, tid, grid))
     step_bytes = sum(b.size for b in host_blocks)
 
     def step_eager(s):
         for fn in fns:
             fn(s)
 
-    replay, graphed = (None, False) if args.eager else capture(step_eager, RING)
-    if graphed:
-        # one replay = RING steps (every ring slot once); steps and warmup are rounded up to whole replays
-        args.warmup = -(-args.warmup // RING) * RING
-        args.steps = max(RING, -(-args.steps // RING) * RING)
-        for _ in range(args.warmup // RING):
-            replay()
+    # Exactly --warmup untimed steps, then exactly --steps timed steps, REPEATS times over; the median repeat is reported.
+    # Graph mode: one graph holds a chunk of consecutive steps (every step on the next ring slot); whole chunks are replayed
+    # and a second graph holds the remainder, so that the number of steps run is the number asked for.
+    chunk = min(args.steps, 4 * RING)
+    replay, graphed = (None, False) if args.eager else capture(step_eager, chunk)
+    rest = args.steps % chunk
+    replay_rest = None
+    if graphed and rest:
+        replay_rest, ok = capture(step_eager, rest)
+        graphed = graphed and ok
+    for i in range(args.warmup):
+        step_eager(i)
+    torch.cuda.synchronize()
+    repeats = []
+    for _ in range(REPEATS):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(args.steps // RING):
-            replay()
+        if graphed:
+            for _c in range(args.steps // chunk):
+                replay()
+            if replay_rest:
+                replay_rest()
+        else:
+            for i in range(args.steps):
+                step_eager(args.warmup + i)
         torch.cuda.synchronize()
-        elapsed = time.perf_counter() - t0
-    else:
-        for i in range(args.warmup):
-            step_eager(i % RING)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for i in range(args.steps):
-            step_eager((args.warmup + i) % RING)
-        torch.cuda.synchronize()
-        elapsed = time.perf_counter() - t0
+        repeats.append(time.perf_counter() - t0)
+    elapsed = float(np.median(repeats))
     ms_per_step = elapsed * 1e3 / args.steps
     value = step_bytes / (elapsed / args.steps) / 1e9
 
-    # per-case launch durations with HIP events on the launch stream (torch's current stream)
+    # per-case launch durations with HIP events on the launch stream (torch's current stream): every case on its own ring of
+    # at least 512 MB of weight copies, at least 200 launches per repeat, median of 5 repeats
     cases = []
-    iters = max(60, args.steps)
-    for (name, tid, n, k), fn, blocks in zip(CASES, fns, host_blocks):
-        us, g = time_calls_us(fn, RING, iters, eager=args.eager)
-        hot, _ = time_calls_us(lambda _s, fn=fn: fn(0), RING, iters, eager=args.eager)
+    for (name, tid, n, k), fn, blocks, ring in zip(CASES, fns, host_blocks, rings):
+        us, g = time_calls_us(fn, len(ring), eager=args.eager)
+        hot, _ = time_calls_us(lambda _s, fn=fn: fn(0), RING, eager=args.eager)
         cases.append({"case": f"{name} matvec {n}x{k} T=1", "weight_bytes": int(blocks.size), "us_per_call": round(us, 3),
                       "gbs": round(blocks.size / us / 1e3, 1), "frac_hbm_peak": round(blocks.size / us / 1e3 / HBM_PEAK_GBS, 4),
-                      "us_per_call_cache_hot": round(hot, 3), "graph": g})
+                      "us_per_call_cache_hot": round(hot, 3), "ring_copies": len(ring), "graph": g})
     dom = cases[DOMINANT]
-    # the dominant kernel alone, for the roofline object: at this size the operator call is the activation pre-pass plus
-    # this kernel (smaller matrices quantize inside the matvec kernel instead), so it is timed on a prepared image
+    # the dominant kernel alone, for the roofline object: timed on a prepared activation image, so that the figure is the
+    # matvec kernel's own launch duration whether or not the operator call quantizes its activation row in the same launch
     d_name, d_tid, d_n, d_k = CASES[DOMINANT]
     image = mod.quantize_activations(x, d_k // 256)
-    kernel_us, _ = time_calls_us(lambda s: mod.gguf_quant_gemm_prequantized(image, rings[DOMINANT][s], d_tid), RING, iters, eager=args.eager)
+    d_ring = rings[DOMINANT]
+    kernel_us, _ = time_calls_us(lambda s: mod.gguf_quant_gemm_prequantized(image, d_ring[s], d_tid), len(d_ring), eager=args.eager)
     kernel_gbs = host_blocks[DOMINANT].size / kernel_us / 1e3
     traffic = None
     if os.path.exists(TRAFFIC_FILE):
@@ -520,9 +598,11 @@ def main() -> None:
             traffic = json.load(f).get("q5_k matvec 17408x5120 T=1")
     roofline = {"bound": "hbm", "achieved": round(kernel_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(kernel_gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
-                "kernel": "k45_mfma_matvec_kernel<Q5K, 5, false, 1> (q5_k matvec 17408x5120, activation image prepared by act_image_256_kernel)",
+                "traffic_source": "profiles/traffic.json: rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE of an earlier run, not measured in this run",
+                "kernel": "q5_k matvec 17408x5120 on a prepared activation image (pllm_gguf_quant_gemm_prequantized)",
                 "bytes_per_launch": dom["weight_bytes"], "us_per_launch": round(kernel_us, 3),
-                "us_per_operator_call": dom["us_per_call"]}
+                "us_per_operator_call": dom["us_per_call"], "frac_per_operator_call": dom["frac_hbm_peak"],
+                "timed_launches_per_repeat": max(MIN_TIMED_LAUNCHES, len(d_ring)), "repeats": REPEATS}
 
     # parity of what was just timed, against the float-activation oracle (small case only: seconds)
     from oracle import gguf_oracle as O
@@ -530,11 +610,21 @@ def main() -> None:
     want = O.matmul_f(x.float().cpu().numpy(), O.dequant_rows(host_blocks[0], "q4_k", 5120))
     parity = O.rel_l2(y_gpu, want)
 
-    cpu = None if args.no_cpu_baseline else cpu_baseline(host_blocks[0], "q4_k", 5120, x.float().cpu().numpy())
-    del rings
+    cpu, cpu_more = None, []
+    if not args.no_cpu_baseline:
+        cpu = cpu_baseline(host_blocks[0], "q4_k", 5120, x.float().cpu().numpy())
+        cpu_more = cpu_baselines_more(host_blocks[0], x.float().cpu().numpy())
+    del rings, d_ring
     torch.cuda.empty_cache()
+    headline = {c["case"]: {"us": c["us_per_call"], "frac": c["frac_hbm_peak"]} for c in cases}
     if not args.no_extra:
-        cases += extra_cases(mod, dev, iters)
+        cases += extra_cases(mod, dev)
+    # the full table goes to stderr; the one line on stdout keeps the records of the BASELINE configurations
+    print("bench.py all cases: " + json.dumps(cases), file=sys.stderr)
+    keep = ("q4_k matvec", "q5_k matvec", "q8_0 matvec", "fp8_e4m3 matvec 17408x5120 T=1", "fused experts", "q4_k prefill", "q5_k prefill",
+            "fp8_e4m3 prefill", "fp8_e4m3 x fp8_e4m3", "iq2_xxs matvec", "iq1_m matvec", "q2_k matvec")
+    short = [{k2: v for k2, v in c.items() if k2 in ("case", "us_per_call", "gbs", "frac_hbm_peak", "tflops", "frac_mfma_peak", "peak")}
+             for c in cases if c["case"].startswith(keep)]
 
     out = {
         "metric": "decode matvec effective HBM GB/s (% of peak) + prefill TFLOPS, per quant type",
@@ -549,13 +639,15 @@ def main() -> None:
         "vs_baseline": None,
         "dtype": "int8 dot (two int8 activation terms), f32 accumulate",
         "data": "synthetic (seeded N(0,0.02) weights quantized to Q4_K/Q5_K blocks, N(0,1) bf16 activations)",
-        "config": {"workload": "Q4_K + Q5_K decode matvec, N x K = 5120x5120 and 17408x5120, T=1, weights rotated through a ring of "
-                               f"{RING} copies per case ({RING * step_bytes >> 20} MiB in all)",
-                   "bytes_per_step": int(step_bytes), "calls_per_step": len(CASES), "hip_graph_replay": graphed},
+        "config": {"workload": "BASELINE config 2: Q4_K + Q5_K decode matvec, 5120x5120 and 17408x5120, T=1, each case on a ring of >= 512 MB of weight copies",
+                   "bytes_per_step": int(step_bytes), "calls_per_step": len(CASES), "hip_graph_replay": graphed,
+                   "repeats": REPEATS, "ms_per_step_repeats": [round(r * 1e3 / args.steps, 5) for r in repeats],
+                   "headline_cases": headline},
         "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "roofline": roofline,
         "cpu_baseline": cpu,
-        "cases": cases,
+        "cpu_baselines_more": cpu_more,
+        "cases": short,
         "parity_rel_l2_vs_float_oracle": parity,
     }
     print(json.dumps(out))

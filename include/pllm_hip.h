@@ -320,14 +320,6 @@ int pllm_moe_route(const void* x, int x_dtype, int64_t tokens, int64_t dim, cons
 int pllm_fp8_act_quant(const void* x, int x_dtype, int64_t rows, int64_t k, uint8_t* codes, float* scales,
                        float eps, int round_scale_pow2, void* stream);
 
-/*
- * Measurement aids with no counterpart in the reference: a streaming copy and a streaming read of
- * nbytes (a multiple of 16) with `blocks` workgroups of 256 threads.  They calibrate HBM byte
- * counters against a transfer of known size.  sink: 4 writable bytes.
- */
-int pllm_diag_stream_copy(const void* src, void* dst, size_t nbytes, int blocks, void* stream);
-int pllm_diag_stream_read(const void* src, void* sink, size_t nbytes, int blocks, void* stream);
-
 #ifdef __cplusplus
 }
 #endif

@@ -15,6 +15,7 @@ PKG = Path(__file__).resolve().parent
 CSRC = PKG / "csrc"
 OBJ_DIR = PKG / "build"
 LIB = PKG / "libpllm_hip.so"
+PROBE_LIB = PKG / "libpllm_probe.so"        # measurement aids (csrc/probe), kept out of the operator library
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
@@ -32,19 +33,25 @@ def _run(cmd: list[str]) -> None:
         print(out, file=sys.stderr)
 
 
-def build_library(verbose: bool = True, jobs: int = 8) -> Path:
+def build_library(verbose: bool = True, jobs: int = 8, incremental: bool = False) -> Path:
+    """Compiles every csrc/*.hip and links the library.  incremental=True (python -m pocketllm_amd.build --incremental) skips
+    sources whose object file is newer than the source and than every header."""
     OBJ_DIR.mkdir(exist_ok=True)
     sources = sorted(CSRC.glob("*.hip"))
     objs = [OBJ_DIR / (s.stem + ".o") for s in sources]
+    newest_header = max(h.stat().st_mtime for h in [*CSRC.glob("*.h"), *CSRC.glob("*.inc"), *(PKG.parent / "include").glob("*.h")])
+    todo = [(s, o) for s, o in zip(sources, objs)
+            if not (incremental and o.exists() and o.stat().st_mtime > max(s.stat().st_mtime, newest_header))]
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
-        futs = [pool.submit(_run, ["hipcc", *HIPCC_FLAGS, "-c", str(s), "-o", str(o)]) for s, o in zip(sources, objs)]
+        futs = [pool.submit(_run, ["hipcc", *HIPCC_FLAGS, "-c", str(s), "-o", str(o)]) for s, o in todo]
         for f in futs:
             f.result()
     _run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", *map(str, objs), "-o", str(LIB)])
+    _run(["hipcc", *HIPCC_FLAGS, "-shared", *map(str, sorted((CSRC / "probe").glob("*.hip"))), "-o", str(PROBE_LIB)])
     if verbose:
         print(f"built {LIB} from {len(sources)} sources")
     return LIB
 
 
 if __name__ == "__main__":
-    build_library()
+    build_library(incremental="--incremental" in sys.argv[1:])

@@ -355,6 +355,11 @@ int pllm_fp8_gemm(const uint8_t* a, const float* a_scale, const uint8_t* weight,
 
 // the tile GEMM serves many rows of 256-aligned k; everything else takes the matvec (no workspace)
 static bool fp8_uses_gemm(int64_t rows, int64_t k, int64_t n) { return k % 256 == 0 && rows >= tile_gemm_min_rows(RowClass::kFp8, n * k); }
+// float32 activations keep the float32 matvec (rel-L2 <= 1e-5 against the float statement of the operator, src/kernels/ops.py:641-648)
+// for every row count below 16; from 16 rows on they take the tile kernel like the 16-bit types (operands rounded to fp16, <= 1e-3).
+static bool fp8_uses_gemm_for(int x_dtype, int64_t rows, int64_t k, int64_t n) {
+    return fp8_uses_gemm(rows, k, n) && (x_dtype != PLLM_F32 || rows >= 16);
+}
 
 size_t pllm_fp8_block_gemm_workspace_bytes(int64_t rows, int64_t k, int64_t n) {
     if (!fits_int(rows) || !fits_int(k) || !fits_int(n) || !fp8_uses_gemm(rows, k, n)) return 0;
@@ -365,7 +370,7 @@ int pllm_fp8_block_gemm(const void* x, int x_dtype, const uint8_t* weight, const
                         int64_t rows, int64_t k, int64_t n, void* workspace, size_t workspace_bytes, void* stream) {
     if (!x || !weight || !scale || !y || !dtype_ok(x_dtype) || !dtype_ok(y_dtype)) return PLLM_ERR_INVALID_ARGUMENT;
     if (!fits_int(rows) || !fits_int(k) || !fits_int(n)) return PLLM_ERR_INVALID_ARGUMENT;
-    if (fp8_uses_gemm(rows, k, n))
+    if (fp8_uses_gemm_for(x_dtype, rows, k, n))
         return pllm::gemm_f16_fp8(x, x_dtype, weight, scale, y, y_dtype, static_cast<int>(rows), static_cast<int>(k), static_cast<int>(n),
                                   workspace, workspace_bytes, static_cast<hipStream_t>(stream));
     if (rows > 65535) return PLLM_ERR_UNSUPPORTED;
@@ -378,7 +383,7 @@ int pllm_fp8_block_gemm_accumulate(const void* x, int x_dtype, const uint8_t* we
     if (!x || !weight || !scale || !y || !dtype_ok(x_dtype) || !dtype_ok(y_dtype)) return PLLM_ERR_INVALID_ARGUMENT;
     if (!fits_int(rows) || !fits_int(k) || !fits_int(n)) return PLLM_ERR_INVALID_ARGUMENT;
     // the matvec only: the row counts pllm_fp8_block_gemm hands to the tile kernel are not served
-    if (rows > 65535 || fp8_uses_gemm(rows, k, n)) return PLLM_ERR_UNSUPPORTED;
+    if (rows > 65535 || fp8_uses_gemm_for(x_dtype, rows, k, n)) return PLLM_ERR_UNSUPPORTED;
     return pllm::fp8_matvec(x, x_dtype, weight, scale, y, y_dtype | pllm::kAccumulateInto, static_cast<int>(rows), static_cast<int>(k),
                             static_cast<int>(n), static_cast<hipStream_t>(stream));
 }

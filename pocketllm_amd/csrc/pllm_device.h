@@ -114,11 +114,13 @@ __device__ __forceinline__ StagedX carve_staged_x(const unsigned char* base, int
 }
 
 // Quantize four activations of one lane; the eight lanes of an aligned group share a 32-block.
-// Rounding and the int8 cast ride on one fused multiply-add each: for |t| < 2^22 the float
-// t + 1.5 * 2^23 has round-to-nearest-even(t) in its low mantissa bits, two's complement included, so
-// its low byte is the code and (sum - 1.5 * 2^23) the rounded value.  |v * inv| <= 127 and
-// |r * inv * 254| <= 127.01 by construction (inv and scale are reciprocal to 2^-22), so neither term
-// needs a clamp.  inv comes from v_rcp_f32: it only steers the rounding, the image carries `scale`.
+// First term: q = rint(fl(v / scale)) with scale = fl(amax / 127), the correctly rounded float32 quotient rounded to the nearest
+// even integer, which is the reference's 32-value activation quantizer (src/csrc/cuda_kernel_impl.cu:7102-7116) bit for bit;
+// |v / scale| <= 127 * (1 + 2^-23), so the clamp of the reference never acts.  The rounding and the int8 cast ride on one
+// addition: for |t| < 2^22 the float t + 1.5 * 2^23 has round-to-nearest-even(t) in its low mantissa bits, two's complement
+// included, so its low byte is the code and (sum - 1.5 * 2^23) the rounded value.  Second term: the residual v - q * scale in
+// units of scale / 254; its reciprocal comes from v_rcp_f32 (it only steers the rounding, the image carries `scale`), and
+// |r * inv * 254| <= 127.01 by construction, so it needs no clamp either.  An all-zero group stores scale 0 and codes 0.
 __device__ __forceinline__ uint32_t pack_low_bytes(uint32_t b0, uint32_t b1, uint32_t b2, uint32_t b3) {
     const uint32_t lo = __builtin_amdgcn_perm(b1, b0, 0x0c0c0400u);
     const uint32_t hi = __builtin_amdgcn_perm(b3, b2, 0x0c0c0400u);
@@ -128,13 +130,13 @@ __device__ __forceinline__ void quantize4(const float v[4], uint32_t& hi, uint32
     constexpr float kRound = 12582912.0f;                       // 1.5 * 2^23
     float am = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
     am = group_max<8>(am);
-    const float inv = am > 0.0f ? 127.0f * __builtin_amdgcn_rcpf(am) : 0.0f;
-    const float inv_lo = inv * 254.0f;
-    scale = am * (1.0f / 127.0f);
+    scale = am / 127.0f;
+    const float divisor = am > 0.0f ? scale : 1.0f;
+    const float inv_lo = am > 0.0f ? (127.0f * 254.0f) * __builtin_amdgcn_rcpf(am) : 0.0f;
     uint32_t qb[4], lb[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const float qm = fmaf(v[i], inv, kRound);
+        const float qm = v[i] / divisor + kRound;
         const float r = fmaf(kRound - qm, scale, v[i]);         // v - q * scale
         qb[i] = __float_as_uint(qm);
         lb[i] = __float_as_uint(fmaf(r, inv_lo, kRound));

@@ -1,7 +1,10 @@
-// Measurement aids: a plain streaming copy and a streaming read of known size.  They calibrate the
-// HBM counters (bytes a counter reports for a known transfer) and show the bandwidth a trivial
-// kernel reaches on the same box; no operator uses them.
-#include "pllm_internal.h"
+// Measurement aids, built into their own library (libpllm_probe.so), not into the operator library: a plain streaming copy
+// and a streaming read of known size.  They calibrate the HBM counters (bytes a counter reports for a known transfer) and
+// show the bandwidth a trivial kernel reaches on the same box; no operator uses them.
+//   int pllm_probe_stream_copy(src, dst, nbytes (a multiple of 16), workgroups of 256 threads, stream)   0 = launched
+//   int pllm_probe_stream_read(src, sink (4 writable bytes), nbytes, workgroups, stream)
+#include <hip/hip_runtime.h>
+#include <stdint.h>
 
 namespace pllm {
 namespace {
@@ -26,18 +29,18 @@ __global__ __launch_bounds__(256) void stream_read_kernel(const uint4* __restric
 
 extern "C" {
 
-int pllm_diag_stream_copy(const void* src, void* dst, size_t nbytes, int blocks, void* stream) {
-    if (!src || !dst || (nbytes & 15) || blocks <= 0) return PLLM_ERR_INVALID_ARGUMENT;
+int pllm_probe_stream_copy(const void* src, void* dst, size_t nbytes, int blocks, void* stream) {
+    if (!src || !dst || (nbytes & 15) || blocks <= 0) return -1;
     hipLaunchKernelGGL(pllm::stream_copy_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
                        static_cast<const uint4*>(src), static_cast<uint4*>(dst), nbytes >> 4);
-    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+    return hipGetLastError() == hipSuccess ? 0 : -2;
 }
 
-int pllm_diag_stream_read(const void* src, void* sink, size_t nbytes, int blocks, void* stream) {
-    if (!src || !sink || (nbytes & 15) || blocks <= 0) return PLLM_ERR_INVALID_ARGUMENT;
+int pllm_probe_stream_read(const void* src, void* sink, size_t nbytes, int blocks, void* stream) {
+    if (!src || !sink || (nbytes & 15) || blocks <= 0) return -1;
     hipLaunchKernelGGL(pllm::stream_read_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
                        static_cast<const uint4*>(src), static_cast<uint32_t*>(sink), nbytes >> 4);
-    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+    return hipGetLastError() == hipSuccess ? 0 : -2;
 }
 
 }  // extern "C"

@@ -20,6 +20,9 @@ def _require_kernel(what: str, attr: str | None = None):
     return mod
 
 
+_GRID_CACHE: dict[tuple[int, str], torch.Tensor] = {}
+
+
 class _BlockModule:
     """Shared state of the block-backed modules: the tensor, the output dtype and the grid argument."""
 
@@ -33,14 +36,16 @@ class _BlockModule:
 
     @staticmethod
     def _grid_for(tensor: QuantizedGGUFTensor) -> torch.Tensor:
+        """The codebook tensor of the tensor's type on the tensor's device (empty for the table-free types), one upload per
+        (type, device) shared by every module."""
         dev = tensor.blocks.device
-        if tensor.type_id == 0:
-            from pocketllm_amd.codebooks import get_iq2xxs_signed_grid_tensor
-            return get_iq2xxs_signed_grid_tensor().to(dev)
-        if tensor.type_id == 2:
-            from pocketllm_amd.codebooks import get_iq1_grid_tensor
-            return get_iq1_grid_tensor().to(dev)
-        return torch.empty(0, dtype=torch.int8, device=dev)
+        key = (int(tensor.type_id) if int(tensor.type_id) in (0, 2, 5, 6) else -1, str(dev))
+        grid = _GRID_CACHE.get(key)
+        if grid is None:
+            from pocketllm_amd.codebooks import grid_tensor_for_type
+            grid = grid_tensor_for_type(key[0]).to(dev)
+            _GRID_CACHE[key] = grid
+        return grid
 
 
 class QuantizedGGUFLinear(_BlockModule):

@@ -278,6 +278,53 @@ def test_activation_image_holds_two_int8_terms_per_value(mod, dtype):
     assert not hi[:, k:].any() and not lo[:, k:].any()
 
 
+def _quantizer_cases(rng, k):
+    """Rows that stress the 32-value quantizer: plain, tiny, huge, an all-zero group, values that sit on or next to rounding
+    ties of x / scale (half-integer multiples of amax / 127, one float32 step above and below), and a group whose largest
+    value is the only non-zero one."""
+    rows = [rng.standard_normal(k), rng.standard_normal(k) * 1e-6, rng.standard_normal(k) * 3e4, rng.standard_normal(k)]
+    rows[3][64:96] = 0.0
+    rows[3][128:160] = 0.0
+    rows[3][130] = -2.5
+    ties = np.empty(k, dtype=np.float32)
+    for g in range(k // 32):
+        amax = np.float32(rng.uniform(0.01, 50.0))
+        scale = np.float32(amax / np.float32(127.0))
+        half = (rng.integers(-126, 126, size=32).astype(np.float32) + np.float32(0.5)) * scale
+        nudge = rng.integers(-1, 2, size=32)
+        half = np.where(nudge > 0, np.nextafter(half, np.float32(np.inf)), np.where(nudge < 0, np.nextafter(half, np.float32(-np.inf)), half))
+        half[0] = amax
+        ties[32 * g:32 * g + 32] = half
+    rows.append(ties)
+    return np.stack(rows).astype(np.float32)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_activation_image_first_term_equals_the_reference_quantizer(mod, dtype):
+    """The first int8 term and the scale of the image are the reference's 32-value activation quantizer
+    (src/csrc/cuda_kernel_impl.cu:7090-7117, restated as oracle.q8_1_quantize): codes equal bit for bit, the stored figure is
+    float32(scale) * float32(1 / 254) bit for bit.  Only an all-zero group differs by design: scale 0 here, 1e-8 there, codes 0
+    in both."""
+    rng = np.random.default_rng(79)
+    dev = torch.device("cuda:0")
+    k, bpr = 2048, 8
+    x_np = _quantizer_cases(rng, k)
+    if dtype == torch.float16:
+        x_np = np.clip(x_np, -6e4, 6e4)
+    x = torch.from_numpy(x_np).to(dev).to(dtype)
+    xf = x.float().cpu().numpy()
+    rows = xf.shape[0]
+    want_q, want_s = O.q8_1_quantize(xf, 32)
+    zero = np.abs(xf).reshape(rows, -1, 32).max(axis=2) == 0
+    assert zero.sum() >= 1
+    image = mod.quantize_activations(x, bpr).cpu().numpy()
+    hi = image[:, :k].view(np.int8)
+    gs = image[:, 2 * k:2 * k + k // 32 * 8].copy().view(np.float32).reshape(rows, k // 32, 2)
+    np.testing.assert_array_equal(hi, want_q)
+    want_gs = np.where(zero, np.float32(0.0), want_s * np.float32(1.0 / 254.0)).astype(np.float32)
+    np.testing.assert_array_equal(gs[..., 0].view(np.uint32), want_gs.view(np.uint32))
+
+
 @pytest.mark.parametrize("type_name", ["q4_k", "q5_k", "q2_k", "q6_k", "iq4_xs", "iq2_xxs", "iq1_m", "iq2_xs", "iq3_xxs"])
 def test_few_row_calls_equal_the_prequantized_path(mod, type_name):
     """Calls of a few rows may quantize the activations inside the matvec kernel; the result is the same bits as quantizing ahead."""

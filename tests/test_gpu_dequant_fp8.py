@@ -118,7 +118,7 @@ def test_fp8_dequant_all_codes_and_block_scales(mod):
     np.testing.assert_array_equal(got2.cpu().numpy(), got)
 
 
-@pytest.mark.parametrize("n,k,rows", [(130, 304, 1), (256, 1024, 1), (17408, 5120, 1), (64, 5120, 3), (33, 300, 2), (16, 40960, 1), (4500, 8192, 1)])
+@pytest.mark.parametrize("n,k,rows", [(130, 304, 1), (256, 1024, 1), (17408, 5120, 1), (64, 5120, 3), (33, 300, 2), (16, 40960, 1), (4500, 8192, 1), (17408, 5120, 6)])
 def test_fp8_matvec_matches_oracle(mod, n, k, rows):
     rng = np.random.default_rng(40 + n)
     if n * k <= 4_000_000:
@@ -134,7 +134,10 @@ def test_fp8_matvec_matches_oracle(mod, n, k, rows):
         y = mod.fp8_block_gemm_forward(xd, torch.from_numpy(codes).to(DEV), torch.from_numpy(scale).to(DEV))
         torch.cuda.synchronize()
         want = O.matmul_f(xd.float().cpu().numpy(), O.dequant_fp8_block(codes, scale))
-        assert O.rel_l2(y.cpu().numpy(), want) <= 1e-5, (n, k, rows, dt)
+        # float32 activations stay on the float32 matvec below 16 rows whatever the matrix size; 16-bit activations may take
+        # the fp16 tile kernel from a few rows on for large matrices (operands rounded to fp16)
+        tol = 1e-3 if (dt != torch.float32 and rows >= 3 and n * k >= (64 << 20)) else 1e-5
+        assert O.rel_l2(y.cpu().numpy(), want) <= tol, (n, k, rows, dt)
 
 
 def test_fp8_act_quant_matches_reference_recipe(mod):

@@ -129,6 +129,64 @@ def test_baseline_config_single_token_shapes(mod):
     assert O.rel_l2(y.cpu().numpy(), want) <= TOL
 
 
+def test_baseline_config_grouped_256_tokens_256_experts(mod):
+    """BASELINE config 5 at T = 256: 256 experts, top-8 softmax routing, 2048 routes, every weight tensor at its full size.
+    The oracle restates the operator for six sampled tokens (their 48 routes, full output rows); every other token is
+    covered by the determinism check and by the finite, non-zero rows."""
+    rng = np.random.default_rng(1005)
+    e, d, inter, topk, t = 256, 3072, 1536, 8, 256
+    w1 = _expert_blocks(rng, "iq2_xxs", e, inter, d)
+    w3 = _expert_blocks(rng, "iq2_xxs", e, inter, d)
+    w2 = _expert_blocks(rng, "iq1_m", e, d, inter)
+    idx, wts = _route(rng, t, e, topk)
+    x = torch.from_numpy(rng.standard_normal((t, d)).astype(np.float32)).to(DEV).to(torch.bfloat16)
+    _, toks, rws, seg = mod.moe_group_routes(torch.from_numpy(idx).to(DEV), torch.from_numpy(wts).to(DEV), 0, e)
+    _, o_toks, o_rws, o_seg = O.group_routes(idx, wts, 0, e)
+    np.testing.assert_array_equal(seg.cpu().numpy(), o_seg)
+    np.testing.assert_array_equal(toks.cpu().numpy(), o_toks)
+    assert len(o_toks) == t * topk
+    grids = (codebooks.get_iq2xxs_signed_grid_tensor().to(DEV), codebooks.get_iq1_grid_tensor().to(DEV))
+    dw1, dw3, dw2 = (torch.from_numpy(a).to(DEV) for a in (w1, w3, w2))
+    tid = O.TYPE_IDS
+    print("case grouped experts 256 tokens x 256 experts", flush=True)
+    y = mod.gguf_moe_prefill_grouped_forward(x, toks, rws, seg, dw1, dw3, dw2, d, tid["iq2_xxs"], d, tid["iq2_xxs"], inter, tid["iq1_m"], grids, 0.0)
+    torch.cuda.synchronize()
+    got = y.cpu().numpy()
+    assert got.shape == (t, d) and np.isfinite(got).all() and (np.abs(got).max(axis=1) > 0).all()
+    route_experts = np.repeat(np.arange(e), np.diff(o_seg))
+    sample = rng.choice(t, size=6, replace=False)
+    keep = np.isin(o_toks, sample)
+    want = O.moe_forward(x.float().cpu().numpy(), o_toks[keep], o_rws[keep], route_experts[keep], w1, w3, w2, "iq2_xxs", "iq2_xxs", "iq1_m", 0.0)
+    assert O.rel_l2(got[sample], want[sample]) <= TOL
+    for tok in sample:
+        assert O.rel_l2(got[tok], want[tok]) <= 2 * TOL, tok
+    y2 = mod.gguf_moe_prefill_grouped_forward(x, toks, rws, seg, dw1, dw3, dw2, d, tid["iq2_xxs"], d, tid["iq2_xxs"], inter, tid["iq1_m"], grids, 0.0)
+    assert torch.equal(y, y2)
+
+
+def test_grouped_experts_more_routes_than_the_reduction_lists(mod):
+    """More than 2048 routes: the route-sum kernel then scans the route table instead of listing a token's routes in LDS."""
+    rng = np.random.default_rng(17)
+    e, d, inter, topk, t = 40, 256, 256, 8, 300
+    w1 = _expert_blocks(rng, "iq2_xxs", e, inter, d)
+    w3 = _expert_blocks(rng, "iq2_xxs", e, inter, d)
+    w2 = _expert_blocks(rng, "iq1_m", e, d, inter)
+    idx, wts = _route(rng, t, e, topk)
+    x = torch.from_numpy(rng.standard_normal((t, d)).astype(np.float32)).to(DEV).to(torch.bfloat16)
+    _, toks, rws, seg = mod.moe_group_routes(torch.from_numpy(idx).to(DEV), torch.from_numpy(wts).to(DEV), 0, e)
+    _, o_toks, o_rws, o_seg = O.group_routes(idx, wts, 0, e)
+    assert len(o_toks) == 2400
+    grids = (codebooks.get_iq2xxs_signed_grid_tensor().to(DEV), codebooks.get_iq1_grid_tensor().to(DEV))
+    dw1, dw3, dw2 = (torch.from_numpy(a).to(DEV) for a in (w1, w3, w2))
+    tid = O.TYPE_IDS
+    print("case grouped experts 2400 routes", flush=True)
+    y = mod.gguf_moe_prefill_grouped_forward(x, toks, rws, seg, dw1, dw3, dw2, d, tid["iq2_xxs"], d, tid["iq2_xxs"], inter, tid["iq1_m"], grids, 0.0)
+    torch.cuda.synchronize()
+    route_experts = np.repeat(np.arange(e), np.diff(o_seg))
+    want = O.moe_forward(x.float().cpu().numpy(), o_toks, o_rws, route_experts, w1, w3, w2, "iq2_xxs", "iq2_xxs", "iq1_m", 0.0)
+    assert O.rel_l2(y.cpu().numpy(), want) <= TOL
+
+
 def test_route_slots_host_compaction(mod):
     idx = torch.tensor([[9, 3, 12, 4, 3]], device=DEV)
     w = torch.tensor([[0.1, 0.2, 0.3, 0.25, 0.15]], device=DEV)
@@ -194,6 +252,19 @@ def test_linear_modules(mod):
         x = torch.randn(3, 512, device=DEV, dtype=torch.float16)
         want = O.matmul_f(x.float().cpu().numpy(), O.dequant_rows(bl, name))
         assert np.abs(lin2(x).float().cpu().numpy() - want).max() < 2e-2
+    # the codebook types: the module brings the grid of its type itself (one upload per type and device)
+    for name in ("iq2_xxs", "iq1_m", "iq2_xs", "iq3_xxs"):
+        bl = GEN[name](rng, 64, 2) if name in GEN else C.random_blocks(rng, name, 64, 2)
+        lin3 = QuantizedGGUFLinear(QuantizedGGUFTensor.from_blocks(torch.from_numpy(bl).to(DEV), name, 512, source_name=name))
+        lin4 = QuantizedGGUFLinear(QuantizedGGUFTensor.from_blocks(torch.from_numpy(bl).to(DEV), name, 512, source_name=name))
+        assert lin3._grid.data_ptr() == lin4._grid.data_ptr()
+        x = torch.randn(3, 512, device=DEV, dtype=torch.float16)
+        want = O.matmul_f(x.float().cpu().numpy(), O.dequant_rows(bl, name))
+        got = lin3(x).float().cpu().numpy()
+        assert O.rel_l2(got, want) < 2e-3, name
+        emb3 = QuantizedGGUFEmbedding(QuantizedGGUFTensor.from_blocks(torch.from_numpy(bl).to(DEV), name, 512, source_name=name))
+        rows = emb3(torch.tensor([5, 63], device=DEV, dtype=torch.int32)).float().cpu().numpy()
+        assert O.rel_l2(rows, O.dequant_rows(bl[[5, 63]], name)) < 2e-3, name
     q8 = Q8_0GGUFLinear(torch.from_numpy(C.pack_q8_0(w)).to(DEV), 512, source_name="q8")
     x = torch.randn(2, 512, device=DEV, dtype=torch.float16)
     want = O.matmul_f(x.float().cpu().numpy(), O.dequant_rows(C.pack_q8_0(w), "q8_0"))

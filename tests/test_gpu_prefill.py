@@ -58,19 +58,29 @@ def test_prefill_3d_input_and_bf16_output(mod):
     assert O.rel_l2(y32.view(32, 192).cpu().numpy(), yd.cpu().numpy()) < 5e-4
 
 
-@pytest.mark.parametrize("type_name,n", [("q4_k", 5120), ("q5_k", 17408)])
-def test_prefill_baseline_shape_sampled(mod, type_name, n):
-    """BASELINE config 3 shape at T = 512; the oracle checks 64 sampled output columns (seconds on the host)."""
-    rng = np.random.default_rng(1003)
-    k, t = 5120, 512
+@pytest.mark.parametrize("type_name", ["q4_k", "q5_k"])
+@pytest.mark.parametrize("n", [5120, 17408])
+def test_prefill_baseline_shapes_sampled(mod, type_name, n):
+    """BASELINE config 3: both shapes, both formats, T = 64, 512 and 2048.  The weights are encoded once per (format, shape);
+    the oracle checks 64 sampled output columns of every token row (seconds on the host)."""
+    rng = np.random.default_rng(1003 + n + len(type_name))
+    k = 5120
     blocks = ENC[type_name]((rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02)))
-    x = torch.from_numpy(rng.standard_normal((t, k)).astype(np.float32)).to(DEV).to(torch.bfloat16)
-    y = mod.gguf_quant_gemm_prefill_forward(x, torch.from_numpy(blocks).to(DEV), k, O.TYPE_IDS[type_name],
-                                            codebooks.grid_tensor_for_type(O.TYPE_IDS[type_name]).to(DEV), out_dtype=torch.float32)
-    torch.cuda.synchronize()
+    dblocks = torch.from_numpy(blocks).to(DEV)
+    grid = codebooks.grid_tensor_for_type(O.TYPE_IDS[type_name]).to(DEV)
     cols = rng.choice(n, size=64, replace=False)
-    want = O.matmul_f(x.float().cpu().numpy(), O.dequant_rows(blocks[cols], type_name, k))
-    assert O.rel_l2(y.cpu().numpy()[:, cols], want) <= 4e-4
+    ref_w = O.dequant_rows(blocks[cols], type_name, k)
+    for t in (64, 512, 2048):
+        x = torch.from_numpy(rng.standard_normal((t, k)).astype(np.float32)).to(DEV).to(torch.bfloat16)
+        print(f"case prefill baseline {type_name} n={n} t={t}", flush=True)
+        y = mod.gguf_quant_gemm_prefill_forward(x, dblocks, k, O.TYPE_IDS[type_name], grid, out_dtype=torch.float32)
+        torch.cuda.synchronize()
+        assert tuple(y.shape) == (t, n)
+        want = O.matmul_f(x.float().cpu().numpy(), ref_w)
+        got = y.cpu().numpy()[:, cols]
+        assert O.rel_l2(got, want) <= 1e-3, (t, O.rel_l2(got, want))
+        row_err = np.sqrt(((got - want) ** 2).sum(axis=1) / np.maximum((want ** 2).sum(axis=1), 1e-300))
+        assert row_err.max() <= 2e-3, (t, row_err.argmax(), row_err.max())
 
 
 @pytest.mark.parametrize("type_name,n,rows", [("q4_k", 17408, 5), ("q5_k", 17408, 7), ("q4_k", 5120, 11), ("q4_k", 5120, 12), ("q5_k", 5120, 15),
