@@ -98,14 +98,16 @@ size_t pllm_q8_0_gemm_workspace_bytes(int64_t rows, int64_t k, int64_t n, int64_
     return pllm::q8_0_matvec_workspace_bytes(static_cast<int>(rows), static_cast<int>(blocks_per_row));
 }
 
-// Calls of up to this many rows skip the activation pre-pass where the kernel can quantize its row itself.  The Q4_K / Q5_K
-// kernel runs one short workgroup per 16 rows and every one of them repeats the quantization: that beats the extra launch
-// (~3 us) up to about a thousand workgroups of a 5120-wide row; the other kernels are longer per workgroup or persistent.
+// Calls of up to this many rows skip the activation pre-pass: the kernels quantize their activation rows themselves.  One row
+// of Q4_K / Q5_K always does (every wave quantizes the slices of its own blocks while its weights are in flight); two to four
+// rows on large Q4_K / Q5_K matrices keep the pre-pass, because only the kernel that reads prepared images shares one pass
+// over the weights between the rows.
 constexpr int64_t kInKernelQuantMaxRows = 4;
 constexpr int64_t kInKernelQuantMaxWeightsK45 = int64_t{64} << 20;
 
-static bool quantizes_in_kernel(int type_id, int64_t n, int64_t bpr) {
-    if (type_id == PLLM_TYPE_Q4_K || type_id == PLLM_TYPE_Q5_K) return n * bpr * 256 <= kInKernelQuantMaxWeightsK45;
+static bool quantizes_in_kernel(int type_id, int64_t rows, int64_t n, int64_t bpr) {
+    if (rows > kInKernelQuantMaxRows) return false;
+    if (type_id == PLLM_TYPE_Q4_K || type_id == PLLM_TYPE_Q5_K) return rows == 1 || n * bpr * 256 <= kInKernelQuantMaxWeightsK45;
     return pllm_gguf_block_bytes(type_id) != 0;
 }
 
@@ -150,7 +152,7 @@ int pllm_gguf_quant_gemm(const void* x, int x_dtype, const uint8_t* blocks, int 
     if (gguf_uses_tile_gemm(type_id, rows, n, blocks_per_row))
         return pllm::gemm_f16(x, x_dtype, blocks, type_id, y, y_dtype, static_cast<int>(rows), static_cast<int>(k), static_cast<int>(n), bpr,
                               workspace, workspace_bytes, s);
-    if (rows <= kInKernelQuantMaxRows && quantizes_in_kernel(type_id, n, blocks_per_row))
+    if (quantizes_in_kernel(type_id, rows, n, blocks_per_row))
         return superblock_matvec(pllm::act_rows_raw(x, x_dtype, static_cast<int>(k)), blocks, type_id, y, y_dtype,
                                  static_cast<int>(rows), static_cast<int>(n), bpr, s);
     const int st = pllm::act_image_256(x, x_dtype, static_cast<int>(rows), static_cast<int>(k), bpr, workspace, s);
@@ -172,7 +174,7 @@ int pllm_gguf_quant_gemm_accumulate(const void* x, int x_dtype, const uint8_t* b
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int bpr = static_cast<int>(blocks_per_row);
     const int into = y_dtype | pllm::kAccumulateInto;
-    if (rows <= kInKernelQuantMaxRows && quantizes_in_kernel(type_id, n, blocks_per_row))
+    if (quantizes_in_kernel(type_id, rows, n, blocks_per_row))
         return superblock_matvec(pllm::act_rows_raw(x, x_dtype, static_cast<int>(k)), blocks, type_id, y, into,
                                  static_cast<int>(rows), static_cast<int>(n), bpr, s);
     const int st = pllm::act_image_256(x, x_dtype, static_cast<int>(rows), static_cast<int>(k), bpr, workspace, s);
@@ -242,7 +244,7 @@ int pllm_gguf_quant_gemm_multi(const void* x, int x_dtype, const float* norm_wei
     // one launch exists in the matrix-core decode kernels; Q2_K (and anything else) is left to one call per matrix
     if (type_id == PLLM_TYPE_Q2_K) return PLLM_ERR_UNSUPPORTED;
     if (rows > 65535 || gguf_uses_tile_gemm(type_id, rows, total_n, blocks_per_row)) return PLLM_ERR_UNSUPPORTED;
-    const bool raw = rows <= kInKernelQuantMaxRows && (norm_weight || quantizes_in_kernel(type_id, total_n, blocks_per_row));
+    const bool raw = rows <= kInKernelQuantMaxRows && (norm_weight || quantizes_in_kernel(type_id, rows, total_n, blocks_per_row));
     if (norm_weight && !raw) return PLLM_ERR_UNSUPPORTED;                    // the normalisation exists inside the kernel only
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int bpr = static_cast<int>(blocks_per_row);
@@ -323,9 +325,8 @@ int pllm_gguf_quant_gemm_pair(const void* x, int x_dtype, const uint8_t* blocks0
     const int R = static_cast<int>(rows), N = static_cast<int>(n);
     const size_t esize = y_dtype == PLLM_F32 ? 4 : 2;
     const bool k45 = type_id0 == type_id1 && (type_id0 == PLLM_TYPE_Q4_K || type_id0 == PLLM_TYPE_Q5_K);
-    const bool raw = rows <= kInKernelQuantMaxRows &&
-                     (k45 ? quantizes_in_kernel(type_id0, 2 * n, blocks_per_row)
-                          : quantizes_in_kernel(type_id0, n, blocks_per_row) && quantizes_in_kernel(type_id1, n, blocks_per_row));
+    const bool raw = k45 ? quantizes_in_kernel(type_id0, rows, 2 * n, blocks_per_row)
+                         : quantizes_in_kernel(type_id0, rows, n, blocks_per_row) && quantizes_in_kernel(type_id1, rows, n, blocks_per_row);
     pllm::ActRows act = pllm::act_rows_raw(x, x_dtype, static_cast<int>(k));
     if (!raw) {
         const int st = pllm::act_image_256(x, x_dtype, R, static_cast<int>(k), bpr, workspace, s);

@@ -58,6 +58,24 @@ __device__ __forceinline__ uint4 fifth_bit(const uint4& w, const uint4& qh, int 
                       w.z | (__builtin_amdgcn_alignbit(qh.z, qh.z, r) & 0x10101010u), w.w | (__builtin_amdgcn_alignbit(qh.w, qh.w, r) & 0x10101010u));
 }
 
+// Which 32-weight group MFMA t's k slice ks carries for the two nibble formats, and the float epilogue of the lane that
+// holds the integer dots v0, v1 (both activation terms folded: 254 * hi + lo) of groups 2 ks and 2 ks + 1 of its row;
+// g2 = {xs0 / 254, sum0, xs1 / 254, sum1} of those groups' activations.
+__device__ __forceinline__ int k45_group_of(int t, int ks) { return 4 * (t >> 1) + 2 * (ks >> 1) + (t & 1); }
+__device__ __forceinline__ float k45_combine(const uint4& hdr, int ks, float v0, float v1, const float4& g2) {
+    const K4Scales sc = k4_unpack(hdr);
+    const uint32_t scw = ((ks & 2) ? sc.sc_hi : sc.sc_lo) >> (16 * (ks & 1));
+    const uint32_t mnw = ((ks & 2) ? sc.mn_hi : sc.mn_lo) >> (16 * (ks & 1));
+    const float d = f16_bits_to_float(hdr.x & 0xffffu);
+    const float dmin = f16_bits_to_float(hdr.x >> 16);
+    const float s0 = static_cast<float>(scw & 0xffu), s1 = static_cast<float>((scw >> 8) & 0xffu);
+    const float m0 = static_cast<float>(mnw & 0xffu), m1 = static_cast<float>((mnw >> 8) & 0xffu);
+    // explicit fused multiply-adds: every kernel that calls this rounds the same way, whatever the compiler would contract
+    const float pos = __builtin_fmaf(s1 * g2.z, v1, (s0 * g2.x) * v0);
+    const float neg = __builtin_fmaf(m1, g2.w, m0 * g2.y);
+    return __builtin_fmaf(d, pos, -(dmin * neg));
+}
+
 // ------------------------------------------------------------------------------------------------
 // Q4_K: 144 B = d(2) dmin(2) scales(12) qs(128).  Lane (n, ks) holds qs[16 ks, +16) and
 // qs[64 + 16 ks, +16).  With p = ks >> 1, h = ks & 1 the first chunk carries weights 16h + (0..15)
@@ -68,6 +86,7 @@ __device__ __forceinline__ uint4 fifth_bit(const uint4& w, const uint4& qh, int 
 // ------------------------------------------------------------------------------------------------
 struct Q4K {
     static constexpr int kBlockBytes = 144;
+    static constexpr int kDepth = 5;                          // blocks in flight per wave that fit 128 registers (four waves per SIMD)
     struct Regs { uint4 hdr; uint4 qa; uint4 qb; };
     static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, int ks) {
         r.hdr = *reinterpret_cast<const uint4*>(blk);
@@ -78,10 +97,13 @@ struct Q4K {
     static __device__ __forceinline__ void codes(const Regs& r, int, uint4 b[4]) {
         b[0] = nib_lo(r.qa); b[1] = nib_hi(r.qa); b[2] = nib_lo(r.qb); b[3] = nib_hi(r.qb);
     }
+    static __device__ __forceinline__ int group_of(int t, int ks) { return k45_group_of(t, ks); }
+    static __device__ __forceinline__ float combine(const Regs& r, int ks, float v0, float v1, const float4& g2) { return k45_combine(r.hdr, ks, v0, v1, g2); }
 };
 
 struct Q5K {
     static constexpr int kBlockBytes = 176;
+    static constexpr int kDepth = 4;
     struct Regs { uint4 hdr; uint4 qh; uint4 qa; uint4 qb; };
     static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, int ks) {
         r.hdr = *reinterpret_cast<const uint4*>(blk);
@@ -96,7 +118,11 @@ struct Q5K {
         b[2] = fifth_bit(nib_lo(r.qb), r.qh, g + 4);
         b[3] = fifth_bit(nib_hi(r.qb), r.qh, g + 5);
     }
+    static __device__ __forceinline__ int group_of(int t, int ks) { return k45_group_of(t, ks); }
+    static __device__ __forceinline__ float combine(const Regs& r, int ks, float v0, float v1, const float4& g2) { return k45_combine(r.hdr, ks, v0, v1, g2); }
 };
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 // R activation rows per workgroup (1, 2 or 4): the weights of a super-block are loaded and split into codes once and multiplied
 // with the images of R rows, which sit side by side in LDS; grid row blockIdx.y serves activation rows R * blockIdx.y ...
@@ -133,7 +159,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void k45_mfma_matvec_kernel(
     int a_off[4], a_step[4], a_row[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-        const int g = 4 * (t >> 1) + 2 * (ks >> 1) + (t & 1);
+        const int g = FMT::group_of(t, ks);
         const bool active = (col >> 1) == g;
         a_off[t] = active ? ((col & 1) ? kpad : 0) + 32 * g + 16 * (ks & 1) : zero_off;
         a_step[t] = active ? 256 : 0;
@@ -177,13 +203,6 @@ __global__ __launch_bounds__(64 * kMaxWaves) void k45_mfma_matvec_kernel(
             if (b < bpr) {                                                   // wave-uniform
                 uint4 bw[4];
                 FMT::codes(regs[it], ks, bw);
-                const K4Scales sc = k4_unpack(regs[it].hdr);
-                const uint32_t scw = ((ks & 2) ? sc.sc_hi : sc.sc_lo) >> (16 * (ks & 1));
-                const uint32_t mnw = ((ks & 2) ? sc.mn_hi : sc.mn_lo) >> (16 * (ks & 1));
-                const float d = f16_bits_to_float(regs[it].hdr.x & 0xffffu);
-                const float dmin = f16_bits_to_float(regs[it].hdr.x >> 16);
-                const float s0 = static_cast<float>(scw & 0xffu), s1 = static_cast<float>((scw >> 8) & 0xffu);
-                const float m0 = static_cast<float>(mnw & 0xffu), m1 = static_cast<float>((mnw >> 8) & 0xffu);
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
                     v4i c = {0, 0, 0, 0};
@@ -196,9 +215,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void k45_mfma_matvec_kernel(
                     const float v0 = static_cast<float>(__mul24(c.x, 254) + c.y);
                     const float v1 = static_cast<float>(__mul24(c.z, 254) + c.w);
                     const float4 g2 = *reinterpret_cast<const float4*>(reinterpret_cast<const unsigned char*>(sx.gs + b * 8 + 2 * ks) + r * image_bytes);   // {xs0, sum0, xs1, sum1}
-                    const float pos = s0 * g2.x * v0 + s1 * g2.z * v1;
-                    const float neg = m0 * g2.y + m1 * g2.w;
-                    acc[r] += d * pos - dmin * neg;
+                    acc[r] += FMT::combine(regs[it], ks, v0, v1, g2);
                 }
             }
         }
@@ -221,6 +238,171 @@ __global__ __launch_bounds__(64 * kMaxWaves) void k45_mfma_matvec_kernel(
 }
 
 // ------------------------------------------------------------------------------------------------
+// The single-launch form for calls of a few raw activation rows: no workgroup-wide image and no barrier ahead of the
+// matrix-core work.  A wave needs the activations of its own super-blocks only (wave w of W takes blocks w, w + W, ...), so it
+// requests those 256-value slices first, then all its weights, and quantizes the slices (the same two-term image, bit for
+// bit) into its own LDS slots while the weights are on their way; memory returns a wave's loads in the order they were
+// issued, so the slices are there long before the first block.  Slot = hi[256] | lo[256] | float2 gs[8] (576 B).  The waves
+// meet only in the final sum.
+constexpr int kSlotBytes = 576;
+
+template <bool X16> struct RawX;
+template <> struct RawX<true> { uint2 v; };                    // four fp16 / bf16 values
+template <> struct RawX<false> { uint4 v; };                   // four float32 values
+
+// Values e0 .. e0 + 3 of the row at element offset xoff, zeros from k on (k >= 4 or k == 0), in two steps so that nothing
+// waits between the requests of consecutive blocks.  request_raw4 is branch-free and only issues the load: four values from
+// an address clamped into the row (the row's last four values for a lane at or past its end; any alignment).  settle_raw4,
+// called where the values are used, shifts them down by the number of values the clamp moved the address.
+__device__ __forceinline__ int raw4_start(int e0, int k) { return max(min(e0, k - 4), 0); }
+template <bool X16>
+__device__ __forceinline__ void request_raw4(RawX<X16>& r, const void* __restrict__ x, size_t xoff, int e0, int k) {
+    const int start = raw4_start(e0, k);
+    if constexpr (X16) {
+        struct __attribute__((packed, aligned(2))) U { uint32_t a, b; };
+        const U u = *reinterpret_cast<const U*>(static_cast<const uint16_t*>(x) + xoff + start);
+        r.v = make_uint2(u.a, u.b);
+    } else {
+        struct __attribute__((packed, aligned(4))) U { u32x4 v; };
+        const U u = *reinterpret_cast<const U*>(static_cast<const uint32_t*>(x) + xoff + start);
+        r.v = make_uint4(u.v.x, u.v.y, u.v.z, u.v.w);
+    }
+}
+template <bool X16>
+__device__ __forceinline__ void settle_raw4(RawX<X16>& r, int e0, int k) {
+    const int moved = k == 0 ? 4 : min(e0 - raw4_start(e0, k), 4);          // 0: all four values lie inside the row; 4: none does
+    if constexpr (X16) {
+        const uint64_t both = (static_cast<uint64_t>(r.v.y) << 32) | r.v.x;
+        const uint64_t kept = moved >= 4 ? 0ull : both >> (16 * moved);
+        r.v = make_uint2(static_cast<uint32_t>(kept), static_cast<uint32_t>(kept >> 32));
+    } else {
+        const uint4 u = r.v;
+        r.v.x = moved == 0 ? u.x : moved == 1 ? u.y : moved == 2 ? u.z : moved == 3 ? u.w : 0u;
+        r.v.y = moved == 0 ? u.y : moved == 1 ? u.z : moved == 2 ? u.w : 0u;
+        r.v.z = moved == 0 ? u.z : moved == 1 ? u.w : 0u;
+        r.v.w = moved == 0 ? u.w : 0u;
+    }
+}
+template <bool X16>
+__device__ __forceinline__ void raw_to_float4(const RawX<X16>& r, int x_dtype, float v[4]) {
+    if constexpr (X16) {
+        if (x_dtype == PLLM_BF16) {
+            v[0] = __uint_as_float(r.v.x << 16); v[1] = __uint_as_float(r.v.x & 0xffff0000u);
+            v[2] = __uint_as_float(r.v.y << 16); v[3] = __uint_as_float(r.v.y & 0xffff0000u);
+        } else {
+            v[0] = f16_bits_to_float(r.v.x & 0xffffu); v[1] = f16_bits_to_float(r.v.x >> 16);
+            v[2] = f16_bits_to_float(r.v.y & 0xffffu); v[3] = f16_bits_to_float(r.v.y >> 16);
+        }
+    } else {
+        v[0] = __uint_as_float(r.v.x); v[1] = __uint_as_float(r.v.y); v[2] = __uint_as_float(r.v.z); v[3] = __uint_as_float(r.v.w);
+    }
+}
+
+// ITERS = blocks a wave walks per pass, DEPTH <= ITERS = blocks it keeps in flight (a block's activation slice is requested
+// right ahead of its weights, so it arrives first).
+template <typename FMT, int ITERS, int DEPTH, bool X16>
+__global__ __launch_bounds__(64 * kMaxWaves) void wave_image_matvec_kernel(
+    const void* __restrict__ x, int x_dtype, int k, const WeightRoute route, const uint8_t* __restrict__ w, void* __restrict__ y,
+    int y_dtype, int n, int bpr) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int tid = threadIdx.x;
+    const int waves = blockDim.x >> 6;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    const int col = lane & 15;
+    const int ks = lane >> 4;
+    constexpr int kWaveBytes = kSlotBytes + 16;                               // the wave's slot, then its 16 zero bytes
+    unsigned char* slot = smem + wave * kWaveBytes;
+    float* partial = reinterpret_cast<float*>(smem + waves * kWaveBytes);    // [waves][16]
+    if (blockIdx.z) {                        // several projections in one launch: this one's matrix, row count and output
+        const int m = blockIdx.z - 1;
+        w = route.more_w[m];
+        y = route.more_y[m];
+        n = route.more_n[m];
+    }
+    if (static_cast<int>(blockIdx.x) * kRowsPerWg >= n) return;             // the grid covers the tallest matrix
+    const int row = blockIdx.x * kRowsPerWg + col;
+    const uint8_t* wrow = w + static_cast<size_t>(row < n ? row : 0) * bpr * FMT::kBlockBytes;
+    const size_t xoff = static_cast<size_t>(blockIdx.y) * k;
+
+    if (lane < 4) reinterpret_cast<uint32_t*>(slot + kSlotBytes)[lane] = 0;
+    float acc = 0.0f;
+    for (int b0 = wave; b0 < bpr; b0 += waves * ITERS) {
+        RawX<X16> raw[DEPTH];
+        typename FMT::Regs regs[DEPTH];
+        auto request_x = [&](int it) {
+            const int b = b0 + it * waves;
+            request_raw4<X16>(raw[it % DEPTH], x, xoff, 256 * b + 4 * lane, b < bpr ? k : 0);
+        };
+        auto request_w = [&](int it) {
+            const int b = b0 + it * waves;
+            FMT::load(regs[it % DEPTH], wrow + static_cast<size_t>(min(b, bpr - 1)) * FMT::kBlockBytes, ks);   // clamped: always a valid address
+        };
+        auto request = [&](int it) {
+            request_x(it);
+            __builtin_amdgcn_sched_barrier(0);                              // keep the issue order: memory returns a wave's loads in it
+            request_w(it);
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        // the activation slices first: they are small, arrive first and are quantized while the weights are on their way
+#pragma unroll
+        for (int it = 0; it < DEPTH; ++it) request_x(it);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int it = 0; it < DEPTH; ++it) request_w(it);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+            const int b = b0 + it * waves;
+            if (b < bpr) {                                                   // wave-uniform
+                // the block's activation slice into the wave's slot: the same two-term image the pre-pass kernel writes
+                float v[4];
+                if (k != 256 * bpr) settle_raw4<X16>(raw[it % DEPTH], 256 * b + 4 * lane, k);   // rows that end inside their last block
+                raw_to_float4<X16>(raw[it % DEPTH], x_dtype, v);
+                uint32_t qh, ql;
+                float scale;
+                quantize4(v, qh, ql, scale);
+                reinterpret_cast<uint32_t*>(slot)[lane] = qh;
+                reinterpret_cast<uint32_t*>(slot + 256)[lane] = ql;
+                const float sum = group_sum<4>((v[0] + v[1]) + (v[2] + v[3]));   // the order in which the pre-pass kernel sums
+                const float sum32 = sum + butterfly_peer<4>(sum);
+                if ((lane & 7) == 0) reinterpret_cast<float2*>(slot + 512)[lane >> 3] = make_float2(scale * kLoInv, sum32);
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();                            // LDS serves a wave's requests in order
+                uint4 bw[4];
+                FMT::codes(regs[it % DEPTH], ks, bw);
+                v4i c = {0, 0, 0, 0};
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    // this lane supplies row m = col = 2 * group + term of MFMA t's A operand, slice ks: codes only where that
+                    // slice belongs to `group`, the zero bytes elsewhere
+                    const int g = FMT::group_of(t, ks);
+                    const int off = (col >> 1) == g ? ((col & 1) ? 256 : 0) + 32 * g + 16 * (ks & 1) : kSlotBytes;
+                    const uint4 a = *reinterpret_cast<const uint4*>(slot + off);
+                    c = __builtin_amdgcn_mfma_i32_16x16x64_i8(as_v4i(a), as_v4i(bw[t]), c, 0, 0, 0);
+                }
+                const float v0 = static_cast<float>(__mul24(c.x, 254) + c.y);
+                const float v1 = static_cast<float>(__mul24(c.z, 254) + c.w);
+                const float4 g2 = *reinterpret_cast<const float4*>(slot + 512 + 16 * ks);   // {xs0, sum0, xs1, sum1}
+                acc += FMT::combine(regs[it % DEPTH], ks, v0, v1, g2);
+                __builtin_amdgcn_wave_barrier();                            // the next block's slice overwrites the slot
+            }
+            if (it + DEPTH < ITERS) request(it + DEPTH);
+        }
+    }
+    acc += __shfl_xor(acc, 16, 64);
+    acc += __shfl_xor(acc, 32, 64);
+    if (ks == 0) partial[wave * kRowsPerWg + col] = acc;
+    __syncthreads();
+    if (tid < kRowsPerWg) {
+        float total = 0.0f;
+        for (int v = 0; v < waves; ++v) total += partial[v * kRowsPerWg + tid];
+        const int out_row = blockIdx.x * kRowsPerWg + tid;
+        if (out_row < n) store_any(y, y_dtype, static_cast<size_t>(blockIdx.y) * n + out_row, total);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
 template <typename KERN>
 int launch_kernel(KERN kern, const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype,
                   int rows, int n, int bpr, int waves, int rows_per_wg, hipStream_t stream) {
@@ -238,6 +420,24 @@ int launch_kernel(KERN kern, const ActRows& act, const WeightRoute& route, const
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 
+template <typename KERN>
+int launch_wave_kernel(KERN kern, const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype,
+                       int rows, int n, int bpr, int waves, hipStream_t stream) {
+    const size_t smem = static_cast<size_t>(waves) * (kSlotBytes + 16) + static_cast<size_t>(waves) * kRowsPerWg * sizeof(float);
+    int tallest = n;
+    for (int m = 0; m < route.extra; ++m) tallest = tallest > route.more_n[m] ? tallest : route.more_n[m];
+    dim3 grid((tallest + kRowsPerWg - 1) / kRowsPerWg, rows, 1 + route.extra);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * waves), smem, stream, act.x, act.x_dtype, act.k, route, w, y, y_dtype, n, bpr);
+    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+}
+
+// float32 activation quads take twice the registers: one block less in flight keeps four waves per SIMD
+template <typename FMT>
+constexpr int wave_depth(int iters, bool x16) {
+    const int cap = FMT::kDepth - (x16 ? 0 : 1);
+    return iters < cap ? iters : cap;
+}
+
 // waves per workgroup and blocks in flight per wave for a row of bpr super-blocks
 void split_blocks(int bpr, int work_items, int& waves, int& iters) {
     waves = 1;
@@ -250,8 +450,27 @@ void split_blocks(int bpr, int work_items, int& waves, int& iters) {
     if (iters == 7) iters = 8;
 }
 
+// the single-launch form: raw rows, no normalisation, no routing
+template <typename FMT>
+int launch_wave(const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream) {
+    int waves, iters;
+    int tiles = (n + kRowsPerWg - 1) / kRowsPerWg;
+    for (int m = 0; m < route.extra; ++m) tiles += (route.more_n[m] + kRowsPerWg - 1) / kRowsPerWg;
+    split_blocks(bpr, tiles * rows, waves, iters);
+#define PLLM_CASE(I) case I: \
+        return act.x_dtype == PLLM_F32 ? launch_wave_kernel(wave_image_matvec_kernel<FMT, I, wave_depth<FMT>(I, false), false>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream) \
+                                       : launch_wave_kernel(wave_image_matvec_kernel<FMT, I, wave_depth<FMT>(I, true), true>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream)
+    switch (iters) {
+        PLLM_CASE(1); PLLM_CASE(2); PLLM_CASE(3); PLLM_CASE(4); PLLM_CASE(5); PLLM_CASE(6);
+        default: PLLM_CASE(8);
+    }
+#undef PLLM_CASE
+}
+
 template <typename FMT, int R>
 int launch_k45_rows(const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream) {
+    if constexpr (R == 1)
+        if (act.x && act.k >= 4 && !act.gamma && !route.expert && !act.row_token) return launch_wave<FMT>(act, route, w, y, y_dtype, rows, n, bpr, stream);
     int waves, iters;
     int tiles = (n + kRowsPerWg - 1) / kRowsPerWg;
     for (int m = 0; m < route.extra; ++m) tiles += (route.more_n[m] + kRowsPerWg - 1) / kRowsPerWg;

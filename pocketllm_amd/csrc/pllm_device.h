@@ -116,11 +116,19 @@ __device__ __forceinline__ StagedX carve_staged_x(const unsigned char* base, int
 // Quantize four activations of one lane; the eight lanes of an aligned group share a 32-block.
 // First term: q = rint(fl(v / scale)) with scale = fl(amax / 127), the correctly rounded float32 quotient rounded to the nearest
 // even integer, which is the reference's 32-value activation quantizer (src/csrc/cuda_kernel_impl.cu:7102-7116) bit for bit;
-// |v / scale| <= 127 * (1 + 2^-23), so the clamp of the reference never acts.  The rounding and the int8 cast ride on one
-// addition: for |t| < 2^22 the float t + 1.5 * 2^23 has round-to-nearest-even(t) in its low mantissa bits, two's complement
-// included, so its low byte is the code and (sum - 1.5 * 2^23) the rounded value.  Second term: the residual v - q * scale in
-// units of scale / 254; its reciprocal comes from v_rcp_f32 (it only steers the rounding, the image carries `scale`), and
-// |r * inv * 254| <= 127.01 by construction, so it needs no clamp either.  An all-zero group stores scale 0 and codes 0.
+// |v / scale| <= 127 * (1 + 2^-23), so the clamp of the reference never acts.  Second term: the residual v - q * scale in
+// units of scale / 254 (|r / scale * 254| <= 127.01 by construction, no clamp either).  An all-zero group stores scale 0, codes 0.
+//
+// How the quotients stay exact without four IEEE divisions per lane:
+//   * scale: q0 = amax * c, scale = fma(fma(-q0, 127, amax), c, q0) with c = fl(1 / 127) is the correctly rounded amax / 127
+//     for every finite float32 (checked exhaustively on the host, tests/test_quantizer_identities.py).
+//   * codes: q = rint(v * y) with y ~= 1 / scale from v_rcp_f32 can differ from rint(fl(v / scale)) only when v / scale lies
+//     within 127 * 2^-21 of a rounding tie.  The residual r = fma(-q, scale, v), which the second term needs anyway, shows it:
+//     |r| < scale * (0.5 - 1e-4) proves q right whatever y was.  If any lane of the wave fails that test (about one
+//     32-block in a hundred), or amax is so small that the products above could leave the normal range, the whole wave
+//     redoes its four codes with true divisions.
+// The rounding and the int8 cast ride on one addition: for |t| < 2^22 the float t + 1.5 * 2^23 has round-to-nearest-even(t)
+// in its low mantissa bits, two's complement included, so its low byte is the code and (sum - 1.5 * 2^23) the rounded value.
 __device__ __forceinline__ uint32_t pack_low_bytes(uint32_t b0, uint32_t b1, uint32_t b2, uint32_t b3) {
     const uint32_t lo = __builtin_amdgcn_perm(b1, b0, 0x0c0c0400u);
     const uint32_t hi = __builtin_amdgcn_perm(b3, b2, 0x0c0c0400u);
@@ -128,18 +136,37 @@ __device__ __forceinline__ uint32_t pack_low_bytes(uint32_t b0, uint32_t b1, uin
 }
 __device__ __forceinline__ void quantize4(const float v[4], uint32_t& hi, uint32_t& lo, float& scale) {
     constexpr float kRound = 12582912.0f;                       // 1.5 * 2^23
+    constexpr float kInv127 = 1.0f / 127.0f;
     float am = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
     am = group_max<8>(am);
-    scale = am / 127.0f;
-    const float divisor = am > 0.0f ? scale : 1.0f;
+    const float s0 = am * kInv127;
+    scale = __builtin_fmaf(__builtin_fmaf(-s0, 127.0f, am), kInv127, s0);
+    const bool normal = am > 1e-30f && am < 1e30f;
+    const float y = normal ? __builtin_amdgcn_rcpf(scale) : 0.0f;
+    const float thr = scale * (0.5f - 1e-4f);
+    float qm[4], r[4];
+    bool sure = normal;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        qm[i] = __builtin_fmaf(v[i], y, kRound);
+        r[i] = __builtin_fmaf(kRound - qm[i], scale, v[i]);     // v - q * scale
+        sure = sure && fabsf(r[i]) < thr;
+    }
+    if (__builtin_amdgcn_ballot_w64(am > 0.0f && !sure) != 0) {  // wave-uniform: a quotient next to a rounding tie, or an extreme amax
+        scale = am / 127.0f;
+        const float divisor = am > 0.0f ? scale : 1.0f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            qm[i] = v[i] / divisor + kRound;
+            r[i] = __builtin_fmaf(kRound - qm[i], scale, v[i]);
+        }
+    }
     const float inv_lo = am > 0.0f ? (127.0f * 254.0f) * __builtin_amdgcn_rcpf(am) : 0.0f;
     uint32_t qb[4], lb[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const float qm = v[i] / divisor + kRound;
-        const float r = fmaf(kRound - qm, scale, v[i]);         // v - q * scale
-        qb[i] = __float_as_uint(qm);
-        lb[i] = __float_as_uint(fmaf(r, inv_lo, kRound));
+        qb[i] = __float_as_uint(qm[i]);
+        lb[i] = __float_as_uint(__builtin_fmaf(r[i], inv_lo, kRound));
     }
     hi = pack_low_bytes(qb[0], qb[1], qb[2], qb[3]);
     lo = pack_low_bytes(lb[0], lb[1], lb[2], lb[3]);
