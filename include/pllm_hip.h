@@ -88,6 +88,20 @@ int pllm_gguf_quant_gemm(const void* x, int x_dtype, const uint8_t* blocks, int 
 size_t pllm_gguf_quant_gemm_workspace_bytes(int type_id, int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row);
 
 /*
+ * pllm_gguf_quant_gemm for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): same arguments without the workspace, same results bit for bit.  It has no counterpart in
+ * the reference, whose operators allocate their temporaries through the framework on every call.  The activation image / the
+ * tile kernel's staging lives in a device array of PLLM_STATIC_SCRATCH_BYTES that the library holds on every GPU it runs on
+ * until the process ends; the call itself calls no hipMalloc, hipFree or other allocating routine.
+ *   - calls whose pllm_gguf_quant_gemm_workspace_bytes(...) exceeds PLLM_STATIC_SCRATCH_BYTES return PLLM_ERR_WORKSPACE;
+ *   - every call on one GPU shares that GPU's array: calls that overlap on one GPU (two streams, two threads) race;
+ *   - the first call on a device looks the array's address up (hipGetSymbolAddress): make it outside graph capture.
+ */
+#define PLLM_STATIC_SCRATCH_BYTES (16u << 20)
+int pllm_gguf_quant_gemm_static_scratch(const void* x, int x_dtype, const uint8_t* blocks, int type_id, void* y, int y_dtype,
+                                        int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row, void* stream);
+
+/*
  * The residual form of pllm_gguf_quant_gemm: y[t, r] += sum_c x[t, c] * W[r, c], the sum formed in float32 and rounded to y's
  * type once.  Replaces the matmul followed by the separate addition of the transformer block's residual connection
  * (src/models/minimax_m2/architecture.py:412-413, `x = x + ...` after the output and expert projections) for decode calls.

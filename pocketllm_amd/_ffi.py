@@ -8,6 +8,7 @@ LIB_PATH = Path(__file__).resolve().parent / "libpllm_hip.so"
 
 PLLM_OK = 0
 PLLM_ERR_UNSUPPORTED = -2        # include/pllm_hip.h: type id or shape outside what the kernels implement
+PLLM_ERR_WORKSPACE = -4          # the caller's workspace (or the library's static array) is too small
 DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
 TYPE_Q8_0 = 100
 
@@ -27,6 +28,7 @@ SIGNATURES = {
     "pllm_gguf_quant_gemm_multi": (_int, [_c_void_p, _int, _c_void_p, ctypes.c_float, _int, _int, _c_void_p, _c_void_p, _int, _c_void_p, _int,
                                           _i64, _i64, _i64, _c_void_p, _size_t, _c_void_p]),
     "pllm_gguf_quant_gemm_accumulate": (_int, [_c_void_p, _int, _c_void_p, _int, _c_void_p, _int, _i64, _i64, _i64, _i64, _c_void_p, _size_t, _c_void_p]),
+    "pllm_gguf_quant_gemm_static_scratch": (_int, [_c_void_p, _int, _c_void_p, _int, _c_void_p, _int, _i64, _i64, _i64, _i64, _c_void_p]),
     "pllm_gguf_quant_gemm_workspace_bytes": (_size_t, [_int, _i64, _i64, _i64, _i64]),
     "pllm_activation_image_bytes": (_size_t, [_i64, _i64]),
     "pllm_quantize_activations": (_int, [_c_void_p, _int, _i64, _i64, _i64, _c_void_p, _size_t, _c_void_p]),

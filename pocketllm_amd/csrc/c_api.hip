@@ -1,4 +1,6 @@
 // extern "C" surface of libpllm_hip: argument validation and dispatch by type and shape.
+#include <mutex>
+
 #include "pllm_internal.h"
 
 namespace {
@@ -189,6 +191,45 @@ size_t pllm_gguf_quant_gemm_workspace_bytes(int type_id, int64_t rows, int64_t k
     if (gguf_uses_tile_gemm(type_id, rows, n, blocks_per_row))
         return pllm::gemm_f16_workspace_bytes(static_cast<int>(rows), static_cast<int>(n), static_cast<int>(blocks_per_row));
     return pllm::act_image_256_bytes(static_cast<int>(blocks_per_row)) * static_cast<size_t>(rows);
+}
+
+// ---- the entry point that allocates nothing ---------------------------------------------------------------------------
+// Device memory for the activation image / the tile kernel's staging lives in a file-scope array instead of a caller's
+// workspace.  Every GPU the library runs on holds its own copy of the array at its own address; the address is looked up once
+// per device (hipGetSymbolAddress, with that device current) and kept.  Host code never passes the array's name to a kernel.
+static __device__ __align__(256) unsigned char scratch[PLLM_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex scratch_mutex;
+void* scratch_address[kMaxDevices];
+
+int static_scratch(void** out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return PLLM_ERR_LAUNCH;
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (!scratch_address[dev]) {
+        void* ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return PLLM_ERR_LAUNCH;
+        scratch_address[dev] = ptr;
+    }
+    *out = scratch_address[dev];
+    return PLLM_OK;
+}
+}  // namespace
+
+int pllm_gguf_quant_gemm_static_scratch(const void* x, int x_dtype, const uint8_t* blocks, int type_id, void* y, int y_dtype,
+                                        int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row, void* stream) {
+    if (!fits_int(rows) || !fits_int(k) || !fits_int(n) || !fits_int(blocks_per_row)) return PLLM_ERR_INVALID_ARGUMENT;
+    if (pllm_gguf_block_bytes(type_id) == 0) return PLLM_ERR_UNSUPPORTED;
+    // sizes beyond the array are refused: "workspace too small" names the limit that was hit
+    if (pllm_gguf_quant_gemm_workspace_bytes(type_id, rows, k, n, blocks_per_row) > PLLM_STATIC_SCRATCH_BYTES) return PLLM_ERR_WORKSPACE;
+    void* ptr = nullptr;
+    const int st = static_scratch(&ptr);
+    if (st != PLLM_OK) return st;
+    // every kernel behind pllm_gguf_quant_gemm writes what it later reads of the workspace (image, staged rows, partial tiles)
+    // within the same call, so nothing has to be cleared between calls
+    return pllm_gguf_quant_gemm(x, x_dtype, blocks, type_id, y, y_dtype, rows, k, n, blocks_per_row, ptr, PLLM_STATIC_SCRATCH_BYTES, stream);
 }
 
 int pllm_fused_rms_norm(const void* x, int x_dtype, const float* weight, void* y, int y_dtype, int64_t rows, int64_t dim, float eps, void* stream) {

@@ -145,6 +145,29 @@ def _dense_gemm(name, x, blocks, row_elems, type_id, signed_grid, out_dtype):
     return y
 
 
+STATIC_SCRATCH_BYTES = 16 << 20
+
+
+def gguf_quant_gemm_static_scratch_forward(x, blocks, row_elems, type_id, signed_grid, y: torch.Tensor) -> torch.Tensor:
+    """gguf_quant_gemm_forward / gguf_quant_gemm_prefill_forward into a caller-owned y, through the entry point that allocates no
+    device memory (pllm_gguf_quant_gemm_static_scratch: its activation image and staging live in a 16 MiB array the library
+    holds on the device).  For callers that cannot allocate: code under graph capture, tight serving loops.  Raises RuntimeError
+    ("workspace too small") for calls that need more than the array; calls that overlap on one GPU race."""
+    row_elems, type_id = int(row_elems), int(type_id)
+    _dense_checks(x, blocks, row_elems, type_id, signed_grid)
+    rows = x.numel() // row_elems
+    n = blocks.size(0)
+    _check(y.is_cuda and y.device == x.device and y.is_contiguous() and y.dtype in _DTYPE_CODE, "y must be a contiguous CUDA tensor of float16, bfloat16 or float32")
+    _check(tuple(y.shape) == (*x.shape[:-1], n), "y must have x's leading shape and blocks.size(0) columns")
+    if rows == 0 or n == 0:
+        return y
+    with _on_device(x.device):
+        st = _lib().pllm_gguf_quant_gemm_static_scratch(x.data_ptr(), _DTYPE_CODE[x.dtype], blocks.data_ptr(), type_id, y.data_ptr(),
+                                                        _DTYPE_CODE[y.dtype], rows, row_elems, n, blocks.size(1), _stream(x.device))
+    _ffi.check(st, "gguf_quant_gemm_static_scratch_forward")
+    return y
+
+
 def gguf_quant_gemm_forward(x, blocks, row_elems, type_id, signed_grid, *, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
     """Decode-regime operator, src/csrc/cuda_kernel.cpp:566-589.  Any row count is accepted."""
     return _dense_gemm("gguf_quant_gemm_forward", x, blocks, row_elems, type_id, signed_grid, out_dtype)
