@@ -88,6 +88,21 @@ int pllm_gguf_quant_gemm(const void* x, int x_dtype, const uint8_t* blocks, int 
 size_t pllm_gguf_quant_gemm_workspace_bytes(int type_id, int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row);
 
 /*
+ * Q4_K / Q5_K matmul with the int8 activation semantics of the reference's MMA prefill path: activations quantized to 32-value
+ * int8 blocks (xs = amax / 127, code = rint(x / xs)), integer dots per 32-weight group on the int8 matrix cores,
+ *   y[t, r] = sum_g xs[t, g] * (d_r sc_{r,g} * dot_g - dmin_r m_{r,g} * sum of the group's activation codes),
+ * d * sc and dmin * m in float32.  Any row count; built for prefill row counts.  Other type ids return PLLM_ERR_UNSUPPORTED.
+ * Replaces the MMA branch of gguf_quant_gemm_prefill_forward (src/csrc/llama_mmq/gguf_mma_wrapper.cu:257-322,
+ * src/csrc/llama_mmq/mmq.cuh:1329-1455, 2083-2200; activation quantizer src/csrc/cuda_kernel_impl.cu:7090-7117).
+ * pllm_gguf_quant_gemm keeps float-activation semantics (fp16 tiles); this entry point is the reference's other statement of
+ * the operator.
+ */
+int pllm_gguf_quant_gemm_q8(const void* x, int x_dtype, const uint8_t* blocks, int type_id, void* y, int y_dtype,
+                            int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row,
+                            void* workspace, size_t workspace_bytes, void* stream);
+size_t pllm_gguf_quant_gemm_q8_workspace_bytes(int type_id, int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row);
+
+/*
  * pllm_gguf_quant_gemm for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc): same arguments without the workspace, same results bit for bit.  It has no counterpart in
  * the reference, whose operators allocate their temporaries through the framework on every call.  The activation image / the

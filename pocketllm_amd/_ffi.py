@@ -28,6 +28,8 @@ SIGNATURES = {
     "pllm_gguf_quant_gemm_multi": (_int, [_c_void_p, _int, _c_void_p, ctypes.c_float, _int, _int, _c_void_p, _c_void_p, _int, _c_void_p, _int,
                                           _i64, _i64, _i64, _c_void_p, _size_t, _c_void_p]),
     "pllm_gguf_quant_gemm_accumulate": (_int, [_c_void_p, _int, _c_void_p, _int, _c_void_p, _int, _i64, _i64, _i64, _i64, _c_void_p, _size_t, _c_void_p]),
+    "pllm_gguf_quant_gemm_q8": (_int, [_c_void_p, _int, _c_void_p, _int, _c_void_p, _int, _i64, _i64, _i64, _i64, _c_void_p, _size_t, _c_void_p]),
+    "pllm_gguf_quant_gemm_q8_workspace_bytes": (_size_t, [_int, _i64, _i64, _i64, _i64]),
     "pllm_gguf_quant_gemm_static_scratch": (_int, [_c_void_p, _int, _c_void_p, _int, _c_void_p, _int, _i64, _i64, _i64, _i64, _c_void_p]),
     "pllm_gguf_quant_gemm_workspace_bytes": (_size_t, [_int, _i64, _i64, _i64, _i64]),
     "pllm_activation_image_bytes": (_size_t, [_i64, _i64]),

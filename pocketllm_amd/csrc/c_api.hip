@@ -193,6 +193,24 @@ size_t pllm_gguf_quant_gemm_workspace_bytes(int type_id, int64_t rows, int64_t k
     return pllm::act_image_256_bytes(static_cast<int>(blocks_per_row)) * static_cast<size_t>(rows);
 }
 
+// Q4_K / Q5_K with int8 activation semantics (activations quantized to 32-value int8 blocks, integer dots on the matrix cores)
+size_t pllm_gguf_quant_gemm_q8_workspace_bytes(int type_id, int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row) {
+    (void)k; (void)n;
+    if (!fits_int(rows) || !fits_int(blocks_per_row) || !pllm::gemm_i8_supports(type_id)) return 0;
+    return pllm::gemm_i8_workspace_bytes(static_cast<int>(rows), static_cast<int>(blocks_per_row));
+}
+
+int pllm_gguf_quant_gemm_q8(const void* x, int x_dtype, const uint8_t* blocks, int type_id, void* y, int y_dtype,
+                            int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row,
+                            void* workspace, size_t workspace_bytes, void* stream) {
+    if (!x || !blocks || !y || !dtype_ok(x_dtype) || !dtype_ok(y_dtype)) return PLLM_ERR_INVALID_ARGUMENT;
+    if (!fits_int(rows) || !fits_int(k) || !fits_int(n) || !fits_int(blocks_per_row) || rows <= 0 || n <= 0 || k <= 0) return PLLM_ERR_INVALID_ARGUMENT;
+    if (blocks_per_row * 256 < k) return PLLM_ERR_INVALID_ARGUMENT;
+    if (!pllm::gemm_i8_supports(type_id)) return PLLM_ERR_UNSUPPORTED;
+    return pllm::gemm_i8(x, x_dtype, blocks, type_id, y, y_dtype, static_cast<int>(rows), static_cast<int>(k), static_cast<int>(n),
+                         static_cast<int>(blocks_per_row), workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
 // ---- the entry point that allocates nothing ---------------------------------------------------------------------------
 // Device memory for the activation image / the tile kernel's staging lives in a file-scope array instead of a caller's
 // workspace.  Every GPU the library runs on holds its own copy of the array at its own address; the address is looked up once

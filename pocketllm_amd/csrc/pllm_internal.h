@@ -113,6 +113,11 @@ int gemm_f16_stage_swiglu(const float* g, const float* u, const float* route_wei
                           hipStream_t stream);
 int gemm_f16_grouped(const void* staged, const uint8_t* w, int type_id, size_t group_stride, const int32_t* seg, int groups,
                      float* y, int rows, int max_group_rows, int n, int bpr, hipStream_t stream);
+// prefill matmul of Q4_K / Q5_K on the int8 matrix cores, activations quantized to 32-value int8 blocks (gemm_i8.hip)
+bool gemm_i8_supports(int type_id);
+size_t gemm_i8_workspace_bytes(int rows, int bpr);
+int gemm_i8(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y, int y_dtype,
+            int rows, int k, int n, int bpr, void* workspace, size_t workspace_bytes, hipStream_t stream);
 // FP8 x FP8 block-scaled matmul on the native FP8 matrix path (gemm_fp8.hip); k a multiple of 128
 int fp8_gemm_native(const uint8_t* a, const float* a_s, const uint8_t* b, const float* b_s, void* y, int y_dtype,
                     int rows, int k, int n, hipStream_t stream);

@@ -145,6 +145,28 @@ def _dense_gemm(name, x, blocks, row_elems, type_id, signed_grid, out_dtype):
     return y
 
 
+def gguf_quant_gemm_q8_forward(x, blocks, row_elems, type_id, signed_grid, *, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """Q4_K / Q5_K matmul with the int8 activation semantics of the reference's MMA prefill path
+    (src/csrc/llama_mmq/gguf_mma_wrapper.cu:257-322): activations quantized to 32-value int8 blocks, integer group dots on the
+    int8 matrix cores, float32 scales.  gguf_quant_gemm_prefill_forward states the same operator with float activations."""
+    row_elems, type_id = int(row_elems), int(type_id)
+    _dense_checks(x, blocks, row_elems, type_id, signed_grid)
+    _check(type_id in (3, 4), "int8-activation matmul serves q4_k and q5_k")
+    rows = x.numel() // row_elems
+    n = blocks.size(0)
+    y = torch.empty(*x.shape[:-1], n, dtype=out_dtype, device=x.device)
+    if rows == 0 or n == 0:
+        return y
+    lib = _lib()
+    with _on_device(x.device):
+        ws_bytes = lib.pllm_gguf_quant_gemm_q8_workspace_bytes(type_id, rows, row_elems, n, blocks.size(1))
+        ws = _workspace(ws_bytes, x.device)
+        st = lib.pllm_gguf_quant_gemm_q8(x.data_ptr(), _DTYPE_CODE[x.dtype], blocks.data_ptr(), type_id, y.data_ptr(), _DTYPE_CODE[out_dtype],
+                                         rows, row_elems, n, blocks.size(1), ws.data_ptr(), ws_bytes, _stream(x.device))
+    _ffi.check(st, "gguf_quant_gemm_q8_forward")
+    return y
+
+
 STATIC_SCRATCH_BYTES = 16 << 20
 
 

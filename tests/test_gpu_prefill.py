@@ -256,3 +256,55 @@ def test_fp8_gemm_native_baseline_shape_sampled(mod):
     xa = O.fp8_e4m3_decode(xa_codes).reshape(t, k // 128, 128) * xs[..., None]
     want = O.matmul_f(xa.reshape(t, k), O.dequant_fp8_block(codes, scale)[cols])
     assert O.rel_l2(y.cpu().numpy()[:, cols], want) <= 2e-4
+
+
+# ---- Q4_K / Q5_K on the int8 matrix cores: int8 activation semantics ------------------------------------
+
+@pytest.mark.parametrize("type_name", ["q4_k", "q5_k"])
+@pytest.mark.parametrize("t,n,k", [(16, 128, 256), (64, 300, 768), (130, 129, 1000), (257, 64, 2048), (1, 40, 512), (700, 200, 512)])
+def test_int8_prefill_matches_the_int8_activation_oracle(mod, type_name, t, n, k):
+    """pllm_gguf_quant_gemm_q8 against oracle.kquant_gemm_q (activations quantized per 32 values, integer group dots, float32
+    scales): the integer part is exact, so the two differ by the order of the float32 sums only.  The distance to the
+    float-activation oracle is the quantization error of the activations (about 5e-3) and is reported, not bounded tightly."""
+    rng = np.random.default_rng(t + n + k)
+    kp = (k + 255) // 256 * 256
+    w = np.zeros((n, kp), dtype=np.float32)
+    w[:, :k] = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
+    blocks = ENC[type_name](w)
+    x_np = rng.standard_normal((t, k)).astype(np.float32)
+    if t > 5:
+        x_np[3] *= 1e4
+        x_np[5] *= 1e-6
+        x_np[2, 64:96] = 0.0                                   # an all-zero activation group
+    grid = torch.empty(0, dtype=torch.int8, device=DEV)
+    for dt in (torch.bfloat16, torch.float32):
+        x = torch.from_numpy(x_np).to(DEV).to(dt)
+        print(f"case int8 prefill {type_name} t={t} n={n} k={k} {dt}", flush=True)
+        y = mod.gguf_quant_gemm_q8_forward(x, torch.from_numpy(blocks).to(DEV), k, O.TYPE_IDS[type_name], grid, out_dtype=torch.float32)
+        torch.cuda.synchronize()
+        xp = np.zeros((t, kp), dtype=np.float32)
+        xp[:, :k] = x.float().cpu().numpy()
+        want = O.kquant_gemm_q(xp, blocks, type_name)
+        got = y.cpu().numpy()
+        row_err = np.sqrt(((got - want) ** 2).sum(axis=1) / np.maximum((want ** 2).sum(axis=1), 1e-300))
+        assert row_err.max() <= 2e-5, (dt, row_err.argmax(), row_err.max())
+        far = O.rel_l2(got, O.matmul_f(xp, O.dequant_rows(blocks, type_name, kp)))
+        assert far <= 2e-2, far
+
+
+@pytest.mark.parametrize("type_name,n", [("q4_k", 5120), ("q5_k", 17408)])
+def test_int8_prefill_baseline_shapes_sampled(mod, type_name, n):
+    """BASELINE config 3 with its own semantics (int8 activation blocks): T = 64 and 2048, 48 sampled columns against the int8 oracle."""
+    rng = np.random.default_rng(1013 + n)
+    k = 5120
+    blocks = ENC[type_name]((rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02)))
+    dblocks = torch.from_numpy(blocks).to(DEV)
+    grid = torch.empty(0, dtype=torch.int8, device=DEV)
+    cols = rng.choice(n, size=48, replace=False)
+    for t in (64, 2048):
+        x = torch.from_numpy(rng.standard_normal((t, k)).astype(np.float32)).to(DEV).to(torch.bfloat16)
+        print(f"case int8 prefill baseline {type_name} n={n} t={t}", flush=True)
+        y = mod.gguf_quant_gemm_q8_forward(x, dblocks, k, O.TYPE_IDS[type_name], grid, out_dtype=torch.float32)
+        torch.cuda.synchronize()
+        want = O.kquant_gemm_q(x.float().cpu().numpy(), blocks[cols], type_name)
+        assert O.rel_l2(y.cpu().numpy()[:, cols], want) <= 2e-5
