@@ -342,7 +342,12 @@ def extra_cases(mod, dev):
     out.append({"case": "decoder layer matmul path, MiniMax-M2 shapes, T=1 (norm + q/k/v projections in one launch, output projection + residual, norm, routing, experts)",
                 "weight_bytes": int(layer_bytes), "us_per_call": round(us, 3), "gbs": round(layer_bytes / us / 1e3, 1),
                 "frac_hbm_peak": round(layer_bytes / us / 1e3 / HBM_PEAK_GBS, 4), "graph": graphed,
-                "note": "7 launches; the experts and the routing gate stay cache-resident between replays (same routes every replay)"})
+                "note": "7 launches; the experts and the routing gate stay cache-resident between replays (same routes every replay)",
+                "decode_tps_62_layers": round(1e6 / (62 * us), 2)})
+    # the reference reports generation speed in this form (src/runtime/generation.py:262-268); one token through 62 such layers
+    # (MiniMax-M2's depth), attention core and logits not included
+    print(f"RESULT prefill_seconds=0.000000 prefill_tokens=0 prefill_tps=0.00 decode_seconds={62 * us * 1e-6:.6f} decode_tokens=1 "
+          f"decode_tps={1e6 / (62 * us):.2f}", file=sys.stderr)
     del w1, w3, w2, wq, wk, wv, wo
     # one dense feed-forward block at T=1, hidden 5120, intermediate 17408, Q4_K: y += W_down (SiLU(W_gate n(x)) * W_up n(x)), as three
     # launches (norm + gate/up in one, SiLU * up into the activation image, down projection with the residual in its store) and as the

@@ -1,0 +1,104 @@
+"""One MiniMax-M2 decoder block composed from the raw-block operators (pocketllm_amd/minimax_block.py) against the oracle chain
+rms_norm -> projections -> attention -> residual -> rms_norm -> route_topk -> moe_forward -> residual, all in float64.
+The block rounds to fp16 between operators as the reference's does (src/models/minimax_m2/architecture.py:409-413), so the
+composed bound is that of fp16 storage, not of the kernels (those are checked on their own at 1e-3)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import gguf_oracle as O
+from pocketllm_amd import block_codec as C
+from pocketllm_amd.cuda_loader import load_cuda_kernel
+from pocketllm_amd.minimax_block import ExpertLayer, MiniMaxAttention, MiniMaxBlock, MiniMaxM2Args, MiniMaxMoE, RMSNorm
+from pocketllm_amd.quantized_ops import QuantizedGGUFLinear
+from pocketllm_amd.quantized_tensor import QuantizedGGUFTensor
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _rope(x, start, rope_dim, base):
+    half = rope_dim // 2
+    pos = np.arange(start, start + x.shape[0], dtype=np.float64)
+    inv = base ** (-(2.0 * np.arange(half)) / rope_dim)
+    f = pos[:, None] * inv[None, :]
+    s, c = np.sin(f)[:, None, :], np.cos(f)[:, None, :]
+    x1, x2 = x[..., :half], x[..., half:rope_dim]
+    return np.concatenate([x1 * c - x2 * s, x1 * s + x2 * c, x[..., rope_dim:]], axis=-1)
+
+
+class _OracleBlock:
+    def __init__(self, a, w, gate, bias, experts, norms):
+        self.a, self.w, self.gate, self.bias, self.experts, self.norms = a, w, gate, bias, experts, norms
+        self.k = np.zeros((0, a.n_kv_heads, a.head_dim))
+        self.v = np.zeros((0, a.n_kv_heads, a.head_dim))
+
+    def __call__(self, x, start):
+        a = self.a
+        h = O.rms_norm(x, self.norms["attn"], a.norm_eps)
+        q = O.rms_norm(h @ self.w["q"].T, self.norms["q"], a.norm_eps).reshape(-1, a.n_heads, a.head_dim)
+        k = O.rms_norm(h @ self.w["k"].T, self.norms["k"], a.norm_eps).reshape(-1, a.n_kv_heads, a.head_dim)
+        v = (h @ self.w["v"].T).reshape(-1, a.n_kv_heads, a.head_dim)
+        q, k = _rope(q, start, a.rope_dim, a.rope_base), _rope(k, start, a.rope_dim, a.rope_base)
+        self.k, self.v = np.concatenate([self.k[:start], k]), np.concatenate([self.v[:start], v])
+        rep = a.n_heads // a.n_kv_heads
+        out = np.zeros((x.shape[0], a.n_heads, a.head_dim))
+        for t in range(x.shape[0]):
+            for hh in range(a.n_heads):
+                kk, vv = self.k[:start + t + 1, hh // rep], self.v[:start + t + 1, hh // rep]
+                s = kk @ q[t, hh] / np.sqrt(a.head_dim)
+                p = np.exp(s - s.max())
+                out[t, hh] = (p / p.sum()) @ vv
+        x1 = x + out.reshape(x.shape[0], -1) @ self.w["o"].T
+        h2 = O.rms_norm(x1, self.norms["ffn"], a.norm_eps)
+        idx, wts = O.route_topk(h2 @ self.gate.T, self.bias, a.top_k)
+        w1, w3, w2 = self.experts
+        rt = np.repeat(np.arange(x.shape[0]), a.top_k)
+        y = O.moe_forward(h2, rt, wts.reshape(-1), idx.reshape(-1), w1, w3, w2, "iq2_xxs", "iq2_xxs", "iq1_m", 0.0)
+        return x1 + y
+
+
+def test_decoder_block_prefill_then_decode():
+    assert load_cuda_kernel() is not None and torch.cuda.is_available()
+    rng = np.random.default_rng(21)
+    a = MiniMaxM2Args(dim=512, n_heads=4, n_kv_heads=2, head_dim=64, rope_dim=32, rope_base=10000.0, n_routed_experts=8, top_k=2,
+                      moe_inter_dim=256, norm_eps=1e-6)
+    shapes = {"q": (a.n_heads * a.head_dim, a.dim), "k": (a.n_kv_heads * a.head_dim, a.dim), "v": (a.n_kv_heads * a.head_dim, a.dim),
+              "o": (a.dim, a.n_heads * a.head_dim)}
+    blocks = {n: C.quantize_q5_k((rng.standard_normal(s) * (0.7 / np.sqrt(s[1]))).astype(np.float32)) for n, s in shapes.items()}
+    lin = {n: QuantizedGGUFLinear(QuantizedGGUFTensor.from_blocks(torch.from_numpy(b).to(DEV), "q5_k", shapes[n][1], source_name=n))
+           for n, b in blocks.items()}
+    norms = {"attn": rng.uniform(0.5, 1.5, a.dim), "ffn": rng.uniform(0.5, 1.5, a.dim), "q": rng.uniform(0.5, 1.5, shapes["q"][0]),
+             "k": rng.uniform(0.5, 1.5, shapes["k"][0])}
+    norms = {n: v.astype(np.float32) for n, v in norms.items()}
+    tn = {n: torch.from_numpy(v).to(DEV) for n, v in norms.items()}
+    gate = (rng.standard_normal((a.n_routed_experts, a.dim)) / np.sqrt(a.dim)).astype(np.float32)
+    bias = (rng.standard_normal(a.n_routed_experts) * 0.1).astype(np.float32)
+    w1 = C.random_iq2_xxs(rng, a.n_routed_experts, a.moe_inter_dim, a.dim // 256, d_range=(0.002, 0.006))
+    w3 = C.random_iq2_xxs(rng, a.n_routed_experts, a.moe_inter_dim, a.dim // 256, d_range=(0.002, 0.006))
+    w2 = C.random_iq1_m(rng, a.n_routed_experts, a.dim, a.moe_inter_dim // 256, d_range=(0.002, 0.006))
+    experts = ExpertLayer(*(QuantizedGGUFTensor.from_blocks(torch.from_numpy(b).to(DEV), name, k)
+                            for b, name, k in ((w1, "iq2_xxs", a.dim), (w3, "iq2_xxs", a.dim), (w2, "iq1_m", a.moe_inter_dim))))
+    moe = MiniMaxMoE(a, torch.from_numpy(gate).to(DEV), torch.from_numpy(bias).to(DEV), experts)
+    attn = MiniMaxAttention(a, lin["q"], lin["k"], lin["v"], lin["o"], RMSNorm(tn["q"], a.norm_eps), RMSNorm(tn["k"], a.norm_eps))
+    block = MiniMaxBlock(a, tn["attn"], tn["ffn"], attn, moe)
+    oracle = _OracleBlock(a, {n: O.dequant_rows(b, "q5_k", shapes[n][1]).astype(np.float64) for n, b in blocks.items()}, gate.astype(np.float64),
+                          bias.astype(np.float64), (w1, w3, w2), {n: v.astype(np.float64) for n, v in norms.items()})
+    block.reset_cache(1, 16)
+    # the experts alone: float32 output of the fused operators rounded once to fp16
+    x_moe = torch.from_numpy(rng.standard_normal((5, a.dim)).astype(np.float32)).to(DEV).to(torch.float16)
+    idx, wts = O.route_topk(x_moe.float().cpu().numpy().astype(np.float64) @ gate.T.astype(np.float64), bias.astype(np.float64), a.top_k)
+    want = O.moe_forward(x_moe.float().cpu().numpy(), np.repeat(np.arange(5), a.top_k), wts.reshape(-1), idx.reshape(-1), w1, w3, w2,
+                         "iq2_xxs", "iq2_xxs", "iq1_m", 0.0)
+    assert O.rel_l2(moe(x_moe).float().cpu().numpy(), want) <= 2e-3
+    assert O.rel_l2(moe(x_moe[:1]).float().cpu().numpy(), want[:1]) <= 2e-3
+    # a prefill of three tokens, then two decode steps against the same cache
+    x0 = rng.standard_normal((3, a.dim)).astype(np.float32)
+    steps = [(x0, 0), (rng.standard_normal((1, a.dim)).astype(np.float32), 3), (rng.standard_normal((1, a.dim)).astype(np.float32), 4)]
+    for x_np, start in steps:
+        x = torch.from_numpy(x_np).to(DEV).to(torch.float16)
+        print(f"case decoder block tokens={x_np.shape[0]} start={start}", flush=True)
+        got = block(x.view(1, -1, a.dim), start).float().cpu().numpy()[0]
+        want = oracle(x.float().cpu().numpy().astype(np.float64), start)
+        assert got.shape == want.shape
+        assert O.rel_l2(got, want) <= 1e-2, (start, O.rel_l2(got, want))
