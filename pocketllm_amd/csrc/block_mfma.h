@@ -25,7 +25,8 @@ typedef __attribute__((address_space(3))) unsigned char* lds_byte_ptr;
 // between.  Issued through inline assembly so that the compiler does not put a wait for it in front
 // of every later LDS read: the kernel waits for its chunks itself (wait_vm).
 __device__ __forceinline__ void lds_dma16(const void* src, uint32_t lds_base) {
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(lds_base) : "memory", "m0");
+    // (lds_base is wave-uniform by contract; the readfirstlane only tells the compiler so)
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(__builtin_amdgcn_readfirstlane(lds_base)) : "memory", "m0");
 }
 template <int N> __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory"); }
 // until at most `newest` of this wave's memory operations are outstanding (they complete in order)

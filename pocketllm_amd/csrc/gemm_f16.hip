@@ -776,7 +776,6 @@ int launch_gemm_mi(const GemmPlan& p, const _Float16* xh, const float* xscale, c
     }
 }
 
-size_t align256(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
 
 }  // namespace
 

@@ -238,7 +238,6 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(const int8_t* __restr
     else store_all([&](size_t at, float v) { static_cast<f16_t*>(y)[at] = from_float<f16_t>(v); });
 }
 
-size_t align256(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
 
 }  // namespace
 

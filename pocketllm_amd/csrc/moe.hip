@@ -491,8 +491,6 @@ int launch_w2_grouped(const unsigned char* h_image, size_t h_stride, int bpr, co
 
 bool dot4_type(int t) { return t == PLLM_TYPE_Q2_K || t == PLLM_TYPE_IQ2_XXS || t == PLLM_TYPE_IQ1_M; }
 
-size_t align256(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
-
 }  // namespace
 }  // namespace pllm
 
@@ -503,9 +501,13 @@ size_t pllm_gguf_moe_workspace_bytes(int64_t tokens, int64_t routes, int64_t dim
     const int bpr_x = static_cast<int>((dim + 255) / 256), bpr_h = static_cast<int>((inter + 255) / 256);
     // images of the tokens and of the routes' hidden rows, per-route outputs, narrow expert ids, and (route-by-route path of the
     // types without fused expert kernels) the float32 gate and up products
-    const size_t dot_path = pllm::act_image_256_bytes(bpr_x) * static_cast<size_t>(tokens) + pllm::act_image_256_bytes(bpr_h) * static_cast<size_t>(routes) +
+    size_t dot_path = pllm::act_image_256_bytes(bpr_x) * static_cast<size_t>(tokens) + pllm::act_image_256_bytes(bpr_h) * static_cast<size_t>(routes) +
                             pllm::align256(static_cast<size_t>(routes) * dim * sizeof(float)) + pllm::align256(static_cast<size_t>(routes) * sizeof(int32_t)) +
                             2 * pllm::align256(static_cast<size_t>(routes) * inter * sizeof(float)) + 256;
+    // (the grouped path with the routes as matrix rows: half-precision activation rows and hidden rows, per-route outputs)
+    const size_t rows_path = pllm::moe_rows_x_bytes(tokens, dim) + pllm::moe_rows_h_bytes(routes, inter) +
+                             pllm::align256(static_cast<size_t>(routes) * dim * sizeof(float)) + 256;
+    if (rows_path > dot_path) dot_path = rows_path;
     if (tokens < pllm::kMoeGemmMinTokens || routes > INT32_MAX) return dot_path;
     const int R = static_cast<int>(routes);
     const size_t tile_path = pllm::gemm_f16_staged_bytes(R, bpr_x) + pllm::gemm_f16_staged_bytes(R, bpr_h) +
@@ -535,6 +537,22 @@ int pllm_gguf_moe_forward(const void* x, int x_dtype, int64_t tokens, int64_t di
     if (!workspace || workspace_bytes < pllm_gguf_moe_workspace_bytes(tokens, routes, dim, inter)) return PLLM_ERR_WORKSPACE;
 
     const int bpr_x = static_cast<int>((dim + 255) / 256), bpr_h = static_cast<int>((inter + 255) / 256);
+    if (seg_starts && tokens > 1 && routes <= kMoeGroupedMaxRoutesPerExpert * n_experts &&
+        moe_rows_supports(w13_type, w2_type, static_cast<int>(dim), static_cast<int>(inter), w1, w3, w2)) {
+        // a few routes per expert, IQ2_XXS / IQ1_M: every expert's weights are decoded once, in half precision, and multiplied with
+        // all its routes at once on the matrix cores
+        unsigned char* x_rows = static_cast<unsigned char*>(workspace);
+        unsigned char* h_rows = x_rows + moe_rows_x_bytes(tokens, dim);
+        float* part = reinterpret_cast<float*>(h_rows + moe_rows_h_bytes(routes, inter));
+        const int R = static_cast<int>(routes), E = static_cast<int>(n_experts), I = static_cast<int>(inter), D = static_cast<int>(dim);
+        int st = moe_rows_w13(x, x_dtype, static_cast<int>(tokens), D, x_rows, route_tokens, seg_starts, route_weights, w1, w3, I, swiglu_limit, h_rows, E, R, s);
+        if (st != PLLM_OK) return st;
+        st = moe_rows_w2(h_rows, I, seg_starts, w2, part, D, E, R, s);
+        if (st != PLLM_OK) return st;
+        dim3 rg(static_cast<unsigned>(tokens), static_cast<unsigned>((dim + 255) / 256));
+        hipLaunchKernelGGL(moe_reduce_kernel, rg, dim3(256), 0, s, part, route_tokens, y, R, D);
+        return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+    }
     if (seg_starts && tokens > 1 && routes <= kMoeGroupedMaxRoutesPerExpert * n_experts &&
         moe_grouped_mfma_supports(w13_type, w2_type, static_cast<int>(dim), static_cast<int>(inter), w1, w3, w2)) {
         // a few routes per expert: every expert's weights are decoded once on the matrix-core path and all its routes pass

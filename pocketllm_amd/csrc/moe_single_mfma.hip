@@ -356,6 +356,400 @@ __global__ __launch_bounds__(64 * kGroupWaves) void moe_grouped_w2_kernel(
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Grouped routes with the ROUTES as matrix rows, in half precision on the matrix cores.
+//
+// The integer weights of IQ2_XXS, magnitude (8, 25 or 43) times group scale (odd, at most 31), are
+// exact in half precision, and so is a bfloat16 / float16 activation once its row is scaled by a power
+// of two (float32 rows go in as two half-precision terms).  v_mfma_f32_16x16x32_f16 per 32-weight
+// group: A row m = route m of a batch of 16 (or route m / 2, term m % 2, of a batch of 8), B column n =
+// weight row n; lane (n, q) = (lane % 16, lane / 16) supplies the eight weights [8 q, 8 q + 8) of the
+// group (grid entry q of the sub-block) as B and the same eight positions of its image row as A, and
+// finds rows 4 q .. 4 q + 3 for weight row n in its C registers.  The matrix cores accumulate over the
+// groups of a block in float32; the block scale goes on per block.  One decode of a block serves the
+// whole batch, no integer fix-up follows the MFMA, and the lanes' A operands are the same for every
+// tile of a run: they are read from memory once per batch and kept in registers.
+//
+// Unit = (expert, run of 16-row tiles).  The tiles' weights (gate and up) arrive by direct-to-LDS
+// loads, double-buffered, one barrier per tile.  Twelve waves = (matrix, sixth of the row's blocks).
+// LDS codebooks: 256 x 8 magnitudes and 128 x 8 sign masks as half-precision vectors, kRowsCopies
+// copies of each entry side by side so that lane l reads copy l % 8: eight neighbouring lanes cover
+// all banks with their 16-byte reads whatever entries they pick.
+// ------------------------------------------------------------------------------------------------
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+
+constexpr int kRowsWaves = 12;
+constexpr int kRowsShares = kRowsWaves / 2;
+constexpr int kRowsBlocks = 2;            // blocks of a row per wave
+constexpr int kRowsCopies = 8;
+constexpr int kRowsTableBytes = (256 + 128) * 16 * kRowsCopies;
+
+// Activation rows as half-precision images: img[token][term][kpad] = x * s (zero beyond dim), s a
+// power of two that brings the row's largest magnitude into [1024, 2048); unscale[token] = 1 / s.
+// TERMS = 2 adds the rounding residual as a second row.
+template <int TERMS>
+__global__ __launch_bounds__(256) void rows_image_kernel(const void* __restrict__ x, int x_dtype, int dim, int kpad, _Float16* __restrict__ img,
+                                                         float* __restrict__ unscale) {
+    __shared__ float part[4];
+    const int token = blockIdx.x, tid = threadIdx.x;
+    const size_t base = static_cast<size_t>(token) * dim;
+    float am = 0.0f;
+    for (int k = tid; k < dim; k += 256) am = fmaxf(am, fabsf(load_any(x, x_dtype, base + k)));
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) am = fmaxf(am, __shfl_xor(am, off, 64));
+    if ((tid & 63) == 0) part[tid >> 6] = am;
+    __syncthreads();
+    am = fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3]));
+    float s = 1.0f;
+    if (am > 0.0f && am < 3.0e38f) {
+        int ex;
+        frexpf(am, &ex);                       // am = m * 2^ex, m in [0.5, 1)
+        s = ldexpf(1.0f, max(-126, min(11 - ex, 126)));
+    }
+    _Float16* row = img + static_cast<size_t>(token) * TERMS * kpad;
+    for (int k = tid; k < kpad; k += 256) {
+        const float v = k < dim ? load_any(x, x_dtype, base + k) * s : 0.0f;
+        const _Float16 h = static_cast<_Float16>(v);
+        row[k] = h;
+        if constexpr (TERMS == 2) row[kpad + k] = static_cast<_Float16>(v - static_cast<float>(h));
+    }
+    if (tid == 0) unscale[token] = 1.0f / s;
+}
+
+__device__ __forceinline__ v8h as_v8h(uint4 u) {
+    union { uint4 u; v8h h; } c;
+    c.u = u;
+    return c.h;
+}
+
+// the half-precision codebooks of IQ2_XXS, kRowsCopies copies per entry, built by the whole workgroup
+__device__ __forceinline__ void rows_tables_iq2xxs(unsigned char* lds, int tid, int threads) {
+    for (int i = tid; i < (256 + 128) * kRowsCopies; i += threads) {
+        const int e = i / kRowsCopies;
+        uint32_t w[4];
+        if (e < 256) {
+            const uint64_t g = PLLM_IQ2XXS_GRID[e];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                union { _Float16 h[2]; uint32_t u; } c;
+                c.h[0] = static_cast<_Float16>(static_cast<float>((g >> (16 * j)) & 0xffu));
+                c.h[1] = static_cast<_Float16>(static_cast<float>((g >> (16 * j + 8)) & 0xffu));
+                w[j] = c.u;
+            }
+        } else {
+            const uint64_t m = PLLM_IQ2XXS_SIGN_MASKS.v[e - 256];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) w[j] = (((m >> (16 * j)) & 1u) ? 0x8000u : 0u) | (((m >> (16 * j + 8)) & 1u) ? 0x80000000u : 0u);
+        }
+        reinterpret_cast<uint4*>(lds)[i] = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+}
+
+// One hidden value h = silu(g) * u * route weight as two half-precision terms, h ~= hi + lo:
+// rows[0 .. h_kpad) and rows[h_kpad .. 2 h_kpad) of the route.  Magnitudes beyond the half-precision
+// range saturate.
+__device__ __forceinline__ void store_hidden_rows(float g, float u, float limit, float route_weight, int i, int inter, _Float16* rows, int h_kpad) {
+    if (limit > 0.0f) {
+        u = fminf(fmaxf(u, -limit), limit);
+        g = fminf(g, limit);
+    }
+    float h = (i < inter) ? g / (1.0f + expf(-g)) * u * route_weight : 0.0f;
+    h = fminf(fmaxf(h, -65504.0f), 65504.0f);
+    const _Float16 hi = static_cast<_Float16>(h);
+    rows[i] = hi;
+    rows[h_kpad + i] = static_cast<_Float16>(h - static_cast<float>(hi));
+}
+
+template <int NB, int TERMS>
+__global__ __launch_bounds__(64 * kRowsWaves) void moe_rows_w13_kernel(
+    const _Float16* __restrict__ x_rows, const float* __restrict__ unscale, int bpr, const int64_t* __restrict__ route_tokens,
+    const int32_t* __restrict__ seg, const float* __restrict__ route_weights, const uint8_t* __restrict__ w1, const uint8_t* __restrict__ w3,
+    int inter, float limit, _Float16* __restrict__ h_rows, int h_kpad, int n_experts, int runs,
+    int tile_off, int tile_stride) {
+    using FMT = IQ2XXSm;
+    extern __shared__ __align__(16) unsigned char smem[];
+    constexpr int kBatch = 16 / TERMS;
+    constexpr int kExchFloats = kBatch * kRowsShares * 2 * 16;              // [route][share][matrix][16]
+    const int kpad = bpr * 256;
+    float* exch = reinterpret_cast<float*>(smem + kRowsTableBytes);          // two of them, by tile parity
+    const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_byte_ptr)smem));
+
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63;
+    const int n = lane & 15, q = lane >> 4;
+    const int mat = wave & 1, share = wave >> 1;
+    const int row_bytes = bpr * FMT::kBlockBytes;
+    const int tile_bytes = 16 * row_bytes;
+    const int tiles = (inter + 15) / 16;
+    const int tiles_per_run = (tiles + runs - 1) / runs;
+    const unsigned char* grid_lane = smem + (lane & (kRowsCopies - 1)) * 16;            // entry e of the lane's copy: + e * 16 * kRowsCopies
+    const unsigned char* sign_lane = grid_lane + 256 * 16 * kRowsCopies;
+    // every block the lane reads starts at the same offset modulo 4 (66-byte blocks, the wave's blocks
+    // an even number of them apart): its sub-blocks are read as aligned dwords and shifted where needed
+    const bool dword_aligned = ((n * bpr + share) & 1) != 0;
+    const uint32_t sh = dword_aligned ? 0u : 16u;
+    const uint32_t id_sel = 0x0c0c0c00u | static_cast<uint32_t>(q + (dword_aligned ? 0 : 2));   // byte q of the sub-block's four grid ids
+
+    rows_tables_iq2xxs(smem, tid, blockDim.x);
+
+    for (int unit = blockIdx.x; unit < n_experts * runs; unit += gridDim.x) {
+        const int expert = unit / runs, run = unit % runs;
+        const int r0 = seg[expert], r1 = seg[expert + 1];
+        if (r0 >= r1) continue;
+        if (run == 0)                          // padding of the hidden rows: zeros, no weights behind them
+            for (int i = tid; i < (h_kpad - 16 * tiles) * 2 * (r1 - r0); i += blockDim.x) {
+                const int r = i / (h_kpad - 16 * tiles), c = i % (h_kpad - 16 * tiles);          // r = (route, term)
+                h_rows[(static_cast<size_t>(2 * r0) + r) * h_kpad + 16 * tiles + c] = static_cast<_Float16>(0.0f);
+            }
+        const int t0 = run * tiles_per_run, t1 = min(tiles, t0 + tiles_per_run);
+        if (t0 >= t1) continue;
+        const size_t expert_pos = static_cast<size_t>(expert) * inter * row_bytes;
+        for (int rc = r0; rc < r1; rc += kBatch) {
+            const int nr = min(kBatch, r1 - rc);
+            {
+                const size_t pos = expert_pos + static_cast<size_t>(t0) * tile_bytes;
+                dma_share<kRowsWaves>(w1 + pos, lds0 + tile_off, tile_bytes, wave, lane);
+                dma_share<kRowsWaves>(w3 + pos, lds0 + tile_off + tile_stride, tile_bytes, wave, lane);
+            }
+            // the lane's image row: the same for every tile of the run (rows past the batch's end repeat its last route)
+            const int my_route = rc + min((TERMS == 2) ? (n >> 1) : n, nr - 1);
+            const _Float16* xrow = x_rows + (static_cast<size_t>(route_tokens[my_route]) * TERMS + ((TERMS == 2) ? (n & 1) : 0)) * kpad + 8 * q;
+            v8h av[NB][8];
+#pragma unroll
+            for (int i = 0; i < NB; ++i) {
+                const int b = min(share + kRowsShares * i, bpr - 1);
+#pragma unroll
+                for (int g = 0; g < 8; ++g) av[i][g] = as_v8h(*reinterpret_cast<const uint4*>(xrow + 256 * b + 32 * g));
+            }
+            // the epilogue's thread (route j, row c of the tile) keeps its route's factors
+            float ep_unscale = 0.0f, ep_weight = 0.0f;
+            if (tid < 16 * nr) {
+                ep_unscale = unscale[route_tokens[rc + (tid >> 4)]];
+                ep_weight = route_weights[rc + (tid >> 4)];
+            }
+            wait_vm<0>();
+            __syncthreads();                   // first tile landed; every wave has left the previous batch (and the tables are built)
+            for (int tile = t0; tile < t1; ++tile) {
+                const int buf = (tile - t0) & 1;
+                if (tile + 1 < t1) {           // the other buffer was last read before the previous tile's barrier
+                    const size_t pos = expert_pos + static_cast<size_t>(tile + 1) * tile_bytes;
+                    const uint32_t dst = lds0 + tile_off + (buf ^ 1) * 2 * tile_stride;
+                    dma_share<kRowsWaves>(w1 + pos, dst, tile_bytes, wave, lane);
+                    dma_share<kRowsWaves>(w3 + pos, dst + tile_stride, tile_bytes, wave, lane);
+                }
+                const unsigned char* tb = smem + tile_off + (2 * buf + mat) * tile_stride;
+                v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                for (int i = 0; i < NB; ++i) {
+                    const int b = share + kRowsShares * i;
+                    if (b < bpr) {             // wave-uniform
+                        const int off = n * row_bytes + b * FMT::kBlockBytes;
+                        const uint32_t* p = reinterpret_cast<const uint32_t*>(tb + ((off + 2) & ~3));
+                        uint32_t dw[17];
+#pragma unroll
+                        for (int j = 0; j < 17; ++j) dw[j] = p[j];
+                        const float d8 = 0.125f * f16_bits_to_float(*reinterpret_cast<const uint16_t*>(tb + off));
+                        v4f c = {0.0f, 0.0f, 0.0f, 0.0f};
+                        // four groups at a time: all their codebook reads are issued before the first is used
+#pragma unroll
+                        for (int g0 = 0; g0 < 8; g0 += 4) {
+                            uint4 mag[4], sgn[4];
+                            uint32_t aux[4];
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) {
+                                const int g = g0 + j;
+                                const uint32_t id = __builtin_amdgcn_perm(dw[2 * g + 1], dw[2 * g], id_sel);
+                                aux[j] = __builtin_amdgcn_alignbit(dw[2 * g + 2], dw[2 * g + 1], sh);
+                                mag[j] = *reinterpret_cast<const uint4*>(grid_lane + id * (16 * kRowsCopies));
+                                sgn[j] = *reinterpret_cast<const uint4*>(sign_lane + ((aux[j] >> (7 * q)) & 127u) * (16 * kRowsCopies));
+                            }
+                            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) {
+                                // the group scale 2 ls + 1 as a pair of halves: 1024 + 2 ls + 1 by integer arithmetic on the bits, then - 1024
+                                union { uint32_t u; v2h h; } ls2;
+                                ls2.u = (aux[j] >> 28) * 0x00020002u + 0x64016401u;
+                                const v2h k1024 = {static_cast<_Float16>(1024.0f), static_cast<_Float16>(1024.0f)};
+                                ls2.h = ls2.h - k1024;
+                                union { uint4 u; v2h h[4]; } bw;
+                                bw.u = make_uint4(mag[j].x ^ sgn[j].x, mag[j].y ^ sgn[j].y, mag[j].z ^ sgn[j].z, mag[j].w ^ sgn[j].w);
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) bw.h[e] = bw.h[e] * ls2.h;
+                                c = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[i][g0 + j], as_v8h(bw.u), c, 0, 0, 0);
+                            }
+                        }
+                        acc += c * d8;
+                    }
+                }
+                float* ex = exch + buf * kExchFloats;
+                if constexpr (TERMS == 1) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) ex[(((4 * q + j) * kRowsShares + share) * 2 + mat) * 16 + n] = acc[j];
+                } else {
+                    ex[(((2 * q) * kRowsShares + share) * 2 + mat) * 16 + n] = acc[0] + acc[1];
+                    ex[(((2 * q + 1) * kRowsShares + share) * 2 + mat) * 16 + n] = acc[2] + acc[3];
+                }
+                wait_vm<0>();
+                __syncthreads();               // sums visible, next tile landed, this tile's buffer free
+                if (tid < 16 * nr) {
+                    const int j = tid >> 4, c = tid & 15;
+                    float g = 0.0f, u = 0.0f;
+#pragma unroll
+                    for (int v = 0; v < kRowsShares; ++v) { g += ex[((j * kRowsShares + v) * 2) * 16 + c]; u += ex[((j * kRowsShares + v) * 2 + 1) * 16 + c]; }
+                    store_hidden_rows(g * ep_unscale, u * ep_unscale, limit, ep_weight, tile * 16 + c, inter, h_rows + static_cast<size_t>(rc + j) * 2 * h_kpad, h_kpad);
+                }
+            }
+            __syncthreads();                   // the epilogue's readers are done before the next batch overwrites anything
+        }
+    }
+}
+
+// Down projection of grouped routes, the routes as matrix rows (IQ1_M): partial[r, :] = W2_e h_r.
+// The codes 8 (c - 1) +- 1 times the 16-weight scale 2 s + 1 (at most 9 * 15) are exact in half
+// precision; a 32-weight group = four codebook entries = one MFMA, lane (n, q) supplying entry q with
+// its own 16-weight scale.  A rows = (route, term) of the hidden rows written by the kernel above, kept
+// in registers for a run of steps.  A step = 64 output rows (four tiles), twelve waves = (tile, third
+// of the row's blocks); the step's weights are one contiguous run of memory.
+// LDS codebook: 4096 x 8 codes as half-precision vectors, index = qs byte | qh nibble << 8.
+constexpr int kRows2Tiles = 4;
+constexpr int kRows2Shares = kRowsWaves / kRows2Tiles;
+constexpr int kRows2Blocks = 3;           // blocks of a row per wave
+constexpr int kRows2TableBytes = 4096 * 16;
+constexpr int kRows2Batch = 8;
+
+__device__ __forceinline__ void rows_tables_iq1m(unsigned char* lds, int tid, int threads) {
+    for (int i = tid; i < 4096; i += threads) {
+        const uint64_t v = PLLM_IQ1_DELTA_CODES.v[i];
+        uint32_t w[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            union { _Float16 h[2]; uint32_t u; } c;
+            c.h[0] = static_cast<_Float16>(static_cast<float>(static_cast<int8_t>(v >> (16 * j))));
+            c.h[1] = static_cast<_Float16>(static_cast<float>(static_cast<int8_t>(v >> (16 * j + 8))));
+            w[j] = c.u;
+        }
+        reinterpret_cast<uint4*>(lds)[i] = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+}
+
+template <int NB>
+__global__ __launch_bounds__(64 * kRowsWaves) void moe_rows_w2_kernel(
+    const _Float16* __restrict__ h_rows, int bpr, const int32_t* __restrict__ seg, const uint8_t* __restrict__ w2, size_t expert_stride,
+    float* __restrict__ partial, int dim, int n_experts, int runs, int tile_off, int step_stride) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    constexpr int kBlockBytes = IQ1Mm::kBlockBytes;
+    constexpr int kStepRows = 16 * kRows2Tiles;
+    constexpr int kExchFloats = kRows2Batch * kRows2Shares * kStepRows;     // [route][share][row of the step]
+    const int kpad = bpr * 256;
+    float* exch = reinterpret_cast<float*>(smem + kRows2TableBytes);         // two of them, by step parity
+    const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_byte_ptr)smem));
+
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63;
+    const int n = lane & 15, q = lane >> 4;
+    const int tile_in_step = wave / kRows2Shares, share = wave % kRows2Shares;
+    const int row_bytes = bpr * kBlockBytes;
+    const int steps = (dim + kStepRows - 1) / kStepRows;
+    const int steps_per_run = (steps + runs - 1) / runs;
+
+    rows_tables_iq1m(smem, tid, blockDim.x);
+
+    for (int unit = blockIdx.x; unit < n_experts * runs; unit += gridDim.x) {
+        const int expert = unit / runs, run = unit % runs;
+        const int r0 = seg[expert], r1 = seg[expert + 1];
+        if (r0 >= r1) continue;
+        const int s0 = run * steps_per_run, s1 = min(steps, s0 + steps_per_run);
+        if (s0 >= s1) continue;
+        const uint8_t* wexp = w2 + static_cast<size_t>(expert) * expert_stride;
+        for (int rc = r0; rc < r1; rc += kRows2Batch) {
+            const int nr = min(kRows2Batch, r1 - rc);
+            dma_share<kRowsWaves>(wexp + static_cast<size_t>(s0) * kStepRows * row_bytes, lds0 + tile_off, min(kStepRows, dim - s0 * kStepRows) * row_bytes, wave, lane);
+            // the lane's row of the hidden values: the same for every step of the run (rows past the batch's end repeat its last route)
+            const _Float16* hrow = h_rows + (static_cast<size_t>(rc + min(n >> 1, nr - 1)) * 2 + (n & 1)) * kpad + 8 * q;
+            v8h av[NB][8];
+#pragma unroll
+            for (int i = 0; i < NB; ++i) {
+                const int b = min(share + kRows2Shares * i, bpr - 1);
+#pragma unroll
+                for (int g = 0; g < 8; ++g) av[i][g] = as_v8h(*reinterpret_cast<const uint4*>(hrow + 256 * b + 32 * g));
+            }
+            wait_vm<0>();
+            __syncthreads();                   // first step landed; every wave has left the previous batch (and the table is built)
+            for (int step = s0; step < s1; ++step) {
+                const int buf = (step - s0) & 1;
+                const int row0 = step * kStepRows, valid_rows = min(kStepRows, dim - row0);   // a multiple of 16
+                if (step + 1 < s1)             // the other buffer was last read before the previous step's barrier
+                    dma_share<kRowsWaves>(wexp + static_cast<size_t>(row0 + kStepRows) * row_bytes, lds0 + tile_off + (buf ^ 1) * step_stride,
+                                          min(kStepRows, dim - row0 - kStepRows) * row_bytes, wave, lane);
+                float* ex = exch + buf * kExchFloats;
+                if (tile_in_step * 16 < valid_rows) {                       // wave-uniform
+                    const unsigned char* tb = smem + tile_off + buf * step_stride + (tile_in_step * 16 + n) * row_bytes;
+                    v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                    for (int i = 0; i < NB; ++i) {
+                        const int b = share + kRows2Shares * i;
+                        if (b < bpr) {         // wave-uniform
+                            const uint2* p = reinterpret_cast<const uint2*>(tb + b * kBlockBytes);     // blocks are 8-byte aligned
+                            uint32_t dw[14];
+#pragma unroll
+                            for (int j = 0; j < 7; ++j) { const uint2 v = p[j]; dw[2 * j] = v.x; dw[2 * j + 1] = v.y; }
+                            const uint32_t s01 = dw[12], s23 = dw[13];
+                            const uint32_t dbits = ((s01 >> 12) & 0xfu) | ((s01 >> 24) & 0xf0u) | ((s23 >> 4) & 0xf00u) | ((s23 >> 16) & 0xf000u);
+                            v4f c = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                            for (int g0 = 0; g0 < 8; g0 += 4) {
+                                uint4 code[4];
+#pragma unroll
+                                for (int j = 0; j < 4; ++j) {
+                                    const int g = g0 + j;
+                                    const uint32_t qs = __builtin_amdgcn_ubfe(dw[g], 8 * q, 8);
+                                    const uint32_t nib = __builtin_amdgcn_ubfe(dw[8 + (g >> 1)], 16 * (g & 1) + 4 * q, 4);
+                                    code[j] = *reinterpret_cast<const uint4*>(smem + (qs | (nib << 8)) * 16);
+                                }
+                                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                                for (int j = 0; j < 4; ++j) {
+                                    const int g = g0 + j;
+                                    // the 16-weight group 2 g + q / 2: field (2 (g % 2) + q / 2) of scale word g / 2
+                                    const uint32_t s3 = __builtin_amdgcn_ubfe(dw[12 + (g >> 2)], 16 * ((g >> 1) & 1) + 6 * (g & 1) + 3 * (q >> 1), 3);
+                                    union { uint32_t u; v2h h; } ls2;
+                                    ls2.u = s3 * 0x00020002u + 0x64016401u;          // 1024 + 2 s + 1 in both halves ...
+                                    const v2h k1024 = {static_cast<_Float16>(1024.0f), static_cast<_Float16>(1024.0f)};
+                                    ls2.h = ls2.h - k1024;                            // ... minus 1024
+                                    union { uint4 u; v2h h[4]; } bw;
+                                    bw.u = code[j];
+#pragma unroll
+                                    for (int e = 0; e < 4; ++e) bw.h[e] = bw.h[e] * ls2.h;
+                                    c = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[i][g], as_v8h(bw.u), c, 0, 0, 0);
+                                }
+                            }
+                            acc += c * (0.125f * f16_bits_to_float(dbits));
+                        }
+                    }
+                    ex[((2 * q) * kRows2Shares + share) * kStepRows + tile_in_step * 16 + n] = acc[0] + acc[1];
+                    ex[((2 * q + 1) * kRows2Shares + share) * kStepRows + tile_in_step * 16 + n] = acc[2] + acc[3];
+                }
+                wait_vm<0>();
+                __syncthreads();               // sums visible, next step landed, this step's buffer free
+                {
+                    const int j = tid / kStepRows, r = tid % kStepRows;
+                    if (j < nr && r < valid_rows) {
+                        float total = 0.0f;
+#pragma unroll
+                        for (int v = 0; v < kRows2Shares; ++v) total += ex[(j * kRows2Shares + v) * kStepRows + r];
+                        partial[static_cast<size_t>(rc + j) * dim + row0 + r] = total;
+                    }
+                }
+            }
+            __syncthreads();                   // the epilogue's readers are done before the next batch overwrites anything
+        }
+    }
+}
+
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 template <typename KERN>
@@ -438,6 +832,62 @@ int launch_grouped_w13(const unsigned char* x_image, size_t x_stride, int bpr, c
         default: return PLLM_ERR_UNSUPPORTED;
     }
 #undef PLLM_CASE
+}
+
+struct RowsW13Plan { int nb, tile_off, tile_stride; size_t smem; };
+
+RowsW13Plan plan_rows_w13(int bpr) {
+    RowsW13Plan p;
+    p.nb = (bpr + kRowsShares - 1) / kRowsShares;
+    const int head = kRowsTableBytes + 2 * 16 * kRowsShares * 2 * 16 * static_cast<int>(sizeof(float));
+    p.tile_off = (head + 1023) & ~1023;
+    p.tile_stride = 16 * bpr * IQ2XXSm::kBlockBytes + 16;                    // block shares are read as aligned dwords: a few bytes past the end
+    p.smem = static_cast<size_t>(p.tile_off) + 4 * p.tile_stride;
+    return p;
+}
+
+template <int NB, int TERMS>
+int launch_rows_w13_nb(const RowsW13Plan& p, const _Float16* x_rows, const float* unscale, int bpr, const int64_t* route_tokens, const int32_t* seg,
+                       const float* route_weights, const uint8_t* w1, const uint8_t* w3, int inter, float limit, _Float16* h_rows,
+                       int h_kpad, int n_experts, int routes, hipStream_t stream) {
+    auto kern = moe_rows_w13_kernel<NB, TERMS>;
+    if (!allow_lds(kern, p.smem)) return PLLM_ERR_UNSUPPORTED;
+    const int resident = resident_workgroups(kern, 64 * kRowsWaves, p.smem);
+    const int tiles = (inter + 15) / 16;
+    const int busy = max(1, min(routes, n_experts));                         // experts that can have routes at all
+    const int runs = max(1, min(tiles, (4 * resident + busy - 1) / busy));
+    const int grid = min(n_experts * runs, resident);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * kRowsWaves), p.smem, stream, x_rows, unscale, bpr, route_tokens, seg, route_weights, w1, w3, inter,
+                       limit, h_rows, h_kpad, n_experts, runs, p.tile_off, p.tile_stride);
+    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+}
+
+struct RowsW2Plan { int nb, tile_off, step_stride; size_t smem; };
+
+RowsW2Plan plan_rows_w2(int bpr) {
+    RowsW2Plan p;
+    p.nb = (bpr + kRows2Shares - 1) / kRows2Shares;
+    const int head = kRows2TableBytes + 2 * kRows2Batch * kRows2Shares * 16 * kRows2Tiles * static_cast<int>(sizeof(float));
+    p.tile_off = (head + 1023) & ~1023;
+    p.step_stride = 16 * kRows2Tiles * bpr * IQ1Mm::kBlockBytes;
+    p.smem = static_cast<size_t>(p.tile_off) + 2 * p.step_stride;
+    return p;
+}
+
+template <int NB>
+int launch_rows_w2_nb(const RowsW2Plan& p, const _Float16* h_rows, int bpr, const int32_t* seg, const uint8_t* w2, float* partial, int dim,
+                      int n_experts, int routes, hipStream_t stream) {
+    auto kern = moe_rows_w2_kernel<NB>;
+    if (!allow_lds(kern, p.smem)) return PLLM_ERR_UNSUPPORTED;
+    const int resident = resident_workgroups(kern, 64 * kRowsWaves, p.smem);
+    const int steps = (dim + 16 * kRows2Tiles - 1) / (16 * kRows2Tiles);
+    const int busy = max(1, min(routes, n_experts));
+    const int runs = max(1, min(steps, (4 * resident + busy - 1) / busy));
+    const int grid = min(n_experts * runs, resident);
+    const size_t expert_stride = static_cast<size_t>(dim) * bpr * IQ1Mm::kBlockBytes;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * kRowsWaves), p.smem, stream, h_rows, bpr, seg, w2, expert_stride, partial, dim, n_experts, runs,
+                       p.tile_off, p.step_stride);
+    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 
 struct GroupedW2Plan { int nb, shares, table_off, tile_off; size_t smem; };
@@ -526,6 +976,56 @@ int moe_grouped_w13_mfma(const unsigned char* x_image, size_t x_stride, int dim,
     if (w13_type == PLLM_TYPE_IQ2_XXS)
         return launch_grouped_w13<IQ2XXSm>(x_image, x_stride, bpr, route_tokens, seg, route_weights, w1, w3, inter, limit, h_image, h_stride, h_kpad, n_experts, stream);
     return launch_grouped_w13<IQ1Mm>(x_image, x_stride, bpr, route_tokens, seg, route_weights, w1, w3, inter, limit, h_image, h_stride, h_kpad, n_experts, stream);
+}
+
+bool moe_rows_supports(int w13_type, int w2_type, int dim, int inter, const uint8_t* w1, const uint8_t* w3, const uint8_t* w2) {
+    if (w13_type != PLLM_TYPE_IQ2_XXS || w2_type != PLLM_TYPE_IQ1_M || dim % 16 != 0 || inter % 16 != 0) return false;
+    if (!aligned16(w1) || !aligned16(w3) || !aligned16(w2)) return false;
+    const RowsW13Plan p13 = plan_rows_w13((dim + 255) / 256);
+    const RowsW2Plan p2 = plan_rows_w2((inter + 255) / 256);
+    return p13.nb <= kRowsBlocks && p13.smem <= 160 * 1024 && p2.nb <= kRows2Blocks && p2.smem <= 160 * 1024;
+}
+
+size_t moe_rows_x_bytes(int64_t tokens, int64_t dim) {
+    const size_t kpad = static_cast<size_t>((dim + 255) / 256) * 256;
+    return align256(static_cast<size_t>(tokens) * 2 * kpad * sizeof(_Float16)) + align256(static_cast<size_t>(tokens) * sizeof(float));
+}
+
+size_t moe_rows_h_bytes(int64_t routes, int64_t inter) {
+    const size_t kpad = static_cast<size_t>((inter + 255) / 256) * 256;
+    return align256(static_cast<size_t>(routes) * 2 * kpad * sizeof(_Float16));
+}
+
+int moe_rows_w13(const void* x, int x_dtype, int tokens, int dim, void* x_rows_ws, const int64_t* route_tokens, const int32_t* seg,
+                 const float* route_weights, const uint8_t* w1, const uint8_t* w3, int inter, float limit, void* h_rows_ws,
+                 int n_experts, int routes, hipStream_t stream) {
+    const int bpr = (dim + 255) / 256, kpad = bpr * 256, h_kpad = (inter + 255) / 256 * 256;
+    _Float16* x_rows = static_cast<_Float16*>(x_rows_ws);
+    _Float16* h_rows = static_cast<_Float16*>(h_rows_ws);
+    float* unscale = reinterpret_cast<float*>(static_cast<unsigned char*>(x_rows_ws) + align256(static_cast<size_t>(tokens) * 2 * kpad * sizeof(_Float16)));
+    const bool two_terms = x_dtype == PLLM_F32;
+    if (two_terms) hipLaunchKernelGGL(rows_image_kernel<2>, dim3(tokens), dim3(256), 0, stream, x, x_dtype, dim, kpad, x_rows, unscale);
+    else hipLaunchKernelGGL(rows_image_kernel<1>, dim3(tokens), dim3(256), 0, stream, x, x_dtype, dim, kpad, x_rows, unscale);
+    if (hipGetLastError() != hipSuccess) return PLLM_ERR_LAUNCH;
+    const RowsW13Plan p = plan_rows_w13(bpr);
+#define PLLM_CASE(N, T) return launch_rows_w13_nb<N, T>(p, x_rows, unscale, bpr, route_tokens, seg, route_weights, w1, w3, inter, limit, h_rows, h_kpad, n_experts, routes, stream)
+    if (p.nb == 1) { if (two_terms) PLLM_CASE(1, 2); PLLM_CASE(1, 1); }
+    if (p.nb == 2) { if (two_terms) PLLM_CASE(2, 2); PLLM_CASE(2, 1); }
+#undef PLLM_CASE
+    return PLLM_ERR_UNSUPPORTED;
+}
+
+int moe_rows_w2(const void* h_rows_ws, int inter, const int32_t* seg, const uint8_t* w2, float* partial, int dim, int n_experts, int routes,
+                hipStream_t stream) {
+    const int bpr = (inter + 255) / 256;
+    const RowsW2Plan p = plan_rows_w2(bpr);
+    const _Float16* h_rows = static_cast<const _Float16*>(h_rows_ws);
+    switch (p.nb) {
+        case 1: return launch_rows_w2_nb<1>(p, h_rows, bpr, seg, w2, partial, dim, n_experts, routes, stream);
+        case 2: return launch_rows_w2_nb<2>(p, h_rows, bpr, seg, w2, partial, dim, n_experts, routes, stream);
+        case 3: return launch_rows_w2_nb<3>(p, h_rows, bpr, seg, w2, partial, dim, n_experts, routes, stream);
+        default: return PLLM_ERR_UNSUPPORTED;
+    }
 }
 
 int moe_grouped_w2_mfma(const unsigned char* h_image, size_t h_stride, int inter, const int32_t* seg, const uint8_t* w2, float* partial, int dim,

@@ -9,6 +9,8 @@
 
 namespace pllm {
 
+inline size_t align256(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
+
 // Set in the output dtype code a matvec launcher receives: the kernels add their result to what y holds (float32 sum,
 // rounded once) instead of overwriting it.
 constexpr int kAccumulateInto = 0x100;
@@ -96,6 +98,16 @@ bool moe_grouped_mfma_supports(int w13_type, int w2_type, int dim, int inter, co
 int moe_grouped_w13_mfma(const unsigned char* x_image, size_t x_stride, int dim, const int64_t* route_tokens, const int32_t* seg,
                          const float* route_weights, const uint8_t* w1, const uint8_t* w3, int w13_type, int inter, float limit,
                          unsigned char* h_image, size_t h_stride, int n_experts, hipStream_t stream);
+// the same two steps with the routes as matrix rows in half precision (IQ2_XXS gate / up, IQ1_M down): x_rows_ws and h_rows_ws
+// are moe_rows_x_bytes(tokens, dim) and moe_rows_h_bytes(routes, inter) bytes of workspace (activation rows, hidden rows)
+bool moe_rows_supports(int w13_type, int w2_type, int dim, int inter, const uint8_t* w1, const uint8_t* w3, const uint8_t* w2);
+size_t moe_rows_x_bytes(int64_t tokens, int64_t dim);
+size_t moe_rows_h_bytes(int64_t routes, int64_t inter);
+int moe_rows_w13(const void* x, int x_dtype, int tokens, int dim, void* x_rows_ws, const int64_t* route_tokens, const int32_t* seg,
+                 const float* route_weights, const uint8_t* w1, const uint8_t* w3, int inter, float limit, void* h_rows_ws,
+                 int n_experts, int routes, hipStream_t stream);
+int moe_rows_w2(const void* h_rows_ws, int inter, const int32_t* seg, const uint8_t* w2, float* partial, int dim, int n_experts, int routes,
+                hipStream_t stream);
 int moe_grouped_w2_mfma(const unsigned char* h_image, size_t h_stride, int inter, const int32_t* seg, const uint8_t* w2, float* partial, int dim,
                         int n_experts, hipStream_t stream);
 
