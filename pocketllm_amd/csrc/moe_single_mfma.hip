@@ -383,7 +383,7 @@ typedef _Float16 v2h __attribute__((ext_vector_type(2)));
 constexpr int kRowsWaves = 12;
 constexpr int kRowsShares = kRowsWaves / 2;
 constexpr int kRowsBlocks = 2;            // blocks of a row per wave
-constexpr int kRowsCopies = 8;
+constexpr int kRowsCopies = 8;            // (the kernel shifts entry numbers by 7 = log2(16 * kRowsCopies))
 constexpr int kRowsTableBytes = (256 + 128) * 16 * kRowsCopies;
 
 // Activation rows as half-precision images: img[token][term][kpad] = x * s (zero beyond dim), s a
@@ -447,19 +447,15 @@ __device__ __forceinline__ void rows_tables_iq2xxs(unsigned char* lds, int tid, 
     }
 }
 
-// One hidden value h = silu(g) * u * route weight as two half-precision terms, h ~= hi + lo:
-// rows[0 .. h_kpad) and rows[h_kpad .. 2 h_kpad) of the route.  Magnitudes beyond the half-precision
-// range saturate.
-__device__ __forceinline__ void store_hidden_rows(float g, float u, float limit, float route_weight, int i, int inter, _Float16* rows, int h_kpad) {
+// One hidden value h = silu(g) * u * route weight, rounded to half precision (the reference rounds it
+// to 8 bits per 32 values); magnitudes beyond the half-precision range saturate.
+__device__ __forceinline__ void store_hidden_rows(float g, float u, float limit, float route_weight, int i, int inter, _Float16* row) {
     if (limit > 0.0f) {
         u = fminf(fmaxf(u, -limit), limit);
         g = fminf(g, limit);
     }
-    float h = (i < inter) ? g / (1.0f + expf(-g)) * u * route_weight : 0.0f;
-    h = fminf(fmaxf(h, -65504.0f), 65504.0f);
-    const _Float16 hi = static_cast<_Float16>(h);
-    rows[i] = hi;
-    rows[h_kpad + i] = static_cast<_Float16>(h - static_cast<float>(hi));
+    const float h = (i < inter) ? g / (1.0f + expf(-g)) * u * route_weight : 0.0f;
+    row[i] = static_cast<_Float16>(fminf(fmaxf(h, -65504.0f), 65504.0f));
 }
 
 template <int NB, int TERMS>
@@ -490,7 +486,8 @@ __global__ __launch_bounds__(64 * kRowsWaves) void moe_rows_w13_kernel(
     // every block the lane reads starts at the same offset modulo 4 (66-byte blocks, the wave's blocks
     // an even number of them apart): its sub-blocks are read as aligned dwords and shifted where needed
     const bool dword_aligned = ((n * bpr + share) & 1) != 0;
-    const uint32_t sh = dword_aligned ? 0u : 16u;
+    uint32_t sh = dword_aligned ? 0u : 16u;
+    asm volatile("" : "+v"(sh));               // (kept a plain shift amount: one v_alignbit per use instead of a byte permute and a select)
     const uint32_t id_sel = 0x0c0c0c00u | static_cast<uint32_t>(q + (dword_aligned ? 0 : 2));   // byte q of the sub-block's four grid ids
 
     rows_tables_iq2xxs(smem, tid, blockDim.x);
@@ -500,9 +497,9 @@ __global__ __launch_bounds__(64 * kRowsWaves) void moe_rows_w13_kernel(
         const int r0 = seg[expert], r1 = seg[expert + 1];
         if (r0 >= r1) continue;
         if (run == 0)                          // padding of the hidden rows: zeros, no weights behind them
-            for (int i = tid; i < (h_kpad - 16 * tiles) * 2 * (r1 - r0); i += blockDim.x) {
-                const int r = i / (h_kpad - 16 * tiles), c = i % (h_kpad - 16 * tiles);          // r = (route, term)
-                h_rows[(static_cast<size_t>(2 * r0) + r) * h_kpad + 16 * tiles + c] = static_cast<_Float16>(0.0f);
+            for (int i = tid; i < (h_kpad - 16 * tiles) * (r1 - r0); i += blockDim.x) {
+                const int r = i / (h_kpad - 16 * tiles), c = i % (h_kpad - 16 * tiles);
+                h_rows[static_cast<size_t>(r0 + r) * h_kpad + 16 * tiles + c] = static_cast<_Float16>(0.0f);
             }
         const int t0 = run * tiles_per_run, t1 = min(tiles, t0 + tiles_per_run);
         if (t0 >= t1) continue;
@@ -563,8 +560,8 @@ __global__ __launch_bounds__(64 * kRowsWaves) void moe_rows_w13_kernel(
                                 const int g = g0 + j;
                                 const uint32_t id = __builtin_amdgcn_perm(dw[2 * g + 1], dw[2 * g], id_sel);
                                 aux[j] = __builtin_amdgcn_alignbit(dw[2 * g + 2], dw[2 * g + 1], sh);
-                                mag[j] = *reinterpret_cast<const uint4*>(grid_lane + id * (16 * kRowsCopies));
-                                sgn[j] = *reinterpret_cast<const uint4*>(sign_lane + ((aux[j] >> (7 * q)) & 127u) * (16 * kRowsCopies));
+                                mag[j] = *reinterpret_cast<const uint4*>(grid_lane + (id << 7));
+                                sgn[j] = *reinterpret_cast<const uint4*>(sign_lane + (__builtin_amdgcn_ubfe(aux[j], 7 * q, 7) << 7));
                             }
                             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -599,7 +596,7 @@ __global__ __launch_bounds__(64 * kRowsWaves) void moe_rows_w13_kernel(
                     float g = 0.0f, u = 0.0f;
 #pragma unroll
                     for (int v = 0; v < kRowsShares; ++v) { g += ex[((j * kRowsShares + v) * 2) * 16 + c]; u += ex[((j * kRowsShares + v) * 2 + 1) * 16 + c]; }
-                    store_hidden_rows(g * ep_unscale, u * ep_unscale, limit, ep_weight, tile * 16 + c, inter, h_rows + static_cast<size_t>(rc + j) * 2 * h_kpad, h_kpad);
+                    store_hidden_rows(g * ep_unscale, u * ep_unscale, limit, ep_weight, tile * 16 + c, inter, h_rows + static_cast<size_t>(rc + j) * h_kpad);
                 }
             }
             __syncthreads();                   // the epilogue's readers are done before the next batch overwrites anything
@@ -610,15 +607,15 @@ __global__ __launch_bounds__(64 * kRowsWaves) void moe_rows_w13_kernel(
 // Down projection of grouped routes, the routes as matrix rows (IQ1_M): partial[r, :] = W2_e h_r.
 // The codes 8 (c - 1) +- 1 times the 16-weight scale 2 s + 1 (at most 9 * 15) are exact in half
 // precision; a 32-weight group = four codebook entries = one MFMA, lane (n, q) supplying entry q with
-// its own 16-weight scale.  A rows = (route, term) of the hidden rows written by the kernel above, kept
-// in registers for a run of steps.  A step = 64 output rows (four tiles), twelve waves = (tile, third
+// its own 16-weight scale.  A rows = the hidden rows of 16 routes written by the kernel above, kept in
+// registers for a run of steps.  A step = 64 output rows (four tiles), twelve waves = (tile, third
 // of the row's blocks); the step's weights are one contiguous run of memory.
 // LDS codebook: 4096 x 8 codes as half-precision vectors, index = qs byte | qh nibble << 8.
 constexpr int kRows2Tiles = 4;
 constexpr int kRows2Shares = kRowsWaves / kRows2Tiles;
 constexpr int kRows2Blocks = 3;           // blocks of a row per wave
 constexpr int kRows2TableBytes = 4096 * 16;
-constexpr int kRows2Batch = 8;
+constexpr int kRows2Batch = 16;
 
 __device__ __forceinline__ void rows_tables_iq1m(unsigned char* lds, int tid, int threads) {
     for (int i = tid; i < 4096; i += threads) {
@@ -669,7 +666,7 @@ __global__ __launch_bounds__(64 * kRowsWaves) void moe_rows_w2_kernel(
             const int nr = min(kRows2Batch, r1 - rc);
             dma_share<kRowsWaves>(wexp + static_cast<size_t>(s0) * kStepRows * row_bytes, lds0 + tile_off, min(kStepRows, dim - s0 * kStepRows) * row_bytes, wave, lane);
             // the lane's row of the hidden values: the same for every step of the run (rows past the batch's end repeat its last route)
-            const _Float16* hrow = h_rows + (static_cast<size_t>(rc + min(n >> 1, nr - 1)) * 2 + (n & 1)) * kpad + 8 * q;
+            const _Float16* hrow = h_rows + static_cast<size_t>(rc + min(n, nr - 1)) * kpad + 8 * q;
             v8h av[NB][8];
 #pragma unroll
             for (int i = 0; i < NB; ++i) {
@@ -730,14 +727,14 @@ __global__ __launch_bounds__(64 * kRowsWaves) void moe_rows_w2_kernel(
                             acc += c * (0.125f * f16_bits_to_float(dbits));
                         }
                     }
-                    ex[((2 * q) * kRows2Shares + share) * kStepRows + tile_in_step * 16 + n] = acc[0] + acc[1];
-                    ex[((2 * q + 1) * kRows2Shares + share) * kStepRows + tile_in_step * 16 + n] = acc[2] + acc[3];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) ex[((4 * q + j) * kRows2Shares + share) * kStepRows + tile_in_step * 16 + n] = acc[j];
                 }
                 wait_vm<0>();
                 __syncthreads();               // sums visible, next step landed, this step's buffer free
-                {
-                    const int j = tid / kStepRows, r = tid % kStepRows;
-                    if (j < nr && r < valid_rows) {
+                for (int o = tid; o < nr * kStepRows; o += blockDim.x) {
+                    const int j = o / kStepRows, r = o % kStepRows;
+                    if (r < valid_rows) {
                         float total = 0.0f;
 #pragma unroll
                         for (int v = 0; v < kRows2Shares; ++v) total += ex[(j * kRows2Shares + v) * kStepRows + r];
@@ -993,7 +990,7 @@ size_t moe_rows_x_bytes(int64_t tokens, int64_t dim) {
 
 size_t moe_rows_h_bytes(int64_t routes, int64_t inter) {
     const size_t kpad = static_cast<size_t>((inter + 255) / 256) * 256;
-    return align256(static_cast<size_t>(routes) * 2 * kpad * sizeof(_Float16));
+    return align256(static_cast<size_t>(routes) * kpad * sizeof(_Float16));
 }
 
 int moe_rows_w13(const void* x, int x_dtype, int tokens, int dim, void* x_rows_ws, const int64_t* route_tokens, const int32_t* seg,
