@@ -21,6 +21,10 @@ constexpr int kMoeGemmMinTokens = 16;
 // epilogue after one decode per expert; measured ~180 us + 0.5 us per route at 256 experts of 1536 x 3072) run ahead
 // of the tile matmuls (cost per expert: the fp16 decode of every weight, ~1450 us for the same experts)
 constexpr int kMoeGroupedMaxRoutesPerExpert = 8;
+// The half-precision form with the routes as matrix rows pays a fixed price per expert that has routes at all (its decode costs
+// more than the integer one, its multiply next to nothing): measured at 256 experts of 1536 x 3072 it overtakes the form above
+// between 1 and 2 routes per expert (32 tokens, top 8: 375 vs 316 us; 64 tokens: 381 vs 472 us; 256 tokens: 500 vs 1126 us).
+constexpr int kMoeRowsMinRoutesPerExpertX2 = 3;
 
 namespace {
 
@@ -537,7 +541,7 @@ int pllm_gguf_moe_forward(const void* x, int x_dtype, int64_t tokens, int64_t di
     if (!workspace || workspace_bytes < pllm_gguf_moe_workspace_bytes(tokens, routes, dim, inter)) return PLLM_ERR_WORKSPACE;
 
     const int bpr_x = static_cast<int>((dim + 255) / 256), bpr_h = static_cast<int>((inter + 255) / 256);
-    if (seg_starts && tokens > 1 && routes <= kMoeGroupedMaxRoutesPerExpert * n_experts &&
+    if (seg_starts && tokens > 1 && routes <= kMoeGroupedMaxRoutesPerExpert * n_experts && 2 * routes >= kMoeRowsMinRoutesPerExpertX2 * n_experts &&
         moe_rows_supports(w13_type, w2_type, static_cast<int>(dim), static_cast<int>(inter), w1, w3, w2)) {
         // a few routes per expert, IQ2_XXS / IQ1_M: every expert's weights are decoded once, in half precision, and multiplied with
         // all its routes at once on the matrix cores

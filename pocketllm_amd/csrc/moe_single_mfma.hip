@@ -389,6 +389,14 @@ constexpr int kRowsTableBytes = (256 + 128) * 16 * kRowsCopies;
 // Activation rows as half-precision images: img[token][term][kpad] = x * s (zero beyond dim), s a
 // power of two that brings the row's largest magnitude into [1024, 2048); unscale[token] = 1 / s.
 // TERMS = 2 adds the rounding residual as a second row.
+// the power of two that brings a row whose largest magnitude is am into [1024, 2048) (1 for rows of zeros or with non-finite values)
+__device__ __forceinline__ float rows_scale(float am) {
+    if (!(am > 0.0f && am < 3.0e38f)) return 1.0f;
+    int ex;
+    frexpf(am, &ex);                           // am = m * 2^ex, m in [0.5, 1)
+    return ldexpf(1.0f, max(-126, min(11 - ex, 126)));
+}
+
 template <int TERMS>
 __global__ __launch_bounds__(256) void rows_image_kernel(const void* __restrict__ x, int x_dtype, int dim, int kpad, _Float16* __restrict__ img,
                                                          float* __restrict__ unscale) {
@@ -402,12 +410,7 @@ __global__ __launch_bounds__(256) void rows_image_kernel(const void* __restrict_
     if ((tid & 63) == 0) part[tid >> 6] = am;
     __syncthreads();
     am = fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3]));
-    float s = 1.0f;
-    if (am > 0.0f && am < 3.0e38f) {
-        int ex;
-        frexpf(am, &ex);                       // am = m * 2^ex, m in [0.5, 1)
-        s = ldexpf(1.0f, max(-126, min(11 - ex, 126)));
-    }
+    const float s = rows_scale(am);
     _Float16* row = img + static_cast<size_t>(token) * TERMS * kpad;
     for (int k = tid; k < kpad; k += 256) {
         const float v = k < dim ? load_any(x, x_dtype, base + k) * s : 0.0f;
@@ -447,22 +450,51 @@ __device__ __forceinline__ void rows_tables_iq2xxs(unsigned char* lds, int tid, 
     }
 }
 
-// One hidden value h = silu(g) * u * route weight, rounded to half precision (the reference rounds it
-// to 8 bits per 32 values); magnitudes beyond the half-precision range saturate.
-__device__ __forceinline__ void store_hidden_rows(float g, float u, float limit, float route_weight, int i, int inter, _Float16* row) {
+// One hidden value h = silu(g) * u * route weight of a 16-row tile (16 neighbouring lanes = the tile), kept in float32,
+// and the tile's largest magnitude: the down projection's rows are scaled per route once all tiles are there.
+__device__ __forceinline__ void store_hidden_rows(float g, float u, float limit, float route_weight, int i, int inter, float* row, float* tile_max) {
     if (limit > 0.0f) {
         u = fminf(fmaxf(u, -limit), limit);
         g = fminf(g, limit);
     }
     const float h = (i < inter) ? g / (1.0f + expf(-g)) * u * route_weight : 0.0f;
-    row[i] = static_cast<_Float16>(fminf(fmaxf(h, -65504.0f), 65504.0f));
+    row[i] = h;
+    float am = fabsf(h);
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) am = fmaxf(am, __shfl_xor(am, off, 64));   // (fmaxf drops NaNs; an infinity stays)
+    if ((i & 15) == 0) tile_max[i >> 4] = am;
+}
+
+// hidden rows of the down projection: h16[route][k] = h[route][k] * s, s the power of two of rows_scale for the route's
+// largest magnitude; unscale[route] = 1 / s.  One workgroup per route.
+__global__ __launch_bounds__(256) void rows_hidden_half_kernel(const float* __restrict__ h, const float* __restrict__ tile_max, int h_kpad,
+                                                               _Float16* __restrict__ h16, float* __restrict__ unscale) {
+    __shared__ float part[4];
+    const int route = blockIdx.x, tid = threadIdx.x;
+    float am = 0.0f;
+    for (int t = tid; t < h_kpad / 16; t += 256) am = fmaxf(am, tile_max[static_cast<size_t>(route) * (h_kpad / 16) + t]);
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) am = fmaxf(am, __shfl_xor(am, off, 64));
+    if ((tid & 63) == 0) part[tid >> 6] = am;
+    __syncthreads();
+    const float s = rows_scale(fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3])));
+    const float4* src = reinterpret_cast<const float4*>(h + static_cast<size_t>(route) * h_kpad);
+    uint2* dst = reinterpret_cast<uint2*>(h16 + static_cast<size_t>(route) * h_kpad);
+    for (int k = tid; k < h_kpad / 4; k += 256) {
+        const float4 v = src[k];
+        union { _Float16 h[4]; uint2 u; } c;
+        c.h[0] = static_cast<_Float16>(v.x * s); c.h[1] = static_cast<_Float16>(v.y * s);
+        c.h[2] = static_cast<_Float16>(v.z * s); c.h[3] = static_cast<_Float16>(v.w * s);
+        dst[k] = c.u;
+    }
+    if (tid == 0) unscale[route] = 1.0f / s;
 }
 
 template <int NB, int TERMS>
 __global__ __launch_bounds__(64 * kRowsWaves) void moe_rows_w13_kernel(
     const _Float16* __restrict__ x_rows, const float* __restrict__ unscale, int bpr, const int64_t* __restrict__ route_tokens,
     const int32_t* __restrict__ seg, const float* __restrict__ route_weights, const uint8_t* __restrict__ w1, const uint8_t* __restrict__ w3,
-    int inter, float limit, _Float16* __restrict__ h_rows, int h_kpad, int n_experts, int runs,
+    int inter, float limit, float* __restrict__ h_rows, float* __restrict__ h_tile_max, int h_kpad, int n_experts, int runs,
     int tile_off, int tile_stride) {
     using FMT = IQ2XXSm;
     extern __shared__ __align__(16) unsigned char smem[];
@@ -499,7 +531,8 @@ __global__ __launch_bounds__(64 * kRowsWaves) void moe_rows_w13_kernel(
         if (run == 0)                          // padding of the hidden rows: zeros, no weights behind them
             for (int i = tid; i < (h_kpad - 16 * tiles) * (r1 - r0); i += blockDim.x) {
                 const int r = i / (h_kpad - 16 * tiles), c = i % (h_kpad - 16 * tiles);
-                h_rows[static_cast<size_t>(r0 + r) * h_kpad + 16 * tiles + c] = static_cast<_Float16>(0.0f);
+                h_rows[static_cast<size_t>(r0 + r) * h_kpad + 16 * tiles + c] = 0.0f;
+                if ((c & 15) == 0) h_tile_max[static_cast<size_t>(r0 + r) * (h_kpad / 16) + tiles + (c >> 4)] = 0.0f;
             }
         const int t0 = run * tiles_per_run, t1 = min(tiles, t0 + tiles_per_run);
         if (t0 >= t1) continue;
@@ -596,7 +629,7 @@ __global__ __launch_bounds__(64 * kRowsWaves) void moe_rows_w13_kernel(
                     float g = 0.0f, u = 0.0f;
 #pragma unroll
                     for (int v = 0; v < kRowsShares; ++v) { g += ex[((j * kRowsShares + v) * 2) * 16 + c]; u += ex[((j * kRowsShares + v) * 2 + 1) * 16 + c]; }
-                    store_hidden_rows(g * ep_unscale, u * ep_unscale, limit, ep_weight, tile * 16 + c, inter, h_rows + static_cast<size_t>(rc + j) * h_kpad);
+                    store_hidden_rows(g * ep_unscale, u * ep_unscale, limit, ep_weight, tile * 16 + c, inter, h_rows + static_cast<size_t>(rc + j) * h_kpad, h_tile_max + static_cast<size_t>(rc + j) * (h_kpad / 16));
                 }
             }
             __syncthreads();                   // the epilogue's readers are done before the next batch overwrites anything
@@ -607,7 +640,7 @@ __global__ __launch_bounds__(64 * kRowsWaves) void moe_rows_w13_kernel(
 // Down projection of grouped routes, the routes as matrix rows (IQ1_M): partial[r, :] = W2_e h_r.
 // The codes 8 (c - 1) +- 1 times the 16-weight scale 2 s + 1 (at most 9 * 15) are exact in half
 // precision; a 32-weight group = four codebook entries = one MFMA, lane (n, q) supplying entry q with
-// its own 16-weight scale.  A rows = the hidden rows of 16 routes written by the kernel above, kept in
+// its own 16-weight scale.  A rows = the hidden rows of 16 routes (rows_hidden_half_kernel), kept in
 // registers for a run of steps.  A step = 64 output rows (four tiles), twelve waves = (tile, third
 // of the row's blocks); the step's weights are one contiguous run of memory.
 // LDS codebook: 4096 x 8 codes as half-precision vectors, index = qs byte | qh nibble << 8.
@@ -634,14 +667,15 @@ __device__ __forceinline__ void rows_tables_iq1m(unsigned char* lds, int tid, in
 
 template <int NB>
 __global__ __launch_bounds__(64 * kRowsWaves) void moe_rows_w2_kernel(
-    const _Float16* __restrict__ h_rows, int bpr, const int32_t* __restrict__ seg, const uint8_t* __restrict__ w2, size_t expert_stride,
-    float* __restrict__ partial, int dim, int n_experts, int runs, int tile_off, int step_stride) {
+    const _Float16* __restrict__ h_rows, const float* __restrict__ h_unscale, int bpr, const int32_t* __restrict__ seg, const uint8_t* __restrict__ w2,
+    size_t expert_stride, float* __restrict__ partial, int dim, int n_experts, int runs, int tile_off, int step_stride) {
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int kBlockBytes = IQ1Mm::kBlockBytes;
     constexpr int kStepRows = 16 * kRows2Tiles;
     constexpr int kExchFloats = kRows2Batch * kRows2Shares * kStepRows;     // [route][share][row of the step]
     const int kpad = bpr * 256;
     float* exch = reinterpret_cast<float*>(smem + kRows2TableBytes);         // two of them, by step parity
+    float* route_unscale = exch + 2 * kExchFloats;                           // [route of the batch]
     const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_byte_ptr)smem));
 
     const int tid = threadIdx.x;
@@ -666,7 +700,9 @@ __global__ __launch_bounds__(64 * kRowsWaves) void moe_rows_w2_kernel(
             const int nr = min(kRows2Batch, r1 - rc);
             dma_share<kRowsWaves>(wexp + static_cast<size_t>(s0) * kStepRows * row_bytes, lds0 + tile_off, min(kStepRows, dim - s0 * kStepRows) * row_bytes, wave, lane);
             // the lane's row of the hidden values: the same for every step of the run (rows past the batch's end repeat its last route)
+            // (rows scaled into half-precision range by a power of two per route: taken out again when the sums are stored)
             const _Float16* hrow = h_rows + static_cast<size_t>(rc + min(n, nr - 1)) * kpad + 8 * q;
+            if (tid < kRows2Batch) route_unscale[tid] = h_unscale[rc + min(tid, nr - 1)];
             v8h av[NB][8];
 #pragma unroll
             for (int i = 0; i < NB; ++i) {
@@ -738,7 +774,7 @@ __global__ __launch_bounds__(64 * kRowsWaves) void moe_rows_w2_kernel(
                         float total = 0.0f;
 #pragma unroll
                         for (int v = 0; v < kRows2Shares; ++v) total += ex[(j * kRows2Shares + v) * kStepRows + r];
-                        partial[static_cast<size_t>(rc + j) * dim + row0 + r] = total;
+                        partial[static_cast<size_t>(rc + j) * dim + row0 + r] = total * route_unscale[j];
                     }
                 }
             }
@@ -845,8 +881,8 @@ RowsW13Plan plan_rows_w13(int bpr) {
 
 template <int NB, int TERMS>
 int launch_rows_w13_nb(const RowsW13Plan& p, const _Float16* x_rows, const float* unscale, int bpr, const int64_t* route_tokens, const int32_t* seg,
-                       const float* route_weights, const uint8_t* w1, const uint8_t* w3, int inter, float limit, _Float16* h_rows,
-                       int h_kpad, int n_experts, int routes, hipStream_t stream) {
+                       const float* route_weights, const uint8_t* w1, const uint8_t* w3, int inter, float limit, float* h_rows,
+                       float* h_tile_max, int h_kpad, int n_experts, int routes, hipStream_t stream) {
     auto kern = moe_rows_w13_kernel<NB, TERMS>;
     if (!allow_lds(kern, p.smem)) return PLLM_ERR_UNSUPPORTED;
     const int resident = resident_workgroups(kern, 64 * kRowsWaves, p.smem);
@@ -855,7 +891,7 @@ int launch_rows_w13_nb(const RowsW13Plan& p, const _Float16* x_rows, const float
     const int runs = max(1, min(tiles, (4 * resident + busy - 1) / busy));
     const int grid = min(n_experts * runs, resident);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * kRowsWaves), p.smem, stream, x_rows, unscale, bpr, route_tokens, seg, route_weights, w1, w3, inter,
-                       limit, h_rows, h_kpad, n_experts, runs, p.tile_off, p.tile_stride);
+                       limit, h_rows, h_tile_max, h_kpad, n_experts, runs, p.tile_off, p.tile_stride);
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 
@@ -864,7 +900,7 @@ struct RowsW2Plan { int nb, tile_off, step_stride; size_t smem; };
 RowsW2Plan plan_rows_w2(int bpr) {
     RowsW2Plan p;
     p.nb = (bpr + kRows2Shares - 1) / kRows2Shares;
-    const int head = kRows2TableBytes + 2 * kRows2Batch * kRows2Shares * 16 * kRows2Tiles * static_cast<int>(sizeof(float));
+    const int head = kRows2TableBytes + (2 * kRows2Batch * kRows2Shares * 16 * kRows2Tiles + kRows2Batch) * static_cast<int>(sizeof(float));
     p.tile_off = (head + 1023) & ~1023;
     p.step_stride = 16 * kRows2Tiles * bpr * IQ1Mm::kBlockBytes;
     p.smem = static_cast<size_t>(p.tile_off) + 2 * p.step_stride;
@@ -872,7 +908,7 @@ RowsW2Plan plan_rows_w2(int bpr) {
 }
 
 template <int NB>
-int launch_rows_w2_nb(const RowsW2Plan& p, const _Float16* h_rows, int bpr, const int32_t* seg, const uint8_t* w2, float* partial, int dim,
+int launch_rows_w2_nb(const RowsW2Plan& p, const _Float16* h_rows, const float* h_unscale, int bpr, const int32_t* seg, const uint8_t* w2, float* partial, int dim,
                       int n_experts, int routes, hipStream_t stream) {
     auto kern = moe_rows_w2_kernel<NB>;
     if (!allow_lds(kern, p.smem)) return PLLM_ERR_UNSUPPORTED;
@@ -882,7 +918,7 @@ int launch_rows_w2_nb(const RowsW2Plan& p, const _Float16* h_rows, int bpr, cons
     const int runs = max(1, min(steps, (4 * resident + busy - 1) / busy));
     const int grid = min(n_experts * runs, resident);
     const size_t expert_stride = static_cast<size_t>(dim) * bpr * IQ1Mm::kBlockBytes;
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * kRowsWaves), p.smem, stream, h_rows, bpr, seg, w2, expert_stride, partial, dim, n_experts, runs,
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * kRowsWaves), p.smem, stream, h_rows, h_unscale, bpr, seg, w2, expert_stride, partial, dim, n_experts, runs,
                        p.tile_off, p.step_stride);
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
@@ -988,39 +1024,53 @@ size_t moe_rows_x_bytes(int64_t tokens, int64_t dim) {
     return align256(static_cast<size_t>(tokens) * 2 * kpad * sizeof(_Float16)) + align256(static_cast<size_t>(tokens) * sizeof(float));
 }
 
-size_t moe_rows_h_bytes(int64_t routes, int64_t inter) {
-    const size_t kpad = static_cast<size_t>((inter + 255) / 256) * 256;
-    return align256(static_cast<size_t>(routes) * kpad * sizeof(_Float16));
+// hidden rows of the routes: float32 values [routes][h_kpad], largest magnitudes per 16-row tile, half-precision rows, 1 / scale
+struct RowsHidden { float* values; float* tile_max; _Float16* half_rows; float* unscale; size_t bytes; };
+
+static RowsHidden rows_hidden(void* ws, int64_t routes, int64_t inter) {
+    const size_t kpad = static_cast<size_t>((inter + 255) / 256) * 256, r = static_cast<size_t>(routes);
+    unsigned char* p = static_cast<unsigned char*>(ws);
+    RowsHidden h;
+    h.values = reinterpret_cast<float*>(p);        p += align256(r * kpad * sizeof(float));
+    h.tile_max = reinterpret_cast<float*>(p);      p += align256(r * (kpad / 16) * sizeof(float));
+    h.half_rows = reinterpret_cast<_Float16*>(p);  p += align256(r * kpad * sizeof(_Float16));
+    h.unscale = reinterpret_cast<float*>(p);       p += align256(r * sizeof(float));
+    h.bytes = static_cast<size_t>(p - static_cast<unsigned char*>(ws));
+    return h;
 }
+
+size_t moe_rows_h_bytes(int64_t routes, int64_t inter) { return rows_hidden(nullptr, routes, inter).bytes; }
 
 int moe_rows_w13(const void* x, int x_dtype, int tokens, int dim, void* x_rows_ws, const int64_t* route_tokens, const int32_t* seg,
                  const float* route_weights, const uint8_t* w1, const uint8_t* w3, int inter, float limit, void* h_rows_ws,
                  int n_experts, int routes, hipStream_t stream) {
     const int bpr = (dim + 255) / 256, kpad = bpr * 256, h_kpad = (inter + 255) / 256 * 256;
     _Float16* x_rows = static_cast<_Float16*>(x_rows_ws);
-    _Float16* h_rows = static_cast<_Float16*>(h_rows_ws);
+    const RowsHidden hid = rows_hidden(h_rows_ws, routes, inter);
     float* unscale = reinterpret_cast<float*>(static_cast<unsigned char*>(x_rows_ws) + align256(static_cast<size_t>(tokens) * 2 * kpad * sizeof(_Float16)));
     const bool two_terms = x_dtype == PLLM_F32;
     if (two_terms) hipLaunchKernelGGL(rows_image_kernel<2>, dim3(tokens), dim3(256), 0, stream, x, x_dtype, dim, kpad, x_rows, unscale);
     else hipLaunchKernelGGL(rows_image_kernel<1>, dim3(tokens), dim3(256), 0, stream, x, x_dtype, dim, kpad, x_rows, unscale);
     if (hipGetLastError() != hipSuccess) return PLLM_ERR_LAUNCH;
     const RowsW13Plan p = plan_rows_w13(bpr);
-#define PLLM_CASE(N, T) return launch_rows_w13_nb<N, T>(p, x_rows, unscale, bpr, route_tokens, seg, route_weights, w1, w3, inter, limit, h_rows, h_kpad, n_experts, routes, stream)
+#define PLLM_CASE(N, T) return launch_rows_w13_nb<N, T>(p, x_rows, unscale, bpr, route_tokens, seg, route_weights, w1, w3, inter, limit, hid.values, hid.tile_max, h_kpad, n_experts, routes, stream)
     if (p.nb == 1) { if (two_terms) PLLM_CASE(1, 2); PLLM_CASE(1, 1); }
     if (p.nb == 2) { if (two_terms) PLLM_CASE(2, 2); PLLM_CASE(2, 1); }
 #undef PLLM_CASE
     return PLLM_ERR_UNSUPPORTED;
 }
 
-int moe_rows_w2(const void* h_rows_ws, int inter, const int32_t* seg, const uint8_t* w2, float* partial, int dim, int n_experts, int routes,
+int moe_rows_w2(void* h_rows_ws, int inter, const int32_t* seg, const uint8_t* w2, float* partial, int dim, int n_experts, int routes,
                 hipStream_t stream) {
     const int bpr = (inter + 255) / 256;
     const RowsW2Plan p = plan_rows_w2(bpr);
-    const _Float16* h_rows = static_cast<const _Float16*>(h_rows_ws);
+    const RowsHidden hid = rows_hidden(const_cast<void*>(h_rows_ws), routes, inter);
+    hipLaunchKernelGGL(rows_hidden_half_kernel, dim3(routes), dim3(256), 0, stream, hid.values, hid.tile_max, bpr * 256, hid.half_rows, hid.unscale);
+    if (hipGetLastError() != hipSuccess) return PLLM_ERR_LAUNCH;
     switch (p.nb) {
-        case 1: return launch_rows_w2_nb<1>(p, h_rows, bpr, seg, w2, partial, dim, n_experts, routes, stream);
-        case 2: return launch_rows_w2_nb<2>(p, h_rows, bpr, seg, w2, partial, dim, n_experts, routes, stream);
-        case 3: return launch_rows_w2_nb<3>(p, h_rows, bpr, seg, w2, partial, dim, n_experts, routes, stream);
+        case 1: return launch_rows_w2_nb<1>(p, hid.half_rows, hid.unscale, bpr, seg, w2, partial, dim, n_experts, routes, stream);
+        case 2: return launch_rows_w2_nb<2>(p, hid.half_rows, hid.unscale, bpr, seg, w2, partial, dim, n_experts, routes, stream);
+        case 3: return launch_rows_w2_nb<3>(p, hid.half_rows, hid.unscale, bpr, seg, w2, partial, dim, n_experts, routes, stream);
         default: return PLLM_ERR_UNSUPPORTED;
     }
 }

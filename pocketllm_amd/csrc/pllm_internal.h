@@ -106,7 +106,7 @@ size_t moe_rows_h_bytes(int64_t routes, int64_t inter);
 int moe_rows_w13(const void* x, int x_dtype, int tokens, int dim, void* x_rows_ws, const int64_t* route_tokens, const int32_t* seg,
                  const float* route_weights, const uint8_t* w1, const uint8_t* w3, int inter, float limit, void* h_rows_ws,
                  int n_experts, int routes, hipStream_t stream);
-int moe_rows_w2(const void* h_rows_ws, int inter, const int32_t* seg, const uint8_t* w2, float* partial, int dim, int n_experts, int routes,
+int moe_rows_w2(void* h_rows_ws, int inter, const int32_t* seg, const uint8_t* w2, float* partial, int dim, int n_experts, int routes,
                 hipStream_t stream);
 int moe_grouped_w2_mfma(const unsigned char* h_image, size_t h_stride, int inter, const int32_t* seg, const uint8_t* w2, float* partial, int dim,
                         int n_experts, hipStream_t stream);

@@ -303,6 +303,70 @@ def test_grouped_experts_matrix_core_path(mod, t13, e, d, inter, topk, t, limit)
     assert torch.equal(y, y2)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_grouped_experts_routes_as_matrix_rows(mod, dtype):
+    """IQ2_XXS / IQ1_M experts at 1.5 routes per expert or more take the half-precision form (routes = rows of the matrix-core
+    product): one expert with 21 routes (two batches of 16, three of 8 for float32 activations, which go in as two terms),
+    experts without routes, an intermediate size that is not a multiple of 256, every activation dtype, rows scaled far
+    away from 1 (the rows are brought into half-precision range by a power of two per token)."""
+    rng = np.random.default_rng(77)
+    e, d, inter, t = 6, 512, 400, 24
+    w1 = _expert_blocks(rng, "iq2_xxs", e, inter, d)
+    w3 = _expert_blocks(rng, "iq2_xxs", e, inter, d)
+    w2 = _expert_blocks(rng, "iq1_m", e, d, inter)
+    idx = np.zeros((t, 2), dtype=np.int64)
+    idx[:21, 0] = 0                                         # 21 tokens choose expert 0 first
+    idx[21:, 0] = 2
+    idx[:, 1] = 1 + 2 * (np.arange(t) % 2) + 2 * (np.arange(t) % 3 == 0)   # second choices over experts 1, 3, 5; expert 4 stays empty
+    wts = rng.uniform(0.1, 0.9, size=(t, 2)).astype(np.float32)
+    xf = rng.standard_normal((t, d)).astype(np.float32)
+    xf[3] *= 3.0e4 if dtype != torch.float16 else 40.0      # (its hidden values) beyond half-precision range before scaling
+    xf[5] *= 2.0e-6                                         # half-precision subnormals before scaling
+    xf[7] = 0.0
+    x = torch.from_numpy(xf).to(DEV).to(dtype)
+    _, toks, rws, seg = mod.moe_group_routes(torch.from_numpy(idx).to(DEV), torch.from_numpy(wts).to(DEV), 0, e)
+    _, o_toks, o_rws, o_seg = O.group_routes(idx, wts, 0, e)
+    counts = np.diff(o_seg)
+    assert counts[0] == 21 and counts[4] == 0 and 2 * len(o_toks) >= 3 * e and len(o_toks) <= 8 * e
+    grids = (codebooks.get_iq2xxs_signed_grid_tensor().to(DEV), codebooks.get_iq1_grid_tensor().to(DEV))
+    dw1, dw3, dw2 = (torch.from_numpy(a).to(DEV) for a in (w1, w3, w2))
+    tid = O.TYPE_IDS
+    print(f"case routes as matrix rows {dtype}", flush=True)
+    y = mod.gguf_moe_prefill_grouped_forward(x, toks, rws, seg, dw1, dw3, dw2, d, tid["iq2_xxs"], d, tid["iq2_xxs"], inter, tid["iq1_m"], grids, 0.0)
+    torch.cuda.synchronize()
+    route_experts = np.repeat(np.arange(e), counts)
+    want = O.moe_forward(x.float().cpu().numpy(), o_toks, o_rws, route_experts, w1, w3, w2, "iq2_xxs", "iq2_xxs", "iq1_m", 0.0)
+    got = y.float().cpu().numpy()
+    for tok in range(t):                                    # per token: the rows differ by ten orders of magnitude
+        if np.abs(want[tok]).max() > 0:
+            assert O.rel_l2(got[tok], want[tok]) <= TOL, tok
+        else:
+            assert not got[tok].any(), tok
+
+
+def test_grouped_experts_below_the_matrix_row_threshold(mod):
+    """Fewer than 1.5 routes per expert: the integer form (one decode per expert, the routes one after the other)."""
+    rng = np.random.default_rng(78)
+    e, d, inter, topk, t = 12, 512, 512, 2, 7
+    w1 = _expert_blocks(rng, "iq2_xxs", e, inter, d)
+    w3 = _expert_blocks(rng, "iq2_xxs", e, inter, d)
+    w2 = _expert_blocks(rng, "iq1_m", e, d, inter)
+    idx, wts = _route(rng, t, e, topk)
+    x = torch.from_numpy(rng.standard_normal((t, d)).astype(np.float32)).to(DEV).to(torch.bfloat16)
+    _, toks, rws, seg = mod.moe_group_routes(torch.from_numpy(idx).to(DEV), torch.from_numpy(wts).to(DEV), 0, e)
+    _, o_toks, o_rws, o_seg = O.group_routes(idx, wts, 0, e)
+    assert 2 * len(o_toks) < 3 * e
+    grids = (codebooks.get_iq2xxs_signed_grid_tensor().to(DEV), codebooks.get_iq1_grid_tensor().to(DEV))
+    dw1, dw3, dw2 = (torch.from_numpy(a).to(DEV) for a in (w1, w3, w2))
+    tid = O.TYPE_IDS
+    print("case grouped experts below the matrix-row threshold", flush=True)
+    y = mod.gguf_moe_prefill_grouped_forward(x, toks, rws, seg, dw1, dw3, dw2, d, tid["iq2_xxs"], d, tid["iq2_xxs"], inter, tid["iq1_m"], grids, 0.0)
+    torch.cuda.synchronize()
+    route_experts = np.repeat(np.arange(e), np.diff(o_seg))
+    want = O.moe_forward(x.float().cpu().numpy(), o_toks, o_rws, route_experts, w1, w3, w2, "iq2_xxs", "iq2_xxs", "iq1_m", 0.0)
+    assert O.rel_l2(y.cpu().numpy(), want) <= TOL
+
+
 @pytest.mark.parametrize("t13,t2,limit", [("iq2_xxs", "iq1_m", 0.0), ("iq2_xxs", "q2_k", 0.7), ("iq1_m", "iq1_m", 0.0)])
 def test_grouped_experts_tile_path(mod, t13, t2, limit):
     """Sixteen tokens or more: the routes of every expert go through the MFMA tile kernel as one batch of matmuls
