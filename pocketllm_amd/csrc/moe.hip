@@ -11,6 +11,8 @@
 //   3. the routed matvec of matvec_dot4.hip computes W2_e h_r per route into a float32 [R, D] scratch.
 //   4. moe_reduce_kernel sums each token's routes in ascending route order: the result does not
 //      depend on scheduling (the reference accumulates with atomicAdd).
+#include <algorithm>
+
 #include "block_dot4.h"
 #include "pllm_internal.h"
 
@@ -343,44 +345,67 @@ __global__ void narrow_experts_kernel(const int64_t* __restrict__ src, int32_t* 
     if (r < routes) dst[r] = static_cast<int32_t>(src[r]);
 }
 
-// y[t, d] = sum_{r : route_tokens[r] == t} partial[r, d], ascending r.  grid (tokens, ceil(dim / 256)).
-// The workgroup first lists the routes of its token in LDS (every thread scans a contiguous run of
-// the route table, an exclusive scan of the per-thread counts keeps the list in route order), then
-// adds them.  route_tokens == nullptr: a single token owns every route.
+// y[t, d] = sum_{r : route_tokens[r] == t} partial[r, d], ascending r.  grid (tokens, column groups): a workgroup owns the
+// columns blockIdx.y * 256 + tid + k * gridDim.y * 256.  It first lists the routes of its token in LDS (every thread scans a
+// contiguous run of the route table, an exclusive scan of the per-thread counts keeps the list in route order), then adds
+// them.  route_tokens == nullptr: a single token owns every route.
 constexpr int kReduceList = 2048;
 __global__ __launch_bounds__(256) void moe_reduce_kernel(const float* __restrict__ partial, const int64_t* __restrict__ route_tokens,
                                                          float* __restrict__ y, int routes, int dim) {
     __shared__ int list[kReduceList];
-    __shared__ int offs[257];
+    __shared__ int wave_total[4];
     const int t = blockIdx.x, tid = threadIdx.x;
-    const int d = blockIdx.y * 256 + tid;
-    float acc = 0.0f;
+    const int d0 = blockIdx.y * 256 + tid, dstep = gridDim.y * 256;
     if (!route_tokens) {
-        if (d < dim)
+        for (int d = d0; d < dim; d += dstep) {
+            float acc = 0.0f;
             for (int r = 0; r < routes; ++r) acc += partial[static_cast<size_t>(r) * dim + d];
+            y[static_cast<size_t>(t) * dim + d] = acc;
+        }
     } else if (routes <= kReduceList) {
         const int per = (routes + 255) / 256;
         const int r0 = min(tid * per, routes), r1 = min(r0 + per, routes);
         int cnt = 0;
         for (int r = r0; r < r1; ++r) cnt += route_tokens[r] == t;
-        offs[tid + 1] = cnt;
-        if (tid == 0) offs[0] = 0;
+        int incl = cnt;                                     // inclusive scan over the wave, then over the four waves
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int v = __shfl_up(incl, off, 64);
+            if ((tid & 63) >= off) incl += v;
+        }
+        if ((tid & 63) == 63) wave_total[tid >> 6] = incl;
         __syncthreads();
-        if (tid == 0)
-            for (int i = 1; i <= 256; ++i) offs[i] += offs[i - 1];
-        __syncthreads();
-        int pos = offs[tid];
+        int pos = incl - cnt, total = 0;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            if (w < (tid >> 6)) pos += wave_total[w];
+            total += wave_total[w];
+        }
         for (int r = r0; r < r1; ++r)
             if (route_tokens[r] == t) list[pos++] = r;
         __syncthreads();
-        const int total = offs[256];
-        if (d < dim)
+        for (int d = d0; d < dim; d += dstep) {
+            float acc = 0.0f;
             for (int i = 0; i < total; ++i) acc += partial[static_cast<size_t>(list[i]) * dim + d];
-    } else if (d < dim) {
-        for (int r = 0; r < routes; ++r)
-            if (route_tokens[r] == t) acc += partial[static_cast<size_t>(r) * dim + d];
+            y[static_cast<size_t>(t) * dim + d] = acc;
+        }
+    } else {
+        for (int d = d0; d < dim; d += dstep) {
+            float acc = 0.0f;
+            for (int r = 0; r < routes; ++r)
+                if (route_tokens[r] == t) acc += partial[static_cast<size_t>(r) * dim + d];
+            y[static_cast<size_t>(t) * dim + d] = acc;
+        }
     }
-    if (d < dim) y[static_cast<size_t>(t) * dim + d] = acc;
+}
+
+// (with many tokens a workgroup takes several column groups, so that the route table is scanned by about a thousand workgroups at most)
+int launch_moe_reduce(const float* partial, const int64_t* route_tokens, float* y, int64_t tokens, int routes, int dim, hipStream_t s) {
+    const int col_groups = (dim + 255) / 256;
+    const int per_token = static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(col_groups, 1024 / std::max<int64_t>(tokens, 1))));
+    hipLaunchKernelGGL(moe_reduce_kernel, dim3(static_cast<unsigned>(tokens), static_cast<unsigned>(per_token)), dim3(256), 0, s, partial, route_tokens, y,
+                       routes, dim);
+    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 
 // ---- route grouping ---------------------------------------------------------------------------
@@ -553,9 +578,7 @@ int pllm_gguf_moe_forward(const void* x, int x_dtype, int64_t tokens, int64_t di
         if (st != PLLM_OK) return st;
         st = moe_rows_w2(h_rows, I, seg_starts, w2, part, D, E, R, s);
         if (st != PLLM_OK) return st;
-        dim3 rg(static_cast<unsigned>(tokens), static_cast<unsigned>((dim + 255) / 256));
-        hipLaunchKernelGGL(moe_reduce_kernel, rg, dim3(256), 0, s, part, route_tokens, y, R, D);
-        return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+        return launch_moe_reduce(part, route_tokens, y, tokens, R, D, s);
     }
     if (seg_starts && tokens > 1 && routes <= kMoeGroupedMaxRoutesPerExpert * n_experts &&
         moe_grouped_mfma_supports(w13_type, w2_type, static_cast<int>(dim), static_cast<int>(inter), w1, w3, w2)) {
@@ -572,9 +595,7 @@ int pllm_gguf_moe_forward(const void* x, int x_dtype, int64_t tokens, int64_t di
         if (st != PLLM_OK) return st;
         st = moe_grouped_w2_mfma(h_img, hs, I, seg_starts, w2, part, D, E, s);
         if (st != PLLM_OK) return st;
-        dim3 rg(static_cast<unsigned>(tokens), static_cast<unsigned>((dim + 255) / 256));
-        hipLaunchKernelGGL(moe_reduce_kernel, rg, dim3(256), 0, s, part, route_tokens, y, R, D);
-        return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+        return launch_moe_reduce(part, route_tokens, y, tokens, R, D, s);
     }
     if (seg_starts && tokens >= kMoeGemmMinTokens) {
         // tile path: gather the routes' activation rows as fp16, gate and up as two batches of tile
@@ -600,9 +621,7 @@ int pllm_gguf_moe_forward(const void* x, int x_dtype, int64_t tokens, int64_t di
         if (st != PLLM_OK) return st;
         st = gemm_f16_grouped(h_staged, w2, w2_type, stride2, seg_starts, E, part, R, max_group, D, bpr_h, s);
         if (st != PLLM_OK) return st;
-        dim3 rg(static_cast<unsigned>(tokens), static_cast<unsigned>((dim + 255) / 256));
-        hipLaunchKernelGGL(moe_reduce_kernel, rg, dim3(256), 0, s, part, route_tokens, y, R, D);
-        return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+        return launch_moe_reduce(part, route_tokens, y, tokens, R, D, s);
     }
     const size_t x_stride = act_image_256_bytes(bpr_x), h_stride = act_image_256_bytes(bpr_h);
     if (!dot4_type(w13_type) || !dot4_type(w2_type)) {
@@ -640,9 +659,7 @@ int pllm_gguf_moe_forward(const void* x, int x_dtype, int64_t tokens, int64_t di
         if (hipGetLastError() != hipSuccess) return PLLM_ERR_LAUNCH;
         st = superblock_matvec(act_rows_from_image(h_image, h_stride), w2, w2_type, partial, PLLM_F32, R, D, bpr_h, s, r2);
         if (st != PLLM_OK) return st;
-        dim3 rg(static_cast<unsigned>(tokens), static_cast<unsigned>((dim + 255) / 256));
-        hipLaunchKernelGGL(moe_reduce_kernel, rg, dim3(256), 0, s, partial, tokens > 1 ? route_tokens : nullptr, y, R, D);
-        return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+        return launch_moe_reduce(partial, tokens > 1 ? route_tokens : nullptr, y, tokens, R, D, s);
     }
     if (tokens == 1 && route_experts && routes * staged_x_bytes(bpr_h * 256) <= 96 * 1024) {
         // single token: two launches.  Gate/up read the raw activation row and the int64 expert ids
@@ -702,9 +719,7 @@ int pllm_gguf_moe_forward(const void* x, int x_dtype, int64_t tokens, int64_t di
             default: st = launch_w2_grouped<Q2K>(h_image, h_stride, bpr_h, seg_starts, w2, stride2, partial, static_cast<int>(dim), E, s); break;
         }
         if (st != PLLM_OK) return st;
-        dim3 rg(static_cast<unsigned>(tokens), static_cast<unsigned>((dim + 255) / 256));
-        hipLaunchKernelGGL(moe_reduce_kernel, rg, dim3(256), 0, s, partial, route_tokens, y, R, static_cast<int>(dim));
-        return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+        return launch_moe_reduce(partial, route_tokens, y, tokens, R, static_cast<int>(dim), s);
     }
     switch (w13_type) {
         case PLLM_TYPE_IQ2_XXS:
@@ -723,9 +738,7 @@ int pllm_gguf_moe_forward(const void* x, int x_dtype, int64_t tokens, int64_t di
     st = dot4_routed_matvec_from_image(h_image, h_stride, w2, w2_type, partial, PLLM_F32, R, static_cast<int>(dim), bpr_h, experts32,
                                        w2_expert_stride, s);
     if (st != PLLM_OK) return st;
-    dim3 rgrid(static_cast<unsigned>(tokens), static_cast<unsigned>((dim + 255) / 256));
-    hipLaunchKernelGGL(moe_reduce_kernel, rgrid, dim3(256), 0, s, partial, tokens > 1 ? route_tokens : nullptr, y, R, static_cast<int>(dim));
-    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+    return launch_moe_reduce(partial, tokens > 1 ? route_tokens : nullptr, y, tokens, R, static_cast<int>(dim), s);
 }
 
 int pllm_moe_group_routes(const void* indices, int indices_are_i64, const float* weights, int64_t tokens, int64_t topk,
