@@ -37,6 +37,19 @@ __device__ __forceinline__ float scale_at(const void* __restrict__ scale, size_t
     else return static_cast<const float*>(scale)[i];
 }
 
+// a scale entry as loaded (no conversion yet, so that the load can stay in flight) and its value
+template <int F16S>
+__device__ __forceinline__ uint32_t scale_raw_at(const void* __restrict__ scale, size_t i) {
+    if constexpr (F16S == 0) return __float_as_uint(static_cast<const float*>(scale)[i]);
+    else return static_cast<const uint16_t*>(scale)[i];
+}
+template <int F16S>
+__device__ __forceinline__ float scale_value(uint32_t raw) {
+    if constexpr (F16S == 1) return f16_bits_to_float(raw);
+    else if constexpr (F16S == 2) return __uint_as_float(raw << 16);
+    else return __uint_as_float(raw);
+}
+
 __device__ __forceinline__ float silu(float v) { return v / (1.0f + __expf(-v)); }
 
 // The activation row as float32 in LDS (k a multiple of 16 on the callers' path): four values per lane and trip, one vector
@@ -86,8 +99,8 @@ __device__ __forceinline__ void stage_row_finish(float* xs, const float (&v)[kSt
 // gate and of the up matrix.
 template <bool SWIGLU>
 __device__ __forceinline__ const Fp8Mat& slot_mat(const Fp8Mat& a, const Fp8Mat& b, int q) { return (SWIGLU && q == 1) ? b : a; }
-template <bool SWIGLU>
-__device__ __forceinline__ int slot_row(int row0, int q, int n) { return min(SWIGLU ? row0 : row0 + q, n - 1); }
+// (plain form: the second slot's row lies rstride rows behind the first one's, in the workgroup's next group of rows)
+__device__ __forceinline__ int slot_row(int row0, int q, int rstride, int n) { return min(row0 + q * rstride, n - 1); }
 
 __device__ __forceinline__ float chunk_dot(const uint4& w, const float* xp) {
     const float4 x0 = *reinterpret_cast<const float4*>(xp);
@@ -111,11 +124,21 @@ __device__ __forceinline__ float chunk_dot(const uint4& w, const float* xp) {
 // row once and then walks groups of 8 weight rows (two per wave) in passes of 64 * 16 * ITERS bytes
 // per row, always holding the loads of its next pass (of the same group or of its next group) in a
 // second register set while it multiplies the current one.
-template <int ITERS, bool SWIGLU>
-__device__ __forceinline__ void fp8_fetch_pass(uint4 (&r)[kRowsPerWave][ITERS], const Fp8Mat& ma, const Fp8Mat& mb, int row0, int n, int chunks, int c0, int lane) {
+// The block scales of a pass travel with its weights, requested ahead of them: loads return in order, so a scale asked for
+// while the pass is multiplied would arrive behind the weights of the pass after it and hold the arithmetic until those are in.
+template <int ITERS, int F16S, bool SWIGLU>
+__device__ __forceinline__ void fp8_fetch_pass(uint4 (&r)[kRowsPerWave][ITERS], uint32_t (&sc)[kRowsPerWave][ITERS], const Fp8Mat& ma, const Fp8Mat& mb,
+                                               int row0, int rstride, int n, int chunks, int c0, int lane) {
 #pragma unroll
     for (int q = 0; q < kRowsPerWave; ++q) {
-        const uint8_t* wrow = slot_mat<SWIGLU>(ma, mb, q).w + static_cast<size_t>(slot_row<SWIGLU>(row0, q, n)) * slot_mat<SWIGLU>(ma, mb, q).wstride;
+        const Fp8Mat& m = slot_mat<SWIGLU>(ma, mb, q);
+        const size_t srow = static_cast<size_t>(slot_row(row0, q, rstride, n) >> 7) * m.sstride;
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) sc[q][it] = scale_raw_at<F16S>(m.scale, srow + (min(c0 + it * 64 + lane, chunks - 1) >> 3));
+    }
+#pragma unroll
+    for (int q = 0; q < kRowsPerWave; ++q) {
+        const uint8_t* wrow = slot_mat<SWIGLU>(ma, mb, q).w + static_cast<size_t>(slot_row(row0, q, rstride, n)) * slot_mat<SWIGLU>(ma, mb, q).wstride;
 #pragma unroll
         for (int it = 0; it < ITERS; ++it) r[q][it] = *reinterpret_cast<const uint4*>(wrow + 16 * min(c0 + it * 64 + lane, chunks - 1));
     }
@@ -149,8 +172,8 @@ __device__ __forceinline__ float floats_dot(const float (&f)[16], const float* x
 
 // R activation rows (xs holds them k floats apart) against the pass's weights: the codes are converted once per chunk
 template <int ITERS, int F16S, bool SWIGLU, int R>
-__device__ __forceinline__ void fp8_multiply_pass(float (&acc)[kRowsPerWave][R], const uint4 (&r)[kRowsPerWave][ITERS], const float* xs, int k,
-                                                  const Fp8Mat& ma, const Fp8Mat& mb, int row0, int n, int chunks, int c0, int lane) {
+__device__ __forceinline__ void fp8_multiply_pass(float (&acc)[kRowsPerWave][R], const uint4 (&r)[kRowsPerWave][ITERS],
+                                                  const uint32_t (&scales)[kRowsPerWave][ITERS], const float* xs, int k, int chunks, int c0, int lane) {
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
         const int c = c0 + it * 64 + lane;
@@ -158,8 +181,7 @@ __device__ __forceinline__ void fp8_multiply_pass(float (&acc)[kRowsPerWave][R],
         const int cc = ok ? c : 0;
 #pragma unroll
         for (int q = 0; q < kRowsPerWave; ++q) {
-            const Fp8Mat& m = slot_mat<SWIGLU>(ma, mb, q);
-            const float sc = scale_at<F16S>(m.scale, static_cast<size_t>(slot_row<SWIGLU>(row0, q, n) >> 7) * m.sstride + (cc >> 3));
+            const float sc = scale_value<F16S>(scales[q][it]);
             if constexpr (R == 1) {
                 const float d = chunk_dot(r[q][it], xs + 16 * cc);
                 acc[q][0] += ok ? d * sc : 0.0f;
@@ -179,7 +201,7 @@ __device__ __forceinline__ void fp8_multiply_pass(float (&acc)[kRowsPerWave][R],
 // activation rows arow0 .. arow0 + R - 1 (those below total_rows) of output row(s) row0
 template <bool SWIGLU, int R>
 __device__ __forceinline__ void fp8_store_rows(float (&acc)[kRowsPerWave][R], void* __restrict__ y, int y_dtype, size_t y_stride, int arow0, int total_rows,
-                                               int row0, int n, int lane) {
+                                               int row0, int rstride, int n, int lane) {
 #pragma unroll
     for (int a = 0; a < R; ++a) {
         float total[kRowsPerWave];
@@ -192,7 +214,7 @@ __device__ __forceinline__ void fp8_store_rows(float (&acc)[kRowsPerWave][R], vo
         } else {
 #pragma unroll
             for (int q = 0; q < kRowsPerWave; ++q)
-                if (lane == 0 && row0 + q < n) store_any(y, y_dtype, yoff + row0 + q, total[q]);
+                if (lane == 0 && row0 + q * rstride < n) store_any(y, y_dtype, yoff + row0 + q * rstride, total[q]);
         }
     }
 }
@@ -209,12 +231,17 @@ __global__ __launch_bounds__(kThreads) void fp8_persistent_matvec_kernel(
     const int wave = tid >> 6;
     const int chunks = k >> 4;
     const int arow0 = blockIdx.y * R;                                        // this workgroup's first activation row
-    constexpr int per_wave = SWIGLU ? 1 : kRowsPerWave;
     constexpr int kPassChunks = 64 * ITERS;
-    const int rows_per_group = kWaves * per_wave, wave_row = wave * per_wave;
-    const int step = gridDim.x;
+    // A group = kWaves rows, one per wave.  SWIGLU: the wave's two slots hold its row of the gate and of the up matrix.  Plain: the
+    // slots hold the wave's rows of two groups, this workgroup's current and its next one (groups are dealt round-robin, so the
+    // workgroups' loads differ by at most one group, not by a pair of them).
+    constexpr int rows_per_group = kWaves;
+    const int wave_row = wave;
+    const int step = SWIGLU ? gridDim.x : 2 * gridDim.x;
+    const int rstride = SWIGLU ? 0 : rows_per_group * static_cast<int>(gridDim.x);
 
     uint4 a[kRowsPerWave][ITERS], b[kRowsPerWave][ITERS];
+    uint32_t sa[kRowsPerWave][ITERS], sb[kRowsPerWave][ITERS];
     float acc[kRowsPerWave][R];
 #pragma unroll
     for (int q = 0; q < kRowsPerWave; ++q)
@@ -226,10 +253,10 @@ __global__ __launch_bounds__(kThreads) void fp8_persistent_matvec_kernel(
         float head[kStageBatch][4];
         const size_t xoff = static_cast<size_t>(arow0) * x_stride;
         stage_row_request(head, x, x_dtype, xoff, k);
-        fp8_fetch_pass<ITERS, SWIGLU>(a, ma, mb, g * rows_per_group + wave_row, n, chunks, 0, lane);
+        fp8_fetch_pass<ITERS, F16S, SWIGLU>(a, sa, ma, mb, g * rows_per_group + wave_row, rstride, n, chunks, 0, lane);
         stage_row_finish(xs, head, x, x_dtype, xoff, k);
     } else {
-        fp8_fetch_pass<ITERS, SWIGLU>(a, ma, mb, g * rows_per_group + wave_row, n, chunks, 0, lane);
+        fp8_fetch_pass<ITERS, F16S, SWIGLU>(a, sa, ma, mb, g * rows_per_group + wave_row, rstride, n, chunks, 0, lane);
 #pragma unroll 1
         for (int r = 0; r < R; ++r)          // rows past the end: the last row again, result dropped
             stage_row_f32(xs + static_cast<size_t>(r) * k, x, x_dtype, static_cast<size_t>(min(arow0 + r, total_rows - 1)) * x_stride, k);
@@ -237,15 +264,17 @@ __global__ __launch_bounds__(kThreads) void fp8_persistent_matvec_kernel(
     __syncthreads();
     while (g < groups) {
         if (++pn == passes) { pn = 0; gn += step; }
-        if (gn < groups) fp8_fetch_pass<ITERS, SWIGLU>(b, ma, mb, gn * rows_per_group + wave_row, n, chunks, pn * kPassChunks, lane);
-        fp8_multiply_pass<ITERS, F16S, SWIGLU, R>(acc, a, xs, k, ma, mb, g * rows_per_group + wave_row, n, chunks, p * kPassChunks, lane);
-        if (p == passes - 1) fp8_store_rows<SWIGLU, R>(acc, y, y_dtype, y_stride, arow0, total_rows, g * rows_per_group + wave_row, n, lane);
+        // (fetched without a condition, past the last group its rows again: a branch around the loads would make the compiler wait
+        // for them at the join, ahead of the arithmetic on the other register set)
+        fp8_fetch_pass<ITERS, F16S, SWIGLU>(b, sb, ma, mb, min(gn, groups - 1) * rows_per_group + wave_row, rstride, n, chunks, pn * kPassChunks, lane);
+        fp8_multiply_pass<ITERS, F16S, SWIGLU, R>(acc, a, sa, xs, k, chunks, p * kPassChunks, lane);
+        if (p == passes - 1) fp8_store_rows<SWIGLU, R>(acc, y, y_dtype, y_stride, arow0, total_rows, g * rows_per_group + wave_row, rstride, n, lane);
         g = gn; p = pn;
         if (g >= groups) break;
         if (++pn == passes) { pn = 0; gn += step; }
-        if (gn < groups) fp8_fetch_pass<ITERS, SWIGLU>(a, ma, mb, gn * rows_per_group + wave_row, n, chunks, pn * kPassChunks, lane);
-        fp8_multiply_pass<ITERS, F16S, SWIGLU, R>(acc, b, xs, k, ma, mb, g * rows_per_group + wave_row, n, chunks, p * kPassChunks, lane);
-        if (p == passes - 1) fp8_store_rows<SWIGLU, R>(acc, y, y_dtype, y_stride, arow0, total_rows, g * rows_per_group + wave_row, n, lane);
+        fp8_fetch_pass<ITERS, F16S, SWIGLU>(a, sa, ma, mb, min(gn, groups - 1) * rows_per_group + wave_row, rstride, n, chunks, pn * kPassChunks, lane);
+        fp8_multiply_pass<ITERS, F16S, SWIGLU, R>(acc, b, sb, xs, k, chunks, p * kPassChunks, lane);
+        if (p == passes - 1) fp8_store_rows<SWIGLU, R>(acc, y, y_dtype, y_stride, arow0, total_rows, g * rows_per_group + wave_row, rstride, n, lane);
         g = gn; p = pn;
     }
 }
@@ -302,8 +331,7 @@ int launch_any(const void* x, int x_dtype, size_t x_stride, const Fp8Mat& ma, co
                            y, y_dtype, y_stride, k, n);
         return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
     }
-    const int rows_per_group = kWaves * (SWIGLU ? 1 : kRowsPerWave);
-    const int groups = (n + rows_per_group - 1) / rows_per_group;
+    const int groups = (n + kWaves - 1) / kWaves;                            // one row per wave; a workgroup multiplies two groups at a time (SWIGLU: one, both matrices)
     const int niter = ((k >> 4) + 63) / 64;
     const int passes = (niter + 5) / 6;
     const int iters = (niter + passes - 1) / passes;
@@ -314,7 +342,7 @@ int launch_any(const void* x, int x_dtype, size_t x_stride, const Fp8Mat& ma, co
     // persistent: the workgroups that fit a compute unit at once (two by registers, fewer when the activation rows fill LDS),
     // groups dealt round-robin
     const int per_cu = std::max(1, std::min(2, static_cast<int>((160 * 1024) / std::max<size_t>(smem, 1))));
-    const int grid_x = std::min(groups, per_cu * compute_units());
+    const int grid_x = std::min(SWIGLU ? groups : (groups + 1) / 2, per_cu * compute_units());
     const dim3 grid(grid_x, (rows + share - 1) / share);
     // (the form with a compile-time pass count keeps both register sets and all accumulators of several rows live at once and spills;
     // several activation rows always run the form with the pass count as a variable)
