@@ -73,9 +73,12 @@ __global__ __launch_bounds__(256, 2) void fp8_gemm_kernel(
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
     uint4 ra0, ra1, ra2, ra3, rb0, rb1, rb2, rb3;
-    float rs = 0.0f;
+    float rs = 0.0f, rws = 0.0f;
+    // the step's codes and both scales: everything a step needs from memory is requested one step ahead (loads return in
+    // order, so a scale asked for inside the step would arrive behind the next step's codes)
     auto fetch = [&](int s) {
         const size_t off = static_cast<size_t>(s) * kStep;
+        rws = bs_src[s];
         ra0 = *reinterpret_cast<const uint4*>(as0 + off); ra1 = *reinterpret_cast<const uint4*>(as1 + off);
         ra2 = *reinterpret_cast<const uint4*>(as2 + off); ra3 = *reinterpret_cast<const uint4*>(as3 + off);
         rb0 = *reinterpret_cast<const uint4*>(bs0 + off); rb1 = *reinterpret_cast<const uint4*>(bs1 + off);
@@ -97,8 +100,8 @@ __global__ __launch_bounds__(256, 2) void fp8_gemm_kernel(
     __syncthreads();
     for (int s = 0; s < steps; ++s) {
         const int buf = s & 1;
-        if (s + 1 < steps) fetch(s + 1);
-        const float ws = bs_src[s];
+        const float ws = rws;
+        fetch(min(s + 1, steps - 1));        // (no branch around the loads: the last step fetches itself again and drops it)
         const unsigned char* at = a_tile + buf * kTile * kRow + (wm * 64 + (lane & 31)) * kRow + 32 * (lane >> 5);
         const unsigned char* bt = b_tile + buf * kTile * kRow + (wn * 64 + (lane & 31)) * kRow + 32 * (lane >> 5);
         floatx16 c[2][2];

@@ -214,6 +214,36 @@ __device__ __forceinline__ void load_row4(float v[4], const void* __restrict__ x
     }
 }
 
+// N pieces of four consecutive values (piece j at element e0[j], whole and 8- / 16-byte aligned: the caller checks), all loads in
+// flight together.  The type is told apart once around the batch: a branch per piece would end every load in a wait of its own.
+template <int N>
+__device__ __forceinline__ void load_rows4_batch(float (&v)[N][4], const void* __restrict__ x, int x_dtype, size_t xoff, const int (&e0)[N]) {
+    if (x_dtype == PLLM_F32) {
+        float4 w[N];
+#pragma unroll
+        for (int j = 0; j < N; ++j) w[j] = *reinterpret_cast<const float4*>(static_cast<const float*>(x) + xoff + e0[j]);
+#pragma unroll
+        for (int j = 0; j < N; ++j) { v[j][0] = w[j].x; v[j][1] = w[j].y; v[j][2] = w[j].z; v[j][3] = w[j].w; }
+    } else {
+        uint2 w[N];
+#pragma unroll
+        for (int j = 0; j < N; ++j) w[j] = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(x) + xoff + e0[j]);
+        if (x_dtype == PLLM_BF16) {
+#pragma unroll
+            for (int j = 0; j < N; ++j) {
+                v[j][0] = __uint_as_float(w[j].x << 16); v[j][1] = __uint_as_float(w[j].x & 0xffff0000u);
+                v[j][2] = __uint_as_float(w[j].y << 16); v[j][3] = __uint_as_float(w[j].y & 0xffff0000u);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < N; ++j) {
+                v[j][0] = f16_bits_to_float(w[j].x & 0xffffu); v[j][1] = f16_bits_to_float(w[j].x >> 16);
+                v[j][2] = f16_bits_to_float(w[j].y & 0xffffu); v[j][3] = f16_bits_to_float(w[j].y >> 16);
+            }
+        }
+    }
+}
+
 // One lane's four values into the image at e0 (hi, lo, and the group figures from the lanes that own them).
 __device__ __forceinline__ void quantize4_to_image(const float v[4], int e0, int8_t* hi, int8_t* lo, float2* gs, float* sum16) {
     uint32_t qh, ql;

@@ -47,7 +47,8 @@ __global__ __launch_bounds__(kThreads) void route_logits_kernel(
 #pragma unroll
     for (int i = 0; i < kHeld; ++i) {
         const int c = lane * 4 + 256 * i;
-        held[i] = c < dim ? *reinterpret_cast<const float4*>(grow + c) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        const float4 gv = *reinterpret_cast<const float4*>(grow + min(c, dim - 4));
+        held[i] = c < dim ? gv : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     }
     // all tokens of the group side by side: their loads are independent and go out together
     const bool xvec = ((reinterpret_cast<uintptr_t>(x) & 15u) == 0) && (x_dtype != PLLM_F32 ? dim % 4 == 0 : true);
@@ -58,16 +59,24 @@ __global__ __launch_bounds__(kThreads) void route_logits_kernel(
         acc[j] = 0.0f;
         xoff[j] = static_cast<size_t>(min(t0 + j, t1 - 1)) * dim;            // past the end: the last token again, result dropped
     }
+    // (no branch around the loads: pieces beyond the row read its last piece again and are dropped; a branch per piece would
+    // make every piece wait for its own round trip)
+    int cpos[kHeld];
 #pragma unroll
-    for (int i = 0; i < kHeld; ++i) {
-        const int c = lane * 4 + 256 * i;
-        if (c < dim) {
+    for (int i = 0; i < kHeld; ++i) cpos[i] = min(lane * 4 + 256 * i, max(dim - 4, 0));
 #pragma unroll
-            for (int j = 0; j < NT; ++j) {
-                float v[4];
-                load_row4(v, x, x_dtype, xoff[j], c, dim, xvec);
-                acc[j] += held[i].x * v[0] + held[i].y * v[1] + held[i].z * v[2] + held[i].w * v[3];
-            }
+    for (int j = 0; j < NT; ++j) {
+        float v[kHeld][4];
+        if (xvec) {
+            load_rows4_batch(v, x, x_dtype, xoff[j], cpos);
+        } else {
+#pragma unroll
+            for (int i = 0; i < kHeld; ++i) load_row4(v[i], x, x_dtype, xoff[j], cpos[i], dim, false);
+        }
+#pragma unroll
+        for (int i = 0; i < kHeld; ++i) {
+            const float d = held[i].x * v[i][0] + held[i].y * v[i][1] + held[i].z * v[i][2] + held[i].w * v[i][3];
+            acc[j] += (lane * 4 + 256 * i < dim) ? d : 0.0f;
         }
     }
     for (int c = lane * 4 + 256 * kHeld; c < dim; c += 256) {               // rows wider than the held part
@@ -136,6 +145,17 @@ __global__ __launch_bounds__(kThreads) void route_logits_mfma_kernel(
 
 __device__ __forceinline__ float wave_max(float v) { return group_max<64>(v); }
 
+// the maximum over the wave as a wave-uniform value: butterflies inside the rows of 16 lanes, then the four rows' results
+// through scalar registers (no LDS crossbar)
+__device__ __forceinline__ float wave_max_uniform(float v) {
+    v = group_max<16>(v);
+    const float r0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0)), r1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+    const float r2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32)), r3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+    return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
+}
+
+// PER = candidates per lane (expert lane + 64 i)
+template <int PER>
 __global__ __launch_bounds__(64) void route_topk_kernel(
     const float* __restrict__ logits, const float* __restrict__ bias, int n_experts, int top_k, int softmax_mode,
     int64_t* __restrict__ indices, float* __restrict__ weights) {
@@ -143,23 +163,19 @@ __global__ __launch_bounds__(64) void route_topk_kernel(
     const size_t t = blockIdx.x;
     const float* row = logits + t * n_experts;
     constexpr float kGone = -3.0e38f;
-    float score[kMaxPerLane], prob[kMaxPerLane];
+    float score[PER], prob[PER], l[PER], bv[PER];
 #pragma unroll
-    for (int i = 0; i < kMaxPerLane; ++i) {
-        const int e = lane + 64 * i;
-        score[i] = kGone;
-        prob[i] = 0.0f;
-        if (e < n_experts) {
-            const float l = row[e];
-            if (softmax_mode) {
-                score[i] = l;
-                prob[i] = l;
-            } else {
-                const float p = 1.0f / (1.0f + expf(-l));
-                prob[i] = p;
-                score[i] = bias ? p + bias[e] : p;
-            }
-        }
+    for (int i = 0; i < PER; ++i) {                                         // all loads first, past the end the last expert again
+        const int e = min(lane + 64 * i, n_experts - 1);
+        l[i] = row[e];
+        bv[i] = bias ? bias[e] : 0.0f;
+    }
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const bool live = lane + 64 * i < n_experts;
+        const float p = softmax_mode ? l[i] : 1.0f / (1.0f + expf(-l[i]));
+        prob[i] = live ? p : 0.0f;
+        score[i] = live ? (softmax_mode ? p : p + bv[i]) : kGone;
     }
     // top_k rounds; lane r keeps the r-th pick
     int my_pick = -1;
@@ -168,21 +184,29 @@ __global__ __launch_bounds__(64) void route_topk_kernel(
         float best = kGone;
         int best_e = 0x7fffffff;
 #pragma unroll
-        for (int i = 0; i < kMaxPerLane; ++i) {                             // ascending expert id inside the lane: strict > keeps the lowest
+        for (int i = 0; i < PER; ++i) {                                     // ascending expert id inside the lane: strict > keeps the lowest
             if (score[i] > best) { best = score[i]; best_e = lane + 64 * i; }
         }
-        const float top = wave_max(best);
-        // the lowest expert id among the lanes that hold the maximum
-        int cand = (best == top) ? best_e : 0x7fffffff;
+        const float top = wave_max_uniform(best);
+        // the lowest expert id among the lanes that hold the maximum: one lane almost always, else a wave-wide minimum
+        const unsigned long long holders = __ballot(best == top);
+        int cand;
+        if (__popcll(holders) == 1) {
+            cand = __builtin_amdgcn_readlane(best_e, static_cast<int>(__ffsll(static_cast<long long>(holders))) - 1);
+        } else {
+            cand = (best == top) ? best_e : 0x7fffffff;
 #pragma unroll
-        for (int off = 1; off < 64; off <<= 1) cand = min(cand, __shfl_xor(cand, off, 64));
+            for (int off = 1; off < 64; off <<= 1) cand = min(cand, __shfl_xor(cand, off, 64));
+            cand = __builtin_amdgcn_readfirstlane(cand);
+        }
         const int owner = cand & 63, slot = cand >> 6;
         float p = 0.0f;
 #pragma unroll
-        for (int i = 0; i < kMaxPerLane; ++i) {
-            if (lane == owner && i == slot) { p = prob[i]; score[i] = kGone; }
+        for (int i = 0; i < PER; ++i) {
+            if (i == slot) p = prob[i];                                     // (wave-uniform slot)
+            if (lane == owner && i == slot) score[i] = kGone;
         }
-        p = __shfl(p, owner, 64);
+        p = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), owner));
         if (lane == r) { my_pick = cand; my_prob = p; }
     }
     // renormalise over the picks (lanes 0 .. top_k - 1)
@@ -226,8 +250,12 @@ int pllm_moe_route(const void* x, int x_dtype, int64_t tokens, int64_t dim, cons
     else
         hipLaunchKernelGGL(route_logits_kernel<kTokensPerWave>, wgs, dim3(kThreads), 0, s, x, x_dtype, gate_weight, logits, static_cast<int>(dim),
                            static_cast<int>(n_experts), static_cast<int>(tokens));
-    hipLaunchKernelGGL(route_topk_kernel, dim3(static_cast<unsigned>(tokens)), dim3(64), 0, s, logits, gate_bias, static_cast<int>(n_experts),
-                       static_cast<int>(top_k), softmax_mode, indices, weights);
+    if (n_experts <= 256)
+        hipLaunchKernelGGL(route_topk_kernel<4>, dim3(static_cast<unsigned>(tokens)), dim3(64), 0, s, logits, gate_bias, static_cast<int>(n_experts),
+                           static_cast<int>(top_k), softmax_mode, indices, weights);
+    else
+        hipLaunchKernelGGL(route_topk_kernel<kMaxPerLane>, dim3(static_cast<unsigned>(tokens)), dim3(64), 0, s, logits, gate_bias,
+                           static_cast<int>(n_experts), static_cast<int>(top_k), softmax_mode, indices, weights);
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 
