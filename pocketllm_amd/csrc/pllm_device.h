@@ -265,6 +265,24 @@ struct RowNorm {
     int round_f16;
 };
 
+// BATCH pieces of four values at base, base + trip, ... of a row of k values padded to kpad (zeros beyond k, pieces beyond kpad
+// untouched): one batch of vector loads when all pieces lie inside the row, piece by piece otherwise (the row's last trips,
+// rows that do not start on a vector boundary).
+template <int BATCH>
+__device__ __forceinline__ void load_row_pieces(float (&v)[BATCH][4], const void* __restrict__ x, int x_dtype, size_t xoff, int base, int trip, int k,
+                                                int kpad, bool vec) {
+    if (vec && base + (BATCH - 1) * trip + 3 < k) {
+        int e0[BATCH];
+#pragma unroll
+        for (int j = 0; j < BATCH; ++j) e0[j] = base + j * trip;
+        load_rows4_batch(v, x, x_dtype, xoff, e0);
+    } else {
+#pragma unroll
+        for (int j = 0; j < BATCH; ++j)
+            if (base + j * trip < kpad) load_row4(v[j], x, x_dtype, xoff, base + j * trip, k, vec);
+    }
+}
+
 template <int BATCH = 6>
 __device__ __forceinline__ void quantize_row_to_lds(unsigned char* lds, const void* __restrict__ x, int x_dtype, size_t xoff, int k, int kpad,
                                                     const RowNorm norm = RowNorm{nullptr, 0.0f, 0}) {
@@ -275,15 +293,27 @@ __device__ __forceinline__ void quantize_row_to_lds(unsigned char* lds, const vo
     // one 8-byte (16-bit inputs) or 16-byte (float32) load per lane and trip when the row starts on that boundary
     const bool vec = x_dtype == PLLM_F32 ? ((reinterpret_cast<uintptr_t>(x) + 4 * xoff) & 15u) == 0
                                          : ((reinterpret_cast<uintptr_t>(x) + 2 * xoff) & 7u) == 0;
+    const bool gvec = (reinterpret_cast<uintptr_t>(norm.gamma) & 15u) == 0;
     const int trip = static_cast<int>(blockDim.x) * 4;
+    const int first = static_cast<int>(threadIdx.x) * 4;
+    const bool one_batch = kpad <= trip * BATCH;                             // the whole row in one batch: read once, also for the norm
+    float v[BATCH][4], g[BATCH][4];
     float rstd = 1.0f;
     if (norm.gamma) {
         // sum of squares of the row: per-wave sums meet in the first floats of the image area, which nobody has written yet
         float ss = 0.0f;
-        for (int e0 = static_cast<int>(threadIdx.x) * 4; e0 < k; e0 += trip) {
-            float v[4];
-            load_row4(v, x, x_dtype, xoff, e0, k, vec);
-            ss += (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
+        if (one_batch) {
+            load_row_pieces<BATCH>(v, x, x_dtype, xoff, first, trip, k, kpad, vec);
+            load_row_pieces<BATCH>(g, norm.gamma, PLLM_F32, 0, first, trip, k, kpad, gvec);   // (now: after the barriers they would cost a round trip of their own)
+#pragma unroll
+            for (int j = 0; j < BATCH; ++j)
+                if (first + j * trip < kpad) ss += (v[j][0] * v[j][0] + v[j][1] * v[j][1]) + (v[j][2] * v[j][2] + v[j][3] * v[j][3]);
+        } else {
+            for (int e0 = first; e0 < k; e0 += trip) {
+                float w[4];
+                load_row4(w, x, x_dtype, xoff, e0, k, vec);
+                ss += (w[0] * w[0] + w[1] * w[1]) + (w[2] * w[2] + w[3] * w[3]);
+            }
         }
         ss = group_sum<64>(ss);
         float* red = reinterpret_cast<float*>(lds);
@@ -294,21 +324,16 @@ __device__ __forceinline__ void quantize_row_to_lds(unsigned char* lds, const vo
         __syncthreads();                                                     // read by everybody before the image overwrites it
         rstd = rsqrtf(total / static_cast<float>(k) + norm.eps);
     }
-    for (int base = static_cast<int>(threadIdx.x) * 4; base < kpad; base += trip * BATCH) {
-        float v[BATCH][4];
-#pragma unroll
-        for (int j = 0; j < BATCH; ++j)
-            if (base + j * trip < kpad) load_row4(v[j], x, x_dtype, xoff, base + j * trip, k, vec);
+    for (int base = first; base < kpad; base += trip * BATCH) {
+        if (!(norm.gamma && one_batch)) load_row_pieces<BATCH>(v, x, x_dtype, xoff, base, trip, k, kpad, vec);
         if (norm.gamma) {
+            if (!one_batch) load_row_pieces<BATCH>(g, norm.gamma, PLLM_F32, 0, base, trip, k, kpad, gvec);
 #pragma unroll
             for (int j = 0; j < BATCH; ++j) {
-                const int e0 = base + j * trip;
-                if (e0 < kpad) {
-                    float g[4];
-                    load_row4(g, norm.gamma, PLLM_F32, 0, e0, k, (reinterpret_cast<uintptr_t>(norm.gamma) & 15u) == 0);
+                if (base + j * trip < kpad) {
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
-                        float t = v[j][i] * rstd * g[i];                     // values past k are zeros on both sides
+                        float t = v[j][i] * rstd * g[j][i];                  // values past k are zeros on both sides
                         if (norm.round_f16) t = static_cast<float>(static_cast<_Float16>(t));
                         v[j][i] = t;
                     }
