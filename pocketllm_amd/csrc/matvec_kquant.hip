@@ -307,10 +307,10 @@ __device__ __forceinline__ void raw_to_float4(const RawX<X16>& r, int x_dtype, f
 
 // ITERS = blocks a wave walks per pass, DEPTH <= ITERS = blocks it keeps in flight (a block's activation slice is requested
 // right ahead of its weights, so it arrives first).
-template <typename FMT, int ITERS, int DEPTH, bool X16>
+template <typename FMT, int ITERS, int DEPTH, bool X16, bool NORM>
 __global__ __launch_bounds__(64 * kMaxWaves) void wave_image_matvec_kernel(
     const void* __restrict__ x, int x_dtype, int k, const WeightRoute route, const uint8_t* __restrict__ w, void* __restrict__ y,
-    int y_dtype, int n, int bpr) {
+    int y_dtype, int n, int bpr, const float* __restrict__ gamma, float eps, int round_f16) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int tid = threadIdx.x;
     const int waves = blockDim.x >> 6;
@@ -334,38 +334,82 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_image_matvec_kernel(
 
     if (lane < 4) reinterpret_cast<uint32_t*>(slot + kSlotBytes)[lane] = 0;
     float acc = 0.0f;
+    // NORM (the row passes through an RMS normalisation first, one pass of the loop below): the wave's slices of all its blocks
+    // are requested at once, with the weights of the first blocks behind them; their squares are the wave's share of the row's
+    // sum, the shares meet in LDS, and the slices are scaled as they are quantized.  No extra pass over the row, one barrier.
+    constexpr int kHeldX = NORM ? ITERS : DEPTH;
+    RawX<X16> raw[kHeldX];
+    RawX<false> graw[NORM ? ITERS : 1];
+    float rstd = 1.0f;
     for (int b0 = wave; b0 < bpr; b0 += waves * ITERS) {
-        RawX<X16> raw[DEPTH];
         typename FMT::Regs regs[DEPTH];
         auto request_x = [&](int it) {
             const int b = b0 + it * waves;
-            request_raw4<X16>(raw[it % DEPTH], x, xoff, 256 * b + 4 * lane, b < bpr ? k : 0);
+            request_raw4<X16>(raw[it % kHeldX], x, xoff, 256 * b + 4 * lane, b < bpr ? k : 0);
         };
         auto request_w = [&](int it) {
             const int b = b0 + it * waves;
             FMT::load(regs[it % DEPTH], wrow + static_cast<size_t>(min(b, bpr - 1)) * FMT::kBlockBytes, ks);   // clamped: always a valid address
         };
         auto request = [&](int it) {
-            request_x(it);
+            if constexpr (!NORM) request_x(it);
             __builtin_amdgcn_sched_barrier(0);                              // keep the issue order: memory returns a wave's loads in it
             request_w(it);
             __builtin_amdgcn_sched_barrier(0);
         };
         // the activation slices first: they are small, arrive first and are quantized while the weights are on their way
 #pragma unroll
-        for (int it = 0; it < DEPTH; ++it) request_x(it);
+        for (int it = 0; it < kHeldX; ++it) request_x(it);
+        if constexpr (NORM) {
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it) {
+                const int b = b0 + it * waves;
+                request_raw4<false>(graw[it], gamma, 0, 256 * b + 4 * lane, b < bpr ? k : 0);
+            }
+        }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int it = 0; it < DEPTH; ++it) request_w(it);
         __builtin_amdgcn_sched_barrier(0);
+        if constexpr (NORM) {
+            float ss = 0.0f;
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it) {
+                const int b = b0 + it * waves;
+                if (k != 256 * bpr) {                                        // rows that end inside their last block
+                    settle_raw4<X16>(raw[it], 256 * b + 4 * lane, b < bpr ? k : 0);
+                    settle_raw4<false>(graw[it], 256 * b + 4 * lane, b < bpr ? k : 0);
+                }
+                float v[4];
+                raw_to_float4<X16>(raw[it], x_dtype, v);
+                if (b < bpr) ss += (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
+            }
+            ss = group_sum<64>(ss);
+            float* shares = partial + waves * kRowsPerWg;                    // [waves]
+            if (lane == 0) shares[wave] = ss;
+            __syncthreads();
+            float total = 0.0f;
+            for (int v = 0; v < waves; ++v) total += shares[v];
+            rstd = rsqrtf(total / static_cast<float>(k) + eps);
+        }
 #pragma unroll
         for (int it = 0; it < ITERS; ++it) {
             const int b = b0 + it * waves;
             if (b < bpr) {                                                   // wave-uniform
                 // the block's activation slice into the wave's slot: the same two-term image the pre-pass kernel writes
                 float v[4];
-                if (k != 256 * bpr) settle_raw4<X16>(raw[it % DEPTH], 256 * b + 4 * lane, k);   // rows that end inside their last block
-                raw_to_float4<X16>(raw[it % DEPTH], x_dtype, v);
+                if constexpr (!NORM)
+                    if (k != 256 * bpr) settle_raw4<X16>(raw[it % kHeldX], 256 * b + 4 * lane, k);   // rows that end inside their last block
+                raw_to_float4<X16>(raw[it % kHeldX], x_dtype, v);
+                if constexpr (NORM) {
+                    const float g[4] = {__uint_as_float(graw[it].v.x), __uint_as_float(graw[it].v.y), __uint_as_float(graw[it].v.z), __uint_as_float(graw[it].v.w)};
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        float t = v[i] * rstd * g[i];                        // values past k are zeros on both sides
+                        if (round_f16) t = static_cast<float>(static_cast<_Float16>(t));
+                        v[i] = t;
+                    }
+                }
                 uint32_t qh, ql;
                 float scale;
                 quantize4(v, qh, ql, scale);
@@ -430,11 +474,12 @@ int launch_kernel(KERN kern, const ActRows& act, const WeightRoute& route, const
 template <typename KERN>
 int launch_wave_kernel(KERN kern, const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype,
                        int rows, int n, int bpr, int waves, hipStream_t stream) {
-    const size_t smem = static_cast<size_t>(waves) * (kSlotBytes + 16) + static_cast<size_t>(waves) * kRowsPerWg * sizeof(float);
+    const size_t smem = static_cast<size_t>(waves) * (kSlotBytes + 16) + static_cast<size_t>(waves) * (kRowsPerWg + 1) * sizeof(float);
     int tallest = n;
     for (int m = 0; m < route.extra; ++m) tallest = tallest > route.more_n[m] ? tallest : route.more_n[m];
     dim3 grid((tallest + kRowsPerWg - 1) / kRowsPerWg, rows, 1 + route.extra);
-    hipLaunchKernelGGL(kern, grid, dim3(64 * waves), smem, stream, act.x, act.x_dtype, act.k, route, w, y, y_dtype, n, bpr);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * waves), smem, stream, act.x, act.x_dtype, act.k, route, w, y, y_dtype, n, bpr, act.gamma, act.eps,
+                       act.round_f16);
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 
@@ -457,16 +502,17 @@ void split_blocks(int bpr, int work_items, int& waves, int& iters) {
     if (iters == 7) iters = 8;
 }
 
-// the single-launch form: raw rows, no normalisation, no routing
-template <typename FMT>
+// the single-launch form: raw rows (with or without an RMS normalisation ahead), no routing
+template <typename FMT, bool NORM>
 int launch_wave(const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream) {
     int waves, iters;
     int tiles = (n + kRowsPerWg - 1) / kRowsPerWg;
     for (int m = 0; m < route.extra; ++m) tiles += (route.more_n[m] + kRowsPerWg - 1) / kRowsPerWg;
     split_blocks(bpr, tiles * rows, waves, iters);
+    if (NORM && waves * iters < bpr) return PLLM_ERR_UNSUPPORTED;             // the normalised form holds a wave's slices of the whole row
 #define PLLM_CASE(I) case I: \
-        return act.x_dtype == PLLM_F32 ? launch_wave_kernel(wave_image_matvec_kernel<FMT, I, wave_depth<FMT>(I, false), false>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream) \
-                                       : launch_wave_kernel(wave_image_matvec_kernel<FMT, I, wave_depth<FMT>(I, true), true>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream)
+        return act.x_dtype == PLLM_F32 ? launch_wave_kernel(wave_image_matvec_kernel<FMT, I, wave_depth<FMT>(I, false), false, NORM>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream) \
+                                       : launch_wave_kernel(wave_image_matvec_kernel<FMT, I, wave_depth<FMT>(I, true), true, NORM>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream)
     switch (iters) {
         PLLM_CASE(1); PLLM_CASE(2); PLLM_CASE(3); PLLM_CASE(4); PLLM_CASE(5); PLLM_CASE(6);
         default: PLLM_CASE(8);
@@ -477,7 +523,11 @@ int launch_wave(const ActRows& act, const WeightRoute& route, const uint8_t* w, 
 template <typename FMT, int R>
 int launch_k45_rows(const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream) {
     if constexpr (R == 1)
-        if (act.x && act.k >= 4 && !act.gamma && !route.expert && !act.row_token) return launch_wave<FMT>(act, route, w, y, y_dtype, rows, n, bpr, stream);
+        if (act.x && act.k >= 4 && !route.expert && !act.row_token) {
+            if (!act.gamma) return launch_wave<FMT, false>(act, route, w, y, y_dtype, rows, n, bpr, stream);
+            const int st = launch_wave<FMT, true>(act, route, w, y, y_dtype, rows, n, bpr, stream);
+            if (st != PLLM_ERR_UNSUPPORTED) return st;                       // (rows too long for it: the workgroup-wide quantizer below)
+        }
     int waves, iters;
     int tiles = (n + kRowsPerWg - 1) / kRowsPerWg;
     for (int m = 0; m < route.extra; ++m) tiles += (route.more_n[m] + kRowsPerWg - 1) / kRowsPerWg;
