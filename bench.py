@@ -607,7 +607,7 @@ def main() -> None:
     roofline = {"bound": "hbm", "achieved": round(kernel_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(kernel_gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
                 "traffic_source": "profiles/traffic.json: rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE of an earlier run, not measured in this run",
-                "kernel": "wave_image_matvec_kernel<Q5K, 5, 4, true> = the q5_k matvec 17408x5120 operator call (one launch, activations quantized in the kernel)",
+                "kernel": "wave_image_matvec_kernel<Q5K, 5, 4, true, false> = the q5_k matvec 17408x5120 operator call (one launch, activations quantized in the kernel)",
                 "bytes_per_launch": dom["weight_bytes"], "us_per_launch": round(kernel_us, 3),
                 "us_per_launch_on_prepared_image": round(image_us, 3),
                 "timed_launches_per_repeat": max(MIN_TIMED_LAUNCHES, len(d_ring)), "repeats": REPEATS}
