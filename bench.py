@@ -600,16 +600,21 @@ def main() -> None:
     image_us, _ = time_calls_us(lambda s: mod.gguf_quant_gemm_prequantized(image, d_ring[s], d_tid), len(d_ring), eager=args.eager)
     kernel_us = dom["us_per_call"]
     kernel_gbs = host_blocks[DOMINANT].size / kernel_us / 1e3
-    traffic = None
+    traffic, traced_us = None, None
     if os.path.exists(TRAFFIC_FILE):
         with open(TRAFFIC_FILE) as f:
-            traffic = json.load(f).get("q5_k matvec 17408x5120 T=1")
+            recorded = json.load(f)
+        traffic = recorded.get("q5_k matvec 17408x5120 T=1")
+        traced_us = recorded.get("q5_k matvec 17408x5120 T=1 rocprofv3 kernel-trace avg us")
     roofline = {"bound": "hbm", "achieved": round(kernel_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(kernel_gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
                 "traffic_source": "profiles/traffic.json: rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE of an earlier run, not measured in this run",
                 "kernel": "wave_image_matvec_kernel<Q5K, 5, 4, true, false> = the q5_k matvec 17408x5120 operator call (one launch, activations quantized in the kernel)",
                 "bytes_per_launch": dom["weight_bytes"], "us_per_launch": round(kernel_us, 3),
                 "us_per_launch_on_prepared_image": round(image_us, 3),
+                # begin-to-end duration of the same kernel in the committed kernel trace (profiles/): the event-timed figure above is
+                # the period of back-to-back launches and carries the gap between graph nodes
+                "us_per_launch_in_committed_kernel_trace": traced_us,
                 "timed_launches_per_repeat": max(MIN_TIMED_LAUNCHES, len(d_ring)), "repeats": REPEATS}
 
     # parity of what was just timed, against the float-activation oracle (small case only: seconds)
