@@ -363,10 +363,15 @@ __global__ __launch_bounds__(256) void moe_reduce_kernel(const float* __restrict
             y[static_cast<size_t>(t) * dim + d] = acc;
         }
     } else if (routes <= kReduceList) {
-        const int per = (routes + 255) / 256;
+        const int per = (routes + 255) / 256;                                // at most kReduceList / 256 = 8
         const int r0 = min(tid * per, routes), r1 = min(r0 + per, routes);
+        // the thread's run of the route table, all loads in flight together (past the run: its last entry again, not counted)
+        int64_t mine[kReduceList / 256];
+#pragma unroll
+        for (int i = 0; i < kReduceList / 256; ++i) mine[i] = route_tokens[min(r0 + i, routes - 1)];
         int cnt = 0;
-        for (int r = r0; r < r1; ++r) cnt += route_tokens[r] == t;
+#pragma unroll
+        for (int i = 0; i < kReduceList / 256; ++i) cnt += (r0 + i < r1) && mine[i] == t;
         int incl = cnt;                                     // inclusive scan over the wave, then over the four waves
 #pragma unroll
         for (int off = 1; off < 64; off <<= 1) {
@@ -381,12 +386,21 @@ __global__ __launch_bounds__(256) void moe_reduce_kernel(const float* __restrict
             if (w < (tid >> 6)) pos += wave_total[w];
             total += wave_total[w];
         }
-        for (int r = r0; r < r1; ++r)
-            if (route_tokens[r] == t) list[pos++] = r;
+#pragma unroll
+        for (int i = 0; i < kReduceList / 256; ++i)
+            if ((r0 + i < r1) && mine[i] == t) list[pos++] = r0 + i;
         __syncthreads();
         for (int d = d0; d < dim; d += dstep) {
             float acc = 0.0f;
-            for (int i = 0; i < total; ++i) acc += partial[static_cast<size_t>(list[i]) * dim + d];
+            int i = 0;
+            for (; i + 8 <= total; i += 8) {                                 // eight routes' values requested together, added in route order
+                float v[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) v[j] = partial[static_cast<size_t>(list[i + j]) * dim + d];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc += v[j];
+            }
+            for (; i < total; ++i) acc += partial[static_cast<size_t>(list[i]) * dim + d];
             y[static_cast<size_t>(t) * dim + d] = acc;
         }
     } else {

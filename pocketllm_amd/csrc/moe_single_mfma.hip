@@ -397,14 +397,32 @@ __device__ __forceinline__ float rows_scale(float am) {
     return ldexpf(1.0f, max(-126, min(11 - ex, 126)));
 }
 
+constexpr int kImageHeld = 4;              // pieces of four values a thread keeps: rows up to 4096 values are read once
 template <int TERMS>
 __global__ __launch_bounds__(256) void rows_image_kernel(const void* __restrict__ x, int x_dtype, int dim, int kpad, _Float16* __restrict__ img,
                                                          float* __restrict__ unscale) {
     __shared__ float part[4];
     const int token = blockIdx.x, tid = threadIdx.x;
     const size_t base = static_cast<size_t>(token) * dim;
+    const bool held = kpad <= 4 * kImageHeld * 256 && dim % 4 == 0 &&
+                      ((reinterpret_cast<uintptr_t>(x) + base * (x_dtype == PLLM_F32 ? 4 : 2)) & 15u) == 0;
+    float v[kImageHeld][4];
     float am = 0.0f;
-    for (int k = tid; k < dim; k += 256) am = fmaxf(am, fabsf(load_any(x, x_dtype, base + k)));
+    if (held) {                                // all of the thread's pieces requested together (beyond the row: its first piece again, dropped)
+        int e0[kImageHeld];
+#pragma unroll
+        for (int j = 0; j < kImageHeld; ++j) e0[j] = 4 * (tid + 256 * j) < dim ? 4 * (tid + 256 * j) : 0;
+        load_rows4_batch(v, x, x_dtype, base, e0);
+#pragma unroll
+        for (int j = 0; j < kImageHeld; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (4 * (tid + 256 * j) >= dim) v[j][i] = 0.0f;
+                am = fmaxf(am, fabsf(v[j][i]));
+            }
+    } else {
+        for (int k = tid; k < dim; k += 256) am = fmaxf(am, fabsf(load_any(x, x_dtype, base + k)));
+    }
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) am = fmaxf(am, __shfl_xor(am, off, 64));
     if ((tid & 63) == 0) part[tid >> 6] = am;
@@ -412,11 +430,29 @@ __global__ __launch_bounds__(256) void rows_image_kernel(const void* __restrict_
     am = fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3]));
     const float s = rows_scale(am);
     _Float16* row = img + static_cast<size_t>(token) * TERMS * kpad;
-    for (int k = tid; k < kpad; k += 256) {
-        const float v = k < dim ? load_any(x, x_dtype, base + k) * s : 0.0f;
-        const _Float16 h = static_cast<_Float16>(v);
-        row[k] = h;
-        if constexpr (TERMS == 2) row[kpad + k] = static_cast<_Float16>(v - static_cast<float>(h));
+    if (held) {
+#pragma unroll
+        for (int j = 0; j < kImageHeld; ++j) {
+            const int k0 = 4 * (tid + 256 * j);
+            if (k0 < kpad) {
+                union { _Float16 h[4]; uint2 u; } hi, lo;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float w = v[j][i] * s;
+                    hi.h[i] = static_cast<_Float16>(w);
+                    lo.h[i] = static_cast<_Float16>(w - static_cast<float>(hi.h[i]));
+                }
+                *reinterpret_cast<uint2*>(row + k0) = hi.u;
+                if constexpr (TERMS == 2) *reinterpret_cast<uint2*>(row + kpad + k0) = lo.u;
+            }
+        }
+    } else {
+        for (int k = tid; k < kpad; k += 256) {
+            const float w = k < dim ? load_any(x, x_dtype, base + k) * s : 0.0f;
+            const _Float16 h = static_cast<_Float16>(w);
+            row[k] = h;
+            if constexpr (TERMS == 2) row[kpad + k] = static_cast<_Float16>(w - static_cast<float>(h));
+        }
     }
     if (tid == 0) unscale[token] = 1.0f / s;
 }
