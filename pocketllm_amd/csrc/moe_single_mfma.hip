@@ -80,17 +80,20 @@ __global__ __launch_bounds__(64 * kW13Waves) void moe_single_w13_kernel(
         if (tid < 16) store_hidden16(0.0f, 0.0f, 0.0f, 0.0f, blockIdx.x * 16 + tid, inter, h_image + static_cast<size_t>(route) * h_image_stride, h_kpad, tid);
         return;
     }
-    // the raw activation row, both matrices' tiles and the codebooks travel to LDS together
+    // the raw activation row, the codebooks and both matrices' tiles travel to LDS together; the row is requested first and
+    // quantized (LDS to LDS) while the tiles are still on their way: loads complete in order, so "all but the tiles'
+    // instructions" means the row has landed
     dma_share<kW13Waves>(static_cast<const unsigned char*>(x), lds0 + raw_off, dim * (x_dtype == PLLM_F32 ? 4 : 2), wave, lane);
-    dma_share<kW13Waves>(w1 + tile_pos, lds0 + tile_off, tile_bytes, wave, lane);
-    dma_share<kW13Waves>(w3 + tile_pos, lds0 + tile_off + tile_stride, tile_bytes, wave, lane);
     FMT::template dma_tables<kW13Waves>(lds0 + table_off, wave, lane);
+    const int tile_loads = dma_share<kW13Waves>(w1 + tile_pos, lds0 + tile_off, tile_bytes, wave, lane) +
+                           dma_share<kW13Waves>(w3 + tile_pos, lds0 + tile_off + tile_stride, tile_bytes, wave, lane);
     if (tid < 4) reinterpret_cast<uint32_t*>(smem + zero_off)[tid] = 0;
     AMap<FMT::kSlots> am;
     FMT::a_map(am, col, ks, kpad, zero_off);
-    wait_vm<0>();
+    wait_vm_all_but(tile_loads);
     __syncthreads();
-    quantize_row_to_lds(smem, smem + raw_off, x_dtype, 0, dim, kpad);       // LDS to LDS
+    quantize_row_to_lds(smem, smem + raw_off, x_dtype, 0, dim, kpad);
+    wait_vm<0>();
     __syncthreads();
 
     const unsigned char* tile = smem + tile_off + mat * tile_stride;
@@ -495,9 +498,8 @@ __device__ __forceinline__ void store_hidden_rows(float g, float u, float limit,
     }
     const float h = (i < inter) ? g / (1.0f + expf(-g)) * u * route_weight : 0.0f;
     row[i] = h;
-    float am = fabsf(h);
-#pragma unroll
-    for (int off = 1; off < 16; off <<= 1) am = fmaxf(am, __shfl_xor(am, off, 64));   // (fmaxf drops NaNs; an infinity stays)
+    // the tile's maximum through DPP row operations (no LDS crossbar); fmaxf drops NaNs, an infinity stays
+    const float am = group_max<16>(fabsf(h));
     if ((i & 15) == 0) tile_max[i >> 4] = am;
 }
 
