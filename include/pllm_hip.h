@@ -249,6 +249,15 @@ size_t pllm_fp8_block_gemm_workspace_bytes(int64_t rows, int64_t k, int64_t n);
  */
 int pllm_fp8_gemm(const uint8_t* a, const float* a_scale, const uint8_t* weight, const float* scale, void* y, int y_dtype,
                   int64_t rows, int64_t k, int64_t n, void* stream);
+/*
+ * The same operator (same reference interface, src/kernels/ops.py:1043-1051) with a caller-provided workspace of
+ * pllm_fp8_gemm_workspace_bytes(rows, k, n) bytes: output tiles that would occupy a fraction of the GPU for a full pass
+ * over K are cut along K, their float32 partial sums go through the workspace and are added in a fixed order (results do
+ * not depend on scheduling).  A null or short workspace runs every tile whole, as pllm_fp8_gemm does.
+ */
+size_t pllm_fp8_gemm_workspace_bytes(int64_t rows, int64_t k, int64_t n);
+int pllm_fp8_gemm_ws(const uint8_t* a, const float* a_scale, const uint8_t* weight, const float* scale, void* y, int y_dtype,
+                     int64_t rows, int64_t k, int64_t n, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * FP8 E4M3 weights with IEEE fp16 scale bits per 128 x 128 block and explicit pitches: the raw-pointer

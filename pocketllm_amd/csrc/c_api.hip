@@ -410,7 +410,20 @@ int pllm_fp8_gemm(const uint8_t* a, const float* a_scale, const uint8_t* weight,
     if (!a || !a_scale || !weight || !scale || !y || !dtype_ok(y_dtype)) return PLLM_ERR_INVALID_ARGUMENT;
     if (!fits_int(rows) || !fits_int(k) || !fits_int(n) || rows <= 0 || n <= 0) return PLLM_ERR_INVALID_ARGUMENT;
     return pllm::fp8_gemm_native(a, a_scale, weight, scale, y, y_dtype, static_cast<int>(rows), static_cast<int>(k), static_cast<int>(n),
-                                 static_cast<hipStream_t>(stream));
+                                 nullptr, 0, static_cast<hipStream_t>(stream));
+}
+
+size_t pllm_fp8_gemm_workspace_bytes(int64_t rows, int64_t k, int64_t n) {
+    if (!fits_int(rows) || !fits_int(k) || !fits_int(n)) return 0;
+    return pllm::fp8_gemm_native_workspace_bytes(static_cast<int>(rows), static_cast<int>(k), static_cast<int>(n));
+}
+
+int pllm_fp8_gemm_ws(const uint8_t* a, const float* a_scale, const uint8_t* weight, const float* scale, void* y, int y_dtype,
+                     int64_t rows, int64_t k, int64_t n, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!a || !a_scale || !weight || !scale || !y || !dtype_ok(y_dtype)) return PLLM_ERR_INVALID_ARGUMENT;
+    if (!fits_int(rows) || !fits_int(k) || !fits_int(n) || rows <= 0 || n <= 0) return PLLM_ERR_INVALID_ARGUMENT;
+    return pllm::fp8_gemm_native(a, a_scale, weight, scale, y, y_dtype, static_cast<int>(rows), static_cast<int>(k), static_cast<int>(n),
+                                 workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
 // the tile GEMM serves many rows of 256-aligned k; everything else takes the matvec (no workspace)

@@ -12,6 +12,8 @@
 // scale.  Which code of a 64-chunk sits in which byte of a lane's operand does not matter as long
 // as both operands agree: lanes 0..31 take bytes [0, 32) and lanes 32..63 bytes [32, 64) of the
 // chunk on both sides.
+#include <algorithm>
+
 #include "pllm_device.h"
 #include "pllm_internal.h"
 
@@ -39,9 +41,13 @@ __device__ __forceinline__ floatx16 mfma_e4m3(const v8i& a, const v8i& b, const 
     return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 127, 0, 127);
 }
 
+// Workgroups [0, full_tiles) take whole tiles (tile = its index, column tiles fastest) and store scaled results into y.
+// Workgroup full_tiles + r takes K steps [slice * per, (slice + 1) * per) of tile full_tiles + r / slices, slice = r % slices, and
+// stores its float32 sums into partial[r][128][128]: the tiles that would occupy a fraction of the machine for a full round of
+// K are cut along K (block scales are per K step, so every slice's sums are final values) and added in slice order afterwards.
 __global__ __launch_bounds__(256, 2) void fp8_gemm_kernel(
     const uint8_t* __restrict__ a, const float* __restrict__ a_s, const uint8_t* __restrict__ b, const float* __restrict__ b_s,
-    void* __restrict__ y, int y_dtype, int rows, int n, int k) {
+    void* __restrict__ y, int y_dtype, int rows, int n, int k, int tiles_n, int full_tiles, int slices, int per, float* __restrict__ partial) {
     extern __shared__ __align__(16) unsigned char smem[];
     unsigned char* a_tile = smem;                                         // [2][kTile * kRow]
     unsigned char* b_tile = smem + 2 * kTile * kRow;                      // [2][kTile * kRow]
@@ -50,8 +56,14 @@ __global__ __launch_bounds__(256, 2) void fp8_gemm_kernel(
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    const int n0 = blockIdx.x * kTile, t0 = blockIdx.y * kTile;
-    const int steps = k / kStep;
+    const int wg = blockIdx.x;
+    const bool whole = wg < full_tiles;
+    const int rest = wg - full_tiles;
+    const int tile = whole ? wg : full_tiles + rest / slices;
+    const int n0 = (tile % tiles_n) * kTile, t0 = (tile / tiles_n) * kTile;
+    const int steps = k / kStep;                                          // row pitch of the scale tables
+    const int s_begin = whole ? 0 : (rest % slices) * per;
+    const int s_end = whole ? steps : min(steps, s_begin + per);
 
     // staging: piece q = tid + 256 i is bytes [16 (q % 8), +16) of tile row q / 8
     const int prow = tid >> 3, pcol = 16 * (tid & 7);
@@ -95,13 +107,13 @@ __global__ __launch_bounds__(256, 2) void fp8_gemm_kernel(
         if (tid < kTile) a_scale[buf * kTile + tid] = rs;
     };
 
-    fetch(0);
+    fetch(s_begin);
     stage(0);
     __syncthreads();
-    for (int s = 0; s < steps; ++s) {
-        const int buf = s & 1;
+    for (int s = s_begin; s < s_end; ++s) {
+        const int buf = (s - s_begin) & 1;
         const float ws = rws;
-        fetch(min(s + 1, steps - 1));        // (no branch around the loads: the last step fetches itself again and drops it)
+        fetch(min(s + 1, s_end - 1));        // (no branch around the loads: the last step fetches itself again and drops it)
         const unsigned char* at = a_tile + buf * kTile * kRow + (wm * 64 + (lane & 31)) * kRow + 32 * (lane >> 5);
         const unsigned char* bt = b_tile + buf * kTile * kRow + (wn * 64 + (lane & 31)) * kRow + 32 * (lane >> 5);
         floatx16 c[2][2];
@@ -137,8 +149,23 @@ __global__ __launch_bounds__(256, 2) void fp8_gemm_kernel(
                     acc[mi][ni][4 * q + 3] += c[mi][ni][4 * q + 3] * f3;
                 }
             }
-        if (s + 1 < steps) stage(buf ^ 1);
+        if (s + 1 < s_end) stage(buf ^ 1);
         __syncthreads();
+    }
+    if (!whole) {                            // raw sums of this slice, [row of the tile][column of the tile]
+        float* dst = partial + static_cast<size_t>(rest) * kTile * kTile;
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni) {
+                const int col = wn * 64 + ni * 32 + (lane & 31);
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int row = wm * 64 + mi * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                    dst[row * kTile + col] = acc[mi][ni][v];
+                }
+            }
+        return;
     }
 
 #pragma unroll
@@ -154,17 +181,81 @@ __global__ __launch_bounds__(256, 2) void fp8_gemm_kernel(
         }
 }
 
+// y[t, n] = sum over the slices, in slice order, of the split tiles' partial sums; one workgroup per 1024 elements of a tile
+__global__ __launch_bounds__(256) void fp8_gemm_reduce_kernel(const float* __restrict__ partial, void* __restrict__ y, int y_dtype, int rows, int n,
+                                                              int tiles_n, int full_tiles, int slices) {
+    const int tile = full_tiles + blockIdx.y;
+    const int n0 = (tile % tiles_n) * kTile, t0 = (tile / tiles_n) * kTile;
+    const int i = (blockIdx.x * 256 + threadIdx.x) * 4;                    // four neighbouring columns of one row
+    const int row = i / kTile, col = i % kTile;
+    const float* src = partial + static_cast<size_t>(blockIdx.y) * slices * kTile * kTile + i;
+    float4 total = *reinterpret_cast<const float4*>(src);
+    for (int sl = 1; sl < slices; ++sl) {
+        const float4 v = *reinterpret_cast<const float4*>(src + static_cast<size_t>(sl) * kTile * kTile);
+        total.x += v.x; total.y += v.y; total.z += v.z; total.w += v.w;
+    }
+    if (t0 + row >= rows) return;
+    const size_t o = static_cast<size_t>(t0 + row) * n + n0 + col;
+    if (n0 + col < n) store_any(y, y_dtype, o, total.x);
+    if (n0 + col + 1 < n) store_any(y, y_dtype, o + 1, total.y);
+    if (n0 + col + 2 < n) store_any(y, y_dtype, o + 2, total.z);
+    if (n0 + col + 3 < n) store_any(y, y_dtype, o + 3, total.w);
+}
+
+struct Fp8GemmPlan { int tiles_n, tiles, full_tiles, slices, per; size_t partial_bytes; };
+
+// Whole rounds of tiles run unsplit; the left-over tiles (all tiles, when there is less than one round) are cut along K so that
+// their workgroups fill the machine about once, as long as the partial sums stay under 64 MB and a slice keeps two steps.
+Fp8GemmPlan plan_fp8_gemm(int rows, int k, int n) {
+    Fp8GemmPlan p;
+    p.tiles_n = (n + kTile - 1) / kTile;
+    p.tiles = p.tiles_n * ((rows + kTile - 1) / kTile);
+    const int resident = 2 * compute_units();
+    const int steps = k / kStep;
+    p.full_tiles = (p.tiles / resident) * resident;
+    const int rem = p.tiles - p.full_tiles;
+    p.slices = 1;
+    p.per = steps;
+    if (rem > 0 && rem * 2 <= resident) {
+        int slices = std::min(resident / rem, std::max(1, steps / 2));
+        slices = std::min<int>(slices, static_cast<int>((static_cast<size_t>(64) << 20) / (static_cast<size_t>(rem) * kTile * kTile * sizeof(float))));
+        if (slices >= 2) {
+            p.per = (steps + slices - 1) / slices;
+            p.slices = (steps + p.per - 1) / p.per;
+        }
+    }
+    if (p.slices == 1) p.full_tiles = p.tiles;
+    p.partial_bytes = p.slices > 1 ? static_cast<size_t>(p.tiles - p.full_tiles) * p.slices * kTile * kTile * sizeof(float) : 0;
+    return p;
+}
+
 }  // namespace
 
+size_t fp8_gemm_native_workspace_bytes(int rows, int k, int n) {
+    if (k % kStep != 0 || k <= 0 || rows <= 0 || n <= 0) return 0;
+    return plan_fp8_gemm(rows, k, n).partial_bytes;
+}
+
 int fp8_gemm_native(const uint8_t* a, const float* a_s, const uint8_t* b, const float* b_s, void* y, int y_dtype,
-                    int rows, int k, int n, hipStream_t stream) {
+                    int rows, int k, int n, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     if (k % kStep != 0 || k <= 0) return PLLM_ERR_UNSUPPORTED;
     if ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15u) return PLLM_ERR_UNSUPPORTED;
     const size_t smem = static_cast<size_t>(4) * kTile * kRow + 2 * kTile * sizeof(float);
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(fp8_gemm_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem)) != hipSuccess)
         return PLLM_ERR_UNSUPPORTED;
-    dim3 grid((n + kTile - 1) / kTile, (rows + kTile - 1) / kTile);
-    hipLaunchKernelGGL(fp8_gemm_kernel, grid, dim3(256), smem, stream, a, a_s, b, b_s, y, y_dtype, rows, n, k);
+    Fp8GemmPlan p = plan_fp8_gemm(rows, k, n);
+    if (p.slices > 1 && (!workspace || workspace_bytes < p.partial_bytes)) {  // no room for partial sums: every tile whole
+        p.slices = 1;
+        p.per = k / kStep;
+        p.full_tiles = p.tiles;
+    }
+    const int rem = p.tiles - p.full_tiles;
+    hipLaunchKernelGGL(fp8_gemm_kernel, dim3(p.full_tiles + rem * p.slices), dim3(256), smem, stream, a, a_s, b, b_s, y, y_dtype, rows, n, k,
+                       p.tiles_n, p.full_tiles, p.slices, p.per, static_cast<float*>(workspace));
+    if (hipGetLastError() != hipSuccess) return PLLM_ERR_LAUNCH;
+    if (rem > 0)
+        hipLaunchKernelGGL(fp8_gemm_reduce_kernel, dim3(kTile * kTile / 1024, rem), dim3(256), 0, stream, static_cast<const float*>(workspace), y,
+                           y_dtype, rows, n, p.tiles_n, p.full_tiles, p.slices);
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 

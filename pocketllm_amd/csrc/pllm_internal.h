@@ -131,8 +131,10 @@ size_t gemm_i8_workspace_bytes(int rows, int bpr);
 int gemm_i8(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y, int y_dtype,
             int rows, int k, int n, int bpr, void* workspace, size_t workspace_bytes, hipStream_t stream);
 // FP8 x FP8 block-scaled matmul on the native FP8 matrix path (gemm_fp8.hip); k a multiple of 128
+// (workspace: fp8_gemm_native_workspace_bytes for the partial sums of tiles cut along K; without it every tile runs whole)
+size_t fp8_gemm_native_workspace_bytes(int rows, int k, int n);
 int fp8_gemm_native(const uint8_t* a, const float* a_s, const uint8_t* b, const float* b_s, void* y, int y_dtype,
-                    int rows, int k, int n, hipStream_t stream);
+                    int rows, int k, int n, void* workspace, size_t workspace_bytes, hipStream_t stream);
 int gemm_f16_fp8(const void* x, int x_dtype, const uint8_t* w, const float* wscale, void* y, int y_dtype,
                  int rows, int k, int n, void* workspace, size_t workspace_bytes, hipStream_t stream);
 int gemm_f16(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y, int y_dtype,

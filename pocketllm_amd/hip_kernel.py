@@ -455,8 +455,10 @@ def fp8_gemm_forward(a: torch.Tensor, a_scale: torch.Tensor, weight: torch.Tenso
     if rows == 0:
         return y
     with _on_device(a8.device):
-        st = _lib().pllm_fp8_gemm(a8.data_ptr(), a_scale.data_ptr(), w8.data_ptr(), scale.data_ptr(), y.data_ptr(), _DTYPE_CODE[out_dtype],
-                                  rows, k, n, _stream(a8.device))
+        need = int(_lib().pllm_fp8_gemm_workspace_bytes(rows, k, n))
+        ws = torch.empty(need, dtype=torch.uint8, device=a8.device) if need else None
+        st = _lib().pllm_fp8_gemm_ws(a8.data_ptr(), a_scale.data_ptr(), w8.data_ptr(), scale.data_ptr(), y.data_ptr(), _DTYPE_CODE[out_dtype],
+                                     rows, k, n, ws.data_ptr() if ws is not None else None, need, _stream(a8.device))
     _ffi.check(st, "fp8_gemm_forward")
     return y
 

@@ -258,6 +258,38 @@ def test_fp8_gemm_native_baseline_shape_sampled(mod):
     assert O.rel_l2(y.cpu().numpy()[:, cols], want) <= 2e-4
 
 
+@pytest.mark.parametrize("t,n,k", [(512, 17408, 5120), (640, 1024, 2048), (100, 3000, 1280)])
+def test_fp8_gemm_native_split_tiles_equal_whole_tiles(mod, t, n, k):
+    """With a workspace the left-over output tiles are cut along K and their partial sums added in slice order; without one
+    every tile runs whole.  Same operands, every output element: the two differ only by the grouping of float32 additions."""
+    from pocketllm_amd import _ffi
+    lib = _ffi.load_library()
+    rng = np.random.default_rng(t + n + k)
+    codes, scale = C.quantize_fp8_block(rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02))
+    a, a_s = mod.fp8_act_quant_forward(torch.from_numpy(rng.standard_normal((t, k)).astype(np.float32)).to(DEV))
+    w, sc = torch.from_numpy(codes).to(DEV), torch.from_numpy(scale).to(DEV)
+    a8 = a.view(torch.uint8)
+    need = int(lib.pllm_fp8_gemm_workspace_bytes(t, k, n))
+    assert need > 0, "shape no longer splits any tile"
+    ws = torch.empty(need, dtype=torch.uint8, device=DEV)
+    y_split = torch.empty(t, n, dtype=torch.float32, device=DEV)
+    y_whole = torch.empty(t, n, dtype=torch.float32, device=DEV)
+    stream = torch.cuda.current_stream().cuda_stream
+    print(f"case fp8 native split t={t} n={n} k={k} workspace={need}", flush=True)
+    assert lib.pllm_fp8_gemm_ws(a8.data_ptr(), a_s.data_ptr(), w.data_ptr(), sc.data_ptr(), y_split.data_ptr(), 0, t, k, n, ws.data_ptr(), need, stream) == 0
+    assert lib.pllm_fp8_gemm(a8.data_ptr(), a_s.data_ptr(), w.data_ptr(), sc.data_ptr(), y_whole.data_ptr(), 0, t, k, n, stream) == 0
+    torch.cuda.synchronize()
+    got, ref = y_split.cpu().numpy(), y_whole.cpu().numpy()
+    assert np.isfinite(got).all()
+    assert O.rel_l2(got, ref) <= 1e-6
+    assert np.abs(got - ref).max() <= 1e-5 * np.abs(ref).max()
+    # a short workspace falls back to whole tiles: bit-identical to the entry point without one
+    y_short = torch.empty(t, n, dtype=torch.float32, device=DEV)
+    assert lib.pllm_fp8_gemm_ws(a8.data_ptr(), a_s.data_ptr(), w.data_ptr(), sc.data_ptr(), y_short.data_ptr(), 0, t, k, n, ws.data_ptr(), 16, stream) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(y_short, y_whole)
+
+
 # ---- Q4_K / Q5_K on the int8 matrix cores: int8 activation semantics ------------------------------------
 
 @pytest.mark.parametrize("type_name", ["q4_k", "q5_k"])
