@@ -119,8 +119,10 @@ namespace pllm {
 int superblock_matvec(const ActRows& act, const uint8_t* blocks, int type_id, void* y, int y_dtype,
                       int rows, int n, int bpr, hipStream_t s, WeightRoute route) {
     switch (type_id) {
-        case PLLM_TYPE_Q2_K:
-            return dot4_matvec_from_image(act, blocks, type_id, y, y_dtype, rows, n, bpr, s, route);
+        case PLLM_TYPE_Q2_K: {
+            const int st = q2k_wave_matvec(act, blocks, y, y_dtype, rows, n, bpr, s, route);
+            return st != PLLM_ERR_UNSUPPORTED ? st : dot4_matvec_from_image(act, blocks, type_id, y, y_dtype, rows, n, bpr, s, route);
+        }
         case PLLM_TYPE_IQ2_XXS:
         case PLLM_TYPE_IQ1_M:
         case PLLM_TYPE_IQ2_XS:

@@ -520,6 +520,156 @@ int launch_wave(const ActRows& act, const WeightRoute& route, const uint8_t* w, 
 #undef PLLM_CASE
 }
 
+// ------------------------------------------------------------------------------------------------
+// Q2_K in the same single-launch frame.  84 B = scales(16) qs(64) d(2) dmin(2): sixteen groups of 16
+// weights, 2-bit codes; group g lies in bytes qs[16 j, 16 j + 16), j = 2 (g / 8) + g % 2, at bit 2 s,
+// s = (g % 8) / 2; scale byte g = scale (low nibble) and min (high nibble).
+//     y = d sum_g sc_g dot(q_g, x_g) - dmin sum_g m_g sum(x_g).
+// A rows = the 16 groups, one MFMA set per activation term; MFMA t carries the weights [64 t, 64 t + 64),
+// groups 4 t .. 4 t + 3, lane (n, ks) supplies group 4 t + ks of weight row n as B and, where its A row
+// (= lane % 16) is that group, the group's 16 activation bytes as A.  C[4 ks .. 4 ks + 3][n] = the lane's
+// own four groups.  The wave's LDS slot adds the sums per 16 activations for the min terms.
+// ------------------------------------------------------------------------------------------------
+constexpr int kQ2SlotBytes = kSlotBytes + 64;       // ... | float sum16[16]
+struct Q2Regs { uint32_t sc; uint4 qa, qb; uint32_t dd; };
+struct __attribute__((packed, aligned(4))) Dwords4 { u32x4 v; };
+
+__device__ __forceinline__ void q2_load(Q2Regs& r, const uint8_t* blk, int ks) {
+    r.sc = *reinterpret_cast<const uint32_t*>(blk + 4 * ks);               // scale bytes of groups 4 ks .. 4 ks + 3
+    const Dwords4 a = *reinterpret_cast<const Dwords4*>(blk + 16 + 16 * (ks & 1));
+    const Dwords4 b = *reinterpret_cast<const Dwords4*>(blk + 48 + 16 * (ks & 1));
+    r.qa = make_uint4(a.v.x, a.v.y, a.v.z, a.v.w);                        // groups 0 .. 7 with the lane's parity
+    r.qb = make_uint4(b.v.x, b.v.y, b.v.z, b.v.w);                        // groups 8 .. 15
+    r.dd = *reinterpret_cast<const uint32_t*>(blk + 80);
+}
+
+template <int ITERS, int DEPTH, bool X16>
+__global__ __launch_bounds__(64 * kMaxWaves) void wave_q2k_matvec_kernel(
+    const void* __restrict__ x, int x_dtype, int k, const WeightRoute route, const uint8_t* __restrict__ w, void* __restrict__ y,
+    int y_dtype, int n, int bpr) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int tid = threadIdx.x;
+    const int waves = blockDim.x >> 6;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    const int col = lane & 15;
+    const int ks = lane >> 4;
+    constexpr int kWaveBytes = kQ2SlotBytes + 16;                            // the wave's slot, then its 16 zero bytes
+    unsigned char* slot = smem + wave * kWaveBytes;
+    float* partial = reinterpret_cast<float*>(smem + waves * kWaveBytes);    // [waves][16]
+    if (blockIdx.z) {                        // several projections in one launch: this one's matrix, row count and output
+        const int m = blockIdx.z - 1;
+        w = route.more_w[m];
+        y = route.more_y[m];
+        n = route.more_n[m];
+    }
+    if (static_cast<int>(blockIdx.x) * kRowsPerWg >= n) return;
+    const int row = blockIdx.x * kRowsPerWg + col;
+    const uint8_t* wrow = w + static_cast<size_t>(row < n ? row : 0) * bpr * 84;
+    const size_t xoff = static_cast<size_t>(blockIdx.y) * k;
+    // the lane's A operand: group `col` of the block, in the one MFMA (t = col / 4) whose slice ks carries that group
+    const bool mine = (col & 3) == ks;
+    const int my_t = col >> 2;
+    const int bit = 2 * (ks >> 1);                                           // codes of MFMA t sit at bit 2 (2 (t % 2) + ks / 2)
+
+    if (lane < 4) reinterpret_cast<uint32_t*>(slot + kQ2SlotBytes)[lane] = 0;
+    float acc = 0.0f;
+    for (int b0 = wave; b0 < bpr; b0 += waves * ITERS) {
+        RawX<X16> raw[DEPTH];
+        Q2Regs regs[DEPTH];
+        auto request_x = [&](int it) {
+            const int b = b0 + it * waves;
+            request_raw4<X16>(raw[it % DEPTH], x, xoff, 256 * b + 4 * lane, b < bpr ? k : 0);
+        };
+        auto request_w = [&](int it) {
+            const int b = b0 + it * waves;
+            q2_load(regs[it % DEPTH], wrow + static_cast<size_t>(min(b, bpr - 1)) * 84, ks);   // clamped: always a valid address
+        };
+#pragma unroll
+        for (int it = 0; it < DEPTH; ++it) request_x(it);
+        __builtin_amdgcn_sched_barrier(0);                                  // keep the issue order: memory returns a wave's loads in it
+#pragma unroll
+        for (int it = 0; it < DEPTH; ++it) request_w(it);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+            const int b = b0 + it * waves;
+            if (b < bpr) {                                                   // wave-uniform
+                float v[4];
+                if (k != 256 * bpr) settle_raw4<X16>(raw[it % DEPTH], 256 * b + 4 * lane, k);
+                raw_to_float4<X16>(raw[it % DEPTH], x_dtype, v);
+                uint32_t qh, ql;
+                float scale;
+                quantize4(v, qh, ql, scale);
+                reinterpret_cast<uint32_t*>(slot)[lane] = qh;
+                reinterpret_cast<uint32_t*>(slot + 256)[lane] = ql;
+                const float sum = group_sum<4>((v[0] + v[1]) + (v[2] + v[3]));   // the order in which the pre-pass kernel sums
+                const float sum32 = sum + butterfly_peer<4>(sum);
+                if ((lane & 7) == 0) reinterpret_cast<float2*>(slot + 512)[lane >> 3] = make_float2(scale * kLoInv, sum32);
+                if ((lane & 3) == 0) reinterpret_cast<float*>(slot + kSlotBytes)[lane >> 2] = sum;
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();                            // LDS serves a wave's requests in order
+                const Q2Regs& r = regs[it % DEPTH];
+                v4i ch = {0, 0, 0, 0}, cl = {0, 0, 0, 0};
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const uint4 piece = t < 2 ? r.qa : r.qb;
+                    const int sh = bit + 4 * (t & 1);
+                    const uint4 bw = make_uint4((piece.x >> sh) & 0x03030303u, (piece.y >> sh) & 0x03030303u,
+                                                (piece.z >> sh) & 0x03030303u, (piece.w >> sh) & 0x03030303u);
+                    const int off = (mine && t == my_t) ? 16 * col : kQ2SlotBytes;
+                    const uint4 ah = *reinterpret_cast<const uint4*>(slot + off);
+                    const uint4 al = *reinterpret_cast<const uint4*>(slot + off + ((mine && t == my_t) ? 256 : 0));
+                    ch = __builtin_amdgcn_mfma_i32_16x16x64_i8(as_v4i(ah), as_v4i(bw), ch, 0, 0, 0);
+                    cl = __builtin_amdgcn_mfma_i32_16x16x64_i8(as_v4i(al), as_v4i(bw), cl, 0, 0, 0);
+                }
+                const float4 g2 = *reinterpret_cast<const float4*>(slot + 512 + 16 * ks);          // {xs, sum} of 32-groups 2 ks, 2 ks + 1
+                const float4 s16 = *reinterpret_cast<const float4*>(slot + kSlotBytes + 16 * ks);  // sums of groups 4 ks .. 4 ks + 3
+                const float vv[4] = {static_cast<float>(__mul24(ch.x, 254) + cl.x), static_cast<float>(__mul24(ch.y, 254) + cl.y),
+                                     static_cast<float>(__mul24(ch.z, 254) + cl.z), static_cast<float>(__mul24(ch.w, 254) + cl.w)};
+                const float xsv[4] = {g2.x, g2.x, g2.z, g2.z};
+                const float smv[4] = {s16.x, s16.y, s16.z, s16.w};
+                float pos = 0.0f, neg = 0.0f;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t sb = (r.sc >> (8 * j)) & 0xffu;
+                    pos += static_cast<float>(sb & 15u) * xsv[j] * vv[j];
+                    neg += static_cast<float>(sb >> 4) * smv[j];
+                }
+                acc += f16_bits_to_float(r.dd & 0xffffu) * pos - f16_bits_to_float(r.dd >> 16) * neg;
+                __builtin_amdgcn_wave_barrier();                            // the next block's slice overwrites the slot
+            }
+            if (it + DEPTH < ITERS) {
+                request_x(it + DEPTH);
+                __builtin_amdgcn_sched_barrier(0);
+                request_w(it + DEPTH);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    }
+    acc += __shfl_xor(acc, 16, 64);
+    acc += __shfl_xor(acc, 32, 64);
+    if (ks == 0) partial[wave * kRowsPerWg + col] = acc;
+    __syncthreads();
+    if (tid < kRowsPerWg) {
+        float total = 0.0f;
+        for (int v = 0; v < waves; ++v) total += partial[v * kRowsPerWg + tid];
+        const int out_row = blockIdx.x * kRowsPerWg + tid;
+        if (out_row < n) store_any(y, y_dtype, static_cast<size_t>(blockIdx.y) * n + out_row, total);
+    }
+}
+
+template <typename KERN>
+int launch_q2k_kernel(KERN kern, const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype,
+                      int rows, int n, int bpr, int waves, hipStream_t stream) {
+    const size_t smem = static_cast<size_t>(waves) * (kQ2SlotBytes + 16) + static_cast<size_t>(waves) * kRowsPerWg * sizeof(float);
+    int tallest = n;
+    for (int m = 0; m < route.extra; ++m) tallest = tallest > route.more_n[m] ? tallest : route.more_n[m];
+    dim3 grid((tallest + kRowsPerWg - 1) / kRowsPerWg, rows, 1 + route.extra);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * waves), smem, stream, act.x, act.x_dtype, act.k, route, w, y, y_dtype, n, bpr);
+    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+}
+
 template <typename FMT, int R>
 int launch_k45_rows(const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream) {
     if constexpr (R == 1)
@@ -567,6 +717,25 @@ int kquant_matvec_from_image(const ActRows& act, const uint8_t* w, int type_id, 
         case PLLM_TYPE_Q5_K: return launch_k45<Q5K>(act, route, w, y, y_dtype, rows, n, bpr, stream);
         default: return PLLM_ERR_UNSUPPORTED;
     }
+}
+
+int q2k_wave_matvec(const ActRows& act, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream, WeightRoute route) {
+    // raw rows without normalisation or routing, blocks on a 4-byte boundary; everything else stays with the v_dot4 kernels
+    if (!act.x || act.k < 4 || act.gamma || route.expert || act.row_token || (reinterpret_cast<uintptr_t>(w) & 3u)) return PLLM_ERR_UNSUPPORTED;
+    for (int m = 0; m < route.extra; ++m)
+        if (reinterpret_cast<uintptr_t>(route.more_w[m]) & 3u) return PLLM_ERR_UNSUPPORTED;
+    int waves, iters;
+    int tiles = (n + kRowsPerWg - 1) / kRowsPerWg;
+    for (int m = 0; m < route.extra; ++m) tiles += (route.more_n[m] + kRowsPerWg - 1) / kRowsPerWg;
+    split_blocks(bpr, tiles * rows, waves, iters);
+#define PLLM_CASE(I, D) case I: \
+        return act.x_dtype == PLLM_F32 ? launch_q2k_kernel(wave_q2k_matvec_kernel<I, D, false>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream) \
+                                       : launch_q2k_kernel(wave_q2k_matvec_kernel<I, D, true>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream)
+    switch (iters) {
+        PLLM_CASE(1, 1); PLLM_CASE(2, 2); PLLM_CASE(3, 3); PLLM_CASE(4, 4); PLLM_CASE(5, 5); PLLM_CASE(6, 6);
+        default: PLLM_CASE(8, 6);
+    }
+#undef PLLM_CASE
 }
 
 }  // namespace pllm
