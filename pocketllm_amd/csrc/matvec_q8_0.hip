@@ -13,6 +13,7 @@
 // cross-lane reduction.
 #include "pllm_device.h"
 #include "pllm_internal.h"
+#include <algorithm>
 
 namespace pllm {
 namespace {
@@ -105,6 +106,192 @@ __global__ __launch_bounds__(kThreads) void q8_0_pair_kernel(
     if (row_ok && slot == 0) store_any(y, y_dtype, static_cast<size_t>(blockIdx.y) * n + row, acc);
 }
 
+// ------------------------------------------------------------------------------------------------
+// Streamed form (rows of a multiple of four pairs, 16-byte aligned matrix): one launch per operator call.
+//
+// The matrix is one contiguous run of 68-byte pairs.  One workgroup of 16 waves per compute unit owns a
+// contiguous range of whole rows and walks it in steps of 64 pairs = 4352 contiguous bytes, wave v taking
+// steps v, v + 16, ...  A step is loaded the way a stream is read: lane l takes 16 bytes at
+// 1024 i + 16 l (five fully coalesced wave instructions, the fifth covering the last 256 bytes four
+// lanes to an address), two steps ahead in registers (more waves beat deeper sets: 12 waves x 3 steps and 8 x 4 ran 1 - 2 us slower).  The wave then turns the step by way of an LDS
+// buffer of its own (no barrier: written and read by the same wave) so that lane l holds pair l (17
+// dwords at 68 l: neighbouring lanes 17 banks apart) and multiplies it as the kernel above does.  A
+// step may hold the end of one row and the start of the next: lanes are told apart by row, each row's
+// part is reduced over the wave into partial[step][row - first row of the step], and after one barrier
+// a thread per row adds the row's parts in step order (deterministic) and stores.
+// The workgroup quantizes the activation row itself into the pair image, once per compute unit, from
+// loads requested ahead of the first weights.
+// ------------------------------------------------------------------------------------------------
+constexpr int kStepBytes = 64 * 68;                            // 4352 = 4 x 1024 + 256
+constexpr int kStreamWaves = 16;
+constexpr int kStreamThreads = 64 * kStreamWaves;
+constexpr int kStreamDepth = 2;                                // steps a wave holds in registers (sixteen waves fit 128 registers each)
+constexpr int kXBatch = 2;                                     // pieces of the activation row a thread requests ahead of the weights
+
+typedef uint32_t v2u __attribute__((ext_vector_type(2)));
+typedef uint32_t v4u __attribute__((ext_vector_type(4)));                   // (a native vector: moves of HIP's uint4 struct between address spaces compile to memcpy calls that keep the sets in memory)
+
+__device__ __forceinline__ const uint8_t* not_past(const uint8_t* p, const uint8_t* last16) { return p < last16 ? p : last16; }
+
+__global__ __launch_bounds__(kStreamThreads) void q8_0_stream_kernel(
+    const void* __restrict__ x, int x_dtype, const uint8_t* __restrict__ w, void* __restrict__ y, int y_dtype,
+    int k, int n, int pairs, uint32_t pairs_magic, int image_bytes, int cols) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    unsigned char* img_hi = smem;
+    unsigned char* img_lo = smem + static_cast<size_t>(pairs) * 80;
+    float* xs = reinterpret_cast<float*>(smem + static_cast<size_t>(pairs) * 160);
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    unsigned char* turn = smem + image_bytes + wave * kStepBytes;              // this wave's buffer
+    float* partial = reinterpret_cast<float*>(smem + image_bytes + kStreamWaves * kStepBytes);   // [step][cols]
+
+    // this workgroup's rows [r0, r1): an even share of the matrix
+    const int r0 = static_cast<int>(static_cast<long long>(blockIdx.x) * n / gridDim.x);
+    const int r1 = static_cast<int>(static_cast<long long>(blockIdx.x + 1) * n / gridDim.x);
+    const int count = (r1 - r0) * pairs;
+    const int steps = (count + 63) >> 6;
+    const uint8_t* base = w + static_cast<size_t>(r0) * pairs * 68;
+    const uint8_t* last16 = w + static_cast<size_t>(n) * pairs * 68 - 16;      // loads past the matrix are bent back to here (their lanes are not used)
+
+    // the first pieces of the activation row, requested ahead of the weights (loads return in order) and left as loaded until the
+    // weights have been requested too: telling the value types apart before that would wait for the pieces inside each branch
+    const size_t xoff = static_cast<size_t>(blockIdx.y) * k;
+    constexpr int trip = kStreamThreads * 4;
+    v4u raw[kXBatch];
+    if (x_dtype == PLLM_F32) {
+#pragma unroll
+        for (int j = 0; j < kXBatch; ++j)
+            raw[j] = *reinterpret_cast<const v4u*>(static_cast<const float*>(x) + xoff + (tid * 4 + j * trip < k ? tid * 4 + j * trip : 0));
+    } else {
+#pragma unroll
+        for (int j = 0; j < kXBatch; ++j) {
+            const v2u t = *reinterpret_cast<const v2u*>(static_cast<const uint16_t*>(x) + xoff + (tid * 4 + j * trip < k ? tid * 4 + j * trip : 0));
+            raw[j] = v4u{t.x, t.y, 0u, 0u};
+        }
+    }
+
+    // step s of the workgroup (past its last step: that one again), always five loads
+    auto fetch = [&](v4u (&r)[5], int s) __attribute__((always_inline)) {
+        const uint8_t* src = base + static_cast<size_t>(min(s, max(steps - 1, 0))) * kStepBytes;
+        r[0] = *reinterpret_cast<const v4u*>(not_past(src + lane * 16, last16));
+        r[1] = *reinterpret_cast<const v4u*>(not_past(src + 1024 + lane * 16, last16));
+        r[2] = *reinterpret_cast<const v4u*>(not_past(src + 2048 + lane * 16, last16));
+        r[3] = *reinterpret_cast<const v4u*>(not_past(src + 3072 + lane * 16, last16));
+        r[4] = *reinterpret_cast<const v4u*>(not_past(src + 4096 + (lane & 15) * 16, last16));
+    };
+    v4u regs[kStreamDepth][5];
+#pragma unroll
+    for (int j = 0; j < kStreamDepth; ++j) fetch(regs[j], wave + j * kStreamWaves);
+
+    float head[kXBatch][4];
+    if (x_dtype == PLLM_F32) {
+#pragma unroll
+        for (int j = 0; j < kXBatch; ++j) {
+            head[j][0] = __uint_as_float(raw[j].x); head[j][1] = __uint_as_float(raw[j].y);
+            head[j][2] = __uint_as_float(raw[j].z); head[j][3] = __uint_as_float(raw[j].w);
+        }
+    } else if (x_dtype == PLLM_BF16) {
+#pragma unroll
+        for (int j = 0; j < kXBatch; ++j) {
+            head[j][0] = __uint_as_float(raw[j].x << 16); head[j][1] = __uint_as_float(raw[j].x & 0xffff0000u);
+            head[j][2] = __uint_as_float(raw[j].y << 16); head[j][3] = __uint_as_float(raw[j].y & 0xffff0000u);
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < kXBatch; ++j) {
+            head[j][0] = f16_bits_to_float(raw[j].x & 0xffffu); head[j][1] = f16_bits_to_float(raw[j].x >> 16);
+            head[j][2] = f16_bits_to_float(raw[j].y & 0xffffu); head[j][3] = f16_bits_to_float(raw[j].y >> 16);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < kXBatch; ++j)
+        if (tid * 4 + j * trip < k) quantize4_to_pair_image(head[j], tid * 4 + j * trip, img_hi, img_lo, xs);
+    for (int b0 = tid * 4 + kXBatch * trip; b0 < k; b0 += trip) {              // rows longer than one batch
+        float v[4];
+        load_row4(v, x, x_dtype, xoff, b0, k, true);
+        quantize4_to_pair_image(v, b0, img_hi, img_lo, xs);
+    }
+    __syncthreads();
+
+    // step s from the register set r, which then takes step s + kStreamDepth * kStreamWaves
+    auto step = [&](v4u (&r)[5], int s) __attribute__((always_inline)) {
+        // turn the step: 16-byte pieces in stream order -> LDS -> this lane's pair
+        *reinterpret_cast<v4u*>(turn + lane * 16) = r[0];
+        *reinterpret_cast<v4u*>(turn + 1024 + lane * 16) = r[1];
+        *reinterpret_cast<v4u*>(turn + 2048 + lane * 16) = r[2];
+        *reinterpret_cast<v4u*>(turn + 3072 + lane * 16) = r[3];
+        if (lane < 16) *reinterpret_cast<v4u*>(turn + 4096 + lane * 16) = r[4];
+        fetch(r, s + kStreamDepth * kStreamWaves);
+        if (s >= steps) return;                                                // wave-uniform
+        const int pidx = 64 * s + lane;
+        const int rowi = static_cast<int>(__umulhi(static_cast<uint32_t>(pidx), pairs_magic));   // row within the workgroup's range
+        const int p = pidx - rowi * pairs;
+        const uint32_t* q = reinterpret_cast<const uint32_t*>(turn + 68 * lane);
+        PairRegs pr;
+        pr.a = make_uint4(q[0], q[1], q[2], q[3]);
+        pr.b = make_uint4(q[4], q[5], q[6], q[7]);
+        pr.c = make_uint4(q[8], q[9], q[10], q[11]);
+        pr.d = make_uint4(q[12], q[13], q[14], q[15]);
+        pr.e = q[16];
+        const float d = pair_dot(pr, p, img_hi, img_lo, xs);
+        const float val = pidx < count ? d : 0.0f;
+        const int first = static_cast<int>(__umulhi(static_cast<uint32_t>(64 * s), pairs_magic));
+        const int last = static_cast<int>(__umulhi(static_cast<uint32_t>(min(64 * s + 63, count - 1)), pairs_magic));
+        for (int rr = first; rr <= last; ++rr) {                               // wave-uniform
+            const float total = group_sum<64>(rowi == rr ? val : 0.0f);
+            if (lane == 0) partial[s * cols + rr - first] = total;
+        }
+    };
+    for (int s = wave; s < steps; s += kStreamDepth * kStreamWaves) {
+#pragma unroll
+        for (int j = 0; j < kStreamDepth; ++j) step(regs[j], s + j * kStreamWaves);
+    }
+    __syncthreads();
+    for (int i = tid; i < r1 - r0; i += kStreamThreads) {
+        const int s_first = (i * pairs) >> 6, s_last = ((i + 1) * pairs - 1) >> 6;
+        float total = 0.0f;
+        for (int s = s_first; s <= s_last; ++s)
+            total += partial[s * cols + i - static_cast<int>(__umulhi(static_cast<uint32_t>(64 * s), pairs_magic))];
+        store_any(y, y_dtype, static_cast<size_t>(blockIdx.y) * n + r0 + i, total);
+    }
+}
+
+struct StreamPlan { int grid_x; int cols; int image_bytes; size_t smem; };
+
+// false when the streamed form does not apply
+bool plan_stream(const void* x, int x_dtype, const uint8_t* w, int k, int n, int bpr, StreamPlan& plan) {
+    if (bpr % 8 != 0 || k != bpr * 32 || (reinterpret_cast<uintptr_t>(w) & 15u)) return false;
+    if (reinterpret_cast<uintptr_t>(x) & (x_dtype == PLLM_F32 ? 15u : 7u)) return false;   // rows are read in vector pieces
+    const int pairs = bpr / 2;
+    const long long total_steps = (static_cast<long long>(n) * pairs + 63) / 64;
+    plan.grid_x = static_cast<int>(std::max<long long>(1, std::min<long long>(compute_units(), (total_steps + kStreamWaves - 1) / kStreamWaves)));
+    const long long rows_per_wg = (n + plan.grid_x - 1) / plan.grid_x;
+    const long long steps = (rows_per_wg * pairs + 63) / 64;
+    // the row index of a pair comes from a multiplication by a rounded-up reciprocal: exact while (pair index) x pairs < 2^32
+    if ((steps * 64 + 64) * pairs >= (1ll << 32)) return false;
+    plan.cols = (62 + pairs) / pairs + 1;                                      // rows that 64 consecutive pairs can touch
+    plan.image_bytes = (pairs * 168 + 15) & ~15;
+    plan.smem = static_cast<size_t>(plan.image_bytes) + static_cast<size_t>(kStreamWaves) * kStepBytes + static_cast<size_t>(steps) * plan.cols * sizeof(float);
+    return plan.smem <= 160 * 1024;
+}
+
+int launch_stream(const void* x, int x_dtype, const uint8_t* w, void* y, int y_dtype, int rows, int k, int n, int pairs, const StreamPlan& plan,
+                  hipStream_t stream) {
+    auto kern = q8_0_stream_kernel;
+    static size_t attr_smem = 0;
+    if (plan.smem > 64 * 1024 && plan.smem > attr_smem) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                static_cast<int>(plan.smem)) != hipSuccess)
+            return PLLM_ERR_UNSUPPORTED;
+        attr_smem = plan.smem;
+    }
+    const uint32_t magic = static_cast<uint32_t>(((1ull << 32) + pairs - 1) / pairs);
+    hipLaunchKernelGGL(kern, dim3(plan.grid_x, rows), dim3(kStreamThreads), plan.smem, stream, x, x_dtype, w, y, y_dtype, k, n, pairs, magic,
+                       plan.image_bytes, plan.cols);
+    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+}
+
 // Any shape, any alignment: one wave per output row, one lane per block, byte loads.  Used when a
 // row holds an odd number of blocks or the base pointer is not dword aligned.
 __global__ __launch_bounds__(kThreads) void q8_0_generic_kernel(
@@ -156,6 +343,8 @@ size_t q8_0_matvec_workspace_bytes(int rows, int bpr) {
 
 int q8_0_matvec(const void* x, int x_dtype, const uint8_t* w, void* y, int y_dtype,
                 int rows, int k, int n, int bpr, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+    StreamPlan plan;
+    if (plan_stream(x, x_dtype, w, k, n, bpr, plan)) return launch_stream(x, x_dtype, w, y, y_dtype, rows, k, n, bpr / 2, plan, stream);
     const bool pair_ok = (bpr % 2 == 0) && ((reinterpret_cast<uintptr_t>(w) & 3u) == 0);
     if (!pair_ok) {
         dim3 grid((n + kWaves - 1) / kWaves, rows);

@@ -112,6 +112,40 @@ def test_q8_0_matvec_matches_oracle(mod, n, k, rows):
         assert err <= 2e-4, (n, k, rows, dt, err)
 
 
+@pytest.mark.parametrize("n,k,rows,dt", [(1, 256, 1, torch.float32), (7, 256, 1, torch.float16), (1000, 256, 2, torch.bfloat16),
+                                         (4099, 1024, 1, torch.float16), (333, 2304, 3, torch.float32), (517, 5120, 1, torch.bfloat16),
+                                         (2050, 24576, 1, torch.float32), (61, 17408, 4, torch.bfloat16)])
+def test_q8_0_streamed_rows_straddling_steps(mod, n, k, rows, dt):
+    """Rows of a multiple of 256 weights on an aligned base take the single-launch kernel, whose 64-pair steps cut
+    through row ends: every output row against the oracle, max-abs as well as norm (a misplaced row would hide in a norm)."""
+    rng = np.random.default_rng(77 + n)
+    blocks = C.pack_q8_0(_weights(rng, n, k))
+    dev = torch.device("cuda:0")
+    print(f"case q8_0 streamed n={n} k={k} rows={rows} {dt}", flush=True)
+    x = torch.from_numpy(rng.standard_normal((rows, k)).astype(np.float32)).to(dev).to(dt)
+    y = mod.q8_0_gemm_forward(x, torch.from_numpy(blocks).to(dev), k, out_dtype=torch.float32)
+    torch.cuda.synchronize()
+    want = O.matmul_f(x.float().cpu().numpy(), O.dequant_rows(blocks, "q8_0", k))
+    got = y.cpu().numpy()
+    assert O.rel_l2(got, want) <= 2e-4
+    assert np.abs(got - want).max() <= 1e-3 * np.abs(want).max()
+
+
+def test_q8_0_unaligned_activation_rows_fall_back(mod):
+    """An activation view that starts 4 bytes into its allocation cannot be read in vector pieces: same result through the other kernels."""
+    rng = np.random.default_rng(5)
+    n, k = 64, 512
+    blocks = C.pack_q8_0(_weights(rng, n, k))
+    dev = torch.device("cuda:0")
+    store = torch.from_numpy(rng.standard_normal(k + 1).astype(np.float32)).to(dev)
+    x = store[1:].view(1, k)
+    y = mod.q8_0_gemm_forward(x, torch.from_numpy(blocks).to(dev), k, out_dtype=torch.float32)
+    y2 = mod.q8_0_gemm_forward(x.clone(), torch.from_numpy(blocks).to(dev), k, out_dtype=torch.float32)
+    torch.cuda.synchronize()
+    want = O.matmul_f(x.cpu().numpy(), O.dequant_rows(blocks, "q8_0", k))
+    assert O.rel_l2(y.cpu().numpy(), want) <= 2e-4 and O.rel_l2(y2.cpu().numpy(), want) <= 2e-4
+
+
 def test_q8_0_random_bytes_and_offset_base(mod):
     rng = np.random.default_rng(3)
     n, bpr = 40, 16
