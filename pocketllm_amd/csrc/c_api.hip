@@ -120,16 +120,23 @@ int superblock_matvec(const ActRows& act, const uint8_t* blocks, int type_id, vo
                       int rows, int n, int bpr, hipStream_t s, WeightRoute route) {
     switch (type_id) {
         case PLLM_TYPE_Q2_K: {
-            const int st = q2k_wave_matvec(act, blocks, y, y_dtype, rows, n, bpr, s, route);
+            const int st = groups16_wave_matvec(act, blocks, type_id, y, y_dtype, rows, n, bpr, s, route);
             return st != PLLM_ERR_UNSUPPORTED ? st : dot4_matvec_from_image(act, blocks, type_id, y, y_dtype, rows, n, bpr, s, route);
+        }
+        case PLLM_TYPE_Q6_K: {
+            const int st = groups16_wave_matvec(act, blocks, type_id, y, y_dtype, rows, n, bpr, s, route);
+            return st != PLLM_ERR_UNSUPPORTED ? st : iq_mfma_matvec_from_image(act, blocks, type_id, y, y_dtype, rows, n, bpr, s, route);
         }
         case PLLM_TYPE_IQ2_XXS:
         case PLLM_TYPE_IQ1_M:
         case PLLM_TYPE_IQ2_XS:
         case PLLM_TYPE_IQ3_XXS:
-        case PLLM_TYPE_IQ4_XS:
-        case PLLM_TYPE_Q6_K:
             return iq_mfma_matvec_from_image(act, blocks, type_id, y, y_dtype, rows, n, bpr, s, route);
+        case PLLM_TYPE_IQ4_XS: {
+            const int st = iq4xs_wave_matvec(act, blocks, y, y_dtype, rows, n, bpr, s, route);
+            if (st != PLLM_ERR_UNSUPPORTED) return st;
+            return iq_mfma_matvec_from_image(act, blocks, type_id, y, y_dtype, rows, n, bpr, s, route);
+        }
         case PLLM_TYPE_Q4_K:
         case PLLM_TYPE_Q5_K:
             return kquant_matvec_from_image(act, blocks, type_id, y, y_dtype, rows, n, bpr, s, route);

@@ -105,6 +105,7 @@ struct Q4K {
         b[0] = nib_lo(r.qa); b[1] = nib_hi(r.qa); b[2] = nib_lo(r.qb); b[3] = nib_hi(r.qb);
     }
     static __device__ __forceinline__ int group_of(int t, int ks) { return k45_group_of(t, ks); }
+    static __device__ __forceinline__ int half_of(int, int ks) { return ks & 1; }   // which 16 weights of the group the slice carries
     static __device__ __forceinline__ float combine(const Regs& r, int ks, float v0, float v1, const float4& g2) { return k45_combine(r.hdr, ks, v0, v1, g2); }
 };
 
@@ -126,10 +127,54 @@ struct Q5K {
         b[3] = fifth_bit(nib_hi(r.qb), r.qh, g + 5);
     }
     static __device__ __forceinline__ int group_of(int t, int ks) { return k45_group_of(t, ks); }
+    static __device__ __forceinline__ int half_of(int, int ks) { return ks & 1; }
     static __device__ __forceinline__ float combine(const Regs& r, int ks, float v0, float v1, const float4& g2) { return k45_combine(r.hdr, ks, v0, v1, g2); }
 };
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// ------------------------------------------------------------------------------------------------
+// IQ4_XS: 136 B = d(2) scales_h(2) scales_l(4) qs(128), blocks 8-byte aligned; w = d (ls - 32) kvalues[code],
+// ls six bits per 32 weights (low four in a nibble of scales_l, high two in scales_h); group g = qs[16 g, +16),
+// weights 0..15 in the low and 16..31 in the high nibbles.  Lane (n, ks) holds qs[32 ks, +32) = groups 2 ks and
+// 2 ks + 1; MFMA t, slice ks carries half t % 2 of group 2 ks + t / 2.  The 16-entry code table sits in four
+// constants; a byte permute picks from its lower and upper half and a third one chooses by bit 3 of the code.
+// ------------------------------------------------------------------------------------------------
+struct IQ4XS {
+    static constexpr int kBlockBytes = 136;
+    static constexpr int kDepth = 5;
+    struct Regs { uint2 hdr; uint4 q0, q1; };
+    struct __attribute__((packed, aligned(8))) Words { u32x4 v; };
+    static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, int ks) {
+        r.hdr = *reinterpret_cast<const uint2*>(blk);
+        const Words a = *reinterpret_cast<const Words*>(blk + 8 + 32 * ks);
+        const Words b = *reinterpret_cast<const Words*>(blk + 24 + 32 * ks);
+        r.q0 = make_uint4(a.v.x, a.v.y, a.v.z, a.v.w);
+        r.q1 = make_uint4(b.v.x, b.v.y, b.v.z, b.v.w);
+    }
+    // four codes (one per byte, 0..15) -> four table values
+    static __device__ __forceinline__ uint32_t values4(uint32_t codes) {
+        const uint32_t low3 = codes & 0x07070707u;
+        const uint32_t lower = __builtin_amdgcn_perm(0xF6EADDCFu, 0xBFAD9881u, low3);   // -127 -104 -83 -65 | -49 -35 -22 -10
+        const uint32_t upper = __builtin_amdgcn_perm(0x71594535u, 0x26190D01u, low3);   // 1 13 25 38 | 53 69 89 113
+        return __builtin_amdgcn_perm(upper, lower, ((codes >> 1) & 0x04040404u) | 0x03020100u);
+    }
+    static __device__ __forceinline__ uint4 values16(const uint4& q, int sh) {
+        return make_uint4(values4((q.x >> sh) & 0x0f0f0f0fu), values4((q.y >> sh) & 0x0f0f0f0fu),
+                          values4((q.z >> sh) & 0x0f0f0f0fu), values4((q.w >> sh) & 0x0f0f0f0fu));
+    }
+    static __device__ __forceinline__ void codes(const Regs& r, int, uint4 b[4]) {
+        b[0] = values16(r.q0, 0); b[1] = values16(r.q0, 4); b[2] = values16(r.q1, 0); b[3] = values16(r.q1, 4);
+    }
+    static __device__ __forceinline__ int group_of(int t, int ks) { return 2 * ks + (t >> 1); }
+    static __device__ __forceinline__ int half_of(int t, int) { return t & 1; }
+    static __device__ __forceinline__ float combine(const Regs& r, int ks, float v0, float v1, const float4& g2) {
+        const uint32_t scales_h = r.hdr.x >> 16, sl = (r.hdr.y >> (8 * ks)) & 0xffu;
+        const int ls0 = static_cast<int>((sl & 15u) | (((scales_h >> (4 * ks)) & 3u) << 4)) - 32;
+        const int ls1 = static_cast<int>((sl >> 4) | (((scales_h >> (4 * ks + 2)) & 3u) << 4)) - 32;
+        return f16_bits_to_float(r.hdr.x & 0xffffu) * (static_cast<float>(ls0) * g2.x * v0 + static_cast<float>(ls1) * g2.z * v1);
+    }
+};
 
 // R activation rows per workgroup (1, 2 or 4): the weights of a super-block are loaded and split into codes once and multiplied
 // with the images of R rows, which sit side by side in LDS; grid row blockIdx.y serves activation rows R * blockIdx.y ...
@@ -428,7 +473,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_image_matvec_kernel(
                     // this lane supplies row m = col = 2 * group + term of MFMA t's A operand, slice ks: codes only where that
                     // slice belongs to `group`, the zero bytes elsewhere
                     const int g = FMT::group_of(t, ks);
-                    const int off = (col >> 1) == g ? ((col & 1) ? 256 : 0) + 32 * g + 16 * (ks & 1) : kSlotBytes;
+                    const int off = (col >> 1) == g ? ((col & 1) ? 256 : 0) + 32 * g + 16 * FMT::half_of(t, ks) : kSlotBytes;
                     const uint4 a = *reinterpret_cast<const uint4*>(slot + off);
                     c = __builtin_amdgcn_mfma_i32_16x16x64_i8(as_v4i(a), as_v4i(bw[t]), c, 0, 0, 0);
                 }
@@ -521,30 +566,96 @@ int launch_wave(const ActRows& act, const WeightRoute& route, const uint8_t* w, 
 }
 
 // ------------------------------------------------------------------------------------------------
-// Q2_K in the same single-launch frame.  84 B = scales(16) qs(64) d(2) dmin(2): sixteen groups of 16
-// weights, 2-bit codes; group g lies in bytes qs[16 j, 16 j + 16), j = 2 (g / 8) + g % 2, at bit 2 s,
-// s = (g % 8) / 2; scale byte g = scale (low nibble) and min (high nibble).
-//     y = d sum_g sc_g dot(q_g, x_g) - dmin sum_g m_g sum(x_g).
-// A rows = the 16 groups, one MFMA set per activation term; MFMA t carries the weights [64 t, 64 t + 64),
-// groups 4 t .. 4 t + 3, lane (n, ks) supplies group 4 t + ks of weight row n as B and, where its A row
-// (= lane % 16) is that group, the group's 16 activation bytes as A.  C[4 ks .. 4 ks + 3][n] = the lane's
-// own four groups.  The wave's LDS slot adds the sums per 16 activations for the min terms.
+// Q2_K and Q6_K in the same single-launch frame: formats of sixteen groups of 16 weights.
+// A rows = the 16 groups, one MFMA set per activation term; lane (n, ks) supplies as B the 16 weights of
+// one group per MFMA t (the format says which) and, where its A row (= lane % 16) is that group, the
+// group's 16 activation bytes as A.  C[4 ks .. 4 ks + 3][n] = groups 4 ks .. 4 ks + 3 of weight row n,
+// whose scales the lane applies.  The wave's LDS slot adds the sums per 16 activations (Q2_K: min
+// terms; Q6_K: codes are left unsigned and the - 32 goes through the sums).
+//   Q2_K, 84 B = scales(16) qs(64) d(2) dmin(2): 2-bit codes; group g lies in bytes qs[16 j, 16 j + 16),
+//     j = 2 (g / 8) + g % 2, at bit 2 ((g % 8) / 2); scale byte g = scale (low nibble), min (high nibble);
+//     y = d sum_g sc_g dot(q_g, x_g) - dmin sum_g m_g sum(x_g).  MFMA t, slice ks: group 4 t + ks.
+//   Q6_K, 210 B = ql(128) qh(64) scales(16 x int8) d(2), blocks 2-byte aligned: code = low nibble | two
+//     high bits << 4, minus 32; lane (n, ks) holds ql[64 h + 16 p ..], ql[64 h + 32 + 16 p ..] and
+//     qh[32 h + 16 p ..] with h = ks / 2, p = ks % 2; MFMA t, slice ks: group 8 h + 2 t + p.
 // ------------------------------------------------------------------------------------------------
 constexpr int kQ2SlotBytes = kSlotBytes + 64;       // ... | float sum16[16]
-struct Q2Regs { uint32_t sc; uint4 qa, qb; uint32_t dd; };
 struct __attribute__((packed, aligned(4))) Dwords4 { u32x4 v; };
-
-__device__ __forceinline__ void q2_load(Q2Regs& r, const uint8_t* blk, int ks) {
-    r.sc = *reinterpret_cast<const uint32_t*>(blk + 4 * ks);               // scale bytes of groups 4 ks .. 4 ks + 3
-    const Dwords4 a = *reinterpret_cast<const Dwords4*>(blk + 16 + 16 * (ks & 1));
-    const Dwords4 b = *reinterpret_cast<const Dwords4*>(blk + 48 + 16 * (ks & 1));
-    r.qa = make_uint4(a.v.x, a.v.y, a.v.z, a.v.w);                        // groups 0 .. 7 with the lane's parity
-    r.qb = make_uint4(b.v.x, b.v.y, b.v.z, b.v.w);                        // groups 8 .. 15
-    r.dd = *reinterpret_cast<const uint32_t*>(blk + 80);
+struct __attribute__((packed, aligned(2))) Words16 { u32x4 v; };          // blocks on a 2-byte boundary: still one 16-byte load
+struct __attribute__((packed, aligned(2))) Words4 { uint32_t v; };
+__device__ __forceinline__ uint4 load16_a2(const uint8_t* p) {
+    const Words16 u = *reinterpret_cast<const Words16*>(p);
+    return make_uint4(u.v.x, u.v.y, u.v.z, u.v.w);
 }
 
-template <int ITERS, int DEPTH, bool X16>
-__global__ __launch_bounds__(64 * kMaxWaves) void wave_q2k_matvec_kernel(
+struct WaveQ2K {
+    static constexpr int kBlockBytes = 84;
+    static constexpr int kAlign = 4;
+    struct Regs { uint32_t sc; uint4 qa, qb; uint32_t dd; };
+    static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, int ks) {
+        r.sc = *reinterpret_cast<const uint32_t*>(blk + 4 * ks);               // scale bytes of groups 4 ks .. 4 ks + 3
+        const Dwords4 a = *reinterpret_cast<const Dwords4*>(blk + 16 + 16 * (ks & 1));
+        const Dwords4 b = *reinterpret_cast<const Dwords4*>(blk + 48 + 16 * (ks & 1));
+        r.qa = make_uint4(a.v.x, a.v.y, a.v.z, a.v.w);                        // groups 0 .. 7 with the lane's parity
+        r.qb = make_uint4(b.v.x, b.v.y, b.v.z, b.v.w);                        // groups 8 .. 15
+        r.dd = *reinterpret_cast<const uint32_t*>(blk + 80);
+    }
+    // the MFMA and slice that carry group `col`
+    static __device__ __forceinline__ int slice_of(int col) { return col & 3; }
+    static __device__ __forceinline__ int mfma_of(int col) { return col >> 2; }
+    static __device__ __forceinline__ uint4 codes(const Regs& r, int t, int ks) {
+        const uint4 piece = t < 2 ? r.qa : r.qb;
+        const int sh = 2 * (ks >> 1) + 4 * (t & 1);                             // codes of MFMA t sit at bit 2 (2 (t % 2) + ks / 2)
+        return make_uint4((piece.x >> sh) & 0x03030303u, (piece.y >> sh) & 0x03030303u, (piece.z >> sh) & 0x03030303u, (piece.w >> sh) & 0x03030303u);
+    }
+    // dots[j], xs[j], sums[j]: integer dot (both terms joined), activation scale and activation sum of group 4 ks + j
+    static __device__ __forceinline__ float finish(const Regs& r, const float (&dots)[4], const float (&xs)[4], const float (&sums)[4]) {
+        float pos = 0.0f, neg = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t sb = (r.sc >> (8 * j)) & 0xffu;
+            pos += static_cast<float>(sb & 15u) * xs[j] * dots[j];
+            neg += static_cast<float>(sb >> 4) * sums[j];
+        }
+        return f16_bits_to_float(r.dd & 0xffffu) * pos - f16_bits_to_float(r.dd >> 16) * neg;
+    }
+};
+
+struct WaveQ6K {
+    static constexpr int kBlockBytes = 210;
+    static constexpr int kAlign = 2;
+    struct Regs { uint4 qa, qb, qh; uint32_t sc, d; };
+    static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, int ks) {
+        const int half = ks >> 1, part = ks & 1;
+        r.qa = load16_a2(blk + 64 * half + 16 * part);
+        r.qb = load16_a2(blk + 64 * half + 32 + 16 * part);
+        r.qh = load16_a2(blk + 128 + 32 * half + 16 * part);
+        r.sc = reinterpret_cast<const Words4*>(blk + 192 + 4 * ks)->v;     // int8 scales of groups 4 ks .. 4 ks + 3
+        r.d = *reinterpret_cast<const uint16_t*>(blk + 208);
+    }
+    static __device__ __forceinline__ int slice_of(int col) { return 2 * (col >> 3) + (col & 1); }
+    static __device__ __forceinline__ int mfma_of(int col) { return (col >> 1) & 3; }
+    static __device__ __forceinline__ uint32_t code4(uint32_t ql, uint32_t qh, int t) {
+        const uint32_t lo = (t < 2 ? ql : ql >> 4) & 0x0f0f0f0fu;
+        const uint32_t hi = (t == 0 ? qh << 4 : t == 1 ? qh << 2 : t == 2 ? qh : qh >> 2) & 0x30303030u;
+        return lo | hi;
+    }
+    static __device__ __forceinline__ uint4 codes(const Regs& r, int t, int) {
+        const uint4 ql = (t & 1) ? r.qb : r.qa;
+        return make_uint4(code4(ql.x, r.qh.x, t), code4(ql.y, r.qh.y, t), code4(ql.z, r.qh.z, t), code4(ql.w, r.qh.w, t));
+    }
+    static __device__ __forceinline__ float finish(const Regs& r, const float (&dots)[4], const float (&xs)[4], const float (&sums)[4]) {
+        const int sc = static_cast<int>(r.sc);
+        const float v = static_cast<float>(static_cast<int8_t>(sc)) * (xs[0] * dots[0] - 32.0f * sums[0]) +
+                        static_cast<float>(static_cast<int8_t>(sc >> 8)) * (xs[1] * dots[1] - 32.0f * sums[1]) +
+                        static_cast<float>(static_cast<int8_t>(sc >> 16)) * (xs[2] * dots[2] - 32.0f * sums[2]) +
+                        static_cast<float>(sc >> 24) * (xs[3] * dots[3] - 32.0f * sums[3]);
+        return f16_bits_to_float(r.d) * v;
+    }
+};
+
+template <typename FMT, int ITERS, int DEPTH, bool X16>
+__global__ __launch_bounds__(64 * kMaxWaves) void wave_groups16_matvec_kernel(
     const void* __restrict__ x, int x_dtype, int k, const WeightRoute route, const uint8_t* __restrict__ w, void* __restrict__ y,
     int y_dtype, int n, int bpr) {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -565,25 +676,24 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_q2k_matvec_kernel(
     }
     if (static_cast<int>(blockIdx.x) * kRowsPerWg >= n) return;
     const int row = blockIdx.x * kRowsPerWg + col;
-    const uint8_t* wrow = w + static_cast<size_t>(row < n ? row : 0) * bpr * 84;
+    const uint8_t* wrow = w + static_cast<size_t>(row < n ? row : 0) * bpr * FMT::kBlockBytes;
     const size_t xoff = static_cast<size_t>(blockIdx.y) * k;
-    // the lane's A operand: group `col` of the block, in the one MFMA (t = col / 4) whose slice ks carries that group
-    const bool mine = (col & 3) == ks;
-    const int my_t = col >> 2;
-    const int bit = 2 * (ks >> 1);                                           // codes of MFMA t sit at bit 2 (2 (t % 2) + ks / 2)
+    // the lane's A operand: group `col` of the block, in the one MFMA whose slice ks carries that group
+    const bool mine = FMT::slice_of(col) == ks;
+    const int my_t = FMT::mfma_of(col);
 
     if (lane < 4) reinterpret_cast<uint32_t*>(slot + kQ2SlotBytes)[lane] = 0;
     float acc = 0.0f;
     for (int b0 = wave; b0 < bpr; b0 += waves * ITERS) {
         RawX<X16> raw[DEPTH];
-        Q2Regs regs[DEPTH];
+        typename FMT::Regs regs[DEPTH];
         auto request_x = [&](int it) {
             const int b = b0 + it * waves;
             request_raw4<X16>(raw[it % DEPTH], x, xoff, 256 * b + 4 * lane, b < bpr ? k : 0);
         };
         auto request_w = [&](int it) {
             const int b = b0 + it * waves;
-            q2_load(regs[it % DEPTH], wrow + static_cast<size_t>(min(b, bpr - 1)) * 84, ks);   // clamped: always a valid address
+            FMT::load(regs[it % DEPTH], wrow + static_cast<size_t>(min(b, bpr - 1)) * FMT::kBlockBytes, ks);   // clamped: always a valid address
         };
 #pragma unroll
         for (int it = 0; it < DEPTH; ++it) request_x(it);
@@ -609,14 +719,11 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_q2k_matvec_kernel(
                 if ((lane & 3) == 0) reinterpret_cast<float*>(slot + kSlotBytes)[lane >> 2] = sum;
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
                 __builtin_amdgcn_wave_barrier();                            // LDS serves a wave's requests in order
-                const Q2Regs& r = regs[it % DEPTH];
+                const typename FMT::Regs& r = regs[it % DEPTH];
                 v4i ch = {0, 0, 0, 0}, cl = {0, 0, 0, 0};
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
-                    const uint4 piece = t < 2 ? r.qa : r.qb;
-                    const int sh = bit + 4 * (t & 1);
-                    const uint4 bw = make_uint4((piece.x >> sh) & 0x03030303u, (piece.y >> sh) & 0x03030303u,
-                                                (piece.z >> sh) & 0x03030303u, (piece.w >> sh) & 0x03030303u);
+                    const uint4 bw = FMT::codes(r, t, ks);
                     const int off = (mine && t == my_t) ? 16 * col : kQ2SlotBytes;
                     const uint4 ah = *reinterpret_cast<const uint4*>(slot + off);
                     const uint4 al = *reinterpret_cast<const uint4*>(slot + off + ((mine && t == my_t) ? 256 : 0));
@@ -629,14 +736,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_q2k_matvec_kernel(
                                      static_cast<float>(__mul24(ch.z, 254) + cl.z), static_cast<float>(__mul24(ch.w, 254) + cl.w)};
                 const float xsv[4] = {g2.x, g2.x, g2.z, g2.z};
                 const float smv[4] = {s16.x, s16.y, s16.z, s16.w};
-                float pos = 0.0f, neg = 0.0f;
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const uint32_t sb = (r.sc >> (8 * j)) & 0xffu;
-                    pos += static_cast<float>(sb & 15u) * xsv[j] * vv[j];
-                    neg += static_cast<float>(sb >> 4) * smv[j];
-                }
-                acc += f16_bits_to_float(r.dd & 0xffffu) * pos - f16_bits_to_float(r.dd >> 16) * neg;
+                acc += FMT::finish(r, vv, xsv, smv);
                 __builtin_amdgcn_wave_barrier();                            // the next block's slice overwrites the slot
             }
             if (it + DEPTH < ITERS) {
@@ -706,6 +806,28 @@ int launch_k45(const ActRows& act, const WeightRoute& route, const uint8_t* w, v
     return launch_k45_rows<FMT, 1>(act, route, w, y, y_dtype, rows, n, bpr, stream);
 }
 
+template <typename FMT>
+int launch_groups16(const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream) {
+    // raw rows without normalisation or routing, blocks on the format's boundary; everything else stays with the other kernels
+    if (!act.x || act.k < 4 || act.gamma || route.expert || act.row_token || (reinterpret_cast<uintptr_t>(w) & (FMT::kAlign - 1))) return PLLM_ERR_UNSUPPORTED;
+    for (int m = 0; m < route.extra; ++m)
+        if (reinterpret_cast<uintptr_t>(route.more_w[m]) & (FMT::kAlign - 1)) return PLLM_ERR_UNSUPPORTED;
+    int waves, iters;
+    int tiles = (n + kRowsPerWg - 1) / kRowsPerWg;
+    for (int m = 0; m < route.extra; ++m) tiles += (route.more_n[m] + kRowsPerWg - 1) / kRowsPerWg;
+    split_blocks(bpr, tiles * rows, waves, iters);
+    constexpr int kMaxDepth = sizeof(typename FMT::Regs) > 48 ? 2 : 6;      // blocks in flight per wave (Q6_K: 2, 3, 4 and 5 ran within 3 % of each other: five waves per SIMD fit with 2)
+#define PLLM_CASE(I) case I: { \
+        constexpr int D = I < kMaxDepth ? I : kMaxDepth; \
+        return act.x_dtype == PLLM_F32 ? launch_q2k_kernel(wave_groups16_matvec_kernel<FMT, I, D, false>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream) \
+                                       : launch_q2k_kernel(wave_groups16_matvec_kernel<FMT, I, D, true>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream); }
+    switch (iters) {
+        PLLM_CASE(1) PLLM_CASE(2) PLLM_CASE(3) PLLM_CASE(4) PLLM_CASE(5) PLLM_CASE(6)
+        default: PLLM_CASE(8)
+    }
+#undef PLLM_CASE
+}
+
 }  // namespace
 
 size_t kquant_matvec_workspace_bytes(int rows, int bpr) { return act_image_256_bytes(bpr) * static_cast<size_t>(rows); }
@@ -719,23 +841,19 @@ int kquant_matvec_from_image(const ActRows& act, const uint8_t* w, int type_id, 
     }
 }
 
-int q2k_wave_matvec(const ActRows& act, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream, WeightRoute route) {
-    // raw rows without normalisation or routing, blocks on a 4-byte boundary; everything else stays with the v_dot4 kernels
-    if (!act.x || act.k < 4 || act.gamma || route.expert || act.row_token || (reinterpret_cast<uintptr_t>(w) & 3u)) return PLLM_ERR_UNSUPPORTED;
+int iq4xs_wave_matvec(const ActRows& act, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream, WeightRoute route) {
+    // raw rows without routing, blocks on an 8-byte boundary; everything else stays with the tile-frame kernel
+    if (!act.x || act.k < 4 || route.expert || act.row_token || (reinterpret_cast<uintptr_t>(w) & 7u)) return PLLM_ERR_UNSUPPORTED;
     for (int m = 0; m < route.extra; ++m)
-        if (reinterpret_cast<uintptr_t>(route.more_w[m]) & 3u) return PLLM_ERR_UNSUPPORTED;
-    int waves, iters;
-    int tiles = (n + kRowsPerWg - 1) / kRowsPerWg;
-    for (int m = 0; m < route.extra; ++m) tiles += (route.more_n[m] + kRowsPerWg - 1) / kRowsPerWg;
-    split_blocks(bpr, tiles * rows, waves, iters);
-#define PLLM_CASE(I, D) case I: \
-        return act.x_dtype == PLLM_F32 ? launch_q2k_kernel(wave_q2k_matvec_kernel<I, D, false>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream) \
-                                       : launch_q2k_kernel(wave_q2k_matvec_kernel<I, D, true>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream)
-    switch (iters) {
-        PLLM_CASE(1, 1); PLLM_CASE(2, 2); PLLM_CASE(3, 3); PLLM_CASE(4, 4); PLLM_CASE(5, 5); PLLM_CASE(6, 6);
-        default: PLLM_CASE(8, 6);
-    }
-#undef PLLM_CASE
+        if (reinterpret_cast<uintptr_t>(route.more_w[m]) & 7u) return PLLM_ERR_UNSUPPORTED;
+    return act.gamma ? launch_wave<IQ4XS, true>(act, route, w, y, y_dtype, rows, n, bpr, stream)
+                     : launch_wave<IQ4XS, false>(act, route, w, y, y_dtype, rows, n, bpr, stream);
+}
+
+int groups16_wave_matvec(const ActRows& act, const uint8_t* w, int type_id, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream, WeightRoute route) {
+    if (type_id == PLLM_TYPE_Q2_K) return launch_groups16<WaveQ2K>(act, route, w, y, y_dtype, rows, n, bpr, stream);
+    if (type_id == PLLM_TYPE_Q6_K) return launch_groups16<WaveQ6K>(act, route, w, y, y_dtype, rows, n, bpr, stream);
+    return PLLM_ERR_UNSUPPORTED;
 }
 
 }  // namespace pllm

@@ -70,8 +70,11 @@ int kquant_matvec_from_image(const ActRows& act, const uint8_t* w, int type_id, 
                              int rows, int n, int bpr, hipStream_t stream, WeightRoute route = WeightRoute{});
 int dot4_matvec_from_image(const ActRows& act, const uint8_t* w, int type_id, void* y, int y_dtype,
                            int rows, int n, int bpr, hipStream_t stream, WeightRoute route = WeightRoute{});
-// Q2_K on raw activation rows in the single-launch frame of matvec_kquant.hip (PLLM_ERR_UNSUPPORTED: take dot4_matvec_from_image)
-int q2k_wave_matvec(const ActRows& act, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream,
+// Q2_K / Q6_K and IQ4_XS on raw activation rows in the single-launch frames of matvec_kquant.hip (PLLM_ERR_UNSUPPORTED: take the
+// kernels for prepared images)
+int iq4xs_wave_matvec(const ActRows& act, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream,
+                      WeightRoute route = WeightRoute{});
+int groups16_wave_matvec(const ActRows& act, const uint8_t* w, int type_id, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream,
                     WeightRoute route = WeightRoute{});
 int iq_mfma_matvec_from_image(const ActRows& act, const uint8_t* w, int type_id, void* y, int y_dtype,
                               int rows, int n, int bpr, hipStream_t stream, WeightRoute route = WeightRoute{});

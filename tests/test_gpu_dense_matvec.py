@@ -362,7 +362,7 @@ def test_activation_image_first_term_equals_the_reference_quantizer(mod, dtype):
 @pytest.mark.parametrize("type_name", ["q4_k", "q5_k", "q2_k", "q6_k", "iq4_xs", "iq2_xxs", "iq1_m", "iq2_xs", "iq3_xxs"])
 def test_few_row_calls_equal_the_prequantized_path(mod, type_name):
     """Calls of a few rows may quantize the activations inside the matvec kernel; the result is the same bits as quantizing ahead
-    (Q2_K: the same activation image and integer dots, summed in another order by a different kernel: equal to float32 rounding)."""
+    (Q2_K, Q6_K, IQ4_XS: the same activation image and integer dots, summed in another order by a different kernel: equal to float32 rounding)."""
     rng = np.random.default_rng(78)
     dev = torch.device("cuda:0")
     tid = O.TYPE_IDS[type_name]
@@ -381,7 +381,7 @@ def test_few_row_calls_equal_the_prequantized_path(mod, type_name):
             print(f"case few-row {type_name} n={n} k={k} rows={rows} {dt}", flush=True)
             y = mod.gguf_quant_gemm_forward(x, blocks, k, tid, codebooks.grid_tensor_for_type(tid).to(dev), out_dtype=torch.float32)
             y_pre = mod.gguf_quant_gemm_prequantized(mod.quantize_activations(x, bpr), blocks, tid, out_dtype=torch.float32)
-            if type_name == "q2_k":
+            if type_name in ("q2_k", "q6_k", "iq4_xs"):
                 assert O.rel_l2(y.cpu().numpy(), y_pre.cpu().numpy()) <= 1e-6
             else:
                 assert torch.equal(y, y_pre)
