@@ -456,6 +456,35 @@ def pmc_pass(mod, dev) -> None:
     print(json.dumps({"pmc_pass": f"{name} matvec {n}x{k}", "weight_bytes": int(blocks.size), "copy_bytes": int(nbytes)}))
 
 
+def decode_pass(mod, dev) -> None:
+    """A few launches of the other dense decode kernels for the profiler: Q8_0 4096x4096 and 17408x5120, FP8 17408x5120,
+    Q2_K, Q6_K and IQ4_XS 17408x5120 (rings of weight copies, so that no launch finds its matrix in cache)."""
+    from pocketllm_amd import block_codec as C, codebooks
+    rng = np.random.default_rng(6006)
+    for n, k in ((4096, 4096), (17408, 5120)):
+        ring = ring_of(C.pack_q8_0((rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02))), dev, 8)
+        x = torch.randn(1, k, device=dev)
+        for i in range(24):
+            mod.q8_0_gemm_forward(x, ring[i % len(ring)], k)
+        del ring
+    codes, scale = C.quantize_fp8_block((rng.standard_normal((17408, 5120), dtype=np.float32) * np.float32(0.02)))
+    ring = ring_of(codes, dev, 8)
+    sc = torch.from_numpy(scale).to(dev)
+    x = torch.randn(1, 5120, device=dev, dtype=torch.bfloat16)
+    for i in range(24):
+        mod.fp8_block_gemm_forward(x, ring[i % len(ring)], sc)
+    del ring
+    for name, tid, blocks in (("q2_k", 1, C.quantize_q2_k((rng.standard_normal((17408, 5120), dtype=np.float32) * np.float32(0.02)))),
+                              ("q6_k", 8, C.random_blocks(rng, "q6_k", 17408, 20)), ("iq4_xs", 7, C.random_blocks(rng, "iq4_xs", 17408, 20))):
+        ring = ring_of(blocks, dev, 8)
+        grid = codebooks.grid_tensor_for_type(tid).to(dev)
+        for i in range(24):
+            mod.gguf_quant_gemm_forward(x, ring[i % len(ring)], 5120, tid, grid)
+        del ring
+    torch.cuda.synchronize()
+    print(json.dumps({"decode_pass": "q8_0 4096x4096 + 17408x5120, fp8 17408x5120, q2_k / q6_k / iq4_xs 17408x5120, 24 launches each"}))
+
+
 def iq_pass(mod, dev) -> None:
     """A few launches of the codebook formats for the profiler: IQ2_XXS 98304x3072 and IQ1_M 196608x1536 matvec, then the
     single-token routed experts of the 256-expert top-8 configuration."""
@@ -509,6 +538,7 @@ def main() -> None:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--pmc-pass", action="store_true", help="short run for rocprofv3 --pmc: dominant kernel + a copy of the same size")
     ap.add_argument("--prefill-pass", action="store_true", help="short run for rocprofv3: a few launches of the MFMA tile kernel")
+    ap.add_argument("--decode-pass", action="store_true", help="short run for rocprofv3: Q8_0, FP8, Q2_K, Q6_K and IQ4_XS decode matvec")
     ap.add_argument("--iq-pass", action="store_true", help="short run for rocprofv3: IQ2_XXS / IQ1_M matvec and the single-token experts")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -529,6 +559,9 @@ def main() -> None:
         return
     if args.prefill_pass:
         prefill_pass(mod, dev)
+        return
+    if args.decode_pass:
+        decode_pass(mod, dev)
         return
     if args.iq_pass:
         iq_pass(mod, dev)

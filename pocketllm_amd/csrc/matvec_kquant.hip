@@ -816,7 +816,7 @@ int launch_groups16(const ActRows& act, const WeightRoute& route, const uint8_t*
     int tiles = (n + kRowsPerWg - 1) / kRowsPerWg;
     for (int m = 0; m < route.extra; ++m) tiles += (route.more_n[m] + kRowsPerWg - 1) / kRowsPerWg;
     split_blocks(bpr, tiles * rows, waves, iters);
-    constexpr int kMaxDepth = sizeof(typename FMT::Regs) > 48 ? 2 : 6;      // blocks in flight per wave (Q6_K: 2, 3, 4 and 5 ran within 3 % of each other: five waves per SIMD fit with 2)
+    constexpr int kMaxDepth = 2;            // blocks in flight per wave: five waves per SIMD fit with 2 (Q6_K with 2, 3, 4 and 5 ran within 3 % of each other, Q2_K 14.6 us with 2 against 15.2 with 5)
 #define PLLM_CASE(I) case I: { \
         constexpr int D = I < kMaxDepth ? I : kMaxDepth; \
         return act.x_dtype == PLLM_F32 ? launch_q2k_kernel(wave_groups16_matvec_kernel<FMT, I, D, false>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream) \
