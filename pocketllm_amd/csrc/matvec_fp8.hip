@@ -19,7 +19,8 @@ constexpr int kWaves = 4;
 constexpr int kThreads = 64 * kWaves;
 // register slots per wave: the fused gate/up form holds the same row of both matrices, the plain form one row (two rows per wave
 // cost 0.8 us at 17408x5120: 19.6 against 18.9 us)
-template <bool SWIGLU> constexpr int slots() { return SWIGLU ? 2 : 1; }
+// (calls on several activation rows keep two rows per wave: 25.8 us against 29.5 at two rows)
+template <bool SWIGLU, int R> constexpr int kSlots = (SWIGLU || R > 1) ? 2 : 1;
 
 typedef float v2f __attribute__((ext_vector_type(2)));
 
@@ -100,7 +101,8 @@ __device__ __forceinline__ void stage_row_finish(float* xs, const float (&v)[kSt
 // Register slots of a wave: one row of the matrix, or (SWIGLU) the same row of the gate and of the up matrix.
 template <bool SWIGLU>
 __device__ __forceinline__ const Fp8Mat& slot_mat(const Fp8Mat& a, const Fp8Mat& b, int q) { return (SWIGLU && q == 1) ? b : a; }
-__device__ __forceinline__ int slot_row(int row0, int n) { return min(row0, n - 1); }
+// (plain form with two slots: the second slot's row lies rstride rows behind the first one's, in the workgroup's next group of rows)
+__device__ __forceinline__ int slot_row(int row0, int q, int rstride, int n) { return min(row0 + q * rstride, n - 1); }
 
 __device__ __forceinline__ float chunk_dot(const uint4& w, const float* xp) {
     const float4 x0 = *reinterpret_cast<const float4*>(xp);
@@ -126,19 +128,19 @@ __device__ __forceinline__ float chunk_dot(const uint4& w, const float* xp) {
 // second register set while it multiplies the current one.
 // The block scales of a pass travel with its weights, requested ahead of them: loads return in order, so a scale asked for
 // while the pass is multiplied would arrive behind the weights of the pass after it and hold the arithmetic until those are in.
-template <int ITERS, int F16S, bool SWIGLU>
-__device__ __forceinline__ void fp8_fetch_pass(uint4 (&r)[slots<SWIGLU>()][ITERS], uint32_t (&sc)[slots<SWIGLU>()][ITERS], const Fp8Mat& ma, const Fp8Mat& mb,
-                                               int row0, int n, int chunks, int c0, int lane) {
+template <int ITERS, int F16S, bool SWIGLU, int SLOTS>
+__device__ __forceinline__ void fp8_fetch_pass(uint4 (&r)[SLOTS][ITERS], uint32_t (&sc)[SLOTS][ITERS], const Fp8Mat& ma, const Fp8Mat& mb,
+                                               int row0, int rstride, int n, int chunks, int c0, int lane) {
 #pragma unroll
-    for (int q = 0; q < slots<SWIGLU>(); ++q) {
+    for (int q = 0; q < SLOTS; ++q) {
         const Fp8Mat& m = slot_mat<SWIGLU>(ma, mb, q);
-        const size_t srow = static_cast<size_t>(slot_row(row0, n) >> 7) * m.sstride;
+        const size_t srow = static_cast<size_t>(slot_row(row0, q, rstride, n) >> 7) * m.sstride;
 #pragma unroll
         for (int it = 0; it < ITERS; ++it) sc[q][it] = scale_raw_at<F16S>(m.scale, srow + (min(c0 + it * 64 + lane, chunks - 1) >> 3));
     }
 #pragma unroll
-    for (int q = 0; q < slots<SWIGLU>(); ++q) {
-        const uint8_t* wrow = slot_mat<SWIGLU>(ma, mb, q).w + static_cast<size_t>(slot_row(row0, n)) * slot_mat<SWIGLU>(ma, mb, q).wstride;
+    for (int q = 0; q < SLOTS; ++q) {
+        const uint8_t* wrow = slot_mat<SWIGLU>(ma, mb, q).w + static_cast<size_t>(slot_row(row0, q, rstride, n)) * slot_mat<SWIGLU>(ma, mb, q).wstride;
 #pragma unroll
         for (int it = 0; it < ITERS; ++it) r[q][it] = *reinterpret_cast<const uint4*>(wrow + 16 * min(c0 + it * 64 + lane, chunks - 1));
     }
@@ -171,16 +173,16 @@ __device__ __forceinline__ float floats_dot(const float (&f)[16], const float* x
 }
 
 // R activation rows (xs holds them k floats apart) against the pass's weights: the codes are converted once per chunk
-template <int ITERS, int F16S, bool SWIGLU, int R>
-__device__ __forceinline__ void fp8_multiply_pass(float (&acc)[slots<SWIGLU>()][R], const uint4 (&r)[slots<SWIGLU>()][ITERS],
-                                                  const uint32_t (&scales)[slots<SWIGLU>()][ITERS], const float* xs, int k, int chunks, int c0, int lane) {
+template <int ITERS, int F16S, bool SWIGLU, int R, int SLOTS>
+__device__ __forceinline__ void fp8_multiply_pass(float (&acc)[SLOTS][R], const uint4 (&r)[SLOTS][ITERS],
+                                                  const uint32_t (&scales)[SLOTS][ITERS], const float* xs, int k, int chunks, int c0, int lane) {
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
         const int c = c0 + it * 64 + lane;
         const bool ok = c < chunks;
         const int cc = ok ? c : 0;
 #pragma unroll
-        for (int q = 0; q < slots<SWIGLU>(); ++q) {
+        for (int q = 0; q < SLOTS; ++q) {
             const float sc = scale_value<F16S>(scales[q][it]);
             if constexpr (R == 1) {
                 const float d = chunk_dot(r[q][it], xs + 16 * cc);
@@ -199,22 +201,22 @@ __device__ __forceinline__ void fp8_multiply_pass(float (&acc)[slots<SWIGLU>()][
 }
 
 // activation rows arow0 .. arow0 + R - 1 (those below total_rows) of output row(s) row0
-template <bool SWIGLU, int R>
-__device__ __forceinline__ void fp8_store_rows(float (&acc)[slots<SWIGLU>()][R], void* __restrict__ y, int y_dtype, size_t y_stride, int arow0, int total_rows,
-                                               int row0, int n, int lane) {
+template <bool SWIGLU, int R, int SLOTS>
+__device__ __forceinline__ void fp8_store_rows(float (&acc)[SLOTS][R], void* __restrict__ y, int y_dtype, size_t y_stride, int arow0, int total_rows,
+                                               int row0, int rstride, int n, int lane) {
 #pragma unroll
     for (int a = 0; a < R; ++a) {
-        float total[slots<SWIGLU>()];
+        float total[SLOTS];
 #pragma unroll
-        for (int q = 0; q < slots<SWIGLU>(); ++q) { total[q] = group_sum<64>(acc[q][a]); acc[q][a] = 0.0f; }
+        for (int q = 0; q < SLOTS; ++q) { total[q] = group_sum<64>(acc[q][a]); acc[q][a] = 0.0f; }
         if (arow0 + a >= total_rows) continue;
         const size_t yoff = static_cast<size_t>(arow0 + a) * y_stride;
         if constexpr (SWIGLU) {
             if (lane == 0 && row0 < n) store_any(y, y_dtype, yoff + row0, silu(total[0]) * total[1]);
         } else {
 #pragma unroll
-            for (int q = 0; q < slots<SWIGLU>(); ++q)
-                if (lane == 0 && row0 < n) store_any(y, y_dtype, yoff + row0, total[q]);
+            for (int q = 0; q < SLOTS; ++q)
+                if (lane == 0 && row0 + q * rstride < n) store_any(y, y_dtype, yoff + row0 + q * rstride, total[q]);
         }
     }
 }
@@ -236,13 +238,16 @@ __global__ __launch_bounds__(kThreads) void fp8_persistent_matvec_kernel(
     // row of the gate and of the up matrix.
     constexpr int rows_per_group = kWaves;
     const int wave_row = wave;
-    const int step = gridDim.x;
+    // two plain slots: the wave's rows of this workgroup's current and next group (groups are dealt round-robin)
+    constexpr bool kTwoPlain = !SWIGLU && kSlots<SWIGLU, R> == 2;
+    const int step = kTwoPlain ? 2 * gridDim.x : gridDim.x;
+    const int rstride = kTwoPlain ? rows_per_group * static_cast<int>(gridDim.x) : 0;
 
-    uint4 a[slots<SWIGLU>()][ITERS], b[slots<SWIGLU>()][ITERS];
-    uint32_t sa[slots<SWIGLU>()][ITERS], sb[slots<SWIGLU>()][ITERS];
-    float acc[slots<SWIGLU>()][R];
+    uint4 a[kSlots<SWIGLU, R>][ITERS], b[kSlots<SWIGLU, R>][ITERS];
+    uint32_t sa[kSlots<SWIGLU, R>][ITERS], sb[kSlots<SWIGLU, R>][ITERS];
+    float acc[kSlots<SWIGLU, R>][R];
 #pragma unroll
-    for (int q = 0; q < slots<SWIGLU>(); ++q)
+    for (int q = 0; q < kSlots<SWIGLU, R>; ++q)
 #pragma unroll
         for (int r = 0; r < R; ++r) acc[q][r] = 0.0f;
     int g = blockIdx.x, p = 0;               // the pass being multiplied
@@ -251,10 +256,10 @@ __global__ __launch_bounds__(kThreads) void fp8_persistent_matvec_kernel(
         float head[kStageBatch][4];
         const size_t xoff = static_cast<size_t>(arow0) * x_stride;
         stage_row_request(head, x, x_dtype, xoff, k);
-        fp8_fetch_pass<ITERS, F16S, SWIGLU>(a, sa, ma, mb, g * rows_per_group + wave_row, n, chunks, 0, lane);
+        fp8_fetch_pass<ITERS, F16S, SWIGLU>(a, sa, ma, mb, g * rows_per_group + wave_row, rstride, n, chunks, 0, lane);
         stage_row_finish(xs, head, x, x_dtype, xoff, k);
     } else {
-        fp8_fetch_pass<ITERS, F16S, SWIGLU>(a, sa, ma, mb, g * rows_per_group + wave_row, n, chunks, 0, lane);
+        fp8_fetch_pass<ITERS, F16S, SWIGLU>(a, sa, ma, mb, g * rows_per_group + wave_row, rstride, n, chunks, 0, lane);
 #pragma unroll 1
         for (int r = 0; r < R; ++r)          // rows past the end: the last row again, result dropped
             stage_row_f32(xs + static_cast<size_t>(r) * k, x, x_dtype, static_cast<size_t>(min(arow0 + r, total_rows - 1)) * x_stride, k);
@@ -264,15 +269,15 @@ __global__ __launch_bounds__(kThreads) void fp8_persistent_matvec_kernel(
         if (++pn == passes) { pn = 0; gn += step; }
         // (fetched without a condition, past the last group its rows again: a branch around the loads would make the compiler wait
         // for them at the join, ahead of the arithmetic on the other register set)
-        fp8_fetch_pass<ITERS, F16S, SWIGLU>(b, sb, ma, mb, min(gn, groups - 1) * rows_per_group + wave_row, n, chunks, pn * kPassChunks, lane);
+        fp8_fetch_pass<ITERS, F16S, SWIGLU>(b, sb, ma, mb, min(gn, groups - 1) * rows_per_group + wave_row, rstride, n, chunks, pn * kPassChunks, lane);
         fp8_multiply_pass<ITERS, F16S, SWIGLU, R>(acc, a, sa, xs, k, chunks, p * kPassChunks, lane);
-        if (p == passes - 1) fp8_store_rows<SWIGLU, R>(acc, y, y_dtype, y_stride, arow0, total_rows, g * rows_per_group + wave_row, n, lane);
+        if (p == passes - 1) fp8_store_rows<SWIGLU, R>(acc, y, y_dtype, y_stride, arow0, total_rows, g * rows_per_group + wave_row, rstride, n, lane);
         g = gn; p = pn;
         if (g >= groups) break;
         if (++pn == passes) { pn = 0; gn += step; }
-        fp8_fetch_pass<ITERS, F16S, SWIGLU>(a, sa, ma, mb, min(gn, groups - 1) * rows_per_group + wave_row, n, chunks, pn * kPassChunks, lane);
+        fp8_fetch_pass<ITERS, F16S, SWIGLU>(a, sa, ma, mb, min(gn, groups - 1) * rows_per_group + wave_row, rstride, n, chunks, pn * kPassChunks, lane);
         fp8_multiply_pass<ITERS, F16S, SWIGLU, R>(acc, b, sb, xs, k, chunks, p * kPassChunks, lane);
-        if (p == passes - 1) fp8_store_rows<SWIGLU, R>(acc, y, y_dtype, y_stride, arow0, total_rows, g * rows_per_group + wave_row, n, lane);
+        if (p == passes - 1) fp8_store_rows<SWIGLU, R>(acc, y, y_dtype, y_stride, arow0, total_rows, g * rows_per_group + wave_row, rstride, n, lane);
         g = gn; p = pn;
     }
 }
@@ -340,9 +345,10 @@ int launch_any(const void* x, int x_dtype, size_t x_stride, const Fp8Mat& ma, co
     // persistent: the workgroups that fit a compute unit at once (two by registers, fewer when the activation rows fill LDS),
     // groups dealt round-robin
     const int per_cu = std::max(1, std::min(2, static_cast<int>((160 * 1024) / std::max<size_t>(smem, 1))));
-    const int grid_x = std::min(groups, per_cu * compute_units());
+    const int grid_x = std::min((!SWIGLU && share > 1) ? (groups + 1) / 2 : groups, per_cu * compute_units());
     const dim3 grid(grid_x, (rows + share - 1) / share);
-    // (the form with a compile-time pass count keeps both register sets and all accumulators of several rows live at once and spills;
+    // (the form with the pass count as a variable needs 70 registers against 168 and is slower on rows of one pass: 21.5 against 18.9 us;
+    // the form with a compile-time pass count keeps both register sets and all accumulators of several rows live at once and spills;
     // several activation rows always run the form with the pass count as a variable)
 #define PLLM_LAUNCH(I, RR) { \
         auto kern = (passes > 1 || RR > 1) ? fp8_persistent_matvec_kernel<I, F16S, SWIGLU, true, RR> : fp8_persistent_matvec_kernel<I, F16S, SWIGLU, false, 1>; \
