@@ -303,14 +303,15 @@ def test_grouped_experts_matrix_core_path(mod, t13, e, d, inter, topk, t, limit)
     assert torch.equal(y, y2)
 
 
+@pytest.mark.parametrize("d", [512, 1024, 2048, 3072])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
-def test_grouped_experts_routes_as_matrix_rows(mod, dtype):
+def test_grouped_experts_routes_as_matrix_rows(mod, dtype, d):
     """IQ2_XXS / IQ1_M experts at 1.5 routes per expert or more take the half-precision form (routes = rows of the matrix-core
     product): one expert with 21 routes (two batches of 16, three of 8 for float32 activations, which go in as two terms),
     experts without routes, an intermediate size that is not a multiple of 256, every activation dtype, rows scaled far
     away from 1 (the rows are brought into half-precision range by a power of two per token)."""
     rng = np.random.default_rng(77)
-    e, d, inter, t = 6, 512, 400, 24
+    e, inter, t = 6, 400, 24           # d: rows of 2, 4, 8 and 12 super-blocks (the gate/up kernel has a form per divisibility of the row)
     w1 = _expert_blocks(rng, "iq2_xxs", e, inter, d)
     w3 = _expert_blocks(rng, "iq2_xxs", e, inter, d)
     w2 = _expert_blocks(rng, "iq1_m", e, d, inter)
@@ -331,7 +332,7 @@ def test_grouped_experts_routes_as_matrix_rows(mod, dtype):
     grids = (codebooks.get_iq2xxs_signed_grid_tensor().to(DEV), codebooks.get_iq1_grid_tensor().to(DEV))
     dw1, dw3, dw2 = (torch.from_numpy(a).to(DEV) for a in (w1, w3, w2))
     tid = O.TYPE_IDS
-    print(f"case routes as matrix rows {dtype}", flush=True)
+    print(f"case routes as matrix rows {dtype} d={d}", flush=True)
     y = mod.gguf_moe_prefill_grouped_forward(x, toks, rws, seg, dw1, dw3, dw2, d, tid["iq2_xxs"], d, tid["iq2_xxs"], inter, tid["iq1_m"], grids, 0.0)
     torch.cuda.synchronize()
     route_experts = np.repeat(np.arange(e), counts)
