@@ -45,7 +45,9 @@ enum {
     PLLM_TYPE_IQ3_XXS = 6, /* 98 B */
     PLLM_TYPE_IQ4_XS = 7,  /* 136 B */
     PLLM_TYPE_Q6_K = 8,    /* 210 B */
-    PLLM_TYPE_Q8_0 = 100   /* 34 B / 32 weights; the reference gives Q8_0 no id, this one is the library's own */
+    PLLM_TYPE_Q8_0 = 100,  /* 34 B / 32 weights; the reference gives Q8_0 no id, this one is the library's own */
+    PLLM_TYPE_Q3_K = 101   /* 110 B; decoded by the reference's reader only (src/loader/gguf/tensor_reader.py:746-776, no id, no kernel):
+                              pllm_gguf_dequantize_rows takes it, the matmul entry points do not */
 };
 
 const char* pllm_status_string(int status);
@@ -202,7 +204,7 @@ int pllm_gguf_quant_gemm_multi(const void* x, int x_dtype, const float* norm_wei
 /*
  * Selected-row dequantization: out[i, :] = dequant(blocks[row_ids[i], :, :])[:k]  (row_ids == NULL
  * selects rows 0 .. n_selected-1 in order).  type_id may also be PLLM_TYPE_Q8_0 (blocks_per_row then
- * counts 32-weight blocks).  Results are bit-identical to the reference's numpy decoders.
+ * counts 32-weight blocks) or PLLM_TYPE_Q3_K.  Results are bit-identical to the reference's numpy decoders.
  *   row_ids int64 [n_selected] (ids outside [0, n_rows) produce zero rows), out [n_selected, k]
  * Replaces gguf_quant_embedding_forward (src/csrc/cuda_kernel.cpp:669-687, kernel
  * src/csrc/cuda_kernel_impl.cu:8387-8423, which serves q4_k/q5_k only) and stands in for the

@@ -50,8 +50,8 @@ _CODEBOOK_FILE = Path(__file__).resolve().parents[1] / "pocketllm_amd" / "csrc" 
 # type_id map of the reference: src/loader/gguf/quant_types.py:3-13, src/csrc/cuda_kernel.cpp:401-412
 TYPE_IDS = {"iq2_xxs": 0, "q2_k": 1, "iq1_m": 2, "q4_k": 3, "q5_k": 4, "iq2_xs": 5, "iq3_xxs": 6, "iq4_xs": 7, "q6_k": 8}
 TYPE_NAMES = {v: k for k, v in TYPE_IDS.items()}
-BLOCK_BYTES = {"q8_0": 34, "iq2_xxs": 66, "q2_k": 84, "iq1_m": 56, "q4_k": 144, "q5_k": 176, "iq4_xs": 136, "q6_k": 210, "iq2_xs": 74, "iq3_xxs": 98}
-BLOCK_ELEMS = {"q8_0": 32, "iq2_xxs": 256, "q2_k": 256, "iq1_m": 256, "q4_k": 256, "q5_k": 256, "iq4_xs": 256, "q6_k": 256, "iq2_xs": 256, "iq3_xxs": 256}
+BLOCK_BYTES = {"q8_0": 34, "iq2_xxs": 66, "q2_k": 84, "iq1_m": 56, "q4_k": 144, "q5_k": 176, "iq4_xs": 136, "q6_k": 210, "iq2_xs": 74, "iq3_xxs": 98, "q3_k": 110}
+BLOCK_ELEMS = {"q8_0": 32, "iq2_xxs": 256, "q2_k": 256, "iq1_m": 256, "q4_k": 256, "q5_k": 256, "iq4_xs": 256, "q6_k": 256, "iq2_xs": 256, "iq3_xxs": 256, "q3_k": 256}
 
 
 # --------------------------------------------------------------------------------------------
@@ -326,6 +326,29 @@ def dequant_q6_k(blocks: np.ndarray) -> np.ndarray:
     return out
 
 
+def dequant_q3_k(blocks: np.ndarray) -> np.ndarray:
+    """Q3_K as the reference's reader decodes it: hmask(32) qs(64) scales(12) d(f16), sixteen groups of 16 weights.
+    Group g: scale = nibble g of the first eight scale bytes (low nibbles for g < 8, high nibbles of byte g - 8 else) minus 8;
+    weight j of the group: two low bits (qs[4 g + j % 4] >> 2 (j // 4)) & 3, minus 4 when bit j % 8 of hmask[2 g + j // 8] is
+    clear; w = (d * scale) * q in float32.  Reference: tensor_reader.py:746-776 (its own layout: the last four scale bytes
+    are not read).  The reference gives this type no type id and no device kernel; only the decoder exists."""
+    assert blocks.dtype == np.uint8 and blocks.shape[-1] == 110
+    hmask = blocks[..., 0:32]
+    qs = blocks[..., 32:96]
+    scales = blocks[..., 96:108]
+    d = _f16(blocks[..., 108:110])
+    out = np.empty(blocks.shape[:-1] + (256,), dtype=np.float32)
+    j = np.arange(16)
+    for g in range(16):
+        nib = (scales[..., g] & 0x0F) if g < 8 else (scales[..., g - 8] >> 4)
+        scale = (nib.astype(np.int16) - 8).astype(np.float32)
+        low = (qs[..., 4 * g + (j & 3)] >> (2 * (j >> 2)).astype(np.uint8)) & 3
+        bit = (hmask[..., 2 * g + (j >> 3)] >> (j & 7).astype(np.uint8)) & 1
+        q = low.astype(np.int16) - np.where(bit == 0, 4, 0).astype(np.int16)
+        out[..., 16 * g:16 * g + 16] = (d * scale)[..., None] * q.astype(np.float32)
+    return out
+
+
 IQ4_KVALUES = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], dtype=np.float32)
 
 
@@ -350,6 +373,7 @@ def dequant_iq4_xs(blocks: np.ndarray) -> np.ndarray:
 
 
 _DECODERS = {
+    "q3_k": dequant_q3_k,
     "q8_0": dequant_q8_0, "q4_k": dequant_q4_k, "q5_k": dequant_q5_k,
     "q2_k": dequant_q2_k, "iq2_xxs": dequant_iq2_xxs, "iq1_m": dequant_iq1_m,
     "q6_k": dequant_q6_k, "iq4_xs": dequant_iq4_xs, "iq2_xs": dequant_iq2_xs, "iq3_xxs": dequant_iq3_xxs,

@@ -11,6 +11,7 @@ PLLM_ERR_UNSUPPORTED = -2        # include/pllm_hip.h: type id or shape outside 
 PLLM_ERR_WORKSPACE = -4          # the caller's workspace (or the library's static array) is too small
 DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
 TYPE_Q8_0 = 100
+TYPE_Q3_K = 101   # dequantization only (the reference decodes it in numpy and gives it no id)
 
 _c_void_p = ctypes.c_void_p
 _i64 = ctypes.c_int64

@@ -121,6 +121,18 @@ __device__ float dequant_iq4_xs(const uint8_t* b, int e) {
     return f16_at(b) * static_cast<float>(ls) * static_cast<float>(kIq4Values[code]);
 }
 
+// Q3_K as the reference's reader decodes it (src/loader/gguf/tensor_reader.py:746-776): 110 B = hmask(32) qs(64) scales(12) d(2);
+// group g = e / 16: scale = nibble g of the first eight scale bytes - 8; two low bits from qs[4 g + j % 4] at 2 (j / 4), minus 4
+// when bit j % 8 of hmask[2 g + j / 8] is clear; (d * scale) * q.
+__device__ float dequant_q3_k(const uint8_t* b, int e) {
+    const int g = e >> 4, j = e & 15;
+    const int nib = g < 8 ? (b[96 + g] & 15) : (b[96 + g - 8] >> 4);
+    const int low = (b[32 + 4 * g + (j & 3)] >> (2 * (j >> 2))) & 3;
+    const int bit = (b[2 * g + (j >> 3)] >> (j & 7)) & 1;
+    const float ds = f16_at(b + 108) * static_cast<float>(nib - 8);
+    return ds * static_cast<float>(low - (bit ? 0 : 4));
+}
+
 // grid (selected rows, ceil(k / 256)), 256 threads
 __global__ __launch_bounds__(256) void dequant_rows_kernel(
     const int64_t* __restrict__ row_ids, const uint8_t* __restrict__ blocks, int type_id, void* __restrict__ out, int out_dtype,
@@ -145,6 +157,7 @@ __global__ __launch_bounds__(256) void dequant_rows_kernel(
                 case PLLM_TYPE_IQ2_XS: v = dequant_iq2_xs(b, e); break;
                 case PLLM_TYPE_IQ3_XXS: v = dequant_iq3_xxs(b, e); break;
                 case PLLM_TYPE_IQ4_XS: v = dequant_iq4_xs(b, e); break;
+                case PLLM_TYPE_Q3_K: v = dequant_q3_k(b, e); break;
                 default: v = dequant_iq1_m(b, e); break;
             }
         }
@@ -180,14 +193,15 @@ int pllm_gguf_dequantize_rows(const int64_t* row_ids, int64_t n_selected, const 
     if (!blocks || !out || n_selected < 0 || n_rows <= 0 || k <= 0 || blocks_per_row <= 0) return PLLM_ERR_INVALID_ARGUMENT;
     if (out_dtype != PLLM_F32 && out_dtype != PLLM_F16 && out_dtype != PLLM_BF16) return PLLM_ERR_INVALID_ARGUMENT;
     const bool q8 = type_id == PLLM_TYPE_Q8_0;
-    if (!q8 && pllm_gguf_block_bytes(type_id) == 0) return PLLM_ERR_UNSUPPORTED;
+    const int block_bytes = type_id == PLLM_TYPE_Q3_K ? 110 : pllm_gguf_block_bytes(type_id);   // (Q3_K: this entry point only)
+    if (!q8 && block_bytes == 0) return PLLM_ERR_UNSUPPORTED;
     if (blocks_per_row * (q8 ? 32 : 256) < k) return PLLM_ERR_INVALID_ARGUMENT;
     if (n_selected == 0) return PLLM_OK;
     if (n_selected > 0x7fffffffLL || (k + 255) / 256 > 65535 || k > 0x7fffffffLL) return PLLM_ERR_UNSUPPORTED;
     dim3 grid(static_cast<unsigned>(n_selected), static_cast<unsigned>((k + 255) / 256));
     hipLaunchKernelGGL(pllm::dequant_rows_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream), row_ids, blocks,
                        q8 ? -1 : type_id, out, out_dtype, static_cast<int>(k), static_cast<int>(blocks_per_row),
-                       q8 ? 34 : pllm_gguf_block_bytes(type_id), n_rows);
+                       q8 ? 34 : block_bytes, n_rows);
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 

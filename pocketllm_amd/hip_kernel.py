@@ -323,18 +323,18 @@ def gguf_q2k_gemm_dp4a_forward(x, blocks, row_elems, *, out_dtype: torch.dtype =
 
 def gguf_dequantize_rows(blocks: torch.Tensor, type_id: int, row_elems: int, row_ids: torch.Tensor | None = None, *,
                          out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
-    """Dequantize whole or selected rows of a raw-block matrix (type_id _ffi.TYPE_Q8_0 for Q8_0 blocks).
+    """Dequantize whole or selected rows of a raw-block matrix (type_id _ffi.TYPE_Q8_0 for Q8_0 blocks, _ffi.TYPE_Q3_K for Q3_K).
 
     No direct counterpart in the reference extension: it is the device form of the numpy decoders of
     src/loader/gguf/tensor_reader.py:543-1009, with bit-identical float32 results.
     """
     type_id, row_elems = int(type_id), int(row_elems)
-    q8 = type_id == _ffi.TYPE_Q8_0
-    if not q8:
+    q8, q3 = type_id == _ffi.TYPE_Q8_0, type_id == _ffi.TYPE_Q3_K
+    if not (q8 or q3):
         _check_type(type_id)
     _check(blocks.dim() == 3 and blocks.is_cuda and blocks.dtype == torch.uint8 and blocks.is_contiguous(),
            "blocks must be a contiguous CUDA uint8 tensor [N, K_blocks, block_bytes]")
-    _check(blocks.size(2) == (34 if q8 else GGUF_BLOCK_BYTES[type_id]), "unexpected GGUF block size for type_id")
+    _check(blocks.size(2) == (34 if q8 else 110 if q3 else GGUF_BLOCK_BYTES[type_id]), "unexpected GGUF block size for type_id")
     _check(row_elems > 0 and blocks.size(1) * (32 if q8 else 256) >= row_elems, "blocks do not cover row_elems")
     if row_ids is not None:
         _check(row_ids.is_cuda and row_ids.dtype == torch.int64 and row_ids.is_contiguous(), "row_ids must be contiguous CUDA int64")

@@ -5,7 +5,7 @@ Run ONLY in the build container, where the reference checkout is mounted:
     python tests/golden/make_reference_fixtures.py /root/reference
 
 It imports the reference's GGUF reader from that checkout, feeds it seeded random blocks of the types
-that no reference-held vector and no compiled reference kernel pins (Q8_0, Q4_K, Q5_K, Q6_K, IQ4_XS, IQ2_XS, IQ3_XXS, and
+that no reference-held vector and no compiled reference kernel pins (Q8_0, Q4_K, Q5_K, Q6_K, IQ4_XS, IQ2_XS, IQ3_XXS, Q3_K, and
 IQ2_XXS, whose compiled CPU kernel takes the sign-expanded grid from its caller) through a one-tensor GGUF file
 in a temporary directory, and stores {blocks, values} as hex in JSON files next to this script, plus
 SHA-256 digests of the two codebook arrays the reference builds (sign-expanded IQ2_XXS grid, IQ1 grid).  The fixtures are data; the reference itself never leaves the container.
@@ -21,9 +21,9 @@ from pathlib import Path
 import numpy as np
 
 HERE = Path(__file__).resolve().parent
-GGML_TYPE = {"q8_0": 8, "q4_k": 12, "q5_k": 13, "iq2_xxs": 16, "q6_k": 14, "iq4_xs": 23, "iq2_xs": 17, "iq3_xxs": 18}
-GEOM = {"q8_0": (32, 34), "q4_k": (256, 144), "q5_k": (256, 176), "iq2_xxs": (256, 66), "q6_k": (256, 210), "iq4_xs": (256, 136), "iq2_xs": (256, 74), "iq3_xxs": (256, 98)}
-F16_FIELDS = {"q8_0": [0], "q4_k": [0, 2], "q5_k": [0, 2], "iq2_xxs": [0], "q6_k": [208], "iq4_xs": [0], "iq2_xs": [0], "iq3_xxs": [0]}
+GGML_TYPE = {"q8_0": 8, "q4_k": 12, "q5_k": 13, "iq2_xxs": 16, "q6_k": 14, "iq4_xs": 23, "iq2_xs": 17, "iq3_xxs": 18, "q3_k": 11}
+GEOM = {"q8_0": (32, 34), "q4_k": (256, 144), "q5_k": (256, 176), "iq2_xxs": (256, 66), "q6_k": (256, 210), "iq4_xs": (256, 136), "iq2_xs": (256, 74), "iq3_xxs": (256, 98), "q3_k": (256, 110)}
+F16_FIELDS = {"q8_0": [0], "q4_k": [0, 2], "q5_k": [0, 2], "iq2_xxs": [0], "q6_k": [208], "iq4_xs": [0], "iq2_xs": [0], "iq3_xxs": [0], "q3_k": [108]}
 ROWS, BLOCKS_PER_ROW = 3, 2
 
 
@@ -67,7 +67,7 @@ def main() -> None:
 
     rng = np.random.default_rng(20240607)
     with tempfile.TemporaryDirectory() as tmp:
-        for type_name in ("q8_0", "q4_k", "q5_k", "iq2_xxs", "q6_k", "iq4_xs", "iq2_xs", "iq3_xxs"):      # new types go last: the stream of random blocks of the earlier ones stays the same
+        for type_name in ("q8_0", "q4_k", "q5_k", "iq2_xxs", "q6_k", "iq4_xs", "iq2_xs", "iq3_xxs", "q3_k"):      # new types go last: the stream of random blocks of the earlier ones stays the same
             elems, nbytes = GEOM[type_name]
             blocks = random_blocks(rng, type_name)
             path = Path(tmp) / f"{type_name}.gguf"

@@ -25,17 +25,17 @@ def _random_blocks(rng, type_name, n, bpr):
     if type_name == "iq1_m":
         return C.random_iq1_m(rng, n, bpr, d_range=(0.001, 0.08))
     blocks = rng.integers(0, 256, size=(n, bpr, bb), dtype=np.uint8)
-    for off in {"q8_0": [0], "q4_k": [0, 2], "q5_k": [0, 2], "q2_k": [80, 82], "iq2_xxs": [0], "q6_k": [208], "iq4_xs": [0], "iq2_xs": [0], "iq3_xxs": [0]}[type_name]:
+    for off in {"q8_0": [0], "q4_k": [0, 2], "q5_k": [0, 2], "q2_k": [80, 82], "iq2_xxs": [0], "q6_k": [208], "iq4_xs": [0], "iq2_xs": [0], "iq3_xxs": [0], "q3_k": [108]}[type_name]:
         vals = rng.uniform(0.001, 0.05, size=(n, bpr)) * rng.choice([-1.0, 1.0], size=(n, bpr))
         blocks[..., off:off + 2] = vals.astype("<f2").view(np.uint8).reshape(n, bpr, 2)
     return blocks
 
 
 def _tid(type_name):
-    return _ffi.TYPE_Q8_0 if type_name == "q8_0" else O.TYPE_IDS[type_name]
+    return {"q8_0": _ffi.TYPE_Q8_0, "q3_k": _ffi.TYPE_Q3_K}.get(type_name) or O.TYPE_IDS[type_name]
 
 
-@pytest.mark.parametrize("type_name", ["q8_0", "q4_k", "q5_k", "q2_k", "iq2_xxs", "iq1_m", "q6_k", "iq4_xs", "iq2_xs", "iq3_xxs"])
+@pytest.mark.parametrize("type_name", ["q8_0", "q4_k", "q5_k", "q2_k", "iq2_xxs", "iq1_m", "q6_k", "iq4_xs", "iq2_xs", "iq3_xxs", "q3_k"])
 def test_dequant_is_bit_exact_on_random_bytes(mod, type_name):
     rng = np.random.default_rng(31)
     n, bpr = 37, (24 if type_name == "q8_0" else 3)
@@ -54,7 +54,8 @@ def test_dequant_is_bit_exact_on_random_bytes(mod, type_name):
 
 @pytest.mark.parametrize("name", ["iq1m_oracle.json", "q8_0_reference_decode.json", "q4_k_reference_decode.json",
                                   "q5_k_reference_decode.json", "iq2_xxs_reference_decode.json", "q6_k_reference_decode.json",
-                                  "iq4_xs_reference_decode.json", "iq2_xs_reference_decode.json", "iq3_xxs_reference_decode.json"])
+                                  "iq4_xs_reference_decode.json", "iq2_xs_reference_decode.json", "iq3_xxs_reference_decode.json",
+                                  "q3_k_reference_decode.json"])
 def test_dequant_matches_golden_vectors(mod, golden_dir, name):
     raw = json.loads((golden_dir / name).read_text())
     blocks = np.frombuffer(bytes.fromhex(raw["blocks_u8"]), dtype=np.uint8)

@@ -34,7 +34,7 @@ def test_iq1m_matches_reference_held_vector(golden_dir):
     np.testing.assert_array_equal(got, values.reshape(raw["n_blocks"], 256))
 
 
-@pytest.mark.parametrize("type_name", ["q8_0", "q4_k", "q5_k", "iq2_xxs", "q6_k", "iq4_xs", "iq2_xs", "iq3_xxs"])
+@pytest.mark.parametrize("type_name", ["q8_0", "q4_k", "q5_k", "iq2_xxs", "q6_k", "iq4_xs", "iq2_xs", "iq3_xxs", "q3_k"])
 def test_decoders_match_reference_decoder_vectors(golden_dir, type_name):
     raw, blocks, values = _load(golden_dir, f"{type_name}_reference_decode.json")
     blocks = blocks.reshape(raw["rows"], raw["blocks_per_row"], raw["block_bytes"])
