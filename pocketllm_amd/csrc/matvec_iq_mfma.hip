@@ -33,10 +33,11 @@ __global__ __launch_bounds__(64 * kWaves) void mfma_tile_matvec_kernel(
     const StagedX sx = carve_staged_x(smem, kpad);
     const int zero_off = image_bytes;                                        // 16 zero bytes
     unsigned char* tables = smem + image_bytes + 16;
-    if (route.expert) w += static_cast<size_t>(route.expert[blockIdx.y]) * route.expert_stride;
-    if (blockIdx.z) {                        // several projections in one launch: this one's matrix, row count and output
+    const size_t woff = route_offset(route, blockIdx.y);
+    w += woff;
+    if (blockIdx.z) {                        // several projections in one launch: this one's matrix (of the same expert), row count and output
         const int m = blockIdx.z - 1;
-        w = route.more_w[m];
+        w = route.more_w[m] + woff;
         y = route.more_y[m];
         n = route.more_n[m];
     }
@@ -60,7 +61,7 @@ __global__ __launch_bounds__(64 * kWaves) void mfma_tile_matvec_kernel(
     float acc = 0.0f;
     bool staged = false;
     if constexpr (RAW)                       // raw activation row: quantized here, before the loads take their registers
-        quantize_row_to_lds(smem, act.x, act.x_dtype, static_cast<size_t>(blockIdx.y) * act.k, act.k, kpad, RowNorm{act.gamma, act.eps, act.round_f16});
+        quantize_row_to_lds(smem, act.x, act.x_dtype, raw_row_of(act, blockIdx.y) * act.k, act.k, kpad, RowNorm{act.gamma, act.eps, act.round_f16});
     for (int b0 = wave; b0 < bpr || !staged; b0 += waves * ITERS) {
         typename FMT::Regs regs[ITERS];
 #pragma unroll
@@ -309,7 +310,7 @@ int launch_fmt(const ActRows& act, const WeightRoute& route, const uint8_t* w, v
     // where shape and alignment allow, else one short workgroup per tile; routed calls and several projections in one launch
     // always take the latter
     if constexpr (FMT::kStreamed)
-        if (!route.expert && !act.row_token && route.extra == 0)
+        if (!routed(route) && !act.row_token && !act.x_broadcast && route.extra == 0)
             if (const int split = stream_split<FMT>(w, n, bpr)) return launch_stream<FMT>(act, w, y, y_dtype, rows, n, bpr, split, stream);
     return launch_tiles<FMT>(act, route, w, y, y_dtype, rows, n, bpr, stream);
 }

@@ -194,10 +194,11 @@ __global__ __launch_bounds__(64 * kMaxWaves) void k45_mfma_matvec_kernel(
     const int lane = tid & 63;
     const int col = lane & 15;        // B/C column = output row within the tile; also A's row index m
     const int ks = lane >> 4;         // k slice of A and B, row quad of C
-    if (route.expert) w += static_cast<size_t>(route.expert[blockIdx.y]) * route.expert_stride;
-    if (blockIdx.z) {                        // several projections in one launch: this one's matrix, row count and output
+    const size_t woff = route_offset(route, blockIdx.y);
+    w += woff;
+    if (blockIdx.z) {                        // several projections in one launch: this one's matrix (of the same expert), row count and output
         const int m = blockIdx.z - 1;
-        w = route.more_w[m];
+        w = route.more_w[m] + woff;
         y = route.more_y[m];
         n = route.more_n[m];
     }
@@ -225,7 +226,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void k45_mfma_matvec_kernel(
     if constexpr (RAW) {                     // quantize before the loads take their registers
 #pragma unroll 1
         for (int r = 0; r < R; ++r)          // rows past the end: the last row again, result dropped
-            quantize_row_to_lds(smem + r * image_bytes, act.x, act.x_dtype, static_cast<size_t>(min(row0 + r, total_rows - 1)) * act.k, act.k, kpad,
+            quantize_row_to_lds(smem + r * image_bytes, act.x, act.x_dtype, raw_row_of(act, min(row0 + r, total_rows - 1)) * act.k, act.k, kpad,
                                 RowNorm{act.gamma, act.eps, act.round_f16});
         if (tid < 4) reinterpret_cast<uint32_t*>(smem + zero_off)[tid] = 0;
         __syncthreads();
@@ -773,7 +774,7 @@ int launch_q2k_kernel(KERN kern, const ActRows& act, const WeightRoute& route, c
 template <typename FMT, int R>
 int launch_k45_rows(const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream) {
     if constexpr (R == 1)
-        if (act.x && act.k >= 4 && !route.expert && !act.row_token) {
+        if (act.x && act.k >= 4 && !routed(route) && !act.row_token && !act.x_broadcast) {
             if (!act.gamma) return launch_wave<FMT, false>(act, route, w, y, y_dtype, rows, n, bpr, stream);
             const int st = launch_wave<FMT, true>(act, route, w, y, y_dtype, rows, n, bpr, stream);
             if (st != PLLM_ERR_UNSUPPORTED) return st;                       // (rows too long for it: the workgroup-wide quantizer below)
@@ -800,7 +801,7 @@ int launch_k45_rows(const ActRows& act, const WeightRoute& route, const uint8_t*
 template <typename FMT>
 int launch_k45(const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream) {
     const size_t image = staged_x_bytes(bpr * 256);
-    const bool plain = !route.expert && !act.row_token && !act.x;
+    const bool plain = !routed(route) && !act.row_token && !act.x;
     if (plain && rows >= 3 && 4 * image <= 52 * 1024) return launch_k45_rows<FMT, 4>(act, route, w, y, y_dtype, rows, n, bpr, stream);
     if (plain && rows >= 2 && 2 * image <= 52 * 1024) return launch_k45_rows<FMT, 2>(act, route, w, y, y_dtype, rows, n, bpr, stream);
     return launch_k45_rows<FMT, 1>(act, route, w, y, y_dtype, rows, n, bpr, stream);
@@ -809,7 +810,7 @@ int launch_k45(const ActRows& act, const WeightRoute& route, const uint8_t* w, v
 template <typename FMT>
 int launch_groups16(const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream) {
     // raw rows without normalisation or routing, blocks on the format's boundary; everything else stays with the other kernels
-    if (!act.x || act.k < 4 || act.gamma || route.expert || act.row_token || (reinterpret_cast<uintptr_t>(w) & (FMT::kAlign - 1))) return PLLM_ERR_UNSUPPORTED;
+    if (!act.x || act.k < 4 || act.gamma || routed(route) || act.row_token || act.x_broadcast || (reinterpret_cast<uintptr_t>(w) & (FMT::kAlign - 1))) return PLLM_ERR_UNSUPPORTED;
     for (int m = 0; m < route.extra; ++m)
         if (reinterpret_cast<uintptr_t>(route.more_w[m]) & (FMT::kAlign - 1)) return PLLM_ERR_UNSUPPORTED;
     int waves, iters;
@@ -843,7 +844,7 @@ int kquant_matvec_from_image(const ActRows& act, const uint8_t* w, int type_id, 
 
 int iq4xs_wave_matvec(const ActRows& act, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream, WeightRoute route) {
     // raw rows without routing, blocks on an 8-byte boundary; everything else stays with the tile-frame kernel
-    if (!act.x || act.k < 4 || route.expert || act.row_token || (reinterpret_cast<uintptr_t>(w) & 7u)) return PLLM_ERR_UNSUPPORTED;
+    if (!act.x || act.k < 4 || routed(route) || act.row_token || act.x_broadcast || (reinterpret_cast<uintptr_t>(w) & 7u)) return PLLM_ERR_UNSUPPORTED;
     for (int m = 0; m < route.extra; ++m)
         if (reinterpret_cast<uintptr_t>(route.more_w[m]) & 7u) return PLLM_ERR_UNSUPPORTED;
     return act.gamma ? launch_wave<IQ4XS, true>(act, route, w, y, y_dtype, rows, n, bpr, stream)

@@ -40,10 +40,11 @@ struct ActRows {
     const void* x;
     int x_dtype;
     int k;
-    const int64_t* row_token;     // routed calls: grid row r reads image row_token[r] (null: image r)
+    const int64_t* row_token;     // routed calls: grid row r reads image (or raw row) row_token[r] (null: row r)
     const float* gamma;           // raw rows only: RMS normalisation ahead of the quantization (null: none)
     float eps;
     int round_f16;
+    int x_broadcast;              // raw rows, routed calls on one token: every grid row reads row 0
 };
 // Routed calls: grid row r multiplies with the matrix at w + expert[r] * expert_stride (null: one matrix for every row).
 struct WeightRoute {
@@ -55,7 +56,21 @@ struct WeightRoute {
     void* more_y[3];
     int more_n[3];
     int extra;
+    const int64_t* expert64;      // the expert numbers as int64 (the form the single-token operators receive them in) instead of `expert`
 };
+inline bool routed(const WeightRoute& r) { return r.expert != nullptr || r.expert64 != nullptr; }
+#ifdef __HIPCC__
+// byte offset of grid row `row`'s matrix
+__device__ __forceinline__ size_t route_offset(const WeightRoute& r, int row) {
+    if (r.expert) return static_cast<size_t>(r.expert[row]) * r.expert_stride;
+    if (r.expert64) return static_cast<size_t>(r.expert64[row]) * r.expert_stride;
+    return 0;
+}
+// the activation row (raw rows) that grid row `row` reads
+__device__ __forceinline__ size_t raw_row_of(const ActRows& a, int row) {
+    return a.x_broadcast ? 0 : (a.row_token ? static_cast<size_t>(a.row_token[row]) : static_cast<size_t>(row));
+}
+#endif
 inline ActRows act_rows_from_image(const unsigned char* image, size_t stride, const int64_t* row_token = nullptr) {
     return ActRows{image, stride, nullptr, 0, 0, row_token, nullptr, 0.0f, 0};
 }
