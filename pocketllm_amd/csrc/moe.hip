@@ -19,6 +19,7 @@
 namespace pllm {
 // from this many tokens on, an expert's routes are multiplied as one tile matmul on the matrix cores
 constexpr int kMoeGemmMinTokens = 16;
+constexpr int kMoeTileMinRoutesPerExpert = 3;   // (128 experts top-8, 2048 -> 768, Q4_K: 79 / 146 / 202 / 259 us route by route at 16 / 32 / 48 / 64 tokens against 190 / 211 / 216 / 220 us as tile matmuls)
 // up to this many routes per expert on average the grouped matrix-core kernels (cost per route: MFMAs and a short
 // epilogue after one decode per expert; measured ~180 us + 0.5 us per route at 256 experts of 1536 x 3072) run ahead
 // of the tile matmuls (cost per expert: the fp16 decode of every weight, ~1450 us for the same experts)
@@ -611,7 +612,10 @@ int pllm_gguf_moe_forward(const void* x, int x_dtype, int64_t tokens, int64_t di
         if (st != PLLM_OK) return st;
         return launch_moe_reduce(part, route_tokens, y, tokens, R, D, s);
     }
-    if (seg_starts && tokens >= kMoeGemmMinTokens) {
+    // (types without fused expert kernels: the tile path decodes every touched expert's three matrices whatever its route count, so
+    // below kMoeTileMinRoutesPerExpert routes per expert on average the route-by-route path below stays cheaper)
+    const bool few_routes_each = (!dot4_type(w13_type) || !dot4_type(w2_type)) && routes < static_cast<int64_t>(kMoeTileMinRoutesPerExpert) * n_experts;
+    if (seg_starts && tokens >= kMoeGemmMinTokens && !few_routes_each) {
         // tile path: gather the routes' activation rows as fp16, gate and up as two batches of tile
         // matmuls (one group per expert), SwiGLU into fp16 hidden rows, down as a third batch, then
         // the ordered sum of every token's routes

@@ -492,6 +492,30 @@ def test_experts_in_every_block_type(mod, t13, t2, tokens):
         assert O.rel_l2(y.cpu().numpy(), want) <= TOL, (t13, t2, tokens, limit)
 
 
+@pytest.mark.parametrize("t13,t2", [("q4_k", "q6_k"), ("iq4_xs", "q5_k")])
+def test_experts_with_few_routes_each_at_sixteen_tokens_or_more(mod, t13, t2):
+    """Types without fused expert kernels, 16 tokens or more but under three routes per expert on average: the route-by-route path
+    (the tile matmuls would decode every touched expert for one or two rows)."""
+    rng = np.random.default_rng(812)
+    e, d, inter, topk, tokens = 40, 512, 512, 2, 24
+    w1 = _any_expert_blocks(rng, t13, e, inter, d)
+    w3 = _any_expert_blocks(rng, t13, e, inter, d)
+    w2 = _any_expert_blocks(rng, t2, e, d, inter)
+    idx, wts = _route(rng, tokens, e, topk)
+    assert tokens * topk < 3 * e
+    x = torch.from_numpy(rng.standard_normal((tokens, d)).astype(np.float32)).to(DEV).to(torch.bfloat16)
+    dw1, dw3, dw2 = (torch.from_numpy(a).to(DEV) for a in (w1, w3, w2))
+    tid = O.TYPE_IDS
+    _, toks, rws, seg = mod.moe_group_routes(torch.from_numpy(idx).to(DEV), torch.from_numpy(wts).to(DEV), 0, e)
+    print(f"case experts few routes each {t13}/{t2}", flush=True)
+    y = mod.gguf_moe_prefill_grouped_forward(x, toks, rws, seg, dw1, dw3, dw2, d, tid[t13], d, tid[t13], inter, tid[t2],
+                                             torch.empty(0, dtype=torch.int8, device=DEV), 0.0)
+    torch.cuda.synchronize()
+    _, o_toks, o_rws, o_seg = O.group_routes(idx, wts, 0, e)
+    want = O.moe_forward(x.float().cpu().numpy(), o_toks, o_rws, np.repeat(np.arange(e), np.diff(o_seg)), w1, w3, w2, t13, t13, t2, 0.0)
+    assert O.rel_l2(y.cpu().numpy(), want) <= TOL
+
+
 def test_expert_grid_families_are_checked(mod):
     e, d, inter = 2, 256, 256
     x = torch.randn(2, d, device=DEV)
