@@ -356,7 +356,7 @@ __device__ __forceinline__ void raw_to_float4(const RawX<X16>& r, int x_dtype, f
 template <typename FMT, int ITERS, int DEPTH, bool X16, bool NORM>
 __global__ __launch_bounds__(64 * kMaxWaves) void wave_image_matvec_kernel(
     const void* __restrict__ x, int x_dtype, int k, const WeightRoute route, const uint8_t* __restrict__ w, void* __restrict__ y,
-    int y_dtype, int n, int bpr, const float* __restrict__ gamma, float eps, int round_f16) {
+    int y_dtype, int n, int bpr, const float* __restrict__ gamma, float eps, int round_f16, const int64_t* __restrict__ row_token, int x_broadcast) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int tid = threadIdx.x;
     const int waves = blockDim.x >> 6;
@@ -367,16 +367,18 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_image_matvec_kernel(
     constexpr int kWaveBytes = kSlotBytes + 16;                               // the wave's slot, then its 16 zero bytes
     unsigned char* slot = smem + wave * kWaveBytes;
     float* partial = reinterpret_cast<float*>(smem + waves * kWaveBytes);    // [waves][16]
+    const size_t woff = route_offset(route, blockIdx.y);                      // routed calls: the grid row's expert
+    w += woff;
     if (blockIdx.z) {                        // several projections in one launch: this one's matrix, row count and output
         const int m = blockIdx.z - 1;
-        w = route.more_w[m];
+        w = route.more_w[m] + woff;
         y = route.more_y[m];
         n = route.more_n[m];
     }
     if (static_cast<int>(blockIdx.x) * kRowsPerWg >= n) return;             // the grid covers the tallest matrix
     const int row = blockIdx.x * kRowsPerWg + col;
     const uint8_t* wrow = w + static_cast<size_t>(row < n ? row : 0) * bpr * FMT::kBlockBytes;
-    const size_t xoff = static_cast<size_t>(blockIdx.y) * k;
+    const size_t xoff = (x_broadcast ? 0 : row_token ? static_cast<size_t>(row_token[blockIdx.y]) : static_cast<size_t>(blockIdx.y)) * k;
 
     if (lane < 4) reinterpret_cast<uint32_t*>(slot + kSlotBytes)[lane] = 0;
     float acc = 0.0f;
@@ -525,7 +527,7 @@ int launch_wave_kernel(KERN kern, const ActRows& act, const WeightRoute& route, 
     for (int m = 0; m < route.extra; ++m) tallest = tallest > route.more_n[m] ? tallest : route.more_n[m];
     dim3 grid((tallest + kRowsPerWg - 1) / kRowsPerWg, rows, 1 + route.extra);
     hipLaunchKernelGGL(kern, grid, dim3(64 * waves), smem, stream, act.x, act.x_dtype, act.k, route, w, y, y_dtype, n, bpr, act.gamma, act.eps,
-                       act.round_f16);
+                       act.round_f16, act.row_token, act.x_broadcast);
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 
@@ -658,7 +660,7 @@ struct WaveQ6K {
 template <typename FMT, int ITERS, int DEPTH, bool X16>
 __global__ __launch_bounds__(64 * kMaxWaves) void wave_groups16_matvec_kernel(
     const void* __restrict__ x, int x_dtype, int k, const WeightRoute route, const uint8_t* __restrict__ w, void* __restrict__ y,
-    int y_dtype, int n, int bpr) {
+    int y_dtype, int n, int bpr, const int64_t* __restrict__ row_token, int x_broadcast) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int tid = threadIdx.x;
     const int waves = blockDim.x >> 6;
@@ -669,16 +671,18 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_groups16_matvec_kernel(
     constexpr int kWaveBytes = kQ2SlotBytes + 16;                            // the wave's slot, then its 16 zero bytes
     unsigned char* slot = smem + wave * kWaveBytes;
     float* partial = reinterpret_cast<float*>(smem + waves * kWaveBytes);    // [waves][16]
+    const size_t woff = route_offset(route, blockIdx.y);                      // routed calls: the grid row's expert
+    w += woff;
     if (blockIdx.z) {                        // several projections in one launch: this one's matrix, row count and output
         const int m = blockIdx.z - 1;
-        w = route.more_w[m];
+        w = route.more_w[m] + woff;
         y = route.more_y[m];
         n = route.more_n[m];
     }
     if (static_cast<int>(blockIdx.x) * kRowsPerWg >= n) return;
     const int row = blockIdx.x * kRowsPerWg + col;
     const uint8_t* wrow = w + static_cast<size_t>(row < n ? row : 0) * bpr * FMT::kBlockBytes;
-    const size_t xoff = static_cast<size_t>(blockIdx.y) * k;
+    const size_t xoff = (x_broadcast ? 0 : row_token ? static_cast<size_t>(row_token[blockIdx.y]) : static_cast<size_t>(blockIdx.y)) * k;
     // the lane's A operand: group `col` of the block, in the one MFMA whose slice ks carries that group
     const bool mine = FMT::slice_of(col) == ks;
     const int my_t = FMT::mfma_of(col);
@@ -767,14 +771,14 @@ int launch_q2k_kernel(KERN kern, const ActRows& act, const WeightRoute& route, c
     int tallest = n;
     for (int m = 0; m < route.extra; ++m) tallest = tallest > route.more_n[m] ? tallest : route.more_n[m];
     dim3 grid((tallest + kRowsPerWg - 1) / kRowsPerWg, rows, 1 + route.extra);
-    hipLaunchKernelGGL(kern, grid, dim3(64 * waves), smem, stream, act.x, act.x_dtype, act.k, route, w, y, y_dtype, n, bpr);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * waves), smem, stream, act.x, act.x_dtype, act.k, route, w, y, y_dtype, n, bpr, act.row_token, act.x_broadcast);
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 
 template <typename FMT, int R>
 int launch_k45_rows(const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream) {
     if constexpr (R == 1)
-        if (act.x && act.k >= 4 && !routed(route) && !act.row_token && !act.x_broadcast) {
+        if (act.x && act.k >= 4 && (!act.gamma || (!routed(route) && !act.row_token && !act.x_broadcast))) {
             if (!act.gamma) return launch_wave<FMT, false>(act, route, w, y, y_dtype, rows, n, bpr, stream);
             const int st = launch_wave<FMT, true>(act, route, w, y, y_dtype, rows, n, bpr, stream);
             if (st != PLLM_ERR_UNSUPPORTED) return st;                       // (rows too long for it: the workgroup-wide quantizer below)
@@ -809,8 +813,8 @@ int launch_k45(const ActRows& act, const WeightRoute& route, const uint8_t* w, v
 
 template <typename FMT>
 int launch_groups16(const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream) {
-    // raw rows without normalisation or routing, blocks on the format's boundary; everything else stays with the other kernels
-    if (!act.x || act.k < 4 || act.gamma || routed(route) || act.row_token || act.x_broadcast || (reinterpret_cast<uintptr_t>(w) & (FMT::kAlign - 1))) return PLLM_ERR_UNSUPPORTED;
+    // raw rows without normalisation, blocks (of every expert) on the format's boundary; everything else stays with the other kernels
+    if (!act.x || act.k < 4 || act.gamma || ((reinterpret_cast<uintptr_t>(w) | route.expert_stride) & (FMT::kAlign - 1))) return PLLM_ERR_UNSUPPORTED;
     for (int m = 0; m < route.extra; ++m)
         if (reinterpret_cast<uintptr_t>(route.more_w[m]) & (FMT::kAlign - 1)) return PLLM_ERR_UNSUPPORTED;
     int waves, iters;
@@ -843,8 +847,9 @@ int kquant_matvec_from_image(const ActRows& act, const uint8_t* w, int type_id, 
 }
 
 int iq4xs_wave_matvec(const ActRows& act, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream, WeightRoute route) {
-    // raw rows without routing, blocks on an 8-byte boundary; everything else stays with the tile-frame kernel
-    if (!act.x || act.k < 4 || routed(route) || act.row_token || act.x_broadcast || (reinterpret_cast<uintptr_t>(w) & 7u)) return PLLM_ERR_UNSUPPORTED;
+    // raw rows, blocks (of every expert) on an 8-byte boundary, no normalisation in routed calls; everything else stays with the tile-frame kernel
+    if (!act.x || act.k < 4 || ((reinterpret_cast<uintptr_t>(w) | route.expert_stride) & 7u)) return PLLM_ERR_UNSUPPORTED;
+    if (act.gamma && (routed(route) || act.row_token || act.x_broadcast)) return PLLM_ERR_UNSUPPORTED;
     for (int m = 0; m < route.extra; ++m)
         if (reinterpret_cast<uintptr_t>(route.more_w[m]) & 7u) return PLLM_ERR_UNSUPPORTED;
     return act.gamma ? launch_wave<IQ4XS, true>(act, route, w, y, y_dtype, rows, n, bpr, stream)

@@ -19,7 +19,7 @@
 namespace pllm {
 // from this many tokens on, an expert's routes are multiplied as one tile matmul on the matrix cores
 constexpr int kMoeGemmMinTokens = 16;
-constexpr int kMoeTileMinRoutesPerExpert = 3;   // (128 experts top-8, 2048 -> 768, Q4_K: 79 / 146 / 202 / 259 us route by route at 16 / 32 / 48 / 64 tokens against 190 / 211 / 216 / 220 us as tile matmuls)
+constexpr int kMoeTileMinRoutesPerExpert = 4;   // (128 experts top-8, 2048 -> 768, Q4_K: 66 / 117 us route by route at 16 / 32 tokens, ~175 / ~230 at 48 / 64, against 190 / 211 / 216 / 220 us as tile matmuls)
 // up to this many routes per expert on average the grouped matrix-core kernels (cost per route: MFMAs and a short
 // epilogue after one decode per expert; measured ~180 us + 0.5 us per route at 256 experts of 1536 x 3072) run ahead
 // of the tile matmuls (cost per expert: the fp16 decode of every weight, ~1450 us for the same experts)

@@ -494,7 +494,7 @@ def test_experts_in_every_block_type(mod, t13, t2, tokens):
 
 @pytest.mark.parametrize("t13,t2", [("q4_k", "q6_k"), ("iq4_xs", "q5_k")])
 def test_experts_with_few_routes_each_at_sixteen_tokens_or_more(mod, t13, t2):
-    """Types without fused expert kernels, 16 tokens or more but under three routes per expert on average: the route-by-route path
+    """Types without fused expert kernels, 16 tokens or more but under four routes per expert on average: the route-by-route path
     (the tile matmuls would decode every touched expert for one or two rows)."""
     rng = np.random.default_rng(812)
     e, d, inter, topk, tokens = 40, 512, 512, 2, 24
@@ -502,7 +502,7 @@ def test_experts_with_few_routes_each_at_sixteen_tokens_or_more(mod, t13, t2):
     w3 = _any_expert_blocks(rng, t13, e, inter, d)
     w2 = _any_expert_blocks(rng, t2, e, d, inter)
     idx, wts = _route(rng, tokens, e, topk)
-    assert tokens * topk < 3 * e
+    assert tokens * topk < 4 * e
     x = torch.from_numpy(rng.standard_normal((tokens, d)).astype(np.float32)).to(DEV).to(torch.bfloat16)
     dw1, dw3, dw2 = (torch.from_numpy(a).to(DEV) for a in (w1, w3, w2))
     tid = O.TYPE_IDS
