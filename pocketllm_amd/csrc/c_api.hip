@@ -439,8 +439,9 @@ int pllm_fp8_gemm_ws(const uint8_t* a, const float* a_scale, const uint8_t* weig
 static bool fp8_uses_gemm(int64_t rows, int64_t k, int64_t n) { return k % 256 == 0 && rows >= tile_gemm_min_rows(RowClass::kFp8, n * k); }
 // float32 activations keep the float32 matvec (rel-L2 <= 1e-5 against the float statement of the operator, src/kernels/ops.py:641-648)
 // for every row count below 16; from 16 rows on they take the tile kernel like the 16-bit types (operands rounded to fp16, <= 1e-3).
+// up to 16 rows of 16-bit activations run the matrix-core form of the matvec (one pass over the weights, exact products)
 static bool fp8_uses_gemm_for(int x_dtype, int64_t rows, int64_t k, int64_t n) {
-    return fp8_uses_gemm(rows, k, n) && (x_dtype != PLLM_F32 || rows >= 16);
+    return fp8_uses_gemm(rows, k, n) && (x_dtype == PLLM_F32 ? rows >= 16 : rows > 16);
 }
 
 size_t pllm_fp8_block_gemm_workspace_bytes(int64_t rows, int64_t k, int64_t n) {
@@ -519,7 +520,7 @@ int pllm_fp8_bf16scale_matmul_rows(const void* x, int x_dtype, const uint8_t* we
 // the workspace).  float32 activations stay on the float32 matvec, row by row: the tile kernel rounds its operands to fp16,
 // which is inside the bound the reference sets for its fp16-storage variants (2e-2) but not the 2e-4 of its float32 ones.
 static bool fp16scale_uses_gemm(int x_dtype, int64_t batch, int64_t rows, int64_t cols, int64_t x_stride, int64_t y_stride, int64_t weight_stride) {
-    return x_dtype != PLLM_F32 && fp8_uses_gemm(batch, cols, rows) && x_stride == cols && y_stride == rows && weight_stride == cols;
+    return x_dtype != PLLM_F32 && batch > 16 && fp8_uses_gemm(batch, cols, rows) && x_stride == cols && y_stride == rows && weight_stride == cols;
 }
 
 static size_t fp16scale_table_bytes(int64_t rows, int64_t cols) {

@@ -315,6 +315,108 @@ __global__ __launch_bounds__(kThreads) void fp8_generic_matvec_kernel(
     if (lane == 0 && row < n) store_any(y, y_dtype, static_cast<size_t>(blockIdx.y) * y_stride + row, acc);
 }
 
+// ------------------------------------------------------------------------------------------------
+// Two to sixteen activation rows of bf16 or fp16 in one pass over the weights, on the matrix cores.
+// E4M3 codes are exact in bf16 and in fp16 (v_cvt_scalef32_pk_{bf16,f16}_fp8 with scale 1), the activations go in as they are,
+// products and sums are float32: v_mfma_f32_16x16x32_{bf16,f16} with A = 16 activation rows x 32 columns, B = 32 columns x 16
+// weight rows, C[row 4 q .. 4 q + 3][weight row n] in lane (n, q).  A workgroup owns 16 weight rows; its eight waves split the
+// row's 128-column scale blocks (wave v: blocks v, v + 8, ...).  Per block a lane loads its weight row's bytes [32 q, 32 q + 32)
+// (whole cache lines per row) and, for each of the block's four MFMAs j, the activations of its row at columns 32 q + 8 j .. + 8 -
+// the MFMA's column order is the lanes' own, the same on both sides.  The block's sum is scaled by the block scale and added to
+// the wave's total; the waves meet in LDS.  The activations come from cache (16 rows x k x 2 bytes); they are requested one
+// block ahead, the weights of a pass of up to kRows16Blocks blocks all at once.
+// ------------------------------------------------------------------------------------------------
+constexpr int kRows16Waves = 8;
+constexpr int kRows16Blocks = 5;                    // scale blocks per wave and pass
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+typedef _Float16 v8hf __attribute__((ext_vector_type(8)));
+typedef _Float16 v2hf __attribute__((ext_vector_type(2)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+template <bool BF16>
+__device__ __forceinline__ v4f rows16_mfma(const uint4& a, uint32_t w_lo, uint32_t w_hi, v4f c) {
+    if constexpr (BF16) {
+        const v2bf p0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w_lo, 1.0f, false), p1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w_lo, 1.0f, true);
+        const v2bf p2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w_hi, 1.0f, false), p3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w_hi, 1.0f, true);
+        const v8bf b = {p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+        union { uint4 u; v8bf v; } av;
+        av.u = a;
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(av.v, b, c, 0, 0, 0);
+    } else {
+        const v2hf p0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w_lo, 1.0f, false), p1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w_lo, 1.0f, true);
+        const v2hf p2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w_hi, 1.0f, false), p3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w_hi, 1.0f, true);
+        const v8hf b = {p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+        union { uint4 u; v8hf v; } av;
+        av.u = a;
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(av.v, b, c, 0, 0, 0);
+    }
+}
+
+// k a multiple of 128, weight base / pitch and activation base / pitch 16-byte aligned; grid (ceil(n / 16), ceil(rows / 16))
+template <int F16S, bool BF16>
+__global__ __launch_bounds__(64 * kRows16Waves) void fp8_rows16_matvec_kernel(
+    const uint16_t* __restrict__ x, size_t x_stride, const Fp8Mat m, void* __restrict__ y, int y_dtype, size_t y_stride,
+    int k, int n, int total_rows) {
+    __shared__ float partial[kRows16Waves][64][4];
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int col = lane & 15, q = lane >> 4;                                // B column (weight row) and A row (activation row); column quarter
+    const int blocks = k >> 7;
+    const int wrow = min(static_cast<int>(blockIdx.x) * 16 + col, n - 1);
+    const int arow = min(static_cast<int>(blockIdx.y) * 16 + col, total_rows - 1);   // rows past the end: the last row again, result dropped
+    const uint8_t* wp = m.w + static_cast<size_t>(wrow) * m.wstride + 32 * q;
+    const uint16_t* xp = x + static_cast<size_t>(arow) * x_stride + 32 * q;
+    const size_t srow = static_cast<size_t>(wrow >> 7) * m.sstride;
+
+    v4f total = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int b0 = wave; b0 < blocks; b0 += kRows16Waves * kRows16Blocks) {
+        uint4 wreg[kRows16Blocks][2];
+        uint32_t sraw[kRows16Blocks];
+#pragma unroll
+        for (int i = 0; i < kRows16Blocks; ++i) {                            // (past the last block: that one again, not used)
+            const int b = min(b0 + i * kRows16Waves, blocks - 1);
+            sraw[i] = scale_raw_at<F16S>(m.scale, srow + b);
+        }
+#pragma unroll
+        for (int i = 0; i < kRows16Blocks; ++i) {
+            const int b = min(b0 + i * kRows16Waves, blocks - 1);
+            wreg[i][0] = *reinterpret_cast<const uint4*>(wp + 128 * b);
+            wreg[i][1] = *reinterpret_cast<const uint4*>(wp + 128 * b + 16);
+        }
+        uint4 areg[2][4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) areg[0][j] = *reinterpret_cast<const uint4*>(xp + 128 * min(b0, blocks - 1) + 8 * j);
+#pragma unroll
+        for (int i = 0; i < kRows16Blocks; ++i) {
+            if (i + 1 < kRows16Blocks) {
+                const int bn = min(b0 + (i + 1) * kRows16Waves, blocks - 1);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) areg[(i + 1) & 1][j] = *reinterpret_cast<const uint4*>(xp + 128 * bn + 8 * j);
+            }
+            if (b0 + i * kRows16Waves < blocks) {                            // wave-uniform
+                v4f c = {0.0f, 0.0f, 0.0f, 0.0f};
+                c = rows16_mfma<BF16>(areg[i & 1][0], wreg[i][0].x, wreg[i][0].y, c);
+                c = rows16_mfma<BF16>(areg[i & 1][1], wreg[i][0].z, wreg[i][0].w, c);
+                c = rows16_mfma<BF16>(areg[i & 1][2], wreg[i][1].x, wreg[i][1].y, c);
+                c = rows16_mfma<BF16>(areg[i & 1][3], wreg[i][1].z, wreg[i][1].w, c);
+                total += c * scale_value<F16S>(sraw[i]);
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) partial[wave][lane][r] = total[r];
+    __syncthreads();
+    if (tid < 256) {
+        const int l = tid >> 2, r = tid & 3;
+        float sum = 0.0f;
+#pragma unroll
+        for (int v = 0; v < kRows16Waves; ++v) sum += partial[v][l][r];
+        const int out_row = static_cast<int>(blockIdx.y) * 16 + 4 * (l >> 4) + r, out_col = static_cast<int>(blockIdx.x) * 16 + (l & 15);
+        if (out_row < total_rows && out_col < n) store_any(y, y_dtype, static_cast<size_t>(out_row) * y_stride + out_col, sum);
+    }
+}
+
 // fp16 scale table with a row pitch -> dense float32 table (what the tile kernel reads)
 __global__ __launch_bounds__(kThreads) void f16_scale_table_kernel(const uint16_t* __restrict__ src, int src_stride, float* __restrict__ dst,
                                                                    int table_rows, int table_cols) {
@@ -334,6 +436,18 @@ int launch_any(const void* x, int x_dtype, size_t x_stride, const Fp8Mat& ma, co
                            y, y_dtype, y_stride, k, n);
         return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
     }
+    if constexpr (!SWIGLU)
+        if (rows >= 2 && (x_dtype == PLLM_BF16 || x_dtype == PLLM_F16) && k % 128 == 0 &&
+            ((reinterpret_cast<uintptr_t>(x) | (x_stride * 2)) & 15u) == 0) {
+            const dim3 grid((n + 15) / 16, (rows + 15) / 16);
+            if (x_dtype == PLLM_BF16)
+                hipLaunchKernelGGL((fp8_rows16_matvec_kernel<F16S, true>), grid, dim3(64 * kRows16Waves), 0, stream, static_cast<const uint16_t*>(x), x_stride,
+                                   ma, y, y_dtype, y_stride, k, n, rows);
+            else
+                hipLaunchKernelGGL((fp8_rows16_matvec_kernel<F16S, false>), grid, dim3(64 * kRows16Waves), 0, stream, static_cast<const uint16_t*>(x), x_stride,
+                                   ma, y, y_dtype, y_stride, k, n, rows);
+            return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+        }
     const int groups = (n + kWaves - 1) / kWaves;                            // one row per wave; a workgroup multiplies two groups at a time (SWIGLU: one, both matrices)
     const int niter = ((k >> 4) + 63) / 64;
     const int passes = (niter + 5) / 6;

@@ -135,10 +135,34 @@ def test_fp8_matvec_matches_oracle(mod, n, k, rows):
         y = mod.fp8_block_gemm_forward(xd, torch.from_numpy(codes).to(DEV), torch.from_numpy(scale).to(DEV))
         torch.cuda.synchronize()
         want = O.matmul_f(xd.float().cpu().numpy(), O.dequant_fp8_block(codes, scale))
-        # float32 activations stay on the float32 matvec below 16 rows whatever the matrix size; 16-bit activations may take
-        # the fp16 tile kernel from a few rows on for large matrices (operands rounded to fp16)
-        tol = 1e-3 if (dt != torch.float32 and rows >= 3 and n * k >= (64 << 20)) else 1e-5
+        # float32 activations stay on the float32 matvec below 16 rows whatever the matrix size; 16-bit activations take the
+        # matrix-core matvec (exact products) up to 16 rows and may take the fp16 tile kernel beyond (operands rounded to fp16)
+        tol = 1e-3 if (dt != torch.float32 and rows > 16 and n * k >= (64 << 20)) else 1e-5
         assert O.rel_l2(y.cpu().numpy(), want) <= tol, (n, k, rows, dt)
+
+
+@pytest.mark.parametrize("n,k,rows", [(33, 384, 2), (16, 128, 5), (130, 1024, 16), (64, 5120, 17), (48, 6144, 9), (5, 256, 40), (33, 384, 40)])
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+def test_fp8_few_rows_on_the_matrix_cores(mod, n, k, rows, dt):
+    """Two or more rows of 16-bit activations with k a multiple of 128: one pass over the weights for every 16 rows, codes and
+    activations exact in the matrix-core operands.  Row counts around 16, weight rows that do not fill a tile, rows of more
+    scale blocks than a wave holds at once; every code value occurs."""
+    rng = np.random.default_rng(90 + n + rows)
+    codes = rng.integers(0, 256, size=(n, k), dtype=np.uint8)
+    codes[(codes & 0x7f) == 0x7f] = 0x3c
+    scale = rng.uniform(0.001, 0.01, size=((n + 127) // 128, (k + 127) // 128)).astype(np.float32)
+    x = torch.from_numpy(rng.standard_normal((rows, k)).astype(np.float32)).to(DEV).to(dt)
+    print(f"case fp8 few rows n={n} k={k} rows={rows} {dt}", flush=True)
+    y = mod.fp8_block_gemm_forward(x, torch.from_numpy(codes).to(DEV), torch.from_numpy(scale).to(DEV))
+    torch.cuda.synchronize()
+    want = O.matmul_f(x.float().cpu().numpy(), O.dequant_fp8_block(codes, scale))
+    got = y.cpu().numpy()
+    assert y.dtype == torch.float32 and got.shape == want.shape
+    # more than 16 rows of a multiple of 256 columns run the fp16 tile kernel (operands rounded to fp16); other column counts
+    # stay here, 16 rows per pass over the weights
+    exact = rows <= 16 or k % 256 != 0
+    assert O.rel_l2(got, want) <= (1e-5 if exact else 1e-3)
+    assert np.abs(got - want).max() <= (1e-4 if exact else 1e-2) * np.abs(want).max()
 
 
 def test_fp8_act_quant_matches_reference_recipe(mod):
