@@ -319,14 +319,13 @@ __global__ __launch_bounds__(kThreads) void fp8_generic_matvec_kernel(
 // Two to sixteen activation rows of bf16 or fp16 in one pass over the weights, on the matrix cores.
 // E4M3 codes are exact in bf16 and in fp16 (v_cvt_scalef32_pk_{bf16,f16}_fp8 with scale 1), the activations go in as they are,
 // products and sums are float32: v_mfma_f32_16x16x32_{bf16,f16} with A = 16 activation rows x 32 columns, B = 32 columns x 16
-// weight rows, C[row 4 q .. 4 q + 3][weight row n] in lane (n, q).  A workgroup owns 16 weight rows; its eight waves split the
-// row's 128-column scale blocks (wave v: blocks v, v + 8, ...).  Per block a lane loads its weight row's bytes [32 q, 32 q + 32)
+// weight rows, C[row 4 q .. 4 q + 3][weight row n] in lane (n, q).  A workgroup owns 16 or 32 weight rows (one or two tiles per wave);
+// its eight or four waves split the row's 128-column scale blocks (wave v: blocks v, v + WAVES, ...).  Per block a lane loads its weight row's bytes [32 q, 32 q + 32)
 // (whole cache lines per row) and, for each of the block's four MFMAs j, the activations of its row at columns 32 q + 8 j .. + 8 -
 // the MFMA's column order is the lanes' own, the same on both sides.  The block's sum is scaled by the block scale and added to
 // the wave's total; the waves meet in LDS.  The activations come from cache (16 rows x k x 2 bytes); they are requested one
 // block ahead, the weights of a pass of up to kRows16Blocks blocks all at once.
 // ------------------------------------------------------------------------------------------------
-constexpr int kRows16Waves = 8;
 constexpr int kRows16Blocks = 5;                    // scale blocks per wave and pass
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
@@ -353,36 +352,48 @@ __device__ __forceinline__ v4f rows16_mfma(const uint4& a, uint32_t w_lo, uint32
     }
 }
 
-// k a multiple of 128, weight base / pitch and activation base / pitch 16-byte aligned; grid (ceil(n / 16), ceil(rows / 16))
-template <int F16S, bool BF16>
-__global__ __launch_bounds__(64 * kRows16Waves) void fp8_rows16_matvec_kernel(
+// k a multiple of 128, weight base / pitch and activation base / pitch 16-byte aligned; grid (ceil(n / (16 TILES)), ceil(rows / 16)).
+// TILES tiles of 16 weight rows per wave share the wave's activation operands.
+template <int F16S, bool BF16, int TILES, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void fp8_rows16_matvec_kernel(
     const uint16_t* __restrict__ x, size_t x_stride, const Fp8Mat m, void* __restrict__ y, int y_dtype, size_t y_stride,
     int k, int n, int total_rows) {
-    __shared__ float partial[kRows16Waves][64][4];
+    __shared__ float partial[WAVES][TILES][64][4];
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
     const int col = lane & 15, q = lane >> 4;                                // B column (weight row) and A row (activation row); column quarter
     const int blocks = k >> 7;
-    const int wrow = min(static_cast<int>(blockIdx.x) * 16 + col, n - 1);
     const int arow = min(static_cast<int>(blockIdx.y) * 16 + col, total_rows - 1);   // rows past the end: the last row again, result dropped
-    const uint8_t* wp = m.w + static_cast<size_t>(wrow) * m.wstride + 32 * q;
     const uint16_t* xp = x + static_cast<size_t>(arow) * x_stride + 32 * q;
-    const size_t srow = static_cast<size_t>(wrow >> 7) * m.sstride;
+    const uint8_t* wp[TILES];
+    size_t srow[TILES];
+#pragma unroll
+    for (int t = 0; t < TILES; ++t) {
+        const int wrow = min((static_cast<int>(blockIdx.x) * TILES + t) * 16 + col, n - 1);
+        wp[t] = m.w + static_cast<size_t>(wrow) * m.wstride + 32 * q;
+        srow[t] = static_cast<size_t>(wrow >> 7) * m.sstride;
+    }
 
-    v4f total = {0.0f, 0.0f, 0.0f, 0.0f};
-    for (int b0 = wave; b0 < blocks; b0 += kRows16Waves * kRows16Blocks) {
-        uint4 wreg[kRows16Blocks][2];
-        uint32_t sraw[kRows16Blocks];
+    v4f total[TILES];
+#pragma unroll
+    for (int t = 0; t < TILES; ++t) total[t] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int b0 = wave; b0 < blocks; b0 += WAVES * kRows16Blocks) {
+        uint4 wreg[kRows16Blocks][TILES][2];
+        uint32_t sraw[kRows16Blocks][TILES];
 #pragma unroll
         for (int i = 0; i < kRows16Blocks; ++i) {                            // (past the last block: that one again, not used)
-            const int b = min(b0 + i * kRows16Waves, blocks - 1);
-            sraw[i] = scale_raw_at<F16S>(m.scale, srow + b);
+            const int b = min(b0 + i * WAVES, blocks - 1);
+#pragma unroll
+            for (int t = 0; t < TILES; ++t) sraw[i][t] = scale_raw_at<F16S>(m.scale, srow[t] + b);
         }
 #pragma unroll
         for (int i = 0; i < kRows16Blocks; ++i) {
-            const int b = min(b0 + i * kRows16Waves, blocks - 1);
-            wreg[i][0] = *reinterpret_cast<const uint4*>(wp + 128 * b);
-            wreg[i][1] = *reinterpret_cast<const uint4*>(wp + 128 * b + 16);
+            const int b = min(b0 + i * WAVES, blocks - 1);
+#pragma unroll
+            for (int t = 0; t < TILES; ++t) {
+                wreg[i][t][0] = *reinterpret_cast<const uint4*>(wp[t] + 128 * b);
+                wreg[i][t][1] = *reinterpret_cast<const uint4*>(wp[t] + 128 * b + 16);
+            }
         }
         uint4 areg[2][4];
 #pragma unroll
@@ -390,31 +401,44 @@ __global__ __launch_bounds__(64 * kRows16Waves) void fp8_rows16_matvec_kernel(
 #pragma unroll
         for (int i = 0; i < kRows16Blocks; ++i) {
             if (i + 1 < kRows16Blocks) {
-                const int bn = min(b0 + (i + 1) * kRows16Waves, blocks - 1);
+                const int bn = min(b0 + (i + 1) * WAVES, blocks - 1);
 #pragma unroll
                 for (int j = 0; j < 4; ++j) areg[(i + 1) & 1][j] = *reinterpret_cast<const uint4*>(xp + 128 * bn + 8 * j);
             }
-            if (b0 + i * kRows16Waves < blocks) {                            // wave-uniform
-                v4f c = {0.0f, 0.0f, 0.0f, 0.0f};
-                c = rows16_mfma<BF16>(areg[i & 1][0], wreg[i][0].x, wreg[i][0].y, c);
-                c = rows16_mfma<BF16>(areg[i & 1][1], wreg[i][0].z, wreg[i][0].w, c);
-                c = rows16_mfma<BF16>(areg[i & 1][2], wreg[i][1].x, wreg[i][1].y, c);
-                c = rows16_mfma<BF16>(areg[i & 1][3], wreg[i][1].z, wreg[i][1].w, c);
-                total += c * scale_value<F16S>(sraw[i]);
+            if (b0 + i * WAVES < blocks) {                                   // wave-uniform
+#pragma unroll
+                for (int t = 0; t < TILES; ++t) {
+                    v4f c = {0.0f, 0.0f, 0.0f, 0.0f};
+                    c = rows16_mfma<BF16>(areg[i & 1][0], wreg[i][t][0].x, wreg[i][t][0].y, c);
+                    c = rows16_mfma<BF16>(areg[i & 1][1], wreg[i][t][0].z, wreg[i][t][0].w, c);
+                    c = rows16_mfma<BF16>(areg[i & 1][2], wreg[i][t][1].x, wreg[i][t][1].y, c);
+                    c = rows16_mfma<BF16>(areg[i & 1][3], wreg[i][t][1].z, wreg[i][t][1].w, c);
+                    total[t] += c * scale_value<F16S>(sraw[i][t]);
+                }
             }
         }
     }
 #pragma unroll
-    for (int r = 0; r < 4; ++r) partial[wave][lane][r] = total[r];
+    for (int t = 0; t < TILES; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) partial[wave][t][lane][r] = total[t][r];
     __syncthreads();
-    if (tid < 256) {
-        const int l = tid >> 2, r = tid & 3;
+    for (int e = tid; e < TILES * 256; e += 64 * WAVES) {
+        const int t = e >> 8, l = (e >> 2) & 63, r = e & 3;
         float sum = 0.0f;
 #pragma unroll
-        for (int v = 0; v < kRows16Waves; ++v) sum += partial[v][l][r];
-        const int out_row = static_cast<int>(blockIdx.y) * 16 + 4 * (l >> 4) + r, out_col = static_cast<int>(blockIdx.x) * 16 + (l & 15);
+        for (int v = 0; v < WAVES; ++v) sum += partial[v][t][l][r];
+        const int out_row = static_cast<int>(blockIdx.y) * 16 + 4 * (l >> 4) + r, out_col = (static_cast<int>(blockIdx.x) * TILES + t) * 16 + (l & 15);
         if (out_row < total_rows && out_col < n) store_any(y, y_dtype, static_cast<size_t>(out_row) * y_stride + out_col, sum);
     }
+}
+
+template <int F16S, bool BF16, int TILES, int WAVES>
+int launch_rows16(const void* x, size_t x_stride, const Fp8Mat& ma, void* y, int y_dtype, size_t y_stride, int rows, int k, int n, hipStream_t stream) {
+    const dim3 grid((n + 16 * TILES - 1) / (16 * TILES), (rows + 15) / 16);
+    hipLaunchKernelGGL((fp8_rows16_matvec_kernel<F16S, BF16, TILES, WAVES>), grid, dim3(64 * WAVES), 0, stream, static_cast<const uint16_t*>(x), x_stride,
+                       ma, y, y_dtype, y_stride, k, n, rows);
+    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 
 // fp16 scale table with a row pitch -> dense float32 table (what the tile kernel reads)
@@ -439,14 +463,15 @@ int launch_any(const void* x, int x_dtype, size_t x_stride, const Fp8Mat& ma, co
     if constexpr (!SWIGLU)
         if (rows >= 2 && (x_dtype == PLLM_BF16 || x_dtype == PLLM_F16) && k % 128 == 0 &&
             ((reinterpret_cast<uintptr_t>(x) | (x_stride * 2)) & 15u) == 0) {
-            const dim3 grid((n + 15) / 16, (rows + 15) / 16);
-            if (x_dtype == PLLM_BF16)
-                hipLaunchKernelGGL((fp8_rows16_matvec_kernel<F16S, true>), grid, dim3(64 * kRows16Waves), 0, stream, static_cast<const uint16_t*>(x), x_stride,
-                                   ma, y, y_dtype, y_stride, k, n, rows);
-            else
-                hipLaunchKernelGGL((fp8_rows16_matvec_kernel<F16S, false>), grid, dim3(64 * kRows16Waves), 0, stream, static_cast<const uint16_t*>(x), x_stride,
-                                   ma, y, y_dtype, y_stride, k, n, rows);
-            return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+            // two tiles per wave halve the activation operands fetched per weight byte; they pay from 8 rows on, on long rows and
+            // on matrices of few tiles (17408x5120 at 2 / 16 rows: 23.5 / 38.4 us with one tile and eight waves, 25.1 / 37.1 with two
+            // and four; 5120x17408: 34.9 / 57.8 against 30.6 / 40.0)
+            const bool two_tiles = rows >= 8 || k >= 8192 || n < 8192;
+            if (two_tiles)
+                return x_dtype == PLLM_BF16 ? launch_rows16<F16S, true, 2, 4>(x, x_stride, ma, y, y_dtype, y_stride, rows, k, n, stream)
+                                            : launch_rows16<F16S, false, 2, 4>(x, x_stride, ma, y, y_dtype, y_stride, rows, k, n, stream);
+            return x_dtype == PLLM_BF16 ? launch_rows16<F16S, true, 1, 8>(x, x_stride, ma, y, y_dtype, y_stride, rows, k, n, stream)
+                                        : launch_rows16<F16S, false, 1, 8>(x, x_stride, ma, y, y_dtype, y_stride, rows, k, n, stream);
         }
     const int groups = (n + kWaves - 1) / kWaves;                            // one row per wave; a workgroup multiplies two groups at a time (SWIGLU: one, both matrices)
     const int niter = ((k >> 4) + 63) / 64;
