@@ -257,9 +257,11 @@ def extra_cases(mod, dev):
     sc = torch.from_numpy(scale).to(dev)
     run("fp8_e4m3 matvec 17408x5120 T=1", codes.size + scale.size * 4,
         lambda s, ring=ring, x=x, sc=sc: mod.fp8_block_gemm_forward(x, ring[s], sc), len(ring))
-    x2 = torch.randn(2, 5120, device=dev, dtype=torch.bfloat16)
-    run("fp8_e4m3 matvec 17408x5120 T=2", codes.size + scale.size * 4,
-        lambda s, ring=ring, x2=x2, sc=sc: mod.fp8_block_gemm_forward(x2, ring[s], sc), len(ring))
+    # a few rows of bf16 activations: one pass over the weights for up to 16 rows on the matrix cores
+    for t in (2, 4, 16):
+        xt = torch.randn(t, 5120, device=dev, dtype=torch.bfloat16)
+        run(f"fp8_e4m3 matvec 17408x5120 T={t}", codes.size + scale.size * 4,
+            lambda s, ring=ring, xt=xt, sc=sc: mod.fp8_block_gemm_forward(xt, ring[s], sc), len(ring))
     del ring
     # the same weights with fp16 scales behind the C++ engine's operator forms: matvec and fused gate/up SwiGLU (float32 activations)
     from pocketllm_amd import qwen_fp8_ops as Q
@@ -320,6 +322,28 @@ def extra_cases(mod, dev):
     out.append({"case": "fused experts iq2_xxs gate/up + iq1_m down, 256 experts top-8, T=256", "weight_bytes": nbytes,
                 "us_per_call": round(us, 3), "gbs": round(nbytes / us / 1e3, 1), "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
                 "tflops": round(flops / us / 1e6, 2), "graph": graphed, "note": f"{touched} of 256 experts touched by the 2048 routes"})
+    # routed experts of a type without fused expert kernels (the common Q4_K checkpoints): 128 experts of 2048 -> 768, top-8, route by
+    # route through the dense decode kernels (random valid blocks: the work does not depend on the values)
+    ek, dk, ik = 128, 2048, 768
+
+    def q4k_random(*lead):
+        b = rng.integers(0, 256, size=tuple(lead) + (144,), dtype=np.uint8)
+        b[..., 0:2] = np.frombuffer(np.float16(0.01).tobytes(), dtype=np.uint8)
+        b[..., 2:4] = np.frombuffer(np.float16(0.005).tobytes(), dtype=np.uint8)
+        return torch.from_numpy(b).to(dev)
+    kw1, kw3, kw2 = q4k_random(ek, ik, dk // 256), q4k_random(ek, ik, dk // 256), q4k_random(ek, dk, ik // 256)
+    kbytes = 8 * (2 * ik * (dk // 256) + dk * (ik // 256)) * 144
+    ksets = [torch.from_numpy(rng.choice(ek, size=8, replace=False).astype(np.int64)).to(dev) for _ in range(8)]
+    kwts = torch.full((8,), 0.125, device=dev)
+    xk = torch.randn(1, dk, device=dev, dtype=torch.bfloat16)
+    run("routed experts q4_k, 128 experts top-8, 2048 -> 768, T=1 (four launches)", kbytes,
+        lambda s: mod.gguf_moe_single_token_forward(xk, ksets[s], kwts, kw1, kw3, kw2, 0.0), 8)
+    idx16 = np.stack([rng.choice(ek, size=8, replace=False) for _ in range(16)]).astype(np.int64)
+    _, ktoks, krws, kseg = mod.moe_group_routes(torch.from_numpy(idx16).to(dev), torch.full((16, 8), 0.125, device=dev), 0, ek)
+    xk16 = torch.randn(16, dk, device=dev, dtype=torch.bfloat16)
+    us, graphed = time_calls_us(lambda s: mod.gguf_moe_prefill_grouped_forward(xk16, ktoks, krws, kseg, kw1, kw3, kw2, dk, 3, dk, 3, ik, 3, empty, 0.0), 4)
+    out.append({"case": "routed experts q4_k, 128 experts top-8, 2048 -> 768, T=16 (128 routes, route by route)", "us_per_call": round(us, 3), "graph": graphed})
+    del kw1, kw3, kw2
     # one decoder layer's quantized-matmul path at T=1, MiniMax-M2 shapes (hidden 3072, 48 query / 8 key-value heads of 128, 256 experts
     # of 1536, top-8): norm + Q5_K q/k/v projections, Q5_K output projection, norm + routing, fused experts.  Attention itself
     # (rotary embedding, cache, softmax) is not on this path: the projection output feeds the next step directly.
