@@ -237,8 +237,8 @@ def extra_cases(mod, dev):
     ring = ring_of(blocks, dev, 12)
     run("q4_k paired projection 2 x 17408x5120 T=1", 2 * blocks.size,
         lambda s, ring=ring: mod.gguf_quant_gemm_pair_forward(x, ring[s], 5120, 3, ring[(s + 6) % 12], 5120, 3, empty), len(ring))
-    # a few activation rows (speculative decoding, small batches): two or four rows share one pass over the weights
-    for t in (2, 4):
+    # a few activation rows (speculative decoding, small batches): up to sixteen rows share one pass over the weights
+    for t in (2, 4, 8, 16):
         xt = torch.randn(t, 5120, device=dev, dtype=torch.bfloat16)
         run(f"q4_k matvec 17408x5120 T={t}", blocks.size, lambda s, ring=ring, xt=xt: mod.gguf_quant_gemm_forward(xt, ring[s], 5120, 3, empty), len(ring))
     del ring

@@ -833,6 +833,195 @@ int launch_groups16(const ActRows& act, const WeightRoute& route, const uint8_t*
 #undef PLLM_CASE
 }
 
+// ------------------------------------------------------------------------------------------------
+// Q4_K / Q5_K, 2 - 16 rows of bf16 or fp16 activations in one pass over the weights: the activation rows are the ROWS of a
+// half-precision matrix-core product and go in as they are (no quantization, no pre-pass).
+//   v_mfma_f32_16x16x32_{bf16,f16}: A = 16 activation rows x the 32 columns of one scale group, B = the group's 32 codes x 16 weight
+//   rows, C[activation row 4 q .. 4 q + 3][weight row n] in lane (n, q), float32.
+// The codes enter B as the exact values M + code (bf16: M = 16 for 4-bit codes, bits 0x4180 | code << 3; M = 32 for 5-bit codes,
+// 0x4200 | code << 2; fp16: 0x4c00 | code << 6 and 0x5000 | code << 5), built from the code bytes with a byte permute and a shift;
+// a second MFMA per group with B = 1 gives the group's activation sums S, which take M back out and carry the min term:
+//   y += d sc_g (C' - M S) - dmin m_g S = (d sc_g) C' - (M d sc_g + dmin m_g) S       per group g, activation row and weight row.
+// Lane (n, q) holds bytes [8 q, 8 q + 8) of each 32-byte chunk j of the block's codes (codes 8 q .. 8 q + 7 of groups 2 j, low
+// nibbles, and 2 j + 1, high nibbles) and reads the activations at the same columns.  A workgroup owns TILES x 16 weight rows per
+// wave, its WAVES waves split the row's super-blocks and meet in LDS; the activation operands and the sums are shared by a
+// wave's tiles.  Weights of kRows16Depth blocks in flight per wave, activations one block ahead.
+// ------------------------------------------------------------------------------------------------
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef _Float16 v8hf __attribute__((ext_vector_type(8)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+constexpr int kRows16Depth = 3;
+
+template <bool BF16>
+__device__ __forceinline__ v4f half_mfma(const uint4& a, const uint4& b, v4f c) {
+    if constexpr (BF16) {
+        union { uint4 u; v8bf v; } av, bv;
+        av.u = a; bv.u = b;
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(av.v, bv.v, c, 0, 0, 0);
+    } else {
+        union { uint4 u; v8hf v; } av, bv;
+        av.u = a; bv.u = b;
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(av.v, bv.v, c, 0, 0, 0);
+    }
+}
+
+// eight code bytes (two dwords) -> eight halves M + code
+template <bool BF16, bool FIVE>
+__device__ __forceinline__ uint4 code_halves(uint32_t c0, uint32_t c1) {
+    constexpr uint32_t kMagic = BF16 ? (FIVE ? 0x42004200u : 0x41804180u) : (FIVE ? 0x50005000u : 0x4c004c00u);
+    constexpr int kShift = BF16 ? (FIVE ? 2 : 3) : (FIVE ? 5 : 6);
+    // bytes [b0, 0, b1, 0] and [b2, 0, b3, 0], then (x << kShift) | magic per half
+    const uint32_t a0 = __builtin_amdgcn_perm(0u, c0, 0x04010400u), a1 = __builtin_amdgcn_perm(0u, c0, 0x04030402u);
+    const uint32_t a2 = __builtin_amdgcn_perm(0u, c1, 0x04010400u), a3 = __builtin_amdgcn_perm(0u, c1, 0x04030402u);
+    return make_uint4((a0 << kShift) | kMagic, (a1 << kShift) | kMagic, (a2 << kShift) | kMagic, (a3 << kShift) | kMagic);
+}
+
+struct Rows16Q4K {
+    static constexpr int kBlockBytes = 144;
+    static constexpr bool kFive = false;
+    struct Regs { uint4 hdr; uint2 q[4]; };
+    static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, int q) {
+        r.hdr = *reinterpret_cast<const uint4*>(blk);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) r.q[j] = *reinterpret_cast<const uint2*>(blk + 16 + 32 * j + 8 * q);
+    }
+    // code bytes of group g = 2 j + nib
+    static __device__ __forceinline__ uint2 codes(const Regs& r, int j, int nib, int) {
+        return nib ? make_uint2((r.q[j].x >> 4) & 0x0f0f0f0fu, (r.q[j].y >> 4) & 0x0f0f0f0fu) : make_uint2(r.q[j].x & 0x0f0f0f0fu, r.q[j].y & 0x0f0f0f0fu);
+    }
+};
+
+struct Rows16Q5K {
+    static constexpr int kBlockBytes = 176;
+    static constexpr bool kFive = true;
+    struct Regs { uint4 hdr; uint2 qh; uint2 q[4]; };
+    static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, int q) {
+        r.hdr = *reinterpret_cast<const uint4*>(blk);
+        r.qh = *reinterpret_cast<const uint2*>(blk + 16 + 8 * q);           // bit g of byte i: the fifth bit of code 8 q + i of group g
+#pragma unroll
+        for (int j = 0; j < 4; ++j) r.q[j] = *reinterpret_cast<const uint2*>(blk + 48 + 32 * j + 8 * q);
+    }
+    static __device__ __forceinline__ uint2 codes(const Regs& r, int j, int nib, int) {
+        const int g = 2 * j + nib;
+        const uint32_t lo = nib ? (r.q[j].x >> 4) & 0x0f0f0f0fu : r.q[j].x & 0x0f0f0f0fu;
+        const uint32_t hi = nib ? (r.q[j].y >> 4) & 0x0f0f0f0fu : r.q[j].y & 0x0f0f0f0fu;
+        // bit g of every qh byte to bit 4: a rotation only wraps bits that the mask drops
+        const uint32_t rot = static_cast<uint32_t>(g + 28) & 31u;
+        return make_uint2(lo | (__builtin_amdgcn_alignbit(r.qh.x, r.qh.x, rot) & 0x10101010u), hi | (__builtin_amdgcn_alignbit(r.qh.y, r.qh.y, rot) & 0x10101010u));
+    }
+};
+
+// k = 256 bpr, weights and activation rows 16-byte aligned; grid (ceil(n / (16 TILES)), ceil(rows / 16)).
+// ITERS = blocks per wave and pass (wave v: blocks v, v + WAVES, ...); every load is issued outside the branches.
+template <typename FMT, bool BF16, int TILES, int WAVES, int ITERS>
+__global__ __launch_bounds__(64 * WAVES) void k45_rows16_kernel(
+    const uint16_t* __restrict__ x, const uint8_t* __restrict__ w, void* __restrict__ y, int y_dtype, int k, int n, int bpr, int total_rows) {
+    __shared__ float partial[WAVES][TILES][64][4];
+    constexpr int DEPTH = ITERS < kRows16Depth ? ITERS : kRows16Depth;
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int col = lane & 15, q = lane >> 4;
+    const int arow = min(static_cast<int>(blockIdx.y) * 16 + col, total_rows - 1);   // rows past the end: the last row again, result dropped
+    const uint16_t* xp = x + static_cast<size_t>(arow) * k + 8 * q;
+    const uint8_t* wp[TILES];
+#pragma unroll
+    for (int t = 0; t < TILES; ++t) {
+        const int wrow = min((static_cast<int>(blockIdx.x) * TILES + t) * 16 + col, n - 1);
+        wp[t] = w + static_cast<size_t>(wrow) * bpr * FMT::kBlockBytes;
+    }
+    constexpr float kM = FMT::kFive ? 32.0f : 16.0f;
+    constexpr uint32_t kOnes = BF16 ? 0x3f803f80u : 0x3c003c00u;
+    const uint4 ones = make_uint4(kOnes, kOnes, kOnes, kOnes);
+
+    v4f total[TILES];
+#pragma unroll
+    for (int t = 0; t < TILES; ++t) total[t] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int b0 = wave; b0 < bpr; b0 += WAVES * ITERS) {
+        typename FMT::Regs regs[DEPTH][TILES];
+        uint4 areg[2][8];
+        auto request_w = [&](int it) {
+            const int b = min(b0 + it * WAVES, bpr - 1);                      // (past the last block: that one again, not used)
+#pragma unroll
+            for (int t = 0; t < TILES; ++t) FMT::load(regs[it % DEPTH][t], wp[t] + static_cast<size_t>(b) * FMT::kBlockBytes, q);
+        };
+        auto request_a = [&](int it) {
+            const int b = min(b0 + it * WAVES, bpr - 1);
+#pragma unroll
+            for (int g = 0; g < 8; ++g) areg[it & 1][g] = *reinterpret_cast<const uint4*>(xp + 256 * b + 32 * g);
+        };
+        request_a(0);
+#pragma unroll
+        for (int it = 0; it < DEPTH; ++it) request_w(it);
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+            if (it + 1 < ITERS) request_a(it + 1);
+            if (b0 + it * WAVES < bpr) {                                     // wave-uniform
+                K4Scales sc[TILES];
+                float dd[TILES], dmin[TILES];
+#pragma unroll
+                for (int t = 0; t < TILES; ++t) {
+                    sc[t] = k4_unpack(regs[it % DEPTH][t].hdr);
+                    dd[t] = f16_bits_to_float(regs[it % DEPTH][t].hdr.x & 0xffffu);
+                    dmin[t] = f16_bits_to_float(regs[it % DEPTH][t].hdr.x >> 16);
+                }
+#pragma unroll
+                for (int g = 0; g < 8; ++g) {
+                    const uint4 a = areg[it & 1][g];
+                    const v4f sums = half_mfma<BF16>(a, ones, v4f{0.0f, 0.0f, 0.0f, 0.0f});
+#pragma unroll
+                    for (int t = 0; t < TILES; ++t) {
+                        const uint2 cb = FMT::codes(regs[it % DEPTH][t], g >> 1, g & 1, q);
+                        const v4f c = half_mfma<BF16>(a, code_halves<BF16, FMT::kFive>(cb.x, cb.y), v4f{0.0f, 0.0f, 0.0f, 0.0f});
+                        const uint32_t scw = (g < 4 ? sc[t].sc_lo : sc[t].sc_hi) >> (8 * (g & 3));
+                        const uint32_t mnw = (g < 4 ? sc[t].mn_lo : sc[t].mn_hi) >> (8 * (g & 3));
+                        const float ca = dd[t] * static_cast<float>(scw & 0xffu);
+                        const float cs = __builtin_fmaf(kM, ca, dmin[t] * static_cast<float>(mnw & 0xffu));
+                        total[t] += c * ca - sums * cs;
+                    }
+                }
+            }
+            if (it + DEPTH < ITERS) request_w(it + DEPTH);
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < TILES; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) partial[wave][t][lane][r] = total[t][r];
+    __syncthreads();
+    for (int e = tid; e < TILES * 256; e += 64 * WAVES) {
+        const int t = e >> 8, l = (e >> 2) & 63, r = e & 3;
+        float sum = 0.0f;
+#pragma unroll
+        for (int v = 0; v < WAVES; ++v) sum += partial[v][t][l][r];
+        const int out_row = static_cast<int>(blockIdx.y) * 16 + 4 * (l >> 4) + r, out_col = (static_cast<int>(blockIdx.x) * TILES + t) * 16 + (l & 15);
+        if (out_row < total_rows && out_col < n) store_any(y, y_dtype, static_cast<size_t>(out_row) * n + out_col, sum);
+    }
+}
+
+template <typename FMT, int TILES, int WAVES, int ITERS>
+int launch_rows16_it(const void* x, int x_dtype, const uint8_t* w, void* y, int y_dtype, int rows, int k, int n, int bpr, hipStream_t stream) {
+    const dim3 grid((n + 16 * TILES - 1) / (16 * TILES), (rows + 15) / 16);
+    if (x_dtype == PLLM_BF16)
+        hipLaunchKernelGGL((k45_rows16_kernel<FMT, true, TILES, WAVES, ITERS>), grid, dim3(64 * WAVES), 0, stream, static_cast<const uint16_t*>(x), w, y, y_dtype, k, n, bpr, rows);
+    else
+        hipLaunchKernelGGL((k45_rows16_kernel<FMT, false, TILES, WAVES, ITERS>), grid, dim3(64 * WAVES), 0, stream, static_cast<const uint16_t*>(x), w, y, y_dtype, k, n, bpr, rows);
+    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+}
+
+template <typename FMT, int TILES, int WAVES>
+int launch_rows16(const void* x, int x_dtype, const uint8_t* w, void* y, int y_dtype, int rows, int k, int n, int bpr, hipStream_t stream) {
+    const int niter = (bpr + WAVES - 1) / WAVES;
+    const int passes = (niter + 5) / 6;
+    switch ((niter + passes - 1) / passes) {
+        case 1: return launch_rows16_it<FMT, TILES, WAVES, 1>(x, x_dtype, w, y, y_dtype, rows, k, n, bpr, stream);
+        case 2: return launch_rows16_it<FMT, TILES, WAVES, 2>(x, x_dtype, w, y, y_dtype, rows, k, n, bpr, stream);
+        case 3: return launch_rows16_it<FMT, TILES, WAVES, 3>(x, x_dtype, w, y, y_dtype, rows, k, n, bpr, stream);
+        case 4: return launch_rows16_it<FMT, TILES, WAVES, 4>(x, x_dtype, w, y, y_dtype, rows, k, n, bpr, stream);
+        case 5: return launch_rows16_it<FMT, TILES, WAVES, 5>(x, x_dtype, w, y, y_dtype, rows, k, n, bpr, stream);
+        default: return launch_rows16_it<FMT, TILES, WAVES, 6>(x, x_dtype, w, y, y_dtype, rows, k, n, bpr, stream);
+    }
+}
+
 }  // namespace
 
 size_t kquant_matvec_workspace_bytes(int rows, int bpr) { return act_image_256_bytes(bpr) * static_cast<size_t>(rows); }
@@ -860,6 +1049,22 @@ int groups16_wave_matvec(const ActRows& act, const uint8_t* w, int type_id, void
     if (type_id == PLLM_TYPE_Q2_K) return launch_groups16<WaveQ2K>(act, route, w, y, y_dtype, rows, n, bpr, stream);
     if (type_id == PLLM_TYPE_Q6_K) return launch_groups16<WaveQ6K>(act, route, w, y, y_dtype, rows, n, bpr, stream);
     return PLLM_ERR_UNSUPPORTED;
+}
+
+// Q4_K / Q5_K on 2 - 16 raw rows of bf16 / fp16 activations whose length is a whole number of super-blocks (PLLM_ERR_UNSUPPORTED otherwise)
+int k45_rows16_matvec(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y, int y_dtype, int rows, int k, int n, int bpr, hipStream_t stream) {
+    if ((type_id != PLLM_TYPE_Q4_K && type_id != PLLM_TYPE_Q5_K) || (x_dtype != PLLM_BF16 && x_dtype != PLLM_F16)) return PLLM_ERR_UNSUPPORTED;
+    if (rows < 2 || k != 256 * bpr || ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) & 15u)) return PLLM_ERR_UNSUPPORTED;
+    // one tile per wave and four waves on matrices of many tiles of short rows; long rows and matrices of few tiles run two tiles per
+    // wave (which share the activation operands) on eight waves (Q4_K, us at 2 / 4 / 8 / 16 rows: 17408x5120 22.7 / 23.8 / 26.3 / 33.9
+    // against 28.4 / 29.6 / 31.4 / 37.4; 5120x17408 30.5 / 32.0 / 36.0 / 46.6 against 30.3 / 31.4 / 33.3 / 38.6; 5120x5120 11.3 / 11.7 /
+    // 12.9 / 15.7 against 10.6 / 10.9 / 11.5 / 13.7)
+    const bool two_tiles = k >= 8192 || n < 8192;
+    if (type_id == PLLM_TYPE_Q4_K)
+        return two_tiles ? launch_rows16<Rows16Q4K, 2, 8>(x, x_dtype, w, y, y_dtype, rows, k, n, bpr, stream)
+                         : launch_rows16<Rows16Q4K, 1, 4>(x, x_dtype, w, y, y_dtype, rows, k, n, bpr, stream);
+    return two_tiles ? launch_rows16<Rows16Q5K, 2, 8>(x, x_dtype, w, y, y_dtype, rows, k, n, bpr, stream)
+                     : launch_rows16<Rows16Q5K, 1, 4>(x, x_dtype, w, y, y_dtype, rows, k, n, bpr, stream);
 }
 
 }  // namespace pllm

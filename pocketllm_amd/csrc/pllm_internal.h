@@ -87,6 +87,9 @@ int dot4_matvec_from_image(const ActRows& act, const uint8_t* w, int type_id, vo
                            int rows, int n, int bpr, hipStream_t stream, WeightRoute route = WeightRoute{});
 // Q2_K / Q6_K and IQ4_XS on raw activation rows in the single-launch frames of matvec_kquant.hip (PLLM_ERR_UNSUPPORTED: take the
 // kernels for prepared images)
+// Q4_K / Q5_K, 2 - 16 raw rows of bf16 / fp16 activations (k a whole number of super-blocks) as rows of a half-precision matrix-core
+// product in one pass over the weights (PLLM_ERR_UNSUPPORTED: not such a call)
+int k45_rows16_matvec(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y, int y_dtype, int rows, int k, int n, int bpr, hipStream_t stream);
 int iq4xs_wave_matvec(const ActRows& act, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream,
                       WeightRoute route = WeightRoute{});
 int groups16_wave_matvec(const ActRows& act, const uint8_t* w, int type_id, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream,

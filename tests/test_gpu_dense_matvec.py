@@ -359,6 +359,32 @@ def test_activation_image_first_term_equals_the_reference_quantizer(mod, dtype):
     np.testing.assert_array_equal(gs[..., 0].view(np.uint32), want_gs.view(np.uint32))
 
 
+@pytest.mark.parametrize("type_name", ["q4_k", "q5_k"])
+@pytest.mark.parametrize("n,k,rows", [(40, 768, 3), (16, 256, 16), (100, 5120, 7), (9000, 1280, 5), (33, 17408, 16), (70, 2304, 11)])
+def test_three_to_sixteen_rows_as_matrix_core_operands(mod, type_name, n, k, rows):
+    """3 - 16 rows of bf16 / fp16 activations of a whole number of super-blocks: one pass over the weights with the rows as
+    half-precision matrix-core operands, codes exact, float32 sums.  Weight rows that do not fill a tile, many tiles of short rows
+    (one tile per wave) and long rows or few tiles (two), more blocks per wave than a pass holds, random bytes in every code field."""
+    rng = np.random.default_rng(500 + n + rows)
+    bpr = k // 256
+    blocks = rng.integers(0, 256, size=(n, bpr, O.BLOCK_BYTES[type_name]), dtype=np.uint8)
+    for off in (0, 2):
+        vals = rng.uniform(0.001, 0.05, size=(n, bpr)) * rng.choice([-1.0, 1.0], size=(n, bpr))
+        blocks[..., off:off + 2] = vals.astype("<f2").view(np.uint8).reshape(n, bpr, 2)
+    dev = torch.device("cuda:0")
+    w = torch.from_numpy(blocks).to(dev)
+    empty = torch.empty(0, dtype=torch.int8, device=dev)
+    for dt in (torch.bfloat16, torch.float16):
+        print(f"case rows as operands {type_name} n={n} k={k} rows={rows} {dt}", flush=True)
+        x = torch.from_numpy(rng.standard_normal((rows, k)).astype(np.float32)).to(dev).to(dt)
+        y = mod.gguf_quant_gemm_forward(x, w, k, O.TYPE_IDS[type_name], empty, out_dtype=torch.float32)
+        torch.cuda.synchronize()
+        want = O.matmul_f(x.float().cpu().numpy(), O.dequant_rows(blocks, type_name, k))
+        got = y.cpu().numpy()
+        assert O.rel_l2(got, want) <= 2e-6
+        assert np.abs(got - want).max() <= 2e-5 * np.abs(want).max()
+
+
 @pytest.mark.parametrize("type_name", ["q4_k", "q5_k", "q2_k", "q6_k", "iq4_xs", "iq2_xxs", "iq1_m", "iq2_xs", "iq3_xxs"])
 def test_few_row_calls_equal_the_prequantized_path(mod, type_name):
     """Calls of a few rows may quantize the activations inside the matvec kernel; the result is the same bits as quantizing ahead
@@ -383,6 +409,11 @@ def test_few_row_calls_equal_the_prequantized_path(mod, type_name):
             y_pre = mod.gguf_quant_gemm_prequantized(mod.quantize_activations(x, bpr), blocks, tid, out_dtype=torch.float32)
             if type_name in ("q2_k", "q6_k", "iq4_xs"):
                 assert O.rel_l2(y.cpu().numpy(), y_pre.cpu().numpy()) <= 1e-6
+            elif type_name in ("q4_k", "q5_k") and rows >= 3 and dt != torch.float32 and k % 256 == 0:
+                # three rows or more of 16-bit activations go in unquantized (half-precision matrix-core operands): closer to the
+                # float statement of the operator than the two-term int8 image, not the same bits
+                want = O.matmul_f(x.float().cpu().numpy(), O.dequant_rows(blocks.cpu().numpy(), type_name, k))
+                assert O.rel_l2(y.cpu().numpy(), want) <= 2e-6 and O.rel_l2(y.cpu().numpy(), y_pre.cpu().numpy()) <= 1e-4
             else:
                 assert torch.equal(y, y_pre)
 
