@@ -326,6 +326,16 @@ int pllm_gguf_quant_gemm_multi(const void* x, int x_dtype, const float* norm_wei
     if (norm_weight && !raw) return PLLM_ERR_UNSUPPORTED;                    // the normalisation exists inside the kernel only
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int bpr = static_cast<int>(blocks_per_row);
+    if (!norm_weight && rows >= 3 && rows <= 16) {   // the single-matrix operator's kernel for these calls, one launch per matrix
+        int m = 0;
+        for (; m < count; ++m) {
+            const int st = pllm::k45_rows16_matvec(x, x_dtype, blocks[m], type_id, y[m], y_dtype, static_cast<int>(rows), static_cast<int>(k),
+                                                   static_cast<int>(n[m]), bpr, s);
+            if (st == PLLM_ERR_UNSUPPORTED) break;   // (a matrix it does not take: every output is written again below)
+            if (st != PLLM_OK) return st;
+        }
+        if (m == count) return PLLM_OK;
+    }
     pllm::ActRows act = pllm::act_rows_raw(x, x_dtype, static_cast<int>(k), norm_weight, eps, round_fp16);
     if (!raw) {
         if (!workspace || workspace_bytes < pllm_activation_image_bytes(rows, blocks_per_row)) return PLLM_ERR_WORKSPACE;
@@ -402,6 +412,22 @@ int pllm_gguf_quant_gemm_pair(const void* x, int x_dtype, const uint8_t* blocks0
     const int bpr = static_cast<int>(blocks_per_row);
     const int R = static_cast<int>(rows), N = static_cast<int>(n);
     const size_t esize = y_dtype == PLLM_F32 ? 4 : 2;
+    if (rows >= 3 && rows <= 16) {             // the kernel the single-matrix operator takes for these calls, once per matrix
+        const int st0 = pllm::k45_rows16_matvec(x, x_dtype, blocks0, type_id0, y, y_dtype, R, static_cast<int>(k), N, bpr, s);
+        if (st0 != PLLM_ERR_UNSUPPORTED) {
+            if (st0 != PLLM_OK) return st0;
+            void* y1 = static_cast<char*>(y) + static_cast<size_t>(rows) * n * esize;
+            const int st1 = pllm::k45_rows16_matvec(x, x_dtype, blocks1, type_id1, y1, y_dtype, R, static_cast<int>(k), N, bpr, s);
+            if (st1 != PLLM_ERR_UNSUPPORTED) return st1;
+            // (mixed pair: the second matrix on the kernels below, as its own operator call would run)
+            if (quantizes_in_kernel(type_id1, rows, n, blocks_per_row))
+                return superblock_matvec(pllm::act_rows_raw(x, x_dtype, static_cast<int>(k)), blocks1, type_id1, y1, y_dtype, R, N, bpr, s);
+            const int sti = pllm::act_image_256(x, x_dtype, R, static_cast<int>(k), bpr, workspace, s);
+            if (sti != PLLM_OK) return sti;
+            return superblock_matvec(pllm::act_rows_from_image(static_cast<const unsigned char*>(workspace), pllm::act_image_256_bytes(bpr)), blocks1,
+                                     type_id1, y1, y_dtype, R, N, bpr, s);
+        }
+    }
     const bool k45 = type_id0 == type_id1 && (type_id0 == PLLM_TYPE_Q4_K || type_id0 == PLLM_TYPE_Q5_K);
     const bool raw = k45 ? quantizes_in_kernel(type_id0, rows, 2 * n, blocks_per_row)
                          : quantizes_in_kernel(type_id0, rows, n, blocks_per_row) && quantizes_in_kernel(type_id1, rows, n, blocks_per_row);

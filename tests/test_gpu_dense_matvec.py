@@ -460,7 +460,7 @@ def test_multi_projection_equals_separate_calls(mod, type_name):
     dev = torch.device("cuda:0")
     tid = O.TYPE_IDS[type_name]
     grid = codebooks.grid_tensor_for_type(tid).to(dev)
-    for k, heights, rows in ((3072, (6144, 1024, 1024), 1), (1002, (40, 130, 16, 7), 3), (512, (33,), 2), (768, (64, 200), 20)):
+    for k, heights, rows in ((3072, (6144, 1024, 1024), 1), (1002, (40, 130, 16, 7), 3), (512, (33,), 2), (768, (64, 200), 20), (1024, (48, 200), 5)):
         bpr = (k + 255) // 256
         mats = []
         for n in heights:
