@@ -14,6 +14,7 @@
 // chunk on both sides.
 #include <algorithm>
 
+#include "block_mfma.h"
 #include "pllm_device.h"
 #include "pllm_internal.h"
 
@@ -202,30 +203,253 @@ __global__ __launch_bounds__(256) void fp8_gemm_reduce_kernel(const float* __res
     if (n0 + col + 3 < n) store_any(y, y_dtype, o + 3, total.w);
 }
 
-struct Fp8GemmPlan { int tiles_n, tiles, full_tiles, slices, per; size_t partial_bytes; };
+// ------------------------------------------------------------------------------------------------
+// More than 128 tokens: a tile of 256 tokens x 128 weight rows per workgroup of eight waves (4 x 2, 64 x 64 each), fed by a
+// ring of three LDS stages that direct-to-LDS loads fill two steps ahead: no registers in between, and nothing of a step
+// waits for memory that was asked for one step earlier.
+//  * Rows lie 128 bytes apart in LDS, unpadded, because a wave instruction of such a load writes one contiguous kilobyte
+//    (eight rows); instead the 16-byte pieces of row r are stored at position piece ^ ((r / 2) % 8), which spreads the
+//    sixteen rows that one pass of a 16-byte LDS read touches over all banks.
+//  * The weights are the matrix instruction's A rows and the tokens its columns, so a lane's sums belong to two tokens
+//    and the activation scale is one factor per lane and token block.
+//  * The activation scales of four steps are one 16-byte load per token (a 4-byte gather per step asks the memory system
+//    for as many separate lines as all the codes of the step), in a ring of two groups.
+//  * The scaling of a step's sums runs on the vector ALU while the matrix cores work on the next four instructions: the
+//    second half of a step's sums is scaled during the first instructions of the next step.
+//  * Tile index -> (token tile, row tile): the workgroups that share a block of weight rows are neighbours on one XCD
+//    (hardware deals workgroups to the eight XCDs in turn), so the block reaches that L2 once.
+// What bounds it: a compute unit keeps a limited number of cache requests outstanding, so bytes per step and unit, not
+// the L2's bandwidth, cap the rate at which a tile's codes arrive.
+// ------------------------------------------------------------------------------------------------
+constexpr int kRingM = 256, kRingN = 128, kRingStages = 3, kRingWaves = 8;
+constexpr int kRingA = kRingM * kStep;                        // bytes of a stage's activation codes
+constexpr int kRingB = kRingN * kStep;
+constexpr int kRingStage = kRingA + kRingB;
+constexpr int kRingScales = 2 * kRingM * 16;                   // two groups of four steps' activation scales
+constexpr int kRingLoads = 6;                                  // code loads per wave and stage
+
+__device__ __forceinline__ void ring_tile_origin(int tile, int tiles_m, int& t0, int& n0) {
+    const int xcd = tile & 7, local = tile >> 3;
+    n0 = ((local / tiles_m) * 8 + xcd) * kRingN;
+    t0 = (local % tiles_m) * kRingM;
+}
+
+// sums of one 32 x 32 block times one factor into the running sums
+__device__ __forceinline__ void ring_scale_into(floatx16& acc, const floatx16& c, float f) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[v] = __builtin_fmaf(c[v], f, acc[v]);
+}
+
+// four neighbouring outputs of one token
+__device__ __forceinline__ void ring_store4(void* y, int y_dtype, size_t at, float v0, float v1, float v2, float v3, bool vector_ok, int valid) {
+    if (vector_ok && valid == 4) {
+        if (y_dtype == PLLM_F32) {
+            *reinterpret_cast<float4*>(static_cast<float*>(y) + at) = make_float4(v0, v1, v2, v3);
+        } else if (y_dtype == PLLM_BF16) {
+            const uint32_t lo = from_float<bf16_t>(v0).bits | (static_cast<uint32_t>(from_float<bf16_t>(v1).bits) << 16);
+            const uint32_t hi = from_float<bf16_t>(v2).bits | (static_cast<uint32_t>(from_float<bf16_t>(v3).bits) << 16);
+            *reinterpret_cast<uint2*>(static_cast<uint16_t*>(y) + at) = make_uint2(lo, hi);
+        } else {
+            typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+            half4 h = {static_cast<_Float16>(v0), static_cast<_Float16>(v1), static_cast<_Float16>(v2), static_cast<_Float16>(v3)};
+            *reinterpret_cast<half4*>(static_cast<_Float16*>(y) + at) = h;
+        }
+        return;
+    }
+    if (valid > 0) store_any(y, y_dtype, at, v0);
+    if (valid > 1) store_any(y, y_dtype, at + 1, v1);
+    if (valid > 2) store_any(y, y_dtype, at + 2, v2);
+    if (valid > 3) store_any(y, y_dtype, at + 3, v3);
+}
+
+__global__ __launch_bounds__(64 * kRingWaves) void fp8_gemm_ring_kernel(
+    const uint8_t* __restrict__ a, const float* __restrict__ a_s, const uint8_t* __restrict__ b, const float* __restrict__ b_s,
+    void* __restrict__ y, int y_dtype, int rows, int n, int k, int tiles_m, int full_tiles, int slices, int per, float* __restrict__ partial) {
+    extern __shared__ __align__(1024) unsigned char smem[];
+    const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_byte_ptr)smem));
+    constexpr int kScaleOff = kRingStages * kRingStage;
+    float* w_scale = reinterpret_cast<float*>(smem + kScaleOff + kRingScales);     // [steps of this workgroup]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wt = wave >> 1, wr = wave & 1;                              // the wave's 64 tokens and 64 weight rows of the tile
+    const int wg = blockIdx.x;
+    const bool whole = wg < full_tiles;
+    const int rest = wg - full_tiles;
+    int t0, n0;
+    ring_tile_origin(whole ? wg : full_tiles + rest / slices, tiles_m, t0, n0);
+    if (n0 >= n) return;                                                  // (row tiles are dealt in eights)
+    const int steps = k / kStep;                                          // a multiple of four
+    const int s_begin = whole ? 0 : (rest % slices) * per;
+    const int s_end = whole ? steps : min(steps, s_begin + per);
+
+    // the weight block's scales of all steps, through ordinary loads, before the first direct-to-LDS load is issued
+    for (int i = tid; i < s_end - s_begin; i += 64 * kRingWaves) w_scale[i] = b_s[static_cast<size_t>(n0 >> 7) * steps + s_begin + i];
+
+    // this wave's pieces of a stage: kilobytes 4 wave .. 4 wave + 3 of the token tile and 2 wave, 2 wave + 1 of the weight
+    // tile (eight rows each; lane = row in the piece, position in the row); waves 0 .. 3: the scales of 64 tokens
+    const int pr = lane >> 3, pc = lane & 7;
+    auto piece_src = [&](const uint8_t* base, int row0, int limit, int piece) {
+        const int row = 8 * piece + pr;
+        return base + static_cast<size_t>(min(row0 + row, limit - 1)) * k + 16 * (pc ^ ((row >> 1) & 7));
+    };
+    const uint8_t* const as0 = piece_src(a, t0, rows, 4 * wave); const uint8_t* const as1 = piece_src(a, t0, rows, 4 * wave + 1);
+    const uint8_t* const as2 = piece_src(a, t0, rows, 4 * wave + 2); const uint8_t* const as3 = piece_src(a, t0, rows, 4 * wave + 3);
+    const uint8_t* const bs0 = piece_src(b, n0, n, 2 * wave); const uint8_t* const bs1 = piece_src(b, n0, n, 2 * wave + 1);
+    const float* const ss = a_s + static_cast<size_t>(min(t0 + (wave & 3) * 64 + lane, rows - 1)) * steps;
+    auto issue = [&](int s, int buf) {
+        const size_t off = static_cast<size_t>(s) * kStep;
+        const uint32_t base = lds0 + buf * kRingStage;
+        lds_dma16(as0 + off, base + (4 * wave) * 1024); lds_dma16(as1 + off, base + (4 * wave + 1) * 1024);
+        lds_dma16(as2 + off, base + (4 * wave + 2) * 1024); lds_dma16(as3 + off, base + (4 * wave + 3) * 1024);
+        lds_dma16(bs0 + off, base + kRingA + (2 * wave) * 1024); lds_dma16(bs1 + off, base + kRingA + (2 * wave + 1) * 1024);
+    };
+    // scales of steps 4 g .. 4 g + 3 (g clamped to the last group); always issued AHEAD of a stage's code loads, so that
+    // "all but the newest six loads have landed" covers them
+    auto issue_scales = [&](int g) {
+        if (wave < 4) {
+            const int gc = min(g, steps / 4 - 1);
+            lds_dma16(ss + 4 * gc, lds0 + kScaleOff + (g & 1) * (kRingM * 16) + wave * 1024);
+        }
+    };
+
+    floatx16 acc[2][2];                      // [32 weight rows i][32 tokens j]
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    // operand reads: lane (row l of a 32-row block, K half hs) takes pieces 4 h + 2 hs and + 1 of its row; the rows of
+    // both operands are l plus multiples of 16, so one set of swizzled positions serves all of them
+    const int l = lane & 31, hs = lane >> 5, x = (l >> 1) & 7;
+    const int o00 = 16 * ((2 * hs) ^ x), o01 = 16 * ((2 * hs + 1) ^ x), o10 = 16 * ((4 + 2 * hs) ^ x), o11 = 16 * ((5 + 2 * hs) ^ x);
+    auto operand2 = [&](const unsigned char* row, int lo, int hi) {
+        const uint4 u = *reinterpret_cast<const uint4*>(row + lo);
+        const uint4 w = *reinterpret_cast<const uint4*>(row + hi);
+        v8i r;
+        r[0] = static_cast<int>(u.x); r[1] = static_cast<int>(u.y); r[2] = static_cast<int>(u.z); r[3] = static_cast<int>(u.w);
+        r[4] = static_cast<int>(w.x); r[5] = static_cast<int>(w.y); r[6] = static_cast<int>(w.z); r[7] = static_cast<int>(w.w);
+        return r;
+    };
+    const floatx16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+
+    issue_scales(s_begin >> 2);
+    issue_scales((s_begin >> 2) + 1);
+    issue(s_begin, 0);
+    issue(min(s_begin + 1, s_end - 1), 1);
+    int buf = 0;
+    floatx16 late0 = zero, late1 = zero;     // the second half (weight rows 32 .. 63) of the previous step's sums, not yet scaled
+    float late_f0 = 0.0f, late_f1 = 0.0f;
+    for (int s = s_begin; s < s_end; ++s) {
+        wait_vm<kRingLoads>();               // this wave's loads of stage s have landed (the newest stage may be on its way) ...
+        __syncthreads();                     // ... and everybody's; nobody reads the stage of step s - 1 any more
+        const int nbuf = buf == 0 ? 2 : buf - 1;
+        if ((s & 3) == 0) issue_scales((s >> 2) + 1);
+        issue(min(s + 2, s_end - 1), nbuf);  // (no branch around the loads: past the end a step is fetched again and dropped)
+        const unsigned char* stage = smem + buf * kRingStage;
+        const unsigned char* tk = stage + (wt * 64 + l) * kStep;
+        const unsigned char* wg_rows = stage + kRingA + (wr * 64 + l) * kStep;
+        const float* tok_scale = reinterpret_cast<const float*>(smem + kScaleOff + ((s >> 2) & 1) * (kRingM * 16)) + (s & 3);
+        const float ws = w_scale[s - s_begin];
+        const float f0 = tok_scale[4 * (wt * 64 + l)] * ws, f1 = tok_scale[4 * (wt * 64 + 32 + l)] * ws;
+        const v8i t0h0 = operand2(tk, o00, o01), t1h0 = operand2(tk + 32 * kStep, o00, o01);
+        const v8i w0h0 = operand2(wg_rows, o00, o01);
+        const v8i t0h1 = operand2(tk, o10, o11), t1h1 = operand2(tk + 32 * kStep, o10, o11);
+        const v8i w0h1 = operand2(wg_rows, o10, o11);
+        const v8i w1h0 = operand2(wg_rows + 32 * kStep, o00, o01), w1h1 = operand2(wg_rows + 32 * kStep, o10, o11);
+        // weight rows 0 .. 31 on the matrix cores while the vector ALU scales the previous step's second half
+        floatx16 c0 = mfma_e4m3(w0h0, t0h0, zero);
+        floatx16 c1 = mfma_e4m3(w0h0, t1h0, zero);
+        ring_scale_into(acc[1][0], late0, late_f0);
+        c0 = mfma_e4m3(w0h1, t0h1, c0);
+        c1 = mfma_e4m3(w0h1, t1h1, c1);
+        ring_scale_into(acc[1][1], late1, late_f1);
+        // weight rows 32 .. 63 while the first half is scaled
+        late0 = mfma_e4m3(w1h0, t0h0, zero);
+        late1 = mfma_e4m3(w1h0, t1h0, zero);
+        ring_scale_into(acc[0][0], c0, f0);
+        late0 = mfma_e4m3(w1h1, t0h1, late0);
+        late1 = mfma_e4m3(w1h1, t1h1, late1);
+        ring_scale_into(acc[0][1], c1, f1);
+        late_f0 = f0; late_f1 = f1;
+        buf = buf == 2 ? 0 : buf + 1;
+    }
+    ring_scale_into(acc[1][0], late0, late_f0);
+    ring_scale_into(acc[1][1], late1, late_f1);
+    wait_vm<0>();                            // the dropped loads past the end: nothing may arrive in LDS after the workgroup has left
+
+    // D[m][n]: lane holds column n = token l of block j and rows m = weight rows 8 * (v / 4) + 4 * hs + v % 4 of block i
+    float* const dst = whole ? nullptr : partial + static_cast<size_t>(rest) * kRingM * kRingN;   // a slice's sums: [token of the tile][row of the tile]
+    const bool vector_ok = (n & 3) == 0 && !(y_dtype & 0x100);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int tok = wt * 64 + j * 32 + l;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int col = wr * 64 + i * 32 + 8 * q + 4 * hs;
+                const float v0 = acc[i][j][4 * q], v1 = acc[i][j][4 * q + 1], v2 = acc[i][j][4 * q + 2], v3 = acc[i][j][4 * q + 3];
+                if (!whole) *reinterpret_cast<float4*>(dst + tok * kRingN + col) = make_float4(v0, v1, v2, v3);
+                else if (t0 + tok < rows) ring_store4(y, y_dtype, static_cast<size_t>(t0 + tok) * n + n0 + col, v0, v1, v2, v3, vector_ok, min(4, n - n0 - col));
+            }
+    }
+}
+
+// the split tiles of the ring kernel: sums over the slices in slice order; one workgroup per 1024 elements of a tile
+__global__ __launch_bounds__(256) void fp8_gemm_ring_reduce_kernel(const float* __restrict__ partial, void* __restrict__ y, int y_dtype, int rows, int n,
+                                                                   int tiles_m, int full_tiles, int slices) {
+    int t0, n0;
+    ring_tile_origin(full_tiles + blockIdx.y, tiles_m, t0, n0);
+    const int i = (blockIdx.x * 256 + threadIdx.x) * 4;                    // four neighbouring columns of one row
+    const int row = i / kRingN, col = i % kRingN;
+    const float* src = partial + static_cast<size_t>(blockIdx.y) * slices * kRingM * kRingN + i;
+    float4 total = *reinterpret_cast<const float4*>(src);
+    for (int sl = 1; sl < slices; ++sl) {
+        const float4 v = *reinterpret_cast<const float4*>(src + static_cast<size_t>(sl) * kRingM * kRingN);
+        total.x += v.x; total.y += v.y; total.z += v.z; total.w += v.w;
+    }
+    if (t0 + row >= rows || n0 >= n) return;
+    const size_t o = static_cast<size_t>(t0 + row) * n + n0 + col;
+    if (n0 + col < n) store_any(y, y_dtype, o, total.x);
+    if (n0 + col + 1 < n) store_any(y, y_dtype, o + 1, total.y);
+    if (n0 + col + 2 < n) store_any(y, y_dtype, o + 2, total.z);
+    if (n0 + col + 3 < n) store_any(y, y_dtype, o + 3, total.w);
+}
+
+
+struct Fp8GemmPlan { bool ring; int tiles_m, tiles_n, tiles, full_tiles, slices, per; size_t partial_bytes; };
 
 // Whole rounds of tiles run unsplit; the left-over tiles (all tiles, when there is less than one round) are cut along K so that
 // their workgroups fill the machine about once, as long as the partial sums stay under 64 MB and a slice keeps two steps.
-Fp8GemmPlan plan_fp8_gemm(int rows, int k, int n) {
+// More than 128 tokens take the ring kernel's 256 x 128 tiles (one workgroup per compute unit, row tiles dealt in eights).
+Fp8GemmPlan plan_fp8_gemm(int rows, int k, int n, bool allow_ring) {
     Fp8GemmPlan p;
+    p.ring = allow_ring && rows > kTile && (k / kStep) % 4 == 0;       // (scales of four steps are one load)
+    const int tile_m = p.ring ? kRingM : kTile;
+    p.tiles_m = (rows + tile_m - 1) / tile_m;
     p.tiles_n = (n + kTile - 1) / kTile;
-    p.tiles = p.tiles_n * ((rows + kTile - 1) / kTile);
-    const int resident = 2 * compute_units();
+    if (p.ring) p.tiles_n = (p.tiles_n + 7) / 8 * 8;
+    p.tiles = p.tiles_n * p.tiles_m;
+    const int resident = (p.ring ? 1 : 2) * compute_units();
     const int steps = k / kStep;
+    const size_t tile_bytes = static_cast<size_t>(tile_m) * kTile * sizeof(float);
     p.full_tiles = (p.tiles / resident) * resident;
     const int rem = p.tiles - p.full_tiles;
     p.slices = 1;
     p.per = steps;
     if (rem > 0 && rem * 2 <= resident) {
         int slices = std::min(resident / rem, std::max(1, steps / 2));
-        slices = std::min<int>(slices, static_cast<int>((static_cast<size_t>(64) << 20) / (static_cast<size_t>(rem) * kTile * kTile * sizeof(float))));
+        slices = std::min<int>(slices, static_cast<int>((static_cast<size_t>(64) << 20) / (static_cast<size_t>(rem) * tile_bytes)));
         if (slices >= 2) {
             p.per = (steps + slices - 1) / slices;
             p.slices = (steps + p.per - 1) / p.per;
         }
     }
     if (p.slices == 1) p.full_tiles = p.tiles;
-    p.partial_bytes = p.slices > 1 ? static_cast<size_t>(p.tiles - p.full_tiles) * p.slices * kTile * kTile * sizeof(float) : 0;
+    p.partial_bytes = p.slices > 1 ? static_cast<size_t>(p.tiles - p.full_tiles) * p.slices * tile_bytes : 0;
     return p;
 }
 
@@ -233,24 +457,37 @@ Fp8GemmPlan plan_fp8_gemm(int rows, int k, int n) {
 
 size_t fp8_gemm_native_workspace_bytes(int rows, int k, int n) {
     if (k % kStep != 0 || k <= 0 || rows <= 0 || n <= 0) return 0;
-    return plan_fp8_gemm(rows, k, n).partial_bytes;
+    return std::max(plan_fp8_gemm(rows, k, n, true).partial_bytes, plan_fp8_gemm(rows, k, n, false).partial_bytes);
 }
 
 int fp8_gemm_native(const uint8_t* a, const float* a_s, const uint8_t* b, const float* b_s, void* y, int y_dtype,
                     int rows, int k, int n, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     if (k % kStep != 0 || k <= 0) return PLLM_ERR_UNSUPPORTED;
     if ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15u) return PLLM_ERR_UNSUPPORTED;
-    const size_t smem = static_cast<size_t>(4) * kTile * kRow + 2 * kTile * sizeof(float);
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(fp8_gemm_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem)) != hipSuccess)
-        return PLLM_ERR_UNSUPPORTED;
-    Fp8GemmPlan p = plan_fp8_gemm(rows, k, n);
+    const size_t steps_bytes = static_cast<size_t>(k / kStep) * sizeof(float);
+    const bool ring_ok = (reinterpret_cast<uintptr_t>(a_s) & 15u) == 0 && static_cast<size_t>(kRingStages) * kRingStage + kRingScales + steps_bytes <= 160 * 1024;
+    Fp8GemmPlan p = plan_fp8_gemm(rows, k, n, ring_ok);
+    const size_t ring_smem = static_cast<size_t>(kRingStages) * kRingStage + kRingScales + static_cast<size_t>(k / kStep) * sizeof(float);
+    const size_t smem = p.ring ? ring_smem : static_cast<size_t>(4) * kTile * kRow + 2 * kTile * sizeof(float);
+    const void* kern = p.ring ? reinterpret_cast<const void*>(fp8_gemm_ring_kernel) : reinterpret_cast<const void*>(fp8_gemm_kernel);
+    if (hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem)) != hipSuccess) return PLLM_ERR_UNSUPPORTED;
     if (p.slices > 1 && (!workspace || workspace_bytes < p.partial_bytes)) {  // no room for partial sums: every tile whole
         p.slices = 1;
         p.per = k / kStep;
         p.full_tiles = p.tiles;
     }
     const int rem = p.tiles - p.full_tiles;
-    hipLaunchKernelGGL(fp8_gemm_kernel, dim3(p.full_tiles + rem * p.slices), dim3(256), smem, stream, a, a_s, b, b_s, y, y_dtype, rows, n, k,
+    const dim3 grid(p.full_tiles + rem * p.slices);
+    if (p.ring) {
+        hipLaunchKernelGGL(fp8_gemm_ring_kernel, grid, dim3(64 * kRingWaves), smem, stream, a, a_s, b, b_s, y, y_dtype, rows, n, k, p.tiles_m,
+                           p.full_tiles, p.slices, p.per, static_cast<float*>(workspace));
+        if (hipGetLastError() != hipSuccess) return PLLM_ERR_LAUNCH;
+        if (rem > 0)
+            hipLaunchKernelGGL(fp8_gemm_ring_reduce_kernel, dim3(kRingM * kRingN / 1024, rem), dim3(256), 0, stream, static_cast<const float*>(workspace),
+                               y, y_dtype, rows, n, p.tiles_m, p.full_tiles, p.slices);
+        return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+    }
+    hipLaunchKernelGGL(fp8_gemm_kernel, grid, dim3(256), smem, stream, a, a_s, b, b_s, y, y_dtype, rows, n, k,
                        p.tiles_n, p.full_tiles, p.slices, p.per, static_cast<float*>(workspace));
     if (hipGetLastError() != hipSuccess) return PLLM_ERR_LAUNCH;
     if (rem > 0)

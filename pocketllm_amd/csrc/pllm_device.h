@@ -145,13 +145,13 @@ __device__ __forceinline__ void quantize4(const float v[4], uint32_t& hi, uint32
     const float y = normal ? __builtin_amdgcn_rcpf(scale) : 0.0f;
     const float thr = scale * (0.5f - 1e-4f);
     float qm[4], r[4];
-    bool sure = normal;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         qm[i] = __builtin_fmaf(v[i], y, kRound);
         r[i] = __builtin_fmaf(kRound - qm[i], scale, v[i]);     // v - q * scale
-        sure = sure && fabsf(r[i]) < thr;
     }
+    // one comparison on the largest residual (a NaN among the values has the same code either way and drops out of the maximum)
+    const bool sure = normal && fmaxf(fmaxf(fabsf(r[0]), fabsf(r[1])), fmaxf(fabsf(r[2]), fabsf(r[3]))) < thr;
     if (__builtin_amdgcn_ballot_w64(am > 0.0f && !sure) != 0) {  // wave-uniform: a quotient next to a rounding tie, or an extreme amax
         scale = am / 127.0f;
         const float divisor = am > 0.0f ? scale : 1.0f;

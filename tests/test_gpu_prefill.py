@@ -218,7 +218,8 @@ def test_prefill_operator_serves_q6_k_and_iq4_xs(mod, type_name, t, n, k):
 
 # ---- FP8 activations x FP8 weights on the native FP8 matrix path -----------------------------------
 
-@pytest.mark.parametrize("t,n,k", [(1, 128, 128), (16, 130, 256), (77, 300, 1024), (200, 512, 5120)])
+@pytest.mark.parametrize("t,n,k", [(1, 128, 128), (16, 130, 256), (77, 300, 1024), (200, 512, 5120), (129, 130, 128), (300, 1100, 1024),
+                                   (513, 2050, 384)])
 def test_fp8_gemm_native_matches_act_quant_semantics(mod, t, n, k):
     """act_quant + fp8_gemm (ops.py:982-1051) against the oracle, which dequantizes both sides and multiplies in
     float64.  The only differences are the matrix core's own summation of 64 products per instruction (full-range
