@@ -214,8 +214,8 @@ __global__ __launch_bounds__(256) void fp8_gemm_reduce_kernel(const float* __res
 //    and the activation scale is one factor per lane and token block.
 //  * The activation scales of four steps are one 16-byte load per token (a 4-byte gather per step asks the memory system
 //    for as many separate lines as all the codes of the step), in a ring of two groups.
-//  * The scaling of a step's sums runs on the vector ALU while the matrix cores work on the next four instructions: the
-//    second half of a step's sums is scaled during the first instructions of the next step.
+//  * The scaling of a step's sums runs on the vector ALU while the matrix cores work on the next instructions; the last
+//    block of a step is scaled during the first instructions of the next step.
 //  * Tile index -> (token tile, row tile): the workgroups that share a block of weight rows are neighbours on one XCD
 //    (hardware deals workgroups to the eight XCDs in turn), so the block reaches that L2 once.
 // What bounds it: a compute unit keeps a limited number of cache requests outstanding, so bytes per step and unit, not
@@ -339,45 +339,52 @@ __global__ __launch_bounds__(64 * kRingWaves) void fp8_gemm_ring_kernel(
     issue_scales((s_begin >> 2) + 1);
     issue(s_begin, 0);
     issue(min(s_begin + 1, s_end - 1), 1);
+    issue(min(s_begin + 2, s_end - 1), 2);
+    wait_vm<2 * kRingLoads>();               // the first stage (and the scales, which are older)
+    __syncthreads();
+    // The loop is cut in the middle of a step: the K half h = 0 of a step's operands is read during the step before, so the
+    // matrix instructions of a step start at once; the one barrier per step sits behind the first four of them, which keep the
+    // matrix cores busy while the waves meet, and the second half's operands are in registers before it.
+    const unsigned char* tk = smem + (wt * 64 + l) * kStep;
+    const unsigned char* wg_rows = smem + kRingA + (wr * 64 + l) * kStep;
+    v8i t0h0 = operand2(tk, o00, o01), t1h0 = operand2(tk + 32 * kStep, o00, o01);
+    v8i w0h0 = operand2(wg_rows, o00, o01), w1h0 = operand2(wg_rows + 32 * kStep, o00, o01);
     int buf = 0;
-    floatx16 late0 = zero, late1 = zero;     // the second half (weight rows 32 .. 63) of the previous step's sums, not yet scaled
-    float late_f0 = 0.0f, late_f1 = 0.0f;
+    floatx16 c11 = zero;                     // weight rows 32 .. 63 x tokens 32 .. 63 of the previous step, not yet scaled
+    float late_f = 0.0f;
     for (int s = s_begin; s < s_end; ++s) {
-        wait_vm<kRingLoads>();               // this wave's loads of stage s have landed (the newest stage may be on its way) ...
-        __syncthreads();                     // ... and everybody's; nobody reads the stage of step s - 1 any more
-        const int nbuf = buf == 0 ? 2 : buf - 1;
-        if ((s & 3) == 0) issue_scales((s >> 2) + 1);
-        issue(min(s + 2, s_end - 1), nbuf);  // (no branch around the loads: past the end a step is fetched again and dropped)
-        const unsigned char* stage = smem + buf * kRingStage;
-        const unsigned char* tk = stage + (wt * 64 + l) * kStep;
-        const unsigned char* wg_rows = stage + kRingA + (wr * 64 + l) * kStep;
         const float* tok_scale = reinterpret_cast<const float*>(smem + kScaleOff + ((s >> 2) & 1) * (kRingM * 16)) + (s & 3);
         const float ws = w_scale[s - s_begin];
         const float f0 = tok_scale[4 * (wt * 64 + l)] * ws, f1 = tok_scale[4 * (wt * 64 + 32 + l)] * ws;
-        const v8i t0h0 = operand2(tk, o00, o01), t1h0 = operand2(tk + 32 * kStep, o00, o01);
-        const v8i w0h0 = operand2(wg_rows, o00, o01);
         const v8i t0h1 = operand2(tk, o10, o11), t1h1 = operand2(tk + 32 * kStep, o10, o11);
-        const v8i w0h1 = operand2(wg_rows, o10, o11);
-        const v8i w1h0 = operand2(wg_rows + 32 * kStep, o00, o01), w1h1 = operand2(wg_rows + 32 * kStep, o10, o11);
-        // weight rows 0 .. 31 on the matrix cores while the vector ALU scales the previous step's second half
-        floatx16 c0 = mfma_e4m3(w0h0, t0h0, zero);
-        floatx16 c1 = mfma_e4m3(w0h0, t1h0, zero);
-        ring_scale_into(acc[1][0], late0, late_f0);
-        c0 = mfma_e4m3(w0h1, t0h1, c0);
-        c1 = mfma_e4m3(w0h1, t1h1, c1);
-        ring_scale_into(acc[1][1], late1, late_f1);
-        // weight rows 32 .. 63 while the first half is scaled
-        late0 = mfma_e4m3(w1h0, t0h0, zero);
-        late1 = mfma_e4m3(w1h0, t1h0, zero);
-        ring_scale_into(acc[0][0], c0, f0);
-        late0 = mfma_e4m3(w1h1, t0h1, late0);
-        late1 = mfma_e4m3(w1h1, t1h1, late1);
-        ring_scale_into(acc[0][1], c1, f1);
-        late_f0 = f0; late_f1 = f1;
+        const v8i w0h1 = operand2(wg_rows, o10, o11), w1h1 = operand2(wg_rows + 32 * kStep, o10, o11);
+        floatx16 c00 = mfma_e4m3(w0h0, t0h0, zero);
+        floatx16 c01 = mfma_e4m3(w0h0, t1h0, zero);
+        floatx16 c10 = mfma_e4m3(w1h0, t0h0, zero);
+        ring_scale_into(acc[1][1], c11, late_f);
+        c11 = mfma_e4m3(w1h0, t1h0, zero);
+        asm volatile("" : "+v"(c00), "+v"(c01), "+v"(c10), "+v"(c11));   // the four instructions above are issued before the wave waits
+
+        wait_vm<kRingLoads>();               // this wave's loads of stage s + 1 have landed (stage s + 2 may be on its way) ...
+        __syncthreads();                     // ... and everybody's; every read of stage s has returned
+        if ((s & 3) == 0) issue_scales((s >> 2) + 1);
+        issue(min(s + 3, s_end - 1), buf);   // (no branch around the loads: past the end a step is fetched again and dropped)
         buf = buf == 2 ? 0 : buf + 1;
+        tk = smem + buf * kRingStage + (wt * 64 + l) * kStep;
+        wg_rows = smem + buf * kRingStage + kRingA + (wr * 64 + l) * kStep;
+        t0h0 = operand2(tk, o00, o01); t1h0 = operand2(tk + 32 * kStep, o00, o01);
+        w0h0 = operand2(wg_rows, o00, o01); w1h0 = operand2(wg_rows + 32 * kStep, o00, o01);
+
+        c00 = mfma_e4m3(w0h1, t0h1, c00);
+        c01 = mfma_e4m3(w0h1, t1h1, c01);
+        c10 = mfma_e4m3(w1h1, t0h1, c10);
+        c11 = mfma_e4m3(w1h1, t1h1, c11);
+        ring_scale_into(acc[0][0], c00, f0);
+        ring_scale_into(acc[0][1], c01, f1);
+        ring_scale_into(acc[1][0], c10, f0);
+        late_f = f1;
     }
-    ring_scale_into(acc[1][0], late0, late_f0);
-    ring_scale_into(acc[1][1], late1, late_f1);
+    ring_scale_into(acc[1][1], c11, late_f);
     wait_vm<0>();                            // the dropped loads past the end: nothing may arrive in LDS after the workgroup has left
 
     // D[m][n]: lane holds column n = token l of block j and rows m = weight rows 8 * (v / 4) + 4 * hs + v % 4 of block i
