@@ -552,6 +552,21 @@ def prefill_pass(mod, dev) -> None:
     print(json.dumps({"prefill_pass": "q4_k 17408x5120 T=2048 x6, fp8 17408x5120 T=512 x6", "flops_q4k": 2.0 * 2048 * k * n, "flops_fp8": 2.0 * 512 * k * n}))
 
 
+def fp8_gemm_pass(mod, dev) -> None:
+    """A few launches of the native FP8 x FP8 matmul for the profiler: 17408x5120 at T=512, then at T=2048."""
+    from pocketllm_amd import block_codec as C
+    rng = np.random.default_rng(6006)
+    k, n = 5120, 17408
+    codes, scale = C.quantize_fp8_block(rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02))
+    codes, scale = torch.from_numpy(codes).to(dev), torch.from_numpy(scale).to(dev)
+    for t in (512, 2048):
+        a, a_s = mod.fp8_act_quant_forward(torch.randn(t, k, device=dev, dtype=torch.bfloat16))
+        for _ in range(8):
+            mod.fp8_gemm_forward(a, a_s, codes, scale)
+    torch.cuda.synchronize()
+    print(json.dumps({"fp8_gemm_pass": "fp8 x fp8 17408x5120, T=512 x8 then T=2048 x8", "flops_512": 2.0 * 512 * k * n, "flops_2048": 2.0 * 2048 * k * n}))
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -563,6 +578,7 @@ def main() -> None:
     ap.add_argument("--pmc-pass", action="store_true", help="short run for rocprofv3 --pmc: dominant kernel + a copy of the same size")
     ap.add_argument("--prefill-pass", action="store_true", help="short run for rocprofv3: a few launches of the MFMA tile kernel")
     ap.add_argument("--decode-pass", action="store_true", help="short run for rocprofv3: Q8_0, FP8, Q2_K, Q6_K and IQ4_XS decode matvec")
+    ap.add_argument("--fp8-gemm-pass", action="store_true", help="short run for rocprofv3: native FP8 x FP8 matmul at T=512 and T=2048")
     ap.add_argument("--iq-pass", action="store_true", help="short run for rocprofv3: IQ2_XXS / IQ1_M matvec and the single-token experts")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -589,6 +605,9 @@ def main() -> None:
         return
     if args.iq_pass:
         iq_pass(mod, dev)
+        return
+    if args.fp8_gemm_pass:
+        fp8_gemm_pass(mod, dev)
         return
     x_np = np.random.default_rng(2002).standard_normal((1, 5120), dtype=np.float32)
     x = torch.from_numpy(x_np).to(dev).to(torch.bfloat16)
