@@ -243,6 +243,33 @@ def test_fp8_gemm_native_matches_act_quant_semantics(mod, t, n, k):
     assert O.rel_l2(y2.float().cpu().numpy(), want) <= 1e-2       # default dtype may be 16-bit
 
 
+@pytest.mark.parametrize("t,n,k", [(300, 1102, 512), (260, 257, 1024)])
+def test_fp8_gemm_native_output_forms_above_128_tokens(mod, t, n, k):
+    """The kernel for more than 128 tokens stores four neighbouring outputs of a token at once where the row length allows it and
+    element by element otherwise; bf16 / fp16 outputs are the float32 ones rounded once; activation scales that do not start on a
+    16-byte boundary take the other kernel (same sums up to the grouping of float32 additions)."""
+    rng = np.random.default_rng(t * n + k)
+    codes, scale = C.quantize_fp8_block(rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02))
+    x_np = rng.standard_normal((t, k)).astype(np.float32)
+    a, a_s = mod.fp8_act_quant_forward(torch.from_numpy(x_np).to(DEV))
+    w, sc = torch.from_numpy(codes).to(DEV), torch.from_numpy(scale).to(DEV)
+    print(f"case fp8 native outputs t={t} n={n} k={k}", flush=True)
+    y32 = mod.fp8_gemm_forward(a, a_s, w, sc)
+    torch.cuda.synchronize()
+    want = O.fp8_gemm_q(x_np, codes, scale)
+    assert O.rel_l2(y32.cpu().numpy(), want) <= 2e-4
+    for dt in (torch.bfloat16, torch.float16):
+        y16 = mod.fp8_gemm_forward(a, a_s, w, sc, out_dtype=dt)
+        assert torch.equal(y16, y32.to(dt)), dt
+    # the same scales four bytes off a 16-byte boundary
+    shifted = torch.empty(a_s.numel() + 1, dtype=torch.float32, device=DEV)[1:].view_as(a_s)
+    shifted.copy_(a_s)
+    assert shifted.data_ptr() % 16 != 0
+    y_other = mod.fp8_gemm_forward(a, shifted, w, sc)
+    torch.cuda.synchronize()
+    assert O.rel_l2(y_other.cpu().numpy(), y32.cpu().numpy()) <= 1e-6
+
+
 def test_fp8_gemm_native_baseline_shape_sampled(mod):
     """BASELINE config 4 at T = 512 with the reference's FP8-activation semantics; 64 sampled columns."""
     rng = np.random.default_rng(1005)
