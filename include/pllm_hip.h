@@ -5,7 +5,11 @@
  * the default stream), enqueues its kernels on that stream and returns without synchronizing.
  * Return value: PLLM_OK or a negative pllm_status; nothing throws.  The library never allocates
  * device memory: outputs and workspaces belong to the caller.  Calls on different streams may run
- * concurrently; there is no mutable global state.
+ * concurrently, with one exception: pllm_gguf_quant_gemm_static_scratch keeps its staging in a
+ * device array that all its calls on one GPU share, so overlapping calls of THAT entry point race
+ * (see its declaration).  The only other state the library keeps is host-side bookkeeping that
+ * never changes a result (the device's compute-unit count, LDS sizes already granted to a kernel,
+ * the address of that array), each guarded for concurrent callers.
  *
  * Each declaration names the reference interface it replaces (paths relative to the PocketLLM
  * checkout).
@@ -93,7 +97,12 @@ size_t pllm_gguf_quant_gemm_workspace_bytes(int type_id, int64_t rows, int64_t k
  * Q4_K / Q5_K matmul with the int8 activation semantics of the reference's MMA prefill path: activations quantized to 32-value
  * int8 blocks (xs = amax / 127, code = rint(x / xs)), integer dots per 32-weight group on the int8 matrix cores,
  *   y[t, r] = sum_g xs[t, g] * (d_r sc_{r,g} * dot_g - dmin_r m_{r,g} * sum of the group's activation codes),
- * d * sc and dmin * m in float32.  Any row count; built for prefill row counts.  Other type ids return PLLM_ERR_UNSUPPORTED.
+ * d * sc and dmin * m in float32.  Up to 65535 rows (more return PLLM_ERR_UNSUPPORTED); built for prefill row counts.  Other
+ * type ids return PLLM_ERR_UNSUPPORTED.
+ * Where this differs from the reference's MMA path: its activation quantizer (src/csrc/llama_mmq/gguf_mma_wrapper.cu:104-119)
+ * stores xs and the group's sum as fp16, the sum being that of the float activations; here xs stays float32 and the min term
+ * uses xs * (sum of the int8 codes).  Both are statements of the same operator with one int8 term per activation; they differ
+ * by the fp16 rounding of xs (2^-11 relative) and by the quantization residual inside the min term.
  * Replaces the MMA branch of gguf_quant_gemm_prefill_forward (src/csrc/llama_mmq/gguf_mma_wrapper.cu:257-322,
  * src/csrc/llama_mmq/mmq.cuh:1329-1455, 2083-2200; activation quantizer src/csrc/cuda_kernel_impl.cu:7090-7117).
  * pllm_gguf_quant_gemm keeps float-activation semantics (fp16 tiles); this entry point is the reference's other statement of
@@ -224,6 +233,9 @@ int pllm_gguf_dequantize_rows(const int64_t* row_ids, int64_t n_selected, const 
  *   Few rows take the bandwidth-bound matvec; 16 rows or more with k a multiple of 256 (5 or more when the matrix has
  *   16M weights, 3 or more when it has 64M) take the MFMA tile kernel, which needs `workspace` (pllm_fp8_block_gemm_workspace_bytes bytes, 256-byte
  *   aligned, private to the call until its kernels have run; the query returns 0 when none is needed).
+ *   Precision: the matvec multiplies in float32 (rel-L2 <= 1e-5 against the float statement); the tile kernel rounds both
+ *   operands to fp16 (<= 1e-3).  float32 activations therefore lose precision at the row count where the tile kernel takes
+ *   over, but never below 16 rows; 16-bit activations of 2 - 16 rows run a matrix-core matvec with exact products.
  */
 int pllm_fp8_block_dequantize(const uint8_t* weight, const float* scale, int64_t n, int64_t k, void* out, int out_dtype, void* stream);
 int pllm_fp8_block_gemm(const void* x, int x_dtype, const uint8_t* weight, const float* scale, void* y, int y_dtype,
@@ -303,8 +315,10 @@ int pllm_fp8_bf16scale_matmul_rows(const void* x, int x_dtype, const uint8_t* we
                                    int64_t weight_stride, int64_t scale_stride, void* stream);
 
 /*
- * Fused routed-expert matmul over raw super-blocks (types Q2_K, IQ2_XXS, IQ1_M; gate/up share a type,
- * the down projection may use another, so IQ2_XXS gate/up with IQ1_M down needs no special case):
+ * Fused routed-expert matmul over raw super-blocks (any of the nine super-block types; gate/up share a
+ * type, the down projection may use another, so IQ2_XXS gate/up with IQ1_M down needs no special case;
+ * pairs of Q2_K / IQ2_XXS / IQ1_M have fused kernels, the other types run route by route through the
+ * dense decode kernels or, from 16 tokens on, as batches of tile matmuls):
  *     y[t] = sum over routes r of token t:  W2_e ( silu(min(W1_e x_t, L)) * clamp(W3_e x_t, +-L) * w_r )
  * with the clamp only when swiglu_limit L > 0.
  *   x [tokens, dim]; w1, w3 [n_experts, inter, ceil(dim/256), bb]; w2 [n_experts, dim, ceil(inter/256), bb]

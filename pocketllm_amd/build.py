@@ -15,7 +15,6 @@ PKG = Path(__file__).resolve().parent
 CSRC = PKG / "csrc"
 OBJ_DIR = PKG / "build"
 LIB = PKG / "libpllm_hip.so"
-PROBE_LIB = PKG / "libpllm_probe.so"        # measurement aids (csrc/probe), kept out of the operator library
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
@@ -47,7 +46,6 @@ def build_library(verbose: bool = True, jobs: int = 8, incremental: bool = False
         for f in futs:
             f.result()
     _run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", *map(str, objs), "-o", str(LIB)])
-    _run(["hipcc", *HIPCC_FLAGS, "-shared", *map(str, sorted((CSRC / "probe").glob("*.hip"))), "-o", str(PROBE_LIB)])
     if verbose:
         print(f"built {LIB} from {len(sources)} sources")
     return LIB

@@ -260,13 +260,8 @@ int launch_stream_raw(const ActRows& act, const uint8_t* w, void* y, int y_dtype
     const int chunk_stride = chunk_bytes + 16;                               // shares are read as aligned dwords: a few bytes past the end
     const size_t smem = static_cast<size_t>(chunk_off) + 2 * chunk_stride;
     if (smem > 160 * 1024) return PLLM_ERR_UNSUPPORTED;
-    static size_t attr_smem = 0;
-    if (smem > 64 * 1024 && smem > attr_smem) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                static_cast<int>(smem)) != hipSuccess)
-            return PLLM_ERR_UNSUPPORTED;
-        attr_smem = smem;
-    }
+    static SmemGrant granted;
+    if (!grant_dynamic_smem(reinterpret_cast<const void*>(kern), smem, granted)) return PLLM_ERR_UNSUPPORTED;
     // resident workgroups per compute unit for this LDS size: asked once per size (the query costs microseconds of host time)
     static size_t occ_smem = ~static_cast<size_t>(0);
     static int occ_per_cu = 1;

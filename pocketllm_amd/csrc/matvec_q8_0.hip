@@ -279,13 +279,8 @@ bool plan_stream(const void* x, int x_dtype, const uint8_t* w, int k, int n, int
 int launch_stream(const void* x, int x_dtype, const uint8_t* w, void* y, int y_dtype, int rows, int k, int n, int pairs, const StreamPlan& plan,
                   hipStream_t stream) {
     auto kern = q8_0_stream_kernel;
-    static size_t attr_smem = 0;
-    if (plan.smem > 64 * 1024 && plan.smem > attr_smem) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                static_cast<int>(plan.smem)) != hipSuccess)
-            return PLLM_ERR_UNSUPPORTED;
-        attr_smem = plan.smem;
-    }
+    static SmemGrant granted;
+    if (!grant_dynamic_smem(reinterpret_cast<const void*>(kern), plan.smem, granted)) return PLLM_ERR_UNSUPPORTED;
     const uint32_t magic = static_cast<uint32_t>(((1ull << 32) + pairs - 1) / pairs);
     hipLaunchKernelGGL(kern, dim3(plan.grid_x, rows), dim3(kStreamThreads), plan.smem, stream, x, x_dtype, w, y, y_dtype, k, n, pairs, magic,
                        plan.image_bytes, plan.cols);

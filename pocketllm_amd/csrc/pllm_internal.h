@@ -5,11 +5,29 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/pllm_hip.h"
 
 namespace pllm {
 
 inline size_t align256(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
+
+// Dynamic LDS above 64 KB has to be granted to a kernel before its launch, on every device it runs on.  `granted` is the
+// caller's per-kernel record (one static instance per launcher): the largest size granted so far per device, so that the
+// attribute call is made only when a call needs more than any before it on that device.  Safe from several threads: a
+// lost race only repeats the attribute call.
+struct SmemGrant { std::atomic<size_t> bytes[16]; };
+inline bool grant_dynamic_smem(const void* kernel, size_t smem, SmemGrant& granted) {
+    if (smem <= 64 * 1024) return true;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return false;
+    std::atomic<size_t>* slot = (dev >= 0 && dev < 16) ? &granted.bytes[dev] : nullptr;
+    if (slot && slot->load(std::memory_order_relaxed) >= smem) return true;
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem)) != hipSuccess) return false;
+    if (slot) slot->store(smem, std::memory_order_relaxed);
+    return true;
+}
 
 // Set in the output dtype code a matvec launcher receives: the kernels add their result to what y holds (float32 sum,
 // rounded once) instead of overwriting it.
