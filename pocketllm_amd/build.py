@@ -19,7 +19,7 @@ LIB = PKG / "libpllm_hip.so"
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-Wno-unused-command-line-argument",
+    "-Wno-unused-command-line-argument", "-Wno-inline-asm",
 ]
 
 

@@ -28,6 +28,11 @@ __device__ __forceinline__ void lds_dma16(const void* src, uint32_t lds_base) {
     // (lds_base is wave-uniform by contract; the readfirstlane only tells the compiler so)
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(__builtin_amdgcn_readfirstlane(lds_base)) : "memory", "m0");
 }
+// the same with the source as a wave-uniform base (scalar registers) plus a 32-bit byte offset per lane: no 64-bit vector
+// arithmetic per copy; lds_base must be a scalar value too (computed from readfirstlane'd or launch-wide quantities only)
+__device__ __forceinline__ void lds_dma16_at(const void* uniform_base, uint32_t lane_off, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(lane_off), "s"(uniform_base), "s"(lds_base) : "memory", "m0");
+}
 template <int N> __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory"); }
 // until at most `newest` of this wave's memory operations are outstanding (they complete in order)
 __device__ __forceinline__ void wait_vm_all_but(int newest) {
@@ -90,9 +95,15 @@ __device__ __forceinline__ void load_a(AOps<SLOTS>& ops, const AMap<SLOTS>& am, 
 // The signed code is (g ^ m) - m bytewise; instead of finishing that per byte, the wave runs two
 // MFMAs per slice, with B = g ^ m and with B = m, and subtracts the accumulators.
 // ------------------------------------------------------------------------------------------------
-struct IQ2XXSm {
+// COPIES > 1: every table entry is stored COPIES times side by side (entry e, copy c at 8 * (e * COPIES + c)) and lane l
+// reads copy l % COPIES, i.e. `tables` is the lane's own pointer (lane_tables).  With 16 copies the 16 lanes that the LDS
+// serves together read from 16 different pairs of banks whatever their indices are: a random 8-byte lookup then costs about 5
+// cycles of the LDS per wave instruction instead of about 12 from a single copy (8.4 with 8 copies), measured on the box.
+template <int COPIES>
+struct IQ2XXSmT {
     static constexpr int kBlockBytes = 66;
-    static constexpr int kTableBytes = IQ2XXS::kTableBytes;
+    static constexpr int kCopies = COPIES;
+    static constexpr int kTableBytes = IQ2XXS::kTableBytes * COPIES;
     static constexpr int kSlots = 4;
     static constexpr bool kStreamed = true;                    // has LDS loaders and table copies for the streamed kernel
     static constexpr int kHoldBlocks = 3;                      // block indices whose activation side a wave may keep in registers
@@ -112,8 +123,20 @@ struct IQ2XXSm {
                          __builtin_amdgcn_alignbit(d3, d2, sh), __builtin_amdgcn_alignbit(d4, d3, sh));
         r.d = *reinterpret_cast<const uint16_t*>(base + off);
     }
-    static __device__ __forceinline__ void stage_tables(unsigned char* lds) { IQ2XXS::stage_tables(lds); }
+    static __device__ __forceinline__ void stage_tables(unsigned char* lds) { static_assert(COPIES == 1, "single copy only"); IQ2XXS::stage_tables(lds); }
     template <int WAVES> static __device__ __forceinline__ void dma_tables(uint32_t lds_base, int wave, int lane);
+    // the lane's view of the tables at `tables` (its copy of every entry)
+    static __device__ __forceinline__ const unsigned char* lane_tables(const unsigned char* tables, int lane) { return tables + 8 * (lane % COPIES); }
+    // the replicated tables, written by the whole workgroup (a barrier must follow): thread e takes entry e from memory
+    static __device__ __forceinline__ void stage_replicated(unsigned char* lds, int tid, int threads) {
+        for (int e = tid; e < 256 + 128; e += threads) {
+            const uint64_t v = e < 256 ? PLLM_IQ2XXS_GRID[e] : PLLM_IQ2XXS_SIGN_MASKS.v[e - 256];
+            const uint32_t lo = static_cast<uint32_t>(v), hi = static_cast<uint32_t>(v >> 32);
+            uint4* dst = reinterpret_cast<uint4*>(lds + static_cast<size_t>(e) * 8 * COPIES);
+#pragma unroll
+            for (int c = 0; c < COPIES / 2; ++c) dst[c] = make_uint4(lo, hi, lo, hi);
+        }
+    }
     static __device__ __forceinline__ void a_map(AMap<kSlots>& am, int col, int ks, int kpad, int zero_off) {
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
@@ -136,14 +159,14 @@ struct IQ2XXSm {
     static __device__ __forceinline__ float block_held(const Regs& r, int, int, const Held& h, const unsigned char*, const AMap<kSlots>&,
                                                        const unsigned char* tables) {
         const uint2* grid = reinterpret_cast<const uint2*>(tables);
-        const uint2* sign = grid + 256;
+        const uint2* sign = grid + 256 * COPIES;
         v4i c = {0, 0, 0, 0}, cm = {0, 0, 0, 0};
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             const uint32_t ids = (t < 2) ? r.q.x : r.q.z, aux = (t < 2) ? r.q.y : r.q.w;
             const int e = 2 * (t & 1);                                         // grid entries e and e + 1 of the sub-block
-            const uint2 g0 = grid[(ids >> (8 * e)) & 0xffu], m0 = sign[(aux >> (7 * e)) & 127u];
-            const uint2 g1 = grid[(ids >> (8 * e + 8)) & 0xffu], m1 = sign[(aux >> (7 * e + 7)) & 127u];
+            const uint2 g0 = grid[((ids >> (8 * e)) & 0xffu) * COPIES], m0 = sign[((aux >> (7 * e)) & 127u) * COPIES];
+            const uint2 g1 = grid[((ids >> (8 * e + 8)) & 0xffu) * COPIES], m1 = sign[((aux >> (7 * e + 7)) & 127u) * COPIES];
             const v4i av = as_v4i(h.a[t].x, h.a[t].y, h.a[t].z, h.a[t].w);
             c = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, as_v4i(g0.x ^ m0.x, g0.y ^ m0.y, g1.x ^ m1.x, g1.y ^ m1.y), c, 0, 0, 0);
             cm = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, as_v4i(m0.x, m0.y, m1.x, m1.y), cm, 0, 0, 0);
@@ -158,13 +181,13 @@ struct IQ2XXSm {
     struct Decoded { v4i b[4]; float ls0, ls1; };
     static __device__ __forceinline__ void decode(const Regs& r, int, const unsigned char* tables, Decoded& o) {
         const uint2* grid = reinterpret_cast<const uint2*>(tables);
-        const uint2* sign = grid + 256;
+        const uint2* sign = grid + 256 * COPIES;
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             const uint32_t ids = (t < 2) ? r.q.x : r.q.z, aux = (t < 2) ? r.q.y : r.q.w;
             const int e = 2 * (t & 1);
-            const uint2 g0 = grid[(ids >> (8 * e)) & 0xffu], m0 = sign[(aux >> (7 * e)) & 127u];
-            const uint2 g1 = grid[(ids >> (8 * e + 8)) & 0xffu], m1 = sign[(aux >> (7 * e + 7)) & 127u];
+            const uint2 g0 = grid[((ids >> (8 * e)) & 0xffu) * COPIES], m0 = sign[((aux >> (7 * e)) & 127u) * COPIES];
+            const uint2 g1 = grid[((ids >> (8 * e + 8)) & 0xffu) * COPIES], m1 = sign[((aux >> (7 * e + 7)) & 127u) * COPIES];
             // negate the masked bytes: (g ^ 0xff) + 1 never carries out of a byte because g >= 8
             o.b[t] = as_v4i((g0.x ^ m0.x) + (m0.x & 0x01010101u), (g0.y ^ m0.y) + (m0.y & 0x01010101u),
                             (g1.x ^ m1.x) + (m1.x & 0x01010101u), (g1.y ^ m1.y) + (m1.y & 0x01010101u));
@@ -191,6 +214,8 @@ struct IQ2XXSm {
         return block_held(r, s, b, h, smem, am, tables);
     }
 };
+
+using IQ2XXSm = IQ2XXSmT<1>;
 
 // ------------------------------------------------------------------------------------------------
 // IQ1_M: 56 B = qs(32) qh(16) scales(8); w = dl (c - 1 + delta) with c in {0, 1, 2} from the
@@ -220,7 +245,9 @@ static __device__ const Iq1DeltaCodes PLLM_IQ1_DELTA_CODES = make_iq1_delta_code
 
 struct IQ1Mm {
     static constexpr int kBlockBytes = 56;
+    static constexpr int kCopies = 1;
     static constexpr int kTableBytes = 32768;
+    static __device__ __forceinline__ const unsigned char* lane_tables(const unsigned char* tables, int) { return tables; }
     static constexpr int kSlots = 8;                           // [term][t]
     static constexpr bool kStreamed = true;
     static constexpr int kHoldBlocks = 0;                      // (its held operands would cost a workgroup per compute unit)
@@ -282,11 +309,23 @@ struct IQ1Mm {
                         ls2 * x8.z * static_cast<float>(__mul24(ch.z, 254) + cl.z) + ls3 * x8.w * static_cast<float>(__mul24(ch.w, 254) + cl.w);
         return f16_bits_to_float(dbits) * v;
     }
+    // the same when each pair of groups shares an activation scale (xa for groups 0 and 1, xb for 2 and 3): the group scales go in as
+    // integers.  |254 ch + cl| <= 16 * 127 * 9 * 255 < 2^23 and the scales are at most 15, so the 24-bit multiplies are exact.
+    static __device__ __forceinline__ float finish_pairs(const Regs& r, int s, const v4i& ch, const v4i& cl, float xa, float xb) {
+        const uint32_t s01 = r.sc.x, s23 = r.sc.y;
+        const uint32_t dbits = ((s01 >> 12) & 0xfu) | ((s01 >> 24) & 0xf0u) | ((s23 >> 4) & 0xf00u) | ((s23 >> 16) & 0xf000u);
+        const uint32_t word = ((s & 2) ? s23 : s01) >> (16 * (s & 1));
+        const int l0 = static_cast<int>(2 * (word & 7u) + 1), l1 = static_cast<int>(2 * ((word >> 3) & 7u) + 1);
+        const int l2 = static_cast<int>(2 * ((word >> 6) & 7u) + 1), l3 = static_cast<int>(2 * ((word >> 9) & 7u) + 1);
+        const int ta = __mul24(l0, __mul24(ch.x, 254) + cl.x) + __mul24(l1, __mul24(ch.y, 254) + cl.y);
+        const int tb = __mul24(l2, __mul24(ch.z, 254) + cl.z) + __mul24(l3, __mul24(ch.w, 254) + cl.w);
+        return f16_bits_to_float(dbits) * (xa * static_cast<float>(ta) + xb * static_cast<float>(tb));
+    }
     static __device__ __forceinline__ float block_held(const Regs& r, int s, int b, const Held& h, const unsigned char* smem,
                                                        const AMap<kSlots>& am, const unsigned char* tables) {
         v4i ch, cl;
         group_dots(r, b, h.a, smem, am, tables, ch, cl);
-        return finish(r, s, ch, cl, make_float4(h.x0, h.x0, h.x1, h.x1));
+        return finish_pairs(r, s, ch, cl, h.x0, h.x1);
     }
     // A block decoded once for several activation vectors: the codes of the lane's four 16-weight
     // groups and their scales times d / 8.
@@ -581,8 +620,10 @@ struct IQ3XXSm {
     }
 };
 
+template <int COPIES>
 template <int WAVES>
-__device__ __forceinline__ void IQ2XXSm::dma_tables(uint32_t lds_base, int wave, int lane) {
+__device__ __forceinline__ void IQ2XXSmT<COPIES>::dma_tables(uint32_t lds_base, int wave, int lane) {
+    static_assert(COPIES == 1, "single copy only");
     dma_share<WAVES>(reinterpret_cast<const unsigned char*>(PLLM_IQ2XXS_GRID), lds_base, 2048, wave, lane);
     dma_share<WAVES>(reinterpret_cast<const unsigned char*>(PLLM_IQ2XXS_SIGN_MASKS.v), lds_base + 2048, 1024, wave, lane);
 }

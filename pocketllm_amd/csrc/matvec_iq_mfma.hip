@@ -12,6 +12,8 @@
 //
 // The codebook lookups happen once per weight and feed 16 rows of dots each, where the v_dot4 form
 // repeats the activation reads and the dots per lane.
+#include <type_traits>
+
 #include "block_mfma.h"
 #include "pllm_internal.h"
 
@@ -82,8 +84,7 @@ __global__ __launch_bounds__(64 * kWaves) void mfma_tile_matvec_kernel(
             if (b < bpr) acc += FMT::block(regs[it], ks, b, smem, am, sx, tables);   // wave-uniform guard
         }
     }
-    acc += __shfl_xor(acc, 16, 64);
-    acc += __shfl_xor(acc, 32, 64);
+    acc = quad_rows_sum(acc);
     if (ks == 0) partial[wave * kRowsPerTile + col] = acc;
     __syncthreads();
     if (tid < kRowsPerTile) {
@@ -141,11 +142,14 @@ int launch_tiles(const ActRows& act, const WeightRoute& route, const uint8_t* w,
 // some multiply while others wait for their chunk.  Needs n % 16 == 0 and a 16-byte aligned matrix.
 // ------------------------------------------------------------------------------------------------
 constexpr int kChunkBudget = 28 * 1024;
+constexpr int kLdsBytes = 160 * 1024;
 
 // NB > 0: a wave meets at most NB block indices (part, part + split, ...) and keeps their activation
 // side in registers across all its chunks; NB == 0: any number, read from LDS every time.
-template <typename FMT, int NB, bool RAW>
-__global__ __launch_bounds__(64 * kWaves) void iq_stream_matvec_kernel(
+// WAVES: 8, several workgroups per compute unit, or 16, one workgroup per compute unit around one set of tables (the form for
+// replicated tables, FMT::kCopies > 1, which take the LDS of several plain ones).
+template <typename FMT, int NB, bool RAW, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void iq_stream_matvec_kernel(
     const ActRows act, const uint8_t* __restrict__ w,
     void* __restrict__ y, int y_dtype, int n, int bpr, int split, int chunks, int chunk_off, int chunk_stride) {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -154,7 +158,6 @@ __global__ __launch_bounds__(64 * kWaves) void iq_stream_matvec_kernel(
     const StagedX sx = carve_staged_x(smem, kpad);
     const int zero_off = image_bytes;                                        // 16 zero bytes
     const int table_off = image_bytes + 16;
-    const unsigned char* tables = smem + table_off;
     float* partial = reinterpret_cast<float*>(smem + table_off + FMT::kTableBytes);   // [waves][16]
     const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_byte_ptr)smem));
 
@@ -162,20 +165,22 @@ __global__ __launch_bounds__(64 * kWaves) void iq_stream_matvec_kernel(
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63;
     const int col = lane & 15, ks = lane >> 4;
-    const int tiles_per_chunk = kWaves / split;
+    const unsigned char* tables = FMT::lane_tables(smem + table_off, lane);
+    const int tiles_per_chunk = WAVES / split;
     const int tile_in_chunk = wave / split, part = wave % split;
     const int row_bytes = bpr * FMT::kBlockBytes;
     const int chunk_rows = tiles_per_chunk * kRowsPerTile;
 
     // activation image, codebooks and the first chunk: all in flight together
-    if constexpr (!RAW) dma_share<kWaves>(act.image + static_cast<size_t>(blockIdx.y) * act.stride, lds0, image_bytes, wave, lane);
-    FMT::template dma_tables<kWaves>(lds0 + table_off, wave, lane);
+    if constexpr (!RAW) dma_share<WAVES>(act.image + static_cast<size_t>(blockIdx.y) * act.stride, lds0, image_bytes, wave, lane);
+    if constexpr (FMT::kCopies == 1) FMT::template dma_tables<WAVES>(lds0 + table_off, wave, lane);
     if (tid < 4) reinterpret_cast<uint32_t*>(smem + zero_off)[tid] = 0;
     AMap<FMT::kSlots> am;
     FMT::a_map(am, col, ks, kpad, zero_off);
 
     int c = blockIdx.x, buf = 0;
-    dma_share<kWaves>(w + static_cast<size_t>(c) * chunk_rows * row_bytes, lds0 + chunk_off, min(chunk_rows, n - c * chunk_rows) * row_bytes, wave, lane);
+    dma_share<WAVES>(w + static_cast<size_t>(c) * chunk_rows * row_bytes, lds0 + chunk_off, min(chunk_rows, n - c * chunk_rows) * row_bytes, wave, lane);
+    if constexpr (FMT::kCopies > 1) FMT::stage_replicated(smem + table_off, tid, 64 * WAVES);   // ordinary stores; the loop's first barrier covers them
     if constexpr (RAW)                       // raw activation row: quantized once per workgroup while the first chunk is on its way
         quantize_row_to_lds(smem, act.x, act.x_dtype, static_cast<size_t>(blockIdx.y) * act.k, act.k, kpad, RowNorm{act.gamma, act.eps, act.round_f16});
     typename FMT::Held held[NB > 0 ? NB : 1];
@@ -187,7 +192,7 @@ __global__ __launch_bounds__(64 * kWaves) void iq_stream_matvec_kernel(
         const int cn = c + gridDim.x;
         int newest = 0;
         if (cn < chunks)
-            newest = dma_share<kWaves>(w + static_cast<size_t>(cn) * chunk_rows * row_bytes, lds0 + chunk_off + (buf ^ 1) * chunk_stride,
+            newest = dma_share<WAVES>(w + static_cast<size_t>(cn) * chunk_rows * row_bytes, lds0 + chunk_off + (buf ^ 1) * chunk_stride,
                                min(chunk_rows, n - cn * chunk_rows) * row_bytes, wave, lane);
         wait_vm_all_but(newest);             // this wave's pieces of chunk c (and of the image and tables) have landed ...
         __syncthreads();                     // ... and everybody else's too
@@ -218,8 +223,7 @@ __global__ __launch_bounds__(64 * kWaves) void iq_stream_matvec_kernel(
                     acc += FMT::block(regs, ks, b, smem, am, sx, tables);
                 }
             }
-            acc += __shfl_xor(acc, 16, 64);
-            acc += __shfl_xor(acc, 32, 64);
+            acc = quad_rows_sum(acc);
             if (split == 1) {
                 if (ks == 0) store_any(y, y_dtype, static_cast<size_t>(blockIdx.y) * n + row0 + tile_in_chunk * kRowsPerTile + col, acc);
             } else if (ks == 0) {
@@ -238,39 +242,203 @@ __global__ __launch_bounds__(64 * kWaves) void iq_stream_matvec_kernel(
     }
 }
 
-// 0 when the streamed form does not apply
-template <typename FMT>
-int stream_split(const uint8_t* w, int n, int bpr) {
-    if (n % kRowsPerTile != 0 || (reinterpret_cast<uintptr_t>(w) & 15u)) return 0;
-    const int tile_bytes = kRowsPerTile * bpr * FMT::kBlockBytes;
-    // the most waves per tile first (smallest chunk) that leaves every wave at least two blocks
-    for (int split = kWaves; split >= 1; split /= 2)
-        if ((split == 1 || bpr >= 2 * split) && (kWaves / split) * tile_bytes <= kChunkBudget) return split;
-    return 0;
+// ------------------------------------------------------------------------------------------------
+// The streamed form for rows of exactly NB * SPLIT super-blocks (every model shape): the row length is a compile-time constant,
+// so are the LDS layout and the number of copy instructions per chunk, and every chunk is whole (the last one is moved back to
+// end at row n; rows it shares with its predecessor are computed twice and stored once).  One barrier per chunk:
+//     wait for my pieces of chunk c | barrier | sums of chunk c - 1 out | request chunk c + 1 | multiply chunk c
+// The barrier says that chunk c has landed AND that everybody has left chunk c - 1, whose buffer the request reuses and whose
+// per-wave sums (kept in two alternating sets) can now be added and stored.  These kernels are bound by the number of
+// instructions a SIMD issues (a step of 16 rows x 256 weights cost ~190 wave instructions in the general form above, a third of
+// them the chunk loop's bookkeeping), not by the LDS or the matrix cores.
+// ------------------------------------------------------------------------------------------------
+template <typename FMT, int NB, int SPLIT, int WAVES>
+struct ExactLayout {
+    static constexpr int kBpr = NB * SPLIT;
+    static constexpr int kKpad = kBpr * 256;
+    static constexpr int kImageBytes = static_cast<int>(staged_x_bytes(kKpad));
+    static constexpr int kZeroOff = kImageBytes;
+    static constexpr int kTableOff = kImageBytes + 16;
+    static constexpr int kPartialOff = kTableOff + FMT::kTableBytes;          // float [2][WAVES][16]
+    static constexpr int kChunkOff = (kPartialOff + 2 * WAVES * 16 * 4 + 1023) & ~1023;
+    static constexpr int kTiles = WAVES / SPLIT;
+    static constexpr int kChunkRows = kTiles * kRowsPerTile;
+    static constexpr int kRowBytes = kBpr * FMT::kBlockBytes;
+    static constexpr int kChunkBytes = kChunkRows * kRowBytes;                // a multiple of 32
+    static constexpr int kChunkStride = kChunkBytes + 16;                     // shares are read as aligned dwords: a few bytes past the end
+    static constexpr int kSmem = kChunkOff + 2 * kChunkStride;
+    static constexpr int kPieces = (kChunkBytes + 1023) / 1024;               // 1 KB copy instructions per chunk, dealt round the waves
+    static constexpr int kPiecesPerWave = (kPieces + WAVES - 1) / WAVES;
+};
+
+template <typename FMT, int NB, int SPLIT, bool RAW, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void iq_stream_exact_kernel(
+    const ActRows act, const uint8_t* __restrict__ w, void* __restrict__ y, int y_dtype, int n, int chunks) {
+    using L = ExactLayout<FMT, NB, SPLIT, WAVES>;
+    extern __shared__ __align__(16) unsigned char smem[];
+    const StagedX sx = carve_staged_x(smem, L::kKpad);
+    float* partial = reinterpret_cast<float*>(smem + L::kPartialOff);
+    const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_byte_ptr)smem));
+
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63;
+    const int col = lane & 15, ks = lane >> 4;
+    const unsigned char* tables = FMT::lane_tables(smem + L::kTableOff, lane);
+    const int tile_in_chunk = wave / SPLIT, part = wave % SPLIT;
+    y = static_cast<unsigned char*>(y) + static_cast<size_t>(blockIdx.y) * n * (y_dtype == PLLM_F32 ? 4 : 2);   // this activation row's outputs
+
+    const uint32_t piece_off = wave * 1024 + lane * 16;
+    // chunk c covers rows [first_row(c), first_row(c) + kChunkRows); all but the last start at c * kChunkRows
+    auto first_row = [&](int c) { return min(c * L::kChunkRows, n - L::kChunkRows); };
+    // whole 1 KB pieces wave, wave + WAVES, ... of a chunk, then the last, shorter piece (scalar bases and targets, one lane offset)
+    constexpr int kWhole = L::kChunkBytes / 1024, kTail = L::kChunkBytes % 1024;
+    auto request = [&](int c, int buf) {
+        const uint8_t* src = w + static_cast<size_t>(first_row(c)) * L::kRowBytes;
+        const uint32_t dst = lds0 + L::kChunkOff + buf * L::kChunkStride + wave * 1024;
+#pragma unroll
+        for (int i = 0; i * WAVES < kWhole; ++i)
+            if ((i + 1) * WAVES <= kWhole || wave + i * WAVES < kWhole) lds_dma16_at(src + i * (WAVES * 1024), piece_off, dst + i * (WAVES * 1024));
+        if constexpr (kTail > 0)
+            if (wave == kWhole % WAVES && lane * 16 < kTail)
+                lds_dma16_at(src + (kWhole / WAVES) * (WAVES * 1024), piece_off, dst + (kWhole / WAVES) * (WAVES * 1024));
+    };
+    // sums of the waves that share a tile, in wave order; rows below `skip` belong to the chunk before
+    auto sums_out = [&](int set, int row0, int skip) {
+        if constexpr (SPLIT > 1) {
+            if (tid < L::kChunkRows && tid >= skip) {
+                const float* ps = partial + set * (WAVES * 16) + (tid / kRowsPerTile) * (SPLIT * 16) + tid % kRowsPerTile;
+                float total = 0.0f;
+#pragma unroll
+                for (int v = 0; v < SPLIT; ++v) total += ps[v * 16];
+                store_plain(y, y_dtype, static_cast<size_t>(row0 + tid), total);
+            }
+        }
+    };
+
+    // activation image, codebooks and the first chunk: all in flight together
+    if constexpr (!RAW) dma_share<WAVES>(act.image + static_cast<size_t>(blockIdx.y) * act.stride, lds0, L::kImageBytes, wave, lane);
+    if constexpr (FMT::kCopies == 1) FMT::template dma_tables<WAVES>(lds0 + L::kTableOff, wave, lane);
+    if (tid < 4) reinterpret_cast<uint32_t*>(smem + L::kZeroOff)[tid] = 0;
+    AMap<FMT::kSlots> am;
+    FMT::a_map(am, col, ks, L::kKpad, L::kZeroOff);
+    int c = blockIdx.x;
+    request(c, 0);
+    if constexpr (FMT::kCopies > 1) FMT::stage_replicated(smem + L::kTableOff, tid, 64 * WAVES);   // ordinary stores; the loop's first barrier covers them
+    if constexpr (RAW)                       // raw activation row: quantized once per workgroup while the first chunk is on its way
+        quantize_row_to_lds(smem, act.x, act.x_dtype, static_cast<size_t>(blockIdx.y) * act.k, act.k, L::kKpad, RowNorm{act.gamma, act.eps, act.round_f16});
+
+    constexpr bool kHold = NB <= FMT::kHoldBlocks;
+    typename FMT::Held held[kHold ? NB : 1];
+    wait_vm<0>();                            // this wave's pieces of the first chunk, of the image and of the tables have landed ...
+    __syncthreads();                         // ... and everybody else's
+    if constexpr (kHold) {
+#pragma unroll
+        for (int i = 0; i < NB; ++i) FMT::hold(held[i], ks, part + i * SPLIT, smem, am, sx);
+    }
+    int buf = 0, set = 0;
+    const int row_off = (tile_in_chunk * kRowsPerTile + col) * L::kRowBytes + part * FMT::kBlockBytes;
+    while (true) {
+        const int cn = c + gridDim.x;
+        if (cn < chunks) request(cn, buf ^ 1);   // the other buffer is free: everybody has passed the barrier behind its last use
+
+        const unsigned char* chunk = smem + L::kChunkOff + buf * L::kChunkStride;
+        float acc = 0.0f;
+#pragma unroll
+        for (int i = 0; i < NB; ++i) {
+            typename FMT::Regs regs;
+            FMT::load_lds(regs, chunk, row_off + i * SPLIT * FMT::kBlockBytes, ks);
+            if constexpr (kHold) acc += FMT::block_held(regs, ks, part + i * SPLIT, held[i], smem, am, tables);
+            else acc += FMT::block(regs, ks, part + i * SPLIT, smem, am, sx, tables);
+            __builtin_amdgcn_sched_barrier(0);                               // one block after the other: interleaved they do not fit the registers
+        }
+        acc = quad_rows_sum(acc);
+        const int row0 = first_row(c), skip = c * L::kChunkRows - row0;
+        if constexpr (SPLIT == 1) {
+            const int r = tile_in_chunk * kRowsPerTile + col;
+            if (ks == 0 && r >= skip) store_plain(y, y_dtype, static_cast<size_t>(row0 + r), acc);
+        } else if (ks == 0) {
+            partial[set * (WAVES * 16) + wave * 16 + col] = acc;
+        }
+        wait_vm<0>();                        // this wave's pieces of the next chunk have landed ...
+        __syncthreads();                     // ... and everybody else's; everybody has left this chunk, whose sums are complete
+        sums_out(set, row0, skip);
+        if (cn >= chunks) break;
+        c = cn; buf ^= 1; set ^= 1;
+    }
 }
 
-template <typename FMT, int NB, bool RAW>
-int launch_stream_raw(const ActRows& act, const uint8_t* w, void* y, int y_dtype,
-                      int rows, int n, int bpr, int split, hipStream_t stream) {
-    auto kern = iq_stream_matvec_kernel<FMT, NB, RAW>;
-    const int tiles_per_chunk = kWaves / split;
-    const int chunk_bytes = tiles_per_chunk * kRowsPerTile * bpr * FMT::kBlockBytes;
-    const size_t head = staged_x_bytes(bpr * 256) + 16 + FMT::kTableBytes + kWaves * kRowsPerTile * sizeof(float);
-    const int chunk_off = static_cast<int>((head + 1023) & ~static_cast<size_t>(1023));
-    const int chunk_stride = chunk_bytes + 16;                               // shares are read as aligned dwords: a few bytes past the end
-    const size_t smem = static_cast<size_t>(chunk_off) + 2 * chunk_stride;
-    if (smem > 160 * 1024) return PLLM_ERR_UNSUPPORTED;
-    static SmemGrant granted;
-    if (!grant_dynamic_smem(reinterpret_cast<const void*>(kern), smem, granted)) return PLLM_ERR_UNSUPPORTED;
-    // resident workgroups per compute unit for this LDS size: asked once per size (the query costs microseconds of host time)
-    static size_t occ_smem = ~static_cast<size_t>(0);
-    static int occ_per_cu = 1;
-    if (smem != occ_smem) {
-        int q = 0;
-        occ_per_cu = (hipOccupancyMaxActiveBlocksPerMultiprocessor(&q, kern, 64 * kWaves, smem) == hipSuccess && q >= 1) ? q : 1;
-        occ_smem = smem;
+template <typename FMT, int NB, int SPLIT, int WAVES>
+int launch_exact(const ActRows& act, const uint8_t* w, void* y, int y_dtype, int rows, int n, hipStream_t stream) {
+    using L = ExactLayout<FMT, NB, SPLIT, WAVES>;
+    static_assert(L::kSmem <= kLdsBytes, "does not fit the LDS");
+    const void* kern = act.x ? reinterpret_cast<const void*>(iq_stream_exact_kernel<FMT, NB, SPLIT, true, WAVES>)
+                             : reinterpret_cast<const void*>(iq_stream_exact_kernel<FMT, NB, SPLIT, false, WAVES>);
+    static SmemGrant granted[2];
+    if (!grant_dynamic_smem(kern, L::kSmem, granted[act.x ? 1 : 0])) return PLLM_ERR_UNSUPPORTED;
+    const int chunks = (n + L::kChunkRows - 1) / L::kChunkRows;
+    const int resident = (kLdsBytes / L::kSmem) * compute_units();           // the LDS is what limits residency here
+    int grid = chunks;
+    if (chunks > resident) {
+        const int rounds = (chunks + resident - 1) / resident;
+        grid = (chunks + rounds - 1) / rounds;
     }
-    const int per_cu = occ_per_cu;
+    if (act.x) hipLaunchKernelGGL((iq_stream_exact_kernel<FMT, NB, SPLIT, true, WAVES>), dim3(grid, rows), dim3(64 * WAVES), L::kSmem, stream, act, w, y, y_dtype, n, chunks);
+    else hipLaunchKernelGGL((iq_stream_exact_kernel<FMT, NB, SPLIT, false, WAVES>), dim3(grid, rows), dim3(64 * WAVES), L::kSmem, stream, act, w, y, y_dtype, n, chunks);
+    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+}
+
+// the exact form for the row lengths it is built for; PLLM_ERR_UNSUPPORTED: take the general one
+template <typename FMT>
+int launch_exact_for(const ActRows& act, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream) {
+    if (n % kRowsPerTile != 0 || (reinterpret_cast<uintptr_t>(w) & 15u) || (y_dtype & kAccumulateInto)) return PLLM_ERR_UNSUPPORTED;
+#define PLLM_EXACT(F, NB, SPLIT, WAVES) \
+    if (bpr == NB * SPLIT && n >= ExactLayout<F, NB, SPLIT, WAVES>::kChunkRows) return launch_exact<F, NB, SPLIT, WAVES>(act, w, y, y_dtype, rows, n, stream)
+    if constexpr (std::is_same<FMT, IQ2XXSm>::value) {
+        PLLM_EXACT(IQ2XXSmT<16>, 3, 4, 16);        // K = 3072
+    } else if constexpr (std::is_same<FMT, IQ1Mm>::value) {
+        PLLM_EXACT(IQ1Mm, 3, 2, 8);                // K = 1536
+    }
+#undef PLLM_EXACT
+    return PLLM_ERR_UNSUPPORTED;
+}
+
+// What a streamed launch looks like: waves per workgroup, waves per tile, LDS layout.  split == 0: the streamed form does not apply.
+struct StreamPlan { int waves, split, chunk_off, chunk_stride; size_t smem; };
+
+template <typename FMT>
+StreamPlan stream_plan(const uint8_t* w, int n, int bpr, int waves, int chunk_budget) {
+    StreamPlan p{waves, 0, 0, 0, 0};
+    if (n % kRowsPerTile != 0 || (reinterpret_cast<uintptr_t>(w) & 15u)) return p;
+    const int tile_bytes = kRowsPerTile * bpr * FMT::kBlockBytes;
+    const size_t head = staged_x_bytes(bpr * 256) + 16 + FMT::kTableBytes + waves * kRowsPerTile * sizeof(float);
+    p.chunk_off = static_cast<int>((head + 1023) & ~static_cast<size_t>(1023));
+    if (chunk_budget <= 0) chunk_budget = (kLdsBytes - p.chunk_off) / 2 - 16;
+    // the most waves per tile first (smallest chunk) that leaves every wave at least two blocks
+    for (int split = waves; split >= 1; split /= 2)
+        if ((split == 1 || bpr >= 2 * split) && (waves / split) * tile_bytes <= chunk_budget) { p.split = split; break; }
+    if (!p.split) return p;
+    p.chunk_stride = (waves / p.split) * tile_bytes + 16;                    // shares are read as aligned dwords: a few bytes past the end
+    p.smem = static_cast<size_t>(p.chunk_off) + 2 * p.chunk_stride;
+    if (p.smem > kLdsBytes) p.split = 0;
+    return p;
+}
+
+template <typename FMT, int NB, bool RAW, int WAVES>
+int launch_stream_raw(const ActRows& act, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, const StreamPlan& p, hipStream_t stream) {
+    auto kern = iq_stream_matvec_kernel<FMT, NB, RAW, WAVES>;
+    const int tiles_per_chunk = WAVES / p.split;
+    static SmemGrant granted;
+    if (!grant_dynamic_smem(reinterpret_cast<const void*>(kern), p.smem, granted)) return PLLM_ERR_UNSUPPORTED;
+    // resident workgroups per compute unit for this LDS size: asked once per size (the query costs microseconds of host time)
+    static std::atomic<size_t> occ_smem{~static_cast<size_t>(0)};
+    static std::atomic<int> occ_per_cu{1};
+    if (p.smem != occ_smem.load(std::memory_order_acquire)) {
+        int q = 0;
+        occ_per_cu.store((hipOccupancyMaxActiveBlocksPerMultiprocessor(&q, kern, 64 * WAVES, p.smem) == hipSuccess && q >= 1) ? q : 1, std::memory_order_relaxed);
+        occ_smem.store(p.smem, std::memory_order_release);
+    }
+    const int per_cu = occ_per_cu.load(std::memory_order_relaxed);
     const int chunks = (n / kRowsPerTile + tiles_per_chunk - 1) / tiles_per_chunk;
     const int resident = per_cu * compute_units();
     int grid = chunks;
@@ -278,24 +446,23 @@ int launch_stream_raw(const ActRows& act, const uint8_t* w, void* y, int y_dtype
         const int rounds = (chunks + resident - 1) / resident;
         grid = (chunks + rounds - 1) / rounds;
     }
-    hipLaunchKernelGGL(kern, dim3(grid, rows), dim3(64 * kWaves), smem, stream, act, w, y, y_dtype, n, bpr, split, chunks,
-                       chunk_off, chunk_stride);
+    hipLaunchKernelGGL(kern, dim3(grid, rows), dim3(64 * WAVES), p.smem, stream, act, w, y, y_dtype, n, bpr, p.split, chunks,
+                       p.chunk_off, p.chunk_stride);
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 
-template <typename FMT, int NB>
-int launch_stream_nb(const ActRows& act, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, int split, hipStream_t stream) {
-    return act.x ? launch_stream_raw<FMT, NB, true>(act, w, y, y_dtype, rows, n, bpr, split, stream)
-                 : launch_stream_raw<FMT, NB, false>(act, w, y, y_dtype, rows, n, bpr, split, stream);
+template <typename FMT, int NB, int WAVES>
+int launch_stream_nb(const ActRows& act, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, const StreamPlan& p, hipStream_t stream) {
+    return act.x ? launch_stream_raw<FMT, NB, true, WAVES>(act, w, y, y_dtype, rows, n, bpr, p, stream)
+                 : launch_stream_raw<FMT, NB, false, WAVES>(act, w, y, y_dtype, rows, n, bpr, p, stream);
 }
 
-template <typename FMT>
-int launch_stream(const ActRows& act, const uint8_t* w, void* y, int y_dtype,
-                  int rows, int n, int bpr, int split, hipStream_t stream) {
-    const int per_wave = (bpr + split - 1) / split;                          // block indices a wave meets
-    if constexpr (FMT::kHoldBlocks >= 2) if (per_wave <= 2) return launch_stream_nb<FMT, 2>(act, w, y, y_dtype, rows, n, bpr, split, stream);
-    if constexpr (FMT::kHoldBlocks >= 3) if (per_wave == 3) return launch_stream_nb<FMT, 3>(act, w, y, y_dtype, rows, n, bpr, split, stream);
-    return launch_stream_nb<FMT, 0>(act, w, y, y_dtype, rows, n, bpr, split, stream);
+template <typename FMT, int WAVES>
+int launch_stream(const ActRows& act, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, const StreamPlan& p, hipStream_t stream) {
+    const int per_wave = (bpr + p.split - 1) / p.split;                      // block indices a wave meets
+    if constexpr (FMT::kHoldBlocks >= 2) if (per_wave <= 2) return launch_stream_nb<FMT, 2, WAVES>(act, w, y, y_dtype, rows, n, bpr, p, stream);
+    if constexpr (FMT::kHoldBlocks >= 3) if (per_wave == 3) return launch_stream_nb<FMT, 3, WAVES>(act, w, y, y_dtype, rows, n, bpr, p, stream);
+    return launch_stream_nb<FMT, 0, WAVES>(act, w, y, y_dtype, rows, n, bpr, p, stream);
 }
 
 template <typename FMT>
@@ -305,8 +472,17 @@ int launch_fmt(const ActRows& act, const WeightRoute& route, const uint8_t* w, v
     // where shape and alignment allow, else one short workgroup per tile; routed calls and several projections in one launch
     // always take the latter
     if constexpr (FMT::kStreamed)
-        if (!routed(route) && !act.row_token && !act.x_broadcast && route.extra == 0)
-            if (const int split = stream_split<FMT>(w, n, bpr)) return launch_stream<FMT>(act, w, y, y_dtype, rows, n, bpr, split, stream);
+        if (!routed(route) && !act.row_token && !act.x_broadcast && route.extra == 0) {
+            const int exact = launch_exact_for<FMT>(act, w, y, y_dtype, rows, n, bpr, stream);
+            if (exact != PLLM_ERR_UNSUPPORTED) return exact;
+            if constexpr (std::is_same<FMT, IQ2XXSm>::value) {
+                // sixteen table copies (conflict-free lookups) around one 16-wave workgroup per compute unit, where the LDS holds it
+                const StreamPlan wide = stream_plan<IQ2XXSmT<16>>(w, n, bpr, 16, 0);
+                if (wide.split) return launch_stream<IQ2XXSmT<16>, 16>(act, w, y, y_dtype, rows, n, bpr, wide, stream);
+            }
+            const StreamPlan p = stream_plan<FMT>(w, n, bpr, kWaves, kChunkBudget);
+            if (p.split) return launch_stream<FMT, kWaves>(act, w, y, y_dtype, rows, n, bpr, p, stream);
+        }
     return launch_tiles<FMT>(act, route, w, y, y_dtype, rows, n, bpr, stream);
 }
 

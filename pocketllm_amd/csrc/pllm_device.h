@@ -57,6 +57,17 @@ __device__ __forceinline__ float butterfly_peer(float v) {
     else return __shfl_xor(v, OFF, 64);
 }
 
+// v summed over the four lanes (l % 16) + {0, 16, 32, 48}, in every lane: the two wide steps of a butterfly through
+// gfx950's row swaps (v_permlane16_swap exchanges odd rows of one operand with even rows of the other, v_permlane32_swap
+// the upper half with the lower half), one vector instruction each and no LDS crossbar.
+__device__ __forceinline__ float quad_rows_sum(float v) {
+    const uint32_t b = __float_as_uint(v);
+    const auto h = __builtin_amdgcn_permlane32_swap(b, b, false, false);      // {v of the lower half, v of the upper half} in both halves
+    const uint32_t s = __float_as_uint(__uint_as_float(h[0]) + __uint_as_float(h[1]));
+    const auto r = __builtin_amdgcn_permlane16_swap(s, s, false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 // Sum / maximum over aligned groups of WIDTH lanes (WIDTH a power of two <= 64); every lane gets the result.
 template <int WIDTH>
 __device__ __forceinline__ float group_sum(float v) {
@@ -100,7 +111,7 @@ struct StagedX {
     const float* sum16;
 };
 
-__host__ __device__ inline size_t staged_x_bytes(int kpad) {
+__host__ __device__ constexpr size_t staged_x_bytes(int kpad) {
     return static_cast<size_t>(kpad) * 2 + static_cast<size_t>(kpad / 32) * 8 + static_cast<size_t>(kpad / 16) * 4;
 }
 
@@ -186,6 +197,13 @@ __device__ __forceinline__ void store_any(void* y, int y_dtype, size_t i, float 
         y_dtype &= ~0x100;
         v += load_any(y, y_dtype, i);
     }
+    if (y_dtype == PLLM_BF16) static_cast<bf16_t*>(y)[i] = from_float<bf16_t>(v);
+    else if (y_dtype == PLLM_F16) static_cast<f16_t*>(y)[i] = from_float<f16_t>(v);
+    else static_cast<float*>(y)[i] = v;
+}
+
+// the same for callers that never accumulate (y_dtype is one of the three plain codes)
+__device__ __forceinline__ void store_plain(void* y, int y_dtype, size_t i, float v) {
     if (y_dtype == PLLM_BF16) static_cast<bf16_t*>(y)[i] = from_float<bf16_t>(v);
     else if (y_dtype == PLLM_F16) static_cast<f16_t*>(y)[i] = from_float<f16_t>(v);
     else static_cast<float*>(y)[i] = v;

@@ -195,7 +195,11 @@ def _grid_for(type_name, dev):
 
 @pytest.mark.parametrize("type_name", ["iq2_xxs", "iq1_m"])
 @pytest.mark.parametrize("n,k,rows", [(16, 256, 1), (50, 768, 1), (1536, 3072, 1), (3072, 1536, 1), (40, 2048, 3), (7, 5120, 1), (21, 1000, 2),
-                                      (176, 768, 2), (208, 5120, 1), (64, 14336, 1)])
+                                      (176, 768, 2), (208, 5120, 1), (64, 14336, 1),
+                                      # rows of 12 and of 6 super-blocks (the streamed kernels built for those lengths): fewer rows than
+                                      # one chunk of 64, exactly one, and row counts whose last chunk is moved back over its predecessor
+                                      (48, 3072, 1), (64, 3072, 2), (80, 3072, 1), (1552, 3072, 2), (32, 1536, 1), (64, 1536, 1), (208, 1536, 2),
+                                      (3088, 1536, 1)])
 def test_iq_matvec_matches_oracle(mod, type_name, n, k, rows):
     rng = np.random.default_rng(500 + n + k)
     gen = C.random_iq2_xxs if type_name == "iq2_xxs" else C.random_iq1_m
