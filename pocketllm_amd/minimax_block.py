@@ -1,28 +1,29 @@
 """One MiniMax-M2 decoder block over the raw-block operators: the callers either side of the quantized matmul path.
 
 Host-side mirror of the reference's src/models/minimax_m2/architecture.py (RMSNorm 57-85, MiniMaxAttention 88-268,
-MiniMaxMoE 271-385, MiniMaxBlock 388-413): same class names, constructor arguments and call shapes, so that a runtime
-written against the reference composes these the same way.  What differs is what runs underneath:
+MiniMaxMoE 271-385, MiniMaxBlock 388-413, MiniMaxTransformer 417-472): same class names, constructor arguments and call
+shapes, so that a runtime written against the reference composes these the same way.  What differs is what runs underneath:
 
   * the projections are QuantizedGGUFLinear modules of this package (raw GGUF blocks, HIP kernels); q, k and v of a
     decode step leave in ONE launch (gguf_quant_gemm_multi_forward) when the three tensors share a format;
   * routing (gate matvec, sigmoid, bias, top-k, renormalisation) is one operator (moe_route) instead of five framework ops;
   * the experts run through gguf_moe_single_token_forward (one token) or moe_group_routes +
-    gguf_moe_prefill_grouped_forward (several tokens), any of the supported expert format pairs.
+    gguf_moe_prefill_grouped_forward (several tokens), any of the supported expert format pairs;
+  * a decode step folds both residual connections and both normalisations it can into the projections: the block's first
+    RMS normalisation runs inside the q / k / v launch, the output projection adds into the residual stream in its store.
 
-The attention core itself (rotary embedding, key/value cache, softmax) is not part of the quantized matmul path and stays
-framework code, as in the reference (architecture.py:158-266).  One GPU: no tensor-parallel reduction.  The native library
-is mandatory; nothing here falls back to a CPU path.
+The attention core itself (rotary phases, key/value store, softmax) is not part of the quantized matmul path; it lives in
+attention_core.py as plain framework arithmetic of this package's own (head-major cache, grouped matrix products, float32
+softmax).  One GPU: no tensor-parallel reduction.  The native library is mandatory; nothing here falls back to a CPU path.
 """
 from __future__ import annotations
 
-import math
 from dataclasses import dataclass
 
 import torch
-import torch.nn.functional as F
 
 from pocketllm_amd import codebooks
+from pocketllm_amd.attention_core import KeyValueCache, RotaryTable, grouped_query_attention
 from pocketllm_amd.cuda_loader import load_cuda_kernel
 from pocketllm_amd.quantized_ops import QuantizedGGUFLinear
 from pocketllm_amd.quantized_tensor import QuantizedGGUFTensor
@@ -60,8 +61,8 @@ class RMSNorm:
         self._cuda = _kernel()
 
     def __call__(self, x: torch.Tensor) -> torch.Tensor:
-        x_flat = x.reshape(-1, x.size(-1)).contiguous()
-        return self._cuda.fused_rms_norm_forward(x_flat, self.weight, self.eps).view(x.shape).to(self.out_dtype)
+        rows = x.contiguous().view(-1, x.size(-1))
+        return self._cuda.fused_rms_norm_forward(rows, self.weight, self.eps, out_dtype=self.out_dtype).view(x.shape)
 
 
 @dataclass
@@ -97,37 +98,30 @@ class MiniMaxMoE:
         return self._cuda.moe_route(x_flat, self.gate_weight, self.gate_bias, int(self.args.top_k))
 
     def __call__(self, x: torch.Tensor) -> torch.Tensor:
-        original_shape = x.shape
-        x_flat = x.reshape(-1, original_shape[-1]).contiguous()
-        indices, weights = self.route(x_flat)
-        e = self.experts
-        if x_flat.size(0) == 1:
-            slots = indices[0]
-            local = (slots >= self.expert_start) & (slots < self.expert_start + self.expert_count)
-            if self.expert_start == 0 and self.expert_count >= int(self.args.n_routed_experts):
-                local_slots, local_weights = slots, weights[0]                 # every expert is resident: nothing to filter
-            else:
-                local_slots, local_weights = slots[local] - self.expert_start, weights[0][local]
-            if local_slots.numel() == 0:
-                y = torch.zeros((1, self.args.dim), device=x.device, dtype=torch.float32)
-            else:
-                y = self._cuda.gguf_moe_single_token_forward(x_flat, local_slots.contiguous(), local_weights.contiguous(),
-                                                             e.w1.blocks, e.w3.blocks, e.w2.blocks, 0.0)
+        tokens = x.reshape(-1, x.size(-1)).contiguous()
+        chosen, gate_w = self.route(tokens)
+        w = self.experts
+        nothing = lambda: tokens.new_zeros((tokens.size(0), self.args.dim), dtype=torch.float32)   # no route lands on a resident expert
+        if tokens.size(0) == 1:
+            ids, ws = chosen[0], gate_w[0]
+            if not (self.expert_start == 0 and self.expert_count >= int(self.args.n_routed_experts)):   # a slice of the experts is resident
+                here = (ids >= self.expert_start) & (ids < self.expert_start + self.expert_count)
+                ids, ws = ids[here] - self.expert_start, ws[here]
+            out = nothing() if ids.numel() == 0 else self._cuda.gguf_moe_single_token_forward(
+                tokens, ids.contiguous(), ws.contiguous(), w.w1.blocks, w.w3.blocks, w.w2.blocks, 0.0)
         else:
-            _ids, route_tokens, route_weights, seg = self._cuda.moe_group_routes(indices, weights, self.expert_start, self.expert_count)
-            if int(route_tokens.numel()) == 0:
-                y = torch.zeros((x_flat.size(0), self.args.dim), device=x.device, dtype=torch.float32)
-            else:
-                y = self._cuda.gguf_moe_prefill_grouped_forward(
-                    x_flat, route_tokens, route_weights, seg, e.w1.blocks, e.w3.blocks, e.w2.blocks,
-                    int(e.w1.row_elems), int(e.w1.type_id), int(e.w3.row_elems), int(e.w3.type_id), int(e.w2.row_elems), int(e.w2.type_id),
-                    self._grid, 0.0)
-        return y.reshape(original_shape).to(self.dtype)
+            _, route_tokens, route_weights, seg = self._cuda.moe_group_routes(chosen, gate_w, self.expert_start, self.expert_count)
+            out = nothing() if route_tokens.numel() == 0 else self._cuda.gguf_moe_prefill_grouped_forward(
+                tokens, route_tokens, route_weights, seg, w.w1.blocks, w.w3.blocks, w.w2.blocks,
+                int(w.w1.row_elems), int(w.w1.type_id), int(w.w3.row_elems), int(w.w3.type_id), int(w.w2.row_elems), int(w.w2.type_id), self._grid, 0.0)
+        return out.view(x.shape).to(self.dtype)
 
 
 class MiniMaxAttention:
-    """architecture.py:88-268: q / k / v projections, per-projection RMS normalisation of q and k, half-split rotary embedding
-    over the first rope_dim values of every head, key/value cache, scaled dot-product attention, output projection."""
+    """The attention half of a block (reference: architecture.py:88-268): q / k / v projections, RMS normalisation of q and k
+    over the whole projection width, rotary phases on the first rope_dim values of every head, key/value store, grouped-query
+    softmax attention, output projection.  `input_norm`, when given, is the block's normalisation of the residual stream: decode
+    steps then run it inside the q / k / v launch."""
 
     def __init__(self, args: MiniMaxM2Args, q_proj: QuantizedGGUFLinear, k_proj: QuantizedGGUFLinear, v_proj: QuantizedGGUFLinear,
                  o_proj: QuantizedGGUFLinear, q_norm: RMSNorm, k_norm: RMSNorm, *, dtype: torch.dtype = torch.float16):
@@ -135,83 +129,48 @@ class MiniMaxAttention:
         self.q_proj, self.k_proj, self.v_proj, self.o_proj = q_proj, k_proj, v_proj, o_proj
         self.q_norm, self.k_norm = q_norm, k_norm
         self.dtype = dtype
-        self.cache_k: torch.Tensor | None = None
-        self.cache_v: torch.Tensor | None = None
         self._cuda = _kernel()
-        tensors = (q_proj.tensor, k_proj.tensor, v_proj.tensor)
-        self._one_launch = len({int(t.type_id) for t in tensors}) == 1 and len({int(t.blocks.size(1)) for t in tensors}) == 1 \
-            and int(tensors[0].type_id) != 1
+        dev = q_proj.tensor.blocks.device
+        self.rotary = RotaryTable(args.rope_dim, args.rope_base, dev, head_dim=args.head_dim)
+        self.store = KeyValueCache(args.n_kv_heads, args.head_dim, dev, dtype)
+        qkv = (q_proj.tensor, k_proj.tensor, v_proj.tensor)
+        # one launch for the three projections needs one format (not Q2_K) and one row length
+        self._fused_qkv = len({(int(t.type_id), int(t.blocks.size(1))) for t in qkv}) == 1 and int(qkv[0].type_id) != 1
 
     def reset_cache(self, batch_size: int, max_seq_len: int) -> None:
-        dev = self.q_proj.tensor.blocks.device
-        shape = (batch_size, max_seq_len, self.args.n_kv_heads, self.args.head_dim)
-        self.cache_k = torch.zeros(shape, device=dev, dtype=self.dtype)
-        self.cache_v = torch.zeros(shape, device=dev, dtype=self.dtype)
+        self.store.allocate(batch_size, max_seq_len)
+        self.rotary.reserve(max_seq_len)
 
-    def _apply_rope(self, x: torch.Tensor, start_pos: int) -> torch.Tensor:
-        rope_dim = int(self.args.rope_dim)
-        if rope_dim <= 0:
-            return x
-        half = rope_dim // 2
-        positions = torch.arange(start_pos, start_pos + x.size(1), device=x.device, dtype=torch.float32)
-        j = torch.arange(half, device=x.device, dtype=torch.float32)
-        inv = torch.pow(torch.full_like(j, float(self.args.rope_base)), -(2.0 * j) / float(rope_dim))
-        freqs = positions[:, None] * inv[None, :]
-        sin = torch.sin(freqs).to(x.dtype)[None, :, None, :]
-        cos = torch.cos(freqs).to(x.dtype)[None, :, None, :]
-        x1, x2 = x[..., :half], x[..., half:rope_dim]
-        parts = [x1 * cos - x2 * sin, x1 * sin + x2 * cos]
-        if rope_dim < x.size(-1):
-            parts.append(x[..., rope_dim:])
-        return torch.cat(parts, dim=-1)
-
-    def _qkv(self, x: torch.Tensor):
+    def project_qkv(self, x: torch.Tensor, input_norm: RMSNorm | None = None):
+        """q, k, v of x [batch, steps, dim] (of input_norm(x) when a normalisation is handed in)."""
         rows = x.numel() // x.size(-1)
-        if self._one_launch and rows <= 4:                  # decode: the three projections of one activation row as one launch
+        if self._fused_qkv and rows <= 4:
             t = self.q_proj.tensor
-            q, k, v = self._cuda.gguf_quant_gemm_multi_forward(
-                x.contiguous(), (self.q_proj.tensor.blocks, self.k_proj.tensor.blocks, self.v_proj.tensor.blocks), int(t.row_elems),
-                int(t.type_id), self.q_proj._grid, out_dtype=self.dtype)
-            return q, k, v
-        return self.q_proj(x), self.k_proj(x), self.v_proj(x)
+            return self._cuda.gguf_quant_gemm_multi_forward(
+                x.contiguous(), [p.tensor.blocks for p in (self.q_proj, self.k_proj, self.v_proj)], int(t.row_elems), int(t.type_id),
+                self.q_proj._grid, norm_weight=None if input_norm is None else input_norm.weight,
+                eps=0.0 if input_norm is None else input_norm.eps, out_dtype=self.dtype)
+        h = x if input_norm is None else input_norm(x)
+        return self.q_proj(h), self.k_proj(h), self.v_proj(h)
+
+    def context(self, x: torch.Tensor, start_pos: int, input_norm: RMSNorm | None = None) -> torch.Tensor:
+        """Everything up to the output projection: [batch, steps, heads * head_dim]."""
+        a = self.args
+        batch, steps = x.size(0), x.size(1)
+        q, k, v = self.project_qkv(x, input_norm)
+        q = self.rotary.rotate(self.q_norm(q).view(batch, steps, a.n_heads, a.head_dim), start_pos)
+        k = self.rotary.rotate(self.k_norm(k).view(batch, steps, a.n_kv_heads, a.head_dim), start_pos)
+        self.store.write(k, v.view(batch, steps, a.n_kv_heads, a.head_dim).to(self.dtype), start_pos)
+        keys, values = self.store.read(batch, start_pos + steps)
+        return grouped_query_attention(q.to(self.dtype), keys, values, start_pos)
 
     def __call__(self, x: torch.Tensor, start_pos: int) -> torch.Tensor:
-        bsz, seqlen, _ = x.shape
-        end_pos = int(start_pos) + int(seqlen)
-        if self.cache_k is None or self.cache_k.size(0) < bsz or self.cache_k.size(1) < end_pos:
-            self.reset_cache(bsz, max(end_pos, 256))
-        a = self.args
-        q_raw, k_raw, v_raw = self._qkv(x)
-        q = self.q_norm(q_raw).view(bsz, seqlen, a.n_heads, a.head_dim)
-        k = self.k_norm(k_raw).view(bsz, seqlen, a.n_kv_heads, a.head_dim)
-        v = v_raw.view(bsz, seqlen, a.n_kv_heads, a.head_dim).to(self.dtype)
-        q = self._apply_rope(q, int(start_pos))
-        k = self._apply_rope(k, int(start_pos))
-        self.cache_k[:bsz, start_pos:end_pos].copy_(k)
-        self.cache_v[:bsz, start_pos:end_pos].copy_(v)
-        q_t = q.transpose(1, 2).contiguous()
-        k_t = self.cache_k[:bsz, :end_pos].transpose(1, 2).contiguous()
-        v_t = self.cache_v[:bsz, :end_pos].transpose(1, 2).contiguous()
-        repeat = a.n_heads // a.n_kv_heads
-        if repeat != 1:
-            k_t = k_t.repeat_interleave(repeat, dim=1)
-            v_t = v_t.repeat_interleave(repeat, dim=1)
-        mask, causal = None, False
-        if seqlen > 1 and int(start_pos) == 0:
-            causal = True
-        elif seqlen > 1:
-            q_pos = torch.arange(start_pos, end_pos, device=x.device)
-            k_pos = torch.arange(0, end_pos, device=x.device)
-            mask = torch.zeros((seqlen, end_pos), device=x.device, dtype=q_t.dtype)
-            mask.masked_fill_(~(k_pos[None, :] <= q_pos[:, None]), float("-inf"))
-        out = F.scaled_dot_product_attention(q_t.to(self.dtype), k_t.to(self.dtype), v_t.to(self.dtype), attn_mask=mask, dropout_p=0.0,
-                                             is_causal=causal, scale=1.0 / math.sqrt(float(a.head_dim)))
-        out = out.transpose(1, 2).contiguous().view(bsz, seqlen, a.n_heads * a.head_dim)
-        return self.o_proj(out)
+        return self.o_proj(self.context(x, int(start_pos)))
 
 
 class MiniMaxBlock:
-    """architecture.py:388-413: x + attention(norm(x)), then x + experts(norm(x)), each sum rounded to the model's dtype."""
+    """One decoder layer (reference: architecture.py:388-413): attention and routed experts, each behind an RMS normalisation
+    and added back to the residual stream, which is kept in the model's dtype."""
 
     def __init__(self, args: MiniMaxM2Args, attn_norm_weight: torch.Tensor, ffn_norm_weight: torch.Tensor, attention: MiniMaxAttention,
                  moe: MiniMaxMoE, *, dtype: torch.dtype = torch.float16):
@@ -221,11 +180,62 @@ class MiniMaxBlock:
         self.attention = attention
         self.moe = moe
         self.dtype = dtype
+        self._cuda = _kernel()
 
     def reset_cache(self, batch_size: int, max_seq_len: int) -> None:
         self.attention.reset_cache(batch_size, max_seq_len)
 
     def __call__(self, x: torch.Tensor, start_pos: int) -> torch.Tensor:
-        x = (x + self.attention(self.attn_norm(x), start_pos)).to(self.dtype)
-        x = (x + self.moe(self.ffn_norm(x))).to(self.dtype)
-        return x
+        start_pos = int(start_pos)
+        stream = x.to(self.dtype).contiguous()
+        if stream is x:
+            stream = x.clone()                                                 # the caller's tensor is not written
+        rows = stream.numel() // stream.size(-1)
+        o = self.attention.o_proj
+        if rows <= 4:
+            # decode: normalisation inside the q / k / v launch, residual added in the output projection's store
+            ctx = self.attention.context(stream, start_pos, input_norm=self.attn_norm)
+            self._cuda.gguf_quant_gemm_accumulate_forward(ctx.contiguous(), o.tensor.blocks, int(o.tensor.row_elems), int(o.tensor.type_id), o._grid,
+                                                          stream)
+        else:
+            stream += self.attention(self.attn_norm(stream), start_pos)
+        stream += self.moe(self.ffn_norm(stream))
+        return stream
+
+
+class MiniMaxTransformer:
+    """The layer stack (reference: architecture.py:417-472): token embedding from raw blocks, the blocks, the final
+    normalisation and the vocabulary projection of the last position (or of all).  One GPU, so logits are whole rows."""
+
+    def __init__(self, args: MiniMaxM2Args, embedding, layers: list[MiniMaxBlock], final_norm_weight: torch.Tensor, lm_head: QuantizedGGUFLinear,
+                 *, device: torch.device, dtype: torch.dtype = torch.float16):
+        self.args = args
+        self.embedding = embedding
+        self.layers = list(layers)
+        self.final_norm = RMSNorm(final_norm_weight, args.norm_eps, out_dtype=dtype)
+        self.lm_head = lm_head
+        self.device = device
+        self.dtype = dtype
+
+    def reset_cache(self, batch_size: int, max_seq_len: int) -> None:
+        for layer in self.layers:
+            layer.reset_cache(batch_size, max_seq_len)
+
+    @torch.inference_mode()
+    def forward(self, tokens: torch.Tensor, start_pos: int = 0, *, return_next_token: bool = False, keep_all_positions: bool = False):
+        """tokens [batch, steps] (or [steps]) at positions start_pos ..; float32 logits [batch, 1 or steps, vocabulary], or the
+        arg-max token ids when return_next_token is set."""
+        ids = tokens.to(self.device)
+        ids = ids.view(1, -1) if ids.dim() == 1 else ids
+        hidden = self.embedding(ids).to(self.dtype)
+        for layer in self.layers:
+            hidden = layer(hidden, int(start_pos))
+        if not keep_all_positions:
+            hidden = hidden[:, -1:, :]
+        logits = self.lm_head(self.final_norm(hidden.contiguous())).float()
+        if return_next_token:
+            best = logits.argmax(dim=-1)
+            return best if keep_all_positions else best[:, -1]
+        return logits
+
+    __call__ = forward

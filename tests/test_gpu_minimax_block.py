@@ -9,8 +9,8 @@ import torch
 from oracle import gguf_oracle as O
 from pocketllm_amd import block_codec as C
 from pocketllm_amd.cuda_loader import load_cuda_kernel
-from pocketllm_amd.minimax_block import ExpertLayer, MiniMaxAttention, MiniMaxBlock, MiniMaxM2Args, MiniMaxMoE, RMSNorm
-from pocketllm_amd.quantized_ops import QuantizedGGUFLinear
+from pocketllm_amd.minimax_block import ExpertLayer, MiniMaxAttention, MiniMaxBlock, MiniMaxM2Args, MiniMaxMoE, MiniMaxTransformer, RMSNorm
+from pocketllm_amd.quantized_ops import QuantizedGGUFEmbedding, QuantizedGGUFLinear
 from pocketllm_amd.quantized_tensor import QuantizedGGUFTensor
 
 pytestmark = pytest.mark.gpu
@@ -102,3 +102,72 @@ def test_decoder_block_prefill_then_decode():
         want = oracle(x.float().cpu().numpy().astype(np.float64), start)
         assert got.shape == want.shape
         assert O.rel_l2(got, want) <= 1e-2, (start, O.rel_l2(got, want))
+
+
+def _small_layer(rng, a, seed_names):
+    """Weights of one layer as (device modules, oracle block)."""
+    shapes = {"q": (a.n_heads * a.head_dim, a.dim), "k": (a.n_kv_heads * a.head_dim, a.dim), "v": (a.n_kv_heads * a.head_dim, a.dim),
+              "o": (a.dim, a.n_heads * a.head_dim)}
+    blocks = {n: C.quantize_q5_k((rng.standard_normal(s) * (0.7 / np.sqrt(s[1]))).astype(np.float32)) for n, s in shapes.items()}
+    lin = {n: QuantizedGGUFLinear(QuantizedGGUFTensor.from_blocks(torch.from_numpy(b).to(DEV), "q5_k", shapes[n][1], source_name=f"{seed_names}.{n}"))
+           for n, b in blocks.items()}
+    norms = {n: rng.uniform(0.5, 1.5, size).astype(np.float32)
+             for n, size in (("attn", a.dim), ("ffn", a.dim), ("q", shapes["q"][0]), ("k", shapes["k"][0]))}
+    tn = {n: torch.from_numpy(v).to(DEV) for n, v in norms.items()}
+    gate = (rng.standard_normal((a.n_routed_experts, a.dim)) / np.sqrt(a.dim)).astype(np.float32)
+    bias = (rng.standard_normal(a.n_routed_experts) * 0.1).astype(np.float32)
+    w1 = C.random_iq2_xxs(rng, a.n_routed_experts, a.moe_inter_dim, a.dim // 256, d_range=(0.002, 0.006))
+    w3 = C.random_iq2_xxs(rng, a.n_routed_experts, a.moe_inter_dim, a.dim // 256, d_range=(0.002, 0.006))
+    w2 = C.random_iq1_m(rng, a.n_routed_experts, a.dim, a.moe_inter_dim // 256, d_range=(0.002, 0.006))
+    experts = ExpertLayer(*(QuantizedGGUFTensor.from_blocks(torch.from_numpy(b).to(DEV), name, k)
+                            for b, name, k in ((w1, "iq2_xxs", a.dim), (w3, "iq2_xxs", a.dim), (w2, "iq1_m", a.moe_inter_dim))))
+    moe = MiniMaxMoE(a, torch.from_numpy(gate).to(DEV), torch.from_numpy(bias).to(DEV), experts)
+    attn = MiniMaxAttention(a, lin["q"], lin["k"], lin["v"], lin["o"], RMSNorm(tn["q"], a.norm_eps), RMSNorm(tn["k"], a.norm_eps))
+    block = MiniMaxBlock(a, tn["attn"], tn["ffn"], attn, moe)
+    oracle = _OracleBlock(a, {n: O.dequant_rows(b, "q5_k", shapes[n][1]).astype(np.float64) for n, b in blocks.items()}, gate.astype(np.float64),
+                          bias.astype(np.float64), (w1, w3, w2), {n: v.astype(np.float64) for n, v in norms.items()})
+    return block, oracle
+
+
+def test_transformer_stack_prefill_then_decode():
+    """Embedding from raw blocks -> two blocks -> final normalisation -> vocabulary projection (architecture.py:417-472) against the
+    float64 chain of the same operators; the stack keeps its residual stream in fp16, which is what bounds the distance."""
+    assert load_cuda_kernel() is not None and torch.cuda.is_available()
+    rng = np.random.default_rng(33)
+    a = MiniMaxM2Args(dim=512, n_heads=4, n_kv_heads=2, head_dim=64, rope_dim=32, rope_base=10000.0, n_routed_experts=8, top_k=2,
+                      moe_inter_dim=256, norm_eps=1e-6)
+    vocab = 640
+    layers = [_small_layer(rng, a, f"blk.{i}") for i in range(2)]
+    emb_blocks = C.quantize_q4_k(rng.standard_normal((vocab, a.dim)).astype(np.float32))
+    head_blocks = C.quantize_q6_k((rng.standard_normal((vocab, a.dim)) / np.sqrt(a.dim)).astype(np.float32))
+    final = rng.uniform(0.5, 1.5, a.dim).astype(np.float32)
+    model = MiniMaxTransformer(
+        a, QuantizedGGUFEmbedding(QuantizedGGUFTensor.from_blocks(torch.from_numpy(emb_blocks).to(DEV), "q4_k", a.dim, source_name="token_embd")),
+        [blk for blk, _ in layers], torch.from_numpy(final).to(DEV),
+        QuantizedGGUFLinear(QuantizedGGUFTensor.from_blocks(torch.from_numpy(head_blocks).to(DEV), "q6_k", a.dim, source_name="output")),
+        device=torch.device(DEV))
+    model.reset_cache(1, 16)
+    emb = O.dequant_rows(emb_blocks, "q4_k", a.dim).astype(np.float64)
+    head = O.dequant_rows(head_blocks, "q6_k", a.dim).astype(np.float64)
+
+    def want_logits(ids, start, all_positions):
+        h = emb[ids]
+        for _, oracle in layers:
+            h = oracle(h, start)
+        h = O.rms_norm(h if all_positions else h[-1:], final.astype(np.float64), a.norm_eps)
+        return h @ head.T
+
+    prompt = rng.integers(0, vocab, size=5)
+    print("case transformer prefill 5 tokens", flush=True)
+    got = model(torch.from_numpy(prompt), 0, keep_all_positions=True).cpu().numpy()[0]
+    want = want_logits(prompt, 0, True)
+    assert got.shape == want.shape == (5, vocab)
+    assert O.rel_l2(got, want) <= 2e-2, O.rel_l2(got, want)
+    for step, tok in enumerate(rng.integers(0, vocab, size=2)):
+        print(f"case transformer decode step {step}", flush=True)
+        got = model(torch.tensor([[int(tok)]]), 5 + step).cpu().numpy()[0]
+        want = want_logits(np.array([tok]), 5 + step, False)
+        assert got.shape == want.shape == (1, vocab)
+        assert O.rel_l2(got, want) <= 2e-2, (step, O.rel_l2(got, want))
+    nxt = model(torch.tensor([[3]]), 7, return_next_token=True)
+    assert nxt.shape == (1,) and 0 <= int(nxt[0]) < vocab
