@@ -113,6 +113,11 @@ static bool quantizes_in_kernel(int type_id, int64_t rows, int64_t n, int64_t bp
     return pllm_gguf_block_bytes(type_id) != 0;
 }
 
+// Q4_K / Q5_K calls of 17 - 48 rows that the tile kernel would otherwise take
+static bool uses_rows64(int type_id, int64_t rows, int64_t n, int64_t bpr, const uint8_t* blocks) {
+    return gguf_uses_tile_gemm(type_id, rows, n, bpr) && pllm::k45_rows64_supports(type_id, static_cast<int>(rows), static_cast<int>(n), static_cast<int>(bpr), blocks);
+}
+
 }  // extern "C"
 
 namespace pllm {
@@ -166,6 +171,10 @@ int pllm_gguf_quant_gemm(const void* x, int x_dtype, const uint8_t* blocks, int 
         const int st16 = pllm::k45_rows16_matvec(x, x_dtype, blocks, type_id, y, y_dtype, static_cast<int>(rows), static_cast<int>(k), static_cast<int>(n), bpr, s);
         if (st16 != PLLM_ERR_UNSUPPORTED) return st16;
     }
+    // Q4_K / Q5_K, 17 - 48 rows: every block decoded once in registers and multiplied into all rows
+    if (uses_rows64(type_id, rows, n, blocks_per_row, blocks))
+        return pllm::k45_rows64_gemm(x, x_dtype, blocks, type_id, y, y_dtype, static_cast<int>(rows), static_cast<int>(k), static_cast<int>(n), bpr,
+                                     workspace, workspace_bytes, s);
     if (gguf_uses_tile_gemm(type_id, rows, n, blocks_per_row))
         return pllm::gemm_f16(x, x_dtype, blocks, type_id, y, y_dtype, static_cast<int>(rows), static_cast<int>(k), static_cast<int>(n), bpr,
                               workspace, workspace_bytes, s);
@@ -207,8 +216,13 @@ int pllm_gguf_quant_gemm_accumulate(const void* x, int x_dtype, const uint8_t* b
 size_t pllm_gguf_quant_gemm_workspace_bytes(int type_id, int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row) {
     (void)k;
     if (!fits_int(rows) || !fits_int(n) || !fits_int(blocks_per_row) || pllm_gguf_block_bytes(type_id) == 0) return 0;
-    if (gguf_uses_tile_gemm(type_id, rows, n, blocks_per_row))
-        return pllm::gemm_f16_workspace_bytes(static_cast<int>(rows), static_cast<int>(n), static_cast<int>(blocks_per_row));
+    if (gguf_uses_tile_gemm(type_id, rows, n, blocks_per_row)) {
+        // (the weights' alignment is not known here: room for either kernel)
+        const size_t tiles = pllm::gemm_f16_workspace_bytes(static_cast<int>(rows), static_cast<int>(n), static_cast<int>(blocks_per_row));
+        const size_t rows64 = uses_rows64(type_id, rows, n, blocks_per_row, nullptr)
+                                  ? pllm::k45_rows64_workspace_bytes(static_cast<int>(rows), static_cast<int>(n), static_cast<int>(blocks_per_row)) : 0;
+        return tiles > rows64 ? tiles : rows64;
+    }
     return pllm::act_image_256_bytes(static_cast<int>(blocks_per_row)) * static_cast<size_t>(rows);
 }
 

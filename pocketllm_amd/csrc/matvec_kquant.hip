@@ -1022,6 +1022,186 @@ int launch_rows16(const void* x, int x_dtype, const uint8_t* w, void* y, int y_d
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Q4_K / Q5_K, 17 - 48 activation rows (the kernel serves up to 128): the token counts between decode and the large tiles.  At these counts the call is bound by
+// streaming and decoding the weights once, so every super-block is fetched by one wave, decoded once in its registers and
+// multiplied into ALL activation rows; the rows reach the waves through LDS, staged once per workgroup and block.
+//   v_mfma_f32_16x16x32_f16: A = 16 activation rows x the 32 columns of a scale group (fp16 rows scaled per row by a power of two,
+//   as the tile kernel stages them: bf16 / fp16 inputs stay exact), B = 32 weights x 16 weight rows.
+// B carries sc_g * code as an exact fp16 integer (at most 63 * 31 = 1953 < 2048): the code enters as 1024 + code (bits
+// 0x6400 | code, one byte permute per two codes) and one packed fused multiply-add, (1024 + code) * sc - 1024 * sc, leaves
+// sc * code with a single rounding, i.e. exactly.  A second B with m_g in every position accumulates m_g times the group's
+// activation sum.  Both accumulate over the eight groups of a block inside the matrix core, so a block costs per 16 rows
+//   y += d * C1 - dmin * C2
+// and no per-group float arithmetic at all.  Workgroup = eight waves = eight tiles of 16 weight rows on one range of blocks; RG
+// groups of 16 activation rows.  LDS per block: [RG][8 groups][64 lanes][16 B] in operand order (a wave's read is one contiguous
+// kilobyte), two blocks at a time.  The matrix is cut along K into `slices` until two workgroups per compute unit exist; the
+// partial sums [slice][row][n] are added in slice order by k45_rows64_reduce_kernel (deterministic).
+// ------------------------------------------------------------------------------------------------
+constexpr int kR64Waves = 8;
+typedef _Float16 v2hf __attribute__((ext_vector_type(2)));
+
+// eight code bytes (two dwords) and the group's 6-bit scale -> eight fp16 values sc * code
+__device__ __forceinline__ uint4 scaled_code_halves(uint32_t c0, uint32_t c1, uint32_t scale) {
+    union { uint32_t u; v2hf h; } s2, off, in, out;
+    const _Float16 sh = static_cast<_Float16>(static_cast<unsigned short>(scale));
+    s2.h = v2hf{sh, sh};
+    off.h = s2.h * static_cast<_Float16>(-1024.0f);                          // exact: at most 63 * 2^10
+    uint32_t r[4];
+    const uint32_t pairs[4] = {__builtin_amdgcn_perm(0x64646464u, c0, 0x04010400u), __builtin_amdgcn_perm(0x64646464u, c0, 0x04030402u),
+                               __builtin_amdgcn_perm(0x64646464u, c1, 0x04010400u), __builtin_amdgcn_perm(0x64646464u, c1, 0x04030402u)};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        in.u = pairs[i];
+        out.h = __builtin_elementwise_fma(in.h, s2.h, off.h);
+        r[i] = out.u;
+    }
+    return make_uint4(r[0], r[1], r[2], r[3]);
+}
+
+template <typename FMT, int RG>
+__global__ __launch_bounds__(64 * kR64Waves) void k45_rows64_kernel(
+    const _Float16* __restrict__ xh, const float* __restrict__ xscale, const uint8_t* __restrict__ w, void* __restrict__ y, int y_dtype,
+    float* __restrict__ partial, int t_rows, int t_pad, int n, int bpr, int kp, int blocks_per_slice) {
+    __shared__ __align__(16) unsigned char abuf[2][RG * 8 * 1024];
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int col = lane & 15, q = lane >> 4;
+    const int wrow = min((static_cast<int>(blockIdx.x) * kR64Waves + wave) * 16 + col, n - 1);   // rows past the end: the last row again, dropped at the store
+    const uint8_t* wp = w + static_cast<size_t>(wrow) * bpr * FMT::kBlockBytes;
+    const int b_begin = static_cast<int>(blockIdx.y) * blocks_per_slice, b_end = min(bpr, b_begin + blocks_per_slice);
+    const int t0 = static_cast<int>(blockIdx.z) * 16 * RG;
+    // staging: wave v moves the pieces (rg, g) = (i, v) of a block, i < RG; lane (col, q) brings 8 values of activation row 16 rg + col
+    const _Float16* ap[RG];
+#pragma unroll
+    for (int i = 0; i < RG; ++i) ap[i] = xh + static_cast<size_t>(min(t0 + 16 * i + col, t_rows - 1)) * kp + 32 * wave + 8 * q;
+
+    v4f acc[RG];
+#pragma unroll
+    for (int i = 0; i < RG; ++i) acc[i] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+
+    auto multiply = [&](const typename FMT::Regs& r, int buf) {
+        const K4Scales sc = k4_unpack(r.hdr);
+        v4f c1[RG], c2[RG];
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {
+            const uint2 cb = FMT::codes(r, g >> 1, g & 1, q);
+            const uint32_t scg = ((g < 4 ? sc.sc_lo : sc.sc_hi) >> (8 * (g & 3))) & 0xffu;
+            const uint32_t mng = ((g < 4 ? sc.mn_lo : sc.mn_hi) >> (8 * (g & 3))) & 0xffu;
+            const uint4 bc = scaled_code_halves(cb.x, cb.y, scg);
+            union { uint32_t u; v2hf h; } m2;
+            const _Float16 mh = static_cast<_Float16>(static_cast<unsigned short>(mng));
+            m2.h = v2hf{mh, mh};
+            const uint4 bm = make_uint4(m2.u, m2.u, m2.u, m2.u);
+#pragma unroll
+            for (int i = 0; i < RG; ++i) {
+                const uint4 a = *reinterpret_cast<const uint4*>(&abuf[buf][(i * 8 + g) * 1024 + lane * 16]);
+                c1[i] = half_mfma<false>(a, bc, g == 0 ? v4f{0.0f, 0.0f, 0.0f, 0.0f} : c1[i]);
+                c2[i] = half_mfma<false>(a, bm, g == 0 ? v4f{0.0f, 0.0f, 0.0f, 0.0f} : c2[i]);
+            }
+        }
+        const float dd = f16_bits_to_float(r.hdr.x & 0xffffu), dmin = f16_bits_to_float(r.hdr.x >> 16);
+#pragma unroll
+        for (int i = 0; i < RG; ++i) acc[i] += c1[i] * dd - c2[i] * dmin;
+    };
+    // Two blocks per trip: everything the trip needs is requested at once (weights of both blocks into registers, activation pieces
+    // of both through registers into the two LDS buffers), one memory round trip, then both blocks are multiplied.  A workgroup's
+    // own trips do not overlap; the two workgroups of a compute unit do, one fetching while the other multiplies.
+    for (int b = b_begin; b < b_end; b += 2) {
+        const int b1 = min(b + 1, b_end - 1);                                // (past the last block: that one again, not used)
+        typename FMT::Regs r0, r1;
+        u32x4 a0[RG], a1[RG];
+        FMT::load(r0, wp + static_cast<size_t>(b) * FMT::kBlockBytes, q);
+        FMT::load(r1, wp + static_cast<size_t>(b1) * FMT::kBlockBytes, q);
+#pragma unroll
+        for (int i = 0; i < RG; ++i) {
+            a0[i] = *reinterpret_cast<const u32x4*>(ap[i] + 256 * b);
+            a1[i] = *reinterpret_cast<const u32x4*>(ap[i] + 256 * b1);
+        }
+        if (b > b_begin) __syncthreads();                                    // everybody has left the buffers of the trip before
+#pragma unroll
+        for (int i = 0; i < RG; ++i) {
+            *reinterpret_cast<u32x4*>(&abuf[0][(i * 8 + wave) * 1024 + lane * 16]) = a0[i];
+            *reinterpret_cast<u32x4*>(&abuf[1][(i * 8 + wave) * 1024 + lane * 16]) = a1[i];
+        }
+        __syncthreads();
+        multiply(r0, 0);
+        if (b + 1 < b_end) multiply(r1, 1);
+    }
+
+    // lane (col, q) holds rows 4 q .. 4 q + 3 of every row group against weight row `col` of the wave's tile
+    const int out_col = (static_cast<int>(blockIdx.x) * kR64Waves + wave) * 16 + col;
+    if (out_col >= n) return;
+#pragma unroll
+    for (int i = 0; i < RG; ++i)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int row = t0 + 16 * i + 4 * q + r;
+            if (row >= t_rows) continue;
+            if (partial) partial[(static_cast<size_t>(blockIdx.y) * t_pad + row) * n + out_col] = acc[i][r];
+            else store_plain(y, y_dtype, static_cast<size_t>(row) * n + out_col, acc[i][r] * xscale[row]);
+        }
+}
+
+// y[t, c] = xscale[t] * sum over the slices, in slice order, of partial[slice][t][c]; four columns per thread
+__global__ __launch_bounds__(256) void k45_rows64_reduce_kernel(const float* __restrict__ partial, const float* __restrict__ xscale, void* __restrict__ y,
+                                                                int y_dtype, int t_rows, int t_pad, int n, int slices) {
+    const int c = (static_cast<int>(blockIdx.x) * 256 + static_cast<int>(threadIdx.x)) * 4, t = blockIdx.y;
+    if (c >= n) return;
+    float4 s = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    const float* src = partial + static_cast<size_t>(t) * n + c;
+    if (c + 3 < n && (n & 3) == 0) {
+        for (int k = 0; k < slices; ++k) {
+            const float4 v = *reinterpret_cast<const float4*>(src + static_cast<size_t>(k) * t_pad * n);
+            s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+        }
+    } else {
+        for (int k = 0; k < slices; ++k) {
+            const float* v = src + static_cast<size_t>(k) * t_pad * n;
+            s.x += v[0];
+            if (c + 1 < n) s.y += v[1];
+            if (c + 2 < n) s.z += v[2];
+            if (c + 3 < n) s.w += v[3];
+        }
+    }
+    const float sc = xscale[t];
+    const size_t o = static_cast<size_t>(t) * n + c;
+    store_plain(y, y_dtype, o, s.x * sc);
+    if (c + 1 < n) store_plain(y, y_dtype, o + 1, s.y * sc);
+    if (c + 2 < n) store_plain(y, y_dtype, o + 2, s.z * sc);
+    if (c + 3 < n) store_plain(y, y_dtype, o + 3, s.w * sc);
+}
+
+// column groups of 128 weight rows, cut along K until about two workgroups per compute unit exist
+struct Rows64Plan { int rg, zs, t_pad, cols, slices, bps; };
+Rows64Plan plan_rows64(int rows, int n, int bpr) {
+    Rows64Plan p;
+    p.rg = rows <= 32 ? 2 : 4;
+    p.zs = (rows + 16 * p.rg - 1) / (16 * p.rg);
+    p.t_pad = p.zs * 16 * p.rg;
+    p.cols = (n + 16 * kR64Waves - 1) / (16 * kR64Waves);
+    const int want = 2 * compute_units() / (p.cols * p.zs);                 // all workgroups resident at once, two per compute unit
+    int slices = want < 1 ? 1 : (want > bpr ? bpr : want);
+    p.bps = (bpr + slices - 1) / slices;
+    p.slices = (bpr + p.bps - 1) / p.bps;
+    return p;
+}
+
+template <typename FMT>
+int launch_rows64(const Rows64Plan& p, const _Float16* xh, const float* xscale, const uint8_t* w, void* y, int y_dtype, float* partial,
+                  int rows, int n, int bpr, hipStream_t stream) {
+    const dim3 grid(p.cols, p.slices, p.zs);
+    float* part = p.slices > 1 ? partial : nullptr;
+    if (p.rg == 2) hipLaunchKernelGGL((k45_rows64_kernel<FMT, 2>), grid, dim3(64 * kR64Waves), 0, stream, xh, xscale, w, y, y_dtype, part, rows, p.t_pad, n, bpr, bpr * 256, p.bps);
+    else hipLaunchKernelGGL((k45_rows64_kernel<FMT, 4>), grid, dim3(64 * kR64Waves), 0, stream, xh, xscale, w, y, y_dtype, part, rows, p.t_pad, n, bpr, bpr * 256, p.bps);
+    if (hipGetLastError() != hipSuccess) return PLLM_ERR_LAUNCH;
+    if (p.slices > 1) {
+        hipLaunchKernelGGL(k45_rows64_reduce_kernel, dim3((n + 1023) / 1024, rows), dim3(256), 0, stream, partial, xscale, y, y_dtype, rows, p.t_pad, n, p.slices);
+        if (hipGetLastError() != hipSuccess) return PLLM_ERR_LAUNCH;
+    }
+    return PLLM_OK;
+}
+
 }  // namespace
 
 size_t kquant_matvec_workspace_bytes(int rows, int bpr) { return act_image_256_bytes(bpr) * static_cast<size_t>(rows); }
@@ -1067,4 +1247,34 @@ int k45_rows16_matvec(const void* x, int x_dtype, const uint8_t* w, int type_id,
                      : launch_rows16<Rows16Q5K, 1, 4>(x, x_dtype, w, y, y_dtype, rows, k, n, bpr, stream);
 }
 
+}  // namespace pllm
+
+namespace pllm {
+// Q4_K / Q5_K on 17 - 48 activation rows (any of the three input types; the rows are staged as scaled fp16 rows first)
+bool k45_rows64_supports(int type_id, int rows, int n, int bpr, const uint8_t* w) {
+    // measured against the tile kernel (Q4_K, operator call in us, this kernel / tiles): 5120x5120 19.1 / 26.2 at 17 rows, 21.4 / 26.2
+    // at 32, 27.9 / 27.7 at 64, 31.9 / 32.8 at 128; 17408x5120 31.0 / 40.9, 32.8 / 41.0, 44.6 / 43.0, 91.5 / 60.3: it takes the calls of up
+    // to 48 rows (the kernel itself serves up to 128)
+    return (type_id == PLLM_TYPE_Q4_K || type_id == PLLM_TYPE_Q5_K) && rows > 16 && rows <= 48 && n >= 16 && bpr >= 1 &&
+           (reinterpret_cast<uintptr_t>(w) & 15u) == 0;
+}
+size_t k45_rows64_workspace_bytes(int rows, int n, int bpr) {
+    const Rows64Plan p = plan_rows64(rows, n, bpr);
+    const size_t part = p.slices > 1 ? align256(static_cast<size_t>(p.slices) * p.t_pad * n * sizeof(float)) : 0;
+    return gemm_f16_staged_bytes(rows, bpr) + part;
+}
+int k45_rows64_gemm(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y, int y_dtype, int rows, int k, int n, int bpr,
+                    void* workspace, size_t workspace_bytes, hipStream_t stream) {
+    if (!k45_rows64_supports(type_id, rows, n, bpr, w) || (y_dtype & kAccumulateInto)) return PLLM_ERR_UNSUPPORTED;
+    if (!workspace || workspace_bytes < k45_rows64_workspace_bytes(rows, n, bpr)) return PLLM_ERR_WORKSPACE;
+    const int st = gemm_f16_stage_rows(x, x_dtype, nullptr, rows, k, bpr, workspace, stream);
+    if (st != PLLM_OK) return st;
+    const size_t rows_bytes = align256(static_cast<size_t>(rows) * bpr * 256 * sizeof(_Float16));
+    const _Float16* xh = static_cast<const _Float16*>(workspace);
+    const float* xscale = reinterpret_cast<const float*>(static_cast<const unsigned char*>(workspace) + rows_bytes);
+    float* partial = reinterpret_cast<float*>(static_cast<unsigned char*>(workspace) + gemm_f16_staged_bytes(rows, bpr));
+    const Rows64Plan p = plan_rows64(rows, n, bpr);
+    return type_id == PLLM_TYPE_Q4_K ? launch_rows64<Rows16Q4K>(p, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, stream)
+                                     : launch_rows64<Rows16Q5K>(p, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, stream);
+}
 }  // namespace pllm

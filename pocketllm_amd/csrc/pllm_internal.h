@@ -108,6 +108,12 @@ int dot4_matvec_from_image(const ActRows& act, const uint8_t* w, int type_id, vo
 // Q4_K / Q5_K, 2 - 16 raw rows of bf16 / fp16 activations (k a whole number of super-blocks) as rows of a half-precision matrix-core
 // product in one pass over the weights (PLLM_ERR_UNSUPPORTED: not such a call)
 int k45_rows16_matvec(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y, int y_dtype, int rows, int k, int n, int bpr, hipStream_t stream);
+// Q4_K / Q5_K on 17 - 48 activation rows: every block decoded once in registers and multiplied into all rows (fp16 matrix cores,
+// exact weights); workspace = staged fp16 rows + partial sums of the slices along K
+bool k45_rows64_supports(int type_id, int rows, int n, int bpr, const uint8_t* w);
+size_t k45_rows64_workspace_bytes(int rows, int n, int bpr);
+int k45_rows64_gemm(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y, int y_dtype, int rows, int k, int n, int bpr,
+                    void* workspace, size_t workspace_bytes, hipStream_t stream);
 int iq4xs_wave_matvec(const ActRows& act, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream,
                       WeightRoute route = WeightRoute{});
 int groups16_wave_matvec(const ActRows& act, const uint8_t* w, int type_id, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream,

@@ -44,6 +44,32 @@ def test_prefill_matches_float_oracle(mod, type_name, t, n, k):
         assert row_err.max() <= tol, (dt, row_err.argmax(), row_err.max())
 
 
+@pytest.mark.parametrize("type_name", ["q4_k", "q5_k"])
+@pytest.mark.parametrize("t,n,k", [(17, 100, 768), (24, 16, 256), (33, 272, 2048), (40, 129, 1000), (48, 5120, 5120), (32, 1000, 5120)])
+def test_prefill_17_to_48_rows_matches_float_oracle(mod, type_name, t, n, k):
+    """The token counts between decode and the large tiles: every block is decoded once in registers (sc * code as exact fp16 integers) and
+    multiplied into all rows on the fp16 matrix cores.  16-bit activations are exact in the operands, so the distance to the float
+    statement is float32 summation order only; float32 activations are rounded to fp16 once (<= 1e-3)."""
+    rng = np.random.default_rng(7 * t + n + k)
+    blocks = ENC[type_name]((rng.standard_normal((n, k)) * 0.02).astype(np.float32))
+    x_np = rng.standard_normal((t, k)).astype(np.float32)
+    x_np[3] *= 1e4                      # per-row power-of-two scaling has to absorb a huge and a tiny row
+    x_np[5] *= 1e-6
+    ref_w = O.dequant_rows(blocks, type_name, k)
+    grid = torch.empty(0, dtype=torch.int8, device=DEV)
+    for dt, tol in ((torch.bfloat16, 5e-6), (torch.float16, 5e-6), (torch.float32, 6e-4)):
+        x = torch.from_numpy(np.clip(x_np, -6e4, 6e4) if dt == torch.float16 else x_np).to(DEV).to(dt)
+        print(f"case prefill rows {type_name} t={t} n={n} k={k} {dt}", flush=True)
+        y = mod.gguf_quant_gemm_prefill_forward(x, torch.from_numpy(blocks).to(DEV), k, O.TYPE_IDS[type_name], grid, out_dtype=torch.float32)
+        torch.cuda.synchronize()
+        want = O.matmul_f(x.float().cpu().numpy(), ref_w)
+        got = y.cpu().numpy()
+        row_err = np.sqrt(((got - want) ** 2).sum(axis=1) / np.maximum((want ** 2).sum(axis=1), 1e-300))
+        assert row_err.max() <= tol, (dt, row_err.argmax(), row_err.max())
+        y16 = mod.gguf_quant_gemm_prefill_forward(x, torch.from_numpy(blocks).to(DEV), k, O.TYPE_IDS[type_name], grid)
+        assert y16.dtype == torch.bfloat16 and torch.equal(y16, y.to(torch.bfloat16))
+
+
 def test_prefill_3d_input_and_bf16_output(mod):
     rng = np.random.default_rng(0)
     blocks = torch.from_numpy(C.quantize_q4_k((rng.standard_normal((192, 512)) * 0.02).astype(np.float32))).to(DEV)
