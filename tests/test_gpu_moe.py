@@ -131,8 +131,9 @@ def test_baseline_config_single_token_shapes(mod):
 
 def test_baseline_config_grouped_256_tokens_256_experts(mod):
     """BASELINE config 5 at T = 256: 256 experts, top-8 softmax routing, 2048 routes, every weight tensor at its full size.
-    The oracle restates the operator for six sampled tokens (their 48 routes, full output rows); every other token is
-    covered by the determinism check and by the finite, non-zero rows."""
+    The oracle restates the operator for 32 sampled tokens (their 256 routes, full output rows); every other token is
+    covered by the determinism check and by the finite, non-zero rows.  The same full-size tensors then serve the single-token
+    operator on routes to the far end of the expert range (ids above 200: offsets of hundreds of megabytes into w1 / w3 / w2)."""
     rng = np.random.default_rng(1005)
     e, d, inter, topk, t = 256, 3072, 1536, 8, 256
     w1 = _expert_blocks(rng, "iq2_xxs", e, inter, d)
@@ -154,7 +155,7 @@ def test_baseline_config_grouped_256_tokens_256_experts(mod):
     got = y.cpu().numpy()
     assert got.shape == (t, d) and np.isfinite(got).all() and (np.abs(got).max(axis=1) > 0).all()
     route_experts = np.repeat(np.arange(e), np.diff(o_seg))
-    sample = rng.choice(t, size=6, replace=False)
+    sample = rng.choice(t, size=32, replace=False)
     keep = np.isin(o_toks, sample)
     want = O.moe_forward(x.float().cpu().numpy(), o_toks[keep], o_rws[keep], route_experts[keep], w1, w3, w2, "iq2_xxs", "iq2_xxs", "iq1_m", 0.0)
     assert O.rel_l2(got[sample], want[sample]) <= TOL
@@ -162,6 +163,14 @@ def test_baseline_config_grouped_256_tokens_256_experts(mod):
         assert O.rel_l2(got[tok], want[tok]) <= 2 * TOL, tok
     y2 = mod.gguf_moe_prefill_grouped_forward(x, toks, rws, seg, dw1, dw3, dw2, d, tid["iq2_xxs"], d, tid["iq2_xxs"], inter, tid["iq1_m"], grids, 0.0)
     assert torch.equal(y, y2)
+    # T = 1 on the same 256-expert tensors, routed to experts at the far end of the range
+    far = np.array([255, 201, 230, 7, 248, 213, 128, 254], dtype=np.int64)
+    fw = rng.uniform(0.05, 0.3, size=topk).astype(np.float32)
+    print("case single token, experts above 200 of 256", flush=True)
+    y1 = mod.gguf_moe_single_token_forward(x[:1].contiguous(), torch.from_numpy(far).to(DEV), torch.from_numpy(fw).to(DEV), dw1, dw3, dw2, 0.0)
+    torch.cuda.synchronize()
+    want1 = O.moe_forward(x[:1].float().cpu().numpy(), np.zeros(topk, dtype=np.int64), fw, far, w1, w3, w2, "iq2_xxs", "iq2_xxs", "iq1_m", 0.0)
+    assert O.rel_l2(y1.cpu().numpy(), want1) <= TOL
 
 
 def test_grouped_experts_more_routes_than_the_reduction_lists(mod):

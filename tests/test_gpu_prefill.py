@@ -162,6 +162,26 @@ def test_fp8_prefill_matches_float_oracle(mod, t, n, k):
         assert O.rel_l2(got, want) <= 1e-3
 
 
+def test_fp8_float32_activations_precision_step_at_16_rows(mod):
+    """float32 activations stay on the float32 matvec (<= 1e-5 against the float statement of soft_fp8_blockfp8_gemm,
+    src/kernels/ops.py:641-648) up to 15 rows and take the fp16 tile kernel from 16 rows on (operands rounded to fp16, <= 1e-3):
+    both sides of the switch are pinned here."""
+    rng = np.random.default_rng(16)
+    n, k = 384, 2048
+    codes, scale = C.quantize_fp8_block((rng.standard_normal((n, k)) * 0.02).astype(np.float32))
+    ref_w = O.dequant_fp8_block(codes, scale)
+    dc, ds = torch.from_numpy(codes).to(DEV), torch.from_numpy(scale).to(DEV)
+    errs = {}
+    for rows in (15, 16):
+        x_np = rng.standard_normal((rows, k)).astype(np.float32)
+        print(f"case fp8 float32 activations rows={rows}", flush=True)
+        y = mod.fp8_block_gemm_forward(torch.from_numpy(x_np).to(DEV), dc, ds, out_dtype=torch.float32)
+        torch.cuda.synchronize()
+        errs[rows] = O.rel_l2(y.cpu().numpy(), O.matmul_f(x_np, ref_w))
+    assert errs[15] <= 1e-5, errs
+    assert errs[16] <= 1e-3, errs
+
+
 def test_fp8_prefill_baseline_shape_sampled(mod):
     """BASELINE config 4 at T = 512 (N = 17408, K = 5120, weights N(0, 0.02) with blockmax/448 scales); 64 sampled columns."""
     rng = np.random.default_rng(1004)

@@ -1,6 +1,9 @@
 """The entry point that allocates nothing (pllm_gguf_quant_gemm_static_scratch) against pllm_gguf_quant_gemm, through the C ABI:
-same bits on calls in a row, the later ones smaller than the first, for a decode call on a pre-quantized image and for a prefill
-call on the tile kernel (both keep their temporaries in the library's device array); oversize calls are refused."""
+same bits on calls in a row, the later ones smaller than the first, for every kind of call that keeps temporaries in the library's
+device array: decode calls whose activation image is written there by the pre-pass (float32 activations of 5 - 8 rows, and a
+Q6_K call of 7 bf16 rows; 16-bit rows of Q4_K / Q5_K at these counts run a kernel without workspace and would test nothing), a
+33-row call (staged fp16 rows and the partial sums of its K slices) and a 96-row call on the tile kernel (staged rows and partial
+tiles); oversize calls are refused."""
 import ctypes
 
 import numpy as np
@@ -36,13 +39,14 @@ def test_static_scratch_entry_point_matches_the_workspace_one():
     assert load_cuda_kernel() is not None and torch.cuda.is_available()
     lib = _ffi.load_library()
     rng = np.random.default_rng(91)
-    enc = {3: C.quantize_q4_k, 4: C.quantize_q5_k}
-    # (type id, rows, n, k): a decode call of 8 rows (activation image in the array), then smaller ones; a prefill call of 96
-    # rows (staged fp16 rows and partial tiles in the array), then a smaller one
-    for type_id, rows, n, k in ((3, 8, 640, 2048), (3, 6, 200, 1024), (4, 5, 48, 512), (4, 96, 520, 1536), (3, 33, 130, 768)):
+    enc = {3: C.quantize_q4_k, 4: C.quantize_q5_k, 8: C.quantize_q6_k}
+    # (type id, rows, n, k, activation type): decode calls on an activation image in the array, each smaller than the one before;
+    # then the two prefill forms, the larger first
+    for type_id, rows, n, k, dt in ((3, 8, 640, 2048, torch.float32), (3, 6, 200, 1024, torch.float32), (4, 5, 48, 512, torch.float32),
+                                    (8, 7, 96, 512, torch.bfloat16), (4, 96, 520, 1536, torch.bfloat16), (3, 33, 130, 768, torch.bfloat16)):
         blocks = torch.from_numpy(enc[type_id]((rng.standard_normal((n, k)) * 0.02).astype(np.float32))).to(DEV)
-        x = torch.from_numpy(rng.standard_normal((rows, k)).astype(np.float32)).to(DEV).to(torch.bfloat16)
-        print(f"case static scratch type={type_id} rows={rows} n={n} k={k}", flush=True)
+        x = torch.from_numpy(rng.standard_normal((rows, k)).astype(np.float32)).to(DEV).to(dt)
+        print(f"case static scratch type={type_id} rows={rows} n={n} k={k} {dt}", flush=True)
         need, want, got = _both(lib, x, blocks, type_id, k)
         assert need > 0, "the case no longer uses a workspace"
         assert not torch.isnan(want).any()
