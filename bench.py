@@ -501,10 +501,18 @@ def prefill_cases(mod, dev):
     for name, tid, enc in (("q4_k", 3, C.quantize_q4_k), ("q5_k", 4, C.quantize_q5_k)):
         for n in (5120, 17408):
             blocks = torch.from_numpy(enc(rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02))).to(dev)
-            for t in (64, 512, 2048):
+            for t in (32, 64, 512, 2048):
                 x = torch.randn(t, k, device=dev, dtype=torch.bfloat16)
                 run(f"{name} prefill {n}x{k} T={t}", t, n,
                     lambda s, x=x, blocks=blocks, tid=tid: mod.gguf_quant_gemm_prefill_forward(x, blocks, k, tid, empty))
+            if n == 17408:
+                # BASELINE config 3 as it is worded: activations quantized to 32-value int8 blocks, integer dots on the int8 matrix cores
+                for t in (512, 2048):
+                    x = torch.randn(t, k, device=dev, dtype=torch.bfloat16)
+                    us, graphed = time_calls_us(lambda s, x=x, blocks=blocks, tid=tid: mod.gguf_quant_gemm_q8_forward(x, blocks, k, tid, empty), 4, iters=40)
+                    tops = 2.0 * t * k * n / us / 1e6
+                    out.append({"case": f"{name} int8-MFMA prefill (int8 activations) {n}x{k} T={t}", "us_per_call": round(us, 3), "tflops": round(tops, 1),
+                                "frac_mfma_peak": round(tops / 5000.0, 4), "peak": "int8 dense 5.0 POP/s", "graph": graphed})
             del blocks
     n = 17408
     for name, tid in (("q6_k", 8), ("iq4_xs", 7), ("iq3_xxs", 6), ("iq2_xs", 5)):   # random valid blocks: the work does not depend on the values
@@ -778,8 +786,10 @@ def main() -> None:
     # the full table goes to stderr; the one line on stdout keeps the records of the BASELINE configurations
     print("bench.py all cases: " + json.dumps(cases), file=sys.stderr)
     keep = ("q4_k matvec", "q5_k matvec", "q8_0 matvec", "fp8_e4m3 matvec 17408x5120 T=1", "fused experts", "q4_k prefill", "q5_k prefill",
-            "fp8_e4m3 prefill", "fp8_e4m3 x fp8_e4m3", "iq2_xxs matvec", "iq1_m matvec", "q2_k matvec")
-    short = [{k2: v for k2, v in c.items() if k2 in ("case", "us_per_call", "gbs", "frac_hbm_peak", "tflops", "frac_mfma_peak", "peak")}
+            "q4_k int8-MFMA", "q5_k int8-MFMA", "fp8_e4m3 prefill", "fp8_e4m3 x fp8_e4m3", "iq2_xxs matvec", "iq1_m matvec", "q2_k matvec",
+            "MiniMaxBlock", "MiniMaxTransformer")
+    short = [{k2: v for k2, v in c.items() if k2 in ("case", "us_per_call", "gbs", "frac_hbm_peak", "tflops", "frac_mfma_peak", "peak", "decode_tps", "prefill_tps",
+                                                     "decode_us_per_token", "decode_tps_62_layers_blocks_only", "decode_tps_62_layers_extrapolated")}
              for c in cases if c["case"].startswith(keep)]
 
     out = {

@@ -500,20 +500,34 @@ def matmul_f(x: np.ndarray, w: np.ndarray) -> np.ndarray:
     return x.astype(np.float64) @ w.astype(np.float64).T
 
 
-def kquant_gemm_q(x: np.ndarray, blocks: np.ndarray, type_name: str) -> np.ndarray:
+def kquant_gemm_q(x: np.ndarray, blocks: np.ndarray, type_name: str, ds4_pair: bool = False) -> np.ndarray:
     """Int8-activation semantics for Q4_K / Q5_K (the prefill path of BASELINE config 3).
 
     acts -> int8 per 32 (q8_1_quantize); per 32-group g:
         y += (d * sc_g) * xs_g * sum_i(q_i * xq_i)  -  (dmin * m_g) * xs_g * sum_i(xq_i)
     with d*sc and dmin*m kept in float32 (the reference's MMQ rounds them to fp16:
     llama_mmq/mmq.cuh:2160-2165, 1374-1378; that loss is not reproduced).  Returns float64 [T, N].
+
+    ds4_pair=True restates the activation side the way the reference's MMA path stores it (llama_mmq/gguf_mma_wrapper.cu:90-126,
+    layout DS4): per 32 values the pair {fp16(amax / 127), fp16(sum of the float activations)}, codes rint(x * (1 / d)) with d the
+    float32 quotient; the min term then uses the stored float sum, y -= (dmin * m_g) * fp16(sum_i x_i), and the dot term the fp16
+    scale.  The library's operator is the default statement; the two are compared in tests/test_oracle_pinning.py.
     """
     assert type_name in ("q4_k", "q5_k")
     n, bpr, _ = blocks.shape
     t, k = x.shape
     assert k == bpr * 256
-    xq, xs = q8_1_quantize(x, 32)
-    xq = xq.astype(np.int64).reshape(t, bpr * 8, 32)
+    if ds4_pair:
+        xg = x.astype(np.float32).reshape(t, bpr * 8, 32)
+        dq = (np.abs(xg).max(axis=-1) / np.float32(127.0)).astype(np.float32)
+        inv = np.where(dq > 0, np.float32(1.0) / np.where(dq > 0, dq, np.float32(1.0)), np.float32(0.0)).astype(np.float32)
+        xq = np.rint(xg * inv[..., None]).astype(np.int64)
+        xs = dq.astype(np.float16).astype(np.float32)
+        fsum = xg.sum(axis=-1, dtype=np.float32).astype(np.float16).astype(np.float64)       # [T, G]
+    else:
+        xq, xs = q8_1_quantize(x, 32)
+        xq = xq.astype(np.int64).reshape(t, bpr * 8, 32)
+        fsum = None
     xsum = xq.sum(axis=-1)                                           # [T, G]
     if type_name == "q4_k":
         d = _f16(blocks[..., 0:2]); dmin = _f16(blocks[..., 2:4]); scales = blocks[..., 4:16]
@@ -544,7 +558,10 @@ def kquant_gemm_q(x: np.ndarray, blocks: np.ndarray, type_name: str) -> np.ndarr
     xs64 = xs.astype(np.float64)
     for g in range(bpr * 8):
         dots = xq[:, g, :] @ q[:, g, :].T                             # exact integers [T, N]
-        out += xs64[:, g:g + 1] * (dots * sc[None, :, g] - xsum[:, g:g + 1] * mn[None, :, g])
+        if fsum is None:
+            out += xs64[:, g:g + 1] * (dots * sc[None, :, g] - xsum[:, g:g + 1] * mn[None, :, g])
+        else:
+            out += xs64[:, g:g + 1] * dots * sc[None, :, g] - fsum[:, g:g + 1] * mn[None, :, g]
     return out
 
 
