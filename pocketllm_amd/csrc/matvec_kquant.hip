@@ -276,8 +276,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void k45_mfma_matvec_kernel(
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         float a = acc[r];
-        a += __shfl_xor(a, 16, 64);
-        a += __shfl_xor(a, 32, 64);
+        a = quad_rows_sum(a);
         if (ks == 0) partial[(r * waves + wave) * kRowsPerWg + col] = a;
     }
     __syncthreads();
@@ -489,8 +488,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_image_matvec_kernel(
             if (it + DEPTH < ITERS) request(it + DEPTH);
         }
     }
-    acc += __shfl_xor(acc, 16, 64);
-    acc += __shfl_xor(acc, 32, 64);
+    acc = quad_rows_sum(acc);
     if (ks == 0) partial[wave * kRowsPerWg + col] = acc;
     __syncthreads();
     if (tid < kRowsPerWg) {
@@ -752,8 +750,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_groups16_matvec_kernel(
             }
         }
     }
-    acc += __shfl_xor(acc, 16, 64);
-    acc += __shfl_xor(acc, 32, 64);
+    acc = quad_rows_sum(acc);
     if (ks == 0) partial[wave * kRowsPerWg + col] = acc;
     __syncthreads();
     if (tid < kRowsPerWg) {

@@ -35,11 +35,8 @@ __device__ __forceinline__ void store_hidden16(float g, float u, float limit, fl
     }
     const float h = (i < inter) ? g / (1.0f + expf(-g)) * u * route_weight : 0.0f;
     float am = fabsf(h), sum = h;
-#pragma unroll
-    for (int off = 1; off < 16; off <<= 1) {
-        am = fmaxf(am, __shfl_xor(am, off, 64));
-        sum += __shfl_xor(sum, off, 64);
-    }
+    am = group_max<16>(am);
+    sum = group_sum<16>(sum);
     const float inv = am > 0.0f ? 127.0f / am : 0.0f;
     const float scale = am * (1.0f / 127.0f);
     const float q = fminf(fmaxf(rintf(h * inv), -127.0f), 127.0f);
@@ -103,8 +100,7 @@ __global__ __launch_bounds__(64 * kW13Waves) void moe_single_w13_kernel(
         FMT::load_lds(regs, tile, col * row_bytes + b * FMT::kBlockBytes, ks);
         acc += FMT::block(regs, ks, b, smem, am, sx, tables);
     }
-    acc += __shfl_xor(acc, 16, 64);
-    acc += __shfl_xor(acc, 32, 64);
+    acc = quad_rows_sum(acc);
     if (ks == 0) exch[(share * 2 + mat) * 16 + col] = acc;
     __syncthreads();
     if (tid < 16) {
@@ -173,8 +169,7 @@ __global__ __launch_bounds__(64 * kW2Waves) void moe_single_w2_kernel(
             acc += FMT::finish(regs, ks, ch, cl, make_float4(0.125f * xs.x, 0.125f * xs.y, 0.125f * xs.z, 0.125f * xs.w));
         }
     }
-    acc += __shfl_xor(acc, 16, 64);
-    acc += __shfl_xor(acc, 32, 64);
+    acc = quad_rows_sum(acc);
     if (ks == 0) partial[wave * 16 + col] = acc;
     __syncthreads();
     if (tid < 16) {
@@ -264,8 +259,7 @@ __global__ __launch_bounds__(64 * kGroupWaves) void moe_grouped_w13_kernel(
                     const int b = share + kShares * i;
                     if (b < bpr) acc += FMT::route_block(dec[i], ks, b, img, am, kpad, ops);   // wave-uniform
                 }
-                acc += __shfl_xor(acc, 16, 64);
-                acc += __shfl_xor(acc, 32, 64);
+                acc = quad_rows_sum(acc);
                 if (ks == 0) exch[((q * kShares + share) * 2 + mat) * 16 + col] = acc;
             }
             __syncthreads();
@@ -344,8 +338,7 @@ __global__ __launch_bounds__(64 * kGroupWaves) void moe_grouped_w2_kernel(
                         const int b = share + shares * i;
                         if (b < bpr) acc += FMT::route_block16(dec[i], ks, b, img, am, kpad, ops);
                     }
-                    acc += __shfl_xor(acc, 16, 64);
-                    acc += __shfl_xor(acc, 32, 64);
+                    acc = quad_rows_sum(acc);
                     if (ks == 0) exch[(q * kGroupWaves + wave) * 16 + col] = acc;
                 }
             __syncthreads();
@@ -426,8 +419,7 @@ __global__ __launch_bounds__(256) void rows_image_kernel(const void* __restrict_
     } else {
         for (int k = tid; k < dim; k += 256) am = fmaxf(am, fabsf(load_any(x, x_dtype, base + k)));
     }
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) am = fmaxf(am, __shfl_xor(am, off, 64));
+    am = group_max<64>(am);
     if ((tid & 63) == 0) part[tid >> 6] = am;
     __syncthreads();
     am = fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3]));
@@ -511,8 +503,7 @@ __global__ __launch_bounds__(256) void rows_hidden_half_kernel(const float* __re
     const int route = blockIdx.x, tid = threadIdx.x;
     float am = 0.0f;
     for (int t = tid; t < h_kpad / 16; t += 256) am = fmaxf(am, tile_max[static_cast<size_t>(route) * (h_kpad / 16) + t]);
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) am = fmaxf(am, __shfl_xor(am, off, 64));
+    am = group_max<64>(am);
     if ((tid & 63) == 0) part[tid >> 6] = am;
     __syncthreads();
     const float s = rows_scale(fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3])));

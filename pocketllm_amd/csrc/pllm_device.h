@@ -57,26 +57,41 @@ __device__ __forceinline__ float butterfly_peer(float v) {
     else return __shfl_xor(v, OFF, 64);
 }
 
-// v summed over the four lanes (l % 16) + {0, 16, 32, 48}, in every lane: the two wide steps of a butterfly through
-// gfx950's row swaps (v_permlane16_swap exchanges odd rows of one operand with even rows of the other, v_permlane32_swap
-// the upper half with the lower half), one vector instruction each and no LDS crossbar.
+// v summed over the four lanes (l % 16) + {0, 16, 32, 48}, in every lane: the two wide steps of a butterfly (lane ^ 16, then
+// lane ^ 32, the order and therefore the bits of the shuffle form) through gfx950's row swaps: v_permlane16_swap exchanges the odd
+// rows of one operand with the even rows of the other, v_permlane32_swap the upper half with the lower half; one vector
+// instruction each and no LDS crossbar.
 __device__ __forceinline__ float quad_rows_sum(float v) {
     const uint32_t b = __float_as_uint(v);
-    const auto h = __builtin_amdgcn_permlane32_swap(b, b, false, false);      // {v of the lower half, v of the upper half} in both halves
+    const auto h = __builtin_amdgcn_permlane16_swap(b, b, false, false);      // {rows 0 0 2 2, rows 1 1 3 3}
     const uint32_t s = __float_as_uint(__uint_as_float(h[0]) + __uint_as_float(h[1]));
-    const auto r = __builtin_amdgcn_permlane16_swap(s, s, false, false);
+    const auto r = __builtin_amdgcn_permlane32_swap(s, s, false, false);      // {lower half twice, upper half twice}
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
 // Sum / maximum over aligned groups of WIDTH lanes (WIDTH a power of two <= 64); every lane gets the result.
+// the wide steps (lane ^ 16, lane ^ 32) of a commutative reduction through the row swaps: both halves of the swapped pair hold
+// the two values every lane needs, in one order or the other
+template <int OFF>
+__device__ __forceinline__ void swapped_pair(float v, float& a, float& b) {
+    const uint32_t bits = __float_as_uint(v);
+    if constexpr (OFF == 16) {
+        const auto h = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+        a = __uint_as_float(h[0]); b = __uint_as_float(h[1]);
+    } else {
+        const auto h = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+        a = __uint_as_float(h[0]); b = __uint_as_float(h[1]);
+    }
+}
 template <int WIDTH>
 __device__ __forceinline__ float group_sum(float v) {
     if constexpr (WIDTH > 1) v += butterfly_peer<1>(v);
     if constexpr (WIDTH > 2) v += butterfly_peer<2>(v);
     if constexpr (WIDTH > 4) v += butterfly_peer<4>(v);
     if constexpr (WIDTH > 8) v += butterfly_peer<8>(v);
-    if constexpr (WIDTH > 16) v += butterfly_peer<16>(v);
-    if constexpr (WIDTH > 32) v += butterfly_peer<32>(v);
+    float a, b;
+    if constexpr (WIDTH > 16) { swapped_pair<16>(v, a, b); v = a + b; }
+    if constexpr (WIDTH > 32) { swapped_pair<32>(v, a, b); v = a + b; }
     return v;
 }
 template <int WIDTH>
@@ -85,8 +100,9 @@ __device__ __forceinline__ float group_max(float v) {
     if constexpr (WIDTH > 2) v = fmaxf(v, butterfly_peer<2>(v));
     if constexpr (WIDTH > 4) v = fmaxf(v, butterfly_peer<4>(v));
     if constexpr (WIDTH > 8) v = fmaxf(v, butterfly_peer<8>(v));
-    if constexpr (WIDTH > 16) v = fmaxf(v, butterfly_peer<16>(v));
-    if constexpr (WIDTH > 32) v = fmaxf(v, butterfly_peer<32>(v));
+    float a, b;
+    if constexpr (WIDTH > 16) { swapped_pair<16>(v, a, b); v = fmaxf(a, b); }
+    if constexpr (WIDTH > 32) { swapped_pair<32>(v, a, b); v = fmaxf(a, b); }
     return v;
 }
 
