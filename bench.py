@@ -642,6 +642,55 @@ def fp8_gemm_pass(mod, dev) -> None:
     print(json.dumps({"fp8_gemm_pass": "fp8 x fp8 17408x5120, T=512 x8 then T=2048 x8", "flops_512": 2.0 * 512 * k * n, "flops_2048": 2.0 * 2048 * k * n}))
 
 
+def experts_rows_pass(mod, dev) -> None:
+    """A few launches of the grouped routed experts for the profiler: 256 tokens, 256 resident experts, top-8 (2048 routes),
+    IQ2_XXS gate/up 1536x3072 and IQ1_M down 3072x1536."""
+    from pocketllm_amd import block_codec as C, codebooks
+    rng = np.random.default_rng(7007)
+    e, d, inter, t = 256, 3072, 1536, 256
+    w1 = torch.from_numpy(C.random_iq2_xxs(rng, e, inter, d // 256, d_range=(0.002, 0.006))).to(dev)
+    w3 = torch.from_numpy(C.random_iq2_xxs(rng, e, inter, d // 256, d_range=(0.002, 0.006))).to(dev)
+    w2 = torch.from_numpy(C.random_iq1_m(rng, e, d, inter // 256, d_range=(0.002, 0.006))).to(dev)
+    logits = torch.from_numpy(rng.standard_normal((t, e)).astype(np.float32))
+    tw, ti = torch.softmax(logits, dim=-1).topk(8, dim=-1)
+    tw = (tw / tw.sum(dim=-1, keepdim=True)).to(dev)
+    _, toks, rws, seg = mod.moe_group_routes(ti.to(dev), tw, 0, e)
+    touched = int((seg[1:] > seg[:-1]).sum().item())
+    xt = torch.randn(t, d, device=dev, dtype=torch.bfloat16)
+    grids = (codebooks.get_iq2xxs_signed_grid_tensor().to(dev), codebooks.get_iq1_grid_tensor().to(dev))
+    for _ in range(6):
+        mod.gguf_moe_prefill_grouped_forward(xt, toks, rws, seg, w1, w3, w2, d, 0, d, 0, inter, 2, grids, 0.0)
+    torch.cuda.synchronize()
+    print(json.dumps({"experts_rows_pass": "iq2_xxs gate/up + iq1_m down, 256 experts top-8, T=256, 6 calls", "experts_touched": touched,
+                      "weight_bytes": touched * (2 * inter * (d // 256) * 66 + d * (inter // 256) * 56), "flops": 2.0 * t * 8 * 3 * inter * d}))
+
+
+def q8_gemm_pass(mod, dev) -> None:
+    """A few launches for the profiler of the two prefill forms that the streamed decode and tile kernels do not cover: the
+    int8-MFMA matmul on int8-quantized activations (Q4_K 17408x5120 at T=512 and T=2048) and the 17 - 48 row kernel (Q4_K and
+    Q5_K 5120x5120 and 17408x5120 at T=32)."""
+    from pocketllm_amd import block_codec as C
+    rng = np.random.default_rng(8008)
+    k = 5120
+    empty = torch.empty(0, dtype=torch.int8, device=dev)
+    for n in (5120, 17408):
+        w = rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02)
+        for tid, enc in ((3, C.quantize_q4_k), (4, C.quantize_q5_k)):
+            blocks = torch.from_numpy(enc(w)).to(dev)
+            x = torch.randn(32, k, device=dev, dtype=torch.bfloat16)
+            for _ in range(8):
+                mod.gguf_quant_gemm_prefill_forward(x, blocks, k, tid, empty)
+            if n == 17408 and tid == 3:
+                for t in (512, 2048):
+                    xt = torch.randn(t, k, device=dev, dtype=torch.bfloat16)
+                    for _ in range(6):
+                        mod.gguf_quant_gemm_q8_forward(xt, blocks, k, tid, empty)
+            del blocks
+    torch.cuda.synchronize()
+    print(json.dumps({"q8_gemm_pass": "q4_k / q5_k 5120x5120 and 17408x5120 at T=32 x8; q4_k 17408x5120 int8 activations T=512 x6, T=2048 x6",
+                      "ops_512": 2.0 * 512 * k * 17408, "ops_2048": 2.0 * 2048 * k * 17408}))
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -655,6 +704,8 @@ def main() -> None:
     ap.add_argument("--decode-pass", action="store_true", help="short run for rocprofv3: Q8_0, FP8, Q2_K, Q6_K and IQ4_XS decode matvec")
     ap.add_argument("--fp8-gemm-pass", action="store_true", help="short run for rocprofv3: native FP8 x FP8 matmul at T=512 and T=2048")
     ap.add_argument("--iq-pass", action="store_true", help="short run for rocprofv3: IQ2_XXS / IQ1_M matvec and the single-token experts")
+    ap.add_argument("--experts-rows-pass", action="store_true", help="short run for rocprofv3: grouped routed experts at T=256")
+    ap.add_argument("--q8-gemm-pass", action="store_true", help="short run for rocprofv3: int8-activation matmul at T=512 / 2048 and the 17 - 48 row kernel at T=32")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU (no sharding, no collectives); run with --gpus 1")
@@ -683,6 +734,12 @@ def main() -> None:
         return
     if args.fp8_gemm_pass:
         fp8_gemm_pass(mod, dev)
+        return
+    if args.experts_rows_pass:
+        experts_rows_pass(mod, dev)
+        return
+    if args.q8_gemm_pass:
+        q8_gemm_pass(mod, dev)
         return
     x_np = np.random.default_rng(2002).standard_normal((1, 5120), dtype=np.float32)
     x = torch.from_numpy(x_np).to(dev).to(torch.bfloat16)
