@@ -159,6 +159,30 @@ int pllm_gguf_quant_gemm_rmsnorm(const void* x, int x_dtype, const float* norm_w
 size_t pllm_gguf_quant_gemm_rmsnorm_workspace_bytes(int type_id, int64_t rows, int64_t k, int64_t n, int64_t blocks_per_row);
 
 /*
+ * Attention of one new token per sequence against a key/value store (a decode step), everything between the q / k / v projections
+ * and the output projection: RMS normalisation of q and k over their whole width (weights may be null: none), rotary phases
+ * out = x * cos_row + partner(x) * sin_row on the first rope_dim values of every head (partner = the value rope_dim / 2 away;
+ * cos_row / sin_row hold head_dim floats for position pos, sin_row with the sign of the first half; rope_dim 0: none), the new
+ * key and value rows written to position pos of the stores, softmax(q k^T / sqrt(head_dim)) v over positions 0 .. pos with every
+ * key/value head shared by heads / kv_heads query heads.  Replaces, for one query position, what the reference runs as separate
+ * framework operators in src/models/minimax_m2/architecture.py:158-266 (q_norm, k_norm, apply_rotary_emb, cache update,
+ * scaled_dot_product_attention).  Not a quantized operator: it is here because those ~17 small launches, not the matmuls,
+ * dominated a decoder block's step.
+ *
+ * q [batch, heads * head_dim], k_new / v_new [batch, kv_heads * head_dim], out [batch, heads * head_dim] and the stores
+ * [batch, kv_heads, capacity, head_dim] (strides in elements) all have type dtype (PLLM_F16 or PLLM_BF16); 16-byte aligned.
+ * head_dim must be 128, heads / kv_heads at most 8 (PLLM_ERR_UNSUPPORTED otherwise).  Float32 arithmetic; the normalized and the
+ * turned values are rounded to dtype where the separate operators round.  Two launches (one when pos < 64).
+ */
+size_t pllm_attention_decode_workspace_bytes(int64_t batch, int64_t heads, int64_t pos);
+int pllm_attention_decode(const void* q, const void* k_new, const void* v_new, int dtype,
+                          const float* q_norm_weight, const float* k_norm_weight, float eps,
+                          const float* cos_row, const float* sin_row, int64_t rope_dim,
+                          void* k_store, void* v_store, int64_t store_batch_stride, int64_t store_head_stride,
+                          int64_t batch, int64_t heads, int64_t kv_heads, int64_t head_dim, int64_t pos,
+                          void* out, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * The two halves of pllm_gguf_quant_gemm, for callers that feed one activation tensor to several
  * matrices (q/k/v, gate/up): quantize once into `image` (pllm_activation_image_bytes bytes, 256-byte
  * aligned), then run any number of matmuls against it (the decode kernels, whatever the row count).  They have no counterpart in the

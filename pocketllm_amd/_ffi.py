@@ -59,6 +59,9 @@ SIGNATURES = {
     "pllm_fp8_gemm_workspace_bytes": (_size_t, [_i64, _i64, _i64]),
     "pllm_fp8_gemm_ws": (_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _int, _i64, _i64, _i64, _c_void_p, _size_t, _c_void_p]),
     "pllm_fused_rms_norm": (_int, [_c_void_p, _int, _c_void_p, _c_void_p, _int, _i64, _i64, ctypes.c_float, _c_void_p]),
+    "pllm_attention_decode_workspace_bytes": (_size_t, [_i64, _i64, _i64]),
+    "pllm_attention_decode": (_int, [_c_void_p, _c_void_p, _c_void_p, _int, _c_void_p, _c_void_p, ctypes.c_float, _c_void_p, _c_void_p, _i64,
+                                     _c_void_p, _c_void_p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _c_void_p, _c_void_p, _size_t, _c_void_p]),
     "pllm_gguf_quant_gemm_rmsnorm": (_int, [_c_void_p, _int, _c_void_p, ctypes.c_float, _int, _c_void_p, _int, _c_void_p, _int,
                                             _i64, _i64, _i64, _i64, _c_void_p, _size_t, _c_void_p]),
     "pllm_gguf_quant_gemm_rmsnorm_workspace_bytes": (_size_t, [_int, _i64, _i64, _i64, _i64]),

@@ -44,6 +44,16 @@ class RotaryTable:
         self._cos = torch.cat((angle.cos(), angle.cos(), torch.ones(count, rest, device=self.device, dtype=torch.float64)), dim=1).float()
         self._sin = torch.cat((-angle.sin(), angle.sin(), torch.zeros(count, rest, device=self.device, dtype=torch.float64)), dim=1).float()
 
+    def rows(self, pos: int) -> tuple[torch.Tensor, torch.Tensor]:
+        """The cos and sin rows (float32, head_dim values each) of one position; all ones / zeros without a rotary part."""
+        if self.half == 0:
+            if self._cos is None:
+                self._cos = torch.ones(1, self.head_dim, device=self.device)
+                self._sin = torch.zeros(1, self.head_dim, device=self.device)
+            return self._cos[0], self._sin[0]
+        self.reserve(pos + 1)
+        return self._cos[pos], self._sin[pos]
+
     def rotate(self, x: torch.Tensor, first_pos: int) -> torch.Tensor:
         """x [batch, steps, heads, head_dim] at positions first_pos .. first_pos + steps - 1; returns a new tensor of x's dtype
         (float32 arithmetic, one rounding)."""

@@ -289,6 +289,33 @@ int pllm_fused_rms_norm(const void* x, int x_dtype, const float* weight, void* y
     return pllm::rms_norm_rows(x, x_dtype, weight, y, y_dtype, static_cast<int>(rows), static_cast<int>(dim), eps, static_cast<hipStream_t>(stream));
 }
 
+size_t pllm_attention_decode_workspace_bytes(int64_t batch, int64_t heads, int64_t pos) {
+    if (!fits_int(batch) || !fits_int(heads) || pos < 0 || pos >= 0x7fffffffLL) return 0;
+    return pllm::attention_decode_workspace_bytes(static_cast<int>(batch), static_cast<int>(heads), static_cast<int>(pos));
+}
+
+int pllm_attention_decode(const void* q, const void* k_new, const void* v_new, int dtype, const float* q_norm_weight, const float* k_norm_weight,
+                          float eps, const float* cos_row, const float* sin_row, int64_t rope_dim, void* k_store, void* v_store,
+                          int64_t store_batch_stride, int64_t store_head_stride, int64_t batch, int64_t heads, int64_t kv_heads, int64_t head_dim,
+                          int64_t pos, void* out, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!q || !k_new || !v_new || !k_store || !v_store || !out || (dtype != PLLM_F16 && dtype != PLLM_BF16)) return PLLM_ERR_INVALID_ARGUMENT;
+    if (!fits_int(batch) || !fits_int(heads) || !fits_int(kv_heads) || !fits_int(head_dim) || pos < 0 || pos >= 0x7fffffffLL || batch > 65535)
+        return PLLM_ERR_INVALID_ARGUMENT;
+    if (rope_dim < 0 || rope_dim > head_dim || (rope_dim > 0 && (!cos_row || !sin_row))) return PLLM_ERR_INVALID_ARGUMENT;
+    if (store_head_stride < (pos + 1) * head_dim || store_batch_stride < kv_heads * store_head_stride) return PLLM_ERR_INVALID_ARGUMENT;
+    if (!pllm::attention_decode_supports(static_cast<int>(heads), static_cast<int>(kv_heads), static_cast<int>(head_dim), static_cast<int>(rope_dim)))
+        return PLLM_ERR_UNSUPPORTED;
+    const uintptr_t all = reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k_new) | reinterpret_cast<uintptr_t>(v_new) |
+                          reinterpret_cast<uintptr_t>(k_store) | reinterpret_cast<uintptr_t>(v_store) | reinterpret_cast<uintptr_t>(out);
+    if ((all & 15u) || (store_batch_stride % 8) || (store_head_stride % 8)) return PLLM_ERR_INVALID_ARGUMENT;
+    const size_t need = pllm_attention_decode_workspace_bytes(batch, heads, pos);
+    if (need > 0 && (!workspace || workspace_bytes < need)) return PLLM_ERR_WORKSPACE;
+    return pllm::attention_decode(q, k_new, v_new, dtype, q_norm_weight, k_norm_weight, eps, cos_row, sin_row, static_cast<int>(rope_dim), k_store, v_store,
+                                  static_cast<size_t>(store_batch_stride), static_cast<size_t>(store_head_stride), static_cast<int>(batch),
+                                  static_cast<int>(heads), static_cast<int>(kv_heads), static_cast<int>(pos), out, workspace,
+                                  static_cast<hipStream_t>(stream));
+}
+
 // normalized rows (fp16) ahead of the matmul's own workspace when the call has too many rows for the in-kernel form
 static size_t rmsnorm_rows_bytes(int64_t rows, int64_t k) {
     return rows <= kInKernelQuantMaxRows ? 0 : (static_cast<size_t>(rows) * static_cast<size_t>(k) * 2 + 255) & ~static_cast<size_t>(255);

@@ -41,6 +41,12 @@ int swiglu_image_256(const void* gate, const void* up, int gu_dtype, float limit
                      hipStream_t stream);
 // y[r, :] = x[r, :] * rsqrt(mean(x[r, :]^2) + eps) * weight (float32 arithmetic, one rounding to y_dtype)
 int rms_norm_rows(const void* x, int x_dtype, const float* weight, void* y, int y_dtype, int rows, int dim, float eps, hipStream_t stream);
+// one decode step of attention (attn_decode.hip): normalisation, rotary phases, store update, grouped-query softmax attention
+size_t attention_decode_workspace_bytes(int batch, int heads, int pos);
+bool attention_decode_supports(int heads, int kv_heads, int head_dim, int rope_dim);
+int attention_decode(const void* q, const void* k_new, const void* v_new, int dtype, const float* q_weight, const float* k_weight, float eps,
+                     const float* cos_row, const float* sin_row, int rope_dim, void* k_store, void* v_store, size_t batch_stride,
+                     size_t head_stride, int batch, int heads, int kv_heads, int pos, void* out, void* workspace, hipStream_t stream);
 size_t act_image_q8pair_bytes(int pairs);
 int act_image_q8pair(const void* x, int x_dtype, int rows, int k, int pairs, void* image, hipStream_t stream);
 

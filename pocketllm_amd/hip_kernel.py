@@ -289,6 +289,48 @@ def fused_rms_norm_forward(x: torch.Tensor, weight: torch.Tensor, eps: float, *,
     return y
 
 
+def attention_decode_forward(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor, keys: torch.Tensor, values: torch.Tensor, pos: int, *,
+                             q_norm_weight: torch.Tensor | None = None, k_norm_weight: torch.Tensor | None = None, eps: float = 1e-6,
+                             cos_row: torch.Tensor | None = None, sin_row: torch.Tensor | None = None, rope_dim: int = 0) -> torch.Tensor:
+    """One decode step of grouped-query attention (the framework operators of src/models/minimax_m2/architecture.py:158-266 for
+    one query position): q [batch, heads * head_dim], k_new / v_new [batch, kv_heads * head_dim]; keys / values
+    [>= batch, kv_heads, capacity, head_dim] are the stores, whose position `pos` this call writes.  RMS normalisation of q and k
+    over their whole width when weights are given, rotary phases from the float32 rows cos_row / sin_row (head_dim values each
+    for this position).  Returns [batch, heads * head_dim] in q's dtype."""
+    _check(q.dim() == 2 and k_new.dim() == 2 and v_new.dim() == 2, "attention_decode: q, k_new, v_new must be 2D [batch, width]")
+    _check(keys.dim() == 4 and values.shape == keys.shape, "attention_decode: stores must be [batch, kv_heads, capacity, head_dim]")
+    _check(q.dtype in (torch.float16, torch.bfloat16), "attention_decode: float16 or bfloat16 only")
+    _check(all(t.dtype == q.dtype for t in (k_new, v_new, keys, values)), "attention_decode: one dtype for q, k, v and the stores")
+    _check(all(t.is_cuda for t in (q, k_new, v_new, keys, values)), "attention_decode: tensors must be CUDA tensors")
+    batch, kv_heads, capacity, head_dim = q.size(0), keys.size(1), keys.size(2), keys.size(3)
+    pos = int(pos)
+    _check(0 <= pos < capacity and keys.size(0) >= batch, "attention_decode: position or batch outside the stores")
+    _check(q.size(1) % head_dim == 0 and k_new.shape == (batch, kv_heads * head_dim) and v_new.shape == k_new.shape,
+           "attention_decode: widths do not match the stores")
+    heads = q.size(1) // head_dim
+    _check(keys.stride(3) == 1 and keys.stride(2) == head_dim and values.stride() == keys.stride(), "attention_decode: stores must be dense per head")
+    for w, width in ((q_norm_weight, heads * head_dim), (k_norm_weight, kv_heads * head_dim)):
+        _check(w is None or (w.is_cuda and w.dtype == torch.float32 and w.is_contiguous() and w.numel() == width), "attention_decode: norm weights must be fp32 [width]")
+    if rope_dim:
+        for r in (cos_row, sin_row):
+            _check(r is not None and r.is_cuda and r.dtype == torch.float32 and r.is_contiguous() and r.numel() == head_dim,
+                   "attention_decode: cos_row / sin_row must be fp32 [head_dim]")
+    q, k_new, v_new = q.contiguous(), k_new.contiguous(), v_new.contiguous()
+    out = torch.empty_like(q)
+    lib = _lib()
+    need = lib.pllm_attention_decode_workspace_bytes(batch, heads, pos)
+    ws = _workspace(need, q.device)
+    with _on_device(q.device):
+        st = lib.pllm_attention_decode(q.data_ptr(), k_new.data_ptr(), v_new.data_ptr(), _DTYPE_CODE[q.dtype],
+                                       None if q_norm_weight is None else q_norm_weight.data_ptr(),
+                                       None if k_norm_weight is None else k_norm_weight.data_ptr(), float(eps),
+                                       None if not rope_dim else cos_row.data_ptr(), None if not rope_dim else sin_row.data_ptr(), int(rope_dim),
+                                       keys.data_ptr(), values.data_ptr(), keys.stride(0), keys.stride(1), batch, heads, kv_heads, head_dim, pos,
+                                       out.data_ptr(), ws.data_ptr(), need, _stream(q.device))
+    _ffi.check(st, "attention_decode_forward")
+    return out
+
+
 def gguf_quant_gemm_rmsnorm_forward(x, norm_weight, eps, blocks, row_elems, type_id, signed_grid, *, round_fp16: bool = True,
                                     out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
     """gguf_quant_gemm_forward(fused_rms_norm_forward(x, norm_weight, eps), ...) as one operator (decode: one launch).

@@ -136,6 +136,9 @@ class MiniMaxAttention:
         qkv = (q_proj.tensor, k_proj.tensor, v_proj.tensor)
         # one launch for the three projections needs one format (not Q2_K) and one row length
         self._fused_qkv = len({(int(t.type_id), int(t.blocks.size(1))) for t in qkv}) == 1 and int(qkv[0].type_id) != 1
+        # the one-operator decode step: 128-wide heads, groups of up to 8, 16-bit stores, both normalisations with one eps
+        self._fused_step = (args.head_dim == 128 and args.n_heads % args.n_kv_heads == 0 and args.n_heads // args.n_kv_heads <= 8 and
+                            dtype in (torch.float16, torch.bfloat16) and q_norm.eps == k_norm.eps and self._cuda is not None and dev.type == "cuda")
 
     def reset_cache(self, batch_size: int, max_seq_len: int) -> None:
         self.store.allocate(batch_size, max_seq_len)
@@ -158,6 +161,14 @@ class MiniMaxAttention:
         a = self.args
         batch, steps = x.size(0), x.size(1)
         q, k, v = self.project_qkv(x, input_norm)
+        if steps == 1 and self._fused_step:
+            # a decode step: normalisation, rotary phases, store update and attention in one operator (two launches)
+            self.store.ensure(batch, start_pos + 1)
+            cos_row, sin_row = self.rotary.rows(start_pos)
+            return self._cuda.attention_decode_forward(
+                q.view(batch, -1).to(self.dtype), k.view(batch, -1).to(self.dtype), v.view(batch, -1).to(self.dtype), self.store.keys, self.store.values,
+                start_pos, q_norm_weight=self.q_norm.weight, k_norm_weight=self.k_norm.weight, eps=self.q_norm.eps, cos_row=cos_row, sin_row=sin_row,
+                rope_dim=2 * self.rotary.half).view(batch, 1, -1)
         q = self.rotary.rotate(self.q_norm(q).view(batch, steps, a.n_heads, a.head_dim), start_pos)
         k = self.rotary.rotate(self.k_norm(k).view(batch, steps, a.n_kv_heads, a.head_dim), start_pos)
         self.store.write(k, v.view(batch, steps, a.n_kv_heads, a.head_dim).to(self.dtype), start_pos)

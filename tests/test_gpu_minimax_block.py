@@ -171,3 +171,22 @@ def test_transformer_stack_prefill_then_decode():
         assert O.rel_l2(got, want) <= 2e-2, (step, O.rel_l2(got, want))
     nxt = model(torch.tensor([[3]]), 7, return_next_token=True)
     assert nxt.shape == (1,) and 0 <= int(nxt[0]) < vocab
+
+
+def test_decoder_block_decode_steps_use_the_one_operator_attention():
+    """128-wide heads: decode steps run normalisation, rotary phases, store update and attention as one operator
+    (attention_decode_forward); the prefill before them and the oracle are as above."""
+    assert load_cuda_kernel() is not None and torch.cuda.is_available()
+    rng = np.random.default_rng(33)
+    a = MiniMaxM2Args(dim=512, n_heads=6, n_kv_heads=2, head_dim=128, rope_dim=64, rope_base=10000.0, n_routed_experts=8, top_k=2,
+                      moe_inter_dim=256, norm_eps=1e-6)
+    block, oracle = _small_layer(rng, a, "wide")
+    assert block.attention._fused_step
+    block.reset_cache(1, 80)
+    steps = [(rng.standard_normal((70, a.dim)).astype(np.float32), 0)] + [(rng.standard_normal((1, a.dim)).astype(np.float32), 70 + i) for i in range(3)]
+    for x_np, start in steps:
+        x = torch.from_numpy(x_np).to(DEV).to(torch.float16)
+        print(f"case wide-head decoder block tokens={x_np.shape[0]} start={start}", flush=True)
+        got = block(x.view(1, -1, a.dim), start).float().cpu().numpy()[0]
+        want = oracle(x.float().cpu().numpy().astype(np.float64), start)
+        assert O.rel_l2(got, want) <= 1e-2, (start, O.rel_l2(got, want))
