@@ -171,7 +171,7 @@ size_t pllm_gguf_quant_gemm_rmsnorm_workspace_bytes(int type_id, int64_t rows, i
  *
  * q [batch, heads * head_dim], k_new / v_new [batch, kv_heads * head_dim], out [batch, heads * head_dim] and the stores
  * [batch, kv_heads, capacity, head_dim] (strides in elements) all have type dtype (PLLM_F16 or PLLM_BF16); 16-byte aligned.
- * head_dim must be 128, heads / kv_heads at most 8 (PLLM_ERR_UNSUPPORTED otherwise).  Float32 arithmetic; the normalized and the
+ * head_dim must be 128, heads at most 64, heads / kv_heads at most 8, pos below 131072 (PLLM_ERR_UNSUPPORTED otherwise).  Float32 arithmetic; the normalized and the
  * turned values are rounded to dtype where the separate operators round.  Two launches (one when pos < 64).
  */
 size_t pllm_attention_decode_workspace_bytes(int64_t batch, int64_t heads, int64_t pos);

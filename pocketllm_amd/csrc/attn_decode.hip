@@ -20,18 +20,28 @@ namespace {
 constexpr int kHeadDim = 128;
 constexpr int kSliceKeys = 64;
 constexpr int kMaxGroup = 8;
+constexpr int kMaxHeads = 64;                  // q rows of up to 64 x 128 values (four 16-byte pieces per thread)
+constexpr int kQPieces = kMaxHeads * kHeadDim / (8 * 256), kKPieces = 2;   // k rows of up to 32 x 128 values
 constexpr int kPartFloats = kHeadDim + 2;     // a slice's result per query head: 128 weighted sums, running maximum, sum of weights
 
-__device__ __forceinline__ float half_bits_to_float(uint32_t bits, bool bf16) {
-    return bf16 ? __uint_as_float(bits << 16) : f16_bits_to_float(bits);
-}
-__device__ __forceinline__ uint16_t float_to_half_bits(float v, bool bf16) {
-    if (bf16) return from_float<bf16_t>(v).bits;
-    union { _Float16 h; uint16_t u; } c;
-    c.h = static_cast<_Float16>(v);
-    return c.u;
-}
-__device__ __forceinline__ void unpack8(const uint4& u, bool bf16, float v[8]) {
+template <bool BF16> struct HalfBits {
+    static __device__ __forceinline__ float to_float(uint32_t bits) {
+        if constexpr (BF16) return __uint_as_float(bits << 16);
+        else return f16_bits_to_float(bits);
+    }
+    static __device__ __forceinline__ uint16_t from(float v) {
+        if constexpr (BF16) return from_float<bf16_t>(v).bits;
+        else {
+            union { _Float16 h; uint16_t u; } c;
+            c.h = static_cast<_Float16>(v);
+            return c.u;
+        }
+    }
+};
+#define half_bits_to_float(bits, bf16) HalfBits<bf16>::to_float(bits)
+#define float_to_half_bits(v, bf16) HalfBits<bf16>::from(v)
+template <bool bf16>
+__device__ __forceinline__ void unpack8(const uint4& u, float v[8]) {
     const uint32_t w[4] = {u.x, u.y, u.z, u.w};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -54,6 +64,8 @@ __device__ __forceinline__ void block_sum2(float& a, float& b, float* red) {
     b = (red[4] + red[5]) + (red[6] + red[7]);
 }
 
+__device__ const float kOne = 1.0f;
+
 struct DecodeArgs {
     const uint16_t* q; const uint16_t* k_new; const uint16_t* v_new;
     const float* q_weight; const float* k_weight;               // RMS normalisation weights over the whole q / k width, or null
@@ -66,17 +78,20 @@ struct DecodeArgs {
     int bf16, heads, kv_heads, rope_half, pos, slices;
 };
 
+// GROUP: the query heads per key/value head the loops are unrolled for (at least the launch's heads / kv_heads)
+template <bool bf16, int GROUP>
 __global__ __launch_bounds__(256) void attn_decode_slice_kernel(const DecodeArgs a) {
     __shared__ float red[8];
     __shared__ __align__(16) float qn[kMaxGroup][kHeadDim];                   // normalized, turned, scaled queries of this key/value head's group
     __shared__ __align__(16) uint16_t new_key[kHeadDim], new_value[kHeadDim]; // the new row as the store holds it
+    __shared__ __align__(16) uint16_t raw_q[kMaxGroup * kHeadDim], raw_k[kHeadDim];   // the group's q heads and this head's k as they came
+    __shared__ float w_q[kMaxGroup * kHeadDim], w_k[kHeadDim], rot_cos[kHeadDim], rot_sin[kHeadDim];
     __shared__ float weight[kMaxGroup][kSliceKeys];                           // scores, then softmax weights
     __shared__ float stats[kMaxGroup][2];
     __shared__ __align__(16) float sums[8][kMaxGroup][kHeadDim];              // weighted value sums per group of eight keys
 
     const int slice = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
     const int tid = threadIdx.x;
-    const bool bf16 = a.bf16 != 0;
     const int group = a.heads / a.kv_heads;
     const int length = a.pos + 1;
     const int j0 = slice * kSliceKeys;
@@ -88,68 +103,94 @@ __global__ __launch_bounds__(256) void attn_decode_slice_kernel(const DecodeArgs
 
     // stored keys and values of the slice first: they are the long round trip.  Keys: thread (key tid / 4, quarter tid % 4) holds
     // 32 values; values: thread (keys 8 (tid / 32) .. + 7, columns 4 (tid % 32) .. + 3).  The new position is not in memory yet.
+    // Every load has a valid address whatever the thread's share (row numbers clamped to the new position, whose row exists and is
+    // replaced below): no load stands under a condition, so all of them are in flight together.
     const int key = tid >> 2, quarter = tid & 3;
-    uint4 kreg[4] = {};
-    const bool key_stored = key < nkeys && j0 + key != a.pos;
-    if (key_stored) {
-        const uint4* src = reinterpret_cast<const uint4*>(kbase + static_cast<size_t>(j0 + key) * kHeadDim + 32 * quarter);
+    uint4 kreg[4];
+    {
+        const uint4* src = reinterpret_cast<const uint4*>(kbase + static_cast<size_t>(min(j0 + key, a.pos)) * kHeadDim + 32 * quarter);
 #pragma unroll
         for (int i = 0; i < 4; ++i) kreg[i] = src[i];
     }
     const int kg = tid >> 5, dpart = tid & 31;
-    uint2 vreg[8] = {};
+    uint2 vreg[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const int j = 8 * kg + i;
-        if (j < nkeys && j0 + j != a.pos) vreg[i] = *reinterpret_cast<const uint2*>(vbase + static_cast<size_t>(j0 + j) * kHeadDim + 4 * dpart);
-    }
+    for (int i = 0; i < 8; ++i)
+        vreg[i] = *reinterpret_cast<const uint2*>(vbase + static_cast<size_t>(min(j0 + 8 * kg + i, a.pos)) * kHeadDim + 4 * dpart);
 
-    // sums of squares of the whole q and k rows of this sequence
+    // the q row, this head's k row, the group's normalisation weights and the rotary rows: requested in one batch behind the
+    // stores' rows, staged in LDS as they are, so that the whole prologue costs one round trip to memory
     const uint16_t* qrow = a.q + static_cast<size_t>(b) * a.heads * kHeadDim;
     const uint16_t* krow = a.k_new + static_cast<size_t>(b) * a.kv_heads * kHeadDim;
+    const int q_width = a.heads * kHeadDim, k_width = a.kv_heads * kHeadDim;
+    uint4 qpiece[kQPieces], kpiece[kKPieces];
+#pragma unroll
+    for (int r = 0; r < kQPieces; ++r) qpiece[r] = *reinterpret_cast<const uint4*>(qrow + min(8 * (tid + 256 * r), q_width - 8));
+#pragma unroll
+    for (int r = 0; r < kKPieces; ++r) kpiece[r] = *reinterpret_cast<const uint4*>(krow + min(8 * (tid + 256 * r), k_width - 8));
+    const float* qw_src = a.q_weight ? a.q_weight + kvh * group * kHeadDim : &kOne;    // null weights: read a one, stride zero
+    const int qw_last = a.q_weight ? group * kHeadDim - 1 : 0;
+    float qw_reg[kMaxGroup * kHeadDim / 256];
+#pragma unroll
+    for (int r = 0; r < kMaxGroup * kHeadDim / 256; ++r) qw_reg[r] = qw_src[min(tid + 256 * r, qw_last)];
+    const float kw_reg = a.k_weight ? a.k_weight[kvh * kHeadDim + (tid & (kHeadDim - 1))] : 1.0f;
+    const float rot_reg = a.cos_row ? (tid < kHeadDim ? a.cos_row[tid] : a.sin_row[tid - kHeadDim]) : (tid < kHeadDim ? 1.0f : 0.0f);
+    const uint16_t v_bits = a.v_new[static_cast<size_t>(b) * k_width + kvh * kHeadDim + (tid & (kHeadDim - 1))];
+
+    // sums of squares of the whole q and k rows; the group's part of q and this head's k go to LDS on the way
     float ssq = 0.0f, ssk = 0.0f;
-    if (a.q_weight)
-        for (int i = 8 * tid; i < a.heads * kHeadDim; i += 8 * 256) {
-            float v[8];
-            unpack8(*reinterpret_cast<const uint4*>(qrow + i), bf16, v);
+#pragma unroll
+    for (int r = 0; r < kQPieces; ++r) {
+        float v[8];
+        unpack8<bf16>(qpiece[r], v);
+        if (8 * (tid + 256 * r) < q_width)
 #pragma unroll
             for (int e = 0; e < 8; ++e) ssq += v[e] * v[e];
-        }
-    if (a.k_weight)
-        for (int i = 8 * tid; i < a.kv_heads * kHeadDim; i += 8 * 256) {
-            float v[8];
-            unpack8(*reinterpret_cast<const uint4*>(krow + i), bf16, v);
+        const int at = 8 * (tid + 256 * r) - kvh * group * kHeadDim;          // position inside the group's part
+        if (at >= 0 && at < group * kHeadDim) *reinterpret_cast<uint4*>(&raw_q[at]) = qpiece[r];
+    }
+#pragma unroll
+    for (int r = 0; r < kKPieces; ++r) {
+        float v[8];
+        unpack8<bf16>(kpiece[r], v);
+        if (8 * (tid + 256 * r) < k_width)
 #pragma unroll
             for (int e = 0; e < 8; ++e) ssk += v[e] * v[e];
-        }
-    block_sum2(ssq, ssk, red);
-    const float rstd_q = a.q_weight ? rsqrtf(ssq / static_cast<float>(a.heads * kHeadDim) + a.eps) : 1.0f;
-    const float rstd_k = a.k_weight ? rsqrtf(ssk / static_cast<float>(a.kv_heads * kHeadDim) + a.eps) : 1.0f;
+        const int at = 8 * (tid + 256 * r) - kvh * kHeadDim;
+        if (at >= 0 && at < kHeadDim) *reinterpret_cast<uint4*>(&raw_k[at]) = kpiece[r];
+    }
+#pragma unroll
+    for (int r = 0; r < kMaxGroup * kHeadDim / 256; ++r)
+        if (tid + 256 * r < group * kHeadDim) w_q[tid + 256 * r] = qw_reg[r];
+    if (tid < kHeadDim) { w_k[tid] = kw_reg; rot_cos[tid] = rot_reg; }
+    else rot_sin[tid - kHeadDim] = rot_reg;
+    block_sum2(ssq, ssk, red);                                                // (its barrier also covers the staging above)
+    const float rstd_q = a.q_weight ? rsqrtf(ssq / static_cast<float>(q_width) + a.eps) : 1.0f;
+    const float rstd_k = a.k_weight ? rsqrtf(ssk / static_cast<float>(k_width) + a.eps) : 1.0f;
 
-    // one normalized value of a row: x * rstd * weight, rounded to the activations' type like a separate normalisation's output
-    auto normed = [&](const uint16_t* row, const float* w, float rstd, int i) {
-        const float x = half_bits_to_float(row[i], bf16);
-        if (!w) return x;
-        return half_bits_to_float(float_to_half_bits(x * rstd * w[i], bf16), bf16);
+    // one normalized value: x * rstd * weight, rounded to the activations' type like a separate normalisation's output; then the
+    // turn out = x cos + partner sin, rounded again like a separate rotary operator's output
+    auto normed = [&](const uint16_t* raw, const float* w, bool on, float rstd, int i) {
+        const float x = half_bits_to_float(raw[i], bf16);
+        return on ? half_bits_to_float(float_to_half_bits(x * rstd * w[i], bf16), bf16) : x;
     };
-    auto turned = [&](const uint16_t* row, const float* w, float rstd, int head, int d) {
-        const float x = normed(row, w, rstd, head * kHeadDim + d);
+    auto turned = [&](const uint16_t* raw, const float* w, bool on, float rstd, int head_at, int d) {
+        const float x = normed(raw, w, on, rstd, head_at + d);
         if (!a.cos_row) return x;
-        const float xp = normed(row, w, rstd, head * kHeadDim + rotary_partner(d, a.rope_half));
-        return half_bits_to_float(float_to_half_bits(__builtin_fmaf(xp, a.sin_row[d], x * a.cos_row[d]), bf16), bf16);
+        const float xp = normed(raw, w, on, rstd, head_at + rotary_partner(d, a.rope_half));
+        return half_bits_to_float(float_to_half_bits(__builtin_fmaf(xp, rot_sin[d], x * rot_cos[d]), bf16), bf16);
     };
-    for (int e = tid; e < group * kHeadDim; e += 256) {
+    for (int e = tid; e < GROUP * kHeadDim; e += 256) {
         const int g = e / kHeadDim, d = e % kHeadDim;
-        qn[g][d] = turned(qrow, a.q_weight, rstd_q, kvh * group + g, d) * a.scale;
+        qn[g][d] = g < group ? turned(raw_q, w_q, a.q_weight != nullptr, rstd_q, g * kHeadDim, d) * a.scale : 0.0f;
     }
     if (has_new && tid < kHeadDim) {
-        const uint16_t kb = float_to_half_bits(turned(krow, a.k_weight, rstd_k, kvh, tid), bf16);
-        const uint16_t vb = a.v_new[static_cast<size_t>(b) * a.kv_heads * kHeadDim + kvh * kHeadDim + tid];
+        const uint16_t kb = float_to_half_bits(turned(raw_k, w_k, a.k_weight != nullptr, rstd_k, 0, tid), bf16);
         new_key[tid] = kb;
-        new_value[tid] = vb;
+        new_value[tid] = v_bits;
         const size_t at = static_cast<size_t>(b) * a.batch_stride + static_cast<size_t>(kvh) * a.head_stride + static_cast<size_t>(a.pos) * kHeadDim + tid;
         a.k_store[at] = kb;
-        a.v_store[at] = vb;
+        a.v_store[at] = v_bits;
     }
     __syncthreads();
 
@@ -162,20 +203,26 @@ __global__ __launch_bounds__(256) void attn_decode_slice_kernel(const DecodeArgs
     {
         float kv[32];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) unpack8(kreg[i], bf16, kv + 8 * i);
-        for (int g = 0; g < group; ++g) {
-            const float4* qv = reinterpret_cast<const float4*>(&qn[g][32 * quarter]);
-            float s = 0.0f;
+        for (int i = 0; i < 4; ++i) unpack8<bf16>(kreg[i], kv + 8 * i);
+        // the heads side by side: GROUP independent sums per pass over the key's values (rows of qn beyond the group hold
+        // zeros and are not stored)
+        float s[GROUP];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const float4 q4 = qv[i];
-                s = __builtin_fmaf(q4.x, kv[4 * i], s);
-                s = __builtin_fmaf(q4.y, kv[4 * i + 1], s);
-                s = __builtin_fmaf(q4.z, kv[4 * i + 2], s);
-                s = __builtin_fmaf(q4.w, kv[4 * i + 3], s);
+        for (int g = 0; g < GROUP; ++g) s[g] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+            for (int g = 0; g < GROUP; ++g) {
+                const float4 q4 = *reinterpret_cast<const float4*>(&qn[g][32 * quarter + 4 * i]);
+                s[g] = __builtin_fmaf(q4.x, kv[4 * i], s[g]);
+                s[g] = __builtin_fmaf(q4.y, kv[4 * i + 1], s[g]);
+                s[g] = __builtin_fmaf(q4.z, kv[4 * i + 2], s[g]);
+                s[g] = __builtin_fmaf(q4.w, kv[4 * i + 3], s[g]);
             }
-            s = group_sum<4>(s);
-            if (quarter == 0) weight[g][key] = key < nkeys ? s : -INFINITY;
+#pragma unroll
+        for (int g = 0; g < GROUP; ++g) {
+            const float t = group_sum<4>(s[g]);
+            if (quarter == 0 && g < group) weight[g][key] = key < nkeys ? t : -INFINITY;
         }
     }
     __syncthreads();
@@ -196,28 +243,29 @@ __global__ __launch_bounds__(256) void attn_decode_slice_kernel(const DecodeArgs
 
     // weighted sums of the values: eight keys and four columns per thread
     {
-        float acc[kMaxGroup][4] = {};
+        float acc[GROUP][4] = {};
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const int j = 8 * kg + i;
             if (j < nkeys) {                 // uniform over the 32 threads of a key group
-                uint2 bits = vreg[i];
-                if (j0 + j == a.pos) bits = *reinterpret_cast<const uint2*>(new_value + 4 * dpart);
+                const uint2 fresh = *reinterpret_cast<const uint2*>(new_value + 4 * dpart);
+                const uint2 bits = j0 + j == a.pos ? fresh : vreg[i];
                 const float v0 = half_bits_to_float(bits.x & 0xffffu, bf16), v1 = half_bits_to_float(bits.x >> 16, bf16);
                 const float v2 = half_bits_to_float(bits.y & 0xffffu, bf16), v3 = half_bits_to_float(bits.y >> 16, bf16);
 #pragma unroll
-                for (int g = 0; g < kMaxGroup; ++g)
-                    if (g < group) {
-                        const float p = weight[g][j];
+                for (int g = 0; g < GROUP; ++g) {
+                    {
+                        const float p = g < group ? weight[g][j] : 0.0f;
                         acc[g][0] = __builtin_fmaf(p, v0, acc[g][0]);
                         acc[g][1] = __builtin_fmaf(p, v1, acc[g][1]);
                         acc[g][2] = __builtin_fmaf(p, v2, acc[g][2]);
                         acc[g][3] = __builtin_fmaf(p, v3, acc[g][3]);
                     }
+                }
             }
         }
 #pragma unroll
-        for (int g = 0; g < kMaxGroup; ++g)
+        for (int g = 0; g < GROUP; ++g)
             if (g < group) *reinterpret_cast<float4*>(&sums[kg][g][4 * dpart]) = make_float4(acc[g][0], acc[g][1], acc[g][2], acc[g][3]);
     }
     __syncthreads();
@@ -237,20 +285,42 @@ __global__ __launch_bounds__(256) void attn_decode_slice_kernel(const DecodeArgs
     }
 }
 
-// out[b, head, :] = sum over slices of sums * exp(m - M) / sum over slices of l * exp(m - M), slices in order
+// out[b, head, :] = sum over slices of sums * exp(m - M) / sum over slices of l * exp(m - M), slices in order.
+// The slices' statistics are fetched side by side (one round trip), the sums in batches of eight.
+constexpr int kMaxSlices = 2048;                // stores of up to 131072 positions
 __global__ __launch_bounds__(kHeadDim) void attn_decode_merge_kernel(const float* __restrict__ part, uint16_t* __restrict__ out, int slices, int bf16) {
+    __shared__ float factor[kMaxSlices];
+    __shared__ float wave_top[2], wave_den[2];
     const size_t row = blockIdx.x;                                            // b * heads + head
     const float* src = part + row * slices * kPartFloats;
     const int d = threadIdx.x;
     float top = -INFINITY;
-    for (int s = 0; s < slices; ++s) top = fmaxf(top, src[s * kPartFloats + kHeadDim]);
-    float num = 0.0f, den = 0.0f;
-    for (int s = 0; s < slices; ++s) {
-        const float f = expf(src[s * kPartFloats + kHeadDim] - top);
-        num = __builtin_fmaf(src[s * kPartFloats + d], f, num);
+    for (int s = d; s < slices; s += kHeadDim) { const float m = src[s * kPartFloats + kHeadDim]; factor[s] = m; top = fmaxf(top, m); }
+    top = group_max<64>(top);
+    if ((d & 63) == 0) wave_top[d >> 6] = top;
+    __syncthreads();
+    top = fmaxf(wave_top[0], wave_top[1]);
+    float den = 0.0f;
+    for (int s = d; s < slices; s += kHeadDim) {
+        const float f = expf(factor[s] - top);
+        factor[s] = f;
         den = __builtin_fmaf(src[s * kPartFloats + kHeadDim + 1], f, den);
     }
-    out[row * kHeadDim + d] = float_to_half_bits(num / den, bf16 != 0);
+    den = group_sum<64>(den);
+    if ((d & 63) == 0) wave_den[d >> 6] = den;
+    __syncthreads();
+    den = wave_den[0] + wave_den[1];
+    float num = 0.0f;
+    int s = 0;
+    for (; s + 8 <= slices; s += 8) {
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = src[(s + i) * kPartFloats + d];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) num = __builtin_fmaf(v[i], factor[s + i], num);
+    }
+    for (; s < slices; ++s) num = __builtin_fmaf(src[s * kPartFloats + d], factor[s], num);
+    out[row * kHeadDim + d] = bf16 ? HalfBits<true>::from(num / den) : HalfBits<false>::from(num / den);
 }
 
 }  // namespace
@@ -261,8 +331,8 @@ size_t attention_decode_workspace_bytes(int batch, int heads, int pos) {
 }
 
 bool attention_decode_supports(int heads, int kv_heads, int head_dim, int rope_dim) {
-    return head_dim == kHeadDim && kv_heads >= 1 && heads % kv_heads == 0 && heads / kv_heads <= kMaxGroup && rope_dim >= 0 &&
-           rope_dim <= kHeadDim && rope_dim % 2 == 0;
+    return head_dim == kHeadDim && kv_heads >= 1 && heads % kv_heads == 0 && heads / kv_heads <= kMaxGroup && heads <= kMaxHeads &&
+           kv_heads * kHeadDim <= kKPieces * 8 * 256 && rope_dim >= 0 && rope_dim <= kHeadDim && rope_dim % 2 == 0;
 }
 
 int attention_decode(const void* q, const void* k_new, const void* v_new, int dtype, const float* q_weight, const float* k_weight, float eps,
@@ -279,7 +349,16 @@ int attention_decode(const void* q, const void* k_new, const void* v_new, int dt
     a.eps = eps; a.scale = 1.0f / sqrtf(static_cast<float>(kHeadDim));
     a.bf16 = dtype == PLLM_BF16; a.heads = heads; a.kv_heads = kv_heads; a.rope_half = rope_dim / 2; a.pos = pos;
     a.slices = pos / kSliceKeys + 1;
-    hipLaunchKernelGGL(attn_decode_slice_kernel, dim3(a.slices, kv_heads, batch), dim3(256), 0, stream, a);
+    if (a.slices > kMaxSlices) return PLLM_ERR_UNSUPPORTED;
+    const int group = heads / kv_heads;
+    const dim3 grid(a.slices, kv_heads, batch);
+#define PLLM_CASE(G) \
+    if (group <= G) { \
+        if (a.bf16) hipLaunchKernelGGL((attn_decode_slice_kernel<true, G>), grid, dim3(256), 0, stream, a); \
+        else hipLaunchKernelGGL((attn_decode_slice_kernel<false, G>), grid, dim3(256), 0, stream, a); \
+    } else
+    PLLM_CASE(1) PLLM_CASE(2) PLLM_CASE(4) PLLM_CASE(6) PLLM_CASE(8) return PLLM_ERR_UNSUPPORTED;
+#undef PLLM_CASE
     if (hipGetLastError() != hipSuccess) return PLLM_ERR_LAUNCH;
     if (a.slices > 1) {
         hipLaunchKernelGGL(attn_decode_merge_kernel, dim3(batch * heads), dim3(kHeadDim), 0, stream, a.part, a.out, a.slices, a.bf16);

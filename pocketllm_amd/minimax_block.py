@@ -161,7 +161,7 @@ class MiniMaxAttention:
         a = self.args
         batch, steps = x.size(0), x.size(1)
         q, k, v = self.project_qkv(x, input_norm)
-        if steps == 1 and self._fused_step:
+        if steps == 1 and self._fused_step and start_pos < 131072:
             # a decode step: normalisation, rotary phases, store update and attention in one operator (two launches)
             self.store.ensure(batch, start_pos + 1)
             cos_row, sin_row = self.rotary.rows(start_pos)
