@@ -97,7 +97,9 @@ class MiniMaxMoE:
         """architecture.py:291-298 as one operator: sigmoid scores, bias for the selection only, top-k, renormalised weights."""
         return self._cuda.moe_route(x_flat, self.gate_weight, self.gate_bias, int(self.args.top_k))
 
-    def __call__(self, x: torch.Tensor) -> torch.Tensor:
+    def __call__(self, x: torch.Tensor, residual: torch.Tensor | None = None) -> torch.Tensor:
+        """The experts' output for x in the model's dtype; with `residual` (x's shape, the model's dtype) it is added into that
+        tensor, which is returned."""
         tokens = x.reshape(-1, x.size(-1)).contiguous()
         chosen, gate_w = self.route(tokens)
         w = self.experts
@@ -114,7 +116,8 @@ class MiniMaxMoE:
             out = nothing() if route_tokens.numel() == 0 else self._cuda.gguf_moe_prefill_grouped_forward(
                 tokens, route_tokens, route_weights, seg, w.w1.blocks, w.w3.blocks, w.w2.blocks,
                 int(w.w1.row_elems), int(w.w1.type_id), int(w.w3.row_elems), int(w.w3.type_id), int(w.w2.row_elems), int(w.w2.type_id), self._grid, 0.0)
-        return out.view(x.shape).to(self.dtype)
+        y = out.view(x.shape).to(self.dtype)
+        return y if residual is None else residual.add_(y)
 
 
 class MiniMaxAttention:
@@ -196,11 +199,13 @@ class MiniMaxBlock:
     def reset_cache(self, batch_size: int, max_seq_len: int) -> None:
         self.attention.reset_cache(batch_size, max_seq_len)
 
-    def __call__(self, x: torch.Tensor, start_pos: int) -> torch.Tensor:
+    def __call__(self, x: torch.Tensor, start_pos: int, *, in_place: bool = False) -> torch.Tensor:
+        """x [batch, steps, dim] at positions start_pos ..; returns the residual stream behind the layer.  in_place: x may be
+        overwritten (a layer stack passing its own tensor from layer to layer); otherwise the caller's tensor is left alone."""
         start_pos = int(start_pos)
         stream = x.to(self.dtype).contiguous()
-        if stream is x:
-            stream = x.clone()                                                 # the caller's tensor is not written
+        if stream is x and not in_place:
+            stream = x.clone()
         rows = stream.numel() // stream.size(-1)
         o = self.attention.o_proj
         if rows <= 4:
@@ -210,8 +215,7 @@ class MiniMaxBlock:
                                                           stream)
         else:
             stream += self.attention(self.attn_norm(stream), start_pos)
-        stream += self.moe(self.ffn_norm(stream))
-        return stream
+        return self.moe(self.ffn_norm(stream), residual=stream)
 
 
 class MiniMaxTransformer:
@@ -240,7 +244,7 @@ class MiniMaxTransformer:
         ids = ids.view(1, -1) if ids.dim() == 1 else ids
         hidden = self.embedding(ids).to(self.dtype)
         for layer in self.layers:
-            hidden = layer(hidden, int(start_pos))
+            hidden = layer(hidden, int(start_pos), in_place=True)                # `hidden` is this call's own tensor
         if not keep_all_positions:
             hidden = hidden[:, -1:, :]
         logits = self.lm_head(self.final_norm(hidden.contiguous())).float()
