@@ -642,6 +642,40 @@ def fp8_gemm_pass(mod, dev) -> None:
     print(json.dumps({"fp8_gemm_pass": "fp8 x fp8 17408x5120, T=512 x8 then T=2048 x8", "flops_512": 2.0 * 512 * k * n, "flops_2048": 2.0 * 2048 * k * n}))
 
 
+def block_pass(mod, dev) -> None:
+    """A few decode steps of one MiniMaxBlock for the profiler: MiniMax-M2 shapes (3072 wide, 48 / 8 heads of 128, 64 resident
+    experts of the 256, top-8, Q6_K projections, IQ2_XXS / IQ1_M experts), position 2047 of a 2048-token store."""
+    from pocketllm_amd import block_codec as C
+    from pocketllm_amd.minimax_block import ExpertLayer, MiniMaxAttention, MiniMaxBlock, MiniMaxM2Args, MiniMaxMoE, RMSNorm
+    from pocketllm_amd.quantized_ops import QuantizedGGUFLinear
+    from pocketllm_amd.quantized_tensor import QuantizedGGUFTensor
+    rng = np.random.default_rng(9009)
+    e, d, inter = 64, 3072, 1536
+    a = MiniMaxM2Args(dim=d, n_heads=48, n_kv_heads=8, head_dim=128, rope_dim=64, rope_base=5.0e6, n_routed_experts=e, top_k=8,
+                      moe_inter_dim=inter, norm_eps=1e-6)
+
+    def lin(n, k):
+        return QuantizedGGUFLinear(QuantizedGGUFTensor.from_blocks(torch.from_numpy(C.random_blocks(rng, "q6_k", n, k // 256)).to(dev), "q6_k", k))
+
+    w1 = torch.from_numpy(C.random_iq2_xxs(rng, e, inter, d // 256, d_range=(0.002, 0.006))).to(dev)
+    w3 = torch.from_numpy(C.random_iq2_xxs(rng, e, inter, d // 256, d_range=(0.002, 0.006))).to(dev)
+    w2 = torch.from_numpy(C.random_iq1_m(rng, e, d, inter // 256, d_range=(0.002, 0.006))).to(dev)
+    experts = ExpertLayer(*(QuantizedGGUFTensor.from_blocks(t, n, k) for t, n, k in ((w1, "iq2_xxs", d), (w3, "iq2_xxs", d), (w2, "iq1_m", inter))))
+    moe = MiniMaxMoE(a, torch.randn(e, d, device=dev) * d ** -0.5, torch.zeros(e, device=dev), experts)
+    attn = MiniMaxAttention(a, lin(6144, d), lin(1024, d), lin(1024, d), lin(d, 6144), RMSNorm(torch.ones(6144, device=dev), 1e-6),
+                            RMSNorm(torch.ones(1024, device=dev), 1e-6))
+    blk = MiniMaxBlock(a, torch.ones(d, device=dev), torch.ones(d, device=dev), attn, moe)
+    blk.reset_cache(1, 2048)
+    blk.attention.store.keys.normal_()
+    blk.attention.store.values.normal_()
+    x = torch.randn(1, 1, d, device=dev, dtype=torch.float16)
+    with torch.inference_mode():
+        for _ in range(12):
+            blk(x, 2047)
+    torch.cuda.synchronize()
+    print(json.dumps({"block_pass": "MiniMaxBlock decode step at position 2047, 12 steps, one token"}))
+
+
 def experts_rows_pass(mod, dev) -> None:
     """A few launches of the grouped routed experts for the profiler: 256 tokens, 256 resident experts, top-8 (2048 routes),
     IQ2_XXS gate/up 1536x3072 and IQ1_M down 3072x1536."""
@@ -705,6 +739,7 @@ def main() -> None:
     ap.add_argument("--fp8-gemm-pass", action="store_true", help="short run for rocprofv3: native FP8 x FP8 matmul at T=512 and T=2048")
     ap.add_argument("--iq-pass", action="store_true", help="short run for rocprofv3: IQ2_XXS / IQ1_M matvec and the single-token experts")
     ap.add_argument("--experts-rows-pass", action="store_true", help="short run for rocprofv3: grouped routed experts at T=256")
+    ap.add_argument("--block-pass", action="store_true", help="short run for rocprofv3: decode steps of one MiniMaxBlock")
     ap.add_argument("--q8-gemm-pass", action="store_true", help="short run for rocprofv3: int8-activation matmul at T=512 / 2048 and the 17 - 48 row kernel at T=32")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -737,6 +772,9 @@ def main() -> None:
         return
     if args.experts_rows_pass:
         experts_rows_pass(mod, dev)
+        return
+    if args.block_pass:
+        block_pass(mod, dev)
         return
     if args.q8_gemm_pass:
         q8_gemm_pass(mod, dev)
