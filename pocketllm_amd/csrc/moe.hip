@@ -27,6 +27,9 @@ constexpr int kMoeGroupedMaxRoutesPerExpert = 8;
 // The half-precision form with the routes as matrix rows pays a fixed price per expert that has routes at all (its decode costs
 // more than the integer one, its multiply next to nothing): measured at 256 experts of 1536 x 3072 it overtakes the form above
 // between 1 and 2 routes per expert (32 tokens, top 8: 375 vs 316 us; 64 tokens: 381 vs 472 us; 256 tokens: 500 vs 1126 us).
+// It has no upper limit: an expert with more than 16 routes is decoded once per batch of 16, and that still beats the tile matmuls,
+// which run every expert's few rows through 64-row tiles (256 experts, top 8, 512 / 1024 / 2048 / 4096 tokens: 0.97 / 1.41 / 2.39 /
+// 4.37 ms against 2.85 / 4.57 / 7.25 / 8.50 ms, routing included).
 constexpr int kMoeRowsMinRoutesPerExpertX2 = 3;
 
 namespace {
@@ -347,9 +350,9 @@ __global__ void narrow_experts_kernel(const int64_t* __restrict__ src, int32_t* 
 }
 
 // y[t, d] = sum_{r : route_tokens[r] == t} partial[r, d], ascending r.  grid (tokens, column groups): a workgroup owns the
-// columns blockIdx.y * 256 + tid + k * gridDim.y * 256.  It first lists the routes of its token in LDS (every thread scans a
-// contiguous run of the route table, an exclusive scan of the per-thread counts keeps the list in route order), then adds
-// them.  route_tokens == nullptr: a single token owns every route.
+// columns blockIdx.y * 256 + tid + k * gridDim.y * 256.  It first lists the routes of its token in LDS (the route table is read in
+// pieces of 2048 routes, every thread a contiguous run of a piece; an exclusive scan of the per-thread counts keeps the list in
+// route order), then adds them.  route_tokens == nullptr: a single token owns every route.
 constexpr int kReduceList = 2048;
 __global__ __launch_bounds__(256) void moe_reduce_kernel(const float* __restrict__ partial, const int64_t* __restrict__ route_tokens,
                                                          float* __restrict__ y, int routes, int dim) {
@@ -363,53 +366,66 @@ __global__ __launch_bounds__(256) void moe_reduce_kernel(const float* __restrict
             for (int r = 0; r < routes; ++r) acc += partial[static_cast<size_t>(r) * dim + d];
             y[static_cast<size_t>(t) * dim + d] = acc;
         }
-    } else if (routes <= kReduceList) {
-        const int per = (routes + 255) / 256;                                // at most kReduceList / 256 = 8
-        const int r0 = min(tid * per, routes), r1 = min(r0 + per, routes);
-        // the thread's run of the route table, all loads in flight together (past the run: its last entry again, not counted)
-        int64_t mine[kReduceList / 256];
-#pragma unroll
-        for (int i = 0; i < kReduceList / 256; ++i) mine[i] = route_tokens[min(r0 + i, routes - 1)];
-        int cnt = 0;
-#pragma unroll
-        for (int i = 0; i < kReduceList / 256; ++i) cnt += (r0 + i < r1) && mine[i] == t;
-        int incl = cnt;                                     // inclusive scan over the wave, then over the four waves
-#pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            const int v = __shfl_up(incl, off, 64);
-            if ((tid & 63) >= off) incl += v;
-        }
-        if ((tid & 63) == 63) wave_total[tid >> 6] = incl;
-        __syncthreads();
-        int pos = incl - cnt, total = 0;
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            if (w < (tid >> 6)) pos += wave_total[w];
-            total += wave_total[w];
-        }
-#pragma unroll
-        for (int i = 0; i < kReduceList / 256; ++i)
-            if ((r0 + i < r1) && mine[i] == t) list[pos++] = r0 + i;
-        __syncthreads();
-        for (int d = d0; d < dim; d += dstep) {
-            float acc = 0.0f;
-            int i = 0;
-            for (; i + 8 <= total; i += 8) {                                 // eight routes' values requested together, added in route order
-                float v[8];
-#pragma unroll
-                for (int j = 0; j < 8; ++j) v[j] = partial[static_cast<size_t>(list[i + j]) * dim + d];
-#pragma unroll
-                for (int j = 0; j < 8; ++j) acc += v[j];
-            }
-            for (; i < total; ++i) acc += partial[static_cast<size_t>(list[i]) * dim + d];
-            y[static_cast<size_t>(t) * dim + d] = acc;
-        }
     } else {
-        for (int d = d0; d < dim; d += dstep) {
-            float acc = 0.0f;
-            for (int r = 0; r < routes; ++r)
-                if (route_tokens[r] == t) acc += partial[static_cast<size_t>(r) * dim + d];
-            y[static_cast<size_t>(t) * dim + d] = acc;
+        // The route table is scanned in pieces of kReduceList routes; a token's routes found so far stay listed in LDS in route
+        // order.  (A token with more routes than the list holds - more than kReduceList experts - falls back to a scan per column.)
+        int listed = 0;
+        for (int c0 = 0; c0 < routes; c0 += kReduceList) {
+            const int chunk = min(kReduceList, routes - c0);
+            const int per = (chunk + 255) / 256;                             // at most kReduceList / 256 = 8
+            const int r0 = c0 + min(tid * per, chunk), r1 = min(r0 + per, c0 + chunk);
+            // the thread's run of the route table, all loads in flight together (past the run: the table's last entry, not counted)
+            int64_t mine[kReduceList / 256];
+#pragma unroll
+            for (int i = 0; i < kReduceList / 256; ++i) mine[i] = route_tokens[min(r0 + i, routes - 1)];
+            int cnt = 0;
+#pragma unroll
+            for (int i = 0; i < kReduceList / 256; ++i) cnt += (r0 + i < r1) && mine[i] == t;
+            int incl = cnt;                                 // inclusive scan over the wave, then over the four waves
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                const int v = __shfl_up(incl, off, 64);
+                if ((tid & 63) >= off) incl += v;
+            }
+            __syncthreads();                                // the previous piece's totals have been read by everybody
+            if ((tid & 63) == 63) wave_total[tid >> 6] = incl;
+            __syncthreads();
+            int pos = listed + incl - cnt, total = 0;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                if (w < (tid >> 6)) pos += wave_total[w];
+                total += wave_total[w];
+            }
+#pragma unroll
+            for (int i = 0; i < kReduceList / 256; ++i)
+                if ((r0 + i < r1) && mine[i] == t) {
+                    if (pos < kReduceList) list[pos] = r0 + i;
+                    ++pos;
+                }
+            listed += total;
+        }
+        __syncthreads();
+        if (listed <= kReduceList) {
+            for (int d = d0; d < dim; d += dstep) {
+                float acc = 0.0f;
+                int i = 0;
+                for (; i + 8 <= listed; i += 8) {                            // eight routes' values requested together, added in route order
+                    float v[8];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) v[j] = partial[static_cast<size_t>(list[i + j]) * dim + d];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) acc += v[j];
+                }
+                for (; i < listed; ++i) acc += partial[static_cast<size_t>(list[i]) * dim + d];
+                y[static_cast<size_t>(t) * dim + d] = acc;
+            }
+        } else {
+            for (int d = d0; d < dim; d += dstep) {
+                float acc = 0.0f;
+                for (int r = 0; r < routes; ++r)
+                    if (route_tokens[r] == t) acc += partial[static_cast<size_t>(r) * dim + d];
+                y[static_cast<size_t>(t) * dim + d] = acc;
+            }
         }
     }
 }
@@ -581,7 +597,7 @@ int pllm_gguf_moe_forward(const void* x, int x_dtype, int64_t tokens, int64_t di
     if (!workspace || workspace_bytes < pllm_gguf_moe_workspace_bytes(tokens, routes, dim, inter)) return PLLM_ERR_WORKSPACE;
 
     const int bpr_x = static_cast<int>((dim + 255) / 256), bpr_h = static_cast<int>((inter + 255) / 256);
-    if (seg_starts && tokens > 1 && routes <= kMoeGroupedMaxRoutesPerExpert * n_experts && 2 * routes >= kMoeRowsMinRoutesPerExpertX2 * n_experts &&
+    if (seg_starts && tokens > 1 && 2 * routes >= kMoeRowsMinRoutesPerExpertX2 * n_experts &&
         moe_rows_supports(w13_type, w2_type, static_cast<int>(dim), static_cast<int>(inter), w1, w3, w2)) {
         // a few routes per expert, IQ2_XXS / IQ1_M: every expert's weights are decoded once, in half precision, and multiplied with
         // all its routes at once on the matrix cores

@@ -174,26 +174,28 @@ def test_baseline_config_grouped_256_tokens_256_experts(mod):
 
 
 def test_grouped_experts_more_routes_than_the_reduction_lists(mod):
-    """More than 2048 routes: the route-sum kernel then scans the route table instead of listing a token's routes in LDS."""
+    """More than 2048 routes (the route-sum kernel reads the route table in pieces of 2048: two pieces, then three) and 60 / 120 routes
+    per expert on average (every expert's routes pass through the matrix-row kernels in several batches of 16)."""
     rng = np.random.default_rng(17)
-    e, d, inter, topk, t = 40, 256, 256, 8, 300
+    e, d, inter, topk = 40, 256, 256, 8
     w1 = _expert_blocks(rng, "iq2_xxs", e, inter, d)
     w3 = _expert_blocks(rng, "iq2_xxs", e, inter, d)
     w2 = _expert_blocks(rng, "iq1_m", e, d, inter)
-    idx, wts = _route(rng, t, e, topk)
-    x = torch.from_numpy(rng.standard_normal((t, d)).astype(np.float32)).to(DEV).to(torch.bfloat16)
-    _, toks, rws, seg = mod.moe_group_routes(torch.from_numpy(idx).to(DEV), torch.from_numpy(wts).to(DEV), 0, e)
-    _, o_toks, o_rws, o_seg = O.group_routes(idx, wts, 0, e)
-    assert len(o_toks) == 2400
     grids = (codebooks.get_iq2xxs_signed_grid_tensor().to(DEV), codebooks.get_iq1_grid_tensor().to(DEV))
     dw1, dw3, dw2 = (torch.from_numpy(a).to(DEV) for a in (w1, w3, w2))
     tid = O.TYPE_IDS
-    print("case grouped experts 2400 routes", flush=True)
-    y = mod.gguf_moe_prefill_grouped_forward(x, toks, rws, seg, dw1, dw3, dw2, d, tid["iq2_xxs"], d, tid["iq2_xxs"], inter, tid["iq1_m"], grids, 0.0)
-    torch.cuda.synchronize()
-    route_experts = np.repeat(np.arange(e), np.diff(o_seg))
-    want = O.moe_forward(x.float().cpu().numpy(), o_toks, o_rws, route_experts, w1, w3, w2, "iq2_xxs", "iq2_xxs", "iq1_m", 0.0)
-    assert O.rel_l2(y.cpu().numpy(), want) <= TOL
+    for t in (300, 600):
+        idx, wts = _route(rng, t, e, topk)
+        x = torch.from_numpy(rng.standard_normal((t, d)).astype(np.float32)).to(DEV).to(torch.bfloat16)
+        _, toks, rws, seg = mod.moe_group_routes(torch.from_numpy(idx).to(DEV), torch.from_numpy(wts).to(DEV), 0, e)
+        _, o_toks, o_rws, o_seg = O.group_routes(idx, wts, 0, e)
+        assert len(o_toks) == 8 * t
+        print(f"case grouped experts {8 * t} routes", flush=True)
+        y = mod.gguf_moe_prefill_grouped_forward(x, toks, rws, seg, dw1, dw3, dw2, d, tid["iq2_xxs"], d, tid["iq2_xxs"], inter, tid["iq1_m"], grids, 0.0)
+        torch.cuda.synchronize()
+        route_experts = np.repeat(np.arange(e), np.diff(o_seg))
+        want = O.moe_forward(x.float().cpu().numpy(), o_toks, o_rws, route_experts, w1, w3, w2, "iq2_xxs", "iq2_xxs", "iq1_m", 0.0)
+        assert O.rel_l2(y.cpu().numpy(), want) <= TOL
 
 
 def test_route_slots_host_compaction(mod):
