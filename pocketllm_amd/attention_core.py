@@ -111,6 +111,10 @@ def grouped_query_attention(q: torch.Tensor, keys: torch.Tensor, values: torch.T
     batch, steps, heads, dim = q.shape
     kv_heads, length = keys.size(1), keys.size(2)
     group = heads // kv_heads
+    if steps > 1 and first_pos == 0 and length == steps and q.is_cuda and q.dtype == keys.dtype and q.dtype in (torch.float16, torch.bfloat16):
+        # a whole prompt at once: the framework's fused causal attention (the routine the reference calls), key/value heads shared
+        out = torch.nn.functional.scaled_dot_product_attention(q.permute(0, 2, 1, 3), keys, values, is_causal=True, enable_gqa=group > 1)
+        return out.permute(0, 2, 1, 3).reshape(batch, steps, heads * dim)
     # [batch, kv_heads, group * steps, head_dim]: row g * steps + s is query head (kv * group + g) at step s
     rows = (q * (float(dim) ** -0.5)).view(batch, steps, kv_heads, group, dim).permute(0, 2, 3, 1, 4).reshape(batch, kv_heads, group * steps, dim)
     scores = torch.matmul(rows.to(keys.dtype), keys.transpose(2, 3))
