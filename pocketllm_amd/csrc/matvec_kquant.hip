@@ -352,7 +352,9 @@ __device__ __forceinline__ void raw_to_float4(const RawX<X16>& r, int x_dtype, f
 
 // ITERS = blocks a wave walks per pass, DEPTH <= ITERS = blocks it keeps in flight (a block's activation slice is requested
 // right ahead of its weights, so it arrives first).
-template <typename FMT, int ITERS, int DEPTH, bool X16, bool NORM>
+// PLAIN: one matrix, one output, activation row = grid row (no routing, no further projections, no row map): the arguments the
+// other forms test one after the other (a scalar load and a wait each) are not read at all.
+template <typename FMT, int ITERS, int DEPTH, bool X16, bool NORM, bool PLAIN = false>
 __global__ __launch_bounds__(64 * kMaxWaves) void wave_image_matvec_kernel(
     const void* __restrict__ x, int x_dtype, int k, const WeightRoute route, const uint8_t* __restrict__ w, void* __restrict__ y,
     int y_dtype, int n, int bpr, const float* __restrict__ gamma, float eps, int round_f16, const int64_t* __restrict__ row_token, int x_broadcast) {
@@ -365,19 +367,22 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_image_matvec_kernel(
     const int ks = lane >> 4;
     constexpr int kWaveBytes = kSlotBytes + 16;                               // the wave's slot, then its 16 zero bytes
     unsigned char* slot = smem + wave * kWaveBytes;
-    float* partial = reinterpret_cast<float*>(smem + waves * kWaveBytes);    // [waves][16]
-    const size_t woff = route_offset(route, blockIdx.y);                      // routed calls: the grid row's expert
-    w += woff;
-    if (blockIdx.z) {                        // several projections in one launch: this one's matrix, row count and output
-        const int m = blockIdx.z - 1;
-        w = route.more_w[m] + woff;
-        y = route.more_y[m];
-        n = route.more_n[m];
+    float* partial = reinterpret_cast<float*>(smem + waves * kWaveBytes);    // [16][kMaxWaves]: a row's shares side by side
+    if constexpr (!PLAIN) {
+        const size_t woff = route_offset(route, blockIdx.y);                  // routed calls: the grid row's expert
+        w += woff;
+        if (blockIdx.z) {                    // several projections in one launch: this one's matrix, row count and output
+            const int m = blockIdx.z - 1;
+            w = route.more_w[m] + woff;
+            y = route.more_y[m];
+            n = route.more_n[m];
+        }
+        if (static_cast<int>(blockIdx.x) * kRowsPerWg >= n) return;         // the grid covers the tallest matrix
     }
-    if (static_cast<int>(blockIdx.x) * kRowsPerWg >= n) return;             // the grid covers the tallest matrix
     const int row = blockIdx.x * kRowsPerWg + col;
     const uint8_t* wrow = w + static_cast<size_t>(row < n ? row : 0) * bpr * FMT::kBlockBytes;
-    const size_t xoff = (x_broadcast ? 0 : row_token ? static_cast<size_t>(row_token[blockIdx.y]) : static_cast<size_t>(blockIdx.y)) * k;
+    const size_t xoff = (PLAIN ? static_cast<size_t>(blockIdx.y)
+                               : x_broadcast ? 0 : row_token ? static_cast<size_t>(row_token[blockIdx.y]) : static_cast<size_t>(blockIdx.y)) * k;
 
     if (lane < 4) reinterpret_cast<uint32_t*>(slot + kSlotBytes)[lane] = 0;
     float acc = 0.0f;
@@ -432,7 +437,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_image_matvec_kernel(
                 if (b < bpr) ss += (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
             }
             ss = group_sum<64>(ss);
-            float* shares = partial + waves * kRowsPerWg;                    // [waves]
+            float* shares = partial + kMaxWaves * kRowsPerWg;                // [waves]
             if (lane == 0) shares[wave] = ss;
             __syncthreads();
             float total = 0.0f;
@@ -459,12 +464,13 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_image_matvec_kernel(
                 }
                 uint32_t qh, ql;
                 float scale;
-                quantize4(v, qh, ql, scale);
+                float sum4;                                                 // the four values as the image holds them, summed (exact): the
+                quantize4_pow2(v, qh, ql, scale, &sum4);                    // min terms cancel against dots of these same rounded values
                 reinterpret_cast<uint32_t*>(slot)[lane] = qh;
                 reinterpret_cast<uint32_t*>(slot + 256)[lane] = ql;
-                const float sum = group_sum<4>((v[0] + v[1]) + (v[2] + v[3]));   // the order in which the pre-pass kernel sums
+                const float sum = group_sum<4>(sum4);
                 const float sum32 = sum + butterfly_peer<4>(sum);
-                if ((lane & 7) == 0) reinterpret_cast<float2*>(slot + 512)[lane >> 3] = make_float2(scale * kLoInv, sum32);
+                if ((lane & 7) == 0) reinterpret_cast<float2*>(slot + 512)[lane >> 3] = make_float2(scale, sum32);
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
                 __builtin_amdgcn_wave_barrier();                            // LDS serves a wave's requests in order
                 uint4 bw[4];
@@ -479,8 +485,8 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_image_matvec_kernel(
                     const uint4 a = *reinterpret_cast<const uint4*>(slot + off);
                     c = __builtin_amdgcn_mfma_i32_16x16x64_i8(as_v4i(a), as_v4i(bw[t]), c, 0, 0, 0);
                 }
-                const float v0 = static_cast<float>(__mul24(c.x, 254) + c.y);
-                const float v1 = static_cast<float>(__mul24(c.z, 254) + c.w);
+                const float v0 = static_cast<float>((c.x << 8) + c.y);       // both terms of the image joined: 256 hi + lo
+                const float v1 = static_cast<float>((c.z << 8) + c.w);
                 const float4 g2 = *reinterpret_cast<const float4*>(slot + 512 + 16 * ks);   // {xs0, sum0, xs1, sum1}
                 acc += FMT::combine(regs[it % DEPTH], ks, v0, v1, g2);
                 __builtin_amdgcn_wave_barrier();                            // the next block's slice overwrites the slot
@@ -489,11 +495,15 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_image_matvec_kernel(
         }
     }
     acc = quad_rows_sum(acc);
-    if (ks == 0) partial[wave * kRowsPerWg + col] = acc;
+    if (ks == 0) partial[col * kMaxWaves + wave] = acc;
     __syncthreads();
-    if (tid < kRowsPerWg) {
-        float total = 0.0f;
-        for (int v = 0; v < waves; ++v) total += partial[v * kRowsPerWg + tid];
+    if (tid < kRowsPerWg) {                  // the waves' shares in wave order, fetched together
+        const float4 lo4 = *reinterpret_cast<const float4*>(partial + tid * kMaxWaves);
+        const float4 hi4 = *reinterpret_cast<const float4*>(partial + tid * kMaxWaves + 4);
+        const float p[kMaxWaves] = {lo4.x, lo4.y, lo4.z, lo4.w, hi4.x, hi4.y, hi4.z, hi4.w};
+        float total = p[0];
+#pragma unroll
+        for (int v = 1; v < kMaxWaves; ++v) total = v < waves ? total + p[v] : total;
         const int out_row = blockIdx.x * kRowsPerWg + tid;
         if (out_row < n) store_any(y, y_dtype, static_cast<size_t>(blockIdx.y) * n + out_row, total);
     }
@@ -520,7 +530,7 @@ int launch_kernel(KERN kern, const ActRows& act, const WeightRoute& route, const
 template <typename KERN>
 int launch_wave_kernel(KERN kern, const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype,
                        int rows, int n, int bpr, int waves, hipStream_t stream) {
-    const size_t smem = static_cast<size_t>(waves) * (kSlotBytes + 16) + static_cast<size_t>(waves) * (kRowsPerWg + 1) * sizeof(float);
+    const size_t smem = static_cast<size_t>(waves) * (kSlotBytes + 16) + static_cast<size_t>(kMaxWaves * kRowsPerWg + waves) * sizeof(float);
     int tallest = n;
     for (int m = 0; m < route.extra; ++m) tallest = tallest > route.more_n[m] ? tallest : route.more_n[m];
     dim3 grid((tallest + kRowsPerWg - 1) / kRowsPerWg, rows, 1 + route.extra);
@@ -556,7 +566,11 @@ int launch_wave(const ActRows& act, const WeightRoute& route, const uint8_t* w, 
     for (int m = 0; m < route.extra; ++m) tiles += (route.more_n[m] + kRowsPerWg - 1) / kRowsPerWg;
     split_blocks(bpr, tiles * rows, waves, iters);
     if (NORM && waves * iters < bpr) return PLLM_ERR_UNSUPPORTED;             // the normalised form holds a wave's slices of the whole row
+    const bool plain = !NORM && !routed(route) && route.extra == 0 && !act.row_token && !act.x_broadcast;
 #define PLLM_CASE(I) case I: \
+        if constexpr (!NORM) if (plain) \
+            return act.x_dtype == PLLM_F32 ? launch_wave_kernel(wave_image_matvec_kernel<FMT, I, wave_depth<FMT>(I, false), false, false, true>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream) \
+                                           : launch_wave_kernel(wave_image_matvec_kernel<FMT, I, wave_depth<FMT>(I, true), true, false, true>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream); \
         return act.x_dtype == PLLM_F32 ? launch_wave_kernel(wave_image_matvec_kernel<FMT, I, wave_depth<FMT>(I, false), false, NORM>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream) \
                                        : launch_wave_kernel(wave_image_matvec_kernel<FMT, I, wave_depth<FMT>(I, true), true, NORM>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream)
     switch (iters) {
@@ -655,7 +669,7 @@ struct WaveQ6K {
     }
 };
 
-template <typename FMT, int ITERS, int DEPTH, bool X16>
+template <typename FMT, int ITERS, int DEPTH, bool X16, bool PLAIN = false>
 __global__ __launch_bounds__(64 * kMaxWaves) void wave_groups16_matvec_kernel(
     const void* __restrict__ x, int x_dtype, int k, const WeightRoute route, const uint8_t* __restrict__ w, void* __restrict__ y,
     int y_dtype, int n, int bpr, const int64_t* __restrict__ row_token, int x_broadcast) {
@@ -668,19 +682,22 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_groups16_matvec_kernel(
     const int ks = lane >> 4;
     constexpr int kWaveBytes = kQ2SlotBytes + 16;                            // the wave's slot, then its 16 zero bytes
     unsigned char* slot = smem + wave * kWaveBytes;
-    float* partial = reinterpret_cast<float*>(smem + waves * kWaveBytes);    // [waves][16]
-    const size_t woff = route_offset(route, blockIdx.y);                      // routed calls: the grid row's expert
-    w += woff;
-    if (blockIdx.z) {                        // several projections in one launch: this one's matrix, row count and output
-        const int m = blockIdx.z - 1;
-        w = route.more_w[m] + woff;
-        y = route.more_y[m];
-        n = route.more_n[m];
+    float* partial = reinterpret_cast<float*>(smem + waves * kWaveBytes);    // [16][kMaxWaves]: a row's shares side by side
+    if constexpr (!PLAIN) {
+        const size_t woff = route_offset(route, blockIdx.y);                  // routed calls: the grid row's expert
+        w += woff;
+        if (blockIdx.z) {                    // several projections in one launch: this one's matrix, row count and output
+            const int m = blockIdx.z - 1;
+            w = route.more_w[m] + woff;
+            y = route.more_y[m];
+            n = route.more_n[m];
+        }
+        if (static_cast<int>(blockIdx.x) * kRowsPerWg >= n) return;
     }
-    if (static_cast<int>(blockIdx.x) * kRowsPerWg >= n) return;
     const int row = blockIdx.x * kRowsPerWg + col;
     const uint8_t* wrow = w + static_cast<size_t>(row < n ? row : 0) * bpr * FMT::kBlockBytes;
-    const size_t xoff = (x_broadcast ? 0 : row_token ? static_cast<size_t>(row_token[blockIdx.y]) : static_cast<size_t>(blockIdx.y)) * k;
+    const size_t xoff = (PLAIN ? static_cast<size_t>(blockIdx.y)
+                               : x_broadcast ? 0 : row_token ? static_cast<size_t>(row_token[blockIdx.y]) : static_cast<size_t>(blockIdx.y)) * k;
     // the lane's A operand: group `col` of the block, in the one MFMA whose slice ks carries that group
     const bool mine = FMT::slice_of(col) == ks;
     const int my_t = FMT::mfma_of(col);
@@ -713,12 +730,13 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_groups16_matvec_kernel(
                 raw_to_float4<X16>(raw[it % DEPTH], x_dtype, v);
                 uint32_t qh, ql;
                 float scale;
-                quantize4(v, qh, ql, scale);
+                float sum4;                                                 // the four values as the image holds them, summed (exact): the
+                quantize4_pow2(v, qh, ql, scale, &sum4);                    // offset terms cancel against dots of these same rounded values
                 reinterpret_cast<uint32_t*>(slot)[lane] = qh;
                 reinterpret_cast<uint32_t*>(slot + 256)[lane] = ql;
-                const float sum = group_sum<4>((v[0] + v[1]) + (v[2] + v[3]));   // the order in which the pre-pass kernel sums
+                const float sum = group_sum<4>(sum4);
                 const float sum32 = sum + butterfly_peer<4>(sum);
-                if ((lane & 7) == 0) reinterpret_cast<float2*>(slot + 512)[lane >> 3] = make_float2(scale * kLoInv, sum32);
+                if ((lane & 7) == 0) reinterpret_cast<float2*>(slot + 512)[lane >> 3] = make_float2(scale, sum32);
                 if ((lane & 3) == 0) reinterpret_cast<float*>(slot + kSlotBytes)[lane >> 2] = sum;
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
                 __builtin_amdgcn_wave_barrier();                            // LDS serves a wave's requests in order
@@ -735,8 +753,8 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_groups16_matvec_kernel(
                 }
                 const float4 g2 = *reinterpret_cast<const float4*>(slot + 512 + 16 * ks);          // {xs, sum} of 32-groups 2 ks, 2 ks + 1
                 const float4 s16 = *reinterpret_cast<const float4*>(slot + kSlotBytes + 16 * ks);  // sums of groups 4 ks .. 4 ks + 3
-                const float vv[4] = {static_cast<float>(__mul24(ch.x, 254) + cl.x), static_cast<float>(__mul24(ch.y, 254) + cl.y),
-                                     static_cast<float>(__mul24(ch.z, 254) + cl.z), static_cast<float>(__mul24(ch.w, 254) + cl.w)};
+                const float vv[4] = {static_cast<float>((ch.x << 8) + cl.x), static_cast<float>((ch.y << 8) + cl.y),
+                                     static_cast<float>((ch.z << 8) + cl.z), static_cast<float>((ch.w << 8) + cl.w)};
                 const float xsv[4] = {g2.x, g2.x, g2.z, g2.z};
                 const float smv[4] = {s16.x, s16.y, s16.z, s16.w};
                 acc += FMT::finish(r, vv, xsv, smv);
@@ -751,11 +769,15 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_groups16_matvec_kernel(
         }
     }
     acc = quad_rows_sum(acc);
-    if (ks == 0) partial[wave * kRowsPerWg + col] = acc;
+    if (ks == 0) partial[col * kMaxWaves + wave] = acc;
     __syncthreads();
-    if (tid < kRowsPerWg) {
-        float total = 0.0f;
-        for (int v = 0; v < waves; ++v) total += partial[v * kRowsPerWg + tid];
+    if (tid < kRowsPerWg) {                  // the waves' shares in wave order, fetched together
+        const float4 lo4 = *reinterpret_cast<const float4*>(partial + tid * kMaxWaves);
+        const float4 hi4 = *reinterpret_cast<const float4*>(partial + tid * kMaxWaves + 4);
+        const float p[kMaxWaves] = {lo4.x, lo4.y, lo4.z, lo4.w, hi4.x, hi4.y, hi4.z, hi4.w};
+        float total = p[0];
+#pragma unroll
+        for (int v = 1; v < kMaxWaves; ++v) total = v < waves ? total + p[v] : total;
         const int out_row = blockIdx.x * kRowsPerWg + tid;
         if (out_row < n) store_any(y, y_dtype, static_cast<size_t>(blockIdx.y) * n + out_row, total);
     }
@@ -764,7 +786,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_groups16_matvec_kernel(
 template <typename KERN>
 int launch_q2k_kernel(KERN kern, const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype,
                       int rows, int n, int bpr, int waves, hipStream_t stream) {
-    const size_t smem = static_cast<size_t>(waves) * (kQ2SlotBytes + 16) + static_cast<size_t>(waves) * kRowsPerWg * sizeof(float);
+    const size_t smem = static_cast<size_t>(waves) * (kQ2SlotBytes + 16) + static_cast<size_t>(kMaxWaves) * kRowsPerWg * sizeof(float);
     int tallest = n;
     for (int m = 0; m < route.extra; ++m) tallest = tallest > route.more_n[m] ? tallest : route.more_n[m];
     dim3 grid((tallest + kRowsPerWg - 1) / kRowsPerWg, rows, 1 + route.extra);
@@ -819,8 +841,12 @@ int launch_groups16(const ActRows& act, const WeightRoute& route, const uint8_t*
     for (int m = 0; m < route.extra; ++m) tiles += (route.more_n[m] + kRowsPerWg - 1) / kRowsPerWg;
     split_blocks(bpr, tiles * rows, waves, iters);
     constexpr int kMaxDepth = 2;            // blocks in flight per wave: five waves per SIMD fit with 2 (Q6_K with 2, 3, 4 and 5 ran within 3 % of each other, Q2_K 14.6 us with 2 against 15.2 with 5)
+    const bool plain = !routed(route) && route.extra == 0 && !act.row_token && !act.x_broadcast;
 #define PLLM_CASE(I) case I: { \
         constexpr int D = I < kMaxDepth ? I : kMaxDepth; \
+        if (plain) \
+            return act.x_dtype == PLLM_F32 ? launch_q2k_kernel(wave_groups16_matvec_kernel<FMT, I, D, false, true>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream) \
+                                           : launch_q2k_kernel(wave_groups16_matvec_kernel<FMT, I, D, true, true>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream); \
         return act.x_dtype == PLLM_F32 ? launch_q2k_kernel(wave_groups16_matvec_kernel<FMT, I, D, false>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream) \
                                        : launch_q2k_kernel(wave_groups16_matvec_kernel<FMT, I, D, true>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream); }
     switch (iters) {

@@ -199,6 +199,32 @@ __device__ __forceinline__ void quantize4(const float v[4], uint32_t& hi, uint32
     lo = pack_low_bytes(lb[0], lb[1], lb[2], lb[3]);
 }
 
+// The same two-term image on a power-of-two scale, for kernels that quantize a slice per wave and block and cannot afford the
+// exact quotients above: x ~= xs * (256 * hi + lo) with xs = 2^(E - 13), E the exponent of the group's largest magnitude, so that
+// |x / xs| < 2^14, hi in [-64, 64], lo in [-128, 127].  No division and no tie test: x / xs is an exponent shift, exact for every
+// value whose lowest mantissa bit is worth xs or more (all bf16 values within 2^-6 of the group's largest; fp16 within 2^-3);
+// smaller values round to the nearest multiple of xs (error <= amax * 2^-15).  One fused multiply-add with 1.5 * 2^23 + 128
+// rounds to nearest even and leaves (q + 128) in the low mantissa bits: byte 1 is hi, byte 0 is lo with its top bit flipped.
+// image_sum: the sum of the four values as the image holds them (exact).  The K-quants' offset terms (- dmin m sum(x), Q6_K's
+// - 32 sum(x)) cancel most of the dot of the unsigned codes; taken from the image the two carry the same rounding and the result
+// is the weights applied to the rounded activations, with the unrounded sums the rounding error is amplified by that cancellation.
+__device__ __forceinline__ void quantize4_pow2(const float v[4], uint32_t& hi, uint32_t& lo, float& xs, float* image_sum) {
+    constexpr float kRound = 12582912.0f + 128.0f;
+    float am = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
+    am = group_max<8>(am);
+    const uint32_t e = max(__float_as_uint(am) >> 23, 14u);     // groups below 2^-113 quantize to zeros
+    const float mult = __uint_as_float((267u - e) << 23);       // 2^(13 - (e - 127))
+    xs = __uint_as_float((e - 13u) << 23);
+    uint32_t t[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) t[i] = __float_as_uint(__builtin_fmaf(v[i], mult, kRound));
+    const uint32_t w01 = __builtin_amdgcn_perm(t[1], t[0], 0x05010400u);   // lo0 lo1 hi0 hi1
+    const uint32_t w23 = __builtin_amdgcn_perm(t[3], t[2], 0x05010400u);
+    lo = __builtin_amdgcn_perm(w23, w01, 0x05040100u) ^ 0x80808080u;
+    hi = __builtin_amdgcn_perm(w23, w01, 0x07060302u);
+    *image_sum = xs * (((__uint_as_float(t[0]) - kRound) + (__uint_as_float(t[1]) - kRound)) + ((__uint_as_float(t[2]) - kRound) + (__uint_as_float(t[3]) - kRound)));
+}
+
 // Runtime-dtype front ends (the dtype is uniform, so the switch costs one scalar branch).
 __device__ __forceinline__ float load_any(const void* x, int x_dtype, size_t i) {
     if (x_dtype == PLLM_BF16) return to_float(static_cast<const bf16_t*>(x)[i]);
