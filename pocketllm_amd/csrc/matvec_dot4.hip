@@ -19,6 +19,7 @@ template <typename FMT, int ITERS, bool RAW>
 __global__ __launch_bounds__(64 * kMaxWaves) void dot4_matvec_kernel(
     const ActRows act, const uint8_t* __restrict__ w,
     void* __restrict__ y, int y_dtype, int n, int bpr, const int32_t* __restrict__ y_expert, size_t expert_stride) {
+    fetch_together(act);
     extern __shared__ __align__(16) unsigned char smem[];
     const int kpad = bpr * 256;
     const int image_bytes = static_cast<int>(staged_x_bytes(kpad));

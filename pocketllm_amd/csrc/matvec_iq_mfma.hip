@@ -29,6 +29,8 @@ constexpr int kWaves = 8;
 template <typename FMT, int ITERS, bool RAW>
 __global__ __launch_bounds__(64 * kWaves) void mfma_tile_matvec_kernel(
     const ActRows act, const WeightRoute route, const uint8_t* __restrict__ w, void* __restrict__ y, int y_dtype, int n, int bpr) {
+    fetch_together(act);
+    fetch_together(route);
     extern __shared__ __align__(16) unsigned char smem[];
     const int kpad = bpr * 256;
     const int image_bytes = static_cast<int>(staged_x_bytes(kpad));

@@ -181,6 +181,8 @@ struct IQ4XS {
 template <typename FMT, int ITERS, bool RAW, int R>
 __global__ __launch_bounds__(64 * kMaxWaves) void k45_mfma_matvec_kernel(
     const ActRows act, const WeightRoute route, const uint8_t* __restrict__ w, void* __restrict__ y, int y_dtype, int n, int bpr, int total_rows) {
+    fetch_together(act);
+    fetch_together(route);
     extern __shared__ __align__(16) unsigned char smem[];
     const int kpad = bpr * 256;
     const int image_bytes = static_cast<int>(staged_x_bytes(kpad));          // a multiple of 16
@@ -358,6 +360,11 @@ template <typename FMT, int ITERS, int DEPTH, bool X16, bool NORM, bool PLAIN = 
 __global__ __launch_bounds__(64 * kMaxWaves) void wave_image_matvec_kernel(
     const void* __restrict__ x, int x_dtype, int k, const WeightRoute route, const uint8_t* __restrict__ w, void* __restrict__ y,
     int y_dtype, int n, int bpr, const float* __restrict__ gamma, float eps, int round_f16, const int64_t* __restrict__ row_token, int x_broadcast) {
+    if constexpr (!PLAIN) {
+        fetch_together(route);
+        asm volatile("" : : "s"(row_token), "s"(x_broadcast));
+    }
+    asm volatile("" : : "s"(x), "s"(k), "s"(w), "s"(y), "s"(n), "s"(bpr));   // the arguments in one batch of scalar loads, one wait
     extern __shared__ __align__(16) unsigned char smem[];
     const int tid = threadIdx.x;
     const int waves = blockDim.x >> 6;
@@ -673,6 +680,11 @@ template <typename FMT, int ITERS, int DEPTH, bool X16, bool PLAIN = false>
 __global__ __launch_bounds__(64 * kMaxWaves) void wave_groups16_matvec_kernel(
     const void* __restrict__ x, int x_dtype, int k, const WeightRoute route, const uint8_t* __restrict__ w, void* __restrict__ y,
     int y_dtype, int n, int bpr, const int64_t* __restrict__ row_token, int x_broadcast) {
+    if constexpr (!PLAIN) {
+        fetch_together(route);
+        asm volatile("" : : "s"(row_token), "s"(x_broadcast));
+    }
+    asm volatile("" : : "s"(x), "s"(k), "s"(w), "s"(y), "s"(n), "s"(bpr));   // the arguments in one batch of scalar loads, one wait
     extern __shared__ __align__(16) unsigned char smem[];
     const int tid = threadIdx.x;
     const int waves = blockDim.x >> 6;

@@ -136,6 +136,7 @@ __device__ __forceinline__ const uint8_t* not_past(const uint8_t* p, const uint8
 __global__ __launch_bounds__(kStreamThreads) void q8_0_stream_kernel(
     const void* __restrict__ x, int x_dtype, const uint8_t* __restrict__ w, void* __restrict__ y, int y_dtype,
     int k, int n, int pairs, uint32_t pairs_magic, int image_bytes, int cols) {
+    asm volatile("" : : "s"(x), "s"(x_dtype), "s"(w), "s"(y), "s"(y_dtype), "s"(k), "s"(n), "s"(pairs), "s"(pairs_magic), "s"(image_bytes), "s"(cols));   // the arguments in one batch of scalar loads, one wait
     extern __shared__ __align__(16) unsigned char smem[];
     unsigned char* img_hi = smem;
     unsigned char* img_lo = smem + static_cast<size_t>(pairs) * 80;

@@ -90,6 +90,16 @@ __device__ __forceinline__ size_t route_offset(const WeightRoute& r, int row) {
     if (r.expert64) return static_cast<size_t>(r.expert64[row]) * r.expert_stride;
     return 0;
 }
+// Kernels that take these structs test their fields one after the other (routed? further projections? a row map?), and the
+// compiler loads each field where it is first needed: a scalar load and a wait per test, several hundred nanoseconds of a
+// short kernel before its first memory request.  Naming the fields as inputs of an empty statement at the top of the kernel
+// makes it fetch them together, behind one wait.
+__device__ __forceinline__ void fetch_together(const ActRows& a) {
+    asm volatile("" : : "s"(a.image), "s"(a.stride), "s"(a.x), "s"(a.x_dtype), "s"(a.k), "s"(a.row_token), "s"(a.gamma), "s"(a.round_f16), "s"(a.x_broadcast));
+}
+__device__ __forceinline__ void fetch_together(const WeightRoute& r) {
+    asm volatile("" : : "s"(r.expert), "s"(r.expert_stride), "s"(r.extra), "s"(r.expert64));
+}
 // the activation row (raw rows) that grid row `row` reads
 __device__ __forceinline__ size_t raw_row_of(const ActRows& a, int row) {
     return a.x_broadcast ? 0 : (a.row_token ? static_cast<size_t>(a.row_token[row]) : static_cast<size_t>(row));
