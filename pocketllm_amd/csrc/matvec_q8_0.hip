@@ -135,8 +135,9 @@ __device__ __forceinline__ const uint8_t* not_past(const uint8_t* p, const uint8
 
 __global__ __launch_bounds__(kStreamThreads) void q8_0_stream_kernel(
     const void* __restrict__ x, int x_dtype, const uint8_t* __restrict__ w, void* __restrict__ y, int y_dtype,
-    int k, int n, int pairs, uint32_t pairs_magic, int image_bytes, int cols) {
-    asm volatile("" : : "s"(x), "s"(x_dtype), "s"(w), "s"(y), "s"(y_dtype), "s"(k), "s"(n), "s"(pairs), "s"(pairs_magic), "s"(image_bytes), "s"(cols));   // the arguments in one batch of scalar loads, one wait
+    int k, int n, int pairs, uint32_t pairs_magic, int image_bytes, int cols, int rows_each, int rows_left) {
+    asm volatile("" : : "s"(x), "s"(x_dtype), "s"(w), "s"(y), "s"(y_dtype), "s"(k), "s"(n), "s"(pairs), "s"(pairs_magic), "s"(image_bytes), "s"(cols),
+                 "s"(rows_each), "s"(rows_left));   // the arguments in one batch of scalar loads, one wait
     extern __shared__ __align__(16) unsigned char smem[];
     unsigned char* img_hi = smem;
     unsigned char* img_lo = smem + static_cast<size_t>(pairs) * 80;
@@ -147,9 +148,12 @@ __global__ __launch_bounds__(kStreamThreads) void q8_0_stream_kernel(
     unsigned char* turn = smem + image_bytes + wave * kStepBytes;              // this wave's buffer
     float* partial = reinterpret_cast<float*>(smem + image_bytes + kStreamWaves * kStepBytes);   // [step][cols]
 
-    // this workgroup's rows [r0, r1): an even share of the matrix
-    const int r0 = static_cast<int>(static_cast<long long>(blockIdx.x) * n / gridDim.x);
-    const int r1 = static_cast<int>(static_cast<long long>(blockIdx.x + 1) * n / gridDim.x);
+    // this workgroup's rows [r0, r1): an even share of the matrix, rows_each = n / grid with one row more for the first
+    // rows_left = n % grid workgroups (quotient and remainder come from the host: a 64-bit division here is ~150 dependent
+    // instructions, twice, ahead of the kernel's first memory request)
+    const int bx = static_cast<int>(blockIdx.x);
+    const int r0 = bx * rows_each + min(bx, rows_left);
+    const int r1 = r0 + rows_each + (bx < rows_left ? 1 : 0);
     const int count = (r1 - r0) * pairs;
     const int steps = (count + 63) >> 6;
     const uint8_t* base = w + static_cast<size_t>(r0) * pairs * 68;
@@ -284,7 +288,7 @@ int launch_stream(const void* x, int x_dtype, const uint8_t* w, void* y, int y_d
     if (!grant_dynamic_smem(reinterpret_cast<const void*>(kern), plan.smem, granted)) return PLLM_ERR_UNSUPPORTED;
     const uint32_t magic = static_cast<uint32_t>(((1ull << 32) + pairs - 1) / pairs);
     hipLaunchKernelGGL(kern, dim3(plan.grid_x, rows), dim3(kStreamThreads), plan.smem, stream, x, x_dtype, w, y, y_dtype, k, n, pairs, magic,
-                       plan.image_bytes, plan.cols);
+                       plan.image_bytes, plan.cols, n / plan.grid_x, n % plan.grid_x);
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 

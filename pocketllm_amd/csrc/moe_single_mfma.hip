@@ -134,16 +134,13 @@ __global__ __launch_bounds__(64 * kW2Waves) void moe_single_w2_kernel(
     const int tile_bytes = 16 * row_bytes;
     const size_t tile_pos = static_cast<size_t>(blockIdx.x) * 16 * row_bytes;
 
-    // 1 KB pieces of the routes' tiles and images, dealt round the waves
-    const int tile_pieces = (tile_bytes + 1023) / 1024, image_pieces = (image_bytes + 1023) / 1024;
-    for (int q = wave; q < routes * tile_pieces; q += kW2Waves) {
-        const int r = q / tile_pieces, o = (q % tile_pieces) * 1024;
-        if (o + lane * 16 < tile_bytes)
-            lds_dma16(w2 + static_cast<size_t>(route_experts[r]) * expert_stride + tile_pos + o + lane * 16, lds0 + tile_off + r * tile_stride + o);
-    }
-    for (int q = wave; q < routes * image_pieces; q += kW2Waves) {
-        const int r = q / image_pieces, o = (q % image_pieces) * 1024;
-        if (o + lane * 16 < image_bytes) lds_dma16(h_image + static_cast<size_t>(r) * h_image_stride + o + lane * 16, lds0 + r * image_bytes + o);
+    // 1 KB pieces of the routes' tiles and images: wave = (route parity, piece mod 8), so that no wave divides to find its share
+    for (int r = wave >> 3; r < routes; r += kW2Waves / 8) {
+        const uint8_t* tile_src = w2 + static_cast<size_t>(route_experts[r]) * expert_stride + tile_pos;
+        for (int o = (wave & 7) * 1024; o < tile_bytes; o += 8 * 1024)
+            if (o + lane * 16 < tile_bytes) lds_dma16(tile_src + o + lane * 16, lds0 + tile_off + r * tile_stride + o);
+        for (int o = (wave & 7) * 1024; o < image_bytes; o += 8 * 1024)
+            if (o + lane * 16 < image_bytes) lds_dma16(h_image + static_cast<size_t>(r) * h_image_stride + o + lane * 16, lds0 + r * image_bytes + o);
     }
     FMT::dma_tables<kW2Waves>(lds0 + table_off, wave, lane);
     if (tid < 4) reinterpret_cast<uint32_t*>(smem + zero_off)[tid] = 0;
