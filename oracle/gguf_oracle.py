@@ -487,6 +487,24 @@ def q8_1_quantize(x: np.ndarray, group: int = 32):
     return q.reshape(t, k), scale
 
 
+def pow2_image(x: np.ndarray, group: int = 32) -> np.ndarray:
+    """The activations as the single-launch decode kernels of this package carry them (no counterpart in the reference, whose
+    decode matvec multiplies float activations, src/csrc/cuda_kernel_impl.cu:6082-6137): per `group` values one power-of-two
+    scale xs = 2^(E - 13), E the exponent of the group's largest magnitude (groups below 2^-113: E clamped, values round to
+    zero), and q = rint(x / xs) with |q| <= 2^14, which the kernels split into two int8 terms q = 256 hi + lo.  Returns the
+    rounded activations xs * q as float64 [T, K]: the kernels' results are the float statement of the operator applied to these.
+    """
+    t, k = x.shape
+    assert k % group == 0
+    xf = x.astype(np.float32).reshape(t, k // group, group)
+    amax = np.abs(xf).max(axis=-1)
+    e = np.maximum(amax.view(np.uint32) >> np.uint32(23), np.uint32(14)).astype(np.int64)      # biased exponent
+    xs = np.ldexp(1.0, (e - 140).astype(np.int64))                                             # 2^(e - 127 - 13), float64
+    q = np.rint(xf.astype(np.float64) / xs[..., None])                                         # exact quotient, ties to even
+    assert np.abs(q).max() <= 16384
+    return (q * xs[..., None]).reshape(t, k)
+
+
 # --------------------------------------------------------------------------------------------
 # matvec / matmul semantics
 # --------------------------------------------------------------------------------------------

@@ -389,6 +389,37 @@ def test_three_to_sixteen_rows_as_matrix_core_operands(mod, type_name, n, k, row
         assert np.abs(got - want).max() <= 2e-5 * np.abs(want).max()
 
 
+@pytest.mark.parametrize("type_name", ["q4_k", "q5_k", "q2_k", "q6_k", "iq4_xs"])
+def test_single_launch_kernels_multiply_the_power_of_two_image(mod, type_name):
+    """One activation row through the single-launch decode kernels: the result is the float statement of the operator applied to
+    the activations rounded onto a power-of-two scale per 32 values (oracle.pow2_image: x ~= 2^(E - 13) q, |q| <= 2^14), the dots
+    and the offset terms both taken from that image.  Against the image the distance is float32 summation error only (a wrong
+    scale, rounding mode or sum would show at 1e-5 or more); N(0, 1) activations in bf16 lie on the image almost everywhere, so
+    there the result is also close to the unrounded operator."""
+    rng = np.random.default_rng(4242)
+    for n, k in ((64, 5120), (48, 20480), (33, 1000)):
+        bpr = (k + 255) // 256
+        if type_name in ("q4_k", "q5_k", "q2_k"):
+            blocks = ENCODERS[type_name](np.pad(_weights(rng, n, k), ((0, 0), (0, bpr * 256 - k))))
+        else:
+            blocks = C.random_blocks(rng, type_name, n, bpr)
+        w = O.dequant_rows(blocks, type_name, k)
+        # a wide range of magnitudes inside every group, and a group of zeros
+        x_np = (rng.standard_normal((1, k)) * np.exp(rng.uniform(-6.0, 2.0, size=(1, k)))).astype(np.float32)
+        x_np[0, 64:96] = 0.0
+        for dt in (torch.float32, torch.bfloat16, torch.float16):
+            print(f"case image {type_name} n={n} k={k} {dt}", flush=True)
+            x_used, y = _run_dense(mod, type_name, blocks, x_np, dt, k)
+            pad = (-k) % 32
+            image = O.pow2_image(np.pad(x_used, ((0, 0), (0, pad))))[:, :k]
+            want_image = O.matmul_f(image, w)
+            err = O.rel_l2(y, want_image)
+            assert err <= 3e-6, (type_name, n, k, dt, err)
+        # N(0, 1) activations in bf16: nearly all of them lie on the image
+        x_used, y = _run_dense(mod, type_name, blocks, rng.standard_normal((1, k)).astype(np.float32), torch.bfloat16, k)
+        assert O.rel_l2(y, O.matmul_f(x_used, w)) <= 2e-5
+
+
 @pytest.mark.parametrize("type_name", ["q4_k", "q5_k", "q2_k", "q6_k", "iq4_xs", "iq2_xxs", "iq1_m", "iq2_xs", "iq3_xxs"])
 def test_few_row_calls_equal_the_prequantized_path(mod, type_name):
     """Calls of a few rows may quantize the activations inside the matvec kernel; the result is the same bits as quantizing ahead
