@@ -8,7 +8,7 @@
 // the reference's dequantize-then-matmul statement).  Codes become floats with v_cvt_pk_f32_fp8,
 // 16 FMAs per lane and chunk; a chunk lies inside one 128-wide scale block, so the block scale is
 // applied once per chunk.  Row sums are 64-lane reductions.
-#include "pllm_device.h"
+#include "block_mfma.h"
 #include "pllm_internal.h"
 #include <algorithm>
 
@@ -122,6 +122,28 @@ __device__ __forceinline__ float chunk_dot(const uint4& w, const float* xp) {
     return s;
 }
 
+// The same with the 16 activations as the caller's bf16 / fp16 values (the row lies in LDS as it came from memory): the values are
+// widened here, which costs vector instructions the kernel has to spare, and the row takes half the LDS reads.  Same products
+// and the same summation order as chunk_dot, so the same bits.
+template <bool BF16>
+__device__ __forceinline__ float chunk_dot16(const uint4& w, const uint16_t* xp) {
+    const uint4 xa = *reinterpret_cast<const uint4*>(xp);
+    const uint4 xb = *reinterpret_cast<const uint4*>(xp + 8);
+    auto lo = [](uint32_t u) { return BF16 ? __uint_as_float(u << 16) : f16_bits_to_float(u & 0xffffu); };
+    auto hi = [](uint32_t u) { return BF16 ? __uint_as_float(u & 0xffff0000u) : f16_bits_to_float(u >> 16); };
+    v2f a;
+    float s;
+    a = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w.x), false); s = a.x * lo(xa.x); s += a.y * hi(xa.x);
+    a = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w.x), true);  s += a.x * lo(xa.y); s += a.y * hi(xa.y);
+    a = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w.y), false); s += a.x * lo(xa.z); s += a.y * hi(xa.z);
+    a = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w.y), true);  s += a.x * lo(xa.w); s += a.y * hi(xa.w);
+    a = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w.z), false); s += a.x * lo(xb.x); s += a.y * hi(xb.x);
+    a = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w.z), true);  s += a.x * lo(xb.y); s += a.y * hi(xb.y);
+    a = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w.w), false); s += a.x * lo(xb.z); s += a.y * hi(xb.z);
+    a = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w.w), true);  s += a.x * lo(xb.w); s += a.y * hi(xb.w);
+    return s;
+}
+
 // k a multiple of 16, weight base and row pitch 16-byte aligned.  Persistent: the grid is sized to be resident at once, a workgroup stages the activation
 // row once and then walks groups of 4 weight rows (one per wave) in passes of 64 * 16 * ITERS bytes
 // per row, always holding the loads of its next pass (of the same group or of its next group) in a
@@ -173,7 +195,8 @@ __device__ __forceinline__ float floats_dot(const float (&f)[16], const float* x
 }
 
 // R activation rows (xs holds them k floats apart) against the pass's weights: the codes are converted once per chunk
-template <int ITERS, int F16S, bool SWIGLU, int R, int SLOTS>
+// XT: what xs holds: 0 / 3 float32 values, 1 bf16 and 2 fp16 values as they came from memory (one activation row only)
+template <int ITERS, int F16S, bool SWIGLU, int R, int XT, int SLOTS>
 __device__ __forceinline__ void fp8_multiply_pass(float (&acc)[SLOTS][R], const uint4 (&r)[SLOTS][ITERS],
                                                   const uint32_t (&scales)[SLOTS][ITERS], const float* xs, int k, int chunks, int c0, int lane) {
 #pragma unroll
@@ -185,7 +208,9 @@ __device__ __forceinline__ void fp8_multiply_pass(float (&acc)[SLOTS][R], const 
         for (int q = 0; q < SLOTS; ++q) {
             const float sc = scale_value<F16S>(scales[q][it]);
             if constexpr (R == 1) {
-                const float d = chunk_dot(r[q][it], xs + 16 * cc);
+                float d;
+                if constexpr (XT == 0 || XT == 3) d = chunk_dot(r[q][it], xs + 16 * cc);
+                else d = chunk_dot16<XT == 1>(r[q][it], reinterpret_cast<const uint16_t*>(xs) + 16 * cc);
                 acc[q][0] += ok ? d * sc : 0.0f;
             } else {
                 float f[16];
@@ -221,7 +246,7 @@ __device__ __forceinline__ void fp8_store_rows(float (&acc)[SLOTS][R], void* __r
     }
 }
 
-template <int ITERS, int F16S, bool SWIGLU, bool LONG_ROWS, int R>
+template <int ITERS, int F16S, bool SWIGLU, bool LONG_ROWS, int R, int XT = 0>
 __global__ __launch_bounds__(kThreads) void fp8_persistent_matvec_kernel(
     const void* __restrict__ x, int x_dtype, size_t x_stride, const Fp8Mat ma, const Fp8Mat mb,
     void* __restrict__ y, int y_dtype, size_t y_stride, int k, int n, int groups, int passes_of_long_rows, int total_rows) {
@@ -252,7 +277,16 @@ __global__ __launch_bounds__(kThreads) void fp8_persistent_matvec_kernel(
         for (int r = 0; r < R; ++r) acc[q][r] = 0.0f;
     int g = blockIdx.x, p = 0;               // the pass being multiplied
     int gn = g, pn = 0;                      // the pass being fetched
-    if constexpr (R == 1) {                  // the activation row is requested first and stored once the weights are on their way
+    if constexpr (R == 1 && XT != 0) {
+        // the row as it is (XT 1, 2: 16-bit values; 3: float32; row start on a 16-byte boundary) straight to LDS, requested ahead of
+        // the weights; loads complete in order, so once no more than the pass's weight loads are outstanding the row (and the
+        // pass's scales, which stand between them) has landed
+        const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_byte_ptr)smem));
+        constexpr int kValueBytes = XT == 3 ? 4 : 2;
+        dma_share<kWaves>(static_cast<const unsigned char*>(x) + static_cast<size_t>(arow0) * x_stride * kValueBytes, lds0, k * kValueBytes, wave, lane);
+        fp8_fetch_pass<ITERS, F16S, SWIGLU>(a, sa, ma, mb, g * rows_per_group + wave_row, rstride, n, chunks, 0, lane);
+        wait_vm<ITERS * kSlots<SWIGLU, R>>();
+    } else if constexpr (R == 1) {           // the activation row is requested first and stored once the weights are on their way
         float head[kStageBatch][4];
         const size_t xoff = static_cast<size_t>(arow0) * x_stride;
         stage_row_request(head, x, x_dtype, xoff, k);
@@ -270,13 +304,13 @@ __global__ __launch_bounds__(kThreads) void fp8_persistent_matvec_kernel(
         // (fetched without a condition, past the last group its rows again: a branch around the loads would make the compiler wait
         // for them at the join, ahead of the arithmetic on the other register set)
         fp8_fetch_pass<ITERS, F16S, SWIGLU>(b, sb, ma, mb, min(gn, groups - 1) * rows_per_group + wave_row, rstride, n, chunks, pn * kPassChunks, lane);
-        fp8_multiply_pass<ITERS, F16S, SWIGLU, R>(acc, a, sa, xs, k, chunks, p * kPassChunks, lane);
+        fp8_multiply_pass<ITERS, F16S, SWIGLU, R, XT>(acc, a, sa, xs, k, chunks, p * kPassChunks, lane);
         if (p == passes - 1) fp8_store_rows<SWIGLU, R>(acc, y, y_dtype, y_stride, arow0, total_rows, g * rows_per_group + wave_row, rstride, n, lane);
         g = gn; p = pn;
         if (g >= groups) break;
         if (++pn == passes) { pn = 0; gn += step; }
         fp8_fetch_pass<ITERS, F16S, SWIGLU>(a, sa, ma, mb, min(gn, groups - 1) * rows_per_group + wave_row, rstride, n, chunks, pn * kPassChunks, lane);
-        fp8_multiply_pass<ITERS, F16S, SWIGLU, R>(acc, b, sb, xs, k, chunks, p * kPassChunks, lane);
+        fp8_multiply_pass<ITERS, F16S, SWIGLU, R, XT>(acc, b, sb, xs, k, chunks, p * kPassChunks, lane);
         if (p == passes - 1) fp8_store_rows<SWIGLU, R>(acc, y, y_dtype, y_stride, arow0, total_rows, g * rows_per_group + wave_row, rstride, n, lane);
         g = gn; p = pn;
     }
@@ -489,8 +523,17 @@ int launch_any(const void* x, int x_dtype, size_t x_stride, const Fp8Mat& ma, co
     // (the form with the pass count as a variable needs 70 registers against 168 and is slower on rows of one pass: 21.5 against 18.9 us;
     // the form with a compile-time pass count keeps both register sets and all accumulators of several rows live at once and spills;
     // several activation rows always run the form with the pass count as a variable)
+    // one activation row that starts on a 16-byte boundary goes to LDS as it is (rows of one pass): 1 bf16, 2 fp16, 3 float32
+    const size_t value_bytes = x_dtype == PLLM_F32 ? 4 : 2;
+    const int xt = (share == 1 && passes == 1 && ((reinterpret_cast<uintptr_t>(x) | (x_stride * value_bytes)) & 15u) == 0)
+                       ? (x_dtype == PLLM_BF16 ? 1 : x_dtype == PLLM_F16 ? 2 : 3) : 0;
 #define PLLM_LAUNCH(I, RR) { \
         auto kern = (passes > 1 || RR > 1) ? fp8_persistent_matvec_kernel<I, F16S, SWIGLU, true, RR> : fp8_persistent_matvec_kernel<I, F16S, SWIGLU, false, 1>; \
+        if constexpr (RR == 1) { \
+            if (xt == 1) kern = fp8_persistent_matvec_kernel<I, F16S, SWIGLU, false, 1, 1>; \
+            else if (xt == 2) kern = fp8_persistent_matvec_kernel<I, F16S, SWIGLU, false, 1, 2>; \
+            else if (xt == 3) kern = fp8_persistent_matvec_kernel<I, F16S, SWIGLU, false, 1, 3>; \
+        } \
         if (smem > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, \
                                                     static_cast<int>(smem)) != hipSuccess) return PLLM_ERR_UNSUPPORTED; \
         hipLaunchKernelGGL(kern, grid, dim3(kThreads), smem, stream, x, x_dtype, x_stride, ma, mb, y, y_dtype, y_stride, k, n, groups, passes, rows); }
