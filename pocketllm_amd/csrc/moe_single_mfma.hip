@@ -53,6 +53,8 @@ __global__ __launch_bounds__(64 * kW13Waves) void moe_single_w13_kernel(
     const void* __restrict__ x, int x_dtype, int dim, int bpr, const int64_t* __restrict__ route_experts,
     const float* __restrict__ route_weights, const uint8_t* __restrict__ w1, const uint8_t* __restrict__ w3, int inter, float limit,
     unsigned char* __restrict__ h_image, size_t h_image_stride, int h_kpad, int raw_off, int tile_off, int tile_stride) {
+    asm volatile("" : : "s"(x), "s"(x_dtype), "s"(dim), "s"(bpr), "s"(route_experts), "s"(route_weights), "s"(w1), "s"(w3), "s"(inter),
+                 "s"(h_image), "s"(h_image_stride), "s"(h_kpad), "s"(raw_off), "s"(tile_off), "s"(tile_stride));   // the arguments in one batch of scalar loads, one wait
     extern __shared__ __align__(16) unsigned char smem[];
     const int kpad = bpr * 256;
     const int image_bytes = static_cast<int>(staged_x_bytes(kpad));
@@ -116,6 +118,8 @@ __global__ __launch_bounds__(64 * kW13Waves) void moe_single_w13_kernel(
 __global__ __launch_bounds__(64 * kW2Waves) void moe_single_w2_kernel(
     const unsigned char* __restrict__ h_image, size_t h_image_stride, int bpr, const int64_t* __restrict__ route_experts, int routes,
     const uint8_t* __restrict__ w2, size_t expert_stride, float* __restrict__ y, int dim, int tile_off, int tile_stride) {
+    asm volatile("" : : "s"(h_image), "s"(h_image_stride), "s"(bpr), "s"(route_experts), "s"(routes), "s"(w2), "s"(expert_stride), "s"(y),
+                 "s"(dim), "s"(tile_off), "s"(tile_stride));   // the arguments in one batch of scalar loads, one wait
     using FMT = IQ1Mm;
     extern __shared__ __align__(16) unsigned char smem[];
     const int kpad = bpr * 256;
