@@ -363,6 +363,19 @@ int pllm_gguf_moe_forward(const void* x, int x_dtype, int64_t tokens, int64_t di
                           float swiglu_limit, float* y, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * The routed experts of ONE token added into y [dim] of y_dtype (the residual stream of a decoder block: y += experts(x),
+ * float32 sum of what y holds and the routes' sum, rounded once), for callers that would otherwise convert and add in two
+ * further launches (the reference's block does: src/models/minimax_m2/architecture.py:404-413).  Same arguments and workspace as
+ * pllm_gguf_moe_forward with tokens == 1.  PLLM_ERR_UNSUPPORTED when the shape or the type pair has no kernel that sums the
+ * routes inside the down projection (IQ2_XXS or IQ1_M gate / up with IQ1_M down, whole 16-row tiles, 16-byte aligned tensors):
+ * call pllm_gguf_moe_forward and add.  No routes: y is left as it is.
+ */
+int pllm_gguf_moe_single_token_accumulate(const void* x, int x_dtype, int64_t dim, int64_t inter, const int64_t* route_experts,
+                                          const float* route_weights, int64_t routes, const uint8_t* w1, const uint8_t* w3, int w13_type,
+                                          const uint8_t* w2, int w2_type, float swiglu_limit, void* y, int y_dtype, void* workspace,
+                                          size_t workspace_bytes, void* stream);
+
+/*
  * Counting sort of the (token, k) routes of indices [tokens, topk] by local expert
  * (local = expert - experts_start, kept when 0 <= local < n_local), stable in (token, k) order.
  *   seg_starts int32 [n_local + 1]; route_tokens int64, route_weights float32, route_experts int32:

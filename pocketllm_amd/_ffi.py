@@ -42,6 +42,8 @@ SIGNATURES = {
     "pllm_gguf_moe_workspace_bytes": (_size_t, [_i64, _i64, _i64, _i64]),
     "pllm_gguf_moe_forward": (_int, [_c_void_p, _int, _i64, _i64, _i64, _c_void_p, _c_void_p, _c_void_p, _i64, _c_void_p, _i64,
                                      _c_void_p, _c_void_p, _int, _c_void_p, _int, ctypes.c_float, _c_void_p, _c_void_p, _size_t, _c_void_p]),
+    "pllm_gguf_moe_single_token_accumulate": (_int, [_c_void_p, _int, _i64, _i64, _c_void_p, _c_void_p, _i64, _c_void_p, _c_void_p, _int, _c_void_p, _int,
+                                                     ctypes.c_float, _c_void_p, _int, _c_void_p, _size_t, _c_void_p]),
     "pllm_moe_group_routes": (_int, [_c_void_p, _int, _c_void_p, _i64, _i64, _i64, _i64, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
     "pllm_gguf_dequantize_rows": (_int, [_c_void_p, _i64, _c_void_p, _int, _i64, _i64, _i64, _c_void_p, _int, _c_void_p]),
     "pllm_fp8_block_dequantize": (_int, [_c_void_p, _c_void_p, _i64, _i64, _c_void_p, _int, _c_void_p]),

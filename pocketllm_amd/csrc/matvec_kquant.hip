@@ -362,7 +362,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_image_matvec_kernel(
     int y_dtype, int n, int bpr, const float* __restrict__ gamma, float eps, int round_f16, const int64_t* __restrict__ row_token, int x_broadcast) {
     if constexpr (!PLAIN) {
         fetch_together(route);
-        asm volatile("" : : "s"(row_token), "s"(x_broadcast));
+        asm volatile("" : : "s"(static_cast<int>(row_token != nullptr)), "s"(x_broadcast));
     }
     asm volatile("" : : "s"(x), "s"(k), "s"(w), "s"(y), "s"(n), "s"(bpr));   // the arguments in one batch of scalar loads, one wait
     extern __shared__ __align__(16) unsigned char smem[];
@@ -682,7 +682,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_groups16_matvec_kernel(
     int y_dtype, int n, int bpr, const int64_t* __restrict__ row_token, int x_broadcast) {
     if constexpr (!PLAIN) {
         fetch_together(route);
-        asm volatile("" : : "s"(row_token), "s"(x_broadcast));
+        asm volatile("" : : "s"(static_cast<int>(row_token != nullptr)), "s"(x_broadcast));
     }
     asm volatile("" : : "s"(x), "s"(k), "s"(w), "s"(y), "s"(n), "s"(bpr));   // the arguments in one batch of scalar loads, one wait
     extern __shared__ __align__(16) unsigned char smem[];

@@ -576,6 +576,30 @@ size_t pllm_gguf_moe_workspace_bytes(int64_t tokens, int64_t routes, int64_t dim
     return dot_path > tile_path ? dot_path : tile_path;
 }
 
+int pllm_gguf_moe_single_token_accumulate(const void* x, int x_dtype, int64_t dim, int64_t inter, const int64_t* route_experts,
+                                          const float* route_weights, int64_t routes, const uint8_t* w1, const uint8_t* w3, int w13_type,
+                                          const uint8_t* w2, int w2_type, float swiglu_limit, void* y, int y_dtype, void* workspace,
+                                          size_t workspace_bytes, void* stream) {
+    using namespace pllm;
+    if (!x || !y || dim <= 0 || inter <= 0 || routes < 0) return PLLM_ERR_INVALID_ARGUMENT;
+    if (x_dtype != PLLM_F32 && x_dtype != PLLM_F16 && x_dtype != PLLM_BF16) return PLLM_ERR_INVALID_ARGUMENT;
+    if (y_dtype != PLLM_F32 && y_dtype != PLLM_F16 && y_dtype != PLLM_BF16) return PLLM_ERR_INVALID_ARGUMENT;
+    if (routes == 0) return PLLM_OK;                                          // nothing to add
+    if (!w1 || !w3 || !w2 || !route_weights || !route_experts) return PLLM_ERR_INVALID_ARGUMENT;
+    if (routes > 65535 || dim > (1 << 24) || inter > (1 << 24)) return PLLM_ERR_UNSUPPORTED;
+    if (!workspace || workspace_bytes < pllm_gguf_moe_workspace_bytes(1, routes, dim, inter)) return PLLM_ERR_WORKSPACE;
+    const int bpr_h = static_cast<int>((inter + 255) / 256);
+    const int R = static_cast<int>(routes), I = static_cast<int>(inter), D = static_cast<int>(dim);
+    if (routes * staged_x_bytes(bpr_h * 256) > 96 * 1024 || !moe_single_mfma_supports(w13_type, w2_type, D, I, R, x, w1, w3, w2))
+        return PLLM_ERR_UNSUPPORTED;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    unsigned char* himg = static_cast<unsigned char*>(workspace);
+    const size_t h_stride = act_image_256_bytes(bpr_h);
+    const int st = moe_single_w13_mfma(x, x_dtype, D, route_experts, route_weights, R, w1, w3, w13_type, I, swiglu_limit, himg, h_stride, s);
+    if (st != PLLM_OK) return st;
+    return moe_single_w2_mfma(himg, h_stride, I, route_experts, R, w2, nullptr, D, s, y, y_dtype);
+}
+
 int pllm_gguf_moe_forward(const void* x, int x_dtype, int64_t tokens, int64_t dim, int64_t inter,
                           const int64_t* route_tokens, const int64_t* route_experts, const int32_t* seg_starts, int64_t n_experts,
                           const float* route_weights, int64_t routes,

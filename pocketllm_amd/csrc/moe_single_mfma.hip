@@ -53,8 +53,9 @@ __global__ __launch_bounds__(64 * kW13Waves) void moe_single_w13_kernel(
     const void* __restrict__ x, int x_dtype, int dim, int bpr, const int64_t* __restrict__ route_experts,
     const float* __restrict__ route_weights, const uint8_t* __restrict__ w1, const uint8_t* __restrict__ w3, int inter, float limit,
     unsigned char* __restrict__ h_image, size_t h_image_stride, int h_kpad, int raw_off, int tile_off, int tile_stride) {
-    asm volatile("" : : "s"(x), "s"(x_dtype), "s"(dim), "s"(bpr), "s"(route_experts), "s"(route_weights), "s"(w1), "s"(w3), "s"(inter),
-                 "s"(h_image), "s"(h_image_stride), "s"(h_kpad), "s"(raw_off), "s"(tile_off), "s"(tile_stride));   // the arguments in one batch of scalar loads, one wait
+    // the arguments in one batch of scalar loads, one wait (not the route tables: their reads must stay scalar loads)
+    asm volatile("" : : "s"(x), "s"(x_dtype), "s"(dim), "s"(bpr), "s"(w1), "s"(w3), "s"(inter), "s"(h_image), "s"(h_image_stride), "s"(h_kpad),
+                 "s"(raw_off), "s"(tile_off), "s"(tile_stride));
     extern __shared__ __align__(16) unsigned char smem[];
     const int kpad = bpr * 256;
     const int image_bytes = static_cast<int>(staged_x_bytes(kpad));
@@ -117,9 +118,11 @@ __global__ __launch_bounds__(64 * kW13Waves) void moe_single_w13_kernel(
 // IQ1_M down projection.  LDS: the routes' hidden images | 16 zero bytes | codebook | partial sums | the routes' tiles.
 __global__ __launch_bounds__(64 * kW2Waves) void moe_single_w2_kernel(
     const unsigned char* __restrict__ h_image, size_t h_image_stride, int bpr, const int64_t* __restrict__ route_experts, int routes,
-    const uint8_t* __restrict__ w2, size_t expert_stride, float* __restrict__ y, int dim, int tile_off, int tile_stride) {
-    asm volatile("" : : "s"(h_image), "s"(h_image_stride), "s"(bpr), "s"(route_experts), "s"(routes), "s"(w2), "s"(expert_stride), "s"(y),
-                 "s"(dim), "s"(tile_off), "s"(tile_stride));   // the arguments in one batch of scalar loads, one wait
+    const uint8_t* __restrict__ w2, size_t expert_stride, float* __restrict__ y, int dim, int tile_off, int tile_stride,
+    void* __restrict__ add_into, int add_dtype) {
+    // the arguments in one batch of scalar loads, one wait (not the route table: its reads must stay scalar loads)
+    asm volatile("" : : "s"(h_image), "s"(h_image_stride), "s"(bpr), "s"(routes), "s"(w2), "s"(expert_stride), "s"(y), "s"(dim), "s"(tile_off),
+                 "s"(tile_stride), "s"(static_cast<int>(add_into != nullptr)), "s"(add_dtype));
     using FMT = IQ1Mm;
     extern __shared__ __align__(16) unsigned char smem[];
     const int kpad = bpr * 256;
@@ -177,7 +180,9 @@ __global__ __launch_bounds__(64 * kW2Waves) void moe_single_w2_kernel(
         float total = 0.0f;
 #pragma unroll
         for (int v = 0; v < kW2Waves; ++v) total += partial[v * 16 + tid];
-        y[blockIdx.x * 16 + tid] = total;
+        // the routes' sum, or the residual stream with the sum added (float32 addition, one rounding to the stream's type)
+        if (add_into) store_any(add_into, add_dtype | 0x100, static_cast<size_t>(blockIdx.x) * 16 + tid, total);
+        else y[blockIdx.x * 16 + tid] = total;
     }
 }
 
@@ -1008,7 +1013,7 @@ int moe_single_w13_mfma(const void* x, int x_dtype, int dim, const int64_t* rout
 }
 
 int moe_single_w2_mfma(const unsigned char* h_image, size_t h_stride, int inter, const int64_t* route_experts, int routes, const uint8_t* w2,
-                       float* y, int dim, hipStream_t stream) {
+                       float* y, int dim, hipStream_t stream, void* add_into, int add_dtype) {
     const int bpr = (inter + 255) / 256;
     const int image_bytes = static_cast<int>(staged_x_bytes(bpr * 256));
     const int tile_bytes = 16 * bpr * IQ1Mm::kBlockBytes;
@@ -1019,7 +1024,7 @@ int moe_single_w2_mfma(const unsigned char* h_image, size_t h_stride, int inter,
     if (!allow_lds(moe_single_w2_kernel, smem)) return PLLM_ERR_UNSUPPORTED;
     const size_t expert_stride = static_cast<size_t>(dim) * bpr * IQ1Mm::kBlockBytes;
     hipLaunchKernelGGL(moe_single_w2_kernel, dim3(dim / 16), dim3(64 * kW2Waves), smem, stream, h_image, h_stride, bpr, route_experts, routes, w2,
-                       expert_stride, y, dim, tile_off, tile_stride);
+                       expert_stride, y, dim, tile_off, tile_stride, add_into, add_dtype);
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 

@@ -93,12 +93,15 @@ __device__ __forceinline__ size_t route_offset(const WeightRoute& r, int row) {
 // Kernels that take these structs test their fields one after the other (routed? further projections? a row map?), and the
 // compiler loads each field where it is first needed: a scalar load and a wait per test, several hundred nanoseconds of a
 // short kernel before its first memory request.  Naming the fields as inputs of an empty statement at the top of the kernel
-// makes it fetch them together, behind one wait.
+// makes it fetch them together, behind one wait.  Pointers to the per-row tables (expert numbers, row maps) go in as the
+// integers the tests compare, not as pointers: a pointer that has been an operand of an asm statement is no longer known to
+// point at memory nobody writes, and its reads turn from scalar loads into vector loads with a full wait behind each.
 __device__ __forceinline__ void fetch_together(const ActRows& a) {
-    asm volatile("" : : "s"(a.image), "s"(a.stride), "s"(a.x), "s"(a.x_dtype), "s"(a.k), "s"(a.row_token), "s"(a.gamma), "s"(a.round_f16), "s"(a.x_broadcast));
+    asm volatile("" : : "s"(a.image), "s"(a.stride), "s"(a.x), "s"(a.x_dtype), "s"(a.k), "s"(static_cast<int>(a.row_token != nullptr)), "s"(static_cast<int>(a.gamma != nullptr)),
+                 "s"(a.round_f16), "s"(a.x_broadcast));
 }
 __device__ __forceinline__ void fetch_together(const WeightRoute& r) {
-    asm volatile("" : : "s"(r.expert), "s"(r.expert_stride), "s"(r.extra), "s"(r.expert64));
+    asm volatile("" : : "s"(static_cast<int>(r.expert != nullptr)), "s"(r.expert_stride), "s"(r.extra), "s"(static_cast<int>(r.expert64 != nullptr)));
 }
 // the activation row (raw rows) that grid row `row` reads
 __device__ __forceinline__ size_t raw_row_of(const ActRows& a, int row) {
@@ -154,7 +157,7 @@ int moe_single_w13_mfma(const void* x, int x_dtype, int dim, const int64_t* rout
                         const uint8_t* w1, const uint8_t* w3, int w13_type, int inter, float limit, unsigned char* h_image, size_t h_stride,
                         hipStream_t stream);
 int moe_single_w2_mfma(const unsigned char* h_image, size_t h_stride, int inter, const int64_t* route_experts, int routes, const uint8_t* w2,
-                       float* y, int dim, hipStream_t stream);
+                       float* y, int dim, hipStream_t stream, void* add_into = nullptr, int add_dtype = 0);
 
 // Routed experts of several tokens on the matrix cores (same file): routes grouped by expert (seg), x images from
 // act_image_256, hidden images with one scale per 16 values, per-route outputs into partial [R, dim].

@@ -694,6 +694,29 @@ def gguf_moe_single_token_forward(x, route_slots, route_weights, w1_blocks, w3_b
                      _TYPE_OF_BLOCK_BYTES[w1_blocks.size(3)], _TYPE_OF_BLOCK_BYTES[w2_blocks.size(3)], swiglu_limit)
 
 
+def gguf_moe_single_token_accumulate_forward(x, route_slots, route_weights, w1_blocks, w3_blocks, w2_blocks, swiglu_limit, y: torch.Tensor) -> bool:
+    """y [1, D] (float16, bfloat16 or float32) += the routed experts of the one token x, inside the down projection's launch
+    (no counterpart in the reference, whose block converts and adds afterwards: src/models/minimax_m2/architecture.py:404-413).
+    Returns False, with y untouched, when the shape or the type pair has no such kernel: take gguf_moe_single_token_forward and add."""
+    _single_token_checks(x, route_slots, route_weights, w1_blocks, w3_blocks, w2_blocks)
+    _check(w1_blocks.size(3) == w3_blocks.size(3) and w1_blocks.size(3) in _TYPE_OF_BLOCK_BYTES, "w1/w3 must be blocks of one supported GGUF type")
+    _check(w2_blocks.size(3) in _TYPE_OF_BLOCK_BYTES, "w2 must be blocks of a supported GGUF type")
+    _check(y.is_cuda and y.is_contiguous() and y.numel() == x.size(-1) and y.dtype in _DTYPE_CODE, "y must be a contiguous CUDA tensor of D values (float16, bfloat16 or float32)")
+    dim, inter, routes = x.size(-1), w1_blocks.size(1), route_weights.numel()
+    lib = _lib()
+    with _on_device(x.device):
+        ws_bytes = lib.pllm_gguf_moe_workspace_bytes(1, routes, dim, inter)
+        ws = _workspace(ws_bytes, x.device)
+        st = lib.pllm_gguf_moe_single_token_accumulate(
+            x.data_ptr(), _DTYPE_CODE[x.dtype], dim, inter, route_slots.data_ptr(), route_weights.data_ptr(), routes,
+            w1_blocks.data_ptr(), w3_blocks.data_ptr(), _TYPE_OF_BLOCK_BYTES[w1_blocks.size(3)], w2_blocks.data_ptr(),
+            _TYPE_OF_BLOCK_BYTES[w2_blocks.size(3)], float(swiglu_limit), y.data_ptr(), _DTYPE_CODE[y.dtype], ws.data_ptr(), ws_bytes, _stream(x.device))
+    if st == _ffi.PLLM_ERR_UNSUPPORTED:
+        return False
+    _ffi.check(st, "gguf_moe_single_token_accumulate_forward")
+    return True
+
+
 def gguf_moe_single_token_iq2_q2k_forward(x, route_slots, route_weights, w1_blocks, w3_blocks, w2_blocks, signed_grid, swiglu_limit) -> torch.Tensor:
     """src/csrc/cuda_kernel.cpp:769-818: float32 [1, D]."""
     _single_token_checks(x, route_slots, route_weights, w1_blocks, w3_blocks, w2_blocks)

@@ -109,8 +109,14 @@ class MiniMaxMoE:
             if not (self.expert_start == 0 and self.expert_count >= int(self.args.n_routed_experts)):   # a slice of the experts is resident
                 here = (ids >= self.expert_start) & (ids < self.expert_start + self.expert_count)
                 ids, ws = ids[here] - self.expert_start, ws[here]
-            out = nothing() if ids.numel() == 0 else self._cuda.gguf_moe_single_token_forward(
-                tokens, ids.contiguous(), ws.contiguous(), w.w1.blocks, w.w3.blocks, w.w2.blocks, 0.0)
+            if ids.numel() == 0:
+                out = nothing()
+            else:
+                # the down projection adds the routes' sum into the residual stream itself where it has a kernel for it
+                if residual is not None and residual.is_contiguous() and self._cuda.gguf_moe_single_token_accumulate_forward(
+                        tokens, ids.contiguous(), ws.contiguous(), w.w1.blocks, w.w3.blocks, w.w2.blocks, 0.0, residual):
+                    return residual
+                out = self._cuda.gguf_moe_single_token_forward(tokens, ids.contiguous(), ws.contiguous(), w.w1.blocks, w.w3.blocks, w.w2.blocks, 0.0)
         else:
             _, route_tokens, route_weights, seg = self._cuda.moe_group_routes(chosen, gate_w, self.expert_start, self.expert_count)
             out = nothing() if route_tokens.numel() == 0 else self._cuda.gguf_moe_prefill_grouped_forward(

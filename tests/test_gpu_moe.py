@@ -129,6 +129,34 @@ def test_baseline_config_single_token_shapes(mod):
     assert O.rel_l2(y.cpu().numpy(), want) <= TOL
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_single_token_experts_added_into_the_residual_stream(mod, dtype):
+    """y += experts(x) inside the down projection's launch: the float32 sum of what y held and the result of the plain operator
+    (bit for bit the same routes' sum), rounded once to y's type; shapes or type pairs without such a kernel report False and
+    leave y alone."""
+    rng = np.random.default_rng(2718)
+    e, d, inter, topk = 16, 3072, 1536, 8
+    w1 = _expert_blocks(rng, "iq2_xxs", e, inter, d)
+    w3 = _expert_blocks(rng, "iq2_xxs", e, inter, d)
+    w2 = _expert_blocks(rng, "iq1_m", e, d, inter)
+    idx, wts = _route(rng, 1, e, topk)
+    x = torch.from_numpy(rng.standard_normal((1, d)).astype(np.float32)).to(DEV).to(torch.bfloat16)
+    slots, rw = torch.from_numpy(idx[0]).to(DEV), torch.from_numpy(wts[0]).to(DEV)
+    dw1, dw3, dw2 = (torch.from_numpy(a).to(DEV) for a in (w1, w3, w2))
+    plain = mod.gguf_moe_single_token_forward(x, slots, rw, dw1, dw3, dw2, 0.0)
+    stream = torch.from_numpy(rng.standard_normal((1, d)).astype(np.float32)).to(DEV).to(dtype)
+    y = stream.clone()
+    print(f"case accumulate {dtype}", flush=True)
+    assert mod.gguf_moe_single_token_accumulate_forward(x, slots, rw, dw1, dw3, dw2, 0.0, y) is True
+    torch.cuda.synchronize()
+    assert torch.equal(y, (stream.float() + plain).to(dtype))
+    # a type pair whose down projection has no such kernel: refused, y untouched
+    w2q = torch.from_numpy(_expert_blocks(rng, "q2_k", e, d, inter)).to(DEV)
+    y2 = stream.clone()
+    assert mod.gguf_moe_single_token_accumulate_forward(x, slots, rw, dw1, dw3, w2q, 0.0, y2) is False
+    assert torch.equal(y2, stream)
+
+
 def test_baseline_config_grouped_256_tokens_256_experts(mod):
     """BASELINE config 5 at T = 256: 256 experts, top-8 softmax routing, 2048 routes, every weight tensor at its full size.
     The oracle restates the operator for 32 sampled tokens (their 256 routes, full output rows); every other token is
