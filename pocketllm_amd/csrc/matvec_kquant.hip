@@ -676,10 +676,13 @@ struct WaveQ6K {
     }
 };
 
-template <typename FMT, int ITERS, int DEPTH, bool X16, bool PLAIN = false>
+// NORM (one pass of the block loop, as in wave_image_matvec_kernel): the wave requests the slices of all its blocks at once, their
+// squares are its share of the row's sum, the shares meet in LDS behind one barrier and the slices are scaled by rstd * gamma
+// as they are quantized.
+template <typename FMT, int ITERS, int DEPTH, bool X16, bool PLAIN = false, bool NORM = false>
 __global__ __launch_bounds__(64 * kMaxWaves) void wave_groups16_matvec_kernel(
     const void* __restrict__ x, int x_dtype, int k, const WeightRoute route, const uint8_t* __restrict__ w, void* __restrict__ y,
-    int y_dtype, int n, int bpr, const int64_t* __restrict__ row_token, int x_broadcast) {
+    int y_dtype, int n, int bpr, const int64_t* __restrict__ row_token, int x_broadcast, const float* __restrict__ gamma, float eps, int round_f16) {
     if constexpr (!PLAIN) {
         fetch_together(route);
         asm volatile("" : : "s"(static_cast<int>(row_token != nullptr)), "s"(x_broadcast));
@@ -716,30 +719,71 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_groups16_matvec_kernel(
 
     if (lane < 4) reinterpret_cast<uint32_t*>(slot + kQ2SlotBytes)[lane] = 0;
     float acc = 0.0f;
+    constexpr int kHeldX = NORM ? ITERS : DEPTH;
+    float rstd = 1.0f;
     for (int b0 = wave; b0 < bpr; b0 += waves * ITERS) {
-        RawX<X16> raw[DEPTH];
+        RawX<X16> raw[kHeldX];
+        RawX<false> graw[NORM ? ITERS : 1];
         typename FMT::Regs regs[DEPTH];
         auto request_x = [&](int it) {
             const int b = b0 + it * waves;
-            request_raw4<X16>(raw[it % DEPTH], x, xoff, 256 * b + 4 * lane, b < bpr ? k : 0);
+            request_raw4<X16>(raw[it % kHeldX], x, xoff, 256 * b + 4 * lane, b < bpr ? k : 0);
         };
         auto request_w = [&](int it) {
             const int b = b0 + it * waves;
             FMT::load(regs[it % DEPTH], wrow + static_cast<size_t>(min(b, bpr - 1)) * FMT::kBlockBytes, ks);   // clamped: always a valid address
         };
 #pragma unroll
-        for (int it = 0; it < DEPTH; ++it) request_x(it);
+        for (int it = 0; it < kHeldX; ++it) request_x(it);
+        if constexpr (NORM) {
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it) {
+                const int b = b0 + it * waves;
+                request_raw4<false>(graw[it], gamma, 0, 256 * b + 4 * lane, b < bpr ? k : 0);
+            }
+        }
         __builtin_amdgcn_sched_barrier(0);                                  // keep the issue order: memory returns a wave's loads in it
 #pragma unroll
         for (int it = 0; it < DEPTH; ++it) request_w(it);
         __builtin_amdgcn_sched_barrier(0);
+        if constexpr (NORM) {
+            float ss = 0.0f;
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it) {
+                const int b = b0 + it * waves;
+                if (k != 256 * bpr) {                                        // rows that end inside their last block
+                    settle_raw4<X16>(raw[it], 256 * b + 4 * lane, b < bpr ? k : 0);
+                    settle_raw4<false>(graw[it], 256 * b + 4 * lane, b < bpr ? k : 0);
+                }
+                float v[4];
+                raw_to_float4<X16>(raw[it], x_dtype, v);
+                if (b < bpr) ss += (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
+            }
+            ss = group_sum<64>(ss);
+            float* shares = partial + kMaxWaves * kRowsPerWg;                // [waves]
+            if (lane == 0) shares[wave] = ss;
+            __syncthreads();
+            float total = 0.0f;
+            for (int v = 0; v < waves; ++v) total += shares[v];
+            rstd = rsqrtf(total / static_cast<float>(k) + eps);
+        }
 #pragma unroll
         for (int it = 0; it < ITERS; ++it) {
             const int b = b0 + it * waves;
             if (b < bpr) {                                                   // wave-uniform
                 float v[4];
-                if (k != 256 * bpr) settle_raw4<X16>(raw[it % DEPTH], 256 * b + 4 * lane, k);
-                raw_to_float4<X16>(raw[it % DEPTH], x_dtype, v);
+                if constexpr (!NORM)
+                    if (k != 256 * bpr) settle_raw4<X16>(raw[it % kHeldX], 256 * b + 4 * lane, k);
+                raw_to_float4<X16>(raw[it % kHeldX], x_dtype, v);
+                if constexpr (NORM) {
+                    const float g[4] = {__uint_as_float(graw[it].v.x), __uint_as_float(graw[it].v.y), __uint_as_float(graw[it].v.z), __uint_as_float(graw[it].v.w)};
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        float t = v[i] * rstd * g[i];                        // values past k are zeros on both sides
+                        if (round_f16) t = static_cast<float>(static_cast<_Float16>(t));
+                        v[i] = t;
+                    }
+                }
                 uint32_t qh, ql;
                 float scale;
                 float sum4;                                                 // the four values as the image holds them, summed (exact): the
@@ -773,7 +817,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_groups16_matvec_kernel(
                 __builtin_amdgcn_wave_barrier();                            // the next block's slice overwrites the slot
             }
             if (it + DEPTH < ITERS) {
-                request_x(it + DEPTH);
+                if constexpr (!NORM) request_x(it + DEPTH);
                 __builtin_amdgcn_sched_barrier(0);
                 request_w(it + DEPTH);
                 __builtin_amdgcn_sched_barrier(0);
@@ -798,11 +842,12 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_groups16_matvec_kernel(
 template <typename KERN>
 int launch_q2k_kernel(KERN kern, const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype,
                       int rows, int n, int bpr, int waves, hipStream_t stream) {
-    const size_t smem = static_cast<size_t>(waves) * (kQ2SlotBytes + 16) + static_cast<size_t>(kMaxWaves) * kRowsPerWg * sizeof(float);
+    const size_t smem = static_cast<size_t>(waves) * (kQ2SlotBytes + 16) + static_cast<size_t>(kMaxWaves * kRowsPerWg + waves) * sizeof(float);
     int tallest = n;
     for (int m = 0; m < route.extra; ++m) tallest = tallest > route.more_n[m] ? tallest : route.more_n[m];
     dim3 grid((tallest + kRowsPerWg - 1) / kRowsPerWg, rows, 1 + route.extra);
-    hipLaunchKernelGGL(kern, grid, dim3(64 * waves), smem, stream, act.x, act.x_dtype, act.k, route, w, y, y_dtype, n, bpr, act.row_token, act.x_broadcast);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * waves), smem, stream, act.x, act.x_dtype, act.k, route, w, y, y_dtype, n, bpr, act.row_token, act.x_broadcast,
+                       act.gamma, act.eps, act.round_f16);
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 
@@ -844,18 +889,24 @@ int launch_k45(const ActRows& act, const WeightRoute& route, const uint8_t* w, v
 
 template <typename FMT>
 int launch_groups16(const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, hipStream_t stream) {
-    // raw rows without normalisation, blocks (of every expert) on the format's boundary; everything else stays with the other kernels
-    if (!act.x || act.k < 4 || act.gamma || ((reinterpret_cast<uintptr_t>(w) | route.expert_stride) & (FMT::kAlign - 1))) return PLLM_ERR_UNSUPPORTED;
+    // raw rows, blocks (of every expert) on the format's boundary; a normalisation ahead only on unrouted rows; everything else stays
+    // with the other kernels
+    if (!act.x || act.k < 4 || ((reinterpret_cast<uintptr_t>(w) | route.expert_stride) & (FMT::kAlign - 1))) return PLLM_ERR_UNSUPPORTED;
+    if (act.gamma && (routed(route) || act.row_token || act.x_broadcast)) return PLLM_ERR_UNSUPPORTED;
     for (int m = 0; m < route.extra; ++m)
         if (reinterpret_cast<uintptr_t>(route.more_w[m]) & (FMT::kAlign - 1)) return PLLM_ERR_UNSUPPORTED;
     int waves, iters;
     int tiles = (n + kRowsPerWg - 1) / kRowsPerWg;
     for (int m = 0; m < route.extra; ++m) tiles += (route.more_n[m] + kRowsPerWg - 1) / kRowsPerWg;
     split_blocks(bpr, tiles * rows, waves, iters);
+    if (act.gamma && waves * iters < bpr) return PLLM_ERR_UNSUPPORTED;        // the normalised form holds a wave's slices of the whole row
     constexpr int kMaxDepth = 2;            // blocks in flight per wave: five waves per SIMD fit with 2 (Q6_K with 2, 3, 4 and 5 ran within 3 % of each other, Q2_K 14.6 us with 2 against 15.2 with 5)
     const bool plain = !routed(route) && route.extra == 0 && !act.row_token && !act.x_broadcast;
 #define PLLM_CASE(I) case I: { \
         constexpr int D = I < kMaxDepth ? I : kMaxDepth; \
+        if (act.gamma) \
+            return act.x_dtype == PLLM_F32 ? launch_q2k_kernel(wave_groups16_matvec_kernel<FMT, I, D, false, false, true>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream) \
+                                           : launch_q2k_kernel(wave_groups16_matvec_kernel<FMT, I, D, true, false, true>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream); \
         if (plain) \
             return act.x_dtype == PLLM_F32 ? launch_q2k_kernel(wave_groups16_matvec_kernel<FMT, I, D, false, true>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream) \
                                            : launch_q2k_kernel(wave_groups16_matvec_kernel<FMT, I, D, true, true>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream); \
