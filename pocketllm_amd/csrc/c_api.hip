@@ -113,9 +113,10 @@ static bool quantizes_in_kernel(int type_id, int64_t rows, int64_t n, int64_t bp
     return pllm_gguf_block_bytes(type_id) != 0;
 }
 
-// Q4_K / Q5_K calls of 17 - 48 rows that the tile kernel would otherwise take
-static bool uses_rows64(int type_id, int64_t rows, int64_t n, int64_t bpr, const uint8_t* blocks) {
-    return gguf_uses_tile_gemm(type_id, rows, n, bpr) && pllm::k45_rows64_supports(type_id, static_cast<int>(rows), static_cast<int>(n), static_cast<int>(bpr), blocks);
+// Q4_K / Q5_K calls of 17 - 48 rows (up to 64 rows of 16-bit activations the kernel reads as they are: raw16) that the tile kernel
+// would otherwise take
+static bool uses_rows64(int type_id, int64_t rows, int64_t n, int64_t bpr, const uint8_t* blocks, bool raw16) {
+    return gguf_uses_tile_gemm(type_id, rows, n, bpr) && pllm::k45_rows64_supports(type_id, static_cast<int>(rows), static_cast<int>(n), static_cast<int>(bpr), blocks, raw16);
 }
 
 }  // extern "C"
@@ -172,7 +173,7 @@ int pllm_gguf_quant_gemm(const void* x, int x_dtype, const uint8_t* blocks, int 
         if (st16 != PLLM_ERR_UNSUPPORTED) return st16;
     }
     // Q4_K / Q5_K, 17 - 48 rows: every block decoded once in registers and multiplied into all rows
-    if (uses_rows64(type_id, rows, n, blocks_per_row, blocks))
+    if (uses_rows64(type_id, rows, n, blocks_per_row, blocks, pllm::k45_rows64_reads_raw(x, x_dtype, static_cast<int>(k), static_cast<int>(n), bpr)))
         return pllm::k45_rows64_gemm(x, x_dtype, blocks, type_id, y, y_dtype, static_cast<int>(rows), static_cast<int>(k), static_cast<int>(n), bpr,
                                      workspace, workspace_bytes, s);
     if (gguf_uses_tile_gemm(type_id, rows, n, blocks_per_row))
@@ -219,7 +220,7 @@ size_t pllm_gguf_quant_gemm_workspace_bytes(int type_id, int64_t rows, int64_t k
     if (gguf_uses_tile_gemm(type_id, rows, n, blocks_per_row)) {
         // (the weights' alignment is not known here: room for either kernel)
         const size_t tiles = pllm::gemm_f16_workspace_bytes(static_cast<int>(rows), static_cast<int>(n), static_cast<int>(blocks_per_row));
-        const size_t rows64 = uses_rows64(type_id, rows, n, blocks_per_row, nullptr)
+        const size_t rows64 = uses_rows64(type_id, rows, n, blocks_per_row, nullptr, true)
                                   ? pllm::k45_rows64_workspace_bytes(static_cast<int>(rows), static_cast<int>(n), static_cast<int>(blocks_per_row)) : 0;
         return tiles > rows64 ? tiles : rows64;
     }

@@ -62,13 +62,17 @@ __global__ __launch_bounds__(256) void act_f16_kernel(const void* __restrict__ x
 // The same for rows of at most 8192 values with 16-bit inputs (the usual case): one wave per row
 // keeps the row in registers between the maximum and the conversion, so x is read once.
 // bits(v) = the value as float32: bf16 is the high half of a float32, fp16 converts in hardware.
-template <bool BF16>
+// WPR = waves per row: 1 (four rows per workgroup) or 4 (one row per workgroup, for calls of few rows: four times the
+// workgroups, a quarter of the row per wave; the waves meet in LDS for the maximum).
+template <bool BF16, int WPR>
 __global__ __launch_bounds__(256) void act_f16_rows_kernel(const uint16_t* __restrict__ x, _Float16* __restrict__ xh,
                                                            float* __restrict__ scale, int rows, int k, int kp, const int64_t* __restrict__ row_map) {
-    const int lane = threadIdx.x & 63, row = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (row >= rows) return;
+    __shared__ float wave_max[4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int row = WPR == 1 ? blockIdx.x * 4 + wave : blockIdx.x, part = WPR == 1 ? 0 : wave;
+    if (row >= rows) return;                       // (a whole workgroup when WPR = 4)
     const uint16_t* src = x + static_cast<size_t>(row_map ? row_map[row] : row) * k;
-    constexpr int kMaxPieces = 16;                 // 16 pieces x 64 lanes x 8 values
+    constexpr int kMaxPieces = 16 / WPR;           // 16 pieces x 64 lanes x 8 values per row
     uint4 piece[kMaxPieces];
     float am = 0.0f;
     auto value = [](uint32_t word, int hi) -> float {
@@ -78,7 +82,7 @@ __global__ __launch_bounds__(256) void act_f16_rows_kernel(const uint16_t* __res
     };
 #pragma unroll
     for (int i = 0; i < kMaxPieces; ++i) {
-        const int e0 = (i * 64 + lane) * 8;
+        const int e0 = ((i * WPR + part) * 64 + lane) * 8;
         piece[i] = make_uint4(0, 0, 0, 0);
         if (e0 < k) piece[i] = *reinterpret_cast<const uint4*>(src + e0);          // k is a multiple of 8 here
         const uint32_t wds[4] = {piece[i].x, piece[i].y, piece[i].z, piece[i].w};
@@ -86,6 +90,11 @@ __global__ __launch_bounds__(256) void act_f16_rows_kernel(const uint16_t* __res
         for (int j = 0; j < 4; ++j) am = fmaxf(am, fmaxf(fabsf(value(wds[j], 0)), fabsf(value(wds[j], 1))));
     }
     am = group_max<64>(am);
+    if constexpr (WPR > 1) {
+        if (lane == 0) wave_max[wave] = am;
+        __syncthreads();
+        am = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
+    }
     int e = 0;
     if (am > 0.0f && am < __uint_as_float(0x7f800000u)) {
         (void)frexpf(am, &e);
@@ -95,7 +104,7 @@ __global__ __launch_bounds__(256) void act_f16_rows_kernel(const uint16_t* __res
     _Float16* out = xh + static_cast<size_t>(row) * kp;
 #pragma unroll
     for (int i = 0; i < kMaxPieces; ++i) {
-        const int e0 = (i * 64 + lane) * 8;
+        const int e0 = ((i * WPR + part) * 64 + lane) * 8;
         if (e0 >= kp) continue;
         const uint32_t wds[4] = {piece[i].x, piece[i].y, piece[i].z, piece[i].w};
         half8 o;
@@ -106,7 +115,7 @@ __global__ __launch_bounds__(256) void act_f16_rows_kernel(const uint16_t* __res
         }
         *reinterpret_cast<half8*>(out + e0) = o;
     }
-    if (lane == 0) scale[row] = ldexpf(1.0f, e);
+    if (lane == 0 && part == 0) scale[row] = ldexpf(1.0f, e);
 }
 
 // Hidden activations of the routed experts, one wave per route: h = silu(min(g, L)) * clamp(u, +-L) * w_r
@@ -802,10 +811,16 @@ float* stage_activations(const void* x, int x_dtype, int rows, int k, int bpr, v
     base += align256(static_cast<size_t>(rows) * sizeof(float));
     const bool narrow = (x_dtype == PLLM_BF16 || x_dtype == PLLM_F16) && k % 8 == 0 && bpr * 256 <= 8192 &&
                         reinterpret_cast<uintptr_t>(x) % 16 == 0;
-    if (narrow && x_dtype == PLLM_BF16)
-        hipLaunchKernelGGL(act_f16_rows_kernel<true>, dim3((rows + 3) / 4), dim3(256), 0, stream, static_cast<const uint16_t*>(x), xh, xscale, rows, k, bpr * 256, row_map);
+    const bool few = rows <= 512;                  // one row per workgroup while that leaves the grid small
+    const uint16_t* x16 = static_cast<const uint16_t*>(x);
+    if (narrow && x_dtype == PLLM_BF16 && few)
+        hipLaunchKernelGGL((act_f16_rows_kernel<true, 4>), dim3(rows), dim3(256), 0, stream, x16, xh, xscale, rows, k, bpr * 256, row_map);
+    else if (narrow && x_dtype == PLLM_BF16)
+        hipLaunchKernelGGL((act_f16_rows_kernel<true, 1>), dim3((rows + 3) / 4), dim3(256), 0, stream, x16, xh, xscale, rows, k, bpr * 256, row_map);
+    else if (narrow && few)
+        hipLaunchKernelGGL((act_f16_rows_kernel<false, 4>), dim3(rows), dim3(256), 0, stream, x16, xh, xscale, rows, k, bpr * 256, row_map);
     else if (narrow)
-        hipLaunchKernelGGL(act_f16_rows_kernel<false>, dim3((rows + 3) / 4), dim3(256), 0, stream, static_cast<const uint16_t*>(x), xh, xscale, rows, k, bpr * 256, row_map);
+        hipLaunchKernelGGL((act_f16_rows_kernel<false, 1>), dim3((rows + 3) / 4), dim3(256), 0, stream, x16, xh, xscale, rows, k, bpr * 256, row_map);
     else
         hipLaunchKernelGGL(act_f16_kernel, dim3(rows), dim3(256), 0, stream, x, x_dtype, xh, xscale, k, bpr * 256, row_map);
     xh_out = xh;

@@ -15,6 +15,7 @@
 // both terms; the lane that holds C[4s .. 4s+3][n] owns groups 2s and 2s+1 of row n and applies
 // their 6-bit scales and mins in float.  Which k sits where inside an MFMA is irrelevant as long
 // as A and B agree, and both are built per (lane / 16, byte) from the same positions.
+#include "block_mfma.h"
 #include "pllm_device.h"
 #include "pllm_internal.h"
 
@@ -1109,11 +1110,10 @@ int launch_rows16(const void* x, int x_dtype, const uint8_t* w, void* y, int y_d
 }
 
 // ------------------------------------------------------------------------------------------------
-// Q4_K / Q5_K, 17 - 48 activation rows (the kernel serves up to 128): the token counts between decode and the large tiles.  At these counts the call is bound by
-// streaming and decoding the weights once, so every super-block is fetched by one wave, decoded once in its registers and
-// multiplied into ALL activation rows; the rows reach the waves through LDS, staged once per workgroup and block.
-//   v_mfma_f32_16x16x32_f16: A = 16 activation rows x the 32 columns of a scale group (fp16 rows scaled per row by a power of two,
-//   as the tile kernel stages them: bf16 / fp16 inputs stay exact), B = 32 weights x 16 weight rows.
+// Q4_K / Q5_K, 17 - 64 activation rows (the kernel serves up to 128): the token counts between decode and the large tiles.  At these
+// counts the call is bound by streaming and decoding the weights once, so every super-block is fetched by one wave, decoded once in
+// its registers and multiplied into ALL activation rows; the rows reach the waves through LDS, staged once per workgroup and block.
+//   v_mfma_f32_16x16x32_f16: A = 16 activation rows x the 32 columns of a scale group as fp16 values, B = 32 weights x 16 weight rows.
 // B carries sc_g * code as an exact fp16 integer (at most 63 * 31 = 1953 < 2048): the code enters as 1024 + code (bits
 // 0x6400 | code, one byte permute per two codes) and one packed fused multiply-add, (1024 + code) * sc - 1024 * sc, leaves
 // sc * code with a single rounding, i.e. exactly.  A second B with m_g in every position accumulates m_g times the group's
@@ -1122,7 +1122,7 @@ int launch_rows16(const void* x, int x_dtype, const uint8_t* w, void* y, int y_d
 // and no per-group float arithmetic at all.  Workgroup = eight waves = eight tiles of 16 weight rows on one range of blocks; RG
 // groups of 16 activation rows.  LDS per block: [RG][8 groups][64 lanes][16 B] in operand order (a wave's read is one contiguous
 // kilobyte), two blocks at a time.  The matrix is cut along K into `slices` until two workgroups per compute unit exist; the
-// partial sums [slice][row][n] are added in slice order by k45_rows64_reduce_kernel (deterministic).
+// partial sums leave in the order the lanes hold them and are added in slice order by k45_rows64_reduce_kernel (deterministic).
 // ------------------------------------------------------------------------------------------------
 constexpr int kR64Waves = 8;
 typedef _Float16 v2hf __attribute__((ext_vector_type(2)));
@@ -1145,11 +1145,64 @@ __device__ __forceinline__ uint4 scaled_code_halves(uint32_t c0, uint32_t c1, ui
     return make_uint4(r[0], r[1], r[2], r[3]);
 }
 
-template <typename FMT, int RG>
-__global__ __launch_bounds__(64 * kR64Waves) void k45_rows64_kernel(
-    const _Float16* __restrict__ xh, const float* __restrict__ xscale, const uint8_t* __restrict__ w, void* __restrict__ y, int y_dtype,
-    float* __restrict__ partial, int t_rows, int t_pad, int n, int bpr, int kp, int blocks_per_slice) {
+// A workgroup's partial sums leave in the order the lanes hold them: [slice][row group z][column group][wave][i][lane] float4s
+// (rows 4 q .. 4 q + 3 of row group i against one weight row), one contiguous kilobyte per wave and store.
+template <int RG>
+__device__ __forceinline__ void rows64_store_partial(float* __restrict__ partial, const v4f (&acc)[RG], int wave, int lane) {
+    const size_t wg = (static_cast<size_t>(blockIdx.y) * gridDim.z + blockIdx.z) * gridDim.x + blockIdx.x;
+    v4f* dst = reinterpret_cast<v4f*>(partial) + (wg * kR64Waves + wave) * (RG * 64) + lane;
+#pragma unroll
+    for (int i = 0; i < RG; ++i) dst[i * 64] = acc[i];
+}
+
+// y[t, c] = xscale[t] * sum over the slices, in slice order, of the partial sums; thread = one float4 of the lane-order layout
+// (four rows of one column), per_slice = float4s per slice
+template <int RG>
+__global__ __launch_bounds__(256) void k45_rows64_reduce_kernel(const float* __restrict__ partial, const float* __restrict__ xscale, void* __restrict__ y,
+                                                                int y_dtype, int t_rows, int n, int cols, int per_slice, int slices) {
+    const int idx = static_cast<int>(blockIdx.x) * 256 + static_cast<int>(threadIdx.x);
+    if (idx >= per_slice) return;
+    const int lane = idx & 63, i = (idx >> 6) % RG, wave = (idx / (64 * RG)) % kR64Waves;
+    const int wg = idx / (64 * RG * kR64Waves), cg = wg % cols, z = wg / cols;
+    const int c = (cg * kR64Waves + wave) * 16 + (lane & 15), t = (z * RG + i) * 16 + 4 * (lane >> 4);
+    if (c >= n || t >= t_rows) return;
+    const v4f* src = reinterpret_cast<const v4f*>(partial) + idx;
+    // eight slices requested at a time, added in slice order
+    v4f s = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    int k = 0;
+    for (; k + 8 <= slices; k += 8) {
+        v4f part[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) part[j] = src[static_cast<size_t>(k + j) * per_slice];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s += part[j];
+    }
+    {
+        v4f part[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) part[j] = src[static_cast<size_t>(min(k + j, slices - 1)) * per_slice];
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            if (k + j < slices) s += part[j];
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+        if (t + r < t_rows) store_plain(y, y_dtype, static_cast<size_t>(t + r) * n + c, xscale ? s[r] * xscale[t + r] : s[r]);
+}
+
+// The rows are 16-bit values, 256 bpr to a row, 16-byte aligned: fp16 rows (the caller's own, or rows staged by a launch before
+// this one under one power of two per row, xscale, which the stores multiply back in) go into the operand-order LDS buffers
+// unchanged.  bf16 rows (BF16, the caller's own: no staging launch) become fp16 on the way: every trip (two blocks) scales each of
+// its rows by the power of two that brings the row's largest magnitude IN THAT TRIP to [2^14, 2^15) (the waves meet in an LDS
+// maximum per row), so the conversion is exact for every value within 2^-28 of that maximum, and the trip's sums are scaled back
+// per row before they join the accumulators.  Four waves per SIMD (two workgroups per compute unit) are what hides a trip's round
+// trip to memory, hence the register bound; the few values it pushes to scratch are loop-invariant addresses.
+template <typename FMT, int RG, bool BF16>
+__global__ __launch_bounds__(64 * kR64Waves, 4) void k45_rows64_kernel(
+    const uint16_t* __restrict__ x, const float* __restrict__ xscale, const uint8_t* __restrict__ w, void* __restrict__ y, int y_dtype,
+    float* __restrict__ partial, int t_rows, int n, int bpr, int blocks_per_slice) {
     __shared__ __align__(16) unsigned char abuf[2][RG * 8 * 1024];
+    __shared__ __align__(16) uint32_t rmax[2][16 * RG];                      // float32 bits of a trip's row maxima (sign dropped); trips alternate
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
     const int col = lane & 15, q = lane >> 4;
@@ -1157,16 +1210,20 @@ __global__ __launch_bounds__(64 * kR64Waves) void k45_rows64_kernel(
     const uint8_t* wp = w + static_cast<size_t>(wrow) * bpr * FMT::kBlockBytes;
     const int b_begin = static_cast<int>(blockIdx.y) * blocks_per_slice, b_end = min(bpr, b_begin + blocks_per_slice);
     const int t0 = static_cast<int>(blockIdx.z) * 16 * RG;
-    // staging: wave v moves the pieces (rg, g) = (i, v) of a block, i < RG; lane (col, q) brings 8 values of activation row 16 rg + col
-    const _Float16* ap[RG];
+    // wave v brings the pieces (rg, g) = (i, v) of a block, i < RG; lane (col, q): 8 values of activation row 16 rg + col
+    uint32_t ao[RG];                                                         // (element offsets: at most 128 rows of bpr blocks)
 #pragma unroll
-    for (int i = 0; i < RG; ++i) ap[i] = xh + static_cast<size_t>(min(t0 + 16 * i + col, t_rows - 1)) * kp + 32 * wave + 8 * q;
+    for (int i = 0; i < RG; ++i) ao[i] = static_cast<uint32_t>(min(t0 + 16 * i + col, t_rows - 1)) * (256u * bpr) + 32u * wave + 8u * q;
+    if constexpr (BF16) {
+        if (tid < 2 * 16 * RG) (&rmax[0][0])[tid] = 0u;
+        __syncthreads();
+    }
 
     v4f acc[RG];
 #pragma unroll
     for (int i = 0; i < RG; ++i) acc[i] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
 
-    auto multiply = [&](const typename FMT::Regs& r, int buf) {
+    auto multiply = [&](const typename FMT::Regs& r, int buf, int trip) {
         const K4Scales sc = k4_unpack(r.hdr);
         v4f c1[RG], c2[RG];
 #pragma unroll
@@ -1188,12 +1245,27 @@ __global__ __launch_bounds__(64 * kR64Waves) void k45_rows64_kernel(
         }
         const float dd = f16_bits_to_float(r.hdr.x & 0xffffu), dmin = f16_bits_to_float(r.hdr.x >> 16);
 #pragma unroll
-        for (int i = 0; i < RG; ++i) acc[i] += c1[i] * dd - c2[i] * dmin;
+        for (int i = 0; i < RG; ++i) {
+            if constexpr (BF16) {
+                // the sums of rows 4 q .. 4 q + 3 go back by 2^(E - 141), E as at the conversion
+                const uint4 mr = *reinterpret_cast<const uint4*>(&rmax[trip][16 * i + 4 * q]);
+                const v4f back = v4f{__uint_as_float((max(mr.x >> 23, 15u) - 14u) << 23), __uint_as_float((max(mr.y >> 23, 15u) - 14u) << 23),
+                                     __uint_as_float((max(mr.z >> 23, 15u) - 14u) << 23), __uint_as_float((max(mr.w >> 23, 15u) - 14u) << 23)};
+                acc[i] += (c1[i] * dd - c2[i] * dmin) * back;
+            } else {
+                acc[i] += c1[i] * dd - c2[i] * dmin;
+            }
+        }
     };
-    // Two blocks per trip: everything the trip needs is requested at once (weights of both blocks into registers, activation pieces
-    // of both through registers into the two LDS buffers), one memory round trip, then both blocks are multiplied.  A workgroup's
-    // own trips do not overlap; the two workgroups of a compute unit do, one fetching while the other multiplies.
-    for (int b = b_begin; b < b_end; b += 2) {
+    // two bf16 values in a dword -> two fp16 values, both times `mult`
+    auto halves = [](uint32_t pair, float mult) -> uint32_t {
+        union { __fp16 __attribute__((ext_vector_type(2))) h; uint32_t u; } o;
+        o.h = __builtin_amdgcn_cvt_pkrtz(__uint_as_float(pair << 16) * mult, __uint_as_float(pair & 0xffff0000u) * mult);
+        return o.u;
+    };
+    // Two blocks per trip, everything a trip needs requested at once; the two workgroups of a compute unit overlap their trips.
+    int trip = 0;
+    for (int b = b_begin; b < b_end; b += 2, trip ^= 1) {
         const int b1 = min(b + 1, b_end - 1);                                // (past the last block: that one again, not used)
         typename FMT::Regs r0, r1;
         u32x4 a0[RG], a1[RG];
@@ -1201,21 +1273,55 @@ __global__ __launch_bounds__(64 * kR64Waves) void k45_rows64_kernel(
         FMT::load(r1, wp + static_cast<size_t>(b1) * FMT::kBlockBytes, q);
 #pragma unroll
         for (int i = 0; i < RG; ++i) {
-            a0[i] = *reinterpret_cast<const u32x4*>(ap[i] + 256 * b);
-            a1[i] = *reinterpret_cast<const u32x4*>(ap[i] + 256 * b1);
+            a0[i] = *reinterpret_cast<const u32x4*>(x + (ao[i] + 256u * b));
+            a1[i] = *reinterpret_cast<const u32x4*>(x + (ao[i] + 256u * b1));
         }
-        if (b > b_begin) __syncthreads();                                    // everybody has left the buffers of the trip before
+        if constexpr (BF16) {
 #pragma unroll
-        for (int i = 0; i < RG; ++i) {
-            *reinterpret_cast<u32x4*>(&abuf[0][(i * 8 + wave) * 1024 + lane * 16]) = a0[i];
-            *reinterpret_cast<u32x4*>(&abuf[1][(i * 8 + wave) * 1024 + lane * 16]) = a1[i];
+            for (int i = 0; i < RG; ++i) {
+                // the larger of two packed magnitudes per half, then of the halves; as float32 bits the comparison is the values'
+                uint32_t m = 0u;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t u0 = a0[i][j] & 0x7fff7fffu, u1 = a1[i][j] & 0x7fff7fffu;
+                    m = max(m, max(max(u0 << 16, u0 & 0xffff0000u), max(u1 << 16, u1 & 0xffff0000u)));
+                }
+                atomicMax(&rmax[trip][16 * i + col], m);
+            }
+            __syncthreads();                                                 // the maxima are whole; everybody has left the buffers of the trip before
+            if (tid < 16 * RG) rmax[trip ^ 1][tid] = 0u;                     // (last read before this barrier, next written after the one below)
+#pragma unroll
+            for (int i = 0; i < RG; ++i) {
+                // exponent field E of the row maximum (at least 15, so that this power of two and the one the sums go back by are
+                // ordinary numbers): the row is multiplied by 2^(141 - E)
+                const uint32_t e = max(rmax[trip][16 * i + col] >> 23, 15u);
+                const float mult = __uint_as_float((268u - e) << 23);
+                u32x4 h0, h1;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    h0[j] = halves(a0[i][j], mult);
+                    h1[j] = halves(a1[i][j], mult);
+                }
+                *reinterpret_cast<u32x4*>(&abuf[0][(i * 8 + wave) * 1024 + lane * 16]) = h0;
+                *reinterpret_cast<u32x4*>(&abuf[1][(i * 8 + wave) * 1024 + lane * 16]) = h1;
+            }
+        } else {
+            if (b > b_begin) __syncthreads();                                // everybody has left the buffers of the trip before
+#pragma unroll
+            for (int i = 0; i < RG; ++i) {
+                *reinterpret_cast<u32x4*>(&abuf[0][(i * 8 + wave) * 1024 + lane * 16]) = a0[i];
+                *reinterpret_cast<u32x4*>(&abuf[1][(i * 8 + wave) * 1024 + lane * 16]) = a1[i];
+            }
         }
         __syncthreads();
-        multiply(r0, 0);
-        if (b + 1 < b_end) multiply(r1, 1);
+        multiply(r0, 0, trip);
+        if (b + 1 < b_end) multiply(r1, 1, trip);
     }
 
-    // lane (col, q) holds rows 4 q .. 4 q + 3 of every row group against weight row `col` of the wave's tile
+    if (partial) {
+        rows64_store_partial<RG>(partial, acc, wave, lane);
+        return;
+    }
     const int out_col = (static_cast<int>(blockIdx.x) * kR64Waves + wave) * 16 + col;
     if (out_col >= n) return;
 #pragma unroll
@@ -1223,39 +1329,8 @@ __global__ __launch_bounds__(64 * kR64Waves) void k45_rows64_kernel(
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int row = t0 + 16 * i + 4 * q + r;
-            if (row >= t_rows) continue;
-            if (partial) partial[(static_cast<size_t>(blockIdx.y) * t_pad + row) * n + out_col] = acc[i][r];
-            else store_plain(y, y_dtype, static_cast<size_t>(row) * n + out_col, acc[i][r] * xscale[row]);
+            if (row < t_rows) store_plain(y, y_dtype, static_cast<size_t>(row) * n + out_col, xscale ? acc[i][r] * xscale[row] : acc[i][r]);
         }
-}
-
-// y[t, c] = xscale[t] * sum over the slices, in slice order, of partial[slice][t][c]; four columns per thread
-__global__ __launch_bounds__(256) void k45_rows64_reduce_kernel(const float* __restrict__ partial, const float* __restrict__ xscale, void* __restrict__ y,
-                                                                int y_dtype, int t_rows, int t_pad, int n, int slices) {
-    const int c = (static_cast<int>(blockIdx.x) * 256 + static_cast<int>(threadIdx.x)) * 4, t = blockIdx.y;
-    if (c >= n) return;
-    float4 s = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-    const float* src = partial + static_cast<size_t>(t) * n + c;
-    if (c + 3 < n && (n & 3) == 0) {
-        for (int k = 0; k < slices; ++k) {
-            const float4 v = *reinterpret_cast<const float4*>(src + static_cast<size_t>(k) * t_pad * n);
-            s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
-        }
-    } else {
-        for (int k = 0; k < slices; ++k) {
-            const float* v = src + static_cast<size_t>(k) * t_pad * n;
-            s.x += v[0];
-            if (c + 1 < n) s.y += v[1];
-            if (c + 2 < n) s.z += v[2];
-            if (c + 3 < n) s.w += v[3];
-        }
-    }
-    const float sc = xscale[t];
-    const size_t o = static_cast<size_t>(t) * n + c;
-    store_plain(y, y_dtype, o, s.x * sc);
-    if (c + 1 < n) store_plain(y, y_dtype, o + 1, s.y * sc);
-    if (c + 2 < n) store_plain(y, y_dtype, o + 2, s.z * sc);
-    if (c + 3 < n) store_plain(y, y_dtype, o + 3, s.w * sc);
 }
 
 // column groups of 128 weight rows, cut along K until about two workgroups per compute unit exist
@@ -1273,16 +1348,18 @@ Rows64Plan plan_rows64(int rows, int n, int bpr) {
     return p;
 }
 
-template <typename FMT>
-int launch_rows64(const Rows64Plan& p, const _Float16* xh, const float* xscale, const uint8_t* w, void* y, int y_dtype, float* partial,
-                  int rows, int n, int bpr, hipStream_t stream) {
+template <typename FMT, bool BF16>
+int launch_rows64(const Rows64Plan& p, const uint16_t* x, const float* xscale, const uint8_t* w, void* y, int y_dtype, float* partial,
+                      int rows, int n, int bpr, hipStream_t stream) {
     const dim3 grid(p.cols, p.slices, p.zs);
     float* part = p.slices > 1 ? partial : nullptr;
-    if (p.rg == 2) hipLaunchKernelGGL((k45_rows64_kernel<FMT, 2>), grid, dim3(64 * kR64Waves), 0, stream, xh, xscale, w, y, y_dtype, part, rows, p.t_pad, n, bpr, bpr * 256, p.bps);
-    else hipLaunchKernelGGL((k45_rows64_kernel<FMT, 4>), grid, dim3(64 * kR64Waves), 0, stream, xh, xscale, w, y, y_dtype, part, rows, p.t_pad, n, bpr, bpr * 256, p.bps);
+    if (p.rg == 2) hipLaunchKernelGGL((k45_rows64_kernel<FMT, 2, BF16>), grid, dim3(64 * kR64Waves), 0, stream, x, xscale, w, y, y_dtype, part, rows, n, bpr, p.bps);
+    else hipLaunchKernelGGL((k45_rows64_kernel<FMT, 4, BF16>), grid, dim3(64 * kR64Waves), 0, stream, x, xscale, w, y, y_dtype, part, rows, n, bpr, p.bps);
     if (hipGetLastError() != hipSuccess) return PLLM_ERR_LAUNCH;
     if (p.slices > 1) {
-        hipLaunchKernelGGL(k45_rows64_reduce_kernel, dim3((n + 1023) / 1024, rows), dim3(256), 0, stream, partial, xscale, y, y_dtype, rows, p.t_pad, n, p.slices);
+        const int per_slice = p.zs * p.cols * kR64Waves * p.rg * 64;
+        if (p.rg == 2) hipLaunchKernelGGL(k45_rows64_reduce_kernel<2>, dim3((per_slice + 255) / 256), dim3(256), 0, stream, partial, xscale, y, y_dtype, rows, n, p.cols, per_slice, p.slices);
+        else hipLaunchKernelGGL(k45_rows64_reduce_kernel<4>, dim3((per_slice + 255) / 256), dim3(256), 0, stream, partial, xscale, y, y_dtype, rows, n, p.cols, per_slice, p.slices);
         if (hipGetLastError() != hipSuccess) return PLLM_ERR_LAUNCH;
     }
     return PLLM_OK;
@@ -1336,31 +1413,50 @@ int k45_rows16_matvec(const void* x, int x_dtype, const uint8_t* w, int type_id,
 }  // namespace pllm
 
 namespace pllm {
-// Q4_K / Q5_K on 17 - 48 activation rows (any of the three input types; the rows are staged as scaled fp16 rows first)
-bool k45_rows64_supports(int type_id, int rows, int n, int bpr, const uint8_t* w) {
-    // measured against the tile kernel (Q4_K, operator call in us, this kernel / tiles): 5120x5120 19.1 / 26.2 at 17 rows, 21.4 / 26.2
-    // at 32, 27.9 / 27.7 at 64, 31.9 / 32.8 at 128; 17408x5120 31.0 / 40.9, 32.8 / 41.0, 44.6 / 43.0, 91.5 / 60.3: it takes the calls of up
-    // to 48 rows (the kernel itself serves up to 128)
-    return (type_id == PLLM_TYPE_Q4_K || type_id == PLLM_TYPE_Q5_K) && rows > 16 && rows <= 48 && n >= 16 && bpr >= 1 &&
+// Q4_K / Q5_K on 17 - 48 activation rows (float32 rows, and bf16 rows on large matrices, are staged as scaled fp16 rows by a launch
+// of their own first; fp16 rows, and bf16 rows on matrices of up to kRows64SmallWeights weights, are read as the caller holds
+// them).  Operator calls in us, Q4_K, 17 / 32 / 48 / 64 rows:
+//   5120x5120    staged 19.1 / 21.4 / - / 27.9     bf16 as held 16.4 / 18.2 / 24.9 / 25.8     fp16 as held 15.4 / 17.1 / 21.3 / 23.3     tile kernel 26.2 / 26.2 / - / 27.7
+//   17408x5120   staged 31.0 / 32.8 / - / 44.6     bf16 as held 32.1 / 33.3 / 52.0 / 51.6     fp16 as held 27.4 / 29.6 / 40.9 / 43.4     tile kernel 40.9 / 41.0 / - / 43.0
+// (converting bf16 rows inside the kernel repeats the conversion in every column group: 136 of them at 17408 weight rows), so rows
+// read as held are served up to 64 on the small matrices and everything else up to 48; the kernels themselves take up to 128.
+constexpr int64_t kRows64SmallWeights = int64_t{48} << 20;
+bool k45_rows64_reads_raw(const void* x, int x_dtype, int k, int n, int bpr) {
+    if (k != 256 * bpr || (reinterpret_cast<uintptr_t>(x) & 15u) != 0) return false;
+    return x_dtype == PLLM_F16 || (x_dtype == PLLM_BF16 && static_cast<int64_t>(n) * k <= kRows64SmallWeights);
+}
+bool k45_rows64_supports(int type_id, int rows, int n, int bpr, const uint8_t* w, bool raw16) {
+    const int most = raw16 && static_cast<int64_t>(n) * bpr * 256 <= kRows64SmallWeights ? 64 : 48;
+    return (type_id == PLLM_TYPE_Q4_K || type_id == PLLM_TYPE_Q5_K) && rows > 16 && rows <= most && n >= 16 && bpr >= 1 &&
            (reinterpret_cast<uintptr_t>(w) & 15u) == 0;
 }
 size_t k45_rows64_workspace_bytes(int rows, int n, int bpr) {
     const Rows64Plan p = plan_rows64(rows, n, bpr);
-    const size_t part = p.slices > 1 ? align256(static_cast<size_t>(p.slices) * p.t_pad * n * sizeof(float)) : 0;
+    const size_t part = p.slices > 1 ? align256(static_cast<size_t>(p.slices) * p.t_pad * p.cols * (16 * kR64Waves) * sizeof(float)) : 0;
     return gemm_f16_staged_bytes(rows, bpr) + part;
 }
 int k45_rows64_gemm(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y, int y_dtype, int rows, int k, int n, int bpr,
                     void* workspace, size_t workspace_bytes, hipStream_t stream) {
-    if (!k45_rows64_supports(type_id, rows, n, bpr, w) || (y_dtype & kAccumulateInto)) return PLLM_ERR_UNSUPPORTED;
+    const bool raw16 = k45_rows64_reads_raw(x, x_dtype, k, n, bpr);
+    if (!k45_rows64_supports(type_id, rows, n, bpr, w, raw16) || (y_dtype & kAccumulateInto)) return PLLM_ERR_UNSUPPORTED;
     if (!workspace || workspace_bytes < k45_rows64_workspace_bytes(rows, n, bpr)) return PLLM_ERR_WORKSPACE;
-    const int st = gemm_f16_stage_rows(x, x_dtype, nullptr, rows, k, bpr, workspace, stream);
-    if (st != PLLM_OK) return st;
-    const size_t rows_bytes = align256(static_cast<size_t>(rows) * bpr * 256 * sizeof(_Float16));
-    const _Float16* xh = static_cast<const _Float16*>(workspace);
-    const float* xscale = reinterpret_cast<const float*>(static_cast<const unsigned char*>(workspace) + rows_bytes);
-    float* partial = reinterpret_cast<float*>(static_cast<unsigned char*>(workspace) + gemm_f16_staged_bytes(rows, bpr));
     const Rows64Plan p = plan_rows64(rows, n, bpr);
-    return type_id == PLLM_TYPE_Q4_K ? launch_rows64<Rows16Q4K>(p, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, stream)
-                                     : launch_rows64<Rows16Q5K>(p, xh, xscale, w, y, y_dtype, partial, rows, n, bpr, stream);
+    float* partial = reinterpret_cast<float*>(static_cast<unsigned char*>(workspace) + gemm_f16_staged_bytes(rows, bpr));
+    const uint16_t* xr = static_cast<const uint16_t*>(x);
+    const float* xscale = nullptr;
+    bool bf16 = x_dtype == PLLM_BF16;
+    if (!raw16) {
+        // staged as fp16 rows of 256 bpr values, each under one power of two (xscale), which the kernel then reads like fp16 rows
+        const int st = gemm_f16_stage_rows(x, x_dtype, nullptr, rows, k, bpr, workspace, stream);
+        if (st != PLLM_OK) return st;
+        xr = static_cast<const uint16_t*>(workspace);
+        xscale = reinterpret_cast<const float*>(static_cast<const unsigned char*>(workspace) + align256(static_cast<size_t>(rows) * bpr * 256 * sizeof(_Float16)));
+        bf16 = false;
+    }
+    if (type_id == PLLM_TYPE_Q4_K)
+        return bf16 ? launch_rows64<Rows16Q4K, true>(p, xr, xscale, w, y, y_dtype, partial, rows, n, bpr, stream)
+                    : launch_rows64<Rows16Q4K, false>(p, xr, xscale, w, y, y_dtype, partial, rows, n, bpr, stream);
+    return bf16 ? launch_rows64<Rows16Q5K, true>(p, xr, xscale, w, y, y_dtype, partial, rows, n, bpr, stream)
+                : launch_rows64<Rows16Q5K, false>(p, xr, xscale, w, y, y_dtype, partial, rows, n, bpr, stream);
 }
 }  // namespace pllm

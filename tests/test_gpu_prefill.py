@@ -70,6 +70,50 @@ def test_prefill_17_to_48_rows_matches_float_oracle(mod, type_name, t, n, k):
         assert y16.dtype == torch.bfloat16 and torch.equal(y16, y.to(torch.bfloat16))
 
 
+@pytest.mark.parametrize("type_name", ["q4_k", "q5_k"])
+@pytest.mark.parametrize("t", [20, 40, 64])
+def test_prefill_17_to_64_rows_read_as_held_rescale_every_trip(mod, type_name, t):
+    """bf16 / fp16 rows whose length is a whole number of super-blocks are read as the caller holds them (no staging launch); bf16
+    values become fp16 inside the kernel under a power of two chosen per row and per trip of two blocks.  Magnitudes that change
+    along a row by 40 orders, rows and trips of zeros and rows near the ends of the bf16 range must all come out as the float
+    statement has them: the conversion is exact, so only float32 summation order is left."""
+    n, k = 4352, 5120                    # 34 column groups, 7 slices of 3 blocks: two trips per workgroup, the second of one block
+    rng = np.random.default_rng(100 + t)
+    blocks = ENC[type_name]((rng.standard_normal((n, k)) * 0.02).astype(np.float32))
+    x_np = rng.standard_normal((t, k)).astype(np.float32)
+    x_np[3] *= 1e4
+    x_np[5] *= 1e-6
+    x_np[7, :512] *= 1e20                # the first trip of the first slice dwarfs everything else in the row ...
+    x_np[7, 512:1024] *= 1e-20           # ... and its second trip and the next slice's first are tiny
+    x_np[8] = 0.0
+    x_np[9, 512:768] = 0.0               # a trip of zeros between ordinary ones
+    x_np[10] *= 1e30
+    x_np[11] *= 1e-30
+    x_np[12, ::2] *= 1e-5                # neighbours five orders apart inside every group
+    ref_w = O.dequant_rows(blocks, type_name, k)
+    grid = torch.empty(0, dtype=torch.int8, device=DEV)
+    w = torch.from_numpy(blocks).to(DEV)
+    for dt in (torch.bfloat16, torch.float16):
+        x = torch.from_numpy(np.clip(x_np, -6e4, 6e4) if dt == torch.float16 else x_np).to(DEV).to(dt)
+        print(f"case prefill rows as held {type_name} t={t} {dt}", flush=True)
+        y = mod.gguf_quant_gemm_prefill_forward(x, w, k, O.TYPE_IDS[type_name], grid, out_dtype=torch.float32)
+        torch.cuda.synchronize()
+        xs = x.float().cpu().numpy().astype(np.float64)
+        want = xs @ ref_w.astype(np.float64).T
+        got = y.cpu().numpy().astype(np.float64)
+        assert np.isfinite(got).all()
+        assert (got[8] == 0.0).all()
+        # per slice of a row the error is relative to that slice's own products (each trip is scaled by itself)
+        bound = (np.abs(xs) @ np.abs(ref_w.astype(np.float64)).T) * 2e-6 + 1e-44
+        assert (np.abs(got - want) <= bound).all(), (dt, np.unravel_index(np.argmax(np.abs(got - want) / bound), got.shape))
+        # a view that is not 16-byte aligned goes through the staging launch: same bits (both conversions are exact)
+        if dt == torch.bfloat16 and t <= 48:
+            pad = torch.zeros(t * k + 1, dtype=dt, device=DEV)
+            pad[1:] = x.reshape(-1)
+            y2 = mod.gguf_quant_gemm_prefill_forward(pad[1:].view(t, k), w, k, O.TYPE_IDS[type_name], grid, out_dtype=torch.float32)
+            assert torch.equal(y2, y)
+
+
 def test_prefill_3d_input_and_bf16_output(mod):
     rng = np.random.default_rng(0)
     blocks = torch.from_numpy(C.quantize_q4_k((rng.standard_normal((192, 512)) * 0.02).astype(np.float32))).to(DEV)
