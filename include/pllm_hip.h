@@ -403,6 +403,19 @@ int pllm_moe_route(const void* x, int x_dtype, int64_t tokens, int64_t dim, cons
                    int64_t n_experts, int64_t top_k, int softmax_mode, float* logits, int64_t* indices, float* weights, void* stream);
 
 /*
+ * pllm_moe_route on rows that are RMS-normalized first, as a decoder block does ahead of its experts
+ * (src/models/minimax_m2/architecture.py:405-412: ffn_norm, then MiniMaxMoE.forward's gate): the normalisation
+ *     x_normed[t, :] = x[t, :] * rsqrt(mean(x[t, :]^2) + eps) * norm_weight      (float32 arithmetic, one rounding to x_normed_dtype)
+ * runs inside the logits launch, the logits are formed on the rounded values, and x_normed [tokens, dim] is written out for the
+ * expert operators that follow: pllm_fused_rms_norm + pllm_moe_route in two launches instead of three.
+ * For up to 4 rows of at most 3072 values (dim % 4 == 0; x, x_normed, norm_weight and gate_weight 16-byte aligned); PLLM_ERR_UNSUPPORTED
+ * otherwise (call the two operators).
+ */
+int pllm_moe_route_rmsnorm(const void* x, int x_dtype, const float* norm_weight, float eps, void* x_normed, int x_normed_dtype,
+                           int64_t tokens, int64_t dim, const float* gate_weight, const float* gate_bias, int64_t n_experts, int64_t top_k,
+                           int softmax_mode, float* logits, int64_t* indices, float* weights, void* stream);
+
+/*
  * FP8 activation quantizer: per (row, 128 values) scale = max(amax, eps) / 448 (rounded up to a power
  * of two when round_scale_pow2 != 0), code = E4M3FN round-to-nearest-even of clamp(x / scale, +-448).
  *   x [rows, k] (k a multiple of 128) -> codes uint8 [rows, k], scales float32 [rows, k / 128]

@@ -68,6 +68,8 @@ SIGNATURES = {
                                             _i64, _i64, _i64, _i64, _c_void_p, _size_t, _c_void_p]),
     "pllm_gguf_quant_gemm_rmsnorm_workspace_bytes": (_size_t, [_int, _i64, _i64, _i64, _i64]),
     "pllm_moe_route": (_int, [_c_void_p, _int, _i64, _i64, _c_void_p, _c_void_p, _i64, _i64, _int, _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
+    "pllm_moe_route_rmsnorm": (_int, [_c_void_p, _int, _c_void_p, ctypes.c_float, _c_void_p, _int, _i64, _i64, _c_void_p, _c_void_p, _i64, _i64, _int,
+                                      _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
     "pllm_fp8_act_quant": (_int, [_c_void_p, _int, _i64, _i64, _c_void_p, _c_void_p, ctypes.c_float, _int, _c_void_p]),
 }
 

@@ -91,14 +91,16 @@ __global__ __launch_bounds__(kThreads) void rms_norm_rows_kernel(
         int e0[kRmsHeld];                                                   // beyond the row: its first piece again, not counted
 #pragma unroll
         for (int j = 0; j < kRmsHeld; ++j) e0[j] = 4 * (static_cast<int>(threadIdx.x) + kThreads * j) < dim ? 4 * (static_cast<int>(threadIdx.x) + kThreads * j) : 0;
+        // (the weights are requested first: the row's loads sit behind a branch on its type, and what is requested after that
+        // branch, or after the barrier, costs a round trip of its own)
+#pragma unroll
+        for (int j = 0; j < kRmsHeld; ++j) load_row4(g[j], weight, PLLM_F32, 0, e0[j], dim, wvec);
         if (vec) {
             load_rows4_batch(v, x, x_dtype, off, e0);
         } else {
 #pragma unroll
             for (int j = 0; j < kRmsHeld; ++j) load_row4(v[j], x, x_dtype, off, e0[j], dim, false);
         }
-#pragma unroll
-        for (int j = 0; j < kRmsHeld; ++j) load_row4(g[j], weight, PLLM_F32, 0, e0[j], dim, wvec);   // (requested now: after the barrier they would cost a round trip of their own)
 #pragma unroll
         for (int j = 0; j < kRmsHeld; ++j)
             if (4 * (threadIdx.x + kThreads * j) < dim) ss += (v[j][0] * v[j][0] + v[j][1] * v[j][1]) + (v[j][2] * v[j][2] + v[j][3] * v[j][3]);

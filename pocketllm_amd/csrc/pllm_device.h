@@ -363,8 +363,10 @@ __device__ __forceinline__ void quantize_row_to_lds(unsigned char* lds, const vo
         // sum of squares of the row: per-wave sums meet in the first floats of the image area, which nobody has written yet
         float ss = 0.0f;
         if (one_batch) {
+            // (the weights first: the row's loads sit behind a branch on its type, and what is requested after that branch, or
+            // after the barriers, costs a round trip of its own)
+            load_row_pieces<BATCH>(g, norm.gamma, PLLM_F32, 0, first, trip, k, kpad, gvec);
             load_row_pieces<BATCH>(v, x, x_dtype, xoff, first, trip, k, kpad, vec);
-            load_row_pieces<BATCH>(g, norm.gamma, PLLM_F32, 0, first, trip, k, kpad, gvec);   // (now: after the barriers they would cost a round trip of their own)
 #pragma unroll
             for (int j = 0; j < BATCH; ++j)
                 if (first + j * trip < kpad) ss += (v[j][0] * v[j][0] + v[j][1] * v[j][1]) + (v[j][2] * v[j][2] + v[j][3] * v[j][3]);

@@ -93,6 +93,79 @@ __global__ __launch_bounds__(kThreads) void route_logits_kernel(
     }
 }
 
+// Decode rows that are RMS-normalized first (the block's normalisation ahead of its experts): one wave per (expert, token).
+// Every wave holds the whole row, so every wave forms the row's sum of squares itself; v = x * rsqrt(mean(x^2) + eps) * weight is
+// rounded to xn_dtype (what a normalisation launch of its own would have stored) and the logit is formed on the rounded values.
+// The wave of expert 0 also writes the normalized row out for the operators that follow.  dim <= 256 * kHeld, dim % 4 == 0,
+// 16-byte aligned rows.
+template <int XN>
+__device__ __forceinline__ float round_to(float v) {
+    if constexpr (XN == PLLM_F16) return static_cast<float>(static_cast<_Float16>(v));
+    if constexpr (XN == PLLM_BF16) return to_float(from_float<bf16_t>(v));
+    return v;
+}
+template <int XN>
+__global__ __launch_bounds__(kThreads) void route_logits_norm_kernel(
+    const void* __restrict__ x, int x_dtype, const float* __restrict__ norm_weight, float eps, void* __restrict__ xn,
+    const float* __restrict__ gate, float* __restrict__ logits, int dim, int n_experts) {
+    const int lane = threadIdx.x & 63;
+    const int e = blockIdx.x * kWavesPerWg + (threadIdx.x >> 6);
+    if (e >= n_experts) return;                                             // whole waves leave together
+    const int t = blockIdx.y;
+    const float* grow = gate + static_cast<size_t>(e) * dim;
+    int cpos[kHeld];
+#pragma unroll
+    for (int i = 0; i < kHeld; ++i) cpos[i] = min(lane * 4 + 256 * i, dim - 4);   // beyond the row: its last piece again, not counted
+    // gate row and norm weights first: the row's loads sit behind a branch on its type, and what is requested after that branch
+    // would wait for a round trip of its own
+    float4 held[kHeld], g[kHeld];
+#pragma unroll
+    for (int i = 0; i < kHeld; ++i) {
+        held[i] = *reinterpret_cast<const float4*>(grow + cpos[i]);
+        g[i] = *reinterpret_cast<const float4*>(norm_weight + cpos[i]);
+    }
+    float v[kHeld][4];
+    load_rows4_batch(v, x, x_dtype, static_cast<size_t>(t) * dim, cpos);
+    float ss = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kHeld; ++i)
+        if (lane * 4 + 256 * i < dim) ss += (v[i][0] * v[i][0] + v[i][1] * v[i][1]) + (v[i][2] * v[i][2] + v[i][3] * v[i][3]);
+    const float rstd = rsqrtf(group_sum<64>(ss) / static_cast<float>(dim) + eps);
+    float acc = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kHeld; ++i) {
+        v[i][0] = round_to<XN>(v[i][0] * rstd * g[i].x);
+        v[i][1] = round_to<XN>(v[i][1] * rstd * g[i].y);
+        v[i][2] = round_to<XN>(v[i][2] * rstd * g[i].z);
+        v[i][3] = round_to<XN>(v[i][3] * rstd * g[i].w);
+        const float d = held[i].x * v[i][0] + held[i].y * v[i][1] + held[i].z * v[i][2] + held[i].w * v[i][3];
+        acc += (lane * 4 + 256 * i < dim) ? d : 0.0f;
+    }
+    // the normalized row leaves piece by piece: the wave of expert i (of expert 0 where there are fewer experts than pieces)
+    // stores piece i, one 8- or 16-byte store per lane
+#pragma unroll
+    for (int i = 0; i < kHeld; ++i) {
+        if (e == (n_experts >= kHeld ? i : 0) && lane * 4 + 256 * i < dim) {
+            const size_t o = static_cast<size_t>(t) * dim + lane * 4 + 256 * i;
+            if constexpr (XN == PLLM_F32) {
+                *reinterpret_cast<float4*>(static_cast<float*>(xn) + o) = make_float4(v[i][0], v[i][1], v[i][2], v[i][3]);
+            } else if constexpr (XN == PLLM_F16) {
+                union { _Float16 h[4]; uint2 u; } pk;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) pk.h[c] = static_cast<_Float16>(v[i][c]);
+                *reinterpret_cast<uint2*>(static_cast<uint16_t*>(xn) + o) = pk.u;
+            } else {
+                // (already bf16 values: the high halves are exact)
+                const uint2 pk = make_uint2((__float_as_uint(v[i][0]) >> 16) | (__float_as_uint(v[i][1]) & 0xffff0000u),
+                                            (__float_as_uint(v[i][2]) >> 16) | (__float_as_uint(v[i][3]) & 0xffff0000u));
+                *reinterpret_cast<uint2*>(static_cast<uint16_t*>(xn) + o) = pk;
+            }
+        }
+    }
+    acc = group_sum<64>(acc);
+    if (lane == 0) logits[static_cast<size_t>(t) * n_experts + e] = acc;
+}
+
 // Many tokens: a workgroup forms the 16 x 16 block logits[t0 .. t0 + 15, e0 .. e0 + 15] on the float32 matrix cores
 // (v_mfma_f32_16x16x4_f32, C[m][n] = sum_k A[m][k] B[k][n] with m = token, n = expert).  Lane (r, q) = (lane % 16, lane / 16)
 // loads four consecutive values of token row r and of gate row r at column k0 + 4 q; value i of both goes to MFMA i of the step,
@@ -250,6 +323,37 @@ int pllm_moe_route(const void* x, int x_dtype, int64_t tokens, int64_t dim, cons
     else
         hipLaunchKernelGGL(route_logits_kernel<kTokensPerWave>, wgs, dim3(kThreads), 0, s, x, x_dtype, gate_weight, logits, static_cast<int>(dim),
                            static_cast<int>(n_experts), static_cast<int>(tokens));
+    if (n_experts <= 256)
+        hipLaunchKernelGGL(route_topk_kernel<4>, dim3(static_cast<unsigned>(tokens)), dim3(64), 0, s, logits, gate_bias, static_cast<int>(n_experts),
+                           static_cast<int>(top_k), softmax_mode, indices, weights);
+    else
+        hipLaunchKernelGGL(route_topk_kernel<kMaxPerLane>, dim3(static_cast<unsigned>(tokens)), dim3(64), 0, s, logits, gate_bias,
+                           static_cast<int>(n_experts), static_cast<int>(top_k), softmax_mode, indices, weights);
+    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+}
+
+int pllm_moe_route_rmsnorm(const void* x, int x_dtype, const float* norm_weight, float eps, void* x_normed, int x_normed_dtype,
+                           int64_t tokens, int64_t dim, const float* gate_weight, const float* gate_bias, int64_t n_experts, int64_t top_k,
+                           int softmax_mode, float* logits, int64_t* indices, float* weights, void* stream) {
+    using namespace pllm;
+    if (!x || !norm_weight || !x_normed || !gate_weight || !logits || !indices || !weights) return PLLM_ERR_INVALID_ARGUMENT;
+    if (x_dtype != PLLM_F32 && x_dtype != PLLM_F16 && x_dtype != PLLM_BF16) return PLLM_ERR_INVALID_ARGUMENT;
+    if (x_normed_dtype != PLLM_F32 && x_normed_dtype != PLLM_F16 && x_normed_dtype != PLLM_BF16) return PLLM_ERR_INVALID_ARGUMENT;
+    if (tokens <= 0 || dim <= 0 || n_experts <= 0 || top_k <= 0 || top_k > n_experts) return PLLM_ERR_INVALID_ARGUMENT;
+    if (n_experts > 64 * kMaxPerLane || top_k > 64) return PLLM_ERR_UNSUPPORTED;
+    // decode rows that a wave can hold whole, everything on vector boundaries; other calls: normalisation and routing as two operators
+    const uintptr_t align = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(norm_weight) | reinterpret_cast<uintptr_t>(gate_weight) |
+                            reinterpret_cast<uintptr_t>(x_normed);
+    if (tokens > 4 || dim > 256 * kHeld || dim < 4 || dim % 4 != 0 || (align & 15u) != 0) return PLLM_ERR_UNSUPPORTED;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const dim3 wgs(static_cast<unsigned>((n_experts + kWavesPerWg - 1) / kWavesPerWg), static_cast<unsigned>(tokens));
+    const int d = static_cast<int>(dim), ne = static_cast<int>(n_experts);
+    if (x_normed_dtype == PLLM_F16)
+        hipLaunchKernelGGL(route_logits_norm_kernel<PLLM_F16>, wgs, dim3(kThreads), 0, s, x, x_dtype, norm_weight, eps, x_normed, gate_weight, logits, d, ne);
+    else if (x_normed_dtype == PLLM_BF16)
+        hipLaunchKernelGGL(route_logits_norm_kernel<PLLM_BF16>, wgs, dim3(kThreads), 0, s, x, x_dtype, norm_weight, eps, x_normed, gate_weight, logits, d, ne);
+    else
+        hipLaunchKernelGGL(route_logits_norm_kernel<PLLM_F32>, wgs, dim3(kThreads), 0, s, x, x_dtype, norm_weight, eps, x_normed, gate_weight, logits, d, ne);
     if (n_experts <= 256)
         hipLaunchKernelGGL(route_topk_kernel<4>, dim3(static_cast<unsigned>(tokens)), dim3(64), 0, s, logits, gate_bias, static_cast<int>(n_experts),
                            static_cast<int>(top_k), softmax_mode, indices, weights);

@@ -798,6 +798,42 @@ def moe_route(x_flat: torch.Tensor, gate_weight: torch.Tensor, gate_bias, top_k:
     return indices, weights
 
 
+def moe_route_rmsnorm(x_flat: torch.Tensor, norm_weight: torch.Tensor, eps: float, gate_weight: torch.Tensor, gate_bias, top_k: int, *,
+                      out_dtype: torch.dtype = torch.float16, softmax: bool = False):
+    """RMS normalisation of the decode rows x_flat [T <= 4, dim] and moe_route on the result (the decoder block's ffn_norm and
+    MiniMaxMoE.route, src/models/minimax_m2/architecture.py:291-298, 405-412) in two launches instead of three:
+    (indices, weights, normalized rows in out_dtype), or None where the library has no such launch (the caller then runs the two
+    operators)."""
+    _check(x_flat.dim() == 2 and gate_weight.dim() == 2 and x_flat.size(1) == gate_weight.size(1), "x_flat [T, dim] and gate_weight [E, dim] must agree on dim")
+    _check(x_flat.is_cuda and gate_weight.is_cuda and x_flat.is_contiguous() and gate_weight.is_contiguous(), "x_flat and gate_weight must be contiguous CUDA tensors")
+    _check_x(x_flat)
+    _check(gate_weight.dtype == torch.float32, "gate_weight must be float32")
+    _check(norm_weight.is_cuda and norm_weight.dtype == torch.float32 and norm_weight.is_contiguous() and norm_weight.numel() == x_flat.size(1),
+           "norm_weight must be a contiguous CUDA float32 tensor [dim]")
+    _check(out_dtype in _DTYPE_CODE, "out_dtype must be float32, float16 or bfloat16")
+    if gate_bias is not None:
+        _check(gate_bias.is_cuda and gate_bias.dtype == torch.float32 and gate_bias.is_contiguous() and gate_bias.numel() == gate_weight.size(0),
+               "gate_bias must be a contiguous CUDA float32 tensor [E]")
+    t, e, k = x_flat.size(0), gate_weight.size(0), int(top_k)
+    _check(0 < k <= e, "top_k must be in 1..E")
+    if t == 0 or t > 4:
+        return None
+    dev = x_flat.device
+    indices = torch.empty(t, k, dtype=torch.int64, device=dev)
+    weights = torch.empty(t, k, dtype=torch.float32, device=dev)
+    logits = torch.empty(t, e, dtype=torch.float32, device=dev)
+    normed = torch.empty(t, x_flat.size(1), dtype=out_dtype, device=dev)
+    with _on_device(dev):
+        st = _lib().pllm_moe_route_rmsnorm(x_flat.data_ptr(), _DTYPE_CODE[x_flat.dtype], norm_weight.data_ptr(), float(eps), normed.data_ptr(),
+                                           _DTYPE_CODE[out_dtype], t, x_flat.size(1), gate_weight.data_ptr(),
+                                           gate_bias.data_ptr() if gate_bias is not None else None, e, k, int(bool(softmax)),
+                                           logits.data_ptr(), indices.data_ptr(), weights.data_ptr(), _stream(dev))
+    if st == _ffi.PLLM_ERR_UNSUPPORTED:
+        return None
+    _ffi.check(st, "moe_route_rmsnorm")
+    return indices, weights, normed
+
+
 def gguf_single_token_route_slots(indices, weights, experts_start_idx, n_local_experts):
     """Host-side compaction of one token's routes (src/csrc/cuda_kernel.cpp:1244-1327):
     [local_ids (CPU int64), route_tokens, route_weights, route_slots, compact_starts (int32)]."""

@@ -97,11 +97,22 @@ class MiniMaxMoE:
         """architecture.py:291-298 as one operator: sigmoid scores, bias for the selection only, top-k, renormalised weights."""
         return self._cuda.moe_route(x_flat, self.gate_weight, self.gate_bias, int(self.args.top_k))
 
-    def __call__(self, x: torch.Tensor, residual: torch.Tensor | None = None) -> torch.Tensor:
+    def __call__(self, x: torch.Tensor, residual: torch.Tensor | None = None, input_norm: RMSNorm | None = None) -> torch.Tensor:
         """The experts' output for x in the model's dtype; with `residual` (x's shape, the model's dtype) it is added into that
-        tensor, which is returned."""
+        tensor, which is returned.  `input_norm`, when given, is the block's normalisation of the residual stream: the experts see
+        input_norm(x), and decode steps run it inside the routing launch."""
         tokens = x.reshape(-1, x.size(-1)).contiguous()
-        chosen, gate_w = self.route(tokens)
+        routed = None
+        if input_norm is not None:
+            if tokens.size(0) <= 4:
+                routed = self._cuda.moe_route_rmsnorm(tokens, input_norm.weight, input_norm.eps, self.gate_weight, self.gate_bias,
+                                                      int(self.args.top_k), out_dtype=input_norm.out_dtype)
+            if routed is None:
+                tokens = input_norm(tokens)
+        if routed is not None:
+            chosen, gate_w, tokens = routed
+        else:
+            chosen, gate_w = self.route(tokens)
         w = self.experts
         nothing = lambda: tokens.new_zeros((tokens.size(0), self.args.dim), dtype=torch.float32)   # no route lands on a resident expert
         if tokens.size(0) == 1:
@@ -221,7 +232,7 @@ class MiniMaxBlock:
                                                           stream)
         else:
             stream += self.attention(self.attn_norm(stream), start_pos)
-        return self.moe(self.ffn_norm(stream), residual=stream)
+        return self.moe(stream, residual=stream, input_norm=self.ffn_norm)
 
 
 class MiniMaxTransformer:

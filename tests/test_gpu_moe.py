@@ -487,6 +487,70 @@ def test_router_matches_the_reference_statement(mod, tokens, dim, n_experts, top
         mod.moe_route(x, gate, None, n_experts + 1)
 
 
+@pytest.mark.parametrize("tokens,dim,n_experts,top_k", [(1, 3072, 256, 8), (4, 3072, 256, 8), (3, 1000, 60, 6), (2, 260, 1024, 64), (1, 64, 8, 8)])
+@pytest.mark.parametrize("x_dtype,out_dtype", [(torch.float16, torch.float16), (torch.bfloat16, torch.bfloat16), (torch.float32, torch.float16),
+                                               (torch.float32, torch.float32)])
+def test_router_on_rows_normalized_in_the_same_launch(mod, tokens, dim, n_experts, top_k, x_dtype, out_dtype):
+    """ffn_norm + MiniMaxMoE.route of a decode step in two launches: the normalized rows against the oracle's float64
+    normalisation (one rounding to the output type), the logits against float64 on the rows the kernel itself wrote, picks and
+    weights against the oracle on the device's logits, and all three against the two-operator chain."""
+    rng = np.random.default_rng(tokens * 131 + dim + n_experts)
+    x = torch.from_numpy((rng.standard_normal((tokens, dim)) * 3.0).astype(np.float32)).to(DEV).to(x_dtype)
+    gamma = torch.from_numpy(rng.uniform(0.5, 1.5, size=dim).astype(np.float32)).to(DEV)
+    gate = torch.from_numpy((rng.standard_normal((n_experts, dim)) / np.sqrt(dim)).astype(np.float32)).to(DEV)
+    bias = torch.from_numpy(rng.uniform(-0.3, 0.3, size=n_experts).astype(np.float32)).to(DEV)
+    eps = 1e-6
+    lib = _ffi.load_library()
+    code = {torch.float32: _ffi.DTYPE_F32, torch.bfloat16: _ffi.DTYPE_BF16, torch.float16: _ffi.DTYPE_F16}
+    logits = torch.empty(tokens, n_experts, device=DEV)
+    idx = torch.empty(tokens, top_k, dtype=torch.int64, device=DEV)
+    w = torch.empty(tokens, top_k, device=DEV)
+    normed = torch.empty(tokens, dim, dtype=out_dtype, device=DEV)
+    print(f"case route+norm t={tokens} dim={dim} e={n_experts} k={top_k} {x_dtype} -> {out_dtype}", flush=True)
+    st = lib.pllm_moe_route_rmsnorm(x.data_ptr(), code[x_dtype], gamma.data_ptr(), eps, normed.data_ptr(), code[out_dtype], tokens, dim,
+                                    gate.data_ptr(), bias.data_ptr(), n_experts, top_k, 0, logits.data_ptr(), idx.data_ptr(), w.data_ptr(),
+                                    torch.cuda.current_stream().cuda_stream)
+    assert st == 0
+    torch.cuda.synchronize()
+    want_rows = O.rms_norm(x.float().cpu().numpy(), gamma.cpu().numpy(), eps)
+    ulp = {torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8, torch.float32: 2.0 ** -22}[out_dtype]
+    got_rows = normed.double().cpu().numpy()
+    atol = 2.0 ** -25 if out_dtype == torch.float16 else 1e-30          # (fp16 values below 6.1e-5 are spaced 2^-24 apart)
+    assert np.all(np.abs(got_rows - want_rows) <= ulp * np.abs(want_rows) * 1.01 + atol)
+    want_logits = got_rows @ gate.double().cpu().numpy().T
+    assert O.rel_l2(logits.cpu().numpy(), want_logits) < 1e-6
+    want_idx, want_w = O.route_topk(logits.cpu().numpy(), bias.cpu().numpy(), top_k, False)
+    got_idx = idx.cpu().numpy()
+    if np.array_equal(got_idx, want_idx):
+        np.testing.assert_allclose(w.cpu().numpy(), want_w, rtol=2e-6, atol=1e-8)
+    else:                                                  # two scores within float32 rounding of each other
+        sc = 1.0 / (1.0 + np.exp(-logits.double().cpu().numpy())) + bias.double().cpu().numpy()[None, :]
+        for t in range(tokens):
+            assert np.abs(np.sort(np.take(sc[t], got_idx[t])) - np.sort(np.take(sc[t], want_idx[t]))).max() < 1e-6
+    # the two-operator chain: same rows up to one unit of the output type where the row's scale rounded the other way, then
+    # the same picks wherever the rows are the same bits
+    rows2 = mod.fused_rms_norm_forward(x, gamma, eps, out_dtype=out_dtype)
+    assert np.all(np.abs(rows2.double().cpu().numpy() - got_rows) <= 2.0 * ulp * np.abs(got_rows) + 2.0 * atol)
+    i2, w2 = mod.moe_route(rows2, gate, bias, top_k)
+    for t in range(tokens):
+        if torch.equal(rows2[t], normed[t]):
+            assert torch.equal(i2[t], idx[t]) and torch.allclose(w2[t], w[t], rtol=1e-5, atol=1e-8)
+    # the operator form
+    out = mod.moe_route_rmsnorm(x, gamma, eps, gate, bias, top_k, out_dtype=out_dtype)
+    assert out is not None and torch.equal(out[0], idx) and torch.equal(out[1], w) and torch.equal(out[2], normed)
+
+
+def test_router_with_normalisation_declines_what_it_has_no_launch_for(mod):
+    gate = torch.randn(16, 4096, device=DEV)
+    assert mod.moe_route_rmsnorm(torch.randn(1, 4096, device=DEV), torch.ones(4096, device=DEV), 1e-6, gate, None, 4) is None      # wider than a wave holds
+    gate = torch.randn(16, 512, device=DEV)
+    assert mod.moe_route_rmsnorm(torch.randn(5, 512, device=DEV), torch.ones(512, device=DEV), 1e-6, gate, None, 4) is None        # more than four rows
+    gate = torch.randn(16, 510, device=DEV)
+    assert mod.moe_route_rmsnorm(torch.randn(1, 510, device=DEV), torch.ones(510, device=DEV), 1e-6, gate, None, 4) is None        # not whole vectors
+    out = mod.moe_route_rmsnorm(torch.randn(2, 512, device=DEV), torch.ones(512, device=DEV), 1e-6, torch.randn(16, 512, device=DEV), None, 4)
+    assert out is not None and tuple(out[2].shape) == (2, 512)
+
+
 def _any_expert_blocks(rng, type_name, e, n, k):
     if type_name in ("iq2_xxs", "iq1_m", "q2_k"):
         return _expert_blocks(rng, type_name, e, n, k)
