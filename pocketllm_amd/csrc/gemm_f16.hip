@@ -730,9 +730,19 @@ struct GemmPlan { int mi; int tiles_n; int tiles; int full_tiles; int slices; };
 // number of K slices that minimises rounds per slice plus the cost of moving the partial tiles.
 GemmPlan plan_gemm(int t_rows, int n, int bpr) {
     GemmPlan p;
-    p.mi = t_rows <= 64 ? 1 : (t_rows <= 128 ? 2 : 4);
-    const int bm = 64 * p.mi, cus = compute_units();
+    const int cus = compute_units();
     p.tiles_n = (n + kBN - 1) / kBN;
+    p.mi = t_rows <= 64 ? 1 : (t_rows <= 128 ? 2 : 4);
+    if (t_rows > 128) {
+        // 128-row tiles instead of 256-row ones where those would leave the machine mostly empty (a quarter of the compute units or
+        // less: half the partial-tile traffic per slice, twice the workgroups before slicing), and where the last 256-row tile
+        // would be half padding while the 128-row tiles still fit one round.  Q4_K, us, 256- / 128-row tiles: 5120x5120 T=129
+        // 49.8 / 42.9, T=256 52.1 / 44.1, T=384 60.9 / 50.8, T=512 64.3 / 63.7, T=1024 92.7 / 114.0; 17408x5120 T=256 83.1 / 107.4,
+        // T=384 152.3 / 138.5, T=512 159.8 / 167.7
+        const int tiles128 = (t_rows + 127) / 128, tiles256 = (t_rows + 255) / 256;
+        if (tiles256 * p.tiles_n * 4 <= cus || ((tiles128 & 1) && tiles128 * p.tiles_n <= cus)) p.mi = 2;
+    }
+    const int bm = 64 * p.mi;
     p.tiles = ((t_rows + bm - 1) / bm) * p.tiles_n;
     p.full_tiles = (p.tiles / cus) * cus;
     const int rem = p.tiles - p.full_tiles;
