@@ -336,7 +336,7 @@ def extra_cases(mod, dev):
     ksets = [torch.from_numpy(rng.choice(ek, size=8, replace=False).astype(np.int64)).to(dev) for _ in range(8)]
     kwts = torch.full((8,), 0.125, device=dev)
     xk = torch.randn(1, dk, device=dev, dtype=torch.bfloat16)
-    run("routed experts q4_k, 128 experts top-8, 2048 -> 768, T=1 (four launches)", kbytes,
+    run("routed experts q4_k, 128 experts top-8, 2048 -> 768, T=1 (two launches)", kbytes,
         lambda s: mod.gguf_moe_single_token_forward(xk, ksets[s], kwts, kw1, kw3, kw2, 0.0), 8)
     idx16 = np.stack([rng.choice(ek, size=8, replace=False) for _ in range(16)]).astype(np.int64)
     _, ktoks, krws, kseg = mod.moe_group_routes(torch.from_numpy(idx16).to(dev), torch.full((16, 8), 0.125, device=dev), 0, ek)

@@ -357,10 +357,14 @@ __device__ __forceinline__ void raw_to_float4(const RawX<X16>& r, int x_dtype, f
 // right ahead of its weights, so it arrives first).
 // PLAIN: one matrix, one output, activation row = grid row (no routing, no further projections, no row map): the arguments the
 // other forms test one after the other (a scalar load and a wait each) are not read at all.
-template <typename FMT, int ITERS, int DEPTH, bool X16, bool NORM, bool PLAIN = false>
+// RSUM (the down projection of one token's routed experts): wave v is route v.  It takes ALL blocks of its own expert's 16 rows
+// against its own activation row, which it forms on the way as SiLU(min(gate, L)) * clamp(up, +-L) * route weight from the gate
+// (x) and up (x_up) products [routes, k]; the sum over the waves at the end is the sum over the routes, in route order.
+template <typename FMT, int ITERS, int DEPTH, bool X16, bool NORM, bool PLAIN = false, bool RSUM = false>
 __global__ __launch_bounds__(64 * kMaxWaves) void wave_image_matvec_kernel(
     const void* __restrict__ x, int x_dtype, int k, const WeightRoute route, const uint8_t* __restrict__ w, void* __restrict__ y,
-    int y_dtype, int n, int bpr, const float* __restrict__ gamma, float eps, int round_f16, const int64_t* __restrict__ row_token, int x_broadcast) {
+    int y_dtype, int n, int bpr, const float* __restrict__ gamma, float eps, int round_f16, const int64_t* __restrict__ row_token, int x_broadcast,
+    const void* __restrict__ x_up, const float* __restrict__ route_w, float limit) {
     if constexpr (!PLAIN) {
         fetch_together(route);
         asm volatile("" : : "s"(static_cast<int>(row_token != nullptr)), "s"(x_broadcast));
@@ -377,7 +381,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_image_matvec_kernel(
     unsigned char* slot = smem + wave * kWaveBytes;
     float* partial = reinterpret_cast<float*>(smem + waves * kWaveBytes);    // [16][kMaxWaves]: a row's shares side by side
     if constexpr (!PLAIN) {
-        const size_t woff = route_offset(route, blockIdx.y);                  // routed calls: the grid row's expert
+        const size_t woff = route_offset(route, RSUM ? __builtin_amdgcn_readfirstlane(wave) : static_cast<int>(blockIdx.y));   // routed calls: the grid row's expert
         w += woff;
         if (blockIdx.z) {                    // several projections in one launch: this one's matrix, row count and output
             const int m = blockIdx.z - 1;
@@ -389,8 +393,10 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_image_matvec_kernel(
     }
     const int row = blockIdx.x * kRowsPerWg + col;
     const uint8_t* wrow = w + static_cast<size_t>(row < n ? row : 0) * bpr * FMT::kBlockBytes;
-    const size_t xoff = (PLAIN ? static_cast<size_t>(blockIdx.y)
+    const size_t xoff = (PLAIN ? static_cast<size_t>(blockIdx.y) : RSUM ? static_cast<size_t>(wave)
                                : x_broadcast ? 0 : row_token ? static_cast<size_t>(row_token[blockIdx.y]) : static_cast<size_t>(blockIdx.y)) * k;
+    const int bstep = RSUM ? 1 : waves;                                       // distance between a wave's blocks
+    const float rw = RSUM ? route_w[__builtin_amdgcn_readfirstlane(wave)] : 1.0f;
 
     if (lane < 4) reinterpret_cast<uint32_t*>(slot + kSlotBytes)[lane] = 0;
     float acc = 0.0f;
@@ -399,16 +405,18 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_image_matvec_kernel(
     // sum, the shares meet in LDS, and the slices are scaled as they are quantized.  No extra pass over the row, one barrier.
     constexpr int kHeldX = NORM ? ITERS : DEPTH;
     RawX<X16> raw[kHeldX];
+    RawX<X16> raw_up[RSUM ? kHeldX : 1];
     RawX<false> graw[NORM ? ITERS : 1];
     float rstd = 1.0f;
-    for (int b0 = wave; b0 < bpr; b0 += waves * ITERS) {
+    for (int b0 = RSUM ? 0 : wave; b0 < bpr; b0 += bstep * ITERS) {
         typename FMT::Regs regs[DEPTH];
         auto request_x = [&](int it) {
-            const int b = b0 + it * waves;
+            const int b = b0 + it * bstep;
             request_raw4<X16>(raw[it % kHeldX], x, xoff, 256 * b + 4 * lane, b < bpr ? k : 0);
+            if constexpr (RSUM) request_raw4<X16>(raw_up[it % kHeldX], x_up, xoff, 256 * b + 4 * lane, b < bpr ? k : 0);
         };
         auto request_w = [&](int it) {
-            const int b = b0 + it * waves;
+            const int b = b0 + it * bstep;
             FMT::load(regs[it % DEPTH], wrow + static_cast<size_t>(min(b, bpr - 1)) * FMT::kBlockBytes, ks);   // clamped: always a valid address
         };
         auto request = [&](int it) {
@@ -423,7 +431,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_image_matvec_kernel(
         if constexpr (NORM) {
 #pragma unroll
             for (int it = 0; it < ITERS; ++it) {
-                const int b = b0 + it * waves;
+                const int b = b0 + it * bstep;
                 request_raw4<false>(graw[it], gamma, 0, 256 * b + 4 * lane, b < bpr ? k : 0);
             }
         }
@@ -435,7 +443,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_image_matvec_kernel(
             float ss = 0.0f;
 #pragma unroll
             for (int it = 0; it < ITERS; ++it) {
-                const int b = b0 + it * waves;
+                const int b = b0 + it * bstep;
                 if (k != 256 * bpr) {                                        // rows that end inside their last block
                     settle_raw4<X16>(raw[it], 256 * b + 4 * lane, b < bpr ? k : 0);
                     settle_raw4<false>(graw[it], 256 * b + 4 * lane, b < bpr ? k : 0);
@@ -454,13 +462,27 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_image_matvec_kernel(
         }
 #pragma unroll
         for (int it = 0; it < ITERS; ++it) {
-            const int b = b0 + it * waves;
+            const int b = b0 + it * bstep;
             if (b < bpr) {                                                   // wave-uniform
                 // the block's activation slice into the wave's slot: the same two-term image the pre-pass kernel writes
                 float v[4];
                 if constexpr (!NORM)
                     if (k != 256 * bpr) settle_raw4<X16>(raw[it % kHeldX], 256 * b + 4 * lane, k);   // rows that end inside their last block
                 raw_to_float4<X16>(raw[it % kHeldX], x_dtype, v);
+                if constexpr (RSUM) {
+                    float u[4];
+                    if (k != 256 * bpr) settle_raw4<X16>(raw_up[it % kHeldX], 256 * b + 4 * lane, k);
+                    raw_to_float4<X16>(raw_up[it % kHeldX], x_dtype, u);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        float g = v[i], uu = u[i];
+                        if (limit > 0.0f) {
+                            uu = fminf(fmaxf(uu, -limit), limit);
+                            g = fminf(g, limit);
+                        }
+                        v[i] = g / (1.0f + expf(-g)) * uu * rw;              // values past k are zeros on both sides
+                    }
+                }
                 if constexpr (NORM) {
                     const float g[4] = {__uint_as_float(graw[it].v.x), __uint_as_float(graw[it].v.y), __uint_as_float(graw[it].v.z), __uint_as_float(graw[it].v.w)};
 #pragma unroll
@@ -543,7 +565,7 @@ int launch_wave_kernel(KERN kern, const ActRows& act, const WeightRoute& route, 
     for (int m = 0; m < route.extra; ++m) tallest = tallest > route.more_n[m] ? tallest : route.more_n[m];
     dim3 grid((tallest + kRowsPerWg - 1) / kRowsPerWg, rows, 1 + route.extra);
     hipLaunchKernelGGL(kern, grid, dim3(64 * waves), smem, stream, act.x, act.x_dtype, act.k, route, w, y, y_dtype, n, bpr, act.gamma, act.eps,
-                       act.round_f16, act.row_token, act.x_broadcast);
+                       act.round_f16, act.row_token, act.x_broadcast, static_cast<const void*>(nullptr), static_cast<const float*>(nullptr), 0.0f);
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 
@@ -586,6 +608,26 @@ int launch_wave(const ActRows& act, const WeightRoute& route, const uint8_t* w, 
         default: PLLM_CASE(8);
     }
 #undef PLLM_CASE
+}
+
+// the routes of one token as the waves of a workgroup (RSUM): float32 gate / up products [routes, k], routes <= kMaxWaves
+template <typename FMT>
+int launch_wave_route_sum(const float* gate, const float* up, const float* route_w, float limit, int k, const WeightRoute& route, const uint8_t* w,
+                          void* y, int y_dtype, int n, int bpr, int routes, hipStream_t stream) {
+    const int passes = (bpr + 5) / 6, iters = (bpr + passes - 1) / passes;
+    const size_t smem = static_cast<size_t>(routes) * (kSlotBytes + 16) + static_cast<size_t>(kMaxWaves * kRowsPerWg + routes) * sizeof(float);
+    const dim3 grid((n + kRowsPerWg - 1) / kRowsPerWg, 1, 1);
+#define PLLM_CASE(I) case I: \
+        hipLaunchKernelGGL((wave_image_matvec_kernel<FMT, I, wave_depth<FMT>(I, false), false, false, false, true>), grid, dim3(64 * routes), smem, stream, \
+                           static_cast<const void*>(gate), PLLM_F32, k, route, w, y, y_dtype, n, bpr, static_cast<const float*>(nullptr), 0.0f, 0, \
+                           static_cast<const int64_t*>(nullptr), 0, static_cast<const void*>(up), route_w, limit); \
+        break
+    switch (iters) {
+        PLLM_CASE(1); PLLM_CASE(2); PLLM_CASE(3); PLLM_CASE(4); PLLM_CASE(5);
+        default: PLLM_CASE(6);
+    }
+#undef PLLM_CASE
+    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -680,10 +722,12 @@ struct WaveQ6K {
 // NORM (one pass of the block loop, as in wave_image_matvec_kernel): the wave requests the slices of all its blocks at once, their
 // squares are its share of the row's sum, the shares meet in LDS behind one barrier and the slices are scaled by rstd * gamma
 // as they are quantized.
-template <typename FMT, int ITERS, int DEPTH, bool X16, bool PLAIN = false, bool NORM = false>
+// RSUM: as in wave_image_matvec_kernel (wave = route of one token's experts, SwiGLU formed on the way, ordered sum at the end).
+template <typename FMT, int ITERS, int DEPTH, bool X16, bool PLAIN = false, bool NORM = false, bool RSUM = false>
 __global__ __launch_bounds__(64 * kMaxWaves) void wave_groups16_matvec_kernel(
     const void* __restrict__ x, int x_dtype, int k, const WeightRoute route, const uint8_t* __restrict__ w, void* __restrict__ y,
-    int y_dtype, int n, int bpr, const int64_t* __restrict__ row_token, int x_broadcast, const float* __restrict__ gamma, float eps, int round_f16) {
+    int y_dtype, int n, int bpr, const int64_t* __restrict__ row_token, int x_broadcast, const float* __restrict__ gamma, float eps, int round_f16,
+    const void* __restrict__ x_up, const float* __restrict__ route_w, float limit) {
     if constexpr (!PLAIN) {
         fetch_together(route);
         asm volatile("" : : "s"(static_cast<int>(row_token != nullptr)), "s"(x_broadcast));
@@ -700,7 +744,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_groups16_matvec_kernel(
     unsigned char* slot = smem + wave * kWaveBytes;
     float* partial = reinterpret_cast<float*>(smem + waves * kWaveBytes);    // [16][kMaxWaves]: a row's shares side by side
     if constexpr (!PLAIN) {
-        const size_t woff = route_offset(route, blockIdx.y);                  // routed calls: the grid row's expert
+        const size_t woff = route_offset(route, RSUM ? __builtin_amdgcn_readfirstlane(wave) : static_cast<int>(blockIdx.y));   // routed calls: the grid row's expert
         w += woff;
         if (blockIdx.z) {                    // several projections in one launch: this one's matrix, row count and output
             const int m = blockIdx.z - 1;
@@ -712,8 +756,10 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_groups16_matvec_kernel(
     }
     const int row = blockIdx.x * kRowsPerWg + col;
     const uint8_t* wrow = w + static_cast<size_t>(row < n ? row : 0) * bpr * FMT::kBlockBytes;
-    const size_t xoff = (PLAIN ? static_cast<size_t>(blockIdx.y)
+    const size_t xoff = (PLAIN ? static_cast<size_t>(blockIdx.y) : RSUM ? static_cast<size_t>(wave)
                                : x_broadcast ? 0 : row_token ? static_cast<size_t>(row_token[blockIdx.y]) : static_cast<size_t>(blockIdx.y)) * k;
+    const int bstep = RSUM ? 1 : waves;                                       // distance between a wave's blocks
+    const float rw = RSUM ? route_w[__builtin_amdgcn_readfirstlane(wave)] : 1.0f;
     // the lane's A operand: group `col` of the block, in the one MFMA whose slice ks carries that group
     const bool mine = FMT::slice_of(col) == ks;
     const int my_t = FMT::mfma_of(col);
@@ -722,16 +768,18 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_groups16_matvec_kernel(
     float acc = 0.0f;
     constexpr int kHeldX = NORM ? ITERS : DEPTH;
     float rstd = 1.0f;
-    for (int b0 = wave; b0 < bpr; b0 += waves * ITERS) {
+    for (int b0 = RSUM ? 0 : wave; b0 < bpr; b0 += bstep * ITERS) {
         RawX<X16> raw[kHeldX];
+        RawX<X16> raw_up[RSUM ? kHeldX : 1];
         RawX<false> graw[NORM ? ITERS : 1];
         typename FMT::Regs regs[DEPTH];
         auto request_x = [&](int it) {
-            const int b = b0 + it * waves;
+            const int b = b0 + it * bstep;
             request_raw4<X16>(raw[it % kHeldX], x, xoff, 256 * b + 4 * lane, b < bpr ? k : 0);
+            if constexpr (RSUM) request_raw4<X16>(raw_up[it % kHeldX], x_up, xoff, 256 * b + 4 * lane, b < bpr ? k : 0);
         };
         auto request_w = [&](int it) {
-            const int b = b0 + it * waves;
+            const int b = b0 + it * bstep;
             FMT::load(regs[it % DEPTH], wrow + static_cast<size_t>(min(b, bpr - 1)) * FMT::kBlockBytes, ks);   // clamped: always a valid address
         };
 #pragma unroll
@@ -739,7 +787,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_groups16_matvec_kernel(
         if constexpr (NORM) {
 #pragma unroll
             for (int it = 0; it < ITERS; ++it) {
-                const int b = b0 + it * waves;
+                const int b = b0 + it * bstep;
                 request_raw4<false>(graw[it], gamma, 0, 256 * b + 4 * lane, b < bpr ? k : 0);
             }
         }
@@ -751,7 +799,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_groups16_matvec_kernel(
             float ss = 0.0f;
 #pragma unroll
             for (int it = 0; it < ITERS; ++it) {
-                const int b = b0 + it * waves;
+                const int b = b0 + it * bstep;
                 if (k != 256 * bpr) {                                        // rows that end inside their last block
                     settle_raw4<X16>(raw[it], 256 * b + 4 * lane, b < bpr ? k : 0);
                     settle_raw4<false>(graw[it], 256 * b + 4 * lane, b < bpr ? k : 0);
@@ -770,12 +818,26 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_groups16_matvec_kernel(
         }
 #pragma unroll
         for (int it = 0; it < ITERS; ++it) {
-            const int b = b0 + it * waves;
+            const int b = b0 + it * bstep;
             if (b < bpr) {                                                   // wave-uniform
                 float v[4];
                 if constexpr (!NORM)
                     if (k != 256 * bpr) settle_raw4<X16>(raw[it % kHeldX], 256 * b + 4 * lane, k);
                 raw_to_float4<X16>(raw[it % kHeldX], x_dtype, v);
+                if constexpr (RSUM) {
+                    float u[4];
+                    if (k != 256 * bpr) settle_raw4<X16>(raw_up[it % kHeldX], 256 * b + 4 * lane, k);
+                    raw_to_float4<X16>(raw_up[it % kHeldX], x_dtype, u);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        float g = v[i], uu = u[i];
+                        if (limit > 0.0f) {
+                            uu = fminf(fmaxf(uu, -limit), limit);
+                            g = fminf(g, limit);
+                        }
+                        v[i] = g / (1.0f + expf(-g)) * uu * rw;              // values past k are zeros on both sides
+                    }
+                }
                 if constexpr (NORM) {
                     const float g[4] = {__uint_as_float(graw[it].v.x), __uint_as_float(graw[it].v.y), __uint_as_float(graw[it].v.z), __uint_as_float(graw[it].v.w)};
 #pragma unroll
@@ -848,7 +910,27 @@ int launch_q2k_kernel(KERN kern, const ActRows& act, const WeightRoute& route, c
     for (int m = 0; m < route.extra; ++m) tallest = tallest > route.more_n[m] ? tallest : route.more_n[m];
     dim3 grid((tallest + kRowsPerWg - 1) / kRowsPerWg, rows, 1 + route.extra);
     hipLaunchKernelGGL(kern, grid, dim3(64 * waves), smem, stream, act.x, act.x_dtype, act.k, route, w, y, y_dtype, n, bpr, act.row_token, act.x_broadcast,
-                       act.gamma, act.eps, act.round_f16);
+                       act.gamma, act.eps, act.round_f16, static_cast<const void*>(nullptr), static_cast<const float*>(nullptr), 0.0f);
+    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+}
+
+// the routes of one token as the waves of a workgroup (RSUM): float32 gate / up products [routes, k], routes <= kMaxWaves
+template <typename FMT>
+int launch_groups16_route_sum(const float* gate, const float* up, const float* route_w, float limit, int k, const WeightRoute& route, const uint8_t* w,
+                              void* y, int y_dtype, int n, int bpr, int routes, hipStream_t stream) {
+    const int passes = (bpr + 5) / 6, iters = (bpr + passes - 1) / passes;
+    const size_t smem = static_cast<size_t>(routes) * (kQ2SlotBytes + 16) + static_cast<size_t>(kMaxWaves * kRowsPerWg + routes) * sizeof(float);
+    const dim3 grid((n + kRowsPerWg - 1) / kRowsPerWg, 1, 1);
+#define PLLM_CASE(I) case I: \
+        hipLaunchKernelGGL((wave_groups16_matvec_kernel<FMT, I, (I < 2 ? I : 2), false, false, false, true>), grid, dim3(64 * routes), smem, stream, \
+                           static_cast<const void*>(gate), PLLM_F32, k, route, w, y, y_dtype, n, bpr, static_cast<const int64_t*>(nullptr), 0, \
+                           static_cast<const float*>(nullptr), 0.0f, 0, static_cast<const void*>(up), route_w, limit); \
+        break
+    switch (iters) {
+        PLLM_CASE(1); PLLM_CASE(2); PLLM_CASE(3); PLLM_CASE(4); PLLM_CASE(5);
+        default: PLLM_CASE(6);
+    }
+#undef PLLM_CASE
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 
@@ -1374,6 +1456,24 @@ int kquant_matvec_from_image(const ActRows& act, const uint8_t* w, int type_id, 
     switch (type_id) {
         case PLLM_TYPE_Q4_K: return launch_k45<Q4K>(act, route, w, y, y_dtype, rows, n, bpr, stream);
         case PLLM_TYPE_Q5_K: return launch_k45<Q5K>(act, route, w, y, y_dtype, rows, n, bpr, stream);
+        default: return PLLM_ERR_UNSUPPORTED;
+    }
+}
+
+// Down projection of one token's routed experts with the SwiGLU ahead of it and the ordered sum over the routes behind it in one
+// launch: y[n] (+)= sum over routes r, in route order, of W_{e(r)} (SiLU(gate[r]) * up[r] * route_w[r]); Q4_K, Q5_K, IQ4_XS, Q6_K
+// and Q2_K, up to kMaxWaves routes (PLLM_ERR_UNSUPPORTED otherwise).  route carries the expert numbers and the expert stride.
+int kquant_route_sum_matvec(const float* gate, const float* up, const float* route_w, float limit, int k, const WeightRoute& route, const uint8_t* w,
+                            int type_id, void* y, int y_dtype, int n, int bpr, int routes, hipStream_t stream) {
+    if (routes < 1 || routes > kMaxWaves || k < 4 || !routed(route) || route.extra != 0) return PLLM_ERR_UNSUPPORTED;
+    const unsigned need = type_id == PLLM_TYPE_Q6_K ? 1u : type_id == PLLM_TYPE_Q2_K ? 3u : type_id == PLLM_TYPE_IQ4_XS ? 7u : 15u;   // the formats' block boundaries
+    if ((reinterpret_cast<uintptr_t>(w) | route.expert_stride) & need) return PLLM_ERR_UNSUPPORTED;
+    switch (type_id) {
+        case PLLM_TYPE_Q4_K: return launch_wave_route_sum<Q4K>(gate, up, route_w, limit, k, route, w, y, y_dtype, n, bpr, routes, stream);
+        case PLLM_TYPE_Q5_K: return launch_wave_route_sum<Q5K>(gate, up, route_w, limit, k, route, w, y, y_dtype, n, bpr, routes, stream);
+        case PLLM_TYPE_IQ4_XS: return launch_wave_route_sum<IQ4XS>(gate, up, route_w, limit, k, route, w, y, y_dtype, n, bpr, routes, stream);
+        case PLLM_TYPE_Q6_K: return launch_groups16_route_sum<WaveQ6K>(gate, up, route_w, limit, k, route, w, y, y_dtype, n, bpr, routes, stream);
+        case PLLM_TYPE_Q2_K: return launch_groups16_route_sum<WaveQ2K>(gate, up, route_w, limit, k, route, w, y, y_dtype, n, bpr, routes, stream);
         default: return PLLM_ERR_UNSUPPORTED;
     }
 }

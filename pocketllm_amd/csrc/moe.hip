@@ -687,7 +687,8 @@ int pllm_gguf_moe_forward(const void* x, int x_dtype, int64_t tokens, int64_t di
         // by route through the dense decode kernels in their routed form (grid row = route, matrix = the route's expert, activation
         // row = the route's token, quantized inside the kernel): gate and up as one launch (grid.z picks the matrix), SwiGLU into
         // hidden images, down, ordered sum per token.  Four launches for one token (its int64 expert numbers are read as they are;
-        // the SwiGLU inside the down projection's activation quantizer instead of a launch of its own ran 22.3 us against 20.4).
+        // the SwiGLU inside the down projection's activation quantizer instead of a launch of its own ran 22.3 us against 20.4 in
+        // the route-per-workgroup form), two where the down format has the routes-as-waves form.
         unsigned char* p = static_cast<unsigned char*>(workspace);
         p += x_stride * tokens;                                              // (the activation images of the layout: unused here)
         unsigned char* h_image = p;  p += h_stride * routes;
@@ -717,6 +718,12 @@ int pllm_gguf_moe_forward(const void* x, int x_dtype, int64_t tokens, int64_t di
         r2.expert_stride = static_cast<size_t>(dim) * bpr_h * pllm_gguf_block_bytes(w2_type);
         int st = superblock_matvec(xa, w1, w13_type, gate, PLLM_F32, R, I, bpr_x, s, r13);
         if (st != PLLM_OK) return st;
+        if (tokens == 1) {
+            // one token, a down format of the single-launch wave kernels: the routes are the waves of a workgroup, which form their
+            // hidden slices from the gate and up products themselves and meet in the ordered sum (two launches in all)
+            const int st2 = kquant_route_sum_matvec(gate, up, route_weights, swiglu_limit, I, r2, w2, w2_type, y, PLLM_F32, D, bpr_h, R, s);
+            if (st2 != PLLM_ERR_UNSUPPORTED) return st2;
+        }
         const int h_kpad = bpr_h * 256;
         hipLaunchKernelGGL(swiglu_image_kernel, dim3((h_kpad / 4 + 255) / 256, R), dim3(256), 0, s, gate, up, route_weights, swiglu_limit, I, h_kpad,
                            h_image, h_stride);

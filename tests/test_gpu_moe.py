@@ -595,6 +595,35 @@ def test_experts_in_every_block_type(mod, t13, t2, tokens):
         assert O.rel_l2(y.cpu().numpy(), want) <= TOL, (t13, t2, tokens, limit)
 
 
+@pytest.mark.parametrize("t2", ["q4_k", "q5_k", "iq4_xs", "q6_k", "q2_k"])
+@pytest.mark.parametrize("topk,inter", [(8, 768), (5, 600), (1, 256)])
+def test_one_token_down_projection_with_the_routes_as_waves(mod, t2, topk, inter):
+    """One token through experts without fused kernels: the down projection forms SiLU(gate) * up * route weight itself, one wave
+    per route, and sums the routes in route order (two launches in all).  Every down format of the single-launch kernels, a row
+    length that ends inside its last super-block, one to eight routes, with and without the clamp; bitwise repeatable."""
+    rng = np.random.default_rng(900 + topk + inter + len(t2))
+    e, d = 12, 512
+    w1 = _any_expert_blocks(rng, "q4_k", e, inter, d)
+    w3 = _any_expert_blocks(rng, "q4_k", e, inter, d)
+    if t2 == "q2_k":                                       # (the helper's Q2_K encoder takes whole super-blocks)
+        wd = (rng.standard_normal((e * d, (inter + 255) // 256 * 256)) * 0.05).astype(np.float32)
+        wd[:, inter:] = 0.0
+        w2 = C.quantize_q2_k(wd).reshape(e, d, (inter + 255) // 256, 84)
+    else:
+        w2 = _any_expert_blocks(rng, t2, e, d, inter)
+    idx, wts = _route(rng, 1, e, topk)
+    x = torch.from_numpy(rng.standard_normal((1, d)).astype(np.float32)).to(DEV).to(torch.bfloat16)
+    dw1, dw3, dw2 = (torch.from_numpy(a).to(DEV) for a in (w1, w3, w2))
+    for limit in (0.0, 0.5):
+        print(f"case routes as waves q4_k/{t2} topk={topk} inter={inter} limit={limit}", flush=True)
+        y = mod.gguf_moe_single_token_forward(x, torch.from_numpy(idx[0]).to(DEV), torch.from_numpy(wts[0]).to(DEV), dw1, dw3, dw2, limit)
+        torch.cuda.synchronize()
+        want = O.moe_forward(x.float().cpu().numpy(), np.zeros(topk, dtype=np.int64), wts[0], idx[0], w1, w3, w2, "q4_k", "q4_k", t2, limit)
+        assert O.rel_l2(y.cpu().numpy(), want) <= TOL, (t2, topk, inter, limit)
+        y2 = mod.gguf_moe_single_token_forward(x, torch.from_numpy(idx[0]).to(DEV), torch.from_numpy(wts[0]).to(DEV), dw1, dw3, dw2, limit)
+        assert torch.equal(y, y2)
+
+
 @pytest.mark.parametrize("t13,t2", [("q4_k", "q6_k"), ("iq4_xs", "q5_k")])
 def test_experts_with_few_routes_each_at_sixteen_tokens_or_more(mod, t13, t2):
     """Types without fused expert kernels, 16 tokens or more but under four routes per expert on average: the route-by-route path
