@@ -367,8 +367,9 @@ int pllm_gguf_moe_forward(const void* x, int x_dtype, int64_t tokens, int64_t di
  * float32 sum of what y holds and the routes' sum, rounded once), for callers that would otherwise convert and add in two
  * further launches (the reference's block does: src/models/minimax_m2/architecture.py:404-413).  Same arguments and workspace as
  * pllm_gguf_moe_forward with tokens == 1.  PLLM_ERR_UNSUPPORTED when the shape or the type pair has no kernel that sums the
- * routes inside the down projection (IQ2_XXS or IQ1_M gate / up with IQ1_M down, whole 16-row tiles, 16-byte aligned tensors):
- * call pllm_gguf_moe_forward and add.  No routes: y is left as it is.
+ * routes inside the down projection: call pllm_gguf_moe_forward and add.  Such kernels exist for IQ2_XXS or IQ1_M gate / up with
+ * IQ1_M down (whole 16-row tiles, 16-byte aligned tensors) and, with any gate / up type outside that family, for Q4_K, Q5_K,
+ * IQ4_XS, Q6_K and Q2_K down with up to 8 routes (expert matrices on their block type's boundary).  No routes: y is left as it is.
  */
 int pllm_gguf_moe_single_token_accumulate(const void* x, int x_dtype, int64_t dim, int64_t inter, const int64_t* route_experts,
                                           const float* route_weights, int64_t routes, const uint8_t* w1, const uint8_t* w3, int w13_type,

@@ -1463,11 +1463,21 @@ int kquant_matvec_from_image(const ActRows& act, const uint8_t* w, int type_id, 
 // Down projection of one token's routed experts with the SwiGLU ahead of it and the ordered sum over the routes behind it in one
 // launch: y[n] (+)= sum over routes r, in route order, of W_{e(r)} (SiLU(gate[r]) * up[r] * route_w[r]); Q4_K, Q5_K, IQ4_XS, Q6_K
 // and Q2_K, up to kMaxWaves routes (PLLM_ERR_UNSUPPORTED otherwise).  route carries the expert numbers and the expert stride.
+bool kquant_route_sum_supports(int type_id, int routes, int k, const uint8_t* w, size_t expert_stride) {
+    if (routes < 1 || routes > kMaxWaves || k < 4) return false;
+    unsigned need;                                                            // the formats' block boundaries
+    switch (type_id) {
+        case PLLM_TYPE_Q4_K: case PLLM_TYPE_Q5_K: need = 15u; break;
+        case PLLM_TYPE_IQ4_XS: need = 7u; break;
+        case PLLM_TYPE_Q2_K: need = 3u; break;
+        case PLLM_TYPE_Q6_K: need = 1u; break;
+        default: return false;
+    }
+    return ((reinterpret_cast<uintptr_t>(w) | expert_stride) & need) == 0;
+}
 int kquant_route_sum_matvec(const float* gate, const float* up, const float* route_w, float limit, int k, const WeightRoute& route, const uint8_t* w,
                             int type_id, void* y, int y_dtype, int n, int bpr, int routes, hipStream_t stream) {
-    if (routes < 1 || routes > kMaxWaves || k < 4 || !routed(route) || route.extra != 0) return PLLM_ERR_UNSUPPORTED;
-    const unsigned need = type_id == PLLM_TYPE_Q6_K ? 1u : type_id == PLLM_TYPE_Q2_K ? 3u : type_id == PLLM_TYPE_IQ4_XS ? 7u : 15u;   // the formats' block boundaries
-    if ((reinterpret_cast<uintptr_t>(w) | route.expert_stride) & need) return PLLM_ERR_UNSUPPORTED;
+    if (!routed(route) || route.extra != 0 || !kquant_route_sum_supports(type_id, routes, k, w, route.expert_stride)) return PLLM_ERR_UNSUPPORTED;
     switch (type_id) {
         case PLLM_TYPE_Q4_K: return launch_wave_route_sum<Q4K>(gate, up, route_w, limit, k, route, w, y, y_dtype, n, bpr, routes, stream);
         case PLLM_TYPE_Q5_K: return launch_wave_route_sum<Q5K>(gate, up, route_w, limit, k, route, w, y, y_dtype, n, bpr, routes, stream);

@@ -590,11 +590,37 @@ int pllm_gguf_moe_single_token_accumulate(const void* x, int x_dtype, int64_t di
     if (!workspace || workspace_bytes < pllm_gguf_moe_workspace_bytes(1, routes, dim, inter)) return PLLM_ERR_WORKSPACE;
     const int bpr_h = static_cast<int>((inter + 255) / 256);
     const int R = static_cast<int>(routes), I = static_cast<int>(inter), D = static_cast<int>(dim);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const size_t h_stride = act_image_256_bytes(bpr_h);
+    if ((!dot4_type(w13_type) || !dot4_type(w2_type)) && pllm_gguf_block_bytes(w13_type) != 0) {
+        // types without fused expert kernels: gate and up as one launch of the routed wave kernels, then the down projection with the
+        // routes as its waves, which adds the ordered sum into y itself (the workspace layout of pllm_gguf_moe_forward's same path)
+        const int bpr_x = static_cast<int>((dim + 255) / 256);
+        const size_t stride2 = static_cast<size_t>(dim) * bpr_h * pllm_gguf_block_bytes(w2_type);
+        if (!kquant_route_sum_supports(w2_type, R, I, w2, stride2)) return PLLM_ERR_UNSUPPORTED;
+        unsigned char* p = static_cast<unsigned char*>(workspace);
+        p += act_image_256_bytes(bpr_x) + h_stride * routes + align256(static_cast<size_t>(routes) * dim * sizeof(float)) +
+             align256(static_cast<size_t>(routes) * sizeof(int32_t));
+        float* gate = reinterpret_cast<float*>(p);  p += align256(static_cast<size_t>(routes) * inter * sizeof(float));
+        float* up = reinterpret_cast<float*>(p);
+        WeightRoute r13{};
+        r13.expert64 = route_experts;
+        WeightRoute r2 = r13;
+        r13.expert_stride = static_cast<size_t>(inter) * bpr_x * pllm_gguf_block_bytes(w13_type);
+        r13.extra = 1;
+        r13.more_w[0] = w3;
+        r13.more_y[0] = up;
+        r13.more_n[0] = I;
+        r2.expert_stride = stride2;
+        ActRows xa = act_rows_raw(x, x_dtype, D);
+        xa.x_broadcast = 1;
+        const int st = superblock_matvec(xa, w1, w13_type, gate, PLLM_F32, R, I, bpr_x, s, r13);
+        if (st != PLLM_OK) return st;
+        return kquant_route_sum_matvec(gate, up, route_weights, swiglu_limit, I, r2, w2, w2_type, y, y_dtype | kAccumulateInto, D, bpr_h, R, s);
+    }
     if (routes * staged_x_bytes(bpr_h * 256) > 96 * 1024 || !moe_single_mfma_supports(w13_type, w2_type, D, I, R, x, w1, w3, w2))
         return PLLM_ERR_UNSUPPORTED;
-    hipStream_t s = static_cast<hipStream_t>(stream);
     unsigned char* himg = static_cast<unsigned char*>(workspace);
-    const size_t h_stride = act_image_256_bytes(bpr_h);
     const int st = moe_single_w13_mfma(x, x_dtype, D, route_experts, route_weights, R, w1, w3, w13_type, I, swiglu_limit, himg, h_stride, s);
     if (st != PLLM_OK) return st;
     return moe_single_w2_mfma(himg, h_stride, I, route_experts, R, w2, nullptr, D, s, y, y_dtype);

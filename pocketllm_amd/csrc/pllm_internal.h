@@ -129,6 +129,7 @@ int dot4_matvec_from_image(const ActRows& act, const uint8_t* w, int type_id, vo
 int k45_rows16_matvec(const void* x, int x_dtype, const uint8_t* w, int type_id, void* y, int y_dtype, int rows, int k, int n, int bpr, hipStream_t stream);
 // Q4_K / Q5_K on 17 - 48 activation rows: every block decoded once in registers and multiplied into all rows (fp16 matrix cores,
 // exact weights); workspace = staged fp16 rows + partial sums of the slices along K
+bool kquant_route_sum_supports(int type_id, int routes, int k, const uint8_t* w, size_t expert_stride);
 int kquant_route_sum_matvec(const float* gate, const float* up, const float* route_w, float limit, int k, const WeightRoute& route, const uint8_t* w,
                             int type_id, void* y, int y_dtype, int n, int bpr, int routes, hipStream_t stream);
 bool k45_rows64_reads_raw(const void* x, int x_dtype, int k, int n, int bpr);

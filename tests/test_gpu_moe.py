@@ -150,6 +150,17 @@ def test_single_token_experts_added_into_the_residual_stream(mod, dtype):
     assert mod.gguf_moe_single_token_accumulate_forward(x, slots, rw, dw1, dw3, dw2, 0.0, y) is True
     torch.cuda.synchronize()
     assert torch.equal(y, (stream.float() + plain).to(dtype))
+    # types without fused expert kernels: the down projection with the routes as its waves adds into y
+    for t13, t2 in (("q4_k", "q6_k"), ("q5_k", "q4_k")):
+        g1, g3, g2 = (torch.from_numpy(_any_expert_blocks(rng, t, 4, n, k)).to(DEV) for t, n, k in ((t13, 512, 768), (t13, 512, 768), (t2, 768, 512)))
+        xs = x[:, :768].contiguous()
+        few = torch.tensor([3, 0, 2], dtype=torch.int64, device=DEV)
+        fw = torch.tensor([0.5, 0.3, 0.2], device=DEV)
+        plain_g = mod.gguf_moe_single_token_forward(xs, few, fw, g1, g3, g2, 0.0)
+        base = stream[:, :768].contiguous()
+        yg = base.clone()
+        assert mod.gguf_moe_single_token_accumulate_forward(xs, few, fw, g1, g3, g2, 0.0, yg) is True
+        assert torch.equal(yg, (base.float() + plain_g).to(dtype))
     # a type pair whose down projection has no such kernel: refused, y untouched
     w2q = torch.from_numpy(_expert_blocks(rng, "q2_k", e, d, inter)).to(DEV)
     y2 = stream.clone()
