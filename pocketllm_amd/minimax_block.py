@@ -248,6 +248,7 @@ class MiniMaxTransformer:
         self.lm_head = lm_head
         self.device = device
         self.dtype = dtype
+        self._cuda = _kernel()
 
     def reset_cache(self, batch_size: int, max_seq_len: int) -> None:
         for layer in self.layers:
@@ -264,7 +265,14 @@ class MiniMaxTransformer:
             hidden = layer(hidden, int(start_pos), in_place=True)                # `hidden` is this call's own tensor
         if not keep_all_positions:
             hidden = hidden[:, -1:, :]
-        logits = self.lm_head(self.final_norm(hidden.contiguous())).float()
+        hidden = hidden.contiguous()
+        head = self.lm_head.tensor
+        if hidden.numel() // hidden.size(-1) <= 4 and int(head.row_start) == 0 and self._cuda is not None and hidden.is_cuda:
+            # decode: the final normalisation inside the vocabulary projection's launch
+            logits = self._cuda.gguf_quant_gemm_rmsnorm_forward(hidden, self.final_norm.weight, self.final_norm.eps, head.blocks, int(head.row_elems),
+                                                                int(head.type_id), self.lm_head._grid, out_dtype=self.lm_head.out_dtype).float()
+        else:
+            logits = self.lm_head(self.final_norm(hidden)).float()
         if return_next_token:
             best = logits.argmax(dim=-1)
             return best if keep_all_positions else best[:, -1]
