@@ -459,6 +459,45 @@ def test_few_row_calls_equal_the_prequantized_path(mod, type_name):
                 assert torch.equal(y, y_pre)
 
 
+@pytest.mark.parametrize("type_name", ["q4_k", "q5_k", "iq4_xs"])
+@pytest.mark.parametrize("n,k", [(17408, 5120), (1041, 1000), (16, 256), (300, 17408)])
+def test_two_rows_in_one_pass_equal_two_single_row_calls(mod, type_name, n, k):
+    """A call of two rows takes both rows through every block a wave fetches and unpacks (one launch, one pass over the weights,
+    whatever the matrix size): each row goes through the same slice image and the same products in the same order as in a call
+    of its own, so the results are the same bits; and they meet the float statement like the single-row call."""
+    rng = np.random.default_rng(n + k)
+    dev = torch.device("cuda:0")
+    tid = O.TYPE_IDS[type_name]
+    bpr = (k + 255) // 256
+    if type_name == "iq4_xs":
+        blocks = C.random_blocks(rng, type_name, n, bpr)
+    else:
+        blocks = rng.integers(0, 256, size=(n, bpr, 144 if type_name == "q4_k" else 176), dtype=np.uint8)
+        blocks[..., 0:2] = np.frombuffer(np.float16(0.01).tobytes(), dtype=np.uint8)
+        blocks[..., 2:4] = np.frombuffer(np.float16(0.005).tobytes(), dtype=np.uint8)
+    dblocks = torch.from_numpy(blocks).to(dev)
+    grid = codebooks.grid_tensor_for_type(tid).to(dev)
+    rows_w = rng.choice(n, size=min(n, 48), replace=False)
+    ref_w = O.dequant_rows(blocks[rows_w], type_name, k)
+    for dt in (torch.bfloat16, torch.float32, torch.float16):
+        x = torch.from_numpy(rng.standard_normal((2, k)).astype(np.float32)).to(dev).to(dt)
+        x[1] *= 37.0
+        print(f"case two rows {type_name} n={n} k={k} {dt}", flush=True)
+        y = mod.gguf_quant_gemm_forward(x, dblocks, k, tid, grid, out_dtype=torch.float32)
+        y0 = mod.gguf_quant_gemm_forward(x[0:1].contiguous(), dblocks, k, tid, grid, out_dtype=torch.float32)
+        y1 = mod.gguf_quant_gemm_forward(x[1:2].contiguous(), dblocks, k, tid, grid, out_dtype=torch.float32)
+        torch.cuda.synchronize()
+        assert tuple(y.shape) == (2, n)
+        assert torch.equal(y[0], y0[0]) and torch.equal(y[1], y1[0])
+        want = O.matmul_f(x.float().cpu().numpy(), ref_w)
+        got = y.cpu().numpy()[:, rows_w]
+        for r in range(2):
+            # (random blocks: scales and mins of every size cancel against each other, which magnifies the image's rounding)
+            assert O.rel_l2(got[r], want[r]) <= (1e-4 if dt == torch.bfloat16 else 1e-3), (dt, r, O.rel_l2(got[r], want[r]))
+        y16 = mod.gguf_quant_gemm_forward(x, dblocks, k, tid, grid)
+        assert torch.equal(y16, y.to(y16.dtype))
+
+
 @pytest.mark.parametrize("type_name", ["q4_k", "q5_k", "q2_k", "q6_k", "iq4_xs", "iq2_xxs", "iq1_m", "iq2_xs", "iq3_xxs"])
 def test_accumulate_adds_the_product_to_y(mod, type_name):
     """The residual form y += W x: equal to the plain operator's float32 product plus the old y, rounded once to y's type,
