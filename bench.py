@@ -580,8 +580,29 @@ def decode_pass(mod, dev) -> None:
         for i in range(24):
             mod.gguf_quant_gemm_forward(x, ring[i % len(ring)], 5120, tid, grid)
         del ring
+    # Q4_K 17408x5120 at two rows (the two-row form of the single-launch kernel) and one token through 8 of 128 Q4_K experts of
+    # 2048 -> 768 (gate / up launch, then the down projection with the routes as its waves); random valid blocks
+    def q4k_random(*lead):
+        b = rng.integers(0, 256, size=tuple(lead) + (144,), dtype=np.uint8)
+        b[..., 0:2] = np.frombuffer(np.float16(0.01).tobytes(), dtype=np.uint8)
+        b[..., 2:4] = np.frombuffer(np.float16(0.005).tobytes(), dtype=np.uint8)
+        return b
+    ring = ring_of(q4k_random(17408, 20), dev, 8)
+    x2 = torch.randn(2, 5120, device=dev, dtype=torch.bfloat16)
+    empty = torch.empty(0, dtype=torch.int8, device=dev)
+    for i in range(24):
+        mod.gguf_quant_gemm_forward(x2, ring[i % len(ring)], 5120, 3, empty)
+    del ring
+    ek, dk, ik = 128, 2048, 768
+    kw1, kw3, kw2 = (torch.from_numpy(q4k_random(*shape)).to(dev) for shape in ((ek, ik, dk // 256), (ek, ik, dk // 256), (ek, dk, ik // 256)))
+    xk = torch.randn(1, dk, device=dev, dtype=torch.bfloat16)
+    kwts = torch.full((8,), 0.125, device=dev)
+    for i in range(24):
+        ids = torch.from_numpy(rng.choice(ek, size=8, replace=False).astype(np.int64)).to(dev)
+        mod.gguf_moe_single_token_forward(xk, ids, kwts, kw1, kw3, kw2, 0.0)
     torch.cuda.synchronize()
-    print(json.dumps({"decode_pass": "q8_0 4096x4096 + 17408x5120, fp8 17408x5120, q2_k / q6_k / iq4_xs 17408x5120, 24 launches each"}))
+    print(json.dumps({"decode_pass": "q8_0 4096x4096 + 17408x5120, fp8 17408x5120, q2_k / q6_k / iq4_xs 17408x5120, q4_k 17408x5120 at two rows, "
+                                     "q4_k experts 128 x (2048 -> 768) top-8 one token; 24 launches each"}))
 
 
 def iq_pass(mod, dev) -> None:
