@@ -360,9 +360,10 @@ __device__ __forceinline__ void raw_to_float4(const RawX<X16>& r, int x_dtype, f
 // RSUM (the down projection of one token's routed experts): wave v is route v.  It takes ALL blocks of its own expert's 16 rows
 // against its own activation row, which it forms on the way as SiLU(min(gate, L)) * clamp(up, +-L) * route weight from the gate
 // (x) and up (x_up) products [routes, k]; the sum over the waves at the end is the sum over the routes, in route order.
-// ROW2 (dense calls of two rows): the wave multiplies every block it fetches and unpacks into both rows, one after the other
-// through the same LDS slot; grid row = the pair of rows.
-template <typename FMT, int ITERS, int DEPTH, bool X16, bool NORM, bool PLAIN = false, bool RSUM = false, bool ROW2 = false>
+// ROWS > 1 (dense calls of two to four rows): the wave multiplies every block it fetches and unpacks into all ROWS rows, one
+// after the other through the same LDS slot; one grid row.  The call's row count travels in round_f16 (no normalisation here):
+// rows past it repeat the last row and are not stored.
+template <typename FMT, int ITERS, int DEPTH, bool X16, bool NORM, bool PLAIN = false, bool RSUM = false, int ROWS = 1>
 __global__ __launch_bounds__(64 * kMaxWaves) void wave_image_matvec_kernel(
     const void* __restrict__ x, int x_dtype, int k, const WeightRoute route, const uint8_t* __restrict__ w, void* __restrict__ y,
     int y_dtype, int n, int bpr, const float* __restrict__ gamma, float eps, int round_f16, const int64_t* __restrict__ row_token, int x_broadcast) {
@@ -402,19 +403,25 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_image_matvec_kernel(
     }
     const int row = blockIdx.x * kRowsPerWg + col;
     const uint8_t* wrow = w + static_cast<size_t>(row < n ? row : 0) * bpr * FMT::kBlockBytes;
-    const size_t xoff = (PLAIN ? static_cast<size_t>(ROW2 ? 2 * blockIdx.y : blockIdx.y) : RSUM ? static_cast<size_t>(wave)
+    const size_t xoff = (PLAIN ? static_cast<size_t>(blockIdx.y) : RSUM ? static_cast<size_t>(wave)
                                : x_broadcast ? 0 : row_token ? static_cast<size_t>(row_token[blockIdx.y]) : static_cast<size_t>(blockIdx.y)) * k;
     const int bstep = RSUM ? 1 : waves;                                       // distance between a wave's blocks
     const float rw = RSUM ? route_w[__builtin_amdgcn_readfirstlane(wave)] : 1.0f;
 
     if (lane < 4) reinterpret_cast<uint32_t*>(slot + kSlotBytes)[lane] = 0;
-    float acc = 0.0f, acc_second = 0.0f;
+    float acc = 0.0f;
+    constexpr int kMore = ROWS > 1 ? ROWS - 1 : 1;                            // further rows of a ROWS call
+    const int total_rows = ROWS > 1 ? round_f16 : 1;
+    float acc_more[kMore];
+#pragma unroll
+    for (int j = 0; j < kMore; ++j) acc_more[j] = 0.0f;
     // NORM (the row passes through an RMS normalisation first, one pass of the loop below): the wave's slices of all its blocks
     // are requested at once, with the weights of the first blocks behind them; their squares are the wave's share of the row's
     // sum, the shares meet in LDS, and the slices are scaled as they are quantized.  No extra pass over the row, one barrier.
     constexpr int kHeldX = NORM ? ITERS : DEPTH;
     RawX<X16> raw[kHeldX];
-    RawX<X16> raw_up[(RSUM || ROW2) ? kHeldX : 1];                            // RSUM: the up products; ROW2: the second row
+    RawX<X16> raw_up[RSUM ? kHeldX : 1];                                       // RSUM: the up products
+    RawX<X16> raw_more[kMore][ROWS > 1 ? kHeldX : 1];                         // ROWS: the further rows' slices
     RawX<false> graw[NORM ? ITERS : 1];
     float rstd = 1.0f;
     for (int b0 = RSUM ? 0 : wave; b0 < bpr; b0 += bstep * ITERS) {
@@ -423,7 +430,11 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_image_matvec_kernel(
             const int b = b0 + it * bstep;
             request_raw4<X16>(raw[it % kHeldX], x, xoff, 256 * b + 4 * lane, b < bpr ? k : 0);
             if constexpr (RSUM) request_raw4<X16>(raw_up[it % kHeldX], x_up, xoff, 256 * b + 4 * lane, b < bpr ? k : 0);
-            if constexpr (ROW2) request_raw4<X16>(raw_up[it % kHeldX], x, xoff + k, 256 * b + 4 * lane, b < bpr ? k : 0);
+            if constexpr (ROWS > 1) {
+#pragma unroll
+                for (int j = 0; j < kMore; ++j)
+                    request_raw4<X16>(raw_more[j][it % kHeldX], x, xoff + static_cast<size_t>(min(j + 1, total_rows - 1)) * k, 256 * b + 4 * lane, b < bpr ? k : 0);
+            }
         };
         auto request_w = [&](int it) {
             const int b = b0 + it * bstep;
@@ -530,11 +541,13 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_image_matvec_kernel(
                 const float4 g2 = *reinterpret_cast<const float4*>(slot + 512 + 16 * ks);   // {xs0, sum0, xs1, sum1}
                 acc += FMT::combine(regs[it % DEPTH], ks, v0, v1, g2);
                 __builtin_amdgcn_wave_barrier();                            // the next block's slice overwrites the slot
-                if constexpr (ROW2) {
-                    // the second row's slice through the same slot, against the codes already unpacked
+                if constexpr (ROWS > 1) {
+#pragma unroll
+                  for (int j = 0; j < kMore; ++j) {
+                    // the next row's slice through the same slot, against the codes already unpacked
                     float u[4];
-                    if (k != 256 * bpr) settle_raw4<X16>(raw_up[it % kHeldX], 256 * b + 4 * lane, k);
-                    raw_to_float4<X16>(raw_up[it % kHeldX], x_dtype, u);
+                    if (k != 256 * bpr) settle_raw4<X16>(raw_more[j][it % kHeldX], 256 * b + 4 * lane, k);
+                    raw_to_float4<X16>(raw_more[j][it % kHeldX], x_dtype, u);
                     uint32_t qh2, ql2;
                     float scale2, sum4b;
                     quantize4_pow2(u, qh2, ql2, scale2, &sum4b);
@@ -556,8 +569,9 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_image_matvec_kernel(
                     const float w0 = static_cast<float>((c2.x << 8) + c2.y);
                     const float w1 = static_cast<float>((c2.z << 8) + c2.w);
                     const float4 h2 = *reinterpret_cast<const float4*>(slot + 512 + 16 * ks);
-                    acc_second += FMT::combine(regs[it % DEPTH], ks, w0, w1, h2);
+                    acc_more[j] += FMT::combine(regs[it % DEPTH], ks, w0, w1, h2);
                     __builtin_amdgcn_wave_barrier();
+                  }
                 }
             }
             if (it + DEPTH < ITERS) request(it + DEPTH);
@@ -565,12 +579,15 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_image_matvec_kernel(
     }
     acc = quad_rows_sum(acc);
     if (ks == 0) partial[col * kMaxWaves + wave] = acc;
-    if constexpr (ROW2) {
-        acc_second = quad_rows_sum(acc_second);
-        if (ks == 0) partial[(kRowsPerWg + col) * kMaxWaves + wave] = acc_second;    // (behind the first row's shares; the launcher sizes for it)
+    if constexpr (ROWS > 1) {
+#pragma unroll
+        for (int j = 0; j < kMore; ++j) {
+            const float more = quad_rows_sum(acc_more[j]);
+            if (ks == 0) partial[((j + 1) * kRowsPerWg + col) * kMaxWaves + wave] = more;   // (behind the first row's shares; the launcher sizes for it)
+        }
     }
     __syncthreads();
-    if (tid < (ROW2 ? 2 : 1) * kRowsPerWg) {   // the waves' shares in wave order, fetched together
+    if (tid < ROWS * kRowsPerWg) {            // the waves' shares in wave order, fetched together
         const float4 lo4 = *reinterpret_cast<const float4*>(partial + tid * kMaxWaves);
         const float4 hi4 = *reinterpret_cast<const float4*>(partial + tid * kMaxWaves + 4);
         const float p[kMaxWaves] = {lo4.x, lo4.y, lo4.z, lo4.w, hi4.x, hi4.y, hi4.z, hi4.w};
@@ -578,8 +595,8 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_image_matvec_kernel(
 #pragma unroll
         for (int v = 1; v < kMaxWaves; ++v) total = v < waves ? total + p[v] : total;
         const int out_row = blockIdx.x * kRowsPerWg + (tid & (kRowsPerWg - 1));
-        const size_t y_row = ROW2 ? 2 * static_cast<size_t>(blockIdx.y) + (tid >= kRowsPerWg ? 1 : 0) : static_cast<size_t>(blockIdx.y);
-        if (out_row < n) store_any(y, y_dtype, y_row * n + out_row, total);
+        const int y_row = ROWS > 1 ? tid / kRowsPerWg : static_cast<int>(blockIdx.y);
+        if (out_row < n && (ROWS == 1 || y_row < total_rows)) store_any(y, y_dtype, static_cast<size_t>(y_row) * n + out_row, total);
     }
 }
 
@@ -603,8 +620,8 @@ int launch_kernel(KERN kern, const ActRows& act, const WeightRoute& route, const
 
 template <typename KERN>
 int launch_wave_kernel(KERN kern, const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype,
-                       int rows, int n, int bpr, int waves, hipStream_t stream, bool two_rows = false) {
-    const size_t smem = static_cast<size_t>(waves) * (kSlotBytes + 16) + static_cast<size_t>((two_rows ? 2 : 1) * kMaxWaves * kRowsPerWg + waves) * sizeof(float);
+                       int rows, int n, int bpr, int waves, hipStream_t stream, int rows_per_pass = 1) {
+    const size_t smem = static_cast<size_t>(waves) * (kSlotBytes + 16) + static_cast<size_t>(rows_per_pass * kMaxWaves * kRowsPerWg + waves) * sizeof(float);
     int tallest = n;
     for (int m = 0; m < route.extra; ++m) tallest = tallest > route.more_n[m] ? tallest : route.more_n[m];
     dim3 grid((tallest + kRowsPerWg - 1) / kRowsPerWg, rows, 1 + route.extra);
@@ -638,14 +655,19 @@ int launch_wave(const ActRows& act, const WeightRoute& route, const uint8_t* w, 
     int waves, iters;
     int tiles = (n + kRowsPerWg - 1) / kRowsPerWg;
     for (int m = 0; m < route.extra; ++m) tiles += (route.more_n[m] + kRowsPerWg - 1) / kRowsPerWg;
-    split_blocks(bpr, tiles * rows, waves, iters);
-    if (NORM && waves * iters < bpr) return PLLM_ERR_UNSUPPORTED;             // the normalised form holds a wave's slices of the whole row
     const bool plain = !NORM && !routed(route) && route.extra == 0 && !act.row_token && !act.x_broadcast;
-    const bool pair = plain && rows == 2;                                     // both rows in one pass over the weights
+    const bool pair = plain && rows == 2, quad = plain && (rows == 3 || rows == 4);   // all rows in one pass over the weights
+    split_blocks(bpr, tiles * (pair || quad ? 1 : rows), waves, iters);       // (one grid row then: the single-row call's split, so the same bits per row)
+    if (NORM && waves * iters < bpr) return PLLM_ERR_UNSUPPORTED;             // the normalised form holds a wave's slices of the whole row
+    ActRows few = act;
+    few.round_f16 = rows;                                                     // (where these forms expect the row count)
 #define PLLM_CASE(I) case I: \
         if constexpr (!NORM) if (pair) \
-            return act.x_dtype == PLLM_F32 ? launch_wave_kernel(wave_image_matvec_kernel<FMT, I, wave_depth<FMT>(I, false), false, false, true, false, true>, act, route, w, y, y_dtype, 1, n, bpr, waves, stream, true) \
-                                           : launch_wave_kernel(wave_image_matvec_kernel<FMT, I, wave_depth<FMT>(I, false), true, false, true, false, true>, act, route, w, y, y_dtype, 1, n, bpr, waves, stream, true); \
+            return act.x_dtype == PLLM_F32 ? launch_wave_kernel(wave_image_matvec_kernel<FMT, I, wave_depth<FMT>(I, false), false, false, true, false, 2>, few, route, w, y, y_dtype, 1, n, bpr, waves, stream, 2) \
+                                           : launch_wave_kernel(wave_image_matvec_kernel<FMT, I, wave_depth<FMT>(I, false), true, false, true, false, 2>, few, route, w, y, y_dtype, 1, n, bpr, waves, stream, 2); \
+        if constexpr (!NORM) if (quad) \
+            return act.x_dtype == PLLM_F32 ? launch_wave_kernel(wave_image_matvec_kernel<FMT, I, (I < 2 ? I : 2), false, false, true, false, 4>, few, route, w, y, y_dtype, 1, n, bpr, waves, stream, 4) \
+                                           : launch_wave_kernel(wave_image_matvec_kernel<FMT, I, wave_depth<FMT>(I, false), true, false, true, false, 4>, few, route, w, y, y_dtype, 1, n, bpr, waves, stream, 4); \
         if constexpr (!NORM) if (plain) \
             return act.x_dtype == PLLM_F32 ? launch_wave_kernel(wave_image_matvec_kernel<FMT, I, wave_depth<FMT>(I, false), false, false, true>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream) \
                                            : launch_wave_kernel(wave_image_matvec_kernel<FMT, I, wave_depth<FMT>(I, true), true, false, true>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream); \
