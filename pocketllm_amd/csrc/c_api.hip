@@ -14,7 +14,7 @@ constexpr int64_t kGemmMinRows = 16;
 // From how many activation rows on the MFMA tile kernel serves a matmul.  The decode kernels read the matrix once per
 // activation row (from cache after the first), the tile kernel decodes it once for up to 64 rows at a fixed cost.  Measured
 // crossovers (us, decode kernel against tile kernel): at 17408x5120 Q4_K 5 rows (46.7 / 44), IQ1_M, IQ2_XS and IQ3_XXS 4 rows
-// (50 - 56 / 45), Q6_K 3 rows (88.6 at 4 rows / 56); at 5120x5120 Q4_K 12 rows (27.0 / 26.1), IQ1_M, IQ2_XS, IQ3_XXS 8 rows
+// (50 - 56 / 45), Q6_K 5 rows (30.7 at 4 rows in the few-row form of its kernel / 54); at 5120x5120 Q4_K 12 rows (27.0 / 26.1), IQ1_M, IQ2_XS, IQ3_XXS 8 rows
 // (27 - 30 / 28.5), Q6_K 5 rows (34.0 / 30.6); FP8 (one matvec per row) 3 rows (34.4 at 2 rows / 42) and 5 rows (22.6 at 4 rows / 24.1).
 enum class RowClass { kKQuant, kCodebook, kQ6K, kFp8 };
 
@@ -24,7 +24,7 @@ static int64_t tile_gemm_min_rows(RowClass cls, int64_t weights) {
     switch (cls) {
         case RowClass::kKQuant: return size == 2 ? 5 : 12;
         case RowClass::kCodebook: return size == 2 ? 4 : 8;
-        case RowClass::kQ6K: return size == 2 ? 3 : 5;
+        case RowClass::kQ6K: return 5;        // (up to four rows: the single-launch kernel's few-row form, 30.7 us at 17408x5120 and four rows against 54.3 on the tiles)
         case RowClass::kFp8: return size == 2 ? 3 : 5;
     }
     return kGemmMinRows;

@@ -793,7 +793,8 @@ struct WaveQ6K {
 // squares are its share of the row's sum, the shares meet in LDS behind one barrier and the slices are scaled by rstd * gamma
 // as they are quantized.
 // RSUM: as in wave_image_matvec_kernel (wave = route of one token's experts, SwiGLU formed on the way, ordered sum at the end).
-template <typename FMT, int ITERS, int DEPTH, bool X16, bool PLAIN = false, bool NORM = false, bool RSUM = false>
+// ROWS > 1: as in wave_image_matvec_kernel (dense calls of two to four rows in one pass over the weights; the row count in round_f16).
+template <typename FMT, int ITERS, int DEPTH, bool X16, bool PLAIN = false, bool NORM = false, bool RSUM = false, int ROWS = 1>
 __global__ __launch_bounds__(64 * kMaxWaves) void wave_groups16_matvec_kernel(
     const void* __restrict__ x, int x_dtype, int k, const WeightRoute route, const uint8_t* __restrict__ w, void* __restrict__ y,
     int y_dtype, int n, int bpr, const int64_t* __restrict__ row_token, int x_broadcast, const float* __restrict__ gamma, float eps, int round_f16) {
@@ -840,17 +841,28 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_groups16_matvec_kernel(
 
     if (lane < 4) reinterpret_cast<uint32_t*>(slot + kQ2SlotBytes)[lane] = 0;
     float acc = 0.0f;
+    constexpr int kMore = ROWS > 1 ? ROWS - 1 : 1;                            // further rows of a ROWS call
+    const int total_rows = ROWS > 1 ? round_f16 : 1;
+    float acc_more[kMore];
+#pragma unroll
+    for (int j = 0; j < kMore; ++j) acc_more[j] = 0.0f;
     constexpr int kHeldX = NORM ? ITERS : DEPTH;
     float rstd = 1.0f;
     for (int b0 = RSUM ? 0 : wave; b0 < bpr; b0 += bstep * ITERS) {
         RawX<X16> raw[kHeldX];
         RawX<X16> raw_up[RSUM ? kHeldX : 1];
+        RawX<X16> raw_more[kMore][ROWS > 1 ? kHeldX : 1];
         RawX<false> graw[NORM ? ITERS : 1];
         typename FMT::Regs regs[DEPTH];
         auto request_x = [&](int it) {
             const int b = b0 + it * bstep;
             request_raw4<X16>(raw[it % kHeldX], x, xoff, 256 * b + 4 * lane, b < bpr ? k : 0);
             if constexpr (RSUM) request_raw4<X16>(raw_up[it % kHeldX], x_up, xoff, 256 * b + 4 * lane, b < bpr ? k : 0);
+            if constexpr (ROWS > 1) {
+#pragma unroll
+                for (int j = 0; j < kMore; ++j)
+                    request_raw4<X16>(raw_more[j][it % kHeldX], x, xoff + static_cast<size_t>(min(j + 1, total_rows - 1)) * k, 256 * b + 4 * lane, b < bpr ? k : 0);
+            }
         };
         auto request_w = [&](int it) {
             const int b = b0 + it * bstep;
@@ -935,9 +947,11 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_groups16_matvec_kernel(
                 __builtin_amdgcn_wave_barrier();                            // LDS serves a wave's requests in order
                 const typename FMT::Regs& r = regs[it % DEPTH];
                 v4i ch = {0, 0, 0, 0}, cl = {0, 0, 0, 0};
+                uint4 kept[ROWS > 1 ? 4 : 1];                                 // the unpacked codes, for the further rows
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
                     const uint4 bw = FMT::codes(r, t, ks);
+                    if constexpr (ROWS > 1) kept[t] = bw;
                     const int off = (mine && t == my_t) ? 16 * col : kQ2SlotBytes;
                     const uint4 ah = *reinterpret_cast<const uint4*>(slot + off);
                     const uint4 al = *reinterpret_cast<const uint4*>(slot + off + ((mine && t == my_t) ? 256 : 0));
@@ -952,6 +966,43 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_groups16_matvec_kernel(
                 const float smv[4] = {s16.x, s16.y, s16.z, s16.w};
                 acc += FMT::finish(r, vv, xsv, smv);
                 __builtin_amdgcn_wave_barrier();                            // the next block's slice overwrites the slot
+                if constexpr (ROWS > 1) {
+#pragma unroll
+                  for (int j = 0; j < kMore; ++j) {
+                    // the next row's slice through the same slot, against the codes already unpacked
+                    float u[4];
+                    if (k != 256 * bpr) settle_raw4<X16>(raw_more[j][it % kHeldX], 256 * b + 4 * lane, k);
+                    raw_to_float4<X16>(raw_more[j][it % kHeldX], x_dtype, u);
+                    uint32_t qh2, ql2;
+                    float scale2, sum4b;
+                    quantize4_pow2(u, qh2, ql2, scale2, &sum4b);
+                    reinterpret_cast<uint32_t*>(slot)[lane] = qh2;
+                    reinterpret_cast<uint32_t*>(slot + 256)[lane] = ql2;
+                    const float sum_b = group_sum<4>(sum4b);
+                    const float sum32_b = sum_b + butterfly_peer<4>(sum_b);
+                    if ((lane & 7) == 0) reinterpret_cast<float2*>(slot + 512)[lane >> 3] = make_float2(scale2, sum32_b);
+                    if ((lane & 3) == 0) reinterpret_cast<float*>(slot + kSlotBytes)[lane >> 2] = sum_b;
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                    __builtin_amdgcn_wave_barrier();
+                    v4i ch2 = {0, 0, 0, 0}, cl2 = {0, 0, 0, 0};
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        const int off = (mine && t == my_t) ? 16 * col : kQ2SlotBytes;
+                        const uint4 ah = *reinterpret_cast<const uint4*>(slot + off);
+                        const uint4 al = *reinterpret_cast<const uint4*>(slot + off + ((mine && t == my_t) ? 256 : 0));
+                        ch2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(as_v4i(ah), as_v4i(kept[t]), ch2, 0, 0, 0);
+                        cl2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(as_v4i(al), as_v4i(kept[t]), cl2, 0, 0, 0);
+                    }
+                    const float4 g2b = *reinterpret_cast<const float4*>(slot + 512 + 16 * ks);
+                    const float4 s16b = *reinterpret_cast<const float4*>(slot + kSlotBytes + 16 * ks);
+                    const float vvb[4] = {static_cast<float>((ch2.x << 8) + cl2.x), static_cast<float>((ch2.y << 8) + cl2.y),
+                                          static_cast<float>((ch2.z << 8) + cl2.z), static_cast<float>((ch2.w << 8) + cl2.w)};
+                    const float xsvb[4] = {g2b.x, g2b.x, g2b.z, g2b.z};
+                    const float smvb[4] = {s16b.x, s16b.y, s16b.z, s16b.w};
+                    acc_more[j] += FMT::finish(r, vvb, xsvb, smvb);
+                    __builtin_amdgcn_wave_barrier();
+                  }
+                }
             }
             if (it + DEPTH < ITERS) {
                 if constexpr (!NORM) request_x(it + DEPTH);
@@ -963,23 +1014,31 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_groups16_matvec_kernel(
     }
     acc = quad_rows_sum(acc);
     if (ks == 0) partial[col * kMaxWaves + wave] = acc;
+    if constexpr (ROWS > 1) {
+#pragma unroll
+        for (int j = 0; j < kMore; ++j) {
+            const float more = quad_rows_sum(acc_more[j]);
+            if (ks == 0) partial[((j + 1) * kRowsPerWg + col) * kMaxWaves + wave] = more;   // (behind the first row's shares; the launcher sizes for it)
+        }
+    }
     __syncthreads();
-    if (tid < kRowsPerWg) {                  // the waves' shares in wave order, fetched together
+    if (tid < ROWS * kRowsPerWg) {            // the waves' shares in wave order, fetched together
         const float4 lo4 = *reinterpret_cast<const float4*>(partial + tid * kMaxWaves);
         const float4 hi4 = *reinterpret_cast<const float4*>(partial + tid * kMaxWaves + 4);
         const float p[kMaxWaves] = {lo4.x, lo4.y, lo4.z, lo4.w, hi4.x, hi4.y, hi4.z, hi4.w};
         float total = p[0];
 #pragma unroll
         for (int v = 1; v < kMaxWaves; ++v) total = v < waves ? total + p[v] : total;
-        const int out_row = blockIdx.x * kRowsPerWg + tid;
-        if (out_row < n) store_any(y, y_dtype, static_cast<size_t>(blockIdx.y) * n + out_row, total);
+        const int out_row = blockIdx.x * kRowsPerWg + (tid & (kRowsPerWg - 1));
+        const int y_row = ROWS > 1 ? tid / kRowsPerWg : static_cast<int>(blockIdx.y);
+        if (out_row < n && (ROWS == 1 || y_row < total_rows)) store_any(y, y_dtype, static_cast<size_t>(y_row) * n + out_row, total);
     }
 }
 
 template <typename KERN>
 int launch_q2k_kernel(KERN kern, const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype,
-                      int rows, int n, int bpr, int waves, hipStream_t stream) {
-    const size_t smem = static_cast<size_t>(waves) * (kQ2SlotBytes + 16) + static_cast<size_t>(kMaxWaves * kRowsPerWg + waves) * sizeof(float);
+                      int rows, int n, int bpr, int waves, hipStream_t stream, int rows_per_pass = 1) {
+    const size_t smem = static_cast<size_t>(waves) * (kQ2SlotBytes + 16) + static_cast<size_t>(rows_per_pass * kMaxWaves * kRowsPerWg + waves) * sizeof(float);
     int tallest = n;
     for (int m = 0; m < route.extra; ++m) tallest = tallest > route.more_n[m] ? tallest : route.more_n[m];
     dim3 grid((tallest + kRowsPerWg - 1) / kRowsPerWg, rows, 1 + route.extra);
@@ -1055,12 +1114,21 @@ int launch_groups16(const ActRows& act, const WeightRoute& route, const uint8_t*
     int waves, iters;
     int tiles = (n + kRowsPerWg - 1) / kRowsPerWg;
     for (int m = 0; m < route.extra; ++m) tiles += (route.more_n[m] + kRowsPerWg - 1) / kRowsPerWg;
-    split_blocks(bpr, tiles * rows, waves, iters);
-    if (act.gamma && waves * iters < bpr) return PLLM_ERR_UNSUPPORTED;        // the normalised form holds a wave's slices of the whole row
-    constexpr int kMaxDepth = 2;            // blocks in flight per wave: five waves per SIMD fit with 2 (Q6_K with 2, 3, 4 and 5 ran within 3 % of each other, Q2_K 14.6 us with 2 against 15.2 with 5)
     const bool plain = !routed(route) && route.extra == 0 && !act.row_token && !act.x_broadcast;
+    const bool pair = plain && !act.gamma && rows == 2, quad = plain && !act.gamma && (rows == 3 || rows == 4);   // all rows in one pass over the weights
+    split_blocks(bpr, tiles * (pair || quad ? 1 : rows), waves, iters);       // (one grid row then: the single-row call's split, so the same bits per row)
+    if (act.gamma && waves * iters < bpr) return PLLM_ERR_UNSUPPORTED;        // the normalised form holds a wave's slices of the whole row
+    ActRows few = act;
+    few.round_f16 = rows;                                                     // (where the few-row forms expect the row count)
+    constexpr int kMaxDepth = 2;            // blocks in flight per wave: five waves per SIMD fit with 2 (Q6_K with 2, 3, 4 and 5 ran within 3 % of each other, Q2_K 14.6 us with 2 against 15.2 with 5)
 #define PLLM_CASE(I) case I: { \
         constexpr int D = I < kMaxDepth ? I : kMaxDepth; \
+        if (pair) \
+            return act.x_dtype == PLLM_F32 ? launch_q2k_kernel(wave_groups16_matvec_kernel<FMT, I, D, false, true, false, false, 2>, few, route, w, y, y_dtype, 1, n, bpr, waves, stream, 2) \
+                                           : launch_q2k_kernel(wave_groups16_matvec_kernel<FMT, I, D, true, true, false, false, 2>, few, route, w, y, y_dtype, 1, n, bpr, waves, stream, 2); \
+        if (quad) \
+            return act.x_dtype == PLLM_F32 ? launch_q2k_kernel(wave_groups16_matvec_kernel<FMT, I, D, false, true, false, false, 4>, few, route, w, y, y_dtype, 1, n, bpr, waves, stream, 4) \
+                                           : launch_q2k_kernel(wave_groups16_matvec_kernel<FMT, I, D, true, true, false, false, 4>, few, route, w, y, y_dtype, 1, n, bpr, waves, stream, 4); \
         if (act.gamma) \
             return act.x_dtype == PLLM_F32 ? launch_q2k_kernel(wave_groups16_matvec_kernel<FMT, I, D, false, false, true>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream) \
                                            : launch_q2k_kernel(wave_groups16_matvec_kernel<FMT, I, D, true, false, true>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream); \

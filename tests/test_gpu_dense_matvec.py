@@ -459,7 +459,7 @@ def test_few_row_calls_equal_the_prequantized_path(mod, type_name):
                 assert torch.equal(y, y_pre)
 
 
-@pytest.mark.parametrize("type_name", ["q4_k", "q5_k", "iq4_xs"])
+@pytest.mark.parametrize("type_name", ["q4_k", "q5_k", "iq4_xs", "q6_k", "q2_k"])
 @pytest.mark.parametrize("n,k", [(17408, 5120), (1041, 1000), (16, 256), (300, 17408), (5120, 5120)])
 def test_two_to_four_rows_in_one_pass_equal_single_row_calls(mod, type_name, n, k):
     """A call of two to four rows takes all its rows through every block a wave fetches and unpacks (one launch, one pass over
@@ -471,8 +471,12 @@ def test_two_to_four_rows_in_one_pass_equal_single_row_calls(mod, type_name, n, 
     dev = torch.device("cuda:0")
     tid = O.TYPE_IDS[type_name]
     bpr = (k + 255) // 256
-    if type_name == "iq4_xs":
+    if type_name in ("iq4_xs", "q6_k"):
         blocks = C.random_blocks(rng, type_name, n, bpr)
+    elif type_name == "q2_k":
+        blocks = rng.integers(0, 256, size=(n, bpr, 84), dtype=np.uint8)
+        blocks[..., 80:82] = np.frombuffer(np.float16(0.01).tobytes(), dtype=np.uint8)
+        blocks[..., 82:84] = np.frombuffer(np.float16(0.005).tobytes(), dtype=np.uint8)
     else:
         blocks = rng.integers(0, 256, size=(n, bpr, 144 if type_name == "q4_k" else 176), dtype=np.uint8)
         blocks[..., 0:2] = np.frombuffer(np.float16(0.01).tobytes(), dtype=np.uint8)
