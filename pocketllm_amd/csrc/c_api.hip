@@ -16,13 +16,14 @@ constexpr int64_t kGemmMinRows = 16;
 // crossovers (us, decode kernel against tile kernel): at 17408x5120 Q4_K 5 rows (46.7 / 44), IQ1_M, IQ2_XS and IQ3_XXS 4 rows
 // (50 - 56 / 45), Q6_K 5 rows (30.7 at 4 rows in the few-row form of its kernel / 54); at 5120x5120 Q4_K 12 rows (27.0 / 26.1), IQ1_M, IQ2_XS, IQ3_XXS 8 rows
 // (27 - 30 / 28.5), Q6_K 5 rows (34.0 / 30.6); FP8 (one matvec per row) 3 rows (34.4 at 2 rows / 42) and 5 rows (22.6 at 4 rows / 24.1).
-enum class RowClass { kKQuant, kCodebook, kQ6K, kFp8 };
+enum class RowClass { kKQuant, kWave8, kCodebook, kQ6K, kFp8 };
 
 static int64_t tile_gemm_min_rows(RowClass cls, int64_t weights) {
     const int size = weights >= (int64_t{64} << 20) ? 2 : (weights >= (int64_t{16} << 20) ? 1 : 0);
     if (size == 0) return kGemmMinRows;
     switch (cls) {
         case RowClass::kKQuant: return size == 2 ? 5 : 12;
+        case RowClass::kWave8: return size == 2 ? 9 : 12;   // (up to eight rows: the few-row form of the single-launch kernel, Q4_K 17408x5120 at 5 - 8 float32 rows 34 - 36 us against 50 on the tiles)
         case RowClass::kCodebook: return size == 2 ? 4 : 8;
         case RowClass::kQ6K: return 5;        // (up to four rows: the single-launch kernel's few-row form, 30.7 us at 17408x5120 and four rows against 54.3 on the tiles)
         case RowClass::kFp8: return size == 2 ? 3 : 5;
@@ -33,6 +34,7 @@ static int64_t tile_gemm_min_rows(RowClass cls, int64_t weights) {
 static bool gguf_uses_tile_gemm(int type_id, int64_t rows, int64_t n, int64_t blocks_per_row) {
     if (!pllm::gemm_f16_supports(type_id)) return false;
     const RowClass cls = type_id == PLLM_TYPE_Q6_K ? RowClass::kQ6K
+                         : (type_id == PLLM_TYPE_Q4_K || type_id == PLLM_TYPE_Q5_K || type_id == PLLM_TYPE_IQ4_XS) ? RowClass::kWave8
                          : (type_id == PLLM_TYPE_IQ1_M || type_id == PLLM_TYPE_IQ2_XS || type_id == PLLM_TYPE_IQ3_XXS) ? RowClass::kCodebook
                                                                                                                        : RowClass::kKQuant;
     return rows >= tile_gemm_min_rows(cls, n * blocks_per_row * 256);
@@ -105,10 +107,12 @@ size_t pllm_q8_0_gemm_workspace_bytes(int64_t rows, int64_t k, int64_t n, int64_
 // block a wave fetches, one pass over the weights for all of them (Q4_K 17408x5120, float32 rows, us at 3 / 4 rows: 20.7 / 20.8
 // against 27.8 / 28.6 with the pre-pass and the kernel that reads prepared images); the other formats run one grid row per row.
 constexpr int64_t kInKernelQuantMaxRows = 4;
+constexpr int64_t kInKernelQuantMaxRowsWave8 = 8;   // Q4_K, Q5_K, IQ4_XS: up to eight rows through every block a wave fetches
 
 static bool quantizes_in_kernel(int type_id, int64_t rows, int64_t n, int64_t bpr) {
-    if (rows > kInKernelQuantMaxRows) return false;
     (void)n; (void)bpr;
+    const bool wave8 = type_id == PLLM_TYPE_Q4_K || type_id == PLLM_TYPE_Q5_K || type_id == PLLM_TYPE_IQ4_XS;
+    if (rows > (wave8 ? kInKernelQuantMaxRowsWave8 : kInKernelQuantMaxRows)) return false;
     return pllm_gguf_block_bytes(type_id) != 0;
 }
 

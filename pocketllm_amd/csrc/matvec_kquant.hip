@@ -587,15 +587,16 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_image_matvec_kernel(
         }
     }
     __syncthreads();
-    if (tid < ROWS * kRowsPerWg) {            // the waves' shares in wave order, fetched together
-        const float4 lo4 = *reinterpret_cast<const float4*>(partial + tid * kMaxWaves);
-        const float4 hi4 = *reinterpret_cast<const float4*>(partial + tid * kMaxWaves + 4);
+    // the waves' shares in wave order, fetched together (a workgroup of one wave walks the rows of an eight-row call in two steps)
+    for (int e = tid; e < ROWS * kRowsPerWg; e += (ROWS * kRowsPerWg > 64 ? 64 * waves : ROWS * kRowsPerWg)) {
+        const float4 lo4 = *reinterpret_cast<const float4*>(partial + e * kMaxWaves);
+        const float4 hi4 = *reinterpret_cast<const float4*>(partial + e * kMaxWaves + 4);
         const float p[kMaxWaves] = {lo4.x, lo4.y, lo4.z, lo4.w, hi4.x, hi4.y, hi4.z, hi4.w};
         float total = p[0];
 #pragma unroll
         for (int v = 1; v < kMaxWaves; ++v) total = v < waves ? total + p[v] : total;
-        const int out_row = blockIdx.x * kRowsPerWg + (tid & (kRowsPerWg - 1));
-        const int y_row = ROWS > 1 ? tid / kRowsPerWg : static_cast<int>(blockIdx.y);
+        const int out_row = blockIdx.x * kRowsPerWg + (e & (kRowsPerWg - 1));
+        const int y_row = ROWS > 1 ? e / kRowsPerWg : static_cast<int>(blockIdx.y);
         if (out_row < n && (ROWS == 1 || y_row < total_rows)) store_any(y, y_dtype, static_cast<size_t>(y_row) * n + out_row, total);
     }
 }
@@ -656,8 +657,8 @@ int launch_wave(const ActRows& act, const WeightRoute& route, const uint8_t* w, 
     int tiles = (n + kRowsPerWg - 1) / kRowsPerWg;
     for (int m = 0; m < route.extra; ++m) tiles += (route.more_n[m] + kRowsPerWg - 1) / kRowsPerWg;
     const bool plain = !NORM && !routed(route) && route.extra == 0 && !act.row_token && !act.x_broadcast;
-    const bool pair = plain && rows == 2, quad = plain && (rows == 3 || rows == 4);   // all rows in one pass over the weights
-    split_blocks(bpr, tiles * (pair || quad ? 1 : rows), waves, iters);       // (one grid row then: the single-row call's split, so the same bits per row)
+    const bool pair = plain && rows == 2, quad = plain && (rows == 3 || rows == 4), oct = plain && rows >= 5 && rows <= 8;   // all rows in one pass over the weights
+    split_blocks(bpr, tiles * (pair || quad || oct ? 1 : rows), waves, iters);   // (one grid row then: the single-row call's split, so the same bits per row)
     if (NORM && waves * iters < bpr) return PLLM_ERR_UNSUPPORTED;             // the normalised form holds a wave's slices of the whole row
     ActRows few = act;
     few.round_f16 = rows;                                                     // (where these forms expect the row count)
@@ -668,6 +669,9 @@ int launch_wave(const ActRows& act, const WeightRoute& route, const uint8_t* w, 
         if constexpr (!NORM) if (quad) \
             return act.x_dtype == PLLM_F32 ? launch_wave_kernel(wave_image_matvec_kernel<FMT, I, (I < 2 ? I : 2), false, false, true, false, 4>, few, route, w, y, y_dtype, 1, n, bpr, waves, stream, 4) \
                                            : launch_wave_kernel(wave_image_matvec_kernel<FMT, I, wave_depth<FMT>(I, false), true, false, true, false, 4>, few, route, w, y, y_dtype, 1, n, bpr, waves, stream, 4); \
+        if constexpr (!NORM) if (oct) \
+            return act.x_dtype == PLLM_F32 ? launch_wave_kernel(wave_image_matvec_kernel<FMT, I, 1, false, false, true, false, 8>, few, route, w, y, y_dtype, 1, n, bpr, waves, stream, 8) \
+                                           : launch_wave_kernel(wave_image_matvec_kernel<FMT, I, (I < 2 ? I : 2), true, false, true, false, 8>, few, route, w, y, y_dtype, 1, n, bpr, waves, stream, 8); \
         if constexpr (!NORM) if (plain) \
             return act.x_dtype == PLLM_F32 ? launch_wave_kernel(wave_image_matvec_kernel<FMT, I, wave_depth<FMT>(I, false), false, false, true>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream) \
                                            : launch_wave_kernel(wave_image_matvec_kernel<FMT, I, wave_depth<FMT>(I, true), true, false, true>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream); \
@@ -1116,6 +1120,7 @@ int launch_groups16(const ActRows& act, const WeightRoute& route, const uint8_t*
     for (int m = 0; m < route.extra; ++m) tiles += (route.more_n[m] + kRowsPerWg - 1) / kRowsPerWg;
     const bool plain = !routed(route) && route.extra == 0 && !act.row_token && !act.x_broadcast;
     const bool pair = plain && !act.gamma && rows == 2, quad = plain && !act.gamma && (rows == 3 || rows == 4);   // all rows in one pass over the weights
+    // (eight rows in this form lost to one grid row per row: Q2_K 5120x5120 22.2 against 16.6 us at five rows)
     split_blocks(bpr, tiles * (pair || quad ? 1 : rows), waves, iters);       // (one grid row then: the single-row call's split, so the same bits per row)
     if (act.gamma && waves * iters < bpr) return PLLM_ERR_UNSUPPORTED;        // the normalised form holds a wave's slices of the whole row
     ActRows few = act;
