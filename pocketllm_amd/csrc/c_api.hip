@@ -17,6 +17,9 @@ constexpr int64_t kGemmMinRows = 16;
 // (50 - 56 / 45), Q6_K 5 rows (30.7 at 4 rows in the few-row form of its kernel / 54); at 5120x5120 Q4_K 12 rows (27.0 / 26.1), IQ1_M, IQ2_XS, IQ3_XXS 8 rows
 // (27 - 30 / 28.5), Q6_K 5 rows (34.0 / 30.6); FP8 (one matvec per row) 3 rows (34.4 at 2 rows / 42) and 5 rows (22.6 at 4 rows / 24.1).
 enum class RowClass { kKQuant, kWave8, kCodebook, kQ6K, kFp8 };
+// Q6_K, five to eight rows: the eight-row form of the single-launch kernel while the matrix is this small (5120x5120 23.7 us against 29.4 - 37.6 on
+// the tiles; level at 17408x5120, 301 against 256 us at 200064x3072)
+constexpr int64_t kQ6KEightRowMaxWeights = int64_t{48} << 20;
 
 static int64_t tile_gemm_min_rows(RowClass cls, int64_t weights) {
     const int size = weights >= (int64_t{64} << 20) ? 2 : (weights >= (int64_t{16} << 20) ? 1 : 0);
@@ -25,7 +28,7 @@ static int64_t tile_gemm_min_rows(RowClass cls, int64_t weights) {
         case RowClass::kKQuant: return size == 2 ? 5 : 12;
         case RowClass::kWave8: return size == 2 ? 9 : 12;   // (up to eight rows: the few-row form of the single-launch kernel, Q4_K 17408x5120 at 5 - 8 float32 rows 34 - 36 us against 50 on the tiles)
         case RowClass::kCodebook: return size == 2 ? 4 : 8;
-        case RowClass::kQ6K: return 5;        // (up to four rows: the single-launch kernel's few-row form, 30.7 us at 17408x5120 and four rows against 54.3 on the tiles)
+        case RowClass::kQ6K: return weights <= kQ6KEightRowMaxWeights ? 9 : 5;        // (up to four rows: the single-launch kernel's few-row form, 30.7 us at 17408x5120 and four rows against 54.3 on the tiles)
         case RowClass::kFp8: return size == 2 ? 3 : 5;
     }
     return kGemmMinRows;
@@ -110,8 +113,8 @@ constexpr int64_t kInKernelQuantMaxRows = 4;
 constexpr int64_t kInKernelQuantMaxRowsWave8 = 8;   // Q4_K, Q5_K, IQ4_XS: up to eight rows through every block a wave fetches
 
 static bool quantizes_in_kernel(int type_id, int64_t rows, int64_t n, int64_t bpr) {
-    (void)n; (void)bpr;
-    const bool wave8 = type_id == PLLM_TYPE_Q4_K || type_id == PLLM_TYPE_Q5_K || type_id == PLLM_TYPE_IQ4_XS;
+    const bool wave8 = type_id == PLLM_TYPE_Q4_K || type_id == PLLM_TYPE_Q5_K || type_id == PLLM_TYPE_IQ4_XS ||
+                       (type_id == PLLM_TYPE_Q6_K && n * bpr * 256 <= kQ6KEightRowMaxWeights);
     if (rows > (wave8 ? kInKernelQuantMaxRowsWave8 : kInKernelQuantMaxRows)) return false;
     return pllm_gguf_block_bytes(type_id) != 0;
 }

@@ -1026,15 +1026,16 @@ __global__ __launch_bounds__(64 * kMaxWaves) void wave_groups16_matvec_kernel(
         }
     }
     __syncthreads();
-    if (tid < ROWS * kRowsPerWg) {            // the waves' shares in wave order, fetched together
-        const float4 lo4 = *reinterpret_cast<const float4*>(partial + tid * kMaxWaves);
-        const float4 hi4 = *reinterpret_cast<const float4*>(partial + tid * kMaxWaves + 4);
+    // the waves' shares in wave order, fetched together (more than 64 results only in the eight-row form, whose workgroup may be one wave)
+    for (int e = tid; e < ROWS * kRowsPerWg; e += (ROWS * kRowsPerWg > 64 ? 64 * waves : ROWS * kRowsPerWg)) {
+        const float4 lo4 = *reinterpret_cast<const float4*>(partial + e * kMaxWaves);
+        const float4 hi4 = *reinterpret_cast<const float4*>(partial + e * kMaxWaves + 4);
         const float p[kMaxWaves] = {lo4.x, lo4.y, lo4.z, lo4.w, hi4.x, hi4.y, hi4.z, hi4.w};
         float total = p[0];
 #pragma unroll
         for (int v = 1; v < kMaxWaves; ++v) total = v < waves ? total + p[v] : total;
-        const int out_row = blockIdx.x * kRowsPerWg + (tid & (kRowsPerWg - 1));
-        const int y_row = ROWS > 1 ? tid / kRowsPerWg : static_cast<int>(blockIdx.y);
+        const int out_row = blockIdx.x * kRowsPerWg + (e & (kRowsPerWg - 1));
+        const int y_row = ROWS > 1 ? e / kRowsPerWg : static_cast<int>(blockIdx.y);
         if (out_row < n && (ROWS == 1 || y_row < total_rows)) store_any(y, y_dtype, static_cast<size_t>(y_row) * n + out_row, total);
     }
 }
@@ -1120,12 +1121,17 @@ int launch_groups16(const ActRows& act, const WeightRoute& route, const uint8_t*
     for (int m = 0; m < route.extra; ++m) tiles += (route.more_n[m] + kRowsPerWg - 1) / kRowsPerWg;
     const bool plain = !routed(route) && route.extra == 0 && !act.row_token && !act.x_broadcast;
     const bool pair = plain && !act.gamma && rows == 2, quad = plain && !act.gamma && (rows == 3 || rows == 4);   // all rows in one pass over the weights
-    // (eight rows in this form lost to one grid row per row: Q2_K 5120x5120 22.2 against 16.6 us at five rows)
-    split_blocks(bpr, tiles * (pair || quad ? 1 : rows), waves, iters);       // (one grid row then: the single-row call's split, so the same bits per row)
+    // eight rows for Q6_K only, one block in flight per wave: the caller sends these while the matrix is small (5120x5120 23.7 us against
+    // 29.4 on the tiles); for Q2_K eight rows lost to one grid row per row (5120x5120 22.2 against 16.6 us at five rows)
+    const bool oct = plain && !act.gamma && rows >= 5 && rows <= 8 && FMT::kBlockBytes == 210;
+    split_blocks(bpr, tiles * (pair || quad || oct ? 1 : rows), waves, iters);       // (one grid row then: the single-row call's split, so the same bits per row)
     if (act.gamma && waves * iters < bpr) return PLLM_ERR_UNSUPPORTED;        // the normalised form holds a wave's slices of the whole row
     ActRows few = act;
     few.round_f16 = rows;                                                     // (where the few-row forms expect the row count)
     constexpr int kMaxDepth = 2;            // blocks in flight per wave: five waves per SIMD fit with 2 (Q6_K with 2, 3, 4 and 5 ran within 3 % of each other, Q2_K 14.6 us with 2 against 15.2 with 5)
+#define PLLM_OCT_CASE(I) if constexpr (FMT::kBlockBytes == 210) if (oct) \
+            return act.x_dtype == PLLM_F32 ? launch_q2k_kernel(wave_groups16_matvec_kernel<FMT, I, 1, false, true, false, false, 8>, few, route, w, y, y_dtype, 1, n, bpr, waves, stream, 8) \
+                                           : launch_q2k_kernel(wave_groups16_matvec_kernel<FMT, I, 1, true, true, false, false, 8>, few, route, w, y, y_dtype, 1, n, bpr, waves, stream, 8);
 #define PLLM_CASE(I) case I: { \
         constexpr int D = I < kMaxDepth ? I : kMaxDepth; \
         if (pair) \
@@ -1134,6 +1140,7 @@ int launch_groups16(const ActRows& act, const WeightRoute& route, const uint8_t*
         if (quad) \
             return act.x_dtype == PLLM_F32 ? launch_q2k_kernel(wave_groups16_matvec_kernel<FMT, I, D, false, true, false, false, 4>, few, route, w, y, y_dtype, 1, n, bpr, waves, stream, 4) \
                                            : launch_q2k_kernel(wave_groups16_matvec_kernel<FMT, I, D, true, true, false, false, 4>, few, route, w, y, y_dtype, 1, n, bpr, waves, stream, 4); \
+        PLLM_OCT_CASE(I) \
         if (act.gamma) \
             return act.x_dtype == PLLM_F32 ? launch_q2k_kernel(wave_groups16_matvec_kernel<FMT, I, D, false, false, true>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream) \
                                            : launch_q2k_kernel(wave_groups16_matvec_kernel<FMT, I, D, true, false, true>, act, route, w, y, y_dtype, rows, n, bpr, waves, stream); \
@@ -1147,6 +1154,7 @@ int launch_groups16(const ActRows& act, const WeightRoute& route, const uint8_t*
         default: PLLM_CASE(8)
     }
 #undef PLLM_CASE
+#undef PLLM_OCT_CASE
 }
 
 // ------------------------------------------------------------------------------------------------

@@ -462,7 +462,7 @@ def test_few_row_calls_equal_the_prequantized_path(mod, type_name):
 @pytest.mark.parametrize("type_name", ["q4_k", "q5_k", "iq4_xs", "q6_k", "q2_k"])
 @pytest.mark.parametrize("n,k", [(17408, 5120), (1041, 1000), (16, 256), (300, 17408), (5120, 5120)])
 def test_two_to_four_rows_in_one_pass_equal_single_row_calls(mod, type_name, n, k):
-    """A call of two to four rows (to eight for Q4_K, Q5_K and IQ4_XS) takes all its rows through every block a wave fetches and
+    """A call of two to four rows (to eight for Q4_K, Q5_K and IQ4_XS, and for Q6_K matrices of up to 48 Mi weights) takes all its rows through every block a wave fetches and
     unpacks (one launch, one pass over the weights, whatever the matrix size): each row goes through the same slice image and the
     same products in the same order as in a call of its own, so the results are the same bits; and they meet the float statement
     like the single-row call.  (Three rows or more of 16-bit Q4_K / Q5_K activations in whole super-blocks go to the kernel that
@@ -485,7 +485,7 @@ def test_two_to_four_rows_in_one_pass_equal_single_row_calls(mod, type_name, n, 
     grid = codebooks.grid_tensor_for_type(tid).to(dev)
     rows_w = rng.choice(n, size=min(n, 48), replace=False)
     ref_w = O.dequant_rows(blocks[rows_w], type_name, k)
-    most = 8 if type_name in ("q4_k", "q5_k", "iq4_xs") else 4
+    most = 8 if type_name in ("q4_k", "q5_k", "iq4_xs") or (type_name == "q6_k" and n * bpr * 256 <= 48 << 20) else 4
     for rows in (2, 3, 4, 5, 8):
         if rows > most:
             continue
@@ -574,9 +574,9 @@ def test_multi_projection_equals_separate_calls(mod, type_name):
             # single calls may stream whole tiles), which sums in another order; with the normalisation the row's sum of squares
             # is summed in another order too, which can move an activation code by one step.  A wrong matrix, height or output
             # would be an error of order one.
-            # (five to eight rows: the single calls of Q4_K / Q5_K / IQ4_XS quantize inside their kernel, on the power-of-two scale,
+            # (five to eight rows: the single calls of Q4_K / Q5_K / IQ4_XS / small Q6_K matrices quantize inside their kernel, on the power-of-two scale,
             # the joint call ahead of it: two images of the same rows, each within ~1e-4 of the float statement for float32 rows)
-            same_image = not (5 <= rows <= 8 and type_name in ("q4_k", "q5_k", "iq4_xs"))
+            same_image = not (5 <= rows <= 8 and type_name in ("q4_k", "q5_k", "iq4_xs", "q6_k"))
             for a, b in zip(got, want):
                 assert a.shape == b.shape and O.rel_l2(a.cpu().numpy(), b.cpu().numpy()) <= (2e-6 if same_image else 2e-4)
             got = mod.gguf_quant_gemm_multi_forward(x, mats, k, tid, grid, norm_weight=gamma, eps=1e-5, out_dtype=torch.float32)
