@@ -150,17 +150,23 @@ constexpr int kLdsBytes = 160 * 1024;
 // side in registers across all its chunks; NB == 0: any number, read from LDS every time.
 // WAVES: 8, several workgroups per compute unit, or 16, one workgroup per compute unit around one set of tables (the form for
 // replicated tables, FMT::kCopies > 1, which take the LDS of several plain ones).
-template <typename FMT, int NB, bool RAW, int WAVES>
+// ROWS > 1 (dense calls of two raw rows; the row count in act.round_f16, one grid row): ROWS activation images lie one
+// behind the other, each with its own zero bytes; every block a wave picks out of a chunk is decoded once and multiplied into
+// all of them (the decode, table lookups and sign masks, is what these kernels spend their time on).
+template <typename FMT, int NB, bool RAW, int WAVES, int ROWS = 1>
 __global__ __launch_bounds__(64 * WAVES) void iq_stream_matvec_kernel(
     const ActRows act, const uint8_t* __restrict__ w,
     void* __restrict__ y, int y_dtype, int n, int bpr, int split, int chunks, int chunk_off, int chunk_stride) {
+    static_assert(ROWS == 1 || (NB == 0 && RAW), "the few-row form quantizes its rows itself and holds nothing");
     extern __shared__ __align__(16) unsigned char smem[];
     const int kpad = bpr * 256;
     const int image_bytes = static_cast<int>(staged_x_bytes(kpad));
     const StagedX sx = carve_staged_x(smem, kpad);
-    const int zero_off = image_bytes;                                        // 16 zero bytes
-    const int table_off = image_bytes + 16;
-    float* partial = reinterpret_cast<float*>(smem + table_off + FMT::kTableBytes);   // [waves][16]
+    const int zero_off = image_bytes;                                        // 16 zero bytes behind every image
+    const int image_stride = image_bytes + 16;
+    const int table_off = ROWS * image_stride;
+    const int total_rows = ROWS > 1 ? act.round_f16 : 1;
+    float* partial = reinterpret_cast<float*>(smem + table_off + FMT::kTableBytes);   // [ROWS][waves][16]
     const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_byte_ptr)smem));
 
     const int tid = threadIdx.x;
@@ -176,14 +182,17 @@ __global__ __launch_bounds__(64 * WAVES) void iq_stream_matvec_kernel(
     // activation image, codebooks and the first chunk: all in flight together
     if constexpr (!RAW) dma_share<WAVES>(act.image + static_cast<size_t>(blockIdx.y) * act.stride, lds0, image_bytes, wave, lane);
     if constexpr (FMT::kCopies == 1) FMT::template dma_tables<WAVES>(lds0 + table_off, wave, lane);
-    if (tid < 4) reinterpret_cast<uint32_t*>(smem + zero_off)[tid] = 0;
+    if (tid < 4 * ROWS) reinterpret_cast<uint32_t*>(smem + (tid >> 2) * image_stride + zero_off)[tid & 3] = 0;
     AMap<FMT::kSlots> am;
     FMT::a_map(am, col, ks, kpad, zero_off);
 
     int c = blockIdx.x, buf = 0;
     dma_share<WAVES>(w + static_cast<size_t>(c) * chunk_rows * row_bytes, lds0 + chunk_off, min(chunk_rows, n - c * chunk_rows) * row_bytes, wave, lane);
     if constexpr (FMT::kCopies > 1) FMT::stage_replicated(smem + table_off, tid, 64 * WAVES);   // ordinary stores; the loop's first barrier covers them
-    if constexpr (RAW)                       // raw activation row: quantized once per workgroup while the first chunk is on its way
+    if constexpr (ROWS > 1) {
+        for (int r = 0; r < total_rows; ++r)
+            quantize_row_to_lds(smem + r * image_stride, act.x, act.x_dtype, static_cast<size_t>(r) * act.k, act.k, kpad);
+    } else if constexpr (RAW)                // raw activation row: quantized once per workgroup while the first chunk is on its way
         quantize_row_to_lds(smem, act.x, act.x_dtype, static_cast<size_t>(blockIdx.y) * act.k, act.k, kpad, RowNorm{act.gamma, act.eps, act.round_f16});
     typename FMT::Held held[NB > 0 ? NB : 1];
     bool holding = false;
@@ -206,6 +215,47 @@ __global__ __launch_bounds__(64 * WAVES) void iq_stream_matvec_kernel(
 
         const unsigned char* chunk = smem + chunk_off + buf * chunk_stride;
         float acc = 0.0f;
+        if constexpr (ROWS > 1) {
+            if (tile_in_chunk * kRowsPerTile < valid_rows) {                 // wave-uniform
+                const int row_off = (tile_in_chunk * kRowsPerTile + col) * row_bytes;
+                float accs[ROWS];
+#pragma unroll
+                for (int r = 0; r < ROWS; ++r) accs[r] = 0.0f;
+                AOps<FMT::kSlots> ops;
+                clear_a(ops);                                                // (the slots that are not the lane's stay zero: never loaded)
+                for (int b = part; b < bpr; b += split) {
+                    typename FMT::Regs regs;
+                    FMT::load_lds(regs, chunk, row_off + b * FMT::kBlockBytes, ks);
+                    typename FMT::Decoded o;
+                    FMT::decode(regs, ks, tables, o);
+#pragma unroll
+                    for (int r = 0; r < ROWS; ++r)
+                        if (r < total_rows) {                                // wave-uniform
+                            accs[r] += FMT::route_block(o, ks, b, smem + r * image_stride, am, kpad, ops);
+                        }
+                }
+#pragma unroll
+                for (int r = 0; r < ROWS; ++r) {
+                    const float sum = quad_rows_sum(accs[r]);
+                    if (ks == 0 && r < total_rows) {
+                        if (split == 1) store_any(y, y_dtype, static_cast<size_t>(r) * n + row0 + tile_in_chunk * kRowsPerTile + col, sum);
+                        else partial[(r * WAVES + wave) * kRowsPerTile + col] = sum;
+                    }
+                }
+            }
+            __syncthreads();                 // this buffer may be overwritten, the partial sums are complete
+            if (split > 1 && tid < valid_rows) {
+                const int t = tid / kRowsPerTile, cc = tid % kRowsPerTile;
+                for (int r = 0; r < total_rows; ++r) {
+                    float total = 0.0f;
+                    for (int v = 0; v < split; ++v) total += partial[(r * WAVES + t * split + v) * kRowsPerTile + cc];
+                    store_any(y, y_dtype, static_cast<size_t>(r) * n + row0 + tid, total);
+                }
+            }
+            c = cn;
+            buf ^= 1;
+            continue;
+        }
         if (tile_in_chunk * kRowsPerTile < valid_rows) {                     // wave-uniform
             const int row_off = (tile_in_chunk * kRowsPerTile + col) * row_bytes;
             if constexpr (NB > 0) {
@@ -409,11 +459,11 @@ int launch_exact_for(const ActRows& act, const uint8_t* w, void* y, int y_dtype,
 struct StreamPlan { int waves, split, chunk_off, chunk_stride; size_t smem; };
 
 template <typename FMT>
-StreamPlan stream_plan(const uint8_t* w, int n, int bpr, int waves, int chunk_budget) {
+StreamPlan stream_plan(const uint8_t* w, int n, int bpr, int waves, int chunk_budget, int rows_per_pass = 1) {
     StreamPlan p{waves, 0, 0, 0, 0};
     if (n % kRowsPerTile != 0 || (reinterpret_cast<uintptr_t>(w) & 15u)) return p;
     const int tile_bytes = kRowsPerTile * bpr * FMT::kBlockBytes;
-    const size_t head = staged_x_bytes(bpr * 256) + 16 + FMT::kTableBytes + waves * kRowsPerTile * sizeof(float);
+    const size_t head = rows_per_pass * (staged_x_bytes(bpr * 256) + 16 + waves * kRowsPerTile * sizeof(float)) + FMT::kTableBytes;
     p.chunk_off = static_cast<int>((head + 1023) & ~static_cast<size_t>(1023));
     if (chunk_budget <= 0) chunk_budget = (kLdsBytes - p.chunk_off) / 2 - 16;
     // the most waves per tile first (smallest chunk) that leaves every wave at least two blocks
@@ -426,9 +476,9 @@ StreamPlan stream_plan(const uint8_t* w, int n, int bpr, int waves, int chunk_bu
     return p;
 }
 
-template <typename FMT, int NB, bool RAW, int WAVES>
+template <typename FMT, int NB, bool RAW, int WAVES, int ROWS = 1>
 int launch_stream_raw(const ActRows& act, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, const StreamPlan& p, hipStream_t stream) {
-    auto kern = iq_stream_matvec_kernel<FMT, NB, RAW, WAVES>;
+    auto kern = iq_stream_matvec_kernel<FMT, NB, RAW, WAVES, ROWS>;
     const int tiles_per_chunk = WAVES / p.split;
     static SmemGrant granted;
     if (!grant_dynamic_smem(reinterpret_cast<const void*>(kern), p.smem, granted)) return PLLM_ERR_UNSUPPORTED;
@@ -453,6 +503,14 @@ int launch_stream_raw(const ActRows& act, const uint8_t* w, void* y, int y_dtype
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 
+// two raw rows through every decoded block: one grid row, the row count where the kernel expects it
+template <typename FMT, int WAVES>
+int launch_stream_few(const ActRows& act, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, const StreamPlan& p, hipStream_t stream) {
+    ActRows few = act;
+    few.round_f16 = rows;
+    return launch_stream_raw<FMT, 0, true, WAVES, 2>(few, w, y, y_dtype, 1, n, bpr, p, stream);
+}
+
 template <typename FMT, int NB, int WAVES>
 int launch_stream_nb(const ActRows& act, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, const StreamPlan& p, hipStream_t stream) {
     return act.x ? launch_stream_raw<FMT, NB, true, WAVES>(act, w, y, y_dtype, rows, n, bpr, p, stream)
@@ -475,6 +533,19 @@ int launch_fmt(const ActRows& act, const WeightRoute& route, const uint8_t* w, v
     // always take the latter
     if constexpr (FMT::kStreamed)
         if (!routed(route) && !act.row_token && !act.x_broadcast && route.extra == 0) {
+            // two raw rows of a large matrix: every block decoded once for both (17408x5120 IQ2_XXS 27.8 -> 22.0 us, IQ1_M 26.3 -> 24.5,
+            // 5120x5120 15.5 -> 11.7 and 14.4 -> 13.5, 200064x3072 88.5 -> 78.5 and 111.8 -> 99.4); below 24M weights two grid rows fill
+            // the machine better (IQ1_M 8192x1536 5.4 against 8.7 us), and with four rows in this form each further row still cost
+            // 6 - 10 us (the multiply side: operand loads and MFMAs per image), level with the tile kernel
+            if (act.x && !act.gamma && rows == 2 && static_cast<int64_t>(n) * bpr * 256 >= (int64_t{24} << 20)) {
+                constexpr int rp = 2;
+                if constexpr (std::is_same<FMT, IQ2XXSm>::value) {
+                    const StreamPlan wide = stream_plan<IQ2XXSmT<16>>(w, n, bpr, 16, 0, rp);
+                    if (wide.split) return launch_stream_few<IQ2XXSmT<16>, 16>(act, w, y, y_dtype, rows, n, bpr, wide, stream);
+                }
+                const StreamPlan p = stream_plan<FMT>(w, n, bpr, kWaves, kChunkBudget, rp);
+                if (p.split) return launch_stream_few<FMT, kWaves>(act, w, y, y_dtype, rows, n, bpr, p, stream);
+            }
             const int exact = launch_exact_for<FMT>(act, w, y, y_dtype, rows, n, bpr, stream);
             if (exact != PLLM_ERR_UNSUPPORTED) return exact;
             if constexpr (std::is_same<FMT, IQ2XXSm>::value) {

@@ -510,6 +510,48 @@ def test_two_to_four_rows_in_one_pass_equal_single_row_calls(mod, type_name, n, 
             assert torch.equal(y16, y.to(y16.dtype))
 
 
+@pytest.mark.parametrize("type_name", ["iq2_xxs", "iq1_m"])
+@pytest.mark.parametrize("n,k", [(17408, 5120), (8192, 3072), (6144, 1536), (48, 256), (1041, 1000), (4112, 7168)])
+def test_codebook_two_to_four_rows_decode_every_block_once(mod, type_name, n, k):
+    """Two rows of IQ2_XXS / IQ1_M on a matrix of 24 Mi weights or more that streams through LDS (whole 16-row tiles, 16-byte
+    aligned): every block is decoded once and multiplied into the images of both rows.  Same activation images and integer dots
+    as in single-row calls, the scales multiplied in another order: within float rounding of them.  Other shapes and three or
+    four rows run one grid row per activation row (or, IQ1_M at four rows on the largest matrix, the tile kernel, which rounds
+    weights and activations to fp16).  All meet the float statement of the operator."""
+    rng = np.random.default_rng(n * 3 + k)
+    dev = torch.device("cuda:0")
+    tid = O.TYPE_IDS[type_name]
+    bpr = (k + 255) // 256
+    blocks = (C.random_iq2_xxs if type_name == "iq2_xxs" else C.random_iq1_m)(rng, n, bpr)
+    dblocks = torch.from_numpy(blocks).to(dev)
+    grid = codebooks.grid_tensor_for_type(tid).to(dev)
+    rows_w = rng.choice(n, size=min(n, 48), replace=False)
+    ref_w = O.dequant_rows(blocks[rows_w], type_name, k)
+    for rows in (2, 3, 4):
+        for dt in (torch.float16, torch.float32, torch.bfloat16):
+            x = torch.from_numpy(rng.standard_normal((rows, k)).astype(np.float32)).to(dev).to(dt)
+            x[1] *= 37.0
+            print(f"case {rows} rows {type_name} n={n} k={k} {dt}", flush=True)
+            y = mod.gguf_quant_gemm_forward(x, dblocks, k, tid, grid, out_dtype=torch.float32)
+            singles = torch.cat([mod.gguf_quant_gemm_forward(x[r:r + 1].contiguous(), dblocks, k, tid, grid, out_dtype=torch.float32) for r in range(rows)])
+            torch.cuda.synchronize()
+            assert tuple(y.shape) == (rows, n)
+            tiles = type_name == "iq1_m" and rows == 4 and n * k >= 64 << 20
+            for r in range(rows):
+                assert O.rel_l2(y[r].cpu().numpy(), singles[r].cpu().numpy()) <= (1e-3 if tiles else 1e-6), (rows, r, dt)
+            want = O.matmul_f(x.float().cpu().numpy(), ref_w)
+            got = y.cpu().numpy()[:, rows_w]
+            for r in range(rows):
+                assert O.rel_l2(got[r], want[r]) <= (1e-3 if tiles else 1e-4), (dt, r, O.rel_l2(got[r], want[r]))
+            if tiles:
+                continue                     # (the residual form declines the tile kernel's row counts)
+            # the residual form adds the same product into y
+            y0 = torch.from_numpy(rng.standard_normal((rows, n)).astype(np.float32)).to(dev)
+            acc = y0.clone()
+            mod.gguf_quant_gemm_accumulate_forward(x, dblocks, k, tid, grid, acc)
+            assert torch.allclose(acc, y0 + y, rtol=1e-6, atol=1e-6 * float(y.abs().max()))
+
+
 @pytest.mark.parametrize("type_name", ["q4_k", "q5_k", "q2_k", "q6_k", "iq4_xs", "iq2_xxs", "iq1_m", "iq2_xs", "iq3_xxs"])
 def test_accumulate_adds_the_product_to_y(mod, type_name):
     """The residual form y += W x: equal to the plain operator's float32 product plus the old y, rounded once to y's type,
