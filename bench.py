@@ -605,6 +605,30 @@ def decode_pass(mod, dev) -> None:
                                      "q4_k experts 128 x (2048 -> 768) top-8 one token; 24 launches each"}))
 
 
+def few_rows_pass(mod, dev) -> None:
+    """Dense calls of two to eight activation rows for the profiler, every one a single pass over its weights: Q4_K 17408x5120 at
+    2, 4 and 8 float32 rows, Q6_K 17408x5120 at 4 rows and 5120x5120 at 8 rows, IQ2_XXS and IQ1_M 17408x5120 at 2 rows (rings of
+    weight copies; 24 launches each)."""
+    from pocketllm_amd import block_codec as C, codebooks
+    rng = np.random.default_rng(8008)
+    q4 = rng.integers(0, 256, size=(17408, 20, 144), dtype=np.uint8)
+    q4[..., 0:2] = np.frombuffer(np.float16(0.01).tobytes(), dtype=np.uint8)
+    q4[..., 2:4] = np.frombuffer(np.float16(0.005).tobytes(), dtype=np.uint8)
+    cases = ((3, q4, 5120, (2, 4, 8)), (8, C.random_blocks(rng, "q6_k", 17408, 20), 5120, (4,)), (8, C.random_blocks(rng, "q6_k", 5120, 20), 5120, (8,)),
+             (0, C.random_iq2_xxs(rng, 17408, 20), 5120, (2,)), (2, C.random_iq1_m(rng, 17408, 20), 5120, (2,)))
+    for tid, blocks, k, row_counts in cases:
+        ring = ring_of(blocks, dev, 8)
+        grid = codebooks.grid_tensor_for_type(tid).to(dev)
+        for rows in row_counts:
+            x = torch.randn(rows, k, device=dev)
+            for i in range(24):
+                mod.gguf_quant_gemm_forward(x, ring[i % len(ring)], k, tid, grid)
+        del ring
+    torch.cuda.synchronize()
+    print(json.dumps({"few_rows_pass": "q4_k 17408x5120 at 2 / 4 / 8 rows, q6_k 17408x5120 at 4 and 5120x5120 at 8 rows, iq2_xxs and iq1_m 17408x5120 "
+                                       "at 2 rows; float32 rows, 24 launches each"}))
+
+
 def iq_pass(mod, dev) -> None:
     """A few launches of the codebook formats for the profiler: IQ2_XXS 98304x3072 and IQ1_M 196608x1536 matvec, then the
     single-token routed experts of the 256-expert top-8 configuration."""
@@ -758,6 +782,7 @@ def main() -> None:
     ap.add_argument("--prefill-pass", action="store_true", help="short run for rocprofv3: a few launches of the MFMA tile kernel")
     ap.add_argument("--decode-pass", action="store_true", help="short run for rocprofv3: Q8_0, FP8, Q2_K, Q6_K and IQ4_XS decode matvec")
     ap.add_argument("--fp8-gemm-pass", action="store_true", help="short run for rocprofv3: native FP8 x FP8 matmul at T=512 and T=2048")
+    ap.add_argument("--few-rows-pass", action="store_true", help="short run for rocprofv3: dense calls of two to eight rows in one pass over the weights")
     ap.add_argument("--iq-pass", action="store_true", help="short run for rocprofv3: IQ2_XXS / IQ1_M matvec and the single-token experts")
     ap.add_argument("--experts-rows-pass", action="store_true", help="short run for rocprofv3: grouped routed experts at T=256")
     ap.add_argument("--block-pass", action="store_true", help="short run for rocprofv3: decode steps of one MiniMaxBlock")
@@ -784,6 +809,9 @@ def main() -> None:
         return
     if args.decode_pass:
         decode_pass(mod, dev)
+        return
+    if args.few_rows_pass:
+        few_rows_pass(mod, dev)
         return
     if args.iq_pass:
         iq_pass(mod, dev)
