@@ -97,6 +97,80 @@ __global__ __launch_bounds__(64 * kWaves) void mfma_tile_matvec_kernel(
     }
 }
 
+// Two raw rows of a dense call in one pass over the weights (formats with block_pair): two activation images in LDS, each with
+// its zero bytes behind it; per row the same image, products and float steps as in a call of its own, so the same bits.
+template <typename FMT, int ITERS>
+__global__ __launch_bounds__(64 * kWaves) void mfma_tile_pair_kernel(
+    const ActRows act, const uint8_t* __restrict__ w, void* __restrict__ y, int y_dtype, int n, int bpr) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int kpad = bpr * 256;
+    const int image_bytes = static_cast<int>(staged_x_bytes(kpad));
+    const int image_stride = image_bytes + 16;
+    unsigned char* tables = smem + 2 * image_stride;
+    float* partial = reinterpret_cast<float*>(tables + FMT::kTableBytes);   // [2][waves][16]
+
+    const int tid = threadIdx.x;
+    const int waves = blockDim.x >> 6;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    const int col = lane & 15, ks = lane >> 4;
+    const int row = blockIdx.x * kRowsPerTile + col;
+    const uint8_t* wrow = w + static_cast<size_t>(row < n ? row : 0) * bpr * FMT::kBlockBytes;
+    AMap<FMT::kSlots> am;
+    FMT::a_map(am, col, ks, kpad, image_bytes);
+
+    float acc0 = 0.0f, acc1 = 0.0f;
+    bool staged = false;
+    quantize_row_to_lds(smem, act.x, act.x_dtype, 0, act.k, kpad);
+    quantize_row_to_lds(smem + image_stride, act.x, act.x_dtype, static_cast<size_t>(act.k), act.k, kpad);
+    for (int b0 = wave; b0 < bpr || !staged; b0 += waves * ITERS) {
+        typename FMT::Regs regs[ITERS];
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+            const int b = min(b0 + it * waves, bpr - 1);                    // clamped: always a valid address
+            FMT::load(regs[it], wrow + static_cast<size_t>(b) * FMT::kBlockBytes, ks);
+        }
+        if (!staged) {                       // first trip of every thread of the workgroup
+            if (tid < 8) reinterpret_cast<uint32_t*>(smem + (tid >> 2) * image_stride + image_bytes)[tid & 3] = 0;
+            FMT::stage_tables(tables);
+            __syncthreads();
+            staged = true;
+        }
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+            const int b = b0 + it * waves;
+            if (b < bpr) FMT::block_pair(regs[it], ks, b, smem, smem + image_stride, am, kpad, tables, acc0, acc1);   // wave-uniform guard
+        }
+    }
+    acc0 = quad_rows_sum(acc0);
+    acc1 = quad_rows_sum(acc1);
+    if (ks == 0) {
+        partial[wave * kRowsPerTile + col] = acc0;
+        partial[(waves + wave) * kRowsPerTile + col] = acc1;
+    }
+    __syncthreads();
+    if (tid < 2 * kRowsPerTile) {
+        const int r = tid / kRowsPerTile, cc = tid % kRowsPerTile;
+        float total = 0.0f;
+        for (int v = 0; v < waves; ++v) total += partial[(r * waves + v) * kRowsPerTile + cc];
+        const int out_row = blockIdx.x * kRowsPerTile + cc;
+        if (out_row < n) store_any(y, y_dtype, static_cast<size_t>(r) * n + out_row, total);
+    }
+}
+
+template <typename FMT, int ITERS>
+int launch_tile_pair(const ActRows& act, const uint8_t* w, void* y, int y_dtype, int n, int bpr, int waves, hipStream_t stream) {
+    const size_t smem = 2 * (staged_x_bytes(bpr * 256) + 16) + FMT::kTableBytes + static_cast<size_t>(2 * waves) * kRowsPerTile * sizeof(float);
+    auto kern = mfma_tile_pair_kernel<FMT, ITERS>;
+    if (smem > 64 * 1024) {
+        if (smem > 160 * 1024) return PLLM_ERR_UNSUPPORTED;
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem)) != hipSuccess)
+            return PLLM_ERR_UNSUPPORTED;
+    }
+    hipLaunchKernelGGL(kern, dim3((n + kRowsPerTile - 1) / kRowsPerTile), dim3(64 * waves), smem, stream, act, w, y, y_dtype, n, bpr);
+    return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
+}
+
 template <typename FMT, int ITERS, bool RAW>
 int launch_tile(const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype,
                 int rows, int n, int bpr, int waves, hipStream_t stream) {
@@ -115,6 +189,12 @@ int launch_tile(const ActRows& act, const WeightRoute& route, const uint8_t* w, 
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 
+// The pair kernel halves the number of workgroups and doubles the image's share of LDS: taken from 512 tiles on and up to rows of
+// 32 super-blocks (IQ3_XXS 17408x5120 32.2 -> 24.7 us, 12288x4096 19.3 -> 15.0, 200064x3072 185 -> 124; IQ2_XS 31.3 -> 29.5,
+// 20.4 -> 15.2, 185 -> 144; at 5120x5120 the two were level and at 5120x17408 two grid rows won, 37.4 against 40.5 us)
+constexpr int kPairMinRows = 8192;
+constexpr int kPairMaxBlocksPerRow = 32;
+
 template <typename FMT>
 int launch_tiles(const ActRows& act, const WeightRoute& route, const uint8_t* w, void* y, int y_dtype,
                  int rows, int n, int bpr, hipStream_t stream) {
@@ -124,6 +204,19 @@ int launch_tiles(const ActRows& act, const WeightRoute& route, const uint8_t* w,
     const int niter = (bpr + waves - 1) / waves;
     const int passes = (niter + 5) / 6;
     const int iters = (niter + passes - 1) / passes;
+    // two raw rows of a large dense matrix: one pass over the weights, every block's codes looked up once
+    if constexpr (FMT::kPair)
+        if (act.x && !act.gamma && rows == 2 && !routed(route) && route.extra == 0 && !act.row_token && !act.x_broadcast &&
+            n >= kPairMinRows && bpr <= kPairMaxBlocksPerRow) {
+            switch (iters) {
+                case 1: return launch_tile_pair<FMT, 1>(act, w, y, y_dtype, n, bpr, waves, stream);
+                case 2: return launch_tile_pair<FMT, 2>(act, w, y, y_dtype, n, bpr, waves, stream);
+                case 3: return launch_tile_pair<FMT, 3>(act, w, y, y_dtype, n, bpr, waves, stream);
+                case 4: return launch_tile_pair<FMT, 4>(act, w, y, y_dtype, n, bpr, waves, stream);
+                case 5: return launch_tile_pair<FMT, 5>(act, w, y, y_dtype, n, bpr, waves, stream);
+                default: return launch_tile_pair<FMT, 6>(act, w, y, y_dtype, n, bpr, waves, stream);
+            }
+        }
 #define PLLM_CASE(I) case I: return act.x ? launch_tile<FMT, I, true>(act, route, w, y, y_dtype, rows, n, bpr, waves, stream) \
                                           : launch_tile<FMT, I, false>(act, route, w, y, y_dtype, rows, n, bpr, waves, stream)
     switch (iters) {
