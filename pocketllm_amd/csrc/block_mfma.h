@@ -106,7 +106,7 @@ struct IQ2XXSmT {
     static constexpr int kTableBytes = IQ2XXS::kTableBytes * COPIES;
     static constexpr int kSlots = 4;
     static constexpr bool kStreamed = true;                    // has LDS loaders and table copies for the streamed kernel
-    static constexpr bool kPair = false;                       // (two rows go through the streamed kernel's own form)
+    static constexpr int kRowsPerPass = 1;                     // (two rows go through the streamed kernel's own form)
     static constexpr int kHoldBlocks = 3;                      // block indices whose activation side a wave may keep in registers
     struct Regs { uint4 q; uint32_t d; };
     static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, int s) {
@@ -251,7 +251,7 @@ struct IQ1Mm {
     static __device__ __forceinline__ const unsigned char* lane_tables(const unsigned char* tables, int) { return tables; }
     static constexpr int kSlots = 8;                           // [term][t]
     static constexpr bool kStreamed = true;
-    static constexpr bool kPair = false;
+    static constexpr int kRowsPerPass = 1;
     static constexpr int kHoldBlocks = 3;                      // (109 registers in the streamed kernels: four waves per SIMD; 23.1 -> 21.3 us at 196608x1536)
     struct Regs { uint2 qs; uint32_t qh; uint2 sc; };
     static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, int s) {
@@ -396,7 +396,7 @@ struct Q6Km {
     static constexpr int kTableBytes = 0;
     static constexpr int kSlots = 8;                           // [term][t]
     static constexpr bool kStreamed = false;
-    static constexpr bool kPair = false;
+    static constexpr int kRowsPerPass = 1;
     struct Regs { uint4 qa, qb, qh; uint32_t sc, d; };
     static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, int s) {
         const int half = s >> 1, part = s & 1;
@@ -458,7 +458,7 @@ struct IQ4XSm {
     static constexpr int kTableBytes = 0;
     static constexpr int kSlots = 4;
     static constexpr bool kStreamed = false;
-    static constexpr bool kPair = false;
+    static constexpr int kRowsPerPass = 1;
     struct Regs { uint4 q0, q1; uint2 hdr; };
     static __device__ __forceinline__ void load(Regs& r, const uint8_t* blk, int s) {
         const uint2* p = reinterpret_cast<const uint2*>(blk);                  // blocks are 8-byte aligned
@@ -565,22 +565,25 @@ struct IQ2XSm {
                         l2 * g2.z * static_cast<float>(__mul24(ch.z, 254) + cl.z) + l3 * g2.z * static_cast<float>(__mul24(ch.w, 254) + cl.w);
         return 0.125f * f16_bits_to_float(r.d) * v;
     }
-    // The block against two activation images (each with its zero bytes behind it, offsets of am relative to the image): the
-    // signed codes are looked up once; per image the same products and the same float steps as block().
-    static constexpr bool kPair = true;
-    static __device__ __forceinline__ void block_pair(const Regs& r, int s, int b, const unsigned char* img0, const unsigned char* img1,
-                                                      const AMap<kSlots>& am, int kpad, const unsigned char* tables, float& acc0, float& acc1) {
+    // The block against R activation images that lie image_stride apart (each with its zero bytes behind it, offsets of am
+    // relative to the image): the signed codes are looked up once; per image the same products and the same float steps as block().
+    static constexpr int kRowsPerPass = 2;                     // (every further row costs as much as the lookups: 8 MFMAs per block)
+    template <int R>
+    static __device__ __forceinline__ void block_rows(const Regs& r, int s, int b, const unsigned char* img0, int image_stride,
+                                                      const AMap<kSlots>& am, int kpad, const unsigned char* tables, float (&acc)[R]) {
         const uint2* grid = reinterpret_cast<const uint2*>(tables);
         const uint2* sign = grid + 512;
-        v4i ch[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}}, cl[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+        v4i ch[R], cl[R];
+#pragma unroll
+        for (int i = 0; i < R; ++i) { ch[i] = v4i{0, 0, 0, 0}; cl[i] = v4i{0, 0, 0, 0}; }
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             const uint32_t pair = t == 0 ? r.q.x : t == 1 ? r.q.y : t == 2 ? r.q.z : r.q.w;
             const uint2 w0 = signed8(grid, sign, pair & 0xffffu), w1 = signed8(grid, sign, pair >> 16);
             const v4i bw = as_v4i(w0.x, w0.y, w1.x, w1.y);
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                const unsigned char* img = i ? img1 : img0;
+            for (int i = 0; i < R; ++i) {
+                const unsigned char* img = img0 + i * image_stride;
                 const uint4 ah = *reinterpret_cast<const uint4*>(img + am.off[t] + b * am.step[t]);
                 const uint4 al = *reinterpret_cast<const uint4*>(img + am.off[4 + t] + b * am.step[4 + t]);
                 ch[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(as_v4i(ah.x, ah.y, ah.z, ah.w), bw, ch[i], 0, 0, 0);
@@ -591,11 +594,11 @@ struct IQ2XSm {
         const float l2 = static_cast<float>(2 * ((r.sc >> 8) & 15u) + 1), l3 = static_cast<float>(2 * (r.sc >> 12) + 1);
         const float d8 = 0.125f * f16_bits_to_float(r.d);
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const float4 g2 = *reinterpret_cast<const float4*>((i ? img1 : img0) + 2 * kpad + (b * 8 + 2 * s) * 8);
+        for (int i = 0; i < R; ++i) {
+            const float4 g2 = *reinterpret_cast<const float4*>(img0 + i * image_stride + 2 * kpad + (b * 8 + 2 * s) * 8);
             const float v = l0 * g2.x * static_cast<float>(__mul24(ch[i].x, 254) + cl[i].x) + l1 * g2.x * static_cast<float>(__mul24(ch[i].y, 254) + cl[i].y) +
                             l2 * g2.z * static_cast<float>(__mul24(ch[i].z, 254) + cl[i].z) + l3 * g2.z * static_cast<float>(__mul24(ch[i].w, 254) + cl[i].w);
-            (i ? acc1 : acc0) += d8 * v;
+            acc[i] += d8 * v;
         }
     }
 };
@@ -655,13 +658,16 @@ struct IQ3XXSm {
         const float ls0 = static_cast<float>(2 * (r.aux0 >> 28) + 1), ls1 = static_cast<float>(2 * (r.aux1 >> 28) + 1);
         return 0.25f * f16_bits_to_float(r.d) * (ls0 * g2.x * v0 + ls1 * g2.z * v1);
     }
-    // The block against two activation images (as IQ2XSm::block_pair): ids and signs looked up once.
-    static constexpr bool kPair = true;
-    static __device__ __forceinline__ void block_pair(const Regs& r, int s, int b, const unsigned char* img0, const unsigned char* img1,
-                                                      const AMap<kSlots>& am, int kpad, const unsigned char* tables, float& acc0, float& acc1) {
+    // The block against R activation images (as IQ2XSm::block_rows): ids and signs looked up once.
+    static constexpr int kRowsPerPass = 2;                     // (four rows lost: 17408x5120 55.7 us against 44.8 on the tile kernel, every workgroup quantizes all rows)
+    template <int R>
+    static __device__ __forceinline__ void block_rows(const Regs& r, int s, int b, const unsigned char* img0, int image_stride,
+                                                      const AMap<kSlots>& am, int kpad, const unsigned char* tables, float (&acc)[R]) {
         const uint32_t* grid = reinterpret_cast<const uint32_t*>(tables);
         const uint2* sign = reinterpret_cast<const uint2*>(tables + 1024);
-        v4i c[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+        v4i c[R];
+#pragma unroll
+        for (int i = 0; i < R; ++i) c[i] = v4i{0, 0, 0, 0};
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             const uint32_t ids = t == 0 ? r.ids.x : t == 1 ? r.ids.y : t == 2 ? r.ids.z : r.ids.w;
@@ -670,19 +676,19 @@ struct IQ3XXSm {
             const v4i bw = as_v4i(signed4(grid[ids & 0xffu], m0.x), signed4(grid[(ids >> 8) & 0xffu], m0.y),
                                   signed4(grid[(ids >> 16) & 0xffu], m1.x), signed4(grid[ids >> 24], m1.y));
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                const uint4 a = *reinterpret_cast<const uint4*>((i ? img1 : img0) + am.off[t] + b * am.step[t]);
+            for (int i = 0; i < R; ++i) {
+                const uint4 a = *reinterpret_cast<const uint4*>(img0 + i * image_stride + am.off[t] + b * am.step[t]);
                 c[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(as_v4i(a.x, a.y, a.z, a.w), bw, c[i], 0, 0, 0);
             }
         }
         const float ls0 = static_cast<float>(2 * (r.aux0 >> 28) + 1), ls1 = static_cast<float>(2 * (r.aux1 >> 28) + 1);
         const float d4 = 0.25f * f16_bits_to_float(r.d);
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < R; ++i) {
             const float v0 = static_cast<float>(__mul24(c[i].x, 254) + c[i].y);
             const float v1 = static_cast<float>(__mul24(c[i].z, 254) + c[i].w);
-            const float4 g2 = *reinterpret_cast<const float4*>((i ? img1 : img0) + 2 * kpad + (b * 8 + 2 * s) * 8);
-            (i ? acc1 : acc0) += d4 * (ls0 * g2.x * v0 + ls1 * g2.z * v1);
+            const float4 g2 = *reinterpret_cast<const float4*>(img0 + i * image_stride + 2 * kpad + (b * 8 + 2 * s) * 8);
+            acc[i] += d4 * (ls0 * g2.x * v0 + ls1 * g2.z * v1);
         }
     }
 };

@@ -97,17 +97,19 @@ __global__ __launch_bounds__(64 * kWaves) void mfma_tile_matvec_kernel(
     }
 }
 
-// Two raw rows of a dense call in one pass over the weights (formats with block_pair): two activation images in LDS, each with
-// its zero bytes behind it; per row the same image, products and float steps as in a call of its own, so the same bits.
-template <typename FMT, int ITERS>
-__global__ __launch_bounds__(64 * kWaves) void mfma_tile_pair_kernel(
+// Two to R raw rows of a dense call in one pass over the weights (formats with block_rows; the row count in act.round_f16): R
+// activation images in LDS, each with its zero bytes behind it; per row the same image, products and float steps as in a call
+// of its own, so the same bits.  An image the call has no row for is a copy of the last row's (computed, not stored).
+template <typename FMT, int ITERS, int R>
+__global__ __launch_bounds__(64 * kWaves) void mfma_tile_rows_kernel(
     const ActRows act, const uint8_t* __restrict__ w, void* __restrict__ y, int y_dtype, int n, int bpr) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int kpad = bpr * 256;
     const int image_bytes = static_cast<int>(staged_x_bytes(kpad));
     const int image_stride = image_bytes + 16;
-    unsigned char* tables = smem + 2 * image_stride;
-    float* partial = reinterpret_cast<float*>(tables + FMT::kTableBytes);   // [2][waves][16]
+    unsigned char* tables = smem + R * image_stride;
+    float* partial = reinterpret_cast<float*>(tables + FMT::kTableBytes);   // [R][waves][16]
+    const int total_rows = act.round_f16;
 
     const int tid = threadIdx.x;
     const int waves = blockDim.x >> 6;
@@ -119,10 +121,12 @@ __global__ __launch_bounds__(64 * kWaves) void mfma_tile_pair_kernel(
     AMap<FMT::kSlots> am;
     FMT::a_map(am, col, ks, kpad, image_bytes);
 
-    float acc0 = 0.0f, acc1 = 0.0f;
+    float acc[R];
+#pragma unroll
+    for (int i = 0; i < R; ++i) acc[i] = 0.0f;
     bool staged = false;
-    quantize_row_to_lds(smem, act.x, act.x_dtype, 0, act.k, kpad);
-    quantize_row_to_lds(smem + image_stride, act.x, act.x_dtype, static_cast<size_t>(act.k), act.k, kpad);
+    for (int i = 0; i < R; ++i)
+        quantize_row_to_lds(smem + i * image_stride, act.x, act.x_dtype, static_cast<size_t>(min(i, total_rows - 1)) * act.k, act.k, kpad);
     for (int b0 = wave; b0 < bpr || !staged; b0 += waves * ITERS) {
         typename FMT::Regs regs[ITERS];
 #pragma unroll
@@ -131,7 +135,7 @@ __global__ __launch_bounds__(64 * kWaves) void mfma_tile_pair_kernel(
             FMT::load(regs[it], wrow + static_cast<size_t>(b) * FMT::kBlockBytes, ks);
         }
         if (!staged) {                       // first trip of every thread of the workgroup
-            if (tid < 8) reinterpret_cast<uint32_t*>(smem + (tid >> 2) * image_stride + image_bytes)[tid & 3] = 0;
+            if (tid < 4 * R) reinterpret_cast<uint32_t*>(smem + (tid >> 2) * image_stride + image_bytes)[tid & 3] = 0;
             FMT::stage_tables(tables);
             __syncthreads();
             staged = true;
@@ -139,35 +143,36 @@ __global__ __launch_bounds__(64 * kWaves) void mfma_tile_pair_kernel(
 #pragma unroll
         for (int it = 0; it < ITERS; ++it) {
             const int b = b0 + it * waves;
-            if (b < bpr) FMT::block_pair(regs[it], ks, b, smem, smem + image_stride, am, kpad, tables, acc0, acc1);   // wave-uniform guard
+            if (b < bpr) FMT::template block_rows<R>(regs[it], ks, b, smem, image_stride, am, kpad, tables, acc);   // wave-uniform guard
         }
     }
-    acc0 = quad_rows_sum(acc0);
-    acc1 = quad_rows_sum(acc1);
-    if (ks == 0) {
-        partial[wave * kRowsPerTile + col] = acc0;
-        partial[(waves + wave) * kRowsPerTile + col] = acc1;
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+        const float sum = quad_rows_sum(acc[i]);
+        if (ks == 0) partial[(i * waves + wave) * kRowsPerTile + col] = sum;
     }
     __syncthreads();
-    if (tid < 2 * kRowsPerTile) {
+    if (tid < R * kRowsPerTile) {
         const int r = tid / kRowsPerTile, cc = tid % kRowsPerTile;
         float total = 0.0f;
         for (int v = 0; v < waves; ++v) total += partial[(r * waves + v) * kRowsPerTile + cc];
         const int out_row = blockIdx.x * kRowsPerTile + cc;
-        if (out_row < n) store_any(y, y_dtype, static_cast<size_t>(r) * n + out_row, total);
+        if (out_row < n && r < total_rows) store_any(y, y_dtype, static_cast<size_t>(r) * n + out_row, total);
     }
 }
 
-template <typename FMT, int ITERS>
-int launch_tile_pair(const ActRows& act, const uint8_t* w, void* y, int y_dtype, int n, int bpr, int waves, hipStream_t stream) {
-    const size_t smem = 2 * (staged_x_bytes(bpr * 256) + 16) + FMT::kTableBytes + static_cast<size_t>(2 * waves) * kRowsPerTile * sizeof(float);
-    auto kern = mfma_tile_pair_kernel<FMT, ITERS>;
+template <typename FMT, int ITERS, int R>
+int launch_tile_rows(const ActRows& act, const uint8_t* w, void* y, int y_dtype, int rows, int n, int bpr, int waves, hipStream_t stream) {
+    const size_t smem = R * (staged_x_bytes(bpr * 256) + 16) + FMT::kTableBytes + static_cast<size_t>(R * waves) * kRowsPerTile * sizeof(float);
+    auto kern = mfma_tile_rows_kernel<FMT, ITERS, R>;
     if (smem > 64 * 1024) {
         if (smem > 160 * 1024) return PLLM_ERR_UNSUPPORTED;
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem)) != hipSuccess)
             return PLLM_ERR_UNSUPPORTED;
     }
-    hipLaunchKernelGGL(kern, dim3((n + kRowsPerTile - 1) / kRowsPerTile), dim3(64 * waves), smem, stream, act, w, y, y_dtype, n, bpr);
+    ActRows few = act;
+    few.round_f16 = rows;                    // (where the kernel expects the row count)
+    hipLaunchKernelGGL(kern, dim3((n + kRowsPerTile - 1) / kRowsPerTile), dim3(64 * waves), smem, stream, few, w, y, y_dtype, n, bpr);
     return hipGetLastError() == hipSuccess ? PLLM_OK : PLLM_ERR_LAUNCH;
 }
 
@@ -204,18 +209,17 @@ int launch_tiles(const ActRows& act, const WeightRoute& route, const uint8_t* w,
     const int niter = (bpr + waves - 1) / waves;
     const int passes = (niter + 5) / 6;
     const int iters = (niter + passes - 1) / passes;
-    // two raw rows of a large dense matrix: one pass over the weights, every block's codes looked up once
-    if constexpr (FMT::kPair)
-        if (act.x && !act.gamma && rows == 2 && !routed(route) && route.extra == 0 && !act.row_token && !act.x_broadcast &&
+    // two raw rows of a tall dense matrix: one pass over the weights, every block's codes looked up once
+    if constexpr (FMT::kRowsPerPass > 1)
+        if (act.x && !act.gamma && rows >= 2 && rows <= FMT::kRowsPerPass && !routed(route) && route.extra == 0 && !act.row_token && !act.x_broadcast &&
             n >= kPairMinRows && bpr <= kPairMaxBlocksPerRow) {
+#define PLLM_ROWS_CASE(I) case I: return rows == 2 ? launch_tile_rows<FMT, I, 2>(act, w, y, y_dtype, rows, n, bpr, waves, stream) \
+                                              : launch_tile_rows<FMT, I, FMT::kRowsPerPass>(act, w, y, y_dtype, rows, n, bpr, waves, stream)
             switch (iters) {
-                case 1: return launch_tile_pair<FMT, 1>(act, w, y, y_dtype, n, bpr, waves, stream);
-                case 2: return launch_tile_pair<FMT, 2>(act, w, y, y_dtype, n, bpr, waves, stream);
-                case 3: return launch_tile_pair<FMT, 3>(act, w, y, y_dtype, n, bpr, waves, stream);
-                case 4: return launch_tile_pair<FMT, 4>(act, w, y, y_dtype, n, bpr, waves, stream);
-                case 5: return launch_tile_pair<FMT, 5>(act, w, y, y_dtype, n, bpr, waves, stream);
-                default: return launch_tile_pair<FMT, 6>(act, w, y, y_dtype, n, bpr, waves, stream);
+                PLLM_ROWS_CASE(1); PLLM_ROWS_CASE(2); PLLM_ROWS_CASE(3); PLLM_ROWS_CASE(4); PLLM_ROWS_CASE(5);
+                default: PLLM_ROWS_CASE(6);
             }
+#undef PLLM_ROWS_CASE
         }
 #define PLLM_CASE(I) case I: return act.x ? launch_tile<FMT, I, true>(act, route, w, y, y_dtype, rows, n, bpr, waves, stream) \
                                           : launch_tile<FMT, I, false>(act, route, w, y, y_dtype, rows, n, bpr, waves, stream)

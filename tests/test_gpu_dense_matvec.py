@@ -555,10 +555,10 @@ def test_codebook_two_to_four_rows_decode_every_block_once(mod, type_name, n, k)
 @pytest.mark.parametrize("type_name", ["iq2_xs", "iq3_xxs"])
 @pytest.mark.parametrize("n,k", [(17408, 5120), (8192, 3072), (8200, 1000), (8192, 8192), (4096, 3072), (8192, 8448)])
 def test_two_rows_of_iq2_xs_iq3_xxs_in_one_pass_equal_single_row_calls(mod, type_name, n, k):
-    """Two rows of IQ2_XS / IQ3_XXS on a matrix of 8192 rows or more and rows of up to 32 super-blocks: both activation images in
-    LDS, every block's codes looked up once; per row the same image, products and float steps as a single-row call, so the same
-    bits (ragged rows and a last tile that is not whole included).  Shorter or wider matrices run one grid row per activation
-    row.  The residual form adds the same product."""
+    """Two rows of IQ2_XS / IQ3_XXS on a matrix of 8192 rows or more and rows of up to 32 super-blocks: both activation images
+    in LDS, every block's codes looked up once; per row the same image, products and float steps as a single-row call, so the
+    same bits (ragged rows and a last tile that is not whole included).  Shorter or wider matrices and three rows run one grid
+    row per activation row: the same bits too.  The residual form adds the same product."""
     rng = np.random.default_rng(n + 7 * k)
     dev = torch.device("cuda:0")
     tid = O.TYPE_IDS[type_name]
@@ -569,24 +569,25 @@ def test_two_rows_of_iq2_xs_iq3_xxs_in_one_pass_equal_single_row_calls(mod, type
     rows_w = rng.choice(n, size=48, replace=False)
     rows_w[0] = n - 1
     ref_w = O.dequant_rows(blocks[rows_w], type_name, k)
-    for dt in (torch.float16, torch.float32, torch.bfloat16):
-        x = torch.from_numpy(rng.standard_normal((2, k)).astype(np.float32)).to(dev).to(dt)
-        x[1] *= 37.0
-        print(f"case two rows {type_name} n={n} k={k} {dt}", flush=True)
-        y = mod.gguf_quant_gemm_forward(x, dblocks, k, tid, grid, out_dtype=torch.float32)
-        singles = torch.cat([mod.gguf_quant_gemm_forward(x[r:r + 1].contiguous(), dblocks, k, tid, grid, out_dtype=torch.float32) for r in range(2)])
-        torch.cuda.synchronize()
-        assert tuple(y.shape) == (2, n) and torch.equal(y, singles)
-        want = O.matmul_f(x.float().cpu().numpy(), ref_w)
-        got = y.cpu().numpy()[:, rows_w]
-        for r in range(2):
-            assert O.rel_l2(got[r], want[r]) <= 1e-4, (dt, r, O.rel_l2(got[r], want[r]))
-        y0 = torch.from_numpy(rng.standard_normal((2, n)).astype(np.float32)).to(dev)
-        acc = y0.clone()
-        mod.gguf_quant_gemm_accumulate_forward(x, dblocks, k, tid, grid, acc)
-        assert torch.equal(acc, y0 + y)
-        y16 = mod.gguf_quant_gemm_forward(x, dblocks, k, tid, grid)
-        assert torch.equal(y16, y.to(y16.dtype))
+    for rows in (2, 3):
+        for dt in (torch.float16, torch.float32, torch.bfloat16):
+            x = torch.from_numpy(rng.standard_normal((rows, k)).astype(np.float32)).to(dev).to(dt)
+            x[1] *= 37.0
+            print(f"case {rows} rows {type_name} n={n} k={k} {dt}", flush=True)
+            y = mod.gguf_quant_gemm_forward(x, dblocks, k, tid, grid, out_dtype=torch.float32)
+            singles = torch.cat([mod.gguf_quant_gemm_forward(x[r:r + 1].contiguous(), dblocks, k, tid, grid, out_dtype=torch.float32) for r in range(rows)])
+            torch.cuda.synchronize()
+            assert tuple(y.shape) == (rows, n) and torch.equal(y, singles)
+            want = O.matmul_f(x.float().cpu().numpy(), ref_w)
+            got = y.cpu().numpy()[:, rows_w]
+            for r in range(rows):
+                assert O.rel_l2(got[r], want[r]) <= 1e-4, (dt, r, O.rel_l2(got[r], want[r]))
+            y0 = torch.from_numpy(rng.standard_normal((rows, n)).astype(np.float32)).to(dev)
+            acc = y0.clone()
+            mod.gguf_quant_gemm_accumulate_forward(x, dblocks, k, tid, grid, acc)
+            assert torch.equal(acc, y0 + y)
+            y16 = mod.gguf_quant_gemm_forward(x, dblocks, k, tid, grid)
+            assert torch.equal(y16, y.to(y16.dtype))
 
 
 @pytest.mark.parametrize("type_name", ["q4_k", "q5_k", "q2_k", "q6_k", "iq4_xs", "iq2_xxs", "iq1_m", "iq2_xs", "iq3_xxs"])
