@@ -607,15 +607,16 @@ def decode_pass(mod, dev) -> None:
 
 def few_rows_pass(mod, dev) -> None:
     """Dense calls of two to eight activation rows for the profiler, every one a single pass over its weights: Q4_K 17408x5120 at
-    2, 4 and 8 float32 rows, Q6_K 17408x5120 at 4 rows and 5120x5120 at 8 rows, IQ2_XXS and IQ1_M 17408x5120 at 2 rows (rings of
-    weight copies; 24 launches each)."""
+    2, 4 and 8 float32 rows, Q6_K 17408x5120 at 4 rows and 5120x5120 at 8 rows, IQ2_XXS, IQ1_M, IQ3_XXS and IQ2_XS 17408x5120
+    at 2 rows (rings of weight copies; 24 launches each)."""
     from pocketllm_amd import block_codec as C, codebooks
     rng = np.random.default_rng(8008)
     q4 = rng.integers(0, 256, size=(17408, 20, 144), dtype=np.uint8)
     q4[..., 0:2] = np.frombuffer(np.float16(0.01).tobytes(), dtype=np.uint8)
     q4[..., 2:4] = np.frombuffer(np.float16(0.005).tobytes(), dtype=np.uint8)
     cases = ((3, q4, 5120, (2, 4, 8)), (8, C.random_blocks(rng, "q6_k", 17408, 20), 5120, (4,)), (8, C.random_blocks(rng, "q6_k", 5120, 20), 5120, (8,)),
-             (0, C.random_iq2_xxs(rng, 17408, 20), 5120, (2,)), (2, C.random_iq1_m(rng, 17408, 20), 5120, (2,)))
+             (0, C.random_iq2_xxs(rng, 17408, 20), 5120, (2,)), (2, C.random_iq1_m(rng, 17408, 20), 5120, (2,)),
+             (6, C.random_blocks(rng, "iq3_xxs", 17408, 20), 5120, (2,)), (5, C.random_blocks(rng, "iq2_xs", 17408, 20), 5120, (2,)))
     for tid, blocks, k, row_counts in cases:
         ring = ring_of(blocks, dev, 8)
         grid = codebooks.grid_tensor_for_type(tid).to(dev)
@@ -625,8 +626,8 @@ def few_rows_pass(mod, dev) -> None:
                 mod.gguf_quant_gemm_forward(x, ring[i % len(ring)], k, tid, grid)
         del ring
     torch.cuda.synchronize()
-    print(json.dumps({"few_rows_pass": "q4_k 17408x5120 at 2 / 4 / 8 rows, q6_k 17408x5120 at 4 and 5120x5120 at 8 rows, iq2_xxs and iq1_m 17408x5120 "
-                                       "at 2 rows; float32 rows, 24 launches each"}))
+    print(json.dumps({"few_rows_pass": "q4_k 17408x5120 at 2 / 4 / 8 rows, q6_k 17408x5120 at 4 and 5120x5120 at 8 rows, iq2_xxs, iq1_m, iq3_xxs and iq2_xs "
+                                       "17408x5120 at 2 rows; float32 rows, 24 launches each"}))
 
 
 def iq_pass(mod, dev) -> None:
